@@ -1,0 +1,128 @@
+"""Build recipe for the native libraries of this package.
+
+``libgs_hip.so``  HIP kernels + C ABI (``include/gs_hip.h``); hipcc, gfx950 only,
+                  no torch dependency.
+``libgs.so``      C++ host layer (``gs::Graph``, ``graph_ops``, TORCH_LIBRARY
+                  registration) on top of the C ABI; built by
+                  :func:`build_host` when its sources are present.
+
+Both are built in-tree, next to this file.  Run ``python -m graph_sampling_amd.build``.
+"""
+import glob
+import os
+import subprocess
+import sys
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_CSRC = os.path.join(_PKG, "csrc")
+_ROOT = os.path.dirname(_PKG)
+
+KERNEL_LIB = os.path.join(_PKG, "libgs_hip.so")
+HOST_LIB = os.path.join(_PKG, "libgs.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+HIP_FLAGS = [
+    "--offload-arch=" + ARCH,
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-ffp-contract=off",
+    "-fhip-fp32-correctly-rounded-divide-sqrt",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-result",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines()
+                    if "is not a recognized feature for this target" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def kernel_sources():
+    return sorted(glob.glob(os.path.join(_CSRC, "*.hip"))) + [os.path.join(_CSRC, "gs_api.cpp")]
+
+
+def build_kernels(verbose=False):
+    """Compile every HIP translation unit for gfx950 and link libgs_hip.so."""
+    objdir = os.path.join(_PKG, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = []
+    procs = []
+    for src in kernel_sources():
+        obj = os.path.join(objdir, os.path.basename(src) + ".o")
+        objs.append(obj)
+        cmd = [HIPCC] + HIP_FLAGS + ["-x", "hip", "-c", src, "-o", obj]
+        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                                            text=True)))
+    for cmd, p in procs:
+        out, _ = p.communicate()
+        out = "\n".join(l for l in out.splitlines()
+                        if "is not a recognized feature for this target" not in l)
+        if p.returncode != 0:
+            raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+        if verbose and out.strip():
+            print(out)
+    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", KERNEL_LIB] + objs)
+    return KERNEL_LIB
+
+
+def host_sources():
+    return sorted(glob.glob(os.path.join(_CSRC, "host", "*.cc")))
+
+
+def build_host(verbose=False):
+    """Compile the C++ host layer against libtorch and link it to libgs_hip.so."""
+    srcs = host_sources()
+    if not srcs:
+        return None
+    import torch
+    from torch.utils import cpp_extension as ce
+    objdir = os.path.join(_PKG, "build")
+    os.makedirs(objdir, exist_ok=True)
+    inc = []
+    for p in ce.include_paths():
+        inc += ["-isystem", p]
+    inc += ["-isystem", "/opt/rocm/include", "-I", os.path.join(_ROOT, "include")]
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    flags = ["-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+             "-D_GLIBCXX_USE_CXX11_ABI=%d" % abi, "-Wno-deprecated-declarations"]
+    objs, procs = [], []
+    for src in srcs:
+        obj = os.path.join(objdir, "host_" + os.path.basename(src) + ".o")
+        objs.append(obj)
+        cmd = ["g++"] + flags + inc + ["-c", src, "-o", obj]
+        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                                            text=True)))
+    for cmd, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+        if verbose and out.strip():
+            print(out)
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    link = ["g++", "-shared", "-o", HOST_LIB] + objs + [
+        "-L" + _PKG, "-lgs_hip", "-Wl,-rpath,$ORIGIN",
+        "-L" + torch_lib, "-lc10", "-ltorch_cpu", "-ltorch", "-lc10_hip", "-ltorch_hip",
+        "-Wl,-rpath," + torch_lib,
+        "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib",
+    ]
+    _run(link)
+    return HOST_LIB
+
+
+def build_all(verbose=False):
+    libs = [build_kernels(verbose)]
+    host = build_host(verbose)
+    if host:
+        libs.append(host)
+    return libs
+
+
+if __name__ == "__main__":
+    for lib in build_all(verbose="-v" in sys.argv):
+        print("built", lib)

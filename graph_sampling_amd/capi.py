@@ -1,0 +1,465 @@
+"""ctypes binding of the C ABI declared in ``include/gs_hip.h``.
+
+torch is used for device memory and the current HIP stream only; every call
+hands raw device pointers and sizes to ``libgs_hip.so``.  There is no fallback:
+if the library is missing, importing a symbol raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libgs_hip.so")
+
+_lib = None
+
+
+class GsError(RuntimeError):
+    """A C-ABI call returned a negative gs_status."""
+
+
+def lib():
+    """The loaded kernel library (raises when it has not been built)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise GsError("%s is missing: run `python -m graph_sampling_amd.build`" % LIB_PATH)
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.gs_status_string.restype = ctypes.c_char_p
+        _lib.gs_status_string.argtypes = [ctypes.c_int]
+        for name in ("gs_slice_workspace_bytes", "gs_sample_workspace_bytes",
+                     "gs_sample_weighted_workspace_bytes", "gs_list_sample_workspace_bytes",
+                     "gs_unique_workspace_bytes", "gs_row_slice_workspace_bytes",
+                     "gs_coo2csc_workspace_bytes"):
+            if hasattr(_lib, name):
+                getattr(_lib, name).restype = ctypes.c_size_t
+    return _lib
+
+
+def _check(status, what):
+    if status != 0:
+        raise GsError("%s failed (%d): %s" % (what, status, lib().gs_status_string(status).decode()))
+
+
+def _ptr(t):
+    if t is None:
+        return ctypes.c_void_p(0)
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def _u64(v):
+    return ctypes.c_uint64(int(v) & 0xFFFFFFFFFFFFFFFF)
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _id_bytes(t):
+    if t.dtype == torch.int64:
+        return 8
+    if t.dtype == torch.int32:
+        return 4
+    raise GsError("node ids must be int64 or int32, got %s" % t.dtype)
+
+
+def _need(t, dtype, name):
+    if t.dtype != dtype:
+        raise GsError("%s must be %s, got %s" % (name, dtype, t.dtype))
+    if not t.is_cuda:
+        raise GsError("%s must live on the GPU (there is no CPU path)" % name)
+    if not t.is_contiguous():
+        raise GsError("%s must be contiguous" % name)
+
+
+def _ids(t, name, like=None):
+    if not t.is_cuda:
+        raise GsError("%s must live on the GPU (there is no CPU path)" % name)
+    if not t.is_contiguous():
+        raise GsError("%s must be contiguous" % name)
+    b = _id_bytes(t)
+    if like is not None and t.dtype != like.dtype:
+        raise GsError("%s must have the dtype of the graph ids (%s), got %s" % (name, like.dtype, t.dtype))
+    return b
+
+
+def _replay(t):
+    """Replay draws are raw uint32 values; torch carries them as int32 bit patterns."""
+    if t.element_size() != 4 or not t.is_cuda or not t.is_contiguous():
+        raise GsError("replay must be a contiguous 4-byte integer tensor on the GPU")
+
+
+class _Workspace:
+    """One growing scratch buffer per device (256-byte aligned by the torch allocator)."""
+
+    def __init__(self):
+        self._buf = {}
+
+    def get(self, nbytes, device):
+        nbytes = max(int(nbytes), 256)
+        key = torch.device(device).index or 0
+        buf = self._buf.get(key)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=device)
+            self._buf[key] = buf
+        return buf
+
+
+_ws = _Workspace()
+
+
+def workspace(nbytes, device):
+    return _ws.get(nbytes, device)
+
+
+# ---------------------------------------------------------------- slicing ----
+def slice_count(indptr, column_ids):
+    """gs_slice_count -> sub_indptr[S+1] (device); total still on the device."""
+    _need(indptr, torch.int64, "indptr")
+    idb = _ids(column_ids, "column_ids")
+    S = column_ids.numel()
+    sub_indptr = torch.empty(S + 1, dtype=torch.int64, device=indptr.device)
+    nbytes = lib().gs_slice_workspace_bytes(_i64(S))
+    ws = workspace(nbytes, indptr.device)
+    _check(lib().gs_slice_count(_ptr(indptr), _ptr(column_ids), idb, _i64(S), _ptr(sub_indptr),
+                                _ptr(ws), ctypes.c_size_t(ws.numel()), _stream(indptr.device)),
+           "gs_slice_count")
+    return sub_indptr
+
+
+def slice_fill(indptr, indices, column_ids, sub_indptr, nnz, with_coo):
+    _need(indptr, torch.int64, "indptr")
+    idb = _ids(indices, "indices")
+    _ids(column_ids, "column_ids", like=indices)
+    S = column_ids.numel()
+    dev = indptr.device
+    sub_indices = torch.empty(nnz, dtype=indices.dtype, device=dev)
+    select_index = torch.empty(nnz, dtype=torch.int64, device=dev)
+    coo_col = torch.empty(nnz, dtype=indices.dtype, device=dev) if with_coo else None
+    _check(lib().gs_slice_fill(_ptr(indptr), _ptr(indices), _ptr(column_ids), idb, _i64(S),
+                               _ptr(sub_indptr), _i64(nnz), _ptr(sub_indices), _ptr(select_index),
+                               _ptr(coo_col), _stream(dev)), "gs_slice_fill")
+    return sub_indices, select_index, coo_col
+
+
+# --------------------------------------------------------------- sampling ----
+def sample_uniform(indptr, indices, column_ids, fanout, replace, seed=0, replay=None,
+                   replay_ptr=None, with_coo=False):
+    """gs_sample_count + gs_sample_uniform_fill on upper-bound buffers.
+
+    Returns (sub_indptr, sub_indices_buf, select_index_buf, coo_col_buf); the
+    buffers have capacity S*fanout and the caller narrows them to
+    sub_indptr[S] once it has read that value."""
+    _need(indptr, torch.int64, "indptr")
+    idb = _ids(indices, "indices")
+    dev = indptr.device
+    if column_ids is None:
+        S = indptr.numel() - 1
+    else:
+        _ids(column_ids, "column_ids", like=indices)
+        S = column_ids.numel()
+    if replay is not None:
+        _replay(replay)
+        _need(replay_ptr, torch.int64, "replay_ptr")
+    sub_indptr = torch.empty(S + 1, dtype=torch.int64, device=dev)
+    cap = S * int(fanout)
+    sub_indices = torch.empty(cap, dtype=indices.dtype, device=dev)
+    select_index = torch.empty(cap, dtype=torch.int64, device=dev)
+    coo_col = torch.empty(cap, dtype=indices.dtype, device=dev) if with_coo else None
+    nbytes = lib().gs_sample_workspace_bytes(_i64(S), _i64(fanout))
+    ws = workspace(nbytes, dev)
+    st = _stream(dev)
+    _check(lib().gs_sample_count(_ptr(indptr), _ptr(column_ids), idb, _i64(S), _i64(fanout),
+                                 int(bool(replace)), _ptr(sub_indptr), _ptr(ws),
+                                 ctypes.c_size_t(ws.numel()), st), "gs_sample_count")
+    _check(lib().gs_sample_uniform_fill(_ptr(indptr), _ptr(indices), _ptr(column_ids), idb, _i64(S),
+                                        _i64(fanout), int(bool(replace)), _u64(seed), _ptr(replay),
+                                        _ptr(replay_ptr), _ptr(sub_indptr), _ptr(sub_indices),
+                                        _ptr(select_index), _ptr(coo_col), _ptr(ws),
+                                        ctypes.c_size_t(ws.numel()), st), "gs_sample_uniform_fill")
+    return sub_indptr, sub_indices, select_index, coo_col
+
+
+def sample_one_keepdim(indptr, indices, column_ids, seed=0, replay=None):
+    _need(indptr, torch.int64, "indptr")
+    idb = _ids(indices, "indices")
+    _ids(column_ids, "column_ids", like=indices)
+    dev = indptr.device
+    S = column_ids.numel()
+    sub_indptr = torch.empty(S + 1, dtype=torch.int64, device=dev)
+    sub_indices = torch.empty(S, dtype=indices.dtype, device=dev)
+    select_index = torch.empty(S, dtype=torch.int64, device=dev)
+    _check(lib().gs_sample_one_keepdim(_ptr(indptr), _ptr(indices), _ptr(column_ids), idb, _i64(S),
+                                       _u64(seed), _ptr(replay), _ptr(sub_indptr), _ptr(sub_indices),
+                                       _ptr(select_index), _stream(dev)), "gs_sample_one_keepdim")
+    return sub_indptr, sub_indices, select_index
+
+
+def sample_weighted(indptr, indices, probs, column_ids, fanout, seed=0, replay=None,
+                    replay_ptr=None, with_coo=False):
+    """gs_sample_count(replace=0) + gs_sample_weighted_fill; same return shape as sample_uniform."""
+    _need(indptr, torch.int64, "indptr")
+    _need(probs, torch.float32, "probs")
+    idb = _ids(indices, "indices")
+    dev = indptr.device
+    if column_ids is None:
+        S = indptr.numel() - 1
+    else:
+        _ids(column_ids, "column_ids", like=indices)
+        S = column_ids.numel()
+    sub_indptr = torch.empty(S + 1, dtype=torch.int64, device=dev)
+    cap = S * int(fanout)
+    sub_indices = torch.empty(cap, dtype=indices.dtype, device=dev)
+    select_index = torch.empty(cap, dtype=torch.int64, device=dev)
+    coo_col = torch.empty(cap, dtype=indices.dtype, device=dev) if with_coo else None
+    nbytes = max(lib().gs_sample_workspace_bytes(_i64(S), _i64(fanout)),
+                 lib().gs_sample_weighted_workspace_bytes(_i64(S), _i64(fanout)))
+    ws = workspace(nbytes, dev)
+    st = _stream(dev)
+    _check(lib().gs_sample_count(_ptr(indptr), _ptr(column_ids), idb, _i64(S), _i64(fanout), 0,
+                                 _ptr(sub_indptr), _ptr(ws), ctypes.c_size_t(ws.numel()), st),
+           "gs_sample_count")
+    _check(lib().gs_sample_weighted_fill(_ptr(indptr), _ptr(indices), _ptr(probs), _ptr(column_ids),
+                                         idb, _i64(S), _i64(fanout), _u64(seed), _ptr(replay),
+                                         _ptr(replay_ptr), _ptr(sub_indptr), _ptr(sub_indices),
+                                         _ptr(select_index), _ptr(coo_col), _ptr(ws),
+                                         ctypes.c_size_t(ws.numel()), st), "gs_sample_weighted_fill")
+    return sub_indptr, sub_indices, select_index, coo_col
+
+
+def list_sample_uniform(data, k, replace, seed=0, replay=None):
+    idb = _ids(data, "data")
+    dev = data.device
+    n = data.numel()
+    out_data = torch.empty(k, dtype=data.dtype, device=dev)
+    out_index = torch.empty(k, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_list_sample_workspace_bytes(_i64(n), _i64(k)), dev)
+    _check(lib().gs_list_sample_uniform(_ptr(data), idb, _i64(n), _i64(k), int(bool(replace)),
+                                        _u64(seed), _ptr(replay), _ptr(out_data), _ptr(out_index),
+                                        _ptr(ws), ctypes.c_size_t(ws.numel()), _stream(dev)),
+           "gs_list_sample_uniform")
+    return out_data, out_index
+
+
+def list_sample_weighted(data, probs, k, seed=0, replay=None):
+    idb = _ids(data, "data")
+    _need(probs, torch.float32, "probs")
+    dev = data.device
+    n = data.numel()
+    out_data = torch.empty(k, dtype=data.dtype, device=dev)
+    out_index = torch.empty(k, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_list_sample_workspace_bytes(_i64(n), _i64(k)), dev)
+    _check(lib().gs_list_sample_weighted(_ptr(data), idb, _ptr(probs), _i64(n), _i64(k), _u64(seed),
+                                         _ptr(replay), _ptr(out_data), _ptr(out_index), _ptr(ws),
+                                         ctypes.c_size_t(ws.numel()), _stream(dev)),
+           "gs_list_sample_weighted")
+    return out_data, out_index
+
+
+# ---------------------------------------------------------- unique/relabel ----
+class _Span(ctypes.Structure):
+    _fields_ = [("ptr", ctypes.c_void_p), ("n", ctypes.c_int64)]
+
+
+def unique_relabel(mapping, queries):
+    """gs_unique_relabel.  mapping / queries: lists of 1-D id tensors (one dtype).
+
+    Returns (frontier_buf, num_unique_dev, [relabelled query tensors]); frontier_buf has
+    capacity sum(len(mapping)) and num_unique_dev is a 1-element int64 device tensor."""
+    dev = mapping[0].device
+    idb = _ids(mapping[0], "mapping[0]")
+    for i, t in enumerate(list(mapping[1:]) + list(queries)):
+        _ids(t, "relabel tensor %d" % (i + 1), like=mapping[0])
+    M = sum(int(t.numel()) for t in mapping)
+    frontier = torch.empty(M, dtype=mapping[0].dtype, device=dev)
+    num_unique = torch.empty(1, dtype=torch.int64, device=dev)
+    outs = [torch.empty_like(q) for q in queries]
+    MapArr = _Span * max(len(mapping), 1)
+    QArr = _Span * max(len(queries), 1)
+    OutArr = ctypes.c_void_p * max(len(queries), 1)
+    m_arr = MapArr(*[_Span(t.data_ptr(), t.numel()) for t in mapping])
+    q_arr = QArr(*[_Span(t.data_ptr(), t.numel()) for t in queries]) if queries else QArr()
+    o_arr = OutArr(*[t.data_ptr() for t in outs]) if queries else OutArr()
+    ws = workspace(lib().gs_unique_workspace_bytes(_i64(M)), dev)
+    _check(lib().gs_unique_relabel(m_arr, len(mapping), q_arr, o_arr, len(queries), idb,
+                                   _ptr(frontier), _ptr(num_unique), _ptr(ws),
+                                   ctypes.c_size_t(ws.numel()), _stream(dev)), "gs_unique_relabel")
+    return frontier, num_unique, outs
+
+
+# ------------------------------------------------------------------ walks ----
+def random_walk(indptr, indices, seeds, length, seed=0, replay=None):
+    _need(indptr, torch.int64, "indptr")
+    idb = _ids(indices, "indices")
+    _ids(seeds, "seeds", like=indices)
+    dev = indptr.device
+    n = seeds.numel()
+    trace = torch.empty((int(length) + 1) * n, dtype=indices.dtype, device=dev)
+    _check(lib().gs_random_walk(_ptr(indptr), _ptr(indices), idb, _ptr(seeds), _i64(n), _i64(length),
+                                _u64(seed), _ptr(replay), _ptr(trace), _stream(dev)),
+           "gs_random_walk")
+    return trace
+
+
+def metapath_walk(indptr_table, indices_table, id_dtype, metapath, seeds, seed=0, replay=None):
+    """indptr_table / indices_table: device int64 tensors holding device addresses."""
+    _need(metapath, torch.int64, "metapath")
+    idb = _ids(seeds, "seeds")
+    if seeds.dtype != id_dtype:
+        raise GsError("seeds must have the dtype of the relation graphs' ids")
+    dev = seeds.device
+    n = seeds.numel()
+    L = metapath.numel()
+    trace = torch.empty((L + 1) * n, dtype=seeds.dtype, device=dev)
+    _check(lib().gs_metapath_walk(_ptr(indptr_table), _ptr(indices_table), idb, _ptr(metapath),
+                                  _i64(L), _ptr(seeds), _i64(n), _u64(seed), _ptr(replay),
+                                  _ptr(trace), _stream(dev)), "gs_metapath_walk")
+    return trace
+
+
+# ------------------------------------------------------------------ SDDMM ----
+OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "copy_lhs": 4, "copy_rhs": 5, "dot": 6}
+
+
+def sddmm_coo(op, row, col, e_ids, lhs, rhs, out, lhs_target, rhs_target, lhs_len, rhs_len,
+              out_len, reduce_size, lhs_off=None, rhs_off=None):
+    if op not in OPS:
+        raise GsError("Unsupported SpMM/SDDMM binary operator: %s" % op)
+    _need(row, torch.int64, "row")
+    _need(col, torch.int64, "col")
+    _need(out, torch.float32, "out")
+    dev = row.device
+    _check(lib().gs_sddmm_coo(OPS[op], _ptr(row), _ptr(col), _ptr(e_ids), _i64(row.numel()),
+                              _ptr(lhs), _ptr(rhs), _ptr(out), int(lhs_target), int(rhs_target),
+                              _i64(lhs_len), _i64(rhs_len), _i64(out_len), _i64(reduce_size),
+                              _ptr(lhs_off), _ptr(rhs_off), _stream(dev)), "gs_sddmm_coo")
+
+
+def sddmm_csc(op, indptr, indices, e_ids, nid_map, lhs, rhs, out, lhs_target, rhs_target, lhs_len,
+              rhs_len, out_len, reduce_size, lhs_off=None, rhs_off=None):
+    if op not in OPS:
+        raise GsError("Unsupported SpMM/SDDMM binary operator: %s" % op)
+    _need(indptr, torch.int64, "indptr")
+    _need(indices, torch.int64, "indices")
+    _need(out, torch.float32, "out")
+    dev = indptr.device
+    _check(lib().gs_sddmm_csc(OPS[op], _ptr(indptr), _ptr(indices), _ptr(e_ids), _ptr(nid_map),
+                              _i64(indptr.numel() - 1), _i64(indices.numel()), _ptr(lhs), _ptr(rhs),
+                              _ptr(out), int(lhs_target), int(rhs_target), _i64(lhs_len),
+                              _i64(rhs_len), _i64(out_len), _i64(reduce_size), _ptr(lhs_off),
+                              _ptr(rhs_off), _stream(dev)), "gs_sddmm_csc")
+
+
+# ------------------------------------------------------------ segment ops ----
+def segment_sum(indptr, e_ids, n_ids, data, powk, out):
+    _need(indptr, torch.int64, "indptr")
+    _need(data, torch.float32, "data")
+    _need(out, torch.float32, "out")
+    _check(lib().gs_segment_sum(_ptr(indptr), _ptr(e_ids), _ptr(n_ids), _ptr(data),
+                                _i64(indptr.numel() - 1), _i64(powk), _ptr(out),
+                                _stream(indptr.device)), "gs_segment_sum")
+
+
+def coo_sum(target, e_ids, data, powk, out):
+    _need(target, torch.int64, "target")
+    _need(data, torch.float32, "data")
+    _need(out, torch.float32, "out")
+    _check(lib().gs_coo_sum(_ptr(target), _ptr(e_ids), _ptr(data), _i64(target.numel()), _i64(powk),
+                            _ptr(out), _stream(target.device)), "gs_coo_sum")
+
+
+def segment_normalize(indptr, e_ids, data, out):
+    _need(indptr, torch.int64, "indptr")
+    _need(data, torch.float32, "data")
+    _need(out, torch.float32, "out")
+    _check(lib().gs_segment_normalize(_ptr(indptr), _ptr(e_ids), _ptr(data),
+                                      _i64(indptr.numel() - 1), _ptr(out), _stream(indptr.device)),
+           "gs_segment_normalize")
+
+
+def e_div_u_sum(row, col, data, divisor, out_data, out_sum):
+    _need(row, torch.int64, "row")
+    _need(col, torch.int64, "col")
+    _need(data, torch.float32, "data")
+    _need(divisor, torch.float32, "divisor")
+    _check(lib().gs_e_div_u_sum(_ptr(row), _ptr(col), _ptr(data), _ptr(divisor), _i64(row.numel()),
+                                _ptr(out_data), _ptr(out_sum), _stream(row.device)),
+           "gs_e_div_u_sum")
+
+
+# ------------------------------------------------------------ row slicing ----
+def row_slice_csc(indptr, indices, row_ids, with_coo):
+    """Two-phase gs_row_slice_csc_*; returns (out_indptr, coo_col|None, out_indices, select_index)."""
+    _need(indptr, torch.int64, "indptr")
+    _need(indices, torch.int64, "indices")
+    _need(row_ids, torch.int64, "row_ids")
+    dev = indptr.device
+    ncols, nnz, nr = indptr.numel() - 1, indices.numel(), row_ids.numel()
+    out_indptr = torch.empty(ncols + 1, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_row_slice_workspace_bytes(_i64(nr), _i64(nnz), _i64(ncols)), dev)
+    st = _stream(dev)
+    _check(lib().gs_row_slice_csc_mark(_ptr(indptr), _ptr(indices), _i64(ncols), _i64(nnz),
+                                       _ptr(row_ids), _i64(nr), _ptr(out_indptr), _ptr(ws),
+                                       ctypes.c_size_t(ws.numel()), st), "gs_row_slice_csc_mark")
+    kept = int(out_indptr[-1].item())
+    out_indices = torch.empty(kept, dtype=torch.int64, device=dev)
+    select_index = torch.empty(kept, dtype=torch.int64, device=dev)
+    coo_col = torch.empty(kept, dtype=torch.int64, device=dev) if with_coo else None
+    _check(lib().gs_row_slice_csc_compact(_ptr(indptr), _ptr(indices), _i64(ncols), _i64(nnz),
+                                          _ptr(out_indptr), _ptr(out_indices), _ptr(select_index),
+                                          _ptr(coo_col), _ptr(ws), ctypes.c_size_t(ws.numel()), st),
+           "gs_row_slice_csc_compact")
+    return out_indptr, coo_col, out_indices, select_index
+
+
+def row_slice_coo(key, other, ids):
+    """Two-phase gs_row_slice_coo_*; returns (relabelled key, other, select_index)."""
+    _need(key, torch.int64, "key")
+    _need(other, torch.int64, "other")
+    _need(ids, torch.int64, "ids")
+    dev = key.device
+    E, n = key.numel(), ids.numel()
+    num_kept = torch.empty(1, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_row_slice_workspace_bytes(_i64(n), _i64(E), _i64(0)), dev)
+    st = _stream(dev)
+    _check(lib().gs_row_slice_coo_mark(_ptr(key), _i64(E), _ptr(ids), _i64(n), _ptr(num_kept),
+                                       _ptr(ws), ctypes.c_size_t(ws.numel()), st),
+           "gs_row_slice_coo_mark")
+    kept = int(num_kept.item())
+    out_key = torch.empty(kept, dtype=torch.int64, device=dev)
+    out_other = torch.empty(kept, dtype=torch.int64, device=dev)
+    select_index = torch.empty(kept, dtype=torch.int64, device=dev)
+    _check(lib().gs_row_slice_coo_compact(_ptr(key), _ptr(other), _i64(E), _ptr(out_key),
+                                          _ptr(out_other), _ptr(select_index), _ptr(ws),
+                                          ctypes.c_size_t(ws.numel()), st), "gs_row_slice_coo_compact")
+    return out_key, out_other, select_index
+
+
+# ------------------------------------------------------- format transform ----
+def csc2coo(indptr, nnz):
+    _need(indptr, torch.int64, "indptr")
+    col = torch.empty(nnz, dtype=torch.int64, device=indptr.device)
+    _check(lib().gs_csc2coo(_ptr(indptr), _i64(indptr.numel() - 1), _i64(nnz), _ptr(col),
+                            _stream(indptr.device)), "gs_csc2coo")
+    return col
+
+
+def coo2csc(key, value, num_keys, is_sorted):
+    """Returns (indptr, sorted value | value, perm | None)."""
+    _need(key, torch.int64, "key")
+    _need(value, torch.int64, "value")
+    dev = key.device
+    E = key.numel()
+    indptr = torch.empty(num_keys + 1, dtype=torch.int64, device=dev)
+    out_value = None if is_sorted else torch.empty(E, dtype=torch.int64, device=dev)
+    perm = None if is_sorted else torch.empty(E, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_coo2csc_workspace_bytes(_i64(E), _i64(num_keys)), dev)
+    _check(lib().gs_coo2csc(_ptr(key), _ptr(value), _i64(E), _i64(num_keys), int(bool(is_sorted)),
+                            _ptr(indptr), _ptr(out_value), _ptr(perm), _ptr(ws),
+                            ctypes.c_size_t(ws.numel()), _stream(dev)), "gs_coo2csc")
+    return indptr, (value if is_sorted else out_value), perm

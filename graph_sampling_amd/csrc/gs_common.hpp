@@ -1,0 +1,285 @@
+// Shared device/host helpers for the gfx950 kernels: status reporting, the
+// Philox draw, wave-level primitives and a tiled exclusive scan.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/gs_hip.h"
+
+namespace gs {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// ---------------------------------------------------------------- status ----
+void set_error_text(const char* fmt, ...);
+
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error_text("%s: %s", what, hipGetErrorString(e));
+    return GS_ERR_LAUNCH;
+  }
+  return GS_OK;
+}
+
+#define GS_REQUIRE(cond, ...)            \
+  do {                                   \
+    if (!(cond)) {                       \
+      ::gs::set_error_text(__VA_ARGS__); \
+      return GS_ERR_INVALID_ARG;         \
+    }                                    \
+  } while (0)
+
+#define GS_RETURN_IF_ERROR(expr) \
+  do {                           \
+    int _s = (expr);             \
+    if (_s != GS_OK) return _s;  \
+  } while (0)
+
+inline bool valid_id_bytes(int b) { return b == 4 || b == 8; }
+
+// Carves 256-byte aligned pieces out of the caller's workspace.
+struct Carver {
+  char* base;
+  size_t cap;
+  size_t off = 0;
+  bool ok = true;
+  Carver(void* p, size_t bytes) : base(static_cast<char*>(p)), cap(bytes) {
+    if ((reinterpret_cast<uintptr_t>(p) & 255u) != 0) ok = false;
+  }
+  template <typename T>
+  T* take(size_t count) {
+    size_t bytes = (count * sizeof(T) + 255u) & ~size_t(255);
+    if (!ok || off + bytes > cap) {
+      ok = false;
+      return nullptr;
+    }
+    T* r = reinterpret_cast<T*>(base + off);
+    off += bytes;
+    return r;
+  }
+};
+inline size_t padded(size_t bytes) { return (bytes + 255u) & ~size_t(255); }
+
+// ---------------------------------------------------------------- Philox ----
+constexpr uint32_t kTagUniform = 1u;
+constexpr uint32_t kTagWeighted = 2u;
+constexpr uint32_t kTagWalk = 3u;
+constexpr uint32_t kTagListUniform = 4u;
+constexpr uint32_t kTagListWeighted = 5u;
+
+struct U4 {
+  uint32_t v[4];
+};
+
+// Philox4x32-10 (Salmon et al., SC'11).
+__device__ __forceinline__ U4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                            uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    uint32_t hi0 = __umulhi(0xD2511F53u, c0);
+    uint32_t lo0 = 0xD2511F53u * c0;
+    uint32_t hi1 = __umulhi(0xCD9E8D57u, c2);
+    uint32_t lo1 = 0xCD9E8D57u * c2;
+    uint32_t n0 = hi1 ^ c1 ^ k0;
+    uint32_t n2 = hi0 ^ c3 ^ k1;
+    c0 = n0;
+    c1 = lo1;
+    c2 = n2;
+    c3 = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  U4 r;
+  r.v[0] = c0;
+  r.v[1] = c1;
+  r.v[2] = c2;
+  r.v[3] = c3;
+  return r;
+}
+
+// The four draws for idx = 4q .. 4q+3 of `row`.
+__device__ __forceinline__ U4 draw_block(uint64_t seed, uint32_t tag, uint64_t row, uint64_t q) {
+  return philox4x32_10(static_cast<uint32_t>(q), static_cast<uint32_t>(row),
+                       static_cast<uint32_t>(row >> 32),
+                       tag | (static_cast<uint32_t>(q >> 32) << 8), static_cast<uint32_t>(seed),
+                       static_cast<uint32_t>(seed >> 32));
+}
+
+__device__ __forceinline__ uint32_t draw_one(uint64_t seed, uint32_t tag, uint64_t row,
+                                             uint64_t idx) {
+  U4 b = draw_block(seed, tag, row, idx >> 2);
+  return b.v[idx & 3];
+}
+
+// A-Res key log2(u)/w, u = ((x>>8)+1) * 2^-24.  Only correctly rounded binary32
+// operations (explicit fmaf, IEEE division) so that a host evaluation of the
+// same recipe gives the same bits; requires -ffp-contract=off.
+__device__ __forceinline__ float log2_u24(uint32_t x) {
+  uint32_t m = (x >> 8) + 1u;
+  int e = 31 - __clz(static_cast<int>(m));
+  float f = static_cast<float>(m) * __uint_as_float(static_cast<uint32_t>(127 - e) << 23);  // m * 2^-e, exact
+  if (f > 1.41421356f) {
+    f = f * 0.5f;
+    e += 1;
+  }
+  float s = __fdiv_rn(f - 1.0f, f + 1.0f);
+  float z = s * s;
+  float p = __fmaf_rn(z, 0.11111111f, 0.14285715f);
+  p = __fmaf_rn(z, p, 0.2f);
+  p = __fmaf_rn(z, p, 0.33333334f);
+  p = __fmaf_rn(z, p, 1.0f);
+  float l = (s * 2.88539008f) * p;
+  return l + static_cast<float>(e - 24);
+}
+
+__device__ __forceinline__ float ares_key(uint32_t x, float w) {
+  if (!(w > 0.0f)) return -__builtin_inff();
+  return __fdiv_rn(log2_u24(x), w);
+}
+
+// Order-preserving map float -> uint32 (larger float => larger uint).
+__device__ __forceinline__ uint32_t float_to_ordered(float f) {
+  uint32_t b = __float_as_uint(f);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+// ------------------------------------------------------------ id helpers ----
+template <typename T>
+__device__ __forceinline__ T ld(const T* p) {
+  return *p;
+}
+
+inline int blocks_for(int64_t n, int per_block) {
+  int64_t b = (n + per_block - 1) / per_block;
+  return static_cast<int>(b < 1 ? 1 : b);
+}
+
+// ------------------------------------------------------------ block scan ----
+// Exclusive scan of one int64 per thread over a block of kThreads threads
+// (multiple of 64).  Returns the exclusive prefix; *total gets the block sum.
+template <int kThreads>
+__device__ __forceinline__ int64_t block_exclusive_scan(int64_t v, int64_t* total,
+                                                        int64_t* lds /* kThreads/64 + 1 */) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  int64_t incl = v;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    int64_t o = __shfl_up(incl, d, kWave);
+    if (lane >= d) incl += o;
+  }
+  if (lane == kWave - 1) lds[wave] = incl;
+  __syncthreads();
+  constexpr int kWaves = kThreads / kWave;
+  if (threadIdx.x == 0) {
+    int64_t acc = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      int64_t t = lds[w];
+      lds[w] = acc;
+      acc += t;
+    }
+    lds[kWaves] = acc;
+  }
+  __syncthreads();
+  int64_t r = lds[wave] + incl - v;
+  *total = lds[kWaves];
+  __syncthreads();
+  return r;
+}
+
+// ------------------------------------------------- device-wide scan (tiled) --
+// out[i] = sum_{j<i} f(j) for i in [0, n]; out has n+1 entries.  Three phases:
+// per-tile sums, a one-block scan of the tile sums, per-tile scan + offset.
+// n <= kScanTile runs as a single launch.
+constexpr int kScanThreads = 256;
+constexpr int kScanItems = 8;
+constexpr int kScanTile = kScanThreads * kScanItems;
+
+inline int64_t scan_num_tiles(int64_t n) { return n <= 0 ? 1 : (n + kScanTile - 1) / kScanTile; }
+inline size_t scan_workspace_bytes(int64_t n) { return padded((scan_num_tiles(n) + 1) * 8); }
+
+template <typename F>
+__global__ void __launch_bounds__(kScanThreads) scan_tile_sums_kernel(F f, int64_t n,
+                                                                      int64_t* tile_sums) {
+  __shared__ int64_t lds[kScanThreads / kWave + 1];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kScanTile;
+  int64_t acc = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    int64_t i = base + k * kScanThreads + threadIdx.x;
+    if (i < n) acc += f(i);
+  }
+  int64_t total;
+  block_exclusive_scan<kScanThreads>(acc, &total, lds);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// in-place exclusive scan of tile_sums[0..m) by one block; tile_sums[m] = total
+static __global__ void __launch_bounds__(kScanThreads) scan_tile_offsets_kernel(int64_t* tile_sums,
+                                                                         int64_t m) {
+  __shared__ int64_t lds[kScanThreads / kWave + 1];
+  int64_t carry = 0;
+  for (int64_t base = 0; base < m; base += kScanThreads) {
+    int64_t i = base + threadIdx.x;
+    int64_t v = i < m ? tile_sums[i] : 0;
+    int64_t total;
+    int64_t ex = block_exclusive_scan<kScanThreads>(v, &total, lds);
+    if (i < m) tile_sums[i] = carry + ex;
+    carry += total;
+  }
+  if (threadIdx.x == 0) tile_sums[m] = carry;
+}
+
+// Thread t of the block owns items base + t*kScanItems .. +kScanItems-1 so the
+// per-thread prefix is a running sum (blocked arrangement).
+template <typename F>
+__global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(F f, int64_t n,
+                                                                  const int64_t* tile_offsets,
+                                                                  int64_t* out) {
+  __shared__ int64_t lds[kScanThreads / kWave + 1];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kScanTile +
+                       static_cast<int64_t>(threadIdx.x) * kScanItems;
+  int64_t v[kScanItems];
+  int64_t acc = 0;
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    int64_t i = base + k;
+    v[k] = i < n ? f(i) : 0;
+    acc += v[k];
+  }
+  int64_t total;
+  int64_t ex = block_exclusive_scan<kScanThreads>(acc, &total, lds);
+  int64_t run = ex + (tile_offsets ? tile_offsets[blockIdx.x] : 0);
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) {
+    int64_t i = base + k;
+    if (i < n) out[i] = run;
+    run += v[k];
+    if (i == n - 1) out[n] = run;
+  }
+  if (n == 0 && blockIdx.x == 0 && threadIdx.x == 0) out[0] = 0;
+}
+
+// Enqueues the scan.  tile_ws: scan_workspace_bytes(n) bytes.
+template <typename F>
+inline int exclusive_scan(F f, int64_t n, int64_t* out, int64_t* tile_ws, hipStream_t stream) {
+  const int64_t tiles = scan_num_tiles(n);
+  if (tiles == 1) {
+    hipLaunchKernelGGL(scan_apply_kernel<F>, dim3(1), dim3(kScanThreads), 0, stream, f, n,
+                       static_cast<const int64_t*>(nullptr), out);
+    return check_launch("scan_apply");
+  }
+  hipLaunchKernelGGL(scan_tile_sums_kernel<F>, dim3(static_cast<unsigned>(tiles)),
+                     dim3(kScanThreads), 0, stream, f, n, tile_ws);
+  hipLaunchKernelGGL(scan_tile_offsets_kernel, dim3(1), dim3(kScanThreads), 0, stream, tile_ws,
+                     tiles);
+  hipLaunchKernelGGL(scan_apply_kernel<F>, dim3(static_cast<unsigned>(tiles)),
+                     dim3(kScanThreads), 0, stream, f, n,
+                     static_cast<const int64_t*>(tile_ws), out);
+  return check_launch("scan");
+}
+
+}  // namespace gs

@@ -1,0 +1,582 @@
+// Column slicing and uniform neighbour sampling for CSC graphs on gfx950.
+//
+// Replaces impl::CSCColSlicingCUDA (reference src/cuda/slicing.cu:170),
+// impl::CSCColSamplingCUDA (src/cuda/sampling.cu:157) and
+// impl::fusion::FusedCSCColSlicingSampling[OneKeepDim]CUDA
+// (src/cuda/fusion/slice_sampling.cu:146,157).
+//
+// Layout of the work:
+//  * offsets: one tiled exclusive scan whose input (degree or min(degree,k)) is
+//    computed on the fly from indptr, so no intermediate degree array exists;
+//  * slice fill: edge-balanced -- every workgroup owns 2048 consecutive OUTPUT
+//    positions and finds their rows by binary search in an LDS copy of the
+//    offsets, so a power-law hub row is spread over many workgroups and all
+//    stores are fully coalesced;
+//  * sampling: rows are binned by degree.  deg <= k copies; k < deg <= 1024 runs
+//    Algorithm R inside a 16-lane group with the k slots in LDS (ds_max); larger
+//    rows keep their slots in the output buffer and are cut into 4096-draw
+//    chunks; the chunks go through a device queue so that a second kernel
+//    spreads them evenly over the chip, and a last pass gathers the ids.
+#include "gs_common.hpp"
+
+namespace gs {
+namespace {
+
+// ------------------------------------------------------------- functors ----
+template <typename IdT>
+struct ColDegree {
+  const int64_t* indptr;
+  const IdT* cols;  // nullptr: identity
+  __device__ __forceinline__ int64_t operator()(int64_t r) const {
+    int64_t c = cols ? static_cast<int64_t>(cols[r]) : r;
+    return indptr[c + 1] - indptr[c];
+  }
+};
+
+template <typename IdT>
+struct ColCount {
+  const int64_t* indptr;
+  const IdT* cols;
+  int64_t k;
+  int replace;
+  __device__ __forceinline__ int64_t operator()(int64_t r) const {
+    int64_t c = cols ? static_cast<int64_t>(cols[r]) : r;
+    int64_t deg = indptr[c + 1] - indptr[c];
+    if (replace) return deg == 0 ? 0 : k;
+    return deg < k ? deg : k;
+  }
+};
+
+// first index i in [0, n) with a[i] > v (n if none)
+template <typename P>
+__device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
+  int64_t lo = 0, hi = n;
+  while (lo < hi) {
+    int64_t mid = (lo + hi) >> 1;
+    if (a[mid] <= v) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+// ----------------------------------------------------------- slice fill ----
+constexpr int kFillThreads = 256;
+constexpr int kFillItems = 8;
+constexpr int kFillTile = kFillThreads * kFillItems;
+constexpr int kFillStage = 1024;  // rows of offsets staged in LDS
+
+template <typename IdT, bool WITH_COO>
+__global__ void __launch_bounds__(kFillThreads)
+slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
+                  const IdT* __restrict__ cols, int64_t S, const int64_t* __restrict__ sub_indptr,
+                  int64_t nnz, IdT* __restrict__ sub_indices, int64_t* __restrict__ select_index,
+                  IdT* __restrict__ coo_col) {
+  __shared__ int64_t s_ptr[kFillStage + 1];
+  __shared__ int64_t s_in[kFillStage];
+  __shared__ int64_t s_rows[2];
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kFillTile;
+  const int64_t p1 = p0 + kFillTile < nnz ? p0 + kFillTile : nnz;
+  if (threadIdx.x < 2) {
+    int64_t p = threadIdx.x == 0 ? p0 : p1 - 1;
+    s_rows[threadIdx.x] = upper_bound(sub_indptr, S + 1, p) - 1;
+  }
+  __syncthreads();
+  const int64_t row_lo = s_rows[0];
+  const int64_t nrows = s_rows[1] - row_lo + 1;
+  const bool staged = nrows <= kFillStage;
+  if (staged) {
+    for (int64_t i = threadIdx.x; i <= nrows; i += kFillThreads) {
+      s_ptr[i] = sub_indptr[row_lo + i];
+      if (i < nrows) {
+        int64_t c = cols ? static_cast<int64_t>(cols[row_lo + i]) : row_lo + i;
+        s_in[i] = indptr[c];
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kFillItems; ++k) {
+    const int64_t p = p0 + k * kFillThreads + threadIdx.x;
+    if (p >= p1) break;
+    int64_t row, q;
+    if (staged) {
+      int64_t i = upper_bound(s_ptr, nrows + 1, p) - 1;
+      row = row_lo + i;
+      q = s_in[i] + (p - s_ptr[i]);
+    } else {
+      row = row_lo + upper_bound(sub_indptr + row_lo, nrows + 1, p) - 1;
+      int64_t c = cols ? static_cast<int64_t>(cols[row]) : row;
+      q = indptr[c] + (p - sub_indptr[row]);
+    }
+    sub_indices[p] = indices[q];
+    select_index[p] = q;
+    if (WITH_COO) coo_col[p] = static_cast<IdT>(row);
+  }
+}
+
+// ------------------------------------------------------------- sampling ----
+constexpr int kSampleThreads = 256;
+constexpr int kGroup = 16;                                   // lanes per row
+constexpr int kGroupsPerBlock = kSampleThreads / kGroup;     // 16
+constexpr int kRowsPerBlock = 64;
+constexpr int kRounds = kRowsPerBlock / kGroupsPerBlock;     // 4
+constexpr int64_t kGroupMaxDeg = 1024;  // larger rows take the chunked path
+constexpr int kChunkIters = 4;
+constexpr int64_t kChunkDraws = int64_t(kSampleThreads) * 4 * kChunkIters;  // 4096
+constexpr int kHubGrid = 2048;           // workgroups draining the chunk queue
+constexpr int kChunkBits = 20;           // chunk index bits of a queue entry
+constexpr int64_t kQueueExtra = 1 << 20; // queue capacity = S + kQueueExtra chunks
+constexpr int64_t kMaxLdsFanout = 768;  // 16 groups * 768 * 4 B = 48 KB
+
+template <typename IdT>
+struct SampleArgs {
+  const int64_t* indptr;
+  const IdT* indices;
+  const IdT* cols;
+  int64_t S;
+  int64_t k;
+  uint64_t seed;
+  const uint32_t* replay;
+  const int64_t* replay_ptr;
+  const int64_t* sub_indptr;
+  IdT* sub_indices;
+  int64_t* select_index;
+  IdT* coo_col;
+  long long* queue;                 // chunk queue entries (row << kChunkBits | chunk), -1 = void
+  unsigned long long* queue_count;  // chunks reserved so far (may exceed queue_cap)
+  int64_t queue_cap;
+};
+
+// Draws idx in [4*q_lo, 4*q_hi) of row r and applies Algorithm R to int64 slots
+// in global memory.  `stride` threads cooperate, this one is number `tid`.
+template <typename IdT>
+__device__ __forceinline__ void reservoir_draws_global(const SampleArgs<IdT>& a, int64_t r,
+                                                       int64_t deg, long long* slot,
+                                                       int64_t q_lo, int64_t q_hi, int tid,
+                                                       int stride) {
+  const int64_t k = a.k;
+  const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[r] : nullptr;
+  for (int64_t q = q_lo + tid; q < q_hi; q += stride) {
+    U4 x;
+    if (!rp) x = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(r), static_cast<uint64_t>(q));
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int64_t idx = q * 4 + t;
+      if (idx >= k && idx < deg) {
+        const uint32_t xv = rp ? rp[idx - k] : x.v[t];
+        const uint32_t num = xv % static_cast<uint32_t>(idx + 1);
+        if (static_cast<int64_t>(num) < k) atomicMax(&slot[num], static_cast<long long>(idx));
+      }
+    }
+  }
+}
+
+template <typename IdT>
+__device__ __forceinline__ void load_row(const SampleArgs<IdT>& a, int64_t r, int64_t* start,
+                                         int64_t* deg, int64_t* out_start) {
+  int64_t c = a.cols ? static_cast<int64_t>(a.cols[r]) : r;
+  *start = a.indptr[c];
+  *deg = a.indptr[c + 1] - *start;
+  *out_start = a.sub_indptr[r];
+}
+
+// Without replacement.  Rows with deg <= k are copied, rows up to kGroupMaxDeg
+// run Algorithm R in LDS (when GROUP_TIER), larger rows only get their slots
+// initialised (slot j = j, stored in select_index) for the chunked passes.
+template <typename IdT, bool WITH_COO, bool GROUP_TIER>
+__global__ void __launch_bounds__(kSampleThreads) sample_rows_kernel(SampleArgs<IdT> a) {
+  extern __shared__ int32_t s_slots[];
+  const int g = threadIdx.x / kGroup;
+  const int lane = threadIdx.x % kGroup;
+  const int64_t k = a.k;
+  int32_t* slot = s_slots + (GROUP_TIER ? g * k : 0);
+  for (int round = 0; round < kRounds; ++round) {
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + round * kGroupsPerBlock + g;
+    int mode = 0;  // 1 copy, 2 reservoir in LDS, 3 chunked
+    int64_t start = 0, deg = 0, out_start = 0;
+    if (r < a.S) {
+      load_row(a, r, &start, &deg, &out_start);
+      mode = deg <= k ? 1 : ((GROUP_TIER && deg <= kGroupMaxDeg) ? 2 : 3);
+    }
+    if (GROUP_TIER) {
+      if (mode == 2)
+        for (int64_t j = lane; j < k; j += kGroup) slot[j] = static_cast<int32_t>(j);
+      __syncthreads();
+      if (mode == 2) {
+        const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[r] : nullptr;
+        for (int64_t q = (k >> 2) + lane; q <= ((deg - 1) >> 2); q += kGroup) {
+          U4 x;
+          if (!rp) x = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(r), static_cast<uint64_t>(q));
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int64_t idx = q * 4 + t;
+            if (idx >= k && idx < deg) {
+              const uint32_t xv = rp ? rp[idx - k] : x.v[t];
+              const uint32_t num = xv % static_cast<uint32_t>(idx + 1);
+              if (static_cast<int64_t>(num) < k) atomicMax(&slot[num], static_cast<int32_t>(idx));
+            }
+          }
+        }
+      }
+      __syncthreads();
+    }
+    if (mode == 1) {
+      for (int64_t j = lane; j < deg; j += kGroup) {
+        a.sub_indices[out_start + j] = a.indices[start + j];
+        a.select_index[out_start + j] = start + j;
+        if (WITH_COO) a.coo_col[out_start + j] = static_cast<IdT>(r);
+      }
+    } else if (mode == 2) {
+      for (int64_t j = lane; j < k; j += kGroup) {
+        const int64_t p = start + slot[j];
+        a.sub_indices[out_start + j] = a.indices[p];
+        a.select_index[out_start + j] = p;
+        if (WITH_COO) a.coo_col[out_start + j] = static_cast<IdT>(r);
+      }
+    } else if (mode == 3) {
+      // slots start as j; the draws are queued as 4096-draw chunks
+      for (int64_t j = lane; j < k; j += kGroup) a.select_index[out_start + j] = j;
+      const int64_t q_lo = k >> 2, q_hi = ((deg - 1) >> 2) + 1;
+      const int64_t q_per_chunk = kChunkDraws / 4;
+      const int64_t nchunks = (q_hi - q_lo + q_per_chunk - 1) / q_per_chunk;
+      unsigned long long base = 0;
+      if (lane == 0) base = atomicAdd(a.queue_count, static_cast<unsigned long long>(nchunks));
+      base = __shfl(base, 0, kGroup);
+      if (static_cast<int64_t>(base) + nchunks <= a.queue_cap) {
+        for (int64_t c = lane; c < nchunks; c += kGroup)
+          a.queue[base + c] = static_cast<long long>((r << kChunkBits) | c);
+      } else {
+        // queue full: void the reserved tail and draw here with this group
+        for (int64_t c = static_cast<int64_t>(base) + lane;
+             c < a.queue_cap && c < static_cast<int64_t>(base) + nchunks; c += kGroup)
+          a.queue[c] = -1;
+        __threadfence();
+        reservoir_draws_global(a, r, deg, reinterpret_cast<long long*>(a.select_index + out_start),
+                               q_lo, q_hi, lane, kGroup);
+      }
+    }
+    if (GROUP_TIER) __syncthreads();
+  }
+}
+
+// Drains the chunk queue: one workgroup per 4096-draw chunk, grid-stride.
+// Slots live in select_index (int64, initialised to j); global atomicMax is
+// rare: a draw at position idx hits a slot with probability k/(idx+1).
+template <typename IdT>
+__global__ void __launch_bounds__(kSampleThreads) sample_hub_draw_kernel(SampleArgs<IdT> a) {
+  const unsigned long long reserved = *a.queue_count;
+  const int64_t n = reserved < static_cast<unsigned long long>(a.queue_cap)
+                        ? static_cast<int64_t>(reserved)
+                        : a.queue_cap;
+  const int64_t q_per_chunk = kChunkDraws / 4;
+  for (int64_t t = blockIdx.x; t < n; t += gridDim.x) {
+    const long long e = a.queue[t];
+    if (e < 0) continue;
+    const int64_t r = e >> kChunkBits;
+    const int64_t c = e & ((1 << kChunkBits) - 1);
+    int64_t start, deg, out_start;
+    load_row(a, r, &start, &deg, &out_start);
+    const int64_t q_lo = (a.k >> 2) + c * q_per_chunk;
+    int64_t q_hi = ((deg - 1) >> 2) + 1;
+    if (q_lo + q_per_chunk < q_hi) q_hi = q_lo + q_per_chunk;
+    reservoir_draws_global(a, r, deg, reinterpret_cast<long long*>(a.select_index + out_start),
+                           q_lo, q_hi, threadIdx.x, kSampleThreads);
+  }
+}
+
+static __global__ void zero_counter_kernel(unsigned long long* p) {
+  if (threadIdx.x == 0) *p = 0;
+}
+
+// Turns the slots of chunked rows into (neighbour id, edge position).
+template <typename IdT, bool WITH_COO>
+__global__ void __launch_bounds__(kSampleThreads)
+sample_hub_gather_kernel(SampleArgs<IdT> a, int64_t min_deg) {
+  const int g = threadIdx.x / kGroup;
+  const int lane = threadIdx.x % kGroup;
+  const int64_t k = a.k;
+  for (int round = 0; round < kRounds; ++round) {
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + round * kGroupsPerBlock + g;
+    if (r >= a.S) continue;
+    int64_t start, deg, out_start;
+    load_row(a, r, &start, &deg, &out_start);
+    if (!(deg > k && deg > min_deg)) continue;
+    for (int64_t j = lane; j < k; j += kGroup) {
+      const int64_t p = start + a.select_index[out_start + j];
+      a.sub_indices[out_start + j] = a.indices[p];
+      a.select_index[out_start + j] = p;
+      if (WITH_COO) a.coo_col[out_start + j] = static_cast<IdT>(r);
+    }
+  }
+}
+
+// With replacement: slot j of row r = draw(r, j) % deg (sampling.cu:29-39).
+template <typename IdT, bool WITH_COO>
+__global__ void __launch_bounds__(kSampleThreads) sample_replace_kernel(SampleArgs<IdT> a) {
+  const int g = threadIdx.x / kGroup;
+  const int lane = threadIdx.x % kGroup;
+  for (int round = 0; round < kRounds; ++round) {
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + round * kGroupsPerBlock + g;
+    if (r >= a.S) continue;
+    int64_t start, deg, out_start;
+    load_row(a, r, &start, &deg, &out_start);
+    const int64_t cnt = a.sub_indptr[r + 1] - out_start;
+    const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[r] : nullptr;
+    for (int64_t q = lane; q * 4 < cnt; q += kGroup) {
+      U4 x;
+      if (!rp) x = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(r), static_cast<uint64_t>(q));
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int64_t j = q * 4 + t;
+        if (j < cnt) {
+          const uint32_t xv = rp ? rp[j] : x.v[t];
+          const int64_t p = start + static_cast<int64_t>(xv % static_cast<uint32_t>(deg));
+          a.sub_indices[out_start + j] = a.indices[p];
+          a.select_index[out_start + j] = p;
+          if (WITH_COO) a.coo_col[out_start + j] = static_cast<IdT>(r);
+        }
+      }
+    }
+  }
+}
+
+// One slot per column, -1 for an empty column (slice_sampling.cu:171-198).
+template <typename IdT>
+__global__ void __launch_bounds__(256)
+sample_one_keepdim_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
+                          const IdT* __restrict__ cols, int64_t S, uint64_t seed,
+                          const uint32_t* __restrict__ replay, int64_t* __restrict__ sub_indptr,
+                          IdT* __restrict__ sub_indices, int64_t* __restrict__ select_index) {
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (r > S) return;
+  sub_indptr[r] = r;
+  if (r == S) return;
+  const int64_t c = static_cast<int64_t>(cols[r]);
+  const int64_t start = indptr[c];
+  const int64_t deg = indptr[c + 1] - start;
+  if (deg == 0) {
+    sub_indices[r] = static_cast<IdT>(-1);
+    select_index[r] = -1;
+  } else {
+    const uint32_t x = replay ? replay[r] : draw_one(seed, kTagUniform, static_cast<uint64_t>(r), 0);
+    const int64_t p = start + static_cast<int64_t>(x % static_cast<uint32_t>(deg));
+    sub_indices[r] = indices[p];
+    select_index[r] = p;
+  }
+}
+
+// ----------------------------------------------------------- host glue -----
+template <typename IdT>
+int slice_count_impl(const int64_t* indptr, const void* cols, int64_t S, int64_t* sub_indptr,
+                     int64_t* tile_ws, hipStream_t stream) {
+  ColDegree<IdT> f{indptr, static_cast<const IdT*>(cols)};
+  return exclusive_scan(f, S, sub_indptr, tile_ws, stream);
+}
+
+template <typename IdT>
+int slice_fill_impl(const int64_t* indptr, const void* indices, const void* cols, int64_t S,
+                    const int64_t* sub_indptr, int64_t nnz, void* sub_indices,
+                    int64_t* select_index, void* coo_col, hipStream_t stream) {
+  if (nnz == 0) return GS_OK;
+  const unsigned grid = static_cast<unsigned>((nnz + kFillTile - 1) / kFillTile);
+  if (coo_col) {
+    hipLaunchKernelGGL((slice_fill_kernel<IdT, true>), dim3(grid), dim3(kFillThreads), 0, stream,
+                       indptr, static_cast<const IdT*>(indices), static_cast<const IdT*>(cols), S,
+                       sub_indptr, nnz, static_cast<IdT*>(sub_indices), select_index,
+                       static_cast<IdT*>(coo_col));
+  } else {
+    hipLaunchKernelGGL((slice_fill_kernel<IdT, false>), dim3(grid), dim3(kFillThreads), 0, stream,
+                       indptr, static_cast<const IdT*>(indices), static_cast<const IdT*>(cols), S,
+                       sub_indptr, nnz, static_cast<IdT*>(sub_indices), select_index,
+                       static_cast<IdT*>(nullptr));
+  }
+  return check_launch("slice_fill");
+}
+
+template <typename IdT>
+int sample_count_impl(const int64_t* indptr, const void* cols, int64_t S, int64_t k, int replace,
+                      int64_t* sub_indptr, int64_t* tile_ws, hipStream_t stream) {
+  ColCount<IdT> f{indptr, static_cast<const IdT*>(cols), k, replace};
+  return exclusive_scan(f, S, sub_indptr, tile_ws, stream);
+}
+
+template <typename IdT, bool WITH_COO>
+int sample_fill_impl(const SampleArgs<IdT>& a, int replace, hipStream_t stream) {
+  if (a.S == 0) return GS_OK;
+  const unsigned grid = static_cast<unsigned>((a.S + kRowsPerBlock - 1) / kRowsPerBlock);
+  if (replace) {
+    hipLaunchKernelGGL((sample_replace_kernel<IdT, WITH_COO>), dim3(grid), dim3(kSampleThreads), 0,
+                       stream, a);
+    return check_launch("sample_replace");
+  }
+  hipLaunchKernelGGL(zero_counter_kernel, dim3(1), dim3(64), 0, stream, a.queue_count);
+  int64_t min_deg;
+  if (a.k <= kMaxLdsFanout) {
+    const size_t lds = static_cast<size_t>(kGroupsPerBlock) * a.k * sizeof(int32_t);
+    hipLaunchKernelGGL((sample_rows_kernel<IdT, WITH_COO, true>), dim3(grid), dim3(kSampleThreads),
+                       lds, stream, a);
+    min_deg = kGroupMaxDeg;
+  } else {
+    hipLaunchKernelGGL((sample_rows_kernel<IdT, WITH_COO, false>), dim3(grid),
+                       dim3(kSampleThreads), 0, stream, a);
+    min_deg = 0;
+  }
+  hipLaunchKernelGGL((sample_hub_draw_kernel<IdT>), dim3(kHubGrid), dim3(kSampleThreads), 0,
+                     stream, a);
+  hipLaunchKernelGGL((sample_hub_gather_kernel<IdT, WITH_COO>), dim3(grid), dim3(kSampleThreads),
+                     0, stream, a, min_deg);
+  return check_launch("sample_rows");
+}
+
+}  // namespace
+}  // namespace gs
+
+using namespace gs;
+
+template <typename IdT>
+static int sample_uniform_fill_t(const int64_t* indptr, const void* indices, const void* column_ids,
+                                 int64_t S, int64_t fanout, int replace, uint64_t seed,
+                                 const uint32_t* replay, const int64_t* replay_ptr,
+                                 const int64_t* sub_indptr, void* sub_indices,
+                                 int64_t* select_index, void* coo_col, long long* queue,
+                                 unsigned long long* queue_count, int64_t queue_cap,
+                                 hipStream_t st) {
+  SampleArgs<IdT> a{indptr,
+                    static_cast<const IdT*>(indices),
+                    static_cast<const IdT*>(column_ids),
+                    S,
+                    fanout,
+                    seed,
+                    replay,
+                    replay_ptr,
+                    sub_indptr,
+                    static_cast<IdT*>(sub_indices),
+                    select_index,
+                    static_cast<IdT*>(coo_col),
+                    queue,
+                    queue_count,
+                    queue_cap};
+  return coo_col ? sample_fill_impl<IdT, true>(a, replace, st)
+                 : sample_fill_impl<IdT, false>(a, replace, st);
+}
+
+extern "C" {
+
+size_t gs_slice_workspace_bytes(int64_t num_cols) { return scan_workspace_bytes(num_cols); }
+
+int gs_slice_count(const int64_t* indptr, const void* column_ids, int id_bytes, int64_t S,
+                   int64_t* sub_indptr, void* workspace, size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && S >= 0, "gs_slice_count: null pointer or negative size");
+  GS_REQUIRE(S == 0 || column_ids, "gs_slice_count: column_ids is null");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_slice_count: id_bytes must be 4 or 8, got %d", id_bytes);
+  Carver ws(workspace, workspace_bytes);
+  int64_t* tiles = ws.take<int64_t>(scan_num_tiles(S) + 1);
+  if (!ws.ok) {
+    set_error_text("gs_slice_count: workspace needs %zu bytes, 256-byte aligned",
+                   gs_slice_workspace_bytes(S));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8 ? slice_count_impl<int64_t>(indptr, column_ids, S, sub_indptr, tiles, st)
+                       : slice_count_impl<int32_t>(indptr, column_ids, S, sub_indptr, tiles, st);
+}
+
+int gs_slice_fill(const int64_t* indptr, const void* indices, const void* column_ids,
+                  int id_bytes, int64_t S, const int64_t* sub_indptr, int64_t nnz,
+                  void* sub_indices, int64_t* select_index, void* coo_col, void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && nnz >= 0, "gs_slice_fill: null pointer or negative size");
+  GS_REQUIRE(nnz == 0 || (indices && column_ids && sub_indices && select_index),
+             "gs_slice_fill: null buffer with nnz > 0");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_slice_fill: id_bytes must be 4 or 8, got %d", id_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8 ? slice_fill_impl<int64_t>(indptr, indices, column_ids, S, sub_indptr, nnz,
+                                                  sub_indices, select_index, coo_col, st)
+                       : slice_fill_impl<int32_t>(indptr, indices, column_ids, S, sub_indptr, nnz,
+                                                  sub_indices, select_index, coo_col, st);
+}
+
+size_t gs_sample_workspace_bytes(int64_t S, int64_t fanout) {
+  (void)fanout;
+  const int64_t s = S < 0 ? 0 : S;
+  return scan_workspace_bytes(s) + padded(8) + padded(static_cast<size_t>(s + kQueueExtra) * 8);
+}
+
+int gs_sample_count(const int64_t* indptr, const void* column_ids, int id_bytes, int64_t S,
+                    int64_t fanout, int replace, int64_t* sub_indptr, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0,
+             "gs_sample_count: null pointer or negative size");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sample_count: id_bytes must be 4 or 8, got %d", id_bytes);
+  Carver ws(workspace, workspace_bytes);
+  int64_t* tiles = ws.take<int64_t>(scan_num_tiles(S) + 1);
+  if (!ws.ok) {
+    set_error_text("gs_sample_count: workspace needs %zu bytes, 256-byte aligned",
+                   gs_sample_workspace_bytes(S, fanout));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8
+             ? sample_count_impl<int64_t>(indptr, column_ids, S, fanout, replace, sub_indptr, tiles, st)
+             : sample_count_impl<int32_t>(indptr, column_ids, S, fanout, replace, sub_indptr, tiles, st);
+}
+
+int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const void* column_ids,
+                           int id_bytes, int64_t S, int64_t fanout, int replace, uint64_t seed,
+                           const uint32_t* replay, const int64_t* replay_ptr,
+                           const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
+                           void* coo_col, void* workspace, size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0,
+             "gs_sample_uniform_fill: null pointer or negative size");
+  GS_REQUIRE(S == 0 || fanout == 0 || (indices && sub_indices && select_index),
+             "gs_sample_uniform_fill: null buffer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sample_uniform_fill: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  GS_REQUIRE((replay == nullptr) == (replay_ptr == nullptr),
+             "gs_sample_uniform_fill: replay and replay_ptr must be given together");
+  if (fanout == 0 || S == 0) return GS_OK;
+  // same carving as gs_sample_count, so one workspace serves both calls
+  Carver ws(workspace, workspace_bytes);
+  ws.take<int64_t>(scan_num_tiles(S) + 1);
+  unsigned long long* queue_count = ws.take<unsigned long long>(1);
+  const int64_t queue_cap = S + kQueueExtra;
+  long long* queue = ws.take<long long>(static_cast<size_t>(queue_cap));
+  if (!ws.ok) {
+    set_error_text("gs_sample_uniform_fill: workspace needs %zu bytes, 256-byte aligned",
+                   gs_sample_workspace_bytes(S, fanout));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8
+             ? sample_uniform_fill_t<int64_t>(indptr, indices, column_ids, S, fanout, replace, seed,
+                                              replay, replay_ptr, sub_indptr, sub_indices,
+                                              select_index, coo_col, queue, queue_count,
+                                              queue_cap, st)
+             : sample_uniform_fill_t<int32_t>(indptr, indices, column_ids, S, fanout, replace, seed,
+                                              replay, replay_ptr, sub_indptr, sub_indices,
+                                              select_index, coo_col, queue, queue_count,
+                                              queue_cap, st);
+}
+
+int gs_sample_one_keepdim(const int64_t* indptr, const void* indices, const void* column_ids,
+                          int id_bytes, int64_t S, uint64_t seed, const uint32_t* replay,
+                          int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
+                          void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && S >= 0, "gs_sample_one_keepdim: null pointer or negative size");
+  GS_REQUIRE(S == 0 || (indices && column_ids && sub_indices && select_index),
+             "gs_sample_one_keepdim: null buffer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sample_one_keepdim: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const unsigned grid = static_cast<unsigned>((S + 1 + 255) / 256);
+  if (id_bytes == 8) {
+    hipLaunchKernelGGL((sample_one_keepdim_kernel<int64_t>), dim3(grid), dim3(256), 0, st, indptr,
+                       static_cast<const int64_t*>(indices), static_cast<const int64_t*>(column_ids),
+                       S, seed, replay, sub_indptr, static_cast<int64_t*>(sub_indices), select_index);
+  } else {
+    hipLaunchKernelGGL((sample_one_keepdim_kernel<int32_t>), dim3(grid), dim3(256), 0, st, indptr,
+                       static_cast<const int32_t*>(indices), static_cast<const int32_t*>(column_ids),
+                       S, seed, replay, sub_indptr, static_cast<int32_t*>(sub_indices), select_index);
+  }
+  return check_launch("sample_one_keepdim");
+}
+
+}  // extern "C"

@@ -1,0 +1,282 @@
+/*
+ * gs_hip.h -- C ABI of the MI355X (gfx950) graph-sampling kernels.
+ *
+ * This is the boundary a binding of czkkkkkk/graph_sampling links against in
+ * place of its `gs::impl::*CUDA` functions (src/cuda/graph_ops.h:10-75,
+ * src/cuda/tensor_ops.h:11-105, src/cuda/sddmm.h, the headers under src/cuda/fusion).  Each
+ * entry point cites the reference routine it replaces.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer unless its name ends in `_host`.
+ *  - Buffers are caller-owned; the library never allocates device memory.
+ *    Scratch is passed as (workspace, workspace_bytes); the matching
+ *    gs_*_workspace_bytes() gives the size.  Workspace must be 256-byte aligned.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Calls
+ *    only enqueue work; they never synchronise.  Data-dependent result sizes
+ *    are left in device memory (last element of an offsets array, or a device
+ *    scalar) for the caller to read after its own synchronisation.
+ *  - Offsets (indptr, sub_indptr, select_index, e_ids) are int64.  Node ids
+ *    (indices, column ids, frontier, relabelled ids) are `id_bytes` wide: 8
+ *    (int64, the reference's only instantiation, src/cuda/slicing.cu:176) or 4
+ *    (int32 extension).
+ *  - Return value: GS_OK or a negative gs_status.  Nothing throws or aborts.
+ *
+ * Randomness.  draw(seed, tag, row, idx) =
+ *     Philox4x32-10(key = seed, ctr = (idx/4, row_lo, row_hi, tag))[idx % 4].
+ * When `replay` is non-NULL the draw is instead read from that uint32 buffer
+ * (layout documented per entry point) so that two implementations fed the same
+ * buffer return identical samples.
+ */
+#ifndef GS_HIP_H_
+#define GS_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum gs_status {
+  GS_OK = 0,
+  GS_ERR_INVALID_ARG = -1,   /* null pointer, negative size, bad id_bytes ... */
+  GS_ERR_WORKSPACE = -2,     /* workspace too small or misaligned */
+  GS_ERR_UNSUPPORTED = -3,   /* combination not implemented (message says which) */
+  GS_ERR_LAUNCH = -4         /* hipGetLastError() after a launch was not hipSuccess */
+} gs_status;
+
+/* Human-readable text for a status code; for GS_ERR_LAUNCH / GS_ERR_UNSUPPORTED
+ * the text of the most recent failure on the calling thread. */
+const char* gs_status_string(int status);
+
+/* Library version (major*10000 + minor*100 + patch). */
+int gs_version(void);
+
+typedef enum gs_op {
+  GS_OP_ADD = 0, GS_OP_SUB = 1, GS_OP_MUL = 2, GS_OP_DIV = 3,
+  GS_OP_COPY_LHS = 4, GS_OP_COPY_RHS = 5, GS_OP_DOT = 6
+} gs_op;
+
+/* ------------------------------------------------------------------------- */
+/* Column slicing: replaces impl::CSCColSlicingCUDA (src/cuda/slicing.cu:170). */
+/* ------------------------------------------------------------------------- */
+size_t gs_slice_workspace_bytes(int64_t num_cols);
+
+/* sub_indptr[0..S] = exclusive scan of deg(column_ids[r]); total in sub_indptr[S]
+ * (slicing.cu:133-147). */
+int gs_slice_count(const int64_t* indptr, const void* column_ids, int id_bytes, int64_t S,
+                   int64_t* sub_indptr, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Neighbour copy (slicing.cu:101-119).  nnz = sub_indptr[S] as read back by the
+ * caller.  coo_col may be NULL (WITH_COO = false). */
+int gs_slice_fill(const int64_t* indptr, const void* indices, const void* column_ids,
+                  int id_bytes, int64_t S, const int64_t* sub_indptr, int64_t nnz,
+                  void* sub_indices, int64_t* select_index, void* coo_col, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Uniform neighbour sampling: replaces impl::CSCColSamplingCUDA              */
+/* (src/cuda/sampling.cu:157; column_ids == NULL: every column 0..S-1 of the   */
+/* CSC) and impl::fusion::FusedCSCColSlicingSamplingCUDA                      */
+/* (src/cuda/fusion/slice_sampling.cu:146; column_ids given).                 */
+/* ------------------------------------------------------------------------- */
+size_t gs_sample_workspace_bytes(int64_t S, int64_t fanout);
+
+/* sub_indptr = exscan(cnt), cnt = replace ? (deg ? fanout : 0) : min(deg, fanout)
+ * (sampling.cu:107-119). */
+int gs_sample_count(const int64_t* indptr, const void* column_ids, int id_bytes, int64_t S,
+                    int64_t fanout, int replace, int64_t* sub_indptr, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* Fill for a sub_indptr made by gs_sample_count on the same stream.  Output
+ * buffers need capacity S*fanout (an upper bound known without reading back).
+ * Without replacement: deg <= fanout copies in order, else Algorithm R with
+ * draw index idx in [fanout, deg) (sampling.cu:44-96); output is in slot order.
+ * With replacement: slot j = draw(r, j) % deg (sampling.cu:13-41).
+ * replay / replay_ptr (both or neither): replay_ptr[S+1] offsets into replay;
+ * row r consumes max(deg-fanout, 0) draws (cnt draws with replacement).
+ * coo_col may be NULL. */
+int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const void* column_ids,
+                           int id_bytes, int64_t S, int64_t fanout, int replace, uint64_t seed,
+                           const uint32_t* replay, const int64_t* replay_ptr,
+                           const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
+                           void* coo_col, void* workspace, size_t workspace_bytes, void* stream);
+
+/* fanout == 1 with replacement through the fused entry: exactly one slot per
+ * column, -1 in both outputs for an empty column; sub_indptr = 0..S.  Replaces
+ * impl::fusion::FusedCSCColSlicingSamplingOneKeepDimCUDA
+ * (src/cuda/fusion/slice_sampling.cu:157).  replay: one draw per column. */
+int gs_sample_one_keepdim(const int64_t* indptr, const void* indices, const void* column_ids,
+                          int id_bytes, int64_t S, uint64_t seed, const uint32_t* replay,
+                          int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
+                          void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Weighted neighbour sampling without replacement (A-Res): replaces          */
+/* impl::CSCColSamplingProbsCUDA (src/cuda/sampling_probs.cu:268).  Key of     */
+/* edge i = log2(u_i)/w_i (monotone in the reference's u^(1/w)), w <= 0 ->     */
+/* -inf; the fanout largest keys are emitted in descending key order, ties by  */
+/* lower position.  probs is indexed by edge position of the input CSC.        */
+/* sub_indptr comes from gs_sample_count(replace = 0).  replay_ptr: a row with */
+/* deg > fanout consumes deg draws, any other row none.                        */
+/* ------------------------------------------------------------------------- */
+size_t gs_sample_weighted_workspace_bytes(int64_t S, int64_t fanout);
+
+int gs_sample_weighted_fill(const int64_t* indptr, const void* indices, const float* probs,
+                            const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+                            uint64_t seed, const uint32_t* replay, const int64_t* replay_ptr,
+                            const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
+                            void* coo_col, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* List sampling: replaces impl::ListSamplingCUDA (src/cuda/list_sampling.cu:79) */
+/* and impl::ListSamplingProbsCUDA (src/cuda/list_sampling_probs.cu:185).       */
+/* The caller handles n <= k without replacement (identity) itself.            */
+/* out_index[k] int64, out_data[k] id_bytes wide.                              */
+/* ------------------------------------------------------------------------- */
+size_t gs_list_sample_workspace_bytes(int64_t n, int64_t k);
+
+/* replay: k draws with replacement, n-k draws (idx = k..n-1) without. */
+int gs_list_sample_uniform(const void* data, int id_bytes, int64_t n, int64_t k, int replace,
+                           uint64_t seed, const uint32_t* replay, void* out_data,
+                           int64_t* out_index, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
+/* A-Res top-k over one list (without replacement); replay: n draws. */
+int gs_list_sample_weighted(const void* data, int id_bytes, const float* probs, int64_t n,
+                            int64_t k, uint64_t seed, const uint32_t* replay, void* out_data,
+                            int64_t* out_index, void* workspace, size_t workspace_bytes,
+                            void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Unique / relabel: replaces impl::TensorUniqueCUDA and impl::RelabelCUDA     */
+/* (src/cuda/unique_reindex.cu:174,179).                                      */
+/* ------------------------------------------------------------------------- */
+typedef struct gs_span {
+  const void* ptr; /* device pointer to ids (id_bytes wide) */
+  int64_t n;       /* number of ids */
+} gs_span;
+
+#define GS_MAX_SPANS 4
+
+size_t gs_unique_workspace_bytes(int64_t num_mapping_items);
+
+/* frontier = distinct ids of concat(mapping[0..n_mapping)) in first-occurrence
+ * order (unique_reindex.cu:106-144); *num_unique (device scalar) = its length.
+ * For every query q: query_out[q][i] = rank of query[q].ptr[i] in frontier, -1
+ * when absent (unique_reindex.cu:154-172).  n_query may be 0 (plain unique).
+ * frontier needs capacity sum(mapping[].n).  Ids must not be -1. */
+int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* query,
+                      void* const* query_out, int n_query, int id_bytes, void* frontier,
+                      int64_t* num_unique, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Random walks: replace impl::fusion::FusedRandomWalkCUDA                    */
+/* (src/cuda/fusion/random_walk.cu:52) and FusedMetapathRandomWalkCUDA         */
+/* (src/cuda/fusion/metapath_random_walk.cu:49).  trace memory is              */
+/* [length+1][n] (step-major); -1 is absorbing; one draw per live step;        */
+/* replay layout [length][n].                                                  */
+/* ------------------------------------------------------------------------- */
+int gs_random_walk(const int64_t* indptr, const void* indices, int id_bytes, const void* seeds,
+                   int64_t n, int64_t length, uint64_t seed, const uint32_t* replay,
+                   void* trace, void* stream);
+
+/* all_indptr / all_indices: device arrays of device pointers, one per relation
+ * (src/hetero_graph.cc:33-50); metapath: device int64[length] relation ids. */
+int gs_metapath_walk(const int64_t* const* all_indptr, const void* const* all_indices,
+                     int id_bytes, const int64_t* metapath, int64_t length, const void* seeds,
+                     int64_t n, uint64_t seed, const uint32_t* replay, void* trace,
+                     void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* SDDMM: replaces impl::SDDMMCOO / impl::SDDMMCSC (src/cuda/sddmm.cu:280,263). */
+/* out[eid, k] = op(lhs[sel_l, lhs_off[k]], rhs[sel_r, rhs_off[k]]) with         */
+/* sel = src(0) / edge(1) / dst(2); dot reduces `reduce_size` trailing items.   */
+/* lhs_off / rhs_off: device int64[out_len] broadcast offsets or NULL           */
+/* (src/bcast.cc:24-75).  Ids are int64 here (id_bytes reserved).               */
+/* ------------------------------------------------------------------------- */
+int gs_sddmm_coo(int op, const int64_t* row, const int64_t* col, const int64_t* e_ids, int64_t E,
+                 const float* lhs, const float* rhs, float* out, int lhs_target, int rhs_target,
+                 int64_t lhs_len, int64_t rhs_len, int64_t out_len, int64_t reduce_size,
+                 const int64_t* lhs_off, const int64_t* rhs_off, void* stream);
+
+/* CSC flavour: src = indices[e], dst = column owning e (through nid_map when
+ * given, sddmm.cu:126-131). */
+int gs_sddmm_csc(int op, const int64_t* indptr, const int64_t* indices, const int64_t* e_ids,
+                 const int64_t* nid_map, int64_t num_cols, int64_t E, const float* lhs,
+                 const float* rhs, float* out, int lhs_target, int rhs_target, int64_t lhs_len,
+                 int64_t rhs_len, int64_t out_len, int64_t reduce_size, const int64_t* lhs_off,
+                 const int64_t* rhs_off, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Segment ops: replace impl::CSCSumCUDA, COOSumCUDA, CSCNormalizeCUDA          */
+/* (src/cuda/graph_ops.cu:92,122,184) and impl::fusion::COOEDivUSum             */
+/* (src/cuda/fusion/edge_map_reduce.cu:10).                                    */
+/* ------------------------------------------------------------------------- */
+/* out[n_ids ? n_ids[s] : s] = sum over segment s of data[e_ids ? e_ids[e] : e]^powk */
+int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const int64_t* n_ids,
+                   const float* data, int64_t num_segments, int64_t powk, float* out,
+                   void* stream);
+
+/* out[target[e]] += data[e_ids ? e_ids[e] : e]^powk  (out pre-zeroed by caller) */
+int gs_coo_sum(const int64_t* target, const int64_t* e_ids, const float* data, int64_t E,
+               int64_t powk, float* out, void* stream);
+
+/* out[d] = data[d] / sum of its segment, d = e_ids ? e_ids[e] : e */
+int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const float* data,
+                         int64_t num_segments, float* out, void* stream);
+
+/* out_data[e] = data[e] / divisor[row[e]]; out_sum[col[e]] += out_data[e] */
+int gs_e_div_u_sum(const int64_t* row, const int64_t* col, const float* data,
+                   const float* divisor, int64_t E, float* out_data, float* out_sum,
+                   void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Row slicing: replaces impl::CSCRowSlicingCUDA and impl::COORowSlicingCUDA    */
+/* (src/cuda/slicing.cu:528,768).  Kept ids are relabelled to their position    */
+/* in row_ids.  Two phases: *_mark computes per-segment kept counts / a mask,   */
+/* the caller reads the total, *_compact writes the survivors in order.         */
+/* ------------------------------------------------------------------------- */
+size_t gs_row_slice_workspace_bytes(int64_t num_row_ids, int64_t nnz, int64_t num_cols);
+
+/* out_indptr[0..num_cols] = exscan of kept edges per column; total in
+ * out_indptr[num_cols]. */
+int gs_row_slice_csc_mark(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
+                          int64_t nnz, const int64_t* row_ids, int64_t num_row_ids,
+                          int64_t* out_indptr, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
+int gs_row_slice_csc_compact(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
+                             int64_t nnz, const int64_t* out_indptr, int64_t* out_indices,
+                             int64_t* select_index, int64_t* coo_col, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
+/* COO: keep edges whose key[e] is in ids.  *num_kept (device scalar). */
+int gs_row_slice_coo_mark(const int64_t* key, int64_t E, const int64_t* ids, int64_t num_ids,
+                          int64_t* num_kept, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
+int gs_row_slice_coo_compact(const int64_t* key, const int64_t* other, int64_t E,
+                             int64_t* out_key, int64_t* out_other, int64_t* select_index,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Format conversion: replaces impl::CSC2COOCUDA and impl::COO2CSCCUDA          */
+/* (src/cuda/format_transform.cu:35,135).                                      */
+/* ------------------------------------------------------------------------- */
+/* col[e] = column owning edge e */
+int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, int64_t* col, void* stream);
+
+size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys);
+
+/* Stable counting sort of (key -> value): indptr[num_keys+1], out_value[E],
+ * perm[E] (= stable argsort of key; the reference's sort_index).  sorted != 0:
+ * only indptr is computed (out_value / perm untouched, may be NULL). */
+int gs_coo2csc(const int64_t* key, const int64_t* value, int64_t E, int64_t num_keys, int sorted,
+               int64_t* indptr, int64_t* out_value, int64_t* perm, void* workspace,
+               size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GS_HIP_H_ */

@@ -1,0 +1,79 @@
+"""GPU parity: unique / relabel through the C ABI vs the CPU oracle and closed forms."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from graph_sampling_amd import capi
+from tests.util import to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _closed_form_unique(x):
+    u, first = np.unique(x, return_index=True)
+    return u[np.argsort(first, kind="stable")]
+
+
+def _run(mapping, queries, dev, idt):
+    dm = [to_dev(m, dev, idt) for m in mapping]
+    # a query that IS a mapping tensor must alias it (the slot-gather path)
+    dq = []
+    for q in queries:
+        hit = [i for i, m in enumerate(mapping) if m is q]
+        dq.append(dm[hit[0]] if hit else to_dev(q, dev, idt))
+    frontier, num, outs = capi.unique_relabel(dm, dq)
+    n = int(num.item())
+    return frontier[:n].cpu().numpy().astype(np.int64), [o.cpu().numpy().astype(np.int64) for o in outs]
+
+
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+@pytest.mark.parametrize("n", [0, 1, 5, 2048, 2049, 100000])
+def test_unique_first_occurrence(dev, idt, n):
+    rng = np.random.default_rng(n)
+    x = rng.integers(0, max(1, n // 3) + 5, size=n).astype(np.int64) * 7919 % 100003
+    frontier, _ = _run([x], [], dev, idt)
+    assert np.array_equal(frontier, _closed_form_unique(x))
+    assert np.array_equal(frontier, O.unique(x))
+
+
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+def test_relabel_seeds_first(dev, idt):
+    rng = np.random.default_rng(0)
+    seeds = rng.permutation(50000)[:1024].astype(np.int64)
+    rows = rng.integers(0, 50000, size=15000).astype(np.int64)
+    other = rng.integers(0, 60000, size=777).astype(np.int64)  # holds ids absent from the mapping
+    frontier, outs = _run([seeds, rows], [rows, other, seeds], dev, idt)
+    want_frontier, want = O.relabel([seeds, rows], [rows, other, seeds])
+    assert np.array_equal(frontier, want_frontier)
+    for g, w in zip(outs, want):
+        assert np.array_equal(g, w)
+    assert np.array_equal(frontier[:1024], seeds)          # seeds occupy the head of the frontier
+    assert np.array_equal(frontier[outs[0]], rows)         # frontier[relabelled] == original
+    assert (outs[1] == -1).any() and np.array_equal(outs[2], np.arange(1024))
+
+
+def test_relabel_reference_vector(dev):
+    # reference tests/test_relabel.cc:7-26: slicing cols 1..3 of the 20x5 graph with relabel
+    rows = np.arange(5, 20, dtype=np.int64)
+    frontier, outs = _run([rows], [rows], dev, torch.int64)
+    assert np.array_equal(frontier, rows)
+    assert np.array_equal(outs[0], np.arange(15))
+
+
+def test_unique_large_consecutive_and_clustered(dev):
+    # consecutive ids (the case that clusters under an identity hash) plus heavy duplication
+    x = np.concatenate([np.arange(300000), np.arange(300000)[::-1], np.full(1000, 42)]).astype(np.int64)
+    frontier, outs = _run([x], [x], dev, torch.int64)
+    assert np.array_equal(frontier, np.arange(300000))
+    assert np.array_equal(frontier[outs[0]], x)
+
+
+def test_four_mapping_spans(dev):
+    rng = np.random.default_rng(4)
+    spans = [rng.integers(0, 5000, size=s).astype(np.int64) for s in (10, 0, 3000, 2049)]
+    frontier, outs = _run(spans, [spans[3], spans[0]], dev, torch.int64)
+    want_frontier, want = O.relabel(spans, [spans[3], spans[0]])
+    assert np.array_equal(frontier, want_frontier)
+    for g, w in zip(outs, want):
+        assert np.array_equal(g, w)
