@@ -148,8 +148,11 @@ def slice_fill(indptr, indices, column_ids, sub_indptr, nnz, with_coo):
 
 
 # --------------------------------------------------------------- sampling ----
+ALGO_AUTO, ALGO_RESERVOIR = 0, 1
+
+
 def sample_uniform(indptr, indices, column_ids, fanout, replace, seed=0, replay=None,
-                   replay_ptr=None, with_coo=False):
+                   replay_ptr=None, with_coo=False, algo=ALGO_AUTO):
     """gs_sample_count + gs_sample_uniform_fill on upper-bound buffers.
 
     Returns (sub_indptr, sub_indices_buf, select_index_buf, coo_col_buf); the
@@ -178,7 +181,8 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace, seed=0, replay=
                                  int(bool(replace)), _ptr(sub_indptr), _ptr(ws),
                                  ctypes.c_size_t(ws.numel()), st), "gs_sample_count")
     _check(lib().gs_sample_uniform_fill(_ptr(indptr), _ptr(indices), _ptr(column_ids), idb, _i64(S),
-                                        _i64(fanout), int(bool(replace)), _u64(seed), _ptr(replay),
+                                        _i64(fanout), int(bool(replace)), int(algo), _u64(seed),
+                                        _ptr(replay),
                                         _ptr(replay_ptr), _ptr(sub_indptr), _ptr(sub_indices),
                                         _ptr(select_index), _ptr(coo_col), _ptr(ws),
                                         ctypes.c_size_t(ws.numel()), st), "gs_sample_uniform_fill")

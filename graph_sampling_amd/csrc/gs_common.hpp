@@ -201,16 +201,23 @@ constexpr int kScanTile = kScanThreads * kScanItems;
 inline int64_t scan_num_tiles(int64_t n) { return n <= 0 ? 1 : (n + kScanTile - 1) / kScanTile; }
 inline size_t scan_workspace_bytes(int64_t n) { return padded((scan_num_tiles(n) + 1) * 8); }
 
+// Evaluates f once per item (f may chase pointers), parks the value in out[i]
+// for the apply pass and reduces the tile.
 template <typename F>
 __global__ void __launch_bounds__(kScanThreads) scan_tile_sums_kernel(F f, int64_t n,
-                                                                      int64_t* tile_sums) {
+                                                                      int64_t* tile_sums,
+                                                                      int64_t* out) {
   __shared__ int64_t lds[kScanThreads / kWave + 1];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kScanTile;
   int64_t acc = 0;
 #pragma unroll
   for (int k = 0; k < kScanItems; ++k) {
     int64_t i = base + k * kScanThreads + threadIdx.x;
-    if (i < n) acc += f(i);
+    if (i < n) {
+      const int64_t v = f(i);
+      out[i] = v;
+      acc += v;
+    }
   }
   int64_t total;
   block_exclusive_scan<kScanThreads>(acc, &total, lds);
@@ -234,12 +241,26 @@ static __global__ void __launch_bounds__(kScanThreads) scan_tile_offsets_kernel(
 }
 
 // Thread t of the block owns items base + t*kScanItems .. +kScanItems-1 so the
-// per-thread prefix is a running sum (blocked arrangement).
-template <typename F>
+// per-thread prefix is a running sum (blocked arrangement).  With `tiles` the
+// item values are read back from out[] (parked there by scan_tile_sums_kernel),
+// without it f is evaluated here.  SELF_PREFIX: `tiles` holds raw tile sums and
+// the block adds up its predecessors itself, which saves the separate one-block
+// offsets kernel when there are few tiles.
+template <typename F, bool SELF_PREFIX>
 __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(F f, int64_t n,
-                                                                  const int64_t* tile_offsets,
+                                                                  const int64_t* tiles,
                                                                   int64_t* out) {
   __shared__ int64_t lds[kScanThreads / kWave + 1];
+  int64_t tile_base = 0;
+  if (tiles) {
+    if (SELF_PREFIX) {
+      int64_t part = 0;
+      for (int64_t t = threadIdx.x; t < blockIdx.x; t += kScanThreads) part += tiles[t];
+      block_exclusive_scan<kScanThreads>(part, &tile_base, lds);
+    } else {
+      tile_base = tiles[blockIdx.x];
+    }
+  }
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kScanTile +
                        static_cast<int64_t>(threadIdx.x) * kScanItems;
   int64_t v[kScanItems];
@@ -247,12 +268,12 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(F f, int64_t n
 #pragma unroll
   for (int k = 0; k < kScanItems; ++k) {
     int64_t i = base + k;
-    v[k] = i < n ? f(i) : 0;
+    v[k] = i < n ? (tiles ? out[i] : f(i)) : 0;
     acc += v[k];
   }
   int64_t total;
   int64_t ex = block_exclusive_scan<kScanThreads>(acc, &total, lds);
-  int64_t run = ex + (tile_offsets ? tile_offsets[blockIdx.x] : 0);
+  int64_t run = ex + tile_base;
 #pragma unroll
   for (int k = 0; k < kScanItems; ++k) {
     int64_t i = base + k;
@@ -263,22 +284,30 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(F f, int64_t n
   if (n == 0 && blockIdx.x == 0 && threadIdx.x == 0) out[0] = 0;
 }
 
+constexpr int64_t kScanSelfPrefixTiles = 4096;
+
 // Enqueues the scan.  tile_ws: scan_workspace_bytes(n) bytes.
 template <typename F>
 inline int exclusive_scan(F f, int64_t n, int64_t* out, int64_t* tile_ws, hipStream_t stream) {
   const int64_t tiles = scan_num_tiles(n);
   if (tiles == 1) {
-    hipLaunchKernelGGL(scan_apply_kernel<F>, dim3(1), dim3(kScanThreads), 0, stream, f, n,
+    hipLaunchKernelGGL((scan_apply_kernel<F, false>), dim3(1), dim3(kScanThreads), 0, stream, f, n,
                        static_cast<const int64_t*>(nullptr), out);
     return check_launch("scan_apply");
   }
   hipLaunchKernelGGL(scan_tile_sums_kernel<F>, dim3(static_cast<unsigned>(tiles)),
-                     dim3(kScanThreads), 0, stream, f, n, tile_ws);
+                     dim3(kScanThreads), 0, stream, f, n, tile_ws, out);
+  if (tiles <= kScanSelfPrefixTiles) {
+    hipLaunchKernelGGL((scan_apply_kernel<F, true>), dim3(static_cast<unsigned>(tiles)),
+                       dim3(kScanThreads), 0, stream, f, n, static_cast<const int64_t*>(tile_ws),
+                       out);
+    return check_launch("scan");
+  }
   hipLaunchKernelGGL(scan_tile_offsets_kernel, dim3(1), dim3(kScanThreads), 0, stream, tile_ws,
                      tiles);
-  hipLaunchKernelGGL(scan_apply_kernel<F>, dim3(static_cast<unsigned>(tiles)),
-                     dim3(kScanThreads), 0, stream, f, n,
-                     static_cast<const int64_t*>(tile_ws), out);
+  hipLaunchKernelGGL((scan_apply_kernel<F, false>), dim3(static_cast<unsigned>(tiles)),
+                     dim3(kScanThreads), 0, stream, f, n, static_cast<const int64_t*>(tile_ws),
+                     out);
   return check_launch("scan");
 }
 

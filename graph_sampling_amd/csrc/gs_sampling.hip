@@ -12,11 +12,15 @@
 //    positions and finds their rows by binary search in an LDS copy of the
 //    offsets, so a power-law hub row is spread over many workgroups and all
 //    stores are fully coalesced;
-//  * sampling: rows are binned by degree.  deg <= k copies; k < deg <= 1024 runs
-//    Algorithm R inside a 16-lane group with the k slots in LDS (ds_max); larger
-//    rows keep their slots in the output buffer and are cut into 4096-draw
-//    chunks; the chunks go through a device queue so that a second kernel
-//    spreads them evenly over the chip, and a last pass gathers the ids.
+//  * sampling, default algorithm (GS_SAMPLE_AUTO): Floyd's k-subset selection,
+//    k draws per row however large the row is, 8/16/32/64 lanes per row with the
+//    draws in parallel and the duplicate check as a cross-lane broadcast chain;
+//  * sampling, GS_SAMPLE_RESERVOIR (the reference's Algorithm R, deg-k draws
+//    per row): rows are binned by degree.  k < deg <= 1024 runs inside a 16-lane
+//    group with the k slots in LDS (ds_max); larger rows keep their slots in
+//    the output buffer and are cut into 4096-draw chunks; the chunks go through
+//    a device queue so that a second kernel spreads them evenly over the chip,
+//    and a last pass gathers the ids.
 #include "gs_common.hpp"
 
 namespace gs {
@@ -309,6 +313,55 @@ sample_hub_gather_kernel(SampleArgs<IdT> a, int64_t min_deg) {
   }
 }
 
+
+// ------------------------------------------------------- Floyd selection ----
+// G lanes (8/16/32/64, >= k) per row.  Lane i owns step i of Floyd's algorithm
+// (Bentley & Floyd, CACM 30(9), 1987): j_i = deg-k+i, t_i = draw(r,i) % (j_i+1),
+// and the chosen position is t_i unless an earlier step already chose it, in
+// which case it is j_i.  All draws and moduli run in parallel; only the k-step
+// "already chosen?" chain is sequential, and it is one cross-lane broadcast
+// per step (lane m's choice is final once steps 0..m-1 have been broadcast).
+// Lane i then writes output i, so a row's outputs are one contiguous run.
+constexpr int kFloydThreads = 256;
+constexpr int64_t kFloydMaxK = GS_FLOYD_MAX_FANOUT;
+
+template <typename IdT, bool WITH_COO, int G>
+__global__ void __launch_bounds__(kFloydThreads) sample_floyd_kernel(SampleArgs<IdT> a) {
+  const int lane = threadIdx.x % G;
+  const int64_t r = (static_cast<int64_t>(blockIdx.x) * kFloydThreads + threadIdx.x) / G;
+  if (r >= a.S) return;
+  const int k = static_cast<int>(a.k);
+  int64_t start, deg, out_start;
+  load_row(a, r, &start, &deg, &out_start);
+  if (deg <= k) {
+    if (lane < deg) {
+      a.sub_indices[out_start + lane] = a.indices[start + lane];
+      a.select_index[out_start + lane] = start + lane;
+      if (WITH_COO) a.coo_col[out_start + lane] = static_cast<IdT>(r);
+    }
+    return;
+  }
+  uint32_t t = 0, j = 0;
+  if (lane < k) {
+    const uint32_t xv = a.replay ? a.replay[a.replay_ptr[r] + lane]
+                                 : draw_one(a.seed, kTagUniform, static_cast<uint64_t>(r),
+                                            static_cast<uint64_t>(lane));
+    j = static_cast<uint32_t>(deg - k + lane);
+    t = xv % (j + 1u);
+  }
+  bool taken = false;
+  for (int m = 0; m < k - 1; ++m) {
+    const uint32_t chosen_m = __shfl(taken ? j : t, m, G);
+    if (lane > m && t == chosen_m) taken = true;
+  }
+  if (lane < k) {
+    const int64_t q = start + (taken ? j : t);
+    a.sub_indices[out_start + lane] = a.indices[q];
+    a.select_index[out_start + lane] = q;
+    if (WITH_COO) a.coo_col[out_start + lane] = static_cast<IdT>(r);
+  }
+}
+
 // With replacement: slot j of row r = draw(r, j) % deg (sampling.cu:29-39).
 template <typename IdT, bool WITH_COO>
 __global__ void __launch_bounds__(kSampleThreads) sample_replace_kernel(SampleArgs<IdT> a) {
@@ -400,13 +453,31 @@ int sample_count_impl(const int64_t* indptr, const void* cols, int64_t S, int64_
 }
 
 template <typename IdT, bool WITH_COO>
-int sample_fill_impl(const SampleArgs<IdT>& a, int replace, hipStream_t stream) {
+int sample_fill_impl(const SampleArgs<IdT>& a, int replace, int algo, hipStream_t stream) {
   if (a.S == 0) return GS_OK;
   const unsigned grid = static_cast<unsigned>((a.S + kRowsPerBlock - 1) / kRowsPerBlock);
   if (replace) {
     hipLaunchKernelGGL((sample_replace_kernel<IdT, WITH_COO>), dim3(grid), dim3(kSampleThreads), 0,
                        stream, a);
     return check_launch("sample_replace");
+  }
+  if (algo == GS_SAMPLE_AUTO && a.k <= kFloydMaxK) {
+    const int g = a.k <= 8 ? 8 : (a.k <= 16 ? 16 : (a.k <= 32 ? 32 : 64));
+    const unsigned fgrid =
+        static_cast<unsigned>((a.S * g + kFloydThreads - 1) / kFloydThreads);
+    if (g == 8)
+      hipLaunchKernelGGL((sample_floyd_kernel<IdT, WITH_COO, 8>), dim3(fgrid), dim3(kFloydThreads),
+                         0, stream, a);
+    else if (g == 16)
+      hipLaunchKernelGGL((sample_floyd_kernel<IdT, WITH_COO, 16>), dim3(fgrid), dim3(kFloydThreads),
+                         0, stream, a);
+    else if (g == 32)
+      hipLaunchKernelGGL((sample_floyd_kernel<IdT, WITH_COO, 32>), dim3(fgrid), dim3(kFloydThreads),
+                         0, stream, a);
+    else
+      hipLaunchKernelGGL((sample_floyd_kernel<IdT, WITH_COO, 64>), dim3(fgrid), dim3(kFloydThreads),
+                         0, stream, a);
+    return check_launch("sample_floyd");
   }
   hipLaunchKernelGGL(zero_counter_kernel, dim3(1), dim3(64), 0, stream, a.queue_count);
   int64_t min_deg;
@@ -438,7 +509,7 @@ static int sample_uniform_fill_t(const int64_t* indptr, const void* indices, con
                                  const uint32_t* replay, const int64_t* replay_ptr,
                                  const int64_t* sub_indptr, void* sub_indices,
                                  int64_t* select_index, void* coo_col, long long* queue,
-                                 unsigned long long* queue_count, int64_t queue_cap,
+                                 unsigned long long* queue_count, int64_t queue_cap, int algo,
                                  hipStream_t st) {
   SampleArgs<IdT> a{indptr,
                     static_cast<const IdT*>(indices),
@@ -455,8 +526,8 @@ static int sample_uniform_fill_t(const int64_t* indptr, const void* indices, con
                     queue,
                     queue_count,
                     queue_cap};
-  return coo_col ? sample_fill_impl<IdT, true>(a, replace, st)
-                 : sample_fill_impl<IdT, false>(a, replace, st);
+  return coo_col ? sample_fill_impl<IdT, true>(a, replace, algo, st)
+                 : sample_fill_impl<IdT, false>(a, replace, algo, st);
 }
 
 extern "C" {
@@ -520,7 +591,8 @@ int gs_sample_count(const int64_t* indptr, const void* column_ids, int id_bytes,
 }
 
 int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const void* column_ids,
-                           int id_bytes, int64_t S, int64_t fanout, int replace, uint64_t seed,
+                           int id_bytes, int64_t S, int64_t fanout, int replace, int algo,
+                           uint64_t seed,
                            const uint32_t* replay, const int64_t* replay_ptr,
                            const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                            void* coo_col, void* workspace, size_t workspace_bytes, void* stream) {
@@ -532,6 +604,8 @@ int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const voi
              id_bytes);
   GS_REQUIRE((replay == nullptr) == (replay_ptr == nullptr),
              "gs_sample_uniform_fill: replay and replay_ptr must be given together");
+  GS_REQUIRE(algo == GS_SAMPLE_AUTO || algo == GS_SAMPLE_RESERVOIR,
+             "gs_sample_uniform_fill: unknown algo %d", algo);
   if (fanout == 0 || S == 0) return GS_OK;
   // same carving as gs_sample_count, so one workspace serves both calls
   Carver ws(workspace, workspace_bytes);
@@ -549,11 +623,11 @@ int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const voi
              ? sample_uniform_fill_t<int64_t>(indptr, indices, column_ids, S, fanout, replace, seed,
                                               replay, replay_ptr, sub_indptr, sub_indices,
                                               select_index, coo_col, queue, queue_count,
-                                              queue_cap, st)
+                                              queue_cap, algo, st)
              : sample_uniform_fill_t<int32_t>(indptr, indices, column_ids, S, fanout, replace, seed,
                                               replay, replay_ptr, sub_indptr, sub_indices,
                                               select_index, coo_col, queue, queue_count,
-                                              queue_cap, st);
+                                              queue_cap, algo, st);
 }
 
 int gs_sample_one_keepdim(const int64_t* indptr, const void* indices, const void* column_ids,

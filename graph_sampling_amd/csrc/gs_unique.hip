@@ -8,12 +8,19 @@
 //  * capacity = power of two >= 2 * items (load <= 0.5; the reference runs at
 //    0.5..1.0, unique_reindex.cu:74-78), Fibonacci hashing, linear probing
 //    (the reference uses the identity hash, which clusters on consecutive ids);
-//  * values are int32 and every item remembers its slot (4 B) so later passes
-//    never probe again;
+//  * 32-bit ids use ONE 64-bit word per slot, (key << 32 | first index): an
+//    insert is a single compare-and-swap in the common case, and a duplicate
+//    lowers the index with a single atomicMin on the same word.  Device-scope
+//    atomics are resolved memory-side on a multi-XCD part, so the number of
+//    atomics per item, not bytes, is what this kernel is made of.  64-bit ids
+//    keep separate key (int64) and index (int32) arrays;
+//  * every item remembers its slot (4 B) so later passes never probe again;
 //  * the mapping tensors are read in place through a span table -- no
 //    concatenated copy is materialised (the reference does torch::cat,
 //    unique_reindex.cu:187-190);
-//  * a query that aliases a mapping span is relabelled by slot gather.
+//  * the rank of a key is prefix[first index], so compaction and every relabel
+//    lookup run in one final kernel; a query that aliases a mapping span is
+//    relabelled by slot gather instead of probing.
 #include "gs_common.hpp"
 
 namespace gs {
@@ -40,101 +47,170 @@ struct Spans {
   }
 };
 
-struct Table {
-  long long* keys;  // -1 = empty
-  int* vals;        // min index, later the rank
+__device__ __forceinline__ uint32_t fib_home(uint64_t key, int shift) {
+  return static_cast<uint32_t>((key * 0x9E3779B97F4A7C15ull) >> shift);
+}
+
+// ---- slot layout for 32-bit ids: (key << 32 | first index), all ones = empty
+struct PackedTable {
+  unsigned long long* slots;
   uint32_t mask;
-  int shift;  // 64 - log2(capacity)
-  __device__ __forceinline__ uint32_t home(long long key) const {
-    return static_cast<uint32_t>((static_cast<uint64_t>(key) * 0x9E3779B97F4A7C15ull) >> shift);
+  int shift;
+  static size_t bytes(int64_t cap) { return padded(cap * 8); }
+  void carve(Carver& ws, int64_t cap) { slots = ws.take<unsigned long long>(cap); }
+  __device__ __forceinline__ void clear(int64_t i) const { slots[i] = ~0ull; }
+  // returns the slot of `key` after recording index i as a candidate first occurrence
+  __device__ __forceinline__ uint32_t insert(long long key, uint32_t i) const {
+    const unsigned long long hi = static_cast<unsigned long long>(static_cast<uint32_t>(key)) << 32;
+    const unsigned long long word = hi | i;
+    uint32_t p = fib_home(static_cast<uint32_t>(key), shift);
+    while (true) {
+      const unsigned long long prev = atomicCAS(&slots[p], ~0ull, word);
+      if (prev == ~0ull) break;
+      if ((prev >> 32) == (hi >> 32)) {
+        if (static_cast<uint32_t>(prev) > i) atomicMin(&slots[p], word);
+        break;
+      }
+      p = (p + 1) & mask;
+    }
+    return p;
+  }
+  __device__ __forceinline__ uint32_t first_index(uint32_t p) const {
+    return static_cast<uint32_t>(slots[p]);
+  }
+  // first index of `key`, or -1 when absent (unique_reindex.cu:44-58)
+  __device__ __forceinline__ int64_t find(long long key) const {
+    const unsigned long long k32 = static_cast<uint32_t>(key);
+    uint32_t p = fib_home(static_cast<uint32_t>(key), shift);
+    while (true) {
+      const unsigned long long s = slots[p];
+      if (s == ~0ull) return -1;
+      if ((s >> 32) == k32) return static_cast<uint32_t>(s);
+      p = (p + 1) & mask;
+    }
   }
 };
 
-__global__ void __launch_bounds__(kThreads) table_init_kernel(Table t, int64_t cap) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (i < cap) {
-    t.keys[i] = -1;
-    t.vals[i] = 0x7fffffff;
+// ---- slot layout for 64-bit ids: key array (-1 = empty) + first-index array
+struct WideTable {
+  long long* keys;
+  int* vals;
+  uint32_t mask;
+  int shift;
+  static size_t bytes(int64_t cap) { return padded(cap * 8) + padded(cap * 4); }
+  void carve(Carver& ws, int64_t cap) {
+    keys = ws.take<long long>(cap);
+    vals = ws.take<int>(cap);
   }
+  __device__ __forceinline__ void clear(int64_t i) const {
+    keys[i] = -1;
+    vals[i] = 0x7fffffff;
+  }
+  // (unique_reindex.cu:13-26 RelabelHashmap::Update)
+  __device__ __forceinline__ uint32_t insert(long long key, uint32_t i) const {
+    uint32_t p = fib_home(static_cast<uint64_t>(key), shift);
+    while (true) {
+      const unsigned long long prev =
+          atomicCAS(reinterpret_cast<unsigned long long*>(&keys[p]), ~0ull,
+                    static_cast<unsigned long long>(key));
+      if (prev == ~0ull || prev == static_cast<unsigned long long>(key)) break;
+      p = (p + 1) & mask;
+    }
+    // values only decrease, so a (possibly stale) read <= i proves the atomic unnecessary
+    if (__atomic_load_n(&vals[p], __ATOMIC_RELAXED) > static_cast<int>(i))
+      atomicMin(&vals[p], static_cast<int>(i));
+    return p;
+  }
+  __device__ __forceinline__ uint32_t first_index(uint32_t p) const {
+    return static_cast<uint32_t>(vals[p]);
+  }
+  __device__ __forceinline__ int64_t find(long long key) const {
+    uint32_t p = fib_home(static_cast<uint64_t>(key), shift);
+    while (true) {
+      const long long cur = keys[p];
+      if (cur == key) return vals[p];
+      if (cur == -1) return -1;
+      p = (p + 1) & mask;
+    }
+  }
+};
+
+template <typename IdT>
+struct TableFor {
+  using type = WideTable;
+};
+template <>
+struct TableFor<int32_t> {
+  using type = PackedTable;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads) table_init_kernel(T t, int64_t cap) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < cap) t.clear(i);
 }
 
 // insert (key -> min index) and remember the slot of every item
-// (unique_reindex.cu:92-99, RelabelHashmap::Update :13-26)
-template <typename IdT>
+// (unique_reindex.cu:92-99)
+template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
-table_insert_kernel(Spans<IdT> x, int64_t M, Table t, int* __restrict__ pos) {
+table_insert_kernel(Spans<IdT> x, int64_t M, T t, uint32_t* __restrict__ pos) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= M) return;
-  const long long key = static_cast<long long>(x.get(i));
-  uint32_t p = t.home(key);
-  while (true) {
-    long long cur = __atomic_load_n(&t.keys[p], __ATOMIC_RELAXED);
-    if (cur == key) break;
-    if (cur == -1) {
-      unsigned long long prev =
-          atomicCAS(reinterpret_cast<unsigned long long*>(&t.keys[p]), ~0ull,
-                    static_cast<unsigned long long>(key));
-      if (prev == ~0ull || prev == static_cast<unsigned long long>(key)) break;
-    }
-    p = (p + 1) & t.mask;
-  }
-  atomicMin(&t.vals[p], static_cast<int>(i));
-  pos[i] = static_cast<int>(p);
+  pos[i] = t.insert(static_cast<long long>(x.get(i)), static_cast<uint32_t>(i));
 }
 
 // 1 when item i is the first occurrence of its key (unique_reindex.cu:106-114)
+template <typename T>
 struct IsFirst {
-  const int* vals;
-  const int* pos;
+  T t;
+  const uint32_t* pos;
   __device__ __forceinline__ int64_t operator()(int64_t i) const {
-    return vals[pos[i]] == static_cast<int>(i) ? 1 : 0;
+    return t.first_index(pos[i]) == static_cast<uint32_t>(i) ? 1 : 0;
   }
 };
 
-// frontier[rank] = key and slot value <- rank (unique_reindex.cu:127-144).  A
-// first occurrence i has rank <= i, every later duplicate has index > i, so
-// overwriting the slot while others still test `vals == my index` is safe.
-template <typename IdT>
+struct Query {
+  const void* in[GS_MAX_SPANS];
+  void* out[GS_MAX_SPANS];
+  int64_t end[GS_MAX_SPANS];    // exclusive end offset in the concatenation of queries
+  int64_t alias[GS_MAX_SPANS];  // >= 0: the query is the mapping span starting there
+  int n;
+};
+
+// Items [0, M): frontier[rank] = key for first occurrences
+// (unique_reindex.cu:127-144).  Items [M, M+Q): relabel lookups
+// (unique_reindex.cu:162-170), rank of a key = prefix[its first index].
+template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
-compact_kernel(Spans<IdT> x, int64_t M, Table t, const int* __restrict__ pos,
-               const int64_t* __restrict__ prefix, IdT* __restrict__ frontier,
-               int64_t* __restrict__ num_unique) {
+finish_kernel(Spans<IdT> x, int64_t M, T t, const uint32_t* __restrict__ pos,
+              const int64_t* __restrict__ prefix, IdT* __restrict__ frontier,
+              int64_t* __restrict__ num_unique, Query qs, int64_t Q) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i == 0) *num_unique = prefix[M];
-  if (i >= M) return;
-  const int p = pos[i];
-  if (t.vals[p] == static_cast<int>(i)) {
-    const int64_t rank = prefix[i];
-    frontier[rank] = x.get(i);
-    t.vals[p] = static_cast<int>(rank);
-  }
-}
-
-// out[i] = rank of q[i] (unique_reindex.cu:162-170); alias >= 0: q is the
-// mapping span starting at concatenation offset `alias`, so reuse its slots.
-template <typename IdT>
-__global__ void __launch_bounds__(kThreads)
-lookup_kernel(const IdT* __restrict__ q, int64_t n, Table t, const int* __restrict__ pos,
-              int64_t alias, IdT* __restrict__ out) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (i >= n) return;
-  if (alias >= 0) {
-    out[i] = static_cast<IdT>(t.vals[pos[alias + i]]);
+  if (i < M) {
+    if (t.first_index(pos[i]) == static_cast<uint32_t>(i)) frontier[prefix[i]] = x.get(i);
     return;
   }
-  const long long key = static_cast<long long>(q[i]);
-  uint32_t p = t.home(key);
-  int r = -1;
-  while (true) {
-    const long long cur = t.keys[p];
-    if (cur == key) {
-      r = t.vals[p];
-      break;
+  const int64_t j = i - M;
+  if (j >= Q) return;
+  int s = 0;
+  int64_t begin = 0;
+#pragma unroll
+  for (int u = 0; u < GS_MAX_SPANS - 1; ++u) {
+    if (u < qs.n - 1 && j >= qs.end[u]) {
+      s = u + 1;
+      begin = qs.end[u];
     }
-    if (cur == -1) break;
-    p = (p + 1) & t.mask;
   }
-  out[i] = static_cast<IdT>(r);
+  const int64_t local = j - begin;
+  int64_t first;
+  if (qs.alias[s] >= 0) {
+    first = t.first_index(pos[qs.alias[s] + local]);
+  } else {
+    first = t.find(static_cast<long long>(static_cast<const IdT*>(qs.in[s])[local]));
+  }
+  static_cast<IdT*>(qs.out[s])[local] = static_cast<IdT>(first < 0 ? -1 : prefix[first]);
 }
 
 int64_t table_capacity(int64_t M) {
@@ -144,9 +220,18 @@ int64_t table_capacity(int64_t M) {
 }
 
 template <typename IdT>
+size_t workspace_bytes_for(int64_t M) {
+  using T = typename TableFor<IdT>::type;
+  const int64_t cap = table_capacity(M);
+  return T::bytes(cap) + padded((M > 0 ? M : 1) * 4) + padded((M + 1) * 8) +
+         scan_workspace_bytes(M);
+}
+
+template <typename IdT>
 int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* query,
                         void* const* query_out, int n_query, void* frontier, int64_t* num_unique,
                         void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  using T = typename TableFor<IdT>::type;
   Spans<IdT> x;
   int64_t M = 0;
   for (int s = 0; s < GS_MAX_SPANS; ++s) {
@@ -161,15 +246,14 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   x.n = n_mapping;
   const int64_t cap = table_capacity(M);
   Carver ws(workspace, workspace_bytes);
-  Table t;
-  t.keys = ws.take<long long>(cap);
-  t.vals = ws.take<int>(cap);
-  int* pos = ws.take<int>(M > 0 ? M : 1);
+  T t;
+  t.carve(ws, cap);
+  uint32_t* pos = ws.take<uint32_t>(M > 0 ? M : 1);
   int64_t* prefix = ws.take<int64_t>(M + 1);
   int64_t* tiles = ws.take<int64_t>(scan_num_tiles(M) + 1);
   if (!ws.ok) {
     set_error_text("gs_unique_relabel: workspace needs %zu bytes, 256-byte aligned",
-                   gs_unique_workspace_bytes(M));
+                   workspace_bytes_for<IdT>(M));
     return GS_ERR_WORKSPACE;
   }
   t.mask = static_cast<uint32_t>(cap - 1);
@@ -177,27 +261,37 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   while ((int64_t(1) << lg) < cap) ++lg;
   t.shift = 64 - lg;
 
-  hipLaunchKernelGGL(table_init_kernel, dim3(blocks_for(cap, kThreads)), dim3(kThreads), 0, stream,
-                     t, cap);
-  if (M > 0)
-    hipLaunchKernelGGL((table_insert_kernel<IdT>), dim3(blocks_for(M, kThreads)), dim3(kThreads), 0,
-                       stream, x, M, t, pos);
-  GS_RETURN_IF_ERROR(check_launch("unique insert"));
-  IsFirst f{t.vals, pos};
-  GS_RETURN_IF_ERROR(exclusive_scan(f, M, prefix, tiles, stream));
-  hipLaunchKernelGGL((compact_kernel<IdT>), dim3(blocks_for(M, kThreads)), dim3(kThreads), 0, stream,
-                     x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique);
+  Query qs;
+  int64_t Q = 0;
+  for (int q = 0; q < GS_MAX_SPANS; ++q) {
+    qs.in[q] = nullptr;
+    qs.out[q] = nullptr;
+    qs.end[q] = 0;
+    qs.alias[q] = -1;
+  }
   for (int q = 0; q < n_query; ++q) {
-    if (query[q].n == 0) continue;
-    int64_t alias = -1, off = 0;
+    qs.in[q] = query[q].ptr;
+    qs.out[q] = query_out[q];
+    Q += query[q].n;
+    qs.end[q] = Q;
+    int64_t off = 0;
     for (int s = 0; s < n_mapping; ++s) {
-      if (mapping[s].ptr == query[q].ptr && mapping[s].n == query[q].n) alias = off;
+      if (mapping[s].ptr == query[q].ptr && mapping[s].n == query[q].n) qs.alias[q] = off;
       off += mapping[s].n;
     }
-    hipLaunchKernelGGL((lookup_kernel<IdT>), dim3(blocks_for(query[q].n, kThreads)), dim3(kThreads),
-                       0, stream, static_cast<const IdT*>(query[q].ptr), query[q].n, t, pos, alias,
-                       static_cast<IdT*>(query_out[q]));
   }
+  qs.n = n_query;
+
+  hipLaunchKernelGGL((table_init_kernel<T>), dim3(blocks_for(cap, kThreads)), dim3(kThreads), 0,
+                     stream, t, cap);
+  if (M > 0)
+    hipLaunchKernelGGL((table_insert_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
+                       0, stream, x, M, t, pos);
+  GS_RETURN_IF_ERROR(check_launch("unique insert"));
+  IsFirst<T> f{t, pos};
+  GS_RETURN_IF_ERROR(exclusive_scan(f, M, prefix, tiles, stream));
+  hipLaunchKernelGGL((finish_kernel<IdT, T>), dim3(blocks_for(M + Q, kThreads)), dim3(kThreads), 0,
+                     stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, qs, Q);
   return check_launch("unique_relabel");
 }
 
@@ -210,9 +304,9 @@ extern "C" {
 
 size_t gs_unique_workspace_bytes(int64_t M) {
   if (M < 0) M = 0;
-  const int64_t cap = table_capacity(M);
-  return padded(cap * 8) + padded(cap * 4) + padded((M > 0 ? M : 1) * 4) + padded((M + 1) * 8) +
-         scan_workspace_bytes(M);
+  const size_t a = workspace_bytes_for<int64_t>(M);
+  const size_t b = workspace_bytes_for<int32_t>(M);
+  return a > b ? a : b;
 }
 
 int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* query,

@@ -81,6 +81,18 @@ int gs_slice_fill(const int64_t* indptr, const void* indices, const void* column
 /* ------------------------------------------------------------------------- */
 size_t gs_sample_workspace_bytes(int64_t S, int64_t fanout);
 
+/* Selection algorithm for uniform sampling WITHOUT replacement on rows with
+ * deg > fanout.  Both give a uniformly distributed fanout-subset.
+ *  GS_SAMPLE_RESERVOIR  the reference's Algorithm R (sampling.cu:70-92): slot j
+ *      starts as j; for idx in [fanout, deg): num = draw(r, idx) % (idx+1), if
+ *      num < fanout then slot[num] = max(slot[num], idx).  deg-fanout draws.
+ *  GS_SAMPLE_AUTO       Floyd's selection when fanout <= GS_FLOYD_MAX_FANOUT
+ *      (else Algorithm R): for step i in [0, fanout), j = deg-fanout+i,
+ *      t = draw(r, i) % (j+1); position t is taken unless already taken, in
+ *      which case j is.  fanout draws whatever the degree; output in step order. */
+typedef enum gs_sample_algo { GS_SAMPLE_AUTO = 0, GS_SAMPLE_RESERVOIR = 1 } gs_sample_algo;
+#define GS_FLOYD_MAX_FANOUT 64
+
 /* sub_indptr = exscan(cnt), cnt = replace ? (deg ? fanout : 0) : min(deg, fanout)
  * (sampling.cu:107-119). */
 int gs_sample_count(const int64_t* indptr, const void* column_ids, int id_bytes, int64_t S,
@@ -89,14 +101,16 @@ int gs_sample_count(const int64_t* indptr, const void* column_ids, int id_bytes,
 
 /* Fill for a sub_indptr made by gs_sample_count on the same stream.  Output
  * buffers need capacity S*fanout (an upper bound known without reading back).
- * Without replacement: deg <= fanout copies in order, else Algorithm R with
- * draw index idx in [fanout, deg) (sampling.cu:44-96); output is in slot order.
+ * Without replacement: deg <= fanout copies in order (sampling.cu:60-69), else
+ * the algorithm `algo` selects; output is in slot / step order (unsorted).
  * With replacement: slot j = draw(r, j) % deg (sampling.cu:13-41).
  * replay / replay_ptr (both or neither): replay_ptr[S+1] offsets into replay;
- * row r consumes max(deg-fanout, 0) draws (cnt draws with replacement).
- * coo_col may be NULL. */
+ * a row with deg > fanout consumes deg-fanout draws (Algorithm R) or fanout
+ * draws (Floyd), other rows none; with replacement every row consumes its
+ * output count.  coo_col may be NULL. */
 int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const void* column_ids,
-                           int id_bytes, int64_t S, int64_t fanout, int replace, uint64_t seed,
+                           int id_bytes, int64_t S, int64_t fanout, int replace, int algo,
+                           uint64_t seed,
                            const uint32_t* replay, const int64_t* replay_ptr,
                            const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                            void* coo_col, void* workspace, size_t workspace_bytes, void* stream);

@@ -15,7 +15,9 @@
  * on the CUDA launch geometry (src/cuda/sampling.cu:51); no test of the
  * reference checks a sampled value, so those streams are "parity unpinned".
  * This restatement keeps the reference *algorithms* (Algorithm R reservoir,
- * A-Res top-k, modulo pick) and defines the draw as a pure function
+ * A-Res top-k, modulo pick) -- plus, as a second selectable algorithm for
+ * uniform sampling without replacement, Floyd's k-subset selection (see
+ * gso_sample_uniform_fill) -- and defines the draw as a pure function
  *     draw(seed, tag, row, idx) = Philox4x32-10(key=seed, ctr=(idx/4,row,tag))[idx%4]
  * or, in replay mode, a lookup in a caller-supplied uint32 buffer.  Philox is
  * pinned by the Random123 known-answer vectors (tests/test_oracle_pins.py).
@@ -158,10 +160,24 @@ void gso_slice_fill(const i64* indptr, const i64* indices, const i64* cols, i64 
 /* ------------------------------------------------------------------------ */
 static inline i64 col_of(const i64* cols, i64 r) { return cols ? cols[r] : r; }
 
+/* Selection algorithm for uniform sampling without replacement.
+ * GSO_ALGO_RESERVOIR: Algorithm R on every row with deg > k, exactly the
+ *   reference (sampling.cu:70-92); a row consumes deg-k draws.
+ * GSO_ALGO_AUTO: rows with deg > k use Floyd's algorithm (Bentley & Floyd,
+ *   CACM 30(9) 1987, "A sample of brilliance") when k <= GSO_FLOYD_MAX_K: k
+ *   draws per row instead of deg-k, the same uniform distribution over
+ *   k-subsets.  Larger k falls back to Algorithm R. */
+#define GSO_ALGO_AUTO 0
+#define GSO_ALGO_RESERVOIR 1
+#define GSO_FLOYD_MAX_K 64
+
+static inline int use_floyd(int algo, i64 k) { return algo == GSO_ALGO_AUTO && k <= GSO_FLOYD_MAX_K; }
+
 /* sub_indptr = exscan(cnt), cnt = replace ? (deg ? k : 0) : min(deg,k)
  * (sampling.cu:107-119).  replay_ptr (optional, may be NULL) = exscan of the
- * number of draws each row consumes: replace ? cnt : max(deg-k,0). */
-i64 gso_sample_count(const i64* indptr, const i64* cols, i64 S, i64 k, int replace,
+ * number of draws each row consumes: replace ? cnt : (deg > k ? (Floyd ? k :
+ * deg-k) : 0). */
+i64 gso_sample_count(const i64* indptr, const i64* cols, i64 S, i64 k, int replace, int algo,
                      i64* sub_indptr, i64* replay_ptr) {
   i64 acc = 0, racc = 0;
   for (i64 r = 0; r < S; ++r) {
@@ -172,7 +188,7 @@ i64 gso_sample_count(const i64* indptr, const i64* cols, i64 S, i64 k, int repla
     acc += cnt;
     if (replay_ptr) {
       replay_ptr[r] = racc;
-      racc += replace ? cnt : (deg > k ? deg - k : 0);
+      racc += replace ? cnt : (deg > k ? (use_floyd(algo, k) ? k : deg - k) : 0);
     }
   }
   sub_indptr[S] = acc;
@@ -181,7 +197,7 @@ i64 gso_sample_count(const i64* indptr, const i64* cols, i64 S, i64 k, int repla
 }
 
 void gso_sample_uniform_fill(const i64* indptr, const i64* indices, const i64* cols,
-                             i64 S, i64 k, int replace, u64 seed, const u32* replay,
+                             i64 S, i64 k, int replace, int algo, u64 seed, const u32* replay,
                              const i64* replay_ptr, const i64* sub_indptr,
                              i64* sub_indices, i64* select_index, i64* coo_col) {
 #pragma omp parallel
@@ -209,6 +225,26 @@ void gso_sample_uniform_fill(const i64* indptr, const i64* indices, const i64* c
         for (i64 j = 0; j < deg; ++j) {
           sub_indices[out_start + j] = indices[in_start + j];
           select_index[out_start + j] = in_start + j;
+          if (coo_col) coo_col[out_start + j] = r;
+        }
+      } else if (use_floyd(algo, k)) {
+        /* Floyd: for step i (j = deg-k+i): t = draw % (j+1); take t unless it
+         * is already taken, then take j.  Output in insertion order. */
+        for (i64 i = 0; i < k; ++i) {
+          i64 j = deg - k + i;
+          u32 x = rp ? rp[i] : gso_draw(seed, GSO_TAG_UNIFORM, (u64)r, (u64)i);
+          i64 t = (i64)(x % (u32)(j + 1));
+          for (i64 m = 0; m < i; ++m)
+            if (slot[m] == t) {
+              t = j;
+              break;
+            }
+          slot[i] = t;
+        }
+        for (i64 j = 0; j < k; ++j) {
+          i64 q = in_start + slot[j];
+          sub_indices[out_start + j] = indices[q];
+          select_index[out_start + j] = q;
           if (coo_col) coo_col[out_start + j] = r;
         }
       } else {

@@ -123,25 +123,34 @@ def slice_columns(indptr, indices, cols, with_coo=True):
 
 
 # ------------------------------------------------------------------ sampling
-def sample_count(indptr, cols, k, replace, want_replay_ptr=False):
+ALGO_AUTO, ALGO_RESERVOIR = 0, 1
+FLOYD_MAX_K = 64
+
+
+def sample_count(indptr, cols, k, replace, want_replay_ptr=False, algo=ALGO_AUTO):
     indptr = _i64(indptr)
     cols = None if cols is None else _i64(cols)
     S = indptr.size - 1 if cols is None else cols.size
     sub_indptr = np.empty(S + 1, dtype=np.int64)
     replay_ptr = np.empty(S + 1, dtype=np.int64) if want_replay_ptr else None
     lib().gso_sample_count(_p(indptr), _p(cols), _c64(S), _c64(k), ctypes.c_int(int(replace)),
-                           _p(sub_indptr), _p(replay_ptr))
+                           ctypes.c_int(int(algo)), _p(sub_indptr), _p(replay_ptr))
     return sub_indptr, replay_ptr
 
 
-def sample_uniform(indptr, indices, cols, k, replace, seed=0, replay=None, with_coo=True):
+def sample_uniform(indptr, indices, cols, k, replace, seed=0, replay=None, with_coo=True,
+                   algo=ALGO_AUTO):
     """src/cuda/sampling.cu:100-154 (cols=None) / fusion/slice_sampling.cu:91-143.
+
+    algo=ALGO_RESERVOIR is the reference's Algorithm R on every row; ALGO_AUTO uses
+    Floyd's selection on rows with deg > k (k <= FLOYD_MAX_K).
 
     Returns (sub_indptr, coo_col|None, sub_indices, select_index)."""
     indptr, indices = _i64(indptr), _i64(indices)
     cols = None if cols is None else _i64(cols)
     S = indptr.size - 1 if cols is None else cols.size
-    sub_indptr, replay_ptr = sample_count(indptr, cols, k, replace, want_replay_ptr=replay is not None)
+    sub_indptr, replay_ptr = sample_count(indptr, cols, k, replace,
+                                          want_replay_ptr=replay is not None, algo=algo)
     nnz = int(sub_indptr[S])
     if replay is not None:
         replay = _u32(replay)
@@ -150,7 +159,8 @@ def sample_uniform(indptr, indices, cols, k, replace, seed=0, replay=None, with_
     select_index = np.empty(nnz, dtype=np.int64)
     coo_col = np.empty(nnz, dtype=np.int64) if with_coo else None
     lib().gso_sample_uniform_fill(_p(indptr), _p(indices), _p(cols), _c64(S), _c64(k),
-                                  ctypes.c_int(int(replace)), _cu64(seed), _p(replay),
+                                  ctypes.c_int(int(replace)), ctypes.c_int(int(algo)),
+                                  _cu64(seed), _p(replay),
                                   _p(replay_ptr), _p(sub_indptr), _p(sub_indices),
                                   _p(select_index), _p(coo_col))
     return sub_indptr, coo_col, sub_indices, select_index

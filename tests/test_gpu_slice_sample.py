@@ -66,10 +66,14 @@ def test_slice_many_empty_columns(dev):
     _cmp(got, O.slice_columns(indptr, indices, cols, True))
 
 
-def _sample_gpu(indptr, indices, cols, k, replace, seed=0, replay=None, replay_ptr=None, with_coo=True):
+ALGOS = [O.ALGO_AUTO, O.ALGO_RESERVOIR]
+
+
+def _sample_gpu(indptr, indices, cols, k, replace, seed=0, replay=None, replay_ptr=None, with_coo=True,
+                algo=O.ALGO_AUTO):
     sub_indptr, si, sel, coo = capi.sample_uniform(indptr, indices, cols, k, replace, seed=seed,
                                                    replay=replay, replay_ptr=replay_ptr,
-                                                   with_coo=with_coo)
+                                                   with_coo=with_coo, algo=algo)
     nnz = int(sub_indptr[-1].item())
     return sub_indptr, None if coo is None else coo[:nnz], si[:nnz], sel[:nnz]
 
@@ -95,11 +99,12 @@ def test_sample_replace_reference_counts(dev, fanout):
     _cmp(got, O.sample_uniform(indptr, indices, None, fanout, True, seed=0))
 
 
+@pytest.mark.parametrize("algo", ALGOS)
 @pytest.mark.parametrize("idt", ID_DTYPES)
 @pytest.mark.parametrize("replace", [False, True])
-@pytest.mark.parametrize("k", [1, 5, 15, 100, 1000])
+@pytest.mark.parametrize("k", [1, 5, 15, 16, 17, 33, 64, 65, 1000])
 @pytest.mark.parametrize("fused", [True, False])
-def test_sample_free_running_matches_oracle(dev, idt, replace, k, fused):
+def test_sample_free_running_matches_oracle(dev, idt, replace, k, fused, algo):
     """Philox is integer-only, so even free-running draws match the oracle bit for bit."""
     indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=5)  # avg deg 32, hubs of several thousand
     if fused:
@@ -109,42 +114,47 @@ def test_sample_free_running_matches_oracle(dev, idt, replace, k, fused):
         dcols = to_dev(cols, dev, idt)
     else:
         cols, dcols = None, None
-    got = _sample_gpu(to_dev(indptr, dev), to_dev(indices, dev, idt), dcols, k, replace, seed=1234 + k)
-    want = O.sample_uniform(indptr, indices, cols, k, replace, seed=1234 + k)
+    got = _sample_gpu(to_dev(indptr, dev), to_dev(indices, dev, idt), dcols, k, replace, seed=1234 + k,
+                      algo=algo)
+    want = O.sample_uniform(indptr, indices, cols, k, replace, seed=1234 + k, algo=algo)
     _cmp(got, want)
 
 
+@pytest.mark.parametrize("algo", ALGOS)
 @pytest.mark.parametrize("replace", [False, True])
 @pytest.mark.parametrize("k", [3, 15, 900])
-def test_sample_replay_matches_oracle(dev, replace, k):
+def test_sample_replay_matches_oracle(dev, replace, k, algo):
     indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=6)
     cols = np.random.default_rng(1).integers(0, indptr.size - 1, size=2000).astype(np.int64)
     cols[:4] = np.argsort(np.diff(indptr))[-4:]
-    _, replay_ptr = O.sample_count(indptr, cols, k, replace, want_replay_ptr=True)
+    _, replay_ptr = O.sample_count(indptr, cols, k, replace, want_replay_ptr=True, algo=algo)
     replay = u32_draws(int(replay_ptr[-1]), seed=k)
-    want = O.sample_uniform(indptr, indices, cols, k, replace, replay=replay)
+    want = O.sample_uniform(indptr, indices, cols, k, replace, replay=replay, algo=algo)
     got = _sample_gpu(to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev), k, replace,
-                      replay=to_dev(replay, dev), replay_ptr=to_dev(replay_ptr, dev))
+                      replay=to_dev(replay, dev), replay_ptr=to_dev(replay_ptr, dev), algo=algo)
     _cmp(got, want)
 
 
+@pytest.mark.parametrize("algo", ALGOS)
 @pytest.mark.parametrize("k", [5, 1000])
-def test_sample_star_hub_many_chunks(dev, k):
+def test_sample_star_hub_many_chunks(dev, k, algo):
     # one column of degree 300k (74 chunks of 4096 draws) among small ones
     degs = np.array([3, 300000, 0, 17, 2000, 70000], dtype=np.int64)
     indptr = np.concatenate([[0], np.cumsum(degs)]).astype(np.int64)
     indices = np.random.default_rng(0).integers(0, 1 << 20, size=int(indptr[-1])).astype(np.int64)
     cols = np.array([1, 0, 5, 1, 2, 3, 4, 5], dtype=np.int64)
-    got = _sample_gpu(to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev), k, False, seed=77)
-    _cmp(got, O.sample_uniform(indptr, indices, cols, k, False, seed=77))
+    got = _sample_gpu(to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev), k, False, seed=77,
+                      algo=algo)
+    _cmp(got, O.sample_uniform(indptr, indices, cols, k, False, seed=77, algo=algo))
 
 
-def test_sample_structural_invariants(dev):
+@pytest.mark.parametrize("algo", ALGOS)
+def test_sample_structural_invariants(dev, algo):
     indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=7)
     cols = np.random.default_rng(2).integers(0, indptr.size - 1, size=4096).astype(np.int64)
     k = 10
     sub_indptr, _, si, sel = _sample_gpu(to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev),
-                                         k, False, seed=99, with_coo=False)
+                                         k, False, seed=99, with_coo=False, algo=algo)
     sub_indptr, si, sel = sub_indptr.cpu().numpy(), si.cpu().numpy(), sel.cpu().numpy()
     deg = indptr[cols + 1] - indptr[cols]
     assert np.array_equal(np.diff(sub_indptr), np.minimum(deg, k))
@@ -155,14 +165,15 @@ def test_sample_structural_invariants(dev):
         assert np.unique(s).size == s.size
 
 
-def test_sample_chi_square_inclusion(dev):
-    """Each edge of a degree-d column is kept with probability k/d (Algorithm R)."""
+@pytest.mark.parametrize("algo", ALGOS)
+def test_sample_chi_square_inclusion(dev, algo):
+    """Each edge of a degree-d column is kept with probability k/d (both algorithms)."""
     d, k, trials = 40, 8, 4000
     indptr = np.array([0, d], dtype=np.int64)  # one column sampled `trials` times
     indices = np.arange(d, dtype=np.int64)
     cols = np.zeros(trials, dtype=np.int64)  # duplicate seeds get independent draws (row-keyed)
     _, _, si, _ = _sample_gpu(to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev), k, False,
-                              seed=2024, with_coo=False)
+                              seed=2024, with_coo=False, algo=algo)
     counts = np.bincount(si.cpu().numpy(), minlength=d).astype(np.float64)
     expect = trials * k / d
     # positions are exchangeable up to the (negligible) dependence inside a draw; 39 dof
