@@ -414,6 +414,8 @@ def row_slice_csc(indptr, indices, row_ids, with_coo):
     out_indices = torch.empty(kept, dtype=torch.int64, device=dev)
     select_index = torch.empty(kept, dtype=torch.int64, device=dev)
     coo_col = torch.empty(kept, dtype=torch.int64, device=dev) if with_coo else None
+    if kept == 0:
+        return out_indptr, coo_col, out_indices, select_index
     _check(lib().gs_row_slice_csc_compact(_ptr(indptr), _ptr(indices), _i64(ncols), _i64(nnz),
                                           _ptr(out_indptr), _ptr(out_indices), _ptr(select_index),
                                           _ptr(coo_col), _ptr(ws), ctypes.c_size_t(ws.numel()), st),
@@ -438,6 +440,8 @@ def row_slice_coo(key, other, ids):
     out_key = torch.empty(kept, dtype=torch.int64, device=dev)
     out_other = torch.empty(kept, dtype=torch.int64, device=dev)
     select_index = torch.empty(kept, dtype=torch.int64, device=dev)
+    if kept == 0:
+        return out_key, out_other, select_index
     _check(lib().gs_row_slice_coo_compact(_ptr(key), _ptr(other), _i64(E), _ptr(out_key),
                                           _ptr(out_other), _ptr(select_index), _ptr(ws),
                                           ctypes.c_size_t(ws.numel()), st), "gs_row_slice_coo_compact")

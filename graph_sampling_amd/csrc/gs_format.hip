@@ -1,0 +1,246 @@
+// Sparse-format conversion on gfx950: CSC -> COO column expansion and
+// COO -> CSC by a stable least-significant-digit radix sort.
+//
+// Replaces impl::CSC2COOCUDA and impl::COO2CSCCUDA (reference
+// src/cuda/format_transform.cu:35,135; the reference leans on cub radix sort,
+// whose stability pins the edge order, format_transform.cu:81-100).
+//
+//  * csc2coo: edge-balanced.  A workgroup owns 2048 consecutive edges, finds the
+//    columns they span with two binary searches, stages that slice of the
+//    offsets in LDS and resolves each edge there (the reference runs a full
+//    global binary search per edge, format_transform.cu:24-33).
+//  * coo2csc: 8-bit digits, only ceil(log2(num_keys)/8) passes
+//    (format_transform.cu:58-72 also sorts just the significant bits).  Each
+//    pass is histogram -> scan -> stable scatter; the scatter ranks equal digits
+//    inside a wave with 8 ballots (no LDS atomics, order preserved) and across
+//    waves with a small LDS table.  indptr then comes from the boundaries of
+//    the sorted keys, one pass, no per-column binary search.
+#include "gs_common.hpp"
+
+namespace gs {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kItems = 8;
+constexpr int kTile = kThreads * kItems;
+constexpr int kStage = 1024;
+
+template <typename P>
+__device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
+  int64_t lo = 0, hi = n;
+  while (lo < hi) {
+    int64_t mid = (lo + hi) >> 1;
+    if (a[mid] <= v) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+__global__ void __launch_bounds__(kThreads)
+csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz,
+               int64_t* __restrict__ col) {
+  __shared__ int64_t s_ptr[kStage + 1];
+  __shared__ int64_t s_rows[2];
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
+  const int64_t p1 = p0 + kTile < nnz ? p0 + kTile : nnz;
+  if (threadIdx.x < 2)
+    s_rows[threadIdx.x] = upper_bound(indptr, num_cols + 1, threadIdx.x == 0 ? p0 : p1 - 1) - 1;
+  __syncthreads();
+  const int64_t row_lo = s_rows[0];
+  const int64_t nrows = s_rows[1] - row_lo + 1;
+  const bool staged = nrows <= kStage;
+  if (staged)
+    for (int64_t i = threadIdx.x; i <= nrows; i += kThreads) s_ptr[i] = indptr[row_lo + i];
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t p = p0 + k * kThreads + threadIdx.x;
+    if (p >= p1) break;
+    col[p] = row_lo + (staged ? upper_bound(s_ptr, nrows + 1, p)
+                              : upper_bound(indptr + row_lo, nrows + 1, p)) - 1;
+  }
+}
+
+// indptr from sorted keys: every boundary between key[e] and key[e+1] fills the
+// offsets of the columns in between (format_transform.cu:123-156 computes the
+// same values with one binary search per column).
+__global__ void __launch_bounds__(kThreads)
+indptr_from_sorted_kernel(const int64_t* __restrict__ key, int64_t E, int64_t num_keys,
+                          int64_t* __restrict__ indptr) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (e > E) return;
+  // boundary e sits between key[e-1] and key[e]; columns in (key[e-1], key[e]] start at e
+  const int64_t lo = e == 0 ? -1 : key[e - 1];
+  const int64_t hi = e == E ? num_keys : key[e];
+  for (int64_t c = lo + 1; c <= hi; ++c) indptr[c] = e;
+}
+
+// ------------------------------------------------------------ radix sort ----
+constexpr int kRadixBits = 8;
+constexpr int kRadix = 1 << kRadixBits;
+constexpr int kWaves = kThreads / kWave;
+
+__device__ __forceinline__ int digit_of(int64_t key, int shift) {
+  return static_cast<int>((static_cast<uint64_t>(key) >> shift) & (kRadix - 1));
+}
+
+// counts[d * num_blocks + b] = items of tile b with digit d
+__global__ void __launch_bounds__(kThreads)
+radix_hist_kernel(const int64_t* __restrict__ keys, int64_t E, int shift, int64_t num_blocks,
+                  int64_t* __restrict__ counts) {
+  __shared__ int s_hist[kRadix];
+  s_hist[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kTile;
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = base + k * kThreads + threadIdx.x;
+    if (i < E) atomicAdd(&s_hist[digit_of(keys[i], shift)], 1);
+  }
+  __syncthreads();
+  counts[static_cast<int64_t>(threadIdx.x) * num_blocks + blockIdx.x] = s_hist[threadIdx.x];
+}
+
+struct LoadI64 {
+  const int64_t* p;
+  __device__ __forceinline__ int64_t operator()(int64_t i) const { return p[i]; }
+};
+
+// Stable scatter of one tile.  Items are visited in index order, 256 per round;
+// inside a round the rank of an item among equal digits is (earlier waves'
+// count) + (lower lanes of its wave with the same digit).
+__global__ void __launch_bounds__(kThreads)
+radix_scatter_kernel(const int64_t* __restrict__ keys_in, const int64_t* __restrict__ perm_in,
+                     int64_t E, int shift, int64_t num_blocks, const int64_t* __restrict__ offsets,
+                     int64_t* __restrict__ keys_out, int64_t* __restrict__ perm_out) {
+  __shared__ int64_t s_base[kRadix];
+  __shared__ int s_cnt[kWaves][kRadix];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  s_base[threadIdx.x] = offsets[static_cast<int64_t>(threadIdx.x) * num_blocks + blockIdx.x];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kTile;
+  for (int k = 0; k < kItems; ++k) {
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) s_cnt[w][threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t i = base + k * kThreads + threadIdx.x;
+    const bool live = i < E;
+    int64_t key = 0;
+    int d = 0;
+    unsigned long long peers = __ballot(live);
+    if (live) {
+      key = keys_in[i];
+      d = digit_of(key, shift);
+    }
+#pragma unroll
+    for (int b = 0; b < kRadixBits; ++b) {
+      const bool bit = (d >> b) & 1;
+      const unsigned long long bal = __ballot(live && bit);
+      peers &= bit ? bal : ~bal;
+    }
+    const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+    if (live && rank == 0) s_cnt[wave][d] = __popcll(peers);
+    __syncthreads();
+    if (live) {
+      int64_t dst = s_base[d] + rank;
+      for (int w = 0; w < wave; ++w) dst += s_cnt[w][d];
+      keys_out[dst] = key;
+      perm_out[dst] = perm_in ? perm_in[i] : i;
+    }
+    __syncthreads();
+    int add = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) add += s_cnt[w][threadIdx.x];
+    s_base[threadIdx.x] += add;
+    __syncthreads();
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+gather_kernel(const int64_t* __restrict__ value, const int64_t* __restrict__ perm, int64_t E,
+              int64_t* __restrict__ out) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < E) out[i] = value[perm[i]];
+}
+
+int num_passes(int64_t num_keys) {
+  int bits = 0;
+  while ((int64_t(1) << bits) < num_keys) ++bits;  // format_transform.cu:58-72
+  return (bits + kRadixBits - 1) / kRadixBits;
+}
+
+}  // namespace
+}  // namespace gs
+
+using namespace gs;
+
+extern "C" {
+
+int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, int64_t* col, void* stream) {
+  GS_REQUIRE(num_cols >= 0 && nnz >= 0, "gs_csc2coo: negative size");
+  GS_REQUIRE(nnz == 0 || (indptr && col), "gs_csc2coo: null pointer");
+  if (nnz == 0) return GS_OK;
+  hipLaunchKernelGGL(csc2coo_kernel, dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), indptr, num_cols, nnz, col);
+  return check_launch("csc2coo");
+}
+
+size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys) {
+  (void)num_keys;
+  if (E < 0) E = 0;
+  const int64_t blocks = blocks_for(E, kTile);
+  const int64_t table = kRadix * blocks;
+  return 3 * padded(static_cast<size_t>(E > 0 ? E : 1) * 8) +  // keys ping-pong, perm pong
+         padded(static_cast<size_t>(table) * 8) + padded(static_cast<size_t>(table + 1) * 8) +
+         scan_workspace_bytes(table);
+}
+
+int gs_coo2csc(const int64_t* key, const int64_t* value, int64_t E, int64_t num_keys, int sorted,
+               int64_t* indptr, int64_t* out_value, int64_t* perm, void* workspace,
+               size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(E >= 0 && num_keys >= 0 && indptr, "gs_coo2csc: negative size or null indptr");
+  GS_REQUIRE(E == 0 || key, "gs_coo2csc: key is null");
+  GS_REQUIRE(sorted || E == 0 || (value && out_value && perm),
+             "gs_coo2csc: value/out_value/perm required when the keys are not sorted");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t* sorted_keys = key;
+  if (!sorted && E > 0) {
+    const int64_t blocks = blocks_for(E, kTile);
+    const int64_t table = kRadix * blocks;
+    Carver ws(workspace, workspace_bytes);
+    int64_t* kbuf[2] = {ws.take<int64_t>(E), ws.take<int64_t>(E)};
+    int64_t* pbuf = ws.take<int64_t>(E);
+    int64_t* counts = ws.take<int64_t>(table);
+    int64_t* offsets = ws.take<int64_t>(table + 1);
+    int64_t* tiles = ws.take<int64_t>(scan_num_tiles(table) + 1);
+    if (!ws.ok) {
+      set_error_text("gs_coo2csc: workspace needs %zu bytes, 256-byte aligned",
+                     gs_coo2csc_workspace_bytes(E, num_keys));
+      return GS_ERR_WORKSPACE;
+    }
+    int passes = num_passes(num_keys);
+    if (passes == 0) passes = 1;  // one key: still produces perm = identity
+    const int64_t* kin = key;
+    const int64_t* pin = nullptr;
+    // perm alternates between `perm` and pbuf so that the last pass lands in `perm`
+    for (int p = 0; p < passes; ++p) {
+      int64_t* kout = kbuf[p & 1];
+      int64_t* pout = ((passes - 1 - p) & 1) ? pbuf : perm;
+      hipLaunchKernelGGL(radix_hist_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0,
+                         st, kin, E, p * kRadixBits, blocks, counts);
+      LoadI64 f{counts};
+      GS_RETURN_IF_ERROR(exclusive_scan(f, table, offsets, tiles, st));
+      hipLaunchKernelGGL(radix_scatter_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kThreads),
+                         0, st, kin, pin, E, p * kRadixBits, blocks, offsets, kout, pout);
+      kin = kout;
+      pin = pout;
+    }
+    sorted_keys = kin;
+    hipLaunchKernelGGL(gather_kernel, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st, value,
+                       perm, E, out_value);
+  }
+  hipLaunchKernelGGL(indptr_from_sorted_kernel, dim3(blocks_for(E + 1, kThreads)), dim3(kThreads),
+                     0, st, sorted_keys, E, num_keys, indptr);
+  return check_launch("coo2csc");
+}
+
+}  // extern "C"

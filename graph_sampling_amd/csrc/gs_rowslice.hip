@@ -1,0 +1,304 @@
+// Row slicing (keep the edges whose row id is in a given set) on gfx950.
+//
+// Replaces impl::CSCRowSlicingCUDA and impl::COORowSlicingCUDA (reference
+// src/cuda/slicing.cu:528,768; node-set table NodeQueryHashmap :40-97).  Kept
+// ids are relabelled to their position in `ids` (slicing.cu:477-480).
+//
+// Mark:    id-set table (capacity 2 * pow2 > n, as slicing.cu:468; Fibonacci
+//          hashing instead of Hash64Shift) -> val[e] = position or -1
+//          -> prefix = exclusive scan of (val >= 0).  For the CSC flavour the
+//          new offsets are simply prefix[indptr[c]]: no per-column count pass,
+//          no warp reduction (slicing.cu:463-466), no torch::nonzero.
+// Compact: survivors are written in edge order from (val, prefix); the owning
+//          column of an edge is found like in the CSC -> COO expansion.
+// When `ids` holds duplicates the reference keeps whichever store lands last
+// (slicing.cu:56); here the largest position wins (atomicMax), deterministically.
+#include "gs_common.hpp"
+
+namespace gs {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kItems = 8;
+constexpr int kTile = kThreads * kItems;
+constexpr int kStage = 1024;
+
+struct IdSet {
+  long long* keys;  // -1 empty
+  long long* vals;
+  uint32_t mask;
+  int shift;
+  __device__ __forceinline__ uint32_t home(long long key) const {
+    return static_cast<uint32_t>((static_cast<uint64_t>(key) * 0x9E3779B97F4A7C15ull) >> shift);
+  }
+  __device__ __forceinline__ int64_t query(long long key) const {
+    uint32_t p = home(key);
+    while (true) {
+      const long long cur = keys[p];
+      if (cur == key) return vals[p];
+      if (cur == -1) return -1;
+      p = (p + 1) & mask;
+    }
+  }
+};
+
+int64_t set_capacity(int64_t n) {
+  int64_t cap = 1024;
+  while (cap < 2 * n + 2) cap <<= 1;
+  return cap;
+}
+
+__global__ void __launch_bounds__(kThreads) set_init_kernel(IdSet t, int64_t cap) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < cap) {
+    t.keys[i] = -1;
+    t.vals[i] = -1;
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+set_insert_kernel(IdSet t, const int64_t* __restrict__ ids, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= n) return;
+  const long long key = ids[i];
+  uint32_t p = t.home(key);
+  while (true) {
+    const unsigned long long prev =
+        atomicCAS(reinterpret_cast<unsigned long long*>(&t.keys[p]), ~0ull,
+                  static_cast<unsigned long long>(key));
+    if (prev == ~0ull || prev == static_cast<unsigned long long>(key)) break;
+    p = (p + 1) & t.mask;
+  }
+  atomicMax(&t.vals[p], static_cast<long long>(i));
+}
+
+__global__ void __launch_bounds__(kThreads)
+mark_kernel(IdSet t, const int64_t* __restrict__ key, int64_t E, int64_t* __restrict__ val) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (e < E) val[e] = t.query(key[e]);
+}
+
+struct Kept {
+  const int64_t* val;
+  __device__ __forceinline__ int64_t operator()(int64_t e) const { return val[e] >= 0 ? 1 : 0; }
+};
+
+__global__ void __launch_bounds__(kThreads)
+new_indptr_kernel(const int64_t* __restrict__ indptr, int64_t num_cols,
+                  const int64_t* __restrict__ prefix, int64_t* __restrict__ out_indptr) {
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (c <= num_cols) out_indptr[c] = prefix[indptr[c]];
+}
+
+__global__ void __launch_bounds__(kThreads)
+copy_total_kernel(const int64_t* __restrict__ prefix, int64_t E, int64_t* __restrict__ total) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) *total = prefix[E];
+}
+
+template <typename P>
+__device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
+  int64_t lo = 0, hi = n;
+  while (lo < hi) {
+    int64_t mid = (lo + hi) >> 1;
+    if (a[mid] <= v) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+// CSC compaction; a workgroup owns 2048 consecutive input edges.
+template <bool WITH_COO>
+__global__ void __launch_bounds__(kThreads)
+csc_compact_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz,
+                   const int64_t* __restrict__ val, const int64_t* __restrict__ prefix,
+                   int64_t* __restrict__ out_indices, int64_t* __restrict__ select_index,
+                   int64_t* __restrict__ coo_col) {
+  __shared__ int64_t s_ptr[kStage + 1];
+  __shared__ int64_t s_rows[2];
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
+  const int64_t p1 = p0 + kTile < nnz ? p0 + kTile : nnz;
+  int64_t row_lo = 0, nrows = 0;
+  bool staged = false;
+  if (WITH_COO) {
+    if (threadIdx.x < 2)
+      s_rows[threadIdx.x] = upper_bound(indptr, num_cols + 1, threadIdx.x == 0 ? p0 : p1 - 1) - 1;
+    __syncthreads();
+    row_lo = s_rows[0];
+    nrows = s_rows[1] - row_lo + 1;
+    staged = nrows <= kStage;
+    if (staged)
+      for (int64_t i = threadIdx.x; i <= nrows; i += kThreads) s_ptr[i] = indptr[row_lo + i];
+    __syncthreads();
+  }
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t e = p0 + k * kThreads + threadIdx.x;
+    if (e >= p1) break;
+    const int64_t v = val[e];
+    if (v < 0) continue;
+    const int64_t w = prefix[e];
+    out_indices[w] = v;
+    select_index[w] = e;
+    if (WITH_COO)
+      coo_col[w] = row_lo + (staged ? upper_bound(s_ptr, nrows + 1, e)
+                                    : upper_bound(indptr + row_lo, nrows + 1, e)) - 1;
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+coo_compact_kernel(const int64_t* __restrict__ other, int64_t E, const int64_t* __restrict__ val,
+                   const int64_t* __restrict__ prefix, int64_t* __restrict__ out_key,
+                   int64_t* __restrict__ out_other, int64_t* __restrict__ select_index) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (e >= E) return;
+  const int64_t v = val[e];
+  if (v < 0) return;
+  const int64_t w = prefix[e];
+  out_key[w] = v;
+  out_other[w] = other[e];
+  select_index[w] = e;
+}
+
+// Workspace layout: [val | prefix | scan tiles | id-set].  The first three
+// depend on the edge count only, so the compact call finds them again without
+// knowing how many ids the mark call was given.
+struct Scratch {
+  IdSet set;
+  int64_t cap;
+  int64_t* val;
+  int64_t* prefix;
+  int64_t* tiles;
+  bool ok;
+};
+
+Scratch carve(void* workspace, size_t bytes, int64_t n_ids, int64_t E, bool with_set) {
+  Scratch s;
+  Carver ws(workspace, bytes);
+  s.val = ws.take<int64_t>(E > 0 ? E : 1);
+  s.prefix = ws.take<int64_t>(E + 1);
+  s.tiles = ws.take<int64_t>(scan_num_tiles(E) + 1);
+  s.cap = 0;
+  if (with_set) {
+    s.cap = set_capacity(n_ids);
+    s.set.keys = ws.take<long long>(s.cap);
+    s.set.vals = ws.take<long long>(s.cap);
+    s.set.mask = static_cast<uint32_t>(s.cap - 1);
+    int lg = 0;
+    while ((int64_t(1) << lg) < s.cap) ++lg;
+    s.set.shift = 64 - lg;
+  }
+  s.ok = ws.ok;
+  return s;
+}
+
+int mark_common(const char* who, const int64_t* key, int64_t E, const int64_t* ids, int64_t n_ids,
+                Scratch& s, hipStream_t st) {
+  hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(s.cap, kThreads)), dim3(kThreads), 0, st,
+                     s.set, s.cap);
+  if (n_ids > 0)
+    hipLaunchKernelGGL(set_insert_kernel, dim3(blocks_for(n_ids, kThreads)), dim3(kThreads), 0, st,
+                       s.set, ids, n_ids);
+  if (E > 0)
+    hipLaunchKernelGGL(mark_kernel, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st, s.set, key,
+                       E, s.val);
+  GS_RETURN_IF_ERROR(check_launch(who));
+  Kept f{s.val};
+  return exclusive_scan(f, E, s.prefix, s.tiles, st);
+}
+
+}  // namespace
+}  // namespace gs
+
+using namespace gs;
+
+extern "C" {
+
+size_t gs_row_slice_workspace_bytes(int64_t num_row_ids, int64_t nnz, int64_t num_cols) {
+  (void)num_cols;
+  if (num_row_ids < 0) num_row_ids = 0;
+  if (nnz < 0) nnz = 0;
+  const int64_t cap = set_capacity(num_row_ids);
+  return 2 * padded(cap * 8) + padded((nnz > 0 ? nnz : 1) * 8) + padded((nnz + 1) * 8) +
+         scan_workspace_bytes(nnz);
+}
+
+int gs_row_slice_csc_mark(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
+                          int64_t nnz, const int64_t* row_ids, int64_t num_row_ids,
+                          int64_t* out_indptr, void* workspace, size_t workspace_bytes,
+                          void* stream) {
+  GS_REQUIRE(num_cols >= 0 && nnz >= 0 && num_row_ids >= 0, "gs_row_slice_csc_mark: negative size");
+  GS_REQUIRE(indptr && out_indptr && (nnz == 0 || indices) && (num_row_ids == 0 || row_ids),
+             "gs_row_slice_csc_mark: null pointer");
+  Scratch s = carve(workspace, workspace_bytes, num_row_ids, nnz, true);
+  if (!s.ok) {
+    set_error_text("gs_row_slice_csc_mark: workspace needs %zu bytes, 256-byte aligned",
+                   gs_row_slice_workspace_bytes(num_row_ids, nnz, num_cols));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  GS_RETURN_IF_ERROR(mark_common("row_slice_csc_mark", indices, nnz, row_ids, num_row_ids, s, st));
+  hipLaunchKernelGGL(new_indptr_kernel, dim3(blocks_for(num_cols + 1, kThreads)), dim3(kThreads), 0,
+                     st, indptr, num_cols, s.prefix, out_indptr);
+  return check_launch("row_slice_csc_mark");
+}
+
+int gs_row_slice_csc_compact(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
+                             int64_t nnz, const int64_t* out_indptr, int64_t* out_indices,
+                             int64_t* select_index, int64_t* coo_col, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+  (void)indices;
+  (void)out_indptr;
+  GS_REQUIRE(num_cols >= 0 && nnz >= 0 && indptr, "gs_row_slice_csc_compact: bad argument");
+  if (nnz == 0) return GS_OK;
+  GS_REQUIRE(out_indices && select_index, "gs_row_slice_csc_compact: null output");
+  Scratch s = carve(workspace, workspace_bytes, 0, nnz, false);
+  if (!s.ok) {
+    set_error_text("gs_row_slice_csc_compact: pass the workspace given to gs_row_slice_csc_mark");
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid(blocks_for(nnz, kTile));
+  if (coo_col)
+    hipLaunchKernelGGL((csc_compact_kernel<true>), grid, dim3(kThreads), 0, st, indptr, num_cols,
+                       nnz, s.val, s.prefix, out_indices, select_index, coo_col);
+  else
+    hipLaunchKernelGGL((csc_compact_kernel<false>), grid, dim3(kThreads), 0, st, indptr, num_cols,
+                       nnz, s.val, s.prefix, out_indices, select_index, coo_col);
+  return check_launch("row_slice_csc_compact");
+}
+
+int gs_row_slice_coo_mark(const int64_t* key, int64_t E, const int64_t* ids, int64_t num_ids,
+                          int64_t* num_kept, void* workspace, size_t workspace_bytes,
+                          void* stream) {
+  GS_REQUIRE(E >= 0 && num_ids >= 0 && num_kept, "gs_row_slice_coo_mark: bad argument");
+  GS_REQUIRE((E == 0 || key) && (num_ids == 0 || ids), "gs_row_slice_coo_mark: null pointer");
+  Scratch s = carve(workspace, workspace_bytes, num_ids, E, true);
+  if (!s.ok) {
+    set_error_text("gs_row_slice_coo_mark: workspace needs %zu bytes, 256-byte aligned",
+                   gs_row_slice_workspace_bytes(num_ids, E, 0));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  GS_RETURN_IF_ERROR(mark_common("row_slice_coo_mark", key, E, ids, num_ids, s, st));
+  hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(64), 0, st, s.prefix, E, num_kept);
+  return check_launch("row_slice_coo_mark");
+}
+
+int gs_row_slice_coo_compact(const int64_t* key, const int64_t* other, int64_t E,
+                             int64_t* out_key, int64_t* out_other, int64_t* select_index,
+                             void* workspace, size_t workspace_bytes, void* stream) {
+  (void)key;
+  GS_REQUIRE(E >= 0, "gs_row_slice_coo_compact: negative size");
+  if (E == 0) return GS_OK;
+  GS_REQUIRE(other && out_key && out_other && select_index, "gs_row_slice_coo_compact: null pointer");
+  Scratch s = carve(workspace, workspace_bytes, 0, E, false);
+  if (!s.ok) {
+    set_error_text("gs_row_slice_coo_compact: pass the workspace given to gs_row_slice_coo_mark");
+    return GS_ERR_WORKSPACE;
+  }
+  hipLaunchKernelGGL(coo_compact_kernel, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), other, E, s.val, s.prefix, out_key,
+                     out_other, select_index);
+  return check_launch("row_slice_coo_compact");
+}
+
+}  // extern "C"

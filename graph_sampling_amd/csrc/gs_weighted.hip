@@ -1,0 +1,354 @@
+// Weighted neighbour sampling without replacement (A-Res) on gfx950.
+//
+// Replaces impl::CSCColSamplingProbsCUDA (reference
+// src/cuda/sampling_probs.cu:268; kernel :25-110, which keeps a faiss
+// WarpSelect heap per warp and is limited to fanout <= 32, :32).
+//
+// Every edge of a row with deg > k gets the key log2(u)/w (same order as the
+// reference's u^(1/w), :71) and the k largest keys win, emitted in descending
+// key order, ties by lower position.  Key and position travel as one 64-bit
+// composite (ordered key << 32 | ~position): composites are distinct, so
+// "largest k" is unambiguous and bit-reproducible.
+//
+// Selection is a wave-level top-k: each of the 64 lanes streams a strided share
+// of the candidates and keeps its own sorted top-k list in LDS
+// (list[j * 64 + lane], conflict-free, touched by its lane only); the final k
+// rounds take the wave-wide maximum of the list heads (6 xor-shuffles of a
+// 64-bit value) and pop it.  Rows up to 2048 edges are one wave each.  Longer
+// rows are cut into 2048-edge chunks that go through a device queue: one wave
+// per chunk writes its local top-k composites, then one wave per long row
+// merges them.  That spreads a 10^5-edge hub over hundreds of waves instead of
+// pinning one warp on it.
+#include "gs_common.hpp"
+
+namespace gs {
+namespace {
+
+constexpr int64_t kChunk = 2048;          // edges per wave task
+constexpr int64_t kMaxFanout = 96;        // 64 lanes * 96 * 8 B = 48 KB of LDS per wave
+constexpr int kQueueGrid = 1024;          // workgroups draining a queue
+constexpr int64_t kQueueExtra = 1 << 19;  // chunk-queue capacity = S + kQueueExtra
+
+template <typename IdT>
+struct WArgs {
+  const int64_t* indptr;
+  const IdT* indices;
+  const float* probs;
+  const IdT* cols;
+  int64_t S;
+  int k;
+  uint64_t seed;
+  const uint32_t* replay;
+  const int64_t* replay_ptr;
+  const int64_t* sub_indptr;
+  IdT* sub_indices;
+  int64_t* select_index;
+  IdT* coo_col;
+  // long rows
+  unsigned long long* counters;  // [0] chunks reserved, [1] long rows
+  long long* chunk_queue;        // row << 20 | chunk, -1 = void
+  int64_t chunk_cap;
+  long long* long_rows;          // 3 entries per long row: row, first queue slot, #chunks
+  unsigned long long* cand;      // chunk_cap * k composites
+};
+
+__device__ __forceinline__ unsigned long long composite(float key, uint32_t pos) {
+  return (static_cast<unsigned long long>(float_to_ordered(key)) << 32) | (0xFFFFFFFFu - pos);
+}
+__device__ __forceinline__ uint32_t composite_pos(unsigned long long c) {
+  return 0xFFFFFFFFu - static_cast<uint32_t>(c);
+}
+
+// insert c into this lane's descending list (at most k entries)
+__device__ __forceinline__ void lane_insert(unsigned long long* list, int lane, int& cnt, int k,
+                                            unsigned long long c) {
+  if (cnt == k && c <= list[(k - 1) * kWave + lane]) return;
+  int j = cnt < k ? cnt : k - 1;
+  while (j > 0 && list[(j - 1) * kWave + lane] < c) {
+    list[j * kWave + lane] = list[(j - 1) * kWave + lane];
+    --j;
+  }
+  list[j * kWave + lane] = c;
+  if (cnt < k) ++cnt;
+}
+
+__device__ __forceinline__ unsigned long long wave_max(unsigned long long v) {
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) {
+    const unsigned long long o = __shfl_xor(v, d, kWave);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+// k rounds of "largest list head wins"; emit(j, composite) is called by every
+// lane with the same arguments (0 = fewer than j+1 candidates existed).
+template <typename Emit>
+__device__ __forceinline__ void wave_drain(const unsigned long long* list, int lane, int cnt, int k,
+                                           Emit emit) {
+  int head = 0;
+  for (int j = 0; j < k; ++j) {
+    const unsigned long long mine = head < cnt ? list[head * kWave + lane] : 0ull;
+    const unsigned long long best = wave_max(mine);
+    if (best != 0ull && mine == best) ++head;
+    emit(j, best);
+  }
+}
+
+template <typename IdT>
+__device__ __forceinline__ unsigned long long edge_composite(const WArgs<IdT>& a, int64_t r,
+                                                             int64_t start, const uint32_t* rp,
+                                                             int64_t i, const U4& x) {
+  const uint32_t xv = rp ? rp[i] : x.v[i & 3];
+  return composite(ares_key(xv, a.probs[start + i]), static_cast<uint32_t>(i));
+}
+
+// stream edges [lo, hi) of row r into the per-lane lists
+template <typename IdT>
+__device__ __forceinline__ void stream_edges(const WArgs<IdT>& a, int64_t r, int64_t start,
+                                             int64_t lo, int64_t hi, unsigned long long* list,
+                                             int lane, int& cnt) {
+  const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[r] : nullptr;
+  // a lane takes 4 consecutive edges (one Philox block) per trip
+  for (int64_t q = (lo >> 2) + lane; q * 4 < hi; q += kWave) {
+    U4 x;
+    if (!rp) x = draw_block(a.seed, kTagWeighted, static_cast<uint64_t>(r), static_cast<uint64_t>(q));
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int64_t i = q * 4 + t;
+      if (i >= lo && i < hi) lane_insert(list, lane, cnt, a.k, edge_composite(a, r, start, rp, i, x));
+    }
+  }
+}
+
+template <typename IdT, bool WITH_COO>
+__device__ __forceinline__ void emit_final(const WArgs<IdT>& a, int64_t r, int64_t start,
+                                           int64_t out_start, int lane, int j,
+                                           unsigned long long c) {
+  if (lane == (j & (kWave - 1)) && c != 0ull) {
+    const int64_t q = start + composite_pos(c);
+    a.sub_indices[out_start + j] = a.indices[q];
+    a.select_index[out_start + j] = q;
+    if (WITH_COO) a.coo_col[out_start + j] = static_cast<IdT>(r);
+  }
+}
+
+// One wave per row.  deg <= k: copy; deg <= kChunk: select here; longer: queue.
+template <typename IdT, bool WITH_COO>
+__global__ void weighted_rows_kernel(WArgs<IdT> a) {
+  extern __shared__ unsigned long long s_lists[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int waves = blockDim.x / kWave;
+  unsigned long long* list = s_lists + static_cast<size_t>(wave) * a.k * kWave;
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * waves + wave;
+  if (r >= a.S) return;
+  const int64_t c = a.cols ? static_cast<int64_t>(a.cols[r]) : r;
+  const int64_t start = a.indptr[c];
+  const int64_t deg = a.indptr[c + 1] - start;
+  const int64_t out_start = a.sub_indptr[r];
+  if (deg <= a.k) {
+    for (int64_t j = lane; j < deg; j += kWave) {
+      a.sub_indices[out_start + j] = a.indices[start + j];
+      a.select_index[out_start + j] = start + j;
+      if (WITH_COO) a.coo_col[out_start + j] = static_cast<IdT>(r);
+    }
+    return;
+  }
+  bool here = deg <= kChunk;
+  if (!here) {
+    const int64_t nchunks = (deg + kChunk - 1) / kChunk;
+    unsigned long long base = 0;
+    if (lane == 0) base = atomicAdd(&a.counters[0], static_cast<unsigned long long>(nchunks));
+    base = __shfl(base, 0, kWave);
+    if (static_cast<int64_t>(base) + nchunks <= a.chunk_cap) {
+      for (int64_t ch = lane; ch < nchunks; ch += kWave)
+        a.chunk_queue[base + ch] = static_cast<long long>((r << 20) | ch);
+      if (lane == 0) {
+        const unsigned long long slot = atomicAdd(&a.counters[1], 1ull);
+        a.long_rows[slot * 3 + 0] = r;
+        a.long_rows[slot * 3 + 1] = static_cast<long long>(base);
+        a.long_rows[slot * 3 + 2] = nchunks;
+      }
+    } else {
+      // queue full: void the reserved tail and select the whole row with this wave
+      for (int64_t ch = static_cast<int64_t>(base) + lane;
+           ch < a.chunk_cap && ch < static_cast<int64_t>(base) + nchunks; ch += kWave)
+        a.chunk_queue[ch] = -1;
+      here = true;
+    }
+  }
+  if (here) {
+    int cnt = 0;
+    stream_edges(a, r, start, 0, deg, list, lane, cnt);
+    wave_drain(list, lane, cnt, a.k, [&](int j, unsigned long long best) {
+      emit_final<IdT, WITH_COO>(a, r, start, out_start, lane, j, best);
+    });
+  }
+}
+
+// One wave per queued chunk: local top-k composites -> cand[slot * k + j].
+template <typename IdT>
+__global__ void weighted_chunks_kernel(WArgs<IdT> a) {
+  extern __shared__ unsigned long long s_lists[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int waves = blockDim.x / kWave;
+  unsigned long long* list = s_lists + static_cast<size_t>(wave) * a.k * kWave;
+  const unsigned long long reserved = a.counters[0];
+  const int64_t n = reserved < static_cast<unsigned long long>(a.chunk_cap)
+                        ? static_cast<int64_t>(reserved)
+                        : a.chunk_cap;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * waves + wave; t < n;
+       t += static_cast<int64_t>(gridDim.x) * waves) {
+    const long long e = a.chunk_queue[t];
+    if (e < 0) continue;
+    const int64_t r = e >> 20;
+    const int64_t ch = e & ((1 << 20) - 1);
+    const int64_t c = a.cols ? static_cast<int64_t>(a.cols[r]) : r;
+    const int64_t start = a.indptr[c];
+    const int64_t deg = a.indptr[c + 1] - start;
+    const int64_t lo = ch * kChunk;
+    const int64_t hi = lo + kChunk < deg ? lo + kChunk : deg;
+    int cnt = 0;
+    stream_edges(a, r, start, lo, hi, list, lane, cnt);
+    unsigned long long* out = a.cand + static_cast<size_t>(t) * a.k;
+    wave_drain(list, lane, cnt, a.k, [&](int j, unsigned long long best) {
+      if (lane == (j & (kWave - 1))) out[j] = best;
+    });
+  }
+}
+
+// One wave per long row: merge its chunks' candidates.
+template <typename IdT, bool WITH_COO>
+__global__ void weighted_merge_kernel(WArgs<IdT> a) {
+  extern __shared__ unsigned long long s_lists[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int waves = blockDim.x / kWave;
+  unsigned long long* list = s_lists + static_cast<size_t>(wave) * a.k * kWave;
+  const int64_t n = static_cast<int64_t>(a.counters[1]);
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * waves + wave; t < n;
+       t += static_cast<int64_t>(gridDim.x) * waves) {
+    const int64_t r = a.long_rows[t * 3 + 0];
+    const int64_t base = a.long_rows[t * 3 + 1];
+    const int64_t m = a.long_rows[t * 3 + 2] * a.k;
+    const int64_t c = a.cols ? static_cast<int64_t>(a.cols[r]) : r;
+    const int64_t start = a.indptr[c];
+    const int64_t out_start = a.sub_indptr[r];
+    const unsigned long long* src = a.cand + static_cast<size_t>(base) * a.k;
+    int cnt = 0;
+    for (int64_t i = lane; i < m; i += kWave) {
+      const unsigned long long cmp = src[i];
+      if (cmp != 0ull) lane_insert(list, lane, cnt, a.k, cmp);
+    }
+    wave_drain(list, lane, cnt, a.k, [&](int j, unsigned long long best) {
+      emit_final<IdT, WITH_COO>(a, r, start, out_start, lane, j, best);
+    });
+  }
+}
+
+static __global__ void zero2_kernel(unsigned long long* p) {
+  if (threadIdx.x < 2) p[threadIdx.x] = 0;
+}
+
+int waves_per_block(int64_t k) {
+  // 48 KB of LDS per workgroup
+  const int64_t per_wave = k * kWave * 8;
+  int w = static_cast<int>((48 * 1024) / per_wave);
+  return w >= 4 ? 4 : (w >= 2 ? 2 : 1);
+}
+
+template <typename IdT, bool WITH_COO>
+int weighted_launch(const WArgs<IdT>& a, hipStream_t st) {
+  const int waves = waves_per_block(a.k);
+  const size_t lds = static_cast<size_t>(waves) * a.k * kWave * 8;
+  const dim3 block(waves * kWave);
+  hipLaunchKernelGGL(zero2_kernel, dim3(1), dim3(64), 0, st, a.counters);
+  hipLaunchKernelGGL((weighted_rows_kernel<IdT, WITH_COO>),
+                     dim3(static_cast<unsigned>((a.S + waves - 1) / waves)), block, lds, st, a);
+  hipLaunchKernelGGL((weighted_chunks_kernel<IdT>), dim3(kQueueGrid), block, lds, st, a);
+  hipLaunchKernelGGL((weighted_merge_kernel<IdT, WITH_COO>), dim3(kQueueGrid), block, lds, st, a);
+  return check_launch("sample_weighted");
+}
+
+template <typename IdT>
+int weighted_impl(const int64_t* indptr, const void* indices, const float* probs, const void* cols,
+                  int64_t S, int64_t k, uint64_t seed, const uint32_t* replay,
+                  const int64_t* replay_ptr, const int64_t* sub_indptr, void* sub_indices,
+                  int64_t* select_index, void* coo_col, void* workspace, size_t workspace_bytes,
+                  hipStream_t st) {
+  Carver ws(workspace, workspace_bytes);
+  WArgs<IdT> a;
+  a.indptr = indptr;
+  a.indices = static_cast<const IdT*>(indices);
+  a.probs = probs;
+  a.cols = static_cast<const IdT*>(cols);
+  a.S = S;
+  a.k = static_cast<int>(k);
+  a.seed = seed;
+  a.replay = replay;
+  a.replay_ptr = replay_ptr;
+  a.sub_indptr = sub_indptr;
+  a.sub_indices = static_cast<IdT*>(sub_indices);
+  a.select_index = select_index;
+  a.coo_col = static_cast<IdT*>(coo_col);
+  a.chunk_cap = S + kQueueExtra;
+  a.counters = ws.take<unsigned long long>(2);
+  a.chunk_queue = ws.take<long long>(static_cast<size_t>(a.chunk_cap));
+  a.long_rows = ws.take<long long>(static_cast<size_t>(S) * 3);
+  a.cand = ws.take<unsigned long long>(static_cast<size_t>(a.chunk_cap) * k);
+  if (!ws.ok) {
+    set_error_text("gs_sample_weighted_fill: workspace needs %zu bytes, 256-byte aligned",
+                   gs_sample_weighted_workspace_bytes(S, k));
+    return GS_ERR_WORKSPACE;
+  }
+  return coo_col ? weighted_launch<IdT, true>(a, st) : weighted_launch<IdT, false>(a, st);
+}
+
+}  // namespace
+}  // namespace gs
+
+using namespace gs;
+
+extern "C" {
+
+size_t gs_sample_weighted_workspace_bytes(int64_t S, int64_t fanout) {
+  if (S < 0) S = 0;
+  if (fanout < 1) fanout = 1;
+  const size_t cap = static_cast<size_t>(S + kQueueExtra);
+  return padded(16) + padded(cap * 8) + padded(static_cast<size_t>(S) * 24) +
+         padded(cap * static_cast<size_t>(fanout) * 8);
+}
+
+int gs_sample_weighted_fill(const int64_t* indptr, const void* indices, const float* probs,
+                            const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+                            uint64_t seed, const uint32_t* replay, const int64_t* replay_ptr,
+                            const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
+                            void* coo_col, void* workspace, size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0,
+             "gs_sample_weighted_fill: null pointer or negative size");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sample_weighted_fill: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  GS_REQUIRE((replay == nullptr) == (replay_ptr == nullptr),
+             "gs_sample_weighted_fill: replay and replay_ptr must be given together");
+  if (S == 0 || fanout == 0) return GS_OK;
+  GS_REQUIRE(indices && probs && sub_indices && select_index,
+             "gs_sample_weighted_fill: null buffer");
+  if (fanout > kMaxFanout) {
+    set_error_text("gs_sample_weighted_fill: fanout %lld above the supported %lld "
+                   "(the reference stops at 32)",
+                   static_cast<long long>(fanout), static_cast<long long>(kMaxFanout));
+    return GS_ERR_UNSUPPORTED;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8
+             ? weighted_impl<int64_t>(indptr, indices, probs, column_ids, S, fanout, seed, replay,
+                                      replay_ptr, sub_indptr, sub_indices, select_index, coo_col,
+                                      workspace, workspace_bytes, st)
+             : weighted_impl<int32_t>(indptr, indices, probs, column_ids, S, fanout, seed, replay,
+                                      replay_ptr, sub_indptr, sub_indices, select_index, coo_col,
+                                      workspace, workspace_bytes, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,102 @@
+"""GPU parity: format conversion and row slicing vs the CPU oracle and closed forms."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from graph_sampling_amd import capi
+from tests.util import graph_12col_4edge, graph_20x5, rmat_csc_np, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def test_csc2coo_reference_vector(dev):
+    # reference tests/test_format_transform.cc:7-28: col = repeat_interleave(arange(20), 5)
+    indptr, _ = graph_20x5()
+    col = capi.csc2coo(to_dev(indptr, dev), 100).cpu().numpy()
+    assert np.array_equal(col, np.repeat(np.arange(20), 5))
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_csc2coo_rmat(dev, seed):
+    indptr, indices = rmat_csc_np(1 << 13, 1 << 17, seed=seed)
+    col = capi.csc2coo(to_dev(indptr, dev), indices.size).cpu().numpy()
+    assert np.array_equal(col, np.repeat(np.arange(indptr.size - 1), np.diff(indptr)))
+    assert np.array_equal(col, O.csc2coo(indptr, indices.size))
+
+
+def test_coo2csc_reference_eids(dev):
+    # reference tests/test_format_transform.cc:54-74: CSC -> CSR of the 12-column graph
+    indptr, indices = graph_12col_4edge()
+    col = np.repeat(np.arange(12), np.diff(indptr))          # [10,10,11,11]
+    ip, val, perm = capi.coo2csc(to_dev(indices, dev), to_dev(col, dev), 12, False)
+    assert np.array_equal(ip.cpu().numpy(), [0, 0, 2, 2] + [4] * 9)
+    assert np.array_equal(val.cpu().numpy(), [10, 11, 10, 11])
+    assert np.array_equal(perm.cpu().numpy(), [0, 2, 1, 3])
+
+
+@pytest.mark.parametrize("num_keys,E", [(1, 50), (7, 1000), (1 << 12, 1 << 17), (300000, 50000), (2_450_000, 200000)])
+def test_coo2csc_unsorted_matches_stable_sort(dev, num_keys, E):
+    rng = np.random.default_rng(E)
+    key = rng.integers(0, num_keys, size=E).astype(np.int64)
+    value = rng.integers(0, 1 << 40, size=E).astype(np.int64)
+    ip, val, perm = capi.coo2csc(to_dev(key, dev), to_dev(value, dev), num_keys, False)
+    want_perm = np.argsort(key, kind="stable")
+    assert np.array_equal(perm.cpu().numpy(), want_perm)
+    assert np.array_equal(val.cpu().numpy(), value[want_perm])
+    want_ip = np.concatenate([[0], np.cumsum(np.bincount(key, minlength=num_keys))])
+    assert np.array_equal(ip.cpu().numpy(), want_ip)
+    o_ip, o_val, o_perm = O.coo2csc(key, value, num_keys, False)
+    assert np.array_equal(o_ip, want_ip) and np.array_equal(o_perm, want_perm) and np.array_equal(o_val, value[want_perm])
+
+
+def test_coo2csc_sorted(dev):
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 15, seed=3)
+    col = np.repeat(np.arange(indptr.size - 1), np.diff(indptr))
+    ip, val, perm = capi.coo2csc(to_dev(col, dev), to_dev(indices, dev), indptr.size - 1, True)
+    assert perm is None
+    assert np.array_equal(ip.cpu().numpy(), indptr)
+    assert np.array_equal(val.cpu().numpy(), indices)
+
+
+def test_row_slice_csc_reference_vector(dev):
+    # reference tests/test_rowwise_slicing.cc:7-20: rows 0,5,..,95 of the 20x5 graph
+    indptr, indices = graph_20x5()
+    rows = np.arange(0, 100, 5, dtype=np.int64)
+    got = capi.row_slice_csc(to_dev(indptr, dev), to_dev(indices, dev), to_dev(rows, dev), True)
+    assert np.array_equal(got[0].cpu().numpy(), np.arange(21))
+    assert np.array_equal(got[2].cpu().numpy(), np.arange(20))
+    want = O.row_slice_csc(indptr, indices, rows, True)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+
+
+@pytest.mark.parametrize("with_coo", [True, False])
+@pytest.mark.parametrize("n_rows", [0, 1, 512, 4000])
+def test_row_slice_csc_rmat(dev, with_coo, n_rows):
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=4)
+    rows = np.random.default_rng(n_rows).permutation(1 << 12)[:n_rows].astype(np.int64)
+    got = capi.row_slice_csc(to_dev(indptr, dev), to_dev(indices, dev), to_dev(rows, dev), with_coo)
+    want = O.row_slice_csc(indptr, indices, rows, with_coo)
+    for g, w in zip(got, want):
+        if w is None:
+            assert g is None
+        else:
+            assert np.array_equal(g.cpu().numpy(), w)
+    # closed form: mask + position lookup
+    mask = np.isin(indices, rows)
+    lut = np.full(1 << 12, -1)
+    lut[rows] = np.arange(n_rows)
+    assert np.array_equal(want[2], lut[indices[mask]])
+    assert np.array_equal(want[3], np.nonzero(mask)[0])
+
+
+def test_row_slice_coo(dev):
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 16, seed=5)
+    col = np.repeat(np.arange(indptr.size - 1), np.diff(indptr))
+    ids = np.random.default_rng(0).permutation(1 << 12)[:512].astype(np.int64)
+    got = capi.row_slice_coo(to_dev(indices, dev), to_dev(col, dev), to_dev(ids, dev))
+    want = O.row_slice_coo(indices, col, ids)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+    mask = np.isin(indices, ids)
+    assert np.array_equal(want[1], col[mask])

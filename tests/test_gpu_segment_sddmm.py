@@ -1,0 +1,207 @@
+"""GPU parity: segment sums / normalise / EDivUSum and SDDMM vs the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from graph_sampling_amd import capi
+from tests.util import graph_12col_4edge, graph_20x5, rmat_csc_np, to_dev
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5  # float values: relative tolerance of the parity contract
+
+
+def _seg_sum(dev, indptr, data, powk, e_ids=None, n_ids=None, out_size=None):
+    out_size = out_size or indptr.size - 1
+    out = torch.zeros(out_size, dtype=torch.float32, device=dev)
+    capi.segment_sum(to_dev(indptr, dev), None if e_ids is None else to_dev(e_ids, dev),
+                     None if n_ids is None else to_dev(n_ids, dev), to_dev(data, dev), powk, out)
+    return out.cpu().numpy()
+
+
+def test_sum_reference_vectors(dev):
+    # reference tests/test_graph_compute.cc:8-74
+    indptr, _ = graph_20x5()
+    ones = np.ones(100, dtype=np.float32)
+    assert np.array_equal(_seg_sum(dev, indptr, ones, 1), np.full(20, 5, np.float32))
+    assert np.array_equal(_seg_sum(dev, indptr, ones, 2), np.full(20, 5, np.float32))
+    data = np.tile(np.arange(1, 6, dtype=np.float32), 20)
+    assert np.array_equal(_seg_sum(dev, indptr, data, 1), np.full(20, 15, np.float32))
+    assert np.array_equal(_seg_sum(dev, indptr, data, 2), np.full(20, 55, np.float32))
+
+
+def test_row_sum_reference_vector_coo(dev):
+    # reference tests/test_graph_compute.cc:93-108: rows 1 and 3 of the 12-column graph
+    indptr, indices = graph_12col_4edge()
+    data = np.arange(3, 7, dtype=np.float32)
+    out = torch.zeros(12, dtype=torch.float32, device=dev)
+    capi.coo_sum(to_dev(indices, dev), None, to_dev(data, dev), 1, out)
+    expected = np.array([0, 8, 0, 10] + [0] * 8, dtype=np.float32)
+    assert np.array_equal(out.cpu().numpy(), expected)
+    assert np.array_equal(O.coo_sum(indices, None, data, 1, 12), expected)
+
+
+@pytest.mark.parametrize("powk", [1, 2, 3])
+@pytest.mark.parametrize("maps", [False, True])
+def test_segment_sum_rmat(dev, powk, maps):
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=4)  # hubs of several thousand edges
+    rng = np.random.default_rng(powk)
+    data = rng.random(indices.size, dtype=np.float32)
+    e_ids = rng.permutation(indices.size).astype(np.int64) if maps else None
+    n_ids = rng.permutation(indptr.size - 1).astype(np.int64) if maps else None
+    got = _seg_sum(dev, indptr, data, powk, e_ids, n_ids)
+    want = O.segment_sum(indptr, e_ids, n_ids, data, powk, indptr.size - 1)
+    np.testing.assert_allclose(got, want, rtol=RTOL)
+    short = np.diff(indptr) <= 32  # short segments are summed in edge order: bit exact
+    idx = np.arange(indptr.size - 1) if n_ids is None else n_ids
+    assert np.array_equal(got[idx[short]], want[idx[short]])
+
+
+def test_segment_sum_mostly_empty(dev):
+    # the layer-wise sampler case: one segment per graph row, almost all empty
+    n = 300000
+    rng = np.random.default_rng(0)
+    deg = np.zeros(n, dtype=np.int64)
+    deg[rng.integers(0, n, 4000)] = rng.integers(1, 33, 4000)  # <= 32 edges: summed in edge order
+    indptr = np.concatenate([[0], np.cumsum(deg)])
+    data = rng.random(int(indptr[-1]), dtype=np.float32)
+    got = _seg_sum(dev, indptr, data, 2)
+    assert np.array_equal(got, O.segment_sum(indptr, None, None, data, 2, n))
+
+
+@pytest.mark.parametrize("maps", [False, True])
+def test_segment_normalize(dev, maps):
+    indptr, indices = rmat_csc_np(1 << 11, 1 << 16, seed=5)
+    rng = np.random.default_rng(1)
+    data = rng.random(indices.size, dtype=np.float32) + 0.1
+    e_ids = rng.permutation(indices.size).astype(np.int64) if maps else None
+    out = torch.empty(indices.size, dtype=torch.float32, device=dev)
+    capi.segment_normalize(to_dev(indptr, dev), None if e_ids is None else to_dev(e_ids, dev),
+                           to_dev(data, dev), out)
+    want = O.segment_normalize(indptr, e_ids, data)
+    np.testing.assert_allclose(out.cpu().numpy(), want, rtol=RTOL)
+    # every non-empty segment sums to 1
+    got = out.cpu().numpy()
+    d = got if e_ids is None else got[e_ids]
+    sums = np.add.reduceat(np.concatenate([d, [0]]), indptr[:-1])[np.diff(indptr) > 0]
+    np.testing.assert_allclose(sums, 1.0, rtol=1e-4)
+
+
+def test_coo_sum_and_e_div_u_sum(dev):
+    indptr, indices = rmat_csc_np(1 << 11, 1 << 16, seed=6)
+    col = O.csc2coo(indptr, indices.size)
+    rng = np.random.default_rng(2)
+    data = rng.random(indices.size, dtype=np.float32)
+    out = torch.zeros(1 << 11, dtype=torch.float32, device=dev)
+    capi.coo_sum(to_dev(indices, dev), None, to_dev(data, dev), 2, out)
+    np.testing.assert_allclose(out.cpu().numpy(), O.coo_sum(indices, None, data, 2, 1 << 11), rtol=1e-4)
+    divisor = rng.random(1 << 11, dtype=np.float32) + 0.5
+    od = torch.zeros(indices.size, dtype=torch.float32, device=dev)
+    osum = torch.zeros(1 << 11, dtype=torch.float32, device=dev)
+    capi.e_div_u_sum(to_dev(indices, dev), to_dev(col, dev), to_dev(data, dev), to_dev(divisor, dev), od, osum)
+    wd, ws = O.e_div_u_sum(indices, col, data, divisor, 1 << 11)
+    assert np.array_equal(od.cpu().numpy(), wd)  # one IEEE division per edge: bit exact
+    np.testing.assert_allclose(osum.cpu().numpy(), ws, rtol=1e-4)
+
+
+# ------------------------------------------------------------------ SDDMM
+def _sddmm_coo_gpu(dev, op, row, col, e_ids, lhs, rhs, lt, rt):
+    ls = lhs.shape if lhs.ndim > 1 else lhs.shape + (1,)
+    rs = rhs.shape if rhs.ndim > 1 else rhs.shape + (1,)
+    b = O.calc_bcast(op, ls, rs)
+    out = torch.zeros((row.size, b["out_len"]), dtype=torch.float32, device=dev)
+    capi.sddmm_coo(op, to_dev(row, dev), to_dev(col, dev), None if e_ids is None else to_dev(e_ids, dev),
+                   to_dev(lhs, dev), to_dev(rhs, dev), out, lt, rt, b["lhs_len"], b["rhs_len"],
+                   b["out_len"], b["reduce_size"],
+                   None if b["lhs_off"] is None else to_dev(b["lhs_off"], dev),
+                   None if b["rhs_off"] is None else to_dev(b["rhs_off"], dev))
+    return out.cpu().numpy()
+
+
+def test_sddmm_reference_vectors(dev):
+    # reference tests/test_sddmm.cc:7-36 (u_add_v on COO) and :95-107 (on CSC)
+    r = np.arange(100, dtype=np.int64)
+    f = np.arange(100, dtype=np.float32)
+    got = _sddmm_coo_gpu(dev, "add", r, r, None, f, f, 0, 2)
+    assert np.array_equal(got[:, 0], f * 2)
+    indptr, indices = graph_20x5()
+    rhs = np.arange(20, dtype=np.float32)
+    out = torch.zeros((100, 1), dtype=torch.float32, device=dev)
+    capi.sddmm_csc("add", to_dev(indptr, dev), to_dev(indices, dev), None, None, to_dev(f, dev),
+                   to_dev(rhs, dev), out, 0, 2, 1, 1, 1, 1)
+    assert np.array_equal(out.cpu().numpy()[:, 0], f + np.repeat(rhs, 5))
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div", "copy_lhs", "copy_rhs", "dot"])
+@pytest.mark.parametrize("targets", [(0, 2), (2, 0), (1, 2), (0, 1)])
+def test_sddmm_coo_ops_targets(dev, op, targets):
+    indptr, indices = rmat_csc_np(1 << 10, 1 << 14, seed=7)
+    col = O.csc2coo(indptr, indices.size)
+    E, N = indices.size, 1 << 10
+    rng = np.random.default_rng(3)
+    lt, rt = targets
+    lhs = rng.random((E if lt == 1 else N, 8), dtype=np.float32) + 0.5
+    rhs = rng.random((E if rt == 1 else N, 8), dtype=np.float32) + 0.5
+    e_ids = rng.permutation(E).astype(np.int64)
+    got = _sddmm_coo_gpu(dev, op, indices, col, e_ids, lhs, rhs, lt, rt)
+    want = O.sddmm_coo(op, indices, col, e_ids, lhs, rhs, lt, rt)
+    if op == "dot":
+        np.testing.assert_allclose(got, want, rtol=RTOL)
+    else:
+        assert np.array_equal(got, want)
+    # closed form (dense gather)
+    sel = {0: indices, 1: e_ids, 2: col}
+    L, R = lhs[sel[lt]], rhs[sel[rt]]
+    dense = {"add": L + R, "sub": L - R, "mul": L * R, "div": L / R, "copy_lhs": L, "copy_rhs": R,
+             "dot": (L * R).sum(1, keepdims=True)}[op]
+    full = np.zeros_like(want)
+    full[e_ids] = dense
+    np.testing.assert_allclose(want, full, rtol=RTOL)
+
+
+def test_sddmm_dot_64_fast_path(dev):
+    # u_dot_v with 64-wide fp32 features (BASELINE config 5)
+    indptr, indices = rmat_csc_np(1 << 11, 1 << 16, seed=8)
+    col = O.csc2coo(indptr, indices.size)
+    rng = np.random.default_rng(4)
+    lhs = rng.standard_normal((1 << 11, 64)).astype(np.float32)
+    rhs = rng.standard_normal((1 << 11, 64)).astype(np.float32)
+    got = _sddmm_coo_gpu(dev, "dot", indices, col, None, lhs, rhs, 0, 2)
+    want = O.sddmm_coo("dot", indices, col, None, lhs, rhs, 0, 2)
+    ref = np.einsum("ij,ij->i", lhs[indices].astype(np.float64), rhs[col].astype(np.float64))
+    scale = np.abs(lhs[indices] * rhs[col]).sum(1)  # error bound relative to the summed magnitudes
+    assert np.all(np.abs(got[:, 0] - ref) <= RTOL * scale + 1e-6)
+    assert np.all(np.abs(want[:, 0] - ref) <= RTOL * scale + 1e-6)
+
+
+def test_sddmm_broadcast(dev):
+    # worked example of the reference (src/bcast.h:20-30): lhs (1,3) op rhs (5,1) -> (5,3)
+    b = O.calc_bcast("add", (7, 1, 3), (7, 5, 1))
+    assert b["lhs_off"].tolist() == [0, 1, 2] * 5
+    assert b["rhs_off"].tolist() == [i for i in range(5) for _ in range(3)]
+    indptr, indices = rmat_csc_np(1 << 8, 1 << 11, seed=9)
+    col = O.csc2coo(indptr, indices.size)
+    rng = np.random.default_rng(5)
+    lhs = rng.random((1 << 8, 1, 3), dtype=np.float32)
+    rhs = rng.random((1 << 8, 5, 1), dtype=np.float32)
+    got = _sddmm_coo_gpu(dev, "mul", indices, col, None, lhs, rhs, 0, 2)
+    want = (lhs[indices] * rhs[col]).reshape(indices.size, 15)
+    assert np.array_equal(got, want)
+    assert np.array_equal(O.sddmm_coo("mul", indices, col, None, lhs, rhs, 0, 2), want)
+
+
+@pytest.mark.parametrize("use_maps", [False, True])
+def test_sddmm_csc(dev, use_maps):
+    indptr, indices = rmat_csc_np(1 << 10, 1 << 14, seed=10)
+    E, N = indices.size, 1 << 10
+    rng = np.random.default_rng(6)
+    lhs = rng.random((N, 4), dtype=np.float32)
+    rhs = rng.random((2 * N, 4), dtype=np.float32)
+    e_ids = rng.permutation(E).astype(np.int64) if use_maps else None
+    nid = (rng.permutation(N) + N).astype(np.int64) if use_maps else None
+    out = torch.zeros((E, 4), dtype=torch.float32, device=dev)
+    capi.sddmm_csc("add", to_dev(indptr, dev), to_dev(indices, dev),
+                   None if e_ids is None else to_dev(e_ids, dev), None if nid is None else to_dev(nid, dev),
+                   to_dev(lhs, dev), to_dev(rhs, dev), out, 0, 2, 4, 4, 4, 1)
+    want = O.sddmm_csc("add", indptr, indices, e_ids, nid, lhs, rhs, 0, 2)
+    assert np.array_equal(out.cpu().numpy(), want)

@@ -1,0 +1,164 @@
+"""GPU parity: weighted (A-Res) neighbour sampling and list sampling vs the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from graph_sampling_amd import capi
+from tests.util import rmat_csc_np, to_dev, u32_draws
+
+pytestmark = pytest.mark.gpu
+
+
+def _weighted_gpu(dev, indptr, indices, probs, cols, k, idt=torch.int64, seed=0, replay=None, replay_ptr=None):
+    dcols = None if cols is None else to_dev(cols, dev, idt)
+    sp, si, sel, coo = capi.sample_weighted(to_dev(indptr, dev), to_dev(indices, dev, idt),
+                                            to_dev(probs, dev), dcols, k, seed=seed,
+                                            replay=None if replay is None else to_dev(replay, dev),
+                                            replay_ptr=None if replay_ptr is None else to_dev(replay_ptr, dev),
+                                            with_coo=True)
+    n = int(sp[-1].item())
+    return sp.cpu().numpy(), coo[:n].cpu().numpy().astype(np.int64), si[:n].cpu().numpy().astype(np.int64), sel[:n].cpu().numpy()
+
+
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+@pytest.mark.parametrize("k", [1, 10, 25, 40, 96])
+@pytest.mark.parametrize("fused", [True, False])
+def test_weighted_free_running_matches_oracle(dev, idt, k, fused):
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=11)  # hubs above the 2048-edge chunk size
+    rng = np.random.default_rng(k)
+    probs = (1.0 - rng.random(indices.size)).astype(np.float32)
+    probs[rng.integers(0, indices.size, 500)] = 0.0  # weight <= 0: never beats a positive weight
+    cols = None
+    if fused:
+        cols = rng.integers(0, indptr.size - 1, size=2000).astype(np.int64)
+        cols[:6] = np.argsort(np.diff(indptr))[-6:]
+    got = _weighted_gpu(dev, indptr, indices, probs, cols, k, idt, seed=99)
+    want = O.sample_weighted(indptr, indices, probs, cols, k, seed=99)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+
+
+def test_weighted_replay_matches_oracle(dev):
+    indptr, indices = rmat_csc_np(1 << 11, 1 << 16, seed=12)
+    k = 12
+    probs = (1.0 - np.random.default_rng(1).random(indices.size)).astype(np.float32)
+    rp = O.weighted_replay_ptr(indptr, None, k)
+    replay = u32_draws(int(rp[-1]), 9)
+    got = _weighted_gpu(dev, indptr, indices, probs, None, k, replay=replay, replay_ptr=rp)
+    want = O.sample_weighted(indptr, indices, probs, None, k, replay=replay)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+
+
+def test_weighted_hub_many_chunks(dev):
+    degs = np.array([5, 100000, 0, 3000, 40], dtype=np.int64)
+    indptr = np.concatenate([[0], np.cumsum(degs)])
+    rng = np.random.default_rng(2)
+    indices = rng.integers(0, 1 << 20, int(indptr[-1])).astype(np.int64)
+    probs = rng.random(indices.size, dtype=np.float32) + 0.01
+    cols = np.array([1, 3, 1, 0, 2, 4], dtype=np.int64)
+    got = _weighted_gpu(dev, indptr, indices, probs, cols, 15, seed=5)
+    want = O.sample_weighted(indptr, indices, probs, cols, 15, seed=5)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+
+
+def test_weighted_special_cases(dev):
+    # one dominant weight is always selected; equal weights -> uniform inclusion
+    d, k, trials = 30, 5, 3000
+    indptr = np.array([0, d], dtype=np.int64)
+    indices = np.arange(d, dtype=np.int64)
+    cols = np.zeros(trials, dtype=np.int64)
+    probs = np.full(d, 1e-3, dtype=np.float32)
+    probs[17] = 1e6
+    _, _, si, _ = _weighted_gpu(dev, indptr, indices, probs, cols, k, seed=1)
+    assert (si.reshape(trials, k) == 17).any(axis=1).all()
+    assert (si.reshape(trials, k)[:, 0] == 17).mean() > 0.99  # and it comes first (largest key)
+    probs = np.ones(d, dtype=np.float32)
+    _, _, si, _ = _weighted_gpu(dev, indptr, indices, probs, cols, k, seed=2)
+    counts = np.bincount(si, minlength=d).astype(np.float64)
+    expect = trials * k / d
+    chi2 = ((counts - expect) ** 2 / (expect * (1 - k / d))).sum()
+    assert chi2 < (d - 1) + 5 * np.sqrt(2 * (d - 1)), chi2
+
+
+def test_weighted_first_pick_proportional_to_weight(dev):
+    """A-Res: the largest key belongs to item i with probability w_i / sum(w)."""
+    w = np.array([1, 2, 3, 4, 10], dtype=np.float32)
+    trials = 20000
+    indptr = np.array([0, 5], dtype=np.int64)
+    cols = np.zeros(trials, dtype=np.int64)
+    _, _, si, _ = _weighted_gpu(dev, indptr, np.arange(5, dtype=np.int64), w, cols, 2, seed=3)
+    first = si.reshape(trials, 2)[:, 0]
+    counts = np.bincount(first, minlength=5).astype(np.float64)
+    expect = trials * w / w.sum()
+    chi2 = ((counts - expect) ** 2 / expect).sum()
+    assert chi2 < 4 + 5 * np.sqrt(8), chi2
+
+
+# --------------------------------------------------------------- list sampling
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+def test_list_uniform_reference_cases(dev, idt):
+    # reference tests/test_listsampling.cc:7-40
+    data = np.arange(1000, dtype=np.int64)
+    d = to_dev(data, dev, idt)
+    sel, idx = capi.list_sample_uniform(d, 2000, True, seed=1)
+    assert sel.numel() == 2000 and np.unique(sel.cpu().numpy()).size <= 1000
+    sel, idx = capi.list_sample_uniform(d, 999, False, seed=1)
+    assert np.unique(sel.cpu().numpy()).size == 999
+    w_sel, w_idx = O.list_sample_uniform(data, 999, False, seed=1)
+    assert np.array_equal(sel.cpu().numpy().astype(np.int64), w_sel) and np.array_equal(idx.cpu().numpy(), w_idx)
+
+
+@pytest.mark.parametrize("replace", [False, True])
+@pytest.mark.parametrize("n,k", [(10, 3), (5000, 512), (200000, 2000)])
+def test_list_uniform_matches_oracle(dev, replace, n, k):
+    data = np.random.default_rng(n).integers(0, 1 << 30, n).astype(np.int64)
+    sel, idx = capi.list_sample_uniform(to_dev(data, dev), k, replace, seed=7)
+    w_sel, w_idx = O.list_sample_uniform(data, k, replace, seed=7)
+    assert np.array_equal(sel.cpu().numpy(), w_sel) and np.array_equal(idx.cpu().numpy(), w_idx)
+    ndraws = k if replace else n - k
+    replay = u32_draws(ndraws, 4)
+    sel, idx = capi.list_sample_uniform(to_dev(data, dev), k, replace, replay=to_dev(replay, dev))
+    w_sel, w_idx = O.list_sample_uniform(data, k, replace, replay=replay)
+    assert np.array_equal(sel.cpu().numpy(), w_sel) and np.array_equal(idx.cpu().numpy(), w_idx)
+
+
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+@pytest.mark.parametrize("n,k", [(10, 3), (5000, 512), (300000, 2000), (300000, 8192), (2500000, 512)])
+def test_list_weighted_matches_oracle(dev, idt, n, k):
+    rng = np.random.default_rng(n + k)
+    data = rng.integers(0, 1 << 30, n).astype(np.int64)
+    probs = rng.random(n, dtype=np.float32)
+    probs[rng.integers(0, n, max(1, n // 10))] = 0.0   # never selected while positive weights remain
+    sel, idx = capi.list_sample_weighted(to_dev(data, dev, idt), to_dev(probs, dev), k, seed=13)
+    w_sel, w_idx = O.list_sample_weighted(data, probs, k, seed=13)
+    assert np.array_equal(idx.cpu().numpy(), w_idx)
+    assert np.array_equal(sel.cpu().numpy().astype(np.int64), w_sel)
+    assert (probs[w_idx] > 0).all()
+
+
+def test_list_weighted_massive_ties(dev):
+    # all weights zero: every key is -inf, ties resolve to the lowest positions
+    n, k = 50000, 100
+    data = np.arange(n, dtype=np.int64) * 3
+    probs = np.zeros(n, dtype=np.float32)
+    sel, idx = capi.list_sample_weighted(to_dev(data, dev), to_dev(probs, dev), k, seed=1)
+    assert np.array_equal(idx.cpu().numpy(), np.arange(k))
+    assert np.array_equal(O.list_sample_weighted(data, probs, k, seed=1)[1], np.arange(k))
+
+
+def test_list_weighted_replay(dev):
+    n, k = 20000, 300
+    rng = np.random.default_rng(8)
+    data = np.arange(n, dtype=np.int64)
+    probs = rng.random(n, dtype=np.float32) + 0.01
+    replay = u32_draws(n, 6)
+    sel, idx = capi.list_sample_weighted(to_dev(data, dev), to_dev(probs, dev), k, replay=to_dev(replay, dev))
+    w_sel, w_idx = O.list_sample_weighted(data, probs, k, replay=replay)
+    assert np.array_equal(idx.cpu().numpy(), w_idx)
+    # closed form: argsort of the keys u^(1/w) computed in float64 (ties/rounding apart, the sets agree)
+    u = ((replay >> 8).astype(np.float64) + 1) / 2.0 ** 24
+    ref = np.argsort(-(np.log2(u) / probs.astype(np.float64)), kind="stable")[:k]
+    assert len(set(ref.tolist()) ^ set(w_idx.tolist())) <= 2
