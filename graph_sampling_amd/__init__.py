@@ -1,4 +1,50 @@
-"""MI355X-native graph-sampling engine: hand-written HIP kernels behind a C ABI,
-with a host layer mirroring the `gs` Graph / Matrix surface of
-czkkkkkk/graph_sampling."""
+"""MI355X-native graph-sampling engine.
+
+Hand-written HIP kernels behind a C ABI (``libgs_hip.so``, ``include/gs_hip.h``), a C++ host
+layer that mirrors the ``gs::Graph`` / ``graph_ops`` API of czkkkkkk/graph_sampling and
+registers ``torch.classes.gs_classes`` / ``torch.ops.gs_ops`` (``libgs.so``), and a thin Python
+layer with the ``Matrix`` / ``HeteroMatrix`` / ``ops`` surface of the reference's ``gs`` package.
+
+``import graph_sampling_amd as gs`` is meant to read like ``import gs``.
+"""
+import os
+
 from .format import _COO, _CSC, _CSR, _DCSC, _DCSR  # noqa: F401
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+HOST_LIB = os.path.join(_PKG, "libgs.so")
+_loaded = False
+
+
+def load_library():
+    """Registers torch.classes.gs_classes.* and torch.ops.gs_ops.* (raises if libgs.so is missing)."""
+    global _loaded
+    if not _loaded:
+        import torch
+        if not os.path.exists(HOST_LIB):
+            raise RuntimeError("%s is missing: run `python -m graph_sampling_amd.build`" % HOST_LIB)
+        torch.classes.load_library(HOST_LIB)
+        _loaded = True
+
+
+def __getattr__(name):
+    # torch-dependent names are resolved lazily so that the ctypes binding
+    # (graph_sampling_amd.capi) can be used without the C++ host layer
+    if name in ("Graph", "HeteroGraph"):
+        import torch
+        load_library()
+        return getattr(torch.classes.gs_classes, name)
+    if name in ("Matrix", "HeteroMatrix"):
+        from . import matrix_api
+        return getattr(matrix_api, name)
+    if name == "ops":
+        import importlib
+        return importlib.import_module(".ops", __name__)
+    raise AttributeError(name)
+
+
+def set_seed(seed):
+    """Seed of the next sampling / walk call made through Graph (then seed+1, ...)."""
+    import torch
+    load_library()
+    torch.ops.gs_ops._CAPI_SetSeed(int(seed))

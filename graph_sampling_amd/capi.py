@@ -126,7 +126,7 @@ def slice_count(indptr, column_ids):
     sub_indptr = torch.empty(S + 1, dtype=torch.int64, device=indptr.device)
     nbytes = lib().gs_slice_workspace_bytes(_i64(S))
     ws = workspace(nbytes, indptr.device)
-    _check(lib().gs_slice_count(_ptr(indptr), _ptr(column_ids), idb, _i64(S), _ptr(sub_indptr),
+    _check(lib().gs_slice_count(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(column_ids), idb, _i64(S), _ptr(sub_indptr),
                                 _ptr(ws), ctypes.c_size_t(ws.numel()), _stream(indptr.device)),
            "gs_slice_count")
     return sub_indptr
@@ -141,7 +141,7 @@ def slice_fill(indptr, indices, column_ids, sub_indptr, nnz, with_coo):
     sub_indices = torch.empty(nnz, dtype=indices.dtype, device=dev)
     select_index = torch.empty(nnz, dtype=torch.int64, device=dev)
     coo_col = torch.empty(nnz, dtype=indices.dtype, device=dev) if with_coo else None
-    _check(lib().gs_slice_fill(_ptr(indptr), _ptr(indices), _ptr(column_ids), idb, _i64(S),
+    _check(lib().gs_slice_fill(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(column_ids), idb, _i64(S),
                                _ptr(sub_indptr), _i64(nnz), _ptr(sub_indices), _ptr(select_index),
                                _ptr(coo_col), _stream(dev)), "gs_slice_fill")
     return sub_indices, select_index, coo_col
@@ -177,10 +177,10 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace, seed=0, replay=
     nbytes = lib().gs_sample_workspace_bytes(_i64(S), _i64(fanout))
     ws = workspace(nbytes, dev)
     st = _stream(dev)
-    _check(lib().gs_sample_count(_ptr(indptr), _ptr(column_ids), idb, _i64(S), _i64(fanout),
+    _check(lib().gs_sample_count(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(column_ids), idb, _i64(S), _i64(fanout),
                                  int(bool(replace)), _ptr(sub_indptr), _ptr(ws),
                                  ctypes.c_size_t(ws.numel()), st), "gs_sample_count")
-    _check(lib().gs_sample_uniform_fill(_ptr(indptr), _ptr(indices), _ptr(column_ids), idb, _i64(S),
+    _check(lib().gs_sample_uniform_fill(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(column_ids), idb, _i64(S),
                                         _i64(fanout), int(bool(replace)), int(algo), _u64(seed),
                                         _ptr(replay),
                                         _ptr(replay_ptr), _ptr(sub_indptr), _ptr(sub_indices),
@@ -198,7 +198,7 @@ def sample_one_keepdim(indptr, indices, column_ids, seed=0, replay=None):
     sub_indptr = torch.empty(S + 1, dtype=torch.int64, device=dev)
     sub_indices = torch.empty(S, dtype=indices.dtype, device=dev)
     select_index = torch.empty(S, dtype=torch.int64, device=dev)
-    _check(lib().gs_sample_one_keepdim(_ptr(indptr), _ptr(indices), _ptr(column_ids), idb, _i64(S),
+    _check(lib().gs_sample_one_keepdim(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(column_ids), idb, _i64(S),
                                        _u64(seed), _ptr(replay), _ptr(sub_indptr), _ptr(sub_indices),
                                        _ptr(select_index), _stream(dev)), "gs_sample_one_keepdim")
     return sub_indptr, sub_indices, select_index
@@ -225,10 +225,10 @@ def sample_weighted(indptr, indices, probs, column_ids, fanout, seed=0, replay=N
                  lib().gs_sample_weighted_workspace_bytes(_i64(S), _i64(fanout)))
     ws = workspace(nbytes, dev)
     st = _stream(dev)
-    _check(lib().gs_sample_count(_ptr(indptr), _ptr(column_ids), idb, _i64(S), _i64(fanout), 0,
+    _check(lib().gs_sample_count(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(column_ids), idb, _i64(S), _i64(fanout), 0,
                                  _ptr(sub_indptr), _ptr(ws), ctypes.c_size_t(ws.numel()), st),
            "gs_sample_count")
-    _check(lib().gs_sample_weighted_fill(_ptr(indptr), _ptr(indices), _ptr(probs), _ptr(column_ids),
+    _check(lib().gs_sample_weighted_fill(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(probs), _ptr(column_ids),
                                          idb, _i64(S), _i64(fanout), _u64(seed), _ptr(replay),
                                          _ptr(replay_ptr), _ptr(sub_indptr), _ptr(sub_indices),
                                          _ptr(select_index), _ptr(coo_col), _ptr(ws),
@@ -304,14 +304,17 @@ def random_walk(indptr, indices, seeds, length, seed=0, replay=None):
     dev = indptr.device
     n = seeds.numel()
     trace = torch.empty((int(length) + 1) * n, dtype=indices.dtype, device=dev)
-    _check(lib().gs_random_walk(_ptr(indptr), _ptr(indices), idb, _ptr(seeds), _i64(n), _i64(length),
+    _check(lib().gs_random_walk(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), idb, _ptr(seeds), _i64(n), _i64(length),
                                 _u64(seed), _ptr(replay), _ptr(trace), _stream(dev)),
            "gs_random_walk")
     return trace
 
 
-def metapath_walk(indptr_table, indices_table, id_dtype, metapath, seeds, seed=0, replay=None):
-    """indptr_table / indices_table: device int64 tensors holding device addresses."""
+def metapath_walk(indptr_table, indices_table, num_nodes_table, id_dtype, metapath, seeds, seed=0,
+                  replay=None):
+    """indptr_table / indices_table: device int64 tensors holding device addresses;
+    num_nodes_table: device int64 tensor, columns per relation."""
+    _need(num_nodes_table, torch.int64, "num_nodes_table")
     _need(metapath, torch.int64, "metapath")
     idb = _ids(seeds, "seeds")
     if seeds.dtype != id_dtype:
@@ -320,7 +323,7 @@ def metapath_walk(indptr_table, indices_table, id_dtype, metapath, seeds, seed=0
     n = seeds.numel()
     L = metapath.numel()
     trace = torch.empty((L + 1) * n, dtype=seeds.dtype, device=dev)
-    _check(lib().gs_metapath_walk(_ptr(indptr_table), _ptr(indices_table), idb, _ptr(metapath),
+    _check(lib().gs_metapath_walk(_ptr(indptr_table), _ptr(indices_table), _ptr(num_nodes_table), idb, _ptr(metapath),
                                   _i64(L), _ptr(seeds), _i64(n), _u64(seed), _ptr(replay),
                                   _ptr(trace), _stream(dev)), "gs_metapath_walk")
     return trace

@@ -69,8 +69,12 @@ indptr_from_sorted_kernel(const int64_t* __restrict__ key, int64_t E, int64_t nu
   const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (e > E) return;
   // boundary e sits between key[e-1] and key[e]; columns in (key[e-1], key[e]] start at e
-  const int64_t lo = e == 0 ? -1 : key[e - 1];
-  const int64_t hi = e == E ? num_keys : key[e];
+  // keys outside [0, num_keys) (an inconsistent caller) are clamped: they can
+  // never index past the num_keys + 1 offsets
+  int64_t lo = e == 0 ? -1 : key[e - 1];
+  int64_t hi = e == E ? num_keys : key[e];
+  if (lo < -1) lo = -1;
+  if (hi > num_keys) hi = num_keys;
   for (int64_t c = lo + 1; c <= hi; ++c) indptr[c] = e;
 }
 

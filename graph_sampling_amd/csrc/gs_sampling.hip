@@ -27,12 +27,21 @@ namespace gs {
 namespace {
 
 // ------------------------------------------------------------- functors ----
+// A column id outside [0, num_cols) is treated as an empty column everywhere in
+// this file, so that stray ids (e.g. the -1 a dead-end walk step hands back) can
+// never turn into a wild read.
+__device__ __forceinline__ bool valid_col(int64_t c, int64_t num_cols) {
+  return static_cast<uint64_t>(c) < static_cast<uint64_t>(num_cols);
+}
+
 template <typename IdT>
 struct ColDegree {
   const int64_t* indptr;
   const IdT* cols;  // nullptr: identity
+  int64_t num_cols;
   __device__ __forceinline__ int64_t operator()(int64_t r) const {
     int64_t c = cols ? static_cast<int64_t>(cols[r]) : r;
+    if (!valid_col(c, num_cols)) return 0;
     return indptr[c + 1] - indptr[c];
   }
 };
@@ -41,11 +50,12 @@ template <typename IdT>
 struct ColCount {
   const int64_t* indptr;
   const IdT* cols;
+  int64_t num_cols;
   int64_t k;
   int replace;
   __device__ __forceinline__ int64_t operator()(int64_t r) const {
     int64_t c = cols ? static_cast<int64_t>(cols[r]) : r;
-    int64_t deg = indptr[c + 1] - indptr[c];
+    int64_t deg = valid_col(c, num_cols) ? indptr[c + 1] - indptr[c] : 0;
     if (replace) return deg == 0 ? 0 : k;
     return deg < k ? deg : k;
   }
@@ -71,7 +81,8 @@ constexpr int kFillStage = 1024;  // rows of offsets staged in LDS
 template <typename IdT, bool WITH_COO>
 __global__ void __launch_bounds__(kFillThreads)
 slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
-                  const IdT* __restrict__ cols, int64_t S, const int64_t* __restrict__ sub_indptr,
+                  const IdT* __restrict__ cols, int64_t num_cols, int64_t S,
+                  const int64_t* __restrict__ sub_indptr,
                   int64_t nnz, IdT* __restrict__ sub_indices, int64_t* __restrict__ select_index,
                   IdT* __restrict__ coo_col) {
   __shared__ int64_t s_ptr[kFillStage + 1];
@@ -92,7 +103,7 @@ slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ in
       s_ptr[i] = sub_indptr[row_lo + i];
       if (i < nrows) {
         int64_t c = cols ? static_cast<int64_t>(cols[row_lo + i]) : row_lo + i;
-        s_in[i] = indptr[c];
+        s_in[i] = valid_col(c, num_cols) ? indptr[c] : 0;  // invalid: empty row, never used
       }
     }
   }
@@ -108,7 +119,7 @@ slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ in
       q = s_in[i] + (p - s_ptr[i]);
     } else {
       row = row_lo + upper_bound(sub_indptr + row_lo, nrows + 1, p) - 1;
-      int64_t c = cols ? static_cast<int64_t>(cols[row]) : row;
+      int64_t c = cols ? static_cast<int64_t>(cols[row]) : row;  // non-empty row => valid id
       q = indptr[c] + (p - sub_indptr[row]);
     }
     sub_indices[p] = indices[q];
@@ -136,6 +147,7 @@ struct SampleArgs {
   const int64_t* indptr;
   const IdT* indices;
   const IdT* cols;
+  int64_t num_cols;
   int64_t S;
   int64_t k;
   uint64_t seed;
@@ -178,8 +190,13 @@ template <typename IdT>
 __device__ __forceinline__ void load_row(const SampleArgs<IdT>& a, int64_t r, int64_t* start,
                                          int64_t* deg, int64_t* out_start) {
   int64_t c = a.cols ? static_cast<int64_t>(a.cols[r]) : r;
-  *start = a.indptr[c];
-  *deg = a.indptr[c + 1] - *start;
+  if (valid_col(c, a.num_cols)) {
+    *start = a.indptr[c];
+    *deg = a.indptr[c + 1] - *start;
+  } else {
+    *start = 0;
+    *deg = 0;
+  }
   *out_start = a.sub_indptr[r];
 }
 
@@ -396,7 +413,7 @@ __global__ void __launch_bounds__(kSampleThreads) sample_replace_kernel(SampleAr
 template <typename IdT>
 __global__ void __launch_bounds__(256)
 sample_one_keepdim_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
-                          const IdT* __restrict__ cols, int64_t S, uint64_t seed,
+                          const IdT* __restrict__ cols, int64_t num_cols, int64_t S, uint64_t seed,
                           const uint32_t* __restrict__ replay, int64_t* __restrict__ sub_indptr,
                           IdT* __restrict__ sub_indices, int64_t* __restrict__ select_index) {
   const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -404,9 +421,10 @@ sample_one_keepdim_kernel(const int64_t* __restrict__ indptr, const IdT* __restr
   sub_indptr[r] = r;
   if (r == S) return;
   const int64_t c = static_cast<int64_t>(cols[r]);
-  const int64_t start = indptr[c];
-  const int64_t deg = indptr[c + 1] - start;
-  if (deg == 0) {
+  const bool ok = valid_col(c, num_cols);
+  const int64_t start = ok ? indptr[c] : 0;
+  const int64_t deg = ok ? indptr[c + 1] - start : 0;
+  if (deg <= 0) {
     sub_indices[r] = static_cast<IdT>(-1);
     select_index[r] = -1;
   } else {
@@ -419,36 +437,38 @@ sample_one_keepdim_kernel(const int64_t* __restrict__ indptr, const IdT* __restr
 
 // ----------------------------------------------------------- host glue -----
 template <typename IdT>
-int slice_count_impl(const int64_t* indptr, const void* cols, int64_t S, int64_t* sub_indptr,
-                     int64_t* tile_ws, hipStream_t stream) {
-  ColDegree<IdT> f{indptr, static_cast<const IdT*>(cols)};
+int slice_count_impl(const int64_t* indptr, int64_t num_cols, const void* cols, int64_t S,
+                     int64_t* sub_indptr, int64_t* tile_ws, hipStream_t stream) {
+  ColDegree<IdT> f{indptr, static_cast<const IdT*>(cols), num_cols};
   return exclusive_scan(f, S, sub_indptr, tile_ws, stream);
 }
 
 template <typename IdT>
-int slice_fill_impl(const int64_t* indptr, const void* indices, const void* cols, int64_t S,
-                    const int64_t* sub_indptr, int64_t nnz, void* sub_indices,
+int slice_fill_impl(const int64_t* indptr, int64_t num_cols, const void* indices,
+                    const void* cols, int64_t S, const int64_t* sub_indptr, int64_t nnz,
+                    void* sub_indices,
                     int64_t* select_index, void* coo_col, hipStream_t stream) {
   if (nnz == 0) return GS_OK;
   const unsigned grid = static_cast<unsigned>((nnz + kFillTile - 1) / kFillTile);
   if (coo_col) {
     hipLaunchKernelGGL((slice_fill_kernel<IdT, true>), dim3(grid), dim3(kFillThreads), 0, stream,
-                       indptr, static_cast<const IdT*>(indices), static_cast<const IdT*>(cols), S,
-                       sub_indptr, nnz, static_cast<IdT*>(sub_indices), select_index,
+                       indptr, static_cast<const IdT*>(indices), static_cast<const IdT*>(cols),
+                       num_cols, S, sub_indptr, nnz, static_cast<IdT*>(sub_indices), select_index,
                        static_cast<IdT*>(coo_col));
   } else {
     hipLaunchKernelGGL((slice_fill_kernel<IdT, false>), dim3(grid), dim3(kFillThreads), 0, stream,
-                       indptr, static_cast<const IdT*>(indices), static_cast<const IdT*>(cols), S,
-                       sub_indptr, nnz, static_cast<IdT*>(sub_indices), select_index,
+                       indptr, static_cast<const IdT*>(indices), static_cast<const IdT*>(cols),
+                       num_cols, S, sub_indptr, nnz, static_cast<IdT*>(sub_indices), select_index,
                        static_cast<IdT*>(nullptr));
   }
   return check_launch("slice_fill");
 }
 
 template <typename IdT>
-int sample_count_impl(const int64_t* indptr, const void* cols, int64_t S, int64_t k, int replace,
-                      int64_t* sub_indptr, int64_t* tile_ws, hipStream_t stream) {
-  ColCount<IdT> f{indptr, static_cast<const IdT*>(cols), k, replace};
+int sample_count_impl(const int64_t* indptr, int64_t num_cols, const void* cols, int64_t S,
+                      int64_t k, int replace, int64_t* sub_indptr, int64_t* tile_ws,
+                      hipStream_t stream) {
+  ColCount<IdT> f{indptr, static_cast<const IdT*>(cols), num_cols, k, replace};
   return exclusive_scan(f, S, sub_indptr, tile_ws, stream);
 }
 
@@ -504,8 +524,8 @@ int sample_fill_impl(const SampleArgs<IdT>& a, int replace, int algo, hipStream_
 using namespace gs;
 
 template <typename IdT>
-static int sample_uniform_fill_t(const int64_t* indptr, const void* indices, const void* column_ids,
-                                 int64_t S, int64_t fanout, int replace, uint64_t seed,
+static int sample_uniform_fill_t(const int64_t* indptr, int64_t num_cols, const void* indices,
+                                 const void* column_ids, int64_t S, int64_t fanout, int replace, uint64_t seed,
                                  const uint32_t* replay, const int64_t* replay_ptr,
                                  const int64_t* sub_indptr, void* sub_indices,
                                  int64_t* select_index, void* coo_col, long long* queue,
@@ -514,6 +534,7 @@ static int sample_uniform_fill_t(const int64_t* indptr, const void* indices, con
   SampleArgs<IdT> a{indptr,
                     static_cast<const IdT*>(indices),
                     static_cast<const IdT*>(column_ids),
+                    num_cols,
                     S,
                     fanout,
                     seed,
@@ -534,9 +555,11 @@ extern "C" {
 
 size_t gs_slice_workspace_bytes(int64_t num_cols) { return scan_workspace_bytes(num_cols); }
 
-int gs_slice_count(const int64_t* indptr, const void* column_ids, int id_bytes, int64_t S,
-                   int64_t* sub_indptr, void* workspace, size_t workspace_bytes, void* stream) {
-  GS_REQUIRE(indptr && sub_indptr && S >= 0, "gs_slice_count: null pointer or negative size");
+int gs_slice_count(const int64_t* indptr, int64_t num_cols, const void* column_ids, int id_bytes,
+                   int64_t S, int64_t* sub_indptr, void* workspace, size_t workspace_bytes,
+                   void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && num_cols >= 0,
+             "gs_slice_count: null pointer or negative size");
   GS_REQUIRE(S == 0 || column_ids, "gs_slice_count: column_ids is null");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_slice_count: id_bytes must be 4 or 8, got %d", id_bytes);
   Carver ws(workspace, workspace_bytes);
@@ -547,22 +570,27 @@ int gs_slice_count(const int64_t* indptr, const void* column_ids, int id_bytes, 
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return id_bytes == 8 ? slice_count_impl<int64_t>(indptr, column_ids, S, sub_indptr, tiles, st)
-                       : slice_count_impl<int32_t>(indptr, column_ids, S, sub_indptr, tiles, st);
+  return id_bytes == 8
+             ? slice_count_impl<int64_t>(indptr, num_cols, column_ids, S, sub_indptr, tiles, st)
+             : slice_count_impl<int32_t>(indptr, num_cols, column_ids, S, sub_indptr, tiles, st);
 }
 
-int gs_slice_fill(const int64_t* indptr, const void* indices, const void* column_ids,
-                  int id_bytes, int64_t S, const int64_t* sub_indptr, int64_t nnz,
-                  void* sub_indices, int64_t* select_index, void* coo_col, void* stream) {
-  GS_REQUIRE(indptr && sub_indptr && S >= 0 && nnz >= 0, "gs_slice_fill: null pointer or negative size");
+int gs_slice_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
+                  const void* column_ids, int id_bytes, int64_t S, const int64_t* sub_indptr,
+                  int64_t nnz, void* sub_indices, int64_t* select_index, void* coo_col,
+                  void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && nnz >= 0 && num_cols >= 0,
+             "gs_slice_fill: null pointer or negative size");
   GS_REQUIRE(nnz == 0 || (indices && column_ids && sub_indices && select_index),
              "gs_slice_fill: null buffer with nnz > 0");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_slice_fill: id_bytes must be 4 or 8, got %d", id_bytes);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return id_bytes == 8 ? slice_fill_impl<int64_t>(indptr, indices, column_ids, S, sub_indptr, nnz,
-                                                  sub_indices, select_index, coo_col, st)
-                       : slice_fill_impl<int32_t>(indptr, indices, column_ids, S, sub_indptr, nnz,
-                                                  sub_indices, select_index, coo_col, st);
+  return id_bytes == 8 ? slice_fill_impl<int64_t>(indptr, num_cols, indices, column_ids, S,
+                                                  sub_indptr, nnz, sub_indices, select_index,
+                                                  coo_col, st)
+                       : slice_fill_impl<int32_t>(indptr, num_cols, indices, column_ids, S,
+                                                  sub_indptr, nnz, sub_indices, select_index,
+                                                  coo_col, st);
 }
 
 size_t gs_sample_workspace_bytes(int64_t S, int64_t fanout) {
@@ -571,11 +599,12 @@ size_t gs_sample_workspace_bytes(int64_t S, int64_t fanout) {
   return scan_workspace_bytes(s) + padded(8) + padded(static_cast<size_t>(s + kQueueExtra) * 8);
 }
 
-int gs_sample_count(const int64_t* indptr, const void* column_ids, int id_bytes, int64_t S,
-                    int64_t fanout, int replace, int64_t* sub_indptr, void* workspace,
+int gs_sample_count(const int64_t* indptr, int64_t num_cols, const void* column_ids, int id_bytes,
+                    int64_t S, int64_t fanout, int replace, int64_t* sub_indptr, void* workspace,
                     size_t workspace_bytes, void* stream) {
-  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0,
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0 && num_cols >= 0,
              "gs_sample_count: null pointer or negative size");
+  GS_REQUIRE(column_ids || S <= num_cols, "gs_sample_count: S exceeds num_cols without column_ids");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sample_count: id_bytes must be 4 or 8, got %d", id_bytes);
   Carver ws(workspace, workspace_bytes);
   int64_t* tiles = ws.take<int64_t>(scan_num_tiles(S) + 1);
@@ -586,18 +615,22 @@ int gs_sample_count(const int64_t* indptr, const void* column_ids, int id_bytes,
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   return id_bytes == 8
-             ? sample_count_impl<int64_t>(indptr, column_ids, S, fanout, replace, sub_indptr, tiles, st)
-             : sample_count_impl<int32_t>(indptr, column_ids, S, fanout, replace, sub_indptr, tiles, st);
+             ? sample_count_impl<int64_t>(indptr, num_cols, column_ids, S, fanout, replace,
+                                          sub_indptr, tiles, st)
+             : sample_count_impl<int32_t>(indptr, num_cols, column_ids, S, fanout, replace,
+                                          sub_indptr, tiles, st);
 }
 
-int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const void* column_ids,
-                           int id_bytes, int64_t S, int64_t fanout, int replace, int algo,
-                           uint64_t seed,
+int gs_sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
+                           const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+                           int replace, int algo, uint64_t seed,
                            const uint32_t* replay, const int64_t* replay_ptr,
                            const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                            void* coo_col, void* workspace, size_t workspace_bytes, void* stream) {
-  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0,
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0 && num_cols >= 0,
              "gs_sample_uniform_fill: null pointer or negative size");
+  GS_REQUIRE(column_ids || S <= num_cols,
+             "gs_sample_uniform_fill: S exceeds num_cols without column_ids");
   GS_REQUIRE(S == 0 || fanout == 0 || (indices && sub_indices && select_index),
              "gs_sample_uniform_fill: null buffer");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sample_uniform_fill: id_bytes must be 4 or 8, got %d",
@@ -620,21 +653,23 @@ int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const voi
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   return id_bytes == 8
-             ? sample_uniform_fill_t<int64_t>(indptr, indices, column_ids, S, fanout, replace, seed,
+             ? sample_uniform_fill_t<int64_t>(indptr, num_cols, indices, column_ids, S, fanout, replace, seed,
                                               replay, replay_ptr, sub_indptr, sub_indices,
                                               select_index, coo_col, queue, queue_count,
                                               queue_cap, algo, st)
-             : sample_uniform_fill_t<int32_t>(indptr, indices, column_ids, S, fanout, replace, seed,
+             : sample_uniform_fill_t<int32_t>(indptr, num_cols, indices, column_ids, S, fanout, replace, seed,
                                               replay, replay_ptr, sub_indptr, sub_indices,
                                               select_index, coo_col, queue, queue_count,
                                               queue_cap, algo, st);
 }
 
-int gs_sample_one_keepdim(const int64_t* indptr, const void* indices, const void* column_ids,
-                          int id_bytes, int64_t S, uint64_t seed, const uint32_t* replay,
+int gs_sample_one_keepdim(const int64_t* indptr, int64_t num_cols, const void* indices,
+                          const void* column_ids, int id_bytes, int64_t S, uint64_t seed,
+                          const uint32_t* replay,
                           int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                           void* stream) {
-  GS_REQUIRE(indptr && sub_indptr && S >= 0, "gs_sample_one_keepdim: null pointer or negative size");
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && num_cols >= 0,
+             "gs_sample_one_keepdim: null pointer or negative size");
   GS_REQUIRE(S == 0 || (indices && column_ids && sub_indices && select_index),
              "gs_sample_one_keepdim: null buffer");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sample_one_keepdim: id_bytes must be 4 or 8, got %d",
@@ -644,11 +679,13 @@ int gs_sample_one_keepdim(const int64_t* indptr, const void* indices, const void
   if (id_bytes == 8) {
     hipLaunchKernelGGL((sample_one_keepdim_kernel<int64_t>), dim3(grid), dim3(256), 0, st, indptr,
                        static_cast<const int64_t*>(indices), static_cast<const int64_t*>(column_ids),
-                       S, seed, replay, sub_indptr, static_cast<int64_t*>(sub_indices), select_index);
+                       num_cols, S, seed, replay, sub_indptr, static_cast<int64_t*>(sub_indices),
+                       select_index);
   } else {
     hipLaunchKernelGGL((sample_one_keepdim_kernel<int32_t>), dim3(grid), dim3(256), 0, st, indptr,
                        static_cast<const int32_t*>(indices), static_cast<const int32_t*>(column_ids),
-                       S, seed, replay, sub_indptr, static_cast<int32_t*>(sub_indices), select_index);
+                       num_cols, S, seed, replay, sub_indptr, static_cast<int32_t*>(sub_indices),
+                       select_index);
   }
   return check_launch("sample_one_keepdim");
 }

@@ -65,7 +65,9 @@ __device__ __forceinline__ void edge_endpoints(const SddmmArgs& a, int64_t e, in
       const int64_t mid = (lo + hi) >> 1;
       if (a.indptr[mid] <= e) lo = mid + 1; else hi = mid;
     }
-    const int64_t c = lo - 1;
+    int64_t c = lo - 1;
+    if (c >= a.num_cols) c = a.num_cols - 1;  // offsets that do not cover every edge
+    if (c < 0) c = 0;
     *dst = a.nid_map ? a.nid_map[c] : c;
   } else {
     *dst = a.col[e];

@@ -18,10 +18,13 @@ namespace {
 
 constexpr int kThreads = 256;
 
+// A node outside [0, num_nodes) has no neighbours (the walker dies there), so a
+// stray seed can never turn into a wild read.
 template <typename IdT>
 __device__ __forceinline__ int64_t step_from(const int64_t* __restrict__ indptr,
-                                             const IdT* __restrict__ indices, int64_t curr,
-                                             uint32_t x) {
+                                             const IdT* __restrict__ indices, int64_t num_nodes,
+                                             int64_t curr, uint32_t x) {
+  if (static_cast<uint64_t>(curr) >= static_cast<uint64_t>(num_nodes)) return -1;
   const int64_t start = indptr[curr];
   const int64_t deg = indptr[curr + 1] - start;
   if (deg <= 0) return -1;
@@ -31,7 +34,7 @@ __device__ __forceinline__ int64_t step_from(const int64_t* __restrict__ indptr,
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 random_walk_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
-                   const IdT* __restrict__ seeds, int64_t n, int64_t length, uint64_t seed,
+                   int64_t num_nodes, const IdT* __restrict__ seeds, int64_t n, int64_t length, uint64_t seed,
                    const uint32_t* __restrict__ replay, IdT* __restrict__ trace) {
   const int64_t w = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (w >= n) return;
@@ -44,7 +47,7 @@ random_walk_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ i
     int64_t pick = -1;
     if (curr >= 0) {
       const uint32_t xv = replay ? replay[t * n + w] : x.v[t & 3];
-      pick = step_from(indptr, indices, curr, xv);
+      pick = step_from(indptr, indices, num_nodes, curr, xv);
     }
     trace[(t + 1) * n + w] = static_cast<IdT>(pick);
     curr = pick;
@@ -55,6 +58,7 @@ template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 metapath_walk_kernel(const int64_t* const* __restrict__ all_indptr,
                      const IdT* const* __restrict__ all_indices,
+                     const int64_t* __restrict__ all_num_nodes,
                      const int64_t* __restrict__ metapath, int64_t length,
                      const IdT* __restrict__ seeds, int64_t n, uint64_t seed,
                      const uint32_t* __restrict__ replay, IdT* __restrict__ trace) {
@@ -70,7 +74,7 @@ metapath_walk_kernel(const int64_t* const* __restrict__ all_indptr,
     if (curr >= 0) {
       const int64_t rel = metapath[t];  // uniform over the wave: scalar loads
       const uint32_t xv = replay ? replay[t * n + w] : x.v[t & 3];
-      pick = step_from(all_indptr[rel], all_indices[rel], curr, xv);
+      pick = step_from(all_indptr[rel], all_indices[rel], all_num_nodes[rel], curr, xv);
     }
     trace[(t + 1) * n + w] = static_cast<IdT>(pick);
     curr = pick;
@@ -84,10 +88,10 @@ using namespace gs;
 
 extern "C" {
 
-int gs_random_walk(const int64_t* indptr, const void* indices, int id_bytes, const void* seeds,
-                   int64_t n, int64_t length, uint64_t seed, const uint32_t* replay,
+int gs_random_walk(const int64_t* indptr, int64_t num_nodes, const void* indices, int id_bytes,
+                   const void* seeds, int64_t n, int64_t length, uint64_t seed, const uint32_t* replay,
                    void* trace, void* stream) {
-  GS_REQUIRE(n >= 0 && length >= 0, "gs_random_walk: negative size");
+  GS_REQUIRE(n >= 0 && length >= 0 && num_nodes >= 0, "gs_random_walk: negative size");
   GS_REQUIRE(n == 0 || (indptr && seeds && trace), "gs_random_walk: null pointer");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_random_walk: id_bytes must be 4 or 8, got %d", id_bytes);
   if (n == 0) return GS_OK;
@@ -95,22 +99,24 @@ int gs_random_walk(const int64_t* indptr, const void* indices, int id_bytes, con
   const dim3 grid(blocks_for(n, kThreads));
   if (id_bytes == 8)
     hipLaunchKernelGGL((random_walk_kernel<int64_t>), grid, dim3(kThreads), 0, st, indptr,
-                       static_cast<const int64_t*>(indices), static_cast<const int64_t*>(seeds), n,
-                       length, seed, replay, static_cast<int64_t*>(trace));
+                       static_cast<const int64_t*>(indices), num_nodes,
+                       static_cast<const int64_t*>(seeds), n, length, seed, replay,
+                       static_cast<int64_t*>(trace));
   else
     hipLaunchKernelGGL((random_walk_kernel<int32_t>), grid, dim3(kThreads), 0, st, indptr,
-                       static_cast<const int32_t*>(indices), static_cast<const int32_t*>(seeds), n,
-                       length, seed, replay, static_cast<int32_t*>(trace));
+                       static_cast<const int32_t*>(indices), num_nodes,
+                       static_cast<const int32_t*>(seeds), n, length, seed, replay,
+                       static_cast<int32_t*>(trace));
   return check_launch("random_walk");
 }
 
 int gs_metapath_walk(const int64_t* const* all_indptr, const void* const* all_indices,
-                     int id_bytes, const int64_t* metapath, int64_t length, const void* seeds,
+                     const int64_t* all_num_nodes, int id_bytes, const int64_t* metapath, int64_t length, const void* seeds,
                      int64_t n, uint64_t seed, const uint32_t* replay, void* trace,
                      void* stream) {
   GS_REQUIRE(n >= 0 && length >= 0, "gs_metapath_walk: negative size");
   GS_REQUIRE(n == 0 || (seeds && trace), "gs_metapath_walk: null pointer");
-  GS_REQUIRE(n == 0 || length == 0 || (all_indptr && all_indices && metapath),
+  GS_REQUIRE(n == 0 || length == 0 || (all_indptr && all_indices && all_num_nodes && metapath),
              "gs_metapath_walk: null relation tables");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_metapath_walk: id_bytes must be 4 or 8, got %d", id_bytes);
   if (n == 0) return GS_OK;
@@ -118,12 +124,14 @@ int gs_metapath_walk(const int64_t* const* all_indptr, const void* const* all_in
   const dim3 grid(blocks_for(n, kThreads));
   if (id_bytes == 8)
     hipLaunchKernelGGL((metapath_walk_kernel<int64_t>), grid, dim3(kThreads), 0, st, all_indptr,
-                       reinterpret_cast<const int64_t* const*>(all_indices), metapath, length,
+                       reinterpret_cast<const int64_t* const*>(all_indices), all_num_nodes, metapath,
+                       length,
                        static_cast<const int64_t*>(seeds), n, seed, replay,
                        static_cast<int64_t*>(trace));
   else
     hipLaunchKernelGGL((metapath_walk_kernel<int32_t>), grid, dim3(kThreads), 0, st, all_indptr,
-                       reinterpret_cast<const int32_t* const*>(all_indices), metapath, length,
+                       reinterpret_cast<const int32_t* const*>(all_indices), all_num_nodes, metapath,
+                       length,
                        static_cast<const int32_t*>(seeds), n, seed, replay,
                        static_cast<int32_t*>(trace));
   return check_launch("metapath_walk");

@@ -35,6 +35,7 @@ struct WArgs {
   const IdT* indices;
   const float* probs;
   const IdT* cols;
+  int64_t num_cols;
   int64_t S;
   int k;
   uint64_t seed;
@@ -144,6 +145,8 @@ __global__ void weighted_rows_kernel(WArgs<IdT> a) {
   const int64_t r = static_cast<int64_t>(blockIdx.x) * waves + wave;
   if (r >= a.S) return;
   const int64_t c = a.cols ? static_cast<int64_t>(a.cols[r]) : r;
+  // an id outside [0, num_cols) is an empty column
+  if (static_cast<uint64_t>(c) >= static_cast<uint64_t>(a.num_cols)) return;
   const int64_t start = a.indptr[c];
   const int64_t deg = a.indptr[c + 1] - start;
   const int64_t out_start = a.sub_indptr[r];
@@ -273,8 +276,8 @@ int weighted_launch(const WArgs<IdT>& a, hipStream_t st) {
 }
 
 template <typename IdT>
-int weighted_impl(const int64_t* indptr, const void* indices, const float* probs, const void* cols,
-                  int64_t S, int64_t k, uint64_t seed, const uint32_t* replay,
+int weighted_impl(const int64_t* indptr, int64_t num_cols, const void* indices, const float* probs,
+                  const void* cols, int64_t S, int64_t k, uint64_t seed, const uint32_t* replay,
                   const int64_t* replay_ptr, const int64_t* sub_indptr, void* sub_indices,
                   int64_t* select_index, void* coo_col, void* workspace, size_t workspace_bytes,
                   hipStream_t st) {
@@ -284,6 +287,7 @@ int weighted_impl(const int64_t* indptr, const void* indices, const float* probs
   a.indices = static_cast<const IdT*>(indices);
   a.probs = probs;
   a.cols = static_cast<const IdT*>(cols);
+  a.num_cols = num_cols;
   a.S = S;
   a.k = static_cast<int>(k);
   a.seed = seed;
@@ -321,13 +325,16 @@ size_t gs_sample_weighted_workspace_bytes(int64_t S, int64_t fanout) {
          padded(cap * static_cast<size_t>(fanout) * 8);
 }
 
-int gs_sample_weighted_fill(const int64_t* indptr, const void* indices, const float* probs,
-                            const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+int gs_sample_weighted_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
+                            const float* probs, const void* column_ids, int id_bytes, int64_t S,
+                            int64_t fanout,
                             uint64_t seed, const uint32_t* replay, const int64_t* replay_ptr,
                             const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                             void* coo_col, void* workspace, size_t workspace_bytes, void* stream) {
-  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0,
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0 && num_cols >= 0,
              "gs_sample_weighted_fill: null pointer or negative size");
+  GS_REQUIRE(column_ids || S <= num_cols,
+             "gs_sample_weighted_fill: S exceeds num_cols without column_ids");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sample_weighted_fill: id_bytes must be 4 or 8, got %d",
              id_bytes);
   GS_REQUIRE((replay == nullptr) == (replay_ptr == nullptr),
@@ -343,10 +350,10 @@ int gs_sample_weighted_fill(const int64_t* indptr, const void* indices, const fl
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   return id_bytes == 8
-             ? weighted_impl<int64_t>(indptr, indices, probs, column_ids, S, fanout, seed, replay,
+             ? weighted_impl<int64_t>(indptr, num_cols, indices, probs, column_ids, S, fanout, seed, replay,
                                       replay_ptr, sub_indptr, sub_indices, select_index, coo_col,
                                       workspace, workspace_bytes, st)
-             : weighted_impl<int32_t>(indptr, indices, probs, column_ids, S, fanout, seed, replay,
+             : weighted_impl<int32_t>(indptr, num_cols, indices, probs, column_ids, S, fanout, seed, replay,
                                       replay_ptr, sub_indptr, sub_indices, select_index, coo_col,
                                       workspace, workspace_bytes, st);
 }

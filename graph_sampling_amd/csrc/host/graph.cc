@@ -1,0 +1,506 @@
+#include "graph.h"
+
+#include "bcast.h"
+#include "graph_ops.h"
+#include "hip_ops.h"
+
+namespace gs {
+
+namespace {
+
+const char* kNoDoublyCompressed =
+    "doubly-compressed formats (_DCSC / _DCSR) are not part of this build";
+
+bool IsCscLike(int64_t format) { return format == _CSC; }
+bool IsCsrLike(int64_t format) { return format == _CSR; }
+
+void RejectCompressed(int64_t format) {
+  TORCH_CHECK(format != _DCSC && format != _DCSR, kNoDoublyCompressed);
+}
+
+torch::Tensor Pick(const torch::optional<torch::Tensor>& ids, const torch::Tensor& local) {
+  return ids.has_value() ? ids.value().index({local}) : local;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ loading
+void Graph::LoadCSC(torch::Tensor indptr, torch::Tensor indices) {
+  csc_ = std::make_shared<CSC>(CSC{indptr, indices, torch::nullopt});
+  num_cols_ = num_rows_ = indptr.numel() - 1;
+  num_edges_ = indices.numel();
+}
+
+void Graph::LoadCSR(torch::Tensor indptr, torch::Tensor indices) {
+  csr_ = std::make_shared<CSR>(CSR{indptr, indices, torch::nullopt});
+  num_cols_ = num_rows_ = indptr.numel() - 1;
+  num_edges_ = indices.numel();
+}
+
+// node count = the larger number of distinct endpoints (reference src/graph.cc:25-35)
+void Graph::LoadCOO(torch::Tensor row, torch::Tensor col) {
+  coo_ = std::make_shared<COO>(COO{row, col, torch::nullopt, false, false});
+  const int64_t nr = std::get<0>(torch::_unique(row)).numel();
+  const int64_t nc = std::get<0>(torch::_unique(col)).numel();
+  num_cols_ = num_rows_ = std::max(nr, nc);
+  num_edges_ = row.numel();
+}
+
+void Graph::LoadCSCWithColIds(torch::Tensor column_ids, torch::Tensor indptr,
+                              torch::Tensor indices) {
+  TORCH_CHECK(column_ids.numel() == indptr.numel() - 1,
+              "length of column_ids is not aligned with indptr");
+  csc_ = std::make_shared<CSC>(CSC{indptr, indices, torch::nullopt});
+  col_ids_ = column_ids;
+  num_cols_ = column_ids.numel();
+  num_rows_ = indices.numel() ? indices.max().item<int64_t>() + 1 : 0;
+  num_edges_ = indices.numel();
+}
+
+void Graph::SetMetaData(torch::optional<torch::Tensor> col_ids,
+                        torch::optional<torch::Tensor> row_ids, int64_t num_cols,
+                        int64_t num_rows) {
+  col_ids_ = col_ids;
+  row_ids_ = row_ids;
+  num_cols_ = num_cols;
+  num_rows_ = num_rows;
+}
+
+void Graph::SetCOOByTensor(torch::Tensor row, torch::Tensor col,
+                           torch::optional<torch::Tensor> e_ids, bool row_sorted, bool col_sorted) {
+  coo_ = std::make_shared<COO>(COO{row, col, e_ids, row_sorted, col_sorted});
+}
+
+torch::TensorOptions Graph::IdOptions() const {
+  if (csc_) return csc_->indices.options();
+  if (csr_) return csr_->indices.options();
+  TORCH_CHECK(coo_ != nullptr, "the graph holds no sparse format");
+  return coo_->row.options();
+}
+
+torch::Tensor Graph::DataOrOnes() {
+  if (data_.has_value()) return data_.value();
+  return torch::ones({num_edges_}, IdOptions().dtype(torch::kFloat32));
+}
+
+// edge data in the order of a format ("col": CSC order, "row": CSR order)
+torch::optional<torch::Tensor> Graph::GetData(std::string order) {
+  torch::Tensor data = DataOrOnes();
+  if (order == "col") {
+    CreateSparseFormat(_CSC);
+    if (csc_->e_ids.has_value()) return data.index({csc_->e_ids.value()});
+  } else if (order == "row") {
+    CreateSparseFormat(_CSR);
+    if (csr_->e_ids.has_value()) return data.index({csr_->e_ids.value()});
+  }
+  return data;
+}
+
+// ------------------------------------------------------------ format caches
+void Graph::CSC2CSR() {
+  SetCOO(GraphCSC2COO(csc_, true));
+  SetCSR(GraphCOO2CSC(coo_, num_rows_, false));
+}
+
+void Graph::CSR2CSC() {
+  SetCOO(GraphCSC2COO(csr_, false));
+  SetCSC(GraphCOO2CSC(coo_, num_cols_, true));
+}
+
+void Graph::CreateSparseFormat(int64_t format) {
+  RejectCompressed(format);
+  if (format == _COO) {
+    if (coo_) return;
+    if (csc_)
+      SetCOO(GraphCSC2COO(csc_, true));
+    else
+      SetCOO(GraphCSC2COO(csr_, false));
+  } else if (format == _CSC) {
+    if (csc_) return;
+    if (coo_)
+      SetCSC(GraphCOO2CSC(coo_, num_cols_, true));
+    else
+      CSR2CSC();
+  } else if (format == _CSR) {
+    if (csr_) return;
+    if (coo_)
+      SetCSR(GraphCOO2CSC(coo_, num_rows_, false));
+    else
+      CSC2CSR();
+  } else {
+    TORCH_CHECK(false, "unknown sparse format flag ", format);
+  }
+}
+
+std::vector<torch::Tensor> Graph::GetCSCTensor() {
+  CreateSparseFormat(_CSC);
+  return {csc_->indptr, csc_->indices, csc_->e_ids.value_or(torch::Tensor())};
+}
+
+std::vector<torch::Tensor> Graph::GetCOOTensor() {
+  CreateSparseFormat(_COO);
+  TORCH_CHECK(coo_->col_sorted, "GetCOOTensor expects a column-sorted COO");
+  return {coo_->row, coo_->col, coo_->e_ids.value_or(torch::Tensor())};
+}
+
+// ------------------------------------------------------------------ helpers
+c10::intrusive_ptr<Graph> Graph::Child(torch::optional<torch::Tensor> col_ids,
+                                       torch::optional<torch::Tensor> row_ids, int64_t num_cols,
+                                       int64_t num_rows) const {
+  return c10::make_intrusive<Graph>(true, col_ids, row_ids, num_cols, num_rows);
+}
+
+// edge data follows the edges: data[e_ids[select_index]] (reference src/graph.cc:295-308)
+void Graph::InheritData(Graph* child, const torch::optional<torch::Tensor>& e_ids,
+                        const torch::Tensor& select_index) const {
+  if (!data_.has_value()) return;
+  torch::Tensor where = e_ids.has_value() ? e_ids.value().index({select_index}) : select_index;
+  child->SetData(data_.value().index({where}));
+}
+
+// a graph with the same structure (shared format caches) and new edge data
+c10::intrusive_ptr<Graph> Graph::SameShape(torch::Tensor data) {
+  auto g = c10::make_intrusive<Graph>(is_subgraph_, col_ids_, row_ids_, num_cols_, num_rows_);
+  g->SetCSC(csc_);
+  g->SetCSR(csr_);
+  g->SetCOO(coo_);
+  g->SetNumEdges(num_edges_);
+  g->SetData(data);
+  return g;
+}
+
+// ------------------------------------------------------------------ slicing
+c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int64_t on_format,
+                                         int64_t output_format, bool relabel) {
+  TORCH_CHECK(axis == 0 || axis == 1, "axis must be 0 (columns) or 1 (rows)");
+  RejectCompressed(on_format);
+  CreateSparseFormat(on_format);
+  const bool with_coo = output_format & _COO;
+
+  torch::optional<torch::Tensor> col_ids = col_ids_, row_ids = row_ids_;
+  int64_t num_cols = num_cols_, num_rows = num_rows_;
+  if (axis == 0) {
+    col_ids = Pick(col_ids_, n_ids);
+    num_cols = n_ids.numel();
+  } else {
+    row_ids = Pick(row_ids_, n_ids);
+    num_rows = n_ids.numel();
+  }
+
+  std::shared_ptr<CSC> out_csc;
+  std::shared_ptr<CSR> out_csr;
+  std::shared_ptr<COO> out_coo;
+  torch::Tensor select_index;
+  torch::optional<torch::Tensor> e_ids;
+  int64_t num_edges = 0;
+
+  if (on_format == _COO) {
+    std::tie(out_coo, select_index) = COOColSlicing(coo_, n_ids, axis);
+    num_edges = out_coo->row.numel();
+    e_ids = coo_->e_ids;
+  } else {
+    // CSC and CSR are the same storage with the roles of rows and columns
+    // swapped: "along" is the axis the offsets run over.
+    const bool on_csc = IsCscLike(on_format);
+    TORCH_CHECK(on_csc || IsCsrLike(on_format), "unknown sparse format flag ", on_format);
+    TORCH_CHECK(output_format != (on_csc ? _CSR : _CSC),
+                "Error in Slicing, Not implementation [on_format = ", on_csc ? "CSC" : "CSR",
+                ", output_format = ", on_csc ? "CSR" : "CSC", "]");
+    std::shared_ptr<CSC> fmt = on_csc ? csc_ : csr_;
+    const bool along = (axis == 0) == on_csc;
+    std::shared_ptr<_TMP> tmp;
+    if (along) {
+      std::tie(tmp, select_index) = CSCColSlicing(fmt, n_ids, with_coo);
+      if (relabel) {
+        // the other side is renumbered by first occurrence (reference src/graph.cc:219-227)
+        torch::Tensor frontier;
+        std::vector<torch::Tensor> renamed;
+        std::tie(frontier, renamed) =
+            BatchTensorRelabel({tmp->coo_in_indices}, {tmp->coo_in_indices});
+        tmp->coo_in_indices = renamed[0];
+        if (on_csc) {
+          row_ids = frontier;
+          num_rows = frontier.numel();
+        } else {
+          col_ids = frontier;
+          num_cols = frontier.numel();
+        }
+      }
+    } else {
+      TORCH_CHECK(!relabel, "Not implemented warning");
+      std::tie(tmp, select_index) = CSCRowSlicing(fmt, n_ids, with_coo);
+    }
+    if (output_format & (on_csc ? _CSC : _CSR)) {
+      auto compressed =
+          std::make_shared<CSC>(CSC{tmp->indptr, tmp->coo_in_indices, torch::nullopt});
+      (on_csc ? out_csc : out_csr) = compressed;
+    }
+    if (with_coo) {
+      out_coo = on_csc ? std::make_shared<COO>(COO{tmp->coo_in_indices, tmp->coo_in_indptr,
+                                                   torch::nullopt, false, true})
+                       : std::make_shared<COO>(COO{tmp->coo_in_indptr, tmp->coo_in_indices,
+                                                   torch::nullopt, true, false});
+    }
+    num_edges = tmp->coo_in_indices.numel();
+    e_ids = fmt->e_ids;
+  }
+
+  auto ret = Child(col_ids, row_ids, num_cols, num_rows);
+  ret->SetNumEdges(num_edges);
+  ret->SetCOO(out_coo);
+  ret->SetCSC(out_csc);
+  ret->SetCSR(out_csr);
+  InheritData(ret.get(), e_ids, select_index);
+  return ret;
+}
+
+// ----------------------------------------------------------------- sampling
+c10::intrusive_ptr<Graph> Graph::SampleImpl(int64_t axis, const torch::Tensor* edge_probs,
+                                            int64_t fanout, bool replace, int64_t on_format,
+                                            int64_t output_format) {
+  RejectCompressed(on_format);
+  CreateSparseFormat(on_format);
+  const bool on_csc = (axis == 0 && on_format == _CSC);
+  const bool on_csr = (axis == 1 && on_format == _CSR);
+  TORCH_CHECK(on_csc || on_csr, "No implementation!");  // reference src/graph.cc:456
+  TORCH_CHECK(output_format != (on_csc ? _CSR : _CSC),
+              "Error in Sampling, Not implementation [on_format = ", on_csc ? "CSC" : "CSR",
+              ", output_format = ", on_csc ? "CSR" : "CSC", "]");
+  const bool with_coo = output_format & _COO;
+  std::shared_ptr<CSC> fmt = on_csc ? csc_ : csr_;
+  std::shared_ptr<_TMP> tmp;
+  torch::Tensor select_index;
+  if (edge_probs)
+    std::tie(tmp, select_index) = CSCColSamplingProbs(fmt, *edge_probs, fanout, replace, with_coo);
+  else
+    std::tie(tmp, select_index) = CSCColSampling(fmt, fanout, replace, with_coo);
+
+  auto ret = Child(col_ids_, row_ids_, num_cols_, num_rows_);
+  if (output_format & (on_csc ? _CSC : _CSR)) {
+    auto compressed = std::make_shared<CSC>(CSC{tmp->indptr, tmp->coo_in_indices, torch::nullopt});
+    if (on_csc) ret->SetCSC(compressed); else ret->SetCSR(compressed);
+  }
+  if (with_coo) {
+    ret->SetCOO(on_csc ? std::make_shared<COO>(COO{tmp->coo_in_indices, tmp->coo_in_indptr,
+                                                   torch::nullopt, false, true})
+                       : std::make_shared<COO>(COO{tmp->coo_in_indptr, tmp->coo_in_indices,
+                                                   torch::nullopt, true, false}));
+  }
+  ret->SetNumEdges(tmp->coo_in_indices.numel());
+  InheritData(ret.get(), fmt->e_ids, select_index);
+  return ret;
+}
+
+c10::intrusive_ptr<Graph> Graph::Sampling(int64_t axis, int64_t fanout, bool replace,
+                                          int64_t on_format, int64_t output_format) {
+  return SampleImpl(axis, nullptr, fanout, replace, on_format, output_format);
+}
+
+c10::intrusive_ptr<Graph> Graph::SamplingProbs(int64_t axis, torch::Tensor edge_probs,
+                                               int64_t fanout, bool replace, int64_t on_format,
+                                               int64_t output_format) {
+  return SampleImpl(axis, &edge_probs, fanout, replace, on_format, output_format);
+}
+
+// slice + sample without materialising the slice; the result holds a CSC only
+// and the kernel is given the LOCAL column index (reference src/graph.cc:531-559)
+c10::intrusive_ptr<Graph> Graph::ColumnwiseFusedSlicingAndSampling(torch::Tensor column_index,
+                                                                   int64_t fanout, bool replace) {
+  TORCH_CHECK(csc_ != nullptr, "fused slicing + sampling needs the CSC format");
+  torch::Tensor col_ids = Pick(col_ids_, column_index);
+  auto ret = Child(col_ids, row_ids_, col_ids.numel(), num_rows_);
+  std::shared_ptr<CSC> sampled;
+  torch::Tensor select_index;
+  std::tie(sampled, select_index) = FusedCSCColSlicingAndSampling(csc_, column_index, fanout, replace);
+  ret->SetCSC(sampled);
+  ret->SetNumEdges(sampled->indices.numel());
+  InheritData(ret.get(), csc_->e_ids, select_index);
+  return ret;
+}
+
+torch::Tensor Graph::RandomWalk(torch::Tensor seeds, int64_t walk_length) {
+  TORCH_CHECK(csc_ != nullptr, "random walks need the CSC format");
+  return FusedRandomWalk(csc_, seeds, walk_length);
+}
+
+// --------------------------------------------------------- edge-data operators
+torch::Tensor Graph::Sum(int64_t axis, int64_t powk, int64_t on_format) {
+  RejectCompressed(on_format);
+  CreateSparseFormat(on_format);
+  torch::Tensor data = DataOrOnes();
+  // one entry per column (axis 0) / row (axis 1) OF THIS GRAPH OBJECT, so a
+  // column slice summed along axis 1 yields a vector over all original rows
+  torch::Tensor out = torch::zeros({axis == 0 ? num_cols_ : num_rows_}, data.options());
+  if (on_format == _COO)
+    COOGraphSum(coo_, data, out, powk, 1 - axis);
+  else if (axis == 0 && on_format == _CSC)
+    CSCGraphSum(csc_, torch::nullopt, data, out, powk);
+  else if (axis == 1 && on_format == _CSR)
+    CSCGraphSum(csr_, torch::nullopt, data, out, powk);
+  else
+    TORCH_CHECK(false, "axis should be 0 or 1? on_format and axis do not match?");
+  return out;
+}
+
+c10::intrusive_ptr<Graph> Graph::Normalize(int64_t axis, int64_t on_format) {
+  RejectCompressed(on_format);
+  CreateSparseFormat(on_format);
+  torch::Tensor data = DataOrOnes();
+  torch::Tensor out = torch::empty_like(data);
+  if (axis == 0 && on_format == _CSC)
+    hip::SegmentNormalize(csc_->indptr, csc_->e_ids, data, out);
+  else if (axis == 1 && on_format == _CSR)
+    hip::SegmentNormalize(csr_->indptr, csr_->e_ids, data, out);
+  else
+    TORCH_CHECK(false, "Not Implementation Error");
+  return SameShape(out);
+}
+
+c10::intrusive_ptr<Graph> Graph::Divide(torch::Tensor divisor, int64_t axis, int64_t on_format) {
+  RejectCompressed(on_format);
+  CreateSparseFormat(on_format);
+  torch::Tensor data = DataOrOnes();
+  torch::Tensor out = torch::zeros({num_edges_}, data.options());
+  if (on_format == _COO)
+    COOGraphDiv(coo_, data, divisor, out, 1 - axis);
+  else if (axis == 0 && on_format == _CSC)
+    CSCGraphDiv(csc_, torch::nullopt, data, divisor, out);
+  else if (axis == 1 && on_format == _CSR)
+    CSCGraphDiv(csr_, torch::nullopt, data, divisor, out);
+  return SameShape(out);
+}
+
+std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> Graph::EDivUSum(torch::Tensor divisor) {
+  CreateSparseFormat(_COO);
+  torch::Tensor data = DataOrOnes();
+  torch::Tensor out = torch::zeros({num_edges_}, data.options());
+  torch::Tensor sum = torch::zeros({num_cols_}, data.options());
+  hip::EDivUSum(coo_->row, coo_->col, data, divisor, out, sum);
+  return {SameShape(out), sum};
+}
+
+// targets: 0 = source (row id), 1 = edge, 2 = destination (column id); on the
+// CSR the compressed axis is the row, so 0 and 2 swap (reference src/graph.cc:975-976)
+void Graph::SDDMM(const std::string& op, torch::Tensor lhs, torch::Tensor rhs, torch::Tensor out,
+                  int64_t lhs_target, int64_t rhs_target, int64_t on_format) {
+  RejectCompressed(on_format);
+  CreateSparseFormat(on_format);
+  const hip::Bcast b = ToDevice(CalcBcastOff(op, lhs, rhs), out);
+  if (on_format == _COO) {
+    hip::SddmmCoo(op, b, coo_->row, coo_->col, coo_->e_ids, lhs, rhs, out,
+                  static_cast<int>(lhs_target), static_cast<int>(rhs_target));
+  } else if (on_format == _CSR) {
+    const int lt = lhs_target == 1 ? 1 : static_cast<int>(2 - lhs_target);
+    const int rt = rhs_target == 1 ? 1 : static_cast<int>(2 - rhs_target);
+    hip::SddmmCsc(op, b, csr_->indptr, csr_->indices, csr_->e_ids, torch::nullopt, lhs, rhs, out, lt, rt);
+  } else if (on_format == _CSC) {
+    hip::SddmmCsc(op, b, csc_->indptr, csc_->indices, csc_->e_ids, torch::nullopt, lhs, rhs, out,
+                  static_cast<int>(lhs_target), static_cast<int>(rhs_target));
+  } else {
+    TORCH_CHECK(false, "SDDMM only supports CSR and COO formats");
+  }
+}
+
+// ---------------------------------------------------------------- node queries
+torch::Tensor Graph::AllValidNode() {
+  TORCH_CHECK(col_ids_.has_value(), "For sampling, col_ids_ is necessary!");
+  torch::Tensor rows;
+  if (row_ids_.has_value()) {
+    rows = row_ids_.value();
+  } else if (csc_) {
+    rows = csc_->indices;
+  } else {
+    if (!coo_) SetCOO(GraphCSC2COO(csr_, false));
+    rows = coo_->row;
+  }
+  return hip::Unique(torch::cat({col_ids_.value(), rows}));
+}
+
+std::tuple<torch::Tensor, int64_t, int64_t, torch::Tensor, torch::Tensor,
+           torch::optional<torch::Tensor>, std::string>
+Graph::Relabel() {
+  TORCH_CHECK(col_ids_.has_value(), "For sampling, col_ids_ is necessary!");
+  torch::Tensor col_ids = col_ids_.value();
+  torch::Tensor frontier;
+  std::vector<torch::Tensor> renamed;
+  if (csc_) {
+    // seeds first: the frontier starts with the column ids (reference src/graph.cc:789-811)
+    torch::Tensor rows = Pick(row_ids_, csc_->indices);
+    std::tie(frontier, renamed) = BatchTensorRelabel({col_ids, rows}, {rows});
+    return {frontier, frontier.numel(), col_ids.numel(), csc_->indptr.clone(), renamed[0],
+            csc_->e_ids, "csc"};
+  }
+  TORCH_CHECK(csr_ || coo_, "Error in Relabel!");
+  if (!coo_) SetCOO(GraphCSC2COO(csr_, false));
+  torch::Tensor coo_col = col_ids.index({coo_->col});
+  torch::Tensor coo_row = Pick(row_ids_, coo_->row);
+  std::tie(frontier, renamed) = BatchTensorRelabel({col_ids, coo_row}, {coo_col, coo_row});
+  return {frontier, frontier.numel(), col_ids.numel(), renamed[1], renamed[0], coo_->e_ids, "coo"};
+}
+
+torch::Tensor Graph::GetRows() {
+  return row_ids_.has_value() ? row_ids_.value() : torch::arange(num_rows_, IdOptions());
+}
+
+torch::Tensor Graph::GetCols() {
+  return col_ids_.has_value() ? col_ids_.value() : torch::arange(num_cols_, IdOptions());
+}
+
+torch::Tensor Graph::GetValidRows() {
+  return Pick(row_ids_, std::get<0>(torch::_unique(GetCOORows(false))));
+}
+
+torch::Tensor Graph::GetValidCols() {
+  return Pick(col_ids_, std::get<0>(torch::_unique(GetCOOCols(false))));
+}
+
+torch::Tensor Graph::GetCOORows(bool is_original) {
+  torch::Tensor rows;
+  if (coo_) {
+    rows = coo_->row;
+  } else if (csc_ && !csc_->e_ids.has_value()) {
+    rows = csc_->indices;
+  } else {
+    TORCH_CHECK(csr_ && !csr_->e_ids.has_value(), "Error in GetCOORows!");
+    SetCOO(GraphCSC2COO(csr_, false));
+    rows = coo_->row;
+  }
+  return is_original ? Pick(row_ids_, rows) : rows;
+}
+
+torch::Tensor Graph::GetCOOCols(bool is_original) {
+  torch::Tensor cols;
+  if (coo_) {
+    cols = coo_->col;
+  } else if (csc_ && !csc_->e_ids.has_value()) {
+    SetCOO(GraphCSC2COO(csc_, true));
+    cols = coo_->col;
+  } else {
+    TORCH_CHECK(csr_ && !csr_->e_ids.has_value(), "Error in GetCOOCols!");
+    cols = csr_->indices;
+  }
+  return is_original ? Pick(col_ids_, cols) : cols;
+}
+
+std::vector<torch::Tensor> Graph::MetaData() {
+  torch::Tensor col_ids = col_ids_.value_or(torch::Tensor());
+  torch::Tensor row_ids = row_ids_.value_or(torch::Tensor());
+  if (csc_) return {col_ids, row_ids, DataOrOnes(), csc_->indptr, csc_->indices};
+  if (csr_) return {col_ids, row_ids, DataOrOnes(), csr_->indptr, csr_->indices};
+  TORCH_CHECK(coo_ != nullptr, "the graph holds no sparse format");
+  return {coo_->row, coo_->col};
+}
+
+std::vector<torch::Tensor> Graph::COOMetaData() {
+  if (!coo_) return {};
+  return {col_ids_.value_or(torch::Tensor()), row_ids_.value_or(torch::Tensor()),
+          data_.value_or(torch::Tensor()), coo_->row, coo_->col};
+}
+
+std::vector<torch::Tensor> Graph::CSCMetaData() {
+  if (!csc_) return {};
+  return {col_ids_.value_or(torch::Tensor()), row_ids_.value_or(torch::Tensor()),
+          data_.value_or(torch::Tensor()), csc_->indptr, csc_->indices};
+}
+
+}  // namespace gs

@@ -1,0 +1,128 @@
+// gs::Graph -- the sparse-matrix object behind torch.classes.gs_classes.Graph.
+//
+// Public API (names, signatures, return orders) follows the reference's
+// src/graph.h:11-128 for everything on the sampling hot path: loading, format
+// caches, slicing, uniform / weighted / fused sampling, relabel, valid-node
+// queries, walks, Sum / Normalize / Divide / EDivUSum and SDDMM.  The batched
+// ("super-batch") methods, FusedBidirSlicing and the doubly-compressed formats
+// are not part of this build and raise a clear error when requested.
+//
+// A Graph keeps up to three cached formats of one matrix (CSC, CSR, COO), the
+// edge data, and the global ids of its local columns / rows.  Children share
+// storage with their parents; CreateSparseFormat fills caches lazily, so a
+// Graph must not be used from two threads at once (same as the reference).
+#pragma once
+
+#include <torch/custom_class.h>
+#include <torch/script.h>
+
+#include <memory>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "graph_storage.h"
+
+namespace gs {
+
+class Graph : public torch::CustomClassHolder {
+ public:
+  explicit Graph(bool is_subgraph) : is_subgraph_(is_subgraph) {}
+  Graph(bool is_subgraph, torch::optional<torch::Tensor> col_ids,
+        torch::optional<torch::Tensor> row_ids, int64_t num_cols, int64_t num_rows)
+      : is_subgraph_(is_subgraph),
+        num_cols_(num_cols),
+        num_rows_(num_rows),
+        col_ids_(col_ids),
+        row_ids_(row_ids) {}
+
+  // ---- loading and raw accessors
+  void LoadCSC(torch::Tensor indptr, torch::Tensor indices);
+  void LoadCOO(torch::Tensor row, torch::Tensor col);
+  void LoadCSR(torch::Tensor indptr, torch::Tensor indices);
+  void LoadCSCWithColIds(torch::Tensor column_ids, torch::Tensor indptr, torch::Tensor indices);
+  void SetMetaData(torch::optional<torch::Tensor> col_ids, torch::optional<torch::Tensor> row_ids,
+                   int64_t num_cols, int64_t num_rows);
+  void SetCSC(std::shared_ptr<CSC> csc) { csc_ = csc; }
+  void SetCSR(std::shared_ptr<CSR> csr) { csr_ = csr; }
+  void SetCOO(std::shared_ptr<COO> coo) { coo_ = coo; }
+  void SetCOOByTensor(torch::Tensor row, torch::Tensor col, torch::optional<torch::Tensor> e_ids,
+                      bool row_sorted, bool col_sorted);
+  void SetData(torch::Tensor data) { data_ = data; }
+  void SetNumEdges(int64_t num_edges) { num_edges_ = num_edges; }
+  std::shared_ptr<CSC> GetCSC() { return csc_; }
+  std::shared_ptr<CSR> GetCSR() { return csr_; }
+  std::shared_ptr<COO> GetCOO() { return coo_; }
+  std::vector<torch::Tensor> GetCSCTensor();
+  std::vector<torch::Tensor> GetCOOTensor();
+  torch::optional<torch::Tensor> GetData(std::string order = "default");
+  int64_t GetNumRows() { return num_rows_; }
+  int64_t GetNumCols() { return num_cols_; }
+  int64_t GetNumEdges() { return num_edges_; }
+
+  // ---- format caches
+  void CSC2CSR();
+  void CSR2CSC();
+  void CreateSparseFormat(int64_t format);
+
+  // ---- structure operators (axis 0: columns, axis 1: rows)
+  c10::intrusive_ptr<Graph> Slicing(torch::Tensor n_ids, int64_t axis, int64_t on_format,
+                                    int64_t output_format, bool relabel = false);
+  c10::intrusive_ptr<Graph> Sampling(int64_t axis, int64_t fanout, bool replace, int64_t on_format,
+                                     int64_t output_format);
+  c10::intrusive_ptr<Graph> SamplingProbs(int64_t axis, torch::Tensor edge_probs, int64_t fanout,
+                                          bool replace, int64_t on_format, int64_t output_format);
+  c10::intrusive_ptr<Graph> ColumnwiseFusedSlicingAndSampling(torch::Tensor column_index,
+                                                              int64_t fanout, bool replace);
+  torch::Tensor RandomWalk(torch::Tensor seeds, int64_t walk_length);
+
+  // ---- edge-data operators
+  torch::Tensor Sum(int64_t axis, int64_t powk, int64_t on_format);
+  c10::intrusive_ptr<Graph> Normalize(int64_t axis, int64_t on_format);
+  c10::intrusive_ptr<Graph> Divide(torch::Tensor divisor, int64_t axis, int64_t on_format);
+  std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> EDivUSum(torch::Tensor divisor);
+  void SDDMM(const std::string& op, torch::Tensor lhs, torch::Tensor rhs, torch::Tensor out,
+             int64_t lhs_target, int64_t rhs_target, int64_t on_format);
+
+  // ---- node queries; a "valid" node is a requested column or a non-isolated row
+  torch::Tensor AllValidNode();
+  torch::Tensor GetRows();
+  torch::Tensor GetCols();
+  torch::Tensor GetValidRows();
+  torch::Tensor GetValidCols();
+  torch::Tensor GetCOORows(bool is_original);  // global ids when is_original, else local
+  torch::Tensor GetCOOCols(bool is_original);
+  // (frontier, #frontier, #columns, offsets-or-row, indices-or-col, e_ids, "csc" | "coo")
+  std::tuple<torch::Tensor, int64_t, int64_t, torch::Tensor, torch::Tensor,
+             torch::optional<torch::Tensor>, std::string>
+  Relabel();
+  std::vector<torch::Tensor> MetaData();
+  std::vector<torch::Tensor> COOMetaData();
+  std::vector<torch::Tensor> CSCMetaData();
+
+ private:
+  c10::intrusive_ptr<Graph> Child(torch::optional<torch::Tensor> col_ids,
+                                  torch::optional<torch::Tensor> row_ids, int64_t num_cols,
+                                  int64_t num_rows) const;
+  c10::intrusive_ptr<Graph> SameShape(torch::Tensor data);
+  torch::Tensor DataOrOnes();
+  torch::TensorOptions IdOptions() const;
+  void InheritData(Graph* child, const torch::optional<torch::Tensor>& e_ids,
+                   const torch::Tensor& select_index) const;
+  c10::intrusive_ptr<Graph> SampleImpl(int64_t axis, const torch::Tensor* edge_probs,
+                                       int64_t fanout, bool replace, int64_t on_format,
+                                       int64_t output_format);
+
+  bool is_subgraph_ = false;
+  int64_t num_cols_ = 0;
+  int64_t num_rows_ = 0;
+  int64_t num_edges_ = 0;
+  std::shared_ptr<CSC> csc_;
+  std::shared_ptr<CSR> csr_;
+  std::shared_ptr<COO> coo_;
+  torch::optional<torch::Tensor> data_;
+  torch::optional<torch::Tensor> col_ids_;  // global id of each local column
+  torch::optional<torch::Tensor> row_ids_;  // global id of each local row
+};
+
+}  // namespace gs

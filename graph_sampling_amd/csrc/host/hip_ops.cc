@@ -1,0 +1,472 @@
+#include "hip_ops.h"
+
+#include <c10/hip/HIPStream.h>
+
+#include <atomic>
+
+#include "gs_hip.h"
+
+namespace gs {
+namespace hip {
+namespace {
+
+std::atomic<uint64_t> g_seed{7777};
+std::atomic<int64_t> g_algo{GS_SAMPLE_AUTO};
+
+void Check(int status, const char* what) {
+  TORCH_CHECK(status == GS_OK, what, " failed (", status, "): ", gs_status_string(status));
+}
+
+void* Stream(const torch::Tensor& t) {
+  return static_cast<void*>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+}
+
+// Device tensors only: the reference has no CPU path either and aborts with
+// "Not implemented warning" (src/graph_ops.cc:27); here that is an exception.
+void NeedDevice(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.defined(), name, " is undefined");
+  TORCH_CHECK(t.is_cuda(), "Not implemented warning: ", name, " must be a GPU tensor");
+  TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+}
+
+int IdBytes(const torch::Tensor& t, const char* name) {
+  NeedDevice(t, name);
+  if (t.scalar_type() == torch::kInt64) return 8;
+  if (t.scalar_type() == torch::kInt32) return 4;
+  TORCH_CHECK(false, name, " must be int64 (or int32), got ", t.scalar_type());
+}
+
+void NeedI64(const torch::Tensor& t, const char* name) {
+  NeedDevice(t, name);
+  TORCH_CHECK(t.scalar_type() == torch::kInt64, name, " must be int64, got ", t.scalar_type());
+}
+
+void NeedF32(const torch::Tensor& t, const char* name) {
+  NeedDevice(t, name);
+  TORCH_CHECK(t.scalar_type() == torch::kFloat32, name, " must be float32, got ", t.scalar_type());
+}
+
+const int64_t* OptI64(const torch::optional<torch::Tensor>& t, const char* name) {
+  if (!t.has_value() || !t.value().defined()) return nullptr;
+  NeedI64(t.value(), name);
+  return t.value().data_ptr<int64_t>();
+}
+
+torch::Tensor Scratch(size_t bytes, const torch::Tensor& like) {
+  return torch::empty({static_cast<int64_t>(bytes < 256 ? 256 : bytes)},
+                      torch::dtype(torch::kUInt8).device(like.device()));
+}
+
+torch::TensorOptions I64(const torch::Tensor& like) {
+  return torch::dtype(torch::kInt64).device(like.device());
+}
+
+int OpCode(const std::string& op) {
+  if (op == "add") return GS_OP_ADD;
+  if (op == "sub") return GS_OP_SUB;
+  if (op == "mul") return GS_OP_MUL;
+  if (op == "div") return GS_OP_DIV;
+  if (op == "copy_lhs") return GS_OP_COPY_LHS;
+  if (op == "copy_rhs") return GS_OP_COPY_RHS;
+  if (op == "dot") return GS_OP_DOT;
+  TORCH_CHECK(false, "Unsupported SpMM/SDDMM binary operator: ", op);
+}
+
+}  // namespace
+
+void SetSeed(uint64_t seed) { g_seed.store(seed); }
+uint64_t NextSeed() { return g_seed.fetch_add(1); }
+void SetSampleAlgo(int64_t algo) {
+  TORCH_CHECK(algo == GS_SAMPLE_AUTO || algo == GS_SAMPLE_RESERVOIR, "unknown sampling algorithm ", algo);
+  g_algo.store(algo);
+}
+
+SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
+                       const torch::Tensor& column_ids, bool with_coo) {
+  NeedI64(indptr, "indptr");
+  const int idb = IdBytes(indices, "indices");
+  TORCH_CHECK(IdBytes(column_ids, "column ids") == idb, "column ids and indices differ in dtype");
+  const int64_t S = column_ids.numel();
+  auto sub_indptr = torch::empty({S + 1}, I64(indptr));
+  auto ws = Scratch(gs_slice_workspace_bytes(S), indptr);
+  void* st = Stream(indptr);
+  Check(gs_slice_count(indptr.data_ptr<int64_t>(), indptr.numel() - 1, column_ids.data_ptr(), idb, S,
+                       sub_indptr.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
+        "gs_slice_count");
+  const int64_t nnz = sub_indptr[S].item<int64_t>();
+  auto sub_indices = torch::empty({nnz}, indices.options());
+  auto select_index = torch::empty({nnz}, I64(indptr));
+  torch::Tensor coo_col;
+  if (with_coo) coo_col = torch::empty({nnz}, indices.options());
+  Check(gs_slice_fill(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), column_ids.data_ptr(), idb, S,
+                      sub_indptr.data_ptr<int64_t>(), nnz, sub_indices.data_ptr(),
+                      select_index.data_ptr<int64_t>(), with_coo ? coo_col.data_ptr() : nullptr, st),
+        "gs_slice_fill");
+  return {sub_indptr, coo_col, sub_indices, select_index};
+}
+
+namespace {
+
+// shared by uniform and weighted sampling: offsets, upper-bound buffers, narrow
+template <typename Fill>
+SliceResult SampleInto(const torch::Tensor& indptr, const torch::Tensor& indices,
+                       const torch::Tensor& column_ids, int64_t fanout, bool replace, bool with_coo,
+                       size_t extra_ws, Fill fill) {
+  NeedI64(indptr, "indptr");
+  const int idb = IdBytes(indices, "indices");
+  const bool fused = column_ids.defined();
+  if (fused)
+    TORCH_CHECK(IdBytes(column_ids, "column ids") == idb, "column ids and indices differ in dtype");
+  TORCH_CHECK(fanout >= 0, "fanout must be non-negative");
+  const int64_t S = fused ? column_ids.numel() : indptr.numel() - 1;
+  auto sub_indptr = torch::empty({S + 1}, I64(indptr));
+  const int64_t cap = S * fanout;
+  auto sub_indices = torch::empty({cap}, indices.options());
+  auto select_index = torch::empty({cap}, I64(indptr));
+  torch::Tensor coo_col;
+  if (with_coo) coo_col = torch::empty({cap}, indices.options());
+  size_t bytes = gs_sample_workspace_bytes(S, fanout);
+  if (extra_ws > bytes) bytes = extra_ws;
+  auto ws = Scratch(bytes, indptr);
+  void* st = Stream(indptr);
+  const void* cols = fused ? column_ids.data_ptr() : nullptr;
+  Check(gs_sample_count(indptr.data_ptr<int64_t>(), indptr.numel() - 1, cols, idb, S, fanout, replace ? 1 : 0,
+                        sub_indptr.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
+        "gs_sample_count");
+  fill(cols, idb, S, sub_indptr, sub_indices, select_index, coo_col, ws, st);
+  const int64_t nnz = sub_indptr[S].item<int64_t>();  // the only host read of the call
+  if (with_coo) coo_col = coo_col.narrow(0, 0, nnz);
+  return {sub_indptr, coo_col, sub_indices.narrow(0, 0, nnz), select_index.narrow(0, 0, nnz)};
+}
+
+}  // namespace
+
+SliceResult ColSampling(const torch::Tensor& indptr, const torch::Tensor& indices,
+                        const torch::Tensor& column_ids, int64_t fanout, bool replace,
+                        bool with_coo) {
+  return SampleInto(
+      indptr, indices, column_ids, fanout, replace, with_coo, 0,
+      [&](const void* cols, int idb, int64_t S, torch::Tensor& sub_indptr, torch::Tensor& sub_indices,
+          torch::Tensor& select_index, torch::Tensor& coo_col, torch::Tensor& ws, void* st) {
+        Check(gs_sample_uniform_fill(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), cols, idb, S,
+                                     fanout, replace ? 1 : 0, static_cast<int>(g_algo.load()),
+                                     NextSeed(), nullptr, nullptr, sub_indptr.data_ptr<int64_t>(),
+                                     sub_indices.data_ptr(), select_index.data_ptr<int64_t>(),
+                                     with_coo ? coo_col.data_ptr() : nullptr, ws.data_ptr(),
+                                     ws.numel(), st),
+              "gs_sample_uniform_fill");
+      });
+}
+
+SliceResult ColSamplingProbs(const torch::Tensor& indptr, const torch::Tensor& indices,
+                             const torch::Tensor& probs, const torch::Tensor& column_ids,
+                             int64_t fanout, bool replace, bool with_coo) {
+  NeedF32(probs, "edge_probs");
+  TORCH_CHECK(!replace,
+              "weighted sampling with replacement is not built (only the A-Res path without "
+              "replacement is)");
+  const int64_t S = column_ids.defined() ? column_ids.numel() : indptr.numel() - 1;
+  return SampleInto(
+      indptr, indices, column_ids, fanout, false, with_coo,
+      gs_sample_weighted_workspace_bytes(S, fanout),
+      [&](const void* cols, int idb, int64_t S_, torch::Tensor& sub_indptr,
+          torch::Tensor& sub_indices, torch::Tensor& select_index, torch::Tensor& coo_col,
+          torch::Tensor& ws, void* st) {
+        Check(gs_sample_weighted_fill(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(),
+                                      probs.data_ptr<float>(), cols, idb, S_, fanout, NextSeed(),
+                                      nullptr, nullptr, sub_indptr.data_ptr<int64_t>(),
+                                      sub_indices.data_ptr(), select_index.data_ptr<int64_t>(),
+                                      with_coo ? coo_col.data_ptr() : nullptr, ws.data_ptr(),
+                                      ws.numel(), st),
+              "gs_sample_weighted_fill");
+      });
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> SampleOneKeepDim(
+    const torch::Tensor& indptr, const torch::Tensor& indices, const torch::Tensor& column_ids) {
+  NeedI64(indptr, "indptr");
+  const int idb = IdBytes(indices, "indices");
+  TORCH_CHECK(IdBytes(column_ids, "column ids") == idb, "column ids and indices differ in dtype");
+  const int64_t S = column_ids.numel();
+  auto sub_indptr = torch::empty({S + 1}, I64(indptr));
+  auto sub_indices = torch::empty({S}, indices.options());
+  auto select_index = torch::empty({S}, I64(indptr));
+  Check(gs_sample_one_keepdim(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), column_ids.data_ptr(),
+                              idb, S, NextSeed(), nullptr, sub_indptr.data_ptr<int64_t>(),
+                              sub_indices.data_ptr(), select_index.data_ptr<int64_t>(),
+                              Stream(indptr)),
+        "gs_sample_one_keepdim");
+  return {sub_indptr, sub_indices, select_index};
+}
+
+std::tuple<torch::Tensor, std::vector<torch::Tensor>> Relabel(
+    const std::vector<torch::Tensor>& mapping, const std::vector<torch::Tensor>& queries) {
+  TORCH_CHECK(!mapping.empty() && mapping.size() <= GS_MAX_SPANS && queries.size() <= GS_MAX_SPANS,
+              "relabel takes 1..", GS_MAX_SPANS, " mapping tensors and at most ", GS_MAX_SPANS,
+              " tensors to relabel");
+  const int idb = IdBytes(mapping[0], "mapping tensor");
+  gs_span m[GS_MAX_SPANS], q[GS_MAX_SPANS];
+  void* out_ptr[GS_MAX_SPANS];
+  int64_t M = 0;
+  for (size_t i = 0; i < mapping.size(); ++i) {
+    TORCH_CHECK(IdBytes(mapping[i], "mapping tensor") == idb, "relabel tensors differ in dtype");
+    m[i] = {mapping[i].data_ptr(), mapping[i].numel()};
+    M += mapping[i].numel();
+  }
+  std::vector<torch::Tensor> outs;
+  for (size_t i = 0; i < queries.size(); ++i) {
+    TORCH_CHECK(IdBytes(queries[i], "tensor to relabel") == idb, "relabel tensors differ in dtype");
+    q[i] = {queries[i].data_ptr(), queries[i].numel()};
+    outs.push_back(torch::empty_like(queries[i]));
+    out_ptr[i] = outs.back().data_ptr();
+  }
+  auto frontier = torch::empty({M}, mapping[0].options());
+  auto num = torch::empty({1}, I64(mapping[0]));
+  auto ws = Scratch(gs_unique_workspace_bytes(M), mapping[0]);
+  Check(gs_unique_relabel(m, static_cast<int>(mapping.size()), q, out_ptr,
+                          static_cast<int>(queries.size()), idb, frontier.data_ptr(),
+                          num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), Stream(mapping[0])),
+        "gs_unique_relabel");
+  const int64_t U = num.item<int64_t>();
+  return {frontier.narrow(0, 0, U), outs};
+}
+
+torch::Tensor Unique(const torch::Tensor& ids) { return std::get<0>(Relabel({ids}, {})); }
+
+torch::Tensor RandomWalk(const torch::Tensor& seeds, int64_t length, const torch::Tensor& indptr,
+                         const torch::Tensor& indices) {
+  NeedI64(indptr, "indptr");
+  const int idb = IdBytes(indices, "indices");
+  TORCH_CHECK(IdBytes(seeds, "seeds") == idb, "seeds and indices differ in dtype");
+  TORCH_CHECK(length >= 0, "walk_length must be non-negative");
+  const int64_t n = seeds.numel();
+  auto trace = torch::empty({n * (length + 1)}, seeds.options());
+  Check(gs_random_walk(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), idb, seeds.data_ptr(), n,
+                       length, NextSeed(), nullptr, trace.data_ptr(), Stream(seeds)),
+        "gs_random_walk");
+  return trace;
+}
+
+torch::Tensor MetapathWalk(const torch::Tensor& seeds, const torch::Tensor& metapath,
+                           const torch::Tensor& indptr_table, const torch::Tensor& indices_table,
+                           const torch::Tensor& num_nodes_table, int id_bytes) {
+  NeedI64(num_nodes_table, "relation sizes");
+  TORCH_CHECK(IdBytes(seeds, "seeds") == id_bytes, "seeds and relation graphs differ in dtype");
+  NeedI64(metapath, "metapath");
+  const int64_t n = seeds.numel();
+  const int64_t L = metapath.numel();
+  auto trace = torch::empty({n * (L + 1)}, seeds.options());
+  Check(gs_metapath_walk(reinterpret_cast<const int64_t* const*>(indptr_table.data_ptr<int64_t>()),
+                         reinterpret_cast<const void* const*>(indices_table.data_ptr<int64_t>()),
+                         num_nodes_table.data_ptr<int64_t>(), id_bytes, metapath.data_ptr<int64_t>(), L, seeds.data_ptr(), n, NextSeed(),
+                         nullptr, trace.data_ptr(), Stream(seeds)),
+        "gs_metapath_walk");
+  return trace;
+}
+
+void SddmmCoo(const std::string& op, const Bcast& b, const torch::Tensor& row,
+              const torch::Tensor& col, const torch::optional<torch::Tensor>& e_ids,
+              const torch::Tensor& lhs, const torch::Tensor& rhs, torch::Tensor out, int lhs_target,
+              int rhs_target) {
+  const int code = OpCode(op);
+  NeedI64(row, "coo row");
+  NeedI64(col, "coo col");
+  NeedF32(out, "out");
+  if (code != GS_OP_COPY_RHS) NeedF32(lhs, "lhs");
+  if (code != GS_OP_COPY_LHS) NeedF32(rhs, "rhs");
+  Check(gs_sddmm_coo(code, row.data_ptr<int64_t>(), col.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"),
+                     row.numel(), lhs.defined() ? lhs.data_ptr<float>() : nullptr,
+                     rhs.defined() ? rhs.data_ptr<float>() : nullptr, out.data_ptr<float>(),
+                     lhs_target, rhs_target, b.lhs_len, b.rhs_len, b.out_len, b.reduce_size,
+                     b.lhs_off.defined() ? b.lhs_off.data_ptr<int64_t>() : nullptr,
+                     b.rhs_off.defined() ? b.rhs_off.data_ptr<int64_t>() : nullptr, Stream(row)),
+        "gs_sddmm_coo");
+}
+
+void SddmmCsc(const std::string& op, const Bcast& b, const torch::Tensor& indptr,
+              const torch::Tensor& indices, const torch::optional<torch::Tensor>& e_ids,
+              const torch::optional<torch::Tensor>& nid_map, const torch::Tensor& lhs,
+              const torch::Tensor& rhs, torch::Tensor out, int lhs_target, int rhs_target) {
+  const int code = OpCode(op);
+  NeedI64(indptr, "indptr");
+  NeedI64(indices, "indices");
+  NeedF32(out, "out");
+  if (code != GS_OP_COPY_RHS) NeedF32(lhs, "lhs");
+  if (code != GS_OP_COPY_LHS) NeedF32(rhs, "rhs");
+  Check(gs_sddmm_csc(code, indptr.data_ptr<int64_t>(), indices.data_ptr<int64_t>(),
+                     OptI64(e_ids, "e_ids"), OptI64(nid_map, "valid ids"), indptr.numel() - 1,
+                     indices.numel(), lhs.defined() ? lhs.data_ptr<float>() : nullptr,
+                     rhs.defined() ? rhs.data_ptr<float>() : nullptr, out.data_ptr<float>(),
+                     lhs_target, rhs_target, b.lhs_len, b.rhs_len, b.out_len, b.reduce_size,
+                     b.lhs_off.defined() ? b.lhs_off.data_ptr<int64_t>() : nullptr,
+                     b.rhs_off.defined() ? b.rhs_off.data_ptr<int64_t>() : nullptr, Stream(indptr)),
+        "gs_sddmm_csc");
+}
+
+void SegmentSum(const torch::Tensor& indptr, const torch::optional<torch::Tensor>& e_ids,
+                const torch::optional<torch::Tensor>& n_ids, const torch::Tensor& data,
+                torch::Tensor out, int64_t powk) {
+  NeedI64(indptr, "indptr");
+  NeedF32(data, "data");
+  NeedF32(out, "out");
+  Check(gs_segment_sum(indptr.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"), OptI64(n_ids, "valid ids"),
+                       data.data_ptr<float>(), indptr.numel() - 1, powk, out.data_ptr<float>(),
+                       Stream(indptr)),
+        "gs_segment_sum");
+}
+
+void CooSum(const torch::Tensor& target, const torch::optional<torch::Tensor>& e_ids,
+            const torch::Tensor& data, torch::Tensor out, int64_t powk) {
+  NeedI64(target, "coo target");
+  NeedF32(data, "data");
+  NeedF32(out, "out");
+  Check(gs_coo_sum(target.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"), data.data_ptr<float>(),
+                   target.numel(), powk, out.data_ptr<float>(), Stream(target)),
+        "gs_coo_sum");
+}
+
+void SegmentNormalize(const torch::Tensor& indptr, const torch::optional<torch::Tensor>& e_ids,
+                      const torch::Tensor& data, torch::Tensor out) {
+  NeedI64(indptr, "indptr");
+  NeedF32(data, "data");
+  NeedF32(out, "out");
+  Check(gs_segment_normalize(indptr.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"),
+                             data.data_ptr<float>(), indptr.numel() - 1, out.data_ptr<float>(),
+                             Stream(indptr)),
+        "gs_segment_normalize");
+}
+
+void EDivUSum(const torch::Tensor& row, const torch::Tensor& col, const torch::Tensor& data,
+              const torch::Tensor& divisor, torch::Tensor out_data, torch::Tensor out_sum) {
+  NeedI64(row, "coo row");
+  NeedI64(col, "coo col");
+  NeedF32(data, "data");
+  NeedF32(divisor, "divisor");
+  Check(gs_e_div_u_sum(row.data_ptr<int64_t>(), col.data_ptr<int64_t>(), data.data_ptr<float>(),
+                       divisor.data_ptr<float>(), row.numel(), out_data.data_ptr<float>(),
+                       out_sum.data_ptr<float>(), Stream(row)),
+        "gs_e_div_u_sum");
+}
+
+SliceResult RowSlicingCsc(const torch::Tensor& indptr, const torch::Tensor& indices,
+                          const torch::Tensor& row_ids, bool with_coo) {
+  NeedI64(indptr, "indptr");
+  NeedI64(indices, "indices");
+  NeedI64(row_ids, "row ids");
+  const int64_t ncols = indptr.numel() - 1, nnz = indices.numel(), nr = row_ids.numel();
+  auto out_indptr = torch::empty({ncols + 1}, I64(indptr));
+  auto ws = Scratch(gs_row_slice_workspace_bytes(nr, nnz, ncols), indptr);
+  void* st = Stream(indptr);
+  Check(gs_row_slice_csc_mark(indptr.data_ptr<int64_t>(), indices.data_ptr<int64_t>(), ncols, nnz,
+                              row_ids.data_ptr<int64_t>(), nr, out_indptr.data_ptr<int64_t>(),
+                              ws.data_ptr(), ws.numel(), st),
+        "gs_row_slice_csc_mark");
+  const int64_t kept = out_indptr[ncols].item<int64_t>();
+  auto out_indices = torch::empty({kept}, I64(indptr));
+  auto select_index = torch::empty({kept}, I64(indptr));
+  torch::Tensor coo_col;
+  if (with_coo) coo_col = torch::empty({kept}, I64(indptr));
+  if (kept > 0)
+    Check(gs_row_slice_csc_compact(indptr.data_ptr<int64_t>(), indices.data_ptr<int64_t>(), ncols,
+                                   nnz, out_indptr.data_ptr<int64_t>(),
+                                   out_indices.data_ptr<int64_t>(), select_index.data_ptr<int64_t>(),
+                                   with_coo ? coo_col.data_ptr<int64_t>() : nullptr, ws.data_ptr(),
+                                   ws.numel(), st),
+          "gs_row_slice_csc_compact");
+  return {out_indptr, coo_col, out_indices, select_index};
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(const torch::Tensor& key,
+                                                                      const torch::Tensor& other,
+                                                                      const torch::Tensor& ids) {
+  NeedI64(key, "coo ids");
+  NeedI64(other, "coo ids");
+  NeedI64(ids, "node ids");
+  const int64_t E = key.numel(), n = ids.numel();
+  auto num = torch::empty({1}, I64(key));
+  auto ws = Scratch(gs_row_slice_workspace_bytes(n, E, 0), key);
+  void* st = Stream(key);
+  Check(gs_row_slice_coo_mark(key.data_ptr<int64_t>(), E, ids.data_ptr<int64_t>(), n,
+                              num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
+        "gs_row_slice_coo_mark");
+  const int64_t kept = num.item<int64_t>();
+  auto out_key = torch::empty({kept}, I64(key));
+  auto out_other = torch::empty({kept}, I64(key));
+  auto select_index = torch::empty({kept}, I64(key));
+  if (kept > 0)
+    Check(gs_row_slice_coo_compact(key.data_ptr<int64_t>(), other.data_ptr<int64_t>(), E,
+                                   out_key.data_ptr<int64_t>(), out_other.data_ptr<int64_t>(),
+                                   select_index.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
+          "gs_row_slice_coo_compact");
+  return {out_key, out_other, select_index};
+}
+
+torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz) {
+  NeedI64(indptr, "indptr");
+  auto col = torch::empty({nnz}, I64(indptr));
+  Check(gs_csc2coo(indptr.data_ptr<int64_t>(), indptr.numel() - 1, nnz, col.data_ptr<int64_t>(),
+                   Stream(indptr)),
+        "gs_csc2coo");
+  return col;
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::optional<torch::Tensor>> Coo2Csc(
+    const torch::Tensor& key, const torch::Tensor& value, int64_t num_keys, bool sorted) {
+  NeedI64(key, "coo key");
+  NeedI64(value, "coo value");
+  const int64_t E = key.numel();
+  auto indptr = torch::empty({num_keys + 1}, I64(key));
+  if (sorted) {
+    Check(gs_coo2csc(key.data_ptr<int64_t>(), value.data_ptr<int64_t>(), E, num_keys, 1,
+                     indptr.data_ptr<int64_t>(), nullptr, nullptr, nullptr, 0, Stream(key)),
+          "gs_coo2csc");
+    return {indptr, value, torch::nullopt};
+  }
+  auto out_value = torch::empty({E}, I64(key));
+  auto perm = torch::empty({E}, I64(key));
+  auto ws = Scratch(gs_coo2csc_workspace_bytes(E, num_keys), key);
+  Check(gs_coo2csc(key.data_ptr<int64_t>(), value.data_ptr<int64_t>(), E, num_keys, 0,
+                   indptr.data_ptr<int64_t>(), out_value.data_ptr<int64_t>(),
+                   perm.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), Stream(key)),
+        "gs_coo2csc");
+  return {indptr, out_value, perm};
+}
+
+std::tuple<torch::Tensor, torch::Tensor> ListSampling(const torch::Tensor& data, int64_t k,
+                                                      bool replace) {
+  const int idb = IdBytes(data, "data");
+  const int64_t n = data.numel();
+  if (n <= k && !replace) return {data, torch::arange(n, I64(data))};  // list_sampling.cu:29-32
+  auto out_data = torch::empty({k}, data.options());
+  auto out_index = torch::empty({k}, I64(data));
+  auto ws = Scratch(gs_list_sample_workspace_bytes(n, k), data);
+  Check(gs_list_sample_uniform(data.data_ptr(), idb, n, k, replace ? 1 : 0, NextSeed(), nullptr,
+                               out_data.data_ptr(), out_index.data_ptr<int64_t>(), ws.data_ptr(),
+                               ws.numel(), Stream(data)),
+        "gs_list_sample_uniform");
+  return {out_data, out_index};
+}
+
+std::tuple<torch::Tensor, torch::Tensor> ListSamplingProbs(const torch::Tensor& data,
+                                                           const torch::Tensor& probs, int64_t k,
+                                                           bool replace) {
+  const int idb = IdBytes(data, "data");
+  NeedF32(probs, "probs");
+  const int64_t n = data.numel();
+  TORCH_CHECK(probs.numel() == n, "data and probs differ in length");
+  if (n <= k && !replace) return {data, torch::arange(n, I64(data))};  // list_sampling_probs.cu:20-23
+  TORCH_CHECK(!replace,
+              "weighted list sampling with replacement is not built (only the A-Res path without "
+              "replacement is)");
+  auto out_data = torch::empty({k}, data.options());
+  auto out_index = torch::empty({k}, I64(data));
+  auto ws = Scratch(gs_list_sample_workspace_bytes(n, k), data);
+  Check(gs_list_sample_weighted(data.data_ptr(), idb, probs.data_ptr<float>(), n, k, NextSeed(),
+                                nullptr, out_data.data_ptr(), out_index.data_ptr<int64_t>(),
+                                ws.data_ptr(), ws.numel(), Stream(data)),
+        "gs_list_sample_weighted");
+  return {out_data, out_index};
+}
+
+}  // namespace hip
+}  // namespace gs

@@ -1,0 +1,93 @@
+// torch::Tensor front end of the C ABI (include/gs_hip.h): allocates outputs
+// and scratch with the torch allocator, passes raw device pointers and the
+// current HIP stream, turns a negative status into a c10::Error.
+//
+// This is the only file of the host layer that knows about the C ABI; it plays
+// the part of the reference's src/cuda/graph_ops.h / tensor_ops.h / sddmm.h.
+#pragma once
+
+#include <torch/torch.h>
+
+#include <string>
+#include <tuple>
+#include <vector>
+
+namespace gs {
+namespace hip {
+
+// {sub_indptr, coo_col (undefined when !with_coo), sub_indices, select_index}
+using SliceResult = std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor>;
+
+// Seed of the next sampling / walk call; every call consumes one value
+// (seed, seed+1, ...).  The reference hard-wires its seeds, so two calls with
+// the same launch geometry repeat the same draws (src/cuda/sampling.cu:138).
+void SetSeed(uint64_t seed);
+uint64_t NextSeed();
+// 0: Floyd selection for deg > fanout (default), 1: the reference's Algorithm R.
+void SetSampleAlgo(int64_t algo);
+
+SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
+                       const torch::Tensor& column_ids, bool with_coo);
+// column_ids undefined: every column of the CSC
+SliceResult ColSampling(const torch::Tensor& indptr, const torch::Tensor& indices,
+                        const torch::Tensor& column_ids, int64_t fanout, bool replace,
+                        bool with_coo);
+SliceResult ColSamplingProbs(const torch::Tensor& indptr, const torch::Tensor& indices,
+                             const torch::Tensor& probs, const torch::Tensor& column_ids,
+                             int64_t fanout, bool replace, bool with_coo);
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> SampleOneKeepDim(
+    const torch::Tensor& indptr, const torch::Tensor& indices, const torch::Tensor& column_ids);
+
+torch::Tensor Unique(const torch::Tensor& ids);
+std::tuple<torch::Tensor, std::vector<torch::Tensor>> Relabel(
+    const std::vector<torch::Tensor>& mapping, const std::vector<torch::Tensor>& queries);
+
+torch::Tensor RandomWalk(const torch::Tensor& seeds, int64_t length, const torch::Tensor& indptr,
+                         const torch::Tensor& indices);
+torch::Tensor MetapathWalk(const torch::Tensor& seeds, const torch::Tensor& metapath,
+                           const torch::Tensor& indptr_table, const torch::Tensor& indices_table,
+                           const torch::Tensor& num_nodes_table, int id_bytes);
+
+struct Bcast {
+  int64_t lhs_len, rhs_len, out_len, reduce_size;
+  torch::Tensor lhs_off, rhs_off;  // undefined when no broadcast
+};
+void SddmmCoo(const std::string& op, const Bcast& b, const torch::Tensor& row,
+              const torch::Tensor& col, const torch::optional<torch::Tensor>& e_ids,
+              const torch::Tensor& lhs, const torch::Tensor& rhs, torch::Tensor out, int lhs_target,
+              int rhs_target);
+void SddmmCsc(const std::string& op, const Bcast& b, const torch::Tensor& indptr,
+              const torch::Tensor& indices, const torch::optional<torch::Tensor>& e_ids,
+              const torch::optional<torch::Tensor>& nid_map, const torch::Tensor& lhs,
+              const torch::Tensor& rhs, torch::Tensor out, int lhs_target, int rhs_target);
+
+void SegmentSum(const torch::Tensor& indptr, const torch::optional<torch::Tensor>& e_ids,
+                const torch::optional<torch::Tensor>& n_ids, const torch::Tensor& data,
+                torch::Tensor out, int64_t powk);
+void CooSum(const torch::Tensor& target, const torch::optional<torch::Tensor>& e_ids,
+            const torch::Tensor& data, torch::Tensor out, int64_t powk);
+void SegmentNormalize(const torch::Tensor& indptr, const torch::optional<torch::Tensor>& e_ids,
+                      const torch::Tensor& data, torch::Tensor out);
+void EDivUSum(const torch::Tensor& row, const torch::Tensor& col, const torch::Tensor& data,
+              const torch::Tensor& divisor, torch::Tensor out_data, torch::Tensor out_sum);
+
+SliceResult RowSlicingCsc(const torch::Tensor& indptr, const torch::Tensor& indices,
+                          const torch::Tensor& row_ids, bool with_coo);
+// {relabelled key, other, select_index}
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(const torch::Tensor& key,
+                                                                      const torch::Tensor& other,
+                                                                      const torch::Tensor& ids);
+
+torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz);
+// {indptr, values in key order, sort permutation (nullopt when already sorted)}
+std::tuple<torch::Tensor, torch::Tensor, torch::optional<torch::Tensor>> Coo2Csc(
+    const torch::Tensor& key, const torch::Tensor& value, int64_t num_keys, bool sorted);
+
+std::tuple<torch::Tensor, torch::Tensor> ListSampling(const torch::Tensor& data, int64_t k,
+                                                      bool replace);
+std::tuple<torch::Tensor, torch::Tensor> ListSamplingProbs(const torch::Tensor& data,
+                                                           const torch::Tensor& probs, int64_t k,
+                                                           bool replace);
+
+}  // namespace hip
+}  // namespace gs

@@ -19,6 +19,10 @@
  *    (indices, column ids, frontier, relabelled ids) are `id_bytes` wide: 8
  *    (int64, the reference's only instantiation, src/cuda/slicing.cu:176) or 4
  *    (int32 extension).
+ *  - `num_cols` / `num_nodes` is the number of columns the offsets describe
+ *    (indptr has num_cols + 1 entries).  A caller-supplied column id or walk
+ *    seed outside [0, num_cols) is treated as an empty column / a dead walker;
+ *    it is never dereferenced.  (The reference reads indptr[id] unchecked.)
  *  - Return value: GS_OK or a negative gs_status.  Nothing throws or aborts.
  *
  * Randomness.  draw(seed, tag, row, idx) =
@@ -64,14 +68,16 @@ size_t gs_slice_workspace_bytes(int64_t num_cols);
 
 /* sub_indptr[0..S] = exclusive scan of deg(column_ids[r]); total in sub_indptr[S]
  * (slicing.cu:133-147). */
-int gs_slice_count(const int64_t* indptr, const void* column_ids, int id_bytes, int64_t S,
-                   int64_t* sub_indptr, void* workspace, size_t workspace_bytes, void* stream);
+int gs_slice_count(const int64_t* indptr, int64_t num_cols, const void* column_ids, int id_bytes,
+                   int64_t S, int64_t* sub_indptr, void* workspace, size_t workspace_bytes,
+                   void* stream);
 
 /* Neighbour copy (slicing.cu:101-119).  nnz = sub_indptr[S] as read back by the
  * caller.  coo_col may be NULL (WITH_COO = false). */
-int gs_slice_fill(const int64_t* indptr, const void* indices, const void* column_ids,
-                  int id_bytes, int64_t S, const int64_t* sub_indptr, int64_t nnz,
-                  void* sub_indices, int64_t* select_index, void* coo_col, void* stream);
+int gs_slice_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
+                  const void* column_ids, int id_bytes, int64_t S, const int64_t* sub_indptr,
+                  int64_t nnz, void* sub_indices, int64_t* select_index, void* coo_col,
+                  void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Uniform neighbour sampling: replaces impl::CSCColSamplingCUDA              */
@@ -95,8 +101,8 @@ typedef enum gs_sample_algo { GS_SAMPLE_AUTO = 0, GS_SAMPLE_RESERVOIR = 1 } gs_s
 
 /* sub_indptr = exscan(cnt), cnt = replace ? (deg ? fanout : 0) : min(deg, fanout)
  * (sampling.cu:107-119). */
-int gs_sample_count(const int64_t* indptr, const void* column_ids, int id_bytes, int64_t S,
-                    int64_t fanout, int replace, int64_t* sub_indptr, void* workspace,
+int gs_sample_count(const int64_t* indptr, int64_t num_cols, const void* column_ids, int id_bytes,
+                    int64_t S, int64_t fanout, int replace, int64_t* sub_indptr, void* workspace,
                     size_t workspace_bytes, void* stream);
 
 /* Fill for a sub_indptr made by gs_sample_count on the same stream.  Output
@@ -108,9 +114,9 @@ int gs_sample_count(const int64_t* indptr, const void* column_ids, int id_bytes,
  * a row with deg > fanout consumes deg-fanout draws (Algorithm R) or fanout
  * draws (Floyd), other rows none; with replacement every row consumes its
  * output count.  coo_col may be NULL. */
-int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const void* column_ids,
-                           int id_bytes, int64_t S, int64_t fanout, int replace, int algo,
-                           uint64_t seed,
+int gs_sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
+                           const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+                           int replace, int algo, uint64_t seed,
                            const uint32_t* replay, const int64_t* replay_ptr,
                            const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                            void* coo_col, void* workspace, size_t workspace_bytes, void* stream);
@@ -119,8 +125,9 @@ int gs_sample_uniform_fill(const int64_t* indptr, const void* indices, const voi
  * column, -1 in both outputs for an empty column; sub_indptr = 0..S.  Replaces
  * impl::fusion::FusedCSCColSlicingSamplingOneKeepDimCUDA
  * (src/cuda/fusion/slice_sampling.cu:157).  replay: one draw per column. */
-int gs_sample_one_keepdim(const int64_t* indptr, const void* indices, const void* column_ids,
-                          int id_bytes, int64_t S, uint64_t seed, const uint32_t* replay,
+int gs_sample_one_keepdim(const int64_t* indptr, int64_t num_cols, const void* indices,
+                          const void* column_ids, int id_bytes, int64_t S, uint64_t seed,
+                          const uint32_t* replay,
                           int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                           void* stream);
 
@@ -135,8 +142,9 @@ int gs_sample_one_keepdim(const int64_t* indptr, const void* indices, const void
 /* ------------------------------------------------------------------------- */
 size_t gs_sample_weighted_workspace_bytes(int64_t S, int64_t fanout);
 
-int gs_sample_weighted_fill(const int64_t* indptr, const void* indices, const float* probs,
-                            const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+int gs_sample_weighted_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
+                            const float* probs, const void* column_ids, int id_bytes, int64_t S,
+                            int64_t fanout,
                             uint64_t seed, const uint32_t* replay, const int64_t* replay_ptr,
                             const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                             void* coo_col, void* workspace, size_t workspace_bytes, void* stream);
@@ -191,16 +199,17 @@ int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* quer
 /* [length+1][n] (step-major); -1 is absorbing; one draw per live step;        */
 /* replay layout [length][n].                                                  */
 /* ------------------------------------------------------------------------- */
-int gs_random_walk(const int64_t* indptr, const void* indices, int id_bytes, const void* seeds,
-                   int64_t n, int64_t length, uint64_t seed, const uint32_t* replay,
+int gs_random_walk(const int64_t* indptr, int64_t num_nodes, const void* indices, int id_bytes,
+                   const void* seeds, int64_t n, int64_t length, uint64_t seed, const uint32_t* replay,
                    void* trace, void* stream);
 
 /* all_indptr / all_indices: device arrays of device pointers, one per relation
- * (src/hetero_graph.cc:33-50); metapath: device int64[length] relation ids. */
+ * (src/hetero_graph.cc:33-50); all_num_nodes: device int64 array, the number of
+ * columns of each relation; metapath: device int64[length] relation ids. */
 int gs_metapath_walk(const int64_t* const* all_indptr, const void* const* all_indices,
-                     int id_bytes, const int64_t* metapath, int64_t length, const void* seeds,
-                     int64_t n, uint64_t seed, const uint32_t* replay, void* trace,
-                     void* stream);
+                     const int64_t* all_num_nodes, int id_bytes, const int64_t* metapath,
+                     int64_t length, const void* seeds, int64_t n, uint64_t seed,
+                     const uint32_t* replay, void* trace, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* SDDMM: replaces impl::SDDMMCOO / impl::SDDMMCSC (src/cuda/sddmm.cu:280,263). */

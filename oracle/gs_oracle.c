@@ -126,11 +126,16 @@ float gso_ares_key(u32 x, float w) {
 /* Column slicing.  src/cuda/slicing.cu:101-168                              */
 /* ------------------------------------------------------------------------ */
 /* sub_indptr = exscan(deg(cols[r])), returns the total. (slicing.cu:133-147) */
-i64 gso_slice_count(const i64* indptr, const i64* cols, i64 S, i64* sub_indptr) {
+/* A column id outside [0, num_cols) counts as an empty column in every routine
+ * below (the reference reads indptr[id] unchecked; the build defines this so
+ * that the -1 a dead-end step returns can be fed back in as a seed). */
+static inline int col_ok(i64 c, i64 num_cols) { return c >= 0 && c < num_cols; }
+
+i64 gso_slice_count(const i64* indptr, i64 num_cols, const i64* cols, i64 S, i64* sub_indptr) {
   i64 acc = 0;
   for (i64 r = 0; r < S; ++r) {
     sub_indptr[r] = acc;
-    acc += indptr[cols[r] + 1] - indptr[cols[r]];
+    if (col_ok(cols[r], num_cols)) acc += indptr[cols[r] + 1] - indptr[cols[r]];
   }
   sub_indptr[S] = acc;
   return acc;
@@ -142,9 +147,10 @@ void gso_slice_fill(const i64* indptr, const i64* indices, const i64* cols, i64 
                     i64* coo_col) {
 #pragma omp parallel for schedule(dynamic, 64)
   for (i64 r = 0; r < S; ++r) {
-    i64 in_start = indptr[cols[r]];
     i64 out_start = sub_indptr[r];
     i64 n = sub_indptr[r + 1] - out_start;
+    if (n == 0) continue;
+    i64 in_start = indptr[cols[r]];
     for (i64 j = 0; j < n; ++j) {
       sub_indices[out_start + j] = indices[in_start + j];
       select_index[out_start + j] = in_start + j;
@@ -177,12 +183,12 @@ static inline int use_floyd(int algo, i64 k) { return algo == GSO_ALGO_AUTO && k
  * (sampling.cu:107-119).  replay_ptr (optional, may be NULL) = exscan of the
  * number of draws each row consumes: replace ? cnt : (deg > k ? (Floyd ? k :
  * deg-k) : 0). */
-i64 gso_sample_count(const i64* indptr, const i64* cols, i64 S, i64 k, int replace, int algo,
-                     i64* sub_indptr, i64* replay_ptr) {
+i64 gso_sample_count(const i64* indptr, i64 num_cols, const i64* cols, i64 S, i64 k, int replace,
+                     int algo, i64* sub_indptr, i64* replay_ptr) {
   i64 acc = 0, racc = 0;
   for (i64 r = 0; r < S; ++r) {
     i64 c = col_of(cols, r);
-    i64 deg = indptr[c + 1] - indptr[c];
+    i64 deg = col_ok(c, num_cols) ? indptr[c + 1] - indptr[c] : 0;
     i64 cnt = replace ? (deg == 0 ? 0 : k) : (deg < k ? deg : k);
     sub_indptr[r] = acc;
     acc += cnt;
@@ -196,7 +202,7 @@ i64 gso_sample_count(const i64* indptr, const i64* cols, i64 S, i64 k, int repla
   return acc;
 }
 
-void gso_sample_uniform_fill(const i64* indptr, const i64* indices, const i64* cols,
+void gso_sample_uniform_fill(const i64* indptr, i64 num_cols, const i64* indices, const i64* cols,
                              i64 S, i64 k, int replace, int algo, u64 seed, const u32* replay,
                              const i64* replay_ptr, const i64* sub_indptr,
                              i64* sub_indices, i64* select_index, i64* coo_col) {
@@ -206,6 +212,7 @@ void gso_sample_uniform_fill(const i64* indptr, const i64* indices, const i64* c
 #pragma omp for schedule(dynamic, 16)
     for (i64 r = 0; r < S; ++r) {
       i64 c = col_of(cols, r);
+      if (!col_ok(c, num_cols)) continue;
       i64 in_start = indptr[c];
       i64 deg = indptr[c + 1] - in_start;
       i64 out_start = sub_indptr[r];
@@ -270,15 +277,15 @@ void gso_sample_uniform_fill(const i64* indptr, const i64* indices, const i64* c
 
 /* fanout == 1 && replace through the fused entry: exactly one slot per column,
  * -1/-1 for an empty column.  src/cuda/fusion/slice_sampling.cu:157-200 */
-void gso_sample_one_keepdim(const i64* indptr, const i64* indices, const i64* cols,
+void gso_sample_one_keepdim(const i64* indptr, i64 num_cols, const i64* indices, const i64* cols,
                             i64 S, u64 seed, const u32* replay, i64* sub_indptr,
                             i64* sub_indices, i64* select_index) {
   for (i64 r = 0; r <= S; ++r) sub_indptr[r] = r;
 #pragma omp parallel for schedule(static)
   for (i64 r = 0; r < S; ++r) {
     i64 c = cols[r];
-    i64 in_start = indptr[c];
-    i64 deg = indptr[c + 1] - in_start;
+    i64 in_start = col_ok(c, num_cols) ? indptr[c] : 0;
+    i64 deg = col_ok(c, num_cols) ? indptr[c + 1] - in_start : 0;
     if (deg == 0) {
       sub_indices[r] = -1;
       select_index[r] = -1;
@@ -316,12 +323,12 @@ static int kp_cmp(const void* a, const void* b) {
   return 0;
 }
 
-i64 gso_weighted_replay_count(const i64* indptr, const i64* cols, i64 S, i64 k,
+i64 gso_weighted_replay_count(const i64* indptr, i64 num_cols, const i64* cols, i64 S, i64 k,
                               i64* replay_ptr) {
   i64 acc = 0;
   for (i64 r = 0; r < S; ++r) {
     i64 c = col_of(cols, r);
-    i64 deg = indptr[c + 1] - indptr[c];
+    i64 deg = col_ok(c, num_cols) ? indptr[c + 1] - indptr[c] : 0;
     replay_ptr[r] = acc;
     acc += deg > k ? deg : 0;
   }
@@ -329,13 +336,14 @@ i64 gso_weighted_replay_count(const i64* indptr, const i64* cols, i64 S, i64 k,
   return acc;
 }
 
-void gso_sample_weighted_fill(const i64* indptr, const i64* indices, const float* probs,
-                              const i64* cols, i64 S, i64 k, u64 seed, const u32* replay,
+void gso_sample_weighted_fill(const i64* indptr, i64 num_cols, const i64* indices,
+                              const float* probs, const i64* cols, i64 S, i64 k, u64 seed, const u32* replay,
                               const i64* replay_ptr, const i64* sub_indptr,
                               i64* sub_indices, i64* select_index, i64* coo_col) {
 #pragma omp parallel for schedule(dynamic, 16)
   for (i64 r = 0; r < S; ++r) {
     i64 c = col_of(cols, r);
+    if (!col_ok(c, num_cols)) continue;
     i64 in_start = indptr[c];
     i64 deg = indptr[c + 1] - in_start;
     i64 out_start = sub_indptr[r];
@@ -520,7 +528,7 @@ i64 gso_relabel(const i64* mapping, i64 n_map, const i64* query, i64 n_query,
 /* [L+1][n] (step-major); -1 is absorbing; one draw per live step.           */
 /* Replay buffer layout: [L][n].                                             */
 /* ------------------------------------------------------------------------ */
-void gso_random_walk(const i64* indptr, const i64* indices, const i64* seeds, i64 n,
+void gso_random_walk(const i64* indptr, i64 num_nodes, const i64* indices, const i64* seeds, i64 n,
                      i64 L, u64 seed, const u32* replay, i64* trace) {
 #pragma omp parallel for schedule(static)
   for (i64 w = 0; w < n; ++w) {
@@ -528,7 +536,7 @@ void gso_random_walk(const i64* indptr, const i64* indices, const i64* seeds, i6
     trace[w] = curr;
     for (i64 t = 0; t < L; ++t) {
       i64 pick = -1;
-      if (curr >= 0) {
+      if (col_ok(curr, num_nodes)) {
         i64 start = indptr[curr];
         i64 deg = indptr[curr + 1] - start;
         if (deg > 0) {
@@ -545,7 +553,7 @@ void gso_random_walk(const i64* indptr, const i64* indices, const i64* seeds, i6
 /* relation of step t is metapath[t]; (indptr, indices) tables per relation
  * (src/hetero_graph.cc:33-50, metapath_random_walk.cu:36-38). */
 void gso_metapath_walk(const i64* const* all_indptr, const i64* const* all_indices,
-                       const i64* metapath, i64 L, const i64* seeds, i64 n, u64 seed,
+                       const i64* all_num_nodes, const i64* metapath, i64 L, const i64* seeds, i64 n, u64 seed,
                        const u32* replay, i64* trace) {
 #pragma omp parallel for schedule(static)
   for (i64 w = 0; w < n; ++w) {
@@ -553,7 +561,7 @@ void gso_metapath_walk(const i64* const* all_indptr, const i64* const* all_indic
     trace[w] = curr;
     for (i64 t = 0; t < L; ++t) {
       i64 pick = -1;
-      if (curr >= 0) {
+      if (col_ok(curr, all_num_nodes[metapath[t]])) {
         const i64* indptr = all_indptr[metapath[t]];
         const i64* indices = all_indices[metapath[t]];
         i64 start = indptr[curr];

@@ -113,7 +113,7 @@ def slice_columns(indptr, indices, cols, with_coo=True):
     indptr, indices, cols = _i64(indptr), _i64(indices), _i64(cols)
     S = cols.size
     sub_indptr = np.empty(S + 1, dtype=np.int64)
-    nnz = lib().gso_slice_count(_p(indptr), _p(cols), _c64(S), _p(sub_indptr))
+    nnz = lib().gso_slice_count(_p(indptr), _c64(indptr.size - 1), _p(cols), _c64(S), _p(sub_indptr))
     sub_indices = np.empty(nnz, dtype=np.int64)
     select_index = np.empty(nnz, dtype=np.int64)
     coo_col = np.empty(nnz, dtype=np.int64) if with_coo else None
@@ -133,7 +133,7 @@ def sample_count(indptr, cols, k, replace, want_replay_ptr=False, algo=ALGO_AUTO
     S = indptr.size - 1 if cols is None else cols.size
     sub_indptr = np.empty(S + 1, dtype=np.int64)
     replay_ptr = np.empty(S + 1, dtype=np.int64) if want_replay_ptr else None
-    lib().gso_sample_count(_p(indptr), _p(cols), _c64(S), _c64(k), ctypes.c_int(int(replace)),
+    lib().gso_sample_count(_p(indptr), _c64(indptr.size - 1), _p(cols), _c64(S), _c64(k), ctypes.c_int(int(replace)),
                            ctypes.c_int(int(algo)), _p(sub_indptr), _p(replay_ptr))
     return sub_indptr, replay_ptr
 
@@ -158,7 +158,7 @@ def sample_uniform(indptr, indices, cols, k, replace, seed=0, replay=None, with_
     sub_indices = np.empty(nnz, dtype=np.int64)
     select_index = np.empty(nnz, dtype=np.int64)
     coo_col = np.empty(nnz, dtype=np.int64) if with_coo else None
-    lib().gso_sample_uniform_fill(_p(indptr), _p(indices), _p(cols), _c64(S), _c64(k),
+    lib().gso_sample_uniform_fill(_p(indptr), _c64(indptr.size - 1), _p(indices), _p(cols), _c64(S), _c64(k),
                                   ctypes.c_int(int(replace)), ctypes.c_int(int(algo)),
                                   _cu64(seed), _p(replay),
                                   _p(replay_ptr), _p(sub_indptr), _p(sub_indices),
@@ -174,7 +174,7 @@ def sample_one_keepdim(indptr, indices, cols, seed=0, replay=None):
     sub_indptr = np.empty(S + 1, dtype=np.int64)
     sub_indices = np.empty(S, dtype=np.int64)
     select_index = np.empty(S, dtype=np.int64)
-    lib().gso_sample_one_keepdim(_p(indptr), _p(indices), _p(cols), _c64(S), _cu64(seed),
+    lib().gso_sample_one_keepdim(_p(indptr), _c64(indptr.size - 1), _p(indices), _p(cols), _c64(S), _cu64(seed),
                                  _p(replay), _p(sub_indptr), _p(sub_indices), _p(select_index))
     return sub_indptr, sub_indices, select_index
 
@@ -184,7 +184,7 @@ def weighted_replay_ptr(indptr, cols, k):
     cols = None if cols is None else _i64(cols)
     S = indptr.size - 1 if cols is None else cols.size
     rp = np.empty(S + 1, dtype=np.int64)
-    lib().gso_weighted_replay_count(_p(indptr), _p(cols), _c64(S), _c64(k), _p(rp))
+    lib().gso_weighted_replay_count(_p(indptr), _c64(indptr.size - 1), _p(cols), _c64(S), _c64(k), _p(rp))
     return rp
 
 
@@ -203,7 +203,7 @@ def sample_weighted(indptr, indices, probs, cols, k, seed=0, replay=None, with_c
     sub_indices = np.empty(nnz, dtype=np.int64)
     select_index = np.empty(nnz, dtype=np.int64)
     coo_col = np.empty(nnz, dtype=np.int64) if with_coo else None
-    lib().gso_sample_weighted_fill(_p(indptr), _p(indices), _p(probs), _p(cols), _c64(S), _c64(k),
+    lib().gso_sample_weighted_fill(_p(indptr), _c64(indptr.size - 1), _p(indices), _p(probs), _p(cols), _c64(S), _c64(k),
                                    _cu64(seed), _p(replay), _p(replay_ptr), _p(sub_indptr),
                                    _p(sub_indices), _p(select_index), _p(coo_col))
     return sub_indptr, coo_col, sub_indices, select_index
@@ -267,7 +267,7 @@ def random_walk(indptr, indices, seeds, length, seed=0, replay=None):
     n = seeds.size
     replay = None if replay is None else _u32(replay)
     trace = np.empty((length + 1) * n, dtype=np.int64)
-    lib().gso_random_walk(_p(indptr), _p(indices), _p(seeds), _c64(n), _c64(length),
+    lib().gso_random_walk(_p(indptr), _c64(indptr.size - 1), _p(indices), _p(seeds), _c64(n), _c64(length),
                           _cu64(seed), _p(replay), _p(trace))
     return trace
 
@@ -283,7 +283,8 @@ def metapath_walk(indptrs, indicess, metapath, seeds, seed=0, replay=None):
     ip = PtrArr(*[a.ctypes.data for a in indptrs])
     ix = PtrArr(*[a.ctypes.data for a in indicess])
     trace = np.empty((L + 1) * n, dtype=np.int64)
-    lib().gso_metapath_walk(ip, ix, _p(metapath), _c64(L), _p(seeds), _c64(n), _cu64(seed),
+    nn = np.array([a.size - 1 for a in indptrs], dtype=np.int64)
+    lib().gso_metapath_walk(ip, ix, _p(nn), _p(metapath), _c64(L), _p(seeds), _c64(n), _cu64(seed),
                             _p(replay), _p(trace))
     return trace
 

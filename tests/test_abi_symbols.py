@@ -36,15 +36,16 @@ def test_status_strings_and_argument_errors_without_a_gpu():
     lib = capi.lib()
     assert lib.gs_version() >= 100
     assert lib.gs_status_string(0) == b"ok"
-    st = lib.gs_slice_count(None, None, 8, ctypes.c_int64(4), None, None, ctypes.c_size_t(0), None)
+    st = lib.gs_slice_count(None, ctypes.c_int64(4), None, 8, ctypes.c_int64(4), None, None,
+                            ctypes.c_size_t(0), None)
     assert st == -1 and b"gs_slice_count" in lib.gs_status_string(st)
     buf = (ctypes.c_int64 * 64)()
-    st = lib.gs_sample_count(buf, buf, 3, ctypes.c_int64(4), ctypes.c_int64(2), 0, buf, None,
-                             ctypes.c_size_t(0), None)
+    st = lib.gs_sample_count(buf, ctypes.c_int64(8), buf, 3, ctypes.c_int64(4), ctypes.c_int64(2), 0,
+                             buf, None, ctypes.c_size_t(0), None)
     assert st == -1 and b"id_bytes" in lib.gs_status_string(st)
     # workspace too small / misaligned is reported, not executed
-    st = lib.gs_sample_count(buf, buf, 8, ctypes.c_int64(4), ctypes.c_int64(2), 0, buf, None,
-                             ctypes.c_size_t(0), None)
+    st = lib.gs_sample_count(buf, ctypes.c_int64(8), buf, 8, ctypes.c_int64(4), ctypes.c_int64(2), 0,
+                             buf, None, ctypes.c_size_t(0), None)
     assert st == -2
     assert lib.gs_sample_workspace_bytes(ctypes.c_int64(1000), ctypes.c_int64(5)) > 0
 

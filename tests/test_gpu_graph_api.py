@@ -1,0 +1,478 @@
+"""The reference's gtest suite (tests/*.cc of czkkkkkk/graph_sampling) re-expressed against
+torch.classes.gs_classes.Graph / HeteroGraph and torch.ops.gs_ops of this build, plus
+end-to-end sampler flows through the Matrix API checked against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import graph_sampling_amd as gs
+from graph_sampling_amd import _COO, _CSC, _CSR, _DCSR
+from oracle import oracle as O
+from tests.util import rmat_csc_np, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def I(dev):
+    return dict(dtype=torch.int64, device=dev)
+
+
+def F(dev):
+    return dict(dtype=torch.float32, device=dev)
+
+
+def graph20(dev):
+    A = gs.Graph(False)
+    indptr = torch.arange(0, 21, **I(dev)) * 5
+    indices = torch.arange(0, 100, **I(dev))
+    A._CAPI_LoadCSC(indptr, indices)
+    return A, indptr, indices
+
+
+def graph12(dev, csr=False):
+    A = gs.Graph(False)
+    indptr = torch.cat([torch.zeros(10, **I(dev)), torch.arange(0, 3, **I(dev)) * 2])
+    indices = torch.arange(1, 4, 2, **I(dev)).repeat(2)
+    (A._CAPI_LoadCSR if csr else A._CAPI_LoadCSC)(indptr, indices)
+    return A, indptr, indices
+
+
+# ---------------------------------------------------- test_colwise_slicing.cc
+def test_colwise_slicing_test1(dev):
+    A, _, _ = graph20(dev)
+    sub = A._CAPI_Slicing(torch.arange(0, 3, **I(dev)), 0, _CSC, _CSC, False)
+    indptr, indices, _ = sub._CAPI_GetCSC()
+    assert indptr.equal(torch.arange(0, 4, **I(dev)) * 5)
+    assert indices.equal(torch.arange(0, 15, **I(dev)))
+
+
+# --------------------------------------------------- test_colwise_sampling.cc
+def test_colwise_sampling_test1(dev):
+    A, indptr, indices = graph20(dev)
+    sub = A._CAPI_Sampling(0, 6, False, _CSC, _CSC)
+    p, i, _ = sub._CAPI_GetCSC()
+    assert p.equal(indptr) and i.equal(indices)
+
+
+@pytest.mark.parametrize("fanout", [6, 4])
+def test_colwise_sampling_test2_3(dev, fanout):
+    A, indptr, indices = graph20(dev)
+    sub = A._CAPI_Sampling(0, fanout, True, _CSC, _CSC)
+    p, i, _ = sub._CAPI_GetCSC()
+    assert p.equal(torch.arange(0, 21, **I(dev)) * fanout)
+    assert i.numel() == 20 * fanout and not i[:100].equal(indices[:i.numel()][:100])
+    assert torch.unique(i).numel() <= 100
+
+
+# ------------------------------------------------------------ test_relabel.cc
+def test_slicing_relabel_test1(dev):
+    A = gs.Graph(False)
+    A._CAPI_LoadCSCWithColIds(torch.arange(0, 20, **I(dev)), torch.arange(0, 21, **I(dev)) * 5,
+                              torch.arange(0, 100, **I(dev)))
+    sub = A._CAPI_Slicing(torch.arange(1, 4, **I(dev)), 0, _CSC, _CSC, True)
+    assert (A._CAPI_GetNumCols(), A._CAPI_GetNumRows()) == (20, 100)
+    assert (sub._CAPI_GetNumCols(), sub._CAPI_GetNumRows()) == (3, 15)
+    p, i, _ = sub._CAPI_GetCSC()
+    assert p.equal(torch.arange(0, 4, **I(dev)) * 5) and i.equal(torch.arange(0, 15, **I(dev)))
+
+
+def test_doubly_compressed_formats_are_rejected(dev):
+    # SlicingRelabel.test2 / RowwiseSlicing.test2 / CSC2DCSR.test1 use _DCSR, which this build omits
+    A, _, _ = graph12(dev)
+    with pytest.raises(RuntimeError, match="doubly-compressed"):
+        A._CAPI_Slicing(torch.arange(5, 6, **I(dev)), 1, _DCSR, _CSR, False)
+
+
+# ---------------------------------------------------- test_rowwise_slicing.cc
+def test_rowwise_slicing_test1(dev):
+    A, _, _ = graph20(dev)
+    sub = A._CAPI_Slicing(torch.arange(0, 100, 5, **I(dev)), 1, _CSC, _CSC, False)
+    p, i, _ = sub._CAPI_GetCSC()
+    assert p.equal(torch.arange(21, **I(dev))) and i.equal(torch.arange(20, **I(dev)))
+
+
+# ------------------------------------------------------- test_listsampling.cc
+def test_list_sampling(dev):
+    data = torch.arange(1000, **I(dev))
+    sel, idx = torch.ops.gs_ops._CAPI_ListSampling(data, 2000, False)
+    assert sel.equal(data)
+    sel, idx = torch.ops.gs_ops._CAPI_ListSampling(data, 2000, True)
+    assert sel.numel() == 2000 and not sel[:1000].equal(data) and torch.unique(sel).numel() <= 1000
+    sel, idx = torch.ops.gs_ops._CAPI_ListSampling(data, 999, False)
+    assert sel.numel() == 999 and torch.unique(sel).numel() == 999
+
+
+# ------------------------------------------------------ test_graph_compute.cc
+def test_graph_sum_test1_to_4(dev):
+    A, _, _ = graph20(dev)
+    assert A._CAPI_Sum(0, 1, _CSC).equal(torch.ones(20, **F(dev)) * 5)
+    assert A._CAPI_Sum(0, 2, _CSC).equal(torch.ones(20, **F(dev)) * 5)
+    data = torch.arange(1, 6, **F(dev))
+    A._CAPI_SetData(data.repeat(20))
+    assert A._CAPI_Sum(0, 1, _CSC).equal(data.sum().repeat(20))
+    assert A._CAPI_Sum(0, 2, _CSC).equal(data.pow(2).sum().repeat(20))
+
+
+@pytest.mark.parametrize("fmt", [_CSR, _COO])
+def test_graph_sum_test5_6(dev, fmt):
+    A, _, _ = graph12(dev)
+    A._CAPI_SetData(torch.arange(3, 7, **F(dev)))
+    if fmt == _CSR:
+        A._CAPI_CSC2CSR()
+    expected = torch.tensor([0, 8, 0, 10] + [0] * 8, **F(dev))
+    assert A._CAPI_Sum(1, 1, fmt).equal(expected)
+
+
+def test_graph_sum_test7(dev):
+    A, _, _ = graph12(dev)
+    A._CAPI_SetData(torch.arange(3, 7, **F(dev)))
+    A._CAPI_Slicing(torch.arange(10, 12, **I(dev)), 0, _CSC, _CSC, False)
+    assert A._CAPI_Sum(1, 1, _CSR).equal(torch.tensor([0, 8, 0, 10] + [0] * 8, **F(dev)))
+
+
+@pytest.mark.parametrize("fmt", [_CSC, _COO])
+def test_graph_div(dev, fmt):
+    A, _, _ = graph20(dev)
+    if fmt == _CSC:
+        out = A._CAPI_Divide(torch.ones(20, **F(dev)) * 10, 0, _CSC)._CAPI_GetData("default")
+        assert torch.isclose(out, torch.ones(100, **F(dev)) / 10).all()
+    divisor = torch.arange(1, 21, **F(dev))
+    out = A._CAPI_Divide(divisor, 0, fmt)._CAPI_GetData("default")
+    assert torch.isclose(out, torch.repeat_interleave(1 / divisor, 5)).all()
+
+
+@pytest.mark.parametrize("fmt", [_CSC, _COO])
+def test_graph_normalize_test1_to_3(dev, fmt):
+    A, _, _ = graph20(dev)
+    out = A._CAPI_Divide(A._CAPI_Sum(0, 1, _CSC), 0, _CSC)._CAPI_GetData("default")
+    assert torch.isclose(out, torch.ones(100, **F(dev)) / 5).all()
+    data = torch.arange(1, 6, **F(dev))
+    A._CAPI_SetData(data.repeat(20))
+    out = A._CAPI_Divide(A._CAPI_Sum(0, 1, fmt), 0, fmt)._CAPI_GetData("default")
+    assert torch.isclose(out, (data / data.sum()).repeat(20)).all()
+
+
+def test_graph_normalize_test4(dev):
+    A, _, _ = graph12(dev)
+    data = torch.arange(3, 7, **F(dev))
+    A._CAPI_SetData(data)
+    g = A._CAPI_Slicing(torch.arange(10, 12, **I(dev)), 0, _CSC, _CSC, False)
+    g = g._CAPI_Divide(g._CAPI_Sum(1, 1, _CSR), 1, _CSR)
+    expected = torch.flatten(data.reshape(2, 2) / data.reshape(2, 2).sum(0))
+    assert g._CAPI_GetData("default").equal(expected)
+
+
+@pytest.mark.parametrize("fmt", [_CSC, _COO])
+def test_graph_normalize_test5_6(dev, fmt):
+    A, _, _ = graph12(dev, csr=True)
+    data = torch.arange(3, 7, **F(dev))
+    A._CAPI_SetData(data)
+    g = A._CAPI_Slicing(torch.arange(10, 12, **I(dev)), 1, _CSR, _CSR, False)
+    g = g._CAPI_Divide(torch.ones(2, **F(dev)), 1, _CSR)
+    g = g._CAPI_Divide(g._CAPI_Sum(0, 1, fmt), 0, fmt)
+    expected = torch.flatten(data.reshape(2, 2) / data.reshape(2, 2).sum(0))
+    assert g._CAPI_GetData("default").equal(expected)
+
+
+def test_normalize_method(dev):
+    A, _, _ = graph20(dev)
+    data = torch.arange(1, 6, **F(dev))
+    A._CAPI_SetData(data.repeat(20))
+    out = A._CAPI_Normalize(0, _CSC)._CAPI_GetData("default")
+    assert torch.isclose(out, (data / data.sum()).repeat(20)).all()
+
+
+# ---------------------------------------------------------------- test_sddmm.cc
+@pytest.mark.parametrize("fmt", [_COO, _CSR, _CSC])
+def test_sddmm_add_coo_loaded(dev, fmt):
+    A = gs.Graph(False)
+    r = torch.arange(0, 100, **I(dev))
+    A._CAPI_LoadCOO(r, r.clone())
+    f = torch.arange(0, 100, **F(dev))
+    out = torch.zeros(100, **F(dev))
+    A._CAPI_SDDMM("add", f, f.clone(), out, 0, 2, fmt)
+    assert out.equal(f * 2)
+
+
+@pytest.mark.parametrize("fmt", [_COO, _CSR, _CSC])
+@pytest.mark.parametrize("with_col_ids", [False, True])
+def test_sddmm_add_csc_loaded(dev, fmt, with_col_ids):
+    if fmt == _CSR and not with_col_ids:
+        pytest.skip("LoadCSC sets num_rows = num_cols = 20 while rows reach 99: no valid CSR")
+    A = gs.Graph(False)
+    indptr = torch.arange(0, 21, **I(dev)) * 5
+    indices = torch.arange(0, 100, **I(dev))
+    if with_col_ids:
+        A._CAPI_LoadCSCWithColIds(torch.arange(2, 22, **I(dev)), indptr, indices)
+    else:
+        A._CAPI_LoadCSC(indptr, indices)
+    lhs = torch.arange(0, 100, **F(dev))
+    rhs = torch.arange(0, 20, **F(dev))
+    out = torch.zeros(100, **F(dev))
+    A._CAPI_SDDMM("add", lhs, rhs, out, 0, 2, fmt)
+    assert out.equal(lhs + torch.repeat_interleave(rhs, 5))
+
+
+def test_sddmm_unknown_op_raises(dev):
+    A, _, _ = graph20(dev)
+    with pytest.raises(RuntimeError, match="Unsupported SpMM/SDDMM binary operator"):
+        A._CAPI_SDDMM("pow", torch.zeros(100, **F(dev)), torch.zeros(20, **F(dev)),
+                      torch.zeros(100, **F(dev)), 0, 2, _COO)
+
+
+# ------------------------------------------------------ test_format_transform.cc
+def test_csc2csr_test1_and_csr2csc(dev):
+    A = gs.Graph(True)
+    col_ids = torch.arange(0, 20, **I(dev))
+    indptr = torch.arange(0, 21, **I(dev)) * 5
+    indices = torch.arange(0, 100, **I(dev))
+    col = torch.repeat_interleave(col_ids, 5)
+    A._CAPI_LoadCSCWithColIds(col_ids, indptr, indices)
+    A._CAPI_CSC2CSR()
+    _, _, _, row, c = A._CAPI_COOMetadata()
+    assert row.equal(indices) and c.equal(col)
+    assert A._CAPI_GetNumRows() == 100
+    assert A._CAPI_GetCOORows(True).equal(indices)
+    assert A._CAPI_AllValidNode().equal(indices)
+    A._CAPI_CSR2CSC()
+    p, i, _ = A._CAPI_GetCSC()
+    assert p.equal(indptr) and i.equal(indices)
+
+
+def test_csc2csr_test2(dev):
+    A = gs.Graph(True)
+    col_ids = torch.arange(0, 21, **I(dev))
+    indptr = torch.cat([torch.zeros(1, **I(dev)), torch.arange(0, 21, **I(dev))]) * 5
+    indices = torch.arange(2, 102, **I(dev))
+    A._CAPI_LoadCSCWithColIds(col_ids, indptr, indices)
+    A._CAPI_CSC2CSR()
+    assert A._CAPI_GetNumRows() == 102
+    assert A._CAPI_AllValidNode().equal(torch.arange(0, 102, **I(dev)))
+    _, _, _, row, c = A._CAPI_COOMetadata()
+    assert c.equal(torch.repeat_interleave(torch.arange(1, 21, **I(dev)), 5))
+
+
+def test_csc2csr_test3_eids(dev):
+    A, _, _ = graph12(dev)
+    A._CAPI_SetData(torch.arange(3, 7, **F(dev)))
+    A._CAPI_CSC2CSR()
+    # the CSR is reachable through Sum / GetData('row'); its edge order is the stable sort by row
+    assert A._CAPI_GetData("row").equal(torch.tensor([3, 5, 4, 6], **F(dev)))
+    assert A._CAPI_GetValidRows().equal(torch.tensor([1, 3], **I(dev)))
+
+
+# -------------------------------------------------- test_hetero_random_walk.cc
+def _hetero(dev, indptr2, indices2):
+    g1, g2 = gs.Graph(False), gs.Graph(False)
+    g1._CAPI_LoadCSC(torch.tensor([0, 0, 1, 2, 3], **I(dev)), torch.tensor([0, 1, 2], **I(dev)))
+    g2._CAPI_LoadCSC(torch.tensor(indptr2, **I(dev)), torch.tensor(indices2, **I(dev)))
+    hg = gs.HeteroGraph()
+    hg._CAPI_LoadFromHomo(["user", "item"], [("user", "follow", "user"), ("user", "view", "item")], [g1, g2])
+    return hg
+
+
+def test_random_walk_one_path(dev):
+    hg = _hetero(dev, [0, 1, 2, 3], [0, 1, 2])
+    seeds = torch.tensor([2, 1], **I(dev))
+    paths = hg._CAPI_MetapathRandomWalkFused(seeds, ["view", "follow", "follow"])
+    assert paths.shape == (2, 4)
+    assert paths.reshape(-1, 2).cpu().equal(torch.tensor([[2, 1], [2, 1], [1, 0], [0, -1]]))
+
+
+def test_random_walk_multi_path(dev):
+    hg = _hetero(dev, [0, 1, 3, 5], [0, 0, 1, 2, 3])
+    seeds = torch.tensor([2, 2, 1, 1, 0], **I(dev))
+    metapath = ["view", "follow", "follow"]
+    tr = hg._CAPI_MetapathRandomWalkFused(seeds, metapath).reshape(-1, 5).cpu().numpy()
+    for w in range(5):
+        for t, et in enumerate(metapath):
+            g = hg._CAPI_GetHomoGraph(et)
+            p, i = [x.cpu().numpy() for x in g._CAPI_GetCSC()[:2]]
+            s, d = tr[t, w], tr[t + 1, w]
+            assert d == -1 or d in i[p[s]:p[s + 1]]
+
+
+# ------------------------------------------------------ end-to-end sampler flows
+def _rmat_matrix(dev, n_log, e_log, seed, with_data=False):
+    indptr, indices = rmat_csc_np(1 << n_log, 1 << e_log, seed=seed)
+    m = gs.Matrix()
+    data = None
+    if with_data:
+        data = (1.0 - np.random.default_rng(seed).random(indices.size)).astype(np.float32)
+    m.load_csc(to_dev(indptr, dev), to_dev(indices, dev), None if data is None else to_dev(data, dev))
+    return m, indptr, indices, data
+
+
+@pytest.mark.parametrize("algo", [0, 1])
+def test_graphsage_fused_flow_matches_oracle(dev, algo):
+    """examples/graphsage: fused_columnwise_slicing_sampling + relabel per layer."""
+    m, indptr, indices, _ = _rmat_matrix(dev, 13, 17, 1)
+    torch.ops.gs_ops._CAPI_SetSampleAlgo(algo)
+    try:
+        seeds = np.random.default_rng(0).permutation(1 << 13)[:256].astype(np.int64)
+        d_seeds = to_dev(seeds, dev)
+        for layer, fanout in enumerate([10, 5]):
+            gs.set_seed(1000 + layer)
+            sub = m.fused_columnwise_slicing_sampling(d_seeds, fanout, False)
+            block = sub.to_dgl_block()
+            sp, _, rows, sel = O.sample_uniform(indptr, indices, seeds, fanout, False, seed=1000 + layer,
+                                                with_coo=False, algo=algo)
+            frontier, (rel,) = O.relabel([seeds, rows], [rows])
+            assert block["format"] == "csc" and block["num_dst"] == seeds.size
+            assert np.array_equal(block["indptr"].cpu().numpy(), sp)
+            assert np.array_equal(block["indices"].cpu().numpy(), rel)
+            assert np.array_equal(block["srcdata_ID"].cpu().numpy(), frontier)
+            assert block["num_src"] == frontier.size
+            assert np.array_equal(sub.all_indices().cpu().numpy(), frontier)
+            assert np.array_equal(sub.row_indices().cpu().numpy(), rows)
+            seeds, d_seeds = frontier, block["srcdata_ID"]
+    finally:
+        torch.ops.gs_ops._CAPI_SetSampleAlgo(0)
+
+
+def test_graphsage_nonfused_flow_matches_oracle(dev):
+    """A[:, seeds] -> columnwise_sampling -> all_indices / to_dgl_block (COO path)."""
+    m, indptr, indices, data = _rmat_matrix(dev, 12, 16, 2, with_data=True)
+    seeds = np.random.default_rng(1).permutation(1 << 12)[:200].astype(np.int64)
+    sliced = m[:, to_dev(seeds, dev)]
+    sp, coo, si, sel = O.slice_columns(indptr, indices, seeds)
+    assert np.array_equal(sliced.row_indices().cpu().numpy(), si)
+    assert np.array_equal(sliced.get_data().cpu().numpy(), data[sel])
+    gs.set_seed(77)
+    sampled = sliced.columnwise_sampling(7, False)
+    # sampling runs over every column of the sliced CSC (built from the column-sorted COO)
+    sp2, coo2, si2, sel2 = O.sample_uniform(sp, si, None, 7, False, seed=77)
+    block = sampled.to_dgl_block()
+    frontier, (rel_col, rel_row) = O.relabel([seeds, si2], [seeds[coo2], si2])
+    assert block["format"] == "coo"
+    assert np.array_equal(block["row"].cpu().numpy(), rel_row)
+    assert np.array_equal(block["col"].cpu().numpy(), rel_col)
+    assert np.array_equal(block["srcdata_ID"].cpu().numpy(), frontier)
+    assert np.array_equal(sampled.get_data().cpu().numpy(), data[sel][sel2])
+
+
+def test_weighted_sampling_flow(dev):
+    m, indptr, indices, data = _rmat_matrix(dev, 11, 15, 3, with_data=True)
+    gs.set_seed(5)
+    sub = m.columnwise_sampling(6, False, bias=to_dev(data, dev))
+    want = O.sample_weighted(indptr, indices, data, None, 6, seed=5)
+    _, _, _, row, col = sub._graph._CAPI_COOMetadata()
+    assert np.array_equal(row.cpu().numpy(), want[2]) and np.array_equal(col.cpu().numpy(), want[1])
+
+
+def test_ladies_flow_matches_oracle(dev):
+    """examples/ladies: U = P[:, seeds]; prob = U.sum(1, powk=2); weighted list sampling of rows;
+    subU = U[nodes, :]; divide by prob; normalise columns; relabel."""
+    m, indptr, indices, data = _rmat_matrix(dev, 12, 16, 4, with_data=True)
+    N = 1 << 12
+    seeds = np.random.default_rng(2).permutation(N)[:128].astype(np.int64)
+    U = m[:, to_dev(seeds, dev)]
+    prob = U.sum(axis=1, powk=2)
+    sp, coo, si, sel = O.slice_columns(indptr, indices, seeds)
+    want_prob = O.coo_sum(si, None, data[sel], 2, N)
+    np.testing.assert_allclose(prob.cpu().numpy(), want_prob, rtol=1e-5)
+
+    row_ids = U.row_ids(remove_isolated=False)
+    assert np.array_equal(row_ids.cpu().numpy(), np.arange(N))
+    gs.set_seed(31)
+    selected, idx = torch.ops.gs_ops._CAPI_ListSamplingWithProbs(row_ids, prob, 64, False)
+    w_sel, w_idx = O.list_sample_weighted(np.arange(N), prob.cpu().numpy(), 64, seed=31)
+    assert np.array_equal(idx.cpu().numpy(), w_idx) and np.array_equal(selected.cpu().numpy(), w_sel)
+    assert (want_prob[w_idx] > 0).all()
+
+    nodes = torch.cat([to_dev(seeds, dev), selected]).unique()
+    subU = U[nodes, :]
+    h_nodes = nodes.cpu().numpy()
+    # row slice on the CSR of U: edges of U whose row is in nodes, in CSR (row-major) order
+    r_ip, r_col, r_perm = O.coo2csc(si, coo, N, False)
+    s_ip, s_row, s_col, s_sel = O.slice_columns(r_ip, r_col, h_nodes)
+    assert subU.get_num_rows() == h_nodes.size and subU.get_num_edges() == s_col.size
+    w_data = data[sel][r_perm][s_sel]
+    assert np.array_equal(subU.get_data().cpu().numpy(), w_data)
+
+    div = subU.divide(prob[nodes], axis=1)
+    w_div = w_data / want_prob[h_nodes][s_row]
+    np.testing.assert_allclose(div.get_data().cpu().numpy(), w_div, rtol=1e-5)
+    norm = div.normalize(axis=0)
+    col_sum = np.bincount(s_col, weights=w_div.astype(np.float64), minlength=seeds.size)
+    np.testing.assert_allclose(norm.get_data().cpu().numpy(), w_div / col_sum[s_col], rtol=1e-4)
+
+    block = subU.to_dgl_block()
+    frontier, (rel_col, rel_row) = O.relabel([seeds, h_nodes[s_row]], [seeds[s_col], h_nodes[s_row]])
+    assert np.array_equal(block["srcdata_ID"].cpu().numpy(), frontier)
+    assert np.array_equal(block["row"].cpu().numpy(), rel_row)
+    assert np.array_equal(block["col"].cpu().numpy(), rel_col)
+
+
+def test_fastgcn_coo_row_slicing_flow(dev):
+    """examples/fastgcn/unbatching_training.py:18-31: _CAPI_slicing(selected, 1, _COO, _COO, False)."""
+    m, indptr, indices, _ = _rmat_matrix(dev, 11, 15, 5)
+    seeds = np.random.default_rng(3).permutation(1 << 11)[:100].astype(np.int64)
+    U = m[:, to_dev(seeds, dev)]
+    selected = np.random.default_rng(4).permutation(1 << 11)[:300].astype(np.int64)
+    sub = U._graph._CAPI_Slicing(to_dev(selected, dev), 1, _COO, _COO, False)
+    sp, coo, si, sel = O.slice_columns(indptr, indices, seeds)
+    k, o, s = O.row_slice_coo(si, coo, selected)
+    _, _, _, row, col = sub._CAPI_COOMetadata()
+    assert np.array_equal(row.cpu().numpy(), k) and np.array_equal(col.cpu().numpy(), o)
+    assert sub._CAPI_GetNumRows() == 300 and sub._CAPI_GetNumEdges() == k.size
+
+
+def test_random_walk_and_metapath_flow(dev):
+    m, indptr, indices, _ = _rmat_matrix(dev, 11, 15, 6)
+    seeds = np.random.default_rng(5).integers(0, 1 << 11, 500).astype(np.int64)
+    gs.set_seed(9)
+    tr = m.random_walk(to_dev(seeds, dev), 10)
+    assert tr.shape == (500, 11)  # memory is [11][500] (reference random_walk.cu:67)
+    assert np.array_equal(tr.reshape(-1).cpu().numpy(), O.random_walk(indptr, indices, seeds, 10, seed=9))
+    m2, ip2, ix2, _ = _rmat_matrix(dev, 11, 15, 7)
+    hm = gs.HeteroMatrix()
+    hm.load_from_homo(["a", "b"], [("a", "r0", "b"), ("b", "r1", "a")], [m, m2])
+    gs.set_seed(10)
+    tr = hm.metapath_random_walk_fused(to_dev(seeds, dev), ["r0", "r1", "r0", "r1"])
+    want = O.metapath_walk([indptr, ip2], [indices, ix2], [0, 1, 0, 1], seeds, seed=10)
+    assert np.array_equal(tr.reshape(-1).cpu().numpy(), want)
+    # the unfused per-step path (hetero_matrix.py:17-24): the -1 of a dead end is fed back in as a
+    # column id; it must come back as -1 again, never be dereferenced
+    steps = hm.metapath_random_walk(to_dev(seeds, dev), ["r0", "r1", "r0"]).cpu().numpy()
+    assert (steps[1] == -1).any()
+    graphs = [(indptr, indices), (ip2, ix2), (indptr, indices)]
+    for t, (ip, ix) in enumerate(graphs):
+        for w in range(500):
+            s, d = steps[t, w], steps[t + 1, w]
+            assert (d == -1) if s == -1 else (d == -1 or d in ix[ip[s]:ip[s + 1]])
+
+
+def test_gsddmm_ops(dev):
+    m, indptr, indices, _ = _rmat_matrix(dev, 10, 14, 8)
+    N, E = 1 << 10, indices.size
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((N, 64)).astype(np.float32)
+    y = rng.standard_normal((N, 64)).astype(np.float32)
+    col = np.repeat(np.arange(N), np.diff(indptr))
+    out = gs.ops.u_dot_v(m, to_dev(x, dev), to_dev(y, dev))
+    ref = np.einsum("ij,ij->i", x[indices].astype(np.float64), y[col].astype(np.float64))
+    scale = np.abs(x[indices] * y[col]).sum(1)
+    assert out.shape == (E, 1)
+    assert np.all(np.abs(out.cpu().numpy()[:, 0] - ref) <= 1e-5 * scale + 1e-6)
+    e = rng.random(E).astype(np.float32) + 0.5
+    u = rng.random(N).astype(np.float32) + 0.5
+    out = gs.ops.e_div_u(m, to_dev(e, dev), to_dev(u, dev))
+    np.testing.assert_allclose(out.cpu().numpy(), e / u[indices], rtol=1e-5)
+    out = gs.ops.u_sub_v(m, to_dev(u, dev), to_dev(u, dev), on_format=_CSC)
+    np.testing.assert_allclose(out.cpu().numpy(), u[indices] - u[col], rtol=1e-6, atol=1e-7)
+
+
+def test_errors_are_exceptions_not_aborts(dev):
+    A = gs.Graph(False)
+    with pytest.raises(RuntimeError, match="not aligned"):
+        A._CAPI_LoadCSCWithColIds(torch.arange(3, **I(dev)), torch.arange(3, **I(dev)), torch.arange(2, **I(dev)))
+    B = gs.Graph(False)
+    B._CAPI_LoadCSC(torch.arange(3), torch.arange(2))  # CPU tensors: the reference LOG(FATAL)s
+    with pytest.raises(RuntimeError, match="Not implemented warning"):
+        B._CAPI_Slicing(torch.arange(1), 0, _CSC, _CSC, False)
+    C, _, _ = graph20(dev)
+    with pytest.raises(RuntimeError, match="Not implementation"):
+        C._CAPI_Slicing(torch.arange(2, **I(dev)), 0, _CSC, _CSR, False)
+    with pytest.raises(RuntimeError, match="No implementation"):
+        C._CAPI_Sampling(1, 3, False, _CSC, _CSC)

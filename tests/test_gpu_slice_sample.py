@@ -197,3 +197,25 @@ def test_one_keepdim(dev, idt):
     want = O.sample_one_keepdim(indptr, indices, cols, replay=replay)
     for g, w in zip(got, want):
         assert np.array_equal(g.cpu().numpy().astype(np.int64), w)
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+def test_out_of_range_column_ids_are_empty_columns(dev, idt):
+    """A stray id (-1 from a dead-end step, or >= num_cols) is an empty column, never dereferenced."""
+    indptr, indices = rmat_csc_np(1 << 10, 1 << 14, seed=12)
+    n = 1 << 10
+    cols = np.random.default_rng(0).integers(0, n, size=600).astype(np.int64)
+    cols[::7] = -1
+    cols[3::11] = n
+    cols[5::13] = n + 12345
+    d_ip, d_ix, d_cols = to_dev(indptr, dev), to_dev(indices, dev, idt), to_dev(cols, dev, idt)
+    _cmp(_slice_gpu(d_ip, d_ix, d_cols, True), O.slice_columns(indptr, indices, cols, True))
+    for algo in ALGOS:
+        for replace in (False, True):
+            got = _sample_gpu(d_ip, d_ix, d_cols, 6, replace, seed=3, algo=algo)
+            _cmp(got, O.sample_uniform(indptr, indices, cols, 6, replace, seed=3, algo=algo))
+    got = capi.sample_one_keepdim(d_ip, d_ix, d_cols, seed=4)
+    want = O.sample_one_keepdim(indptr, indices, cols, seed=4)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy().astype(np.int64), w)
+    assert (want[1][::7] == -1).all()

@@ -15,7 +15,8 @@ def _tables(indptrs, indicess, dev, idt):
     d_ix = [to_dev(a, dev, idt) for a in indicess]
     ip_tab = torch.tensor([t.data_ptr() for t in d_ip], dtype=torch.int64, device=dev)
     ix_tab = torch.tensor([t.data_ptr() for t in d_ix], dtype=torch.int64, device=dev)
-    return d_ip, d_ix, ip_tab, ix_tab
+    nn_tab = torch.tensor([t.numel() - 1 for t in d_ip], dtype=torch.int64, device=dev)
+    return d_ip, d_ix, ip_tab, ix_tab, nn_tab
 
 
 def test_metapath_reference_unique_path(dev):
@@ -25,7 +26,7 @@ def test_metapath_reference_unique_path(dev):
     keep = _tables([indptr1, indptr2], [indices1, indices2], dev, torch.int64)
     metapath = np.array([1, 0, 0], dtype=np.int64)  # view, follow, follow
     seeds = np.array([2, 1], dtype=np.int64)
-    trace = capi.metapath_walk(keep[2], keep[3], torch.int64, to_dev(metapath, dev), to_dev(seeds, dev),
+    trace = capi.metapath_walk(keep[2], keep[3], keep[4], torch.int64, to_dev(metapath, dev), to_dev(seeds, dev),
                                seed=3)
     expected = np.array([2, 1, 2, 1, 1, 0, 0, -1], dtype=np.int64)  # step-major [4][2]
     assert np.array_equal(trace.cpu().numpy(), expected)
@@ -41,7 +42,7 @@ def test_metapath_reference_multi_path_edges_exist(dev):
     keep = _tables([indptr1, indptr2], [indices1, indices2], dev, torch.int64)
     metapath = np.array([1, 0, 0], dtype=np.int64)
     seeds = np.array([2, 2, 1, 1, 0], dtype=np.int64)
-    trace = capi.metapath_walk(keep[2], keep[3], torch.int64, to_dev(metapath, dev), to_dev(seeds, dev),
+    trace = capi.metapath_walk(keep[2], keep[3], keep[4], torch.int64, to_dev(metapath, dev), to_dev(seeds, dev),
                                seed=11).cpu().numpy().reshape(4, 5)
     for w in range(5):
         for t in range(3):
@@ -95,7 +96,7 @@ def test_metapath_walk_rmat(dev, idt):
     keep = _tables(indptrs, indicess, dev, idt)
     metapath = np.array([0, 1, 2, 1] * 4, dtype=np.int64)
     seeds = np.random.default_rng(3).integers(0, 1 << 11, size=4096).astype(np.int64)
-    got = capi.metapath_walk(keep[2], keep[3], idt, to_dev(metapath, dev), to_dev(seeds, dev, idt), seed=8)
+    got = capi.metapath_walk(keep[2], keep[3], keep[4], idt, to_dev(metapath, dev), to_dev(seeds, dev, idt), seed=8)
     want = O.metapath_walk(indptrs, indicess, metapath, seeds, seed=8)
     assert np.array_equal(got.cpu().numpy().astype(np.int64), want)
 
@@ -111,3 +112,13 @@ def test_walk_next_hop_chi_square(dev):
     counts = np.bincount(hop, minlength=d + 1)[1:].astype(np.float64)
     chi2 = ((counts - n / d) ** 2 / (n / d)).sum()
     assert chi2 < (d - 1) + 5 * np.sqrt(2 * (d - 1)), chi2
+
+
+def test_walk_out_of_range_seeds_die(dev):
+    indptr, indices = rmat_csc_np(1 << 10, 1 << 14, seed=13)
+    seeds = np.array([5, -1, 1 << 10, 7, (1 << 10) + 999, -7], dtype=np.int64)
+    got = capi.random_walk(to_dev(indptr, dev), to_dev(indices, dev), to_dev(seeds, dev), 4, seed=1)
+    want = O.random_walk(indptr, indices, seeds, 4, seed=1)
+    assert np.array_equal(got.cpu().numpy(), want)
+    tr = want.reshape(5, 6)
+    assert (tr[1:, [1, 2, 4, 5]] == -1).all()

@@ -162,3 +162,13 @@ def test_list_weighted_replay(dev):
     u = ((replay >> 8).astype(np.float64) + 1) / 2.0 ** 24
     ref = np.argsort(-(np.log2(u) / probs.astype(np.float64)), kind="stable")[:k]
     assert len(set(ref.tolist()) ^ set(w_idx.tolist())) <= 2
+
+
+def test_weighted_out_of_range_column_ids(dev):
+    indptr, indices = rmat_csc_np(1 << 10, 1 << 14, seed=14)
+    probs = np.random.default_rng(1).random(indices.size, dtype=np.float32) + 0.1
+    cols = np.array([3, -1, 1 << 10, 900, 1 << 20, 17], dtype=np.int64)
+    got = _weighted_gpu(dev, indptr, indices, probs, cols, 4, seed=2)
+    want = O.sample_weighted(indptr, indices, probs, cols, 4, seed=2)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
