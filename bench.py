@@ -4,8 +4,12 @@
 One step = one [15,10,5] minibatch over 1024 fresh seed nodes on a synthetic
 R-MAT graph: per layer a fused column slice + uniform sample without
 replacement, then unique/relabel of (seeds, sampled rows); the frontier feeds
-the next layer.  Everything runs through the C ABI of libgs_hip.so with the
-graph resident in HBM.  Prints ONE JSON line (sampled edges per second).
+the next layer.  The step is written against the drop-in Graph class (the
+reference's _CAPI_* method names), which calls the HIP kernels of libgs_hip.so
+through its C ABI; the graph is resident in HBM.  Prints ONE JSON line (sampled
+edges per second) carrying the roofline of the dominant kernel (timed with
+hipEvents on the launch stream by the library's own hook) and a host-core
+baseline of the same minibatches.
 """
 import argparse
 import ctypes
@@ -26,6 +30,9 @@ WORKLOADS = {
 FANOUTS = (15, 10, 5)
 BATCH = 1024
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per sampler launch read from hardware counters (FETCH_SIZE + WRITE_SIZE,
+# scaled by a copy kernel of known size); None until a counter run has been taken.
+TRAFFIC_BYTES_PER_LAUNCH = None
 
 
 def parse():
@@ -37,55 +44,107 @@ def parse():
     ap.add_argument("--cpu-steps", type=int, default=-1,
                     help="minibatches timed for the host-core baseline (-1: sized to ~15 s)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one plain device copy of the indices array (a kernel of known "
+                         "traffic to scale hardware byte counters by)")
     return ap.parse_args()
 
 
-class HipEvents:
-    """hipEvent pairs on the stream the kernels run on (torch's current stream)."""
+class KernelTimer:
+    """The library's launch-site timing hook: hipEvent pairs around every launch of
+    one named site, recorded on the stream the kernel is launched on."""
 
-    def __init__(self):
-        self.hip = ctypes.CDLL("libamdhip64.so")
+    def __init__(self, lib):
+        self.lib = lib
+        lib.gs_profile_enable.argtypes = [ctypes.c_char_p]
+        lib.gs_profile_collect.argtypes = [ctypes.POINTER(ctypes.c_double),
+                                           ctypes.POINTER(ctypes.c_int64),
+                                           ctypes.POINTER(ctypes.c_double), ctypes.c_int64]
 
-    def create(self):
-        ev = ctypes.c_void_p()
-        assert self.hip.hipEventCreate(ctypes.byref(ev)) == 0
-        return ev
+    def enable(self, site):
+        assert self.lib.gs_profile_enable(site.encode() if site else None) == 0
 
-    def record(self, ev, stream):
-        assert self.hip.hipEventRecord(ev, ctypes.c_void_p(stream)) == 0
-
-    def elapsed_ms(self, a, b):
-        ms = ctypes.c_float()
-        assert self.hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
-        return ms.value
+    def collect(self):
+        total = ctypes.c_double()
+        n = ctypes.c_int64()
+        per = (ctypes.c_double * 4096)()
+        assert self.lib.gs_profile_collect(ctypes.byref(total), ctypes.byref(n), per, 4096) == 0
+        return total.value, n.value, list(per[:n.value])
 
 
-def minibatch(capi, torch, indptr, indices, seeds, step_seed):
-    """One GraphSAGE minibatch.  Returns (#sampled edges, per-layer sizes, final frontier)."""
+# launch sites of one minibatch step and the bytes each launch must move at the
+# least (id_bytes b; S seeds, E sampled edges, M = S + E items, U unique ids):
+#   sample_floyd  : per seed  column id b + two offsets 16 + output offset 8,
+#                   per edge  neighbour gather b + sub_indices b + select_index 8
+#   table_insert  : per item  id b + one 8-byte slot read-modify-write 16 + slot index 4
+#   unique_finish : per item  slot index 4 + slot 8 + rank 8, relabeled id b, frontier b per U
+SITES = ("sample_floyd", "table_insert", "unique_finish", "scan_tile_sums", "scan_apply",
+         "table_init")
+
+
+def floyd_bytes(b, S, E):
+    return S * (b + 24) + E * (2 * b + 8)
+
+
+def insert_bytes(b, S, E):
+    return (S + E) * (b + 20)
+
+
+SITE_BYTES = {"sample_floyd": floyd_bytes, "table_insert": insert_bytes}
+SITE_KERNEL = {
+    "sample_floyd": "sample_floyd_kernel (fused column slice + uniform sample, all three layers)",
+    "table_insert": "table_insert_kernel (hash insert of seeds + sampled rows, all three layers)",
+}
+
+
+def minibatch(graph, seeds):
+    """One GraphSAGE minibatch through the drop-in Graph API, exactly the calls of the
+    reference's examples (examples/graphsage/batching.py:125-138): per layer
+    _CAPI_FusedColumnwiseSlicingSampling(seeds, fanout, False) then _CAPI_Relabel().
+    Returns (#sampled edges, per-layer (S, E, U), final frontier)."""
     total = 0
     sizes = []
-    for layer, k in enumerate(FANOUTS):
-        sub_indptr, sub_indices, select_index, _ = capi.sample_uniform(
-            indptr, indices, seeds, k, False, seed=step_seed * 16 + layer)
-        E = int(sub_indptr[-1].item())
-        rows = sub_indices[:E]
-        frontier, num, outs = capi.unique_relabel([seeds, rows], [rows])
-        U = int(num.item())
-        sizes.append((seeds.numel(), E, U))
+    for k in FANOUTS:
+        sub = graph._CAPI_FusedColumnwiseSlicingSampling(seeds, k, False)
+        frontier, num_src, num_dst, indptr, indices, e_ids, fmt = sub._CAPI_Relabel()
+        E = indices.numel()
+        sizes.append((num_dst, E, num_src))
         total += E
-        seeds = frontier[:U]
+        seeds = frontier
     return total, sizes, seeds
 
 
-def cpu_minibatch(O, np, indptr, indices, seeds, step_seed):
+def cpu_minibatch(O, np, indptr, indices, seeds, step):
     total = 0
     for layer, k in enumerate(FANOUTS):
         sub_indptr, _, sub_indices, _ = O.sample_uniform(indptr, indices, seeds, k, False,
-                                                         seed=step_seed * 16 + layer, with_coo=False)
+                                                         seed=step * len(FANOUTS) + layer,
+                                                         with_coo=False)
         frontier, _ = O.relabel([seeds, sub_indices], [sub_indices])
         total += int(sub_indptr[-1])
         seeds = frontier
-    return total
+    return total, seeds
+
+
+def saturated(torch, graph, timer, nodes, idt, dev, b):
+    """The same sampler launch at a size that fills the chip (4M seed columns drawn with
+    repetition, fanout 10): what the kernel reaches once launch latency is amortised."""
+    S = 1 << 22
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    cols = torch.randint(0, nodes, (S,), generator=gen, device=dev).to(idt)
+    timer.enable("sample_floyd")
+    E = 0
+    for _ in range(4):
+        sub = graph._CAPI_FusedColumnwiseSlicingSampling(cols, 10, False)
+        E = sub._CAPI_GetNumEdges()
+    torch.cuda.synchronize()
+    ms, n, per = timer.collect()
+    timer.enable("")
+    t = min(per[1:]) * 1e-3
+    achieved = floyd_bytes(b, S, E) / t / 1e9
+    return {"seeds": S, "fanout": 10, "sampled_edges": E, "launch_us": t * 1e6,
+            "achieved": achieved, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS}
 
 
 def main():
@@ -96,12 +155,13 @@ def main():
         sys.exit(2)
     import numpy as np
     import torch
+    import graph_sampling_amd as gs
     from graph_sampling_amd import capi, rmat
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
-    capi.lib()  # fail loudly when the HIP library is missing
+    timer = KernelTimer(capi.lib())  # fails loudly when the HIP library is missing
     dev = torch.device("cuda:0")
     nodes, edges, idt = WORKLOADS[args.workload]
     idt = getattr(torch, idt)
@@ -110,6 +170,12 @@ def main():
     indptr, indices = rmat.rmat_csc(nodes, edges, seed=0, device=dev, index_dtype=idt)
     torch.cuda.synchronize()
     gen_s = time.perf_counter() - t0
+
+    graph = gs.Graph(False)
+    graph._CAPI_LoadCSC(indptr, indices)
+    if args.calibration_copy:
+        torch.empty_like(indices).copy_(indices)
+        torch.cuda.synchronize()
 
     gen = torch.Generator(device=dev)
     gen.manual_seed(2)
@@ -120,24 +186,46 @@ def main():
     seed_sets = [fresh_seeds() for _ in range(args.warmup + args.steps)]
     torch.cuda.synchronize()
 
+    # the Graph API draws seed, seed+1, ... per sampling call: 3 calls per step
+    torch.ops.gs_ops._CAPI_SetSeed(0)
     for i in range(args.warmup):
-        minibatch(capi, torch, indptr, indices, seed_sets[i], i)
+        minibatch(graph, seed_sets[i])
     torch.cuda.synchronize()
 
+    # which launch site holds the most GPU time: one untimed step per site
+    site_ms = {}
+    probe = seed_sets[0]
+    for site in SITES:
+        timer.enable(site)
+        minibatch(graph, probe)
+        torch.cuda.synchronize()
+        site_ms[site] = timer.collect()[0]
+    dominant = max(SITE_BYTES, key=lambda k: site_ms[k])
+
+    torch.ops.gs_ops._CAPI_SetSeed(args.warmup * len(FANOUTS))
+    timer.enable(dominant)
     lat = []
     sampled = 0
     layer_sizes = None
+    first = None
+    algo_bytes = 0
+    b = 4 if idt == torch.int32 else 8
+    torch.cuda.synchronize()
     t_begin = time.perf_counter()
     for i in range(args.steps):
         t1 = time.perf_counter()
-        n, sizes, _ = minibatch(capi, torch, indptr, indices, seed_sets[args.warmup + i],
-                                args.warmup + i)
+        n, sizes, frontier = minibatch(graph, seed_sets[args.warmup + i])
         torch.cuda.synchronize()
         lat.append(time.perf_counter() - t1)
         sampled += n
         layer_sizes = sizes
+        algo_bytes += sum(SITE_BYTES[dominant](b, S, E) for S, E, _ in sizes)
+        if first is None:
+            first = (n, frontier)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t_begin
+    k_ms, k_launches, _ = timer.collect()
+    timer.enable("")
     lat.sort()
     p50 = lat[len(lat) // 2] * 1e3
     p90 = lat[min(len(lat) - 1, int(len(lat) * 0.9))] * 1e3
@@ -163,20 +251,43 @@ def main():
         "roofline": None,
         "cpu_baseline": None,
     }
+    if k_launches:
+        avg_s = k_ms * 1e-3 / k_launches
+        achieved = algo_bytes / k_launches / avg_s / 1e9
+        out["roofline"] = {
+            "bound": "hbm",
+            "kernel": SITE_KERNEL[dominant],
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+            "launches": k_launches,
+            "avg_launch_us": avg_s * 1e6,
+            "algorithmic_bytes_per_launch": algo_bytes / k_launches,
+            "share_of_gpu_time_by_site_ms": {k: round(v, 4) for k, v in site_ms.items()},
+        }
+        out["roofline_saturated"] = saturated(torch, graph, timer, nodes, idt, dev, b)
 
     if not args.no_cpu:
         from oracle import oracle as O
         h_indptr = indptr.cpu().numpy()
         h_indices = indices.cpu().numpy().astype(np.int64)
         h_seeds = [s.cpu().numpy().astype(np.int64) for s in seed_sets[args.warmup:]]
-        cpu_minibatch(O, np, h_indptr, h_indices, h_seeds[0], args.warmup)  # warm
+        # the checker: step 0 of the timed region must agree with the oracle bit for bit
+        n_ref, f_ref = cpu_minibatch(O, np, h_indptr, h_indices, h_seeds[0], args.warmup)
+        if n_ref != first[0] or not np.array_equal(f_ref, first[1].cpu().numpy()):
+            print("bench.py: GPU minibatch differs from the oracle on the same seeds and draws",
+                  file=sys.stderr)
+            sys.exit(1)
         t1 = time.perf_counter()
         done = 0
         cpu_edges = 0
         budget = 15.0
         limit = args.cpu_steps if args.cpu_steps > 0 else len(h_seeds)
         while done < limit and (args.cpu_steps > 0 or time.perf_counter() - t1 < budget):
-            cpu_edges += cpu_minibatch(O, np, h_indptr, h_indices, h_seeds[done], args.warmup + done)
+            cpu_edges += cpu_minibatch(O, np, h_indptr, h_indices, h_seeds[done],
+                                       args.warmup + done)[0]
             done += 1
         cpu_s = time.perf_counter() - t1
         out["cpu_baseline"] = {
@@ -185,7 +296,8 @@ def main():
             "cores": O.num_threads(),
             "kind": "port",
             "sample": "%d of the same minibatches (same seeds and draws) through the C oracle, "
-                      "OpenMP over rows; unique is single-threaded" % done,
+                      "OpenMP over rows; unique is single-threaded; step 0 compared with the "
+                      "GPU result bit for bit" % done,
             "ms_per_step": cpu_s / done * 1e3,
         }
     print(json.dumps(out))

@@ -39,6 +39,21 @@ inline int check_launch(const char* what) {
 
 inline bool valid_id_bytes(int b) { return b == 4 || b == 8; }
 
+// ------------------------------------------------------------- profiling ----
+// Optional per-kernel timing for benchmarks: when gs_profile_enable(name) names
+// this launch site, the launch is bracketed by a hipEvent pair on its stream
+// (see gs_profile_collect).  Off by default: one relaxed load per launch.
+void profile_begin(const char* name, hipStream_t stream, int* slot);
+void profile_end(hipStream_t stream, int slot);
+struct ProfileScope {
+  hipStream_t stream;
+  int slot = -1;
+  ProfileScope(const char* name, hipStream_t s) : stream(s) { profile_begin(name, s, &slot); }
+  ~ProfileScope() {
+    if (slot >= 0) profile_end(stream, slot);
+  }
+};
+
 // Carves 256-byte aligned pieces out of the caller's workspace.
 struct Carver {
   char* base;
@@ -295,9 +310,13 @@ inline int exclusive_scan(F f, int64_t n, int64_t* out, int64_t* tile_ws, hipStr
                        static_cast<const int64_t*>(nullptr), out);
     return check_launch("scan_apply");
   }
-  hipLaunchKernelGGL(scan_tile_sums_kernel<F>, dim3(static_cast<unsigned>(tiles)),
-                     dim3(kScanThreads), 0, stream, f, n, tile_ws, out);
+  {
+    ProfileScope prof("scan_tile_sums", stream);
+    hipLaunchKernelGGL(scan_tile_sums_kernel<F>, dim3(static_cast<unsigned>(tiles)),
+                       dim3(kScanThreads), 0, stream, f, n, tile_ws, out);
+  }
   if (tiles <= kScanSelfPrefixTiles) {
+    ProfileScope prof("scan_apply", stream);
     hipLaunchKernelGGL((scan_apply_kernel<F, true>), dim3(static_cast<unsigned>(tiles)),
                        dim3(kScanThreads), 0, stream, f, n, static_cast<const int64_t*>(tile_ws),
                        out);

@@ -482,6 +482,7 @@ int sample_fill_impl(const SampleArgs<IdT>& a, int replace, int algo, hipStream_
     return check_launch("sample_replace");
   }
   if (algo == GS_SAMPLE_AUTO && a.k <= kFloydMaxK) {
+    ProfileScope prof("sample_floyd", stream);
     const int g = a.k <= 8 ? 8 : (a.k <= 16 ? 16 : (a.k <= 32 ? 32 : 64));
     const unsigned fgrid =
         static_cast<unsigned>((a.S * g + kFloydThreads - 1) / kFloydThreads);

@@ -134,6 +134,7 @@ int sddmm_dispatch(int op, const SddmmArgs& a, hipStream_t st) {
   if (op == GS_OP_DOT && !a.lhs_off && !a.rhs_off && a.out_len == 1 && a.R % 4 == 0 && a.R >= 16 &&
       aligned) {
     const unsigned grid = static_cast<unsigned>((a.E * kDotGroup + kThreads - 1) / kThreads);
+    ProfileScope prof("sddmm_dot", st);
     hipLaunchKernelGGL(sddmm_dot_rows_kernel, dim3(grid), dim3(kThreads), 0, st, a);
     return check_launch("sddmm_dot");
   }

@@ -282,14 +282,20 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   }
   qs.n = n_query;
 
-  hipLaunchKernelGGL((table_init_kernel<T>), dim3(blocks_for(cap, kThreads)), dim3(kThreads), 0,
-                     stream, t, cap);
-  if (M > 0)
+  {
+    ProfileScope prof("table_init", stream);
+    hipLaunchKernelGGL((table_init_kernel<T>), dim3(blocks_for(cap, kThreads)), dim3(kThreads), 0,
+                       stream, t, cap);
+  }
+  if (M > 0) {
+    ProfileScope prof("table_insert", stream);
     hipLaunchKernelGGL((table_insert_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
                        0, stream, x, M, t, pos);
+  }
   GS_RETURN_IF_ERROR(check_launch("unique insert"));
   IsFirst<T> f{t, pos};
   GS_RETURN_IF_ERROR(exclusive_scan(f, M, prefix, tiles, stream));
+  ProfileScope prof("unique_finish", stream);
   hipLaunchKernelGGL((finish_kernel<IdT, T>), dim3(blocks_for(M + Q, kThreads)), dim3(kThreads), 0,
                      stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, qs, Q);
   return check_launch("unique_relabel");

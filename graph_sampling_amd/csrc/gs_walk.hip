@@ -97,6 +97,7 @@ int gs_random_walk(const int64_t* indptr, int64_t num_nodes, const void* indices
   if (n == 0) return GS_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(blocks_for(n, kThreads));
+  ProfileScope prof("random_walk", st);
   if (id_bytes == 8)
     hipLaunchKernelGGL((random_walk_kernel<int64_t>), grid, dim3(kThreads), 0, st, indptr,
                        static_cast<const int64_t*>(indices), num_nodes,
@@ -122,6 +123,7 @@ int gs_metapath_walk(const int64_t* const* all_indptr, const void* const* all_in
   if (n == 0) return GS_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(blocks_for(n, kThreads));
+  ProfileScope prof("metapath_walk", st);
   if (id_bytes == 8)
     hipLaunchKernelGGL((metapath_walk_kernel<int64_t>), grid, dim3(kThreads), 0, st, all_indptr,
                        reinterpret_cast<const int64_t* const*>(all_indices), all_num_nodes, metapath,

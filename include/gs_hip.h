@@ -56,6 +56,18 @@ const char* gs_status_string(int status);
 /* Library version (major*10000 + minor*100 + patch). */
 int gs_version(void);
 
+/* Optional timing of one launch site, for benchmarks (no counterpart in the
+ * reference).  gs_profile_enable("name") makes every later launch of that site
+ * record a hipEvent pair on its stream (up to 4096 launches); NULL or ""
+ * disables.  Sites: "sample_floyd", "table_init", "table_insert",
+ * "unique_finish", "scan_tile_sums", "scan_apply", "random_walk",
+ * "metapath_walk", "sddmm_dot".  gs_profile_collect waits for the recorded
+ * events, returns their summed duration and count (and, when per_launch_ms is
+ * given, the first `cap` individual durations in launch order) and clears the
+ * ring.  The events are created by the library and live until the process ends. */
+int gs_profile_enable(const char* launch_site);
+int gs_profile_collect(double* total_ms, int64_t* launches, double* per_launch_ms, int64_t cap);
+
 typedef enum gs_op {
   GS_OP_ADD = 0, GS_OP_SUB = 1, GS_OP_MUL = 2, GS_OP_DIV = 3,
   GS_OP_COPY_LHS = 4, GS_OP_COPY_RHS = 5, GS_OP_DOT = 6
