@@ -30,9 +30,11 @@ WORKLOADS = {
 FANOUTS = (15, 10, 5)
 BATCH = 1024
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per sampler launch read from hardware counters (FETCH_SIZE + WRITE_SIZE,
-# scaled by a copy kernel of known size); None until a counter run has been taken.
-TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per launch of the roofline kernel on the default workload, read from hardware
+# counters (2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE; the factors come from a device copy of
+# known size): profiles/sample_floyd_rmat-2.45M-124M_hbm_counters.txt.  The counters cannot
+# be read from inside this process, so the figure is carried here.
+TRAFFIC_BYTES_PER_LAUNCH = {("rmat-2.45M-124M", "sample_floyd"): 12343562}
 
 
 def parse():
@@ -261,7 +263,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, dominant)),
             "launches": k_launches,
             "avg_launch_us": avg_s * 1e6,
             "algorithmic_bytes_per_launch": algo_bytes / k_launches,
