@@ -31,6 +31,7 @@ def lib():
         for name in ("gs_slice_workspace_bytes", "gs_sample_workspace_bytes",
                      "gs_sample_weighted_workspace_bytes", "gs_list_sample_workspace_bytes",
                      "gs_unique_workspace_bytes", "gs_row_slice_workspace_bytes",
+                     "gs_sample_fused_state_bytes",
                      "gs_coo2csc_workspace_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
@@ -189,6 +190,82 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace, seed=0, replay=
     return sub_indptr, sub_indices, select_index, coo_col
 
 
+_fused_state = {}
+
+
+def fused_state(nbytes, device):
+    """The zero-filled state buffer of gs_sample_uniform_fused for the current stream: cleared
+    once when (re)allocated, left zero by every call."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _fused_state.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.zeros(max(int(nbytes), 4096), dtype=torch.uint8, device=device)
+        _fused_state[key] = buf
+    return buf
+
+
+class Mailbox:
+    """gs_mailbox in pinned host memory plus the host side of the protocol."""
+
+    def __init__(self):
+        self.buf = torch.zeros(2, dtype=torch.int64).pin_memory()
+        self.next_ticket = 1
+
+    def ptr(self):
+        return ctypes.c_void_p(self.buf.data_ptr())
+
+    def ticket(self):
+        t = self.next_ticket
+        self.next_ticket += 1
+        return t
+
+    def wait(self, ticket, device, spins=200_000_000):
+        words = (ctypes.c_int64 * 2).from_address(self.buf.data_ptr())
+        stream = torch.cuda.current_stream(device)
+        n = 0
+        while words[1] != ticket:
+            n += 1
+            if n % 4096 == 0 and stream.query() and words[1] != ticket:
+                raise GsError("the stream drained without posting mailbox ticket %d" % ticket)
+            if n > spins:
+                raise GsError("timed out waiting for mailbox ticket %d" % ticket)
+        return int(words[0])
+
+
+def sample_uniform_fused(indptr, indices, column_ids, fanout, replace, seed=0, replay=None,
+                         replay_ptr=None, with_coo=False, mailbox=None):
+    """gs_sample_uniform_fused: one launch.  Same return shape as sample_uniform; with a
+    Mailbox also returns the ticket to wait on as a fifth element."""
+    _need(indptr, torch.int64, "indptr")
+    idb = _ids(indices, "indices")
+    dev = indptr.device
+    if column_ids is None:
+        S = indptr.numel() - 1
+    else:
+        _ids(column_ids, "column_ids", like=indices)
+        S = column_ids.numel()
+    if replay is not None:
+        _replay(replay)
+        _need(replay_ptr, torch.int64, "replay_ptr")
+    sub_indptr = torch.empty(S + 1, dtype=torch.int64, device=dev)
+    cap = S * int(fanout)
+    sub_indices = torch.empty(cap, dtype=indices.dtype, device=dev)
+    select_index = torch.empty(cap, dtype=torch.int64, device=dev)
+    coo_col = torch.empty(cap, dtype=indices.dtype, device=dev) if with_coo else None
+    state = fused_state(lib().gs_sample_fused_state_bytes(_i64(S)), dev)
+    ticket = mailbox.ticket() if mailbox is not None else 0
+    _check(lib().gs_sample_uniform_fused(
+        _ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(column_ids), idb, _i64(S),
+        _i64(fanout), int(bool(replace)), _u64(seed), _ptr(replay), _ptr(replay_ptr),
+        _ptr(sub_indptr), _ptr(sub_indices), _ptr(select_index), _ptr(coo_col), _i64(cap),
+        _ptr(state), ctypes.c_size_t(state.numel()),
+        mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0), _i64(ticket), _stream(dev)),
+        "gs_sample_uniform_fused")
+    if mailbox is not None:
+        return sub_indptr, sub_indices, select_index, coo_col, ticket
+    return sub_indptr, sub_indices, select_index, coo_col
+
+
 def sample_one_keepdim(indptr, indices, column_ids, seed=0, replay=None):
     _need(indptr, torch.int64, "indptr")
     idb = _ids(indices, "indices")
@@ -270,11 +347,12 @@ class _Span(ctypes.Structure):
     _fields_ = [("ptr", ctypes.c_void_p), ("n", ctypes.c_int64)]
 
 
-def unique_relabel(mapping, queries):
-    """gs_unique_relabel.  mapping / queries: lists of 1-D id tensors (one dtype).
+def unique_relabel(mapping, queries, mailbox=None):
+    """gs_unique_relabel[_notify].  mapping / queries: lists of 1-D id tensors (one dtype).
 
     Returns (frontier_buf, num_unique_dev, [relabelled query tensors]); frontier_buf has
-    capacity sum(len(mapping)) and num_unique_dev is a 1-element int64 device tensor."""
+    capacity sum(len(mapping)) and num_unique_dev is a 1-element int64 device tensor.  With a
+    Mailbox the ticket to wait on is appended."""
     dev = mapping[0].device
     idb = _ids(mapping[0], "mapping[0]")
     for i, t in enumerate(list(mapping[1:]) + list(queries)):
@@ -290,6 +368,14 @@ def unique_relabel(mapping, queries):
     q_arr = QArr(*[_Span(t.data_ptr(), t.numel()) for t in queries]) if queries else QArr()
     o_arr = OutArr(*[t.data_ptr() for t in outs]) if queries else OutArr()
     ws = workspace(lib().gs_unique_workspace_bytes(_i64(M)), dev)
+    if mailbox is not None:
+        ticket = mailbox.ticket()
+        _check(lib().gs_unique_relabel_notify(m_arr, len(mapping), q_arr, o_arr, len(queries), idb,
+                                              _ptr(frontier), _ptr(num_unique), _ptr(ws),
+                                              ctypes.c_size_t(ws.numel()), mailbox.ptr(),
+                                              _i64(ticket), _stream(dev)),
+               "gs_unique_relabel_notify")
+        return frontier, num_unique, outs, ticket
     _check(lib().gs_unique_relabel(m_arr, len(mapping), q_arr, o_arr, len(queries), idb,
                                    _ptr(frontier), _ptr(num_unique), _ptr(ws),
                                    ctypes.c_size_t(ws.numel()), _stream(dev)), "gs_unique_relabel")

@@ -330,4 +330,108 @@ inline int exclusive_scan(F f, int64_t n, int64_t* out, int64_t* tile_ws, hipStr
   return check_launch("scan");
 }
 
+
+// ------------------------------------------- single-pass scan (look-back) ----
+// Chained-scan building blocks for kernels that count, scan and write in one
+// launch.  Every tile owns one 64-bit status word {flag:2 | value:62}: flag 0 =
+// nothing yet, 1 = the tile's own sum, 2 = the inclusive prefix up to and
+// including the tile.  A tile publishes its sum, then wave 0 walks back over its
+// predecessors 64 at a time until it meets an inclusive prefix.
+//
+// Tiles take their number from an atomic ticket, so every predecessor of a
+// tile is already resident on the device and publishes without waiting on
+// anyone: the walk cannot deadlock.  The wait is bounded all the same: after
+// kLookbackSpinLimit polls the tile gives up, raises *error and carries on with
+// a zero, so every wave reaches the end of the kernel.
+//
+// The status words, the ticket and the error word must be zero when the kernel
+// starts.
+struct LookbackState {
+  unsigned long long* status;  // one per tile
+  unsigned int* ticket;
+  unsigned int* done;   // tiles that have finished (for self-cleaning users)
+  unsigned int* error;
+};
+
+constexpr unsigned long long kLbSum = 1ull << 62;
+constexpr unsigned long long kLbInclusive = 2ull << 62;
+constexpr unsigned long long kLbValue = (1ull << 62) - 1;
+constexpr int kLookbackSpinLimit = 1 << 20;
+
+inline size_t lookback_state_bytes(int64_t tiles) { return padded((tiles > 0 ? tiles : 1) * 8) + 256; }
+
+inline LookbackState carve_lookback(Carver& ws, int64_t tiles) {
+  LookbackState st;
+  st.status = ws.take<unsigned long long>(tiles > 0 ? tiles : 1);
+  unsigned int* words = ws.take<unsigned int>(64);
+  st.ticket = words;
+  st.done = words ? words + 1 : nullptr;
+  st.error = words ? words + 2 : nullptr;
+  return st;
+}
+
+__device__ __forceinline__ unsigned long long lb_load(const unsigned long long* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void lb_store(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Thread 0 draws the tile number; returns it to every thread (uses one LDS word).
+__device__ __forceinline__ unsigned int lookback_take_ticket(const LookbackState& st,
+                                                             unsigned int* lds_word) {
+  if (threadIdx.x == 0) *lds_word = atomicAdd(st.ticket, 1u);
+  __syncthreads();
+  return *lds_word;
+}
+
+// Call with all 64 lanes of wave 0.  Publishes `total` for `tile` and returns the
+// sum of all earlier tiles.
+__device__ __forceinline__ int64_t lookback_exclusive_prefix(const LookbackState& st,
+                                                             unsigned int tile, int64_t total) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const unsigned long long mine = static_cast<unsigned long long>(total) & kLbValue;
+  if (tile == 0) {
+    if (lane == 0) lb_store(&st.status[0], kLbInclusive | mine);
+    return 0;
+  }
+  if (lane == 0) lb_store(&st.status[tile], kLbSum | mine);
+  int64_t running = 0;
+  int64_t newest = static_cast<int64_t>(tile) - 1;  // lane l reads tile newest - l
+  while (true) {
+    const int64_t j = newest - lane;
+    unsigned long long s = kLbInclusive;  // before tile 0: inclusive prefix 0
+    if (j >= 0) {
+      int polls = 0;
+      while (((s = lb_load(&st.status[j])) >> 62) == 0) {
+        if (++polls > kLookbackSpinLimit) {
+          __hip_atomic_store(st.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          s = kLbInclusive;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+    }
+    const unsigned long long closed = __ballot((s >> 62) == 2);
+    const int first = closed ? __ffsll(static_cast<long long>(closed)) - 1 : kWave;
+    int64_t v = lane <= first ? static_cast<int64_t>(s & kLbValue) : 0;
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_xor(v, d, kWave);
+    running += v;
+    if (closed) break;
+    newest -= kWave;
+  }
+  __threadfence();  // an error raised above is visible before the prefix that hides it
+  if (lane == 0) lb_store(&st.status[tile], kLbInclusive | ((static_cast<unsigned long long>(running) + mine) & kLbValue));
+  return running;
+}
+
+// ----------------------------------------------------------- host mailbox ----
+// {total, ticket} in pinned host memory, written with system scope, total first.
+__device__ __forceinline__ void post_mailbox(gs_mailbox* box, int64_t total, int64_t ticket) {
+  if (!box) return;
+  __hip_atomic_store(&box->total, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  __hip_atomic_store(&box->ticket, ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 }  // namespace gs

@@ -519,6 +519,216 @@ int sample_fill_impl(const SampleArgs<IdT>& a, int replace, int algo, hipStream_
   return check_launch("sample_rows");
 }
 
+
+// ------------------------------------------- one-launch slice + sample ----
+// Counting, the scan of the counts and the fill in ONE kernel: a workgroup
+// takes a tile of 256 rows, one row per lane reads its column id and offsets
+// (256 independent random reads in flight per workgroup instead of the same
+// read repeated by every lane of a row group), the tile's counts are scanned in
+// LDS, the tile prefix comes from a look-back over earlier tiles, and then the
+// row groups of G lanes draw and gather exactly as sample_floyd_kernel /
+// sample_replace_kernel do, reading (start, degree, output offset) from LDS.
+// The outputs must hold S * fanout entries; the true total lands in
+// sub_indptr[S] (and in the host mailbox when one is given).
+constexpr int kFusedThreads = 256;
+constexpr int kFusedRows = 256;
+
+template <typename IdT>
+struct FusedArgs {
+  const int64_t* indptr;
+  const IdT* indices;
+  const IdT* cols;
+  int64_t num_cols;
+  int64_t S;
+  int64_t k;
+  uint64_t seed;
+  const uint32_t* replay;
+  const int64_t* replay_ptr;
+  int64_t* sub_indptr;
+  IdT* sub_indices;
+  int64_t* select_index;
+  IdT* coo_col;
+  LookbackState lb;
+  gs_mailbox* box;
+  int64_t box_ticket;
+};
+
+template <typename IdT, int G, bool REPLACE>
+__global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<IdT> a) {
+  __shared__ int64_t s_start[kFusedRows];
+  __shared__ int64_t s_deg[kFusedRows];
+  __shared__ int64_t s_out[kFusedRows];
+  __shared__ int64_t s_scan[kFusedThreads / kWave + 1];
+  __shared__ int64_t s_prefix;
+  __shared__ unsigned int s_word;
+  const unsigned int tile = lookback_take_ticket(a.lb, &s_word);
+  const unsigned int tiles = gridDim.x;
+  const int64_t row0 = static_cast<int64_t>(tile) * kFusedRows;
+  const int k = static_cast<int>(a.k);
+
+  // ---- phase 1: one row per lane
+  int64_t start = 0, deg = 0, cnt = 0;
+  {
+    const int64_t r = row0 + threadIdx.x;
+    if (r < a.S) {
+      const int64_t c = a.cols ? static_cast<int64_t>(a.cols[r]) : r;
+      if (valid_col(c, a.num_cols)) {
+        start = a.indptr[c];
+        deg = a.indptr[c + 1] - start;
+      }
+      cnt = REPLACE ? (deg > 0 ? a.k : 0) : (deg < a.k ? deg : a.k);
+    }
+  }
+  int64_t tile_total;
+  const int64_t local = block_exclusive_scan<kFusedThreads>(cnt, &tile_total, s_scan);
+  if (threadIdx.x < kWave) {
+    const int64_t before = lookback_exclusive_prefix(a.lb, tile, tile_total);
+    if (threadIdx.x == 0) s_prefix = before;
+  }
+  __syncthreads();
+  {
+    const int64_t out = s_prefix + local;
+    s_start[threadIdx.x] = start;
+    s_deg[threadIdx.x] = deg;
+    s_out[threadIdx.x] = out;
+    const int64_t r = row0 + threadIdx.x;
+    if (r < a.S) a.sub_indptr[r] = out;
+  }
+  if (tile == tiles - 1 && threadIdx.x == 0) {
+    int64_t total = s_prefix + tile_total;
+    if (__hip_atomic_load(a.lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) total = -1;
+    a.sub_indptr[a.S] = total;
+    post_mailbox(a.box, total, a.box_ticket);
+  }
+  __syncthreads();
+
+  // ---- phase 2: G lanes per row
+  constexpr int kGroups = kFusedThreads / G;
+  const int lane = threadIdx.x % G;
+  for (int row = threadIdx.x / G; row < kFusedRows; row += kGroups) {
+    const int64_t r = row0 + row;
+    if (r >= a.S) break;
+    const int64_t st = s_start[row];
+    const int64_t d = s_deg[row];
+    const int64_t out = s_out[row];
+    if (REPLACE) {
+      if (d == 0) continue;
+      const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[r] : nullptr;
+      for (int64_t q = lane; q * 4 < a.k; q += G) {
+        U4 x;
+        if (!rp) x = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(r), static_cast<uint64_t>(q));
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int64_t j = q * 4 + t;
+          if (j < a.k) {
+            const uint32_t xv = rp ? rp[j] : x.v[t];
+            const int64_t p = st + static_cast<int64_t>(xv % static_cast<uint32_t>(d));
+            a.sub_indices[out + j] = a.indices[p];
+            a.select_index[out + j] = p;
+            if (a.coo_col) a.coo_col[out + j] = static_cast<IdT>(r);
+          }
+        }
+      }
+      continue;
+    }
+    if (d <= k) {
+      if (lane < d) {
+        a.sub_indices[out + lane] = a.indices[st + lane];
+        a.select_index[out + lane] = st + lane;
+        if (a.coo_col) a.coo_col[out + lane] = static_cast<IdT>(r);
+      }
+      continue;
+    }
+    uint32_t t = 0, j = 0;
+    if (lane < k) {
+      const uint32_t xv = a.replay ? a.replay[a.replay_ptr[r] + lane]
+                                   : draw_one(a.seed, kTagUniform, static_cast<uint64_t>(r),
+                                              static_cast<uint64_t>(lane));
+      j = static_cast<uint32_t>(d - k + lane);
+      t = xv % (j + 1u);
+    }
+    bool taken = false;
+    for (int m = 0; m < k - 1; ++m) {
+      const uint32_t chosen_m = __shfl(taken ? j : t, m, G);
+      if (lane > m && t == chosen_m) taken = true;
+    }
+    if (lane < k) {
+      const int64_t q = st + (taken ? j : t);
+      a.sub_indices[out + lane] = a.indices[q];
+      a.select_index[out + lane] = q;
+      if (a.coo_col) a.coo_col[out + lane] = static_cast<IdT>(r);
+    }
+  }
+
+  // ---- leave the look-back state zeroed for the next call
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();
+    s_word = atomicAdd(a.lb.done, 1u) == tiles - 1 ? 1u : 0u;
+  }
+  __syncthreads();
+  if (s_word) {
+    for (unsigned int i = threadIdx.x; i < tiles; i += kFusedThreads) a.lb.status[i] = 0ull;
+    if (threadIdx.x == 0) {
+      *a.lb.ticket = 0u;
+      *a.lb.done = 0u;
+      *a.lb.error = 0u;
+    }
+  }
+}
+
+template <typename IdT, bool REPLACE>
+int sample_fused_launch(const FusedArgs<IdT>& a, hipStream_t stream) {
+  const unsigned grid = static_cast<unsigned>((a.S + kFusedRows - 1) / kFusedRows);
+  ProfileScope prof("sample_fused", stream);
+  const int g = a.k <= 8 ? 8 : (a.k <= 16 ? 16 : (a.k <= 32 ? 32 : 64));
+  if (g == 8)
+    hipLaunchKernelGGL((sample_fused_kernel<IdT, 8, REPLACE>), dim3(grid), dim3(kFusedThreads), 0,
+                       stream, a);
+  else if (g == 16)
+    hipLaunchKernelGGL((sample_fused_kernel<IdT, 16, REPLACE>), dim3(grid), dim3(kFusedThreads), 0,
+                       stream, a);
+  else if (g == 32)
+    hipLaunchKernelGGL((sample_fused_kernel<IdT, 32, REPLACE>), dim3(grid), dim3(kFusedThreads), 0,
+                       stream, a);
+  else
+    hipLaunchKernelGGL((sample_fused_kernel<IdT, 64, REPLACE>), dim3(grid), dim3(kFusedThreads), 0,
+                       stream, a);
+  return check_launch("sample_fused");
+}
+
+static __global__ void post_zero_kernel(int64_t* sub_indptr, gs_mailbox* box, int64_t ticket) {
+  if (threadIdx.x == 0) {
+    sub_indptr[0] = 0;
+    post_mailbox(box, 0, ticket);
+  }
+}
+
+template <typename IdT>
+int sample_fused_t(const int64_t* indptr, int64_t num_cols, const void* indices,
+                   const void* column_ids, int64_t S, int64_t fanout, int replace, uint64_t seed,
+                   const uint32_t* replay, const int64_t* replay_ptr, int64_t* sub_indptr,
+                   void* sub_indices, int64_t* select_index, void* coo_col, LookbackState lb,
+                   gs_mailbox* box, int64_t ticket, hipStream_t st) {
+  FusedArgs<IdT> a{indptr,
+                   static_cast<const IdT*>(indices),
+                   static_cast<const IdT*>(column_ids),
+                   num_cols,
+                   S,
+                   fanout,
+                   seed,
+                   replay,
+                   replay_ptr,
+                   sub_indptr,
+                   static_cast<IdT*>(sub_indices),
+                   select_index,
+                   static_cast<IdT*>(coo_col),
+                   lb,
+                   box,
+                   ticket};
+  return replace ? sample_fused_launch<IdT, true>(a, st) : sample_fused_launch<IdT, false>(a, st);
+}
+
 }  // namespace
 }  // namespace gs
 
@@ -663,6 +873,60 @@ int gs_sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const void* 
                                               select_index, coo_col, queue, queue_count,
                                               queue_cap, algo, st);
 }
+
+size_t gs_sample_fused_state_bytes(int64_t S) {
+  const int64_t s = S < 0 ? 0 : S;
+  return lookback_state_bytes((s + kFusedRows - 1) / kFusedRows);
+}
+
+int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void* indices,
+                            const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+                            int replace, uint64_t seed, const uint32_t* replay,
+                            const int64_t* replay_ptr, int64_t* sub_indptr, void* sub_indices,
+                            int64_t* select_index, void* coo_col, int64_t capacity,
+                            void* zeroed_state, size_t state_bytes, gs_mailbox* mailbox,
+                            int64_t mailbox_ticket, void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0 && num_cols >= 0,
+             "gs_sample_uniform_fused: null pointer or negative size");
+  GS_REQUIRE(column_ids || S <= num_cols,
+             "gs_sample_uniform_fused: S exceeds num_cols without column_ids");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sample_uniform_fused: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  GS_REQUIRE((replay == nullptr) == (replay_ptr == nullptr),
+             "gs_sample_uniform_fused: replay and replay_ptr must be given together");
+  if (!replace && fanout > GS_FLOYD_MAX_FANOUT) {
+    set_error_text("gs_sample_uniform_fused: fanout %lld without replacement exceeds %d; use "
+                   "gs_sample_count + gs_sample_uniform_fill",
+                   static_cast<long long>(fanout), GS_FLOYD_MAX_FANOUT);
+    return GS_ERR_UNSUPPORTED;
+  }
+  GS_REQUIRE(S == 0 || fanout == 0 || capacity >= S * fanout,
+             "gs_sample_uniform_fused: outputs must hold S * fanout = %lld entries, capacity is %lld",
+             static_cast<long long>(S * fanout), static_cast<long long>(capacity));
+  GS_REQUIRE(S == 0 || fanout == 0 || (indices && sub_indices && select_index),
+             "gs_sample_uniform_fused: null buffer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (S == 0) {
+    hipLaunchKernelGGL(post_zero_kernel, dim3(1), dim3(64), 0, st, sub_indptr, mailbox,
+                       mailbox_ticket);
+    return check_launch("sample_fused");
+  }
+  Carver ws(zeroed_state, state_bytes);
+  LookbackState lb = carve_lookback(ws, (S + kFusedRows - 1) / kFusedRows);
+  if (!ws.ok) {
+    set_error_text("gs_sample_uniform_fused: state needs %zu zeroed bytes, 256-byte aligned",
+                   gs_sample_fused_state_bytes(S));
+    return GS_ERR_WORKSPACE;
+  }
+  return id_bytes == 8
+             ? sample_fused_t<int64_t>(indptr, num_cols, indices, column_ids, S, fanout, replace,
+                                       seed, replay, replay_ptr, sub_indptr, sub_indices,
+                                       select_index, coo_col, lb, mailbox, mailbox_ticket, st)
+             : sample_fused_t<int32_t>(indptr, num_cols, indices, column_ids, S, fanout, replace,
+                                       seed, replay, replay_ptr, sub_indptr, sub_indices,
+                                       select_index, coo_col, lb, mailbox, mailbox_ticket, st);
+}
+
 
 int gs_sample_one_keepdim(const int64_t* indptr, int64_t num_cols, const void* indices,
                           const void* column_ids, int id_bytes, int64_t S, uint64_t seed,

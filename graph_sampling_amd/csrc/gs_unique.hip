@@ -18,9 +18,10 @@
 //  * the mapping tensors are read in place through a span table -- no
 //    concatenated copy is materialised (the reference does torch::cat,
 //    unique_reindex.cu:187-190);
-//  * the rank of a key is prefix[first index], so compaction and every relabel
-//    lookup run in one final kernel; a query that aliases a mapping span is
-//    relabelled by slot gather instead of probing.
+//  * first-occurrence flags, their scan and the compaction run in ONE launch
+//    (chained scan with look-back); the rank of a key is prefix[first index],
+//    so every relabel lookup is two gathers in a last kernel, and a query that
+//    aliases a mapping span is relabelled by slot gather instead of probing.
 #include "gs_common.hpp"
 
 namespace gs {
@@ -144,10 +145,18 @@ struct TableFor<int32_t> {
   using type = PackedTable;
 };
 
+// empties the table and zeroes the look-back state of the compaction pass
 template <typename T>
-__global__ void __launch_bounds__(kThreads) table_init_kernel(T t, int64_t cap) {
+__global__ void __launch_bounds__(kThreads) table_init_kernel(T t, int64_t cap, LookbackState lb,
+                                                              int64_t tiles) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i < cap) t.clear(i);
+  if (i < tiles) lb.status[i] = 0ull;
+  if (i == 0) {
+    *lb.ticket = 0u;
+    *lb.done = 0u;
+    *lb.error = 0u;
+  }
 }
 
 // insert (key -> min index) and remember the slot of every item
@@ -160,16 +169,6 @@ table_insert_kernel(Spans<IdT> x, int64_t M, T t, uint32_t* __restrict__ pos) {
   pos[i] = t.insert(static_cast<long long>(x.get(i)), static_cast<uint32_t>(i));
 }
 
-// 1 when item i is the first occurrence of its key (unique_reindex.cu:106-114)
-template <typename T>
-struct IsFirst {
-  T t;
-  const uint32_t* pos;
-  __device__ __forceinline__ int64_t operator()(int64_t i) const {
-    return t.first_index(pos[i]) == static_cast<uint32_t>(i) ? 1 : 0;
-  }
-};
-
 struct Query {
   const void* in[GS_MAX_SPANS];
   void* out[GS_MAX_SPANS];
@@ -178,21 +177,65 @@ struct Query {
   int n;
 };
 
-// Items [0, M): frontier[rank] = key for first occurrences
-// (unique_reindex.cu:127-144).  Items [M, M+Q): relabel lookups
-// (unique_reindex.cu:162-170), rank of a key = prefix[its first index].
+// One launch for flags, their scan and the compaction: a tile of 2048 items,
+// eight consecutive items per lane.  prefix[i] = number of first occurrences
+// before item i (the rank of item i's key when i is a first occurrence),
+// frontier[rank] = key (unique_reindex.cu:106-144).  The last tile knows the
+// number of unique ids and reports it.
+constexpr int kCompactItems = 8;
+constexpr int kCompactTile = kThreads * kCompactItems;
+
 template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
-finish_kernel(Spans<IdT> x, int64_t M, T t, const uint32_t* __restrict__ pos,
-              const int64_t* __restrict__ prefix, IdT* __restrict__ frontier,
-              int64_t* __restrict__ num_unique, Query qs, int64_t Q) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (i == 0) *num_unique = prefix[M];
-  if (i < M) {
-    if (t.first_index(pos[i]) == static_cast<uint32_t>(i)) frontier[prefix[i]] = x.get(i);
-    return;
+compact_kernel(Spans<IdT> x, int64_t M, T t, const uint32_t* __restrict__ pos,
+               int64_t* __restrict__ prefix, IdT* __restrict__ frontier,
+               int64_t* __restrict__ num_unique, LookbackState lb, gs_mailbox* box,
+               int64_t box_ticket) {
+  __shared__ int64_t s_scan[kThreads / kWave + 1];
+  __shared__ int64_t s_prefix;
+  __shared__ unsigned int s_word;
+  const unsigned int tile = lookback_take_ticket(lb, &s_word);
+  const int64_t base = static_cast<int64_t>(tile) * kCompactTile +
+                       static_cast<int64_t>(threadIdx.x) * kCompactItems;
+  bool first[kCompactItems];
+  int64_t mine = 0;
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) {
+    const int64_t i = base + k;
+    first[k] = i < M && t.first_index(pos[i]) == static_cast<uint32_t>(i);
+    mine += first[k] ? 1 : 0;
   }
-  const int64_t j = i - M;
+  int64_t tile_total;
+  const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
+  if (threadIdx.x < kWave) {
+    const int64_t before = lookback_exclusive_prefix(lb, tile, tile_total);
+    if (threadIdx.x == 0) s_prefix = before;
+  }
+  __syncthreads();
+  int64_t run = s_prefix + local;
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) {
+    const int64_t i = base + k;
+    if (i < M) {
+      prefix[i] = run;
+      if (first[k]) frontier[run] = x.get(i);
+    }
+    run += first[k] ? 1 : 0;
+  }
+  if (tile == gridDim.x - 1 && threadIdx.x == 0) {
+    int64_t total = s_prefix + tile_total;
+    if (__hip_atomic_load(lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) total = -1;
+    *num_unique = total;
+    post_mailbox(box, total, box_ticket);
+  }
+}
+
+// Relabel lookups (unique_reindex.cu:162-170): rank of a key = prefix[its first index].
+template <typename IdT, typename T>
+__global__ void __launch_bounds__(kThreads)
+lookup_kernel(T t, const uint32_t* __restrict__ pos, const int64_t* __restrict__ prefix, Query qs,
+              int64_t Q) {
+  const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (j >= Q) return;
   int s = 0;
   int64_t begin = 0;
@@ -213,6 +256,10 @@ finish_kernel(Spans<IdT> x, int64_t M, T t, const uint32_t* __restrict__ pos,
   static_cast<IdT*>(qs.out[s])[local] = static_cast<IdT>(first < 0 ? -1 : prefix[first]);
 }
 
+inline int64_t compact_num_tiles(int64_t M) {
+  return M <= 0 ? 1 : (M + kCompactTile - 1) / kCompactTile;
+}
+
 int64_t table_capacity(int64_t M) {
   int64_t cap = 1024;
   while (cap < 2 * M) cap <<= 1;
@@ -224,13 +271,14 @@ size_t workspace_bytes_for(int64_t M) {
   using T = typename TableFor<IdT>::type;
   const int64_t cap = table_capacity(M);
   return T::bytes(cap) + padded((M > 0 ? M : 1) * 4) + padded((M + 1) * 8) +
-         scan_workspace_bytes(M);
+         lookback_state_bytes(compact_num_tiles(M));
 }
 
 template <typename IdT>
 int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* query,
                         void* const* query_out, int n_query, void* frontier, int64_t* num_unique,
-                        void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                        void* workspace, size_t workspace_bytes, gs_mailbox* box,
+                        int64_t box_ticket, hipStream_t stream) {
   using T = typename TableFor<IdT>::type;
   Spans<IdT> x;
   int64_t M = 0;
@@ -250,7 +298,8 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   t.carve(ws, cap);
   uint32_t* pos = ws.take<uint32_t>(M > 0 ? M : 1);
   int64_t* prefix = ws.take<int64_t>(M + 1);
-  int64_t* tiles = ws.take<int64_t>(scan_num_tiles(M) + 1);
+  const int64_t tiles = compact_num_tiles(M);
+  LookbackState lb = carve_lookback(ws, tiles);
   if (!ws.ok) {
     set_error_text("gs_unique_relabel: workspace needs %zu bytes, 256-byte aligned",
                    workspace_bytes_for<IdT>(M));
@@ -284,20 +333,26 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
 
   {
     ProfileScope prof("table_init", stream);
-    hipLaunchKernelGGL((table_init_kernel<T>), dim3(blocks_for(cap, kThreads)), dim3(kThreads), 0,
-                       stream, t, cap);
+    const int64_t n_init = cap > tiles ? cap : tiles;
+    hipLaunchKernelGGL((table_init_kernel<T>), dim3(blocks_for(n_init, kThreads)), dim3(kThreads),
+                       0, stream, t, cap, lb, tiles);
   }
   if (M > 0) {
     ProfileScope prof("table_insert", stream);
     hipLaunchKernelGGL((table_insert_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
                        0, stream, x, M, t, pos);
   }
-  GS_RETURN_IF_ERROR(check_launch("unique insert"));
-  IsFirst<T> f{t, pos};
-  GS_RETURN_IF_ERROR(exclusive_scan(f, M, prefix, tiles, stream));
-  ProfileScope prof("unique_finish", stream);
-  hipLaunchKernelGGL((finish_kernel<IdT, T>), dim3(blocks_for(M + Q, kThreads)), dim3(kThreads), 0,
-                     stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, qs, Q);
+  {
+    ProfileScope prof("unique_compact", stream);
+    hipLaunchKernelGGL((compact_kernel<IdT, T>), dim3(static_cast<unsigned>(tiles)), dim3(kThreads),
+                       0, stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, lb,
+                       box, box_ticket);
+  }
+  if (Q > 0) {
+    ProfileScope prof("unique_finish", stream);
+    hipLaunchKernelGGL((lookup_kernel<IdT, T>), dim3(blocks_for(Q, kThreads)), dim3(kThreads), 0,
+                       stream, t, pos, prefix, qs, Q);
+  }
   return check_launch("unique_relabel");
 }
 
@@ -315,10 +370,10 @@ size_t gs_unique_workspace_bytes(int64_t M) {
   return a > b ? a : b;
 }
 
-int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* query,
-                      void* const* query_out, int n_query, int id_bytes, void* frontier,
-                      int64_t* num_unique, void* workspace, size_t workspace_bytes,
-                      void* stream) {
+int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_span* query,
+                             void* const* query_out, int n_query, int id_bytes, void* frontier,
+                             int64_t* num_unique, void* workspace, size_t workspace_bytes,
+                             gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream) {
   GS_REQUIRE(mapping && n_mapping >= 1 && n_mapping <= GS_MAX_SPANS,
              "gs_unique_relabel: 1..%d mapping spans required, got %d", GS_MAX_SPANS, n_mapping);
   GS_REQUIRE(n_query >= 0 && n_query <= GS_MAX_SPANS && (n_query == 0 || (query && query_out)),
@@ -343,10 +398,18 @@ int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* quer
   hipStream_t st = static_cast<hipStream_t>(stream);
   return id_bytes == 8 ? unique_relabel_impl<int64_t>(mapping, n_mapping, query, query_out, n_query,
                                                       frontier, num_unique, workspace,
-                                                      workspace_bytes, st)
+                                                      workspace_bytes, mailbox, mailbox_ticket, st)
                        : unique_relabel_impl<int32_t>(mapping, n_mapping, query, query_out, n_query,
                                                       frontier, num_unique, workspace,
-                                                      workspace_bytes, st);
+                                                      workspace_bytes, mailbox, mailbox_ticket, st);
+}
+
+int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* query,
+                      void* const* query_out, int n_query, int id_bytes, void* frontier,
+                      int64_t* num_unique, void* workspace, size_t workspace_bytes,
+                      void* stream) {
+  return gs_unique_relabel_notify(mapping, n_mapping, query, query_out, n_query, id_bytes, frontier,
+                                  num_unique, workspace, workspace_bytes, nullptr, 0, stream);
 }
 
 }  // extern "C"

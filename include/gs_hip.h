@@ -56,11 +56,24 @@ const char* gs_status_string(int status);
 /* Library version (major*10000 + minor*100 + patch). */
 int gs_version(void);
 
+/* Result mailbox: 16 bytes of pinned, device-visible host memory (hipHostMalloc).
+ * Entry points that take one let the kernel that produces a total (sampled edge
+ * count, number of unique ids) also store {total, ticket} there with system
+ * scope, total first.  The host may then spin on `ticket` instead of
+ * synchronising the stream; work queued later on the same stream is still
+ * ordered after the producing kernel.  NULL = no mailbox.  No counterpart in the
+ * reference, which reads totals back with a blocking copy
+ * (src/cuda/sampling.cu:124, src/cuda/unique_reindex.cu:120). */
+typedef struct gs_mailbox {
+  int64_t total;
+  int64_t ticket;
+} gs_mailbox;
+
 /* Optional timing of one launch site, for benchmarks (no counterpart in the
  * reference).  gs_profile_enable("name") makes every later launch of that site
  * record a hipEvent pair on its stream (up to 4096 launches); NULL or ""
- * disables.  Sites: "sample_floyd", "table_init", "table_insert",
- * "unique_finish", "scan_tile_sums", "scan_apply", "random_walk",
+ * disables.  Sites: "sample_fused", "sample_floyd", "table_init", "table_insert",
+ * "unique_compact", "unique_finish", "scan_tile_sums", "scan_apply", "random_walk",
  * "metapath_walk", "sddmm_dot".  gs_profile_collect waits for the recorded
  * events, returns their summed duration and count (and, when per_launch_ms is
  * given, the first `cap` individual durations in launch order) and clears the
@@ -133,6 +146,31 @@ int gs_sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const void* 
                            const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                            void* coo_col, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Column slice + uniform sample in ONE launch: count, offsets and fill together
+ * (the same results as gs_sample_count + gs_sample_uniform_fill with
+ * GS_SAMPLE_AUTO, bit for bit).  Replaces
+ * impl::fusion::FusedCSCColSlicingSamplingCUDA (src/cuda/fusion/slice_sampling.cu:146)
+ * and, with column_ids == NULL, impl::CSCColSamplingCUDA (src/cuda/sampling.cu:157),
+ * without their mid-call host read.
+ *   - without replacement fanout must be <= GS_FLOYD_MAX_FANOUT (else
+ *     GS_ERR_UNSUPPORTED: use the two-phase calls);
+ *   - sub_indices / select_index / coo_col hold `capacity` >= S*fanout entries;
+ *     the true total is written to sub_indptr[S] (-1 if the kernel gave up
+ *     waiting on another tile, which a healthy device never does) and to the
+ *     mailbox when one is given;
+ *   - zeroed_state: gs_sample_fused_state_bytes(S) bytes, 256-byte aligned, ALL
+ *     ZERO on entry; the kernel leaves them zero again, so one buffer cleared
+ *     once serves every later call on the same stream.  Two calls running at the
+ *     same time must not share it. */
+size_t gs_sample_fused_state_bytes(int64_t S);
+int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void* indices,
+                            const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+                            int replace, uint64_t seed, const uint32_t* replay,
+                            const int64_t* replay_ptr, int64_t* sub_indptr, void* sub_indices,
+                            int64_t* select_index, void* coo_col, int64_t capacity,
+                            void* zeroed_state, size_t state_bytes, gs_mailbox* mailbox,
+                            int64_t mailbox_ticket, void* stream);
+
 /* fanout == 1 with replacement through the fused entry: exactly one slot per
  * column, -1 in both outputs for an empty column; sub_indptr = 0..S.  Replaces
  * impl::fusion::FusedCSCColSlicingSamplingOneKeepDimCUDA
@@ -203,6 +241,14 @@ int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* quer
                       void* const* query_out, int n_query, int id_bytes, void* frontier,
                       int64_t* num_unique, void* workspace, size_t workspace_bytes,
                       void* stream);
+
+/* The same, and the kernel that learns the number of unique ids also posts it to
+ * `mailbox` (see gs_mailbox; NULL = plain gs_unique_relabel).  *num_unique and the
+ * mailbox read -1 if the compaction gave up waiting on another tile. */
+int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_span* query,
+                             void* const* query_out, int n_query, int id_bytes, void* frontier,
+                             int64_t* num_unique, void* workspace, size_t workspace_bytes,
+                             gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Random walks: replace impl::fusion::FusedRandomWalkCUDA                    */

@@ -1,0 +1,150 @@
+"""GPU parity: the one-launch slice + sample (gs_sample_uniform_fused) and the result mailbox,
+against the CPU oracle and against the two-phase calls."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from graph_sampling_amd import capi
+from tests.util import graph_20x5, rmat_csc_np, to_dev, u32_draws
+
+pytestmark = pytest.mark.gpu
+
+ID_DTYPES = [torch.int64, torch.int32]
+
+
+def _narrow(res):
+    sub_indptr, sub_indices, select_index, coo_col = res[:4]
+    nnz = int(sub_indptr[-1].item())
+    return (sub_indptr, None if coo_col is None else coo_col[:nnz], sub_indices[:nnz],
+            select_index[:nnz])
+
+
+def _cmp(got, want):
+    for g, w in zip(got, want):
+        if w is None:
+            assert g is None
+            continue
+        g = g.cpu().numpy().astype(np.int64)
+        assert g.shape == w.shape, (g.shape, w.shape)
+        assert np.array_equal(g, w)
+
+
+def _state_is_clean(dev):
+    for buf in capi._fused_state.values():
+        assert int(buf.count_nonzero().item()) == 0, "the look-back state was not left zeroed"
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("replace", [False, True])
+@pytest.mark.parametrize("k", [1, 5, 8, 9, 15, 16, 17, 33, 64])
+@pytest.mark.parametrize("fused_cols", [True, False])
+def test_fused_matches_oracle(dev, idt, replace, k, fused_cols):
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=5)
+    if fused_cols:
+        cols = np.random.default_rng(k).integers(0, indptr.size - 1, size=3000).astype(np.int64)
+        cols[:8] = np.argsort(np.diff(indptr))[-8:]
+        dcols = to_dev(cols, dev, idt)
+    else:
+        cols, dcols = None, None
+    got = _narrow(capi.sample_uniform_fused(to_dev(indptr, dev), to_dev(indices, dev, idt), dcols, k,
+                                            replace, seed=99 + k, with_coo=True))
+    _cmp(got, O.sample_uniform(indptr, indices, cols, k, replace, seed=99 + k, with_coo=True))
+    _state_is_clean(dev)
+
+
+@pytest.mark.parametrize("replace", [False, True])
+@pytest.mark.parametrize("k", [70, 200])
+def test_fused_large_fanout(dev, replace, k):
+    """With replacement any fanout runs; without, fanouts above 64 are refused (two-phase path)."""
+    indptr, indices = rmat_csc_np(1 << 10, 1 << 15, seed=8)
+    cols = np.random.default_rng(3).integers(0, 1 << 10, size=500).astype(np.int64)
+    args = (to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev), k, replace)
+    if not replace:
+        with pytest.raises(capi.GsError, match="exceeds 64"):
+            capi.sample_uniform_fused(*args, seed=1)
+        return
+    _cmp(_narrow(capi.sample_uniform_fused(*args, seed=1, with_coo=True)),
+         O.sample_uniform(indptr, indices, cols, k, replace, seed=1))
+
+
+@pytest.mark.parametrize("S", [0, 1, 255, 256, 257, 16384, 16385, 70001])
+def test_fused_tile_boundaries_and_long_lookback(dev, S):
+    """Row counts around the 256-row tile and past 64 tiles (more than one look-back window)."""
+    indptr, indices = rmat_csc_np(1 << 13, 1 << 17, seed=2)
+    cols = np.random.default_rng(S).integers(0, 1 << 13, size=S).astype(np.int64)
+    d = (to_dev(indptr, dev), to_dev(indices, dev, torch.int32), to_dev(cols, dev, torch.int32))
+    for replace in (False, True):
+        got = _narrow(capi.sample_uniform_fused(*d, 7, replace, seed=S, with_coo=True))
+        _cmp(got, O.sample_uniform(indptr, indices, cols, 7, replace, seed=S))
+    _state_is_clean(dev)
+
+
+def test_fused_equals_two_phase_at_benchmark_shape(dev):
+    """Layer-3-like shape: 45k seed columns, fanout 5; the two entry points agree bit for bit."""
+    indptr, indices = rmat_csc_np(1 << 16, 1 << 21, seed=4)
+    cols = np.random.default_rng(0).integers(0, 1 << 16, size=45000).astype(np.int64)
+    d = (to_dev(indptr, dev), to_dev(indices, dev, torch.int32), to_dev(cols, dev, torch.int32))
+    a = _narrow(capi.sample_uniform_fused(*d, 5, False, seed=11))
+    b = capi.sample_uniform(*d, 5, False, seed=11)
+    nnz = int(b[0][-1].item())
+    assert torch.equal(a[0], b[0])
+    assert torch.equal(a[2], b[1][:nnz]) and torch.equal(a[3], b[2][:nnz])
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_fused_replay(dev, replace):
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=6)
+    cols = np.random.default_rng(1).integers(0, indptr.size - 1, size=2000).astype(np.int64)
+    cols[:4] = np.argsort(np.diff(indptr))[-4:]
+    _, replay_ptr = O.sample_count(indptr, cols, 15, replace, want_replay_ptr=True)
+    replay = u32_draws(int(replay_ptr[-1]), seed=15)
+    want = O.sample_uniform(indptr, indices, cols, 15, replace, replay=replay)
+    got = _narrow(capi.sample_uniform_fused(to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev),
+                                            15, replace, replay=to_dev(replay, dev),
+                                            replay_ptr=to_dev(replay_ptr, dev), with_coo=True))
+    _cmp(got, want)
+
+
+def test_fused_reference_identity_vector(dev):
+    """tests/test_colwise_sampling.cc:7-20 of the reference: fanout >= degree copies in order."""
+    indptr, indices = graph_20x5()
+    got = _narrow(capi.sample_uniform_fused(to_dev(indptr, dev), to_dev(indices, dev), None, 5, False))
+    assert np.array_equal(got[0].cpu().numpy(), indptr)
+    assert np.array_equal(got[2].cpu().numpy(), indices)
+
+
+def test_fused_out_of_range_columns(dev):
+    indptr, indices = rmat_csc_np(1 << 10, 1 << 14, seed=12)
+    n = 1 << 10
+    cols = np.random.default_rng(0).integers(0, n, size=600).astype(np.int64)
+    cols[::7] = -1
+    cols[3::11] = n
+    cols[5::13] = n + 12345
+    d = (to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev))
+    for replace in (False, True):
+        _cmp(_narrow(capi.sample_uniform_fused(*d, 6, replace, seed=3, with_coo=True)),
+             O.sample_uniform(indptr, indices, cols, 6, replace, seed=3))
+
+
+def test_mailbox_reports_totals(dev):
+    """The kernels post {total, ticket} to pinned host memory; the host never syncs the stream."""
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=5)
+    d_ip, d_ix = to_dev(indptr, dev), to_dev(indices, dev, torch.int32)
+    box = capi.Mailbox()
+    for it in range(20):
+        S = [0, 1, 300, 5000, 20000][it % 5]
+        cols = np.random.default_rng(it).integers(0, 1 << 12, size=S).astype(np.int64)
+        d_cols = to_dev(cols, dev, torch.int32)
+        res = capi.sample_uniform_fused(d_ip, d_ix, d_cols, 10, False, seed=it, mailbox=box)
+        nnz = box.wait(res[4], dev)
+        want = O.sample_uniform(indptr, indices, cols, 10, False, seed=it)
+        assert nnz == int(want[0][-1])
+        sub = res[1][:nnz]
+        frontier, num, outs, ticket = capi.unique_relabel([d_cols, sub], [sub], mailbox=box)
+        U = box.wait(ticket, dev)
+        f_want, r_want = O.relabel([cols, want[2]], [want[2]])
+        assert U == f_want.size
+        assert np.array_equal(frontier[:U].cpu().numpy().astype(np.int64), f_want)
+        assert np.array_equal(outs[0].cpu().numpy().astype(np.int64), r_want[0])
+        assert int(num.item()) == U
