@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0
 # counters (2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE; the factors come from a device copy of
 # known size): profiles/sample_floyd_rmat-2.45M-124M_hbm_counters.txt.  The counters cannot
 # be read from inside this process, so the figure is carried here.
-TRAFFIC_BYTES_PER_LAUNCH = {("rmat-2.45M-124M", "sample_floyd"): 12343562}
+TRAFFIC_BYTES_PER_LAUNCH = {}
 
 
 def parse():
@@ -76,12 +76,11 @@ class KernelTimer:
 
 # launch sites of one minibatch step and the bytes each launch must move at the
 # least (id_bytes b; S seeds, E sampled edges, M = S + E items, U unique ids):
-#   sample_floyd  : per seed  column id b + two offsets 16 + output offset 8,
+#   sample_fused  : per seed  column id b + two offsets 16 + output offset 8,
 #                   per edge  neighbour gather b + sub_indices b + select_index 8
 #   table_insert  : per item  id b + one 8-byte slot read-modify-write 16 + slot index 4
 #   unique_finish : per item  slot index 4 + slot 8 + rank 8, relabeled id b, frontier b per U
-SITES = ("sample_floyd", "table_insert", "unique_finish", "scan_tile_sums", "scan_apply",
-         "table_init")
+SITES = ("sample_fused", "table_init", "table_insert", "unique_compact", "unique_finish")
 
 
 def floyd_bytes(b, S, E):
@@ -92,9 +91,10 @@ def insert_bytes(b, S, E):
     return (S + E) * (b + 20)
 
 
-SITE_BYTES = {"sample_floyd": floyd_bytes, "table_insert": insert_bytes}
+SITE_BYTES = {"sample_fused": floyd_bytes, "table_insert": insert_bytes}
 SITE_KERNEL = {
-    "sample_floyd": "sample_floyd_kernel (fused column slice + uniform sample, all three layers)",
+    "sample_fused": "sample_fused_kernel (column slice + count + scan + uniform sample in one "
+                    "launch, all three layers)",
     "table_insert": "table_insert_kernel (hash insert of seeds + sampled rows, all three layers)",
 }
 
@@ -129,13 +129,14 @@ def cpu_minibatch(O, np, indptr, indices, seeds, step):
 
 
 def saturated(torch, graph, timer, nodes, idt, dev, b):
-    """The same sampler launch at a size that fills the chip (4M seed columns drawn with
-    repetition, fanout 10): what the kernel reaches once launch latency is amortised."""
-    S = 1 << 22
+    """The same sampler launch at the largest size the host layer routes to it (2^18 seed
+    columns drawn with repetition, fanout 10): what the kernel reaches once launch latency is
+    amortised."""
+    S = 1 << 18
     gen = torch.Generator(device=dev)
     gen.manual_seed(5)
     cols = torch.randint(0, nodes, (S,), generator=gen, device=dev).to(idt)
-    timer.enable("sample_floyd")
+    timer.enable("sample_fused")
     E = 0
     for _ in range(4):
         sub = graph._CAPI_FusedColumnwiseSlicingSampling(cols, 10, False)

@@ -193,15 +193,22 @@ def sample_uniform(indptr, indices, column_ids, fanout, replace, seed=0, replay=
 _fused_state = {}
 
 
+MAX_EPOCH = (1 << 14) - 1
+
+
 def fused_state(nbytes, device):
-    """The zero-filled state buffer of gs_sample_uniform_fused for the current stream: cleared
-    once when (re)allocated, left zero by every call."""
+    """(state buffer, epoch) of gs_sample_uniform_fused for the current stream: zero-filled when
+    (re)allocated and whenever the epoch counter wraps."""
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)
-    buf = _fused_state.get(key)
+    buf, epoch = _fused_state.get(key, (None, 0))
     if buf is None or buf.numel() < nbytes:
-        buf = torch.zeros(max(int(nbytes), 4096), dtype=torch.uint8, device=device)
-        _fused_state[key] = buf
-    return buf
+        buf, epoch = torch.zeros(max(int(nbytes), 65536), dtype=torch.uint8, device=device), 0
+    if epoch == MAX_EPOCH:
+        buf.zero_()
+        epoch = 0
+    epoch += 1
+    _fused_state[key] = (buf, epoch)
+    return buf, epoch
 
 
 class Mailbox:
@@ -252,13 +259,13 @@ def sample_uniform_fused(indptr, indices, column_ids, fanout, replace, seed=0, r
     sub_indices = torch.empty(cap, dtype=indices.dtype, device=dev)
     select_index = torch.empty(cap, dtype=torch.int64, device=dev)
     coo_col = torch.empty(cap, dtype=indices.dtype, device=dev) if with_coo else None
-    state = fused_state(lib().gs_sample_fused_state_bytes(_i64(S)), dev)
+    state, epoch = fused_state(lib().gs_sample_fused_state_bytes(_i64(S)), dev)
     ticket = mailbox.ticket() if mailbox is not None else 0
     _check(lib().gs_sample_uniform_fused(
         _ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(column_ids), idb, _i64(S),
         _i64(fanout), int(bool(replace)), _u64(seed), _ptr(replay), _ptr(replay_ptr),
         _ptr(sub_indptr), _ptr(sub_indices), _ptr(select_index), _ptr(coo_col), _i64(cap),
-        _ptr(state), ctypes.c_size_t(state.numel()),
+        _ptr(state), ctypes.c_size_t(state.numel()), ctypes.c_uint32(epoch),
         mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0), _i64(ticket), _stream(dev)),
         "gs_sample_uniform_fused")
     if mailbox is not None:

@@ -333,43 +333,55 @@ inline int exclusive_scan(F f, int64_t n, int64_t* out, int64_t* tile_ws, hipStr
 
 // ------------------------------------------- single-pass scan (look-back) ----
 // Chained-scan building blocks for kernels that count, scan and write in one
-// launch.  Every tile owns one 64-bit status word {flag:2 | value:62}: flag 0 =
-// nothing yet, 1 = the tile's own sum, 2 = the inclusive prefix up to and
-// including the tile.  A tile publishes its sum, then wave 0 walks back over its
-// predecessors 64 at a time until it meets an inclusive prefix.
+// launch.  Every tile (= workgroup, in blockIdx order) owns one 64-bit status
+// word {flag:2 | epoch:14 | value:48}: flag 0 = nothing yet, 1 = the tile's own
+// sum, 2 = the inclusive prefix up to and including the tile.  A word whose
+// epoch is not the launch's epoch counts as "nothing yet", so the array needs no
+// clearing between launches: it is zero-filled once and every launch passes an
+// epoch (1..16383) that no earlier launch on the same array has used since.
+// Nothing in the protocol is a same-address read-modify-write: on a multi-XCD
+// part those serialise memory-side, and one per workgroup costs more than the
+// rest of the kernel.
 //
-// Tiles take their number from an atomic ticket, so every predecessor of a
-// tile is already resident on the device and publishes without waiting on
-// anyone: the walk cannot deadlock.  The wait is bounded all the same: after
-// kLookbackSpinLimit polls the tile gives up, raises *error and carries on with
-// a zero, so every wave reaches the end of the kernel.
-//
-// The status words, the ticket and the error word must be zero when the kernel
-// starts.
+// A tile publishes its sum, then wave 0 walks back over its predecessors, 8
+// windows of 64 per round trip, until it meets an inclusive prefix.  Workgroups
+// are dispatched in blockIdx order, so the lowest unfinished tile is always
+// resident and never waits on anyone: the walk cannot deadlock.  The wait is
+// bounded all the same: after kLookbackSpinLimit polls the tile gives up,
+// raises *error (sticky until the state is zero-filled again) and carries on
+// with a zero, so every wave reaches the end of the kernel.
 struct LookbackState {
   unsigned long long* status;  // one per tile
-  unsigned int* ticket;
-  unsigned int* done;   // tiles that have finished (for self-cleaning users)
   unsigned int* error;
+  unsigned int epoch;
 };
 
-constexpr unsigned long long kLbSum = 1ull << 62;
-constexpr unsigned long long kLbInclusive = 2ull << 62;
-constexpr unsigned long long kLbValue = (1ull << 62) - 1;
+constexpr int kLbValueBits = 48;
+constexpr unsigned long long kLbValue = (1ull << kLbValueBits) - 1;
+constexpr unsigned int kLbMaxEpoch = (1u << 14) - 1;
 constexpr int kLookbackSpinLimit = 1 << 20;
+constexpr int kLookbackBurst = 8;  // windows of 64 predecessors requested together
 
 inline size_t lookback_state_bytes(int64_t tiles) { return padded((tiles > 0 ? tiles : 1) * 8) + 256; }
 
-inline LookbackState carve_lookback(Carver& ws, int64_t tiles) {
+inline LookbackState carve_lookback(Carver& ws, int64_t tiles, unsigned int epoch) {
   LookbackState st;
+  st.error = ws.take<unsigned int>(64);  // first, so that it does not move with the tile count
   st.status = ws.take<unsigned long long>(tiles > 0 ? tiles : 1);
-  unsigned int* words = ws.take<unsigned int>(64);
-  st.ticket = words;
-  st.done = words ? words + 1 : nullptr;
-  st.error = words ? words + 2 : nullptr;
+  st.epoch = epoch;
   return st;
 }
 
+__device__ __forceinline__ unsigned long long lb_word(unsigned int flag, unsigned int epoch,
+                                                      int64_t value) {
+  return (static_cast<unsigned long long>(flag) << 62) |
+         (static_cast<unsigned long long>(epoch) << kLbValueBits) |
+         (static_cast<unsigned long long>(value) & kLbValue);
+}
+// flag of a status word as seen by a launch with this epoch (0 when it is stale)
+__device__ __forceinline__ unsigned int lb_flag(unsigned long long s, unsigned int epoch) {
+  return ((s >> kLbValueBits) & kLbMaxEpoch) == epoch ? static_cast<unsigned int>(s >> 62) : 0u;
+}
 __device__ __forceinline__ unsigned long long lb_load(const unsigned long long* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -377,52 +389,60 @@ __device__ __forceinline__ void lb_store(unsigned long long* p, unsigned long lo
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Thread 0 draws the tile number; returns it to every thread (uses one LDS word).
-__device__ __forceinline__ unsigned int lookback_take_ticket(const LookbackState& st,
-                                                             unsigned int* lds_word) {
-  if (threadIdx.x == 0) *lds_word = atomicAdd(st.ticket, 1u);
-  __syncthreads();
-  return *lds_word;
+// Any one thread: makes the tile's own sum visible to its successors.  Call it as
+// early as possible; whatever the tile does between this and the walk below
+// gives its predecessors time to publish theirs.
+__device__ __forceinline__ void lookback_publish_sum(const LookbackState& st, unsigned int tile,
+                                                     int64_t total) {
+  lb_store(&st.status[tile], lb_word(tile == 0 ? 2u : 1u, st.epoch, total));
 }
 
-// Call with all 64 lanes of wave 0.  Publishes `total` for `tile` and returns the
-// sum of all earlier tiles.
+// Call with all 64 lanes of wave 0, after lookback_publish_sum.  Returns the sum
+// of all earlier tiles and publishes the tile's inclusive prefix.
 __device__ __forceinline__ int64_t lookback_exclusive_prefix(const LookbackState& st,
                                                              unsigned int tile, int64_t total) {
   const int lane = threadIdx.x & (kWave - 1);
-  const unsigned long long mine = static_cast<unsigned long long>(total) & kLbValue;
-  if (tile == 0) {
-    if (lane == 0) lb_store(&st.status[0], kLbInclusive | mine);
-    return 0;
-  }
-  if (lane == 0) lb_store(&st.status[tile], kLbSum | mine);
+  if (tile == 0) return 0;
+  const unsigned long long before_first = lb_word(2u, st.epoch, 0);  // "tile -1": inclusive 0
   int64_t running = 0;
-  int64_t newest = static_cast<int64_t>(tile) - 1;  // lane l reads tile newest - l
-  while (true) {
-    const int64_t j = newest - lane;
-    unsigned long long s = kLbInclusive;  // before tile 0: inclusive prefix 0
-    if (j >= 0) {
-      int polls = 0;
-      while (((s = lb_load(&st.status[j])) >> 62) == 0) {
-        if (++polls > kLookbackSpinLimit) {
-          __hip_atomic_store(st.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          s = kLbInclusive;
-          break;
+  int64_t newest = static_cast<int64_t>(tile) - 1;  // lane l reads tile newest - l (- 64 per window)
+  bool closed_seen = false;
+  while (!closed_seen) {
+    // a burst of windows is requested at once so that their latencies overlap
+    unsigned long long s[kLookbackBurst];
+#pragma unroll
+    for (int w = 0; w < kLookbackBurst; ++w) {
+      const int64_t j = newest - w * kWave - lane;
+      s[w] = j >= 0 ? lb_load(&st.status[j]) : before_first;
+    }
+#pragma unroll
+    for (int w = 0; w < kLookbackBurst; ++w) {
+      if (!closed_seen) {
+        const int64_t j = newest - w * kWave - lane;
+        int polls = 0;
+        while (lb_flag(s[w], st.epoch) == 0) {
+          if (++polls > kLookbackSpinLimit) {
+            __hip_atomic_store(st.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s[w] = before_first;
+            break;
+          }
+          // a poll is a round trip to memory shared by every tile: keep them sparse
+          if (polls < 4) __builtin_amdgcn_s_sleep(8); else __builtin_amdgcn_s_sleep(64);
+          s[w] = lb_load(&st.status[j]);
         }
-        __builtin_amdgcn_s_sleep(2);
+        const unsigned long long closed = __ballot(lb_flag(s[w], st.epoch) == 2);
+        const int first = closed ? __ffsll(static_cast<long long>(closed)) - 1 : kWave;
+        int64_t v = lane <= first ? static_cast<int64_t>(s[w] & kLbValue) : 0;
+#pragma unroll
+        for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_xor(v, d, kWave);
+        running += v;
+        closed_seen = closed != 0;
       }
     }
-    const unsigned long long closed = __ballot((s >> 62) == 2);
-    const int first = closed ? __ffsll(static_cast<long long>(closed)) - 1 : kWave;
-    int64_t v = lane <= first ? static_cast<int64_t>(s & kLbValue) : 0;
-#pragma unroll
-    for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_xor(v, d, kWave);
-    running += v;
-    if (closed) break;
-    newest -= kWave;
+    newest -= kLookbackBurst * kWave;
   }
   __threadfence();  // an error raised above is visible before the prefix that hides it
-  if (lane == 0) lb_store(&st.status[tile], kLbInclusive | ((static_cast<unsigned long long>(running) + mine) & kLbValue));
+  if (lane == 0) lb_store(&st.status[tile], lb_word(2u, st.epoch, running + total));
   return running;
 }
 

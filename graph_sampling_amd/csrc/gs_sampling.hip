@@ -521,17 +521,24 @@ int sample_fill_impl(const SampleArgs<IdT>& a, int replace, int algo, hipStream_
 
 
 // ------------------------------------------- one-launch slice + sample ----
-// Counting, the scan of the counts and the fill in ONE kernel: a workgroup
-// takes a tile of 256 rows, one row per lane reads its column id and offsets
-// (256 independent random reads in flight per workgroup instead of the same
-// read repeated by every lane of a row group), the tile's counts are scanned in
-// LDS, the tile prefix comes from a look-back over earlier tiles, and then the
-// row groups of G lanes draw and gather exactly as sample_floyd_kernel /
-// sample_replace_kernel do, reading (start, degree, output offset) from LDS.
+// Counting, the scan of the counts and the fill in ONE kernel.  A workgroup
+// takes a tile of 256 rows:
+//  1. one row per lane reads its column id and offsets (256 independent random
+//     reads in flight per workgroup), the tile's counts are scanned in LDS and
+//     the tile prefix comes from a look-back over earlier tiles;
+//  2. without replacement every lane runs Floyd's selection for its own row in
+//     registers (a fully unrolled k x k duplicate check, four draws per Philox
+//     block) and parks the k chosen positions in LDS;
+//  3. the tile's outputs are then written edge-parallel: lane e finds its row by
+//     binary search in the LDS offsets, so every gather of a lane is independent
+//     of the others and every store is fully coalesced.
 // The outputs must hold S * fanout entries; the true total lands in
-// sub_indptr[S] (and in the host mailbox when one is given).
+// sub_indptr[S] (and in the host mailbox when one is given).  No workgroup does a
+// read-modify-write on a shared address (see the look-back notes).
 constexpr int kFusedThreads = 256;
 constexpr int kFusedRows = 256;
+constexpr int kFusedBatch = 4;  // gathers a lane keeps in flight in the fill
+constexpr int kPickStride = kFusedRows + 1;  // odd stride: conflict-free by row and by step
 
 template <typename IdT>
 struct FusedArgs {
@@ -553,146 +560,141 @@ struct FusedArgs {
   int64_t box_ticket;
 };
 
-template <typename IdT, int G, bool REPLACE>
+template <typename IdT, int KMAX, bool REPLACE>
 __global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<IdT> a) {
+  extern __shared__ uint32_t s_pick[];  // [k][kPickStride], without replacement only
   __shared__ int64_t s_start[kFusedRows];
-  __shared__ int64_t s_deg[kFusedRows];
-  __shared__ int64_t s_out[kFusedRows];
+  __shared__ uint32_t s_deg[kFusedRows];
+  __shared__ uint32_t s_rel[kFusedRows + 1];  // output offsets relative to the tile's first
   __shared__ int64_t s_scan[kFusedThreads / kWave + 1];
   __shared__ int64_t s_prefix;
-  __shared__ unsigned int s_word;
-  const unsigned int tile = lookback_take_ticket(a.lb, &s_word);
+  const unsigned int tile = blockIdx.x;
   const unsigned int tiles = gridDim.x;
   const int64_t row0 = static_cast<int64_t>(tile) * kFusedRows;
   const int k = static_cast<int>(a.k);
+  const int64_t my_row = row0 + threadIdx.x;
 
-  // ---- phase 1: one row per lane
+  // ---- 1. one row per lane
   int64_t start = 0, deg = 0, cnt = 0;
-  {
-    const int64_t r = row0 + threadIdx.x;
-    if (r < a.S) {
-      const int64_t c = a.cols ? static_cast<int64_t>(a.cols[r]) : r;
-      if (valid_col(c, a.num_cols)) {
-        start = a.indptr[c];
-        deg = a.indptr[c + 1] - start;
-      }
-      cnt = REPLACE ? (deg > 0 ? a.k : 0) : (deg < a.k ? deg : a.k);
+  if (my_row < a.S) {
+    const int64_t c = a.cols ? static_cast<int64_t>(a.cols[my_row]) : my_row;
+    if (valid_col(c, a.num_cols)) {
+      start = a.indptr[c];
+      deg = a.indptr[c + 1] - start;
     }
+    cnt = REPLACE ? (deg > 0 ? a.k : 0) : (deg < a.k ? deg : a.k);
   }
   int64_t tile_total;
   const int64_t local = block_exclusive_scan<kFusedThreads>(cnt, &tile_total, s_scan);
+  if (threadIdx.x == 0) lookback_publish_sum(a.lb, tile, tile_total);
+  s_start[threadIdx.x] = start;
+  s_deg[threadIdx.x] = static_cast<uint32_t>(deg);
+  s_rel[threadIdx.x] = static_cast<uint32_t>(local);
+  if (threadIdx.x == 0) s_rel[kFusedRows] = static_cast<uint32_t>(tile_total);
+
+  // ---- 2. Floyd's selection, one row per lane, positions to LDS
+  if (!REPLACE && cnt > 0) {
+    if (deg <= a.k) {
+      for (int i = 0; i < static_cast<int>(deg); ++i) s_pick[i * kPickStride + threadIdx.x] = i;
+    } else {
+      const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[my_row] : nullptr;
+      uint32_t chosen[KMAX];
+      U4 blk;
+#pragma unroll
+      for (int i = 0; i < KMAX; ++i) {
+        if (i < k) {
+          if ((i & 3) == 0 && !rp)
+            blk = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(my_row),
+                             static_cast<uint64_t>(i >> 2));
+          const uint32_t xv = rp ? rp[i] : blk.v[i & 3];
+          const uint32_t j = static_cast<uint32_t>(deg - a.k + i);
+          const uint32_t t = xv % (j + 1u);
+          bool taken = false;
+#pragma unroll
+          for (int m = 0; m < i; ++m) taken |= chosen[m] == t;
+          chosen[i] = taken ? j : t;
+          s_pick[i * kPickStride + threadIdx.x] = chosen[i];
+        }
+      }
+    }
+  }
   if (threadIdx.x < kWave) {
     const int64_t before = lookback_exclusive_prefix(a.lb, tile, tile_total);
     if (threadIdx.x == 0) s_prefix = before;
   }
   __syncthreads();
-  {
-    const int64_t out = s_prefix + local;
-    s_start[threadIdx.x] = start;
-    s_deg[threadIdx.x] = deg;
-    s_out[threadIdx.x] = out;
-    const int64_t r = row0 + threadIdx.x;
-    if (r < a.S) a.sub_indptr[r] = out;
-  }
+  const int64_t out0 = s_prefix;
+  if (my_row < a.S) a.sub_indptr[my_row] = out0 + local;
   if (tile == tiles - 1 && threadIdx.x == 0) {
-    int64_t total = s_prefix + tile_total;
+    int64_t total = out0 + tile_total;
     if (__hip_atomic_load(a.lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) total = -1;
     a.sub_indptr[a.S] = total;
     post_mailbox(a.box, total, a.box_ticket);
   }
-  __syncthreads();
 
-  // ---- phase 2: G lanes per row
-  constexpr int kGroups = kFusedThreads / G;
-  const int lane = threadIdx.x % G;
-  for (int row = threadIdx.x / G; row < kFusedRows; row += kGroups) {
-    const int64_t r = row0 + row;
-    if (r >= a.S) break;
-    const int64_t st = s_start[row];
-    const int64_t d = s_deg[row];
-    const int64_t out = s_out[row];
-    if (REPLACE) {
-      if (d == 0) continue;
-      const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[r] : nullptr;
-      for (int64_t q = lane; q * 4 < a.k; q += G) {
-        U4 x;
-        if (!rp) x = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(r), static_cast<uint64_t>(q));
+  // ---- 3. edge-parallel gather and store, kFusedBatch gathers in flight per lane
+  const uint32_t n_out = static_cast<uint32_t>(tile_total);
+  const IdT* __restrict__ indices = a.indices;
+  for (uint32_t base = threadIdx.x; base < n_out; base += kFusedThreads * kFusedBatch) {
+    int64_t q[kFusedBatch];
+    int64_t r[kFusedBatch];
+    IdT v[kFusedBatch];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int64_t j = q * 4 + t;
-          if (j < a.k) {
-            const uint32_t xv = rp ? rp[j] : x.v[t];
-            const int64_t p = st + static_cast<int64_t>(xv % static_cast<uint32_t>(d));
-            a.sub_indices[out + j] = a.indices[p];
-            a.select_index[out + j] = p;
-            if (a.coo_col) a.coo_col[out + j] = static_cast<IdT>(r);
-          }
+    for (int u = 0; u < kFusedBatch; ++u) {
+      const uint32_t e = base + u * kFusedThreads;
+      q[u] = -1;
+      if (e < n_out) {
+        int lo = 0, hi = kFusedRows;  // last row with s_rel[row] <= e
+        while (lo < hi) {
+          const int mid = (lo + hi) >> 1;
+          if (s_rel[mid] <= e) lo = mid + 1; else hi = mid;
         }
+        const int row = lo - 1;
+        const uint32_t j = e - s_rel[row];
+        r[u] = row0 + row;
+        uint32_t pick;
+        if (REPLACE) {
+          const uint32_t xv = a.replay ? a.replay[a.replay_ptr[r[u]] + j]
+                                       : draw_one(a.seed, kTagUniform, static_cast<uint64_t>(r[u]),
+                                                  static_cast<uint64_t>(j));
+          pick = xv % s_deg[row];
+        } else {
+          pick = s_pick[j * kPickStride + row];
+        }
+        q[u] = s_start[row] + pick;
+        v[u] = indices[q[u]];
       }
-      continue;
     }
-    if (d <= k) {
-      if (lane < d) {
-        a.sub_indices[out + lane] = a.indices[st + lane];
-        a.select_index[out + lane] = st + lane;
-        if (a.coo_col) a.coo_col[out + lane] = static_cast<IdT>(r);
+#pragma unroll
+    for (int u = 0; u < kFusedBatch; ++u) {
+      const uint32_t e = base + u * kFusedThreads;
+      if (q[u] >= 0) {
+        a.sub_indices[out0 + e] = v[u];
+        a.select_index[out0 + e] = q[u];
+        if (a.coo_col) a.coo_col[out0 + e] = static_cast<IdT>(r[u]);
       }
-      continue;
-    }
-    uint32_t t = 0, j = 0;
-    if (lane < k) {
-      const uint32_t xv = a.replay ? a.replay[a.replay_ptr[r] + lane]
-                                   : draw_one(a.seed, kTagUniform, static_cast<uint64_t>(r),
-                                              static_cast<uint64_t>(lane));
-      j = static_cast<uint32_t>(d - k + lane);
-      t = xv % (j + 1u);
-    }
-    bool taken = false;
-    for (int m = 0; m < k - 1; ++m) {
-      const uint32_t chosen_m = __shfl(taken ? j : t, m, G);
-      if (lane > m && t == chosen_m) taken = true;
-    }
-    if (lane < k) {
-      const int64_t q = st + (taken ? j : t);
-      a.sub_indices[out + lane] = a.indices[q];
-      a.select_index[out + lane] = q;
-      if (a.coo_col) a.coo_col[out + lane] = static_cast<IdT>(r);
-    }
-  }
-
-  // ---- leave the look-back state zeroed for the next call
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    __threadfence();
-    s_word = atomicAdd(a.lb.done, 1u) == tiles - 1 ? 1u : 0u;
-  }
-  __syncthreads();
-  if (s_word) {
-    for (unsigned int i = threadIdx.x; i < tiles; i += kFusedThreads) a.lb.status[i] = 0ull;
-    if (threadIdx.x == 0) {
-      *a.lb.ticket = 0u;
-      *a.lb.done = 0u;
-      *a.lb.error = 0u;
     }
   }
 }
 
-template <typename IdT, bool REPLACE>
-int sample_fused_launch(const FusedArgs<IdT>& a, hipStream_t stream) {
+template <typename IdT>
+int sample_fused_launch(const FusedArgs<IdT>& a, bool replace, hipStream_t stream) {
   const unsigned grid = static_cast<unsigned>((a.S + kFusedRows - 1) / kFusedRows);
   ProfileScope prof("sample_fused", stream);
-  const int g = a.k <= 8 ? 8 : (a.k <= 16 ? 16 : (a.k <= 32 ? 32 : 64));
-  if (g == 8)
-    hipLaunchKernelGGL((sample_fused_kernel<IdT, 8, REPLACE>), dim3(grid), dim3(kFusedThreads), 0,
+  if (replace) {
+    hipLaunchKernelGGL((sample_fused_kernel<IdT, 1, true>), dim3(grid), dim3(kFusedThreads), 0,
                        stream, a);
-  else if (g == 16)
-    hipLaunchKernelGGL((sample_fused_kernel<IdT, 16, REPLACE>), dim3(grid), dim3(kFusedThreads), 0,
+    return check_launch("sample_fused");
+  }
+  const size_t lds = static_cast<size_t>(a.k) * kPickStride * sizeof(uint32_t);
+  if (a.k <= 8)
+    hipLaunchKernelGGL((sample_fused_kernel<IdT, 8, false>), dim3(grid), dim3(kFusedThreads), lds,
                        stream, a);
-  else if (g == 32)
-    hipLaunchKernelGGL((sample_fused_kernel<IdT, 32, REPLACE>), dim3(grid), dim3(kFusedThreads), 0,
+  else if (a.k <= 16)
+    hipLaunchKernelGGL((sample_fused_kernel<IdT, 16, false>), dim3(grid), dim3(kFusedThreads), lds,
                        stream, a);
   else
-    hipLaunchKernelGGL((sample_fused_kernel<IdT, 64, REPLACE>), dim3(grid), dim3(kFusedThreads), 0,
+    hipLaunchKernelGGL((sample_fused_kernel<IdT, 32, false>), dim3(grid), dim3(kFusedThreads), lds,
                        stream, a);
   return check_launch("sample_fused");
 }
@@ -726,7 +728,7 @@ int sample_fused_t(const int64_t* indptr, int64_t num_cols, const void* indices,
                    lb,
                    box,
                    ticket};
-  return replace ? sample_fused_launch<IdT, true>(a, st) : sample_fused_launch<IdT, false>(a, st);
+  return sample_fused_launch<IdT>(a, replace != 0, st);
 }
 
 }  // namespace
@@ -884,8 +886,8 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
                             int replace, uint64_t seed, const uint32_t* replay,
                             const int64_t* replay_ptr, int64_t* sub_indptr, void* sub_indices,
                             int64_t* select_index, void* coo_col, int64_t capacity,
-                            void* zeroed_state, size_t state_bytes, gs_mailbox* mailbox,
-                            int64_t mailbox_ticket, void* stream) {
+                            void* state, size_t state_bytes, uint32_t epoch,
+                            gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream) {
   GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0 && num_cols >= 0,
              "gs_sample_uniform_fused: null pointer or negative size");
   GS_REQUIRE(column_ids || S <= num_cols,
@@ -894,10 +896,10 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
              id_bytes);
   GS_REQUIRE((replay == nullptr) == (replay_ptr == nullptr),
              "gs_sample_uniform_fused: replay and replay_ptr must be given together");
-  if (!replace && fanout > GS_FLOYD_MAX_FANOUT) {
+  if (!replace && fanout > GS_FUSED_MAX_FANOUT) {
     set_error_text("gs_sample_uniform_fused: fanout %lld without replacement exceeds %d; use "
                    "gs_sample_count + gs_sample_uniform_fill",
-                   static_cast<long long>(fanout), GS_FLOYD_MAX_FANOUT);
+                   static_cast<long long>(fanout), GS_FUSED_MAX_FANOUT);
     return GS_ERR_UNSUPPORTED;
   }
   GS_REQUIRE(S == 0 || fanout == 0 || capacity >= S * fanout,
@@ -911,10 +913,14 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
                        mailbox_ticket);
     return check_launch("sample_fused");
   }
-  Carver ws(zeroed_state, state_bytes);
-  LookbackState lb = carve_lookback(ws, (S + kFusedRows - 1) / kFusedRows);
+  GS_REQUIRE(epoch >= 1 && epoch <= kLbMaxEpoch,
+             "gs_sample_uniform_fused: epoch must be 1..%u, got %u", kLbMaxEpoch, epoch);
+  GS_REQUIRE(S * fanout <= static_cast<int64_t>(kLbValue),
+             "gs_sample_uniform_fused: S * fanout exceeds 2^48");
+  Carver ws(state, state_bytes);
+  LookbackState lb = carve_lookback(ws, (S + kFusedRows - 1) / kFusedRows, epoch);
   if (!ws.ok) {
-    set_error_text("gs_sample_uniform_fused: state needs %zu zeroed bytes, 256-byte aligned",
+    set_error_text("gs_sample_uniform_fused: state needs %zu bytes, 256-byte aligned",
                    gs_sample_fused_state_bytes(S));
     return GS_ERR_WORKSPACE;
   }

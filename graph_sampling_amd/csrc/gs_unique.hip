@@ -152,11 +152,7 @@ __global__ void __launch_bounds__(kThreads) table_init_kernel(T t, int64_t cap, 
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i < cap) t.clear(i);
   if (i < tiles) lb.status[i] = 0ull;
-  if (i == 0) {
-    *lb.ticket = 0u;
-    *lb.done = 0u;
-    *lb.error = 0u;
-  }
+  if (i == 0) *lb.error = 0u;
 }
 
 // insert (key -> min index) and remember the slot of every item
@@ -193,8 +189,7 @@ compact_kernel(Spans<IdT> x, int64_t M, T t, const uint32_t* __restrict__ pos,
                int64_t box_ticket) {
   __shared__ int64_t s_scan[kThreads / kWave + 1];
   __shared__ int64_t s_prefix;
-  __shared__ unsigned int s_word;
-  const unsigned int tile = lookback_take_ticket(lb, &s_word);
+  const unsigned int tile = blockIdx.x;
   const int64_t base = static_cast<int64_t>(tile) * kCompactTile +
                        static_cast<int64_t>(threadIdx.x) * kCompactItems;
   bool first[kCompactItems];
@@ -207,6 +202,10 @@ compact_kernel(Spans<IdT> x, int64_t M, T t, const uint32_t* __restrict__ pos,
   }
   int64_t tile_total;
   const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
+  if (threadIdx.x == 0) lookback_publish_sum(lb, tile, tile_total);
+  IdT key[kCompactItems];  // in flight while wave 0 walks back
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) key[k] = first[k] ? x.get(base + k) : IdT(0);
   if (threadIdx.x < kWave) {
     const int64_t before = lookback_exclusive_prefix(lb, tile, tile_total);
     if (threadIdx.x == 0) s_prefix = before;
@@ -218,7 +217,7 @@ compact_kernel(Spans<IdT> x, int64_t M, T t, const uint32_t* __restrict__ pos,
     const int64_t i = base + k;
     if (i < M) {
       prefix[i] = run;
-      if (first[k]) frontier[run] = x.get(i);
+      if (first[k]) frontier[run] = key[k];
     }
     run += first[k] ? 1 : 0;
   }
@@ -299,7 +298,7 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   uint32_t* pos = ws.take<uint32_t>(M > 0 ? M : 1);
   int64_t* prefix = ws.take<int64_t>(M + 1);
   const int64_t tiles = compact_num_tiles(M);
-  LookbackState lb = carve_lookback(ws, tiles);
+  LookbackState lb = carve_lookback(ws, tiles, 1u);  // cleared by table_init on every call
   if (!ws.ok) {
     set_error_text("gs_unique_relabel: workspace needs %zu bytes, 256-byte aligned",
                    workspace_bytes_for<IdT>(M));

@@ -1,8 +1,10 @@
 #include "hip_ops.h"
 
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
 
 #include <atomic>
+#include <map>
 
 #include "gs_hip.h"
 
@@ -12,6 +14,7 @@ namespace {
 
 std::atomic<uint64_t> g_seed{7777};
 std::atomic<int64_t> g_algo{GS_SAMPLE_AUTO};
+constexpr int64_t kOneLaunchMaxColumns = 1 << 18;
 
 void Check(int status, const char* what) {
   TORCH_CHECK(status == GS_OK, what, " failed (", status, "): ", gs_status_string(status));
@@ -55,6 +58,68 @@ const int64_t* OptI64(const torch::optional<torch::Tensor>& t, const char* name)
 torch::Tensor Scratch(size_t bytes, const torch::Tensor& like) {
   return torch::empty({static_cast<int64_t>(bytes < 256 ? 256 : bytes)},
                       torch::dtype(torch::kUInt8).device(like.device()));
+}
+
+// ---- result mailbox: totals arrive in pinned host memory, no stream sync ----
+struct HostBox {
+  torch::Tensor buf;  // 2 x int64, pinned
+  gs_mailbox* box = nullptr;
+  int64_t next = 1;
+};
+
+HostBox& Box(int device) {
+  thread_local std::map<int, HostBox> boxes;
+  HostBox& b = boxes[device];
+  if (!b.box) {
+    b.buf = torch::zeros({2}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+    b.box = reinterpret_cast<gs_mailbox*>(b.buf.data_ptr<int64_t>());
+  }
+  return b;
+}
+
+// Spins until the kernel has posted `ticket`; every few thousand polls it asks
+// the stream whether it has drained or failed, so a kernel that never posts
+// turns into an error, not a hang.
+int64_t WaitBox(HostBox& b, int64_t ticket, void* stream, const char* what) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  for (uint64_t n = 1;; ++n) {
+    if (__atomic_load_n(&b.box->ticket, __ATOMIC_ACQUIRE) == ticket) break;
+    if ((n & 0xFFF) == 0) {
+      const hipError_t q = hipStreamQuery(st);
+      if (q == hipSuccess) {
+        if (__atomic_load_n(&b.box->ticket, __ATOMIC_ACQUIRE) == ticket) break;
+        TORCH_CHECK(false, what, ": the stream drained without reporting a total");
+      }
+      TORCH_CHECK(q == hipErrorNotReady, what, ": ", hipGetErrorString(q));
+    }
+    __builtin_ia32_pause();
+  }
+  const int64_t total = __atomic_load_n(&b.box->total, __ATOMIC_RELAXED);
+  TORCH_CHECK(total >= 0, what, ": a tile gave up waiting for its predecessors");
+  return total;
+}
+
+// Look-back state of the one-launch sampler, one per (device, stream): zero-filled
+// when it is (re)allocated and when the epoch counter wraps, never in between.
+struct FusedStateBuf {
+  torch::Tensor buf;
+  uint32_t epoch = 0;
+};
+
+FusedStateBuf& FusedState(size_t bytes, const torch::Tensor& like, void* stream) {
+  thread_local std::map<std::pair<int, void*>, FusedStateBuf> states;
+  FusedStateBuf& s = states[{like.device().index(), stream}];
+  if (!s.buf.defined() || static_cast<size_t>(s.buf.numel()) < bytes) {
+    const int64_t n = static_cast<int64_t>(bytes < 65536 ? 65536 : bytes);
+    s.buf = torch::zeros({n}, torch::dtype(torch::kUInt8).device(like.device()));
+    s.epoch = 0;
+  }
+  if (s.epoch == 16383) {
+    s.buf.zero_();
+    s.epoch = 0;
+  }
+  ++s.epoch;
+  return s;
 }
 
 torch::TensorOptions I64(const torch::Tensor& like) {
@@ -141,9 +206,51 @@ SliceResult SampleInto(const torch::Tensor& indptr, const torch::Tensor& indices
 
 }  // namespace
 
+// One launch, no mid-call host read; the total arrives through the mailbox.
+SliceResult ColSamplingOneLaunch(const torch::Tensor& indptr, const torch::Tensor& indices,
+                                 const torch::Tensor& column_ids, int64_t fanout, bool replace,
+                                 bool with_coo) {
+  NeedI64(indptr, "indptr");
+  const int idb = IdBytes(indices, "indices");
+  const bool fused = column_ids.defined();
+  if (fused)
+    TORCH_CHECK(IdBytes(column_ids, "column ids") == idb, "column ids and indices differ in dtype");
+  const int64_t S = fused ? column_ids.numel() : indptr.numel() - 1;
+  auto sub_indptr = torch::empty({S + 1}, I64(indptr));
+  const int64_t cap = S * fanout;
+  auto sub_indices = torch::empty({cap}, indices.options());
+  auto select_index = torch::empty({cap}, I64(indptr));
+  torch::Tensor coo_col;
+  if (with_coo) coo_col = torch::empty({cap}, indices.options());
+  void* st = Stream(indptr);
+  FusedStateBuf& state = FusedState(gs_sample_fused_state_bytes(S), indptr, st);
+  HostBox& box = Box(indptr.device().index());
+  const int64_t ticket = box.next++;
+  Check(gs_sample_uniform_fused(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(),
+                                fused ? column_ids.data_ptr() : nullptr, idb, S, fanout,
+                                replace ? 1 : 0, NextSeed(), nullptr, nullptr,
+                                sub_indptr.data_ptr<int64_t>(), sub_indices.data_ptr(),
+                                select_index.data_ptr<int64_t>(),
+                                with_coo ? coo_col.data_ptr() : nullptr, cap,
+                                state.buf.data_ptr(), state.buf.numel(), state.epoch, box.box,
+                                ticket, st),
+        "gs_sample_uniform_fused");
+  const int64_t nnz = WaitBox(box, ticket, st, "gs_sample_uniform_fused");
+  if (with_coo) coo_col = coo_col.narrow(0, 0, nnz);
+  return {sub_indptr, coo_col, sub_indices.narrow(0, 0, nnz), select_index.narrow(0, 0, nnz)};
+}
+
 SliceResult ColSampling(const torch::Tensor& indptr, const torch::Tensor& indices,
                         const torch::Tensor& column_ids, int64_t fanout, bool replace,
                         bool with_coo) {
+  TORCH_CHECK(fanout >= 0, "fanout must be non-negative");
+  // One launch wins while launch and round-trip latency dominate (measured: 3-4x at 45k
+  // columns); past a few hundred thousand columns the chained scan's per-tile walk costs
+  // more than the two extra launches of the count / fill pair save.
+  const int64_t S = column_ids.defined() ? column_ids.numel() : indptr.numel() - 1;
+  if (g_algo.load() == GS_SAMPLE_AUTO && S <= kOneLaunchMaxColumns &&
+      (replace || fanout <= GS_FUSED_MAX_FANOUT))
+    return ColSamplingOneLaunch(indptr, indices, column_ids, fanout, replace, with_coo);
   return SampleInto(
       indptr, indices, column_ids, fanout, replace, with_coo, 0,
       [&](const void* cols, int idb, int64_t S, torch::Tensor& sub_indptr, torch::Tensor& sub_indices,
@@ -223,11 +330,15 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> Relabel(
   auto frontier = torch::empty({M}, mapping[0].options());
   auto num = torch::empty({1}, I64(mapping[0]));
   auto ws = Scratch(gs_unique_workspace_bytes(M), mapping[0]);
-  Check(gs_unique_relabel(m, static_cast<int>(mapping.size()), q, out_ptr,
-                          static_cast<int>(queries.size()), idb, frontier.data_ptr(),
-                          num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), Stream(mapping[0])),
+  void* st = Stream(mapping[0]);
+  HostBox& box = Box(mapping[0].device().index());
+  const int64_t ticket = box.next++;
+  Check(gs_unique_relabel_notify(m, static_cast<int>(mapping.size()), q, out_ptr,
+                                 static_cast<int>(queries.size()), idb, frontier.data_ptr(),
+                                 num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), box.box, ticket,
+                                 st),
         "gs_unique_relabel");
-  const int64_t U = num.item<int64_t>();
+  const int64_t U = WaitBox(box, ticket, st, "gs_unique_relabel");
   return {frontier.narrow(0, 0, U), outs};
 }
 

@@ -123,6 +123,8 @@ size_t gs_sample_workspace_bytes(int64_t S, int64_t fanout);
  *      which case j is.  fanout draws whatever the degree; output in step order. */
 typedef enum gs_sample_algo { GS_SAMPLE_AUTO = 0, GS_SAMPLE_RESERVOIR = 1 } gs_sample_algo;
 #define GS_FLOYD_MAX_FANOUT 64
+/* largest fanout without replacement of the one-launch gs_sample_uniform_fused */
+#define GS_FUSED_MAX_FANOUT 32
 
 /* sub_indptr = exscan(cnt), cnt = replace ? (deg ? fanout : 0) : min(deg, fanout)
  * (sampling.cu:107-119). */
@@ -152,24 +154,26 @@ int gs_sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const void* 
  * impl::fusion::FusedCSCColSlicingSamplingCUDA (src/cuda/fusion/slice_sampling.cu:146)
  * and, with column_ids == NULL, impl::CSCColSamplingCUDA (src/cuda/sampling.cu:157),
  * without their mid-call host read.
- *   - without replacement fanout must be <= GS_FLOYD_MAX_FANOUT (else
+ *   - without replacement fanout must be <= GS_FUSED_MAX_FANOUT (else
  *     GS_ERR_UNSUPPORTED: use the two-phase calls);
  *   - sub_indices / select_index / coo_col hold `capacity` >= S*fanout entries;
  *     the true total is written to sub_indptr[S] (-1 if the kernel gave up
  *     waiting on another tile, which a healthy device never does) and to the
  *     mailbox when one is given;
- *   - zeroed_state: gs_sample_fused_state_bytes(S) bytes, 256-byte aligned, ALL
- *     ZERO on entry; the kernel leaves them zero again, so one buffer cleared
- *     once serves every later call on the same stream.  Two calls running at the
- *     same time must not share it. */
+ *   - state: gs_sample_fused_state_bytes(S) bytes, 256-byte aligned, zero-filled
+ *     before its first use; epoch: 1..16383, different from the epoch of every
+ *     earlier call on this buffer since it was last zero-filled (count up from
+ *     1; zero-fill and start again after 16383).  Tiles mark their progress in
+ *     `state` with the epoch, so nothing is cleared between calls.  Two calls
+ *     running at the same time must not share a buffer. */
 size_t gs_sample_fused_state_bytes(int64_t S);
 int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void* indices,
                             const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
                             int replace, uint64_t seed, const uint32_t* replay,
                             const int64_t* replay_ptr, int64_t* sub_indptr, void* sub_indices,
                             int64_t* select_index, void* coo_col, int64_t capacity,
-                            void* zeroed_state, size_t state_bytes, gs_mailbox* mailbox,
-                            int64_t mailbox_ticket, void* stream);
+                            void* state, size_t state_bytes, uint32_t epoch,
+                            gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
 
 /* fanout == 1 with replacement through the fused entry: exactly one slot per
  * column, -1 in both outputs for an empty column; sub_indptr = 0..S.  Replaces
