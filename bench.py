@@ -77,14 +77,15 @@ class KernelTimer:
 # launch sites of one minibatch step and the bytes each launch must move at the
 # least (id_bytes b; S seeds, E sampled edges, M = S + E items, U unique ids):
 #   sample_fused  : per seed  column id b + two offsets 16 + output offset 8,
-#                   per edge  neighbour gather b + sub_indices b + select_index 8
+#                   per edge  neighbour gather b + sub_indices b (no select_index: the graph
+#                   carries no edge data, so the host layer does not ask for it)
 #   table_insert  : per item  id b + one 8-byte slot read-modify-write 16 + slot index 4
 #   unique_finish : per item  slot index 4 + slot 8 + rank 8, relabeled id b, frontier b per U
 SITES = ("sample_fused", "table_init", "table_insert", "unique_compact", "unique_finish")
 
 
 def floyd_bytes(b, S, E):
-    return S * (b + 24) + E * (2 * b + 8)
+    return S * (b + 24) + E * 2 * b
 
 
 def insert_bytes(b, S, E):
@@ -207,7 +208,6 @@ def main():
 
     torch.ops.gs_ops._CAPI_SetSeed(args.warmup * len(FANOUTS))
     timer.enable(dominant)
-    lat = []
     sampled = 0
     layer_sizes = None
     first = None
@@ -216,10 +216,9 @@ def main():
     torch.cuda.synchronize()
     t_begin = time.perf_counter()
     for i in range(args.steps):
-        t1 = time.perf_counter()
+        # a step ends when the host holds every tensor size of the minibatch (the last
+        # relabel hands back the frontier length); nothing else synchronises inside the loop
         n, sizes, frontier = minibatch(graph, seed_sets[args.warmup + i])
-        torch.cuda.synchronize()
-        lat.append(time.perf_counter() - t1)
         sampled += n
         layer_sizes = sizes
         algo_bytes += sum(SITE_BYTES[dominant](b, S, E) for S, E, _ in sizes)
@@ -229,6 +228,16 @@ def main():
     elapsed = time.perf_counter() - t_begin
     k_ms, k_launches, _ = timer.collect()
     timer.enable("")
+
+    # latency of one minibatch with the device drained before and after it (untimed pass over
+    # the same seed sets)
+    lat = []
+    for i in range(args.steps):
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        minibatch(graph, seed_sets[args.warmup + i])
+        torch.cuda.synchronize()
+        lat.append(time.perf_counter() - t1)
     lat.sort()
     p50 = lat[len(lat) // 2] * 1e3
     p90 = lat[min(len(lat) - 1, int(len(lat) * 0.9))] * 1e3

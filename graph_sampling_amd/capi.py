@@ -354,7 +354,7 @@ class _Span(ctypes.Structure):
     _fields_ = [("ptr", ctypes.c_void_p), ("n", ctypes.c_int64)]
 
 
-def unique_relabel(mapping, queries, mailbox=None):
+def unique_relabel(mapping, queries, mailbox=None, last_span_len=None):
     """gs_unique_relabel[_notify].  mapping / queries: lists of 1-D id tensors (one dtype).
 
     Returns (frontier_buf, num_unique_dev, [relabelled query tensors]); frontier_buf has
@@ -375,11 +375,14 @@ def unique_relabel(mapping, queries, mailbox=None):
     q_arr = QArr(*[_Span(t.data_ptr(), t.numel()) for t in queries]) if queries else QArr()
     o_arr = OutArr(*[t.data_ptr() for t in outs]) if queries else OutArr()
     ws = workspace(lib().gs_unique_workspace_bytes(_i64(M)), dev)
-    if mailbox is not None:
-        ticket = mailbox.ticket()
+    if mailbox is not None or last_span_len is not None:
+        # last_span_len: 1-element int64 device tensor holding the true length of mapping[-1]
+        ticket = mailbox.ticket() if mailbox is not None else 0
         _check(lib().gs_unique_relabel_notify(m_arr, len(mapping), q_arr, o_arr, len(queries), idb,
                                               _ptr(frontier), _ptr(num_unique), _ptr(ws),
-                                              ctypes.c_size_t(ws.numel()), mailbox.ptr(),
+                                              ctypes.c_size_t(ws.numel()), _ptr(last_span_len),
+                                              mailbox.ptr() if mailbox is not None
+                                              else ctypes.c_void_p(0),
                                               _i64(ticket), _stream(dev)),
                "gs_unique_relabel_notify")
         return frontier, num_unique, outs, ticket

@@ -670,7 +670,7 @@ __global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<I
       const uint32_t e = base + u * kFusedThreads;
       if (q[u] >= 0) {
         a.sub_indices[out0 + e] = v[u];
-        a.select_index[out0 + e] = q[u];
+        if (a.select_index) a.select_index[out0 + e] = q[u];
         if (a.coo_col) a.coo_col[out0 + e] = static_cast<IdT>(r[u]);
       }
     }
@@ -905,7 +905,7 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
   GS_REQUIRE(S == 0 || fanout == 0 || capacity >= S * fanout,
              "gs_sample_uniform_fused: outputs must hold S * fanout = %lld entries, capacity is %lld",
              static_cast<long long>(S * fanout), static_cast<long long>(capacity));
-  GS_REQUIRE(S == 0 || fanout == 0 || (indices && sub_indices && select_index),
+  GS_REQUIRE(S == 0 || fanout == 0 || (indices && sub_indices),
              "gs_sample_uniform_fused: null buffer");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (S == 0) {

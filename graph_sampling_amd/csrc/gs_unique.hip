@@ -34,6 +34,16 @@ struct Spans {
   const IdT* ptr[GS_MAX_SPANS];
   int64_t end[GS_MAX_SPANS];  // exclusive end offset of each span in the concatenation
   int n;
+  // When last_len is set the last span's length lives on the device (a total an
+  // earlier kernel on the stream produced and the host has not read yet):
+  // items = fixed + max(*last_len, 0), and the host-side count is only a bound.
+  const int64_t* last_len;
+  int64_t fixed;
+  __device__ __forceinline__ int64_t items(int64_t host_items) const {
+    if (!last_len) return host_items;
+    const int64_t n_last = *last_len;
+    return fixed + (n_last > 0 ? n_last : 0);
+  }
   __device__ __forceinline__ IdT get(int64_t i) const {
     int s = 0;
     int64_t begin = 0;
@@ -159,9 +169,9 @@ __global__ void __launch_bounds__(kThreads) table_init_kernel(T t, int64_t cap, 
 // (unique_reindex.cu:92-99)
 template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
-table_insert_kernel(Spans<IdT> x, int64_t M, T t, uint32_t* __restrict__ pos) {
+table_insert_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ pos) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (i >= M) return;
+  if (i >= x.items(M_bound)) return;
   pos[i] = t.insert(static_cast<long long>(x.get(i)), static_cast<uint32_t>(i));
 }
 
@@ -183,12 +193,13 @@ constexpr int kCompactTile = kThreads * kCompactItems;
 
 template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
-compact_kernel(Spans<IdT> x, int64_t M, T t, const uint32_t* __restrict__ pos,
+compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ pos,
                int64_t* __restrict__ prefix, IdT* __restrict__ frontier,
                int64_t* __restrict__ num_unique, LookbackState lb, gs_mailbox* box,
                int64_t box_ticket) {
   __shared__ int64_t s_scan[kThreads / kWave + 1];
   __shared__ int64_t s_prefix;
+  const int64_t M = x.items(M_bound);
   const unsigned int tile = blockIdx.x;
   const int64_t base = static_cast<int64_t>(tile) * kCompactTile +
                        static_cast<int64_t>(threadIdx.x) * kCompactItems;
@@ -233,8 +244,13 @@ compact_kernel(Spans<IdT> x, int64_t M, T t, const uint32_t* __restrict__ pos,
 template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
 lookup_kernel(T t, const uint32_t* __restrict__ pos, const int64_t* __restrict__ prefix, Query qs,
-              int64_t Q) {
+              int64_t Q_bound, const int64_t* __restrict__ q_len) {
   const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  int64_t Q = Q_bound;
+  if (q_len) {  // one query that aliases the device-sized last mapping span
+    Q = *q_len;
+    if (Q > Q_bound) Q = Q_bound;
+  }
   if (j >= Q) return;
   int s = 0;
   int64_t begin = 0;
@@ -276,8 +292,8 @@ size_t workspace_bytes_for(int64_t M) {
 template <typename IdT>
 int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* query,
                         void* const* query_out, int n_query, void* frontier, int64_t* num_unique,
-                        void* workspace, size_t workspace_bytes, gs_mailbox* box,
-                        int64_t box_ticket, hipStream_t stream) {
+                        void* workspace, size_t workspace_bytes, const int64_t* last_span_len,
+                        gs_mailbox* box, int64_t box_ticket, hipStream_t stream) {
   using T = typename TableFor<IdT>::type;
   Spans<IdT> x;
   int64_t M = 0;
@@ -291,6 +307,8 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
     x.end[s] = M;
   }
   x.n = n_mapping;
+  x.last_len = last_span_len;
+  x.fixed = M - mapping[n_mapping - 1].n;
   const int64_t cap = table_capacity(M);
   Carver ws(workspace, workspace_bytes);
   T t;
@@ -350,7 +368,7 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   if (Q > 0) {
     ProfileScope prof("unique_finish", stream);
     hipLaunchKernelGGL((lookup_kernel<IdT, T>), dim3(blocks_for(Q, kThreads)), dim3(kThreads), 0,
-                       stream, t, pos, prefix, qs, Q);
+                       stream, t, pos, prefix, qs, Q, last_span_len);
   }
   return check_launch("unique_relabel");
 }
@@ -372,7 +390,8 @@ size_t gs_unique_workspace_bytes(int64_t M) {
 int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_span* query,
                              void* const* query_out, int n_query, int id_bytes, void* frontier,
                              int64_t* num_unique, void* workspace, size_t workspace_bytes,
-                             gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream) {
+                             const int64_t* last_span_len, gs_mailbox* mailbox,
+                             int64_t mailbox_ticket, void* stream) {
   GS_REQUIRE(mapping && n_mapping >= 1 && n_mapping <= GS_MAX_SPANS,
              "gs_unique_relabel: 1..%d mapping spans required, got %d", GS_MAX_SPANS, n_mapping);
   GS_REQUIRE(n_query >= 0 && n_query <= GS_MAX_SPANS && (n_query == 0 || (query && query_out)),
@@ -394,13 +413,20 @@ int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_spa
                    static_cast<long long>(M));
     return GS_ERR_UNSUPPORTED;
   }
+  if (last_span_len) {
+    const gs_span& last = mapping[n_mapping - 1];
+    GS_REQUIRE(n_query == 0 || (n_query == 1 && query[0].ptr == last.ptr && query[0].n == last.n),
+               "gs_unique_relabel_notify: with a device-side length the only query allowed is "
+               "the last mapping span itself");
+  }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return id_bytes == 8 ? unique_relabel_impl<int64_t>(mapping, n_mapping, query, query_out, n_query,
-                                                      frontier, num_unique, workspace,
-                                                      workspace_bytes, mailbox, mailbox_ticket, st)
-                       : unique_relabel_impl<int32_t>(mapping, n_mapping, query, query_out, n_query,
-                                                      frontier, num_unique, workspace,
-                                                      workspace_bytes, mailbox, mailbox_ticket, st);
+  return id_bytes == 8
+             ? unique_relabel_impl<int64_t>(mapping, n_mapping, query, query_out, n_query, frontier,
+                                            num_unique, workspace, workspace_bytes, last_span_len,
+                                            mailbox, mailbox_ticket, st)
+             : unique_relabel_impl<int32_t>(mapping, n_mapping, query, query_out, n_query, frontier,
+                                            num_unique, workspace, workspace_bytes, last_span_len,
+                                            mailbox, mailbox_ticket, st);
 }
 
 int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* query,
@@ -408,7 +434,8 @@ int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* quer
                       int64_t* num_unique, void* workspace, size_t workspace_bytes,
                       void* stream) {
   return gs_unique_relabel_notify(mapping, n_mapping, query, query_out, n_query, id_bytes, frontier,
-                                  num_unique, workspace, workspace_bytes, nullptr, 0, stream);
+                                  num_unique, workspace, workspace_bytes, nullptr, nullptr, 0,
+                                  stream);
 }
 
 }  // extern "C"

@@ -79,12 +79,14 @@ torch::TensorOptions Graph::IdOptions() const {
 }
 
 torch::Tensor Graph::DataOrOnes() {
+  Settle();
   if (data_.has_value()) return data_.value();
   return torch::ones({num_edges_}, IdOptions().dtype(torch::kFloat32));
 }
 
 // edge data in the order of a format ("col": CSC order, "row": CSR order)
 torch::optional<torch::Tensor> Graph::GetData(std::string order) {
+  Settle();
   torch::Tensor data = DataOrOnes();
   if (order == "col") {
     CreateSparseFormat(_CSC);
@@ -98,16 +100,19 @@ torch::optional<torch::Tensor> Graph::GetData(std::string order) {
 
 // ------------------------------------------------------------ format caches
 void Graph::CSC2CSR() {
+  Settle();
   SetCOO(GraphCSC2COO(csc_, true));
   SetCSR(GraphCOO2CSC(coo_, num_rows_, false));
 }
 
 void Graph::CSR2CSC() {
+  Settle();
   SetCOO(GraphCSC2COO(csr_, false));
   SetCSC(GraphCOO2CSC(coo_, num_cols_, true));
 }
 
 void Graph::CreateSparseFormat(int64_t format) {
+  Settle();
   RejectCompressed(format);
   if (format == _COO) {
     if (coo_) return;
@@ -133,11 +138,13 @@ void Graph::CreateSparseFormat(int64_t format) {
 }
 
 std::vector<torch::Tensor> Graph::GetCSCTensor() {
+  Settle();
   CreateSparseFormat(_CSC);
   return {csc_->indptr, csc_->indices, csc_->e_ids.value_or(torch::Tensor())};
 }
 
 std::vector<torch::Tensor> Graph::GetCOOTensor() {
+  Settle();
   CreateSparseFormat(_COO);
   TORCH_CHECK(coo_->col_sorted, "GetCOOTensor expects a column-sorted COO");
   return {coo_->row, coo_->col, coo_->e_ids.value_or(torch::Tensor())};
@@ -160,6 +167,7 @@ void Graph::InheritData(Graph* child, const torch::optional<torch::Tensor>& e_id
 
 // a graph with the same structure (shared format caches) and new edge data
 c10::intrusive_ptr<Graph> Graph::SameShape(torch::Tensor data) {
+  Settle();
   auto g = c10::make_intrusive<Graph>(is_subgraph_, col_ids_, row_ids_, num_cols_, num_rows_);
   g->SetCSC(csc_);
   g->SetCSR(csr_);
@@ -172,6 +180,7 @@ c10::intrusive_ptr<Graph> Graph::SameShape(torch::Tensor data) {
 // ------------------------------------------------------------------ slicing
 c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int64_t on_format,
                                          int64_t output_format, bool relabel) {
+  Settle();
   TORCH_CHECK(axis == 0 || axis == 1, "axis must be 0 (columns) or 1 (rows)");
   RejectCompressed(on_format);
   CreateSparseFormat(on_format);
@@ -258,6 +267,7 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
 c10::intrusive_ptr<Graph> Graph::SampleImpl(int64_t axis, const torch::Tensor* edge_probs,
                                             int64_t fanout, bool replace, int64_t on_format,
                                             int64_t output_format) {
+  Settle();
   RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   const bool on_csc = (axis == 0 && on_format == _CSC);
@@ -304,11 +314,32 @@ c10::intrusive_ptr<Graph> Graph::SamplingProbs(int64_t axis, torch::Tensor edge_
 
 // slice + sample without materialising the slice; the result holds a CSC only
 // and the kernel is given the LOCAL column index (reference src/graph.cc:531-559)
+void Graph::Settle() {
+  if (!pending_) return;
+  std::shared_ptr<hip::PendingSample> p = std::move(pending_);
+  pending_.reset();
+  const int64_t nnz = p->Wait();
+  auto csc = std::make_shared<CSC>();
+  csc->indptr = p->sub_indptr;
+  csc->indices = p->indices.narrow(0, 0, nnz);
+  csc_ = csc;
+  num_edges_ = nnz;
+}
+
 c10::intrusive_ptr<Graph> Graph::ColumnwiseFusedSlicingAndSampling(torch::Tensor column_index,
                                                                    int64_t fanout, bool replace) {
+  Settle();
   TORCH_CHECK(csc_ != nullptr, "fused slicing + sampling needs the CSC format");
   torch::Tensor col_ids = Pick(col_ids_, column_index);
   auto ret = Child(col_ids, row_ids_, col_ids.numel(), num_rows_);
+  // No edge data to carry over: nothing on the host needs the edge count yet, so the
+  // child is handed back while the sampler runs and settles when it is first used.
+  if (hip::DeferredSampling() && !data_.has_value() && !(fanout == 1 && replace) &&
+      hip::OneLaunchApplies(column_index.numel(), fanout, replace)) {
+    ret->pending_ = hip::ColSamplingDeferred(csc_->indptr, csc_->indices, column_index, fanout,
+                                             replace, false, false);
+    return ret;
+  }
   std::shared_ptr<CSC> sampled;
   torch::Tensor select_index;
   std::tie(sampled, select_index) = FusedCSCColSlicingAndSampling(csc_, column_index, fanout, replace);
@@ -319,12 +350,14 @@ c10::intrusive_ptr<Graph> Graph::ColumnwiseFusedSlicingAndSampling(torch::Tensor
 }
 
 torch::Tensor Graph::RandomWalk(torch::Tensor seeds, int64_t walk_length) {
+  Settle();
   TORCH_CHECK(csc_ != nullptr, "random walks need the CSC format");
   return FusedRandomWalk(csc_, seeds, walk_length);
 }
 
 // --------------------------------------------------------- edge-data operators
 torch::Tensor Graph::Sum(int64_t axis, int64_t powk, int64_t on_format) {
+  Settle();
   RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
@@ -343,6 +376,7 @@ torch::Tensor Graph::Sum(int64_t axis, int64_t powk, int64_t on_format) {
 }
 
 c10::intrusive_ptr<Graph> Graph::Normalize(int64_t axis, int64_t on_format) {
+  Settle();
   RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
@@ -357,6 +391,7 @@ c10::intrusive_ptr<Graph> Graph::Normalize(int64_t axis, int64_t on_format) {
 }
 
 c10::intrusive_ptr<Graph> Graph::Divide(torch::Tensor divisor, int64_t axis, int64_t on_format) {
+  Settle();
   RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
@@ -371,6 +406,7 @@ c10::intrusive_ptr<Graph> Graph::Divide(torch::Tensor divisor, int64_t axis, int
 }
 
 std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> Graph::EDivUSum(torch::Tensor divisor) {
+  Settle();
   CreateSparseFormat(_COO);
   torch::Tensor data = DataOrOnes();
   torch::Tensor out = torch::zeros({num_edges_}, data.options());
@@ -383,6 +419,7 @@ std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> Graph::EDivUSum(torch::Tens
 // CSR the compressed axis is the row, so 0 and 2 swap (reference src/graph.cc:975-976)
 void Graph::SDDMM(const std::string& op, torch::Tensor lhs, torch::Tensor rhs, torch::Tensor out,
                   int64_t lhs_target, int64_t rhs_target, int64_t on_format) {
+  Settle();
   RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   const hip::Bcast b = ToDevice(CalcBcastOff(op, lhs, rhs), out);
@@ -403,6 +440,7 @@ void Graph::SDDMM(const std::string& op, torch::Tensor lhs, torch::Tensor rhs, t
 
 // ---------------------------------------------------------------- node queries
 torch::Tensor Graph::AllValidNode() {
+  Settle();
   TORCH_CHECK(col_ids_.has_value(), "For sampling, col_ids_ is necessary!");
   torch::Tensor rows;
   if (row_ids_.has_value()) {
@@ -423,6 +461,22 @@ Graph::Relabel() {
   torch::Tensor col_ids = col_ids_.value();
   torch::Tensor frontier;
   std::vector<torch::Tensor> renamed;
+  if (pending_ && !row_ids_.has_value()) {
+    // straight behind the sampler: its edge count stays on the device until the end
+    std::shared_ptr<hip::PendingSample> p = std::move(pending_);
+    pending_.reset();
+    torch::Tensor indptr_copy = p->sub_indptr.clone();
+    torch::Tensor relabeled;
+    int64_t nnz;
+    std::tie(frontier, relabeled, nnz) = hip::RelabelDeferred(col_ids, *p);
+    auto csc = std::make_shared<CSC>();
+    csc->indptr = p->sub_indptr;
+    csc->indices = p->indices.narrow(0, 0, nnz);
+    csc_ = csc;
+    num_edges_ = nnz;
+    return {frontier, frontier.numel(), col_ids.numel(), indptr_copy, relabeled, csc_->e_ids, "csc"};
+  }
+  Settle();
   if (csc_) {
     // seeds first: the frontier starts with the column ids (reference src/graph.cc:789-811)
     torch::Tensor rows = Pick(row_ids_, csc_->indices);
@@ -447,14 +501,17 @@ torch::Tensor Graph::GetCols() {
 }
 
 torch::Tensor Graph::GetValidRows() {
+  Settle();
   return Pick(row_ids_, std::get<0>(torch::_unique(GetCOORows(false))));
 }
 
 torch::Tensor Graph::GetValidCols() {
+  Settle();
   return Pick(col_ids_, std::get<0>(torch::_unique(GetCOOCols(false))));
 }
 
 torch::Tensor Graph::GetCOORows(bool is_original) {
+  Settle();
   torch::Tensor rows;
   if (coo_) {
     rows = coo_->row;
@@ -469,6 +526,7 @@ torch::Tensor Graph::GetCOORows(bool is_original) {
 }
 
 torch::Tensor Graph::GetCOOCols(bool is_original) {
+  Settle();
   torch::Tensor cols;
   if (coo_) {
     cols = coo_->col;
@@ -483,6 +541,7 @@ torch::Tensor Graph::GetCOOCols(bool is_original) {
 }
 
 std::vector<torch::Tensor> Graph::MetaData() {
+  Settle();
   torch::Tensor col_ids = col_ids_.value_or(torch::Tensor());
   torch::Tensor row_ids = row_ids_.value_or(torch::Tensor());
   if (csc_) return {col_ids, row_ids, DataOrOnes(), csc_->indptr, csc_->indices};
@@ -492,12 +551,14 @@ std::vector<torch::Tensor> Graph::MetaData() {
 }
 
 std::vector<torch::Tensor> Graph::COOMetaData() {
+  Settle();
   if (!coo_) return {};
   return {col_ids_.value_or(torch::Tensor()), row_ids_.value_or(torch::Tensor()),
           data_.value_or(torch::Tensor()), coo_->row, coo_->col};
 }
 
 std::vector<torch::Tensor> Graph::CSCMetaData() {
+  Settle();
   if (!csc_) return {};
   return {col_ids_.value_or(torch::Tensor()), row_ids_.value_or(torch::Tensor()),
           data_.value_or(torch::Tensor()), csc_->indptr, csc_->indices};

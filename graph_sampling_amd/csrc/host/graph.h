@@ -25,6 +25,10 @@
 
 namespace gs {
 
+namespace hip {
+struct PendingSample;
+}
+
 class Graph : public torch::CustomClassHolder {
  public:
   explicit Graph(bool is_subgraph) : is_subgraph_(is_subgraph) {}
@@ -43,22 +47,46 @@ class Graph : public torch::CustomClassHolder {
   void LoadCSCWithColIds(torch::Tensor column_ids, torch::Tensor indptr, torch::Tensor indices);
   void SetMetaData(torch::optional<torch::Tensor> col_ids, torch::optional<torch::Tensor> row_ids,
                    int64_t num_cols, int64_t num_rows);
-  void SetCSC(std::shared_ptr<CSC> csc) { csc_ = csc; }
-  void SetCSR(std::shared_ptr<CSR> csr) { csr_ = csr; }
-  void SetCOO(std::shared_ptr<COO> coo) { coo_ = coo; }
+  void SetCSC(std::shared_ptr<CSC> csc) {
+    Settle();
+    csc_ = csc;
+  }
+  void SetCSR(std::shared_ptr<CSR> csr) {
+    Settle();
+    csr_ = csr;
+  }
+  void SetCOO(std::shared_ptr<COO> coo) {
+    Settle();
+    coo_ = coo;
+  }
   void SetCOOByTensor(torch::Tensor row, torch::Tensor col, torch::optional<torch::Tensor> e_ids,
                       bool row_sorted, bool col_sorted);
   void SetData(torch::Tensor data) { data_ = data; }
-  void SetNumEdges(int64_t num_edges) { num_edges_ = num_edges; }
-  std::shared_ptr<CSC> GetCSC() { return csc_; }
-  std::shared_ptr<CSR> GetCSR() { return csr_; }
-  std::shared_ptr<COO> GetCOO() { return coo_; }
+  void SetNumEdges(int64_t num_edges) {
+    Settle();
+    num_edges_ = num_edges;
+  }
+  std::shared_ptr<CSC> GetCSC() {
+    Settle();
+    return csc_;
+  }
+  std::shared_ptr<CSR> GetCSR() {
+    Settle();
+    return csr_;
+  }
+  std::shared_ptr<COO> GetCOO() {
+    Settle();
+    return coo_;
+  }
   std::vector<torch::Tensor> GetCSCTensor();
   std::vector<torch::Tensor> GetCOOTensor();
   torch::optional<torch::Tensor> GetData(std::string order = "default");
   int64_t GetNumRows() { return num_rows_; }
   int64_t GetNumCols() { return num_cols_; }
-  int64_t GetNumEdges() { return num_edges_; }
+  int64_t GetNumEdges() {
+    Settle();
+    return num_edges_;
+  }
 
   // ---- format caches
   void CSC2CSR();
@@ -112,6 +140,14 @@ class Graph : public torch::CustomClassHolder {
   c10::intrusive_ptr<Graph> SampleImpl(int64_t axis, const torch::Tensor* edge_probs,
                                        int64_t fanout, bool replace, int64_t on_format,
                                        int64_t output_format);
+
+  // A graph made by the fused sampler may still be waiting for its edge count: the
+  // sampled ids sit in a buffer of the capacity columns x fanout and the count is
+  // on its way to a host mailbox.  Settle() collects it and installs the CSC; every
+  // public method does that first, except Relabel(), which queues its kernels
+  // behind the sampler with the count still on the device.
+  void Settle();
+  std::shared_ptr<hip::PendingSample> pending_;
 
   bool is_subgraph_ = false;
   int64_t num_cols_ = 0;

@@ -15,6 +15,7 @@ namespace {
 std::atomic<uint64_t> g_seed{7777};
 std::atomic<int64_t> g_algo{GS_SAMPLE_AUTO};
 constexpr int64_t kOneLaunchMaxColumns = 1 << 18;
+std::atomic<bool> g_deferred{true};
 
 void Check(int status, const char* what) {
   TORCH_CHECK(status == GS_OK, what, " failed (", status, "): ", gs_status_string(status));
@@ -60,41 +61,54 @@ torch::Tensor Scratch(size_t bytes, const torch::Tensor& like) {
                       torch::dtype(torch::kUInt8).device(like.device()));
 }
 
-// ---- result mailbox: totals arrive in pinned host memory, no stream sync ----
-struct HostBox {
-  torch::Tensor buf;  // 2 x int64, pinned
-  gs_mailbox* box = nullptr;
+// ---- result mailboxes: totals arrive in pinned host memory, no stream sync ----
+// A ring of kBoxes {total, ticket} pairs per (thread, device); call number t posts
+// to slot t % kBoxes, so a total stays readable until kBoxes later calls have
+// been issued.
+constexpr int64_t kBoxes = 64;
+constexpr int64_t kLost = -2;  // the slot was reused before anyone read it
+
+struct HostBoxes {
+  torch::Tensor buf;  // kBoxes x {total, ticket}, pinned
+  gs_mailbox* ring = nullptr;
   int64_t next = 1;
+  gs_mailbox* slot(int64_t ticket) const { return ring + ticket % kBoxes; }
 };
 
-HostBox& Box(int device) {
-  thread_local std::map<int, HostBox> boxes;
-  HostBox& b = boxes[device];
-  if (!b.box) {
-    b.buf = torch::zeros({2}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
-    b.box = reinterpret_cast<gs_mailbox*>(b.buf.data_ptr<int64_t>());
+HostBoxes& Boxes(int device) {
+  thread_local std::map<int, HostBoxes> boxes;
+  HostBoxes& b = boxes[device];
+  if (!b.ring) {
+    b.buf = torch::zeros({kBoxes * 2}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+    b.ring = reinterpret_cast<gs_mailbox*>(b.buf.data_ptr<int64_t>());
   }
   return b;
 }
 
 // Spins until the kernel has posted `ticket`; every few thousand polls it asks
 // the stream whether it has drained or failed, so a kernel that never posts
-// turns into an error, not a hang.
-int64_t WaitBox(HostBox& b, int64_t ticket, void* stream, const char* what) {
+// turns into an error (or kLost when a later call took the slot), not a hang.
+int64_t WaitBox(const gs_mailbox* box, int64_t ticket, void* stream, const char* what) {
   hipStream_t st = static_cast<hipStream_t>(stream);
   for (uint64_t n = 1;; ++n) {
-    if (__atomic_load_n(&b.box->ticket, __ATOMIC_ACQUIRE) == ticket) break;
+    const int64_t seen = __atomic_load_n(&box->ticket, __ATOMIC_ACQUIRE);
+    if (seen == ticket) break;
+    if (seen > ticket) return kLost;
     if ((n & 0xFFF) == 0) {
       const hipError_t q = hipStreamQuery(st);
       if (q == hipSuccess) {
-        if (__atomic_load_n(&b.box->ticket, __ATOMIC_ACQUIRE) == ticket) break;
+        const int64_t again = __atomic_load_n(&box->ticket, __ATOMIC_ACQUIRE);
+        if (again == ticket) break;
+        if (again > ticket) return kLost;
         TORCH_CHECK(false, what, ": the stream drained without reporting a total");
       }
       TORCH_CHECK(q == hipErrorNotReady, what, ": ", hipGetErrorString(q));
     }
     __builtin_ia32_pause();
   }
-  const int64_t total = __atomic_load_n(&b.box->total, __ATOMIC_RELAXED);
+  const int64_t total = __atomic_load_n(&box->total, __ATOMIC_RELAXED);
+  // the slot may have been rewritten between the two loads
+  if (__atomic_load_n(&box->ticket, __ATOMIC_ACQUIRE) != ticket) return kLost;
   TORCH_CHECK(total >= 0, what, ": a tile gave up waiting for its predecessors");
   return total;
 }
@@ -206,50 +220,81 @@ SliceResult SampleInto(const torch::Tensor& indptr, const torch::Tensor& indices
 
 }  // namespace
 
-// One launch, no mid-call host read; the total arrives through the mailbox.
-SliceResult ColSamplingOneLaunch(const torch::Tensor& indptr, const torch::Tensor& indices,
-                                 const torch::Tensor& column_ids, int64_t fanout, bool replace,
-                                 bool with_coo) {
+int64_t PendingSample::Wait() const {
+  int64_t nnz = WaitBox(Boxes(device).slot(ticket), ticket, stream, "gs_sample_uniform_fused");
+  if (nnz == kLost) {
+    nnz = sub_indptr[S].item<int64_t>();
+    TORCH_CHECK(nnz >= 0, "gs_sample_uniform_fused: a tile gave up waiting for its predecessors");
+  }
+  return nnz;
+}
+
+void SetDeferredSampling(bool on) { g_deferred.store(on); }
+bool DeferredSampling() { return g_deferred.load(); }
+
+bool OneLaunchApplies(int64_t S, int64_t fanout, bool replace) {
+  // One launch wins while launch and round-trip latency dominate (measured: 3-4x at 45k
+  // columns); past a few hundred thousand columns the chained scan's per-tile walk costs
+  // more than the two extra launches of the count / fill pair save.
+  return g_algo.load() == GS_SAMPLE_AUTO && S <= kOneLaunchMaxColumns &&
+         (replace || fanout <= GS_FUSED_MAX_FANOUT);
+}
+
+// One launch, no host read: the total is posted to a mailbox and collected by Wait().
+std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
+                                                   const torch::Tensor& indices,
+                                                   const torch::Tensor& column_ids, int64_t fanout,
+                                                   bool replace, bool with_coo, bool with_select) {
   NeedI64(indptr, "indptr");
   const int idb = IdBytes(indices, "indices");
   const bool fused = column_ids.defined();
   if (fused)
     TORCH_CHECK(IdBytes(column_ids, "column ids") == idb, "column ids and indices differ in dtype");
-  const int64_t S = fused ? column_ids.numel() : indptr.numel() - 1;
-  auto sub_indptr = torch::empty({S + 1}, I64(indptr));
-  const int64_t cap = S * fanout;
-  auto sub_indices = torch::empty({cap}, indices.options());
-  auto select_index = torch::empty({cap}, I64(indptr));
-  torch::Tensor coo_col;
-  if (with_coo) coo_col = torch::empty({cap}, indices.options());
-  void* st = Stream(indptr);
-  FusedStateBuf& state = FusedState(gs_sample_fused_state_bytes(S), indptr, st);
-  HostBox& box = Box(indptr.device().index());
-  const int64_t ticket = box.next++;
+  TORCH_CHECK(fanout >= 0, "fanout must be non-negative");
+  auto p = std::make_shared<PendingSample>();
+  p->S = fused ? column_ids.numel() : indptr.numel() - 1;
+  p->sub_indptr = torch::empty({p->S + 1}, I64(indptr));
+  const int64_t cap = p->S * fanout;
+  p->indices = torch::empty({cap}, indices.options());
+  if (with_select) p->select_index = torch::empty({cap}, I64(indptr));
+  if (with_coo) p->coo_col = torch::empty({cap}, indices.options());
+  p->stream = Stream(indptr);
+  p->device = indptr.device().index();
+  FusedStateBuf& state = FusedState(gs_sample_fused_state_bytes(p->S), indptr, p->stream);
+  HostBoxes& boxes = Boxes(p->device);
+  p->ticket = boxes.next++;
   Check(gs_sample_uniform_fused(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(),
-                                fused ? column_ids.data_ptr() : nullptr, idb, S, fanout,
+                                fused ? column_ids.data_ptr() : nullptr, idb, p->S, fanout,
                                 replace ? 1 : 0, NextSeed(), nullptr, nullptr,
-                                sub_indptr.data_ptr<int64_t>(), sub_indices.data_ptr(),
-                                select_index.data_ptr<int64_t>(),
-                                with_coo ? coo_col.data_ptr() : nullptr, cap,
-                                state.buf.data_ptr(), state.buf.numel(), state.epoch, box.box,
-                                ticket, st),
+                                p->sub_indptr.data_ptr<int64_t>(), p->indices.data_ptr(),
+                                with_select ? p->select_index.data_ptr<int64_t>() : nullptr,
+                                with_coo ? p->coo_col.data_ptr() : nullptr, cap,
+                                state.buf.data_ptr(), state.buf.numel(), state.epoch,
+                                boxes.slot(p->ticket), p->ticket, p->stream),
         "gs_sample_uniform_fused");
-  const int64_t nnz = WaitBox(box, ticket, st, "gs_sample_uniform_fused");
-  if (with_coo) coo_col = coo_col.narrow(0, 0, nnz);
-  return {sub_indptr, coo_col, sub_indices.narrow(0, 0, nnz), select_index.narrow(0, 0, nnz)};
+  return p;
 }
+
+namespace {
+
+SliceResult ColSamplingOneLaunch(const torch::Tensor& indptr, const torch::Tensor& indices,
+                                 const torch::Tensor& column_ids, int64_t fanout, bool replace,
+                                 bool with_coo) {
+  auto p = ColSamplingDeferred(indptr, indices, column_ids, fanout, replace, with_coo, true);
+  const int64_t nnz = p->Wait();
+  torch::Tensor coo_col;
+  if (with_coo) coo_col = p->coo_col.narrow(0, 0, nnz);
+  return {p->sub_indptr, coo_col, p->indices.narrow(0, 0, nnz), p->select_index.narrow(0, 0, nnz)};
+}
+
+}  // namespace
 
 SliceResult ColSampling(const torch::Tensor& indptr, const torch::Tensor& indices,
                         const torch::Tensor& column_ids, int64_t fanout, bool replace,
                         bool with_coo) {
   TORCH_CHECK(fanout >= 0, "fanout must be non-negative");
-  // One launch wins while launch and round-trip latency dominate (measured: 3-4x at 45k
-  // columns); past a few hundred thousand columns the chained scan's per-tile walk costs
-  // more than the two extra launches of the count / fill pair save.
   const int64_t S = column_ids.defined() ? column_ids.numel() : indptr.numel() - 1;
-  if (g_algo.load() == GS_SAMPLE_AUTO && S <= kOneLaunchMaxColumns &&
-      (replace || fanout <= GS_FUSED_MAX_FANOUT))
+  if (OneLaunchApplies(S, fanout, replace))
     return ColSamplingOneLaunch(indptr, indices, column_ids, fanout, replace, with_coo);
   return SampleInto(
       indptr, indices, column_ids, fanout, replace, with_coo, 0,
@@ -331,15 +376,47 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> Relabel(
   auto num = torch::empty({1}, I64(mapping[0]));
   auto ws = Scratch(gs_unique_workspace_bytes(M), mapping[0]);
   void* st = Stream(mapping[0]);
-  HostBox& box = Box(mapping[0].device().index());
-  const int64_t ticket = box.next++;
+  HostBoxes& boxes = Boxes(mapping[0].device().index());
+  const int64_t ticket = boxes.next++;
   Check(gs_unique_relabel_notify(m, static_cast<int>(mapping.size()), q, out_ptr,
                                  static_cast<int>(queries.size()), idb, frontier.data_ptr(),
-                                 num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), box.box, ticket,
-                                 st),
+                                 num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), nullptr,
+                                 boxes.slot(ticket), ticket, st),
         "gs_unique_relabel");
-  const int64_t U = WaitBox(box, ticket, st, "gs_unique_relabel");
+  int64_t U = WaitBox(boxes.slot(ticket), ticket, st, "gs_unique_relabel");
+  if (U == kLost) U = num.item<int64_t>();
+  TORCH_CHECK(U >= 0, "gs_unique_relabel: a tile gave up waiting for its predecessors");
   return {frontier.narrow(0, 0, U), outs};
+}
+
+// Relabel of (column ids, sampled ids) while the sampler's total is still on the
+// device: everything is sized for the sampler's capacity, the kernels read the
+// true length from sub_indptr[S], and both totals are collected at the end.
+std::tuple<torch::Tensor, torch::Tensor, int64_t> RelabelDeferred(const torch::Tensor& col_ids,
+                                                                  const PendingSample& p) {
+  const int idb = IdBytes(col_ids, "column ids");
+  TORCH_CHECK(IdBytes(p.indices, "sampled ids") == idb, "relabel tensors differ in dtype");
+  const int64_t cap = p.indices.numel();
+  const int64_t M = col_ids.numel() + cap;
+  gs_span m[2] = {{col_ids.data_ptr(), col_ids.numel()}, {p.indices.data_ptr(), cap}};
+  gs_span q[1] = {{p.indices.data_ptr(), cap}};
+  auto renamed = torch::empty_like(p.indices);
+  void* out_ptr[1] = {renamed.data_ptr()};
+  auto frontier = torch::empty({M}, col_ids.options());
+  auto num = torch::empty({1}, I64(col_ids));
+  auto ws = Scratch(gs_unique_workspace_bytes(M), col_ids);
+  HostBoxes& boxes = Boxes(p.device);
+  const int64_t ticket = boxes.next++;
+  Check(gs_unique_relabel_notify(m, 2, q, out_ptr, 1, idb, frontier.data_ptr(),
+                                 num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(),
+                                 p.sub_indptr.data_ptr<int64_t>() + p.S, boxes.slot(ticket), ticket,
+                                 p.stream),
+        "gs_unique_relabel");
+  const int64_t nnz = p.Wait();
+  int64_t U = WaitBox(boxes.slot(ticket), ticket, p.stream, "gs_unique_relabel");
+  if (U == kLost) U = num.item<int64_t>();
+  TORCH_CHECK(U >= 0, "gs_unique_relabel: a tile gave up waiting for its predecessors");
+  return {frontier.narrow(0, 0, U), renamed.narrow(0, 0, nnz), nnz};
 }
 
 torch::Tensor Unique(const torch::Tensor& ids) { return std::get<0>(Relabel({ids}, {})); }

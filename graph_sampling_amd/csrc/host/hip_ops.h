@@ -8,6 +8,7 @@
 
 #include <torch/torch.h>
 
+#include <memory>
 #include <string>
 #include <tuple>
 #include <vector>
@@ -32,6 +33,35 @@ SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices
 SliceResult ColSampling(const torch::Tensor& indptr, const torch::Tensor& indices,
                         const torch::Tensor& column_ids, int64_t fanout, bool replace,
                         bool with_coo);
+// A one-launch sample whose total the host has not read yet.  The buffers have
+// the capacity S * fanout; Wait() collects the total from its mailbox (no stream
+// synchronisation), after which the caller narrows them.
+struct PendingSample {
+  torch::Tensor sub_indptr;    // [S + 1], final
+  torch::Tensor indices;       // capacity
+  torch::Tensor select_index;  // capacity; undefined when not requested
+  torch::Tensor coo_col;       // capacity; undefined when not requested
+  int64_t S = 0;
+  int64_t ticket = 0;
+  void* stream = nullptr;
+  int device = 0;
+  int64_t Wait() const;
+};
+// Whether the fused sampler may hand back a graph before its edge count has reached the
+// host (default on).  Off: every call settles before it returns, as the reference does.
+void SetDeferredSampling(bool on);
+bool DeferredSampling();
+// whether ColSampling would take the one-launch path for this call
+bool OneLaunchApplies(int64_t S, int64_t fanout, bool replace);
+std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
+                                                   const torch::Tensor& indices,
+                                                   const torch::Tensor& column_ids, int64_t fanout,
+                                                   bool replace, bool with_coo, bool with_select);
+// {frontier, relabelled sampled ids, number of sampled ids}: unique / relabel of
+// (column ids, sampled ids) queued behind the sampler without reading its total
+std::tuple<torch::Tensor, torch::Tensor, int64_t> RelabelDeferred(const torch::Tensor& col_ids,
+                                                                  const PendingSample& p);
+
 SliceResult ColSamplingProbs(const torch::Tensor& indptr, const torch::Tensor& indices,
                              const torch::Tensor& probs, const torch::Tensor& column_ids,
                              int64_t fanout, bool replace, bool with_coo);

@@ -156,7 +156,8 @@ int gs_sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const void* 
  * without their mid-call host read.
  *   - without replacement fanout must be <= GS_FUSED_MAX_FANOUT (else
  *     GS_ERR_UNSUPPORTED: use the two-phase calls);
- *   - sub_indices / select_index / coo_col hold `capacity` >= S*fanout entries;
+ *   - sub_indices / select_index / coo_col hold `capacity` >= S*fanout entries
+ *     (select_index and coo_col may be NULL when the caller has no use for them);
  *     the true total is written to sub_indptr[S] (-1 if the kernel gave up
  *     waiting on another tile, which a healthy device never does) and to the
  *     mailbox when one is given;
@@ -246,13 +247,22 @@ int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* quer
                       int64_t* num_unique, void* workspace, size_t workspace_bytes,
                       void* stream);
 
-/* The same, and the kernel that learns the number of unique ids also posts it to
- * `mailbox` (see gs_mailbox; NULL = plain gs_unique_relabel).  *num_unique and the
- * mailbox read -1 if the compaction gave up waiting on another tile. */
+/* The same, for callers that keep the host out of the loop:
+ *   - mailbox (NULL = none): the kernel that learns the number of unique ids also
+ *     posts it there (see gs_mailbox).  *num_unique and the mailbox read -1 if the
+ *     compaction gave up waiting on another tile.
+ *   - last_span_len (NULL = none): device address of the true length of the LAST
+ *     mapping span, for a span whose length an earlier kernel on the stream
+ *     produced and the host has not read (the sampled ids of
+ *     gs_sample_uniform_fused, length sub_indptr[S]).  mapping[n_mapping-1].n is
+ *     then only its capacity; launches, table and frontier are sized for it and the
+ *     kernels read the length themselves (a negative value counts as 0).  The only
+ *     query allowed in this mode is that same span, cut to the same length. */
 int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_span* query,
                              void* const* query_out, int n_query, int id_bytes, void* frontier,
                              int64_t* num_unique, void* workspace, size_t workspace_bytes,
-                             gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
+                             const int64_t* last_span_len, gs_mailbox* mailbox,
+                             int64_t mailbox_ticket, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Random walks: replace impl::fusion::FusedRandomWalkCUDA                    */

@@ -157,3 +157,25 @@ def test_mailbox_reports_totals(dev):
         assert np.array_equal(frontier[:U].cpu().numpy().astype(np.int64), f_want)
         assert np.array_equal(outs[0].cpu().numpy().astype(np.int64), r_want[0])
         assert int(num.item()) == U
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+def test_relabel_with_device_side_length(dev, idt):
+    """Sampler -> relabel with no host read in between: the relabel kernels take the length of the
+    sampled ids from sub_indptr[S] on the device and treat the padded tail as absent."""
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=5)
+    d_ip, d_ix = to_dev(indptr, dev), to_dev(indices, dev, idt)
+    box = capi.Mailbox()
+    for it, S in enumerate([0, 1, 300, 5000, 20000, 7]):
+        cols = np.random.default_rng(it).integers(0, 1 << 12, size=S).astype(np.int64)
+        d_cols = to_dev(cols, dev, idt)
+        sub_indptr, sub, sel, _ = capi.sample_uniform_fused(d_ip, d_ix, d_cols, 10, False, seed=it)
+        frontier, num, outs, ticket = capi.unique_relabel([d_cols, sub], [sub], mailbox=box,
+                                                          last_span_len=sub_indptr[S:])
+        U = box.wait(ticket, dev)
+        nnz = int(sub_indptr[S].item())
+        want = O.sample_uniform(indptr, indices, cols, 10, False, seed=it)
+        f_want, r_want = O.relabel([cols, want[2]], [want[2]])
+        assert nnz == int(want[0][-1]) and U == f_want.size
+        assert np.array_equal(frontier[:U].cpu().numpy().astype(np.int64), f_want)
+        assert np.array_equal(outs[0][:nnz].cpu().numpy().astype(np.int64), r_want[0])
