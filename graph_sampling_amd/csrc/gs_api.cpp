@@ -20,6 +20,8 @@ char g_profile_name[64] = "";
 std::mutex g_profile_mu;
 std::vector<hipEvent_t> g_start, g_stop;
 int g_used = 0;
+int g_stride = 1;     // time every g_stride-th launch of the site
+int g_seen = 0;       // launches of the site since enable
 constexpr int kMaxPairs = 4096;
 }  // namespace
 
@@ -35,6 +37,7 @@ void profile_begin(const char* name, hipStream_t stream, int* slot) {
   if (!g_profile_on.load(std::memory_order_relaxed)) return;
   std::lock_guard<std::mutex> lock(g_profile_mu);
   if (std::strcmp(name, g_profile_name) != 0 || g_used >= kMaxPairs) return;
+  if (g_seen++ % g_stride != 0) return;
   if (g_used == static_cast<int>(g_start.size())) {
     hipEvent_t a, b;
     if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) return;
@@ -69,9 +72,16 @@ const char* gs_status_string(int status) {
 
 int gs_version(void) { return 100; }
 
+int gs_profile_stride(int every) {
+  std::lock_guard<std::mutex> lock(gs::g_profile_mu);
+  gs::g_stride = every < 1 ? 1 : every;
+  return GS_OK;
+}
+
 int gs_profile_enable(const char* launch_site) {
   std::lock_guard<std::mutex> lock(gs::g_profile_mu);
   gs::g_used = 0;
+  gs::g_seen = 0;
   if (!launch_site || !launch_site[0]) {
     gs::g_profile_on.store(false);
     gs::g_profile_name[0] = 0;

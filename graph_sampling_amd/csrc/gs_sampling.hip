@@ -537,7 +537,7 @@ int sample_fill_impl(const SampleArgs<IdT>& a, int replace, int algo, hipStream_
 // read-modify-write on a shared address (see the look-back notes).
 constexpr int kFusedThreads = 256;
 constexpr int kFusedRows = 256;
-constexpr int kFusedBatch = 4;  // gathers a lane keeps in flight in the fill
+constexpr int kFusedBatch = 8;  // gathers a lane keeps in flight in the fill
 constexpr int kPickStride = kFusedRows + 1;  // odd stride: conflict-free by row and by step
 
 template <typename IdT>

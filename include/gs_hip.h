@@ -79,6 +79,10 @@ typedef struct gs_mailbox {
  * given, the first `cap` individual durations in launch order) and clears the
  * ring.  The events are created by the library and live until the process ends. */
 int gs_profile_enable(const char* launch_site);
+/* Time only every `every`-th launch of the enabled site (default 1 = all): an event
+ * pair costs a few microseconds of queue time, which matters when the timed kernels
+ * are themselves that short. */
+int gs_profile_stride(int every);
 int gs_profile_collect(double* total_ms, int64_t* launches, double* per_launch_ms, int64_t cap);
 
 typedef enum gs_op {
