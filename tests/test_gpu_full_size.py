@@ -1,0 +1,245 @@
+"""GPU parity at the benchmark configurations' full sizes.
+
+Where the CPU oracle finishes in seconds the comparison is exact (the whole GraphSAGE minibatch,
+the whole walk trace, the layer-wise sampler's layer); where it does not, the checks are the
+size-independent properties of the operation (every sampled edge exists, positions are distinct
+within a row, relabelling inverts through the frontier, absorbing -1) and, for SDDMM, a torch fp32
+gather-and-dot of the same tensors.  Graphs come from the seeded on-device R-MAT generator."""
+import numpy as np
+import pytest
+import torch
+
+import graph_sampling_amd as gs
+from graph_sampling_amd import _COO, _CSC, _CSR, capi, rmat
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+FANOUTS = (15, 10, 5)
+
+
+def _host(t):
+    return t.cpu().numpy().astype(np.int64)
+
+
+@pytest.fixture(scope="module")
+def sage_graph(dev):
+    """R-MAT 2.45 M nodes / 124 M edges, int64 offsets, int32 ids (the GraphSAGE configuration)."""
+    indptr, indices = rmat.rmat_csc(2_450_000, 124_000_000, seed=0, device=dev, index_dtype=torch.int32)
+    return indptr, indices, _host(indptr), _host(indices)
+
+
+def test_graphsage_minibatch_full_size_matches_oracle(dev, sage_graph):
+    """Two [15,10,5] minibatches of 1024 seeds through the Graph API: every layer's offsets,
+    relabelled ids and frontier equal the oracle's on the same seeds and draws."""
+    indptr, indices, h_indptr, h_indices = sage_graph
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(indptr, indices)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2)
+    torch.ops.gs_ops._CAPI_SetSeed(500)
+    call = 500
+    for _ in range(2):
+        seeds = torch.randperm(2_450_000, generator=gen, device=dev)[:1024].to(torch.int32)
+        h_seeds = _host(seeds)
+        for k in FANOUTS:
+            sub = g._CAPI_FusedColumnwiseSlicingSampling(seeds, k, False)
+            frontier, n_src, n_dst, ptr, idx, e_ids, fmt = sub._CAPI_Relabel()
+            sp, _, rows, _ = O.sample_uniform(h_indptr, h_indices, h_seeds, k, False, seed=call,
+                                              with_coo=False)
+            call += 1
+            want_frontier, (want_idx,) = O.relabel([h_seeds, rows], [rows])
+            assert fmt == "csc" and n_dst == h_seeds.size and n_src == want_frontier.size
+            assert np.array_equal(_host(ptr), sp)
+            assert np.array_equal(_host(idx), want_idx)
+            assert np.array_equal(_host(frontier), want_frontier)
+            assert sub._CAPI_GetNumEdges() == rows.size
+            assert np.array_equal(_host(sub._CAPI_GetCSC()[1]), rows)
+            seeds, h_seeds = frontier, want_frontier
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_sampler_properties_full_size(dev, sage_graph, replace):
+    """2^18 columns, fanout 10, checked without the oracle: counts, positions inside the column,
+    ids read from those positions, distinct positions per row without replacement; and the
+    one-launch and two-phase entry points agree bit for bit."""
+    indptr, indices, _, _ = sage_graph
+    S, k = 1 << 18, 10
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(9)
+    cols = torch.randint(0, 2_450_000, (S,), generator=gen, device=dev).to(torch.int32)
+    sub_indptr, sub, sel, coo = capi.sample_uniform_fused(indptr, indices, cols, k, replace, seed=4,
+                                                          with_coo=True)
+    nnz = int(sub_indptr[-1].item())
+    sub, sel, coo = sub[:nnz], sel[:nnz], coo[:nnz].long()
+    c = cols.long()
+    start, deg = indptr[c], indptr[c + 1] - indptr[c]
+    want_cnt = torch.where(deg > 0, torch.full_like(deg, k), deg) if replace else deg.clamp(max=k)
+    assert torch.equal(sub_indptr[1:] - sub_indptr[:-1], want_cnt)
+    assert torch.equal(coo, torch.repeat_interleave(torch.arange(S, device=dev), want_cnt))
+    assert bool(((sel >= start[coo]) & (sel < start[coo] + deg[coo])).all())
+    assert torch.equal(indices[sel], sub)
+    if not replace:
+        assert torch.unique(coo * (1 << 31) + (sel - start[coo])).numel() == nnz
+        full = deg <= k  # rows that fit are copied in order
+        first = sub_indptr[:-1][full]
+        assert torch.equal(sel[first[deg[full] > 0]], start[full][deg[full] > 0])
+    two = capi.sample_uniform(indptr, indices, cols, k, replace, seed=4, with_coo=True)
+    assert torch.equal(two[0], sub_indptr)
+    assert torch.equal(two[1][:nnz], sub) and torch.equal(two[2][:nnz], sel)
+
+
+def test_relabel_properties_full_size(dev, sage_graph):
+    """1.3 M ids with heavy repetition: the frontier is the distinct ids, seeds first, in
+    first-occurrence order, and relabelling inverts through it."""
+    indptr, indices, _, _ = sage_graph
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(3)
+    seeds = torch.randperm(2_450_000, generator=gen, device=dev)[:100_000].to(torch.int32)
+    sub_indptr, sub, _, _ = capi.sample_uniform_fused(indptr, indices, seeds, 12, False, seed=8)
+    sub = sub[:int(sub_indptr[-1].item())]
+    frontier, num, (rel,) = capi.unique_relabel([seeds, sub], [sub])
+    U = int(num.item())
+    frontier = frontier[:U]
+    assert torch.equal(frontier[:seeds.numel()], seeds)
+    assert U == torch.unique(torch.cat([seeds, sub])).numel() == torch.unique(frontier).numel()
+    assert torch.equal(frontier[rel.long()], sub)
+    # first-occurrence order: the rank of an id's first appearance grows with its position
+    cat = torch.cat([seeds, sub]).long()
+    first_pos = torch.full((2_450_000,), cat.numel(), dtype=torch.int64, device=dev)
+    first_pos.scatter_reduce_(0, cat, torch.arange(cat.numel(), device=dev), reduce="amin")
+    fp = first_pos[frontier.long()]
+    assert bool((fp[1:] > fp[:-1]).all())
+
+
+def test_random_walk_full_size_matches_oracle(dev):
+    """R-MAT 4 M nodes / 200 M edges, 1 M uniform starts, 80 steps: the 81 M-entry trace equals the
+    oracle's; independently, every step is an edge of the graph and -1 is absorbing."""
+    N, E, n, L = 4_000_000, 200_000_000, 1_000_000, 80
+    indptr, indices = rmat.rmat_csc(N, E, seed=0, device=dev, index_dtype=torch.int32)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4)
+    starts = torch.randint(0, N, (n,), generator=gen, device=dev).to(torch.int32)
+    trace = capi.random_walk(indptr, indices, starts, L, seed=21)
+    want = O.random_walk(_host(indptr), _host(indices), _host(starts), L, seed=21)
+    assert np.array_equal(_host(trace), want)
+    t = trace.view(L + 1, n).long()
+    assert torch.equal(t[0], starts.long())
+    dead = t == -1
+    assert bool((dead[1:] | ~dead[:-1]).all())  # once -1, always -1
+    # a live walker only dies in a column without neighbours
+    deg = indptr[1:] - indptr[:-1]
+    died = dead[1:] & ~dead[:-1]
+    assert bool((deg[t[:-1][died]] == 0).all())
+    # edge existence, step by step, against the sorted list of (column, neighbour) keys
+    col_of_edge = torch.repeat_interleave(torch.arange(N, device=dev), deg)
+    keys = torch.sort(col_of_edge * N + indices.long()).values
+    del col_of_edge
+    for s in range(0, L, 8):
+        c, r = t[s:s + 8].reshape(-1), t[s + 1:s + 9].reshape(-1)
+        live = r >= 0
+        q = c[live] * N + r[live]
+        pos = torch.searchsorted(keys, q).clamp(max=keys.numel() - 1)
+        assert torch.equal(keys[pos], q)
+
+
+def test_metapath_walk_full_size_matches_oracle(dev):
+    """Four bipartite relations (R-MAT 1 M x 2 M, 50 M edges each), metapath of 4 repeated 4 times,
+    1 M walkers, through HeteroGraph: the trace equals the oracle's."""
+    U, I_, T = 1_000_000, 2_000_000, 1_000_000
+    rel = {  # name: (src type size = rows, dst type size = columns)
+        "item_to_user": (I_, U), "user_to_item": (U, I_), "tag_to_item": (T, I_), "item_to_tag": (I_, T)}
+    graphs, host = {}, {}
+    for i, (name, (n_src, n_dst)) in enumerate(rel.items()):
+        ip, ix = rmat.rmat_csc(n_dst, 50_000_000, seed=10 + i, device=dev, num_src_nodes=n_src)
+        g = gs.Graph(False)
+        g._CAPI_LoadCSC(ip, ix)
+        graphs[name], host[name] = g, (_host(ip), _host(ix))
+    hg = gs.HeteroGraph()
+    # a walker sitting on a column of relation (src, name, dst) moves to one of its rows
+    hg._CAPI_LoadFromHomo(["user", "item", "tag"],
+                          [("item", "item_to_user", "user"), ("user", "user_to_item", "item"),
+                           ("tag", "tag_to_item", "item"), ("item", "item_to_tag", "tag")],
+                          [graphs[n] for n in rel])
+    # users -> items -> tags -> items -> users, four times
+    path = ["item_to_user", "tag_to_item", "item_to_tag", "user_to_item"] * 4
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(6)
+    starts = torch.randint(0, U, (1_000_000,), generator=gen, device=dev)
+    torch.ops.gs_ops._CAPI_SetSeed(77)
+    trace = hg._CAPI_MetapathRandomWalkFused(starts, path)
+    names = list(rel)
+    want = O.metapath_walk([host[n][0] for n in names], [host[n][1] for n in names],
+                           [names.index(p) for p in path], _host(starts), seed=77)
+    assert trace.shape == (1_000_000, 17)
+    assert np.array_equal(_host(trace.reshape(-1)), want)
+
+
+def test_ladies_layer_full_size_matches_oracle(dev, sage_graph):
+    """One LADIES layer on the 2.45 M-node graph with fp32 edge weights in (0, 1]: slice 512 seed
+    columns, row probability = sum of squared weights, weighted list sampling of 512 of the 2.45 M
+    rows, row slice, divide, normalise -- each stage against the oracle."""
+    indptr, indices32, h_indptr, h_indices = sage_graph
+    N = 2_450_000
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    weights = 1.0 - torch.rand(indices32.numel(), generator=gen, device=dev)
+    h_w = weights.cpu().numpy()
+    m = gs.Matrix()
+    m.load_csc(indptr, indices32.long(), weights)
+    seeds = torch.randperm(N, generator=gen, device=dev)[:512]
+    h_seeds = _host(seeds)
+    Uu = m[:, seeds]
+    prob = Uu.sum(axis=1, powk=2)
+    sp, coo, si, sel = O.slice_columns(h_indptr, h_indices, h_seeds)
+    want_prob = O.coo_sum(si, None, h_w[sel], 2, N)
+    np.testing.assert_allclose(prob.cpu().numpy(), want_prob, rtol=1e-5)
+
+    gs.set_seed(31)
+    row_ids = Uu.row_ids(remove_isolated=False)
+    selected, idx = torch.ops.gs_ops._CAPI_ListSamplingWithProbs(row_ids, prob, 512, False)
+    w_sel, w_idx = O.list_sample_weighted(np.arange(N), prob.cpu().numpy(), 512, seed=31)
+    assert np.array_equal(_host(idx), w_idx) and np.array_equal(_host(selected), w_sel)
+    assert (want_prob[w_idx] > 0).all()
+
+    nodes = torch.cat([seeds, selected]).unique()
+    h_nodes = _host(nodes)
+    subU = Uu[nodes, :]
+    r_ip, r_col, r_perm = O.coo2csc(si, coo, N, False)
+    s_ip, s_row, s_col, s_sel = O.slice_columns(r_ip, r_col, h_nodes)
+    w_data = h_w[sel][r_perm][s_sel]
+    assert subU.get_num_edges() == s_col.size
+    assert np.array_equal(subU.get_data().cpu().numpy(), w_data)
+    div = subU.divide(prob[nodes], axis=1)
+    w_div = w_data / want_prob[h_nodes][s_row]
+    np.testing.assert_allclose(div.get_data().cpu().numpy(), w_div, rtol=1e-5)
+    norm = div.normalize(axis=0)
+    col_sum = np.bincount(s_col, weights=w_div.astype(np.float64), minlength=h_seeds.size)
+    np.testing.assert_allclose(norm.get_data().cpu().numpy(), w_div / col_sum[s_col], rtol=1e-4)
+
+
+def test_sddmm_dot_on_sampled_blocks_full_size(dev, sage_graph):
+    """u_dot_v with 64-dim fp32 node features over the sampled edges of a [15,10,5] minibatch
+    (global row ids into a 2.45 M x 64 feature matrix), against a torch fp32 gather-and-dot; 1e-5
+    relative, the tolerance the dot product's summation order allows."""
+    indptr, indices, _, _ = sage_graph
+    N = 2_450_000
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(12)
+    feat = torch.randn(N, 64, generator=gen, device=dev)
+    m = gs.Matrix()
+    m.load_csc(indptr, indices.long())
+    seeds = torch.randperm(N, generator=gen, device=dev)[:1024]
+    gs.set_seed(3)
+    for k in FANOUTS:
+        sub = m.fused_columnwise_slicing_sampling(seeds, k, False)
+        rows = sub.row_indices()                  # global ids of the sampled neighbours
+        g = sub._graph
+        ptr = g._CAPI_GetCSC()[0]
+        col_local = torch.repeat_interleave(torch.arange(seeds.numel(), device=dev), ptr[1:] - ptr[:-1])
+        rhs = feat[seeds]
+        out = torch.zeros(rows.numel(), 1, device=dev)
+        g._CAPI_SDDMM("dot", feat, rhs, out, 0, 2, _CSC)
+        want = (feat[rows] * rhs[col_local]).sum(-1, keepdim=True)
+        torch.testing.assert_close(out, want, rtol=1e-5, atol=1e-5)
+        seeds = sub.all_indices()
