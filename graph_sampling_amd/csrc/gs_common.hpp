@@ -426,8 +426,8 @@ __device__ __forceinline__ int64_t lookback_exclusive_prefix(const LookbackState
             s[w] = before_first;
             break;
           }
-          // a poll is a round trip to memory shared by every tile: keep them sparse
-          if (polls < 4) __builtin_amdgcn_s_sleep(8); else __builtin_amdgcn_s_sleep(64);
+          // a poll is itself a round trip to memory; back off only when the wait is long
+          if (polls > 16) __builtin_amdgcn_s_sleep(32);
           s[w] = lb_load(&st.status[j]);
         }
         const unsigned long long closed = __ballot(lb_flag(s[w], st.epoch) == 2);
@@ -441,7 +441,8 @@ __device__ __forceinline__ int64_t lookback_exclusive_prefix(const LookbackState
     }
     newest -= kLookbackBurst * kWave;
   }
-  __threadfence();  // an error raised above is visible before the prefix that hides it
+  // (an error raised above was stored with device scope before this point)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   if (lane == 0) lb_store(&st.status[tile], lb_word(2u, st.epoch, running + total));
   return running;
 }

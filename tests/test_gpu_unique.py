@@ -77,3 +77,32 @@ def test_four_mapping_spans(dev):
     assert np.array_equal(frontier, want_frontier)
     for g, w in zip(outs, want):
         assert np.array_equal(g, w)
+
+
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+@pytest.mark.parametrize("n", [512 * 2048 - 1, 512 * 2048, 512 * 2048 + 1, 3_000_000])
+def test_relabel_million_items(dev, idt, n):
+    """Around 2^20 items (512 compaction tiles: several look-back bursts) and 3 M, with an aliased
+    and a plain query, heavy and light repetition."""
+    rng = np.random.default_rng(n)
+    seeds = rng.permutation(5_000_000)[:1000].astype(np.int64)
+    rows = np.concatenate([rng.integers(0, 2000, size=n // 2),            # hubs: heavy repetition
+                           rng.integers(0, 5_000_000, size=n - 1000 - n // 2)]).astype(np.int64)
+    rng.shuffle(rows)
+    probe = rng.integers(0, 5_000_100, size=5000).astype(np.int64)        # some absent ids
+    frontier, (rel_rows, rel_probe) = _run([seeds, rows], [rows, probe], dev, idt)
+    want_frontier, (want_rows, want_probe) = O.relabel([seeds, rows], [rows, probe])
+    assert np.array_equal(frontier, want_frontier)
+    assert np.array_equal(rel_rows, want_rows)
+    assert np.array_equal(rel_probe, want_probe)
+    assert (want_probe == -1).any()
+
+
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+def test_relabel_every_item_the_same_key(dev, idt):
+    """All tiles fight for one slot; one first occurrence in tile 0, every other tile has none."""
+    x = np.full(300_000, 12345, dtype=np.int64)
+    y = np.arange(300_000, dtype=np.int64) % 3
+    frontier, (rx, ry) = _run([x, y], [x, y], dev, idt)
+    assert np.array_equal(frontier, np.array([12345, 0, 1, 2]))
+    assert (rx == 0).all() and np.array_equal(ry, y + 1)
