@@ -34,14 +34,14 @@ HBM_PEAK_GBS = 8000.0
 # counters (2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE; the factors come from a device copy of
 # known size): profiles/sample_fused_rmat-2.45M-124M_hbm_counters.txt.  The counters cannot
 # be read from inside this process, so the figure is carried here.
-TRAFFIC_BYTES_PER_LAUNCH = {("rmat-2.45M-124M", "sample_fused"): 11628433}
+TRAFFIC_BYTES_PER_LAUNCH = {("rmat-2.45M-124M", "sample_fused"): 11629021}
 
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="rmat-2.45M-124M", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-steps", type=int, default=-1,
                     help="minibatches timed for the host-core baseline (-1: sized to ~15 s)")
@@ -83,6 +83,7 @@ class KernelTimer:
 #   table_insert  : per item  id b + one 8-byte slot read-modify-write 16 + slot index 4
 #   unique_finish : per item  slot index 4 + slot 8 + rank 8, relabeled id b, frontier b per U
 SITES = ("sample_fused", "table_init", "table_insert", "unique_compact", "unique_finish")
+# (unique_finish is the relabel lookup kernel)
 
 
 def floyd_bytes(b, S, E):
@@ -131,10 +132,9 @@ def cpu_minibatch(O, np, indptr, indices, seeds, step):
 
 
 def saturated(torch, graph, timer, nodes, idt, dev, b):
-    """The same sampler launch at the largest size the host layer routes to it (2^18 seed
-    columns drawn with repetition, fanout 10): what the kernel reaches once launch latency is
-    amortised."""
-    S = 1 << 18
+    """The same sampler launch at a size that fills the chip (4M seed columns drawn with
+    repetition, fanout 10): what the kernel reaches once launch latency is amortised."""
+    S = 1 << 22
     gen = torch.Generator(device=dev)
     gen.manual_seed(5)
     cols = torch.randint(0, nodes, (S,), generator=gen, device=dev).to(idt)
