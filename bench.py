@@ -119,6 +119,20 @@ def minibatch(graph, seeds):
     return total, sizes, seeds
 
 
+def minibatch_nonfused(graph, seeds):
+    """The same minibatch through the unfused operators of the Matrix API (A[:, seeds] ->
+    columnwise_sampling -> relabel; python/gs/matrix_api/matrix.py:66-84 of the reference):
+    _CAPI_Slicing(seeds, 0, _CSC, _COO) materialises every neighbour of the seeds first."""
+    total = 0
+    for k in FANOUTS:
+        sliced = graph._CAPI_Slicing(seeds, 0, 2, 1, False)
+        sub = sliced._CAPI_Sampling(0, k, False, 2, 1)
+        frontier, num_src, num_dst, row, col, e_ids, fmt = sub._CAPI_Relabel()
+        total += row.numel()
+        seeds = frontier
+    return total
+
+
 def cpu_minibatch(O, np, indptr, indices, seeds, step):
     total = 0
     for layer, k in enumerate(FANOUTS):
@@ -246,6 +260,18 @@ def main():
     p50 = lat[len(lat) // 2] * 1e3
     p90 = lat[min(len(lat) - 1, int(len(lat) * 0.9))] * 1e3
 
+    # the unfused operator sequence on the same seed sets (reported beside the headline)
+    nf_steps = min(args.steps, 50)
+    for i in range(3):
+        minibatch_nonfused(graph, seed_sets[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    nf_edges = 0
+    for i in range(nf_steps):
+        nf_edges += minibatch_nonfused(graph, seed_sets[args.warmup + i])
+    torch.cuda.synchronize()
+    nf_s = time.perf_counter() - t1
+
     out = {
         "metric": "sampled edges/sec (GSEPS), GraphSAGE [15,10,5] batch 1024, slice+sample+relabel",
         "value": sampled / elapsed,
@@ -264,6 +290,9 @@ def main():
         "config": {"workload": args.workload, "nodes": nodes, "edges": edges, "batch": BATCH,
                    "fanouts": list(FANOUTS), "last_step_layers_S_E_U": layer_sizes,
                    "graph_build_s": round(gen_s, 2)},
+        "unfused_path": {"ms_per_step": nf_s / nf_steps * 1e3, "value": nf_edges / nf_s,
+                         "steps": nf_steps,
+                         "what": "Slicing -> Sampling -> Relabel per layer instead of the fused sampler"},
         "roofline": None,
         "cpu_baseline": None,
     }

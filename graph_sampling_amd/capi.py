@@ -433,11 +433,11 @@ def sddmm_coo(op, row, col, e_ids, lhs, rhs, out, lhs_target, rhs_target, lhs_le
               out_len, reduce_size, lhs_off=None, rhs_off=None):
     if op not in OPS:
         raise GsError("Unsupported SpMM/SDDMM binary operator: %s" % op)
-    _need(row, torch.int64, "row")
-    _need(col, torch.int64, "col")
+    idb = _ids(row, "row")
+    _ids(col, "col", like=row)
     _need(out, torch.float32, "out")
     dev = row.device
-    _check(lib().gs_sddmm_coo(OPS[op], _ptr(row), _ptr(col), _ptr(e_ids), _i64(row.numel()),
+    _check(lib().gs_sddmm_coo(OPS[op], _ptr(row), _ptr(col), idb, _ptr(e_ids), _i64(row.numel()),
                               _ptr(lhs), _ptr(rhs), _ptr(out), int(lhs_target), int(rhs_target),
                               _i64(lhs_len), _i64(rhs_len), _i64(out_len), _i64(reduce_size),
                               _ptr(lhs_off), _ptr(rhs_off), _stream(dev)), "gs_sddmm_coo")
@@ -448,10 +448,12 @@ def sddmm_csc(op, indptr, indices, e_ids, nid_map, lhs, rhs, out, lhs_target, rh
     if op not in OPS:
         raise GsError("Unsupported SpMM/SDDMM binary operator: %s" % op)
     _need(indptr, torch.int64, "indptr")
-    _need(indices, torch.int64, "indices")
+    idb = _ids(indices, "indices")
+    if nid_map is not None:
+        _ids(nid_map, "nid_map", like=indices)
     _need(out, torch.float32, "out")
     dev = indptr.device
-    _check(lib().gs_sddmm_csc(OPS[op], _ptr(indptr), _ptr(indices), _ptr(e_ids), _ptr(nid_map),
+    _check(lib().gs_sddmm_csc(OPS[op], _ptr(indptr), _ptr(indices), idb, _ptr(e_ids), _ptr(nid_map),
                               _i64(indptr.numel() - 1), _i64(indices.numel()), _ptr(lhs), _ptr(rhs),
                               _ptr(out), int(lhs_target), int(rhs_target), _i64(lhs_len),
                               _i64(rhs_len), _i64(out_len), _i64(reduce_size), _ptr(lhs_off),
@@ -463,17 +465,18 @@ def segment_sum(indptr, e_ids, n_ids, data, powk, out):
     _need(indptr, torch.int64, "indptr")
     _need(data, torch.float32, "data")
     _need(out, torch.float32, "out")
-    _check(lib().gs_segment_sum(_ptr(indptr), _ptr(e_ids), _ptr(n_ids), _ptr(data),
+    idb = _ids(n_ids, "n_ids") if n_ids is not None else 8
+    _check(lib().gs_segment_sum(_ptr(indptr), _ptr(e_ids), _ptr(n_ids), idb, _ptr(data),
                                 _i64(indptr.numel() - 1), _i64(powk), _ptr(out),
                                 _stream(indptr.device)), "gs_segment_sum")
 
 
 def coo_sum(target, e_ids, data, powk, out):
-    _need(target, torch.int64, "target")
+    idb = _ids(target, "target")
     _need(data, torch.float32, "data")
     _need(out, torch.float32, "out")
-    _check(lib().gs_coo_sum(_ptr(target), _ptr(e_ids), _ptr(data), _i64(target.numel()), _i64(powk),
-                            _ptr(out), _stream(target.device)), "gs_coo_sum")
+    _check(lib().gs_coo_sum(_ptr(target), idb, _ptr(e_ids), _ptr(data), _i64(target.numel()),
+                            _i64(powk), _ptr(out), _stream(target.device)), "gs_coo_sum")
 
 
 def segment_normalize(indptr, e_ids, data, out):
@@ -486,87 +489,87 @@ def segment_normalize(indptr, e_ids, data, out):
 
 
 def e_div_u_sum(row, col, data, divisor, out_data, out_sum):
-    _need(row, torch.int64, "row")
-    _need(col, torch.int64, "col")
+    idb = _ids(row, "row")
+    _ids(col, "col", like=row)
     _need(data, torch.float32, "data")
     _need(divisor, torch.float32, "divisor")
-    _check(lib().gs_e_div_u_sum(_ptr(row), _ptr(col), _ptr(data), _ptr(divisor), _i64(row.numel()),
-                                _ptr(out_data), _ptr(out_sum), _stream(row.device)),
-           "gs_e_div_u_sum")
+    _check(lib().gs_e_div_u_sum(_ptr(row), _ptr(col), idb, _ptr(data), _ptr(divisor),
+                                _i64(row.numel()), _ptr(out_data), _ptr(out_sum),
+                                _stream(row.device)), "gs_e_div_u_sum")
 
 
 # ------------------------------------------------------------ row slicing ----
 def row_slice_csc(indptr, indices, row_ids, with_coo):
     """Two-phase gs_row_slice_csc_*; returns (out_indptr, coo_col|None, out_indices, select_index)."""
     _need(indptr, torch.int64, "indptr")
-    _need(indices, torch.int64, "indices")
-    _need(row_ids, torch.int64, "row_ids")
+    idb = _ids(indices, "indices")
+    _ids(row_ids, "row_ids", like=indices)
     dev = indptr.device
     ncols, nnz, nr = indptr.numel() - 1, indices.numel(), row_ids.numel()
     out_indptr = torch.empty(ncols + 1, dtype=torch.int64, device=dev)
     ws = workspace(lib().gs_row_slice_workspace_bytes(_i64(nr), _i64(nnz), _i64(ncols)), dev)
     st = _stream(dev)
-    _check(lib().gs_row_slice_csc_mark(_ptr(indptr), _ptr(indices), _i64(ncols), _i64(nnz),
+    _check(lib().gs_row_slice_csc_mark(_ptr(indptr), _ptr(indices), idb, _i64(ncols), _i64(nnz),
                                        _ptr(row_ids), _i64(nr), _ptr(out_indptr), _ptr(ws),
                                        ctypes.c_size_t(ws.numel()), st), "gs_row_slice_csc_mark")
     kept = int(out_indptr[-1].item())
-    out_indices = torch.empty(kept, dtype=torch.int64, device=dev)
+    out_indices = torch.empty(kept, dtype=indices.dtype, device=dev)
     select_index = torch.empty(kept, dtype=torch.int64, device=dev)
-    coo_col = torch.empty(kept, dtype=torch.int64, device=dev) if with_coo else None
+    coo_col = torch.empty(kept, dtype=indices.dtype, device=dev) if with_coo else None
     if kept == 0:
         return out_indptr, coo_col, out_indices, select_index
-    _check(lib().gs_row_slice_csc_compact(_ptr(indptr), _ptr(indices), _i64(ncols), _i64(nnz),
-                                          _ptr(out_indptr), _ptr(out_indices), _ptr(select_index),
-                                          _ptr(coo_col), _ptr(ws), ctypes.c_size_t(ws.numel()), st),
+    _check(lib().gs_row_slice_csc_compact(_ptr(indptr), _i64(ncols), _i64(nnz), idb,
+                                          _ptr(out_indices), _ptr(select_index), _ptr(coo_col),
+                                          _ptr(ws), ctypes.c_size_t(ws.numel()), st),
            "gs_row_slice_csc_compact")
     return out_indptr, coo_col, out_indices, select_index
 
 
 def row_slice_coo(key, other, ids):
     """Two-phase gs_row_slice_coo_*; returns (relabelled key, other, select_index)."""
-    _need(key, torch.int64, "key")
-    _need(other, torch.int64, "other")
-    _need(ids, torch.int64, "ids")
+    idb = _ids(key, "key")
+    _ids(other, "other", like=key)
+    _ids(ids, "ids", like=key)
     dev = key.device
     E, n = key.numel(), ids.numel()
     num_kept = torch.empty(1, dtype=torch.int64, device=dev)
     ws = workspace(lib().gs_row_slice_workspace_bytes(_i64(n), _i64(E), _i64(0)), dev)
     st = _stream(dev)
-    _check(lib().gs_row_slice_coo_mark(_ptr(key), _i64(E), _ptr(ids), _i64(n), _ptr(num_kept),
+    _check(lib().gs_row_slice_coo_mark(_ptr(key), idb, _i64(E), _ptr(ids), _i64(n), _ptr(num_kept),
                                        _ptr(ws), ctypes.c_size_t(ws.numel()), st),
            "gs_row_slice_coo_mark")
     kept = int(num_kept.item())
-    out_key = torch.empty(kept, dtype=torch.int64, device=dev)
-    out_other = torch.empty(kept, dtype=torch.int64, device=dev)
+    out_key = torch.empty(kept, dtype=key.dtype, device=dev)
+    out_other = torch.empty(kept, dtype=key.dtype, device=dev)
     select_index = torch.empty(kept, dtype=torch.int64, device=dev)
     if kept == 0:
         return out_key, out_other, select_index
-    _check(lib().gs_row_slice_coo_compact(_ptr(key), _ptr(other), _i64(E), _ptr(out_key),
+    _check(lib().gs_row_slice_coo_compact(_ptr(other), idb, _i64(E), _ptr(out_key),
                                           _ptr(out_other), _ptr(select_index), _ptr(ws),
                                           ctypes.c_size_t(ws.numel()), st), "gs_row_slice_coo_compact")
     return out_key, out_other, select_index
 
 
 # ------------------------------------------------------- format transform ----
-def csc2coo(indptr, nnz):
+def csc2coo(indptr, nnz, id_dtype=torch.int64):
     _need(indptr, torch.int64, "indptr")
-    col = torch.empty(nnz, dtype=torch.int64, device=indptr.device)
+    col = torch.empty(nnz, dtype=id_dtype, device=indptr.device)
     _check(lib().gs_csc2coo(_ptr(indptr), _i64(indptr.numel() - 1), _i64(nnz), _ptr(col),
-                            _stream(indptr.device)), "gs_csc2coo")
+                            _id_bytes(col), _stream(indptr.device)), "gs_csc2coo")
     return col
 
 
 def coo2csc(key, value, num_keys, is_sorted):
     """Returns (indptr, sorted value | value, perm | None)."""
-    _need(key, torch.int64, "key")
-    _need(value, torch.int64, "value")
+    idb = _ids(key, "key")
+    _ids(value, "value", like=key)
     dev = key.device
     E = key.numel()
     indptr = torch.empty(num_keys + 1, dtype=torch.int64, device=dev)
-    out_value = None if is_sorted else torch.empty(E, dtype=torch.int64, device=dev)
+    out_value = None if is_sorted else torch.empty(E, dtype=value.dtype, device=dev)
     perm = None if is_sorted else torch.empty(E, dtype=torch.int64, device=dev)
     ws = workspace(lib().gs_coo2csc_workspace_bytes(_i64(E), _i64(num_keys)), dev)
-    _check(lib().gs_coo2csc(_ptr(key), _ptr(value), _i64(E), _i64(num_keys), int(bool(is_sorted)),
-                            _ptr(indptr), _ptr(out_value), _ptr(perm), _ptr(ws),
+    _check(lib().gs_coo2csc(_ptr(key), _ptr(value), idb, _i64(E), _i64(num_keys),
+                            int(bool(is_sorted)), _ptr(indptr), _ptr(out_value), _ptr(perm), _ptr(ws),
                             ctypes.c_size_t(ws.numel()), _stream(dev)), "gs_coo2csc")
     return indptr, (value if is_sorted else out_value), perm

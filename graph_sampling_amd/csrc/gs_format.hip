@@ -35,9 +35,10 @@ __device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
   return lo;
 }
 
+template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz,
-               int64_t* __restrict__ col) {
+               IdT* __restrict__ col) {
   __shared__ int64_t s_ptr[kStage + 1];
   __shared__ int64_t s_rows[2];
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
@@ -55,24 +56,25 @@ csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz
   for (int k = 0; k < kItems; ++k) {
     const int64_t p = p0 + k * kThreads + threadIdx.x;
     if (p >= p1) break;
-    col[p] = row_lo + (staged ? upper_bound(s_ptr, nrows + 1, p)
-                              : upper_bound(indptr + row_lo, nrows + 1, p)) - 1;
+    col[p] = static_cast<IdT>(row_lo + (staged ? upper_bound(s_ptr, nrows + 1, p)
+                                               : upper_bound(indptr + row_lo, nrows + 1, p)) - 1);
   }
 }
 
 // indptr from sorted keys: every boundary between key[e] and key[e+1] fills the
 // offsets of the columns in between (format_transform.cu:123-156 computes the
 // same values with one binary search per column).
+template <typename KeyT>
 __global__ void __launch_bounds__(kThreads)
-indptr_from_sorted_kernel(const int64_t* __restrict__ key, int64_t E, int64_t num_keys,
+indptr_from_sorted_kernel(const KeyT* __restrict__ key, int64_t E, int64_t num_keys,
                           int64_t* __restrict__ indptr) {
   const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (e > E) return;
   // boundary e sits between key[e-1] and key[e]; columns in (key[e-1], key[e]] start at e
   // keys outside [0, num_keys) (an inconsistent caller) are clamped: they can
   // never index past the num_keys + 1 offsets
-  int64_t lo = e == 0 ? -1 : key[e - 1];
-  int64_t hi = e == E ? num_keys : key[e];
+  int64_t lo = e == 0 ? -1 : static_cast<int64_t>(key[e - 1]);
+  int64_t hi = e == E ? num_keys : static_cast<int64_t>(key[e]);
   if (lo < -1) lo = -1;
   if (hi > num_keys) hi = num_keys;
   for (int64_t c = lo + 1; c <= hi; ++c) indptr[c] = e;
@@ -87,9 +89,11 @@ __device__ __forceinline__ int digit_of(int64_t key, int shift) {
   return static_cast<int>((static_cast<uint64_t>(key) >> shift) & (kRadix - 1));
 }
 
-// counts[d * num_blocks + b] = items of tile b with digit d
+// counts[d * num_blocks + b] = items of tile b with digit d.  KeyT is the
+// caller's id type in the first pass and int64 (the ping-pong buffers) after it.
+template <typename KeyT>
 __global__ void __launch_bounds__(kThreads)
-radix_hist_kernel(const int64_t* __restrict__ keys, int64_t E, int shift, int64_t num_blocks,
+radix_hist_kernel(const KeyT* __restrict__ keys, int64_t E, int shift, int64_t num_blocks,
                   int64_t* __restrict__ counts) {
   __shared__ int s_hist[kRadix];
   s_hist[threadIdx.x] = 0;
@@ -98,7 +102,7 @@ radix_hist_kernel(const int64_t* __restrict__ keys, int64_t E, int shift, int64_
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
     const int64_t i = base + k * kThreads + threadIdx.x;
-    if (i < E) atomicAdd(&s_hist[digit_of(keys[i], shift)], 1);
+    if (i < E) atomicAdd(&s_hist[digit_of(static_cast<int64_t>(keys[i]), shift)], 1);
   }
   __syncthreads();
   counts[static_cast<int64_t>(threadIdx.x) * num_blocks + blockIdx.x] = s_hist[threadIdx.x];
@@ -112,8 +116,9 @@ struct LoadI64 {
 // Stable scatter of one tile.  Items are visited in index order, 256 per round;
 // inside a round the rank of an item among equal digits is (earlier waves'
 // count) + (lower lanes of its wave with the same digit).
+template <typename KeyT>
 __global__ void __launch_bounds__(kThreads)
-radix_scatter_kernel(const int64_t* __restrict__ keys_in, const int64_t* __restrict__ perm_in,
+radix_scatter_kernel(const KeyT* __restrict__ keys_in, const int64_t* __restrict__ perm_in,
                      int64_t E, int shift, int64_t num_blocks, const int64_t* __restrict__ offsets,
                      int64_t* __restrict__ keys_out, int64_t* __restrict__ perm_out) {
   __shared__ int64_t s_base[kRadix];
@@ -132,7 +137,7 @@ radix_scatter_kernel(const int64_t* __restrict__ keys_in, const int64_t* __restr
     int d = 0;
     unsigned long long peers = __ballot(live);
     if (live) {
-      key = keys_in[i];
+      key = static_cast<int64_t>(keys_in[i]);
       d = digit_of(key, shift);
     }
 #pragma unroll
@@ -159,9 +164,10 @@ radix_scatter_kernel(const int64_t* __restrict__ keys_in, const int64_t* __restr
   }
 }
 
+template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
-gather_kernel(const int64_t* __restrict__ value, const int64_t* __restrict__ perm, int64_t E,
-              int64_t* __restrict__ out) {
+gather_kernel(const IdT* __restrict__ value, const int64_t* __restrict__ perm, int64_t E,
+              IdT* __restrict__ out) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i < E) out[i] = value[perm[i]];
 }
@@ -172,6 +178,61 @@ int num_passes(int64_t num_keys) {
   return (bits + kRadixBits - 1) / kRadixBits;
 }
 
+template <typename IdT>
+int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, int sorted,
+                 int64_t* indptr, IdT* out_value, int64_t* perm, void* workspace,
+                 size_t workspace_bytes, hipStream_t st) {
+  if (sorted || E == 0) {
+    hipLaunchKernelGGL((indptr_from_sorted_kernel<IdT>), dim3(blocks_for(E + 1, kThreads)),
+                       dim3(kThreads), 0, st, key, E, num_keys, indptr);
+    return check_launch("coo2csc");
+  }
+  const int64_t blocks = blocks_for(E, kTile);
+  const int64_t table = kRadix * blocks;
+  Carver ws(workspace, workspace_bytes);
+  int64_t* kbuf[2] = {ws.take<int64_t>(E), ws.take<int64_t>(E)};
+  int64_t* pbuf = ws.take<int64_t>(E);
+  int64_t* counts = ws.take<int64_t>(table);
+  int64_t* offsets = ws.take<int64_t>(table + 1);
+  int64_t* tiles = ws.take<int64_t>(scan_num_tiles(table) + 1);
+  if (!ws.ok) {
+    set_error_text("gs_coo2csc: workspace needs %zu bytes, 256-byte aligned",
+                   gs_coo2csc_workspace_bytes(E, num_keys));
+    return GS_ERR_WORKSPACE;
+  }
+  int passes = num_passes(num_keys);
+  if (passes == 0) passes = 1;  // one key: still produces perm = identity
+  const int64_t* kin = nullptr;  // null: the first pass reads the caller's keys
+  const int64_t* pin = nullptr;
+  // perm alternates between `perm` and pbuf so that the last pass lands in `perm`
+  for (int p = 0; p < passes; ++p) {
+    int64_t* kout = kbuf[p & 1];
+    int64_t* pout = ((passes - 1 - p) & 1) ? pbuf : perm;
+    if (p == 0)
+      hipLaunchKernelGGL((radix_hist_kernel<IdT>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kThreads), 0, st, key, E, 0, blocks, counts);
+    else
+      hipLaunchKernelGGL((radix_hist_kernel<int64_t>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kThreads), 0, st, kin, E, p * kRadixBits, blocks, counts);
+    LoadI64 f{counts};
+    GS_RETURN_IF_ERROR(exclusive_scan(f, table, offsets, tiles, st));
+    if (p == 0)
+      hipLaunchKernelGGL((radix_scatter_kernel<IdT>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kThreads), 0, st, key, pin, E, 0, blocks, offsets, kout, pout);
+    else
+      hipLaunchKernelGGL((radix_scatter_kernel<int64_t>), dim3(static_cast<unsigned>(blocks)),
+                         dim3(kThreads), 0, st, kin, pin, E, p * kRadixBits, blocks, offsets, kout,
+                         pout);
+    kin = kout;
+    pin = pout;
+  }
+  hipLaunchKernelGGL((gather_kernel<IdT>), dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st,
+                     value, perm, E, out_value);
+  hipLaunchKernelGGL((indptr_from_sorted_kernel<int64_t>), dim3(blocks_for(E + 1, kThreads)),
+                     dim3(kThreads), 0, st, kin, E, num_keys, indptr);
+  return check_launch("coo2csc");
+}
+
 }  // namespace
 }  // namespace gs
 
@@ -179,12 +240,19 @@ using namespace gs;
 
 extern "C" {
 
-int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, int64_t* col, void* stream) {
+int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, void* col, int id_bytes,
+               void* stream) {
   GS_REQUIRE(num_cols >= 0 && nnz >= 0, "gs_csc2coo: negative size");
   GS_REQUIRE(nnz == 0 || (indptr && col), "gs_csc2coo: null pointer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_csc2coo: id_bytes must be 4 or 8, got %d", id_bytes);
   if (nnz == 0) return GS_OK;
-  hipLaunchKernelGGL(csc2coo_kernel, dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
-                     static_cast<hipStream_t>(stream), indptr, num_cols, nnz, col);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (id_bytes == 8)
+    hipLaunchKernelGGL((csc2coo_kernel<int64_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
+                       st, indptr, num_cols, nnz, static_cast<int64_t*>(col));
+  else
+    hipLaunchKernelGGL((csc2coo_kernel<int32_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
+                       st, indptr, num_cols, nnz, static_cast<int32_t*>(col));
   return check_launch("csc2coo");
 }
 
@@ -198,53 +266,24 @@ size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys) {
          scan_workspace_bytes(table);
 }
 
-int gs_coo2csc(const int64_t* key, const int64_t* value, int64_t E, int64_t num_keys, int sorted,
-               int64_t* indptr, int64_t* out_value, int64_t* perm, void* workspace,
+int gs_coo2csc(const void* key, const void* value, int id_bytes, int64_t E, int64_t num_keys,
+               int sorted, int64_t* indptr, void* out_value, int64_t* perm, void* workspace,
                size_t workspace_bytes, void* stream) {
   GS_REQUIRE(E >= 0 && num_keys >= 0 && indptr, "gs_coo2csc: negative size or null indptr");
   GS_REQUIRE(E == 0 || key, "gs_coo2csc: key is null");
   GS_REQUIRE(sorted || E == 0 || (value && out_value && perm),
              "gs_coo2csc: value/out_value/perm required when the keys are not sorted");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_coo2csc: id_bytes must be 4 or 8, got %d", id_bytes);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const int64_t* sorted_keys = key;
-  if (!sorted && E > 0) {
-    const int64_t blocks = blocks_for(E, kTile);
-    const int64_t table = kRadix * blocks;
-    Carver ws(workspace, workspace_bytes);
-    int64_t* kbuf[2] = {ws.take<int64_t>(E), ws.take<int64_t>(E)};
-    int64_t* pbuf = ws.take<int64_t>(E);
-    int64_t* counts = ws.take<int64_t>(table);
-    int64_t* offsets = ws.take<int64_t>(table + 1);
-    int64_t* tiles = ws.take<int64_t>(scan_num_tiles(table) + 1);
-    if (!ws.ok) {
-      set_error_text("gs_coo2csc: workspace needs %zu bytes, 256-byte aligned",
-                     gs_coo2csc_workspace_bytes(E, num_keys));
-      return GS_ERR_WORKSPACE;
-    }
-    int passes = num_passes(num_keys);
-    if (passes == 0) passes = 1;  // one key: still produces perm = identity
-    const int64_t* kin = key;
-    const int64_t* pin = nullptr;
-    // perm alternates between `perm` and pbuf so that the last pass lands in `perm`
-    for (int p = 0; p < passes; ++p) {
-      int64_t* kout = kbuf[p & 1];
-      int64_t* pout = ((passes - 1 - p) & 1) ? pbuf : perm;
-      hipLaunchKernelGGL(radix_hist_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0,
-                         st, kin, E, p * kRadixBits, blocks, counts);
-      LoadI64 f{counts};
-      GS_RETURN_IF_ERROR(exclusive_scan(f, table, offsets, tiles, st));
-      hipLaunchKernelGGL(radix_scatter_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kThreads),
-                         0, st, kin, pin, E, p * kRadixBits, blocks, offsets, kout, pout);
-      kin = kout;
-      pin = pout;
-    }
-    sorted_keys = kin;
-    hipLaunchKernelGGL(gather_kernel, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st, value,
-                       perm, E, out_value);
-  }
-  hipLaunchKernelGGL(indptr_from_sorted_kernel, dim3(blocks_for(E + 1, kThreads)), dim3(kThreads),
-                     0, st, sorted_keys, E, num_keys, indptr);
-  return check_launch("coo2csc");
+  return id_bytes == 8
+             ? coo2csc_impl<int64_t>(static_cast<const int64_t*>(key),
+                                     static_cast<const int64_t*>(value), E, num_keys, sorted,
+                                     indptr, static_cast<int64_t*>(out_value), perm, workspace,
+                                     workspace_bytes, st)
+             : coo2csc_impl<int32_t>(static_cast<const int32_t*>(key),
+                                     static_cast<const int32_t*>(value), E, num_keys, sorted,
+                                     indptr, static_cast<int32_t*>(out_value), perm, workspace,
+                                     workspace_bytes, st);
 }
 
 }  // extern "C"

@@ -56,11 +56,12 @@ __global__ void __launch_bounds__(kThreads) set_init_kernel(IdSet t, int64_t cap
   }
 }
 
+template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
-set_insert_kernel(IdSet t, const int64_t* __restrict__ ids, int64_t n) {
+set_insert_kernel(IdSet t, const IdT* __restrict__ ids, int64_t n) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= n) return;
-  const long long key = ids[i];
+  const long long key = static_cast<long long>(ids[i]);
   uint32_t p = t.home(key);
   while (true) {
     const unsigned long long prev =
@@ -72,10 +73,11 @@ set_insert_kernel(IdSet t, const int64_t* __restrict__ ids, int64_t n) {
   atomicMax(&t.vals[p], static_cast<long long>(i));
 }
 
+template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
-mark_kernel(IdSet t, const int64_t* __restrict__ key, int64_t E, int64_t* __restrict__ val) {
+mark_kernel(IdSet t, const IdT* __restrict__ key, int64_t E, int64_t* __restrict__ val) {
   const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (e < E) val[e] = t.query(key[e]);
+  if (e < E) val[e] = t.query(static_cast<long long>(key[e]));
 }
 
 struct Kept {
@@ -106,12 +108,12 @@ __device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
 }
 
 // CSC compaction; a workgroup owns 2048 consecutive input edges.
-template <bool WITH_COO>
+template <bool WITH_COO, typename IdT>
 __global__ void __launch_bounds__(kThreads)
 csc_compact_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz,
                    const int64_t* __restrict__ val, const int64_t* __restrict__ prefix,
-                   int64_t* __restrict__ out_indices, int64_t* __restrict__ select_index,
-                   int64_t* __restrict__ coo_col) {
+                   IdT* __restrict__ out_indices, int64_t* __restrict__ select_index,
+                   IdT* __restrict__ coo_col) {
   __shared__ int64_t s_ptr[kStage + 1];
   __shared__ int64_t s_rows[2];
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
@@ -136,24 +138,25 @@ csc_compact_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t
     const int64_t v = val[e];
     if (v < 0) continue;
     const int64_t w = prefix[e];
-    out_indices[w] = v;
+    out_indices[w] = static_cast<IdT>(v);
     select_index[w] = e;
     if (WITH_COO)
-      coo_col[w] = row_lo + (staged ? upper_bound(s_ptr, nrows + 1, e)
-                                    : upper_bound(indptr + row_lo, nrows + 1, e)) - 1;
+      coo_col[w] = static_cast<IdT>(row_lo + (staged ? upper_bound(s_ptr, nrows + 1, e)
+                                                     : upper_bound(indptr + row_lo, nrows + 1, e)) - 1);
   }
 }
 
+template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
-coo_compact_kernel(const int64_t* __restrict__ other, int64_t E, const int64_t* __restrict__ val,
-                   const int64_t* __restrict__ prefix, int64_t* __restrict__ out_key,
-                   int64_t* __restrict__ out_other, int64_t* __restrict__ select_index) {
+coo_compact_kernel(const IdT* __restrict__ other, int64_t E, const int64_t* __restrict__ val,
+                   const int64_t* __restrict__ prefix, IdT* __restrict__ out_key,
+                   IdT* __restrict__ out_other, int64_t* __restrict__ select_index) {
   const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (e >= E) return;
   const int64_t v = val[e];
   if (v < 0) return;
   const int64_t w = prefix[e];
-  out_key[w] = v;
+  out_key[w] = static_cast<IdT>(v);
   out_other[w] = other[e];
   select_index[w] = e;
 }
@@ -190,16 +193,17 @@ Scratch carve(void* workspace, size_t bytes, int64_t n_ids, int64_t E, bool with
   return s;
 }
 
-int mark_common(const char* who, const int64_t* key, int64_t E, const int64_t* ids, int64_t n_ids,
+template <typename IdT>
+int mark_common(const char* who, const void* key, int64_t E, const void* ids, int64_t n_ids,
                 Scratch& s, hipStream_t st) {
   hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(s.cap, kThreads)), dim3(kThreads), 0, st,
                      s.set, s.cap);
   if (n_ids > 0)
-    hipLaunchKernelGGL(set_insert_kernel, dim3(blocks_for(n_ids, kThreads)), dim3(kThreads), 0, st,
-                       s.set, ids, n_ids);
+    hipLaunchKernelGGL(set_insert_kernel<IdT>, dim3(blocks_for(n_ids, kThreads)), dim3(kThreads), 0,
+                       st, s.set, static_cast<const IdT*>(ids), n_ids);
   if (E > 0)
-    hipLaunchKernelGGL(mark_kernel, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st, s.set, key,
-                       E, s.val);
+    hipLaunchKernelGGL(mark_kernel<IdT>, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st, s.set,
+                       static_cast<const IdT*>(key), E, s.val);
   GS_RETURN_IF_ERROR(check_launch(who));
   Kept f{s.val};
   return exclusive_scan(f, E, s.prefix, s.tiles, st);
@@ -221,13 +225,15 @@ size_t gs_row_slice_workspace_bytes(int64_t num_row_ids, int64_t nnz, int64_t nu
          scan_workspace_bytes(nnz);
 }
 
-int gs_row_slice_csc_mark(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
-                          int64_t nnz, const int64_t* row_ids, int64_t num_row_ids,
+int gs_row_slice_csc_mark(const int64_t* indptr, const void* indices, int id_bytes,
+                          int64_t num_cols, int64_t nnz, const void* row_ids, int64_t num_row_ids,
                           int64_t* out_indptr, void* workspace, size_t workspace_bytes,
                           void* stream) {
   GS_REQUIRE(num_cols >= 0 && nnz >= 0 && num_row_ids >= 0, "gs_row_slice_csc_mark: negative size");
   GS_REQUIRE(indptr && out_indptr && (nnz == 0 || indices) && (num_row_ids == 0 || row_ids),
              "gs_row_slice_csc_mark: null pointer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_row_slice_csc_mark: id_bytes must be 4 or 8, got %d",
+             id_bytes);
   Scratch s = carve(workspace, workspace_bytes, num_row_ids, nnz, true);
   if (!s.ok) {
     set_error_text("gs_row_slice_csc_mark: workspace needs %zu bytes, 256-byte aligned",
@@ -235,19 +241,21 @@ int gs_row_slice_csc_mark(const int64_t* indptr, const int64_t* indices, int64_t
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  GS_RETURN_IF_ERROR(mark_common("row_slice_csc_mark", indices, nnz, row_ids, num_row_ids, s, st));
+  GS_RETURN_IF_ERROR(id_bytes == 8 ? mark_common<int64_t>("row_slice_csc_mark", indices, nnz, row_ids,
+                                                          num_row_ids, s, st)
+                                   : mark_common<int32_t>("row_slice_csc_mark", indices, nnz, row_ids,
+                                                          num_row_ids, s, st));
   hipLaunchKernelGGL(new_indptr_kernel, dim3(blocks_for(num_cols + 1, kThreads)), dim3(kThreads), 0,
                      st, indptr, num_cols, s.prefix, out_indptr);
   return check_launch("row_slice_csc_mark");
 }
 
-int gs_row_slice_csc_compact(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
-                             int64_t nnz, const int64_t* out_indptr, int64_t* out_indices,
-                             int64_t* select_index, int64_t* coo_col, void* workspace,
-                             size_t workspace_bytes, void* stream) {
-  (void)indices;
-  (void)out_indptr;
+int gs_row_slice_csc_compact(const int64_t* indptr, int64_t num_cols, int64_t nnz, int id_bytes,
+                             void* out_indices, int64_t* select_index, void* coo_col,
+                             void* workspace, size_t workspace_bytes, void* stream) {
   GS_REQUIRE(num_cols >= 0 && nnz >= 0 && indptr, "gs_row_slice_csc_compact: bad argument");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_row_slice_csc_compact: id_bytes must be 4 or 8, got %d",
+             id_bytes);
   if (nnz == 0) return GS_OK;
   GS_REQUIRE(out_indices && select_index, "gs_row_slice_csc_compact: null output");
   Scratch s = carve(workspace, workspace_bytes, 0, nnz, false);
@@ -257,20 +265,35 @@ int gs_row_slice_csc_compact(const int64_t* indptr, const int64_t* indices, int6
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(blocks_for(nnz, kTile));
-  if (coo_col)
-    hipLaunchKernelGGL((csc_compact_kernel<true>), grid, dim3(kThreads), 0, st, indptr, num_cols,
-                       nnz, s.val, s.prefix, out_indices, select_index, coo_col);
-  else
-    hipLaunchKernelGGL((csc_compact_kernel<false>), grid, dim3(kThreads), 0, st, indptr, num_cols,
-                       nnz, s.val, s.prefix, out_indices, select_index, coo_col);
+  if (id_bytes == 8) {
+    int64_t* oi = static_cast<int64_t*>(out_indices);
+    int64_t* cc = static_cast<int64_t*>(coo_col);
+    if (coo_col)
+      hipLaunchKernelGGL((csc_compact_kernel<true, int64_t>), grid, dim3(kThreads), 0, st, indptr,
+                         num_cols, nnz, s.val, s.prefix, oi, select_index, cc);
+    else
+      hipLaunchKernelGGL((csc_compact_kernel<false, int64_t>), grid, dim3(kThreads), 0, st, indptr,
+                         num_cols, nnz, s.val, s.prefix, oi, select_index, cc);
+  } else {
+    int32_t* oi = static_cast<int32_t*>(out_indices);
+    int32_t* cc = static_cast<int32_t*>(coo_col);
+    if (coo_col)
+      hipLaunchKernelGGL((csc_compact_kernel<true, int32_t>), grid, dim3(kThreads), 0, st, indptr,
+                         num_cols, nnz, s.val, s.prefix, oi, select_index, cc);
+    else
+      hipLaunchKernelGGL((csc_compact_kernel<false, int32_t>), grid, dim3(kThreads), 0, st, indptr,
+                         num_cols, nnz, s.val, s.prefix, oi, select_index, cc);
+  }
   return check_launch("row_slice_csc_compact");
 }
 
-int gs_row_slice_coo_mark(const int64_t* key, int64_t E, const int64_t* ids, int64_t num_ids,
-                          int64_t* num_kept, void* workspace, size_t workspace_bytes,
-                          void* stream) {
+int gs_row_slice_coo_mark(const void* key, int id_bytes, int64_t E, const void* ids,
+                          int64_t num_ids, int64_t* num_kept, void* workspace,
+                          size_t workspace_bytes, void* stream) {
   GS_REQUIRE(E >= 0 && num_ids >= 0 && num_kept, "gs_row_slice_coo_mark: bad argument");
   GS_REQUIRE((E == 0 || key) && (num_ids == 0 || ids), "gs_row_slice_coo_mark: null pointer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_row_slice_coo_mark: id_bytes must be 4 or 8, got %d",
+             id_bytes);
   Scratch s = carve(workspace, workspace_bytes, num_ids, E, true);
   if (!s.ok) {
     set_error_text("gs_row_slice_coo_mark: workspace needs %zu bytes, 256-byte aligned",
@@ -278,16 +301,19 @@ int gs_row_slice_coo_mark(const int64_t* key, int64_t E, const int64_t* ids, int
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  GS_RETURN_IF_ERROR(mark_common("row_slice_coo_mark", key, E, ids, num_ids, s, st));
+  GS_RETURN_IF_ERROR(id_bytes == 8
+                         ? mark_common<int64_t>("row_slice_coo_mark", key, E, ids, num_ids, s, st)
+                         : mark_common<int32_t>("row_slice_coo_mark", key, E, ids, num_ids, s, st));
   hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(64), 0, st, s.prefix, E, num_kept);
   return check_launch("row_slice_coo_mark");
 }
 
-int gs_row_slice_coo_compact(const int64_t* key, const int64_t* other, int64_t E,
-                             int64_t* out_key, int64_t* out_other, int64_t* select_index,
-                             void* workspace, size_t workspace_bytes, void* stream) {
-  (void)key;
+int gs_row_slice_coo_compact(const void* other, int id_bytes, int64_t E, void* out_key,
+                             void* out_other, int64_t* select_index, void* workspace,
+                             size_t workspace_bytes, void* stream) {
   GS_REQUIRE(E >= 0, "gs_row_slice_coo_compact: negative size");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_row_slice_coo_compact: id_bytes must be 4 or 8, got %d",
+             id_bytes);
   if (E == 0) return GS_OK;
   GS_REQUIRE(other && out_key && out_other && select_index, "gs_row_slice_coo_compact: null pointer");
   Scratch s = carve(workspace, workspace_bytes, 0, E, false);
@@ -295,9 +321,18 @@ int gs_row_slice_coo_compact(const int64_t* key, const int64_t* other, int64_t E
     set_error_text("gs_row_slice_coo_compact: pass the workspace given to gs_row_slice_coo_mark");
     return GS_ERR_WORKSPACE;
   }
-  hipLaunchKernelGGL(coo_compact_kernel, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0,
-                     static_cast<hipStream_t>(stream), other, E, s.val, s.prefix, out_key,
-                     out_other, select_index);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid(blocks_for(E, kThreads));
+  if (id_bytes == 8)
+    hipLaunchKernelGGL(coo_compact_kernel<int64_t>, grid, dim3(kThreads), 0, st,
+                       static_cast<const int64_t*>(other), E, s.val, s.prefix,
+                       static_cast<int64_t*>(out_key), static_cast<int64_t*>(out_other),
+                       select_index);
+  else
+    hipLaunchKernelGGL(coo_compact_kernel<int32_t>, grid, dim3(kThreads), 0, st,
+                       static_cast<const int32_t*>(other), E, s.val, s.prefix,
+                       static_cast<int32_t*>(out_key), static_cast<int32_t*>(out_other),
+                       select_index);
   return check_launch("row_slice_coo_compact");
 }
 

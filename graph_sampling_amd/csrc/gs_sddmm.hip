@@ -38,14 +38,15 @@ __device__ __forceinline__ int64_t select3(int target, int64_t src, int64_t eid,
   return target == 0 ? src : (target == 1 ? eid : dst);
 }
 
+template <typename IdT>
 struct SddmmArgs {
   const float* lhs;
   const float* rhs;
   float* out;
-  const int64_t* row;      // COO: row ids; CSC: indices
-  const int64_t* col;      // COO: col ids; CSC: nullptr
+  const IdT* row;          // COO: row ids; CSC: indices
+  const IdT* col;          // COO: col ids; CSC: nullptr
   const int64_t* indptr;   // CSC only
-  const int64_t* nid_map;  // CSC only, optional
+  const IdT* nid_map;      // CSC only, optional
   const int64_t* e_ids;    // optional
   int64_t num_cols;        // CSC only
   int64_t E;
@@ -55,9 +56,10 @@ struct SddmmArgs {
   int lhs_target, rhs_target;
 };
 
-__device__ __forceinline__ void edge_endpoints(const SddmmArgs& a, int64_t e, int64_t* src,
+template <typename IdT>
+__device__ __forceinline__ void edge_endpoints(const SddmmArgs<IdT>& a, int64_t e, int64_t* src,
                                                int64_t* dst, int64_t* eid) {
-  *src = a.row[e];
+  *src = static_cast<int64_t>(a.row[e]);
   if (a.indptr) {
     // last column c with indptr[c] <= e
     int64_t lo = 0, hi = a.num_cols + 1;
@@ -68,16 +70,16 @@ __device__ __forceinline__ void edge_endpoints(const SddmmArgs& a, int64_t e, in
     int64_t c = lo - 1;
     if (c >= a.num_cols) c = a.num_cols - 1;  // offsets that do not cover every edge
     if (c < 0) c = 0;
-    *dst = a.nid_map ? a.nid_map[c] : c;
+    *dst = a.nid_map ? static_cast<int64_t>(a.nid_map[c]) : c;
   } else {
-    *dst = a.col[e];
+    *dst = static_cast<int64_t>(a.col[e]);
   }
   *eid = a.e_ids ? a.e_ids[e] : e;
 }
 
 // blockDim = (tx, 256/tx): tx walks the out_len positions of an edge
-template <int OP>
-__global__ void __launch_bounds__(kThreads) sddmm_generic_kernel(SddmmArgs a) {
+template <int OP, typename IdT>
+__global__ void __launch_bounds__(kThreads) sddmm_generic_kernel(SddmmArgs<IdT> a) {
   const int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.y + threadIdx.y;
   if (e >= a.E) return;
   int64_t src, dst, eid;
@@ -96,7 +98,8 @@ __global__ void __launch_bounds__(kThreads) sddmm_generic_kernel(SddmmArgs a) {
 
 // dot, no broadcast, out_len == 1, R % 4 == 0 and 16-byte aligned rows.
 constexpr int kDotGroup = 16;
-__global__ void __launch_bounds__(kThreads) sddmm_dot_rows_kernel(SddmmArgs a) {
+template <typename IdT>
+__global__ void __launch_bounds__(kThreads) sddmm_dot_rows_kernel(SddmmArgs<IdT> a) {
   const int lane = threadIdx.x % kDotGroup;
   const int64_t e = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) / kDotGroup;
   if (e >= a.E) return;
@@ -117,16 +120,17 @@ __global__ void __launch_bounds__(kThreads) sddmm_dot_rows_kernel(SddmmArgs a) {
   if (lane == 0) a.out[eid] = acc;
 }
 
-template <int OP>
-void launch_generic(const SddmmArgs& a, hipStream_t st) {
+template <int OP, typename IdT>
+void launch_generic(const SddmmArgs<IdT>& a, hipStream_t st) {
   int tx = 1;
   while (tx < a.out_len && tx < kThreads) tx <<= 1;
   const int ty = kThreads / tx;
   const unsigned grid = static_cast<unsigned>((a.E + ty - 1) / ty);
-  hipLaunchKernelGGL((sddmm_generic_kernel<OP>), dim3(grid), dim3(tx, ty), 0, st, a);
+  hipLaunchKernelGGL((sddmm_generic_kernel<OP, IdT>), dim3(grid), dim3(tx, ty), 0, st, a);
 }
 
-int sddmm_dispatch(int op, const SddmmArgs& a, hipStream_t st) {
+template <typename IdT>
+int sddmm_dispatch(int op, const SddmmArgs<IdT>& a, hipStream_t st) {
   if (a.E == 0 || a.out_len == 0) return GS_OK;
   const bool aligned = (reinterpret_cast<uintptr_t>(a.lhs) % 16 == 0) &&
                        (reinterpret_cast<uintptr_t>(a.rhs) % 16 == 0) && a.lhs_len % 4 == 0 &&
@@ -135,17 +139,17 @@ int sddmm_dispatch(int op, const SddmmArgs& a, hipStream_t st) {
       aligned) {
     const unsigned grid = static_cast<unsigned>((a.E * kDotGroup + kThreads - 1) / kThreads);
     ProfileScope prof("sddmm_dot", st);
-    hipLaunchKernelGGL(sddmm_dot_rows_kernel, dim3(grid), dim3(kThreads), 0, st, a);
+    hipLaunchKernelGGL(sddmm_dot_rows_kernel<IdT>, dim3(grid), dim3(kThreads), 0, st, a);
     return check_launch("sddmm_dot");
   }
   switch (op) {
-    case GS_OP_ADD: launch_generic<GS_OP_ADD>(a, st); break;
-    case GS_OP_SUB: launch_generic<GS_OP_SUB>(a, st); break;
-    case GS_OP_MUL: launch_generic<GS_OP_MUL>(a, st); break;
-    case GS_OP_DIV: launch_generic<GS_OP_DIV>(a, st); break;
-    case GS_OP_COPY_LHS: launch_generic<GS_OP_COPY_LHS>(a, st); break;
-    case GS_OP_COPY_RHS: launch_generic<GS_OP_COPY_RHS>(a, st); break;
-    case GS_OP_DOT: launch_generic<GS_OP_DOT>(a, st); break;
+    case GS_OP_ADD: launch_generic<GS_OP_ADD, IdT>(a, st); break;
+    case GS_OP_SUB: launch_generic<GS_OP_SUB, IdT>(a, st); break;
+    case GS_OP_MUL: launch_generic<GS_OP_MUL, IdT>(a, st); break;
+    case GS_OP_DIV: launch_generic<GS_OP_DIV, IdT>(a, st); break;
+    case GS_OP_COPY_LHS: launch_generic<GS_OP_COPY_LHS, IdT>(a, st); break;
+    case GS_OP_COPY_RHS: launch_generic<GS_OP_COPY_RHS, IdT>(a, st); break;
+    case GS_OP_DOT: launch_generic<GS_OP_DOT, IdT>(a, st); break;
     default:
       set_error_text("Unsupported SpMM/SDDMM binary operator: %d", op);  // macro.h:30
       return GS_ERR_UNSUPPORTED;
@@ -173,29 +177,47 @@ using namespace gs;
 
 extern "C" {
 
-int gs_sddmm_coo(int op, const int64_t* row, const int64_t* col, const int64_t* e_ids, int64_t E,
-                 const float* lhs, const float* rhs, float* out, int lhs_target, int rhs_target,
-                 int64_t lhs_len, int64_t rhs_len, int64_t out_len, int64_t reduce_size,
-                 const int64_t* lhs_off, const int64_t* rhs_off, void* stream) {
+int gs_sddmm_coo(int op, const void* row, const void* col, int id_bytes, const int64_t* e_ids,
+                 int64_t E, const float* lhs, const float* rhs, float* out, int lhs_target,
+                 int rhs_target, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
+                 int64_t reduce_size, const int64_t* lhs_off, const int64_t* rhs_off, void* stream) {
   GS_RETURN_IF_ERROR(check_common("gs_sddmm_coo", op, E, lhs, rhs, out, lhs_target, rhs_target,
                                   lhs_len, rhs_len, out_len, reduce_size));
   GS_REQUIRE(E == 0 || (row && col), "gs_sddmm_coo: null row/col");
-  SddmmArgs a{lhs, rhs, out, row, col, nullptr, nullptr, e_ids, 0, E, lhs_len, rhs_len, out_len,
-              reduce_size, lhs_off, rhs_off, lhs_target, rhs_target};
-  return sddmm_dispatch(op, a, static_cast<hipStream_t>(stream));
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sddmm_coo: id_bytes must be 4 or 8, got %d", id_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (id_bytes == 8) {
+    SddmmArgs<int64_t> a{lhs, rhs, out, static_cast<const int64_t*>(row),
+                         static_cast<const int64_t*>(col), nullptr, nullptr, e_ids, 0, E, lhs_len,
+                         rhs_len, out_len, reduce_size, lhs_off, rhs_off, lhs_target, rhs_target};
+    return sddmm_dispatch(op, a, st);
+  }
+  SddmmArgs<int32_t> a{lhs, rhs, out, static_cast<const int32_t*>(row),
+                       static_cast<const int32_t*>(col), nullptr, nullptr, e_ids, 0, E, lhs_len,
+                       rhs_len, out_len, reduce_size, lhs_off, rhs_off, lhs_target, rhs_target};
+  return sddmm_dispatch(op, a, st);
 }
 
-int gs_sddmm_csc(int op, const int64_t* indptr, const int64_t* indices, const int64_t* e_ids,
-                 const int64_t* nid_map, int64_t num_cols, int64_t E, const float* lhs,
-                 const float* rhs, float* out, int lhs_target, int rhs_target, int64_t lhs_len,
-                 int64_t rhs_len, int64_t out_len, int64_t reduce_size, const int64_t* lhs_off,
-                 const int64_t* rhs_off, void* stream) {
+int gs_sddmm_csc(int op, const int64_t* indptr, const void* indices, int id_bytes,
+                 const int64_t* e_ids, const void* nid_map, int64_t num_cols, int64_t E,
+                 const float* lhs, const float* rhs, float* out, int lhs_target, int rhs_target,
+                 int64_t lhs_len, int64_t rhs_len, int64_t out_len, int64_t reduce_size,
+                 const int64_t* lhs_off, const int64_t* rhs_off, void* stream) {
   GS_RETURN_IF_ERROR(check_common("gs_sddmm_csc", op, E, lhs, rhs, out, lhs_target, rhs_target,
                                   lhs_len, rhs_len, out_len, reduce_size));
   GS_REQUIRE(num_cols >= 0 && (E == 0 || (indptr && indices)), "gs_sddmm_csc: null indptr/indices");
-  SddmmArgs a{lhs, rhs, out, indices, nullptr, indptr, nid_map, e_ids, num_cols, E, lhs_len,
-              rhs_len, out_len, reduce_size, lhs_off, rhs_off, lhs_target, rhs_target};
-  return sddmm_dispatch(op, a, static_cast<hipStream_t>(stream));
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_sddmm_csc: id_bytes must be 4 or 8, got %d", id_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (id_bytes == 8) {
+    SddmmArgs<int64_t> a{lhs, rhs, out, static_cast<const int64_t*>(indices), nullptr, indptr,
+                         static_cast<const int64_t*>(nid_map), e_ids, num_cols, E, lhs_len, rhs_len,
+                         out_len, reduce_size, lhs_off, rhs_off, lhs_target, rhs_target};
+    return sddmm_dispatch(op, a, st);
+  }
+  SddmmArgs<int32_t> a{lhs, rhs, out, static_cast<const int32_t*>(indices), nullptr, indptr,
+                       static_cast<const int32_t*>(nid_map), e_ids, num_cols, E, lhs_len, rhs_len,
+                       out_len, reduce_size, lhs_off, rhs_off, lhs_target, rhs_target};
+  return sddmm_dispatch(op, a, st);
 }
 
 }  // extern "C"

@@ -36,10 +36,10 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // NORMALIZE = false: out[nmap ? nmap[s] : s] = sum f(data[d])
 // NORMALIZE = true : out[d] = data[d] / sum data[d],  d = emap ? emap[e] : e
-template <bool NORMALIZE>
+template <bool NORMALIZE, typename IdT>
 __global__ void __launch_bounds__(kThreads)
 segment_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ emap,
-               const int64_t* __restrict__ nmap, const float* __restrict__ data, int64_t num_seg,
+               const IdT* __restrict__ nmap, const float* __restrict__ data, int64_t num_seg,
                int powk, float* __restrict__ out) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t s = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
@@ -80,13 +80,14 @@ segment_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ e
       }
     }
   } else {
-    out[nmap ? nmap[s] : s] = acc;
+    out[nmap ? static_cast<int64_t>(nmap[s]) : s] = acc;
   }
 }
 
 // out[target[e]] += f(data[emap ? emap[e] : e])   (graph_ops.cu:45-64)
+template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
-coo_sum_kernel(const int64_t* __restrict__ target, const int64_t* __restrict__ emap,
+coo_sum_kernel(const IdT* __restrict__ target, const int64_t* __restrict__ emap,
                const float* __restrict__ data, int64_t E, int powk, float* __restrict__ out) {
   const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (e >= E) return;
@@ -94,8 +95,9 @@ coo_sum_kernel(const int64_t* __restrict__ target, const int64_t* __restrict__ e
 }
 
 // edge_map_reduce.cu:15-23
+template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
-e_div_u_sum_kernel(const int64_t* __restrict__ row, const int64_t* __restrict__ col,
+e_div_u_sum_kernel(const IdT* __restrict__ row, const IdT* __restrict__ col,
                    const float* __restrict__ data, const float* __restrict__ divisor, int64_t E,
                    float* __restrict__ out_data, float* __restrict__ out_sum) {
   const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
@@ -112,26 +114,43 @@ using namespace gs;
 
 extern "C" {
 
-int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const int64_t* n_ids,
+int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const void* n_ids, int id_bytes,
                    const float* data, int64_t num_segments, int64_t powk, float* out,
                    void* stream) {
   GS_REQUIRE(num_segments >= 0 && powk >= 1, "gs_segment_sum: negative size or powk < 1");
   GS_REQUIRE(num_segments == 0 || (indptr && data && out), "gs_segment_sum: null pointer");
+  GS_REQUIRE(!n_ids || valid_id_bytes(id_bytes), "gs_segment_sum: id_bytes must be 4 or 8, got %d",
+             id_bytes);
   if (num_segments == 0) return GS_OK;
-  hipLaunchKernelGGL((segment_kernel<false>), dim3(blocks_for(num_segments, kThreads)),
-                     dim3(kThreads), 0, static_cast<hipStream_t>(stream), indptr, e_ids, n_ids,
-                     data, num_segments, static_cast<int>(powk), out);
+  const dim3 grid(blocks_for(num_segments, kThreads));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (n_ids && id_bytes == 4)
+    hipLaunchKernelGGL((segment_kernel<false, int32_t>), grid, dim3(kThreads), 0, st, indptr, e_ids,
+                       static_cast<const int32_t*>(n_ids), data, num_segments,
+                       static_cast<int>(powk), out);
+  else
+    hipLaunchKernelGGL((segment_kernel<false, int64_t>), grid, dim3(kThreads), 0, st, indptr, e_ids,
+                       static_cast<const int64_t*>(n_ids), data, num_segments,
+                       static_cast<int>(powk), out);
   return check_launch("segment_sum");
 }
 
-int gs_coo_sum(const int64_t* target, const int64_t* e_ids, const float* data, int64_t E,
+int gs_coo_sum(const void* target, int id_bytes, const int64_t* e_ids, const float* data, int64_t E,
                int64_t powk, float* out, void* stream) {
   GS_REQUIRE(E >= 0 && powk >= 1, "gs_coo_sum: negative size or powk < 1");
   GS_REQUIRE(E == 0 || (target && data && out), "gs_coo_sum: null pointer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_coo_sum: id_bytes must be 4 or 8, got %d", id_bytes);
   if (E == 0) return GS_OK;
-  hipLaunchKernelGGL(coo_sum_kernel, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0,
-                     static_cast<hipStream_t>(stream), target, e_ids, data, E,
-                     static_cast<int>(powk), out);
+  const dim3 grid(blocks_for(E, kThreads));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (id_bytes == 8)
+    hipLaunchKernelGGL(coo_sum_kernel<int64_t>, grid, dim3(kThreads), 0, st,
+                       static_cast<const int64_t*>(target), e_ids, data, E, static_cast<int>(powk),
+                       out);
+  else
+    hipLaunchKernelGGL(coo_sum_kernel<int32_t>, grid, dim3(kThreads), 0, st,
+                       static_cast<const int32_t*>(target), e_ids, data, E, static_cast<int>(powk),
+                       out);
   return check_launch("coo_sum");
 }
 
@@ -140,22 +159,30 @@ int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const floa
   GS_REQUIRE(num_segments >= 0, "gs_segment_normalize: negative size");
   GS_REQUIRE(num_segments == 0 || (indptr && data && out), "gs_segment_normalize: null pointer");
   if (num_segments == 0) return GS_OK;
-  hipLaunchKernelGGL((segment_kernel<true>), dim3(blocks_for(num_segments, kThreads)),
+  hipLaunchKernelGGL((segment_kernel<true, int64_t>), dim3(blocks_for(num_segments, kThreads)),
                      dim3(kThreads), 0, static_cast<hipStream_t>(stream), indptr, e_ids,
                      static_cast<const int64_t*>(nullptr), data, num_segments, 1, out);
   return check_launch("segment_normalize");
 }
 
-int gs_e_div_u_sum(const int64_t* row, const int64_t* col, const float* data,
+int gs_e_div_u_sum(const void* row, const void* col, int id_bytes, const float* data,
                    const float* divisor, int64_t E, float* out_data, float* out_sum,
                    void* stream) {
   GS_REQUIRE(E >= 0, "gs_e_div_u_sum: negative size");
   GS_REQUIRE(E == 0 || (row && col && data && divisor && out_data && out_sum),
              "gs_e_div_u_sum: null pointer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_e_div_u_sum: id_bytes must be 4 or 8, got %d", id_bytes);
   if (E == 0) return GS_OK;
-  hipLaunchKernelGGL(e_div_u_sum_kernel, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0,
-                     static_cast<hipStream_t>(stream), row, col, data, divisor, E, out_data,
-                     out_sum);
+  const dim3 grid(blocks_for(E, kThreads));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (id_bytes == 8)
+    hipLaunchKernelGGL(e_div_u_sum_kernel<int64_t>, grid, dim3(kThreads), 0, st,
+                       static_cast<const int64_t*>(row), static_cast<const int64_t*>(col), data,
+                       divisor, E, out_data, out_sum);
+  else
+    hipLaunchKernelGGL(e_div_u_sum_kernel<int32_t>, grid, dim3(kThreads), 0, st,
+                       static_cast<const int32_t*>(row), static_cast<const int32_t*>(col), data,
+                       divisor, E, out_data, out_sum);
   return check_launch("e_div_u_sum");
 }
 

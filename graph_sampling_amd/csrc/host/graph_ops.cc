@@ -110,7 +110,7 @@ void COOGraphDiv(std::shared_ptr<COO> coo, torch::Tensor data, torch::Tensor div
 
 std::shared_ptr<COO> GraphCSC2COO(std::shared_ptr<CSC> csc, bool CSC2COO) {
   auto coo = std::make_shared<COO>();
-  torch::Tensor expanded = hip::Csc2CooCols(csc->indptr, csc->indices.numel());
+  torch::Tensor expanded = hip::Csc2CooCols(csc->indptr, csc->indices.numel(), csc->indices);
   if (CSC2COO) {
     coo->row = csc->indices;
     coo->col = expanded;

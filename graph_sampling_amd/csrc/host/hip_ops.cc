@@ -56,6 +56,13 @@ const int64_t* OptI64(const torch::optional<torch::Tensor>& t, const char* name)
   return t.value().data_ptr<int64_t>();
 }
 
+// optional node-id tensor of the width `idb`
+const void* OptIds(const torch::optional<torch::Tensor>& t, int idb, const char* name) {
+  if (!t.has_value() || !t.value().defined()) return nullptr;
+  TORCH_CHECK(IdBytes(t.value(), name) == idb, name, " must have the dtype of the graph ids");
+  return t.value().data_ptr();
+}
+
 torch::Tensor Scratch(size_t bytes, const torch::Tensor& like) {
   return torch::empty({static_cast<int64_t>(bytes < 256 ? 256 : bytes)},
                       torch::dtype(torch::kUInt8).device(like.device()));
@@ -457,12 +464,12 @@ void SddmmCoo(const std::string& op, const Bcast& b, const torch::Tensor& row,
               const torch::Tensor& lhs, const torch::Tensor& rhs, torch::Tensor out, int lhs_target,
               int rhs_target) {
   const int code = OpCode(op);
-  NeedI64(row, "coo row");
-  NeedI64(col, "coo col");
+  const int idb = IdBytes(row, "coo row");
+  TORCH_CHECK(IdBytes(col, "coo col") == idb, "coo row and col differ in dtype");
   NeedF32(out, "out");
   if (code != GS_OP_COPY_RHS) NeedF32(lhs, "lhs");
   if (code != GS_OP_COPY_LHS) NeedF32(rhs, "rhs");
-  Check(gs_sddmm_coo(code, row.data_ptr<int64_t>(), col.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"),
+  Check(gs_sddmm_coo(code, row.data_ptr(), col.data_ptr(), idb, OptI64(e_ids, "e_ids"),
                      row.numel(), lhs.defined() ? lhs.data_ptr<float>() : nullptr,
                      rhs.defined() ? rhs.data_ptr<float>() : nullptr, out.data_ptr<float>(),
                      lhs_target, rhs_target, b.lhs_len, b.rhs_len, b.out_len, b.reduce_size,
@@ -477,12 +484,12 @@ void SddmmCsc(const std::string& op, const Bcast& b, const torch::Tensor& indptr
               const torch::Tensor& rhs, torch::Tensor out, int lhs_target, int rhs_target) {
   const int code = OpCode(op);
   NeedI64(indptr, "indptr");
-  NeedI64(indices, "indices");
+  const int idb = IdBytes(indices, "indices");
   NeedF32(out, "out");
   if (code != GS_OP_COPY_RHS) NeedF32(lhs, "lhs");
   if (code != GS_OP_COPY_LHS) NeedF32(rhs, "rhs");
-  Check(gs_sddmm_csc(code, indptr.data_ptr<int64_t>(), indices.data_ptr<int64_t>(),
-                     OptI64(e_ids, "e_ids"), OptI64(nid_map, "valid ids"), indptr.numel() - 1,
+  Check(gs_sddmm_csc(code, indptr.data_ptr<int64_t>(), indices.data_ptr(), idb,
+                     OptI64(e_ids, "e_ids"), OptIds(nid_map, idb, "valid ids"), indptr.numel() - 1,
                      indices.numel(), lhs.defined() ? lhs.data_ptr<float>() : nullptr,
                      rhs.defined() ? rhs.data_ptr<float>() : nullptr, out.data_ptr<float>(),
                      lhs_target, rhs_target, b.lhs_len, b.rhs_len, b.out_len, b.reduce_size,
@@ -497,18 +504,19 @@ void SegmentSum(const torch::Tensor& indptr, const torch::optional<torch::Tensor
   NeedI64(indptr, "indptr");
   NeedF32(data, "data");
   NeedF32(out, "out");
-  Check(gs_segment_sum(indptr.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"), OptI64(n_ids, "valid ids"),
-                       data.data_ptr<float>(), indptr.numel() - 1, powk, out.data_ptr<float>(),
+  const int idb = n_ids.has_value() && n_ids.value().defined() ? IdBytes(n_ids.value(), "valid ids") : 8;
+  Check(gs_segment_sum(indptr.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"),
+                       OptIds(n_ids, idb, "valid ids"), idb, data.data_ptr<float>(), indptr.numel() - 1, powk, out.data_ptr<float>(),
                        Stream(indptr)),
         "gs_segment_sum");
 }
 
 void CooSum(const torch::Tensor& target, const torch::optional<torch::Tensor>& e_ids,
             const torch::Tensor& data, torch::Tensor out, int64_t powk) {
-  NeedI64(target, "coo target");
+  const int idb = IdBytes(target, "coo target");
   NeedF32(data, "data");
   NeedF32(out, "out");
-  Check(gs_coo_sum(target.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"), data.data_ptr<float>(),
+  Check(gs_coo_sum(target.data_ptr(), idb, OptI64(e_ids, "e_ids"), data.data_ptr<float>(),
                    target.numel(), powk, out.data_ptr<float>(), Stream(target)),
         "gs_coo_sum");
 }
@@ -526,11 +534,11 @@ void SegmentNormalize(const torch::Tensor& indptr, const torch::optional<torch::
 
 void EDivUSum(const torch::Tensor& row, const torch::Tensor& col, const torch::Tensor& data,
               const torch::Tensor& divisor, torch::Tensor out_data, torch::Tensor out_sum) {
-  NeedI64(row, "coo row");
-  NeedI64(col, "coo col");
+  const int idb = IdBytes(row, "coo row");
+  TORCH_CHECK(IdBytes(col, "coo col") == idb, "coo row and col differ in dtype");
   NeedF32(data, "data");
   NeedF32(divisor, "divisor");
-  Check(gs_e_div_u_sum(row.data_ptr<int64_t>(), col.data_ptr<int64_t>(), data.data_ptr<float>(),
+  Check(gs_e_div_u_sum(row.data_ptr(), col.data_ptr(), idb, data.data_ptr<float>(),
                        divisor.data_ptr<float>(), row.numel(), out_data.data_ptr<float>(),
                        out_sum.data_ptr<float>(), Stream(row)),
         "gs_e_div_u_sum");
@@ -539,26 +547,25 @@ void EDivUSum(const torch::Tensor& row, const torch::Tensor& col, const torch::T
 SliceResult RowSlicingCsc(const torch::Tensor& indptr, const torch::Tensor& indices,
                           const torch::Tensor& row_ids, bool with_coo) {
   NeedI64(indptr, "indptr");
-  NeedI64(indices, "indices");
-  NeedI64(row_ids, "row ids");
+  const int idb = IdBytes(indices, "indices");
+  TORCH_CHECK(IdBytes(row_ids, "row ids") == idb, "row ids and indices differ in dtype");
   const int64_t ncols = indptr.numel() - 1, nnz = indices.numel(), nr = row_ids.numel();
   auto out_indptr = torch::empty({ncols + 1}, I64(indptr));
   auto ws = Scratch(gs_row_slice_workspace_bytes(nr, nnz, ncols), indptr);
   void* st = Stream(indptr);
-  Check(gs_row_slice_csc_mark(indptr.data_ptr<int64_t>(), indices.data_ptr<int64_t>(), ncols, nnz,
-                              row_ids.data_ptr<int64_t>(), nr, out_indptr.data_ptr<int64_t>(),
-                              ws.data_ptr(), ws.numel(), st),
+  Check(gs_row_slice_csc_mark(indptr.data_ptr<int64_t>(), indices.data_ptr(), idb, ncols, nnz,
+                              row_ids.data_ptr(), nr, out_indptr.data_ptr<int64_t>(), ws.data_ptr(),
+                              ws.numel(), st),
         "gs_row_slice_csc_mark");
   const int64_t kept = out_indptr[ncols].item<int64_t>();
-  auto out_indices = torch::empty({kept}, I64(indptr));
+  auto out_indices = torch::empty({kept}, indices.options());
   auto select_index = torch::empty({kept}, I64(indptr));
   torch::Tensor coo_col;
-  if (with_coo) coo_col = torch::empty({kept}, I64(indptr));
+  if (with_coo) coo_col = torch::empty({kept}, indices.options());
   if (kept > 0)
-    Check(gs_row_slice_csc_compact(indptr.data_ptr<int64_t>(), indices.data_ptr<int64_t>(), ncols,
-                                   nnz, out_indptr.data_ptr<int64_t>(),
-                                   out_indices.data_ptr<int64_t>(), select_index.data_ptr<int64_t>(),
-                                   with_coo ? coo_col.data_ptr<int64_t>() : nullptr, ws.data_ptr(),
+    Check(gs_row_slice_csc_compact(indptr.data_ptr<int64_t>(), ncols, nnz, idb,
+                                   out_indices.data_ptr(), select_index.data_ptr<int64_t>(),
+                                   with_coo ? coo_col.data_ptr() : nullptr, ws.data_ptr(),
                                    ws.numel(), st),
           "gs_row_slice_csc_compact");
   return {out_indptr, coo_col, out_indices, select_index};
@@ -567,32 +574,33 @@ SliceResult RowSlicingCsc(const torch::Tensor& indptr, const torch::Tensor& indi
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(const torch::Tensor& key,
                                                                       const torch::Tensor& other,
                                                                       const torch::Tensor& ids) {
-  NeedI64(key, "coo ids");
-  NeedI64(other, "coo ids");
-  NeedI64(ids, "node ids");
+  const int idb = IdBytes(key, "coo ids");
+  TORCH_CHECK(IdBytes(other, "coo ids") == idb && IdBytes(ids, "node ids") == idb,
+              "coo ids and node ids differ in dtype");
   const int64_t E = key.numel(), n = ids.numel();
   auto num = torch::empty({1}, I64(key));
   auto ws = Scratch(gs_row_slice_workspace_bytes(n, E, 0), key);
   void* st = Stream(key);
-  Check(gs_row_slice_coo_mark(key.data_ptr<int64_t>(), E, ids.data_ptr<int64_t>(), n,
-                              num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
+  Check(gs_row_slice_coo_mark(key.data_ptr(), idb, E, ids.data_ptr(), n, num.data_ptr<int64_t>(),
+                              ws.data_ptr(), ws.numel(), st),
         "gs_row_slice_coo_mark");
   const int64_t kept = num.item<int64_t>();
-  auto out_key = torch::empty({kept}, I64(key));
-  auto out_other = torch::empty({kept}, I64(key));
+  auto out_key = torch::empty({kept}, key.options());
+  auto out_other = torch::empty({kept}, key.options());
   auto select_index = torch::empty({kept}, I64(key));
   if (kept > 0)
-    Check(gs_row_slice_coo_compact(key.data_ptr<int64_t>(), other.data_ptr<int64_t>(), E,
-                                   out_key.data_ptr<int64_t>(), out_other.data_ptr<int64_t>(),
-                                   select_index.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
+    Check(gs_row_slice_coo_compact(other.data_ptr(), idb, E, out_key.data_ptr(),
+                                   out_other.data_ptr(), select_index.data_ptr<int64_t>(),
+                                   ws.data_ptr(), ws.numel(), st),
           "gs_row_slice_coo_compact");
   return {out_key, out_other, select_index};
 }
 
-torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz) {
+torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz, const torch::Tensor& ids_like) {
   NeedI64(indptr, "indptr");
-  auto col = torch::empty({nnz}, I64(indptr));
-  Check(gs_csc2coo(indptr.data_ptr<int64_t>(), indptr.numel() - 1, nnz, col.data_ptr<int64_t>(),
+  const int idb = IdBytes(ids_like, "indices");
+  auto col = torch::empty({nnz}, ids_like.options());
+  Check(gs_csc2coo(indptr.data_ptr<int64_t>(), indptr.numel() - 1, nnz, col.data_ptr(), idb,
                    Stream(indptr)),
         "gs_csc2coo");
   return col;
@@ -600,22 +608,22 @@ torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz) {
 
 std::tuple<torch::Tensor, torch::Tensor, torch::optional<torch::Tensor>> Coo2Csc(
     const torch::Tensor& key, const torch::Tensor& value, int64_t num_keys, bool sorted) {
-  NeedI64(key, "coo key");
-  NeedI64(value, "coo value");
+  const int idb = IdBytes(key, "coo key");
+  TORCH_CHECK(IdBytes(value, "coo value") == idb, "coo key and value differ in dtype");
   const int64_t E = key.numel();
   auto indptr = torch::empty({num_keys + 1}, I64(key));
   if (sorted) {
-    Check(gs_coo2csc(key.data_ptr<int64_t>(), value.data_ptr<int64_t>(), E, num_keys, 1,
+    Check(gs_coo2csc(key.data_ptr(), value.data_ptr(), idb, E, num_keys, 1,
                      indptr.data_ptr<int64_t>(), nullptr, nullptr, nullptr, 0, Stream(key)),
           "gs_coo2csc");
     return {indptr, value, torch::nullopt};
   }
-  auto out_value = torch::empty({E}, I64(key));
+  auto out_value = torch::empty({E}, value.options());
   auto perm = torch::empty({E}, I64(key));
   auto ws = Scratch(gs_coo2csc_workspace_bytes(E, num_keys), key);
-  Check(gs_coo2csc(key.data_ptr<int64_t>(), value.data_ptr<int64_t>(), E, num_keys, 0,
-                   indptr.data_ptr<int64_t>(), out_value.data_ptr<int64_t>(),
-                   perm.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), Stream(key)),
+  Check(gs_coo2csc(key.data_ptr(), value.data_ptr(), idb, E, num_keys, 0,
+                   indptr.data_ptr<int64_t>(), out_value.data_ptr(), perm.data_ptr<int64_t>(),
+                   ws.data_ptr(), ws.numel(), Stream(key)),
         "gs_coo2csc");
   return {indptr, out_value, perm};
 }

@@ -108,7 +108,8 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(const torc
                                                                       const torch::Tensor& other,
                                                                       const torch::Tensor& ids);
 
-torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz);
+// col[e] = column owning edge e, in the dtype of `ids_like`
+torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz, const torch::Tensor& ids_like);
 // {indptr, values in key order, sort permutation (nullopt when already sorted)}
 std::tuple<torch::Tensor, torch::Tensor, torch::optional<torch::Tensor>> Coo2Csc(
     const torch::Tensor& key, const torch::Tensor& value, int64_t num_keys, bool sorted);

@@ -292,33 +292,34 @@ int gs_metapath_walk(const int64_t* const* all_indptr, const void* const* all_in
 /* out[eid, k] = op(lhs[sel_l, lhs_off[k]], rhs[sel_r, rhs_off[k]]) with         */
 /* sel = src(0) / edge(1) / dst(2); dot reduces `reduce_size` trailing items.   */
 /* lhs_off / rhs_off: device int64[out_len] broadcast offsets or NULL           */
-/* (src/bcast.cc:24-75).  Ids are int64 here (id_bytes reserved).               */
+/* (src/bcast.cc:24-75).  row / col / indices / nid_map are id_bytes wide.      */
 /* ------------------------------------------------------------------------- */
-int gs_sddmm_coo(int op, const int64_t* row, const int64_t* col, const int64_t* e_ids, int64_t E,
+int gs_sddmm_coo(int op, const void* row, const void* col, int id_bytes, const int64_t* e_ids,
+                 int64_t E, const float* lhs, const float* rhs, float* out, int lhs_target,
+                 int rhs_target, int64_t lhs_len, int64_t rhs_len, int64_t out_len,
+                 int64_t reduce_size, const int64_t* lhs_off, const int64_t* rhs_off, void* stream);
+
+/* CSC flavour: src = indices[e], dst = column owning e (through nid_map when
+ * given, sddmm.cu:126-131). */
+int gs_sddmm_csc(int op, const int64_t* indptr, const void* indices, int id_bytes,
+                 const int64_t* e_ids, const void* nid_map, int64_t num_cols, int64_t E,
                  const float* lhs, const float* rhs, float* out, int lhs_target, int rhs_target,
                  int64_t lhs_len, int64_t rhs_len, int64_t out_len, int64_t reduce_size,
                  const int64_t* lhs_off, const int64_t* rhs_off, void* stream);
 
-/* CSC flavour: src = indices[e], dst = column owning e (through nid_map when
- * given, sddmm.cu:126-131). */
-int gs_sddmm_csc(int op, const int64_t* indptr, const int64_t* indices, const int64_t* e_ids,
-                 const int64_t* nid_map, int64_t num_cols, int64_t E, const float* lhs,
-                 const float* rhs, float* out, int lhs_target, int rhs_target, int64_t lhs_len,
-                 int64_t rhs_len, int64_t out_len, int64_t reduce_size, const int64_t* lhs_off,
-                 const int64_t* rhs_off, void* stream);
-
 /* ------------------------------------------------------------------------- */
 /* Segment ops: replace impl::CSCSumCUDA, COOSumCUDA, CSCNormalizeCUDA          */
 /* (src/cuda/graph_ops.cu:92,122,184) and impl::fusion::COOEDivUSum             */
-/* (src/cuda/fusion/edge_map_reduce.cu:10).                                    */
+/* (src/cuda/fusion/edge_map_reduce.cu:10).  Node ids (n_ids, target, row, col) */
+/* are id_bytes wide; e_ids are positions, always int64.                        */
 /* ------------------------------------------------------------------------- */
 /* out[n_ids ? n_ids[s] : s] = sum over segment s of data[e_ids ? e_ids[e] : e]^powk */
-int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const int64_t* n_ids,
+int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const void* n_ids, int id_bytes,
                    const float* data, int64_t num_segments, int64_t powk, float* out,
                    void* stream);
 
 /* out[target[e]] += data[e_ids ? e_ids[e] : e]^powk  (out pre-zeroed by caller) */
-int gs_coo_sum(const int64_t* target, const int64_t* e_ids, const float* data, int64_t E,
+int gs_coo_sum(const void* target, int id_bytes, const int64_t* e_ids, const float* data, int64_t E,
                int64_t powk, float* out, void* stream);
 
 /* out[d] = data[d] / sum of its segment, d = e_ids ? e_ids[e] : e */
@@ -326,7 +327,7 @@ int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const floa
                          int64_t num_segments, float* out, void* stream);
 
 /* out_data[e] = data[e] / divisor[row[e]]; out_sum[col[e]] += out_data[e] */
-int gs_e_div_u_sum(const int64_t* row, const int64_t* col, const float* data,
+int gs_e_div_u_sum(const void* row, const void* col, int id_bytes, const float* data,
                    const float* divisor, int64_t E, float* out_data, float* out_sum,
                    void* stream);
 
@@ -334,45 +335,48 @@ int gs_e_div_u_sum(const int64_t* row, const int64_t* col, const float* data,
 /* Row slicing: replaces impl::CSCRowSlicingCUDA and impl::COORowSlicingCUDA    */
 /* (src/cuda/slicing.cu:528,768).  Kept ids are relabelled to their position    */
 /* in row_ids.  Two phases: *_mark computes per-segment kept counts / a mask,   */
-/* the caller reads the total, *_compact writes the survivors in order.         */
+/* the caller reads the total, *_compact writes the survivors in order.  Ids    */
+/* in and out are id_bytes wide; select_index is int64.                         */
 /* ------------------------------------------------------------------------- */
 size_t gs_row_slice_workspace_bytes(int64_t num_row_ids, int64_t nnz, int64_t num_cols);
 
 /* out_indptr[0..num_cols] = exscan of kept edges per column; total in
  * out_indptr[num_cols]. */
-int gs_row_slice_csc_mark(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
-                          int64_t nnz, const int64_t* row_ids, int64_t num_row_ids,
+int gs_row_slice_csc_mark(const int64_t* indptr, const void* indices, int id_bytes,
+                          int64_t num_cols, int64_t nnz, const void* row_ids, int64_t num_row_ids,
                           int64_t* out_indptr, void* workspace, size_t workspace_bytes,
                           void* stream);
 
-int gs_row_slice_csc_compact(const int64_t* indptr, const int64_t* indices, int64_t num_cols,
-                             int64_t nnz, const int64_t* out_indptr, int64_t* out_indices,
-                             int64_t* select_index, int64_t* coo_col, void* workspace,
-                             size_t workspace_bytes, void* stream);
+/* the workspace is the one the mark call filled */
+int gs_row_slice_csc_compact(const int64_t* indptr, int64_t num_cols, int64_t nnz, int id_bytes,
+                             void* out_indices, int64_t* select_index, void* coo_col,
+                             void* workspace, size_t workspace_bytes, void* stream);
 
 /* COO: keep edges whose key[e] is in ids.  *num_kept (device scalar). */
-int gs_row_slice_coo_mark(const int64_t* key, int64_t E, const int64_t* ids, int64_t num_ids,
-                          int64_t* num_kept, void* workspace, size_t workspace_bytes,
-                          void* stream);
+int gs_row_slice_coo_mark(const void* key, int id_bytes, int64_t E, const void* ids,
+                          int64_t num_ids, int64_t* num_kept, void* workspace,
+                          size_t workspace_bytes, void* stream);
 
-int gs_row_slice_coo_compact(const int64_t* key, const int64_t* other, int64_t E,
-                             int64_t* out_key, int64_t* out_other, int64_t* select_index,
-                             void* workspace, size_t workspace_bytes, void* stream);
+int gs_row_slice_coo_compact(const void* other, int id_bytes, int64_t E, void* out_key,
+                             void* out_other, int64_t* select_index, void* workspace,
+                             size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Format conversion: replaces impl::CSC2COOCUDA and impl::COO2CSCCUDA          */
 /* (src/cuda/format_transform.cu:35,135).                                      */
 /* ------------------------------------------------------------------------- */
-/* col[e] = column owning edge e */
-int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, int64_t* col, void* stream);
+/* col[e] = column owning edge e (id_bytes wide) */
+int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, void* col, int id_bytes,
+               void* stream);
 
 size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys);
 
-/* Stable counting sort of (key -> value): indptr[num_keys+1], out_value[E],
- * perm[E] (= stable argsort of key; the reference's sort_index).  sorted != 0:
- * only indptr is computed (out_value / perm untouched, may be NULL). */
-int gs_coo2csc(const int64_t* key, const int64_t* value, int64_t E, int64_t num_keys, int sorted,
-               int64_t* indptr, int64_t* out_value, int64_t* perm, void* workspace,
+/* Stable counting sort of (key -> value), both id_bytes wide: indptr[num_keys+1],
+ * out_value[E], perm[E] (int64; = stable argsort of key, the reference's
+ * sort_index).  sorted != 0: only indptr is computed (out_value / perm
+ * untouched, may be NULL). */
+int gs_coo2csc(const void* key, const void* value, int id_bytes, int64_t E, int64_t num_keys,
+               int sorted, int64_t* indptr, void* out_value, int64_t* perm, void* workspace,
                size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus

@@ -1,12 +1,15 @@
 """GPU parity: format conversion and row slicing vs the CPU oracle and closed forms."""
 import numpy as np
 import pytest
+import torch
 
 from oracle import oracle as O
 from graph_sampling_amd import capi
 from tests.util import graph_12col_4edge, graph_20x5, rmat_csc_np, to_dev
 
 pytestmark = pytest.mark.gpu
+
+ID_DTYPES = [torch.int64, torch.int32]
 
 
 def test_csc2coo_reference_vector(dev):
@@ -16,10 +19,13 @@ def test_csc2coo_reference_vector(dev):
     assert np.array_equal(col, np.repeat(np.arange(20), 5))
 
 
+@pytest.mark.parametrize("idt", ID_DTYPES)
 @pytest.mark.parametrize("seed", [1, 2])
-def test_csc2coo_rmat(dev, seed):
+def test_csc2coo_rmat(dev, seed, idt):
     indptr, indices = rmat_csc_np(1 << 13, 1 << 17, seed=seed)
-    col = capi.csc2coo(to_dev(indptr, dev), indices.size).cpu().numpy()
+    col = capi.csc2coo(to_dev(indptr, dev), indices.size, idt)
+    assert col.dtype == idt
+    col = col.cpu().numpy()
     assert np.array_equal(col, np.repeat(np.arange(indptr.size - 1), np.diff(indptr)))
     assert np.array_equal(col, O.csc2coo(indptr, indices.size))
 
@@ -34,12 +40,14 @@ def test_coo2csc_reference_eids(dev):
     assert np.array_equal(perm.cpu().numpy(), [0, 2, 1, 3])
 
 
+@pytest.mark.parametrize("idt", ID_DTYPES)
 @pytest.mark.parametrize("num_keys,E", [(1, 50), (7, 1000), (1 << 12, 1 << 17), (300000, 50000), (2_450_000, 200000)])
-def test_coo2csc_unsorted_matches_stable_sort(dev, num_keys, E):
+def test_coo2csc_unsorted_matches_stable_sort(dev, num_keys, E, idt):
     rng = np.random.default_rng(E)
     key = rng.integers(0, num_keys, size=E).astype(np.int64)
-    value = rng.integers(0, 1 << 40, size=E).astype(np.int64)
-    ip, val, perm = capi.coo2csc(to_dev(key, dev), to_dev(value, dev), num_keys, False)
+    value = rng.integers(0, 1 << (40 if idt == torch.int64 else 31), size=E).astype(np.int64)
+    ip, val, perm = capi.coo2csc(to_dev(key, dev, idt), to_dev(value, dev, idt), num_keys, False)
+    assert val.dtype == idt and perm.dtype == torch.int64
     want_perm = np.argsort(key, kind="stable")
     assert np.array_equal(perm.cpu().numpy(), want_perm)
     assert np.array_equal(val.cpu().numpy(), value[want_perm])
@@ -49,10 +57,11 @@ def test_coo2csc_unsorted_matches_stable_sort(dev, num_keys, E):
     assert np.array_equal(o_ip, want_ip) and np.array_equal(o_perm, want_perm) and np.array_equal(o_val, value[want_perm])
 
 
-def test_coo2csc_sorted(dev):
+@pytest.mark.parametrize("idt", ID_DTYPES)
+def test_coo2csc_sorted(dev, idt):
     indptr, indices = rmat_csc_np(1 << 12, 1 << 15, seed=3)
     col = np.repeat(np.arange(indptr.size - 1), np.diff(indptr))
-    ip, val, perm = capi.coo2csc(to_dev(col, dev), to_dev(indices, dev), indptr.size - 1, True)
+    ip, val, perm = capi.coo2csc(to_dev(col, dev, idt), to_dev(indices, dev, idt), indptr.size - 1, True)
     assert perm is None
     assert np.array_equal(ip.cpu().numpy(), indptr)
     assert np.array_equal(val.cpu().numpy(), indices)
@@ -70,12 +79,15 @@ def test_row_slice_csc_reference_vector(dev):
         assert np.array_equal(g.cpu().numpy(), w)
 
 
+@pytest.mark.parametrize("idt", ID_DTYPES)
 @pytest.mark.parametrize("with_coo", [True, False])
 @pytest.mark.parametrize("n_rows", [0, 1, 512, 4000])
-def test_row_slice_csc_rmat(dev, with_coo, n_rows):
+def test_row_slice_csc_rmat(dev, with_coo, n_rows, idt):
     indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=4)
     rows = np.random.default_rng(n_rows).permutation(1 << 12)[:n_rows].astype(np.int64)
-    got = capi.row_slice_csc(to_dev(indptr, dev), to_dev(indices, dev), to_dev(rows, dev), with_coo)
+    got = capi.row_slice_csc(to_dev(indptr, dev), to_dev(indices, dev, idt), to_dev(rows, dev, idt),
+                             with_coo)
+    assert got[2].dtype == idt and got[3].dtype == torch.int64
     want = O.row_slice_csc(indptr, indices, rows, with_coo)
     for g, w in zip(got, want):
         if w is None:
@@ -90,11 +102,12 @@ def test_row_slice_csc_rmat(dev, with_coo, n_rows):
     assert np.array_equal(want[3], np.nonzero(mask)[0])
 
 
-def test_row_slice_coo(dev):
+@pytest.mark.parametrize("idt", ID_DTYPES)
+def test_row_slice_coo(dev, idt):
     indptr, indices = rmat_csc_np(1 << 12, 1 << 16, seed=5)
     col = np.repeat(np.arange(indptr.size - 1), np.diff(indptr))
     ids = np.random.default_rng(0).permutation(1 << 12)[:512].astype(np.int64)
-    got = capi.row_slice_coo(to_dev(indices, dev), to_dev(col, dev), to_dev(ids, dev))
+    got = capi.row_slice_coo(to_dev(indices, dev, idt), to_dev(col, dev, idt), to_dev(ids, dev, idt))
     want = O.row_slice_coo(indices, col, ids)
     for g, w in zip(got, want):
         assert np.array_equal(g.cpu().numpy(), w)

@@ -476,3 +476,90 @@ def test_errors_are_exceptions_not_aborts(dev):
         C._CAPI_Slicing(torch.arange(2, **I(dev)), 0, _CSC, _CSR, False)
     with pytest.raises(RuntimeError, match="No implementation"):
         C._CAPI_Sampling(1, 3, False, _CSC, _CSC)
+
+
+# ------------------------------------------------ deferred edge count (pending graphs)
+def _fused_child(dev, seed=5):
+    m, indptr, indices, _ = _rmat_matrix(dev, 12, 16, 9)
+    seeds = np.random.default_rng(seed).permutation(1 << 12)[:300].astype(np.int64)
+    gs.set_seed(4242)
+    sub = m._graph._CAPI_FusedColumnwiseSlicingSampling(to_dev(seeds, dev), 6, False)
+    want = O.sample_uniform(indptr, indices, seeds, 6, False, seed=4242, with_coo=False)
+    return m, sub, seeds, want
+
+
+@pytest.mark.parametrize("first_use", ["num_edges", "csc", "sum", "slicing", "coo_rows", "relabel_twice"])
+def test_pending_graph_settles_on_first_use(dev, first_use):
+    """The fused sampler returns before its edge count has reached the host; whichever method
+    touches the graph first must see the finished CSC."""
+    m, sub, seeds, (sp, _, rows, _) = _fused_child(dev)
+    if first_use == "num_edges":
+        assert sub._CAPI_GetNumEdges() == rows.size
+    elif first_use == "csc":
+        ptr, idx = sub._CAPI_GetCSC()[:2]
+        assert np.array_equal(ptr.cpu().numpy(), sp) and np.array_equal(idx.cpu().numpy(), rows)
+    elif first_use == "sum":
+        s = sub._CAPI_Sum(0, 1, _CSC)
+        assert np.array_equal(s.cpu().numpy(), np.diff(sp).astype(np.float32))
+    elif first_use == "slicing":
+        child = sub._CAPI_Slicing(torch.arange(0, 10, **I(dev)), 0, _CSC, _CSC, False)
+        assert child._CAPI_GetNumEdges() == sp[10]
+    elif first_use == "coo_rows":
+        assert np.array_equal(sub._CAPI_GetCOORows(False).cpu().numpy(), rows)
+    else:
+        a = sub._CAPI_Relabel()
+        b = sub._CAPI_Relabel()  # the second call finds a settled graph
+        for x, y in zip(a[:5], b[:5]):
+            assert torch.equal(x, y) if torch.is_tensor(x) else x == y
+        frontier, (rel,) = O.relabel([seeds, rows], [rows])
+        assert np.array_equal(a[0].cpu().numpy(), frontier) and np.array_equal(a[4].cpu().numpy(), rel)
+        assert sub._CAPI_GetNumEdges() == rows.size
+
+
+def test_pending_graph_outlives_its_mailbox_slot(dev):
+    """A pending graph kept aside while more calls go by than there are mailbox slots still settles
+    (its count is then read from the device)."""
+    m, sub, seeds, (sp, _, rows, _) = _fused_child(dev)
+    d_seeds = to_dev(seeds, dev)
+    for _ in range(80):
+        m._graph._CAPI_FusedColumnwiseSlicingSampling(d_seeds[:50], 3, False)._CAPI_Relabel()
+    assert sub._CAPI_GetNumEdges() == rows.size
+    assert np.array_equal(sub._CAPI_GetCSC()[1].cpu().numpy(), rows)
+
+
+def test_deferred_sampling_switch_gives_identical_results(dev):
+    outs = []
+    for mode in (True, False):
+        torch.ops.gs_ops._CAPI_SetDeferredSampling(mode)
+        try:
+            _, sub, _, _ = _fused_child(dev, seed=8)
+            outs.append(sub._CAPI_Relabel())
+        finally:
+            torch.ops.gs_ops._CAPI_SetDeferredSampling(True)
+    for x, y in zip(outs[0][:5], outs[1][:5]):
+        assert torch.equal(x, y) if torch.is_tensor(x) else x == y
+
+
+def test_unfused_graphsage_flow_with_int32_ids(dev):
+    """A graph loaded with int32 ids goes through Slicing -> Sampling -> Relabel (COO <-> CSC
+    conversions, sampling over all columns, relabel of both COO sides) and matches the oracle."""
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 16, seed=2)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev, torch.int32))
+    seeds = np.random.default_rng(1).permutation(1 << 12)[:200].astype(np.int64)
+    sliced = g._CAPI_Slicing(to_dev(seeds, dev, torch.int32), 0, _CSC, _COO, False)
+    gs.set_seed(77)
+    sampled = sliced._CAPI_Sampling(0, 7, False, _CSC, _COO)
+    frontier, n_src, n_dst, row, col, e_ids, fmt = sampled._CAPI_Relabel()
+    sp, coo, si, sel = O.slice_columns(indptr, indices, seeds)
+    sp2, coo2, si2, sel2 = O.sample_uniform(sp, si, None, 7, False, seed=77)
+    want_frontier, (rel_col, rel_row) = O.relabel([seeds, si2], [seeds[coo2], si2])
+    assert fmt == "coo" and frontier.dtype == torch.int32 and row.dtype == torch.int32
+    assert np.array_equal(frontier.cpu().numpy(), want_frontier)
+    assert np.array_equal(row.cpu().numpy(), rel_row) and np.array_equal(col.cpu().numpy(), rel_col)
+    # CSR of the int32 graph (stable sort on rows) and a row slice on it
+    g._CAPI_CSC2CSR()
+    r_ip, r_col, r_perm = O.coo2csc(indices, O.csc2coo(indptr, indices.size), 1 << 12, False)
+    meta = g._CAPI_Slicing(to_dev(seeds, dev, torch.int32), 1, _CSR, _CSR, False)._CAPI_Metadata()
+    w_ip, _, w_col, _ = O.slice_columns(r_ip, r_col, seeds)
+    assert np.array_equal(meta[3].cpu().numpy(), w_ip) and np.array_equal(meta[4].cpu().numpy(), w_col)

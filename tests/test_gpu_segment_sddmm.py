@@ -9,13 +9,14 @@ from tests.util import graph_12col_4edge, graph_20x5, rmat_csc_np, to_dev
 
 pytestmark = pytest.mark.gpu
 RTOL = 1e-5  # float values: relative tolerance of the parity contract
+ID_DTYPES = [torch.int64, torch.int32]
 
 
-def _seg_sum(dev, indptr, data, powk, e_ids=None, n_ids=None, out_size=None):
+def _seg_sum(dev, indptr, data, powk, e_ids=None, n_ids=None, out_size=None, idt=torch.int64):
     out_size = out_size or indptr.size - 1
     out = torch.zeros(out_size, dtype=torch.float32, device=dev)
     capi.segment_sum(to_dev(indptr, dev), None if e_ids is None else to_dev(e_ids, dev),
-                     None if n_ids is None else to_dev(n_ids, dev), to_dev(data, dev), powk, out)
+                     None if n_ids is None else to_dev(n_ids, dev, idt), to_dev(data, dev), powk, out)
     return out.cpu().numpy()
 
 
@@ -41,15 +42,16 @@ def test_row_sum_reference_vector_coo(dev):
     assert np.array_equal(O.coo_sum(indices, None, data, 1, 12), expected)
 
 
+@pytest.mark.parametrize("idt", ID_DTYPES)
 @pytest.mark.parametrize("powk", [1, 2, 3])
 @pytest.mark.parametrize("maps", [False, True])
-def test_segment_sum_rmat(dev, powk, maps):
+def test_segment_sum_rmat(dev, powk, maps, idt):
     indptr, indices = rmat_csc_np(1 << 12, 1 << 17, seed=4)  # hubs of several thousand edges
     rng = np.random.default_rng(powk)
     data = rng.random(indices.size, dtype=np.float32)
     e_ids = rng.permutation(indices.size).astype(np.int64) if maps else None
     n_ids = rng.permutation(indptr.size - 1).astype(np.int64) if maps else None
-    got = _seg_sum(dev, indptr, data, powk, e_ids, n_ids)
+    got = _seg_sum(dev, indptr, data, powk, e_ids, n_ids, idt=idt)
     want = O.segment_sum(indptr, e_ids, n_ids, data, powk, indptr.size - 1)
     np.testing.assert_allclose(got, want, rtol=RTOL)
     short = np.diff(indptr) <= 32  # short segments are summed in edge order: bit exact
@@ -87,30 +89,33 @@ def test_segment_normalize(dev, maps):
     np.testing.assert_allclose(sums, 1.0, rtol=1e-4)
 
 
-def test_coo_sum_and_e_div_u_sum(dev):
+@pytest.mark.parametrize("idt", ID_DTYPES)
+def test_coo_sum_and_e_div_u_sum(dev, idt):
     indptr, indices = rmat_csc_np(1 << 11, 1 << 16, seed=6)
     col = O.csc2coo(indptr, indices.size)
     rng = np.random.default_rng(2)
     data = rng.random(indices.size, dtype=np.float32)
     out = torch.zeros(1 << 11, dtype=torch.float32, device=dev)
-    capi.coo_sum(to_dev(indices, dev), None, to_dev(data, dev), 2, out)
+    capi.coo_sum(to_dev(indices, dev, idt), None, to_dev(data, dev), 2, out)
     np.testing.assert_allclose(out.cpu().numpy(), O.coo_sum(indices, None, data, 2, 1 << 11), rtol=1e-4)
     divisor = rng.random(1 << 11, dtype=np.float32) + 0.5
     od = torch.zeros(indices.size, dtype=torch.float32, device=dev)
     osum = torch.zeros(1 << 11, dtype=torch.float32, device=dev)
-    capi.e_div_u_sum(to_dev(indices, dev), to_dev(col, dev), to_dev(data, dev), to_dev(divisor, dev), od, osum)
+    capi.e_div_u_sum(to_dev(indices, dev, idt), to_dev(col, dev, idt), to_dev(data, dev),
+                     to_dev(divisor, dev), od, osum)
     wd, ws = O.e_div_u_sum(indices, col, data, divisor, 1 << 11)
     assert np.array_equal(od.cpu().numpy(), wd)  # one IEEE division per edge: bit exact
     np.testing.assert_allclose(osum.cpu().numpy(), ws, rtol=1e-4)
 
 
 # ------------------------------------------------------------------ SDDMM
-def _sddmm_coo_gpu(dev, op, row, col, e_ids, lhs, rhs, lt, rt):
+def _sddmm_coo_gpu(dev, op, row, col, e_ids, lhs, rhs, lt, rt, idt=torch.int64):
     ls = lhs.shape if lhs.ndim > 1 else lhs.shape + (1,)
     rs = rhs.shape if rhs.ndim > 1 else rhs.shape + (1,)
     b = O.calc_bcast(op, ls, rs)
     out = torch.zeros((row.size, b["out_len"]), dtype=torch.float32, device=dev)
-    capi.sddmm_coo(op, to_dev(row, dev), to_dev(col, dev), None if e_ids is None else to_dev(e_ids, dev),
+    capi.sddmm_coo(op, to_dev(row, dev, idt), to_dev(col, dev, idt),
+                   None if e_ids is None else to_dev(e_ids, dev),
                    to_dev(lhs, dev), to_dev(rhs, dev), out, lt, rt, b["lhs_len"], b["rhs_len"],
                    b["out_len"], b["reduce_size"],
                    None if b["lhs_off"] is None else to_dev(b["lhs_off"], dev),
@@ -159,14 +164,15 @@ def test_sddmm_coo_ops_targets(dev, op, targets):
     np.testing.assert_allclose(want, full, rtol=RTOL)
 
 
-def test_sddmm_dot_64_fast_path(dev):
+@pytest.mark.parametrize("idt", ID_DTYPES)
+def test_sddmm_dot_64_fast_path(dev, idt):
     # u_dot_v with 64-wide fp32 features (BASELINE config 5)
     indptr, indices = rmat_csc_np(1 << 11, 1 << 16, seed=8)
     col = O.csc2coo(indptr, indices.size)
     rng = np.random.default_rng(4)
     lhs = rng.standard_normal((1 << 11, 64)).astype(np.float32)
     rhs = rng.standard_normal((1 << 11, 64)).astype(np.float32)
-    got = _sddmm_coo_gpu(dev, "dot", indices, col, None, lhs, rhs, 0, 2)
+    got = _sddmm_coo_gpu(dev, "dot", indices, col, None, lhs, rhs, 0, 2, idt=idt)
     want = O.sddmm_coo("dot", indices, col, None, lhs, rhs, 0, 2)
     ref = np.einsum("ij,ij->i", lhs[indices].astype(np.float64), rhs[col].astype(np.float64))
     scale = np.abs(lhs[indices] * rhs[col]).sum(1)  # error bound relative to the summed magnitudes
@@ -190,8 +196,9 @@ def test_sddmm_broadcast(dev):
     assert np.array_equal(O.sddmm_coo("mul", indices, col, None, lhs, rhs, 0, 2), want)
 
 
+@pytest.mark.parametrize("idt", ID_DTYPES)
 @pytest.mark.parametrize("use_maps", [False, True])
-def test_sddmm_csc(dev, use_maps):
+def test_sddmm_csc(dev, use_maps, idt):
     indptr, indices = rmat_csc_np(1 << 10, 1 << 14, seed=10)
     E, N = indices.size, 1 << 10
     rng = np.random.default_rng(6)
@@ -200,8 +207,9 @@ def test_sddmm_csc(dev, use_maps):
     e_ids = rng.permutation(E).astype(np.int64) if use_maps else None
     nid = (rng.permutation(N) + N).astype(np.int64) if use_maps else None
     out = torch.zeros((E, 4), dtype=torch.float32, device=dev)
-    capi.sddmm_csc("add", to_dev(indptr, dev), to_dev(indices, dev),
-                   None if e_ids is None else to_dev(e_ids, dev), None if nid is None else to_dev(nid, dev),
+    capi.sddmm_csc("add", to_dev(indptr, dev), to_dev(indices, dev, idt),
+                   None if e_ids is None else to_dev(e_ids, dev),
+                   None if nid is None else to_dev(nid, dev, idt),
                    to_dev(lhs, dev), to_dev(rhs, dev), out, 0, 2, 4, 4, 4, 1)
     want = O.sddmm_csc("add", indptr, indices, e_ids, nid, lhs, rhs, 0, 2)
     assert np.array_equal(out.cpu().numpy(), want)
