@@ -123,7 +123,7 @@ slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ in
       q = indptr[c] + (p - sub_indptr[row]);
     }
     sub_indices[p] = indices[q];
-    select_index[p] = q;
+    if (select_index) select_index[p] = q;
     if (WITH_COO) coo_col[p] = static_cast<IdT>(row);
   }
 }
@@ -794,7 +794,7 @@ int gs_slice_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
                   void* stream) {
   GS_REQUIRE(indptr && sub_indptr && S >= 0 && nnz >= 0 && num_cols >= 0,
              "gs_slice_fill: null pointer or negative size");
-  GS_REQUIRE(nnz == 0 || (indices && column_ids && sub_indices && select_index),
+  GS_REQUIRE(nnz == 0 || (indices && column_ids && sub_indices),
              "gs_slice_fill: null buffer with nnz > 0");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_slice_fill: id_bytes must be 4 or 8, got %d", id_bytes);
   hipStream_t st = static_cast<hipStream_t>(stream);

@@ -122,13 +122,17 @@ void Graph::CreateSparseFormat(int64_t format) {
       SetCOO(GraphCSC2COO(csr_, false));
   } else if (format == _CSC) {
     if (csc_) return;
-    if (coo_)
+    if (spare_csc_)
+      SetCSC(std::move(spare_csc_));
+    else if (coo_)
       SetCSC(GraphCOO2CSC(coo_, num_cols_, true));
     else
       CSR2CSC();
   } else if (format == _CSR) {
     if (csr_) return;
-    if (coo_)
+    if (spare_csr_)
+      SetCSR(std::move(spare_csr_));
+    else if (coo_)
       SetCSR(GraphCOO2CSC(coo_, num_rows_, false));
     else
       CSC2CSR();
@@ -196,8 +200,8 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
     num_rows = n_ids.numel();
   }
 
-  std::shared_ptr<CSC> out_csc;
-  std::shared_ptr<CSR> out_csr;
+  std::shared_ptr<CSC> out_csc, spare_csc;
+  std::shared_ptr<CSR> out_csr, spare_csr;
   std::shared_ptr<COO> out_coo;
   torch::Tensor select_index;
   torch::optional<torch::Tensor> e_ids;
@@ -219,7 +223,7 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
     const bool along = (axis == 0) == on_csc;
     std::shared_ptr<_TMP> tmp;
     if (along) {
-      std::tie(tmp, select_index) = CSCColSlicing(fmt, n_ids, with_coo);
+      std::tie(tmp, select_index) = CSCColSlicing(fmt, n_ids, with_coo, data_.has_value());
       if (relabel) {
         // the other side is renumbered by first occurrence (reference src/graph.cc:219-227)
         torch::Tensor frontier;
@@ -243,6 +247,12 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
       auto compressed =
           std::make_shared<CSC>(CSC{tmp->indptr, tmp->coo_in_indices, torch::nullopt});
       (on_csc ? out_csc : out_csr) = compressed;
+    } else if (along && tmp->indptr.defined()) {
+      // the slice produced the offsets anyway: keep them aside so that a later
+      // CreateSparseFormat finds the compressed format without re-deriving it from the COO
+      auto compressed =
+          std::make_shared<CSC>(CSC{tmp->indptr, tmp->coo_in_indices, torch::nullopt});
+      (on_csc ? spare_csc : spare_csr) = compressed;
     }
     if (with_coo) {
       out_coo = on_csc ? std::make_shared<COO>(COO{tmp->coo_in_indices, tmp->coo_in_indptr,
@@ -259,6 +269,8 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
   ret->SetCOO(out_coo);
   ret->SetCSC(out_csc);
   ret->SetCSR(out_csr);
+  ret->spare_csc_ = spare_csc;
+  ret->spare_csr_ = spare_csr;
   InheritData(ret.get(), e_ids, select_index);
   return ret;
 }

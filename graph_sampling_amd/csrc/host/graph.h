@@ -149,6 +149,12 @@ class Graph : public torch::CustomClassHolder {
   void Settle();
   std::shared_ptr<hip::PendingSample> pending_;
 
+  // Compressed form a slice computed on the way to a COO-only result: not a format of
+  // the graph yet (getters and Relabel do not see it), just what CreateSparseFormat
+  // installs instead of converting the COO back.
+  std::shared_ptr<CSC> spare_csc_;
+  std::shared_ptr<CSR> spare_csr_;
+
   bool is_subgraph_ = false;
   int64_t num_cols_ = 0;
   int64_t num_rows_ = 0;

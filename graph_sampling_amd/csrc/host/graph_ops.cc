@@ -17,8 +17,8 @@ std::pair<std::shared_ptr<_TMP>, torch::Tensor> Wrap(hip::SliceResult r) {
 
 std::pair<std::shared_ptr<_TMP>, torch::Tensor> CSCColSlicing(std::shared_ptr<CSC> csc,
                                                               torch::Tensor node_ids,
-                                                              bool with_coo) {
-  return Wrap(hip::ColSlicing(csc->indptr, csc->indices, node_ids, with_coo));
+                                                              bool with_coo, bool with_select) {
+  return Wrap(hip::ColSlicing(csc->indptr, csc->indices, node_ids, with_coo, with_select));
 }
 
 std::pair<std::shared_ptr<_TMP>, torch::Tensor> CSCRowSlicing(std::shared_ptr<CSC> csc,

@@ -15,9 +15,10 @@
 
 namespace gs {
 
+// with_select false: the returned select_index is undefined (the caller has no edge data)
 std::pair<std::shared_ptr<_TMP>, torch::Tensor> CSCColSlicing(std::shared_ptr<CSC> csc,
                                                               torch::Tensor node_ids,
-                                                              bool with_coo);
+                                                              bool with_coo, bool with_select = true);
 
 std::pair<std::shared_ptr<_TMP>, torch::Tensor> CSCRowSlicing(std::shared_ptr<CSC> csc,
                                                               torch::Tensor node_ids,

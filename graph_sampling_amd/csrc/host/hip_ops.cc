@@ -168,7 +168,7 @@ void SetSampleAlgo(int64_t algo) {
 }
 
 SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
-                       const torch::Tensor& column_ids, bool with_coo) {
+                       const torch::Tensor& column_ids, bool with_coo, bool with_select) {
   NeedI64(indptr, "indptr");
   const int idb = IdBytes(indices, "indices");
   TORCH_CHECK(IdBytes(column_ids, "column ids") == idb, "column ids and indices differ in dtype");
@@ -181,12 +181,14 @@ SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices
         "gs_slice_count");
   const int64_t nnz = sub_indptr[S].item<int64_t>();
   auto sub_indices = torch::empty({nnz}, indices.options());
-  auto select_index = torch::empty({nnz}, I64(indptr));
+  torch::Tensor select_index;
+  if (with_select) select_index = torch::empty({nnz}, I64(indptr));
   torch::Tensor coo_col;
   if (with_coo) coo_col = torch::empty({nnz}, indices.options());
   Check(gs_slice_fill(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), column_ids.data_ptr(), idb, S,
                       sub_indptr.data_ptr<int64_t>(), nnz, sub_indices.data_ptr(),
-                      select_index.data_ptr<int64_t>(), with_coo ? coo_col.data_ptr() : nullptr, st),
+                      with_select ? select_index.data_ptr<int64_t>() : nullptr,
+                      with_coo ? coo_col.data_ptr() : nullptr, st),
         "gs_slice_fill");
   return {sub_indptr, coo_col, sub_indices, select_index};
 }

@@ -27,8 +27,9 @@ uint64_t NextSeed();
 // 0: Floyd selection for deg > fanout (default), 1: the reference's Algorithm R.
 void SetSampleAlgo(int64_t algo);
 
+// with_select false: select_index comes back undefined (nothing to gather edge data for)
 SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
-                       const torch::Tensor& column_ids, bool with_coo);
+                       const torch::Tensor& column_ids, bool with_coo, bool with_select = true);
 // column_ids undefined: every column of the CSC
 SliceResult ColSampling(const torch::Tensor& indptr, const torch::Tensor& indices,
                         const torch::Tensor& column_ids, int64_t fanout, bool replace,

@@ -102,7 +102,8 @@ int gs_slice_count(const int64_t* indptr, int64_t num_cols, const void* column_i
                    void* stream);
 
 /* Neighbour copy (slicing.cu:101-119).  nnz = sub_indptr[S] as read back by the
- * caller.  coo_col may be NULL (WITH_COO = false). */
+ * caller.  coo_col may be NULL (WITH_COO = false); select_index may be NULL when
+ * the caller has no edge data to gather. */
 int gs_slice_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
                   const void* column_ids, int id_bytes, int64_t S, const int64_t* sub_indptr,
                   int64_t nnz, void* sub_indices, int64_t* select_index, void* coo_col,
