@@ -13,8 +13,8 @@
 //    (format_transform.cu:58-72 also sorts just the significant bits).  Each
 //    pass is histogram -> scan -> stable scatter; the scatter ranks equal digits
 //    inside a wave with 8 ballots (no LDS atomics, order preserved) and across
-//    waves with a small LDS table.  indptr then comes from the boundaries of
-//    the sorted keys, one pass, no per-column binary search.
+//    waves with a small LDS table.  indptr then comes from one binary search
+//    per column in the sorted keys.
 #include "gs_common.hpp"
 
 namespace gs {
@@ -61,23 +61,24 @@ csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz
   }
 }
 
-// indptr from sorted keys: every boundary between key[e] and key[e+1] fills the
-// offsets of the columns in between (format_transform.cu:123-156 computes the
-// same values with one binary search per column).
+// indptr from sorted keys: indptr[c] = number of keys < c, one binary search per
+// column (format_transform.cu:123-156 does the same).  A boundary-driven fill
+// (every edge writes the offsets of the columns between it and its predecessor)
+// was tried first and is worse at both ends: with few edges and millions of
+// columns one lane fills a gap of a million offsets by itself, with many edges
+// and few columns it reads every key to find a handful of boundaries.
 template <typename KeyT>
 __global__ void __launch_bounds__(kThreads)
 indptr_from_sorted_kernel(const KeyT* __restrict__ key, int64_t E, int64_t num_keys,
                           int64_t* __restrict__ indptr) {
-  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (e > E) return;
-  // boundary e sits between key[e-1] and key[e]; columns in (key[e-1], key[e]] start at e
-  // keys outside [0, num_keys) (an inconsistent caller) are clamped: they can
-  // never index past the num_keys + 1 offsets
-  int64_t lo = e == 0 ? -1 : static_cast<int64_t>(key[e - 1]);
-  int64_t hi = e == E ? num_keys : static_cast<int64_t>(key[e]);
-  if (lo < -1) lo = -1;
-  if (hi > num_keys) hi = num_keys;
-  for (int64_t c = lo + 1; c <= hi; ++c) indptr[c] = e;
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (c > num_keys) return;
+  int64_t lo = 0, hi = E;  // first position whose key is >= c
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (static_cast<int64_t>(key[mid]) < c) lo = mid + 1; else hi = mid;
+  }
+  indptr[c] = lo;
 }
 
 // ------------------------------------------------------------ radix sort ----
@@ -183,7 +184,7 @@ int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, 
                  int64_t* indptr, IdT* out_value, int64_t* perm, void* workspace,
                  size_t workspace_bytes, hipStream_t st) {
   if (sorted || E == 0) {
-    hipLaunchKernelGGL((indptr_from_sorted_kernel<IdT>), dim3(blocks_for(E + 1, kThreads)),
+    hipLaunchKernelGGL((indptr_from_sorted_kernel<IdT>), dim3(blocks_for(num_keys + 1, kThreads)),
                        dim3(kThreads), 0, st, key, E, num_keys, indptr);
     return check_launch("coo2csc");
   }
@@ -228,7 +229,7 @@ int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, 
   }
   hipLaunchKernelGGL((gather_kernel<IdT>), dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st,
                      value, perm, E, out_value);
-  hipLaunchKernelGGL((indptr_from_sorted_kernel<int64_t>), dim3(blocks_for(E + 1, kThreads)),
+  hipLaunchKernelGGL((indptr_from_sorted_kernel<int64_t>), dim3(blocks_for(num_keys + 1, kThreads)),
                      dim3(kThreads), 0, st, kin, E, num_keys, indptr);
   return check_launch("coo2csc");
 }
