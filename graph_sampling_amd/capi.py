@@ -392,6 +392,33 @@ def unique_relabel(mapping, queries, mailbox=None, last_span_len=None):
     return frontier, num_unique, outs
 
 
+def batch_csr_relabel(seeds, seeds_ptr, ids, ids_ptr, mailbox=None):
+    """gs_batch_csr_relabel.  Returns (unique_buf, unique_ptr, relabelled ids, num_unique_dev
+    [, ticket]); unique_buf has the capacity len(seeds) + len(ids)."""
+    idb = _ids(seeds, "seeds")
+    _ids(ids, "ids", like=seeds)
+    _need(seeds_ptr, torch.int64, "seeds_ptr")
+    _need(ids_ptr, torch.int64, "ids_ptr")
+    dev = seeds.device
+    B = seeds_ptr.numel() - 1
+    M = seeds.numel() + ids.numel()
+    unique = torch.empty(M, dtype=seeds.dtype, device=dev)
+    unique_ptr = torch.empty(B + 1, dtype=torch.int64, device=dev)
+    out_ids = torch.empty_like(ids)
+    num_unique = torch.empty(1, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_unique_workspace_bytes(_i64(M)), dev)
+    ticket = mailbox.ticket() if mailbox is not None else 0
+    _check(lib().gs_batch_csr_relabel(_ptr(seeds), _ptr(seeds_ptr), _ptr(ids), _ptr(ids_ptr), _i64(B),
+                                      _i64(seeds.numel()), _i64(ids.numel()), idb, _ptr(unique),
+                                      _ptr(unique_ptr), _ptr(out_ids), _ptr(num_unique), _ptr(ws),
+                                      ctypes.c_size_t(ws.numel()),
+                                      mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0),
+                                      _i64(ticket), _stream(dev)), "gs_batch_csr_relabel")
+    if mailbox is not None:
+        return unique, unique_ptr, out_ids, num_unique, ticket
+    return unique, unique_ptr, out_ids, num_unique
+
+
 # ------------------------------------------------------------------ walks ----
 def random_walk(indptr, indices, seeds, length, seed=0, replay=None):
     _need(indptr, torch.int64, "indptr")

@@ -179,6 +179,23 @@ int num_passes(int64_t num_keys) {
   return (bits + kRadixBits - 1) / kRadixBits;
 }
 
+// Offsets of B consecutive column ranges, each re-based to start at 0 and laid
+// out one after the other (batch b: offsets[b+1]-offsets[b]+1 entries starting
+// at offsets[b] + b).  One output entry per lane, batch by binary search.
+__global__ void __launch_bounds__(kThreads)
+indptr_split_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ offsets,
+                    int64_t B, int64_t total, int64_t* __restrict__ out) {
+  const int64_t q = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (q >= total) return;
+  int64_t lo = 0, hi = B - 1;  // last b with offsets[b] + b <= q
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) >> 1;
+    if (offsets[mid] + mid <= q) lo = mid; else hi = mid - 1;
+  }
+  const int64_t begin = offsets[lo];
+  out[q] = indptr[begin + (q - begin - lo)] - indptr[begin];
+}
+
 template <typename IdT>
 int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, int sorted,
                  int64_t* indptr, IdT* out_value, int64_t* perm, void* workspace,
@@ -285,6 +302,16 @@ int gs_coo2csc(const void* key, const void* value, int id_bytes, int64_t E, int6
                                      static_cast<const int32_t*>(value), E, num_keys, sorted,
                                      indptr, static_cast<int32_t*>(out_value), perm, workspace,
                                      workspace_bytes, st);
+}
+
+int gs_indptr_split(const int64_t* indptr, const int64_t* offsets, int64_t num_batches,
+                    int64_t total, int64_t* out, void* stream) {
+  GS_REQUIRE(num_batches >= 0 && total >= 0, "gs_indptr_split: negative size");
+  if (num_batches == 0 || total == 0) return GS_OK;
+  GS_REQUIRE(indptr && offsets && out, "gs_indptr_split: null pointer");
+  hipLaunchKernelGGL(indptr_split_kernel, dim3(blocks_for(total, kThreads)), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), indptr, offsets, num_batches, total, out);
+  return check_launch("indptr_split");
 }
 
 }  // extern "C"

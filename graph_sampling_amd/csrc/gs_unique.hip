@@ -44,6 +44,7 @@ struct Spans {
     const int64_t n_last = *last_len;
     return fixed + (n_last > 0 ? n_last : 0);
   }
+  __device__ __forceinline__ long long key(int64_t i) const { return static_cast<long long>(get(i)); }
   __device__ __forceinline__ IdT get(int64_t i) const {
     int s = 0;
     int64_t begin = 0;
@@ -167,12 +168,12 @@ __global__ void __launch_bounds__(kThreads) table_init_kernel(T t, int64_t cap, 
 
 // insert (key -> min index) and remember the slot of every item
 // (unique_reindex.cu:92-99)
-template <typename IdT, typename T>
+template <typename X, typename T>
 __global__ void __launch_bounds__(kThreads)
-table_insert_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ pos) {
+table_insert_kernel(X x, int64_t M_bound, T t, uint32_t* __restrict__ pos) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= x.items(M_bound)) return;
-  pos[i] = t.insert(static_cast<long long>(x.get(i)), static_cast<uint32_t>(i));
+  pos[i] = t.insert(x.key(i), static_cast<uint32_t>(i));
 }
 
 struct Query {
@@ -191,9 +192,9 @@ struct Query {
 constexpr int kCompactItems = 8;
 constexpr int kCompactTile = kThreads * kCompactItems;
 
-template <typename IdT, typename T>
+template <typename IdT, typename X, typename T>
 __global__ void __launch_bounds__(kThreads)
-compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ pos,
+compact_kernel(X x, int64_t M_bound, T t, const uint32_t* __restrict__ pos,
                int64_t* __restrict__ prefix, IdT* __restrict__ frontier,
                int64_t* __restrict__ num_unique, LookbackState lb, gs_mailbox* box,
                int64_t box_ticket) {
@@ -356,12 +357,12 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   }
   if (M > 0) {
     ProfileScope prof("table_insert", stream);
-    hipLaunchKernelGGL((table_insert_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
+    hipLaunchKernelGGL((table_insert_kernel<Spans<IdT>, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
                        0, stream, x, M, t, pos);
   }
   {
     ProfileScope prof("unique_compact", stream);
-    hipLaunchKernelGGL((compact_kernel<IdT, T>), dim3(static_cast<unsigned>(tiles)), dim3(kThreads),
+    hipLaunchKernelGGL((compact_kernel<IdT, Spans<IdT>, T>), dim3(static_cast<unsigned>(tiles)), dim3(kThreads),
                        0, stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, lb,
                        box, box_ticket);
   }
@@ -371,6 +372,120 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
                        stream, t, pos, prefix, qs, Q, last_span_len);
   }
   return check_launch("unique_relabel");
+}
+
+
+// ------------------------------------------------ batched (super-batch) relabel ----
+// B independent relabels in one pass: replaces impl::BatchCSRRelabelCUDA (reference
+// src/cuda/batch_relabel.cu:331; kernels :90-232).  Batch b owns seeds
+// [seeds_ptr[b], seeds_ptr[b+1]) and ids [indices_ptr[b], indices_ptr[b+1]); its
+// frontier is the distinct values of (its seeds, then its ids) in first-occurrence
+// order, the frontiers are concatenated by batch, and every id is renamed to its
+// rank inside its own batch's frontier.
+//
+// The reference gives every batch a hash table of its own.  Here the items are
+// laid out virtually as [seeds_0, ids_0, seeds_1, ids_1, ...] (the order the
+// reference's prefix array has, batch_relabel.cu:152,163), the key is the pair
+// (batch, id) packed into 64 bits, and the single-table machinery above runs
+// once over all of them: one insert pass, one chained-scan compaction, one
+// lookup pass whatever the number of batches.
+constexpr int kBatchIdBits = 40;
+
+template <typename IdT>
+struct BatchItems {
+  const IdT* seeds;
+  const int64_t* seeds_ptr;
+  const IdT* ids;
+  const int64_t* ids_ptr;
+  int64_t B;
+  __device__ __forceinline__ int64_t items(int64_t host_items) const { return host_items; }
+  __device__ __forceinline__ int64_t start(int64_t b) const { return seeds_ptr[b] + ids_ptr[b]; }
+  // batch of the item at position i of the interleaved layout
+  __device__ __forceinline__ int64_t batch_of(int64_t i) const {
+    int64_t lo = 0, hi = B;  // last b with start(b) <= i
+    while (lo < hi) {
+      const int64_t mid = (lo + hi + 1) >> 1;
+      if (start(mid) <= i) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+  }
+  __device__ __forceinline__ IdT get_in(int64_t b, int64_t i) const {
+    const int64_t off = i - start(b);
+    const int64_t n_seeds = seeds_ptr[b + 1] - seeds_ptr[b];
+    return off < n_seeds ? seeds[seeds_ptr[b] + off] : ids[ids_ptr[b] + off - n_seeds];
+  }
+  __device__ __forceinline__ IdT get(int64_t i) const { return get_in(batch_of(i), i); }
+  __device__ __forceinline__ long long key(int64_t i) const {
+    const int64_t b = batch_of(i);
+    return static_cast<long long>((static_cast<unsigned long long>(b) << kBatchIdBits) |
+                                  static_cast<unsigned long long>(get_in(b, i)));
+  }
+};
+
+// ids -> rank inside their batch's frontier; unique_ptr[b] = frontier offset of batch b
+template <typename IdT, typename T>
+__global__ void __launch_bounds__(kThreads)
+batch_finish_kernel(BatchItems<IdT> x, int64_t num_ids, T t, const uint32_t* __restrict__ pos,
+                    const int64_t* __restrict__ prefix, const int64_t* __restrict__ num_unique,
+                    IdT* __restrict__ out_ids, int64_t* __restrict__ unique_ptr) {
+  const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  const int64_t M = x.seeds_ptr[x.B] + x.ids_ptr[x.B];
+  if (j < num_ids) {
+    int64_t lo = 0, hi = x.B;  // last b with ids_ptr[b] <= j
+    while (lo < hi) {
+      const int64_t mid = (lo + hi + 1) >> 1;
+      if (x.ids_ptr[mid] <= j) lo = mid; else hi = mid - 1;
+    }
+    const int64_t b = lo;
+    const int64_t p = x.start(b) + (x.seeds_ptr[b + 1] - x.seeds_ptr[b]) + (j - x.ids_ptr[b]);
+    const int64_t base = x.start(b) < M ? prefix[x.start(b)] : *num_unique;
+    out_ids[j] = static_cast<IdT>(prefix[t.first_index(pos[p])] - base);
+    return;
+  }
+  const int64_t b = j - num_ids;
+  if (b <= x.B) unique_ptr[b] = x.start(b) < M ? prefix[x.start(b)] : *num_unique;
+}
+
+template <typename IdT>
+int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* ids,
+                       const int64_t* ids_ptr, int64_t B, int64_t num_seeds, int64_t num_ids,
+                       void* unique, int64_t* unique_ptr, void* out_ids, int64_t* num_unique,
+                       void* workspace, size_t workspace_bytes, gs_mailbox* box,
+                       int64_t box_ticket, hipStream_t stream) {
+  using T = WideTable;
+  const int64_t M = num_seeds + num_ids;
+  const int64_t cap = table_capacity(M);
+  Carver ws(workspace, workspace_bytes);
+  T t;
+  t.carve(ws, cap);
+  uint32_t* pos = ws.take<uint32_t>(M > 0 ? M : 1);
+  int64_t* prefix = ws.take<int64_t>(M + 1);
+  const int64_t tiles = compact_num_tiles(M);
+  LookbackState lb = carve_lookback(ws, tiles, 1u);
+  if (!ws.ok) {
+    set_error_text("gs_batch_csr_relabel: workspace needs %zu bytes, 256-byte aligned",
+                   gs_unique_workspace_bytes(M));
+    return GS_ERR_WORKSPACE;
+  }
+  t.mask = static_cast<uint32_t>(cap - 1);
+  int lg = 0;
+  while ((int64_t(1) << lg) < cap) ++lg;
+  t.shift = 64 - lg;
+  BatchItems<IdT> x{static_cast<const IdT*>(seeds), seeds_ptr, static_cast<const IdT*>(ids), ids_ptr,
+                    B};
+  const int64_t n_init = cap > tiles ? cap : tiles;
+  hipLaunchKernelGGL((table_init_kernel<T>), dim3(blocks_for(n_init, kThreads)), dim3(kThreads), 0,
+                     stream, t, cap, lb, tiles);
+  if (M > 0)
+    hipLaunchKernelGGL((table_insert_kernel<BatchItems<IdT>, T>), dim3(blocks_for(M, kThreads)),
+                       dim3(kThreads), 0, stream, x, M, t, pos);
+  hipLaunchKernelGGL((compact_kernel<IdT, BatchItems<IdT>, T>), dim3(static_cast<unsigned>(tiles)),
+                     dim3(kThreads), 0, stream, x, M, t, pos, prefix, static_cast<IdT*>(unique),
+                     num_unique, lb, box, box_ticket);
+  hipLaunchKernelGGL((batch_finish_kernel<IdT, T>), dim3(blocks_for(num_ids + B + 1, kThreads)),
+                     dim3(kThreads), 0, stream, x, num_ids, t, pos, prefix, num_unique,
+                     static_cast<IdT*>(out_ids), unique_ptr);
+  return check_launch("batch_csr_relabel");
 }
 
 }  // namespace
@@ -436,6 +551,34 @@ int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* quer
   return gs_unique_relabel_notify(mapping, n_mapping, query, query_out, n_query, id_bytes, frontier,
                                   num_unique, workspace, workspace_bytes, nullptr, nullptr, 0,
                                   stream);
+}
+
+int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void* ids,
+                         const int64_t* ids_ptr, int64_t num_batches, int64_t num_seeds,
+                         int64_t num_ids, int id_bytes, void* unique, int64_t* unique_ptr,
+                         void* out_ids, int64_t* num_unique, void* workspace,
+                         size_t workspace_bytes, gs_mailbox* mailbox, int64_t mailbox_ticket,
+                         void* stream) {
+  GS_REQUIRE(num_batches >= 1 && num_seeds >= 0 && num_ids >= 0,
+             "gs_batch_csr_relabel: at least one batch and non-negative sizes required");
+  GS_REQUIRE(seeds_ptr && ids_ptr && unique_ptr && num_unique, "gs_batch_csr_relabel: null pointer");
+  GS_REQUIRE((num_seeds == 0 || seeds) && (num_ids == 0 || (ids && out_ids)) &&
+                 (num_seeds + num_ids == 0 || unique),
+             "gs_batch_csr_relabel: null buffer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_batch_csr_relabel: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  if (num_batches >= (int64_t(1) << (63 - kBatchIdBits)) || num_seeds + num_ids >= (int64_t(1) << 30)) {
+    set_error_text("gs_batch_csr_relabel: at most 2^%d batches and 2^30 items", 63 - kBatchIdBits);
+    return GS_ERR_UNSUPPORTED;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8
+             ? batch_relabel_impl<int64_t>(seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds,
+                                           num_ids, unique, unique_ptr, out_ids, num_unique,
+                                           workspace, workspace_bytes, mailbox, mailbox_ticket, st)
+             : batch_relabel_impl<int32_t>(seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds,
+                                           num_ids, unique, unique_ptr, out_ids, num_unique,
+                                           workspace, workspace_bytes, mailbox, mailbox_ticket, st);
 }
 
 }  // extern "C"

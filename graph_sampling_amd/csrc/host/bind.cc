@@ -58,6 +58,7 @@ TORCH_LIBRARY(gs_classes, m) {
       GS_DEF2("_CAPI_RandomWalk", "_CAPI_random_walk", &Graph::RandomWalk)
       GS_DEF2("_CAPI_SDDMM", "_CAPI_sddmm", &Graph::SDDMM)
       GS_DEF2("_CAPI_GetCSC", "_CAPI_get_csc", &Graph::GetCSCTensor)
+      GS_DEF2("_CAPI_GetBatchCSC", "GetBatchCSC", &Graph::GetBatchCSC)
       GS_DEF2("_CAPI_GetCOO", "_CAPI_get_coo", &Graph::GetCOOTensor)
       GS_DEF2("_CAPI_SetCOO", "_CAPI_set_coo", &Graph::SetCOOByTensor)
       GS_DEF2("_CAPI_SetMetadata", "_CAPI_set_metadata", &Graph::SetMetaData)
@@ -81,6 +82,12 @@ TORCH_LIBRARY(gs_ops, m) {
   m.def("_CAPI_SplitByOffset", &SplitByOffset);
   m.def("SplitByOffset", &SplitByOffset);
   m.def("_CAPI_Unique", &UniqueOp);
+  m.def("_CAPI_IndptrSplitByOffset", &IndptrSplitByOffset);
+  m.def("IndptrSplitByOffset", &IndptrSplitByOffset);
+  m.def("_CAPI_IndptrSplitBySize", &IndptrSplitBySize);
+  m.def("IndptrSplitBySize", &IndptrSplitBySize);
+  m.def("_CAPI_BatchCSRRelabel", &BatchCSRRelabel);
+  m.def("BatchCSRRelabel", &BatchCSRRelabel);
   // not in the reference: reproducible sampling (its seeds are compile-time constants)
   m.def("_CAPI_SetSeed", &SetSeed);
   m.def("_CAPI_SetSampleAlgo", &SetSampleAlgo);

@@ -147,6 +147,13 @@ std::vector<torch::Tensor> Graph::GetCSCTensor() {
   return {csc_->indptr, csc_->indices, csc_->e_ids.value_or(torch::Tensor())};
 }
 
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> Graph::GetBatchCSC(
+    torch::Tensor seeds_ptr) {
+  Settle();
+  CreateSparseFormat(_CSC);
+  return {csc_->indptr, csc_->indices, csc_->indptr.index({seeds_ptr})};
+}
+
 std::vector<torch::Tensor> Graph::GetCOOTensor() {
   Settle();
   CreateSparseFormat(_COO);

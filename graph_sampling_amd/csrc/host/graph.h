@@ -80,6 +80,9 @@ class Graph : public torch::CustomClassHolder {
   }
   std::vector<torch::Tensor> GetCSCTensor();
   std::vector<torch::Tensor> GetCOOTensor();
+  // (indptr, indices, indices_ptr): the CSC of a super-batch whose columns are cut into
+  // batches at seeds_ptr, with the matching cut of the edges (examples/graphsage/batching.py:68)
+  std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> GetBatchCSC(torch::Tensor seeds_ptr);
   torch::optional<torch::Tensor> GetData(std::string order = "default");
   int64_t GetNumRows() { return num_rows_; }
   int64_t GetNumCols() { return num_cols_; }

@@ -428,6 +428,48 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t> RelabelDeferred(const torch::T
   return {frontier.narrow(0, 0, U), renamed.narrow(0, 0, nnz), nnz};
 }
 
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(
+    const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& ids,
+    const torch::Tensor& ids_ptr) {
+  const int idb = IdBytes(seeds, "seeds");
+  TORCH_CHECK(IdBytes(ids, "indices") == idb, "seeds and indices differ in dtype");
+  NeedI64(seeds_ptr, "seeds_ptr");
+  NeedI64(ids_ptr, "indices_ptr");
+  TORCH_CHECK(seeds_ptr.numel() == ids_ptr.numel() && seeds_ptr.numel() >= 2,
+              "seeds_ptr and indices_ptr must both hold num_batches + 1 offsets");
+  const int64_t B = seeds_ptr.numel() - 1;
+  const int64_t M = seeds.numel() + ids.numel();
+  auto unique = torch::empty({M}, seeds.options());
+  auto unique_ptr = torch::empty({B + 1}, I64(seeds));
+  auto out_ids = torch::empty_like(ids);
+  auto num = torch::empty({1}, I64(seeds));
+  auto ws = Scratch(gs_unique_workspace_bytes(M), seeds);
+  void* st = Stream(seeds);
+  HostBoxes& boxes = Boxes(seeds.device().index());
+  const int64_t ticket = boxes.next++;
+  Check(gs_batch_csr_relabel(seeds.data_ptr(), seeds_ptr.data_ptr<int64_t>(), ids.data_ptr(),
+                             ids_ptr.data_ptr<int64_t>(), B, seeds.numel(), ids.numel(), idb,
+                             unique.data_ptr(), unique_ptr.data_ptr<int64_t>(), out_ids.data_ptr(),
+                             num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), boxes.slot(ticket),
+                             ticket, st),
+        "gs_batch_csr_relabel");
+  int64_t U = WaitBox(boxes.slot(ticket), ticket, st, "gs_batch_csr_relabel");
+  if (U == kLost) U = num.item<int64_t>();
+  TORCH_CHECK(U >= 0, "gs_batch_csr_relabel: a tile gave up waiting for its predecessors");
+  return {unique.narrow(0, 0, U), unique_ptr, out_ids};
+}
+
+torch::Tensor IndptrSplit(const torch::Tensor& indptr, const torch::Tensor& offsets,
+                          int64_t total) {
+  NeedI64(indptr, "indptr");
+  NeedI64(offsets, "offsets");
+  auto out = torch::empty({total}, I64(indptr));
+  Check(gs_indptr_split(indptr.data_ptr<int64_t>(), offsets.data_ptr<int64_t>(),
+                        offsets.numel() - 1, total, out.data_ptr<int64_t>(), Stream(indptr)),
+        "gs_indptr_split");
+  return out;
+}
+
 torch::Tensor Unique(const torch::Tensor& ids) { return std::get<0>(Relabel({ids}, {})); }
 
 torch::Tensor RandomWalk(const torch::Tensor& seeds, int64_t length, const torch::Tensor& indptr,

@@ -73,6 +73,14 @@ torch::Tensor Unique(const torch::Tensor& ids);
 std::tuple<torch::Tensor, std::vector<torch::Tensor>> Relabel(
     const std::vector<torch::Tensor>& mapping, const std::vector<torch::Tensor>& queries);
 
+// {unique (batch frontiers back to back), unique_ptr, relabelled ids}: one relabel per batch
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(
+    const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& ids,
+    const torch::Tensor& ids_ptr);
+// the batches' offsets, re-based, back to back (host_offsets: the same offsets on the host)
+torch::Tensor IndptrSplit(const torch::Tensor& indptr, const torch::Tensor& offsets,
+                          int64_t total);
+
 torch::Tensor RandomWalk(const torch::Tensor& seeds, int64_t length, const torch::Tensor& indptr,
                          const torch::Tensor& indices);
 torch::Tensor MetapathWalk(const torch::Tensor& seeds, const torch::Tensor& metapath,

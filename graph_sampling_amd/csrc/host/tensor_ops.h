@@ -20,4 +20,14 @@ std::tuple<torch::Tensor, torch::Tensor> ListSamplingProbs(torch::Tensor data, t
 // data split at the given offsets (offset[i]..offset[i+1])
 std::vector<torch::Tensor> SplitByOffset(torch::Tensor data, torch::Tensor offset);
 
+// Offsets of a batched CSC cut at the batches' column ranges, each piece re-based to
+// start at 0 (reference src/cuda/batch_split.cu:70-94; BySize: equal ranges, :31-46).
+std::vector<torch::Tensor> IndptrSplitByOffset(torch::Tensor indptr, torch::Tensor offsets);
+std::vector<torch::Tensor> IndptrSplitBySize(torch::Tensor indptr, int64_t size);
+
+// One relabel per batch (reference src/cuda/batch_relabel.cu:331):
+// (unique_tensor, unique_tensor_ptr, relabelled indices, indices_ptr).
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> BatchCSRRelabel(
+    torch::Tensor seeds, torch::Tensor seeds_ptr, torch::Tensor indices, torch::Tensor indices_ptr);
+
 }  // namespace gs

@@ -269,6 +269,21 @@ int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_spa
                              const int64_t* last_span_len, gs_mailbox* mailbox,
                              int64_t mailbox_ticket, void* stream);
 
+/* B relabels in one pass ("super-batch"): replaces impl::BatchCSRRelabelCUDA
+ * (src/cuda/batch_relabel.cu:331).  Batch b owns seeds[seeds_ptr[b]..seeds_ptr[b+1])
+ * and ids[ids_ptr[b]..ids_ptr[b+1]) (both *_ptr: device int64[num_batches+1]).
+ * unique (capacity num_seeds+num_ids) = the batches' frontiers one after the other,
+ * each the distinct values of (its seeds, then its ids) in first-occurrence order;
+ * unique_ptr[num_batches+1] = their offsets; out_ids[j] = rank of ids[j] inside its own
+ * batch's frontier; *num_unique (and the mailbox, when given) = total frontier length.
+ * Ids must lie in [0, 2^40).  Workspace: gs_unique_workspace_bytes(num_seeds+num_ids). */
+int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void* ids,
+                         const int64_t* ids_ptr, int64_t num_batches, int64_t num_seeds,
+                         int64_t num_ids, int id_bytes, void* unique, int64_t* unique_ptr,
+                         void* out_ids, int64_t* num_unique, void* workspace,
+                         size_t workspace_bytes, gs_mailbox* mailbox, int64_t mailbox_ticket,
+                         void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Random walks: replace impl::fusion::FusedRandomWalkCUDA                    */
 /* (src/cuda/fusion/random_walk.cu:52) and FusedMetapathRandomWalkCUDA         */
@@ -379,6 +394,14 @@ size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys);
 int gs_coo2csc(const void* key, const void* value, int id_bytes, int64_t E, int64_t num_keys,
                int sorted, int64_t* indptr, void* out_value, int64_t* perm, void* workspace,
                size_t workspace_bytes, void* stream);
+
+/* Offsets of a batched CSC cut into its batches: replaces
+ * impl::SplitIndptrByOffsetCUDA / SplitIndptrBySizeCUDA (src/cuda/batch_split.cu:101,96).
+ * offsets: device int64[num_batches+1], column ranges of the batches; out (length
+ * total = offsets[num_batches] - offsets[0] + num_batches): batch b's
+ * offsets[b+1]-offsets[b]+1 entries, re-based to start at 0, one batch after the other. */
+int gs_indptr_split(const int64_t* indptr, const int64_t* offsets, int64_t num_batches,
+                    int64_t total, int64_t* out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -261,6 +261,26 @@ def relabel(mapping_tensors, to_be_relabeled):
 
 
 # --------------------------------------------------------------------- walks
+def batch_csr_relabel(seeds, seeds_ptr, indices, indices_ptr):
+    """src/cuda/batch_relabel.cu:236-328: one relabel per batch, results concatenated.
+
+    Returns (unique, unique_ptr, relabelled indices): batch b's frontier is the distinct values
+    of (its seeds, then its indices) in first-occurrence order, and its indices are renamed to
+    their rank inside that frontier."""
+    seeds, indices = _i64(seeds), _i64(indices)
+    seeds_ptr, indices_ptr = _i64(seeds_ptr), _i64(indices_ptr)
+    uniques, outs, ptr = [], [], [0]
+    for b in range(seeds_ptr.size - 1):
+        s_b = seeds[seeds_ptr[b]:seeds_ptr[b + 1]]
+        i_b = indices[indices_ptr[b]:indices_ptr[b + 1]]
+        frontier, (rel,) = relabel([s_b, i_b], [i_b])
+        uniques.append(frontier)
+        outs.append(rel)
+        ptr.append(ptr[-1] + frontier.size)
+    cat = lambda xs: np.concatenate(xs) if xs else np.empty(0, np.int64)  # noqa: E731
+    return cat(uniques), np.asarray(ptr, dtype=np.int64), cat(outs)
+
+
 def random_walk(indptr, indices, seeds, length, seed=0, replay=None):
     """src/cuda/fusion/random_walk.cu:52-68 -> flat trace, memory [L+1][n]"""
     indptr, indices, seeds = _i64(indptr), _i64(indices), _i64(seeds)

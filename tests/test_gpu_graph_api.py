@@ -563,3 +563,50 @@ def test_unfused_graphsage_flow_with_int32_ids(dev):
     meta = g._CAPI_Slicing(to_dev(seeds, dev, torch.int32), 1, _CSR, _CSR, False)._CAPI_Metadata()
     w_ip, _, w_col, _ = O.slice_columns(r_ip, r_col, seeds)
     assert np.array_equal(meta[3].cpu().numpy(), w_ip) and np.array_equal(meta[4].cpu().numpy(), w_col)
+
+
+# ------------------------------------------------------------ super-batch GraphSAGE
+def test_super_batch_graphsage_flow_matches_oracle(dev):
+    """examples/graphsage/batching.py:59-88: B minibatches sampled as one call, GetBatchCSC,
+    BatchCSRRelabel, then the splits; every piece equals what the oracle gives batch by batch."""
+    m, indptr, indices, _ = _rmat_matrix(dev, 13, 17, 1)
+    g = m._graph
+    B, small = 16, 64
+    rng = np.random.default_rng(3)
+    seeds = np.concatenate([rng.permutation(1 << 13)[:small] for _ in range(B)]).astype(np.int64)
+    seeds_ptr = np.arange(B + 1, dtype=np.int64) * small
+    d_seeds, d_ptr = to_dev(seeds, dev), to_dev(seeds_ptr, dev)
+    for layer, fanout in enumerate([10, 5]):
+        gs.set_seed(900 + layer)
+        sub = g._CAPI_FusedColumnwiseSlicingSampling(d_seeds, fanout, False)
+        ptr, idx, idx_ptr = sub._CAPI_GetBatchCSC(d_ptr)
+        uni, uni_ptr, rel, idx_ptr2 = torch.ops.gs_ops.BatchCSRRelabel(d_seeds, d_ptr, idx, idx_ptr)
+        sp, _, rows, _ = O.sample_uniform(indptr, indices, seeds, fanout, False, seed=900 + layer,
+                                          with_coo=False)
+        w_idx_ptr = sp[seeds_ptr]
+        w_uni, w_uni_ptr, w_rel = O.batch_csr_relabel(seeds, seeds_ptr, rows, w_idx_ptr)
+        assert np.array_equal(ptr.cpu().numpy(), sp) and np.array_equal(idx.cpu().numpy(), rows)
+        assert np.array_equal(idx_ptr.cpu().numpy(), w_idx_ptr) and torch.equal(idx_ptr, idx_ptr2)
+        assert np.array_equal(uni.cpu().numpy(), w_uni)
+        assert np.array_equal(uni_ptr.cpu().numpy(), w_uni_ptr)
+        assert np.array_equal(rel.cpu().numpy(), w_rel)
+        unit = torch.ops.gs_ops.SplitByOffset(uni, uni_ptr)
+        ptrt = torch.ops.gs_ops.IndptrSplitByOffset(ptr, d_ptr)
+        indt = torch.ops.gs_ops.SplitByOffset(rel, idx_ptr)
+        assert len(unit) == len(ptrt) == len(indt) == B
+        for b in range(B):
+            lo, hi = seeds_ptr[b], seeds_ptr[b + 1]
+            # each piece is the block a separate relabel of that minibatch would give
+            f, (r,) = O.relabel([seeds[lo:hi], rows[sp[lo]:sp[hi]]], [rows[sp[lo]:sp[hi]]])
+            assert np.array_equal(unit[b].cpu().numpy(), f)
+            assert np.array_equal(indt[b].cpu().numpy(), r)
+            assert np.array_equal(ptrt[b].cpu().numpy(), sp[lo:hi + 1] - sp[lo])
+        seeds, seeds_ptr, d_seeds, d_ptr = w_uni, w_uni_ptr, uni, uni_ptr
+
+
+def test_indptr_split_by_size(dev):
+    indptr = np.concatenate([[0], np.cumsum(np.random.default_rng(0).integers(0, 9, size=103))])
+    pieces = torch.ops.gs_ops.IndptrSplitBySize(to_dev(indptr.astype(np.int64), dev), 10)
+    assert len(pieces) == 10  # the ragged tail of 3 columns is dropped, as in the reference
+    for b, p in enumerate(pieces):
+        assert np.array_equal(p.cpu().numpy(), indptr[10 * b:10 * b + 11] - indptr[10 * b])

@@ -106,3 +106,39 @@ def test_relabel_every_item_the_same_key(dev, idt):
     frontier, (rx, ry) = _run([x, y], [x, y], dev, idt)
     assert np.array_equal(frontier, np.array([12345, 0, 1, 2]))
     assert (rx == 0).all() and np.array_equal(ry, y + 1)
+
+
+def _batches(rng, B, n_nodes, max_seeds, max_ids, empty_every=0):
+    seeds, ids, sp, ip = [], [], [0], [0]
+    for b in range(B):
+        ns = 0 if empty_every and b % empty_every == 1 else int(rng.integers(1, max_seeds + 1))
+        ni = 0 if empty_every and b % empty_every == 2 else int(rng.integers(0, max_ids + 1))
+        seeds.append(rng.permutation(n_nodes)[:ns])
+        ids.append(rng.integers(0, n_nodes, size=ni))
+        sp.append(sp[-1] + ns)
+        ip.append(ip[-1] + ni)
+    cat = lambda xs: np.concatenate(xs).astype(np.int64) if xs else np.empty(0, np.int64)  # noqa: E731
+    return cat(seeds), np.array(sp, dtype=np.int64), cat(ids), np.array(ip, dtype=np.int64)
+
+
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+@pytest.mark.parametrize("B,max_seeds,max_ids,empty_every", [(1, 50, 400, 0), (7, 30, 300, 3),
+                                                               (64, 256, 4000, 0), (300, 8, 40, 5)])
+def test_batch_csr_relabel_matches_oracle(dev, idt, B, max_seeds, max_ids, empty_every):
+    """Every batch is relabelled on its own: the same id in two batches gets two ranks."""
+    rng = np.random.default_rng(B)
+    seeds, sp, ids, ip = _batches(rng, B, 3000, max_seeds, max_ids, empty_every)
+    unique, unique_ptr, out_ids, num = capi.batch_csr_relabel(to_dev(seeds, dev, idt), to_dev(sp, dev),
+                                                              to_dev(ids, dev, idt), to_dev(ip, dev))
+    w_unique, w_ptr, w_out = O.batch_csr_relabel(seeds, sp, ids, ip)
+    U = int(num.item())
+    assert U == w_unique.size
+    assert np.array_equal(unique_ptr.cpu().numpy(), w_ptr)
+    assert np.array_equal(unique[:U].cpu().numpy().astype(np.int64), w_unique)
+    assert np.array_equal(out_ids.cpu().numpy().astype(np.int64), w_out)
+    # closed form per batch, independent of the oracle's hash table
+    for b in range(B):
+        x = np.concatenate([seeds[sp[b]:sp[b + 1]], ids[ip[b]:ip[b + 1]]])
+        f = _closed_form_unique(x)
+        assert np.array_equal(w_unique[w_ptr[b]:w_ptr[b + 1]], f)
+        assert np.array_equal(f[w_out[ip[b]:ip[b + 1]]], ids[ip[b]:ip[b + 1]])
