@@ -31,7 +31,7 @@ def lib():
         for name in ("gs_slice_workspace_bytes", "gs_sample_workspace_bytes",
                      "gs_sample_weighted_workspace_bytes", "gs_list_sample_workspace_bytes",
                      "gs_unique_workspace_bytes", "gs_row_slice_workspace_bytes",
-                     "gs_sample_fused_state_bytes",
+                     "gs_sample_fused_state_bytes", "gs_batch_relabel_workspace_bytes",
                      "gs_coo2csc_workspace_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
@@ -406,7 +406,7 @@ def batch_csr_relabel(seeds, seeds_ptr, ids, ids_ptr, mailbox=None):
     unique_ptr = torch.empty(B + 1, dtype=torch.int64, device=dev)
     out_ids = torch.empty_like(ids)
     num_unique = torch.empty(1, dtype=torch.int64, device=dev)
-    ws = workspace(lib().gs_unique_workspace_bytes(_i64(M)), dev)
+    ws = workspace(lib().gs_batch_relabel_workspace_bytes(_i64(M)), dev)
     ticket = mailbox.ticket() if mailbox is not None else 0
     _check(lib().gs_batch_csr_relabel(_ptr(seeds), _ptr(seeds_ptr), _ptr(ids), _ptr(ids_ptr), _i64(B),
                                       _i64(seeds.numel()), _i64(ids.numel()), idb, _ptr(unique),

@@ -44,7 +44,6 @@ struct Spans {
     const int64_t n_last = *last_len;
     return fixed + (n_last > 0 ? n_last : 0);
   }
-  __device__ __forceinline__ long long key(int64_t i) const { return static_cast<long long>(get(i)); }
   __device__ __forceinline__ IdT get(int64_t i) const {
     int s = 0;
     int64_t begin = 0;
@@ -168,12 +167,12 @@ __global__ void __launch_bounds__(kThreads) table_init_kernel(T t, int64_t cap, 
 
 // insert (key -> min index) and remember the slot of every item
 // (unique_reindex.cu:92-99)
-template <typename X, typename T>
+template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
-table_insert_kernel(X x, int64_t M_bound, T t, uint32_t* __restrict__ pos) {
+table_insert_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ pos) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= x.items(M_bound)) return;
-  pos[i] = t.insert(x.key(i), static_cast<uint32_t>(i));
+  pos[i] = t.insert(static_cast<long long>(x.get(i)), static_cast<uint32_t>(i));
 }
 
 struct Query {
@@ -192,9 +191,9 @@ struct Query {
 constexpr int kCompactItems = 8;
 constexpr int kCompactTile = kThreads * kCompactItems;
 
-template <typename IdT, typename X, typename T>
+template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
-compact_kernel(X x, int64_t M_bound, T t, const uint32_t* __restrict__ pos,
+compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ pos,
                int64_t* __restrict__ prefix, IdT* __restrict__ frontier,
                int64_t* __restrict__ num_unique, LookbackState lb, gs_mailbox* box,
                int64_t box_ticket) {
@@ -357,12 +356,12 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   }
   if (M > 0) {
     ProfileScope prof("table_insert", stream);
-    hipLaunchKernelGGL((table_insert_kernel<Spans<IdT>, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
+    hipLaunchKernelGGL((table_insert_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
                        0, stream, x, M, t, pos);
   }
   {
     ProfileScope prof("unique_compact", stream);
-    hipLaunchKernelGGL((compact_kernel<IdT, Spans<IdT>, T>), dim3(static_cast<unsigned>(tiles)), dim3(kThreads),
+    hipLaunchKernelGGL((compact_kernel<IdT, T>), dim3(static_cast<unsigned>(tiles)), dim3(kThreads),
                        0, stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, lb,
                        box, box_ticket);
   }
@@ -383,13 +382,21 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
 // order, the frontiers are concatenated by batch, and every id is renamed to its
 // rank inside its own batch's frontier.
 //
-// The reference gives every batch a hash table of its own.  Here the items are
-// laid out virtually as [seeds_0, ids_0, seeds_1, ids_1, ...] (the order the
-// reference's prefix array has, batch_relabel.cu:152,163), the key is the pair
-// (batch, id) packed into 64 bits, and the single-table machinery above runs
-// once over all of them: one insert pass, one chained-scan compaction, one
-// lookup pass whatever the number of batches.
-constexpr int kBatchIdBits = 40;
+//  * The items are laid out virtually as [seeds_0, ids_0, seeds_1, ids_1, ...]
+//    (the order the reference's prefix array has, batch_relabel.cu:152,163), so
+//    one insert pass, one chained-scan compaction and one lookup pass serve all
+//    batches.
+//  * Like the reference, every batch hashes into a region of its own
+//    (batch_relabel.cu:243-256), here twice its item count, carved out of one
+//    array at 2 * start(b) with no size rounded to a power of two (the home slot
+//    is a multiply-high of the hash by the region length).  Regions matter for
+//    locality: consecutive items belong to the same batch, so the slots the chip
+//    is hammering at any moment span a few megabytes instead of the whole table
+//    (64 minibatches of layer 3: 270 MB), and the key needs no batch number, so
+//    32-bit ids keep the one-word (key | first index) slot and its single CAS.
+//  * A workgroup's items span one or two batches; it looks the range up once and
+//    its lanes search inside it.
+constexpr int64_t kRegionFactor = 2;
 
 template <typename IdT>
 struct BatchItems {
@@ -398,11 +405,9 @@ struct BatchItems {
   const IdT* ids;
   const int64_t* ids_ptr;
   int64_t B;
-  __device__ __forceinline__ int64_t items(int64_t host_items) const { return host_items; }
   __device__ __forceinline__ int64_t start(int64_t b) const { return seeds_ptr[b] + ids_ptr[b]; }
-  // batch of the item at position i of the interleaved layout
-  __device__ __forceinline__ int64_t batch_of(int64_t i) const {
-    int64_t lo = 0, hi = B;  // last b with start(b) <= i
+  // last b in [lo, hi] with start(b) <= i
+  __device__ __forceinline__ int64_t batch_of(int64_t i, int64_t lo, int64_t hi) const {
     while (lo < hi) {
       const int64_t mid = (lo + hi + 1) >> 1;
       if (start(mid) <= i) lo = mid; else hi = mid - 1;
@@ -414,36 +419,216 @@ struct BatchItems {
     const int64_t n_seeds = seeds_ptr[b + 1] - seeds_ptr[b];
     return off < n_seeds ? seeds[seeds_ptr[b] + off] : ids[ids_ptr[b] + off - n_seeds];
   }
-  __device__ __forceinline__ IdT get(int64_t i) const { return get_in(batch_of(i), i); }
-  __device__ __forceinline__ long long key(int64_t i) const {
-    const int64_t b = batch_of(i);
-    return static_cast<long long>((static_cast<unsigned long long>(b) << kBatchIdBits) |
-                                  static_cast<unsigned long long>(get_in(b, i)));
+  // batches of the first and the last item of a workgroup's range, through LDS
+  __device__ __forceinline__ void block_range(int64_t first, int64_t last, int64_t* lds2,
+                                              int64_t* lo, int64_t* hi) const {
+    if (threadIdx.x < 2) lds2[threadIdx.x] = batch_of(threadIdx.x == 0 ? first : last, 0, B - 1);
+    __syncthreads();
+    *lo = lds2[0];
+    *hi = lds2[1];
   }
 };
 
-// ids -> rank inside their batch's frontier; unique_ptr[b] = frontier offset of batch b
-template <typename IdT, typename T>
+__device__ __forceinline__ uint32_t hash32(unsigned long long key) {
+  return static_cast<uint32_t>((key * 0x9E3779B97F4A7C15ull) >> 32);
+}
+
+// one region per batch, slots (key << 32 | first index), all ones = empty
+struct PackedRegions {
+  unsigned long long* slots;
+  static size_t bytes(int64_t cap) { return padded(cap * 8); }
+  void carve(Carver& ws, int64_t cap) { slots = ws.take<unsigned long long>(cap); }
+  __device__ __forceinline__ void clear(int64_t i) const { slots[i] = ~0ull; }
+  __device__ __forceinline__ uint32_t insert(int64_t begin, int64_t len, long long key,
+                                             uint32_t i) const {
+    const unsigned long long hi = static_cast<unsigned long long>(static_cast<uint32_t>(key)) << 32;
+    const unsigned long long word = hi | i;
+    int64_t p = begin + static_cast<int64_t>((static_cast<unsigned long long>(hash32(
+                                                  static_cast<uint32_t>(key))) *
+                                              static_cast<unsigned long long>(len)) >>
+                                             32);
+    while (true) {
+      const unsigned long long prev = atomicCAS(&slots[p], ~0ull, word);
+      if (prev == ~0ull) break;
+      if ((prev >> 32) == (hi >> 32)) {
+        if (static_cast<uint32_t>(prev) > i) atomicMin(&slots[p], word);
+        break;
+      }
+      if (++p == begin + len) p = begin;
+    }
+    return static_cast<uint32_t>(p);
+  }
+  __device__ __forceinline__ uint32_t first_index(uint32_t p) const {
+    return static_cast<uint32_t>(slots[p]);
+  }
+};
+
+// the same with 64-bit keys: key array (-1 = empty) + first-index array
+struct WideRegions {
+  long long* keys;
+  int* vals;
+  static size_t bytes(int64_t cap) { return padded(cap * 8) + padded(cap * 4); }
+  void carve(Carver& ws, int64_t cap) {
+    keys = ws.take<long long>(cap);
+    vals = ws.take<int>(cap);
+  }
+  __device__ __forceinline__ void clear(int64_t i) const {
+    keys[i] = -1;
+    vals[i] = 0x7fffffff;
+  }
+  __device__ __forceinline__ uint32_t insert(int64_t begin, int64_t len, long long key,
+                                             uint32_t i) const {
+    int64_t p = begin + static_cast<int64_t>((static_cast<unsigned long long>(hash32(
+                                                  static_cast<unsigned long long>(key))) *
+                                              static_cast<unsigned long long>(len)) >>
+                                             32);
+    while (true) {
+      const unsigned long long prev =
+          atomicCAS(reinterpret_cast<unsigned long long*>(&keys[p]), ~0ull,
+                    static_cast<unsigned long long>(key));
+      if (prev == ~0ull || prev == static_cast<unsigned long long>(key)) break;
+      if (++p == begin + len) p = begin;
+    }
+    if (__atomic_load_n(&vals[p], __ATOMIC_RELAXED) > static_cast<int>(i))
+      atomicMin(&vals[p], static_cast<int>(i));
+    return static_cast<uint32_t>(p);
+  }
+  __device__ __forceinline__ uint32_t first_index(uint32_t p) const {
+    return static_cast<uint32_t>(vals[p]);
+  }
+};
+
+template <typename IdT>
+struct RegionsFor {
+  using type = WideRegions;
+};
+template <>
+struct RegionsFor<int32_t> {
+  using type = PackedRegions;
+};
+
+template <typename R>
+__global__ void __launch_bounds__(kThreads) regions_init_kernel(R t, int64_t cap, LookbackState lb,
+                                                                int64_t tiles) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < cap) t.clear(i);
+  if (i < tiles) lb.status[i] = 0ull;
+  if (i == 0) *lb.error = 0u;
+}
+
+template <typename IdT, typename R>
 __global__ void __launch_bounds__(kThreads)
-batch_finish_kernel(BatchItems<IdT> x, int64_t num_ids, T t, const uint32_t* __restrict__ pos,
-                    const int64_t* __restrict__ prefix, const int64_t* __restrict__ num_unique,
-                    IdT* __restrict__ out_ids, int64_t* __restrict__ unique_ptr) {
-  const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  const int64_t M = x.seeds_ptr[x.B] + x.ids_ptr[x.B];
-  if (j < num_ids) {
-    int64_t lo = 0, hi = x.B;  // last b with ids_ptr[b] <= j
+batch_insert_kernel(BatchItems<IdT> x, int64_t M, R t, uint32_t* __restrict__ pos) {
+  __shared__ int64_t s_range[2];
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads;
+  const int64_t last = first + kThreads - 1 < M ? first + kThreads - 1 : M - 1;
+  int64_t lo, hi;
+  x.block_range(first, last, s_range, &lo, &hi);
+  const int64_t i = first + threadIdx.x;
+  if (i >= M) return;
+  const int64_t b = x.batch_of(i, lo, hi);
+  const int64_t begin = x.start(b);
+  pos[i] = t.insert(kRegionFactor * begin, kRegionFactor * (x.start(b + 1) - begin),
+                    static_cast<long long>(x.get_in(b, i)), static_cast<uint32_t>(i));
+}
+
+// flags, chained scan and compaction over all batches at once (see compact_kernel)
+template <typename IdT, typename R>
+__global__ void __launch_bounds__(kThreads)
+batch_compact_kernel(BatchItems<IdT> x, int64_t M, R t, const uint32_t* __restrict__ pos,
+                     int64_t* __restrict__ prefix, IdT* __restrict__ unique,
+                     int64_t* __restrict__ num_unique, LookbackState lb, gs_mailbox* box,
+                     int64_t box_ticket) {
+  __shared__ int64_t s_scan[kThreads / kWave + 1];
+  __shared__ int64_t s_prefix;
+  __shared__ int64_t s_range[2];
+  const unsigned int tile = blockIdx.x;
+  const int64_t tile_first = static_cast<int64_t>(tile) * kCompactTile;
+  const int64_t tile_last = tile_first + kCompactTile - 1 < M ? tile_first + kCompactTile - 1 : M - 1;
+  int64_t lo = 0, hi = 0;
+  if (M > 0) x.block_range(tile_first, tile_last, s_range, &lo, &hi);
+  const int64_t base = tile_first + static_cast<int64_t>(threadIdx.x) * kCompactItems;
+  bool first[kCompactItems];
+  int64_t mine = 0;
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) {
+    const int64_t i = base + k;
+    first[k] = i < M && t.first_index(pos[i]) == static_cast<uint32_t>(i);
+    mine += first[k] ? 1 : 0;
+  }
+  int64_t tile_total;
+  const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
+  if (threadIdx.x == 0) lookback_publish_sum(lb, tile, tile_total);
+  IdT key[kCompactItems];  // in flight while wave 0 walks back
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k)
+    key[k] = first[k] ? x.get_in(x.batch_of(base + k, lo, hi), base + k) : IdT(0);
+  if (threadIdx.x < kWave) {
+    const int64_t before = lookback_exclusive_prefix(lb, tile, tile_total);
+    if (threadIdx.x == 0) s_prefix = before;
+  }
+  __syncthreads();
+  int64_t run = s_prefix + local;
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) {
+    const int64_t i = base + k;
+    if (i < M) {
+      prefix[i] = run;
+      if (first[k]) unique[run] = key[k];
+    }
+    run += first[k] ? 1 : 0;
+  }
+  if (tile == gridDim.x - 1 && threadIdx.x == 0) {
+    int64_t total = s_prefix + tile_total;
+    if (__hip_atomic_load(lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) total = -1;
+    *num_unique = total;
+    post_mailbox(box, total, box_ticket);
+  }
+}
+
+// ids -> rank inside their batch's frontier; unique_ptr[b] = frontier offset of batch b
+template <typename IdT, typename R>
+__global__ void __launch_bounds__(kThreads)
+batch_finish_kernel(BatchItems<IdT> x, int64_t num_ids, int64_t M, R t,
+                    const uint32_t* __restrict__ pos, const int64_t* __restrict__ prefix,
+                    const int64_t* __restrict__ num_unique, IdT* __restrict__ out_ids,
+                    int64_t* __restrict__ unique_ptr) {
+  __shared__ int64_t s_range[2];
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads;
+  if (first < num_ids) {  // a workgroup of id lookups
+    const int64_t last = first + kThreads - 1 < num_ids ? first + kThreads - 1 : num_ids - 1;
+    if (threadIdx.x < 2) {
+      const int64_t j = threadIdx.x == 0 ? first : last;
+      int64_t lo = 0, hi = x.B - 1;  // last b with ids_ptr[b] <= j
+      while (lo < hi) {
+        const int64_t mid = (lo + hi + 1) >> 1;
+        if (x.ids_ptr[mid] <= j) lo = mid; else hi = mid - 1;
+      }
+      s_range[threadIdx.x] = lo;
+    }
+    __syncthreads();
+    const int64_t j = first + threadIdx.x;
+    if (j >= num_ids) return;
+    int64_t lo = s_range[0], hi = s_range[1];
     while (lo < hi) {
       const int64_t mid = (lo + hi + 1) >> 1;
       if (x.ids_ptr[mid] <= j) lo = mid; else hi = mid - 1;
     }
     const int64_t b = lo;
-    const int64_t p = x.start(b) + (x.seeds_ptr[b + 1] - x.seeds_ptr[b]) + (j - x.ids_ptr[b]);
-    const int64_t base = x.start(b) < M ? prefix[x.start(b)] : *num_unique;
-    out_ids[j] = static_cast<IdT>(prefix[t.first_index(pos[p])] - base);
+    const int64_t begin = x.start(b);
+    const int64_t p = begin + (x.seeds_ptr[b + 1] - x.seeds_ptr[b]) + (j - x.ids_ptr[b]);
+    out_ids[j] = static_cast<IdT>(prefix[t.first_index(pos[p])] - prefix[begin]);
     return;
   }
-  const int64_t b = j - num_ids;
+  const int64_t b = first + threadIdx.x - (num_ids + kThreads - 1) / kThreads * kThreads;
   if (b <= x.B) unique_ptr[b] = x.start(b) < M ? prefix[x.start(b)] : *num_unique;
+}
+
+template <typename IdT>
+size_t batch_workspace_bytes_for(int64_t M) {
+  using R = typename RegionsFor<IdT>::type;
+  return R::bytes(kRegionFactor * (M > 0 ? M : 1)) + padded((M > 0 ? M : 1) * 4) +
+         padded((M + 1) * 8) + lookback_state_bytes(compact_num_tiles(M));
 }
 
 template <typename IdT>
@@ -452,11 +637,11 @@ int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* 
                        void* unique, int64_t* unique_ptr, void* out_ids, int64_t* num_unique,
                        void* workspace, size_t workspace_bytes, gs_mailbox* box,
                        int64_t box_ticket, hipStream_t stream) {
-  using T = WideTable;
+  using R = typename RegionsFor<IdT>::type;
   const int64_t M = num_seeds + num_ids;
-  const int64_t cap = table_capacity(M);
+  const int64_t cap = kRegionFactor * (M > 0 ? M : 1);
   Carver ws(workspace, workspace_bytes);
-  T t;
+  R t;
   t.carve(ws, cap);
   uint32_t* pos = ws.take<uint32_t>(M > 0 ? M : 1);
   int64_t* prefix = ws.take<int64_t>(M + 1);
@@ -464,26 +649,24 @@ int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* 
   LookbackState lb = carve_lookback(ws, tiles, 1u);
   if (!ws.ok) {
     set_error_text("gs_batch_csr_relabel: workspace needs %zu bytes, 256-byte aligned",
-                   gs_unique_workspace_bytes(M));
+                   batch_workspace_bytes_for<IdT>(M));
     return GS_ERR_WORKSPACE;
   }
-  t.mask = static_cast<uint32_t>(cap - 1);
-  int lg = 0;
-  while ((int64_t(1) << lg) < cap) ++lg;
-  t.shift = 64 - lg;
   BatchItems<IdT> x{static_cast<const IdT*>(seeds), seeds_ptr, static_cast<const IdT*>(ids), ids_ptr,
                     B};
   const int64_t n_init = cap > tiles ? cap : tiles;
-  hipLaunchKernelGGL((table_init_kernel<T>), dim3(blocks_for(n_init, kThreads)), dim3(kThreads), 0,
-                     stream, t, cap, lb, tiles);
+  hipLaunchKernelGGL((regions_init_kernel<R>), dim3(blocks_for(n_init, kThreads)), dim3(kThreads),
+                     0, stream, t, cap, lb, tiles);
   if (M > 0)
-    hipLaunchKernelGGL((table_insert_kernel<BatchItems<IdT>, T>), dim3(blocks_for(M, kThreads)),
-                       dim3(kThreads), 0, stream, x, M, t, pos);
-  hipLaunchKernelGGL((compact_kernel<IdT, BatchItems<IdT>, T>), dim3(static_cast<unsigned>(tiles)),
+    hipLaunchKernelGGL((batch_insert_kernel<IdT, R>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
+                       0, stream, x, M, t, pos);
+  hipLaunchKernelGGL((batch_compact_kernel<IdT, R>), dim3(static_cast<unsigned>(tiles)),
                      dim3(kThreads), 0, stream, x, M, t, pos, prefix, static_cast<IdT*>(unique),
                      num_unique, lb, box, box_ticket);
-  hipLaunchKernelGGL((batch_finish_kernel<IdT, T>), dim3(blocks_for(num_ids + B + 1, kThreads)),
-                     dim3(kThreads), 0, stream, x, num_ids, t, pos, prefix, num_unique,
+  const int64_t id_blocks = (num_ids + kThreads - 1) / kThreads;
+  const int64_t ptr_blocks = (B + 1 + kThreads - 1) / kThreads;
+  hipLaunchKernelGGL((batch_finish_kernel<IdT, R>), dim3(static_cast<unsigned>(id_blocks + ptr_blocks)),
+                     dim3(kThreads), 0, stream, x, num_ids, M, t, pos, prefix, num_unique,
                      static_cast<IdT*>(out_ids), unique_ptr);
   return check_launch("batch_csr_relabel");
 }
@@ -553,6 +736,13 @@ int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* quer
                                   stream);
 }
 
+size_t gs_batch_relabel_workspace_bytes(int64_t num_items) {
+  if (num_items < 0) num_items = 0;
+  const size_t a = batch_workspace_bytes_for<int64_t>(num_items);
+  const size_t b = batch_workspace_bytes_for<int32_t>(num_items);
+  return a > b ? a : b;
+}
+
 int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void* ids,
                          const int64_t* ids_ptr, int64_t num_batches, int64_t num_seeds,
                          int64_t num_ids, int id_bytes, void* unique, int64_t* unique_ptr,
@@ -567,8 +757,9 @@ int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void
              "gs_batch_csr_relabel: null buffer");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_batch_csr_relabel: id_bytes must be 4 or 8, got %d",
              id_bytes);
-  if (num_batches >= (int64_t(1) << (63 - kBatchIdBits)) || num_seeds + num_ids >= (int64_t(1) << 30)) {
-    set_error_text("gs_batch_csr_relabel: at most 2^%d batches and 2^30 items", 63 - kBatchIdBits);
+  if (num_seeds + num_ids >= (int64_t(1) << 30)) {
+    set_error_text("gs_batch_csr_relabel: %lld items exceed the supported 2^30",
+                   static_cast<long long>(num_seeds + num_ids));
     return GS_ERR_UNSUPPORTED;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);

@@ -443,7 +443,7 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(
   auto unique_ptr = torch::empty({B + 1}, I64(seeds));
   auto out_ids = torch::empty_like(ids);
   auto num = torch::empty({1}, I64(seeds));
-  auto ws = Scratch(gs_unique_workspace_bytes(M), seeds);
+  auto ws = Scratch(gs_batch_relabel_workspace_bytes(M), seeds);
   void* st = Stream(seeds);
   HostBoxes& boxes = Boxes(seeds.device().index());
   const int64_t ticket = boxes.next++;

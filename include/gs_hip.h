@@ -276,7 +276,8 @@ int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_spa
  * each the distinct values of (its seeds, then its ids) in first-occurrence order;
  * unique_ptr[num_batches+1] = their offsets; out_ids[j] = rank of ids[j] inside its own
  * batch's frontier; *num_unique (and the mailbox, when given) = total frontier length.
- * Ids must lie in [0, 2^40).  Workspace: gs_unique_workspace_bytes(num_seeds+num_ids). */
+ * Ids must not be -1.  Workspace: gs_batch_relabel_workspace_bytes(num_seeds+num_ids). */
+size_t gs_batch_relabel_workspace_bytes(int64_t num_items);
 int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void* ids,
                          const int64_t* ids_ptr, int64_t num_batches, int64_t num_seeds,
                          int64_t num_ids, int id_bytes, void* unique, int64_t* unique_ptr,
