@@ -32,7 +32,7 @@ def lib():
                      "gs_sample_weighted_workspace_bytes", "gs_list_sample_workspace_bytes",
                      "gs_unique_workspace_bytes", "gs_row_slice_workspace_bytes",
                      "gs_sample_fused_state_bytes", "gs_batch_relabel_workspace_bytes",
-                     "gs_coo2csc_workspace_bytes"):
+                     "gs_coo2csc_workspace_bytes", "gs_col_row_slice_workspace_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
     return _lib
@@ -575,6 +575,43 @@ def row_slice_coo(key, other, ids):
                                           _ptr(out_other), _ptr(select_index), _ptr(ws),
                                           ctypes.c_size_t(ws.numel()), st), "gs_row_slice_coo_compact")
     return out_key, out_other, select_index
+
+
+def col_row_slice(indptr, indices, column_ids, row_ids, col_ptr=None, row_ptr=None,
+                  encoding_size=0):
+    """gs_slice_count + gs_col_row_slice_{mark,compact}; returns (out_indptr, out_indices,
+    select_index (position in the virtual column slice), parent_index (position in indices))."""
+    _need(indptr, torch.int64, "indptr")
+    idb = _ids(indices, "indices")
+    _ids(column_ids, "column_ids", like=indices)
+    _ids(row_ids, "row_ids", like=indices)
+    dev = indptr.device
+    S, nr = column_ids.numel(), row_ids.numel()
+    B = 0
+    if col_ptr is not None:
+        _need(col_ptr, torch.int64, "col_ptr")
+        _need(row_ptr, torch.int64, "row_ptr")
+        B = col_ptr.numel() - 1
+    sub_indptr = slice_count(indptr, column_ids)
+    D = int(sub_indptr[-1].item())
+    out_indptr = torch.empty(S + 1, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_col_row_slice_workspace_bytes(_i64(nr), _i64(D)), dev)
+    st = _stream(dev)
+    _check(lib().gs_col_row_slice_mark(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), idb,
+                                       _ptr(column_ids), _i64(S), _ptr(sub_indptr), _i64(D),
+                                       _ptr(row_ids), _i64(nr), _ptr(col_ptr), _ptr(row_ptr),
+                                       _i64(B), _i64(encoding_size), _ptr(out_indptr), _ptr(ws),
+                                       ctypes.c_size_t(ws.numel()), st), "gs_col_row_slice_mark")
+    kept = int(out_indptr[-1].item())
+    out_indices = torch.empty(kept, dtype=indices.dtype, device=dev)
+    select_index = torch.empty(kept, dtype=torch.int64, device=dev)
+    parent_index = torch.empty(kept, dtype=torch.int64, device=dev)
+    if kept > 0:
+        _check(lib().gs_col_row_slice_compact(_i64(D), idb, _ptr(out_indices), _ptr(select_index),
+                                              _ptr(parent_index), _ptr(ws),
+                                              ctypes.c_size_t(ws.numel()), st),
+               "gs_col_row_slice_compact")
+    return out_indptr, out_indices, select_index, parent_index
 
 
 # ------------------------------------------------------- format transform ----

@@ -161,8 +161,105 @@ coo_compact_kernel(const IdT* __restrict__ other, int64_t E, const int64_t* __re
   select_index[w] = e;
 }
 
-// Workspace layout: [val | prefix | scan tiles | id-set].  The first three
-// depend on the edge count only, so the compact call finds them again without
+// ------------------------------------------- column slice + row slice in one go ----
+// Induced-subgraph slicing: of the columns `cols`, keep the edges whose row is in the id
+// set (reference src/cuda/fusion/column_row_slicing.cu:102-211; batched :225-355).  The
+// column slice is never materialised: position p of the virtual sliced edge array is
+// resolved to its column by binary search in the slice offsets (staged in LDS when the
+// workgroup's 2048 positions span few columns) and to its position in the parent's
+// indices from there; that parent position is kept for the compaction.
+//
+// Batched flavour (B > 0): columns and ids are cut into B batches at col_ptr / id_ptr; a
+// column of batch b keeps the rows found in batch b's ids.  The table key is
+// id + b * encoding_size and the value the id itself (rows keep their global id,
+// column_row_slicing.cu:272), exactly as the reference composes it.
+template <typename IdT>
+__global__ void __launch_bounds__(kThreads)
+set_insert_batched_kernel(IdSet t, const IdT* __restrict__ ids, int64_t n,
+                          const int64_t* __restrict__ id_ptr, int64_t B, int64_t enc) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= n) return;
+  const int64_t b = upper_bound(id_ptr, B + 1, i) - 1;
+  if (b < 0 || b >= B) return;
+  const long long id = static_cast<long long>(ids[i]);
+  const long long key = id + b * enc;
+  if (key == -1) return;
+  uint32_t p = t.home(key);
+  while (true) {
+    const unsigned long long prev =
+        atomicCAS(reinterpret_cast<unsigned long long*>(&t.keys[p]), ~0ull,
+                  static_cast<unsigned long long>(key));
+    if (prev == ~0ull || prev == static_cast<unsigned long long>(key)) break;
+    p = (p + 1) & t.mask;
+  }
+  atomicMax(&t.vals[p], id);
+}
+
+template <typename IdT>
+__global__ void __launch_bounds__(kThreads)
+sliced_mark_kernel(IdSet t, const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
+                   const IdT* __restrict__ cols, int64_t S, const int64_t* __restrict__ sub_indptr,
+                   int64_t D, const int64_t* __restrict__ col_ptr, int64_t B, int64_t enc,
+                   int64_t* __restrict__ val, int64_t* __restrict__ src) {
+  __shared__ int64_t s_ptr[kStage + 1];
+  __shared__ int64_t s_rows[2];
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
+  const int64_t p1 = p0 + kTile < D ? p0 + kTile : D;
+  if (threadIdx.x < 2)
+    s_rows[threadIdx.x] = upper_bound(sub_indptr, S + 1, threadIdx.x == 0 ? p0 : p1 - 1) - 1;
+  __syncthreads();
+  const int64_t row_lo = s_rows[0];
+  const int64_t nrows = s_rows[1] - row_lo + 1;
+  const bool staged = nrows <= kStage;
+  if (staged)
+    for (int64_t i = threadIdx.x; i <= nrows; i += kThreads) s_ptr[i] = sub_indptr[row_lo + i];
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t p = p0 + k * kThreads + threadIdx.x;
+    if (p >= p1) break;
+    const int64_t lr = (staged ? upper_bound(s_ptr, nrows + 1, p)
+                               : upper_bound(sub_indptr + row_lo, nrows + 1, p)) - 1;
+    const int64_t r = row_lo + lr;
+    const int64_t first = staged ? s_ptr[lr] : sub_indptr[r];
+    // a column that owns a position of the slice has passed the range check of the count
+    const int64_t c = static_cast<int64_t>(cols[r]);
+    const int64_t q = indptr[c] + (p - first);
+    const long long id = static_cast<long long>(indices[q]);
+    src[p] = q;
+    if (B > 0) {
+      const int64_t b = upper_bound(col_ptr, B + 1, r) - 1;
+      val[p] = (b >= 0 && b < B && t.query(id + b * enc) >= 0) ? id : -1;
+    } else {
+      val[p] = t.query(id);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+sliced_indptr_kernel(const int64_t* __restrict__ sub_indptr, int64_t S,
+                     const int64_t* __restrict__ prefix, int64_t* __restrict__ out_indptr) {
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (r <= S) out_indptr[r] = prefix[sub_indptr[r]];
+}
+
+template <typename IdT>
+__global__ void __launch_bounds__(kThreads)
+sliced_compact_kernel(int64_t D, const int64_t* __restrict__ val, const int64_t* __restrict__ prefix,
+                      const int64_t* __restrict__ src, IdT* __restrict__ out_indices,
+                      int64_t* __restrict__ select_index, int64_t* __restrict__ parent_index) {
+  const int64_t p = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (p >= D) return;
+  const int64_t v = val[p];
+  if (v < 0) return;
+  const int64_t w = prefix[p];
+  out_indices[w] = static_cast<IdT>(v);
+  if (select_index) select_index[w] = p;
+  if (parent_index) parent_index[w] = src[p];
+}
+
+// Workspace layout: [val | prefix | scan tiles | (parent positions) | id-set].  All but
+// the last depend on the edge count only, so the compact call finds them again without
 // knowing how many ids the mark call was given.
 struct Scratch {
   IdSet set;
@@ -170,15 +267,18 @@ struct Scratch {
   int64_t* val;
   int64_t* prefix;
   int64_t* tiles;
+  int64_t* src;
   bool ok;
 };
 
-Scratch carve(void* workspace, size_t bytes, int64_t n_ids, int64_t E, bool with_set) {
+Scratch carve(void* workspace, size_t bytes, int64_t n_ids, int64_t E, bool with_set,
+              bool with_src = false) {
   Scratch s;
   Carver ws(workspace, bytes);
   s.val = ws.take<int64_t>(E > 0 ? E : 1);
   s.prefix = ws.take<int64_t>(E + 1);
   s.tiles = ws.take<int64_t>(scan_num_tiles(E) + 1);
+  s.src = with_src ? ws.take<int64_t>(E > 0 ? E : 1) : nullptr;
   s.cap = 0;
   if (with_set) {
     s.cap = set_capacity(n_ids);
@@ -334,6 +434,90 @@ int gs_row_slice_coo_compact(const void* other, int id_bytes, int64_t E, void* o
                        static_cast<int32_t*>(out_key), static_cast<int32_t*>(out_other),
                        select_index);
   return check_launch("row_slice_coo_compact");
+}
+
+size_t gs_col_row_slice_workspace_bytes(int64_t num_row_ids, int64_t D) {
+  if (D < 0) D = 0;
+  return gs_row_slice_workspace_bytes(num_row_ids, D, 0) + padded((D > 0 ? D : 1) * 8);
+}
+
+int gs_col_row_slice_mark(const int64_t* indptr, int64_t num_cols, const void* indices,
+                          int id_bytes, const void* column_ids, int64_t S,
+                          const int64_t* sub_indptr, int64_t D, const void* row_ids,
+                          int64_t num_row_ids, const int64_t* col_batch_ptr,
+                          const int64_t* row_batch_ptr, int64_t num_batches,
+                          int64_t encoding_size, int64_t* out_indptr, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  (void)num_cols;
+  GS_REQUIRE(S >= 0 && D >= 0 && num_row_ids >= 0 && num_batches >= 0,
+             "gs_col_row_slice_mark: negative size");
+  GS_REQUIRE(indptr && sub_indptr && out_indptr && (D == 0 || indices) && (S == 0 || column_ids) &&
+                 (num_row_ids == 0 || row_ids),
+             "gs_col_row_slice_mark: null pointer");
+  GS_REQUIRE(num_batches == 0 || (col_batch_ptr && row_batch_ptr && encoding_size > 0),
+             "gs_col_row_slice_mark: a batched call needs both batch offsets and an encoding size");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_col_row_slice_mark: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  Scratch s = carve(workspace, workspace_bytes, num_row_ids, D, true, true);
+  if (!s.ok) {
+    set_error_text("gs_col_row_slice_mark: workspace needs %zu bytes, 256-byte aligned",
+                   gs_col_row_slice_workspace_bytes(num_row_ids, D));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(s.cap, kThreads)), dim3(kThreads), 0, st,
+                     s.set, s.cap);
+  auto run = [&](auto tag) {
+    using IdT = decltype(tag);
+    const IdT* ids = static_cast<const IdT*>(row_ids);
+    if (num_row_ids > 0) {
+      if (num_batches > 0)
+        hipLaunchKernelGGL(set_insert_batched_kernel<IdT>, dim3(blocks_for(num_row_ids, kThreads)),
+                           dim3(kThreads), 0, st, s.set, ids, num_row_ids, row_batch_ptr,
+                           num_batches, encoding_size);
+      else
+        hipLaunchKernelGGL(set_insert_kernel<IdT>, dim3(blocks_for(num_row_ids, kThreads)),
+                           dim3(kThreads), 0, st, s.set, ids, num_row_ids);
+    }
+    if (D > 0)
+      hipLaunchKernelGGL(sliced_mark_kernel<IdT>, dim3(blocks_for(D, kTile)), dim3(kThreads), 0, st,
+                         s.set, indptr, static_cast<const IdT*>(indices),
+                         static_cast<const IdT*>(column_ids), S, sub_indptr, D, col_batch_ptr,
+                         num_batches, encoding_size, s.val, s.src);
+  };
+  if (id_bytes == 8) run(int64_t{}); else run(int32_t{});
+  GS_RETURN_IF_ERROR(check_launch("col_row_slice_mark"));
+  Kept f{s.val};
+  GS_RETURN_IF_ERROR(exclusive_scan(f, D, s.prefix, s.tiles, st));
+  hipLaunchKernelGGL(sliced_indptr_kernel, dim3(blocks_for(S + 1, kThreads)), dim3(kThreads), 0, st,
+                     sub_indptr, S, s.prefix, out_indptr);
+  return check_launch("col_row_slice_mark");
+}
+
+int gs_col_row_slice_compact(int64_t D, int id_bytes, void* out_indices, int64_t* select_index,
+                             int64_t* parent_index, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+  GS_REQUIRE(D >= 0, "gs_col_row_slice_compact: negative size");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_col_row_slice_compact: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  if (D == 0) return GS_OK;
+  GS_REQUIRE(out_indices, "gs_col_row_slice_compact: null output");
+  Scratch s = carve(workspace, workspace_bytes, 0, D, false, true);
+  if (!s.ok) {
+    set_error_text("gs_col_row_slice_compact: pass the workspace given to gs_col_row_slice_mark");
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid(blocks_for(D, kThreads));
+  if (id_bytes == 8)
+    hipLaunchKernelGGL(sliced_compact_kernel<int64_t>, grid, dim3(kThreads), 0, st, D, s.val,
+                       s.prefix, s.src, static_cast<int64_t*>(out_indices), select_index,
+                       parent_index);
+  else
+    hipLaunchKernelGGL(sliced_compact_kernel<int32_t>, grid, dim3(kThreads), 0, st, D, s.val,
+                       s.prefix, s.src, static_cast<int32_t*>(out_indices), select_index,
+                       parent_index);
+  return check_launch("col_row_slice_compact");
 }
 
 }  // extern "C"

@@ -36,6 +36,9 @@ TORCH_LIBRARY(gs_classes, m) {
       GS_DEF2("_CAPI_SamplingWithProbs", "_CAPI_sampling_with_probs", &Graph::SamplingProbs)
       GS_DEF2("_CAPI_FusedColumnwiseSlicingSampling", "_CAPI_fused_columnwise_slicing_sampling",
               &Graph::ColumnwiseFusedSlicingAndSampling)
+      GS_DEF2("_CAPI_FusionSlicing", "_CAPI_fusion_slicing", &Graph::FusedBidirSlicing)
+      GS_DEF2("_CAPI_BatchFusionSlicing", "_CAPI_batch_fusion_slicing",
+              &Graph::BatchFusedBidirSlicing)
       GS_DEF2("_CAPI_LoadCSC", "_CAPI_load_csc", &Graph::LoadCSC)
       GS_DEF2("_CAPI_LoadCSR", "_CAPI_load_csr", &Graph::LoadCSR)
       GS_DEF2("_CAPI_LoadCOO", "_CAPI_load_coo", &Graph::LoadCOO)

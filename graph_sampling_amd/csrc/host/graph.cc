@@ -368,6 +368,43 @@ c10::intrusive_ptr<Graph> Graph::ColumnwiseFusedSlicingAndSampling(torch::Tensor
   return ret;
 }
 
+// The reference hands the kernel the GLOBAL ids of the seeds (src/graph.cc:120-128), which
+// only works on a graph without id maps, and gathers the parent's edge data with positions
+// of the virtual column slice (:131-137).  Here the kernel gets the local seeds and edge
+// data follows the position in the parent's indices.
+c10::intrusive_ptr<Graph> Graph::FusedBidirSlicing(torch::Tensor column_seeds,
+                                                   torch::Tensor row_seeds) {
+  Settle();
+  CreateSparseFormat(_CSC);
+  auto ret = Child(Pick(col_ids_, column_seeds), Pick(row_ids_, row_seeds), column_seeds.numel(),
+                   row_seeds.numel());
+  std::shared_ptr<CSC> sliced;
+  torch::Tensor select_index, parent_index;
+  std::tie(sliced, select_index) =
+      FusedCSCColRowSlicing(csc_, column_seeds, row_seeds, &parent_index);
+  ret->SetCSC(sliced);
+  ret->SetNumEdges(sliced->indices.numel());
+  InheritData(ret.get(), csc_->e_ids, parent_index);
+  return ret;
+}
+
+c10::intrusive_ptr<Graph> Graph::BatchFusedBidirSlicing(torch::Tensor column_seeds,
+                                                        torch::Tensor col_ptr,
+                                                        torch::Tensor row_seeds,
+                                                        torch::Tensor row_ptr) {
+  Settle();
+  CreateSparseFormat(_CSC);
+  auto ret = Child(Pick(col_ids_, column_seeds), row_ids_, column_seeds.numel(), num_rows_);
+  auto sliced = std::make_shared<CSC>();
+  torch::Tensor select_index, parent_index;
+  std::tie(sliced->indptr, sliced->indices, select_index, parent_index) = hip::ColRowSlicing(
+      csc_->indptr, csc_->indices, column_seeds, row_seeds, col_ptr, row_ptr, num_rows_);
+  ret->SetCSC(sliced);
+  ret->SetNumEdges(sliced->indices.numel());
+  InheritData(ret.get(), csc_->e_ids, parent_index);
+  return ret;
+}
+
 torch::Tensor Graph::RandomWalk(torch::Tensor seeds, int64_t walk_length) {
   Settle();
   TORCH_CHECK(csc_ != nullptr, "random walks need the CSC format");

@@ -2,10 +2,9 @@
 //
 // Public API (names, signatures, return orders) follows the reference's
 // src/graph.h:11-128 for everything on the sampling hot path: loading, format
-// caches, slicing, uniform / weighted / fused sampling, relabel, valid-node
-// queries, walks, Sum / Normalize / Divide / EDivUSum and SDDMM.  The batched
-// ("super-batch") methods, FusedBidirSlicing and the doubly-compressed formats
-// are not part of this build and raise a clear error when requested.
+// caches, slicing, uniform / weighted / fused sampling, induced-subgraph slicing,
+// relabel, valid-node queries, walks, Sum / Normalize / Divide / EDivUSum and SDDMM,
+// and the batched ("super-batch") methods.
 //
 // A Graph keeps up to three cached formats of one matrix (CSC, CSR, COO), the
 // edge data, and the global ids of its local columns / rows.  Children share
@@ -105,6 +104,13 @@ class Graph : public torch::CustomClassHolder {
                                           bool replace, int64_t on_format, int64_t output_format);
   c10::intrusive_ptr<Graph> ColumnwiseFusedSlicingAndSampling(torch::Tensor column_index,
                                                               int64_t fanout, bool replace);
+  // induced subgraph: columns column_seeds, rows row_seeds (renamed to their position in
+  // row_seeds), CSC only (reference src/graph.cc:116-141)
+  c10::intrusive_ptr<Graph> FusedBidirSlicing(torch::Tensor column_seeds, torch::Tensor row_seeds);
+  // one induced subgraph per batch, columns and rows cut at col_ptr / row_ptr; rows keep
+  // their ids (reference src/graph.cc:143-171)
+  c10::intrusive_ptr<Graph> BatchFusedBidirSlicing(torch::Tensor column_seeds, torch::Tensor col_ptr,
+                                                   torch::Tensor row_seeds, torch::Tensor row_ptr);
   torch::Tensor RandomWalk(torch::Tensor seeds, int64_t walk_length);
 
   // ---- edge-data operators

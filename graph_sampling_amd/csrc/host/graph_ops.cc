@@ -74,6 +74,17 @@ std::pair<std::shared_ptr<CSC>, torch::Tensor> FusedCSCColSlicingAndSampling(
   return {out, select_index};
 }
 
+std::pair<std::shared_ptr<CSC>, torch::Tensor> FusedCSCColRowSlicing(
+    std::shared_ptr<CSC> csc, torch::Tensor column_ids, torch::Tensor row_ids,
+    torch::Tensor* parent_index) {
+  auto out = std::make_shared<CSC>();
+  torch::Tensor select_index, parent;
+  std::tie(out->indptr, out->indices, select_index, parent) =
+      hip::ColRowSlicing(csc->indptr, csc->indices, column_ids, row_ids);
+  if (parent_index) *parent_index = parent;
+  return {out, select_index};
+}
+
 torch::Tensor TensorUnique(torch::Tensor node_ids) { return hip::Unique(node_ids); }
 
 std::tuple<torch::Tensor, std::vector<torch::Tensor>> BatchTensorRelabel(

@@ -39,6 +39,13 @@ std::pair<std::shared_ptr<_TMP>, torch::Tensor> CSCColSamplingProbs(std::shared_
 std::pair<std::shared_ptr<CSC>, torch::Tensor> FusedCSCColSlicingAndSampling(
     std::shared_ptr<CSC> csc, torch::Tensor node_ids, int64_t fanout, bool replace);
 
+// {CSC of the induced subgraph, select_index}.  select_index holds positions in the virtual
+// column slice, as the reference's does (src/cuda/fusion/column_row_slicing.cu:204-209);
+// parent_index, when asked for, receives the positions in csc->indices.
+std::pair<std::shared_ptr<CSC>, torch::Tensor> FusedCSCColRowSlicing(
+    std::shared_ptr<CSC> csc, torch::Tensor column_ids, torch::Tensor row_ids,
+    torch::Tensor* parent_index = nullptr);
+
 torch::Tensor TensorUnique(torch::Tensor node_ids);
 
 std::tuple<torch::Tensor, std::vector<torch::Tensor>> BatchTensorRelabel(

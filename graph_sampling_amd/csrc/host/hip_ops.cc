@@ -640,6 +640,51 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(const torc
   return {out_key, out_other, select_index};
 }
 
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ColRowSlicing(
+    const torch::Tensor& indptr, const torch::Tensor& indices, const torch::Tensor& column_ids,
+    const torch::Tensor& row_ids, const torch::optional<torch::Tensor>& col_ptr,
+    const torch::optional<torch::Tensor>& row_ptr, int64_t encoding_size) {
+  NeedI64(indptr, "indptr");
+  const int idb = IdBytes(indices, "indices");
+  TORCH_CHECK(IdBytes(column_ids, "column ids") == idb && IdBytes(row_ids, "row ids") == idb,
+              "column ids, row ids and indices differ in dtype");
+  const int64_t S = column_ids.numel(), nr = row_ids.numel(), ncols = indptr.numel() - 1;
+  const bool batched = col_ptr.has_value();
+  TORCH_CHECK(batched == row_ptr.has_value(), "column and row batch offsets come together");
+  int64_t B = 0;
+  if (batched) {
+    B = col_ptr.value().numel() - 1;
+    TORCH_CHECK(row_ptr.value().numel() == B + 1, "column and row batch offsets differ in length");
+    TORCH_CHECK(encoding_size > 0, "a batched slice needs a positive encoding size");
+  }
+  void* st = Stream(indptr);
+  auto sub_indptr = torch::empty({S + 1}, I64(indptr));
+  {
+    auto ws = Scratch(gs_slice_workspace_bytes(S), indptr);
+    Check(gs_slice_count(indptr.data_ptr<int64_t>(), ncols, column_ids.data_ptr(), idb, S,
+                         sub_indptr.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
+          "gs_slice_count");
+  }
+  const int64_t D = sub_indptr[S].item<int64_t>();
+  auto out_indptr = torch::empty({S + 1}, I64(indptr));
+  auto ws = Scratch(gs_col_row_slice_workspace_bytes(nr, D), indptr);
+  Check(gs_col_row_slice_mark(indptr.data_ptr<int64_t>(), ncols, indices.data_ptr(), idb,
+                              column_ids.data_ptr(), S, sub_indptr.data_ptr<int64_t>(), D,
+                              row_ids.data_ptr(), nr, OptI64(col_ptr, "column batch offsets"),
+                              OptI64(row_ptr, "row batch offsets"), B, encoding_size,
+                              out_indptr.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
+        "gs_col_row_slice_mark");
+  const int64_t kept = out_indptr[S].item<int64_t>();
+  auto out_indices = torch::empty({kept}, indices.options());
+  auto select_index = torch::empty({kept}, I64(indptr));
+  auto parent_index = torch::empty({kept}, I64(indptr));
+  if (kept > 0)
+    Check(gs_col_row_slice_compact(D, idb, out_indices.data_ptr(), select_index.data_ptr<int64_t>(),
+                                   parent_index.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
+          "gs_col_row_slice_compact");
+  return {out_indptr, out_indices, select_index, parent_index};
+}
+
 torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz, const torch::Tensor& ids_like) {
   NeedI64(indptr, "indptr");
   const int idb = IdBytes(ids_like, "indices");

@@ -117,6 +117,16 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(const torc
                                                                       const torch::Tensor& other,
                                                                       const torch::Tensor& ids);
 
+// Induced-subgraph slice (columns column_ids, rows in row_ids) without writing the column
+// slice: {out_indptr, out_indices, select_index, parent_index}.  select_index counts
+// positions in the virtual column slice (the reference's nonzero(mask)); parent_index is the
+// position of the edge in `indices`.  With batch offsets: a column of batch b keeps the rows
+// of batch b's ids and rows keep their global id.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ColRowSlicing(
+    const torch::Tensor& indptr, const torch::Tensor& indices, const torch::Tensor& column_ids,
+    const torch::Tensor& row_ids, const torch::optional<torch::Tensor>& col_ptr = torch::nullopt,
+    const torch::optional<torch::Tensor>& row_ptr = torch::nullopt, int64_t encoding_size = 0);
+
 // col[e] = column owning edge e, in the dtype of `ids_like`
 torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz, const torch::Tensor& ids_like);
 // {indptr, values in key order, sort permutation (nullopt when already sorted)}

@@ -378,6 +378,31 @@ int gs_row_slice_coo_compact(const void* other, int id_bytes, int64_t E, void* o
                              void* out_other, int64_t* select_index, void* workspace,
                              size_t workspace_bytes, void* stream);
 
+/* Column slice and row slice in one pass (induced subgraph): replaces
+ * impl::fusion::CSCColRowSlicingCUDA and BatchCSCColRowSlicingCUDA
+ * (src/cuda/fusion/column_row_slicing.cu:213,356).  Of the columns column_ids, keep the
+ * edges whose row is in row_ids; the column slice itself is never written.
+ *   sub_indptr, D: offsets and total of the plain column slice, from gs_slice_count.
+ *   num_batches == 0: kept rows are renamed to their position in row_ids (:133-141).
+ *   num_batches  > 0: columns and row ids are cut into batches at col_batch_ptr /
+ *     row_batch_ptr (device int64[num_batches+1]); a column of batch b keeps the rows found
+ *     in batch b's ids, under the key id + b*encoding_size, and rows keep their id (:272).
+ * mark: out_indptr[S+1] = offsets of the result, total in out_indptr[S].
+ * compact (same workspace): out_indices; select_index = position in the virtual column
+ * slice (what the reference returns, :204-209); parent_index = position in the parent's
+ * indices (what edge data has to be gathered with).  Either index array may be NULL. */
+size_t gs_col_row_slice_workspace_bytes(int64_t num_row_ids, int64_t D);
+int gs_col_row_slice_mark(const int64_t* indptr, int64_t num_cols, const void* indices,
+                          int id_bytes, const void* column_ids, int64_t S,
+                          const int64_t* sub_indptr, int64_t D, const void* row_ids,
+                          int64_t num_row_ids, const int64_t* col_batch_ptr,
+                          const int64_t* row_batch_ptr, int64_t num_batches,
+                          int64_t encoding_size, int64_t* out_indptr, void* workspace,
+                          size_t workspace_bytes, void* stream);
+int gs_col_row_slice_compact(int64_t D, int id_bytes, void* out_indices, int64_t* select_index,
+                             int64_t* parent_index, void* workspace, size_t workspace_bytes,
+                             void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Format conversion: replaces impl::CSC2COOCUDA and impl::COO2CSCCUDA          */
 /* (src/cuda/format_transform.cu:35,135).                                      */

@@ -461,6 +461,48 @@ def row_slice_coo(key, other, ids):
     return ok[:m].copy(), oo[:m].copy(), sel[:m].copy()
 
 
+def _last_position_lookup(ids):
+    """(sorted distinct ids, position of the LAST occurrence of each)"""
+    n = ids.size
+    uniq, first_rev = np.unique(ids[::-1], return_index=True)
+    return uniq, (n - 1 - first_rev).astype(np.int64)
+
+
+def _lookup(uniq, vals, x):
+    """vals[i] where uniq[i] == x, else -1"""
+    if uniq.size == 0:
+        return np.full(x.shape, -1, dtype=np.int64)
+    pos = np.minimum(np.searchsorted(uniq, x), uniq.size - 1)
+    return np.where(uniq[pos] == x, vals[pos], -1).astype(np.int64)
+
+
+def col_row_slice(indptr, indices, cols, row_ids, col_ptr=None, row_ptr=None, encoding_size=0):
+    """src/cuda/fusion/column_row_slicing.cu:147-211 (one id set: kept rows renamed to their
+    position in row_ids) and :277-355 (batched: key id + b*encoding_size, rows keep their id)
+    -> (out_indptr, out_indices, select_index, parent_index).
+
+    select_index is what the reference returns, nonzero(out_mask): positions in the virtual
+    column slice (:204-209).  parent_index is the position of the same edge in `indices`."""
+    indptr, indices, cols, row_ids = _i64(indptr), _i64(indices), _i64(cols), _i64(row_ids)
+    sub_indptr, coo_col, sub_indices, parent = slice_columns(indptr, indices, cols, with_coo=True)
+    if col_ptr is None:
+        uniq, last = _last_position_lookup(row_ids)
+        val = _lookup(uniq, last, sub_indices)
+    else:
+        col_ptr, row_ptr = _i64(col_ptr), _i64(row_ptr)
+        nb = col_ptr.size - 1
+        row_batch = np.repeat(np.arange(nb, dtype=np.int64), np.diff(row_ptr))
+        col_batch = np.repeat(np.arange(nb, dtype=np.int64), np.diff(col_ptr))
+        uniq = np.unique(row_ids + row_batch * encoding_size)
+        found = _lookup(uniq, np.zeros(uniq.size, np.int64),
+                        sub_indices + col_batch[coo_col] * encoding_size)
+        val = np.where(found == 0, sub_indices, -1)
+    keep = val >= 0
+    select_index = np.flatnonzero(keep).astype(np.int64)
+    kept_before = np.concatenate([[0], np.cumsum(keep)]).astype(np.int64)
+    return kept_before[sub_indptr], val[keep], select_index, parent[select_index]
+
+
 # ---------------------------------------------------------- format transform
 def csc2coo(indptr, nnz):
     """src/cuda/format_transform.cu:35-46 -> col vector"""
