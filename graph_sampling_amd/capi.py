@@ -32,7 +32,8 @@ def lib():
                      "gs_sample_weighted_workspace_bytes", "gs_list_sample_workspace_bytes",
                      "gs_unique_workspace_bytes", "gs_row_slice_workspace_bytes",
                      "gs_sample_fused_state_bytes", "gs_batch_relabel_workspace_bytes",
-                     "gs_coo2csc_workspace_bytes", "gs_col_row_slice_workspace_bytes"):
+                     "gs_coo2csc_workspace_bytes", "gs_col_row_slice_workspace_bytes",
+                     "gs_index_search_workspace_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
     return _lib
@@ -417,6 +418,138 @@ def batch_csr_relabel(seeds, seeds_ptr, ids, ids_ptr, mailbox=None):
     if mailbox is not None:
         return unique, unique_ptr, out_ids, num_unique, ticket
     return unique, unique_ptr, out_ids, num_unique
+
+
+def batch_coo_relabel(seeds, seeds_ptr, coo_row, coo_col, coo_ptr):
+    """gs_batch_coo_relabel.  Returns (unique_buf, unique_ptr, out_row, out_col, num_unique_dev)."""
+    idb = _ids(seeds, "seeds")
+    _ids(coo_row, "coo_row", like=seeds)
+    _ids(coo_col, "coo_col", like=seeds)
+    _need(seeds_ptr, torch.int64, "seeds_ptr")
+    _need(coo_ptr, torch.int64, "coo_ptr")
+    dev = seeds.device
+    B = seeds_ptr.numel() - 1
+    M = seeds.numel() + coo_row.numel()
+    unique = torch.empty(M, dtype=seeds.dtype, device=dev)
+    unique_ptr = torch.empty(B + 1, dtype=torch.int64, device=dev)
+    out_row, out_col = torch.empty_like(coo_row), torch.empty_like(coo_col)
+    num_unique = torch.empty(1, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_batch_relabel_workspace_bytes(_i64(M)), dev)
+    _check(lib().gs_batch_coo_relabel(_ptr(seeds), _ptr(seeds_ptr), _ptr(coo_row), _ptr(coo_col),
+                                      _ptr(coo_ptr), _i64(B), _i64(seeds.numel()),
+                                      _i64(coo_row.numel()), idb, _ptr(unique), _ptr(unique_ptr),
+                                      _ptr(out_row), _ptr(out_col), _ptr(num_unique), _ptr(ws),
+                                      ctypes.c_size_t(ws.numel()), ctypes.c_void_p(0), _i64(0),
+                                      _stream(dev)), "gs_batch_coo_relabel")
+    return unique, unique_ptr, out_row, out_col, num_unique
+
+
+# ------------------------------------------------------- super-batch helpers ----
+def batch_encode(data, ptr, encoding_size):
+    idb = _ids(data, "data")
+    _need(ptr, torch.int64, "ptr")
+    out = torch.empty_like(data)
+    _check(lib().gs_batch_encode(_ptr(data), idb, _i64(data.numel()), _ptr(ptr),
+                                 _i64(ptr.numel() - 1), _i64(encoding_size), _ptr(out),
+                                 _stream(data.device)), "gs_batch_encode")
+    return out
+
+
+def batch_decode(data, encoding_size):
+    """Returns (decoded ids, batch numbers)."""
+    idb = _ids(data, "data")
+    out, batch = torch.empty_like(data), torch.empty_like(data)
+    _check(lib().gs_batch_decode(_ptr(data), idb, _i64(data.numel()), _i64(encoding_size),
+                                 _ptr(out), _ptr(batch), _stream(data.device)), "gs_batch_decode")
+    return out, batch
+
+
+def batch_offsets(data, num_batches, encoding_size):
+    """Returns (offsets [num_batches+1], decoded ids) of encoded data sorted by batch."""
+    idb = _ids(data, "data")
+    ptr = torch.empty(num_batches + 1, dtype=torch.int64, device=data.device)
+    out = torch.empty_like(data)
+    _check(lib().gs_batch_offsets(_ptr(data), idb, _i64(data.numel()), _i64(num_batches),
+                                  _i64(encoding_size), _ptr(ptr), _ptr(out), _stream(data.device)),
+           "gs_batch_offsets")
+    return ptr, out
+
+
+def _ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def batch_concat(datas, ptrs):
+    """gs_batch_concat_{offsets,fill}.  Returns (total, key, total_ptr)."""
+    idb = _ids(datas[0], "data")
+    for d in datas:
+        _ids(d, "data", like=datas[0])
+    for p in ptrs:
+        _need(p, torch.int64, "offsets")
+    dev = datas[0].device
+    B = ptrs[0].numel() - 1
+    total_ptr = torch.empty(B + 1, dtype=torch.int64, device=dev)
+    st = _stream(dev)
+    _check(lib().gs_batch_concat_offsets(_ptr_array(ptrs), len(ptrs), _i64(B), _ptr(total_ptr), st),
+           "gs_batch_concat_offsets")
+    total = sum(int(d.numel()) for d in datas)
+    out = torch.empty(total, dtype=datas[0].dtype, device=dev)
+    key = torch.empty(total, dtype=datas[0].dtype, device=dev)
+    _check(lib().gs_batch_concat_fill(_ptr_array(datas), _ptr_array(ptrs), len(ptrs), _i64(B),
+                                      _i64(max(int(d.numel()) for d in datas)), idb,
+                                      _ptr(total_ptr), _ptr(out), _ptr(key), st),
+           "gs_batch_concat_fill")
+    return out, key, total_ptr
+
+
+def batch_split(data, data_ptr, data_key, out_ptrs):
+    """gs_batch_split.  out_ptrs: offsets of every segment; returns the filled segments."""
+    idb = _ids(data, "data")
+    _need(data_ptr, torch.int64, "data_ptr")
+    dev = data.device
+    host = [int(p[-1].item()) for p in out_ptrs]
+    outs = [torch.empty(n, dtype=data.dtype, device=dev) for n in host]
+    _check(lib().gs_batch_split(_ptr(data), _ptr(data_ptr), _ptr(data_key), idb, _i64(data.numel()),
+                                _i64(data_ptr.numel() - 1), _ptr_array(outs), _ptr_array(out_ptrs),
+                                len(outs), _stream(dev)), "gs_batch_split")
+    return outs
+
+
+def coo_filter(key, row, col, ids, key_ptr=None, ids_ptr=None):
+    """gs_coo_filter_{mark,compact}.  Returns (row, col, batch offsets | None, select_index)."""
+    idb = _ids(key, "key")
+    for t in (row, col, ids):
+        _ids(t, "ids", like=key)
+    dev = key.device
+    E, n = key.numel(), ids.numel()
+    B = 0 if key_ptr is None else key_ptr.numel() - 1
+    num_kept = torch.empty(1, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_row_slice_workspace_bytes(_i64(n), _i64(E), _i64(0)), dev)
+    st = _stream(dev)
+    _check(lib().gs_coo_filter_mark(_ptr(key), idb, _i64(E), _ptr(key_ptr), _ptr(ids), _i64(n),
+                                    _ptr(ids_ptr), _i64(B), _ptr(num_kept), _ptr(ws),
+                                    ctypes.c_size_t(ws.numel()), st), "gs_coo_filter_mark")
+    kept = int(num_kept.item())
+    out_row = torch.empty(kept, dtype=key.dtype, device=dev)
+    out_col = torch.empty(kept, dtype=key.dtype, device=dev)
+    select_index = torch.empty(kept, dtype=torch.int64, device=dev)
+    out_ptr = torch.empty(B + 1, dtype=torch.int64, device=dev) if B else None
+    _check(lib().gs_coo_filter_compact(_ptr(row), _ptr(col), idb, _i64(E), _ptr(key_ptr), _i64(B),
+                                       _ptr(out_row), _ptr(out_col), _ptr(select_index),
+                                       _ptr(out_ptr), _ptr(ws), ctypes.c_size_t(ws.numel()), st),
+           "gs_coo_filter_compact")
+    return out_row, out_col, out_ptr, select_index
+
+
+def index_search(data, keys):
+    idb = _ids(data, "data")
+    _ids(keys, "keys", like=data)
+    out = torch.empty_like(keys)
+    ws = workspace(lib().gs_index_search_workspace_bytes(_i64(data.numel())), data.device)
+    _check(lib().gs_index_search(_ptr(data), _i64(data.numel()), _ptr(keys), _i64(keys.numel()), idb,
+                                 _ptr(out), _ptr(ws), ctypes.c_size_t(ws.numel()),
+                                 _stream(data.device)), "gs_index_search")
+    return out
 
 
 # ------------------------------------------------------------------ walks ----

@@ -258,6 +258,55 @@ sliced_compact_kernel(int64_t D, const int64_t* __restrict__ val, const int64_t*
   if (parent_index) parent_index[w] = src[p];
 }
 
+// ------------------------------------------------- batched membership filter ----
+// Edge e belongs to the batch whose range of key_ptr holds e; it survives when key[e] is
+// among the ids of the same batch.  Replaces the per-batch tables of
+// impl::BatchCOOSlicingCUDA / BatchCOORowSlicingCUDA (reference src/cuda/batch_slicing.cu:
+// 150-232, src/cuda/slicing.cu:659-770) by one table keyed with id + (batch << 44).
+constexpr int kBatchShift = 44;
+
+template <typename IdT>
+__global__ void __launch_bounds__(kThreads)
+mark_batched_kernel(IdSet t, const IdT* __restrict__ key, int64_t E,
+                    const int64_t* __restrict__ key_ptr, int64_t B, int64_t* __restrict__ val) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (e >= E) return;
+  const int64_t b = upper_bound(key_ptr, B + 1, e) - 1;
+  val[e] = (b >= 0 && b < B)
+               ? t.query(static_cast<long long>(key[e]) + (static_cast<long long>(b) << kBatchShift))
+               : -1;
+}
+
+template <typename IdT>
+__global__ void __launch_bounds__(kThreads)
+filter_compact_kernel(const IdT* __restrict__ row, const IdT* __restrict__ col, int64_t E,
+                      const int64_t* __restrict__ val, const int64_t* __restrict__ prefix,
+                      IdT* __restrict__ out_row, IdT* __restrict__ out_col,
+                      int64_t* __restrict__ select_index) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (e >= E || val[e] < 0) return;
+  const int64_t w = prefix[e];
+  out_row[w] = row[e];
+  out_col[w] = col[e];
+  if (select_index) select_index[w] = e;
+}
+
+__global__ void __launch_bounds__(kThreads)
+filter_batch_ptr_kernel(const int64_t* __restrict__ key_ptr, int64_t B,
+                        const int64_t* __restrict__ prefix, int64_t* __restrict__ out_ptr) {
+  const int64_t b = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (b <= B) out_ptr[b] = prefix[key_ptr[b]];
+}
+
+// position of each key in `data` (-1 when absent): impl::IndexHashMapInsertCUDA +
+// IndexHashMapSearchCUDA (reference src/cuda/index_search.cu:83-140)
+template <typename IdT>
+__global__ void __launch_bounds__(kThreads)
+search_kernel(IdSet t, const IdT* __restrict__ keys, int64_t m, IdT* __restrict__ out) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < m) out[i] = static_cast<IdT>(t.query(static_cast<long long>(keys[i])));
+}
+
 // Workspace layout: [val | prefix | scan tiles | (parent positions) | id-set].  All but
 // the last depend on the edge count only, so the compact call finds them again without
 // knowing how many ids the mark call was given.
@@ -518,6 +567,126 @@ int gs_col_row_slice_compact(int64_t D, int id_bytes, void* out_indices, int64_t
                        s.prefix, s.src, static_cast<int32_t*>(out_indices), select_index,
                        parent_index);
   return check_launch("col_row_slice_compact");
+}
+
+int gs_coo_filter_mark(const void* key, int id_bytes, int64_t E, const int64_t* key_batch_ptr,
+                       const void* ids, int64_t num_ids, const int64_t* ids_batch_ptr,
+                       int64_t num_batches, int64_t* num_kept, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(E >= 0 && num_ids >= 0 && num_batches >= 0 && num_kept,
+             "gs_coo_filter_mark: bad argument");
+  GS_REQUIRE((E == 0 || key) && (num_ids == 0 || ids), "gs_coo_filter_mark: null pointer");
+  GS_REQUIRE(num_batches == 0 || (key_batch_ptr && ids_batch_ptr),
+             "gs_coo_filter_mark: a batched call needs both batch offsets");
+  GS_REQUIRE(num_batches < (int64_t(1) << (62 - kBatchShift)),
+             "gs_coo_filter_mark: too many batches");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_coo_filter_mark: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  if (num_batches == 0) {
+    Scratch s0 = carve(workspace, workspace_bytes, num_ids, E, true);
+    if (!s0.ok) {
+      set_error_text("gs_coo_filter_mark: workspace needs %zu bytes, 256-byte aligned",
+                     gs_row_slice_workspace_bytes(num_ids, E, 0));
+      return GS_ERR_WORKSPACE;
+    }
+    hipStream_t st0 = static_cast<hipStream_t>(stream);
+    GS_RETURN_IF_ERROR(id_bytes == 8 ? mark_common<int64_t>("coo_filter_mark", key, E, ids, num_ids,
+                                                            s0, st0)
+                                     : mark_common<int32_t>("coo_filter_mark", key, E, ids, num_ids,
+                                                            s0, st0));
+    hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(64), 0, st0, s0.prefix, E, num_kept);
+    return check_launch("coo_filter_mark");
+  }
+  Scratch s = carve(workspace, workspace_bytes, num_ids, E, true);
+  if (!s.ok) {
+    set_error_text("gs_coo_filter_mark: workspace needs %zu bytes, 256-byte aligned",
+                   gs_row_slice_workspace_bytes(num_ids, E, 0));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(s.cap, kThreads)), dim3(kThreads), 0, st,
+                     s.set, s.cap);
+  auto run = [&](auto tag) {
+    using IdT = decltype(tag);
+    if (num_ids > 0)
+      hipLaunchKernelGGL(set_insert_batched_kernel<IdT>, dim3(blocks_for(num_ids, kThreads)),
+                         dim3(kThreads), 0, st, s.set, static_cast<const IdT*>(ids), num_ids,
+                         ids_batch_ptr, num_batches, int64_t(1) << kBatchShift);
+    if (E > 0)
+      hipLaunchKernelGGL(mark_batched_kernel<IdT>, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0,
+                         st, s.set, static_cast<const IdT*>(key), E, key_batch_ptr, num_batches,
+                         s.val);
+  };
+  if (id_bytes == 8) run(int64_t{}); else run(int32_t{});
+  GS_RETURN_IF_ERROR(check_launch("coo_filter_mark"));
+  Kept f{s.val};
+  GS_RETURN_IF_ERROR(exclusive_scan(f, E, s.prefix, s.tiles, st));
+  hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(64), 0, st, s.prefix, E, num_kept);
+  return check_launch("coo_filter_mark");
+}
+
+int gs_coo_filter_compact(const void* row, const void* col, int id_bytes, int64_t E,
+                          const int64_t* key_batch_ptr, int64_t num_batches, void* out_row,
+                          void* out_col, int64_t* select_index, int64_t* out_batch_ptr,
+                          void* workspace, size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(E >= 0 && num_batches >= 0, "gs_coo_filter_compact: negative size");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_coo_filter_compact: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  GS_REQUIRE(!out_batch_ptr || (num_batches > 0 && key_batch_ptr),
+             "gs_coo_filter_compact: batch offsets of the result need those of the input");
+  Scratch s = carve(workspace, workspace_bytes, 0, E, false);
+  if (!s.ok) {
+    set_error_text("gs_coo_filter_compact: pass the workspace given to gs_coo_filter_mark");
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (out_batch_ptr)
+    hipLaunchKernelGGL(filter_batch_ptr_kernel, dim3(blocks_for(num_batches + 1, kThreads)),
+                       dim3(kThreads), 0, st, key_batch_ptr, num_batches, s.prefix, out_batch_ptr);
+  if (E > 0) {
+    GS_REQUIRE(row && col && out_row && out_col, "gs_coo_filter_compact: null pointer");
+    const dim3 grid(blocks_for(E, kThreads));
+    if (id_bytes == 8)
+      hipLaunchKernelGGL(filter_compact_kernel<int64_t>, grid, dim3(kThreads), 0, st,
+                         static_cast<const int64_t*>(row), static_cast<const int64_t*>(col), E,
+                         s.val, s.prefix, static_cast<int64_t*>(out_row),
+                         static_cast<int64_t*>(out_col), select_index);
+    else
+      hipLaunchKernelGGL(filter_compact_kernel<int32_t>, grid, dim3(kThreads), 0, st,
+                         static_cast<const int32_t*>(row), static_cast<const int32_t*>(col), E,
+                         s.val, s.prefix, static_cast<int32_t*>(out_row),
+                         static_cast<int32_t*>(out_col), select_index);
+  }
+  return check_launch("coo_filter_compact");
+}
+
+size_t gs_index_search_workspace_bytes(int64_t n) { return gs_row_slice_workspace_bytes(n, 0, 0); }
+
+int gs_index_search(const void* data, int64_t n, const void* keys, int64_t m, int id_bytes,
+                    void* out, void* workspace, size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(n >= 0 && m >= 0, "gs_index_search: negative size");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_index_search: id_bytes must be 4 or 8, got %d", id_bytes);
+  GS_REQUIRE((n == 0 || data) && (m == 0 || (keys && out)), "gs_index_search: null pointer");
+  Scratch s = carve(workspace, workspace_bytes, n, 0, true);
+  if (!s.ok) {
+    set_error_text("gs_index_search: workspace needs %zu bytes, 256-byte aligned",
+                   gs_index_search_workspace_bytes(n));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(s.cap, kThreads)), dim3(kThreads), 0, st,
+                     s.set, s.cap);
+  auto run = [&](auto tag) {
+    using IdT = decltype(tag);
+    if (n > 0)
+      hipLaunchKernelGGL(set_insert_kernel<IdT>, dim3(blocks_for(n, kThreads)), dim3(kThreads), 0,
+                         st, s.set, static_cast<const IdT*>(data), n);
+    if (m > 0)
+      hipLaunchKernelGGL(search_kernel<IdT>, dim3(blocks_for(m, kThreads)), dim3(kThreads), 0, st,
+                         s.set, static_cast<const IdT*>(keys), m, static_cast<IdT*>(out));
+  };
+  if (id_bytes == 8) run(int64_t{}); else run(int32_t{});
+  return check_launch("index_search");
 }
 
 }  // extern "C"

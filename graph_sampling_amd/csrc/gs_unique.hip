@@ -461,6 +461,20 @@ struct PackedRegions {
   __device__ __forceinline__ uint32_t first_index(uint32_t p) const {
     return static_cast<uint32_t>(slots[p]);
   }
+  // slot of a key that may be absent (0xFFFFFFFF then); the region is never full
+  __device__ __forceinline__ uint32_t find(int64_t begin, int64_t len, long long key) const {
+    const unsigned long long hi = static_cast<uint32_t>(key);
+    int64_t p = begin + static_cast<int64_t>((static_cast<unsigned long long>(hash32(
+                                                  static_cast<uint32_t>(key))) *
+                                              static_cast<unsigned long long>(len)) >>
+                                             32);
+    while (true) {
+      const unsigned long long w = slots[p];
+      if (w == ~0ull) return 0xFFFFFFFFu;
+      if ((w >> 32) == hi) return static_cast<uint32_t>(p);
+      if (++p == begin + len) p = begin;
+    }
+  }
 };
 
 // the same with 64-bit keys: key array (-1 = empty) + first-index array
@@ -495,6 +509,18 @@ struct WideRegions {
   }
   __device__ __forceinline__ uint32_t first_index(uint32_t p) const {
     return static_cast<uint32_t>(vals[p]);
+  }
+  __device__ __forceinline__ uint32_t find(int64_t begin, int64_t len, long long key) const {
+    int64_t p = begin + static_cast<int64_t>((static_cast<unsigned long long>(hash32(
+                                                  static_cast<unsigned long long>(key))) *
+                                              static_cast<unsigned long long>(len)) >>
+                                             32);
+    while (true) {
+      const long long cur = keys[p];
+      if (cur == -1) return 0xFFFFFFFFu;
+      if (cur == key) return static_cast<uint32_t>(p);
+      if (++p == begin + len) p = begin;
+    }
   }
 };
 
@@ -592,7 +618,8 @@ __global__ void __launch_bounds__(kThreads)
 batch_finish_kernel(BatchItems<IdT> x, int64_t num_ids, int64_t M, R t,
                     const uint32_t* __restrict__ pos, const int64_t* __restrict__ prefix,
                     const int64_t* __restrict__ num_unique, IdT* __restrict__ out_ids,
-                    int64_t* __restrict__ unique_ptr) {
+                    int64_t* __restrict__ unique_ptr, const IdT* __restrict__ extra,
+                    IdT* __restrict__ out_extra) {
   __shared__ int64_t s_range[2];
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads;
   if (first < num_ids) {  // a workgroup of id lookups
@@ -618,6 +645,14 @@ batch_finish_kernel(BatchItems<IdT> x, int64_t num_ids, int64_t M, R t,
     const int64_t begin = x.start(b);
     const int64_t p = begin + (x.seeds_ptr[b + 1] - x.seeds_ptr[b]) + (j - x.ids_ptr[b]);
     out_ids[j] = static_cast<IdT>(prefix[t.first_index(pos[p])] - prefix[begin]);
+    if (extra) {
+      // a second array cut like the ids (the other end of a COO edge): looked up, -1 if absent
+      const uint32_t slot = t.find(kRegionFactor * begin, kRegionFactor * (x.start(b + 1) - begin),
+                                   static_cast<long long>(extra[j]));
+      out_extra[j] = slot == 0xFFFFFFFFu
+                         ? IdT(-1)
+                         : static_cast<IdT>(prefix[t.first_index(slot)] - prefix[begin]);
+    }
     return;
   }
   const int64_t b = first + threadIdx.x - (num_ids + kThreads - 1) / kThreads * kThreads;
@@ -636,7 +671,8 @@ int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* 
                        const int64_t* ids_ptr, int64_t B, int64_t num_seeds, int64_t num_ids,
                        void* unique, int64_t* unique_ptr, void* out_ids, int64_t* num_unique,
                        void* workspace, size_t workspace_bytes, gs_mailbox* box,
-                       int64_t box_ticket, hipStream_t stream) {
+                       int64_t box_ticket, hipStream_t stream, const void* extra = nullptr,
+                       void* out_extra = nullptr) {
   using R = typename RegionsFor<IdT>::type;
   const int64_t M = num_seeds + num_ids;
   const int64_t cap = kRegionFactor * (M > 0 ? M : 1);
@@ -667,7 +703,8 @@ int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* 
   const int64_t ptr_blocks = (B + 1 + kThreads - 1) / kThreads;
   hipLaunchKernelGGL((batch_finish_kernel<IdT, R>), dim3(static_cast<unsigned>(id_blocks + ptr_blocks)),
                      dim3(kThreads), 0, stream, x, num_ids, M, t, pos, prefix, num_unique,
-                     static_cast<IdT*>(out_ids), unique_ptr);
+                     static_cast<IdT*>(out_ids), unique_ptr, static_cast<const IdT*>(extra),
+                     static_cast<IdT*>(out_extra));
   return check_launch("batch_csr_relabel");
 }
 
@@ -770,6 +807,38 @@ int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void
              : batch_relabel_impl<int32_t>(seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds,
                                            num_ids, unique, unique_ptr, out_ids, num_unique,
                                            workspace, workspace_bytes, mailbox, mailbox_ticket, st);
+}
+
+int gs_batch_coo_relabel(const void* seeds, const int64_t* seeds_ptr, const void* coo_row,
+                         const void* coo_col, const int64_t* coo_ptr, int64_t num_batches,
+                         int64_t num_seeds, int64_t num_edges, int id_bytes, void* unique,
+                         int64_t* unique_ptr, void* out_row, void* out_col, int64_t* num_unique,
+                         void* workspace, size_t workspace_bytes, gs_mailbox* mailbox,
+                         int64_t mailbox_ticket, void* stream) {
+  GS_REQUIRE(num_batches >= 1 && num_seeds >= 0 && num_edges >= 0,
+             "gs_batch_coo_relabel: at least one batch and non-negative sizes required");
+  GS_REQUIRE(seeds_ptr && coo_ptr && unique_ptr && num_unique, "gs_batch_coo_relabel: null pointer");
+  GS_REQUIRE((num_seeds == 0 || seeds) &&
+                 (num_edges == 0 || (coo_row && coo_col && out_row && out_col)) &&
+                 (num_seeds + num_edges == 0 || unique),
+             "gs_batch_coo_relabel: null buffer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_batch_coo_relabel: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  if (num_seeds + num_edges >= (int64_t(1) << 30)) {
+    set_error_text("gs_batch_coo_relabel: %lld items exceed the supported 2^30",
+                   static_cast<long long>(num_seeds + num_edges));
+    return GS_ERR_UNSUPPORTED;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8
+             ? batch_relabel_impl<int64_t>(seeds, seeds_ptr, coo_row, coo_ptr, num_batches,
+                                           num_seeds, num_edges, unique, unique_ptr, out_row,
+                                           num_unique, workspace, workspace_bytes, mailbox,
+                                           mailbox_ticket, st, coo_col, out_col)
+             : batch_relabel_impl<int32_t>(seeds, seeds_ptr, coo_row, coo_ptr, num_batches,
+                                           num_seeds, num_edges, unique, unique_ptr, out_row,
+                                           num_unique, workspace, workspace_bytes, mailbox,
+                                           mailbox_ticket, st, coo_col, out_col);
 }
 
 }  // extern "C"

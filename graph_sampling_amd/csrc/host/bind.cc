@@ -39,6 +39,10 @@ TORCH_LIBRARY(gs_classes, m) {
       GS_DEF2("_CAPI_FusionSlicing", "_CAPI_fusion_slicing", &Graph::FusedBidirSlicing)
       GS_DEF2("_CAPI_BatchFusionSlicing", "_CAPI_batch_fusion_slicing",
               &Graph::BatchFusedBidirSlicing)
+      GS_DEF2("_CAPI_BatchSlicing", "_CAPI_batch_slicing", &Graph::BatchSlicing)
+      GS_DEF2("_CAPI_Split", "_CAPI_split", &Graph::Split)
+      GS_DEF2("_CAPI_Decode", "_CAPI_decode", &Graph::Decode)
+      GS_DEF2("_CAPI_GetBatchCOO", "GetBatchCOO", &Graph::GetBatchCOO)
       GS_DEF2("_CAPI_LoadCSC", "_CAPI_load_csc", &Graph::LoadCSC)
       GS_DEF2("_CAPI_LoadCSR", "_CAPI_load_csr", &Graph::LoadCSR)
       GS_DEF2("_CAPI_LoadCOO", "_CAPI_load_coo", &Graph::LoadCOO)
@@ -91,6 +95,38 @@ TORCH_LIBRARY(gs_ops, m) {
   m.def("IndptrSplitBySize", &IndptrSplitBySize);
   m.def("_CAPI_BatchCSRRelabel", &BatchCSRRelabel);
   m.def("BatchCSRRelabel", &BatchCSRRelabel);
+  m.def("_CAPI_BatchCSRRelabelByKey", &BatchCSRRelabelByKey);
+  m.def("BatchCSRRelabelByKey", &BatchCSRRelabelByKey);
+  m.def("_CAPI_BatchCOORelabel", &BatchCOORelabel);
+  m.def("BatchCOORelabel", &BatchCOORelabel);
+  m.def("_CAPI_BatchCOORelabelByKey", &BatchCOORelabelByKey);
+  m.def("BatchCOORelabelByKey", &BatchCOORelabelByKey);
+  m.def("_CAPI_BatchConcat", &BatchConcat);
+  m.def("BatchConcat", &BatchConcat);
+  m.def("_CAPI_BatchSplit", &BatchSplit);
+  m.def("BatchSplit", &BatchSplit);
+  m.def("_CAPI_BatchUnique", &BatchUnique);
+  m.def("BatchUnique", &BatchUnique);
+  m.def("_CAPI_BatchUniqueByKey", &BatchUniqueByKey);
+  m.def("BatchUniqueByKey", &BatchUniqueByKey);
+  m.def("_CAPI_BatchUnique2", &BatchUnique2);
+  m.def("BatchUnique2", &BatchUnique2);
+  m.def("_CAPI_BatchUniqueByKey2", &BatchUniqueByKey2);
+  m.def("BatchUniqueByKey2", &BatchUniqueByKey2);
+  m.def("_CAPI_BatchEncode", &BatchEncode);
+  m.def("BatchEncode", &BatchEncode);
+  m.def("_CAPI_BatchDecode", &BatchDecode);
+  m.def("BatchDecode", &BatchDecode);
+  m.def("_CAPI_GetBatchOffsets", &GetBatchOffsets);
+  m.def("GetBatchOffsets", &GetBatchOffsets);
+  m.def("_CAPI_BatchCOOSlicing", &BatchCOOSlicing);
+  m.def("BatchCOOSlicing", &BatchCOOSlicing);
+  m.def("_CAPI_COORowSlicingGlobalId", &COORowSlicingGlobalId);
+  m.def("COORowSlicingGlobalId", &COORowSlicingGlobalId);
+  m.def("_CAPI_BatchListSamplingWithProbs", &BatchListSamplingProbs);
+  m.def("batch_list_sampling_with_probs", &BatchListSamplingProbs);
+  m.def("_CAPI_IndexSearch", &IndexSearch);
+  m.def("index_search", &IndexSearch);
   // not in the reference: reproducible sampling (its seeds are compile-time constants)
   m.def("_CAPI_SetSeed", &SetSeed);
   m.def("_CAPI_SetSampleAlgo", &SetSampleAlgo);

@@ -3,6 +3,7 @@
 #include "bcast.h"
 #include "graph_ops.h"
 #include "hip_ops.h"
+#include "tensor_ops.h"
 
 namespace gs {
 
@@ -403,6 +404,95 @@ c10::intrusive_ptr<Graph> Graph::BatchFusedBidirSlicing(torch::Tensor column_see
   ret->SetNumEdges(sliced->indices.numel());
   InheritData(ret.get(), csc_->e_ids, parent_index);
   return ret;
+}
+
+std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> Graph::BatchSlicing(
+    torch::Tensor n_ids, torch::Tensor nid_ptr, int64_t axis, int64_t on_format,
+    int64_t output_format, bool relabel, bool encoding) {
+  Settle();
+  TORCH_CHECK(axis == 0, "batch slicing only suppurt column slicing now");  // src/graph.cc:335
+  TORCH_CHECK(on_format == _CSC, "Not Implementatin Error");                // src/graph.cc:364
+  CreateSparseFormat(_CSC);
+  const bool with_coo = output_format & _COO;
+  const int64_t num_batches = nid_ptr.numel() - 1;
+  torch::optional<torch::Tensor> col_ids =
+      col_ids_.has_value() ? col_ids_.value().index({n_ids})
+                           : hip::BatchEncode(n_ids, nid_ptr, num_rows_);
+  torch::optional<torch::Tensor> row_ids = row_ids_;
+  int64_t num_rows = num_rows_ * num_batches;
+
+  std::shared_ptr<_TMP> tmp;
+  torch::Tensor select_index;
+  std::tie(tmp, select_index) = CSCColSlicing(csc_, n_ids, with_coo, data_.has_value());
+  torch::Tensor coo_offsets = tmp->indptr.index({nid_ptr});
+  if (encoding) tmp->coo_in_indices = hip::BatchEncode(tmp->coo_in_indices, coo_offsets, num_rows_);
+  if (relabel) {
+    torch::Tensor frontier;
+    std::vector<torch::Tensor> renamed;
+    std::tie(frontier, renamed) = BatchTensorRelabel({tmp->coo_in_indices}, {tmp->coo_in_indices});
+    tmp->coo_in_indices = renamed[0];
+    row_ids = frontier;
+    num_rows = frontier.numel();
+  }
+  auto ret = Child(col_ids, row_ids, n_ids.numel(), num_rows);
+  if (output_format & _CSC)
+    ret->SetCSC(std::make_shared<CSC>(CSC{tmp->indptr, tmp->coo_in_indices, torch::nullopt}));
+  if (with_coo)
+    ret->SetCOO(std::make_shared<COO>(
+        COO{tmp->coo_in_indices, tmp->coo_in_indptr, torch::nullopt, false, true}));
+  ret->SetNumEdges(tmp->coo_in_indices.numel());
+  InheritData(ret.get(), csc_->e_ids, select_index);
+  return {ret, coo_offsets};
+}
+
+std::vector<c10::intrusive_ptr<Graph>> Graph::Split(int64_t split_size) {
+  Settle();
+  TORCH_CHECK(split_size > 0, "split_size must be positive");
+  CreateSparseFormat(_CSC);
+  const int64_t n = csc_->indptr.numel() - 1;
+  std::vector<int64_t> cuts;
+  for (int64_t c = 0; c < n; c += split_size) cuts.push_back(c);
+  cuts.push_back(n);
+  if (n == 0) return {};
+  auto offsets = torch::tensor(cuts, torch::dtype(torch::kInt64)).to(csc_->indptr.device());
+  std::vector<torch::Tensor> ptrs = IndptrSplitByOffset(csc_->indptr, offsets);
+  std::vector<torch::Tensor> idx = SplitByOffset(csc_->indices, csc_->indptr.index({offsets}));
+  std::vector<torch::Tensor> eid, nid;
+  if (csc_->e_ids.has_value())
+    eid = SplitByOffset(csc_->e_ids.value(), csc_->indptr.index({offsets}));
+  if (col_ids_.has_value()) nid = torch::split(col_ids_.value(), split_size);
+  std::vector<torch::Tensor> data;
+  if (data_.has_value() && !csc_->e_ids.has_value())
+    data = SplitByOffset(data_.value(), csc_->indptr.index({offsets}));
+  std::vector<c10::intrusive_ptr<Graph>> out;
+  for (size_t i = 0; i < ptrs.size(); ++i) {
+    auto g = Child(col_ids_.has_value() ? torch::optional<torch::Tensor>(nid[i]) : torch::nullopt,
+                   row_ids_, ptrs[i].numel() - 1, num_rows_);
+    g->SetCSC(std::make_shared<CSC>(
+        CSC{ptrs[i], idx[i],
+            csc_->e_ids.has_value() ? torch::optional<torch::Tensor>(eid[i]) : torch::nullopt}));
+    g->SetNumEdges(idx[i].numel());
+    // the reference drops the edge data here (src/graph.cc:997-1012); a piece keeps its
+    // share of it: through the parent's e_ids when there are any, else cut like the edges
+    if (data_.has_value()) g->SetData(csc_->e_ids.has_value() ? data_.value() : data[i]);
+    out.push_back(g);
+  }
+  return out;
+}
+
+// The reference's guard is inverted (it aborts exactly when the ids are there,
+// src/graph.cc:1036-1037); the intent, "needs both id maps", is what is checked here.
+void Graph::Decode(int64_t encoding_size) {
+  TORCH_CHECK(col_ids_.has_value() && row_ids_.has_value(),
+              "Error: Decoding should have both row and column id");
+  col_ids_ = hip::BatchDecode(col_ids_.value(), encoding_size);
+  row_ids_ = hip::BatchDecode(row_ids_.value(), encoding_size);
+}
+
+std::tuple<torch::Tensor, torch::Tensor> Graph::GetBatchCOO() {
+  Settle();
+  CreateSparseFormat(_COO);
+  return {coo_->row, coo_->col};
 }
 
 torch::Tensor Graph::RandomWalk(torch::Tensor seeds, int64_t walk_length) {

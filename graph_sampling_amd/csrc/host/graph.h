@@ -111,6 +111,19 @@ class Graph : public torch::CustomClassHolder {
   // their ids (reference src/graph.cc:143-171)
   c10::intrusive_ptr<Graph> BatchFusedBidirSlicing(torch::Tensor column_seeds, torch::Tensor col_ptr,
                                                    torch::Tensor row_seeds, torch::Tensor row_ptr);
+  // ---- super-batch methods (reference src/graph.cc:312-391,987-1040)
+  // Column slice of all batches at once (n_ids cut at nid_ptr): (graph, edge offsets of the
+  // batches).  Without id maps the columns are named batch * num_rows + id; with
+  // `encoding` so are the rows, and the graph counts num_rows * num_batches rows.
+  std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> BatchSlicing(
+      torch::Tensor n_ids, torch::Tensor nid_ptr, int64_t axis, int64_t on_format,
+      int64_t output_format, bool relabel, bool encoding);
+  // the CSC cut into graphs of split_size columns each (the last may be shorter)
+  std::vector<c10::intrusive_ptr<Graph>> Split(int64_t split_size);
+  // column and row ids taken modulo encoding_size
+  void Decode(int64_t encoding_size);
+  // (row, col) of the column-sorted COO
+  std::tuple<torch::Tensor, torch::Tensor> GetBatchCOO();
   torch::Tensor RandomWalk(torch::Tensor seeds, int64_t walk_length);
 
   // ---- edge-data operators

@@ -753,5 +753,186 @@ std::tuple<torch::Tensor, torch::Tensor> ListSamplingProbs(const torch::Tensor& 
   return {out_data, out_index};
 }
 
+// --------------------------------------------------------- super-batch helpers
+namespace {
+int64_t NumBatches(const torch::Tensor& ptr, const char* name) {
+  NeedI64(ptr, name);
+  TORCH_CHECK(ptr.numel() >= 2, name, " must hold num_batches + 1 offsets");
+  return ptr.numel() - 1;
+}
+}  // namespace
+
+torch::Tensor BatchEncode(const torch::Tensor& data, const torch::Tensor& ptr, int64_t enc) {
+  const int idb = IdBytes(data, "data");
+  const int64_t B = NumBatches(ptr, "data_ptr");
+  auto out = torch::empty_like(data);
+  Check(gs_batch_encode(data.data_ptr(), idb, data.numel(), ptr.data_ptr<int64_t>(), B, enc,
+                        out.data_ptr(), Stream(data)),
+        "gs_batch_encode");
+  return out;
+}
+
+torch::Tensor BatchDecode(const torch::Tensor& in, int64_t enc) {
+  const int idb = IdBytes(in, "data");
+  auto out = torch::empty_like(in);
+  Check(gs_batch_decode(in.data_ptr(), idb, in.numel(), enc, out.data_ptr(), nullptr, Stream(in)),
+        "gs_batch_decode");
+  return out;
+}
+
+std::tuple<torch::Tensor, torch::Tensor> BatchOffsets(const torch::Tensor& in, int64_t B,
+                                                      int64_t enc) {
+  const int idb = IdBytes(in, "data");
+  auto ptr = torch::empty({B + 1}, I64(in));
+  auto out = torch::empty_like(in);
+  Check(gs_batch_offsets(in.data_ptr(), idb, in.numel(), B, enc, ptr.data_ptr<int64_t>(),
+                         out.data_ptr(), Stream(in)),
+        "gs_batch_offsets");
+  return {ptr, out};
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchConcat(
+    const std::vector<torch::Tensor>& data, const std::vector<torch::Tensor>& offsets) {
+  TORCH_CHECK(!data.empty() && data.size() == offsets.size(),
+              "BatchConcat takes as many offset tensors as data tensors, at least one");
+  TORCH_CHECK(data.size() <= GS_MAX_SEGMENTS, "BatchConcat: at most ", GS_MAX_SEGMENTS,
+              " tensors, got ", data.size());
+  const int idb = IdBytes(data[0], "data");
+  const int64_t B = NumBatches(offsets[0], "offsets");
+  std::vector<const void*> dp;
+  std::vector<const int64_t*> pp;
+  int64_t longest = 0;
+  for (size_t s = 0; s < data.size(); ++s) {
+    TORCH_CHECK(IdBytes(data[s], "data") == idb, "BatchConcat: data tensors differ in dtype");
+    TORCH_CHECK(NumBatches(offsets[s], "offsets") == B, "BatchConcat: offsets differ in length");
+    dp.push_back(data[s].data_ptr());
+    pp.push_back(offsets[s].data_ptr<int64_t>());
+    longest = std::max(longest, data[s].numel());
+  }
+  void* st = Stream(data[0]);
+  auto total_ptr = torch::empty({B + 1}, I64(data[0]));
+  Check(gs_batch_concat_offsets(pp.data(), static_cast<int>(pp.size()), B,
+                                total_ptr.data_ptr<int64_t>(), st),
+        "gs_batch_concat_offsets");
+  int64_t total = 0;
+  for (const auto& d : data) total += d.numel();  // = total_ptr[B] when the offsets cover the data
+  auto out = torch::empty({total}, data[0].options());
+  auto key = torch::empty({total}, data[0].options());
+  Check(gs_batch_concat_fill(dp.data(), pp.data(), static_cast<int>(pp.size()), B, longest, idb,
+                             total_ptr.data_ptr<int64_t>(), out.data_ptr(), key.data_ptr(), st),
+        "gs_batch_concat_fill");
+  return {out, key, total_ptr};
+}
+
+void BatchSplit(const torch::Tensor& data, const torch::Tensor& data_ptr,
+                const torch::optional<torch::Tensor>& data_key,
+                const std::vector<torch::Tensor>& outs, const std::vector<torch::Tensor>& out_ptrs) {
+  TORCH_CHECK(!outs.empty() && outs.size() == out_ptrs.size(),
+              "BatchSplit takes as many offset tensors as output tensors, at least one");
+  TORCH_CHECK(outs.size() <= GS_MAX_SEGMENTS, "BatchSplit: at most ", GS_MAX_SEGMENTS,
+              " tensors, got ", outs.size());
+  const int idb = IdBytes(data, "data");
+  const int64_t B = NumBatches(data_ptr, "data_ptr");
+  std::vector<void*> dp;
+  std::vector<const int64_t*> pp;
+  for (size_t s = 0; s < outs.size(); ++s) {
+    TORCH_CHECK(IdBytes(outs[s], "output") == idb, "BatchSplit: outputs differ in dtype from data");
+    TORCH_CHECK(NumBatches(out_ptrs[s], "output offsets") == B,
+                "BatchSplit: offsets differ in length");
+    dp.push_back(outs[s].data_ptr());
+    pp.push_back(out_ptrs[s].data_ptr<int64_t>());
+  }
+  const void* key = nullptr;
+  if (data_key.has_value() && data_key.value().defined()) {
+    TORCH_CHECK(IdBytes(data_key.value(), "data_key") == idb && data_key.value().numel() == data.numel(),
+                "BatchSplit: data_key must match data");
+    key = data_key.value().data_ptr();
+  }
+  Check(gs_batch_split(data.data_ptr(), data_ptr.data_ptr<int64_t>(), key, idb, data.numel(), B,
+                       dp.data(), pp.data(), static_cast<int>(pp.size()), Stream(data)),
+        "gs_batch_split");
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> BatchCooRelabel(
+    const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& coo_col,
+    const torch::Tensor& coo_row, const torch::Tensor& coo_ptr) {
+  const int idb = IdBytes(seeds, "seeds");
+  TORCH_CHECK(IdBytes(coo_row, "coo_row") == idb && IdBytes(coo_col, "coo_col") == idb,
+              "seeds and edges differ in dtype");
+  TORCH_CHECK(coo_row.numel() == coo_col.numel(), "coo_row and coo_col differ in length");
+  const int64_t B = NumBatches(seeds_ptr, "seeds_ptr");
+  TORCH_CHECK(NumBatches(coo_ptr, "coo_ptr") == B, "seeds_ptr and coo_ptr differ in length");
+  const int64_t M = seeds.numel() + coo_row.numel();
+  auto unique = torch::empty({M}, seeds.options());
+  auto unique_ptr = torch::empty({B + 1}, I64(seeds));
+  auto out_row = torch::empty_like(coo_row);
+  auto out_col = torch::empty_like(coo_col);
+  auto num = torch::empty({1}, I64(seeds));
+  auto ws = Scratch(gs_batch_relabel_workspace_bytes(M), seeds);
+  void* st = Stream(seeds);
+  HostBoxes& boxes = Boxes(seeds.device().index());
+  const int64_t ticket = boxes.next++;
+  Check(gs_batch_coo_relabel(seeds.data_ptr(), seeds_ptr.data_ptr<int64_t>(), coo_row.data_ptr(),
+                             coo_col.data_ptr(), coo_ptr.data_ptr<int64_t>(), B, seeds.numel(),
+                             coo_row.numel(), idb, unique.data_ptr(),
+                             unique_ptr.data_ptr<int64_t>(), out_row.data_ptr(), out_col.data_ptr(),
+                             num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(),
+                             boxes.slot(ticket), ticket, st),
+        "gs_batch_coo_relabel");
+  int64_t U = WaitBox(boxes.slot(ticket), ticket, st, "gs_batch_coo_relabel");
+  if (U == kLost) U = num.item<int64_t>();
+  TORCH_CHECK(U >= 0, "gs_batch_coo_relabel: a tile gave up waiting for its predecessors");
+  return {unique.narrow(0, 0, U), unique_ptr, out_row, out_col};
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> CooFilter(
+    const torch::Tensor& key, const torch::Tensor& row, const torch::Tensor& col,
+    const torch::optional<torch::Tensor>& key_ptr, const torch::Tensor& ids,
+    const torch::optional<torch::Tensor>& ids_ptr) {
+  const int idb = IdBytes(key, "coo ids");
+  TORCH_CHECK(IdBytes(row, "coo ids") == idb && IdBytes(col, "coo ids") == idb &&
+                  IdBytes(ids, "node ids") == idb,
+              "coo ids and node ids differ in dtype");
+  const int64_t E = key.numel(), n = ids.numel();
+  TORCH_CHECK(row.numel() == E && col.numel() == E, "coo_row and coo_col differ in length");
+  TORCH_CHECK(key_ptr.has_value() == ids_ptr.has_value(), "batch offsets come in pairs");
+  int64_t B = 0;
+  if (key_ptr.has_value()) {
+    B = NumBatches(key_ptr.value(), "batch_ptr");
+    TORCH_CHECK(NumBatches(ids_ptr.value(), "neighbors_ptr") == B, "batch offsets differ in length");
+  }
+  auto num = torch::empty({1}, I64(key));
+  auto ws = Scratch(gs_row_slice_workspace_bytes(n, E, 0), key);
+  void* st = Stream(key);
+  Check(gs_coo_filter_mark(key.data_ptr(), idb, E, OptI64(key_ptr, "batch_ptr"), ids.data_ptr(), n,
+                           OptI64(ids_ptr, "neighbors_ptr"), B, num.data_ptr<int64_t>(),
+                           ws.data_ptr(), ws.numel(), st),
+        "gs_coo_filter_mark");
+  const int64_t kept = num.item<int64_t>();
+  auto out_row = torch::empty({kept}, key.options());
+  auto out_col = torch::empty({kept}, key.options());
+  auto select_index = torch::empty({kept}, I64(key));
+  torch::Tensor out_ptr;
+  if (B > 0) out_ptr = torch::empty({B + 1}, I64(key));
+  Check(gs_coo_filter_compact(row.data_ptr(), col.data_ptr(), idb, E, OptI64(key_ptr, "batch_ptr"),
+                              B, out_row.data_ptr(), out_col.data_ptr(),
+                              select_index.data_ptr<int64_t>(),
+                              B > 0 ? out_ptr.data_ptr<int64_t>() : nullptr, ws.data_ptr(),
+                              ws.numel(), st),
+        "gs_coo_filter_compact");
+  return {out_row, out_col, out_ptr, select_index};
+}
+
+torch::Tensor IndexSearch(const torch::Tensor& data, const torch::Tensor& keys) {
+  const int idb = IdBytes(data, "data");
+  TORCH_CHECK(IdBytes(keys, "keys") == idb, "data and keys differ in dtype");
+  auto out = torch::empty_like(keys);
+  auto ws = Scratch(gs_index_search_workspace_bytes(data.numel()), data);
+  Check(gs_index_search(data.data_ptr(), data.numel(), keys.data_ptr(), keys.numel(), idb,
+                        out.data_ptr(), ws.data_ptr(), ws.numel(), Stream(data)),
+        "gs_index_search");
+  return out;
+}
+
 }  // namespace hip
 }  // namespace gs

@@ -139,5 +139,31 @@ std::tuple<torch::Tensor, torch::Tensor> ListSamplingProbs(const torch::Tensor& 
                                                            const torch::Tensor& probs, int64_t k,
                                                            bool replace);
 
+// ---- super-batch helpers (a batched array = flat array + int64 offsets [B+1])
+torch::Tensor BatchEncode(const torch::Tensor& data, const torch::Tensor& ptr, int64_t enc);
+torch::Tensor BatchDecode(const torch::Tensor& in, int64_t enc);
+// {offsets [B+1], decoded ids} of an encoded array sorted by batch
+std::tuple<torch::Tensor, torch::Tensor> BatchOffsets(const torch::Tensor& in, int64_t B,
+                                                      int64_t enc);
+// {concatenation batch by batch, batch of each item, its offsets}
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchConcat(
+    const std::vector<torch::Tensor>& data, const std::vector<torch::Tensor>& offsets);
+// scatters `data` back into outs (the inverse of BatchConcat)
+void BatchSplit(const torch::Tensor& data, const torch::Tensor& data_ptr,
+                const torch::optional<torch::Tensor>& data_key,
+                const std::vector<torch::Tensor>& outs, const std::vector<torch::Tensor>& out_ptrs);
+// {unique, unique_ptr, relabelled row, relabelled col}
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> BatchCooRelabel(
+    const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& coo_col,
+    const torch::Tensor& coo_row, const torch::Tensor& coo_ptr);
+// edges whose key is among ids (of the same batch, with offsets): {row, col, offsets of the
+// result (undefined without batches), select_index}; ids are kept, not renamed
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> CooFilter(
+    const torch::Tensor& key, const torch::Tensor& row, const torch::Tensor& col,
+    const torch::optional<torch::Tensor>& key_ptr, const torch::Tensor& ids,
+    const torch::optional<torch::Tensor>& ids_ptr);
+// position of each key in data, -1 when absent
+torch::Tensor IndexSearch(const torch::Tensor& data, const torch::Tensor& keys);
+
 }  // namespace hip
 }  // namespace gs

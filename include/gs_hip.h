@@ -285,6 +285,18 @@ int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void
                          size_t workspace_bytes, gs_mailbox* mailbox, int64_t mailbox_ticket,
                          void* stream);
 
+/* The COO flavour: replaces impl::BatchCOORelabelCUDA (src/cuda/batch_relabel.cu:482).
+ * Batch b owns seeds[seeds_ptr[b]..) and the edges [coo_ptr[b], coo_ptr[b+1]); its frontier
+ * is the distinct values of (its seeds, then its coo_row) in first-occurrence order.
+ * out_row[j] / out_col[j] = rank of coo_row[j] / coo_col[j] in the frontier of j's batch
+ * (-1 for a column id that is not in it, batch_relabel.cu:352-374). */
+int gs_batch_coo_relabel(const void* seeds, const int64_t* seeds_ptr, const void* coo_row,
+                         const void* coo_col, const int64_t* coo_ptr, int64_t num_batches,
+                         int64_t num_seeds, int64_t num_edges, int id_bytes, void* unique,
+                         int64_t* unique_ptr, void* out_row, void* out_col, int64_t* num_unique,
+                         void* workspace, size_t workspace_bytes, gs_mailbox* mailbox,
+                         int64_t mailbox_ticket, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Random walks: replace impl::fusion::FusedRandomWalkCUDA                    */
 /* (src/cuda/fusion/random_walk.cu:52) and FusedMetapathRandomWalkCUDA         */
@@ -403,6 +415,31 @@ int gs_col_row_slice_compact(int64_t D, int id_bytes, void* out_indices, int64_t
                              int64_t* parent_index, void* workspace, size_t workspace_bytes,
                              void* stream);
 
+/* Membership filter of a COO that keeps global ids: replaces
+ * impl::COORowSlicingGlobalIdCUDA, BatchCOOSlicingCUDA (src/cuda/batch_slicing.cu:325,232)
+ * and BatchCOORowSlicingCUDA (src/cuda/slicing.cu:774).  Edge e survives when key[e] is
+ * among `ids`; with num_batches > 0 the edges are cut into batches at key_batch_ptr and
+ * the ids at ids_batch_ptr (device int64[num_batches+1]) and an edge is looked up among
+ * the ids of its own batch (ids below 2^44).  mark: *num_kept (device scalar).  compact
+ * (same workspace, gs_row_slice_workspace_bytes(num_ids, E, 0)): out_row / out_col = the
+ * surviving edges in order, select_index (may be NULL) their positions, out_batch_ptr (may
+ * be NULL) the batch offsets of the result. */
+int gs_coo_filter_mark(const void* key, int id_bytes, int64_t E, const int64_t* key_batch_ptr,
+                       const void* ids, int64_t num_ids, const int64_t* ids_batch_ptr,
+                       int64_t num_batches, int64_t* num_kept, void* workspace,
+                       size_t workspace_bytes, void* stream);
+int gs_coo_filter_compact(const void* row, const void* col, int id_bytes, int64_t E,
+                          const int64_t* key_batch_ptr, int64_t num_batches, void* out_row,
+                          void* out_col, int64_t* select_index, int64_t* out_batch_ptr,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
+/* out[i] = position of keys[i] in data, -1 when absent (the last position when data holds
+ * a value twice): replaces impl::IndexHashMapInsertCUDA + IndexHashMapSearchCUDA
+ * (src/cuda/index_search.cu:83,116; src/tensor_ops.cc:24-33).  out is id_bytes wide. */
+size_t gs_index_search_workspace_bytes(int64_t n);
+int gs_index_search(const void* data, int64_t n, const void* keys, int64_t m, int id_bytes,
+                    void* out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Format conversion: replaces impl::CSC2COOCUDA and impl::COO2CSCCUDA          */
 /* (src/cuda/format_transform.cu:35,135).                                      */
@@ -428,6 +465,46 @@ int gs_coo2csc(const void* key, const void* value, int id_bytes, int64_t E, int6
  * offsets[b+1]-offsets[b]+1 entries, re-based to start at 0, one batch after the other. */
 int gs_indptr_split(const int64_t* indptr, const int64_t* offsets, int64_t num_batches,
                     int64_t total, int64_t* out, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Super-batch plumbing.  A batched array is a flat array plus device int64     */
+/* offsets [num_batches+1].                                                    */
+/* ------------------------------------------------------------------------- */
+/* out[i] = data[i] + batch(i) * encoding_size: replaces impl::BatchEncodeCUDA
+ * (src/cuda/batch_coding.cu:74).  32-bit ids: num_batches * encoding_size must fit. */
+int gs_batch_encode(const void* data, int id_bytes, int64_t n, const int64_t* ptr,
+                    int64_t num_batches, int64_t encoding_size, void* out, void* stream);
+
+/* out_data[i] = in[i] mod encoding_size, out_batch[i] = in[i] / encoding_size (either may be
+ * NULL): replaces impl::BatchDecodeCUDA (src/cuda/batch_coding.cu:96). */
+int gs_batch_decode(const void* in, int id_bytes, int64_t n, int64_t encoding_size, void* out_data,
+                    void* out_batch, void* stream);
+
+/* `in` encoded and sorted by batch: out_ptr[num_batches+1] = the batches' offsets, out_data
+ * (may be NULL) the decoded ids: replaces impl::GetBatchOffsets (src/cuda/batch_coding.cu:110). */
+int gs_batch_offsets(const void* in, int id_bytes, int64_t n, int64_t num_batches,
+                     int64_t encoding_size, int64_t* out_ptr, void* out_data, void* stream);
+
+/* Concatenation batch by batch: replaces impl::BatchConcatCUDA
+ * (src/cuda/batch_concat.cu:117).  The *_host arguments are HOST arrays of num_segments
+ * device pointers.  offsets: out_ptr[b] = sum over segments of their ptr[b] (total in
+ * out_ptr[num_batches]).  fill: batch b of `out` = batch b of segment 0, then of segment
+ * 1, ...; out_key[i] (may be NULL) = the batch of item i.  max_segment_len: the longest
+ * segment (sizes the launch). */
+#define GS_MAX_SEGMENTS 8
+int gs_batch_concat_offsets(const int64_t* const* segment_ptrs_host, int num_segments,
+                            int64_t num_batches, int64_t* out_ptr, void* stream);
+int gs_batch_concat_fill(const void* const* segment_data_host,
+                         const int64_t* const* segment_ptrs_host, int num_segments,
+                         int64_t num_batches, int64_t max_segment_len, int id_bytes,
+                         const int64_t* out_ptr, void* out, void* out_key, void* stream);
+
+/* The inverse: replaces impl::BatchSplit2CUDA (src/cuda/batch_split2.cu:100).  Item i of
+ * batch b (= data_key[i], or found from data_ptr when data_key is NULL) goes to the
+ * segment whose share of batch b holds its local position, at out_ptrs[s][b] + ... */
+int gs_batch_split(const void* data, const int64_t* data_ptr, const void* data_key, int id_bytes,
+                   int64_t n, int64_t num_batches, void* const* out_data_host,
+                   const int64_t* const* out_ptrs_host, int num_segments, void* stream);
 
 #ifdef __cplusplus
 }

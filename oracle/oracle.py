@@ -281,6 +281,122 @@ def batch_csr_relabel(seeds, seeds_ptr, indices, indices_ptr):
     return cat(uniques), np.asarray(ptr, dtype=np.int64), cat(outs)
 
 
+def batch_coo_relabel(seeds, seeds_ptr, coo_col, coo_row, coo_ptr):
+    """src/cuda/batch_relabel.cu:377-480: per batch, frontier = distinct (seeds, then coo_row)
+    in first-occurrence order; rows and columns renamed to their rank in it (-1 when absent).
+
+    Returns (unique, unique_ptr, out_row, out_col)."""
+    seeds, coo_col, coo_row = _i64(seeds), _i64(coo_col), _i64(coo_row)
+    seeds_ptr, coo_ptr = _i64(seeds_ptr), _i64(coo_ptr)
+    uniques, rows, cols, ptr = [], [], [], [0]
+    for b in range(seeds_ptr.size - 1):
+        s_b = seeds[seeds_ptr[b]:seeds_ptr[b + 1]]
+        r_b = coo_row[coo_ptr[b]:coo_ptr[b + 1]]
+        c_b = coo_col[coo_ptr[b]:coo_ptr[b + 1]]
+        frontier, (rel_r, rel_c) = relabel([s_b, r_b], [r_b, c_b])
+        uniques.append(frontier)
+        rows.append(rel_r)
+        cols.append(rel_c)
+        ptr.append(ptr[-1] + frontier.size)
+    cat = lambda xs: np.concatenate(xs) if xs else np.empty(0, np.int64)  # noqa: E731
+    return cat(uniques), np.asarray(ptr, dtype=np.int64), cat(rows), cat(cols)
+
+
+# -------------------------------------------------------- super-batch helpers
+def _batch_ids(ptr, n):
+    ptr = _i64(ptr)
+    return np.repeat(np.arange(ptr.size - 1, dtype=np.int64), np.diff(ptr))[:n]
+
+
+def batch_encode(data, ptr, encoding_size):
+    """src/cuda/batch_coding.cu:11-28,74-94: data[i] + batch(i) * encoding_size"""
+    data = _i64(data)
+    return data + _batch_ids(ptr, data.size) * encoding_size
+
+
+def batch_decode(data, encoding_size):
+    """src/cuda/batch_coding.cu:96-108 -> (in mod size, in // size)"""
+    data = _i64(data)
+    batch = data // encoding_size
+    return data - batch * encoding_size, batch
+
+
+def batch_offsets(data, num_batches, encoding_size):
+    """src/cuda/batch_coding.cu:110-120 -> (ptr, decoded): ptr[b+1] = #items of batch <= b"""
+    decoded, batch = batch_decode(data, encoding_size)
+    ptr = np.zeros(num_batches + 1, dtype=np.int64)
+    ptr[1:] = np.searchsorted(batch, np.arange(num_batches), side="right")
+    return ptr, decoded
+
+
+def batch_concat(datas, ptrs):
+    """src/cuda/batch_concat.cu:13-119 -> (total, key, total_ptr): batch b of the result is
+    batch b of every input, one input after the other"""
+    datas, ptrs = [_i64(d) for d in datas], [_i64(p) for p in ptrs]
+    nb = ptrs[0].size - 1
+    total, key = [], []
+    for b in range(nb):
+        for d, p in zip(datas, ptrs):
+            total.append(d[p[b]:p[b + 1]])
+            key.append(np.full(p[b + 1] - p[b], b, dtype=np.int64))
+    cat = lambda xs: np.concatenate(xs) if xs else np.empty(0, np.int64)  # noqa: E731
+    return cat(total), cat(key), np.sum(ptrs, axis=0).astype(np.int64)
+
+
+def batch_split(data, data_ptr, out_ptrs):
+    """src/cuda/batch_split2.cu:12-100: the inverse of batch_concat -> list of segments"""
+    data, data_ptr = _i64(data), _i64(data_ptr)
+    out_ptrs = [_i64(p) for p in out_ptrs]
+    outs = [np.empty(p[-1], dtype=np.int64) for p in out_ptrs]
+    for b in range(data_ptr.size - 1):
+        at = data_ptr[b]
+        for o, p in zip(outs, out_ptrs):
+            n = p[b + 1] - p[b]
+            o[p[b]:p[b + 1]] = data[at:at + n]
+            at += n
+    return outs
+
+
+def batch_unique(data, data_ptr, sort=False):
+    """src/cuda/batch_unique.cu:131-207 (first-occurrence order) and, with sort, what
+    :209-275 is for (ascending inside every batch) -> (unique, unique_ptr, unique_key)"""
+    data, data_ptr = _i64(data), _i64(data_ptr)
+    uniques, ptr = [], [0]
+    for b in range(data_ptr.size - 1):
+        u = unique(data[data_ptr[b]:data_ptr[b + 1]])
+        uniques.append(np.sort(u) if sort else u)
+        ptr.append(ptr[-1] + u.size)
+    out = np.concatenate(uniques) if uniques else np.empty(0, np.int64)
+    ptr = np.asarray(ptr, dtype=np.int64)
+    return out, ptr, _batch_ids(ptr, out.size)
+
+
+def coo_filter(key, row, col, ids, key_ptr=None, ids_ptr=None):
+    """src/cuda/batch_slicing.cu:150-232 (batched) and :281-329 (one id set): the edges
+    whose key is among the ids (of their own batch), ids kept
+    -> (row, col, offsets of the batches | None, select_index)"""
+    key, row, col, ids = _i64(key), _i64(row), _i64(col), _i64(ids)
+    if key_ptr is None:
+        keep = np.isin(key, ids)
+        out_ptr = None
+    else:
+        key_ptr, ids_ptr = _i64(key_ptr), _i64(ids_ptr)
+        keep = np.zeros(key.size, dtype=bool)
+        for b in range(key_ptr.size - 1):
+            lo, hi = key_ptr[b], key_ptr[b + 1]
+            keep[lo:hi] = np.isin(key[lo:hi], ids[ids_ptr[b]:ids_ptr[b + 1]])
+        out_ptr = np.concatenate([[0], np.cumsum(keep)])[key_ptr].astype(np.int64)
+    sel = np.flatnonzero(keep).astype(np.int64)
+    return row[sel], col[sel], out_ptr, sel
+
+
+def index_search(data, keys):
+    """src/cuda/index_search.cu:83-140, src/tensor_ops.cc:24-33: position of every key in
+    data, -1 when absent (the last position of a repeated value)"""
+    uniq, last = _last_position_lookup(_i64(data))
+    return _lookup(uniq, last, _i64(keys))
+
+
 def random_walk(indptr, indices, seeds, length, seed=0, replay=None):
     """src/cuda/fusion/random_walk.cu:52-68 -> flat trace, memory [L+1][n]"""
     indptr, indices, seeds = _i64(indptr), _i64(indices), _i64(seeds)

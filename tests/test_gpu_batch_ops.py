@@ -1,0 +1,297 @@
+"""GPU parity: the super-batch helpers (encode / decode / offsets, concat / split, per-batch
+unique and COO relabel, batched COO filters, index search) vs the numpy oracle, through the
+C ABI and through torch.ops.gs_ops / Graph."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from graph_sampling_amd import capi
+from tests.util import rmat_csc_np, to_dev
+
+pytestmark = pytest.mark.gpu
+
+ID_DTYPES = [torch.int64, torch.int32]
+
+
+def _np(t):
+    return t.cpu().numpy().astype(np.int64)
+
+
+def _ptr(sizes):
+    return np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("sizes", [[5], [0, 3, 0, 0, 7], [300, 1, 0, 5000, 257, 256]])
+def test_encode_decode_offsets(dev, sizes, idt):
+    ptr = _ptr(sizes)
+    enc = 1 << 20
+    data = np.random.default_rng(len(sizes)).integers(0, enc, size=ptr[-1]).astype(np.int64)
+    got = capi.batch_encode(to_dev(data, dev, idt), to_dev(ptr, dev), enc)
+    want = O.batch_encode(data, ptr, enc)
+    assert np.array_equal(_np(got), want)
+    dec, batch = capi.batch_decode(got, enc)
+    assert np.array_equal(_np(dec), data)
+    assert np.array_equal(_np(batch), np.repeat(np.arange(len(sizes)), sizes))
+    g_ptr, g_dec = capi.batch_offsets(got, len(sizes), enc)
+    w_ptr, w_dec = O.batch_offsets(want, len(sizes), enc)
+    assert np.array_equal(_np(g_ptr), w_ptr) and np.array_equal(w_ptr, ptr)
+    assert np.array_equal(_np(g_dec), w_dec)
+
+
+def test_encode_refuses_what_does_not_fit_32_bits(dev):
+    data = torch.zeros(4, dtype=torch.int32, device=dev)
+    ptr = torch.tensor([0, 2, 4], device=dev)
+    with pytest.raises(capi.GsError, match="32-bit"):
+        capi.batch_encode(data, ptr, 1 << 31)
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("B,nseg", [(1, 1), (4, 2), (33, 3), (7, 8)])
+def test_concat_split_round_trip(dev, B, nseg, idt):
+    rng = np.random.default_rng(B * 10 + nseg)
+    ptrs = [_ptr(rng.integers(0, 400, size=B)) for _ in range(nseg)]
+    datas = [rng.integers(0, 1 << 30, size=p[-1]).astype(np.int64) for p in ptrs]
+    d_ptrs = [to_dev(p, dev) for p in ptrs]
+    got = capi.batch_concat([to_dev(d, dev, idt) for d in datas], d_ptrs)
+    want = O.batch_concat(datas, ptrs)
+    for g, w in zip(got, want):
+        assert np.array_equal(_np(g), w)
+    # and back: with the batch of every item given, and found from the offsets
+    for key in (got[1], None):
+        back = capi.batch_split(got[0], got[2], key, d_ptrs)
+        for b, d in zip(back, datas):
+            assert np.array_equal(_np(b), d)
+    for b, d in zip(O.batch_split(want[0], want[2], ptrs), datas):
+        assert np.array_equal(b, d)
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+def test_ops_concat_split_unique(dev, idt):
+    import graph_sampling_amd as gs
+    gs.load_library()
+    ops = torch.ops.gs_ops
+    rng = np.random.default_rng(0)
+    ptrs = [_ptr(rng.integers(0, 300, size=9)) for _ in range(2)]
+    datas = [rng.integers(0, 200, size=p[-1]).astype(np.int64) for p in ptrs]
+    t_d = [to_dev(d, dev, idt) for d in datas]
+    t_p = [to_dev(p, dev) for p in ptrs]
+    total, key, total_ptr = ops.BatchConcat(t_d, t_p)
+    w_total, w_key, w_ptr = O.batch_concat(datas, ptrs)
+    assert np.array_equal(_np(total), w_total) and np.array_equal(_np(key), w_key)
+    assert np.array_equal(_np(total_ptr), w_ptr)
+    outs = [torch.empty_like(d) for d in t_d]
+    ops.BatchSplit(total, total_ptr, key, outs, t_p)
+    for o, d in zip(outs, datas):
+        assert np.array_equal(_np(o), d)
+    for name, sort in (("BatchUnique", False), ("BatchUnique2", True)):
+        u, u_ptr, u_key = getattr(ops, name)(total, total_ptr)
+        w_u, w_uptr, w_ukey = O.batch_unique(w_total, w_ptr, sort=sort)
+        assert np.array_equal(_np(u), w_u) and np.array_equal(_np(u_ptr), w_uptr)
+        assert np.array_equal(_np(u_key), w_ukey)
+    u, u_ptr, u_key = ops.BatchUniqueByKey(total, total_ptr, key)
+    assert np.array_equal(_np(u), O.batch_unique(w_total, w_ptr)[0])
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("B", [1, 5, 64])
+def test_batch_coo_relabel(dev, B, idt):
+    rng = np.random.default_rng(B)
+    seeds_ptr = _ptr(rng.integers(0, 50, size=B))
+    coo_ptr = _ptr(rng.integers(0, 900, size=B))
+    seeds = rng.integers(0, 500, size=seeds_ptr[-1]).astype(np.int64)
+    row = rng.integers(0, 500, size=coo_ptr[-1]).astype(np.int64)
+    # columns are mostly seeds of the same batch; some are strangers and come back as -1
+    col = rng.integers(0, 500, size=coo_ptr[-1]).astype(np.int64)
+    got = capi.batch_coo_relabel(to_dev(seeds, dev, idt), to_dev(seeds_ptr, dev),
+                                 to_dev(row, dev, idt), to_dev(col, dev, idt), to_dev(coo_ptr, dev))
+    w_u, w_uptr, w_row, w_col = O.batch_coo_relabel(seeds, seeds_ptr, col, row, coo_ptr)
+    n_u = int(got[4].item())
+    assert n_u == w_u.size
+    assert np.array_equal(_np(got[0][:n_u]), w_u) and np.array_equal(_np(got[1]), w_uptr)
+    assert np.array_equal(_np(got[2]), w_row) and np.array_equal(_np(got[3]), w_col)
+    assert (w_col == -1).any() and (w_row >= 0).all()
+    # through the op, with the reference's argument and result order
+    import graph_sampling_amd as gs
+    gs.load_library()
+    u, u_ptr, o_row, o_col, o_ptr = torch.ops.gs_ops.BatchCOORelabel(
+        to_dev(seeds, dev, idt), to_dev(seeds_ptr, dev), to_dev(col, dev, idt),
+        to_dev(row, dev, idt), to_dev(coo_ptr, dev))
+    assert np.array_equal(_np(u), w_u) and np.array_equal(_np(o_row), w_row)
+    assert np.array_equal(_np(o_col), w_col) and np.array_equal(_np(o_ptr), coo_ptr)
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("B", [0, 1, 6, 40])
+def test_coo_filter(dev, B, idt):
+    rng = np.random.default_rng(B + 100)
+    n = 1 << 10
+    if B == 0:
+        E, key_ptr, ids_ptr = 20000, None, None
+        ids = rng.permutation(n)[:300].astype(np.int64)
+    else:
+        key_ptr = _ptr(rng.integers(0, 3000, size=B))
+        id_sizes = rng.integers(0, 200, size=B)
+        ids_ptr = _ptr(id_sizes)
+        E = key_ptr[-1]
+        ids = np.concatenate([rng.permutation(n)[:s] for s in id_sizes] + [np.empty(0, np.int64)]).astype(np.int64)
+    row = rng.integers(0, n, size=E).astype(np.int64)
+    col = rng.integers(0, n, size=E).astype(np.int64)
+    got = capi.coo_filter(to_dev(row, dev, idt), to_dev(row, dev, idt), to_dev(col, dev, idt),
+                          to_dev(ids, dev, idt),
+                          None if B == 0 else to_dev(key_ptr, dev),
+                          None if B == 0 else to_dev(ids_ptr, dev))
+    want = O.coo_filter(row, row, col, ids, key_ptr, ids_ptr)
+    for g, w in zip(got, want):
+        if w is None:
+            assert g is None
+        else:
+            assert np.array_equal(_np(g), w)
+
+
+def test_ops_coo_slicing_and_global_id(dev):
+    import graph_sampling_amd as gs
+    gs.load_library()
+    ops = torch.ops.gs_ops
+    rng = np.random.default_rng(7)
+    n, B = 512, 5
+    key_ptr = _ptr(rng.integers(100, 2000, size=B))
+    id_sizes = rng.integers(1, 100, size=B)
+    ids_ptr = _ptr(id_sizes)
+    ids = np.concatenate([rng.permutation(n)[:s] for s in id_sizes]).astype(np.int64)
+    row = rng.integers(0, n, size=key_ptr[-1]).astype(np.int64)
+    col = rng.integers(0, n, size=key_ptr[-1]).astype(np.int64)
+    for axis, key in ((0, col), (1, row)):
+        r, c, p = ops.BatchCOOSlicing(axis, to_dev(row, dev), to_dev(col, dev), to_dev(key_ptr, dev),
+                                      to_dev(ids, dev), to_dev(ids_ptr, dev))
+        w = O.coo_filter(key, row, col, ids, key_ptr, ids_ptr)
+        assert np.array_equal(_np(r), w[0]) and np.array_equal(_np(c), w[1]) and np.array_equal(_np(p), w[2])
+    r, c = ops.COORowSlicingGlobalId(to_dev(row, dev), to_dev(col, dev), to_dev(ids[:50], dev))
+    w = O.coo_filter(row, row, col, ids[:50])
+    assert np.array_equal(_np(r), w[0]) and np.array_equal(_np(c), w[1])
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+def test_index_search(dev, idt):
+    rng = np.random.default_rng(3)
+    data = rng.permutation(1 << 16)[:5000].astype(np.int64)
+    data[10] = data[3]      # a repeated value reports its last position
+    keys = rng.integers(0, 1 << 16, size=20000).astype(np.int64)
+    got = capi.index_search(to_dev(data, dev, idt), to_dev(keys, dev, idt))
+    want = O.index_search(data, keys)
+    assert np.array_equal(_np(got), want)
+    assert (want >= 0).any() and (want == -1).any()
+    hit = want >= 0
+    assert np.array_equal(data[want[hit]], keys[hit])
+    import graph_sampling_amd as gs
+    gs.load_library()
+    assert np.array_equal(_np(torch.ops.gs_ops.index_search(to_dev(data, dev, idt), to_dev(keys, dev, idt))), want)
+
+
+def test_batch_list_sampling_with_probs(dev):
+    import graph_sampling_amd as gs
+    gs.load_library()
+    rng = np.random.default_rng(5)
+    rng_ptr = _ptr([3000, 10, 0, 800])
+    probs = (1.0 - rng.random(rng_ptr[-1])).astype(np.float32)
+    probs[5:40] = 0.0           # never picked while positive weights remain
+    k = 100
+    idx, out_ptr = torch.ops.gs_ops.batch_list_sampling_with_probs(
+        to_dev(probs, dev), k, False, to_dev(rng_ptr, dev))
+    idx, out_ptr = _np(idx), _np(out_ptr)
+    assert np.array_equal(out_ptr, [0, 100, 110, 110, 210])
+    for b in range(4):
+        got = idx[out_ptr[b]:out_ptr[b + 1]]
+        assert np.unique(got).size == got.size
+        assert ((got >= rng_ptr[b]) & (got < rng_ptr[b + 1])).all()
+    assert np.array_equal(idx[100:110], np.arange(3000, 3010))   # a short range is taken whole
+    assert not np.isin(idx[:100], np.arange(5, 40)).any()
+
+
+def test_graph_batch_slicing_split_decode(dev):
+    import graph_sampling_amd as gs
+    n = 1 << 10
+    indptr, indices = rmat_csc_np(n, 1 << 14, seed=11)
+    data = np.random.default_rng(0).random(indices.size).astype(np.float32)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev))
+    g._CAPI_SetData(to_dev(data, dev))
+    nid_ptr = np.array([0, 100, 100, 260], dtype=np.int64)
+    n_ids = np.random.default_rng(1).integers(0, n, size=260).astype(np.int64)
+    for encoding in (False, True):
+        sub, offsets = g._CAPI_BatchSlicing(to_dev(n_ids, dev), to_dev(nid_ptr, dev), 0, gs._CSC,
+                                            gs._CSC + gs._COO, False, encoding)
+        s_ptr, s_col, s_idx, s_sel = O.slice_columns(indptr, indices, n_ids, True)
+        ptr, idx, _ = sub._CAPI_GetCSC()
+        assert np.array_equal(_np(ptr), s_ptr)
+        assert np.array_equal(_np(offsets), s_ptr[nid_ptr])
+        want_idx = O.batch_encode(s_idx, s_ptr[nid_ptr], n) if encoding else s_idx
+        assert np.array_equal(_np(idx), want_idx)
+        row, col = sub._CAPI_GetBatchCOO()
+        assert np.array_equal(_np(row), want_idx) and np.array_equal(_np(col), s_col)
+        assert np.array_equal(sub._CAPI_GetData("default").cpu().numpy(), data[s_sel])
+        assert np.array_equal(_np(sub._CAPI_GetCols()), O.batch_encode(n_ids, nid_ptr, n))
+        assert sub._CAPI_GetNumRows() == 3 * n and sub._CAPI_GetNumCols() == 260
+    # Split: pieces of 300 columns, the last one shorter; edge data follows
+    pieces = g._CAPI_Split(300)
+    assert [p._CAPI_GetNumCols() for p in pieces] == [300, 300, 300, 124]
+    for i, p in enumerate(pieces):
+        lo, hi = i * 300, min((i + 1) * 300, n)
+        ptr, idx, _ = p._CAPI_GetCSC()
+        assert np.array_equal(_np(ptr), indptr[lo:hi + 1] - indptr[lo])
+        assert np.array_equal(_np(idx), indices[indptr[lo]:indptr[hi]])
+        assert np.array_equal(p._CAPI_GetData("default").cpu().numpy(), data[indptr[lo]:indptr[hi]])
+    # Decode: ids back to one batch's range
+    sub, _ = g._CAPI_BatchSlicing(to_dev(n_ids, dev), to_dev(nid_ptr, dev), 0, gs._CSC, gs._CSC,
+                                  True, True)
+    rows_before = _np(sub._CAPI_GetRows())
+    sub._CAPI_Decode(n)
+    assert np.array_equal(_np(sub._CAPI_GetCols()), n_ids)
+    assert np.array_equal(_np(sub._CAPI_GetRows()), rows_before % n)
+
+
+def test_fastgcn_super_batch_equals_batch_by_batch(dev):
+    """The flow of the reference's examples/fastgcn/batching.py:70-106 on B small batches at
+    once against the same steps done one batch at a time."""
+    import graph_sampling_amd as gs
+    gs.load_library()
+    ops = torch.ops.gs_ops
+    n, B, bs = 1 << 11, 6, 64
+    indptr, indices = rmat_csc_np(n, 1 << 15, seed=12)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev))
+    rng = np.random.default_rng(2)
+    seeds = rng.permutation(n)[:B * bs].astype(np.int64)
+    seeds_ptr = np.arange(B + 1, dtype=np.int64) * bs
+    t_seeds, t_seeds_ptr = to_dev(seeds, dev), to_dev(seeds_ptr, dev)
+
+    sub = g._CAPI_Slicing(t_seeds, 0, gs._CSC, gs._CSC + gs._COO, False)
+    _, idx, idx_ptr = sub.GetBatchCSC(t_seeds_ptr)
+    encoded = ops.BatchEncode(idx, idx_ptr, n)
+    neighbors = torch.unique(encoded)
+    nb_ptr, nb_ids = ops.GetBatchOffsets(neighbors, B, n)
+    # "selected": every third neighbour of each batch, in encoded form
+    keep = torch.arange(neighbors.numel(), device=dev) % 3 == 0
+    selected = neighbors[keep]
+    coo_row, coo_col = sub.GetBatchCOO()
+    s_row, s_col = ops.COORowSlicingGlobalId(encoded, coo_col, selected)
+    s_ptr, s_row = ops.GetBatchOffsets(s_row, B, n)
+    u, u_ptr, r_row, r_col, r_ptr = ops.BatchCOORelabel(t_seeds, t_seeds_ptr, s_col, s_row, s_ptr)
+    # columns of the sliced COO are local to the super-batch (0..B*bs): relabel them as ids of seeds
+    u, u_ptr, r_row, r_col = _np(u), _np(u_ptr), _np(r_row), _np(r_col)
+    s_ptr = _np(s_ptr)
+    nb_ptr, nb_ids, neighbors_np = _np(nb_ptr), _np(nb_ids), _np(neighbors)
+    for b in range(B):
+        sb = seeds[b * bs:(b + 1) * bs]
+        _, cc, ii, _ = O.slice_columns(indptr, indices, sb, True)
+        nb = np.unique(ii)
+        assert np.array_equal(nb_ids[nb_ptr[b]:nb_ptr[b + 1]], nb)
+        sel_b = _np(selected)[(_np(selected) // n) == b] % n
+        keep_e = np.isin(ii, sel_b)
+        rows_b, cols_b = ii[keep_e], cc[keep_e] + b * bs
+        lo, hi = s_ptr[b], s_ptr[b + 1]
+        assert np.array_equal(_np(s_row)[lo:hi], rows_b) and np.array_equal(_np(s_col)[lo:hi], cols_b)
+        frontier, (w_row, w_col) = O.relabel([sb, rows_b], [rows_b, cols_b])
+        assert np.array_equal(u[u_ptr[b]:u_ptr[b + 1]], frontier)
+        assert np.array_equal(r_row[lo:hi], w_row) and np.array_equal(r_col[lo:hi], w_col)

@@ -374,3 +374,68 @@ def test_oracle_reproduces_committed_goldens():
     assert np.array_equal(tr, GOLD["walk_trace"])
     fr, rel = O.relabel([cols, GOLD["floyd_sub_indices"]], [GOLD["floyd_sub_indices"]])
     assert np.array_equal(fr, GOLD["relabel_frontier"]) and np.array_equal(rel[0], GOLD["relabel_rows"])
+
+
+# ------------------------------------------------- induced subgraph, super-batch
+def test_col_row_slice_against_an_edge_loop():
+    indptr, indices = rmat_csc_np(64, 600, seed=1)
+    rng = np.random.default_rng(0)
+    cols = rng.integers(0, 64, size=20)
+    rows = rng.permutation(64)[:25]
+    got = O.col_row_slice(indptr, indices, cols, rows)
+    pos = {int(r): i for i, r in enumerate(rows)}
+    ptr, idx, sel, par, p = [0], [], [], [], 0
+    for c in cols:
+        for e in range(indptr[c], indptr[c + 1]):
+            if int(indices[e]) in pos:
+                idx.append(pos[int(indices[e])])
+                sel.append(p)
+                par.append(e)
+            p += 1
+        ptr.append(len(idx))
+    for g, w in zip(got, (ptr, idx, sel, par)):
+        assert np.array_equal(g, w)
+    # batched: rows keep their id; a column only sees the ids of its own batch
+    col_ptr, row_ptr = np.array([0, 8, 20]), np.array([0, 10, 25])
+    got = O.col_row_slice(indptr, indices, cols, rows, col_ptr, row_ptr, 64)
+    ptr, idx = [0], []
+    for r, c in enumerate(cols):
+        b = 0 if r < 8 else 1
+        mine = set(rows[row_ptr[b]:row_ptr[b + 1]].tolist())
+        idx += [int(v) for v in indices[indptr[c]:indptr[c + 1]] if int(v) in mine]
+        ptr.append(len(idx))
+    assert np.array_equal(got[0], ptr) and np.array_equal(got[1], idx)
+
+
+def test_batch_helpers_worked_examples():
+    # two inputs, two batches: batch 0 = [1,2 | 10], batch 1 = [3,4,5 | 20,30]
+    d = [np.array([1, 2, 3, 4, 5]), np.array([10, 20, 30])]
+    p = [np.array([0, 2, 5]), np.array([0, 1, 3])]
+    total, key, total_ptr = O.batch_concat(d, p)
+    assert total.tolist() == [1, 2, 10, 3, 4, 5, 20, 30]
+    assert key.tolist() == [0, 0, 0, 1, 1, 1, 1, 1] and total_ptr.tolist() == [0, 3, 8]
+    back = O.batch_split(total, total_ptr, p)
+    assert back[0].tolist() == [1, 2, 3, 4, 5] and back[1].tolist() == [10, 20, 30]
+    # encode / decode / offsets; batch 1 is empty
+    enc = O.batch_encode(np.array([5, 6, 7, 8]), np.array([0, 1, 1, 4]), 100)
+    assert enc.tolist() == [5, 206, 207, 208]
+    assert [a.tolist() for a in O.batch_decode(enc, 100)] == [[5, 6, 7, 8], [0, 2, 2, 2]]
+    ptr, dec = O.batch_offsets(enc, 3, 100)
+    assert ptr.tolist() == [0, 1, 1, 4] and dec.tolist() == [5, 6, 7, 8]
+    # per-batch unique: first occurrence, or ascending
+    assert [a.tolist() for a in O.batch_unique(np.array([3, 1, 3, 2, 2, 9]), np.array([0, 3, 6]))] == \
+        [[3, 1, 2, 9], [0, 2, 4], [0, 0, 1, 1]]
+    assert O.batch_unique(np.array([3, 1, 3, 2, 2, 9]), np.array([0, 3, 6]), sort=True)[0].tolist() == \
+        [1, 3, 2, 9]
+    # position lookup, last occurrence of a repeated value
+    assert O.index_search(np.array([5, 6, 5]), np.array([5, 7, 6])).tolist() == [2, -1, 1]
+    # COO relabel: batch 0 seeds [4], edges (7->4), (4->4); batch 1 seeds [5,6], edges (9->5), (5->6)
+    u, u_ptr, row, col = O.batch_coo_relabel(np.array([4, 5, 6]), np.array([0, 1, 3]),
+                                             np.array([4, 4, 5, 6]), np.array([7, 4, 9, 5]),
+                                             np.array([0, 2, 4]))
+    assert u.tolist() == [4, 7, 5, 6, 9] and u_ptr.tolist() == [0, 2, 5]
+    assert row.tolist() == [1, 0, 2, 0] and col.tolist() == [0, 0, 0, 1]
+    # batched filter: the id 3 belongs to batch 1 only
+    r, c, ptr, sel = O.coo_filter(np.array([3, 4, 3, 5]), np.array([3, 4, 3, 5]), np.array([0, 1, 2, 3]),
+                                  np.array([4, 3]), np.array([0, 2, 4]), np.array([0, 1, 2]))
+    assert r.tolist() == [4, 3] and c.tolist() == [1, 2] and ptr.tolist() == [0, 1, 2] and sel.tolist() == [1, 2]
