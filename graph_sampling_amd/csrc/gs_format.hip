@@ -38,7 +38,7 @@ __device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz,
-               IdT* __restrict__ col) {
+               const IdT* __restrict__ ids, IdT* __restrict__ col) {
   __shared__ int64_t s_ptr[kStage + 1];
   __shared__ int64_t s_rows[2];
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
@@ -56,8 +56,40 @@ csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz
   for (int k = 0; k < kItems; ++k) {
     const int64_t p = p0 + k * kThreads + threadIdx.x;
     if (p >= p1) break;
-    col[p] = static_cast<IdT>(row_lo + (staged ? upper_bound(s_ptr, nrows + 1, p)
-                                               : upper_bound(indptr + row_lo, nrows + 1, p)) - 1);
+    const int64_t c = row_lo + (staged ? upper_bound(s_ptr, nrows + 1, p)
+                                       : upper_bound(indptr + row_lo, nrows + 1, p)) - 1;
+    // doubly-compressed: stored column c stands for node ids[c] (format_transform.cu:48-60)
+    col[p] = ids ? ids[c] : static_cast<IdT>(c);
+  }
+}
+
+// CSC -> doubly-compressed CSC: the columns that own at least one edge, in order, and
+// their offsets (what format_transform.cu:172-203 builds from the sorted COO).
+struct NonEmptyColumn {
+  const int64_t* indptr;
+  __device__ __forceinline__ int64_t operator()(int64_t c) const {
+    return indptr[c + 1] > indptr[c] ? 1 : 0;
+  }
+};
+
+template <typename IdT>
+__global__ void __launch_bounds__(kThreads)
+compress_kernel(const int64_t* __restrict__ indptr, int64_t num_cols,
+                const int64_t* __restrict__ prefix, IdT* __restrict__ val_ids,
+                int64_t* __restrict__ out_indptr, int64_t* __restrict__ num_valid) {
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (c > num_cols) return;
+  if (c == num_cols) {
+    const int64_t total = prefix[num_cols];
+    out_indptr[total] = indptr[num_cols];
+    *num_valid = total;
+    return;
+  }
+  const int64_t begin = indptr[c];
+  if (indptr[c + 1] > begin) {
+    const int64_t w = prefix[c];
+    val_ids[w] = static_cast<IdT>(c);
+    out_indptr[w] = begin;
   }
 }
 
@@ -267,11 +299,63 @@ int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, void* col, 
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (id_bytes == 8)
     hipLaunchKernelGGL((csc2coo_kernel<int64_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
-                       st, indptr, num_cols, nnz, static_cast<int64_t*>(col));
+                       st, indptr, num_cols, nnz, static_cast<const int64_t*>(nullptr),
+                       static_cast<int64_t*>(col));
   else
     hipLaunchKernelGGL((csc2coo_kernel<int32_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
-                       st, indptr, num_cols, nnz, static_cast<int32_t*>(col));
+                       st, indptr, num_cols, nnz, static_cast<const int32_t*>(nullptr),
+                       static_cast<int32_t*>(col));
   return check_launch("csc2coo");
+}
+
+int gs_dcsc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, const void* ids, void* col,
+                int id_bytes, void* stream) {
+  GS_REQUIRE(num_cols >= 0 && nnz >= 0, "gs_dcsc2coo: negative size");
+  GS_REQUIRE(nnz == 0 || (indptr && col && ids), "gs_dcsc2coo: null pointer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_dcsc2coo: id_bytes must be 4 or 8, got %d", id_bytes);
+  if (nnz == 0) return GS_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (id_bytes == 8)
+    hipLaunchKernelGGL((csc2coo_kernel<int64_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
+                       st, indptr, num_cols, nnz, static_cast<const int64_t*>(ids),
+                       static_cast<int64_t*>(col));
+  else
+    hipLaunchKernelGGL((csc2coo_kernel<int32_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
+                       st, indptr, num_cols, nnz, static_cast<const int32_t*>(ids),
+                       static_cast<int32_t*>(col));
+  return check_launch("dcsc2coo");
+}
+
+size_t gs_csc_compress_workspace_bytes(int64_t num_cols) {
+  if (num_cols < 0) num_cols = 0;
+  return padded(static_cast<size_t>(num_cols + 1) * 8) + scan_workspace_bytes(num_cols);
+}
+
+int gs_csc_compress(const int64_t* indptr, int64_t num_cols, int id_bytes, void* val_ids,
+                    int64_t* out_indptr, int64_t* num_valid, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(num_cols >= 0 && indptr && out_indptr && num_valid && (num_cols == 0 || val_ids),
+             "gs_csc_compress: bad argument");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_csc_compress: id_bytes must be 4 or 8, got %d", id_bytes);
+  Carver ws(workspace, workspace_bytes);
+  int64_t* prefix = ws.take<int64_t>(num_cols + 1);
+  int64_t* tiles = ws.take<int64_t>(scan_num_tiles(num_cols) + 1);
+  if (!ws.ok) {
+    set_error_text("gs_csc_compress: workspace needs %zu bytes, 256-byte aligned",
+                   gs_csc_compress_workspace_bytes(num_cols));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  NonEmptyColumn f{indptr};
+  GS_RETURN_IF_ERROR(exclusive_scan(f, num_cols, prefix, tiles, st));
+  const dim3 grid(blocks_for(num_cols + 1, kThreads));
+  if (id_bytes == 8)
+    hipLaunchKernelGGL(compress_kernel<int64_t>, grid, dim3(kThreads), 0, st, indptr, num_cols,
+                       prefix, static_cast<int64_t*>(val_ids), out_indptr, num_valid);
+  else
+    hipLaunchKernelGGL(compress_kernel<int32_t>, grid, dim3(kThreads), 0, st, indptr, num_cols,
+                       prefix, static_cast<int32_t*>(val_ids), out_indptr, num_valid);
+  return check_launch("csc_compress");
 }
 
 size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys) {

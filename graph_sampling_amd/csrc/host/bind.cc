@@ -65,12 +65,17 @@ TORCH_LIBRARY(gs_classes, m) {
       GS_DEF2("_CAPI_RandomWalk", "_CAPI_random_walk", &Graph::RandomWalk)
       GS_DEF2("_CAPI_SDDMM", "_CAPI_sddmm", &Graph::SDDMM)
       GS_DEF2("_CAPI_GetCSC", "_CAPI_get_csc", &Graph::GetCSCTensor)
+      GS_DEF2("_CAPI_GetCSR", "_CAPI_get_csr", &Graph::GetCSRTensor)
       GS_DEF2("_CAPI_GetBatchCSC", "GetBatchCSC", &Graph::GetBatchCSC)
       GS_DEF2("_CAPI_GetCOO", "_CAPI_get_coo", &Graph::GetCOOTensor)
       GS_DEF2("_CAPI_SetCOO", "_CAPI_set_coo", &Graph::SetCOOByTensor)
       GS_DEF2("_CAPI_SetMetadata", "_CAPI_set_metadata", &Graph::SetMetaData)
       GS_DEF2("_CAPI_CSC2CSR", "_CAPI_csc2csr", &Graph::CSC2CSR)
       GS_DEF2("_CAPI_CSR2CSC", "_CAPI_csr2csc", &Graph::CSR2CSC)
+      GS_DEF2("_CAPI_CSC2DCSR", "_CAPI_csc2dcsr", &Graph::CSC2DCSR)
+      GS_DEF2("_CAPI_CSR2DCSC", "_CAPI_csr2dcsc", &Graph::CSR2DCSC)
+      GS_DEF2("_CAPI_SetValidCols", "_CAPI_set_valid_cols", &Graph::SetValidCols)
+      GS_DEF2("_CAPI_SetValidRows", "_CAPI_set_valid_rows", &Graph::SetValidRows)
       GS_DEF2("_CAPI_CreateSparseFormat", "_CAPI_create_sparse_format", &Graph::CreateSparseFormat);
 
   m.class_<HeteroGraph>("HeteroGraph")

@@ -9,15 +9,9 @@ namespace gs {
 
 namespace {
 
-const char* kNoDoublyCompressed =
-    "doubly-compressed formats (_DCSC / _DCSR) are not part of this build";
-
-bool IsCscLike(int64_t format) { return format == _CSC; }
-bool IsCsrLike(int64_t format) { return format == _CSR; }
-
-void RejectCompressed(int64_t format) {
-  TORCH_CHECK(format != _DCSC && format != _DCSR, kNoDoublyCompressed);
-}
+// _DCSC / _DCSR are the CSC / CSR with only the non-empty columns / rows stored
+bool IsCscLike(int64_t format) { return format == _CSC || format == _DCSC; }
+bool IsCsrLike(int64_t format) { return format == _CSR || format == _DCSR; }
 
 torch::Tensor Pick(const torch::optional<torch::Tensor>& ids, const torch::Tensor& local) {
   return ids.has_value() ? ids.value().index({local}) : local;
@@ -90,10 +84,10 @@ torch::optional<torch::Tensor> Graph::GetData(std::string order) {
   Settle();
   torch::Tensor data = DataOrOnes();
   if (order == "col") {
-    CreateSparseFormat(_CSC);
+    if (!csc_) CreateSparseFormat(_CSC);  // a doubly-compressed CSC orders the edges alike
     if (csc_->e_ids.has_value()) return data.index({csc_->e_ids.value()});
   } else if (order == "row") {
-    CreateSparseFormat(_CSR);
+    if (!csr_) CreateSparseFormat(_CSR);
     if (csr_->e_ids.has_value()) return data.index({csr_->e_ids.value()});
   }
   return data;
@@ -102,27 +96,64 @@ torch::optional<torch::Tensor> Graph::GetData(std::string order) {
 // ------------------------------------------------------------ format caches
 void Graph::CSC2CSR() {
   Settle();
-  SetCOO(GraphCSC2COO(csc_, true));
+  CreateSparseFormat(_COO);
   SetCSR(GraphCOO2CSC(coo_, num_rows_, false));
 }
 
 void Graph::CSR2CSC() {
   Settle();
-  SetCOO(GraphCSC2COO(csr_, false));
+  CreateSparseFormat(_COO);
   SetCSC(GraphCOO2CSC(coo_, num_cols_, true));
 }
 
+void Graph::CSC2DCSR() {
+  Settle();
+  CreateSparseFormat(_COO);
+  std::shared_ptr<CSR> csr;
+  torch::Tensor val;
+  std::tie(csr, val) = GraphCOO2DCSC(coo_, num_rows_, false);
+  val_row_ids_ = val;
+  SetCSR(csr);
+}
+
+void Graph::CSR2DCSC() {
+  Settle();
+  CreateSparseFormat(_COO);
+  std::shared_ptr<CSC> csc;
+  torch::Tensor val;
+  std::tie(csc, val) = GraphCOO2DCSC(coo_, num_cols_, true);
+  val_col_ids_ = val;
+  SetCSC(csc);
+}
+
+// reference src/graph.cc:585-644
 void Graph::CreateSparseFormat(int64_t format) {
   Settle();
-  RejectCompressed(format);
   if (format == _COO) {
     if (coo_) return;
     if (csc_)
-      SetCOO(GraphCSC2COO(csc_, true));
+      SetCOO(val_col_ids_.has_value() ? GraphDCSC2COO(csc_, val_col_ids_.value(), true)
+                                      : GraphCSC2COO(csc_, true));
     else
-      SetCOO(GraphCSC2COO(csr_, false));
+      SetCOO(val_row_ids_.has_value() ? GraphDCSC2COO(csr_, val_row_ids_.value(), false)
+                                      : GraphCSC2COO(csr_, false));
+  } else if (format == _DCSC) {
+    if (csc_) {
+      TORCH_CHECK(val_col_ids_.has_value(), "Require DCSC, get CSC instead");
+      return;
+    }
+    CSR2DCSC();
+  } else if (format == _DCSR) {
+    if (csr_) {
+      TORCH_CHECK(val_row_ids_.has_value(), "Require DCSR, get CSR instead");
+      return;
+    }
+    CSC2DCSR();
   } else if (format == _CSC) {
-    if (csc_) return;
+    if (csc_) {
+      TORCH_CHECK(!val_col_ids_.has_value(), "Require CSC, get DCSC instead");
+      return;
+    }
     if (spare_csc_)
       SetCSC(std::move(spare_csc_));
     else if (coo_)
@@ -130,7 +161,10 @@ void Graph::CreateSparseFormat(int64_t format) {
     else
       CSR2CSC();
   } else if (format == _CSR) {
-    if (csr_) return;
+    if (csr_) {
+      TORCH_CHECK(!val_row_ids_.has_value(), "Require CSR, get DCSR instead");
+      return;
+    }
     if (spare_csr_)
       SetCSR(std::move(spare_csr_));
     else if (coo_)
@@ -144,7 +178,7 @@ void Graph::CreateSparseFormat(int64_t format) {
 
 std::vector<torch::Tensor> Graph::GetCSCTensor() {
   Settle();
-  CreateSparseFormat(_CSC);
+  if (!csc_) CreateSparseFormat(_CSC);
   return {csc_->indptr, csc_->indices, csc_->e_ids.value_or(torch::Tensor())};
 }
 
@@ -153,6 +187,12 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> Graph::GetBatchCSC(
   Settle();
   CreateSparseFormat(_CSC);
   return {csc_->indptr, csc_->indices, csc_->indptr.index({seeds_ptr})};
+}
+
+std::vector<torch::Tensor> Graph::GetCSRTensor() {
+  Settle();
+  if (!csr_) CreateSparseFormat(_CSR);
+  return {csr_->indptr, csr_->indices, csr_->e_ids.value_or(torch::Tensor())};
 }
 
 std::vector<torch::Tensor> Graph::GetCOOTensor() {
@@ -186,6 +226,8 @@ c10::intrusive_ptr<Graph> Graph::SameShape(torch::Tensor data) {
   g->SetCOO(coo_);
   g->SetNumEdges(num_edges_);
   g->SetData(data);
+  g->val_col_ids_ = val_col_ids_;
+  g->val_row_ids_ = val_row_ids_;
   return g;
 }
 
@@ -194,9 +236,9 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
                                          int64_t output_format, bool relabel) {
   Settle();
   TORCH_CHECK(axis == 0 || axis == 1, "axis must be 0 (columns) or 1 (rows)");
-  RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   const bool with_coo = output_format & _COO;
+  torch::optional<torch::Tensor> new_val_cols, new_val_rows;
 
   torch::optional<torch::Tensor> col_ids = col_ids_, row_ids = row_ids_;
   int64_t num_cols = num_cols_, num_rows = num_rows_;
@@ -228,10 +270,17 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
                 "Error in Slicing, Not implementation [on_format = ", on_csc ? "CSC" : "CSR",
                 ", output_format = ", on_csc ? "CSR" : "CSC", "]");
     std::shared_ptr<CSC> fmt = on_csc ? csc_ : csr_;
+    const torch::optional<torch::Tensor>& stored = on_csc ? val_col_ids_ : val_row_ids_;
     const bool along = (axis == 0) == on_csc;
     std::shared_ptr<_TMP> tmp;
     if (along) {
-      std::tie(tmp, select_index) = CSCColSlicing(fmt, n_ids, with_coo, data_.has_value());
+      // the result has one (possibly empty) column per requested id, so it is never
+      // doubly compressed, whatever the input was (reference src/graph.cc:213-217)
+      if (stored.has_value())
+        std::tie(tmp, select_index) =
+            DCSCColSlicing(fmt, stored.value(), n_ids, with_coo, data_.has_value());
+      else
+        std::tie(tmp, select_index) = CSCColSlicing(fmt, n_ids, with_coo, data_.has_value());
       if (relabel) {
         // the other side is renumbered by first occurrence (reference src/graph.cc:219-227)
         torch::Tensor frontier;
@@ -250,8 +299,12 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
     } else {
       TORCH_CHECK(!relabel, "Not implemented warning");
       std::tie(tmp, select_index) = CSCRowSlicing(fmt, n_ids, with_coo);
+      // the stored columns stay the same ones (reference src/graph.cc:231,254)
+      (on_csc ? new_val_cols : new_val_rows) = stored;
+      if (with_coo && stored.has_value())
+        tmp->coo_in_indptr = stored.value().index({tmp->coo_in_indptr});
     }
-    if (output_format & (on_csc ? _CSC : _CSR)) {
+    if (output_format & (on_csc ? (_CSC | _DCSC) : (_CSR | _DCSR))) {
       auto compressed =
           std::make_shared<CSC>(CSC{tmp->indptr, tmp->coo_in_indices, torch::nullopt});
       (on_csc ? out_csc : out_csr) = compressed;
@@ -279,6 +332,8 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
   ret->SetCSR(out_csr);
   ret->spare_csc_ = spare_csc;
   ret->spare_csr_ = spare_csr;
+  if (out_csc) ret->val_col_ids_ = new_val_cols;
+  if (out_csr) ret->val_row_ids_ = new_val_rows;
   InheritData(ret.get(), e_ids, select_index);
   return ret;
 }
@@ -288,7 +343,6 @@ c10::intrusive_ptr<Graph> Graph::SampleImpl(int64_t axis, const torch::Tensor* e
                                             int64_t fanout, bool replace, int64_t on_format,
                                             int64_t output_format) {
   Settle();
-  RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   const bool on_csc = (axis == 0 && on_format == _CSC);
   const bool on_csr = (axis == 1 && on_format == _CSR);
@@ -504,7 +558,6 @@ torch::Tensor Graph::RandomWalk(torch::Tensor seeds, int64_t walk_length) {
 // --------------------------------------------------------- edge-data operators
 torch::Tensor Graph::Sum(int64_t axis, int64_t powk, int64_t on_format) {
   Settle();
-  RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
   // one entry per column (axis 0) / row (axis 1) OF THIS GRAPH OBJECT, so a
@@ -512,10 +565,10 @@ torch::Tensor Graph::Sum(int64_t axis, int64_t powk, int64_t on_format) {
   torch::Tensor out = torch::zeros({axis == 0 ? num_cols_ : num_rows_}, data.options());
   if (on_format == _COO)
     COOGraphSum(coo_, data, out, powk, 1 - axis);
-  else if (axis == 0 && on_format == _CSC)
-    CSCGraphSum(csc_, torch::nullopt, data, out, powk);
-  else if (axis == 1 && on_format == _CSR)
-    CSCGraphSum(csr_, torch::nullopt, data, out, powk);
+  else if (axis == 0 && IsCscLike(on_format))
+    CSCGraphSum(csc_, val_col_ids_, data, out, powk);
+  else if (axis == 1 && IsCsrLike(on_format))
+    CSCGraphSum(csr_, val_row_ids_, data, out, powk);
   else
     TORCH_CHECK(false, "axis should be 0 or 1? on_format and axis do not match?");
   return out;
@@ -523,13 +576,12 @@ torch::Tensor Graph::Sum(int64_t axis, int64_t powk, int64_t on_format) {
 
 c10::intrusive_ptr<Graph> Graph::Normalize(int64_t axis, int64_t on_format) {
   Settle();
-  RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
   torch::Tensor out = torch::empty_like(data);
-  if (axis == 0 && on_format == _CSC)
+  if (axis == 0 && IsCscLike(on_format))
     hip::SegmentNormalize(csc_->indptr, csc_->e_ids, data, out);
-  else if (axis == 1 && on_format == _CSR)
+  else if (axis == 1 && IsCsrLike(on_format))
     hip::SegmentNormalize(csr_->indptr, csr_->e_ids, data, out);
   else
     TORCH_CHECK(false, "Not Implementation Error");
@@ -538,16 +590,15 @@ c10::intrusive_ptr<Graph> Graph::Normalize(int64_t axis, int64_t on_format) {
 
 c10::intrusive_ptr<Graph> Graph::Divide(torch::Tensor divisor, int64_t axis, int64_t on_format) {
   Settle();
-  RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
   torch::Tensor out = torch::zeros({num_edges_}, data.options());
   if (on_format == _COO)
     COOGraphDiv(coo_, data, divisor, out, 1 - axis);
-  else if (axis == 0 && on_format == _CSC)
-    CSCGraphDiv(csc_, torch::nullopt, data, divisor, out);
-  else if (axis == 1 && on_format == _CSR)
-    CSCGraphDiv(csr_, torch::nullopt, data, divisor, out);
+  else if (axis == 0 && IsCscLike(on_format))
+    CSCGraphDiv(csc_, val_col_ids_, data, divisor, out);
+  else if (axis == 1 && IsCsrLike(on_format))
+    CSCGraphDiv(csr_, val_row_ids_, data, divisor, out);
   return SameShape(out);
 }
 
@@ -566,18 +617,18 @@ std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> Graph::EDivUSum(torch::Tens
 void Graph::SDDMM(const std::string& op, torch::Tensor lhs, torch::Tensor rhs, torch::Tensor out,
                   int64_t lhs_target, int64_t rhs_target, int64_t on_format) {
   Settle();
-  RejectCompressed(on_format);
   CreateSparseFormat(on_format);
   const hip::Bcast b = ToDevice(CalcBcastOff(op, lhs, rhs), out);
   if (on_format == _COO) {
     hip::SddmmCoo(op, b, coo_->row, coo_->col, coo_->e_ids, lhs, rhs, out,
                   static_cast<int>(lhs_target), static_cast<int>(rhs_target));
-  } else if (on_format == _CSR) {
+  } else if (IsCsrLike(on_format)) {
     const int lt = lhs_target == 1 ? 1 : static_cast<int>(2 - lhs_target);
     const int rt = rhs_target == 1 ? 1 : static_cast<int>(2 - rhs_target);
-    hip::SddmmCsc(op, b, csr_->indptr, csr_->indices, csr_->e_ids, torch::nullopt, lhs, rhs, out, lt, rt);
-  } else if (on_format == _CSC) {
-    hip::SddmmCsc(op, b, csc_->indptr, csc_->indices, csc_->e_ids, torch::nullopt, lhs, rhs, out,
+    hip::SddmmCsc(op, b, csr_->indptr, csr_->indices, csr_->e_ids, val_row_ids_, lhs, rhs, out, lt,
+                  rt);
+  } else if (IsCscLike(on_format)) {
+    hip::SddmmCsc(op, b, csc_->indptr, csc_->indices, csc_->e_ids, val_col_ids_, lhs, rhs, out,
                   static_cast<int>(lhs_target), static_cast<int>(rhs_target));
   } else {
     TORCH_CHECK(false, "SDDMM only supports CSR and COO formats");
@@ -594,7 +645,7 @@ torch::Tensor Graph::AllValidNode() {
   } else if (csc_) {
     rows = csc_->indices;
   } else {
-    if (!coo_) SetCOO(GraphCSC2COO(csr_, false));
+    CreateSparseFormat(_COO);
     rows = coo_->row;
   }
   return hip::Unique(torch::cat({col_ids_.value(), rows}));
@@ -624,14 +675,16 @@ Graph::Relabel() {
   }
   Settle();
   if (csc_) {
-    // seeds first: the frontier starts with the column ids (reference src/graph.cc:789-811)
+    // seeds first: the frontier starts with the column ids (reference src/graph.cc:789-811);
+    // of a doubly-compressed CSC only the stored columns count (:790-791)
+    if (val_col_ids_.has_value()) col_ids = col_ids.index({val_col_ids_.value()});
     torch::Tensor rows = Pick(row_ids_, csc_->indices);
     std::tie(frontier, renamed) = BatchTensorRelabel({col_ids, rows}, {rows});
     return {frontier, frontier.numel(), col_ids.numel(), csc_->indptr.clone(), renamed[0],
             csc_->e_ids, "csc"};
   }
   TORCH_CHECK(csr_ || coo_, "Error in Relabel!");
-  if (!coo_) SetCOO(GraphCSC2COO(csr_, false));
+  CreateSparseFormat(_COO);
   torch::Tensor coo_col = col_ids.index({coo_->col});
   torch::Tensor coo_row = Pick(row_ids_, coo_->row);
   std::tie(frontier, renamed) = BatchTensorRelabel({col_ids, coo_row}, {coo_col, coo_row});
@@ -648,12 +701,14 @@ torch::Tensor Graph::GetCols() {
 
 torch::Tensor Graph::GetValidRows() {
   Settle();
-  return Pick(row_ids_, std::get<0>(torch::_unique(GetCOORows(false))));
+  return Pick(row_ids_, val_row_ids_.has_value() ? val_row_ids_.value()
+                                                 : std::get<0>(torch::_unique(GetCOORows(false))));
 }
 
 torch::Tensor Graph::GetValidCols() {
   Settle();
-  return Pick(col_ids_, std::get<0>(torch::_unique(GetCOOCols(false))));
+  return Pick(col_ids_, val_col_ids_.has_value() ? val_col_ids_.value()
+                                                 : std::get<0>(torch::_unique(GetCOOCols(false))));
 }
 
 torch::Tensor Graph::GetCOORows(bool is_original) {
@@ -665,7 +720,7 @@ torch::Tensor Graph::GetCOORows(bool is_original) {
     rows = csc_->indices;
   } else {
     TORCH_CHECK(csr_ && !csr_->e_ids.has_value(), "Error in GetCOORows!");
-    SetCOO(GraphCSC2COO(csr_, false));
+    CreateSparseFormat(_COO);
     rows = coo_->row;
   }
   return is_original ? Pick(row_ids_, rows) : rows;
@@ -677,7 +732,7 @@ torch::Tensor Graph::GetCOOCols(bool is_original) {
   if (coo_) {
     cols = coo_->col;
   } else if (csc_ && !csc_->e_ids.has_value()) {
-    SetCOO(GraphCSC2COO(csc_, true));
+    CreateSparseFormat(_COO);
     cols = coo_->col;
   } else {
     TORCH_CHECK(csr_ && !csr_->e_ids.has_value(), "Error in GetCOOCols!");

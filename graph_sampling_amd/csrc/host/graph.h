@@ -61,6 +61,9 @@ class Graph : public torch::CustomClassHolder {
   void SetCOOByTensor(torch::Tensor row, torch::Tensor col, torch::optional<torch::Tensor> e_ids,
                       bool row_sorted, bool col_sorted);
   void SetData(torch::Tensor data) { data_ = data; }
+  // ids of the stored columns / rows when the CSC / CSR is doubly compressed
+  void SetValidCols(torch::Tensor val_cols) { val_col_ids_ = val_cols; }
+  void SetValidRows(torch::Tensor val_rows) { val_row_ids_ = val_rows; }
   void SetNumEdges(int64_t num_edges) {
     Settle();
     num_edges_ = num_edges;
@@ -79,6 +82,9 @@ class Graph : public torch::CustomClassHolder {
   }
   std::vector<torch::Tensor> GetCSCTensor();
   std::vector<torch::Tensor> GetCOOTensor();
+  // (indptr, indices, e_ids) of the row-compressed format as it is held (CSR or DCSR);
+  // made from the others as a CSR when the graph has none
+  std::vector<torch::Tensor> GetCSRTensor();
   // (indptr, indices, indices_ptr): the CSC of a super-batch whose columns are cut into
   // batches at seeds_ptr, with the matching cut of the edges (examples/graphsage/batching.py:68)
   std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> GetBatchCSC(torch::Tensor seeds_ptr);
@@ -93,6 +99,8 @@ class Graph : public torch::CustomClassHolder {
   // ---- format caches
   void CSC2CSR();
   void CSR2CSC();
+  void CSC2DCSR();
+  void CSR2DCSC();
   void CreateSparseFormat(int64_t format);
 
   // ---- structure operators (axis 0: columns, axis 1: rows)
@@ -187,6 +195,10 @@ class Graph : public torch::CustomClassHolder {
   torch::optional<torch::Tensor> data_;
   torch::optional<torch::Tensor> col_ids_;  // global id of each local column
   torch::optional<torch::Tensor> row_ids_;  // global id of each local row
+  // set when csc_ / csr_ is doubly compressed: stored column (row) i is local column
+  // (row) val_col_ids_[i]; columns (rows) without edges are not stored
+  torch::optional<torch::Tensor> val_col_ids_;
+  torch::optional<torch::Tensor> val_row_ids_;
 };
 
 }  // namespace gs

@@ -150,6 +150,39 @@ std::shared_ptr<CSC> GraphCOO2CSC(std::shared_ptr<COO> coo, int64_t num_items, b
   return csc;
 }
 
+// sort by the compressed side, then keep only the offsets of the non-empty columns
+std::pair<std::shared_ptr<CSC>, torch::Tensor> GraphCOO2DCSC(std::shared_ptr<COO> coo,
+                                                             int64_t num_items, bool COO2DCSC) {
+  std::shared_ptr<CSC> full = GraphCOO2CSC(coo, num_items, COO2DCSC);
+  torch::Tensor val_ids;
+  std::tie(full->indptr, val_ids) = hip::CscCompress(full->indptr, full->indices);
+  return {full, val_ids};
+}
+
+std::shared_ptr<COO> GraphDCSC2COO(std::shared_ptr<CSC> csc, torch::Tensor ids, bool DCSC2COO) {
+  auto coo = std::make_shared<COO>();
+  torch::Tensor expanded = hip::Dcsc2CooCols(csc->indptr, csc->indices.numel(), ids);
+  if (DCSC2COO) {
+    coo->row = csc->indices;
+    coo->col = expanded;
+    coo->col_sorted = true;
+  } else {
+    coo->row = expanded;
+    coo->col = csc->indices;
+    coo->row_sorted = true;
+  }
+  coo->e_ids = csc->e_ids;
+  return coo;
+}
+
+std::pair<std::shared_ptr<_TMP>, torch::Tensor> DCSCColSlicing(std::shared_ptr<CSC> csc,
+                                                               torch::Tensor nid_map,
+                                                               torch::Tensor node_ids,
+                                                               bool with_coo, bool with_select) {
+  return Wrap(hip::DcscColSlicing(csc->indptr, csc->indices, nid_map, node_ids, with_coo,
+                                  with_select));
+}
+
 torch::Tensor FusedRandomWalk(std::shared_ptr<CSC> csc, torch::Tensor seeds, int64_t walk_length) {
   // flat [walk_length+1][n] buffer handed out with shape [n, walk_length+1]
   // (reference src/cuda/fusion/random_walk.cu:67)

@@ -68,6 +68,16 @@ std::shared_ptr<COO> GraphCSC2COO(std::shared_ptr<CSC> csc, bool CSC2COO);
 
 std::shared_ptr<CSC> GraphCOO2CSC(std::shared_ptr<COO> coo, int64_t num_items, bool COO2CSC);
 
+// doubly-compressed counterparts (reference src/graph_ops.cc:62-104,156-171)
+std::pair<std::shared_ptr<CSC>, torch::Tensor> GraphCOO2DCSC(std::shared_ptr<COO> coo,
+                                                             int64_t num_items, bool COO2DCSC);
+std::shared_ptr<COO> GraphDCSC2COO(std::shared_ptr<CSC> csc, torch::Tensor ids, bool DCSC2COO);
+std::pair<std::shared_ptr<_TMP>, torch::Tensor> DCSCColSlicing(std::shared_ptr<CSC> csc,
+                                                               torch::Tensor nid_map,
+                                                               torch::Tensor node_ids,
+                                                               bool with_coo,
+                                                               bool with_select = true);
+
 torch::Tensor FusedRandomWalk(std::shared_ptr<CSC> csc, torch::Tensor seeds, int64_t walk_length);
 
 }  // namespace gs

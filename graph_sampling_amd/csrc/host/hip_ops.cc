@@ -685,6 +685,42 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ColRowSli
   return {out_indptr, out_indices, select_index, parent_index};
 }
 
+SliceResult DcscColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
+                           const torch::Tensor& nid_map, const torch::Tensor& column_ids,
+                           bool with_coo, bool with_select) {
+  // position of every requested column among the stored ones; -1 (not stored) is outside
+  // [0, num_cols) and therefore an empty column for the slice kernels
+  return ColSlicing(indptr, indices, IndexSearch(nid_map, column_ids), with_coo, with_select);
+}
+
+torch::Tensor Dcsc2CooCols(const torch::Tensor& indptr, int64_t nnz, const torch::Tensor& ids) {
+  NeedI64(indptr, "indptr");
+  const int idb = IdBytes(ids, "valid ids");
+  TORCH_CHECK(ids.numel() == indptr.numel() - 1, "one id per stored column expected");
+  auto col = torch::empty({nnz}, ids.options());
+  Check(gs_dcsc2coo(indptr.data_ptr<int64_t>(), indptr.numel() - 1, nnz, ids.data_ptr(),
+                    col.data_ptr(), idb, Stream(indptr)),
+        "gs_dcsc2coo");
+  return col;
+}
+
+std::tuple<torch::Tensor, torch::Tensor> CscCompress(const torch::Tensor& indptr,
+                                                     const torch::Tensor& ids_like) {
+  NeedI64(indptr, "indptr");
+  const int idb = IdBytes(ids_like, "indices");
+  const int64_t n = indptr.numel() - 1;
+  auto val_ids = torch::empty({n}, ids_like.options());
+  auto out_indptr = torch::empty({n + 1}, I64(indptr));
+  auto num = torch::empty({1}, I64(indptr));
+  auto ws = Scratch(gs_csc_compress_workspace_bytes(n), indptr);
+  Check(gs_csc_compress(indptr.data_ptr<int64_t>(), n, idb, val_ids.data_ptr(),
+                        out_indptr.data_ptr<int64_t>(), num.data_ptr<int64_t>(), ws.data_ptr(),
+                        ws.numel(), Stream(indptr)),
+        "gs_csc_compress");
+  const int64_t kept = num.item<int64_t>();
+  return {out_indptr.narrow(0, 0, kept + 1), val_ids.narrow(0, 0, kept)};
+}
+
 torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz, const torch::Tensor& ids_like) {
   NeedI64(indptr, "indptr");
   const int idb = IdBytes(ids_like, "indices");

@@ -127,6 +127,17 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ColRowSli
     const torch::Tensor& row_ids, const torch::optional<torch::Tensor>& col_ptr = torch::nullopt,
     const torch::optional<torch::Tensor>& row_ptr = torch::nullopt, int64_t encoding_size = 0);
 
+// ---- doubly-compressed formats (only the non-empty columns are stored; ids name them)
+// column slice of a DCSC: a requested column that is not stored is an empty column
+SliceResult DcscColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
+                           const torch::Tensor& nid_map, const torch::Tensor& column_ids,
+                           bool with_coo, bool with_select = true);
+// col[e] = ids[stored column owning e]
+torch::Tensor Dcsc2CooCols(const torch::Tensor& indptr, int64_t nnz, const torch::Tensor& ids);
+// {offsets of the non-empty columns, their ids}
+std::tuple<torch::Tensor, torch::Tensor> CscCompress(const torch::Tensor& indptr,
+                                                     const torch::Tensor& ids_like);
+
 // col[e] = column owning edge e, in the dtype of `ids_like`
 torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz, const torch::Tensor& ids_like);
 // {indptr, values in key order, sort permutation (nullopt when already sorted)}

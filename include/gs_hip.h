@@ -448,6 +448,19 @@ int gs_index_search(const void* data, int64_t n, const void* keys, int64_t m, in
 int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, void* col, int id_bytes,
                void* stream);
 
+/* Doubly-compressed CSC (only the columns that own an edge are stored; ids[c] names stored
+ * column c).  gs_dcsc2coo: col[e] = ids[column owning e], replaces impl::DCSC2COOCUDA
+ * (src/cuda/format_transform.cu:48).  gs_csc_compress: CSC -> DCSC, the second half of
+ * impl::COO2DCSCCUDA (src/cuda/format_transform.cu:172-203; the first half, the sort, is
+ * gs_coo2csc): val_ids (capacity num_cols) = the non-empty columns in order, out_indptr
+ * (capacity num_cols + 1) = their offsets, *num_valid (device scalar) = how many. */
+int gs_dcsc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, const void* ids, void* col,
+                int id_bytes, void* stream);
+size_t gs_csc_compress_workspace_bytes(int64_t num_cols);
+int gs_csc_compress(const int64_t* indptr, int64_t num_cols, int id_bytes, void* val_ids,
+                    int64_t* out_indptr, int64_t* num_valid, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
 size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys);
 
 /* Stable counting sort of (key -> value), both id_bytes wide: indptr[num_keys+1],

@@ -76,11 +76,111 @@ def test_slicing_relabel_test1(dev):
     assert p.equal(torch.arange(0, 4, **I(dev)) * 5) and i.equal(torch.arange(0, 15, **I(dev)))
 
 
-def test_doubly_compressed_formats_are_rejected(dev):
-    # SlicingRelabel.test2 / RowwiseSlicing.test2 / CSC2DCSR.test1 use _DCSR, which this build omits
-    A, _, _ = graph12(dev)
-    with pytest.raises(RuntimeError, match="doubly-compressed"):
-        A._CAPI_Slicing(torch.arange(5, 6, **I(dev)), 1, _DCSR, _CSR, False)
+def _graph12_rows(dev, lo, hi):
+    A = gs.Graph(False)
+    indptr = torch.cat([torch.zeros(10, **I(dev)), torch.arange(0, 3, **I(dev)) * 2])
+    A._CAPI_LoadCSC(indptr, torch.arange(lo, hi, **I(dev)).repeat(2))
+    return A
+
+
+def test_slicing_relabel_test2_dcsr(dev):
+    # tests/test_relabel.cc:28-52
+    A = _graph12_rows(dev, 5, 7)
+    A._CAPI_CSC2DCSR()
+    sub = A._CAPI_Slicing(torch.arange(5, 6, **I(dev)), 1, _DCSR, _CSR, True)
+    assert (A._CAPI_GetNumCols(), A._CAPI_GetNumRows()) == (12, 12)
+    assert (sub._CAPI_GetNumCols(), sub._CAPI_GetNumRows()) == (2, 1)
+    p, i, _ = sub._CAPI_GetCSR()
+    assert p.numel() == 2 and i.equal(torch.arange(0, 2, **I(dev)))
+    assert sub._CAPI_GetCols().equal(torch.arange(10, 12, **I(dev)))
+
+
+def test_rowwise_slicing_test2_dcsr(dev):
+    # tests/test_rowwise_slicing.cc:22-38
+    A = _graph12_rows(dev, 5, 7)
+    A._CAPI_CSC2DCSR()
+    sub = A._CAPI_Slicing(torch.arange(5, 6, **I(dev)), 1, _DCSR, _CSR, False)
+    p, i, _ = sub._CAPI_GetCSR()
+    assert p.numel() == 2 and i.equal(torch.arange(10, 12, **I(dev)))
+    # a row that is not stored comes back as an empty row
+    sub = A._CAPI_Slicing(torch.tensor([0, 6, 11], **I(dev)), 1, _DCSR, _CSR, False)
+    p, i, _ = sub._CAPI_GetCSR()
+    assert p.tolist() == [0, 0, 2, 2] and i.equal(torch.arange(10, 12, **I(dev)))
+
+
+def test_csc2dcsr_test1(dev):
+    # tests/test_format_transform.cc:100-116
+    A = gs.Graph(False)
+    indptr = torch.cat([torch.zeros(10, **I(dev)), torch.arange(0, 3, **I(dev)) * 2])
+    A._CAPI_LoadCSC(indptr, torch.arange(1, 4, 2, **I(dev)).repeat(2))
+    A._CAPI_CSC2DCSR()
+    p, i, _ = A._CAPI_GetCSR()
+    assert p.numel() == 3 and p.tolist() == [0, 2, 4]
+    assert i.equal(torch.arange(10, 12, **I(dev)).repeat(2))
+    assert A._CAPI_GetValidRows().equal(torch.arange(1, 4, 2, **I(dev)))
+    with pytest.raises(RuntimeError, match="Require CSR, get DCSR instead"):
+        A._CAPI_CreateSparseFormat(_CSR)
+
+
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+def test_doubly_compressed_round_trip_and_edge_ops(dev, idt):
+    """DCSC built from a COO with many empty columns: conversion back, column slice, sums,
+    divide and SDDMM agree with the same graph held as a plain CSC."""
+    from oracle import oracle as O
+    from tests.util import to_dev
+    rng = np.random.default_rng(0)
+    n, E = 5000, 3000
+    row = rng.integers(0, n, size=E).astype(np.int64)
+    col = rng.integers(0, 40, size=E).astype(np.int64) * 100      # 40 columns own all edges
+    w = rng.random(E).astype(np.float32)
+
+    def make():
+        g = gs.Graph(False)
+        g._CAPI_LoadCOO(to_dev(row, dev, idt), to_dev(col, dev, idt))
+        g._CAPI_SetMetadata(None, None, n, n)
+        g._CAPI_SetData(to_dev(w, dev))
+        return g
+
+    d, c = make(), make()
+    d._CAPI_CreateSparseFormat(8)      # _DCSC
+    c._CAPI_CreateSparseFormat(_CSC)
+    dp, di, _ = d._CAPI_GetCSC()
+    w_ptr, w_val, w_perm = O.coo2csc(col, row, n, False)
+    stored = np.flatnonzero(np.diff(w_ptr))
+    assert np.array_equal(dp.cpu().numpy(), np.concatenate([w_ptr[stored], [E]]))
+    assert np.array_equal(di.cpu().numpy(), w_val)
+    assert np.array_equal(d._CAPI_GetValidCols().cpu().numpy(), stored)
+    # sums over columns land at the stored columns' ids
+    assert torch.equal(d._CAPI_Sum(0, 2, 8), c._CAPI_Sum(0, 2, _CSC))
+    div = torch.rand(n, device=dev) + 0.5
+    assert torch.equal(d._CAPI_Divide(div, 0, 8)._CAPI_GetData("col"),
+                       c._CAPI_Divide(div, 0, _CSC)._CAPI_GetData("col"))
+    # column slice: stored, not stored and repeated columns
+    ids = to_dev(np.array([100, 101, 3900, 100, 4999, 0]), dev, idt)
+    sd = d._CAPI_Slicing(ids, 0, 8, _CSC + _COO, False)
+    sc = c._CAPI_Slicing(ids, 0, _CSC, _CSC + _COO, False)
+    for a, b in zip(sd._CAPI_GetCSC()[:2], sc._CAPI_GetCSC()[:2]):
+        assert torch.equal(a, b)
+    assert torch.equal(sd._CAPI_GetData("default"), sc._CAPI_GetData("default"))
+    # SDDMM u_add_v on the compressed format uses the stored columns' ids for the v side
+    lhs, rhs = torch.rand(n, 1, device=dev), torch.rand(n, 1, device=dev)
+    out_d, out_c = torch.zeros(E, 1, device=dev), torch.zeros(E, 1, device=dev)
+    d._CAPI_SDDMM("add", lhs, rhs, out_d, 0, 2, 8)
+    c._CAPI_SDDMM("add", lhs, rhs, out_c, 0, 2, _CSC)
+    assert torch.equal(out_d, out_c)
+    # back to COO: the stored columns' ids, not their positions
+    e = gs.Graph(False)
+    e._CAPI_LoadCOO(to_dev(row, dev, idt), to_dev(col, dev, idt))
+    e._CAPI_SetMetadata(None, None, n, n)
+    e._CAPI_CreateSparseFormat(8)
+    p, i, _ = e._CAPI_GetCSC()
+    f = gs.Graph(False)
+    f._CAPI_LoadCSC(p, i)
+    f._CAPI_SetMetadata(None, None, n, n)
+    f._CAPI_SetValidCols(e._CAPI_GetValidCols())
+    r2, c2 = f._CAPI_GetBatchCOO()
+    assert np.array_equal(c2.cpu().numpy(), np.sort(col, kind="stable"))
+    assert np.array_equal(r2.cpu().numpy(), w_val)
 
 
 # ---------------------------------------------------- test_rowwise_slicing.cc
