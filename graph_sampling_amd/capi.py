@@ -321,6 +321,42 @@ def sample_weighted(indptr, indices, probs, column_ids, fanout, seed=0, replay=N
     return sub_indptr, sub_indices, select_index, coo_col
 
 
+def sample_weighted_replace(indptr, indices, probs, column_ids, fanout, seed=0, replay=None,
+                            with_coo=False):
+    """gs_sample_count(replace=1) + gs_sample_weighted_replace; returns (sub_indptr, sub_indices,
+    select_index, coo_col), the buffers at capacity S * fanout."""
+    _need(indptr, torch.int64, "indptr")
+    _need(probs, torch.float32, "probs")
+    idb = _ids(indices, "indices")
+    dev = indptr.device
+    if column_ids is None:
+        S = indptr.numel() - 1
+        cdf_ptr, cdf_len = indptr, indices.numel()
+    else:
+        _ids(column_ids, "column_ids", like=indices)
+        S = column_ids.numel()
+        cdf_ptr = slice_count(indptr, column_ids)
+        cdf_len = int(cdf_ptr[-1].item())
+    sub_indptr = torch.empty(S + 1, dtype=torch.int64, device=dev)
+    cap = S * int(fanout)
+    sub_indices = torch.empty(cap, dtype=indices.dtype, device=dev)
+    select_index = torch.empty(cap, dtype=torch.int64, device=dev)
+    coo_col = torch.empty(cap, dtype=indices.dtype, device=dev) if with_coo else None
+    cdf = torch.empty(max(cdf_len, 1), dtype=torch.float32, device=dev)
+    ws = workspace(lib().gs_sample_workspace_bytes(_i64(S), _i64(fanout)), dev)
+    st = _stream(dev)
+    _check(lib().gs_sample_count(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(column_ids), idb,
+                                 _i64(S), _i64(fanout), 1, _ptr(sub_indptr), _ptr(ws),
+                                 ctypes.c_size_t(ws.numel()), st), "gs_sample_count")
+    _check(lib().gs_sample_weighted_replace(_ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices),
+                                            _ptr(probs), _ptr(column_ids), idb, _i64(S),
+                                            _i64(fanout), _u64(seed), _ptr(replay), _ptr(sub_indptr),
+                                            _ptr(cdf_ptr), _ptr(cdf), _ptr(sub_indices),
+                                            _ptr(select_index), _ptr(coo_col), st),
+           "gs_sample_weighted_replace")
+    return sub_indptr, sub_indices, select_index, coo_col
+
+
 def list_sample_uniform(data, k, replace, seed=0, replay=None):
     idb = _ids(data, "data")
     dev = data.device

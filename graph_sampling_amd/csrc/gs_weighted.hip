@@ -310,6 +310,87 @@ int weighted_impl(const int64_t* indptr, int64_t num_cols, const void* indices, 
   return coo_col ? weighted_launch<IdT, true>(a, st) : weighted_launch<IdT, false>(a, st);
 }
 
+// ------------------------------------------------ with replacement (inverse CDF) ----
+// Replaces _CSRRowWiseSampleReplaceKernel (reference src/cuda/sampling_probs.cu:112-183).
+// One wave per column: the prefix sums of max(prob, 0) are built 64 edges at a time with a
+// Kogge-Stone scan over the wave (x[i] += x[i-d], d = 1..32; the running total enters the
+// next chunk through its first element, as in the reference's WarpScan loop :147-160) and
+// kept in the caller's scratch; then every lane draws picks and searches them.  The order
+// of the float additions is fixed by that scheme, so a host evaluation of the same steps
+// gives the same bits.
+template <typename IdT, bool WITH_COO>
+__global__ void __launch_bounds__(256)
+weighted_replace_kernel(const int64_t* __restrict__ indptr, int64_t num_cols,
+                        const IdT* __restrict__ indices, const float* __restrict__ probs,
+                        const IdT* __restrict__ cols, int64_t S, int64_t k, uint64_t seed,
+                        const uint32_t* __restrict__ replay, const int64_t* __restrict__ sub_indptr,
+                        const int64_t* __restrict__ cdf_ptr, float* __restrict__ cdf,
+                        IdT* __restrict__ sub_indices, int64_t* __restrict__ select_index,
+                        IdT* __restrict__ coo_col) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (r >= S) return;
+  const int64_t c = cols ? static_cast<int64_t>(cols[r]) : r;
+  if (c < 0 || c >= num_cols) return;
+  const int64_t start = indptr[c];
+  const int64_t deg = indptr[c + 1] - start;
+  if (deg <= 0) return;
+  float* my_cdf = cdf + cdf_ptr[r];
+  float carry = 0.0f;
+  for (int64_t base = 0; base < deg; base += kWave) {
+    float x = base + lane < deg ? probs[start + base + lane] : 0.0f;
+    if (lane == 0) x += carry;
+    x = x > 0.0f ? x : 0.0f;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const float y = __shfl_up(x, d, kWave);
+      if (lane >= d) x += y;
+    }
+    carry = __shfl(x, kWave - 1, kWave);
+    if (base + lane < deg) my_cdf[base + lane] = x;
+  }
+  // the wave's own stores must have landed before other lanes read them back
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+  const float total = carry;
+  const int64_t out_start = sub_indptr[r];
+  for (int64_t j = lane; j < k; j += kWave) {
+    const uint32_t xd = replay ? replay[r * k + j]
+                               : draw_one(seed, kTagWeighted, static_cast<uint64_t>(r),
+                                          static_cast<uint64_t>(j));
+    const float u = static_cast<float>((xd >> 8) + 1u) * 5.9604644775390625e-08f;
+    const float rnd = u * total;
+    int64_t lo = 0, hi = deg;
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (my_cdf[mid] <= rnd) lo = mid + 1; else hi = mid;
+    }
+    if (lo > deg - 1) lo = deg - 1;
+    sub_indices[out_start + j] = indices[start + lo];
+    select_index[out_start + j] = start + lo;
+    if (WITH_COO) coo_col[out_start + j] = static_cast<IdT>(r);
+  }
+}
+
+template <typename IdT>
+int weighted_replace_impl(const int64_t* indptr, int64_t num_cols, const void* indices,
+                          const float* probs, const void* cols, int64_t S, int64_t k, uint64_t seed,
+                          const uint32_t* replay, const int64_t* sub_indptr, const int64_t* cdf_ptr,
+                          float* cdf, void* sub_indices, int64_t* select_index, void* coo_col,
+                          hipStream_t st) {
+  const dim3 grid(static_cast<unsigned>((S + 3) / 4)), block(4 * kWave);
+  if (coo_col)
+    hipLaunchKernelGGL((weighted_replace_kernel<IdT, true>), grid, block, 0, st, indptr, num_cols,
+                       static_cast<const IdT*>(indices), probs, static_cast<const IdT*>(cols), S, k,
+                       seed, replay, sub_indptr, cdf_ptr, cdf, static_cast<IdT*>(sub_indices),
+                       select_index, static_cast<IdT*>(coo_col));
+  else
+    hipLaunchKernelGGL((weighted_replace_kernel<IdT, false>), grid, block, 0, st, indptr, num_cols,
+                       static_cast<const IdT*>(indices), probs, static_cast<const IdT*>(cols), S, k,
+                       seed, replay, sub_indptr, cdf_ptr, cdf, static_cast<IdT*>(sub_indices),
+                       select_index, static_cast<IdT*>(coo_col));
+  return check_launch("sample_weighted_replace");
+}
+
 }  // namespace
 }  // namespace gs
 
@@ -356,6 +437,31 @@ int gs_sample_weighted_fill(const int64_t* indptr, int64_t num_cols, const void*
              : weighted_impl<int32_t>(indptr, num_cols, indices, probs, column_ids, S, fanout, seed, replay,
                                       replay_ptr, sub_indptr, sub_indices, select_index, coo_col,
                                       workspace, workspace_bytes, st);
+}
+
+int gs_sample_weighted_replace(const int64_t* indptr, int64_t num_cols, const void* indices,
+                               const float* probs, const void* column_ids, int id_bytes, int64_t S,
+                               int64_t fanout, uint64_t seed, const uint32_t* replay,
+                               const int64_t* sub_indptr, const int64_t* cdf_ptr, float* cdf,
+                               void* sub_indices, int64_t* select_index, void* coo_col,
+                               void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && cdf_ptr && S >= 0 && fanout >= 0 && num_cols >= 0,
+             "gs_sample_weighted_replace: null pointer or negative size");
+  GS_REQUIRE(column_ids || S <= num_cols,
+             "gs_sample_weighted_replace: S exceeds num_cols without column_ids");
+  GS_REQUIRE(valid_id_bytes(id_bytes),
+             "gs_sample_weighted_replace: id_bytes must be 4 or 8, got %d", id_bytes);
+  if (S == 0 || fanout == 0) return GS_OK;
+  GS_REQUIRE(indices && probs && cdf && sub_indices && select_index,
+             "gs_sample_weighted_replace: null buffer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8
+             ? weighted_replace_impl<int64_t>(indptr, num_cols, indices, probs, column_ids, S,
+                                              fanout, seed, replay, sub_indptr, cdf_ptr, cdf,
+                                              sub_indices, select_index, coo_col, st)
+             : weighted_replace_impl<int32_t>(indptr, num_cols, indices, probs, column_ids, S,
+                                              fanout, seed, replay, sub_indptr, cdf_ptr, cdf,
+                                              sub_indices, select_index, coo_col, st);
 }
 
 }  // extern "C"

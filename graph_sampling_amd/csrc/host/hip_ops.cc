@@ -323,10 +323,37 @@ SliceResult ColSamplingProbs(const torch::Tensor& indptr, const torch::Tensor& i
                              const torch::Tensor& probs, const torch::Tensor& column_ids,
                              int64_t fanout, bool replace, bool with_coo) {
   NeedF32(probs, "edge_probs");
-  TORCH_CHECK(!replace,
-              "weighted sampling with replacement is not built (only the A-Res path without "
-              "replacement is)");
   const int64_t S = column_ids.defined() ? column_ids.numel() : indptr.numel() - 1;
+  if (replace) {
+    // inverse-CDF picks; the prefix sums of every column live in a scratch laid out like
+    // the edges themselves (the offsets of the input, or of the column slice)
+    torch::Tensor cdf_ptr = indptr;
+    int64_t cdf_len = indices.numel();
+    if (column_ids.defined()) {
+      NeedI64(indptr, "indptr");
+      cdf_ptr = torch::empty({S + 1}, I64(indptr));
+      auto sws = Scratch(gs_slice_workspace_bytes(S), indptr);
+      Check(gs_slice_count(indptr.data_ptr<int64_t>(), indptr.numel() - 1, column_ids.data_ptr(),
+                           IdBytes(column_ids, "column ids"), S, cdf_ptr.data_ptr<int64_t>(),
+                           sws.data_ptr(), sws.numel(), Stream(indptr)),
+            "gs_slice_count");
+      cdf_len = cdf_ptr[S].item<int64_t>();
+    }
+    auto cdf = torch::empty({cdf_len > 0 ? cdf_len : 1}, probs.options());
+    return SampleInto(
+        indptr, indices, column_ids, fanout, true, with_coo, 0,
+        [&](const void* cols, int idb, int64_t S_, torch::Tensor& sub_indptr,
+            torch::Tensor& sub_indices, torch::Tensor& select_index, torch::Tensor& coo_col,
+            torch::Tensor&, void* st) {
+          Check(gs_sample_weighted_replace(
+                    indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(),
+                    probs.data_ptr<float>(), cols, idb, S_, fanout, NextSeed(), nullptr,
+                    sub_indptr.data_ptr<int64_t>(), cdf_ptr.data_ptr<int64_t>(),
+                    cdf.data_ptr<float>(), sub_indices.data_ptr(),
+                    select_index.data_ptr<int64_t>(), with_coo ? coo_col.data_ptr() : nullptr, st),
+                "gs_sample_weighted_replace");
+        });
+  }
   return SampleInto(
       indptr, indices, column_ids, fanout, false, with_coo,
       gs_sample_weighted_workspace_bytes(S, fanout),

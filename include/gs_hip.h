@@ -209,6 +209,23 @@ int gs_sample_weighted_fill(const int64_t* indptr, int64_t num_cols, const void*
                             const int64_t* sub_indptr, void* sub_indices, int64_t* select_index,
                             void* coo_col, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Weighted neighbour sampling WITH replacement (inverse CDF): replaces
+ * _CSRRowWiseSampleReplaceKernel (src/cuda/sampling_probs.cu:112-183).  A column with
+ * deg > 0 gets fanout picks.  cdf = inclusive prefix of max(probs, 0) over the column's
+ * edges, built 64 edges at a time by a Kogge-Stone scan (x[i] += x[i-d], d = 1, 2, .., 32)
+ * whose running total enters the next chunk through its first element.  Pick j of row r:
+ * u = ((draw(r, j) >> 8) + 1) * 2^-24, rand = u * cdf[deg-1], item = first position with
+ * cdf > rand, clamped to deg-1.  sub_indptr comes from gs_sample_count(replace = 1).
+ * cdf_ptr[S+1]: offsets of the columns' edges inside the scratch `cdf` (cdf_ptr[S] floats):
+ * indptr itself when column_ids == NULL, else the sub_indptr of gs_slice_count.
+ * replay: S * fanout draws, [r * fanout + j]. */
+int gs_sample_weighted_replace(const int64_t* indptr, int64_t num_cols, const void* indices,
+                               const float* probs, const void* column_ids, int id_bytes, int64_t S,
+                               int64_t fanout, uint64_t seed, const uint32_t* replay,
+                               const int64_t* sub_indptr, const int64_t* cdf_ptr, float* cdf,
+                               void* sub_indices, int64_t* select_index, void* coo_col,
+                               void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* List sampling: replaces impl::ListSamplingCUDA (src/cuda/list_sampling.cu:79) */
 /* and impl::ListSamplingProbsCUDA (src/cuda/list_sampling_probs.cu:185).       */

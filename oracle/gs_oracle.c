@@ -374,6 +374,70 @@ void gso_sample_weighted_fill(const i64* indptr, i64 num_cols, const i64* indice
 }
 
 /* ------------------------------------------------------------------------ */
+/* Weighted column sampling WITH replacement (inverse CDF).                   */
+/* src/cuda/sampling_probs.cu:112-183.  cdf = inclusive prefix of             */
+/* max(prob, 0) over the column's edges.  The reference scans warp-sized      */
+/* chunks with cub::WarpScan and carries the running total into the first     */
+/* element of the next chunk (:147-160); restated here with 64-wide chunks    */
+/* and the scan written out as its Kogge-Stone steps (x[i] += x[i-d] for      */
+/* d = 1, 2, .., 32), so that the float additions happen in one fixed order.  */
+/* Pick j of row r: u = ((draw >> 8) + 1) * 2^-24 in (0, 1], rand = u * total,*/
+/* item = first position with cdf > rand, clamped to deg-1 (:164-171).        */
+/* Replay: replay[r * k + j].  The concrete picks are parity unpinned         */
+/* (no test of the reference calls SamplingProbs).                            */
+/* ------------------------------------------------------------------------ */
+static void cdf_chunks64(const float* prob, i64 deg, float* cdf) {
+  float carry = 0.0f;
+  for (i64 base = 0; base < deg; base += 64) {
+    float x[64], y[64];
+    for (int l = 0; l < 64; ++l) {
+      float v = base + l < deg ? prob[base + l] : 0.0f;
+      if (l == 0) v += carry;
+      x[l] = v > 0.0f ? v : 0.0f;
+    }
+    for (int d = 1; d < 64; d <<= 1) {
+      for (int l = 0; l < 64; ++l) y[l] = l >= d ? x[l] + x[l - d] : x[l];
+      memcpy(x, y, sizeof(x));
+    }
+    carry = x[63];
+    for (int l = 0; l < 64 && base + l < deg; ++l) cdf[base + l] = x[l];
+  }
+}
+
+void gso_sample_weighted_replace(const i64* indptr, i64 num_cols, const i64* indices,
+                                 const float* probs, const i64* cols, i64 S, i64 k, u64 seed,
+                                 const u32* replay, const i64* sub_indptr, i64* sub_indices,
+                                 i64* select_index, i64* coo_col) {
+#pragma omp parallel for schedule(dynamic, 16)
+  for (i64 r = 0; r < S; ++r) {
+    i64 c = col_of(cols, r);
+    if (!col_ok(c, num_cols)) continue;
+    i64 in_start = indptr[c];
+    i64 deg = indptr[c + 1] - in_start;
+    if (deg <= 0) continue;
+    i64 out_start = sub_indptr[r];
+    float* cdf = (float*)malloc(sizeof(float) * (size_t)deg);
+    cdf_chunks64(probs + in_start, deg, cdf);
+    const float total = cdf[deg - 1];
+    for (i64 j = 0; j < k; ++j) {
+      u32 x = replay ? replay[r * k + j] : gso_draw(seed, GSO_TAG_WEIGHTED, (u64)r, (u64)j);
+      float u = (float)((x >> 8) + 1u) * 5.9604644775390625e-08f; /* 2^-24, exact */
+      float rnd = u * total;
+      i64 lo = 0, hi = deg; /* first position with cdf > rnd */
+      while (lo < hi) {
+        i64 mid = (lo + hi) >> 1;
+        if (cdf[mid] <= rnd) lo = mid + 1; else hi = mid;
+      }
+      if (lo > deg - 1) lo = deg - 1;
+      sub_indices[out_start + j] = indices[in_start + lo];
+      select_index[out_start + j] = in_start + lo;
+      if (coo_col) coo_col[out_start + j] = r;
+    }
+    free(cdf);
+  }
+}
+
+/* ------------------------------------------------------------------------ */
 /* List sampling.  src/cuda/list_sampling.cu:20-77 (uniform, Algorithm R over */
 /* positions), src/cuda/list_sampling_probs.cu:11-91 (A-Res, keys sorted      */
 /* descending, first k).  Returns the number of picks written.               */

@@ -209,6 +209,25 @@ def sample_weighted(indptr, indices, probs, cols, k, seed=0, replay=None, with_c
     return sub_indptr, coo_col, sub_indices, select_index
 
 
+def sample_weighted_replace(indptr, indices, probs, cols, k, seed=0, replay=None, with_coo=True):
+    """src/cuda/sampling_probs.cu:112-183 (with replacement, inverse CDF)."""
+    indptr, indices, probs = _i64(indptr), _i64(indices), _f32(probs)
+    cols = None if cols is None else _i64(cols)
+    S = indptr.size - 1 if cols is None else cols.size
+    sub_indptr, _ = sample_count(indptr, cols, k, True)
+    nnz = int(sub_indptr[S])
+    if replay is not None:
+        replay = _u32(replay)
+        assert replay.size >= S * k
+    sub_indices = np.empty(nnz, dtype=np.int64)
+    select_index = np.empty(nnz, dtype=np.int64)
+    coo_col = np.empty(nnz, dtype=np.int64) if with_coo else None
+    lib().gso_sample_weighted_replace(_p(indptr), _c64(indptr.size - 1), _p(indices), _p(probs),
+                                      _p(cols), _c64(S), _c64(k), _cu64(seed), _p(replay),
+                                      _p(sub_indptr), _p(sub_indices), _p(select_index), _p(coo_col))
+    return sub_indptr, coo_col, sub_indices, select_index
+
+
 def list_sample_uniform(data, k, replace, seed=0, replay=None):
     """src/cuda/list_sampling.cu:20-77 -> (select, index)"""
     data = _i64(data)

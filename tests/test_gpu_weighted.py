@@ -172,3 +172,76 @@ def test_weighted_out_of_range_column_ids(dev):
     want = O.sample_weighted(indptr, indices, probs, cols, 4, seed=2)
     for g, w in zip(got, want):
         assert np.array_equal(g, w)
+
+
+# ------------------------------------------------ with replacement (inverse CDF)
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("fanout", [1, 7, 100])
+def test_weighted_replace_matches_oracle(dev, fanout, fused, idt):
+    n = 1 << 11
+    indptr, indices = rmat_csc_np(n, 1 << 16, seed=21)
+    rng = np.random.default_rng(fanout)
+    probs = rng.random(indices.size).astype(np.float32)
+    probs[rng.random(indices.size) < 0.1] = 0.0
+    probs[rng.random(indices.size) < 0.02] = -1.0       # negative weights count as zero
+    cols = rng.integers(0, n, size=300).astype(np.int64) if fused else None
+    S = 300 if fused else n
+    t_cols = None if cols is None else to_dev(cols, dev, idt)
+    for replay in (None, u32_draws(S * fanout, seed=5)):
+        got = capi.sample_weighted_replace(to_dev(indptr, dev), to_dev(indices, dev, idt),
+                                           to_dev(probs, dev), t_cols, fanout, seed=11,
+                                           replay=None if replay is None else to_dev(replay, dev),
+                                           with_coo=True)
+        want = O.sample_weighted_replace(indptr, indices, probs, cols, fanout, seed=11, replay=replay)
+        nnz = int(want[0][-1])
+        assert np.array_equal(got[0].cpu().numpy(), want[0])
+        assert np.array_equal(got[1][:nnz].cpu().numpy().astype(np.int64), want[2])
+        assert np.array_equal(got[2][:nnz].cpu().numpy(), want[3])
+        assert np.array_equal(got[3][:nnz].cpu().numpy().astype(np.int64), want[1])
+    # structure: fanout picks for every non-empty column, each inside the column, never an
+    # edge of weight <= 0 while the column has a positive one
+    c_of = np.arange(n) if cols is None else cols
+    deg = np.diff(indptr)[c_of]
+    assert np.array_equal(np.diff(want[0]), np.where(deg > 0, fanout, 0))
+    sel = want[3]
+    owner = want[1]
+    assert ((sel >= indptr[c_of[owner]]) & (sel < indptr[c_of[owner] + 1])).all()
+    has_pos = np.array([(probs[indptr[c]:indptr[c + 1]] > 0).any() for c in c_of])
+    assert (probs[sel][has_pos[owner]] > 0).all()
+
+
+def test_weighted_replace_hub_column_and_frequencies(dev):
+    # one column of 20000 edges (313 scan chunks): frequencies follow the weights
+    deg, k = 20000, 200000
+    indptr = np.array([0, deg], dtype=np.int64)
+    indices = np.arange(deg, dtype=np.int64)
+    probs = np.ones(deg, dtype=np.float32)
+    probs[:10] = 500.0                      # ten heavy edges share 5000 / 24990 of the mass
+    got = capi.sample_weighted_replace(to_dev(indptr, dev), to_dev(indices, dev), to_dev(probs, dev),
+                                       None, k, seed=3)
+    want = O.sample_weighted_replace(indptr, indices, probs, None, k, seed=3)
+    assert np.array_equal(got[1].cpu().numpy(), want[2])
+    heavy = (want[2] < 10).sum()
+    p = 5000.0 / 24990.0
+    assert abs(heavy - k * p) < 6 * np.sqrt(k * p * (1 - p))
+    counts = np.bincount(want[2][want[2] < 10], minlength=10)
+    assert counts.min() > 0.8 * k * p / 10 and counts.max() < 1.2 * k * p / 10
+
+
+def test_graph_sampling_with_probs_replace(dev):
+    import graph_sampling_amd as gs
+    n = 1 << 10
+    indptr, indices = rmat_csc_np(n, 1 << 14, seed=22)
+    probs = np.random.default_rng(0).random(indices.size).astype(np.float32)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev))
+    g._CAPI_SetData(to_dev(probs, dev))
+    torch.ops.gs_ops._CAPI_SetSeed(99)
+    sub = g._CAPI_SamplingWithProbs(0, to_dev(probs, dev).unsqueeze(1), 5, True, gs._CSC, gs._COO)
+    want = O.sample_weighted_replace(indptr, indices, probs, None, 5, seed=99)
+    row, col = sub._CAPI_GetBatchCOO()
+    assert np.array_equal(row.cpu().numpy(), want[2]) and np.array_equal(col.cpu().numpy(), want[1])
+    # the PASS sampler reads the picked edges' weights back in column order
+    assert np.array_equal(sub._CAPI_GetData("col").cpu().numpy(), probs[want[3]])
+    assert sub._CAPI_GetNumEdges() == want[2].size == 5 * int((np.diff(indptr) > 0).sum())

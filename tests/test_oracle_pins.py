@@ -186,6 +186,40 @@ def test_weighted_closed_form_and_special_cases():
     assert si2.tolist() == np.argsort(-u, kind="stable")[:4].tolist()
 
 
+def test_weighted_replace_closed_form_and_special_cases():
+    # integer weights: every order of float additions gives the same prefix sums, so the
+    # picks must equal a plain cumsum + searchsorted; 150 edges = three scan chunks
+    rng = np.random.default_rng(4)
+    deg, k = 150, 4000
+    indptr = np.array([0, 0, deg], dtype=np.int64)               # column 0 is empty
+    indices = rng.permutation(1000)[:deg].astype(np.int64)
+    w = rng.integers(0, 6, size=deg).astype(np.float32)
+    w[7] = -3.0                                                   # counts as zero
+    draws = u32_draws(2 * k, seed=9)
+    ptr, col, idx, sel = O.sample_weighted_replace(indptr, indices, w, None, k, replay=draws)
+    assert ptr.tolist() == [0, 0, k] and (col == 1).all()
+    cdf = np.cumsum(np.maximum(w, 0), dtype=np.float32)
+    u = ((draws[k:] >> 8).astype(np.float32) + np.float32(1)) * np.float32(2.0 ** -24)
+    want = np.minimum(np.searchsorted(cdf, u * cdf[-1], side="right"), deg - 1)
+    assert np.array_equal(sel, want) and np.array_equal(idx, indices[want])
+    assert (w[sel] > 0).all()
+    # frequencies follow the weights (chi-square over the edges with positive weight)
+    pos = np.flatnonzero(w > 0)
+    obs = np.bincount(sel, minlength=deg)[pos]
+    exp = k * w[pos] / w[pos].sum()
+    assert ((obs - exp) ** 2 / exp).sum() < pos.size + 6 * math.sqrt(2 * pos.size)
+    # one edge carries all the weight: it is every pick
+    one = np.zeros(deg, dtype=np.float32)
+    one[42] = 2.5
+    assert (O.sample_weighted_replace(indptr, indices, one, None, 50, seed=1)[3] == 42).all()
+    # the Philox draw of pick j of row r is draw(seed, tag 2, r, j)
+    _, _, _, a = O.sample_weighted_replace(indptr, indices, w, None, 8, seed=77)
+    d = np.array([O.draw(77, 2, 1, j) for j in range(8)], dtype=np.uint32)
+    _, _, _, b = O.sample_weighted_replace(indptr, indices, w, None, 8,
+                                           replay=np.concatenate([np.zeros(8, np.uint32), d]))
+    assert np.array_equal(a, b)
+
+
 def test_list_sampling_reference_and_closed_form():
     v = REF["list_sampling"]
     data = np.arange(v["n"])
