@@ -33,7 +33,8 @@ def lib():
                      "gs_unique_workspace_bytes", "gs_row_slice_workspace_bytes",
                      "gs_sample_fused_state_bytes", "gs_batch_relabel_workspace_bytes",
                      "gs_coo2csc_workspace_bytes", "gs_col_row_slice_workspace_bytes",
-                     "gs_index_search_workspace_bytes"):
+                     "gs_index_search_workspace_bytes", "gs_relabel_table_bytes",
+                     "gs_relabel_sampled_workspace_bytes", "gs_relabel_sampled_state_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
     return _lib
@@ -272,6 +273,47 @@ def sample_uniform_fused(indptr, indices, column_ids, fanout, replace, seed=0, r
     if mailbox is not None:
         return sub_indptr, sub_indices, select_index, coo_col, ticket
     return sub_indptr, sub_indices, select_index, coo_col
+
+
+class RelabelTable:
+    """The persistent hash table of gs_relabel_sampled (prepared once, left empty by every call)."""
+
+    def __init__(self, max_items, id_dtype, device):
+        self.idb = 8 if id_dtype == torch.int64 else 4
+        nbytes = lib().gs_relabel_table_bytes(_i64(max_items), self.idb)
+        self.buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+        self.prepare()
+
+    def prepare(self):
+        _check(lib().gs_relabel_table_init(_ptr(self.buf), ctypes.c_size_t(self.buf.numel()),
+                                           self.idb, _stream(self.buf.device)),
+               "gs_relabel_table_init")
+
+
+def relabel_sampled(seed_keys, sub_indptr, sub_indices, table, mailbox=None):
+    """gs_relabel_sampled behind a sampler whose total is still on the device (sub_indptr[S]).
+    Returns (frontier buffer, num_unique (device), relabelled sampled ids at capacity[, ticket])."""
+    idb = _ids(seed_keys, "seed_keys")
+    _ids(sub_indices, "sampled ids", like=seed_keys)
+    dev = seed_keys.device
+    S, cap = seed_keys.numel(), sub_indices.numel()
+    M = S + cap
+    frontier = torch.empty(M, dtype=seed_keys.dtype, device=dev)
+    out_ids = torch.empty(cap, dtype=seed_keys.dtype, device=dev)
+    num_unique = torch.empty(1, dtype=torch.int64, device=dev)
+    ws = workspace(lib().gs_relabel_sampled_workspace_bytes(_i64(M)), dev)
+    state, epoch = fused_state(lib().gs_relabel_sampled_state_bytes(_i64(M)), dev)
+    ticket = mailbox.ticket() if mailbox is not None else 0
+    _check(lib().gs_relabel_sampled(
+        _ptr(seed_keys), _i64(S), _ptr(sub_indices), _i64(cap),
+        ctypes.c_void_p(sub_indptr.data_ptr() + 8 * S), idb, _ptr(table.buf),
+        ctypes.c_size_t(table.buf.numel()), _ptr(frontier), _ptr(out_ids), _ptr(num_unique),
+        _ptr(ws), ctypes.c_size_t(ws.numel()), _ptr(state), ctypes.c_size_t(state.numel()),
+        ctypes.c_uint32(epoch), mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0),
+        _i64(ticket), _stream(dev)), "gs_relabel_sampled")
+    if mailbox is not None:
+        return frontier, num_unique, out_ids, ticket
+    return frontier, num_unique, out_ids
 
 
 def sample_one_keepdim(indptr, indices, column_ids, seed=0, replay=None):

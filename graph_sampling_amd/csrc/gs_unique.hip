@@ -23,6 +23,7 @@
 //    so every relabel lookup is two gathers in a last kernel, and a query that
 //    aliases a mapping span is relabelled by slot gather instead of probing.
 #include "gs_common.hpp"
+#include "gs_table.hpp"
 
 namespace gs {
 namespace {
@@ -56,103 +57,6 @@ struct Spans {
     }
     return ptr[s][i - begin];
   }
-};
-
-__device__ __forceinline__ uint32_t fib_home(uint64_t key, int shift) {
-  return static_cast<uint32_t>((key * 0x9E3779B97F4A7C15ull) >> shift);
-}
-
-// ---- slot layout for 32-bit ids: (key << 32 | first index), all ones = empty
-struct PackedTable {
-  unsigned long long* slots;
-  uint32_t mask;
-  int shift;
-  static size_t bytes(int64_t cap) { return padded(cap * 8); }
-  void carve(Carver& ws, int64_t cap) { slots = ws.take<unsigned long long>(cap); }
-  __device__ __forceinline__ void clear(int64_t i) const { slots[i] = ~0ull; }
-  // returns the slot of `key` after recording index i as a candidate first occurrence
-  __device__ __forceinline__ uint32_t insert(long long key, uint32_t i) const {
-    const unsigned long long hi = static_cast<unsigned long long>(static_cast<uint32_t>(key)) << 32;
-    const unsigned long long word = hi | i;
-    uint32_t p = fib_home(static_cast<uint32_t>(key), shift);
-    while (true) {
-      const unsigned long long prev = atomicCAS(&slots[p], ~0ull, word);
-      if (prev == ~0ull) break;
-      if ((prev >> 32) == (hi >> 32)) {
-        if (static_cast<uint32_t>(prev) > i) atomicMin(&slots[p], word);
-        break;
-      }
-      p = (p + 1) & mask;
-    }
-    return p;
-  }
-  __device__ __forceinline__ uint32_t first_index(uint32_t p) const {
-    return static_cast<uint32_t>(slots[p]);
-  }
-  // first index of `key`, or -1 when absent (unique_reindex.cu:44-58)
-  __device__ __forceinline__ int64_t find(long long key) const {
-    const unsigned long long k32 = static_cast<uint32_t>(key);
-    uint32_t p = fib_home(static_cast<uint32_t>(key), shift);
-    while (true) {
-      const unsigned long long s = slots[p];
-      if (s == ~0ull) return -1;
-      if ((s >> 32) == k32) return static_cast<uint32_t>(s);
-      p = (p + 1) & mask;
-    }
-  }
-};
-
-// ---- slot layout for 64-bit ids: key array (-1 = empty) + first-index array
-struct WideTable {
-  long long* keys;
-  int* vals;
-  uint32_t mask;
-  int shift;
-  static size_t bytes(int64_t cap) { return padded(cap * 8) + padded(cap * 4); }
-  void carve(Carver& ws, int64_t cap) {
-    keys = ws.take<long long>(cap);
-    vals = ws.take<int>(cap);
-  }
-  __device__ __forceinline__ void clear(int64_t i) const {
-    keys[i] = -1;
-    vals[i] = 0x7fffffff;
-  }
-  // (unique_reindex.cu:13-26 RelabelHashmap::Update)
-  __device__ __forceinline__ uint32_t insert(long long key, uint32_t i) const {
-    uint32_t p = fib_home(static_cast<uint64_t>(key), shift);
-    while (true) {
-      const unsigned long long prev =
-          atomicCAS(reinterpret_cast<unsigned long long*>(&keys[p]), ~0ull,
-                    static_cast<unsigned long long>(key));
-      if (prev == ~0ull || prev == static_cast<unsigned long long>(key)) break;
-      p = (p + 1) & mask;
-    }
-    // values only decrease, so a (possibly stale) read <= i proves the atomic unnecessary
-    if (__atomic_load_n(&vals[p], __ATOMIC_RELAXED) > static_cast<int>(i))
-      atomicMin(&vals[p], static_cast<int>(i));
-    return p;
-  }
-  __device__ __forceinline__ uint32_t first_index(uint32_t p) const {
-    return static_cast<uint32_t>(vals[p]);
-  }
-  __device__ __forceinline__ int64_t find(long long key) const {
-    uint32_t p = fib_home(static_cast<uint64_t>(key), shift);
-    while (true) {
-      const long long cur = keys[p];
-      if (cur == key) return vals[p];
-      if (cur == -1) return -1;
-      p = (p + 1) & mask;
-    }
-  }
-};
-
-template <typename IdT>
-struct TableFor {
-  using type = WideTable;
-};
-template <>
-struct TableFor<int32_t> {
-  using type = PackedTable;
 };
 
 // empties the table and zeroes the look-back state of the compaction pass
@@ -196,7 +100,7 @@ __global__ void __launch_bounds__(kThreads)
 compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ pos,
                int64_t* __restrict__ prefix, IdT* __restrict__ frontier,
                int64_t* __restrict__ num_unique, LookbackState lb, gs_mailbox* box,
-               int64_t box_ticket) {
+               int64_t box_ticket, uint32_t* __restrict__ first_out) {
   __shared__ int64_t s_scan[kThreads / kWave + 1];
   __shared__ int64_t s_prefix;
   const int64_t M = x.items(M_bound);
@@ -208,8 +112,11 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) {
     const int64_t i = base + k;
-    first[k] = i < M && t.first_index(pos[i]) == static_cast<uint32_t>(i);
+    const uint32_t fi = i < M ? t.first_index(pos[i]) : 0u;
+    first[k] = i < M && fi == static_cast<uint32_t>(i);
     mine += first[k] ? 1 : 0;
+    // kept for a last pass that must not read the table any more (it empties it)
+    if (first_out && i < M) first_out[i] = fi;
   }
   int64_t tile_total;
   const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
@@ -271,14 +178,33 @@ lookup_kernel(T t, const uint32_t* __restrict__ pos, const int64_t* __restrict__
   static_cast<IdT*>(qs.out[s])[local] = static_cast<IdT>(first < 0 ? -1 : prefix[first]);
 }
 
-inline int64_t compact_num_tiles(int64_t M) {
-  return M <= 0 ? 1 : (M + kCompactTile - 1) / kCompactTile;
+// Last pass of a relabel on a table that outlives the call (gs_relabel_sampled): item i >= S is
+// sampled id number i - S, renamed to prefix[its first index]; every item then empties
+// its slot, so the table is clean again for the next call without a clearing pass.  Nothing
+// here reads the table: the first indices were set aside by the compaction.
+template <typename IdT, typename T>
+__global__ void __launch_bounds__(kThreads)
+finish_linked_kernel(T t, const uint32_t* __restrict__ pos, const uint32_t* __restrict__ first,
+                     const int64_t* __restrict__ prefix, int64_t S, int64_t M_bound,
+                     const int64_t* __restrict__ sampled_len, IdT* __restrict__ out_ids) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  int64_t n = *sampled_len;
+  if (n < 0) n = 0;
+  int64_t M = S + n;
+  if (M > M_bound) M = M_bound;
+  if (i >= M) return;
+  if (i >= S) out_ids[i - S] = static_cast<IdT>(prefix[first[i]]);
+  t.clear(pos[i]);
 }
 
-int64_t table_capacity(int64_t M) {
-  int64_t cap = 1024;
-  while (cap < 2 * M) cap <<= 1;
-  return cap;
+template <typename T>
+__global__ void __launch_bounds__(kThreads) table_clear_kernel(T t, int64_t cap) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < cap) t.clear(i);
+}
+
+inline int64_t compact_num_tiles(int64_t M) {
+  return M <= 0 ? 1 : (M + kCompactTile - 1) / kCompactTile;
 }
 
 template <typename IdT>
@@ -322,10 +248,7 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
                    workspace_bytes_for<IdT>(M));
     return GS_ERR_WORKSPACE;
   }
-  t.mask = static_cast<uint32_t>(cap - 1);
-  int lg = 0;
-  while ((int64_t(1) << lg) < cap) ++lg;
-  t.shift = 64 - lg;
+  table_shape(t, cap);
 
   Query qs;
   int64_t Q = 0;
@@ -363,7 +286,7 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
     ProfileScope prof("unique_compact", stream);
     hipLaunchKernelGGL((compact_kernel<IdT, T>), dim3(static_cast<unsigned>(tiles)), dim3(kThreads),
                        0, stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, lb,
-                       box, box_ticket);
+                       box, box_ticket, static_cast<uint32_t*>(nullptr));
   }
   if (Q > 0) {
     ProfileScope prof("unique_finish", stream);
@@ -373,6 +296,65 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   return check_launch("unique_relabel");
 }
 
+
+template <typename IdT>
+int relabel_sampled_impl(const void* seed_keys, int64_t S, const void* sampled, int64_t capacity,
+                         const int64_t* sampled_len, void* table, size_t table_bytes,
+                         void* frontier, void* out_ids, int64_t* num_unique, void* workspace,
+                         size_t workspace_bytes, void* state, size_t state_bytes, uint32_t epoch,
+                         gs_mailbox* box, int64_t box_ticket, hipStream_t stream) {
+  using T = typename TableFor<IdT>::type;
+  const int64_t M = S + capacity;
+  T t;
+  if (!shape_linked_table<T>(table, table_bytes, M, &t)) {
+    set_error_text("gs_relabel_sampled: the table holds fewer than the %lld slots this call "
+                   "needs (or is misaligned)",
+                   static_cast<long long>(linked_table_capacity(M)));
+    return GS_ERR_WORKSPACE;
+  }
+  Carver ws(workspace, workspace_bytes);
+  int64_t* prefix = ws.take<int64_t>(M + 1);
+  uint32_t* first = ws.take<uint32_t>(M > 0 ? M : 1);
+  uint32_t* pos = ws.take<uint32_t>(M > 0 ? M : 1);
+  const int64_t tiles = compact_num_tiles(M);
+  Carver sc(state, state_bytes);
+  LookbackState lb = carve_lookback(sc, tiles, epoch);
+  if (!ws.ok || !sc.ok) {
+    set_error_text("gs_relabel_sampled: workspace needs %zu bytes and state %zu bytes, 256-byte aligned",
+                   gs_relabel_sampled_workspace_bytes(M), gs_relabel_sampled_state_bytes(M));
+    return GS_ERR_WORKSPACE;
+  }
+  Spans<IdT> x;
+  for (int s = 0; s < GS_MAX_SPANS; ++s) {
+    x.ptr[s] = nullptr;
+    x.end[s] = 0;
+  }
+  x.ptr[0] = static_cast<const IdT*>(seed_keys);
+  x.end[0] = S;
+  x.ptr[1] = static_cast<const IdT*>(sampled);
+  x.end[1] = M;
+  x.n = 2;
+  x.last_len = sampled_len;
+  x.fixed = S;
+  if (M > 0) {
+    ProfileScope prof("table_insert", stream);
+    hipLaunchKernelGGL((table_insert_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
+                       0, stream, x, M, t, pos);
+  }
+  {
+    ProfileScope prof("unique_compact", stream);
+    hipLaunchKernelGGL((compact_kernel<IdT, T>), dim3(static_cast<unsigned>(tiles)), dim3(kThreads),
+                       0, stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, lb,
+                       box, box_ticket, first);
+  }
+  if (M > 0) {
+    ProfileScope prof("unique_finish", stream);
+    hipLaunchKernelGGL((finish_linked_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
+                       0, stream, t, pos, first, prefix, S, M, sampled_len,
+                       static_cast<IdT*>(out_ids));
+  }
+  return check_launch("relabel_sampled");
+}
 
 // ------------------------------------------------ batched (super-batch) relabel ----
 // B independent relabels in one pass: replaces impl::BatchCSRRelabelCUDA (reference
@@ -839,6 +821,76 @@ int gs_batch_coo_relabel(const void* seeds, const int64_t* seeds_ptr, const void
                                            num_seeds, num_edges, unique, unique_ptr, out_row,
                                            num_unique, workspace, workspace_bytes, mailbox,
                                            mailbox_ticket, st, coo_col, out_col);
+}
+
+size_t gs_relabel_table_bytes(int64_t max_items, int id_bytes) {
+  if (max_items < 1) max_items = 1;
+  const int64_t cap = linked_table_capacity(max_items);
+  return id_bytes == 4 ? PackedTable::bytes(cap) : WideTable::bytes(cap);
+}
+
+int gs_relabel_table_init(void* table, size_t table_bytes, int id_bytes, void* stream) {
+  GS_REQUIRE(table, "gs_relabel_table_init: null pointer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_relabel_table_init: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (id_bytes == 4) {
+    const int64_t cap = linked_table_slots<PackedTable>(table_bytes);
+    PackedTable t;
+    GS_REQUIRE(cap > 0 && shape_linked_table<PackedTable>(table, table_bytes, cap / 8, &t),
+               "gs_relabel_table_init: buffer too small or misaligned");
+    hipLaunchKernelGGL(table_clear_kernel<PackedTable>, dim3(blocks_for(cap, kThreads)),
+                       dim3(kThreads), 0, st, t, cap);
+  } else {
+    const int64_t cap = linked_table_slots<WideTable>(table_bytes);
+    WideTable t;
+    GS_REQUIRE(cap > 0 && shape_linked_table<WideTable>(table, table_bytes, cap / 8, &t),
+               "gs_relabel_table_init: buffer too small or misaligned");
+    hipLaunchKernelGGL(table_clear_kernel<WideTable>, dim3(blocks_for(cap, kThreads)),
+                       dim3(kThreads), 0, st, t, cap);
+  }
+  return check_launch("relabel_table_init");
+}
+
+size_t gs_relabel_sampled_workspace_bytes(int64_t num_items) {
+  if (num_items < 1) num_items = 1;
+  return padded(static_cast<size_t>(num_items + 1) * 8) +
+         2 * padded(static_cast<size_t>(num_items) * 4);
+}
+
+size_t gs_relabel_sampled_state_bytes(int64_t num_items) {
+  return lookback_state_bytes(compact_num_tiles(num_items));
+}
+
+int gs_relabel_sampled(const void* seed_keys, int64_t S, const void* sampled, int64_t capacity,
+                       const int64_t* sampled_len, int id_bytes, void* table, size_t table_bytes,
+                       void* frontier, void* out_ids, int64_t* num_unique, void* workspace,
+                       size_t workspace_bytes, void* state, size_t state_bytes, uint32_t epoch,
+                       gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream) {
+  GS_REQUIRE(S >= 0 && capacity >= 0 && sampled_len && table && num_unique && state,
+             "gs_relabel_sampled: null pointer or negative size");
+  GS_REQUIRE((S == 0 || seed_keys) && (capacity == 0 || (sampled && out_ids)) &&
+                 (S + capacity == 0 || frontier),
+             "gs_relabel_sampled: null buffer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_relabel_sampled: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  GS_REQUIRE(epoch >= 1 && epoch <= kLbMaxEpoch, "gs_relabel_sampled: epoch must be in 1..%u",
+             kLbMaxEpoch);
+  if (S + capacity >= (int64_t(1) << 31)) {
+    set_error_text("gs_relabel_sampled: %lld items exceed the supported 2^31",
+                   static_cast<long long>(S + capacity));
+    return GS_ERR_UNSUPPORTED;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8
+             ? relabel_sampled_impl<int64_t>(seed_keys, S, sampled, capacity, sampled_len, table,
+                                             table_bytes, frontier, out_ids, num_unique, workspace,
+                                             workspace_bytes, state, state_bytes, epoch, mailbox,
+                                             mailbox_ticket, st)
+             : relabel_sampled_impl<int32_t>(seed_keys, S, sampled, capacity, sampled_len, table,
+                                             table_bytes, frontier, out_ids, num_unique, workspace,
+                                             workspace_bytes, state, state_bytes, epoch, mailbox,
+                                             mailbox_ticket, st);
 }
 
 }  // extern "C"

@@ -143,6 +143,34 @@ FusedStateBuf& FusedState(size_t bytes, const torch::Tensor& like, void* stream)
   return s;
 }
 
+// Hash table of the relabel that follows the sampler, one per (thread, device, stream, id
+// width): prepared when it is (re)allocated or after a failed call, left empty by every
+// call, so no call starts by clearing it.
+struct RelabelTable {
+  torch::Tensor buf;
+  int64_t items = 0;   // number of mapping items it was sized for
+  bool clean = false;  // false: has to be prepared before the next use
+};
+
+RelabelTable& RelabelTableFor(const torch::Tensor& like, void* stream, int idb, int64_t items) {
+  thread_local std::map<std::tuple<int, void*, int>, RelabelTable> tables;
+  RelabelTable& t = tables[{like.device().index(), stream, idb}];
+  if (!t.buf.defined() || t.items < items) {
+    int64_t want = 1 << 16;
+    while (want < items) want <<= 1;
+    t.buf = torch::empty({static_cast<int64_t>(gs_relabel_table_bytes(want, idb))},
+                         torch::dtype(torch::kUInt8).device(like.device()));
+    t.items = want;
+    t.clean = false;
+  }
+  if (!t.clean) {
+    Check(gs_relabel_table_init(t.buf.data_ptr(), t.buf.numel(), idb, stream),
+          "gs_relabel_table_init");
+    t.clean = true;
+  }
+  return t;
+}
+
 torch::TensorOptions I64(const torch::Tensor& like) {
   return torch::dtype(torch::kInt64).device(like.device());
 }
@@ -433,25 +461,29 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t> RelabelDeferred(const torch::T
   const int idb = IdBytes(col_ids, "column ids");
   TORCH_CHECK(IdBytes(p.indices, "sampled ids") == idb, "relabel tensors differ in dtype");
   const int64_t cap = p.indices.numel();
-  const int64_t M = col_ids.numel() + cap;
-  gs_span m[2] = {{col_ids.data_ptr(), col_ids.numel()}, {p.indices.data_ptr(), cap}};
-  gs_span q[1] = {{p.indices.data_ptr(), cap}};
+  const int64_t S = col_ids.numel();
+  const int64_t M = S + cap;
   auto renamed = torch::empty_like(p.indices);
-  void* out_ptr[1] = {renamed.data_ptr()};
   auto frontier = torch::empty({M}, col_ids.options());
   auto num = torch::empty({1}, I64(col_ids));
-  auto ws = Scratch(gs_unique_workspace_bytes(M), col_ids);
+  auto ws = Scratch(gs_relabel_sampled_workspace_bytes(M), col_ids);
+  RelabelTable& table = RelabelTableFor(col_ids, p.stream, idb, M);
+  FusedStateBuf& state = FusedState(gs_relabel_sampled_state_bytes(M), col_ids, p.stream);
   HostBoxes& boxes = Boxes(p.device);
   const int64_t ticket = boxes.next++;
-  Check(gs_unique_relabel_notify(m, 2, q, out_ptr, 1, idb, frontier.data_ptr(),
-                                 num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(),
-                                 p.sub_indptr.data_ptr<int64_t>() + p.S, boxes.slot(ticket), ticket,
-                                 p.stream),
-        "gs_unique_relabel");
+  table.clean = false;  // until both totals have come back
+  Check(gs_relabel_sampled(col_ids.data_ptr(), S, p.indices.data_ptr(), cap,
+                           p.sub_indptr.data_ptr<int64_t>() + p.S, idb, table.buf.data_ptr(),
+                           table.buf.numel(), frontier.data_ptr(), renamed.data_ptr(),
+                           num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(),
+                           state.buf.data_ptr(), state.buf.numel(), state.epoch,
+                           boxes.slot(ticket), ticket, p.stream),
+        "gs_relabel_sampled");
   const int64_t nnz = p.Wait();
-  int64_t U = WaitBox(boxes.slot(ticket), ticket, p.stream, "gs_unique_relabel");
+  int64_t U = WaitBox(boxes.slot(ticket), ticket, p.stream, "gs_relabel_sampled");
   if (U == kLost) U = num.item<int64_t>();
-  TORCH_CHECK(U >= 0, "gs_unique_relabel: a tile gave up waiting for its predecessors");
+  TORCH_CHECK(U >= 0, "gs_relabel_sampled: a tile gave up waiting for its predecessors");
+  table.clean = true;
   return {frontier.narrow(0, 0, U), renamed.narrow(0, 0, nnz), nnz};
 }
 

@@ -286,6 +286,32 @@ int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_spa
                              const int64_t* last_span_len, gs_mailbox* mailbox,
                              int64_t mailbox_ticket, void* stream);
 
+/* The relabel that follows a sampler, on a hash table that outlives the calls (no
+ * counterpart in the reference, which allocates and fills a fresh table per call,
+ * src/cuda/unique_reindex.cu:86-88).  Same result as gs_unique_relabel_notify with the
+ * mapping (seed_keys[0..S), sampled[0..*sampled_len)) and `sampled` as the one query:
+ * frontier (capacity S + capacity), out_ids (capacity), *num_unique and the mailbox.
+ *   table: gs_relabel_table_bytes(max_items, id_bytes) bytes, 256-byte aligned, prepared
+ *     once with gs_relabel_table_init; max_items >= S + capacity of every call.  The last
+ *     kernel of a call empties exactly the slots the call used, so no call starts by
+ *     clearing the table and its size costs nothing per call (it is kept at a load of at
+ *     most 1/8).  A call that failed half-way (*num_unique == -1) leaves it undefined:
+ *     prepare it again.  One call at a time per table.
+ *   sampled_len: device address of the true number of sampled ids (sub_indptr + S of the
+ *     sampler); `capacity` only bounds it.
+ *   workspace: gs_relabel_sampled_workspace_bytes(S + capacity); state / epoch: as for
+ *     gs_sample_uniform_fused, gs_relabel_sampled_state_bytes(S + capacity) bytes (the
+ *     sampler's state buffer may be shared when large enough, with a fresh epoch). */
+size_t gs_relabel_table_bytes(int64_t max_items, int id_bytes);
+int gs_relabel_table_init(void* table, size_t table_bytes, int id_bytes, void* stream);
+size_t gs_relabel_sampled_workspace_bytes(int64_t num_items);
+size_t gs_relabel_sampled_state_bytes(int64_t num_items);
+int gs_relabel_sampled(const void* seed_keys, int64_t S, const void* sampled, int64_t capacity,
+                       const int64_t* sampled_len, int id_bytes, void* table, size_t table_bytes,
+                       void* frontier, void* out_ids, int64_t* num_unique, void* workspace,
+                       size_t workspace_bytes, void* state, size_t state_bytes, uint32_t epoch,
+                       gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
+
 /* B relabels in one pass ("super-batch"): replaces impl::BatchCSRRelabelCUDA
  * (src/cuda/batch_relabel.cu:331).  Batch b owns seeds[seeds_ptr[b]..seeds_ptr[b+1])
  * and ids[ids_ptr[b]..ids_ptr[b+1]) (both *_ptr: device int64[num_batches+1]).

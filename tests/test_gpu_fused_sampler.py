@@ -179,3 +179,37 @@ def test_relabel_with_device_side_length(dev, idt):
         assert nnz == int(want[0][-1]) and U == f_want.size
         assert np.array_equal(frontier[:U].cpu().numpy().astype(np.int64), f_want)
         assert np.array_equal(outs[0][:nnz].cpu().numpy().astype(np.int64), r_want[0])
+
+
+# ------------------------------ relabel behind the sampler on a persistent table
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+@pytest.mark.parametrize("S,fanout,replace", [(1, 3, False), (700, 15, False), (5000, 5, False),
+                                               (40000, 5, False), (3000, 4, True)])
+def test_relabel_sampled_matches_the_one_call_relabel(dev, S, fanout, replace, idt):
+    n = 1 << 14
+    indptr, indices = rmat_csc_np(n, 1 << 19, seed=31)
+    rng = np.random.default_rng(S)
+    cols = rng.integers(0, n, size=S).astype(np.int64)            # duplicates among the seeds
+    keys = cols + 1000                                            # the ids the columns go by
+    t_ptr, t_idx = to_dev(indptr, dev), to_dev(indices, dev, idt)
+    t_cols, t_keys = to_dev(cols, dev, idt), to_dev(keys, dev, idt)
+    table = capi.RelabelTable(S + S * fanout + 100000, idt, dev)
+    # several calls in a row on the same table: every call leaves it empty
+    for seed in (5, 6, 7):
+        sp, si, _, _ = capi.sample_uniform_fused(t_ptr, t_idx, t_cols, fanout, replace, seed=seed)
+        frontier, num, out = capi.relabel_sampled(t_keys, sp, si, table)
+        w_sp, _, w_si, _ = O.sample_uniform(indptr, indices, cols, fanout, replace, seed=seed, with_coo=False)
+        w_frontier, (w_out,) = O.relabel([keys, w_si], [w_si])
+        E = int(w_sp[-1])
+        assert np.array_equal(si[:E].cpu().numpy().astype(np.int64), w_si)
+        assert int(num.item()) == w_frontier.size
+        assert np.array_equal(frontier[:w_frontier.size].cpu().numpy().astype(np.int64), w_frontier)
+        assert np.array_equal(out[:E].cpu().numpy().astype(np.int64), w_out)
+    torch.cuda.synchronize()
+    words = table.buf.view(torch.int64)
+    if idt == torch.int32:
+        assert bool((words == -1).all())
+    else:
+        slots = words.numel() * 8 // 12 // 1024 * 1024     # keys (8 B) then first indices (4 B)
+        cap = 1 << (slots.bit_length() - 1)
+        assert bool((words[:cap] == -1).all())
