@@ -142,3 +142,24 @@ def test_batch_csr_relabel_matches_oracle(dev, idt, B, max_seeds, max_ids, empty
         f = _closed_form_unique(x)
         assert np.array_equal(w_unique[w_ptr[b]:w_ptr[b + 1]], f)
         assert np.array_equal(f[w_out[ip[b]:ip[b + 1]]], ids[ip[b]:ip[b + 1]])
+
+
+# a few tiles of the compaction, with keys all distinct, in long runs, and in between
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+@pytest.mark.parametrize("n", [8191, 8192, 8193, 16383, 16384, 16385])
+@pytest.mark.parametrize("spread", ["distinct", "few", "mixed"])
+def test_relabel_few_tiles_by_key_spread(dev, idt, n, spread):
+    rng = np.random.default_rng(n)
+    if spread == "distinct":
+        rows = (rng.permutation(1 << 20)[:n - 100].astype(np.int64) * 7 + 3)
+    elif spread == "few":           # long runs of the same key
+        rows = rng.integers(0, 17, size=n - 100).astype(np.int64) * 65537
+    else:
+        rows = rng.integers(0, n // 2, size=n - 100).astype(np.int64)
+    seeds = rows[rng.permutation(rows.size)[:100]]
+    other = rng.integers(0, 1 << 21, size=999).astype(np.int64)
+    frontier, outs = _run([seeds, rows], [rows, other], dev, idt)
+    want_frontier, want = O.relabel([seeds, rows], [rows, other])
+    assert np.array_equal(frontier, want_frontier)
+    for g, w in zip(outs, want):
+        assert np.array_equal(g, w)
