@@ -153,6 +153,33 @@ def super_batch(torch, graph, seed_sets):
     return total, blocks
 
 
+def concurrent(torch, graph, seed_sets, workers):
+    """The same minibatches with `workers` of them in flight: one host thread and one stream
+    each, as a loader with sampler workers would run them.  The per-minibatch results do not
+    depend on the interleaving (every thread counts its own seeds)."""
+    import threading
+    dev = seed_sets[0].device
+    edges = [0] * workers
+
+    def work(k):
+        stream = torch.cuda.Stream(device=dev)
+        with torch.cuda.stream(stream):
+            for i in range(k, len(seed_sets), workers):
+                torch.ops.gs_ops._CAPI_SetThreadSeed(i * len(FANOUTS))
+                edges[k] += minibatch(graph, seed_sets[i])[0]
+            stream.synchronize()
+
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(workers)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    return sum(edges), time.perf_counter() - t1
+
+
 def cpu_minibatch(O, np, indptr, indices, seeds, step):
     total = 0
     for layer, k in enumerate(FANOUTS):
@@ -310,6 +337,14 @@ def main():
               "what": "fused sampling + GetBatchCSC + BatchCSRRelabel + splits over 64 minibatches "
                       "of 1024 seeds at once; every minibatch is relabelled on its own"}
 
+    # the same minibatches, four in flight (reported beside the headline)
+    WORKERS = 4
+    concurrent(torch, graph, seed_sets[:4 * WORKERS], WORKERS)
+    cc_edges, cc_s = concurrent(torch, graph, seed_sets[args.warmup:], WORKERS)
+    cc = {"workers": WORKERS, "ms_per_step": cc_s / args.steps * 1e3, "value": cc_edges / cc_s,
+          "what": "the timed minibatches again with four in flight, one host thread and one "
+                  "stream each"}
+
     out = {
         "metric": "sampled edges/sec (GSEPS), GraphSAGE [15,10,5] batch 1024, slice+sample+relabel",
         "value": sampled / elapsed,
@@ -332,6 +367,7 @@ def main():
                          "steps": nf_steps,
                          "what": "Slicing -> Sampling -> Relabel per layer instead of the fused sampler"},
         "super_batch": sb,
+        "concurrent": cc,
         "roofline": None,
         "cpu_baseline": None,
     }

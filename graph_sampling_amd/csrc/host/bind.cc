@@ -16,6 +16,7 @@ using namespace gs;
 
 namespace {
 void SetSeed(int64_t seed) { hip::SetSeed(static_cast<uint64_t>(seed)); }
+void SetThreadSeed(int64_t seed) { hip::SetThreadSeed(static_cast<uint64_t>(seed)); }
 void SetSampleAlgo(int64_t algo) { hip::SetSampleAlgo(algo); }
 void SetDeferredSampling(bool on) { hip::SetDeferredSampling(on); }
 torch::Tensor UniqueOp(torch::Tensor ids) { return TensorUnique(ids); }
@@ -134,6 +135,7 @@ TORCH_LIBRARY(gs_ops, m) {
   m.def("index_search", &IndexSearch);
   // not in the reference: reproducible sampling (its seeds are compile-time constants)
   m.def("_CAPI_SetSeed", &SetSeed);
+  m.def("_CAPI_SetThreadSeed", &SetThreadSeed);
   m.def("_CAPI_SetSampleAlgo", &SetSampleAlgo);
   // not in the reference: off = every sampling call settles its edge count before returning
   m.def("_CAPI_SetDeferredSampling", &SetDeferredSampling);

@@ -188,8 +188,18 @@ int OpCode(const std::string& op) {
 
 }  // namespace
 
+namespace {
+// a thread that called SetThreadSeed counts its own seeds from then on
+thread_local bool t_own_seed = false;
+thread_local uint64_t t_seed = 0;
+}  // namespace
+
 void SetSeed(uint64_t seed) { g_seed.store(seed); }
-uint64_t NextSeed() { return g_seed.fetch_add(1); }
+void SetThreadSeed(uint64_t seed) {
+  t_own_seed = true;
+  t_seed = seed;
+}
+uint64_t NextSeed() { return t_own_seed ? t_seed++ : g_seed.fetch_add(1); }
 void SetSampleAlgo(int64_t algo) {
   TORCH_CHECK(algo == GS_SAMPLE_AUTO || algo == GS_SAMPLE_RESERVOIR, "unknown sampling algorithm ", algo);
   g_algo.store(algo);

@@ -710,3 +710,53 @@ def test_indptr_split_by_size(dev):
     assert len(pieces) == 10  # the ragged tail of 3 columns is dropped, as in the reference
     for b, p in enumerate(pieces):
         assert np.array_equal(p.cpu().numpy(), indptr[10 * b:10 * b + 11] - indptr[10 * b])
+
+
+def test_sampler_threads_on_their_own_streams_are_reproducible(dev):
+    """Four host threads, one stream each, run GraphSAGE minibatches at the same time; with a
+    seed of its own per minibatch every result equals the oracle's, however they interleave."""
+    import threading
+    n = 1 << 15
+    indptr, indices = rmat_csc_np(n, 1 << 20, seed=41)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev, torch.int32))
+    rng = np.random.default_rng(7)
+    batches = [rng.permutation(n)[:256].astype(np.int64) for _ in range(24)]
+    t_batches = [to_dev(b, dev, torch.int32) for b in batches]
+    fanouts = (7, 5)
+    got = [None] * len(batches)
+    errors = []
+
+    def work(k, workers):
+        try:
+            stream = torch.cuda.Stream(device=dev)
+            with torch.cuda.stream(stream):
+                for i in range(k, len(batches), workers):
+                    torch.ops.gs_ops._CAPI_SetThreadSeed(1000 + i * len(fanouts))
+                    seeds, layers = t_batches[i], []
+                    for f in fanouts:
+                        sub = g._CAPI_FusedColumnwiseSlicingSampling(seeds, f, False)
+                        frontier, _, _, ptr, idx, _, _ = sub._CAPI_Relabel()
+                        layers.append((ptr, idx, frontier))
+                        seeds = frontier
+                    stream.synchronize()
+                    got[i] = [tuple(t.cpu().numpy().astype(np.int64) for t in l) for l in layers]
+        except Exception as e:   # surfaced below: an assert in a thread is otherwise lost
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(k, 4)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i, b in enumerate(batches):
+        seeds = b
+        for l, f in enumerate(fanouts):
+            w_ptr, _, w_rows, _ = O.sample_uniform(indptr, indices, seeds, f, False,
+                                                   seed=1000 + i * len(fanouts) + l, with_coo=False)
+            w_frontier, (w_idx,) = O.relabel([seeds, w_rows], [w_rows])
+            ptr, idx, frontier = got[i][l]
+            assert np.array_equal(ptr, w_ptr) and np.array_equal(idx, w_idx)
+            assert np.array_equal(frontier, w_frontier)
+            seeds = w_frontier
