@@ -46,6 +46,9 @@ def parse():
     ap.add_argument("--cpu-steps", type=int, default=-1,
                     help="minibatches timed for the host-core baseline (-1: sized to ~15 s)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="skip the passes reported beside the headline (unfused operators, "
+                         "super-batch, four in flight): for profiling the timed step alone")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain device copy of the indices array (a kernel of known "
                          "traffic to scale hardware byte counters by)")
@@ -308,22 +311,27 @@ def main():
     p90 = lat[min(len(lat) - 1, int(len(lat) * 0.9))] * 1e3
 
     # the unfused operator sequence on the same seed sets (reported beside the headline)
-    nf_steps = min(args.steps, 50)
-    for i in range(3):
-        minibatch_nonfused(graph, seed_sets[i])
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    nf_edges = 0
-    for i in range(nf_steps):
-        nf_edges += minibatch_nonfused(graph, seed_sets[args.warmup + i])
-    torch.cuda.synchronize()
-    nf_s = time.perf_counter() - t1
+    extras = not args.headline_only
+    nf = None
+    if extras:
+        nf_steps = min(args.steps, 50)
+        for i in range(3):
+            minibatch_nonfused(graph, seed_sets[i])
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        nf_edges = 0
+        for i in range(nf_steps):
+            nf_edges += minibatch_nonfused(graph, seed_sets[args.warmup + i])
+        torch.cuda.synchronize()
+        nf_s = time.perf_counter() - t1
+        nf = {"ms_per_step": nf_s / nf_steps * 1e3, "value": nf_edges / nf_s, "steps": nf_steps,
+              "what": "Slicing -> Sampling -> Relabel per layer instead of the fused sampler"}
 
     # the same minibatches, SUPER of them per call (reported beside the headline)
     SUPER = 64
     groups = [seed_sets[i:i + SUPER] for i in range(0, len(seed_sets) - SUPER + 1, SUPER)][:8]
     sb = None
-    if groups:
+    if groups and extras:
         super_batch(torch, graph, groups[0])
         torch.cuda.synchronize()
         t1 = time.perf_counter()
@@ -339,11 +347,14 @@ def main():
 
     # the same minibatches, four in flight (reported beside the headline)
     WORKERS = 4
-    concurrent(torch, graph, seed_sets[:4 * WORKERS], WORKERS)
-    cc_edges, cc_s = concurrent(torch, graph, seed_sets[args.warmup:], WORKERS)
-    cc = {"workers": WORKERS, "ms_per_step": cc_s / args.steps * 1e3, "value": cc_edges / cc_s,
-          "what": "the timed minibatches again with four in flight, one host thread and one "
-                  "stream each"}
+    cc = None
+    if extras:
+        concurrent(torch, graph, seed_sets[:4 * WORKERS], WORKERS)
+        cc_edges, cc_s = concurrent(torch, graph, seed_sets[args.warmup:], WORKERS)
+        cc = {"workers": WORKERS, "ms_per_step": cc_s / args.steps * 1e3,
+              "value": cc_edges / cc_s,
+              "what": "the timed minibatches again with four in flight, one host thread and one "
+                      "stream each"}
 
     out = {
         "metric": "sampled edges/sec (GSEPS), GraphSAGE [15,10,5] batch 1024, slice+sample+relabel",
@@ -363,9 +374,7 @@ def main():
         "config": {"workload": args.workload, "nodes": nodes, "edges": edges, "batch": BATCH,
                    "fanouts": list(FANOUTS), "last_step_layers_S_E_U": layer_sizes,
                    "graph_build_s": round(gen_s, 2)},
-        "unfused_path": {"ms_per_step": nf_s / nf_steps * 1e3, "value": nf_edges / nf_s,
-                         "steps": nf_steps,
-                         "what": "Slicing -> Sampling -> Relabel per layer instead of the fused sampler"},
+        "unfused_path": nf,
         "super_batch": sb,
         "concurrent": cc,
         "roofline": None,
