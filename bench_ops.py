@@ -1,0 +1,185 @@
+#!/usr/bin/env python3
+"""Timings of the operators around the headline path (one MI355X), one JSON line each.
+
+bench.py measures the GraphSAGE minibatch; this script times the other rows of the scope
+table at the sizes of their configurations -- induced-subgraph slicing, the doubly-compressed
+conversions, weighted sampling with and without replacement, the super-batch helpers, walks,
+SDDMM, segment sums, row slicing -- through the same C ABI (graph_sampling_amd/capi.py), with
+`algorithmic` = the bytes the operator must move at the least (stated per line) over the
+median of the timed calls.  Timing: torch.cuda.Event pairs on the current stream, which is the
+stream the C ABI is given; a call is all the launches of the operator, host reads included
+where the operator has one.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+HBM_PEAK_GBS = 8000.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--nodes", type=int, default=2_450_000)
+    ap.add_argument("--edges", type=int, default=124_000_000)
+    ap.add_argument("--reps", type=int, default=10)
+    ap.add_argument("--only", default="", help="comma-separated operator names")
+    args = ap.parse_args()
+    import torch
+    from graph_sampling_amd import capi, rmat
+
+    if not torch.cuda.is_available():
+        print("bench_ops.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    capi.lib()
+    dev = torch.device("cuda:0")
+    N, E = args.nodes, args.edges
+    idt = torch.int32
+    b = 4
+    indptr, indices = rmat.rmat_csc(N, E, seed=0, device=dev, index_dtype=idt)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+    weights = 1.0 - torch.rand(E, generator=gen, device=dev)
+    only = set(x for x in args.only.split(",") if x)
+
+    def rand_ids(n, hi=N):
+        return torch.randint(0, hi, (n,), generator=gen, device=dev).to(idt)
+
+    def perm_ids(n):
+        return torch.randperm(N, generator=gen, device=dev)[:n].to(idt)
+
+    def run(name, what, fn, bytes_of):
+        if only and name not in only:
+            return
+        for _ in range(2):
+            out = fn()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(args.reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = fn()
+            e1.record()
+            e1.synchronize()
+            times.append(e0.elapsed_time(e1) * 1e-3)
+        times.sort()
+        t = times[len(times) // 2]
+        nbytes, units, unit_name = bytes_of(out)
+        print(json.dumps({"op": name, "what": what, "ms": t * 1e3, unit_name: units,
+                          "per_s": units / t, "algorithmic_bytes": nbytes,
+                          "achieved_GBs": nbytes / t / 1e9,
+                          "frac_of_hbm_peak": nbytes / t / 1e9 / HBM_PEAK_GBS}), flush=True)
+
+    # ---- column slice of a third-layer frontier (45k columns) ---------------------------------
+    cols45k = perm_ids(45_000)
+
+    def slice45k():
+        offsets = capi.slice_count(indptr, cols45k)
+        return capi.slice_fill(indptr, indices, cols45k, offsets, int(offsets[-1].item()), False)
+
+    run("slice", "gs_slice_count + gs_slice_fill, 45k columns, with select_index; 16 B per edge",
+        slice45k, lambda o: (o[0].numel() * (2 * b + 8) + 45_000 * 32, o[0].numel(), "edges"))
+
+    # ---- induced subgraph: 100k columns, 200k admissible rows ---------------------------------
+    c100k, r200k = perm_ids(100_000), perm_ids(200_000)
+    D = int(capi.slice_count(indptr, c100k)[-1].item())
+    run("col_row_slice", "gs_col_row_slice_*: 100k columns x 200k rows, D = %d edges looked at; "
+        "b + 16 B per edge looked at (id read, mark, scan), 2b + 16 per edge kept" % D,
+        lambda: capi.col_row_slice(indptr, indices, c100k, r200k),
+        lambda o: (D * (b + 16) + o[1].numel() * (2 * b + 16), D, "edges"))
+
+    # ---- row slicing of a column slice (FastGCN layer: keep 512 sampled rows) -----------------
+    sp = capi.slice_count(indptr, cols45k)
+    nnz = int(sp[-1].item())
+    s_idx, s_sel, s_col = capi.slice_fill(indptr, indices, cols45k, sp, nnz, True)
+    rows512 = perm_ids(512)
+    run("row_slice_coo", "gs_row_slice_coo_*: %d edges, 512 row ids; b + 16 B per edge" % nnz,
+        lambda: capi.row_slice_coo(s_idx, s_col, rows512),
+        lambda o: (nnz * (b + 16), nnz, "edges"))
+
+    # ---- weighted sampling of the same slice ---------------------------------------------------
+    w_slice = weights[:nnz].contiguous()
+    run("sample_weighted", "gs_sample_weighted_fill (A-Res, fanout 10) over the 45k-column slice; "
+        "b + 4 B per edge read, 2b + 8 per edge kept",
+        lambda: capi.sample_weighted(sp, s_idx, w_slice, None, 10),
+        lambda o: (nnz * (b + 4) + 450_000 * (2 * b + 8), nnz, "edges"))
+    run("sample_weighted_replace", "gs_sample_weighted_replace (inverse CDF, fanout 10) over the "
+        "same slice; 4 B read + 4 B prefix write per edge, 2b + 8 per pick",
+        lambda: capi.sample_weighted_replace(sp, s_idx, w_slice, None, 10),
+        lambda o: (nnz * 8 + 450_000 * (2 * b + 8), nnz, "edges"))
+
+    # ---- doubly-compressed conversions -----------------------------------------------------------
+    run("csc2coo", "gs_csc2coo over the whole graph; 8 B offsets per column + b per edge written",
+        lambda: capi.csc2coo(indptr, E, idt),
+        lambda o: (E * b + N * 8, E, "edges"))
+
+    # ---- super-batch helpers on a third-layer super-batch (64 x 45k columns, 14M edges) -------
+    B = 64
+    M = 14_000_000
+    ptr = (torch.arange(B + 1, device=dev, dtype=torch.int64) * (M // B))
+    data = rand_ids(M)
+    run("batch_encode", "gs_batch_encode, 14M ids in 64 batches; 2b per id",
+        lambda: capi.batch_encode(data, ptr, N),
+        lambda o: (M * 2 * b, M, "ids"))
+    enc = capi.batch_encode(data, ptr, N)  # fits 32 bits: 64 * 2.45M
+    run("batch_decode", "gs_batch_decode (ids and batch numbers); 3b per id",
+        lambda: capi.batch_decode(enc, N),
+        lambda o: (M * 3 * b, M, "ids"))
+    ptr2 = (torch.arange(B + 1, device=dev, dtype=torch.int64) * 1024)
+    seeds64 = rand_ids(B * 1024)
+    run("batch_concat", "gs_batch_concat_*: 64k seeds ++ 14M ids batch by batch; 3b per id (value "
+        "in, value and batch number out)",
+        lambda: capi.batch_concat([seeds64, data], [ptr2, ptr]),
+        lambda o: ((M + B * 1024) * 3 * b, M + B * 1024, "ids"))
+    total, key, total_ptr = capi.batch_concat([seeds64, data], [ptr2, ptr])
+    run("batch_split", "gs_batch_split, the inverse; 3b per id",
+        lambda: capi.batch_split(total, total_ptr, key, [ptr2, ptr]),
+        lambda o: ((M + B * 1024) * 3 * b, M + B * 1024, "ids"))
+    run("batch_csr_relabel", "gs_batch_csr_relabel: 64 relabels of (1024 seeds, 218k ids) in one "
+        "pass; about 70 B per item (insert, compaction, lookup)",
+        lambda: capi.batch_csr_relabel(seeds64, ptr2, data, ptr),
+        lambda o: ((M + B * 1024) * 70, M + B * 1024, "items"))
+    col14 = rand_ids(M)
+    run("batch_coo_relabel", "gs_batch_coo_relabel: the same with both ends of 14M edges renamed",
+        lambda: capi.batch_coo_relabel(seeds64, ptr2, data, col14, ptr),
+        lambda o: ((M + B * 1024) * 70 + M * (2 * b + 8), M + B * 1024, "items"))
+    ids_ptr = (torch.arange(B + 1, device=dev, dtype=torch.int64) * 4000)
+    chosen = rand_ids(B * 4000)
+    run("coo_filter_batched", "gs_coo_filter_*: 14M edges in 64 batches against 4000 chosen ids per "
+        "batch; b + 16 B per edge (key, mark, scan)",
+        lambda: capi.coo_filter(data, data, col14, chosen, ptr, ids_ptr),
+        lambda o: (M * (b + 16) + o[0].numel() * 4 * b, M, "edges"))
+    run("index_search", "gs_index_search: 14M keys against 256k stored ids; 2b per key",
+        lambda: capi.index_search(chosen, data),
+        lambda o: (M * 2 * b, M, "keys"))
+
+    # ---- unique / relabel of one large frontier --------------------------------------------------
+    big = rand_ids(16_000_000)
+    run("unique_relabel", "gs_unique_relabel: 16M ids, relabelled in place; about 70 B per item",
+        lambda: capi.unique_relabel([big], [big]),
+        lambda o: (16_000_000 * 70, 16_000_000, "items"))
+
+    # ---- walks, SDDMM, segment sum at their configuration sizes ---------------------------------
+    starts = rand_ids(1_000_000)
+    run("random_walk", "gs_random_walk: 1M walkers x 80 steps on this graph; 28 B per live step",
+        lambda: capi.random_walk(indptr, indices, starts, 80, seed=3),
+        lambda o: (int((o[1_000_000:] >= 0).sum().item()) * 28,
+                   int((o[1_000_000:] >= 0).sum().item()), "steps"))
+    feat = torch.rand(N, 64, generator=gen, device=dev)
+    er, ec = rand_ids(8_000_000), rand_ids(8_000_000)
+    out_e = torch.empty(8_000_000, 1, device=dev)
+    run("sddmm_dot", "gs_sddmm_coo u_dot_v, 64-d fp32 features, 8M random edges; 532 B per edge",
+        lambda: capi.sddmm_coo("dot", er, ec, None, feat, feat, out_e, 0, 2, 64, 64, 1, 64, None, None),
+        lambda o: (8_000_000 * 532, 8_000_000, "edges"))
+    out_n = torch.empty(N, device=dev)
+    run("segment_sum", "gs_segment_sum of w^2 over every column of the graph; 4 B per edge + 20 B "
+        "per column",
+        lambda: capi.segment_sum(indptr, None, None, weights, 2, out_n),
+        lambda o: (E * 4 + N * 20, E, "edges"))
+
+
+if __name__ == "__main__":
+    main()

@@ -34,7 +34,8 @@ def lib():
                      "gs_sample_fused_state_bytes", "gs_batch_relabel_workspace_bytes",
                      "gs_coo2csc_workspace_bytes", "gs_col_row_slice_workspace_bytes",
                      "gs_index_search_workspace_bytes", "gs_relabel_table_bytes",
-                     "gs_relabel_sampled_workspace_bytes", "gs_relabel_sampled_state_bytes"):
+                     "gs_relabel_sampled_workspace_bytes", "gs_relabel_sampled_state_bytes",
+                     "gs_segment_workspace_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
     return _lib
@@ -704,9 +705,13 @@ def segment_sum(indptr, e_ids, n_ids, data, powk, out):
     _need(data, torch.float32, "data")
     _need(out, torch.float32, "out")
     idb = _ids(n_ids, "n_ids") if n_ids is not None else 8
+    nseg = indptr.numel() - 1
+    nnz = e_ids.numel() if e_ids is not None else data.numel()
+    ws = workspace(lib().gs_segment_workspace_bytes(_i64(nseg), _i64(nnz)), indptr.device)
     _check(lib().gs_segment_sum(_ptr(indptr), _ptr(e_ids), _ptr(n_ids), idb, _ptr(data),
-                                _i64(indptr.numel() - 1), _i64(powk), _ptr(out),
-                                _stream(indptr.device)), "gs_segment_sum")
+                                _i64(nseg), _i64(nnz), _i64(powk), _ptr(out), _ptr(ws),
+                                ctypes.c_size_t(ws.numel()), _stream(indptr.device)),
+           "gs_segment_sum")
 
 
 def coo_sum(target, e_ids, data, powk, out):
@@ -721,9 +726,12 @@ def segment_normalize(indptr, e_ids, data, out):
     _need(indptr, torch.int64, "indptr")
     _need(data, torch.float32, "data")
     _need(out, torch.float32, "out")
-    _check(lib().gs_segment_normalize(_ptr(indptr), _ptr(e_ids), _ptr(data),
-                                      _i64(indptr.numel() - 1), _ptr(out), _stream(indptr.device)),
-           "gs_segment_normalize")
+    nseg = indptr.numel() - 1
+    nnz = e_ids.numel() if e_ids is not None else data.numel()
+    ws = workspace(lib().gs_segment_workspace_bytes(_i64(nseg), _i64(nnz)), indptr.device)
+    _check(lib().gs_segment_normalize(_ptr(indptr), _ptr(e_ids), _ptr(data), _i64(nseg), _i64(nnz),
+                                      _ptr(out), _ptr(ws), ctypes.c_size_t(ws.numel()),
+                                      _stream(indptr.device)), "gs_segment_normalize")
 
 
 def e_div_u_sum(row, col, data, divisor, out_data, out_sum):

@@ -618,9 +618,12 @@ void SegmentSum(const torch::Tensor& indptr, const torch::optional<torch::Tensor
   NeedF32(data, "data");
   NeedF32(out, "out");
   const int idb = n_ids.has_value() && n_ids.value().defined() ? IdBytes(n_ids.value(), "valid ids") : 8;
+  const int64_t nseg = indptr.numel() - 1;
+  const int64_t nnz = e_ids.has_value() && e_ids.value().defined() ? e_ids.value().numel() : data.numel();
+  auto ws = Scratch(gs_segment_workspace_bytes(nseg, nnz), indptr);
   Check(gs_segment_sum(indptr.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"),
-                       OptIds(n_ids, idb, "valid ids"), idb, data.data_ptr<float>(), indptr.numel() - 1, powk, out.data_ptr<float>(),
-                       Stream(indptr)),
+                       OptIds(n_ids, idb, "valid ids"), idb, data.data_ptr<float>(), nseg, nnz, powk,
+                       out.data_ptr<float>(), ws.data_ptr(), ws.numel(), Stream(indptr)),
         "gs_segment_sum");
 }
 
@@ -639,9 +642,12 @@ void SegmentNormalize(const torch::Tensor& indptr, const torch::optional<torch::
   NeedI64(indptr, "indptr");
   NeedF32(data, "data");
   NeedF32(out, "out");
+  const int64_t nseg = indptr.numel() - 1;
+  const int64_t nnz = e_ids.has_value() && e_ids.value().defined() ? e_ids.value().numel() : data.numel();
+  auto ws = Scratch(gs_segment_workspace_bytes(nseg, nnz), indptr);
   Check(gs_segment_normalize(indptr.data_ptr<int64_t>(), OptI64(e_ids, "e_ids"),
-                             data.data_ptr<float>(), indptr.numel() - 1, out.data_ptr<float>(),
-                             Stream(indptr)),
+                             data.data_ptr<float>(), nseg, nnz, out.data_ptr<float>(), ws.data_ptr(),
+                             ws.numel(), Stream(indptr)),
         "gs_segment_normalize");
 }
 

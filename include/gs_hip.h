@@ -385,10 +385,15 @@ int gs_sddmm_csc(int op, const int64_t* indptr, const void* indices, int id_byte
 /* (src/cuda/fusion/edge_map_reduce.cu:10).  Node ids (n_ids, target, row, col) */
 /* are id_bytes wide; e_ids are positions, always int64.                        */
 /* ------------------------------------------------------------------------- */
-/* out[n_ids ? n_ids[s] : s] = sum over segment s of data[e_ids ? e_ids[e] : e]^powk */
+/* workspace of gs_segment_sum / gs_segment_normalize; nnz = indptr[num_segments] */
+size_t gs_segment_workspace_bytes(int64_t num_segments, int64_t nnz);
+
+/* out[n_ids ? n_ids[s] : s] = sum over segment s of data[e_ids ? e_ids[e] : e]^powk.
+ * A segment of at most 16 edges is summed in edge order; a longer one in 64-edge pieces
+ * aligned to the edge array (a fixed order, but not the sequential one). */
 int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const void* n_ids, int id_bytes,
-                   const float* data, int64_t num_segments, int64_t powk, float* out,
-                   void* stream);
+                   const float* data, int64_t num_segments, int64_t nnz, int64_t powk, float* out,
+                   void* workspace, size_t workspace_bytes, void* stream);
 
 /* out[target[e]] += data[e_ids ? e_ids[e] : e]^powk  (out pre-zeroed by caller) */
 int gs_coo_sum(const void* target, int id_bytes, const int64_t* e_ids, const float* data, int64_t E,
@@ -396,7 +401,8 @@ int gs_coo_sum(const void* target, int id_bytes, const int64_t* e_ids, const flo
 
 /* out[d] = data[d] / sum of its segment, d = e_ids ? e_ids[e] : e */
 int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const float* data,
-                         int64_t num_segments, float* out, void* stream);
+                         int64_t num_segments, int64_t nnz, float* out, void* workspace,
+                         size_t workspace_bytes, void* stream);
 
 /* out_data[e] = data[e] / divisor[row[e]]; out_sum[col[e]] += out_data[e] */
 int gs_e_div_u_sum(const void* row, const void* col, int id_bytes, const float* data,

@@ -54,9 +54,55 @@ def test_segment_sum_rmat(dev, powk, maps, idt):
     got = _seg_sum(dev, indptr, data, powk, e_ids, n_ids, idt=idt)
     want = O.segment_sum(indptr, e_ids, n_ids, data, powk, indptr.size - 1)
     np.testing.assert_allclose(got, want, rtol=RTOL)
-    short = np.diff(indptr) <= 32  # short segments are summed in edge order: bit exact
+    short = np.diff(indptr) <= 16  # short segments are summed in edge order: bit exact
     idx = np.arange(indptr.size - 1) if n_ids is None else n_ids
     assert np.array_equal(got[idx[short]], want[idx[short]])
+
+
+@pytest.mark.parametrize("case", ["hub_over_chunks", "chunk_aligned", "empties_then_long",
+                                  "one_segment", "short_over_chunk_border"])
+@pytest.mark.parametrize("maps", [False, True])
+def test_segment_sum_pieces_across_chunks(dev, case, maps):
+    # long segments are summed by chunks of 1024 edges of the edge array: segments that start,
+    # cover and end chunks, with short and empty segments around them
+    rng = np.random.default_rng(7)
+    deg = {
+        "hub_over_chunks": [3, 0, 5000, 2, 17, 0, 0, 1030, 16, 2500, 1],
+        "chunk_aligned": [1024, 2048, 1024, 0, 1024],
+        "empties_then_long": [0] * 3000 + [40] + [0] * 2000 + [3000] + [0] * 100,
+        "one_segment": [10000],
+        "short_over_chunk_border": [1020, 8, 1020, 16, 17, 2000],
+    }[case]
+    indptr = np.concatenate([[0], np.cumsum(np.asarray(deg, dtype=np.int64))])
+    nnz, n = int(indptr[-1]), len(deg)
+    data = rng.random(nnz, dtype=np.float32)
+    e_ids = rng.permutation(nnz).astype(np.int64) if maps else None
+    n_ids = rng.permutation(n).astype(np.int64) if maps else None
+    got = _seg_sum(dev, indptr, data, 2, e_ids, n_ids)
+    src = data if e_ids is None else data[e_ids]
+    want = np.zeros(n)
+    for s in range(n):  # float64: the order of the additions is not the sequential one
+        want[s if n_ids is None else n_ids[s]] = np.sum(src[indptr[s]:indptr[s + 1]].astype(np.float64) ** 2)
+    np.testing.assert_allclose(got, want, rtol=RTOL)
+    assert np.array_equal(got, _seg_sum(dev, indptr, data, 2, e_ids, n_ids))  # fixed order
+    # normalize over the same layout
+    out = torch.empty(nnz, dtype=torch.float32, device=dev)
+    capi.segment_normalize(to_dev(indptr, dev), None if e_ids is None else to_dev(e_ids, dev),
+                           to_dev(data + 0.1, dev), out)
+    src = (data + 0.1) if e_ids is None else (data + 0.1)[e_ids]
+    want_n = np.empty(nnz)
+    for s in range(n):
+        seg = src[indptr[s]:indptr[s + 1]].astype(np.float64)
+        pos = np.arange(indptr[s], indptr[s + 1]) if e_ids is None else e_ids[indptr[s]:indptr[s + 1]]
+        want_n[pos] = seg / seg.sum()
+    np.testing.assert_allclose(out.cpu().numpy(), want_n, rtol=RTOL)
+
+
+def test_segment_sum_edge_count_is_an_upper_bound(dev):
+    # the data array may be longer than the offsets cover: the rest is not read into any sum
+    indptr = np.array([0, 2000, 2003], dtype=np.int64)
+    data = np.ones(5000, dtype=np.float32)
+    assert np.array_equal(_seg_sum(dev, indptr, data, 1), np.array([2000, 3], np.float32))
 
 
 def test_segment_sum_mostly_empty(dev):
@@ -64,7 +110,7 @@ def test_segment_sum_mostly_empty(dev):
     n = 300000
     rng = np.random.default_rng(0)
     deg = np.zeros(n, dtype=np.int64)
-    deg[rng.integers(0, n, 4000)] = rng.integers(1, 33, 4000)  # <= 32 edges: summed in edge order
+    deg[rng.integers(0, n, 4000)] = rng.integers(1, 17, 4000)  # <= 16 edges: summed in edge order
     indptr = np.concatenate([[0], np.cumsum(deg)])
     data = rng.random(int(indptr[-1]), dtype=np.float32)
     got = _seg_sum(dev, indptr, data, 2)
