@@ -37,9 +37,12 @@ def __getattr__(name):
     if name in ("Matrix", "HeteroMatrix"):
         from . import matrix_api
         return getattr(matrix_api, name)
-    if name == "ops":
+    if name == "Block":
+        from . import block
+        return block.Block
+    if name in ("ops", "jit"):
         import importlib
-        return importlib.import_module(".ops", __name__)
+        return importlib.import_module("." + name, __name__)
     raise AttributeError(name)
 
 

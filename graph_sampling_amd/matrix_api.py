@@ -2,11 +2,14 @@
 (python/gs/matrix_api/matrix.py:13-119, hetero_matrix.py:6-27), on torch.classes.gs_classes.
 
 Method names, argument order and the format flag each method passes are those of the
-reference; `to_dgl_block` returns the relabel tuple as a small dict because DGL is not a
-dependency of this package.
+reference; `to_dgl_block` returns this package's own `Block` because DGL is not a dependency.
+Methods are written so that `graph_sampling_amd.jit` can trace them: no branch depends on a
+tensor's value.
 """
 import torch
+import torch.fx
 
+from . import block as _block
 from . import load_library
 from .format import _COO, _CSC, _CSR
 
@@ -60,9 +63,9 @@ class Matrix(object):
     def __getitem__(self, data):
         ret = self._graph
         r_slice, c_slice = data[0], data[1]
-        if isinstance(c_slice, torch.Tensor):
+        if isinstance(c_slice, (torch.Tensor, torch.fx.Proxy)):
             ret = ret._CAPI_Slicing(c_slice, 0, _CSC, _COO, False)
-        if isinstance(r_slice, torch.Tensor):
+        if isinstance(r_slice, (torch.Tensor, torch.fx.Proxy)):
             ret = ret._CAPI_Slicing(r_slice, 1, _CSR, _COO, False)
         return Matrix(ret)
 
@@ -95,19 +98,12 @@ class Matrix(object):
         self._graph._CAPI_Relabel()
         return self
 
-    def to_dgl_block(self):
-        """The pieces DGL's create_block would be given (python/gs/matrix_api/matrix.py:41-64)."""
-        frontier, num_src, num_dst, t1, t2, e_ids, fmt = self._graph._CAPI_Relabel()
-        block = {"format": fmt, "num_src": num_src, "num_dst": num_dst, "srcdata_ID": frontier,
-                 "edata_ID": e_ids}
-        if fmt == "coo":
-            block["row"], block["col"] = t1, t2
-        else:
-            block["indptr"], block["indices"] = t1, t2
-        data = self._graph._CAPI_GetData('default')
-        if data is not None:
-            block["edata_w"] = data[e_ids] if e_ids is not None else data
-        return block
+    def to_block(self):
+        """Relabels and returns the `Block` a model consumes (the reference's `to_dgl_block`,
+        python/gs/matrix_api/matrix.py:40-64, without DGL)."""
+        return _block.make_block(self._graph._CAPI_Relabel(), self._graph._CAPI_GetData('default'))
+
+    to_dgl_block = to_block
 
 
 class HeteroMatrix(object):

@@ -418,14 +418,19 @@ def test_graphsage_fused_flow_matches_oracle(dev, algo):
             sp, _, rows, sel = O.sample_uniform(indptr, indices, seeds, fanout, False, seed=1000 + layer,
                                                 with_coo=False, algo=algo)
             frontier, (rel,) = O.relabel([seeds, rows], [rows])
-            assert block["format"] == "csc" and block["num_dst"] == seeds.size
-            assert np.array_equal(block["indptr"].cpu().numpy(), sp)
-            assert np.array_equal(block["indices"].cpu().numpy(), rel)
-            assert np.array_equal(block["srcdata_ID"].cpu().numpy(), frontier)
-            assert block["num_src"] == frontier.size
+            assert block.format == "csc" and block.num_dst_nodes() == seeds.size
+            assert np.array_equal(block.csc()[0].cpu().numpy(), sp)
+            assert np.array_equal(block.csc()[1].cpu().numpy(), rel)
+            assert np.array_equal(block.srcdata["_ID"].cpu().numpy(), frontier)
+            assert np.array_equal(block.dstdata["_ID"].cpu().numpy(), seeds)
+            assert block.num_src_nodes() == frontier.size and block.num_edges() == rel.size
+            assert np.array_equal(block.in_degrees().cpu().numpy(), np.diff(sp))
+            src, dst = block.edges()  # COO view made by the library's CSC -> COO kernel
+            assert np.array_equal(src.cpu().numpy(), rel)
+            assert np.array_equal(dst.cpu().numpy(), np.repeat(np.arange(seeds.size), np.diff(sp)))
             assert np.array_equal(sub.all_indices().cpu().numpy(), frontier)
             assert np.array_equal(sub.row_indices().cpu().numpy(), rows)
-            seeds, d_seeds = frontier, block["srcdata_ID"]
+            seeds, d_seeds = frontier, block.srcdata["_ID"]
     finally:
         torch.ops.gs_ops._CAPI_SetSampleAlgo(0)
 
@@ -444,11 +449,20 @@ def test_graphsage_nonfused_flow_matches_oracle(dev):
     sp2, coo2, si2, sel2 = O.sample_uniform(sp, si, None, 7, False, seed=77)
     block = sampled.to_dgl_block()
     frontier, (rel_col, rel_row) = O.relabel([seeds, si2], [seeds[coo2], si2])
-    assert block["format"] == "coo"
-    assert np.array_equal(block["row"].cpu().numpy(), rel_row)
-    assert np.array_equal(block["col"].cpu().numpy(), rel_col)
-    assert np.array_equal(block["srcdata_ID"].cpu().numpy(), frontier)
+    assert block.format == "coo"
+    assert np.array_equal(block.edges()[0].cpu().numpy(), rel_row)
+    assert np.array_equal(block.edges()[1].cpu().numpy(), rel_col)
+    assert np.array_equal(block.srcdata["_ID"].cpu().numpy(), frontier)
     assert np.array_equal(sampled.get_data().cpu().numpy(), data[sel][sel2])
+    assert np.array_equal(block.edata["w"].cpu().numpy(), data[sel][sel2])
+    # by-destination view and the sparse matrix a model multiplies with: A[dst, src] = sum of w
+    ptr, src, order = block.csc()
+    assert ptr.numel() == seeds.size + 1 and int(ptr[-1]) == rel_row.size
+    dense = np.zeros((seeds.size, frontier.size))
+    np.add.at(dense, (rel_col, rel_row), data[sel][sel2].astype(np.float64))
+    feat = torch.randn(frontier.size, 8, device=dev)
+    np.testing.assert_allclose((block.adj() @ feat).cpu().numpy(),
+                               dense @ feat.cpu().numpy().astype(np.float64), rtol=1e-4, atol=1e-5)
 
 
 def test_weighted_sampling_flow(dev):
@@ -499,9 +513,9 @@ def test_ladies_flow_matches_oracle(dev):
 
     block = subU.to_dgl_block()
     frontier, (rel_col, rel_row) = O.relabel([seeds, h_nodes[s_row]], [seeds[s_col], h_nodes[s_row]])
-    assert np.array_equal(block["srcdata_ID"].cpu().numpy(), frontier)
-    assert np.array_equal(block["row"].cpu().numpy(), rel_row)
-    assert np.array_equal(block["col"].cpu().numpy(), rel_col)
+    assert np.array_equal(block.srcdata["_ID"].cpu().numpy(), frontier)
+    assert np.array_equal(block.edges()[0].cpu().numpy(), rel_row)
+    assert np.array_equal(block.edges()[1].cpu().numpy(), rel_col)
 
 
 def test_fastgcn_coo_row_slicing_flow(dev):
