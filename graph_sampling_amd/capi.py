@@ -291,9 +291,10 @@ class RelabelTable:
                "gs_relabel_table_init")
 
 
-def relabel_sampled(seed_keys, sub_indptr, sub_indices, table, mailbox=None):
+def relabel_sampled(seed_keys, sub_indptr, sub_indices, table, mailbox=None, offsets_copy=None):
     """gs_relabel_sampled behind a sampler whose total is still on the device (sub_indptr[S]).
-    Returns (frontier buffer, num_unique (device), relabelled sampled ids at capacity[, ticket])."""
+    Returns (frontier buffer, num_unique (device), relabelled sampled ids at capacity[, ticket]);
+    `offsets_copy` (int64[S + 1]) receives a copy of sub_indptr."""
     idb = _ids(seed_keys, "seed_keys")
     _ids(sub_indices, "sampled ids", like=seed_keys)
     dev = seed_keys.device
@@ -309,6 +310,7 @@ def relabel_sampled(seed_keys, sub_indptr, sub_indices, table, mailbox=None):
         _ptr(seed_keys), _i64(S), _ptr(sub_indices), _i64(cap),
         ctypes.c_void_p(sub_indptr.data_ptr() + 8 * S), idb, _ptr(table.buf),
         ctypes.c_size_t(table.buf.numel()), _ptr(frontier), _ptr(out_ids), _ptr(num_unique),
+        _ptr(offsets_copy),
         _ptr(ws), ctypes.c_size_t(ws.numel()), _ptr(state), ctypes.c_size_t(state.numel()),
         ctypes.c_uint32(epoch), mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0),
         _i64(ticket), _stream(dev)), "gs_relabel_sampled")

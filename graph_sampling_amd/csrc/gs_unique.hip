@@ -186,8 +186,12 @@ template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
 finish_linked_kernel(T t, const uint32_t* __restrict__ pos, const uint32_t* __restrict__ first,
                      const int64_t* __restrict__ prefix, int64_t S, int64_t M_bound,
-                     const int64_t* __restrict__ sampled_len, IdT* __restrict__ out_ids) {
+                     const int64_t* __restrict__ sampled_len, IdT* __restrict__ out_ids,
+                     int64_t* __restrict__ offsets_copy) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  // the sampler's S + 1 offsets end at sampled_len: a second copy for the caller who hands
+  // the relabelled block out beside the sampled graph (saves a device copy per call)
+  if (offsets_copy && i <= S) offsets_copy[i] = (sampled_len - S)[i];
   int64_t n = *sampled_len;
   if (n < 0) n = 0;
   int64_t M = S + n;
@@ -300,7 +304,8 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
 template <typename IdT>
 int relabel_sampled_impl(const void* seed_keys, int64_t S, const void* sampled, int64_t capacity,
                          const int64_t* sampled_len, void* table, size_t table_bytes,
-                         void* frontier, void* out_ids, int64_t* num_unique, void* workspace,
+                         void* frontier, void* out_ids, int64_t* num_unique,
+                         int64_t* offsets_copy, void* workspace,
                          size_t workspace_bytes, void* state, size_t state_bytes, uint32_t epoch,
                          gs_mailbox* box, int64_t box_ticket, hipStream_t stream) {
   using T = typename TableFor<IdT>::type;
@@ -347,11 +352,12 @@ int relabel_sampled_impl(const void* seed_keys, int64_t S, const void* sampled, 
                        0, stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, lb,
                        box, box_ticket, first);
   }
-  if (M > 0) {
+  if (M > 0 || offsets_copy) {
     ProfileScope prof("unique_finish", stream);
-    hipLaunchKernelGGL((finish_linked_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
-                       0, stream, t, pos, first, prefix, S, M, sampled_len,
-                       static_cast<IdT*>(out_ids));
+    const int64_t threads = offsets_copy && S + 1 > M ? S + 1 : M;
+    hipLaunchKernelGGL((finish_linked_kernel<IdT, T>), dim3(blocks_for(threads, kThreads)),
+                       dim3(kThreads), 0, stream, t, pos, first, prefix, S, M, sampled_len,
+                       static_cast<IdT*>(out_ids), offsets_copy);
   }
   return check_launch("relabel_sampled");
 }
@@ -864,7 +870,8 @@ size_t gs_relabel_sampled_state_bytes(int64_t num_items) {
 
 int gs_relabel_sampled(const void* seed_keys, int64_t S, const void* sampled, int64_t capacity,
                        const int64_t* sampled_len, int id_bytes, void* table, size_t table_bytes,
-                       void* frontier, void* out_ids, int64_t* num_unique, void* workspace,
+                       void* frontier, void* out_ids, int64_t* num_unique,
+                       int64_t* offsets_copy, void* workspace,
                        size_t workspace_bytes, void* state, size_t state_bytes, uint32_t epoch,
                        gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream) {
   GS_REQUIRE(S >= 0 && capacity >= 0 && sampled_len && table && num_unique && state,
@@ -884,12 +891,12 @@ int gs_relabel_sampled(const void* seed_keys, int64_t S, const void* sampled, in
   hipStream_t st = static_cast<hipStream_t>(stream);
   return id_bytes == 8
              ? relabel_sampled_impl<int64_t>(seed_keys, S, sampled, capacity, sampled_len, table,
-                                             table_bytes, frontier, out_ids, num_unique, workspace,
-                                             workspace_bytes, state, state_bytes, epoch, mailbox,
+                                             table_bytes, frontier, out_ids, num_unique, offsets_copy,
+                                             workspace, workspace_bytes, state, state_bytes, epoch, mailbox,
                                              mailbox_ticket, st)
              : relabel_sampled_impl<int32_t>(seed_keys, S, sampled, capacity, sampled_len, table,
-                                             table_bytes, frontier, out_ids, num_unique, workspace,
-                                             workspace_bytes, state, state_bytes, epoch, mailbox,
+                                             table_bytes, frontier, out_ids, num_unique, offsets_copy,
+                                             workspace, workspace_bytes, state, state_bytes, epoch, mailbox,
                                              mailbox_ticket, st);
 }
 

@@ -662,10 +662,9 @@ Graph::Relabel() {
     // straight behind the sampler: its edge count stays on the device until the end
     std::shared_ptr<hip::PendingSample> p = std::move(pending_);
     pending_.reset();
-    torch::Tensor indptr_copy = p->sub_indptr.clone();
-    torch::Tensor relabeled;
+    torch::Tensor indptr_copy, relabeled;  // the copy stands in for indptr.clone()
     int64_t nnz;
-    std::tie(frontier, relabeled, nnz) = hip::RelabelDeferred(col_ids, *p);
+    std::tie(frontier, relabeled, nnz, indptr_copy) = hip::RelabelDeferred(col_ids, *p);
     auto csc = std::make_shared<CSC>();
     csc->indptr = p->sub_indptr;
     csc->indices = p->indices.narrow(0, 0, nnz);

@@ -466,8 +466,8 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> Relabel(
 // Relabel of (column ids, sampled ids) while the sampler's total is still on the
 // device: everything is sized for the sampler's capacity, the kernels read the
 // true length from sub_indptr[S], and both totals are collected at the end.
-std::tuple<torch::Tensor, torch::Tensor, int64_t> RelabelDeferred(const torch::Tensor& col_ids,
-                                                                  const PendingSample& p) {
+std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred(
+    const torch::Tensor& col_ids, const PendingSample& p) {
   const int idb = IdBytes(col_ids, "column ids");
   TORCH_CHECK(IdBytes(p.indices, "sampled ids") == idb, "relabel tensors differ in dtype");
   const int64_t cap = p.indices.numel();
@@ -476,6 +476,7 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t> RelabelDeferred(const torch::T
   auto renamed = torch::empty_like(p.indices);
   auto frontier = torch::empty({M}, col_ids.options());
   auto num = torch::empty({1}, I64(col_ids));
+  auto offsets_copy = torch::empty_like(p.sub_indptr);
   auto ws = Scratch(gs_relabel_sampled_workspace_bytes(M), col_ids);
   RelabelTable& table = RelabelTableFor(col_ids, p.stream, idb, M);
   FusedStateBuf& state = FusedState(gs_relabel_sampled_state_bytes(M), col_ids, p.stream);
@@ -485,8 +486,8 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t> RelabelDeferred(const torch::T
   Check(gs_relabel_sampled(col_ids.data_ptr(), S, p.indices.data_ptr(), cap,
                            p.sub_indptr.data_ptr<int64_t>() + p.S, idb, table.buf.data_ptr(),
                            table.buf.numel(), frontier.data_ptr(), renamed.data_ptr(),
-                           num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(),
-                           state.buf.data_ptr(), state.buf.numel(), state.epoch,
+                           num.data_ptr<int64_t>(), offsets_copy.data_ptr<int64_t>(), ws.data_ptr(),
+                           ws.numel(), state.buf.data_ptr(), state.buf.numel(), state.epoch,
                            boxes.slot(ticket), ticket, p.stream),
         "gs_relabel_sampled");
   const int64_t nnz = p.Wait();
@@ -494,7 +495,7 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t> RelabelDeferred(const torch::T
   if (U == kLost) U = num.item<int64_t>();
   TORCH_CHECK(U >= 0, "gs_relabel_sampled: a tile gave up waiting for its predecessors");
   table.clean = true;
-  return {frontier.narrow(0, 0, U), renamed.narrow(0, 0, nnz), nnz};
+  return {frontier.narrow(0, 0, U), renamed.narrow(0, 0, nnz), nnz, offsets_copy};
 }
 
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(

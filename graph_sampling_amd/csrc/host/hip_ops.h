@@ -62,10 +62,11 @@ std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
                                                    const torch::Tensor& indices,
                                                    const torch::Tensor& column_ids, int64_t fanout,
                                                    bool replace, bool with_coo, bool with_select);
-// {frontier, relabelled sampled ids, number of sampled ids}: unique / relabel of
-// (column ids, sampled ids) queued behind the sampler without reading its total
-std::tuple<torch::Tensor, torch::Tensor, int64_t> RelabelDeferred(const torch::Tensor& col_ids,
-                                                                  const PendingSample& p);
+// {frontier, relabelled sampled ids, number of sampled ids, copy of the sampler's
+// offsets}: unique / relabel of (column ids, sampled ids) queued behind the sampler without
+// reading its total
+std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred(
+    const torch::Tensor& col_ids, const PendingSample& p);
 
 SliceResult ColSamplingProbs(const torch::Tensor& indptr, const torch::Tensor& indices,
                              const torch::Tensor& probs, const torch::Tensor& column_ids,

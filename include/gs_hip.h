@@ -299,6 +299,9 @@ int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_spa
  *     prepare it again.  One call at a time per table.
  *   sampled_len: device address of the true number of sampled ids (sub_indptr + S of the
  *     sampler); `capacity` only bounds it.
+ *   offsets_copy: NULL, or S + 1 slots that receive a copy of the sampler's offsets
+ *     (sampled_len[-S .. 0]): Graph::Relabel returns `indptr.clone()` (src/graph.cc:807),
+ *     and the copy made here costs no launch of its own.
  *   workspace: gs_relabel_sampled_workspace_bytes(S + capacity); state / epoch: as for
  *     gs_sample_uniform_fused, gs_relabel_sampled_state_bytes(S + capacity) bytes (the
  *     sampler's state buffer may be shared when large enough, with a fresh epoch). */
@@ -308,7 +311,8 @@ size_t gs_relabel_sampled_workspace_bytes(int64_t num_items);
 size_t gs_relabel_sampled_state_bytes(int64_t num_items);
 int gs_relabel_sampled(const void* seed_keys, int64_t S, const void* sampled, int64_t capacity,
                        const int64_t* sampled_len, int id_bytes, void* table, size_t table_bytes,
-                       void* frontier, void* out_ids, int64_t* num_unique, void* workspace,
+                       void* frontier, void* out_ids, int64_t* num_unique,
+                       int64_t* offsets_copy, void* workspace,
                        size_t workspace_bytes, void* state, size_t state_bytes, uint32_t epoch,
                        gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
 

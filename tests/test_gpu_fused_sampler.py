@@ -197,7 +197,9 @@ def test_relabel_sampled_matches_the_one_call_relabel(dev, S, fanout, replace, i
     # several calls in a row on the same table: every call leaves it empty
     for seed in (5, 6, 7):
         sp, si, _, _ = capi.sample_uniform_fused(t_ptr, t_idx, t_cols, fanout, replace, seed=seed)
-        frontier, num, out = capi.relabel_sampled(t_keys, sp, si, table)
+        copy = torch.full_like(sp, -7)
+        frontier, num, out = capi.relabel_sampled(t_keys, sp, si, table, offsets_copy=copy)
+        assert torch.equal(copy, sp)  # the sampler's offsets, copied by the last kernel
         w_sp, _, w_si, _ = O.sample_uniform(indptr, indices, cols, fanout, replace, seed=seed, with_coo=False)
         w_frontier, (w_out,) = O.relabel([keys, w_si], [w_si])
         E = int(w_sp[-1])
