@@ -180,6 +180,68 @@ def main():
         lambda: capi.segment_sum(indptr, None, None, weights, 2, out_n),
         lambda o: (E * 4 + N * 20, E, "edges"))
 
+    # ---- whole samplers through the Matrix layer (wall clock, device drained around each) -------
+    import graph_sampling_amd as gs
+    from graph_sampling_amd import jit
+
+    def flow(name, what, fn, units_of, unit_name):
+        if only and name not in only:
+            return
+        for _ in range(3):
+            out = fn()
+        times = []
+        for _ in range(max(args.reps, 10)):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = fn()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        t = times[len(times) // 2]
+        units = units_of(out)
+        print(json.dumps({"op": name, "what": what, "ms": t * 1e3, unit_name: units,
+                          "per_s": units / t}), flush=True)
+
+    A = gs.Matrix().load_csc(indptr, indices, weights)
+
+    def ladies(A, seeds, fanouts):  # the sampler of examples/ladies/ladies_raw.py:8-27
+        ret = []
+        for fanout in fanouts:
+            U = A[:, seeds]
+            prob = U.sum(axis=1, powk=2)
+            selected, _ = torch.ops.gs_ops.list_sampling_with_probs(U.row_ids(unique=False), prob,
+                                                                    fanout, False)
+            nodes = torch.cat((seeds, selected)).unique()
+            subU = U[nodes, :].divide(prob[nodes], axis=1).normalize(axis=0)
+            seeds = subU.all_indices()
+            ret.insert(0, subU.to_dgl_block())
+        return seeds, ret
+
+    def graphsage(A, seeds, fanouts):  # written unfused, as examples/graphsage does before jit
+        ret = []
+        for k in fanouts:
+            sub = A[:, seeds].columnwise_sampling(k, False)
+            seeds = sub.all_indices()
+            ret.insert(0, sub.to_dgl_block())
+        return seeds, ret
+
+    seeds512 = torch.randperm(N, generator=gen, device=dev)[:512].to(idt)
+    seeds1024 = torch.randperm(N, generator=gen, device=dev)[:1024].to(idt)
+    edges_of = lambda o: sum(blk.num_edges() for blk in o[1])
+    flow("flow_ladies", "LADIES, 2 layers of 512 picks from 512 seeds (slice, row sums of w^2 over "
+         "2.45M rows, weighted pick, row slice, divide, normalise, relabel)",
+         lambda: ladies(A, seeds512, [512, 512]), edges_of, "edges")
+    ladies_c = jit.compile(ladies, (A, seeds512, [512, 512]))
+    flow("flow_ladies_compiled", "the same sampler through jit.compile",
+         lambda: ladies_c(A, seeds512, [512, 512]), edges_of, "edges")
+    flow("flow_graphsage_unfused", "GraphSAGE [15,10,5], 1024 seeds, written as slice -> sample -> "
+         "all_indices -> block through the Matrix layer",
+         lambda: graphsage(A, seeds1024, [15, 10, 5]), edges_of, "edges")
+    sage_c = jit.compile(graphsage, (A, seeds1024, [15, 10, 5]))
+    flow("flow_graphsage_compiled", "the same sampler through jit.compile (fused slice+sample, one "
+         "relabel per layer)",
+         lambda: sage_c(A, seeds1024, [15, 10, 5]), edges_of, "edges")
+
 
 if __name__ == "__main__":
     main()

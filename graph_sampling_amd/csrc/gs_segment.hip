@@ -10,17 +10,20 @@
 //    in edge order (bit-identical to a sequential sum).  The typical
 //    layer-wise-sampler call has millions of mostly empty segments
 //    (graph.cc:657: one per graph row): one coalesced pass over the offsets and
-//    one over the output.
-//  * by edge, for everything longer: a wave owns 1024 consecutive edges whatever
-//    segments they belong to, 64 at a time with coalesced loads; a lane finds
-//    the segment of its edge among the offsets the chunk spans, a segmented scan
-//    over the lanes folds the edges of one segment, and a run that is still open
-//    at the end of a step is carried into the next.  A segment that lies inside
-//    the chunk is written at once; the pieces of a segment that crosses chunk
-//    borders go to a carry array and are added up, in chunk order, by the chunk
-//    that holds the segment's head.  A 300 000-edge hub is thus 290 chunks of
-//    work for 290 waves, and the order of the additions is fixed by the layout
-//    alone, so results repeat from run to run.
+//    one over the output.  The same pass enters every longer segment in the list
+//    of the 1024-edge chunk its first edge falls in, and as the "incoming"
+//    segment of every later chunk it reaches into.
+//  * by edge, for the longer ones: a wave owns one chunk of 1024 consecutive
+//    edges.  Its lanes pick up the chunk's segments (at most 61 can start in it,
+//    plus the incoming one), mark where each starts and stops in an LDS array of
+//    one int per edge, and a running "latest mark" over the edges then tells
+//    every edge its owner without any search; a segmented scan folds 64 edges
+//    per step, coalesced.  A segment that lies inside the chunk is written at
+//    once; the pieces of a segment that crosses chunk borders go to a carry
+//    array and are added up, in chunk order, by the chunk that holds its first
+//    edge.  A 300 000-edge hub is 290 chunks of work for 290 waves, millions of
+//    empty segments cost the by-edge pass nothing, and the order of the additions
+//    is fixed by the layout alone, so results repeat from run to run.
 #include "gs_common.hpp"
 
 namespace gs {
@@ -29,7 +32,9 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int64_t kLaneMaxLen = 16;
-constexpr int64_t kChunk = 1024;  // edges per wave in the by-edge pass
+constexpr int64_t kChunk = 1024;   // edges per wave in the by-edge pass
+constexpr int kChunkList = 64;     // list slots per chunk: 1024 / 17 + 1 = 61 segments can start in one
+constexpr int kIncomingLane = kWave - 1;
 
 __device__ __forceinline__ float powk_f(float x, int powk) {
   if (powk == 1) return x;  // graph_ops.cu:30
@@ -38,14 +43,23 @@ __device__ __forceinline__ float powk_f(float x, int powk) {
   return p;
 }
 
-// last g in [lo, hi] with indptr[g] <= e
-__device__ __forceinline__ int64_t segment_of(const int64_t* __restrict__ indptr, int64_t lo,
-                                              int64_t hi, int64_t e) {
-  while (lo < hi) {
-    const int64_t mid = (lo + hi + 1) >> 1;
-    if (indptr[mid] <= e) lo = mid; else hi = mid - 1;
+// Per-chunk bookkeeping of the by-edge pass, all in the caller's workspace.
+struct Chunks {
+  unsigned int* any_long;  // does any segment exceed kLaneMaxLen?
+  unsigned int* count;     // [chunks] long segments starting in the chunk
+  int* list;               // [chunks][kChunkList] their ids
+  int* incoming;           // [chunks] long segment that starts earlier and reaches into the chunk, or -1
+  int* outgoing;           // [chunks] long segment that starts here and goes on after the chunk, or -1
+  float* carry;            // [chunks][2]: piece of the incoming segment, piece of the outgoing one
+};
+
+__global__ void __launch_bounds__(kThreads) clear_chunks_kernel(Chunks ck, int64_t chunks) {
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (c == 0) *ck.any_long = 0u;
+  if (c < chunks) {
+    ck.count[c] = 0u;
+    ck.incoming[c] = -1;
   }
-  return lo;
 }
 
 // ---- by segment: the short ones.  NORMALIZE writes out[d] = data[d] / sum instead.
@@ -53,8 +67,7 @@ template <bool NORMALIZE, typename IdT>
 __global__ void __launch_bounds__(kThreads)
 short_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ emap,
                       const IdT* __restrict__ nmap, const float* __restrict__ data,
-                      int64_t num_seg, int powk, float* __restrict__ out,
-                      unsigned int* __restrict__ any_long) {
+                      int64_t num_seg, int powk, float* __restrict__ out, Chunks ck) {
   const int64_t s = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   int64_t begin = 0, end = 0;
   if (s < num_seg) {
@@ -62,8 +75,29 @@ short_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restr
     end = indptr[s + 1];
   }
   const int64_t len = end - begin;
-  if (__ballot(len > kLaneMaxLen) && (threadIdx.x & (kWave - 1)) == 0) *any_long = 1u;
-  if (s >= num_seg || len > kLaneMaxLen) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const bool is_long = len > kLaneMaxLen;
+  // the long segments of a wave enter their chunks' lists, one atomic per chunk touched
+  unsigned long long todo = __ballot(is_long);
+  if (todo && lane == 0) *ck.any_long = 1u;
+  const int64_t c0 = begin / kChunk;
+  while (todo) {
+    const int64_t c = __shfl(c0, __ffsll(static_cast<long long>(todo)) - 1, kWave);
+    const unsigned long long same = __ballot(is_long && c0 == c);
+    const int leader = __ffsll(static_cast<long long>(same)) - 1;
+    unsigned int base = 0;
+    if (lane == leader) base = atomicAdd(ck.count + c, static_cast<unsigned int>(__popcll(same)));
+    base = __shfl(base, leader, kWave);
+    if (is_long && c0 == c)
+      ck.list[c * kChunkList + base + __popcll(same & ((1ull << lane) - 1ull))] = static_cast<int>(s);
+    todo &= ~same;
+  }
+  if (s >= num_seg) return;
+  if (is_long) {
+    const int64_t c1 = (end - 1) / kChunk;
+    for (int64_t c = c0 + 1; c <= c1; ++c) ck.incoming[c] = static_cast<int>(s);
+    return;
+  }
   float acc = 0.0f;
   for (int64_t e = begin; e < end; ++e) acc += powk_f(data[emap ? emap[e] : e], powk);
   if (NORMALIZE) {
@@ -76,121 +110,128 @@ short_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restr
   }
 }
 
-__global__ void clear_flag_kernel(unsigned int* flag) {
-  if (threadIdx.x == 0) *flag = 0u;
-}
-
 // ---- by edge: the long ones.
-// Which segment owns an edge is found without a search per edge: every segment that starts
-// inside the chunk marks its first edge in an LDS array of one int per edge (empty segments
-// share a position; the highest id wins, which is the one that owns the edge), and a running
-// maximum over the edges then gives each its segment, relative to the segment of the chunk's
-// first edge.
-struct ChunkSpan {
-  int64_t begin, end, g_lo;
+// What a lane knows of the chunk's long segments: lane l < count holds the l-th of the list,
+// the last lane the incoming one.
+struct Owned {
+  int g;           // segment, -1 = none
+  int64_t b, e;    // its edge range
 };
 
-__device__ __forceinline__ ChunkSpan mark_heads(const int64_t* __restrict__ indptr,
-                                                int64_t num_seg, int64_t nnz, int64_t c, int lane,
-                                                int* head) {
-  ChunkSpan span;
-  span.begin = c * kChunk;
-  span.end = span.begin + kChunk < nnz ? span.begin + kChunk : nnz;
-  int64_t edge_g = 0;
-  if (lane < 2) edge_g = segment_of(indptr, 0, num_seg - 1, lane == 0 ? span.begin : span.end - 1);
-  span.g_lo = __shfl(edge_g, 0, kWave);
-  const int64_t g_hi = __shfl(edge_g, 1, kWave);
-  for (int i = lane; i < kChunk; i += kWave) head[i] = 0;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  for (int64_t g = span.g_lo + 1 + lane; g <= g_hi; g += kWave)
-    atomicMax(&head[indptr[g] - span.begin], static_cast<int>(g - span.g_lo));
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  return span;
+__device__ __forceinline__ Owned load_owned(const int64_t* __restrict__ indptr, const Chunks& ck,
+                                            int64_t c, int lane) {
+  Owned o;
+  o.g = -1;
+  o.b = o.e = 0;
+  const int n = static_cast<int>(ck.count[c]);
+  if (lane < n) o.g = ck.list[c * kChunkList + lane];
+  if (lane == kIncomingLane) o.g = ck.incoming[c];
+  if (o.g >= 0) {
+    o.b = indptr[o.g];
+    o.e = indptr[o.g + 1];
+  }
+  return o;
 }
 
-// segment (relative to g_lo) of the edge at offset `at` of the chunk; carried = the last
-// lane's answer of the step before
-__device__ __forceinline__ int owner_of(const int* head, int at, bool live, int carried, int lane) {
-  int g = live ? head[at] : 0;
+// mark[p] = lane + 2 where the lane's segment starts (or the chunk does, for the incoming
+// one), 1 where a segment stops and no other starts, 0 elsewhere
+__device__ __forceinline__ void write_marks(int* mark, const Owned& o, int64_t begin, int64_t end,
+                                            int lane) {
+  for (int i = lane; i < kChunk; i += kWave) mark[i] = 0;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  if (o.g >= 0) {
+    atomicMax(&mark[(o.b > begin ? o.b : begin) - begin], lane + 2);
+    if (o.e < end) atomicMax(&mark[o.e - begin], 1);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// The latest mark at or before each edge of a 64-edge step, as (position + 1) << 8 | mark, so
+// that a maximum over the lanes is "the latest"; carried = the last lane's answer of the step
+// before.  Equal values = same run of edges.
+__device__ __forceinline__ int latest_mark(const int* mark, int at, bool live, int carried,
+                                           int lane) {
+  const int m = live ? mark[at] : 0;
+  int packed = m ? ((at + 1) << 8 | m) : 0;
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
-    const int y = __shfl_up(g, d, kWave);
-    if (lane >= d && y > g) g = y;
+    const int y = __shfl_up(packed, d, kWave);
+    if (lane >= d && y > packed) packed = y;
   }
-  return g > carried ? g : carried;
+  return packed > carried ? packed : carried;
 }
 
-// sums is indexed by segment (nmap applied when given); carry holds two floats per chunk:
-// [2c] the piece of a segment that began before chunk c, [2c+1] the piece of a segment that
-// begins in chunk c and goes on after it.
+// sums is indexed by segment (nmap applied when given)
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ emap,
                      const IdT* __restrict__ nmap, const float* __restrict__ data,
-                     int64_t num_seg, int64_t nnz, int powk, float* __restrict__ sums,
-                     float* __restrict__ carry, const unsigned int* __restrict__ any_long) {
-  __shared__ int s_head[kWaves][kChunk];
-  if (*any_long == 0u) return;
+                     int64_t num_seg, int64_t nnz, int powk, float* __restrict__ sums, Chunks ck) {
+  __shared__ int s_mark[kWaves][kChunk];
+  if (*ck.any_long == 0u) return;
   if (indptr[num_seg] < nnz) nnz = indptr[num_seg];  // the caller's count is an upper bound
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t c = static_cast<int64_t>(blockIdx.x) * kWaves + threadIdx.x / kWave;
-  if (c * kChunk >= nnz) return;
-  int* head = s_head[threadIdx.x / kWave];
-  const ChunkSpan span = mark_heads(indptr, num_seg, nnz, c, lane, head);
-  const int64_t begin = span.begin, end = span.end;
-  int g_carried = 0;     // segment of the last edge of the step before
-  bool open = false;     // that segment's run goes on into this step
+  const int64_t begin = c * kChunk;
+  if (begin >= nnz) return;
+  const int64_t end = begin + kChunk < nnz ? begin + kChunk : nnz;
+  int* mark = s_mark[threadIdx.x / kWave];
+  const Owned own = load_owned(indptr, ck, c, lane);
+  write_marks(mark, own, begin, end, lane);
+  int carried = 0;       // latest mark at the end of the step before
+  bool open = false;     // a long segment's run was cut by the end of that step
   float acc_open = 0.0f;
+  int out_g = -1;        // long segment that starts here and goes on after the chunk
   float v = begin + lane < end ? powk_f(data[emap ? emap[begin + lane] : begin + lane], powk) : 0.0f;
   for (int64_t base = begin; base < end; base += kWave) {
     const int64_t e = base + lane;
     const bool live = e < end;
     const int64_t en = e + kWave;
     const float v_next = en < end ? powk_f(data[emap ? emap[en] : en], powk) : 0.0f;
-    const int g_any = owner_of(head, static_cast<int>(e - begin), live, g_carried, lane);
-    const int g = live ? g_any : -1;
-    float x = v;
+    const int latest = latest_mark(mark, static_cast<int>(e - begin), live, carried, lane);
+    const int run = live ? latest : -1;
+    const int owner = (latest & 0xFF) - 2;  // the lane that holds the edge's segment; < 0: a short one's
+    float x = live && owner >= 0 ? v : 0.0f;
 #pragma unroll
     for (int d = 1; d < kWave; d <<= 1) {
       const float y = __shfl_up(x, d, kWave);
-      const int gy = __shfl_up(g, d, kWave);
-      if (lane >= d && gy == g) x += y;
+      const int ry = __shfl_up(run, d, kWave);
+      if (lane >= d && ry == run) x += y;
     }
-    const int g_next = __shfl_down(g, 1, kWave);
-    const bool run_end = live && (lane == kWave - 1 || g_next != g);
-    if (run_end && open && g == g_carried) x += acc_open;  // only the first run can match
-    bool closed = false, is_long = false, began_here = false;
-    if (run_end) {
-      const int64_t seg_b = indptr[span.g_lo + g], seg_e = indptr[span.g_lo + g + 1];
-      closed = e == seg_e - 1;
-      is_long = seg_e - seg_b > kLaneMaxLen;
-      began_here = seg_b >= begin;
-      if (closed && is_long) {
-        if (began_here) {
-          const int64_t gg = span.g_lo + g;
-          sums[nmap ? static_cast<int64_t>(nmap[gg]) : gg] = x;
-        } else {
-          carry[2 * c] = x;
-        }
-      }
+    const int run_next = __shfl_down(run, 1, kWave);
+    const bool run_end = live && owner >= 0 && (lane == kWave - 1 || run_next != run);
+    if (run_end && open && run == carried) x += acc_open;  // only the first run of a step can match
+    const int src = owner >= 0 ? owner : 0;
+    const int64_t seg_b = __shfl(own.b, src, kWave);
+    const int64_t seg_e = __shfl(own.e, src, kWave);
+    const int seg_g = __shfl(own.g, src, kWave);
+    const bool closed = run_end && e == seg_e - 1;
+    const bool began_here = seg_b >= begin;
+    if (closed) {
+      if (began_here)
+        sums[nmap ? static_cast<int64_t>(nmap[seg_g]) : seg_g] = x;
+      else
+        ck.carry[2 * c] = x;
     }
     // at most one run is cut by the end of the step: the last live lane's
     const unsigned long long cut = __ballot(run_end && !closed);
-    g_carried = __shfl(g_any, kWave - 1, kWave);  // unused lanes repeat the last edge's
+    carried = __shfl(latest, kWave - 1, kWave);  // unused lanes repeat the last edge's
     open = cut != 0;
     if (open) {
-      const int src = __ffsll(static_cast<long long>(cut)) - 1;
-      acc_open = __shfl(x, src, kWave);
+      const int at = __ffsll(static_cast<long long>(cut)) - 1;
+      acc_open = __shfl(x, at, kWave);
       if (base + kWave >= end) {  // cut by the end of the chunk: hand the piece on
-        const int longs = __shfl(static_cast<int>(is_long), src, kWave);
-        const int here = __shfl(static_cast<int>(began_here), src, kWave);
-        if (longs && lane == 0) carry[here ? 2 * c + 1 : 2 * c] = acc_open;
+        const int here = __shfl(static_cast<int>(began_here), at, kWave);
+        const int g = __shfl(seg_g, at, kWave);
+        if (lane == 0) ck.carry[here ? 2 * c + 1 : 2 * c] = acc_open;
+        if (here) out_g = g;
       }
     }
     v = v_next;
   }
+  if (lane == 0) ck.outgoing[c] = out_g;
 }
 
 // one lane per chunk: a chunk that holds the head of a long segment going on after it adds
@@ -198,19 +239,16 @@ long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restri
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 carry_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ nmap, int64_t num_seg,
-             int64_t nnz, const float* __restrict__ carry, float* __restrict__ sums,
-             const unsigned int* __restrict__ any_long) {
-  if (*any_long == 0u) return;
-  if (indptr[num_seg] < nnz) nnz = indptr[num_seg];  // the caller's count is an upper bound
+             int64_t nnz, float* __restrict__ sums, Chunks ck) {
+  if (*ck.any_long == 0u) return;
+  if (indptr[num_seg] < nnz) nnz = indptr[num_seg];
   const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  const int64_t begin = c * kChunk;
-  if (begin >= nnz) return;
-  const int64_t end = begin + kChunk < nnz ? begin + kChunk : nnz;
-  const int64_t g = segment_of(indptr, 0, num_seg - 1, end - 1);
-  const int64_t seg_b = indptr[g], seg_e = indptr[g + 1];
-  if (seg_e <= end || seg_b < begin || seg_e - seg_b <= kLaneMaxLen) return;
-  float total = carry[2 * c + 1];
-  for (int64_t k = c + 1; k * kChunk < seg_e; ++k) total += carry[2 * k];
+  if (c * kChunk >= nnz) return;
+  const int g = ck.outgoing[c];
+  if (g < 0) return;
+  const int64_t seg_e = indptr[g + 1];
+  float total = ck.carry[2 * c + 1];
+  for (int64_t k = c + 1; k * kChunk < seg_e; ++k) total += ck.carry[2 * k];
   sums[nmap ? static_cast<int64_t>(nmap[g]) : g] = total;
 }
 
@@ -218,50 +256,62 @@ carry_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ nmap, i
 __global__ void __launch_bounds__(kThreads)
 long_divide_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ emap,
                    const float* __restrict__ data, int64_t num_seg, int64_t nnz,
-                   const float* __restrict__ sums, float* __restrict__ out,
-                   const unsigned int* __restrict__ any_long) {
-  __shared__ int s_head[kWaves][kChunk];
-  if (*any_long == 0u) return;
-  if (indptr[num_seg] < nnz) nnz = indptr[num_seg];  // the caller's count is an upper bound
+                   const float* __restrict__ sums, float* __restrict__ out, Chunks ck) {
+  __shared__ int s_mark[kWaves][kChunk];
+  if (*ck.any_long == 0u) return;
+  if (indptr[num_seg] < nnz) nnz = indptr[num_seg];
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t c = static_cast<int64_t>(blockIdx.x) * kWaves + threadIdx.x / kWave;
-  if (c * kChunk >= nnz) return;
-  int* head = s_head[threadIdx.x / kWave];
-  const ChunkSpan span = mark_heads(indptr, num_seg, nnz, c, lane, head);
-  int g_carried = 0;
-  for (int64_t base = span.begin; base < span.end; base += kWave) {
+  const int64_t begin = c * kChunk;
+  if (begin >= nnz) return;
+  const int64_t end = begin + kChunk < nnz ? begin + kChunk : nnz;
+  int* mark = s_mark[threadIdx.x / kWave];
+  const Owned own = load_owned(indptr, ck, c, lane);
+  write_marks(mark, own, begin, end, lane);
+  const float own_sum = own.g >= 0 ? sums[own.g] : 0.0f;
+  int carried = 0;
+  for (int64_t base = begin; base < end; base += kWave) {
     const int64_t e = base + lane;
-    const bool live = e < span.end;
-    const int g = owner_of(head, static_cast<int>(e - span.begin), live, g_carried, lane);
-    g_carried = __shfl(g, kWave - 1, kWave);
-    if (live) {
-      const int64_t gg = span.g_lo + g;
-      if (indptr[gg + 1] - indptr[gg] > kLaneMaxLen) {
-        const int64_t d = emap ? emap[e] : e;
-        out[d] = data[d] / sums[gg];
-      }
+    const bool live = e < end;
+    const int latest = latest_mark(mark, static_cast<int>(e - begin), live, carried, lane);
+    carried = __shfl(latest, kWave - 1, kWave);
+    const int owner = (latest & 0xFF) - 2;
+    const float total = __shfl(own_sum, owner >= 0 ? owner : 0, kWave);
+    if (live && owner >= 0) {
+      const int64_t d = emap ? emap[e] : e;
+      out[d] = data[d] / total;
     }
   }
 }
 
+inline int64_t num_chunks(int64_t nnz) { return nnz <= 0 ? 1 : (nnz + kChunk - 1) / kChunk; }
+
 struct SegmentScratch {
-  unsigned int* any_long;
-  float* carry;
+  Chunks ck;
   float* sums;  // normalize only
   bool ok;
 };
 
-inline int64_t num_chunks(int64_t nnz) { return nnz <= 0 ? 1 : (nnz + kChunk - 1) / kChunk; }
-
 SegmentScratch carve_segment(void* workspace, size_t bytes, int64_t nnz, int64_t num_seg,
                              bool with_sums) {
   Carver ws(workspace, bytes);
+  const int64_t chunks = num_chunks(nnz);
   SegmentScratch s;
-  s.any_long = ws.take<unsigned int>(64);
-  s.carry = ws.take<float>(2 * num_chunks(nnz));
+  s.ck.any_long = ws.take<unsigned int>(64);
+  s.ck.count = ws.take<unsigned int>(chunks);
+  s.ck.list = ws.take<int>(chunks * kChunkList);
+  s.ck.incoming = ws.take<int>(chunks);
+  s.ck.outgoing = ws.take<int>(chunks);
+  s.ck.carry = ws.take<float>(2 * chunks);
   s.sums = with_sums ? ws.take<float>(num_seg > 0 ? num_seg : 1) : nullptr;
   s.ok = ws.ok;
   return s;
+}
+
+size_t segment_workspace_bytes(int64_t num_seg, int64_t nnz) {
+  const size_t chunks = static_cast<size_t>(num_chunks(nnz));
+  return padded(256) + 3 * padded(chunks * 4) + padded(chunks * kChunkList * 4) +
+         padded(chunks * 8) + padded(static_cast<size_t>(num_seg > 0 ? num_seg : 1) * 4);
 }
 
 template <typename IdT>
@@ -269,15 +319,16 @@ int segment_sum_impl(const int64_t* indptr, const int64_t* emap, const void* nma
                      const float* data, int64_t num_seg, int64_t nnz, int powk, float* out,
                      const SegmentScratch& s, hipStream_t st) {
   const IdT* nm = static_cast<const IdT*>(nmap);
-  hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(64), 0, st, s.any_long);
+  const int64_t chunks = num_chunks(nnz);
+  hipLaunchKernelGGL(clear_chunks_kernel, dim3(blocks_for(chunks, kThreads)), dim3(kThreads), 0, st,
+                     s.ck, chunks);
   hipLaunchKernelGGL((short_segments_kernel<false, IdT>), dim3(blocks_for(num_seg, kThreads)),
-                     dim3(kThreads), 0, st, indptr, emap, nm, data, num_seg, powk, out, s.any_long);
+                     dim3(kThreads), 0, st, indptr, emap, nm, data, num_seg, powk, out, s.ck);
   if (nnz > kLaneMaxLen) {
-    const int64_t chunks = num_chunks(nnz);
     hipLaunchKernelGGL(long_segments_kernel<IdT>, dim3(blocks_for(chunks, kWaves)), dim3(kThreads),
-                       0, st, indptr, emap, nm, data, num_seg, nnz, powk, out, s.carry, s.any_long);
+                       0, st, indptr, emap, nm, data, num_seg, nnz, powk, out, s.ck);
     hipLaunchKernelGGL(carry_kernel<IdT>, dim3(blocks_for(chunks, kThreads)), dim3(kThreads), 0, st,
-                       indptr, nm, num_seg, nnz, s.carry, out, s.any_long);
+                       indptr, nm, num_seg, nnz, out, s.ck);
   }
   return check_launch("segment_sum");
 }
@@ -313,9 +364,7 @@ using namespace gs;
 extern "C" {
 
 size_t gs_segment_workspace_bytes(int64_t num_segments, int64_t nnz) {
-  if (num_segments < 1) num_segments = 1;
-  return padded(256) + padded(static_cast<size_t>(2 * num_chunks(nnz)) * 4) +
-         padded(static_cast<size_t>(num_segments) * 4);
+  return segment_workspace_bytes(num_segments, nnz);
 }
 
 int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const void* n_ids, int id_bytes,
@@ -327,6 +376,7 @@ int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const void* n_id
              "gs_segment_sum: null pointer");
   GS_REQUIRE(!n_ids || valid_id_bytes(id_bytes), "gs_segment_sum: id_bytes must be 4 or 8, got %d",
              id_bytes);
+  GS_REQUIRE(num_segments < (int64_t(1) << 31), "gs_segment_sum: more than 2^31 segments");
   if (num_segments == 0) return GS_OK;
   SegmentScratch s = carve_segment(workspace, workspace_bytes, nnz, num_segments, false);
   if (!s.ok) {
@@ -364,7 +414,8 @@ int gs_coo_sum(const void* target, int id_bytes, const int64_t* e_ids, const flo
 int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const float* data,
                          int64_t num_segments, int64_t nnz, float* out, void* workspace,
                          size_t workspace_bytes, void* stream) {
-  GS_REQUIRE(num_segments >= 0 && nnz >= 0, "gs_segment_normalize: negative size");
+  GS_REQUIRE(num_segments >= 0 && nnz >= 0 && num_segments < (int64_t(1) << 31),
+             "gs_segment_normalize: negative size or more than 2^31 segments");
   GS_REQUIRE(num_segments == 0 || nnz == 0 || (indptr && data && out),
              "gs_segment_normalize: null pointer");
   if (num_segments == 0 || nnz == 0) return GS_OK;
@@ -376,19 +427,19 @@ int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const floa
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t* no_map = nullptr;
-  hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(64), 0, st, s.any_long);
+  const int64_t chunks = num_chunks(nnz);
+  hipLaunchKernelGGL(clear_chunks_kernel, dim3(blocks_for(chunks, kThreads)), dim3(kThreads), 0, st,
+                     s.ck, chunks);
   hipLaunchKernelGGL((short_segments_kernel<true, int64_t>), dim3(blocks_for(num_segments, kThreads)),
-                     dim3(kThreads), 0, st, indptr, e_ids, no_map, data, num_segments, 1, out,
-                     s.any_long);
+                     dim3(kThreads), 0, st, indptr, e_ids, no_map, data, num_segments, 1, out, s.ck);
   if (nnz > kLaneMaxLen) {
-    const int64_t chunks = num_chunks(nnz);
     hipLaunchKernelGGL(long_segments_kernel<int64_t>, dim3(blocks_for(chunks, kWaves)),
                        dim3(kThreads), 0, st, indptr, e_ids, no_map, data, num_segments, nnz, 1,
-                       s.sums, s.carry, s.any_long);
+                       s.sums, s.ck);
     hipLaunchKernelGGL(carry_kernel<int64_t>, dim3(blocks_for(chunks, kThreads)), dim3(kThreads), 0,
-                       st, indptr, no_map, num_segments, nnz, s.carry, s.sums, s.any_long);
+                       st, indptr, no_map, num_segments, nnz, s.sums, s.ck);
     hipLaunchKernelGGL(long_divide_kernel, dim3(blocks_for(chunks, kWaves)), dim3(kThreads), 0, st,
-                       indptr, e_ids, data, num_segments, nnz, s.sums, out, s.any_long);
+                       indptr, e_ids, data, num_segments, nnz, s.sums, out, s.ck);
   }
   return check_launch("segment_normalize");
 }
