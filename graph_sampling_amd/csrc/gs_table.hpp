@@ -24,10 +24,20 @@ struct PackedTable {
   void carve(Carver& ws, int64_t cap) { slots = ws.take<unsigned long long>(cap); }
   __device__ __forceinline__ void clear(int64_t i) const { slots[i] = ~0ull; }
   // returns the slot of `key` after recording index i as a candidate first occurrence
+  // PEEK reads the slot first and leaves the compare-and-swap out when it is taken: worth a
+  // load when keys repeat a lot (90 k edge ends over 1000 nodes queue up on the same words
+  // otherwise), a loss when most keys are new.  A stale read is harmless: a slot only goes
+  // from empty to a key, and its index only goes down.
+  template <bool PEEK = false>
   __device__ __forceinline__ uint32_t insert(long long key, uint32_t i) const {
     uint32_t p = home(key);
-    while (!landed(key, i, p, probe(key, i, p))) p = (p + 1) & mask;
-    return p;
+    while (true) {
+      unsigned long long prev = ~0ull;
+      if (PEEK) prev = __hip_atomic_load(&slots[p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (prev == ~0ull) prev = probe(key, i, p);
+      if (landed(key, i, p, prev)) return p;
+      p = (p + 1) & mask;
+    }
   }
   // The insert in its two halves: probe issues the compare-and-swap on slot p and returns what the slot held; landed
   // acts on that: true when p is the key's slot (an index already there is lowered when
@@ -80,10 +90,18 @@ struct WideTable {
     vals[i] = 0x7fffffff;
   }
   // (unique_reindex.cu:13-26 RelabelHashmap::Update)
+  template <bool PEEK = false>
   __device__ __forceinline__ uint32_t insert(long long key, uint32_t i) const {
     uint32_t p = home(key);
-    while (!landed(key, i, p, probe(key, i, p))) p = (p + 1) & mask;
-    return p;
+    while (true) {
+      unsigned long long prev = ~0ull;
+      if (PEEK)
+        prev = __hip_atomic_load(reinterpret_cast<unsigned long long*>(&keys[p]), __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+      if (prev == ~0ull) prev = probe(key, i, p);
+      if (landed(key, i, p, prev)) return p;
+      p = (p + 1) & mask;
+    }
   }
   __device__ __forceinline__ uint32_t home(long long key) const {
     return fib_home(static_cast<uint64_t>(key), shift);

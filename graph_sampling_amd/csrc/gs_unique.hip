@@ -71,12 +71,12 @@ __global__ void __launch_bounds__(kThreads) table_init_kernel(T t, int64_t cap, 
 
 // insert (key -> min index) and remember the slot of every item
 // (unique_reindex.cu:92-99)
-template <typename IdT, typename T>
+template <typename IdT, typename T, bool PEEK>
 __global__ void __launch_bounds__(kThreads)
 table_insert_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ pos) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= x.items(M_bound)) return;
-  pos[i] = t.insert(static_cast<long long>(x.get(i)), static_cast<uint32_t>(i));
+  pos[i] = t.template insert<PEEK>(static_cast<long long>(x.get(i)), static_cast<uint32_t>(i));
 }
 
 struct Query {
@@ -283,8 +283,8 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   }
   if (M > 0) {
     ProfileScope prof("table_insert", stream);
-    hipLaunchKernelGGL((table_insert_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
-                       0, stream, x, M, t, pos);
+    hipLaunchKernelGGL((table_insert_kernel<IdT, T, true>), dim3(blocks_for(M, kThreads)),
+                       dim3(kThreads), 0, stream, x, M, t, pos);
   }
   {
     ProfileScope prof("unique_compact", stream);
@@ -343,8 +343,10 @@ int relabel_sampled_impl(const void* seed_keys, int64_t S, const void* sampled, 
   x.fixed = S;
   if (M > 0) {
     ProfileScope prof("table_insert", stream);
-    hipLaunchKernelGGL((table_insert_kernel<IdT, T>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
-                       0, stream, x, M, t, pos);
+    // no peek here: sampled neighbours are mostly new keys, and the extra read costs the
+    // GraphSAGE step 7 % (0.152 ms against 0.142)
+    hipLaunchKernelGGL((table_insert_kernel<IdT, T, false>), dim3(blocks_for(M, kThreads)),
+                       dim3(kThreads), 0, stream, x, M, t, pos);
   }
   {
     ProfileScope prof("unique_compact", stream);
