@@ -75,8 +75,12 @@ template <typename IdT, typename T, bool PEEK>
 __global__ void __launch_bounds__(kThreads)
 table_insert_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ pos) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= M_bound) return;
+  // the key is read before the device-side length is known (the buffers hold M_bound items
+  // whatever the length turns out to be): one round trip instead of two
+  const IdT key = x.get(i);
   if (i >= x.items(M_bound)) return;
-  pos[i] = t.template insert<PEEK>(static_cast<long long>(x.get(i)), static_cast<uint32_t>(i));
+  pos[i] = t.template insert<PEEK>(static_cast<long long>(key), static_cast<uint32_t>(i));
 }
 
 struct Query {
@@ -112,7 +116,9 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) {
     const int64_t i = base + k;
-    const uint32_t fi = i < M ? t.first_index(pos[i]) : 0u;
+    // read under the host's bound, not the device-side length, so that the reads do not wait
+    // for it; a slot number beyond the length is whatever the workspace held: masked
+    const uint32_t fi = i < M_bound ? t.first_index(pos[i] & t.mask) : 0u;
     first[k] = i < M && fi == static_cast<uint32_t>(i);
     mine += first[k] ? 1 : 0;
     // kept for a last pass that must not read the table any more (it empties it)
@@ -192,13 +198,17 @@ finish_linked_kernel(T t, const uint32_t* __restrict__ pos, const uint32_t* __re
   // the sampler's S + 1 offsets end at sampled_len: a second copy for the caller who hands
   // the relabelled block out beside the sampled graph (saves a device copy per call)
   if (offsets_copy && i <= S) offsets_copy[i] = (sampled_len - S)[i];
+  // reads go by the host's bound so that they do not wait for the device-side length
+  const uint32_t f = i < M_bound ? first[i] : 0u;
+  const int64_t rank = prefix[f < M_bound ? f : 0u];
+  const uint32_t p = i < M_bound ? pos[i] : 0u;
   int64_t n = *sampled_len;
   if (n < 0) n = 0;
   int64_t M = S + n;
   if (M > M_bound) M = M_bound;
   if (i >= M) return;
-  if (i >= S) out_ids[i - S] = static_cast<IdT>(prefix[first[i]]);
-  t.clear(pos[i]);
+  if (i >= S) out_ids[i - S] = static_cast<IdT>(rank);
+  t.clear(p);
 }
 
 template <typename T>
