@@ -136,11 +136,11 @@ __device__ __forceinline__ Owned load_owned(const int64_t* __restrict__ indptr, 
 // mark[p] = lane + 2 where the lane's segment starts (or the chunk does, for the incoming
 // one), 1 where a segment stops and no other starts, 0 elsewhere
 __device__ __forceinline__ void write_marks(int* mark, const Owned& o, int64_t begin, int64_t end,
-                                            int lane) {
+                                            int lane, bool skip = false) {
   for (int i = lane; i < kChunk; i += kWave) mark[i] = 0;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
-  if (o.g >= 0) {
+  if (o.g >= 0 && !skip) {
     atomicMax(&mark[(o.b > begin ? o.b : begin) - begin], lane + 2);
     if (o.e < end) atomicMax(&mark[o.e - begin], 1);
   }
@@ -148,13 +148,38 @@ __device__ __forceinline__ void write_marks(int* mark, const Owned& o, int64_t b
   __builtin_amdgcn_wave_barrier();
 }
 
-// The latest mark at or before each edge of a 64-edge step, as (position + 1) << 8 | mark, so
-// that a maximum over the lanes is "the latest"; carried = the last lane's answer of the step
-// before.  Equal values = same run of edges.
-__device__ __forceinline__ int latest_mark(const int* mark, int at, bool live, int carried,
-                                           int lane) {
-  const int m = live ? mark[at] : 0;
-  int packed = m ? ((at + 1) << 8 | m) : 0;
+// A step is 256 edges, four consecutive ones per lane (one 16-byte read of the marks, one of
+// the data).  A long segment has at least 17 edges, so inside a lane's four at most one long
+// run ends (at the lane's first mark) and at most one begins (at its last mark); what lies
+// between belongs to short segments.  Lanes therefore exchange one value each: the cross-lane
+// work per edge is a quarter of a lane-per-edge scan's.
+constexpr int kLaneEdges = 4;
+constexpr int kStep = kWave * kLaneEdges;
+
+struct LaneMarks {
+  int first_k, last_k;  // first and last marked edge among the lane's four, -1 = none
+  int last_packed;      // (position + 1) << 8 | mark of the last one, 0 = none
+};
+
+__device__ __forceinline__ LaneMarks scan_lane_marks(const int (&m)[kLaneEdges], int at0) {
+  LaneMarks lm;
+  lm.first_k = lm.last_k = -1;
+  lm.last_packed = 0;
+#pragma unroll
+  for (int k = 0; k < kLaneEdges; ++k) {
+    if (m[k]) {
+      if (lm.first_k < 0) lm.first_k = k;
+      lm.last_k = k;
+      lm.last_packed = (at0 + k + 1) << 8 | m[k];
+    }
+  }
+  return lm;
+}
+
+// latest mark at or before the end of each lane (inclusive) given the lanes' own last marks;
+// positions grow with the lane, so a maximum is "the latest"
+__device__ __forceinline__ int latest_inclusive(int last_packed, int carried, int lane) {
+  int packed = last_packed;
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
     const int y = __shfl_up(packed, d, kWave);
@@ -163,13 +188,15 @@ __device__ __forceinline__ int latest_mark(const int* mark, int at, bool live, i
   return packed > carried ? packed : carried;
 }
 
+__device__ __forceinline__ int owner_of_mark(int packed) { return (packed & 0xFF) - 2; }
+
 // sums is indexed by segment (nmap applied when given)
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ emap,
                      const IdT* __restrict__ nmap, const float* __restrict__ data,
                      int64_t num_seg, int64_t nnz, int powk, float* __restrict__ sums, Chunks ck) {
-  __shared__ int s_mark[kWaves][kChunk];
+  __shared__ __attribute__((aligned(16))) int s_mark[kWaves][kChunk];
   if (*ck.any_long == 0u) return;
   if (indptr[num_seg] < nnz) nnz = indptr[num_seg];  // the caller's count is an upper bound
   const int lane = threadIdx.x & (kWave - 1);
@@ -179,57 +206,95 @@ long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restri
   const int64_t end = begin + kChunk < nnz ? begin + kChunk : nnz;
   int* mark = s_mark[threadIdx.x / kWave];
   const Owned own = load_owned(indptr, ck, c, lane);
-  write_marks(mark, own, begin, end, lane);
+  // An incoming segment of which fewer than four edges are left would start and stop inside
+  // the first lane, the one case of a run that does not reach beyond a lane: it gets no marks
+  // and lane 0 adds it up by itself.
+  const int64_t in_left = __shfl(own.g >= 0 ? own.e - begin : int64_t(0), kIncomingLane, kWave);
+  const int tiny = in_left < kLaneEdges ? static_cast<int>(in_left) : 0;
+  write_marks(mark, own, begin, end, lane, tiny > 0 && lane == kIncomingLane);
   int carried = 0;       // latest mark at the end of the step before
-  bool open = false;     // a long segment's run was cut by the end of that step
+  bool open = false;     // that mark's segment is a long one: its run goes on
   float acc_open = 0.0f;
-  int out_g = -1;        // long segment that starts here and goes on after the chunk
-  float v = begin + lane < end ? powk_f(data[emap ? emap[begin + lane] : begin + lane], powk) : 0.0f;
-  for (int64_t base = begin; base < end; base += kWave) {
-    const int64_t e = base + lane;
-    const bool live = e < end;
-    const int64_t en = e + kWave;
-    const float v_next = en < end ? powk_f(data[emap ? emap[en] : en], powk) : 0.0f;
-    const int latest = latest_mark(mark, static_cast<int>(e - begin), live, carried, lane);
-    const int run = live ? latest : -1;
-    const int owner = (latest & 0xFF) - 2;  // the lane that holds the edge's segment; < 0: a short one's
-    float x = live && owner >= 0 ? v : 0.0f;
+  for (int64_t base = begin; base < end; base += kStep) {
+    const int at0 = static_cast<int>(base - begin) + lane * kLaneEdges;
+    const int64_t e0 = base + lane * kLaneEdges;
+    int m[kLaneEdges];
+    float v[kLaneEdges];
+    {
+      const int4 mm = *reinterpret_cast<const int4*>(mark + at0);
+      m[0] = mm.x; m[1] = mm.y; m[2] = mm.z; m[3] = mm.w;
+    }
+#pragma unroll
+    for (int k = 0; k < kLaneEdges; ++k) {
+      const int64_t e = e0 + k;
+      if (e >= end) m[k] = 0;
+      v[k] = e < end ? powk_f(data[emap ? emap[e] : e], powk) : 0.0f;
+    }
+    if (tiny > 0 && base == begin && lane == 0) {
+      float piece = 0.0f;
+#pragma unroll
+      for (int k = 0; k < kLaneEdges - 1; ++k)
+        if (k < tiny) piece += v[k];
+      ck.carry[2 * c] = piece;
+    }
+    const LaneMarks lm = scan_lane_marks(m, at0);
+    const bool has_mark = lm.first_k >= 0;
+    float pre = 0.0f, post = 0.0f;  // edges before the first mark; from the last mark on
+#pragma unroll
+    for (int k = 0; k < kLaneEdges; ++k) {
+      if (!has_mark || k < lm.first_k) pre += v[k];
+      if (has_mark && k >= lm.last_k) post += v[k];
+    }
+    const int incl = latest_inclusive(lm.last_packed, carried, lane);
+    int in_packed = __shfl_up(incl, 1, kWave);  // the mark in force where the lane begins
+    if (lane == 0) in_packed = carried;
+    const int in_owner = owner_of_mark(in_packed);
+    // one value per lane: the start of a run where the lane holds a mark, else its four edges
+    float x = has_mark ? (owner_of_mark(incl) >= 0 ? post : 0.0f) : (in_owner >= 0 ? pre : 0.0f);
 #pragma unroll
     for (int d = 1; d < kWave; d <<= 1) {
       const float y = __shfl_up(x, d, kWave);
-      const int ry = __shfl_up(run, d, kWave);
-      if (lane >= d && ry == run) x += y;
+      const int iy = __shfl_up(incl, d, kWave);
+      if (lane >= d && iy == incl) x += y;
     }
-    const int run_next = __shfl_down(run, 1, kWave);
-    const bool run_end = live && owner >= 0 && (lane == kWave - 1 || run_next != run);
-    if (run_end && open && run == carried) x += acc_open;  // only the first run of a step can match
-    const int src = owner >= 0 ? owner : 0;
-    const int64_t seg_b = __shfl(own.b, src, kWave);
-    const int64_t seg_e = __shfl(own.e, src, kWave);
-    const int seg_g = __shfl(own.g, src, kWave);
-    const bool closed = run_end && e == seg_e - 1;
-    const bool began_here = seg_b >= begin;
-    if (closed) {
-      if (began_here)
-        sums[nmap ? static_cast<int64_t>(nmap[seg_g]) : seg_g] = x;
+    float x_prev = __shfl_up(x, 1, kWave);  // the incoming run's sum over the lanes before
+    if (lane == 0) x_prev = 0.0f;
+    const int src = in_owner >= 0 ? in_owner : 0;
+    const int64_t in_b = __shfl(own.b, src, kWave);
+    const int in_g = __shfl(own.g, src, kWave);
+    if (has_mark && in_owner >= 0) {  // the incoming long run stops at this lane's first mark
+      float total = x_prev + pre;
+      if (open && in_packed == carried) total += acc_open;
+      if (in_b >= begin)
+        sums[nmap ? static_cast<int64_t>(nmap[in_g]) : in_g] = total;
       else
-        ck.carry[2 * c] = x;
+        ck.carry[2 * c] = total;
     }
-    // at most one run is cut by the end of the step: the last live lane's
-    const unsigned long long cut = __ballot(run_end && !closed);
-    carried = __shfl(latest, kWave - 1, kWave);  // unused lanes repeat the last edge's
-    open = cut != 0;
-    if (open) {
-      const int at = __ffsll(static_cast<long long>(cut)) - 1;
-      acc_open = __shfl(x, at, kWave);
-      if (base + kWave >= end) {  // cut by the end of the chunk: hand the piece on
-        const int here = __shfl(static_cast<int>(began_here), at, kWave);
-        const int g = __shfl(seg_g, at, kWave);
-        if (lane == 0) ck.carry[here ? 2 * c + 1 : 2 * c] = acc_open;
-        if (here) out_g = g;
+    const int last = __shfl(incl, kWave - 1, kWave);
+    const float x_last = __shfl(x, kWave - 1, kWave);
+    const bool goes_on = owner_of_mark(last) >= 0;
+    acc_open = goes_on ? x_last + (open && last == carried ? acc_open : 0.0f) : 0.0f;
+    open = goes_on;
+    carried = last;
+  }
+  // the run in force at the end of the chunk
+  int out_g = -1;
+  if (open) {
+    const int owner = owner_of_mark(carried);
+    const int64_t ob = __shfl(own.b, owner, kWave);
+    const int64_t oe = __shfl(own.e, owner, kWave);
+    const int og = __shfl(own.g, owner, kWave);
+    if (lane == 0) {
+      if (oe == end) {
+        if (ob >= begin)
+          sums[nmap ? static_cast<int64_t>(nmap[og]) : og] = acc_open;
+        else
+          ck.carry[2 * c] = acc_open;
+      } else {
+        ck.carry[ob >= begin ? 2 * c + 1 : 2 * c] = acc_open;
       }
     }
-    v = v_next;
+    if (oe != end && ob >= begin) out_g = og;
   }
   if (lane == 0) ck.outgoing[c] = out_g;
 }
@@ -257,7 +322,7 @@ __global__ void __launch_bounds__(kThreads)
 long_divide_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ emap,
                    const float* __restrict__ data, int64_t num_seg, int64_t nnz,
                    const float* __restrict__ sums, float* __restrict__ out, Chunks ck) {
-  __shared__ int s_mark[kWaves][kChunk];
+  __shared__ __attribute__((aligned(16))) int s_mark[kWaves][kChunk];
   if (*ck.any_long == 0u) return;
   if (indptr[num_seg] < nnz) nnz = indptr[num_seg];
   const int lane = threadIdx.x & (kWave - 1);
@@ -270,16 +335,32 @@ long_divide_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict
   write_marks(mark, own, begin, end, lane);
   const float own_sum = own.g >= 0 ? sums[own.g] : 0.0f;
   int carried = 0;
-  for (int64_t base = begin; base < end; base += kWave) {
-    const int64_t e = base + lane;
-    const bool live = e < end;
-    const int latest = latest_mark(mark, static_cast<int>(e - begin), live, carried, lane);
-    carried = __shfl(latest, kWave - 1, kWave);
-    const int owner = (latest & 0xFF) - 2;
-    const float total = __shfl(own_sum, owner >= 0 ? owner : 0, kWave);
-    if (live && owner >= 0) {
-      const int64_t d = emap ? emap[e] : e;
-      out[d] = data[d] / total;
+  for (int64_t base = begin; base < end; base += kStep) {
+    const int at0 = static_cast<int>(base - begin) + lane * kLaneEdges;
+    const int64_t e0 = base + lane * kLaneEdges;
+    int m[kLaneEdges];
+    {
+      const int4 mm = *reinterpret_cast<const int4*>(mark + at0);
+      m[0] = mm.x; m[1] = mm.y; m[2] = mm.z; m[3] = mm.w;
+    }
+#pragma unroll
+    for (int k = 0; k < kLaneEdges; ++k)
+      if (e0 + k >= end) m[k] = 0;
+    const LaneMarks lm = scan_lane_marks(m, at0);
+    const int incl = latest_inclusive(lm.last_packed, carried, lane);
+    int cur = __shfl_up(incl, 1, kWave);
+    if (lane == 0) cur = carried;
+    carried = __shfl(incl, kWave - 1, kWave);
+#pragma unroll
+    for (int k = 0; k < kLaneEdges; ++k) {
+      if (m[k]) cur = (at0 + k + 1) << 8 | m[k];
+      const int owner = owner_of_mark(cur);
+      const float total = __shfl(own_sum, owner >= 0 ? owner : 0, kWave);
+      const int64_t e = e0 + k;
+      if (e < end && owner >= 0) {
+        const int64_t d = emap ? emap[e] : e;
+        out[d] = data[d] / total;
+      }
     }
   }
 }

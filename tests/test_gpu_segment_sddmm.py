@@ -60,7 +60,7 @@ def test_segment_sum_rmat(dev, powk, maps, idt):
 
 
 @pytest.mark.parametrize("case", ["hub_over_chunks", "chunk_aligned", "empties_then_long",
-                                  "one_segment", "short_over_chunk_border"])
+                                  "one_segment", "short_over_chunk_border", "few_edges_into_next_chunk"])
 @pytest.mark.parametrize("maps", [False, True])
 def test_segment_sum_pieces_across_chunks(dev, case, maps):
     # long segments are summed by chunks of 1024 edges of the edge array: segments that start,
@@ -72,6 +72,9 @@ def test_segment_sum_pieces_across_chunks(dev, case, maps):
         "empties_then_long": [0] * 3000 + [40] + [0] * 2000 + [3000] + [0] * 100,
         "one_segment": [10000],
         "short_over_chunk_border": [1020, 8, 1020, 16, 17, 2000],
+        # long segments of which 1, 19 and 3 edges reach into the next chunk, and one that starts
+        # one edge before a border
+        "few_edges_into_next_chunk": [1007, 18, 3, 1019, 20, 17, 991, 40],
     }[case]
     indptr = np.concatenate([[0], np.cumsum(np.asarray(deg, dtype=np.int64))])
     nnz, n = int(indptr[-1]), len(deg)
