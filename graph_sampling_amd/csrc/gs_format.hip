@@ -5,10 +5,11 @@
 // src/cuda/format_transform.cu:35,135; the reference leans on cub radix sort,
 // whose stability pins the edge order, format_transform.cu:81-100).
 //
-//  * csc2coo: edge-balanced.  A workgroup owns 2048 consecutive edges, finds the
-//    columns they span with two binary searches, stages that slice of the
-//    offsets in LDS and resolves each edge there (the reference runs a full
-//    global binary search per edge, format_transform.cu:24-33).
+//  * csc2coo: edge-balanced.  A workgroup owns 4096 consecutive edges, finds the
+//    columns they span with two binary searches, lets those columns mark their
+//    first edge in LDS and turns the marks into column numbers with a running
+//    maximum (the reference runs a full global binary search per edge,
+//    format_transform.cu:24-33).
 //  * coo2csc: 8-bit digits, only ceil(log2(num_keys)/8) passes
 //    (format_transform.cu:58-72 also sorts just the significant bits).  Each
 //    pass is histogram -> scan -> stable scatter; the scatter ranks equal digits
@@ -23,7 +24,6 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kItems = 8;
 constexpr int kTile = kThreads * kItems;
-constexpr int kStage = 1024;
 
 template <typename P>
 __device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
@@ -35,31 +35,69 @@ __device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
   return lo;
 }
 
+constexpr int kCooItems = 16;
+constexpr int kCooTile = kThreads * kCooItems;
+
+// A workgroup owns kCooTile consecutive edges.  The columns that start inside the tile mark
+// their first edge in LDS (column-parallel, coalesced reads of the offsets; of several empty
+// columns at one position the highest wins, which is the owner), and a running maximum
+// over the marks gives every edge its column: sixteen consecutive edges per thread, one
+// maximum per thread across the workgroup.  No search per edge.
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz,
                const IdT* __restrict__ ids, IdT* __restrict__ col) {
-  __shared__ int64_t s_ptr[kStage + 1];
+  __shared__ int s_mark[kCooTile];
   __shared__ int64_t s_rows[2];
-  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
-  const int64_t p1 = p0 + kTile < nnz ? p0 + kTile : nnz;
+  __shared__ int s_wave[kThreads / kWave];
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kCooTile;
+  const int64_t p1 = p0 + kCooTile < nnz ? p0 + kCooTile : nnz;
   if (threadIdx.x < 2)
     s_rows[threadIdx.x] = upper_bound(indptr, num_cols + 1, threadIdx.x == 0 ? p0 : p1 - 1) - 1;
+  for (int i = threadIdx.x; i < kCooTile; i += kThreads) s_mark[i] = 0;
   __syncthreads();
-  const int64_t row_lo = s_rows[0];
-  const int64_t nrows = s_rows[1] - row_lo + 1;
-  const bool staged = nrows <= kStage;
-  if (staged)
-    for (int64_t i = threadIdx.x; i <= nrows; i += kThreads) s_ptr[i] = indptr[row_lo + i];
+  const int64_t row_lo = s_rows[0], row_hi = s_rows[1];
+  // columns row_lo + 1 .. row_hi start inside the tile (row_lo holds its first edge)
+  for (int64_t r = row_lo + 1 + threadIdx.x; r <= row_hi; r += kThreads)
+    atomicMax(&s_mark[indptr[r] - p0], static_cast<int>(r - row_lo));
+  __syncthreads();
+  const int at0 = threadIdx.x * kCooItems;
+  int m[kCooItems];
+  int run = 0;
+#pragma unroll
+  for (int k = 0; k < kCooItems; ++k) {
+    const int v = s_mark[at0 + k];
+    run = v > run ? v : run;
+    m[k] = run;  // relative to what holds where the thread begins
+  }
+  // exclusive running maximum of the threads' last values
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  int incl = run;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int y = __shfl_up(incl, d, kWave);
+    if (lane >= d && y > incl) incl = y;
+  }
+  if (lane == kWave - 1) s_wave[wave] = incl;
+  __syncthreads();
+  int before = __shfl_up(incl, 1, kWave);
+  if (lane == 0) before = 0;
+  for (int w = 0; w < wave; ++w) before = s_wave[w] > before ? s_wave[w] : before;
+  // column numbers (relative to row_lo) go back into the marks' place, so that the stores
+  // below are coalesced whatever the id width
   __syncthreads();
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
-    const int64_t p = p0 + k * kThreads + threadIdx.x;
-    if (p >= p1) break;
-    const int64_t c = row_lo + (staged ? upper_bound(s_ptr, nrows + 1, p)
-                                       : upper_bound(indptr + row_lo, nrows + 1, p)) - 1;
-    // doubly-compressed: stored column c stands for node ids[c] (format_transform.cu:48-60)
-    col[p] = ids ? ids[c] : static_cast<IdT>(c);
+  for (int k = 0; k < kCooItems; ++k) s_mark[at0 + k] = m[k] > before ? m[k] : before;
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kCooItems; ++k) {
+    const int i = k * kThreads + threadIdx.x;
+    const int64_t p = p0 + i;
+    if (p < p1) {
+      const int64_t c = row_lo + s_mark[i];
+      // doubly-compressed: stored column c stands for node ids[c] (format_transform.cu:48-60)
+      col[p] = ids ? ids[c] : static_cast<IdT>(c);
+    }
   }
 }
 
@@ -298,11 +336,11 @@ int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, void* col, 
   if (nnz == 0) return GS_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (id_bytes == 8)
-    hipLaunchKernelGGL((csc2coo_kernel<int64_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
+    hipLaunchKernelGGL((csc2coo_kernel<int64_t>), dim3(blocks_for(nnz, kCooTile)), dim3(kThreads), 0,
                        st, indptr, num_cols, nnz, static_cast<const int64_t*>(nullptr),
                        static_cast<int64_t*>(col));
   else
-    hipLaunchKernelGGL((csc2coo_kernel<int32_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
+    hipLaunchKernelGGL((csc2coo_kernel<int32_t>), dim3(blocks_for(nnz, kCooTile)), dim3(kThreads), 0,
                        st, indptr, num_cols, nnz, static_cast<const int32_t*>(nullptr),
                        static_cast<int32_t*>(col));
   return check_launch("csc2coo");
@@ -316,11 +354,11 @@ int gs_dcsc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, const void
   if (nnz == 0) return GS_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (id_bytes == 8)
-    hipLaunchKernelGGL((csc2coo_kernel<int64_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
+    hipLaunchKernelGGL((csc2coo_kernel<int64_t>), dim3(blocks_for(nnz, kCooTile)), dim3(kThreads), 0,
                        st, indptr, num_cols, nnz, static_cast<const int64_t*>(ids),
                        static_cast<int64_t*>(col));
   else
-    hipLaunchKernelGGL((csc2coo_kernel<int32_t>), dim3(blocks_for(nnz, kTile)), dim3(kThreads), 0,
+    hipLaunchKernelGGL((csc2coo_kernel<int32_t>), dim3(blocks_for(nnz, kCooTile)), dim3(kThreads), 0,
                        st, indptr, num_cols, nnz, static_cast<const int32_t*>(ids),
                        static_cast<int32_t*>(col));
   return check_launch("dcsc2coo");
