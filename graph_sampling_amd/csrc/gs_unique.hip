@@ -448,7 +448,9 @@ struct PackedRegions {
                                               static_cast<unsigned long long>(len)) >>
                                              32);
     while (true) {
-      const unsigned long long prev = atomicCAS(&slots[p], ~0ull, word);
+      // a look before the compare-and-swap: a slot that is taken needs none
+      unsigned long long prev = __hip_atomic_load(&slots[p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (prev == ~0ull) prev = atomicCAS(&slots[p], ~0ull, word);
       if (prev == ~0ull) break;
       if ((prev >> 32) == (hi >> 32)) {
         if (static_cast<uint32_t>(prev) > i) atomicMin(&slots[p], word);
