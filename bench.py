@@ -356,6 +356,30 @@ def main():
               "what": "the timed minibatches again with four in flight, one host thread and one "
                       "stream each"}
 
+    # the same again by the C++ layer's own pool of sampler threads (no interpreter in the
+    # loop), 32 minibatches per call as a loader with that prefetch depth would ask for them
+    pool = None
+    if extras:
+        ops = torch.ops.gs_ops
+        DEPTH = 32
+        timed_sets = seed_sets[args.warmup:]
+        ops._CAPI_SampleBlocks(graph, seed_sets[:DEPTH], FANOUTS, False, WORKERS, 0)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        pool_edges = 0
+        for c0 in range(0, len(timed_sets), DEPTH):
+            res = ops._CAPI_SampleBlocks(graph, timed_sets[c0:c0 + DEPTH], FANOUTS, False, WORKERS,
+                                         c0 * len(FANOUTS))
+            pool_edges += sum(int(parts[3 * l + 2].numel()) for parts in res
+                              for l in range(len(FANOUTS)))
+            del res
+        torch.cuda.synchronize()
+        pool_s = time.perf_counter() - t1
+        pool = {"workers": WORKERS, "minibatches_per_call": DEPTH,
+                "ms_per_step": pool_s / len(timed_sets) * 1e3, "value": pool_edges / pool_s,
+                "what": "the timed minibatches through gs_ops._CAPI_SampleBlocks: four host threads "
+                        "of the C++ layer, one stream each"}
+
     out = {
         "metric": "sampled edges/sec (GSEPS), GraphSAGE [15,10,5] batch 1024, slice+sample+relabel",
         "value": sampled / elapsed,
@@ -377,6 +401,7 @@ def main():
         "unfused_path": nf,
         "super_batch": sb,
         "concurrent": cc,
+        "sampler_pool": pool,
         "roofline": None,
         "cpu_baseline": None,
     }

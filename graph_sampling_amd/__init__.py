@@ -51,3 +51,25 @@ def set_seed(seed):
     import torch
     load_library()
     torch.ops.gs_ops._CAPI_SetSeed(int(seed))
+
+
+def sample_blocks(matrix, seed_sets, fanouts, replace=False, workers=4, seed=0):
+    """GraphSAGE-style minibatches sampled side by side by `workers` host threads of the C++
+    layer, one stream each (fused slice + sample, relabel, next seeds = frontier, per layer).
+    Returns [(input_nodes, [Block, ...] innermost layer first)] in the order of `seed_sets`;
+    minibatch i draws with seeds `seed + i * len(fanouts) + layer` whichever thread runs it."""
+    import torch
+    from .block import Block
+    load_library()
+    graph = getattr(matrix, "_graph", matrix)
+    flat = torch.ops.gs_ops._CAPI_SampleBlocks(graph, list(seed_sets), list(fanouts), bool(replace),
+                                               int(workers), int(seed))
+    out = []
+    for parts in flat:
+        blocks = []
+        for l in range(len(fanouts)):
+            frontier, indptr, indices = parts[3 * l:3 * l + 3]
+            blocks.insert(0, Block(frontier.numel(), indptr.numel() - 1, "csc", indptr, indices,
+                                   frontier))
+        out.append((parts[-3], blocks))
+    return out

@@ -10,6 +10,7 @@
 #include "graph_ops.h"
 #include "hetero_graph.h"
 #include "hip_ops.h"
+#include "sampler_pool.h"
 #include "tensor_ops.h"
 
 using namespace gs;
@@ -136,6 +137,7 @@ TORCH_LIBRARY(gs_ops, m) {
   // not in the reference: reproducible sampling (its seeds are compile-time constants)
   m.def("_CAPI_SetSeed", &SetSeed);
   m.def("_CAPI_SetThreadSeed", &SetThreadSeed);
+  m.def("_CAPI_SampleBlocks", &SampleBlocks);
   m.def("_CAPI_SetSampleAlgo", &SetSampleAlgo);
   // not in the reference: off = every sampling call settles its edge count before returning
   m.def("_CAPI_SetDeferredSampling", &SetDeferredSampling);

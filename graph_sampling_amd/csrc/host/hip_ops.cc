@@ -189,12 +189,15 @@ int OpCode(const std::string& op) {
 }  // namespace
 
 namespace {
-// a thread that called SetThreadSeed counts its own seeds from then on
+// a thread that called SetThreadSeed counts its own seeds until it calls SetSeed
 thread_local bool t_own_seed = false;
 thread_local uint64_t t_seed = 0;
 }  // namespace
 
-void SetSeed(uint64_t seed) { g_seed.store(seed); }
+void SetSeed(uint64_t seed) {
+  g_seed.store(seed);
+  t_own_seed = false;  // the caller is back on the shared counter
+}
 void SetThreadSeed(uint64_t seed) {
   t_own_seed = true;
   t_seed = seed;

@@ -24,8 +24,8 @@ using SliceResult = std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torc
 // the same launch geometry repeat the same draws (src/cuda/sampling.cu:138).
 void SetSeed(uint64_t seed);
 // The same for the calling thread only, which from then on no longer draws from the
-// shared counter: for several sampler threads whose draws must not depend on how they
-// interleave.
+// shared counter (until it calls SetSeed): for several sampler threads whose draws must
+// not depend on how they interleave.
 void SetThreadSeed(uint64_t seed);
 uint64_t NextSeed();
 // 0: Floyd selection for deg > fanout (default), 1: the reference's Algorithm R.

@@ -1,0 +1,161 @@
+// Minibatches sampled side by side: a pool of host threads, one HIP stream each.
+//
+// No counterpart in the reference, whose samplers are Python loops over Graph methods
+// (examples/graphsage/graphsage_fused.py:28-46) and which answers launch latency with
+// super-batches.  At batch 1024 a layer is a chain of dependent round trips that leaves the
+// chip almost idle; independent minibatches fill it.  Host threads outside Python share no
+// interpreter lock, every thread keeps its own relabel table, look-back state and mailboxes
+// (they are thread-local in hip_ops.cc), and minibatch i always draws with the seeds
+// first_seed + i * layers + layer, so the result does not depend on which thread took it.
+// How far it scales is set by the hardware queues a process gets (4 by default, one of them
+// the null stream's: a fourth worker shares a queue with the third and the two take turns)
+// and by the kernels slowing each other down: two workers give about 1.5 x one, more add little.
+// The results keep their capacity-sized buffers alive, so a caller should ask for a few
+// minibatches per worker at a time, as a loader's prefetch depth would, not for an epoch.
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+
+#include <condition_variable>
+#include <exception>
+#include <functional>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <thread>
+
+#include "graph.h"
+#include "hip_ops.h"
+#include "sampler_pool.h"
+
+namespace gs {
+namespace {
+
+// The threads live as long as the process: what a thread keeps between calls -- its stream
+// (the caching allocator keeps memory per stream; a fresh stream per call would send every
+// allocation to hipMalloc), its relabel table, its mailboxes -- is only worth having when the
+// next call finds it again.  The pool is never torn down: at exit the threads are parked on a
+// condition variable and own device memory that must not be released after the runtime is gone.
+class Worker {
+ public:
+  Worker() : thread_([this] { Loop(); }) {}
+  void Start(std::function<void()> task) {
+    std::lock_guard<std::mutex> hold(lock_);
+    task_ = std::move(task);
+    busy_ = true;
+    wake_.notify_one();
+  }
+  void Wait() {
+    std::unique_lock<std::mutex> hold(lock_);
+    idle_.wait(hold, [this] { return !busy_; });
+  }
+
+ private:
+  void Loop() {
+    for (;;) {
+      std::function<void()> task;
+      {
+        std::unique_lock<std::mutex> hold(lock_);
+        wake_.wait(hold, [this] { return busy_; });
+        task = std::move(task_);
+      }
+      task();
+      {
+        std::lock_guard<std::mutex> hold(lock_);
+        busy_ = false;
+      }
+      idle_.notify_all();
+    }
+  }
+  std::mutex lock_;
+  std::condition_variable wake_, idle_;
+  std::function<void()> task_;
+  bool busy_ = false;
+  std::thread thread_;
+};
+
+struct Pool {
+  std::mutex one_call;  // calls take turns
+  std::vector<std::unique_ptr<Worker>> workers;
+};
+
+Pool& ThePool() {
+  static Pool* pool = new Pool;  // never deleted, see above
+  return *pool;
+}
+
+// the stream a pool thread uses on a device, taken once
+c10::hip::HIPStream WorkerStream(int device) {
+  thread_local std::map<int, c10::hip::HIPStream> streams;
+  auto it = streams.find(device);
+  if (it == streams.end())
+    it = streams.emplace(device, c10::hip::getStreamFromPool(/*isHighPriority=*/false, device)).first;
+  return it->second;
+}
+
+}  // namespace
+
+std::vector<std::vector<torch::Tensor>> SampleBlocks(const c10::intrusive_ptr<Graph>& graph,
+                                                     std::vector<torch::Tensor> seed_sets,
+                                                     std::vector<int64_t> fanouts, bool replace,
+                                                     int64_t workers, int64_t first_seed) {
+  const int64_t n = static_cast<int64_t>(seed_sets.size());
+  const int64_t layers = static_cast<int64_t>(fanouts.size());
+  std::vector<std::vector<torch::Tensor>> out(n);
+  if (n == 0 || layers == 0) return out;
+  TORCH_CHECK(workers >= 1 && workers <= 16, "workers must be in 1..16, got ", workers);
+  for (const auto& s : seed_sets)
+    TORCH_CHECK(s.defined() && s.is_cuda() && s.device() == seed_sets[0].device(),
+                "every seed set must be a tensor on the same GPU");
+  const auto device = seed_sets[0].device();
+  graph->CreateSparseFormat(_CSC);  // the one lazy step of the shared graph, done before the threads start
+  // what the caller queued so far (the seeds) must be visible to the workers' streams
+  const auto caller = c10::hip::getCurrentHIPStream(device.index());
+  hipEvent_t ready;
+  TORCH_CHECK(hipEventCreateWithFlags(&ready, hipEventDisableTiming) == hipSuccess,
+              "hipEventCreate failed");
+  TORCH_CHECK(hipEventRecord(ready, caller.stream()) == hipSuccess, "hipEventRecord failed");
+
+  const int64_t nthreads = workers < n ? workers : n;
+  std::exception_ptr failure;
+  std::mutex failure_lock;
+  auto work = [&](int64_t k) {
+    try {
+      c10::hip::HIPGuard device_guard(device.index());
+      const auto stream = WorkerStream(device.index());
+      c10::hip::HIPStreamGuard stream_guard(stream);
+      TORCH_CHECK(hipStreamWaitEvent(stream.stream(), ready, 0) == hipSuccess,
+                  "hipStreamWaitEvent failed");
+      for (int64_t i = k; i < n; i += nthreads) {
+        hip::SetThreadSeed(static_cast<uint64_t>(first_seed + i * layers));
+        torch::Tensor seeds = seed_sets[i];
+        out[i].reserve(3 * layers);
+        for (int64_t l = 0; l < layers; ++l) {
+          auto sub = graph->ColumnwiseFusedSlicingAndSampling(seeds, fanouts[l], replace);
+          auto r = sub->Relabel();
+          out[i].push_back(std::get<0>(r));  // frontier: source ids of the block, seeds first
+          out[i].push_back(std::get<3>(r));  // offsets over the destinations
+          out[i].push_back(std::get<4>(r));  // source positions in the frontier
+          seeds = std::get<0>(r);
+        }
+      }
+      TORCH_CHECK(hipStreamSynchronize(stream.stream()) == hipSuccess, "hipStreamSynchronize failed");
+    } catch (...) {
+      std::lock_guard<std::mutex> hold(failure_lock);
+      if (!failure) failure = std::current_exception();
+    }
+  };
+  {
+    Pool& pool = ThePool();
+    std::lock_guard<std::mutex> turn(pool.one_call);
+    while (static_cast<int64_t>(pool.workers.size()) < nthreads)
+      pool.workers.push_back(std::make_unique<Worker>());
+    for (int64_t k = 0; k < nthreads; ++k) pool.workers[k]->Start([&work, k] { work(k); });
+    for (int64_t k = 0; k < nthreads; ++k) pool.workers[k]->Wait();
+  }
+  (void)hipEventDestroy(ready);
+  if (failure) std::rethrow_exception(failure);
+  return out;
+}
+
+}  // namespace gs

@@ -774,3 +774,40 @@ def test_sampler_threads_on_their_own_streams_are_reproducible(dev):
             assert np.array_equal(ptr, w_ptr) and np.array_equal(idx, w_idx)
             assert np.array_equal(frontier, w_frontier)
             seeds = w_frontier
+
+
+@pytest.mark.parametrize("workers", [1, 4])
+def test_sample_blocks_pool_equals_the_python_loop(dev, workers):
+    """gs.sample_blocks (host threads of the C++ layer, one stream each) against the same
+    minibatches sampled one after the other through the Graph methods with the same seeds."""
+    m, indptr, indices, _ = _rmat_matrix(dev, 13, 17, 21)
+    fanouts = [7, 5, 3]
+    rng = np.random.default_rng(8)
+    sets = [to_dev(rng.permutation(1 << 13)[:64 + 16 * i].astype(np.int64), dev) for i in range(11)]
+    got = gs.sample_blocks(m, sets, fanouts, replace=False, workers=workers, seed=500)
+    assert len(got) == len(sets)
+    for i, seeds in enumerate(sets):
+        torch.ops.gs_ops._CAPI_SetThreadSeed(500 + i * len(fanouts))
+        blocks = []
+        for k in fanouts:
+            sub = m.fused_columnwise_slicing_sampling(seeds, k, False)
+            blk = sub.to_dgl_block()
+            blocks.insert(0, blk)
+            seeds = blk.srcdata["_ID"]
+        nodes, got_blocks = got[i]
+        assert torch.equal(nodes, seeds)
+        for a, b in zip(got_blocks, blocks):
+            assert a.num_dst_nodes() == b.num_dst_nodes() and a.num_src_nodes() == b.num_src_nodes()
+            assert torch.equal(a.srcdata["_ID"], b.srcdata["_ID"])
+            assert torch.equal(a.csc()[0], b.csc()[0]) and torch.equal(a.csc()[1], b.csc()[1])
+    gs.set_seed(0)  # back to the shared counter for the tests that follow
+
+
+def test_sample_blocks_rejects_bad_arguments(dev):
+    m, _, _, _ = _rmat_matrix(dev, 10, 13, 2)
+    seeds = torch.arange(10, device=dev)
+    with pytest.raises(RuntimeError, match="workers"):
+        gs.sample_blocks(m, [seeds], [3], workers=0)
+    with pytest.raises(RuntimeError, match="same GPU"):
+        gs.sample_blocks(m, [seeds.cpu()], [3])
+    assert gs.sample_blocks(m, [], [3]) == []
