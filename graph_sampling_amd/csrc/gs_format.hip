@@ -330,7 +330,8 @@ extern "C" {
 
 int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, void* col, int id_bytes,
                void* stream) {
-  GS_REQUIRE(num_cols >= 0 && nnz >= 0, "gs_csc2coo: negative size");
+  GS_REQUIRE(num_cols >= 0 && nnz >= 0 && num_cols < (int64_t(1) << 31),
+             "gs_csc2coo: negative size or more than 2^31 columns");
   GS_REQUIRE(nnz == 0 || (indptr && col), "gs_csc2coo: null pointer");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_csc2coo: id_bytes must be 4 or 8, got %d", id_bytes);
   if (nnz == 0) return GS_OK;
@@ -348,7 +349,8 @@ int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, void* col, 
 
 int gs_dcsc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, const void* ids, void* col,
                 int id_bytes, void* stream) {
-  GS_REQUIRE(num_cols >= 0 && nnz >= 0, "gs_dcsc2coo: negative size");
+  GS_REQUIRE(num_cols >= 0 && nnz >= 0 && num_cols < (int64_t(1) << 31),
+             "gs_dcsc2coo: negative size or more than 2^31 columns");
   GS_REQUIRE(nnz == 0 || (indptr && col && ids), "gs_dcsc2coo: null pointer");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_dcsc2coo: id_bytes must be 4 or 8, got %d", id_bytes);
   if (nnz == 0) return GS_OK;
