@@ -243,3 +243,47 @@ def test_sddmm_dot_on_sampled_blocks_full_size(dev, sage_graph):
         want = (feat[rows] * rhs[col_local]).sum(-1, keepdim=True)
         torch.testing.assert_close(out, want, rtol=1e-5, atol=1e-5)
         seeds = sub.all_indices()
+
+
+def test_segment_sums_and_column_expansion_full_size(dev, sage_graph):
+    """Per-column sum of w^2 and per-column normalisation over all 124 M edges (columns from empty
+    to 297 k edges, so every path of the segment kernels runs: by lane, by chunk, pieces across
+    chunks), and the CSC -> COO column expansion of the whole graph.  The CPU oracle sums in edge
+    order, which at this size is neither fast nor what a 300 k-term fp32 sum should be compared
+    with; the checks are a float64 segment reduction of the same data (1e-5 relative), exactness
+    of columns of at most 16 edges against an fp32 sequential sum, run-to-run identity, and
+    "every non-empty column's normalised weights add up to 1"."""
+    indptr, indices, h_indptr, _ = sage_graph
+    N, E = indptr.numel() - 1, indices.numel()
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(21)
+    w = 1.0 - torch.rand(E, generator=gen, device=dev)
+    lens = indptr[1:] - indptr[:-1]
+    out = torch.empty(N, device=dev)
+    capi.segment_sum(indptr, None, None, w, 2, out)
+    ref = torch.segment_reduce(w.double() ** 2, "sum", lengths=lens, initial=0.0)
+    assert bool((out[lens == 0] == 0).all())
+    rel = ((out.double() - ref).abs() / ref.clamp(min=1e-300))[lens > 0]
+    assert float(rel.max()) < 1e-5
+    again = torch.empty(N, device=dev)
+    capi.segment_sum(indptr, None, None, w, 2, again)
+    assert torch.equal(out, again)
+    # short columns: the sequential fp32 sum, bit for bit (a sample of them on the host)
+    short = torch.nonzero((lens > 0) & (lens <= 16)).flatten()[:20000].cpu().numpy()
+    h_w = w.cpu().numpy()
+    h_out = out.cpu().numpy()
+    for c in short[::50]:
+        acc = np.float32(0)
+        for x in h_w[h_indptr[c]:h_indptr[c + 1]]:
+            acc = np.float32(acc + np.float32(x * x))
+        assert h_out[c] == acc
+    norm = torch.empty(E, device=dev)
+    capi.segment_normalize(indptr, None, w, norm)
+    totals = torch.segment_reduce(norm.double(), "sum", lengths=lens, initial=0.0)
+    assert float((totals[lens > 0] - 1.0).abs().max()) < 1e-4
+    seg = torch.repeat_interleave(torch.arange(N, device=dev), lens)
+    col = capi.csc2coo(indptr, E, torch.int32)
+    assert torch.equal(col.long(), seg)
+    picks = torch.randint(0, E, (1_000_000,), generator=gen, device=dev)
+    want = w[picks].double() / torch.segment_reduce(w.double(), "sum", lengths=lens, initial=0.0)[seg[picks]]
+    assert float(((norm[picks].double() - want).abs() / want).max()) < 1e-5
