@@ -811,3 +811,8 @@ def test_sample_blocks_rejects_bad_arguments(dev):
     with pytest.raises(RuntimeError, match="same GPU"):
         gs.sample_blocks(m, [seeds.cpu()], [3])
     assert gs.sample_blocks(m, [], [3]) == []
+    # an error inside a worker comes back as an exception, and the pool goes on working
+    with pytest.raises(RuntimeError, match="fanout"):
+        gs.sample_blocks(m, [seeds, seeds], [3, -1], workers=2)
+    nodes, blocks = gs.sample_blocks(m, [seeds], [3], workers=2)[0]
+    assert blocks[0].num_dst_nodes() == 10 and nodes.numel() == blocks[0].num_src_nodes()
