@@ -182,6 +182,21 @@ def main():
     run("sddmm_dot", "gs_sddmm_coo u_dot_v, 64-d fp32 features, 8M random edges; 532 B per edge",
         lambda: capi.sddmm_coo("dot", er, ec, None, feat, feat, out_e, 0, 2, 64, 64, 1, 64, None, None),
         lambda o: (8_000_000 * 532, 8_000_000, "edges"))
+    # Divide(divisor, axis=0) on the CSC: out[e] = w[e] / divisor[column of e], scalar per edge
+    divisor = torch.rand(N, generator=gen, device=dev) + 0.5
+    out_w = torch.empty(E, 1, device=dev)
+    run("sddmm_div_csc", "gs_sddmm_csc e_div_v over the whole graph (edge weight / per-column scalar): "
+        "4 B read + 4 B written per edge, 12 B per column",
+        lambda: capi.sddmm_csc("div", indptr, indices, None, None, weights, divisor, out_w, 1, 2,
+                               1, 1, 1, 1, None, None),
+        lambda o: (E * 8 + N * 12, E, "edges"))
+    # Divide(divisor, axis=1) on the COO form: out[e] = w[e] / divisor[row of e], a random read per edge
+    coo_col = capi.csc2coo(indptr, E, idt)
+    run("sddmm_div_coo_rows", "gs_sddmm_coo e_div_u over the whole graph (edge weight / scalar of the "
+        "edge's row): 4 + b read, 4 written and one random 4-byte read per edge",
+        lambda: capi.sddmm_coo("div", indices, coo_col, None, weights, divisor, out_w, 1, 0,
+                               1, 1, 1, 1, None, None),
+        lambda o: (E * (12 + b), E, "edges"))
     out_n = torch.empty(N, device=dev)
     run("segment_sum", "gs_segment_sum of w^2 over every column of the graph; 4 B per edge + 20 B "
         "per column",
