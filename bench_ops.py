@@ -176,6 +176,21 @@ def main():
         lambda: capi.random_walk(indptr, indices, starts, 80, seed=3),
         lambda o: (int((o[1_000_000:] >= 0).sum().item()) * 28,
                    int((o[1_000_000:] >= 0).sum().item()), "steps"))
+    if not only or "metapath_walk" in only:
+        # three bipartite relations (1M x 2M nodes, 50M edges each), metapath of 4 repeated 4 times
+        rels = [rmat.rmat_csc(2_000_000, 50_000_000, seed=30 + r, device=dev, index_dtype=idt,
+                              num_src_nodes=2_000_000) for r in range(3)]
+        ptr_tab = torch.tensor([r[0].data_ptr() for r in rels], dtype=torch.int64, device=dev)
+        idx_tab = torch.tensor([r[1].data_ptr() for r in rels], dtype=torch.int64, device=dev)
+        n_tab = torch.tensor([r[0].numel() - 1 for r in rels], dtype=torch.int64, device=dev)
+        path = torch.tensor([0, 1, 2, 1] * 4, dtype=torch.int64, device=dev)
+        mstarts = rand_ids(1_000_000, 2_000_000)
+        run("metapath_walk", "gs_metapath_walk: 1M walkers x 16 steps over three 50M-edge relations; "
+            "28 B per live step",
+            lambda: capi.metapath_walk(ptr_tab, idx_tab, n_tab, idt, path, mstarts, seed=4),
+            lambda o: (int((o[1_000_000:] >= 0).sum().item()) * 28,
+                       int((o[1_000_000:] >= 0).sum().item()), "steps"))
+        del rels
     feat = torch.rand(N, 64, generator=gen, device=dev)
     er, ec = rand_ids(8_000_000), rand_ids(8_000_000)
     out_e = torch.empty(8_000_000, 1, device=dev)
@@ -197,6 +212,32 @@ def main():
         lambda: capi.sddmm_coo("div", indices, coo_col, None, weights, divisor, out_w, 1, 0,
                                1, 1, 1, 1, None, None),
         lambda o: (E * (12 + b), E, "edges"))
+    # ---- the layer-wise samplers' picks: 512 of 2.45M rows, by weight and uniformly -------------
+    row_prob = torch.rand(N, generator=gen, device=dev)
+    row_prob[torch.rand(N, generator=gen, device=dev) < 0.7] = 0.0  # most rows unreachable
+    all_rows = torch.arange(N, device=dev, dtype=idt)
+    run("list_sample_weighted", "gs_list_sample_weighted: 512 of 2.45M rows without replacement "
+        "(70% of the weights zero); 4 B per row and select level + 16 B per pick",
+        lambda: capi.list_sample_weighted(all_rows, row_prob, 512, seed=3),
+        lambda o: (N * 4 + 512 * 16, N, "items"))
+    run("list_sample_uniform", "gs_list_sample_uniform: 512 of 2.45M rows without replacement",
+        lambda: capi.list_sample_uniform(all_rows, 512, False, seed=3),
+        lambda o: (512 * (b + 16), 512, "items"))
+    # row probabilities straight off a column slice's COO rows (atomic adds into 2.45M sums)
+    out_p = torch.zeros(N, device=dev)
+    run("coo_sum", "gs_coo_sum of w^2 over the rows of a 512-column slice's edges into 2.45M sums",
+        lambda: capi.coo_sum(indices[:2_000_000], None, weights[:2_000_000], 2, out_p),
+        lambda o: (2_000_000 * (b + 4 + 8), 2_000_000, "edges"))
+    out_nrm = torch.empty(E, device=dev)
+    run("segment_normalize", "gs_segment_normalize over every column of the graph; 4 B read twice + "
+        "4 B written per edge, 16 B per column",
+        lambda: capi.segment_normalize(indptr, None, weights, out_nrm),
+        lambda o: (E * 12 + N * 16, E, "edges"))
+    keep_rows = torch.randperm(N, generator=gen, device=dev)[:200_000].to(idt)
+    run("row_slice_csc", "gs_row_slice_csc_*: the whole graph cut down to 200k of its rows (mark, scan, "
+        "compact); b + 16 B per edge looked at, 2b + 8 per edge kept",
+        lambda: capi.row_slice_csc(indptr, indices, keep_rows, True),
+        lambda o: (E * (b + 16) + int(o[2].numel()) * (2 * b + 8), E, "edges"))
     out_n = torch.empty(N, device=dev)
     run("segment_sum", "gs_segment_sum of w^2 over every column of the graph; 4 B per edge + 20 B "
         "per column",

@@ -421,7 +421,9 @@ coo_sum_kernel(const IdT* __restrict__ target, const int64_t* __restrict__ emap,
                const float* __restrict__ data, int64_t E, int powk, float* __restrict__ out) {
   const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (e >= E) return;
-  atomicAdd(out + target[e], powk_f(data[emap ? emap[e] : e], powk));
+  // the hardware's fp32 add at the memory side, not a compare-and-swap loop (which is what a
+  // plain atomicAdd(float*) compiles to here, and which retries without end on a hub row)
+  unsafeAtomicAdd(out + target[e], powk_f(data[emap ? emap[e] : e], powk));
 }
 
 // edge_map_reduce.cu:15-23
@@ -434,7 +436,7 @@ e_div_u_sum_kernel(const IdT* __restrict__ row, const IdT* __restrict__ col,
   if (e >= E) return;
   const float v = data[e] / divisor[row[e]];
   out_data[e] = v;
-  atomicAdd(out_sum + col[e], v);
+  unsafeAtomicAdd(out_sum + col[e], v);
 }
 
 }  // namespace
