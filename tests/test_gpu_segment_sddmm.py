@@ -101,6 +101,27 @@ def test_segment_sum_pieces_across_chunks(dev, case, maps):
     np.testing.assert_allclose(out.cpu().numpy(), want_n, rtol=RTOL)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_segment_sum_random_layouts(dev, seed):
+    # random mixes of empty, short, just-long and multi-chunk segments: wherever the chunk borders
+    # fall, sums and normalised weights agree with float64
+    rng = np.random.default_rng(100 + seed)
+    n = int(rng.integers(1, 600))
+    deg = rng.choice([0, 1, 5, 16, 17, 18, 30, 100, 1030, 2500, 3], size=n,
+                     p=[.2, .1, .1, .1, .1, .1, .1, .1, .03, .02, .05])
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    nnz = int(indptr[-1])
+    data = (rng.random(nnz, dtype=np.float32) + np.float32(0.05))
+    got = _seg_sum(dev, indptr, data, 1)
+    want = np.array([data[indptr[s]:indptr[s + 1]].astype(np.float64).sum() for s in range(n)])
+    np.testing.assert_allclose(got, want, rtol=RTOL)
+    if nnz:
+        out = torch.empty(nnz, dtype=torch.float32, device=dev)
+        capi.segment_normalize(to_dev(indptr, dev), None, to_dev(data, dev), out)
+        want_n = data.astype(np.float64) / np.repeat(want, deg)
+        np.testing.assert_allclose(out.cpu().numpy(), want_n, rtol=RTOL)
+
+
 def test_segment_sum_edge_count_is_an_upper_bound(dev):
     # the data array may be longer than the offsets cover: the rest is not read into any sum
     indptr = np.array([0, 2000, 2003], dtype=np.int64)
