@@ -2,13 +2,15 @@
 """Timings of the operators around the headline path (one MI355X), one JSON line each.
 
 bench.py measures the GraphSAGE minibatch; this script times the other rows of the scope
-table at the sizes of their configurations -- induced-subgraph slicing, the doubly-compressed
-conversions, weighted sampling with and without replacement, the super-batch helpers, walks,
-SDDMM, segment sums, row slicing -- through the same C ABI (graph_sampling_amd/capi.py), with
-`algorithmic` = the bytes the operator must move at the least (stated per line) over the
-median of the timed calls.  Timing: torch.cuda.Event pairs on the current stream, which is the
-stream the C ABI is given; a call is all the launches of the operator, host reads included
-where the operator has one.
+table at the sizes of their configurations -- induced-subgraph slicing, format conversions,
+weighted sampling with and without replacement, list sampling, the super-batch helpers,
+walks, SDDMM, segment and COO sums, row slicing -- through the same C ABI
+(graph_sampling_amd/capi.py), with `algorithmic` = the bytes the operator must move at the
+least (stated per line) over the median of the timed calls, and four whole samplers (LADIES
+and GraphSAGE written against Matrix, as written and through jit.compile) by wall clock.
+Timing of the operators: torch.cuda.Event pairs on the current stream, which is the stream the
+C ABI is given; a call is all the launches of the operator, host reads included where the
+operator has one.
 """
 import argparse
 import json
