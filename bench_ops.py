@@ -172,6 +172,7 @@ def main():
         lambda: capi.unique_relabel([big], [big]),
         lambda o: (16_000_000 * 70, 16_000_000, "items"))
 
+    divisor = torch.rand(N, generator=gen, device=dev) + 0.5
     # ---- walks, SDDMM, segment sum at their configuration sizes ---------------------------------
     starts = rand_ids(1_000_000)
     run("random_walk", "gs_random_walk: 1M walkers x 80 steps on this graph; 28 B per live step",
@@ -200,7 +201,6 @@ def main():
         lambda: capi.sddmm_coo("dot", er, ec, None, feat, feat, out_e, 0, 2, 64, 64, 1, 64, None, None),
         lambda o: (8_000_000 * 532, 8_000_000, "edges"))
     # Divide(divisor, axis=0) on the CSC: out[e] = w[e] / divisor[column of e], scalar per edge
-    divisor = torch.rand(N, generator=gen, device=dev) + 0.5
     out_w = torch.empty(E, 1, device=dev)
     run("sddmm_div_csc", "gs_sddmm_csc e_div_v over the whole graph (edge weight / per-column scalar): "
         "4 B read + 4 B written per edge, 12 B per column",
@@ -230,6 +230,13 @@ def main():
     run("coo_sum", "gs_coo_sum of w^2 over the rows of a 512-column slice's edges into 2.45M sums",
         lambda: capi.coo_sum(indices[:2_000_000], None, weights[:2_000_000], 2, out_p),
         lambda o: (2_000_000 * (b + 4 + 8), 2_000_000, "edges"))
+    coo_cols2m = capi.csc2coo(indptr, E, idt)[:2_000_000]
+    out_c = torch.zeros(N, device=dev)
+    out_d = torch.empty(2_000_000, device=dev)
+    run("e_div_u_sum", "gs_e_div_u_sum over the same 2M edges: w / divisor[row], summed per column",
+        lambda: capi.e_div_u_sum(indices[:2_000_000], coo_cols2m, weights[:2_000_000], divisor,
+                                 out_d, out_c),
+        lambda o: (2_000_000 * (2 * b + 4 + 4 + 4 + 8), 2_000_000, "edges"))
     out_nrm = torch.empty(E, device=dev)
     run("segment_normalize", "gs_segment_normalize over every column of the graph; 4 B read twice + "
         "4 B written per edge, 16 B per column",
