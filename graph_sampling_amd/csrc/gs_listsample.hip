@@ -79,6 +79,7 @@ struct SelectState {
   unsigned long long prefix;     // digits chosen so far, in place
   unsigned long long remaining;  // how many of the matching items are still wanted
   unsigned long long gathered;   // survivor counter
+  unsigned long long done;       // every item under the prefix is wanted: lower digits do not matter
 };
 
 __device__ __forceinline__ unsigned long long list_composite(uint32_t okey, int64_t i) {
@@ -92,6 +93,7 @@ select_init_kernel(uint32_t* hist, SelectState* st, int64_t k) {
     st->prefix = 0;
     st->remaining = static_cast<unsigned long long>(k);
     st->gathered = 0;
+    st->done = 0;
   }
 }
 
@@ -129,6 +131,7 @@ __global__ void __launch_bounds__(kThreads)
 level_hist_kernel(const uint32_t* __restrict__ okey, int64_t n, int level,
                   const SelectState* __restrict__ st, uint32_t* __restrict__ hist) {
   __shared__ uint32_t s_hist[kBins];
+  if (st->done) return;  // the pick of an earlier level took its whole bin: nothing left to split
   for (int i = threadIdx.x; i < kBins; i += kThreads) s_hist[i] = 0;
   __syncthreads();
   const unsigned long long prefix = st->prefix;
@@ -150,6 +153,7 @@ level_hist_kernel(const uint32_t* __restrict__ okey, int64_t n, int level,
 __global__ void __launch_bounds__(kThreads)
 level_pick_kernel(const uint32_t* __restrict__ hist, int level, SelectState* st) {
   __shared__ unsigned long long s_tail[kThreads];  // items in the bins owned by threads > t
+  if (st->done) return;
   const unsigned long long want = st->remaining;   // read before anyone updates it
   const uint32_t* h = hist + level * kBins;
   constexpr int kPer = kBins / kThreads;  // 8 consecutive bins per thread
@@ -174,6 +178,9 @@ level_pick_kernel(const uint32_t* __restrict__ hist, int level, SelectState* st)
       if (want <= above + cnt) {
         st->prefix |= static_cast<unsigned long long>(threadIdx.x * kPer + j) << c_shift[level];
         st->remaining = want - above;
+        // all of the bin is wanted (typically a bin of one): with the lower digits left at zero
+        // "composite >= prefix" already selects exactly the wanted items
+        if (want - above == cnt) st->done = 1;
         break;
       }
       above += cnt;
