@@ -393,8 +393,11 @@ int gs_sddmm_csc(int op, const int64_t* indptr, const void* indices, int id_byte
 size_t gs_segment_workspace_bytes(int64_t num_segments, int64_t nnz);
 
 /* out[n_ids ? n_ids[s] : s] = sum over segment s of data[e_ids ? e_ids[e] : e]^powk.
- * A segment of at most 16 edges is summed in edge order; a longer one in 64-edge pieces
- * aligned to the edge array (a fixed order, but not the sequential one). */
+ * Replaces impl::CSCSumCUDA (src/cuda/graph_ops.cu:92).  nnz: number of edges the offsets
+ * cover (an upper bound will do).  A segment of at most 16 edges is summed in edge order; a
+ * longer one by 1024-edge chunks of the edge array, four edges per lane, pieces across chunk
+ * borders added in chunk order: a fixed order that depends on the layout only, but not the
+ * sequential one. */
 int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const void* n_ids, int id_bytes,
                    const float* data, int64_t num_segments, int64_t nnz, int64_t powk, float* out,
                    void* workspace, size_t workspace_bytes, void* stream);
