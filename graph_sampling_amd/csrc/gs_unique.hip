@@ -715,7 +715,52 @@ int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* 
 
 using namespace gs;
 
+namespace gs {
+namespace {
+// kind: 0 compare-and-swap, 1 atomic minimum, 2 read, 3 write
+template <int KIND>
+__global__ void __launch_bounds__(kThreads)
+probe_kernel(unsigned long long* __restrict__ table, uint32_t mask,
+             const uint32_t* __restrict__ keys, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t key = keys[i];
+  unsigned long long* slot = table + (fib_home(key, 32) & mask);
+  const unsigned long long word = (static_cast<unsigned long long>(key) << 32) | static_cast<uint32_t>(i);
+  if (KIND == 0) {
+    if (atomicCAS(slot, ~0ull, word) == 1ull) table[0] = 0ull;  // keeps the result alive
+  } else if (KIND == 1) {
+    if (atomicMin(slot, word) == 1ull) table[0] = 0ull;
+  } else if (KIND == 2) {
+    if (*slot == 1ull) table[0] = 0ull;
+  } else {
+    *slot = word;
+  }
+}
+}  // namespace
+}  // namespace gs
+
 extern "C" {
+
+int gs_probe_random_access(int kind, uint64_t* table, int64_t slots, const uint32_t* keys,
+                           int64_t n, void* stream) {
+  GS_REQUIRE(kind >= 0 && kind <= 3, "gs_probe_random_access: kind must be 0..3, got %d", kind);
+  GS_REQUIRE(table && keys && n >= 0 && slots >= 1 && slots <= (int64_t(1) << 32) &&
+                 (slots & (slots - 1)) == 0,
+             "gs_probe_random_access: null pointer or a slot count that is not a power of two");
+  if (n == 0) return GS_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  unsigned long long* t = reinterpret_cast<unsigned long long*>(table);
+  const uint32_t mask = static_cast<uint32_t>(slots - 1);
+  const dim3 grid(blocks_for(n, kThreads)), block(kThreads);
+  switch (kind) {
+    case 0: hipLaunchKernelGGL(probe_kernel<0>, grid, block, 0, st, t, mask, keys, n); break;
+    case 1: hipLaunchKernelGGL(probe_kernel<1>, grid, block, 0, st, t, mask, keys, n); break;
+    case 2: hipLaunchKernelGGL(probe_kernel<2>, grid, block, 0, st, t, mask, keys, n); break;
+    default: hipLaunchKernelGGL(probe_kernel<3>, grid, block, 0, st, t, mask, keys, n); break;
+  }
+  return check_launch("probe_random_access");
+}
 
 size_t gs_unique_workspace_bytes(int64_t M) {
   if (M < 0) M = 0;

@@ -85,6 +85,13 @@ int gs_profile_enable(const char* launch_site);
 int gs_profile_stride(int every);
 int gs_profile_collect(double* total_ms, int64_t* launches, double* per_launch_ms, int64_t cap);
 
+/* Memory-system probe for benchmarks (no counterpart in the reference): n accesses of 8 bytes
+ * at hashed positions of a table of `slots` 64-bit words (a power of two), one per key, so
+ * that the rates of the hash-table kernels can be read against what the memory system gives:
+ * kind 0 = compare-and-swap, 1 = atomic minimum, 2 = plain read, 3 = plain write. */
+int gs_probe_random_access(int kind, uint64_t* table, int64_t slots, const uint32_t* keys,
+                           int64_t n, void* stream);
+
 typedef enum gs_op {
   GS_OP_ADD = 0, GS_OP_SUB = 1, GS_OP_MUL = 2, GS_OP_DIV = 3,
   GS_OP_COPY_LHS = 4, GS_OP_COPY_RHS = 5, GS_OP_DOT = 6
