@@ -279,15 +279,18 @@ def sample_uniform_fused(indptr, indices, column_ids, fanout, replace, seed=0, r
 class RelabelTable:
     """The persistent hash table of gs_relabel_sampled (prepared once, left empty by every call)."""
 
-    def __init__(self, max_items, id_dtype, device):
+    def __init__(self, max_items, id_dtype, device, narrow=False):
+        """narrow: 64-bit ids on the one-word slots of 32-bit ids (gs_relabel_sampled_narrow)."""
         self.idb = 8 if id_dtype == torch.int64 else 4
+        self.narrow = bool(narrow) and self.idb == 8
         nbytes = lib().gs_relabel_table_bytes(_i64(max_items), self.idb)
         self.buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
         self.prepare()
 
     def prepare(self):
         _check(lib().gs_relabel_table_init(_ptr(self.buf), ctypes.c_size_t(self.buf.numel()),
-                                           self.idb, _stream(self.buf.device)),
+                                           4 if self.narrow else self.idb,
+                                           _stream(self.buf.device)),
                "gs_relabel_table_init")
 
 
@@ -306,14 +309,23 @@ def relabel_sampled(seed_keys, sub_indptr, sub_indices, table, mailbox=None, off
     ws = workspace(lib().gs_relabel_sampled_workspace_bytes(_i64(M)), dev)
     state, epoch = fused_state(lib().gs_relabel_sampled_state_bytes(_i64(M)), dev)
     ticket = mailbox.ticket() if mailbox is not None else 0
-    _check(lib().gs_relabel_sampled(
-        _ptr(seed_keys), _i64(S), _ptr(sub_indices), _i64(cap),
-        ctypes.c_void_p(sub_indptr.data_ptr() + 8 * S), idb, _ptr(table.buf),
-        ctypes.c_size_t(table.buf.numel()), _ptr(frontier), _ptr(out_ids), _ptr(num_unique),
-        _ptr(offsets_copy),
-        _ptr(ws), ctypes.c_size_t(ws.numel()), _ptr(state), ctypes.c_size_t(state.numel()),
-        ctypes.c_uint32(epoch), mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0),
-        _i64(ticket), _stream(dev)), "gs_relabel_sampled")
+    box = mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0)
+    if table.narrow:
+        _check(lib().gs_relabel_sampled_narrow(
+            _ptr(seed_keys), _i64(S), _ptr(sub_indices), _i64(cap),
+            ctypes.c_void_p(sub_indptr.data_ptr() + 8 * S), _ptr(table.buf),
+            ctypes.c_size_t(table.buf.numel()), _ptr(frontier), _ptr(out_ids), _ptr(num_unique),
+            _ptr(offsets_copy), _ptr(ws), ctypes.c_size_t(ws.numel()), _ptr(state),
+            ctypes.c_size_t(state.numel()), ctypes.c_uint32(epoch), box, _i64(ticket),
+            _stream(dev)), "gs_relabel_sampled_narrow")
+    else:
+        _check(lib().gs_relabel_sampled(
+            _ptr(seed_keys), _i64(S), _ptr(sub_indices), _i64(cap),
+            ctypes.c_void_p(sub_indptr.data_ptr() + 8 * S), idb, _ptr(table.buf),
+            ctypes.c_size_t(table.buf.numel()), _ptr(frontier), _ptr(out_ids), _ptr(num_unique),
+            _ptr(offsets_copy), _ptr(ws), ctypes.c_size_t(ws.numel()), _ptr(state),
+            ctypes.c_size_t(state.numel()), ctypes.c_uint32(epoch), box, _i64(ticket),
+            _stream(dev)), "gs_relabel_sampled")
     if mailbox is not None:
         return frontier, num_unique, out_ids, ticket
     return frontier, num_unique, out_ids

@@ -23,6 +23,8 @@
 //    so every relabel lookup is two gathers in a last kernel, and a query that
 //    aliases a mapping span is relabelled by slot gather instead of probing.
 #include "gs_common.hpp"
+#include <type_traits>
+
 #include "gs_table.hpp"
 
 namespace gs {
@@ -71,15 +73,23 @@ __global__ void __launch_bounds__(kThreads) table_init_kernel(T t, int64_t cap, 
 
 // insert (key -> min index) and remember the slot of every item
 // (unique_reindex.cu:92-99)
+// too_wide: set to 2 when T keeps 32 bits of a key and a key does not fit them (64-bit ids
+// on the one-word slots); the compaction then reports -2 instead of a count
 template <typename IdT, typename T, bool PEEK>
 __global__ void __launch_bounds__(kThreads)
-table_insert_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ pos) {
+table_insert_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ pos,
+                    unsigned int* __restrict__ too_wide) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= M_bound) return;
   // the key is read before the device-side length is known (the buffers hold M_bound items
   // whatever the length turns out to be): one round trip instead of two
   const IdT key = x.get(i);
   if (i >= x.items(M_bound)) return;
+  if (sizeof(IdT) == 8 && too_wide && (static_cast<unsigned long long>(key) >> 32) != 0ull) {
+    *too_wide = 2u;
+    pos[i] = 0u;
+    return;
+  }
   pos[i] = t.template insert<PEEK>(static_cast<long long>(key), static_cast<uint32_t>(i));
 }
 
@@ -147,7 +157,8 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
   }
   if (tile == gridDim.x - 1 && threadIdx.x == 0) {
     int64_t total = s_prefix + tile_total;
-    if (__hip_atomic_load(lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) total = -1;
+    const unsigned int err = __hip_atomic_load(lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (err) total = err == 2u ? -2 : -1;  // 2: a key did not fit the one-word slots
     *num_unique = total;
     post_mailbox(box, total, box_ticket);
   }
@@ -294,7 +305,7 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   if (M > 0) {
     ProfileScope prof("table_insert", stream);
     hipLaunchKernelGGL((table_insert_kernel<IdT, T, true>), dim3(blocks_for(M, kThreads)),
-                       dim3(kThreads), 0, stream, x, M, t, pos);
+                       dim3(kThreads), 0, stream, x, M, t, pos, static_cast<unsigned int*>(nullptr));
   }
   {
     ProfileScope prof("unique_compact", stream);
@@ -311,14 +322,13 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
 }
 
 
-template <typename IdT>
+template <typename IdT, typename T>
 int relabel_sampled_impl(const void* seed_keys, int64_t S, const void* sampled, int64_t capacity,
                          const int64_t* sampled_len, void* table, size_t table_bytes,
                          void* frontier, void* out_ids, int64_t* num_unique,
                          int64_t* offsets_copy, void* workspace,
                          size_t workspace_bytes, void* state, size_t state_bytes, uint32_t epoch,
                          gs_mailbox* box, int64_t box_ticket, hipStream_t stream) {
-  using T = typename TableFor<IdT>::type;
   const int64_t M = S + capacity;
   T t;
   if (!shape_linked_table<T>(table, table_bytes, M, &t)) {
@@ -355,8 +365,10 @@ int relabel_sampled_impl(const void* seed_keys, int64_t S, const void* sampled, 
     ProfileScope prof("table_insert", stream);
     // no peek here: sampled neighbours are mostly new keys, and the extra read costs the
     // GraphSAGE step 7 % (0.152 ms against 0.142)
+    constexpr bool kNarrow = sizeof(IdT) == 8 && std::is_same<T, PackedTable>::value;
     hipLaunchKernelGGL((table_insert_kernel<IdT, T, false>), dim3(blocks_for(M, kThreads)),
-                       dim3(kThreads), 0, stream, x, M, t, pos);
+                       dim3(kThreads), 0, stream, x, M, t, pos,
+                       kNarrow ? lb.error : static_cast<unsigned int*>(nullptr));
   }
   {
     ProfileScope prof("unique_compact", stream);
@@ -949,14 +961,39 @@ int gs_relabel_sampled(const void* seed_keys, int64_t S, const void* sampled, in
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   return id_bytes == 8
-             ? relabel_sampled_impl<int64_t>(seed_keys, S, sampled, capacity, sampled_len, table,
-                                             table_bytes, frontier, out_ids, num_unique, offsets_copy,
-                                             workspace, workspace_bytes, state, state_bytes, epoch, mailbox,
-                                             mailbox_ticket, st)
-             : relabel_sampled_impl<int32_t>(seed_keys, S, sampled, capacity, sampled_len, table,
-                                             table_bytes, frontier, out_ids, num_unique, offsets_copy,
-                                             workspace, workspace_bytes, state, state_bytes, epoch, mailbox,
-                                             mailbox_ticket, st);
+             ? relabel_sampled_impl<int64_t, WideTable>(
+                   seed_keys, S, sampled, capacity, sampled_len, table, table_bytes, frontier,
+                   out_ids, num_unique, offsets_copy, workspace, workspace_bytes, state,
+                   state_bytes, epoch, mailbox, mailbox_ticket, st)
+             : relabel_sampled_impl<int32_t, PackedTable>(
+                   seed_keys, S, sampled, capacity, sampled_len, table, table_bytes, frontier,
+                   out_ids, num_unique, offsets_copy, workspace, workspace_bytes, state,
+                   state_bytes, epoch, mailbox, mailbox_ticket, st);
+}
+
+int gs_relabel_sampled_narrow(const void* seed_keys, int64_t S, const void* sampled,
+                              int64_t capacity, const int64_t* sampled_len, void* table,
+                              size_t table_bytes, void* frontier, void* out_ids,
+                              int64_t* num_unique, int64_t* offsets_copy, void* workspace,
+                              size_t workspace_bytes, void* state, size_t state_bytes,
+                              uint32_t epoch, gs_mailbox* mailbox, int64_t mailbox_ticket,
+                              void* stream) {
+  GS_REQUIRE(S >= 0 && capacity >= 0 && sampled_len && table && num_unique && state,
+             "gs_relabel_sampled_narrow: null pointer or negative size");
+  GS_REQUIRE((S == 0 || seed_keys) && (capacity == 0 || (sampled && out_ids)) &&
+                 (S + capacity == 0 || frontier),
+             "gs_relabel_sampled_narrow: null buffer");
+  GS_REQUIRE(epoch >= 1 && epoch <= kLbMaxEpoch,
+             "gs_relabel_sampled_narrow: epoch must be in 1..%u", kLbMaxEpoch);
+  if (S + capacity >= (int64_t(1) << 31)) {
+    set_error_text("gs_relabel_sampled_narrow: %lld items exceed the supported 2^31",
+                   static_cast<long long>(S + capacity));
+    return GS_ERR_UNSUPPORTED;
+  }
+  return relabel_sampled_impl<int64_t, PackedTable>(
+      seed_keys, S, sampled, capacity, sampled_len, table, table_bytes, frontier, out_ids,
+      num_unique, offsets_copy, workspace, workspace_bytes, state, state_bytes, epoch, mailbox,
+      mailbox_ticket, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -73,7 +73,8 @@ torch::Tensor Scratch(size_t bytes, const torch::Tensor& like) {
 // to slot t % kBoxes, so a total stays readable until kBoxes later calls have
 // been issued.
 constexpr int64_t kBoxes = 64;
-constexpr int64_t kLost = -2;  // the slot was reused before anyone read it
+constexpr int64_t kLost = -3;     // the slot was reused before anyone read it
+constexpr int64_t kTooWide = -2;  // posted by the narrow relabel: a key needs more than 32 bits
 
 struct HostBoxes {
   torch::Tensor buf;  // kBoxes x {total, ticket}, pinned
@@ -116,7 +117,8 @@ int64_t WaitBox(const gs_mailbox* box, int64_t ticket, void* stream, const char*
   const int64_t total = __atomic_load_n(&box->total, __ATOMIC_RELAXED);
   // the slot may have been rewritten between the two loads
   if (__atomic_load_n(&box->ticket, __ATOMIC_ACQUIRE) != ticket) return kLost;
-  TORCH_CHECK(total >= 0, what, ": a tile gave up waiting for its predecessors");
+  TORCH_CHECK(total >= 0 || total == kTooWide, what,
+              ": a tile gave up waiting for its predecessors");
   return total;
 }
 
@@ -150,6 +152,9 @@ struct RelabelTable {
   torch::Tensor buf;
   int64_t items = 0;   // number of mapping items it was sized for
   bool clean = false;  // false: has to be prepared before the next use
+  // 64-bit ids on the one-word slots of 32-bit ids (gs_relabel_sampled_narrow) until a key
+  // turns up that does not fit 32 bits
+  bool narrow = true;
 };
 
 RelabelTable& RelabelTableFor(const torch::Tensor& like, void* stream, int idb, int64_t items) {
@@ -164,7 +169,8 @@ RelabelTable& RelabelTableFor(const torch::Tensor& like, void* stream, int idb, 
     t.clean = false;
   }
   if (!t.clean) {
-    Check(gs_relabel_table_init(t.buf.data_ptr(), t.buf.numel(), idb, stream),
+    Check(gs_relabel_table_init(t.buf.data_ptr(), t.buf.numel(), idb == 8 && t.narrow ? 4 : idb,
+                                stream),
           "gs_relabel_table_init");
     t.clean = true;
   }
@@ -484,18 +490,40 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred
   RelabelTable& table = RelabelTableFor(col_ids, p.stream, idb, M);
   FusedStateBuf& state = FusedState(gs_relabel_sampled_state_bytes(M), col_ids, p.stream);
   HostBoxes& boxes = Boxes(p.device);
-  const int64_t ticket = boxes.next++;
-  table.clean = false;  // until both totals have come back
-  Check(gs_relabel_sampled(col_ids.data_ptr(), S, p.indices.data_ptr(), cap,
-                           p.sub_indptr.data_ptr<int64_t>() + p.S, idb, table.buf.data_ptr(),
-                           table.buf.numel(), frontier.data_ptr(), renamed.data_ptr(),
-                           num.data_ptr<int64_t>(), offsets_copy.data_ptr<int64_t>(), ws.data_ptr(),
-                           ws.numel(), state.buf.data_ptr(), state.buf.numel(), state.epoch,
-                           boxes.slot(ticket), ticket, p.stream),
-        "gs_relabel_sampled");
-  const int64_t nnz = p.Wait();
-  int64_t U = WaitBox(boxes.slot(ticket), ticket, p.stream, "gs_relabel_sampled");
-  if (U == kLost) U = num.item<int64_t>();
+  int64_t nnz = -1, U = kTooWide;
+  for (int attempt = 0; attempt < 2 && U == kTooWide; ++attempt) {
+    const int64_t ticket = boxes.next++;
+    table.clean = false;  // until both totals have come back
+    if (idb == 8 && table.narrow) {
+      Check(gs_relabel_sampled_narrow(col_ids.data_ptr(), S, p.indices.data_ptr(), cap,
+                                      p.sub_indptr.data_ptr<int64_t>() + p.S, table.buf.data_ptr(),
+                                      table.buf.numel(), frontier.data_ptr(), renamed.data_ptr(),
+                                      num.data_ptr<int64_t>(), offsets_copy.data_ptr<int64_t>(),
+                                      ws.data_ptr(), ws.numel(), state.buf.data_ptr(),
+                                      state.buf.numel(), state.epoch, boxes.slot(ticket), ticket,
+                                      p.stream),
+            "gs_relabel_sampled_narrow");
+    } else {
+      Check(gs_relabel_sampled(col_ids.data_ptr(), S, p.indices.data_ptr(), cap,
+                               p.sub_indptr.data_ptr<int64_t>() + p.S, idb, table.buf.data_ptr(),
+                               table.buf.numel(), frontier.data_ptr(), renamed.data_ptr(),
+                               num.data_ptr<int64_t>(), offsets_copy.data_ptr<int64_t>(),
+                               ws.data_ptr(), ws.numel(), state.buf.data_ptr(), state.buf.numel(),
+                               state.epoch, boxes.slot(ticket), ticket, p.stream),
+            "gs_relabel_sampled");
+    }
+    if (nnz < 0) nnz = p.Wait();
+    U = WaitBox(boxes.slot(ticket), ticket, p.stream, "gs_relabel_sampled");
+    if (U == kLost) U = num.item<int64_t>();
+    if (U == kTooWide) {
+      // an id beyond 32 bits: from now on this table takes the two-array slots
+      TORCH_CHECK(idb == 8 && table.narrow, "gs_relabel_sampled: unexpected status");
+      table.narrow = false;
+      state.buf.zero_();  // the error word is sticky
+      RelabelTableFor(col_ids, p.stream, idb, M);                               // prepares it again
+      FusedState(gs_relabel_sampled_state_bytes(M), col_ids, p.stream);       // next epoch
+    }
+  }
   TORCH_CHECK(U >= 0, "gs_relabel_sampled: a tile gave up waiting for its predecessors");
   table.clean = true;
   return {frontier.narrow(0, 0, U), renamed.narrow(0, 0, nnz), nnz, offsets_copy};

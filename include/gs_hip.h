@@ -323,6 +323,22 @@ int gs_relabel_sampled(const void* seed_keys, int64_t S, const void* sampled, in
                        size_t workspace_bytes, void* state, size_t state_bytes, uint32_t epoch,
                        gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
 
+/* gs_relabel_sampled for 64-bit ids whose values fit 32 bits (node ids of any graph below
+ * 4.29 G nodes): the table is used with the one-word slots of 32-bit ids -- one
+ * compare-and-swap per insert instead of compare-and-swap, read and minimum -- while ids,
+ * frontier and out_ids stay 64-bit.  The table must have been prepared with
+ * gs_relabel_table_init(..., id_bytes = 4) (a buffer sized by gs_relabel_table_bytes(..., 8)
+ * is large enough for both layouts).  If a key does not fit, *num_unique and the mailbox read
+ * -2, nothing else written is valid, and the error word of `state` stays set: zero `state`,
+ * prepare the table again with id_bytes = 8 and call gs_relabel_sampled. */
+int gs_relabel_sampled_narrow(const void* seed_keys, int64_t S, const void* sampled,
+                              int64_t capacity, const int64_t* sampled_len, void* table,
+                              size_t table_bytes, void* frontier, void* out_ids,
+                              int64_t* num_unique, int64_t* offsets_copy, void* workspace,
+                              size_t workspace_bytes, void* state, size_t state_bytes,
+                              uint32_t epoch, gs_mailbox* mailbox, int64_t mailbox_ticket,
+                              void* stream);
+
 /* B relabels in one pass ("super-batch"): replaces impl::BatchCSRRelabelCUDA
  * (src/cuda/batch_relabel.cu:331).  Batch b owns seeds[seeds_ptr[b]..seeds_ptr[b+1])
  * and ids[ids_ptr[b]..ids_ptr[b+1]) (both *_ptr: device int64[num_batches+1]).

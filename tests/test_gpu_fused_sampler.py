@@ -215,3 +215,30 @@ def test_relabel_sampled_matches_the_one_call_relabel(dev, S, fanout, replace, i
         slots = words.numel() * 8 // 12 // 1024 * 1024     # keys (8 B) then first indices (4 B)
         cap = 1 << (slots.bit_length() - 1)
         assert bool((words[:cap] == -1).all())
+
+
+def test_relabel_sampled_narrow_slots_for_64_bit_ids(dev):
+    """64-bit ids that fit 32 bits on the one-word slots: same frontier and renamed ids as the
+    two-array table; an id beyond 32 bits is reported (-2) instead of being truncated."""
+    n = 1 << 13
+    indptr, indices = rmat_csc_np(n, 1 << 17, seed=9)
+    cols = np.random.default_rng(4).integers(0, n, size=900).astype(np.int64)
+    t_ptr, t_idx, t_cols = to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev)
+    narrow = capi.RelabelTable(900 * 11 + 50000, torch.int64, dev, narrow=True)
+    for shift in (0, 4_000_000_000, (1 << 33)):           # the last one does not fit 32 bits
+        keys = cols + shift
+        t_keys = to_dev(keys, dev)
+        sp, si, _, _ = capi.sample_uniform_fused(t_ptr, t_idx, t_cols, 10, False, seed=3)
+        w_sp, _, w_si, _ = O.sample_uniform(indptr, indices, cols, 10, False, seed=3, with_coo=False)
+        frontier, num, out = capi.relabel_sampled(t_keys, sp, si, narrow)
+        if shift == (1 << 33):
+            assert int(num.item()) == -2
+            break
+        w_frontier, (w_out,) = O.relabel([keys, w_si], [w_si])
+        E = int(w_sp[-1])
+        assert int(num.item()) == w_frontier.size
+        assert np.array_equal(frontier[:w_frontier.size].cpu().numpy(), w_frontier)
+        assert np.array_equal(out[:E].cpu().numpy(), w_out)
+    torch.cuda.synchronize()
+    # the sticky error word of the look-back state must not leak into later calls of this process
+    capi._fused_state.clear()

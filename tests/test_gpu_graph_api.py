@@ -816,3 +816,31 @@ def test_sample_blocks_rejects_bad_arguments(dev):
         gs.sample_blocks(m, [seeds, seeds], [3, -1], workers=2)
     nodes, blocks = gs.sample_blocks(m, [seeds], [3], workers=2)[0]
     assert blocks[0].num_dst_nodes() == 10 and nodes.numel() == blocks[0].num_src_nodes()
+
+
+def test_relabel_falls_back_when_64_bit_ids_exceed_32_bits(dev):
+    """Graph.Relabel behind the fused sampler uses one-word table slots for 64-bit ids; column ids
+    beyond 32 bits make it switch to the two-array slots, with the same result as the oracle."""
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 16, seed=13)
+    big = np.int64(1) << 35
+    g = gs.Graph(False)
+    col_ids = np.arange(1 << 12, dtype=np.int64) + big        # the columns go by huge ids
+    g._CAPI_LoadCSCWithColIds(to_dev(col_ids, dev), to_dev(indptr, dev), to_dev(indices, dev))
+    seeds = np.random.default_rng(2).permutation(1 << 12)[:300].astype(np.int64)
+    for rep in range(2):  # the second call runs on the switched table
+        gs.set_seed(90 + rep)
+        sub = g._CAPI_FusedColumnwiseSlicingSampling(to_dev(seeds, dev), 6, False)
+        frontier, n_src, n_dst, ptr, idx, _, fmt = sub._CAPI_Relabel()
+        sp, _, rows, _ = O.sample_uniform(indptr, indices, seeds, 6, False, seed=90 + rep, with_coo=False)
+        w_frontier, (w_idx,) = O.relabel([col_ids[seeds], rows], [rows])
+        assert np.array_equal(frontier.cpu().numpy(), w_frontier)
+        assert np.array_equal(idx.cpu().numpy(), w_idx)
+        assert np.array_equal(ptr.cpu().numpy(), sp)
+    # ids that fit again keep working on the switched table
+    g2 = gs.Graph(False)
+    g2._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev))
+    gs.set_seed(95)
+    sub = g2._CAPI_FusedColumnwiseSlicingSampling(to_dev(seeds, dev), 6, False)
+    frontier = sub._CAPI_Relabel()[0]
+    sp, _, rows, _ = O.sample_uniform(indptr, indices, seeds, 6, False, seed=95, with_coo=False)
+    assert np.array_equal(frontier.cpu().numpy(), O.relabel([seeds, rows], [rows])[0])
