@@ -448,14 +448,17 @@ class _Span(ctypes.Structure):
     _fields_ = [("ptr", ctypes.c_void_p), ("n", ctypes.c_int64)]
 
 
-def unique_relabel(mapping, queries, mailbox=None, last_span_len=None):
+NARROW_IDS = 0x100  # GS_NARROW_IDS: 64-bit ids that fit 32 bits, on one-word table slots
+
+
+def unique_relabel(mapping, queries, mailbox=None, last_span_len=None, narrow=False):
     """gs_unique_relabel[_notify].  mapping / queries: lists of 1-D id tensors (one dtype).
 
     Returns (frontier_buf, num_unique_dev, [relabelled query tensors]); frontier_buf has
     capacity sum(len(mapping)) and num_unique_dev is a 1-element int64 device tensor.  With a
     Mailbox the ticket to wait on is appended."""
     dev = mapping[0].device
-    idb = _ids(mapping[0], "mapping[0]")
+    idb = _ids(mapping[0], "mapping[0]") | (NARROW_IDS if narrow else 0)
     for i, t in enumerate(list(mapping[1:]) + list(queries)):
         _ids(t, "relabel tensor %d" % (i + 1), like=mapping[0])
     M = sum(int(t.numel()) for t in mapping)
@@ -486,10 +489,10 @@ def unique_relabel(mapping, queries, mailbox=None, last_span_len=None):
     return frontier, num_unique, outs
 
 
-def batch_csr_relabel(seeds, seeds_ptr, ids, ids_ptr, mailbox=None):
+def batch_csr_relabel(seeds, seeds_ptr, ids, ids_ptr, mailbox=None, narrow=False):
     """gs_batch_csr_relabel.  Returns (unique_buf, unique_ptr, relabelled ids, num_unique_dev
     [, ticket]); unique_buf has the capacity len(seeds) + len(ids)."""
-    idb = _ids(seeds, "seeds")
+    idb = _ids(seeds, "seeds") | (NARROW_IDS if narrow else 0)
     _ids(ids, "ids", like=seeds)
     _need(seeds_ptr, torch.int64, "seeds_ptr")
     _need(ids_ptr, torch.int64, "ids_ptr")
@@ -513,9 +516,9 @@ def batch_csr_relabel(seeds, seeds_ptr, ids, ids_ptr, mailbox=None):
     return unique, unique_ptr, out_ids, num_unique
 
 
-def batch_coo_relabel(seeds, seeds_ptr, coo_row, coo_col, coo_ptr):
+def batch_coo_relabel(seeds, seeds_ptr, coo_row, coo_col, coo_ptr, narrow=False):
     """gs_batch_coo_relabel.  Returns (unique_buf, unique_ptr, out_row, out_col, num_unique_dev)."""
-    idb = _ids(seeds, "seeds")
+    idb = _ids(seeds, "seeds") | (NARROW_IDS if narrow else 0)
     _ids(coo_row, "coo_row", like=seeds)
     _ids(coo_col, "coo_col", like=seeds)
     _need(seeds_ptr, torch.int64, "seeds_ptr")

@@ -168,7 +168,7 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
 template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
 lookup_kernel(T t, const uint32_t* __restrict__ pos, const int64_t* __restrict__ prefix, Query qs,
-              int64_t Q_bound, const int64_t* __restrict__ q_len) {
+              int64_t Q_bound, const int64_t* __restrict__ q_len, int64_t M) {
   const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   int64_t Q = Q_bound;
   if (q_len) {  // one query that aliases the device-sized last mapping span
@@ -190,9 +190,15 @@ lookup_kernel(T t, const uint32_t* __restrict__ pos, const int64_t* __restrict__
   if (qs.alias[s] >= 0) {
     first = t.first_index(pos[qs.alias[s] + local]);
   } else {
-    first = t.find(static_cast<long long>(static_cast<const IdT*>(qs.in[s])[local]));
+    const IdT key = static_cast<const IdT*>(qs.in[s])[local];
+    const bool fits = sizeof(IdT) == 4 || !std::is_same<T, PackedTable>::value ||
+                      (static_cast<unsigned long long>(key) >> 32) == 0ull;
+    first = fits ? t.find(static_cast<long long>(key)) : -1;
   }
-  static_cast<IdT*>(qs.out[s])[local] = static_cast<IdT>(first < 0 ? -1 : prefix[first]);
+  // first >= M only when the insert pass gave up (an id too wide for the slots): the outputs
+  // are void then, but no index may leave the arrays
+  static_cast<IdT*>(qs.out[s])[local] =
+      static_cast<IdT>(first < 0 || first >= M ? -1 : prefix[first]);
 }
 
 // Last pass of a relabel on a table that outlives the call (gs_relabel_sampled): item i >= S is
@@ -240,12 +246,11 @@ size_t workspace_bytes_for(int64_t M) {
          lookback_state_bytes(compact_num_tiles(M));
 }
 
-template <typename IdT>
+template <typename IdT, typename T>
 int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* query,
                         void* const* query_out, int n_query, void* frontier, int64_t* num_unique,
                         void* workspace, size_t workspace_bytes, const int64_t* last_span_len,
                         gs_mailbox* box, int64_t box_ticket, hipStream_t stream) {
-  using T = typename TableFor<IdT>::type;
   Spans<IdT> x;
   int64_t M = 0;
   for (int s = 0; s < GS_MAX_SPANS; ++s) {
@@ -304,8 +309,10 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   }
   if (M > 0) {
     ProfileScope prof("table_insert", stream);
+    constexpr bool kNarrow = sizeof(IdT) == 8 && std::is_same<T, PackedTable>::value;
     hipLaunchKernelGGL((table_insert_kernel<IdT, T, true>), dim3(blocks_for(M, kThreads)),
-                       dim3(kThreads), 0, stream, x, M, t, pos, static_cast<unsigned int*>(nullptr));
+                       dim3(kThreads), 0, stream, x, M, t, pos,
+                       kNarrow ? lb.error : static_cast<unsigned int*>(nullptr));
   }
   {
     ProfileScope prof("unique_compact", stream);
@@ -316,7 +323,7 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   if (Q > 0) {
     ProfileScope prof("unique_finish", stream);
     hipLaunchKernelGGL((lookup_kernel<IdT, T>), dim3(blocks_for(Q, kThreads)), dim3(kThreads), 0,
-                       stream, t, pos, prefix, qs, Q, last_span_len);
+                       stream, t, pos, prefix, qs, Q, last_span_len, M);
   }
   return check_launch("unique_relabel");
 }
@@ -558,7 +565,8 @@ __global__ void __launch_bounds__(kThreads) regions_init_kernel(R t, int64_t cap
 
 template <typename IdT, typename R>
 __global__ void __launch_bounds__(kThreads)
-batch_insert_kernel(BatchItems<IdT> x, int64_t M, R t, uint32_t* __restrict__ pos) {
+batch_insert_kernel(BatchItems<IdT> x, int64_t M, R t, uint32_t* __restrict__ pos,
+                    unsigned int* __restrict__ too_wide) {
   __shared__ int64_t s_range[2];
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads;
   const int64_t last = first + kThreads - 1 < M ? first + kThreads - 1 : M - 1;
@@ -568,8 +576,14 @@ batch_insert_kernel(BatchItems<IdT> x, int64_t M, R t, uint32_t* __restrict__ po
   if (i >= M) return;
   const int64_t b = x.batch_of(i, lo, hi);
   const int64_t begin = x.start(b);
+  const IdT key = x.get_in(b, i);
+  if (sizeof(IdT) == 8 && too_wide && (static_cast<unsigned long long>(key) >> 32) != 0ull) {
+    *too_wide = 2u;  // 64-bit ids on one-word slots, and this one does not fit: reported as -2
+    pos[i] = static_cast<uint32_t>(kRegionFactor * begin);
+    return;
+  }
   pos[i] = t.insert(kRegionFactor * begin, kRegionFactor * (x.start(b + 1) - begin),
-                    static_cast<long long>(x.get_in(b, i)), static_cast<uint32_t>(i));
+                    static_cast<long long>(key), static_cast<uint32_t>(i));
 }
 
 // flags, chained scan and compaction over all batches at once (see compact_kernel)
@@ -620,7 +634,8 @@ batch_compact_kernel(BatchItems<IdT> x, int64_t M, R t, const uint32_t* __restri
   }
   if (tile == gridDim.x - 1 && threadIdx.x == 0) {
     int64_t total = s_prefix + tile_total;
-    if (__hip_atomic_load(lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) total = -1;
+    const unsigned int err = __hip_atomic_load(lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (err) total = err == 2u ? -2 : -1;
     *num_unique = total;
     post_mailbox(box, total, box_ticket);
   }
@@ -658,14 +673,20 @@ batch_finish_kernel(BatchItems<IdT> x, int64_t num_ids, int64_t M, R t,
     const int64_t b = lo;
     const int64_t begin = x.start(b);
     const int64_t p = begin + (x.seeds_ptr[b + 1] - x.seeds_ptr[b]) + (j - x.ids_ptr[b]);
-    out_ids[j] = static_cast<IdT>(prefix[t.first_index(pos[p])] - prefix[begin]);
+    // an index beyond M only when the insert pass gave up (an id too wide for the slots): the
+    // outputs are void then, but no index may leave the arrays
+    const uint32_t fi = t.first_index(pos[p]);
+    out_ids[j] = static_cast<IdT>(fi < M ? prefix[fi] - prefix[begin] : -1);
     if (extra) {
       // a second array cut like the ids (the other end of a COO edge): looked up, -1 if absent
-      const uint32_t slot = t.find(kRegionFactor * begin, kRegionFactor * (x.start(b + 1) - begin),
-                                   static_cast<long long>(extra[j]));
-      out_extra[j] = slot == 0xFFFFFFFFu
-                         ? IdT(-1)
-                         : static_cast<IdT>(prefix[t.first_index(slot)] - prefix[begin]);
+      const bool fits = sizeof(IdT) == 4 || !std::is_same<R, PackedRegions>::value ||
+                        (static_cast<unsigned long long>(extra[j]) >> 32) == 0ull;
+      const uint32_t slot =
+          fits ? t.find(kRegionFactor * begin, kRegionFactor * (x.start(b + 1) - begin),
+                        static_cast<long long>(extra[j]))
+               : 0xFFFFFFFFu;
+      const uint32_t fe = slot == 0xFFFFFFFFu ? 0xFFFFFFFFu : t.first_index(slot);
+      out_extra[j] = fe < M ? static_cast<IdT>(prefix[fe] - prefix[begin]) : IdT(-1);
     }
     return;
   }
@@ -680,14 +701,13 @@ size_t batch_workspace_bytes_for(int64_t M) {
          padded((M + 1) * 8) + lookback_state_bytes(compact_num_tiles(M));
 }
 
-template <typename IdT>
+template <typename IdT, typename R>
 int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* ids,
                        const int64_t* ids_ptr, int64_t B, int64_t num_seeds, int64_t num_ids,
                        void* unique, int64_t* unique_ptr, void* out_ids, int64_t* num_unique,
                        void* workspace, size_t workspace_bytes, gs_mailbox* box,
                        int64_t box_ticket, hipStream_t stream, const void* extra = nullptr,
                        void* out_extra = nullptr) {
-  using R = typename RegionsFor<IdT>::type;
   const int64_t M = num_seeds + num_ids;
   const int64_t cap = kRegionFactor * (M > 0 ? M : 1);
   Carver ws(workspace, workspace_bytes);
@@ -709,7 +729,10 @@ int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* 
                      0, stream, t, cap, lb, tiles);
   if (M > 0)
     hipLaunchKernelGGL((batch_insert_kernel<IdT, R>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
-                       0, stream, x, M, t, pos);
+                       0, stream, x, M, t, pos,
+                       sizeof(IdT) == 8 && std::is_same<R, PackedRegions>::value
+                           ? lb.error
+                           : static_cast<unsigned int*>(nullptr));
   hipLaunchKernelGGL((batch_compact_kernel<IdT, R>), dim3(static_cast<unsigned>(tiles)),
                      dim3(kThreads), 0, stream, x, M, t, pos, prefix, static_cast<IdT*>(unique),
                      num_unique, lb, box, box_ticket);
@@ -790,7 +813,10 @@ int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_spa
              "gs_unique_relabel: 1..%d mapping spans required, got %d", GS_MAX_SPANS, n_mapping);
   GS_REQUIRE(n_query >= 0 && n_query <= GS_MAX_SPANS && (n_query == 0 || (query && query_out)),
              "gs_unique_relabel: 0..%d query spans required, got %d", GS_MAX_SPANS, n_query);
-  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_unique_relabel: id_bytes must be 4 or 8, got %d", id_bytes);
+  const bool narrow = (id_bytes & GS_NARROW_IDS) != 0;
+  id_bytes &= ~GS_NARROW_IDS;
+  GS_REQUIRE(valid_id_bytes(id_bytes) && (!narrow || id_bytes == 8),
+             "gs_unique_relabel: id_bytes must be 4, 8 or 8 | GS_NARROW_IDS, got %d", id_bytes);
   GS_REQUIRE(num_unique, "gs_unique_relabel: num_unique is null");
   int64_t M = 0;
   for (int s = 0; s < n_mapping; ++s) {
@@ -814,13 +840,19 @@ int gs_unique_relabel_notify(const gs_span* mapping, int n_mapping, const gs_spa
                "the last mapping span itself");
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return id_bytes == 8
-             ? unique_relabel_impl<int64_t>(mapping, n_mapping, query, query_out, n_query, frontier,
-                                            num_unique, workspace, workspace_bytes, last_span_len,
-                                            mailbox, mailbox_ticket, st)
-             : unique_relabel_impl<int32_t>(mapping, n_mapping, query, query_out, n_query, frontier,
-                                            num_unique, workspace, workspace_bytes, last_span_len,
-                                            mailbox, mailbox_ticket, st);
+  if (id_bytes == 4)
+    return unique_relabel_impl<int32_t, PackedTable>(mapping, n_mapping, query, query_out, n_query,
+                                                     frontier, num_unique, workspace,
+                                                     workspace_bytes, last_span_len, mailbox,
+                                                     mailbox_ticket, st);
+  return narrow ? unique_relabel_impl<int64_t, PackedTable>(mapping, n_mapping, query, query_out,
+                                                            n_query, frontier, num_unique, workspace,
+                                                            workspace_bytes, last_span_len, mailbox,
+                                                            mailbox_ticket, st)
+                : unique_relabel_impl<int64_t, WideTable>(mapping, n_mapping, query, query_out,
+                                                          n_query, frontier, num_unique, workspace,
+                                                          workspace_bytes, last_span_len, mailbox,
+                                                          mailbox_ticket, st);
 }
 
 int gs_unique_relabel(const gs_span* mapping, int n_mapping, const gs_span* query,
@@ -851,21 +883,28 @@ int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void
   GS_REQUIRE((num_seeds == 0 || seeds) && (num_ids == 0 || (ids && out_ids)) &&
                  (num_seeds + num_ids == 0 || unique),
              "gs_batch_csr_relabel: null buffer");
-  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_batch_csr_relabel: id_bytes must be 4 or 8, got %d",
-             id_bytes);
+  const bool narrow = (id_bytes & GS_NARROW_IDS) != 0;
+  id_bytes &= ~GS_NARROW_IDS;
+  GS_REQUIRE(valid_id_bytes(id_bytes) && (!narrow || id_bytes == 8),
+             "gs_batch_csr_relabel: id_bytes must be 4, 8 or 8 | GS_NARROW_IDS, got %d", id_bytes);
   if (num_seeds + num_ids >= (int64_t(1) << 30)) {
     set_error_text("gs_batch_csr_relabel: %lld items exceed the supported 2^30",
                    static_cast<long long>(num_seeds + num_ids));
     return GS_ERR_UNSUPPORTED;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return id_bytes == 8
-             ? batch_relabel_impl<int64_t>(seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds,
-                                           num_ids, unique, unique_ptr, out_ids, num_unique,
-                                           workspace, workspace_bytes, mailbox, mailbox_ticket, st)
-             : batch_relabel_impl<int32_t>(seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds,
-                                           num_ids, unique, unique_ptr, out_ids, num_unique,
-                                           workspace, workspace_bytes, mailbox, mailbox_ticket, st);
+  if (id_bytes == 4)
+    return batch_relabel_impl<int32_t, PackedRegions>(
+        seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds, num_ids, unique, unique_ptr, out_ids,
+        num_unique, workspace, workspace_bytes, mailbox, mailbox_ticket, st);
+  return narrow ? batch_relabel_impl<int64_t, PackedRegions>(
+                      seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds, num_ids, unique,
+                      unique_ptr, out_ids, num_unique, workspace, workspace_bytes, mailbox,
+                      mailbox_ticket, st)
+                : batch_relabel_impl<int64_t, WideRegions>(
+                      seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds, num_ids, unique,
+                      unique_ptr, out_ids, num_unique, workspace, workspace_bytes, mailbox,
+                      mailbox_ticket, st);
 }
 
 int gs_batch_coo_relabel(const void* seeds, const int64_t* seeds_ptr, const void* coo_row,
@@ -881,23 +920,29 @@ int gs_batch_coo_relabel(const void* seeds, const int64_t* seeds_ptr, const void
                  (num_edges == 0 || (coo_row && coo_col && out_row && out_col)) &&
                  (num_seeds + num_edges == 0 || unique),
              "gs_batch_coo_relabel: null buffer");
-  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_batch_coo_relabel: id_bytes must be 4 or 8, got %d",
-             id_bytes);
+  const bool narrow = (id_bytes & GS_NARROW_IDS) != 0;
+  id_bytes &= ~GS_NARROW_IDS;
+  GS_REQUIRE(valid_id_bytes(id_bytes) && (!narrow || id_bytes == 8),
+             "gs_batch_coo_relabel: id_bytes must be 4, 8 or 8 | GS_NARROW_IDS, got %d", id_bytes);
   if (num_seeds + num_edges >= (int64_t(1) << 30)) {
     set_error_text("gs_batch_coo_relabel: %lld items exceed the supported 2^30",
                    static_cast<long long>(num_seeds + num_edges));
     return GS_ERR_UNSUPPORTED;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return id_bytes == 8
-             ? batch_relabel_impl<int64_t>(seeds, seeds_ptr, coo_row, coo_ptr, num_batches,
-                                           num_seeds, num_edges, unique, unique_ptr, out_row,
-                                           num_unique, workspace, workspace_bytes, mailbox,
-                                           mailbox_ticket, st, coo_col, out_col)
-             : batch_relabel_impl<int32_t>(seeds, seeds_ptr, coo_row, coo_ptr, num_batches,
-                                           num_seeds, num_edges, unique, unique_ptr, out_row,
-                                           num_unique, workspace, workspace_bytes, mailbox,
-                                           mailbox_ticket, st, coo_col, out_col);
+  if (id_bytes == 4)
+    return batch_relabel_impl<int32_t, PackedRegions>(
+        seeds, seeds_ptr, coo_row, coo_ptr, num_batches, num_seeds, num_edges, unique, unique_ptr,
+        out_row, num_unique, workspace, workspace_bytes, mailbox, mailbox_ticket, st, coo_col,
+        out_col);
+  return narrow ? batch_relabel_impl<int64_t, PackedRegions>(
+                      seeds, seeds_ptr, coo_row, coo_ptr, num_batches, num_seeds, num_edges, unique,
+                      unique_ptr, out_row, num_unique, workspace, workspace_bytes, mailbox,
+                      mailbox_ticket, st, coo_col, out_col)
+                : batch_relabel_impl<int64_t, WideRegions>(
+                      seeds, seeds_ptr, coo_row, coo_ptr, num_batches, num_seeds, num_edges, unique,
+                      unique_ptr, out_row, num_unique, workspace, workspace_bytes, mailbox,
+                      mailbox_ticket, st, coo_col, out_col);
 }
 
 size_t gs_relabel_table_bytes(int64_t max_items, int id_bytes) {

@@ -76,6 +76,11 @@ constexpr int64_t kBoxes = 64;
 constexpr int64_t kLost = -3;     // the slot was reused before anyone read it
 constexpr int64_t kTooWide = -2;  // posted by the narrow relabel: a key needs more than 32 bits
 
+// 64-bit ids go on the one-word table slots of 32-bit ids (GS_NARROW_IDS) until this thread
+// meets one that does not fit 32 bits; from then on it asks for the two-array slots.
+thread_local bool t_narrow_ids = true;
+int TableIds(int idb) { return idb == 8 && t_narrow_ids ? (8 | GS_NARROW_IDS) : idb; }
+
 struct HostBoxes {
   torch::Tensor buf;  // kBoxes x {total, ticket}, pinned
   gs_mailbox* ring = nullptr;
@@ -460,14 +465,18 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> Relabel(
   auto ws = Scratch(gs_unique_workspace_bytes(M), mapping[0]);
   void* st = Stream(mapping[0]);
   HostBoxes& boxes = Boxes(mapping[0].device().index());
-  const int64_t ticket = boxes.next++;
-  Check(gs_unique_relabel_notify(m, static_cast<int>(mapping.size()), q, out_ptr,
-                                 static_cast<int>(queries.size()), idb, frontier.data_ptr(),
-                                 num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), nullptr,
-                                 boxes.slot(ticket), ticket, st),
-        "gs_unique_relabel");
-  int64_t U = WaitBox(boxes.slot(ticket), ticket, st, "gs_unique_relabel");
-  if (U == kLost) U = num.item<int64_t>();
+  int64_t U = kTooWide;
+  for (int attempt = 0; attempt < 2 && U == kTooWide; ++attempt) {
+    const int64_t ticket = boxes.next++;
+    Check(gs_unique_relabel_notify(m, static_cast<int>(mapping.size()), q, out_ptr,
+                                   static_cast<int>(queries.size()), TableIds(idb),
+                                   frontier.data_ptr(), num.data_ptr<int64_t>(), ws.data_ptr(),
+                                   ws.numel(), nullptr, boxes.slot(ticket), ticket, st),
+          "gs_unique_relabel");
+    U = WaitBox(boxes.slot(ticket), ticket, st, "gs_unique_relabel");
+    if (U == kLost) U = num.item<int64_t>();
+    if (U == kTooWide) t_narrow_ids = false;
+  }
   TORCH_CHECK(U >= 0, "gs_unique_relabel: a tile gave up waiting for its predecessors");
   return {frontier.narrow(0, 0, U), outs};
 }
@@ -547,15 +556,19 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(
   auto ws = Scratch(gs_batch_relabel_workspace_bytes(M), seeds);
   void* st = Stream(seeds);
   HostBoxes& boxes = Boxes(seeds.device().index());
-  const int64_t ticket = boxes.next++;
-  Check(gs_batch_csr_relabel(seeds.data_ptr(), seeds_ptr.data_ptr<int64_t>(), ids.data_ptr(),
-                             ids_ptr.data_ptr<int64_t>(), B, seeds.numel(), ids.numel(), idb,
-                             unique.data_ptr(), unique_ptr.data_ptr<int64_t>(), out_ids.data_ptr(),
-                             num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), boxes.slot(ticket),
-                             ticket, st),
-        "gs_batch_csr_relabel");
-  int64_t U = WaitBox(boxes.slot(ticket), ticket, st, "gs_batch_csr_relabel");
-  if (U == kLost) U = num.item<int64_t>();
+  int64_t U = kTooWide;
+  for (int attempt = 0; attempt < 2 && U == kTooWide; ++attempt) {
+    const int64_t ticket = boxes.next++;
+    Check(gs_batch_csr_relabel(seeds.data_ptr(), seeds_ptr.data_ptr<int64_t>(), ids.data_ptr(),
+                               ids_ptr.data_ptr<int64_t>(), B, seeds.numel(), ids.numel(),
+                               TableIds(idb), unique.data_ptr(), unique_ptr.data_ptr<int64_t>(),
+                               out_ids.data_ptr(), num.data_ptr<int64_t>(), ws.data_ptr(),
+                               ws.numel(), boxes.slot(ticket), ticket, st),
+          "gs_batch_csr_relabel");
+    U = WaitBox(boxes.slot(ticket), ticket, st, "gs_batch_csr_relabel");
+    if (U == kLost) U = num.item<int64_t>();
+    if (U == kTooWide) t_narrow_ids = false;
+  }
   TORCH_CHECK(U >= 0, "gs_batch_csr_relabel: a tile gave up waiting for its predecessors");
   return {unique.narrow(0, 0, U), unique_ptr, out_ids};
 }
@@ -1014,16 +1027,20 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> BatchCooR
   auto ws = Scratch(gs_batch_relabel_workspace_bytes(M), seeds);
   void* st = Stream(seeds);
   HostBoxes& boxes = Boxes(seeds.device().index());
-  const int64_t ticket = boxes.next++;
-  Check(gs_batch_coo_relabel(seeds.data_ptr(), seeds_ptr.data_ptr<int64_t>(), coo_row.data_ptr(),
-                             coo_col.data_ptr(), coo_ptr.data_ptr<int64_t>(), B, seeds.numel(),
-                             coo_row.numel(), idb, unique.data_ptr(),
-                             unique_ptr.data_ptr<int64_t>(), out_row.data_ptr(), out_col.data_ptr(),
-                             num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(),
-                             boxes.slot(ticket), ticket, st),
-        "gs_batch_coo_relabel");
-  int64_t U = WaitBox(boxes.slot(ticket), ticket, st, "gs_batch_coo_relabel");
-  if (U == kLost) U = num.item<int64_t>();
+  int64_t U = kTooWide;
+  for (int attempt = 0; attempt < 2 && U == kTooWide; ++attempt) {
+    const int64_t ticket = boxes.next++;
+    Check(gs_batch_coo_relabel(seeds.data_ptr(), seeds_ptr.data_ptr<int64_t>(), coo_row.data_ptr(),
+                               coo_col.data_ptr(), coo_ptr.data_ptr<int64_t>(), B, seeds.numel(),
+                               coo_row.numel(), TableIds(idb), unique.data_ptr(),
+                               unique_ptr.data_ptr<int64_t>(), out_row.data_ptr(),
+                               out_col.data_ptr(), num.data_ptr<int64_t>(), ws.data_ptr(),
+                               ws.numel(), boxes.slot(ticket), ticket, st),
+          "gs_batch_coo_relabel");
+    U = WaitBox(boxes.slot(ticket), ticket, st, "gs_batch_coo_relabel");
+    if (U == kLost) U = num.item<int64_t>();
+    if (U == kTooWide) t_narrow_ids = false;
+  }
   TORCH_CHECK(U >= 0, "gs_batch_coo_relabel: a tile gave up waiting for its predecessors");
   return {unique.narrow(0, 0, U), unique_ptr, out_row, out_col};
 }

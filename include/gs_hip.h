@@ -69,6 +69,15 @@ typedef struct gs_mailbox {
   int64_t ticket;
 } gs_mailbox;
 
+/* Or-ed into id_bytes = 8 of gs_unique_relabel[_notify], gs_batch_csr_relabel and
+ * gs_batch_coo_relabel: the 64-bit ids are promised to fit 32 bits (node ids of any graph below
+ * 4.29 G nodes do), and the hash table uses the one-word slots of 32-bit ids -- one
+ * compare-and-swap per insert instead of compare-and-swap, read and minimum.  Ids, frontier
+ * and outputs stay 64-bit.  If a mapping id does not fit, *num_unique and the mailbox read -2
+ * and nothing else written is valid: call again without the flag.  (The reference's API is
+ * int64 throughout; this is how that costs no more than int32.) */
+#define GS_NARROW_IDS 0x100
+
 /* Optional timing of one launch site, for benchmarks (no counterpart in the
  * reference).  gs_profile_enable("name") makes every later launch of that site
  * record a hipEvent pair on its stream (up to 4096 launches); NULL or ""

@@ -295,3 +295,25 @@ def test_fastgcn_super_batch_equals_batch_by_batch(dev):
         frontier, (w_row, w_col) = O.relabel([sb, rows_b], [rows_b, cols_b])
         assert np.array_equal(u[u_ptr[b]:u_ptr[b + 1]], frontier)
         assert np.array_equal(r_row[lo:hi], w_row) and np.array_equal(r_col[lo:hi], w_col)
+
+
+def test_batch_relabel_64_bit_ids_narrow_and_fallback(dev):
+    """The host layer first tries one-word slots for 64-bit ids and falls back to the two-array
+    slots when an id does not fit 32 bits; both give the oracle's result."""
+    import graph_sampling_amd as gs
+    gs.load_library()
+    rng = np.random.default_rng(3)
+    B = 5
+    seeds_ptr = np.arange(B + 1, dtype=np.int64) * 40
+    ids_ptr = np.concatenate([[0], np.cumsum(rng.integers(50, 300, B))]).astype(np.int64)
+    for offset in (0, 3_000_000_000, 1 << 34):
+        seeds = rng.integers(0, 500, seeds_ptr[-1]).astype(np.int64) + offset
+        ids = rng.integers(0, 500, ids_ptr[-1]).astype(np.int64) + offset
+        uni, uni_ptr, rel, _ = torch.ops.gs_ops.BatchCSRRelabel(
+            to_dev(seeds, dev), to_dev(seeds_ptr, dev), to_dev(ids, dev), to_dev(ids_ptr, dev))
+        for b in range(B):
+            f, (r,) = O.relabel([seeds[seeds_ptr[b]:seeds_ptr[b + 1]], ids[ids_ptr[b]:ids_ptr[b + 1]]],
+                                [ids[ids_ptr[b]:ids_ptr[b + 1]]])
+            lo, hi = int(uni_ptr[b]), int(uni_ptr[b + 1])
+            assert np.array_equal(uni[lo:hi].cpu().numpy(), f)
+            assert np.array_equal(rel[ids_ptr[b]:ids_ptr[b + 1]].cpu().numpy(), r)

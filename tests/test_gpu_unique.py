@@ -163,3 +163,33 @@ def test_relabel_few_tiles_by_key_spread(dev, idt, n, spread):
     assert np.array_equal(frontier, want_frontier)
     for g, w in zip(outs, want):
         assert np.array_equal(g, w)
+
+
+def test_64_bit_ids_on_one_word_slots(dev):
+    """GS_NARROW_IDS: 64-bit ids that fit 32 bits give the same frontier and ranks as the
+    two-array table, lookups of ids beyond 32 bits come back absent, and a mapping id beyond
+    32 bits is reported (-2) rather than truncated."""
+    rng = np.random.default_rng(12)
+    a = rng.integers(0, 5000, 30000).astype(np.int64) + 4_000_000_000     # still below 2^32
+    b = rng.integers(0, 5000, 20000).astype(np.int64) + 4_000_000_000
+    q = np.concatenate([b[:1000], np.array([1 << 40, (1 << 32) + 5], dtype=np.int64)])
+    for narrow in (False, True):
+        frontier, num, outs = capi.unique_relabel([to_dev(a, dev), to_dev(b, dev)],
+                                                  [to_dev(b, dev), to_dev(q, dev)], narrow=narrow)
+        w_frontier, w_outs = O.relabel([a, b], [b, q])
+        U = int(num.item())
+        assert U == w_frontier.size
+        assert np.array_equal(frontier[:U].cpu().numpy(), w_frontier)
+        assert np.array_equal(outs[0].cpu().numpy(), w_outs[0])
+        assert np.array_equal(outs[1].cpu().numpy(), w_outs[1])
+        assert outs[1][-1].item() == -1 and outs[1][-2].item() == -1
+    big = a.copy()
+    big[777] = (1 << 36) + 1
+    _, num, _ = capi.unique_relabel([to_dev(big, dev)], [], narrow=True)
+    assert int(num.item()) == -2
+    # the same with lookups queued behind the pass that gave up: void outputs, but the call ends
+    t_big = to_dev(big, dev)
+    _, num, _ = capi.unique_relabel([t_big], [t_big, to_dev(q, dev)], narrow=True)
+    assert int(num.item()) == -2
+    frontier, num, _ = capi.unique_relabel([to_dev(big, dev)], [], narrow=False)
+    assert np.array_equal(frontier[:int(num.item())].cpu().numpy(), O.relabel([big], [])[0])
