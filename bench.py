@@ -356,6 +356,25 @@ def main():
               "what": "the timed minibatches again with four in flight, one host thread and one "
                       "stream each"}
 
+    # the same minibatches with 64-bit ids, the reference's only id type (beside the headline)
+    wide = None
+    if extras and idt == torch.int32 and edges <= 200_000_000:
+        graph64 = gs.Graph(False)
+        graph64._CAPI_LoadCSC(indptr, indices.long())
+        sets64 = [s.long() for s in seed_sets]
+        for i in range(args.warmup):
+            minibatch(graph64, sets64[i])
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        wide_edges = 0
+        for i in range(args.steps):
+            wide_edges += minibatch(graph64, sets64[args.warmup + i])[0]
+        torch.cuda.synchronize()
+        wide_s = time.perf_counter() - t1
+        wide = {"ms_per_step": wide_s / args.steps * 1e3, "value": wide_edges / wide_s,
+                "what": "the timed minibatches on the same graph with int64 ids"}
+        del graph64, sets64
+
     # the same again by the C++ layer's own pool of sampler threads (no interpreter in the
     # loop), 32 minibatches per call as a loader with that prefetch depth would ask for them
     pool = None
@@ -402,6 +421,7 @@ def main():
         "super_batch": sb,
         "concurrent": cc,
         "sampler_pool": pool,
+        "int64_ids": wide,
         "roofline": None,
         "cpu_baseline": None,
     }
