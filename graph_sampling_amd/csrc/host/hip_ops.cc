@@ -528,7 +528,10 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred
       // an id beyond 32 bits: from now on this table takes the two-array slots
       TORCH_CHECK(idb == 8 && table.narrow, "gs_relabel_sampled: unexpected status");
       table.narrow = false;
-      state.buf.zero_();  // the error word is sticky
+      // the error word is sticky: clear the state on the stream the kernels run on
+      TORCH_CHECK(hipMemsetAsync(state.buf.data_ptr(), 0, state.buf.numel(),
+                                 static_cast<hipStream_t>(p.stream)) == hipSuccess,
+                  "hipMemsetAsync failed");
       RelabelTableFor(col_ids, p.stream, idb, M);                               // prepares it again
       FusedState(gs_relabel_sampled_state_bytes(M), col_ids, p.stream);       // next epoch
     }
