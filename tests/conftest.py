@@ -12,6 +12,15 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """The tests load the libraries that are built; only when there are none do they build."""
+    pkg = os.path.join(ROOT, "graph_sampling_amd")
+    if all(os.path.exists(os.path.join(pkg, name)) for name in ("libgs_hip.so", "libgs.so")):
+        return
+    from graph_sampling_amd import build
+    build.build_all()
+
+
 @pytest.fixture(scope="session")
 def dev():
     import torch
