@@ -107,7 +107,11 @@ def build_host(verbose=False):
     torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
     link = ["g++", "-shared", "-o", HOST_LIB] + objs + [
         "-L" + _PKG, "-lgs_hip", "-Wl,-rpath,$ORIGIN",
-        "-L" + torch_lib, "-lc10", "-ltorch_cpu", "-ltorch", "-lc10_hip", "-ltorch_hip",
+        "-L" + torch_lib, "-lc10", "-ltorch_cpu", "-ltorch", "-lc10_hip",
+        # libtorch_hip registers the GPU backend from its static initialisers; nothing here
+        # refers to a symbol of it, so the linker would drop it and a C++ program that loads
+        # only this library would find no GPU
+        "-Wl,--no-as-needed", "-ltorch_hip", "-Wl,--as-needed",
         "-Wl,-rpath," + torch_lib,
         "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib",
     ]
@@ -115,11 +119,44 @@ def build_host(verbose=False):
     return HOST_LIB
 
 
+CPP_CHECK_SRC = os.path.join(_ROOT, "tests", "cpp", "host_api_check.cc")
+CPP_CHECK_BIN = os.path.join(_ROOT, "tests", "cpp", "host_api_check")
+
+
+def build_cpp_check(verbose=False):
+    """Compile the C++ caller of the host layer (tests/cpp) against the public headers and
+    link it to libgs.so: proof that gs::Graph and the free functions can be used from C++."""
+    if not os.path.exists(CPP_CHECK_SRC):
+        return None
+    import torch
+    from torch.utils import cpp_extension as ce
+    inc = []
+    for p in ce.include_paths():
+        inc += ["-isystem", p]
+    inc += ["-isystem", "/opt/rocm/include", "-I", os.path.join(_CSRC, "host")]
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = ["g++", "-O1", "-std=c++17", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % abi, "-Wno-deprecated-declarations"] + inc + [
+        CPP_CHECK_SRC, "-o", CPP_CHECK_BIN,
+        "-L" + _PKG, "-lgs", "-lgs_hip", "-Wl,-rpath,$ORIGIN/../../graph_sampling_amd",
+        "-L" + torch_lib, "-lc10", "-ltorch_cpu", "-ltorch", "-lc10_hip", "-ltorch_hip",
+        "-Wl,-rpath," + torch_lib,
+        "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"]
+    out = _run(cmd)
+    if verbose and out.strip():
+        print(out)
+    return CPP_CHECK_BIN
+
+
 def build_all(verbose=False):
     libs = [build_kernels(verbose)]
     host = build_host(verbose)
     if host:
         libs.append(host)
+        check = build_cpp_check(verbose)
+        if check:
+            libs.append(check)
     return libs
 
 
