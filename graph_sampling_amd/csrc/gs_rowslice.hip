@@ -5,12 +5,22 @@
 // ids are relabelled to their position in `ids` (slicing.cu:477-480).
 //
 // Mark:    id-set table (capacity 2 * pow2 > n, as slicing.cu:468; Fibonacci
-//          hashing instead of Hash64Shift) -> val[e] = position or -1
-//          -> prefix = exclusive scan of (val >= 0).  For the CSC flavour the
-//          new offsets are simply prefix[indptr[c]]: no per-column count pass,
-//          no warp reduction (slicing.cu:463-466), no torch::nonzero.
-// Compact: survivors are written in edge order from (val, prefix); the owning
-//          column of an edge is found like in the CSC -> COO expansion.
+//          hashing instead of Hash64Shift) with a one-bit-per-hash filter in front of
+//          it: most edges of a slice are not kept, and those leave after one read of a
+//          bit array that stays in the caches instead of a chain of 8-byte slots.
+//          What the pass leaves behind per edge is ONE BIT (kept or not) in 64-edge
+//          words, the number of kept edges of the tile before each word, the count of
+//          each 2048-edge tile, and the new ids of the kept edges packed to the front
+//          of the tile's range of a scratch array.  An exclusive scan of the tile
+//          counts (one entry per 2048 edges) gives every tile its place in the result.
+//          For the CSC flavour the new offsets are kept_before(indptr[c]): no
+//          per-column count pass, no warp reduction (slicing.cu:463-466), no
+//          torch::nonzero.
+// Compact: tiles without kept edges leave at once; the others copy their packed ids
+//          and write edge positions (and owning columns, found like in the CSC -> COO
+//          expansion) at tile base + rank from the bit words.
+// The induced-subgraph slice and the batched membership filter below mark and compact the
+// same way.
 // When `ids` holds duplicates the reference keeps whichever store lands last
 // (slicing.cu:56); here the largest position wins (atomicMax), deterministically.
 #include "gs_common.hpp"
@@ -28,8 +38,23 @@ struct IdSet {
   long long* vals;
   uint32_t mask;
   int shift;
+  // bit (hash of key) is set for every key of the set: a clear bit proves absence
+  uint32_t* filter;
+  int filter_shift;
   __device__ __forceinline__ uint32_t home(long long key) const {
     return static_cast<uint32_t>((static_cast<uint64_t>(key) * 0x9E3779B97F4A7C15ull) >> shift);
+  }
+  __device__ __forceinline__ uint32_t filter_bit(long long key) const {
+    return static_cast<uint32_t>((static_cast<uint64_t>(key) * 0xD6E8FEB86659FD93ull) >>
+                                 filter_shift);
+  }
+  __device__ __forceinline__ bool maybe(long long key) const {
+    const uint32_t b = filter_bit(key);
+    return (filter[b >> 5] >> (b & 31)) & 1u;
+  }
+  __device__ __forceinline__ void admit(long long key) const {
+    const uint32_t b = filter_bit(key);
+    atomicOr(&filter[b >> 5], 1u << (b & 31));
   }
   __device__ __forceinline__ int64_t query(long long key) const {
     uint32_t p = home(key);
@@ -48,12 +73,22 @@ int64_t set_capacity(int64_t n) {
   return cap;
 }
 
-__global__ void __launch_bounds__(kThreads) set_init_kernel(IdSet t, int64_t cap) {
+// bits of the filter: 32 per id (3 % of the absent keys pass), between 1 KB and 1 MB
+int64_t filter_bits(int64_t n) {
+  int64_t bits = 8192;
+  while (bits < 32 * n && bits < (int64_t(1) << 23)) bits <<= 1;
+  return bits;
+}
+
+// clears the table and the filter; the grid covers the longer of the two
+__global__ void __launch_bounds__(kThreads)
+set_init_kernel(IdSet t, int64_t cap, int64_t filter_words) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i < cap) {
     t.keys[i] = -1;
     t.vals[i] = -1;
   }
+  if (i < filter_words) t.filter[i] = 0;
 }
 
 template <typename IdT>
@@ -71,30 +106,7 @@ set_insert_kernel(IdSet t, const IdT* __restrict__ ids, int64_t n) {
     p = (p + 1) & t.mask;
   }
   atomicMax(&t.vals[p], static_cast<long long>(i));
-}
-
-template <typename IdT>
-__global__ void __launch_bounds__(kThreads)
-mark_kernel(IdSet t, const IdT* __restrict__ key, int64_t E, int64_t* __restrict__ val) {
-  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (e < E) val[e] = t.query(static_cast<long long>(key[e]));
-}
-
-struct Kept {
-  const int64_t* val;
-  __device__ __forceinline__ int64_t operator()(int64_t e) const { return val[e] >= 0 ? 1 : 0; }
-};
-
-__global__ void __launch_bounds__(kThreads)
-new_indptr_kernel(const int64_t* __restrict__ indptr, int64_t num_cols,
-                  const int64_t* __restrict__ prefix, int64_t* __restrict__ out_indptr) {
-  const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (c <= num_cols) out_indptr[c] = prefix[indptr[c]];
-}
-
-__global__ void __launch_bounds__(kThreads)
-copy_total_kernel(const int64_t* __restrict__ prefix, int64_t E, int64_t* __restrict__ total) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) *total = prefix[E];
+  t.admit(key);
 }
 
 template <typename P>
@@ -107,15 +119,165 @@ __device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
   return lo;
 }
 
-// CSC compaction; a workgroup owns 2048 consecutive input edges.
+// ------------------------------------------------------------ survivor marks ----
+constexpr int kWords = kTile / kWave;  // 64-edge words of a tile
+
+// What the mark pass leaves for the compaction: one bit per edge, the kept edges of the
+// tile before each word, and (after the scan) the kept edges before each tile.
+struct Marks {
+  unsigned long long* mask;  // [n / 64 + 1]
+  int32_t* word_rank;        // [n / 64 + 1]
+  int64_t* tile_counts;      // [tiles]
+  int64_t* tile_base;        // [tiles + 1], exclusive scan of tile_counts
+  int64_t n;
+  int64_t tiles;
+  // kept edges among the first i, 0 <= i <= n
+  __device__ __forceinline__ int64_t kept_before(int64_t i) const {
+    if (i >= n) return tile_base[tiles];
+    const int64_t w = i >> 6;
+    const unsigned long long below = mask[w] & ((1ull << (i & 63)) - 1ull);
+    return tile_base[i / kTile] + word_rank[w] + __popcll(below);
+  }
+};
+
+struct LoadCounts {
+  const int64_t* p;
+  __device__ __forceinline__ int64_t operator()(int64_t i) const { return p[i]; }
+};
+
+// key of edge e for the id set; false: the edge cannot be kept
+template <typename IdT>
+struct PlainKey {
+  const IdT* key;
+  __device__ __forceinline__ bool operator()(int64_t e, long long* out) const {
+    *out = static_cast<long long>(key[e]);
+    return true;
+  }
+};
+
+constexpr int kBatchShift = 44;
+
+// edge e belongs to the batch whose range of key_ptr holds it; set keys are id + (batch << 44)
+template <typename IdT>
+struct BatchedKey {
+  const IdT* key;
+  const int64_t* key_ptr;
+  int64_t B;
+  __device__ __forceinline__ bool operator()(int64_t e, long long* out) const {
+    int64_t lo = 0, hi = B + 1;  // first b with key_ptr[b] > e
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (key_ptr[mid] <= e) lo = mid + 1; else hi = mid;
+    }
+    const int64_t b = lo - 1;
+    if (b < 0 || b >= B) return false;
+    *out = static_cast<long long>(key[e]) + (static_cast<long long>(b) << kBatchShift);
+    return true;
+  }
+};
+
+// Tail of a mark pass.  The workgroup owns the 2048 positions from p0, position
+// p0 + k * 256 + thread in round k, so that a wave's ballot in round k is the word of 64
+// consecutive positions (word k * 4 + wave of the tile).  vals[k] >= 0: kept, and the
+// value to pack to the front of the tile's range (with src[k] beside it when WITH_SRC).
+// Every thread of the workgroup calls this.
+template <typename IdT, bool WITH_VALUES, bool WITH_SRC>
+__device__ __forceinline__ void publish_marks(const int64_t (&vals)[kItems],
+                                              const int64_t (&src)[kItems], int64_t p0, int64_t n,
+                                              const Marks& m, IdT* __restrict__ packed,
+                                              int64_t* __restrict__ packed_src, int* s_pop,
+                                              int* s_rank) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  unsigned long long bal[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    bal[k] = __ballot(vals[k] >= 0);
+    const int w = k * (kThreads / kWave) + wave;
+    if (lane == 0) {
+      s_pop[w] = __popcll(bal[k]);
+      if (p0 + static_cast<int64_t>(w) * kWave < n) m.mask[(p0 >> 6) + w] = bal[k];
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < kWave) {
+    const int v = threadIdx.x < kWords ? s_pop[threadIdx.x] : 0;
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < kWords; d <<= 1) {
+      const int o = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl += o;
+    }
+    if (threadIdx.x < kWords) {
+      s_rank[threadIdx.x] = incl - v;
+      if (p0 + static_cast<int64_t>(threadIdx.x) * kWave < n)
+        m.word_rank[(p0 >> 6) + threadIdx.x] = incl - v;
+    }
+    if (threadIdx.x == kWords - 1) m.tile_counts[blockIdx.x] = incl;
+  }
+  if (WITH_VALUES || WITH_SRC) {
+    __syncthreads();
+    const unsigned long long lower = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int k = 0; k < kItems; ++k)
+      if (vals[k] >= 0) {
+        const int64_t at =
+            p0 + s_rank[k * (kThreads / kWave) + wave] + __popcll(bal[k] & lower);
+        if (WITH_VALUES) packed[at] = static_cast<IdT>(vals[k]);
+        if (WITH_SRC) packed_src[at] = src[k];
+      }
+  }
+}
+
+// One tile of 2048 edges per workgroup.  The eight keys of a thread, their filter bits and
+// their table probes are issued as three batches of independent loads.
+template <typename IdT, typename KeyOf, bool WITH_VALUES>
+__global__ void __launch_bounds__(kThreads)
+mark_tiles_kernel(IdSet t, KeyOf key_of, int64_t E, Marks m, IdT* __restrict__ packed) {
+  __shared__ int s_pop[kWords];
+  __shared__ int s_rank[kWords];
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
+  long long keys[kItems];
+  bool pass[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t e = p0 + k * kThreads + threadIdx.x;
+    keys[k] = -1;
+    pass[k] = e < E && key_of(e, &keys[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < kItems; ++k)
+    if (pass[k]) pass[k] = t.maybe(keys[k]);
+  int64_t vals[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) vals[k] = pass[k] ? t.query(keys[k]) : -1;
+  publish_marks<IdT, WITH_VALUES, false>(vals, vals, p0, E, m, packed, nullptr, s_pop, s_rank);
+}
+
+__global__ void __launch_bounds__(kThreads)
+new_indptr_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, Marks m,
+                  int64_t* __restrict__ out_indptr) {
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (c <= num_cols) out_indptr[c] = m.kept_before(indptr[c]);
+}
+
+__global__ void __launch_bounds__(kWave) copy_total_kernel(Marks m, int64_t* __restrict__ total) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) *total = m.tile_base[m.tiles];
+}
+
+// CSC compaction; a workgroup owns the 2048 input edges its mark workgroup owned.
 template <bool WITH_COO, typename IdT>
 __global__ void __launch_bounds__(kThreads)
-csc_compact_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz,
-                   const int64_t* __restrict__ val, const int64_t* __restrict__ prefix,
-                   IdT* __restrict__ out_indices, int64_t* __restrict__ select_index,
-                   IdT* __restrict__ coo_col) {
+csc_compact_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz, Marks m,
+                   const IdT* __restrict__ packed, IdT* __restrict__ out_indices,
+                   int64_t* __restrict__ select_index, IdT* __restrict__ coo_col) {
   __shared__ int64_t s_ptr[kStage + 1];
   __shared__ int64_t s_rows[2];
+  const int64_t base = m.tile_base[blockIdx.x];
+  const int64_t count = m.tile_base[blockIdx.x + 1] - base;
+  if (count == 0) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
   const int64_t p1 = p0 + kTile < nnz ? p0 + kTile : nnz;
   int64_t row_lo = 0, nrows = 0;
@@ -131,34 +293,51 @@ csc_compact_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t
       for (int64_t i = threadIdx.x; i <= nrows; i += kThreads) s_ptr[i] = indptr[row_lo + i];
     __syncthreads();
   }
+  for (int64_t r = threadIdx.x; r < count; r += kThreads) out_indices[base + r] = packed[p0 + r];
+  const unsigned long long lower = (1ull << lane) - 1ull;
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
-    const int64_t e = p0 + k * kThreads + threadIdx.x;
-    if (e >= p1) break;
-    const int64_t v = val[e];
-    if (v < 0) continue;
-    const int64_t w = prefix[e];
-    out_indices[w] = static_cast<IdT>(v);
-    select_index[w] = e;
+    const int w = k * (kThreads / kWave) + wave;
+    const int64_t e = p0 + static_cast<int64_t>(w) * kWave + lane;
+    if (e - lane >= p1) break;
+    const unsigned long long bits = m.mask[(p0 >> 6) + w];
+    if (!((bits >> lane) & 1ull)) continue;
+    const int64_t pos = base + m.word_rank[(p0 >> 6) + w] + __popcll(bits & lower);
+    select_index[pos] = e;
     if (WITH_COO)
-      coo_col[w] = static_cast<IdT>(row_lo + (staged ? upper_bound(s_ptr, nrows + 1, e)
-                                                     : upper_bound(indptr + row_lo, nrows + 1, e)) - 1);
+      coo_col[pos] = static_cast<IdT>(row_lo + (staged ? upper_bound(s_ptr, nrows + 1, e)
+                                                       : upper_bound(indptr + row_lo, nrows + 1, e)) - 1);
   }
 }
 
-template <typename IdT>
+// COO compaction and the membership filter's: KEY_OUT writes the packed new ids of the
+// key side (row slice); otherwise both endpoints are copied as they are (filter).
+template <bool KEY_OUT, typename IdT>
 __global__ void __launch_bounds__(kThreads)
-coo_compact_kernel(const IdT* __restrict__ other, int64_t E, const int64_t* __restrict__ val,
-                   const int64_t* __restrict__ prefix, IdT* __restrict__ out_key,
+coo_compact_kernel(const IdT* __restrict__ key, const IdT* __restrict__ other, int64_t E, Marks m,
+                   const IdT* __restrict__ packed, IdT* __restrict__ out_key,
                    IdT* __restrict__ out_other, int64_t* __restrict__ select_index) {
-  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (e >= E) return;
-  const int64_t v = val[e];
-  if (v < 0) return;
-  const int64_t w = prefix[e];
-  out_key[w] = static_cast<IdT>(v);
-  out_other[w] = other[e];
-  select_index[w] = e;
+  const int64_t base = m.tile_base[blockIdx.x];
+  const int64_t count = m.tile_base[blockIdx.x + 1] - base;
+  if (count == 0) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
+  if (KEY_OUT)
+    for (int64_t r = threadIdx.x; r < count; r += kThreads) out_key[base + r] = packed[p0 + r];
+  const unsigned long long lower = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int w = k * (kThreads / kWave) + wave;
+    const int64_t e = p0 + static_cast<int64_t>(w) * kWave + lane;
+    if (e - lane >= E) break;
+    const unsigned long long bits = m.mask[(p0 >> 6) + w];
+    if (!((bits >> lane) & 1ull)) continue;
+    const int64_t pos = base + m.word_rank[(p0 >> 6) + w] + __popcll(bits & lower);
+    if (!KEY_OUT) out_key[pos] = key[e];
+    out_other[pos] = other[e];
+    if (select_index) select_index[pos] = e;
+  }
 }
 
 // ------------------------------------------- column slice + row slice in one go ----
@@ -193,16 +372,19 @@ set_insert_batched_kernel(IdSet t, const IdT* __restrict__ ids, int64_t n,
     p = (p + 1) & t.mask;
   }
   atomicMax(&t.vals[p], id);
+  t.admit(key);
 }
 
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 sliced_mark_kernel(IdSet t, const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
                    const IdT* __restrict__ cols, int64_t S, const int64_t* __restrict__ sub_indptr,
-                   int64_t D, const int64_t* __restrict__ col_ptr, int64_t B, int64_t enc,
-                   int64_t* __restrict__ val, int64_t* __restrict__ src) {
+                   int64_t D, const int64_t* __restrict__ col_ptr, int64_t B, int64_t enc, Marks m,
+                   IdT* __restrict__ packed, int64_t* __restrict__ packed_src) {
   __shared__ int64_t s_ptr[kStage + 1];
   __shared__ int64_t s_rows[2];
+  __shared__ int s_pop[kWords];
+  __shared__ int s_rank[kWords];
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
   const int64_t p1 = p0 + kTile < D ? p0 + kTile : D;
   if (threadIdx.x < 2)
@@ -214,88 +396,91 @@ sliced_mark_kernel(IdSet t, const int64_t* __restrict__ indptr, const IdT* __res
   if (staged)
     for (int64_t i = threadIdx.x; i <= nrows; i += kThreads) s_ptr[i] = sub_indptr[row_lo + i];
   __syncthreads();
+  long long keys[kItems], ids[kItems];
+  int64_t src[kItems];
+  bool pass[kItems];
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
     const int64_t p = p0 + k * kThreads + threadIdx.x;
-    if (p >= p1) break;
+    keys[k] = ids[k] = -1;
+    src[k] = 0;
+    pass[k] = false;
+    if (p >= p1) continue;
     const int64_t lr = (staged ? upper_bound(s_ptr, nrows + 1, p)
                                : upper_bound(sub_indptr + row_lo, nrows + 1, p)) - 1;
     const int64_t r = row_lo + lr;
     const int64_t first = staged ? s_ptr[lr] : sub_indptr[r];
     // a column that owns a position of the slice has passed the range check of the count
     const int64_t c = static_cast<int64_t>(cols[r]);
-    const int64_t q = indptr[c] + (p - first);
-    const long long id = static_cast<long long>(indices[q]);
-    src[p] = q;
+    src[k] = indptr[c] + (p - first);
+    ids[k] = static_cast<long long>(indices[src[k]]);
     if (B > 0) {
       const int64_t b = upper_bound(col_ptr, B + 1, r) - 1;
-      val[p] = (b >= 0 && b < B && t.query(id + b * enc) >= 0) ? id : -1;
+      pass[k] = b >= 0 && b < B;
+      keys[k] = ids[k] + b * enc;
     } else {
-      val[p] = t.query(id);
+      pass[k] = true;
+      keys[k] = ids[k];
     }
   }
+#pragma unroll
+  for (int k = 0; k < kItems; ++k)
+    if (pass[k]) pass[k] = t.maybe(keys[k]);
+  int64_t vals[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t v = pass[k] ? t.query(keys[k]) : -1;
+    vals[k] = (B > 0 && v >= 0) ? ids[k] : v;  // batched: rows keep their id
+  }
+  publish_marks<IdT, true, true>(vals, src, p0, D, m, packed, packed_src, s_pop, s_rank);
 }
 
 __global__ void __launch_bounds__(kThreads)
-sliced_indptr_kernel(const int64_t* __restrict__ sub_indptr, int64_t S,
-                     const int64_t* __restrict__ prefix, int64_t* __restrict__ out_indptr) {
+sliced_indptr_kernel(const int64_t* __restrict__ sub_indptr, int64_t S, Marks m,
+                     int64_t* __restrict__ out_indptr) {
   const int64_t r = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (r <= S) out_indptr[r] = prefix[sub_indptr[r]];
+  if (r <= S) out_indptr[r] = m.kept_before(sub_indptr[r]);
 }
 
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
-sliced_compact_kernel(int64_t D, const int64_t* __restrict__ val, const int64_t* __restrict__ prefix,
-                      const int64_t* __restrict__ src, IdT* __restrict__ out_indices,
+sliced_compact_kernel(int64_t D, Marks m, const IdT* __restrict__ packed,
+                      const int64_t* __restrict__ packed_src, IdT* __restrict__ out_indices,
                       int64_t* __restrict__ select_index, int64_t* __restrict__ parent_index) {
-  const int64_t p = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (p >= D) return;
-  const int64_t v = val[p];
-  if (v < 0) return;
-  const int64_t w = prefix[p];
-  out_indices[w] = static_cast<IdT>(v);
-  if (select_index) select_index[w] = p;
-  if (parent_index) parent_index[w] = src[p];
+  const int64_t base = m.tile_base[blockIdx.x];
+  const int64_t count = m.tile_base[blockIdx.x + 1] - base;
+  if (count == 0) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
+  for (int64_t r = threadIdx.x; r < count; r += kThreads) {
+    out_indices[base + r] = packed[p0 + r];
+    if (parent_index) parent_index[base + r] = packed_src[p0 + r];
+  }
+  if (!select_index) return;
+  const unsigned long long lower = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int w = k * (kThreads / kWave) + wave;
+    const int64_t p = p0 + static_cast<int64_t>(w) * kWave + lane;
+    if (p - lane >= D) break;
+    const unsigned long long bits = m.mask[(p0 >> 6) + w];
+    if ((bits >> lane) & 1ull)
+      select_index[base + m.word_rank[(p0 >> 6) + w] + __popcll(bits & lower)] = p;
+  }
 }
 
 // ------------------------------------------------- batched membership filter ----
 // Edge e belongs to the batch whose range of key_ptr holds e; it survives when key[e] is
 // among the ids of the same batch.  Replaces the per-batch tables of
 // impl::BatchCOOSlicingCUDA / BatchCOORowSlicingCUDA (reference src/cuda/batch_slicing.cu:
-// 150-232, src/cuda/slicing.cu:659-770) by one table keyed with id + (batch << 44).
-constexpr int kBatchShift = 44;
-
-template <typename IdT>
+// 150-232, src/cuda/slicing.cu:659-770) by one table keyed with id + (batch << 44)
+// (BatchedKey above); mark and compaction are the row slice's.
 __global__ void __launch_bounds__(kThreads)
-mark_batched_kernel(IdSet t, const IdT* __restrict__ key, int64_t E,
-                    const int64_t* __restrict__ key_ptr, int64_t B, int64_t* __restrict__ val) {
-  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (e >= E) return;
-  const int64_t b = upper_bound(key_ptr, B + 1, e) - 1;
-  val[e] = (b >= 0 && b < B)
-               ? t.query(static_cast<long long>(key[e]) + (static_cast<long long>(b) << kBatchShift))
-               : -1;
-}
-
-template <typename IdT>
-__global__ void __launch_bounds__(kThreads)
-filter_compact_kernel(const IdT* __restrict__ row, const IdT* __restrict__ col, int64_t E,
-                      const int64_t* __restrict__ val, const int64_t* __restrict__ prefix,
-                      IdT* __restrict__ out_row, IdT* __restrict__ out_col,
-                      int64_t* __restrict__ select_index) {
-  const int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (e >= E || val[e] < 0) return;
-  const int64_t w = prefix[e];
-  out_row[w] = row[e];
-  out_col[w] = col[e];
-  if (select_index) select_index[w] = e;
-}
-
-__global__ void __launch_bounds__(kThreads)
-filter_batch_ptr_kernel(const int64_t* __restrict__ key_ptr, int64_t B,
-                        const int64_t* __restrict__ prefix, int64_t* __restrict__ out_ptr) {
+filter_batch_ptr_kernel(const int64_t* __restrict__ key_ptr, int64_t B, Marks m,
+                        int64_t* __restrict__ out_ptr) {
   const int64_t b = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (b <= B) out_ptr[b] = prefix[key_ptr[b]];
+  if (b <= B) out_ptr[b] = m.kept_before(key_ptr[b]);
 }
 
 // position of each key in `data` (-1 when absent): impl::IndexHashMapInsertCUDA +
@@ -307,55 +492,114 @@ search_kernel(IdSet t, const IdT* __restrict__ keys, int64_t m, IdT* __restrict_
   if (i < m) out[i] = static_cast<IdT>(t.query(static_cast<long long>(keys[i])));
 }
 
-// Workspace layout: [val | prefix | scan tiles | (parent positions) | id-set].  All but
-// the last depend on the edge count only, so the compact call finds them again without
-// knowing how many ids the mark call was given.
-struct Scratch {
+// Workspace layout: [marks | (parent positions) | id-set keys | id-set values | filter].
+// The marks (bit words, word ranks, tile counts and bases, scan tiles, packed new ids)
+// and the parent positions depend on the edge count only, so the compact call finds them
+// again without knowing how many ids the mark call was given.
+void carve_set(Carver& ws, int64_t n_ids, IdSet* set, int64_t* cap, int64_t* filter_words) {
+  *cap = set_capacity(n_ids);
+  set->keys = ws.take<long long>(*cap);
+  set->vals = ws.take<long long>(*cap);
+  set->mask = static_cast<uint32_t>(*cap - 1);
+  int lg = 0;
+  while ((int64_t(1) << lg) < *cap) ++lg;
+  set->shift = 64 - lg;
+  const int64_t bits = filter_bits(n_ids);
+  *filter_words = bits / 32;
+  set->filter = ws.take<uint32_t>(*filter_words);
+  lg = 0;
+  while ((int64_t(1) << lg) < bits) ++lg;
+  set->filter_shift = 64 - lg;
+}
+
+size_t set_bytes(int64_t n_ids) {
+  return 2 * padded(set_capacity(n_ids) * 8) + padded(filter_bits(n_ids) / 8);
+}
+
+struct MarkScratch {
   IdSet set;
   int64_t cap;
-  int64_t* val;
-  int64_t* prefix;
-  int64_t* tiles;
-  int64_t* src;
+  int64_t filter_words;
+  Marks m;
+  int64_t* scan_tiles;
+  void* packed;
+  int64_t* packed_src;
   bool ok;
 };
 
-Scratch carve(void* workspace, size_t bytes, int64_t n_ids, int64_t E, bool with_set,
-              bool with_src = false) {
-  Scratch s;
+// tiles of an array of E positions; none when it is empty
+int64_t mark_tiles(int64_t E) { return (E + kTile - 1) / kTile; }
+
+size_t marks_bytes(int64_t E) {
+  const int64_t words = E / kWave + 1;
+  const int64_t tiles = mark_tiles(E);
+  return padded(words * 8) + padded(words * 4) + padded((tiles + 1) * 8) + padded((tiles + 2) * 8) +
+         scan_workspace_bytes(tiles) + padded((E > 0 ? E : 1) * 8);
+}
+
+MarkScratch carve_marks(void* workspace, size_t bytes, int64_t n_ids, int64_t E, bool with_set,
+                        bool with_src = false) {
+  MarkScratch s;
   Carver ws(workspace, bytes);
-  s.val = ws.take<int64_t>(E > 0 ? E : 1);
-  s.prefix = ws.take<int64_t>(E + 1);
-  s.tiles = ws.take<int64_t>(scan_num_tiles(E) + 1);
-  s.src = with_src ? ws.take<int64_t>(E > 0 ? E : 1) : nullptr;
+  const int64_t words = E / kWave + 1;
+  s.m.n = E;
+  s.m.tiles = mark_tiles(E);
+  s.m.mask = ws.take<unsigned long long>(words);
+  s.m.word_rank = ws.take<int32_t>(words);
+  s.m.tile_counts = ws.take<int64_t>(s.m.tiles + 1);
+  s.m.tile_base = ws.take<int64_t>(s.m.tiles + 2);
+  s.scan_tiles = ws.take<int64_t>(scan_num_tiles(s.m.tiles) + 1);
+  s.packed = ws.take<int64_t>(E > 0 ? E : 1);
+  s.packed_src = with_src ? ws.take<int64_t>(E > 0 ? E : 1) : nullptr;
   s.cap = 0;
-  if (with_set) {
-    s.cap = set_capacity(n_ids);
-    s.set.keys = ws.take<long long>(s.cap);
-    s.set.vals = ws.take<long long>(s.cap);
-    s.set.mask = static_cast<uint32_t>(s.cap - 1);
-    int lg = 0;
-    while ((int64_t(1) << lg) < s.cap) ++lg;
-    s.set.shift = 64 - lg;
-  }
+  s.filter_words = 0;
+  if (with_set) carve_set(ws, n_ids, &s.set, &s.cap, &s.filter_words);
   s.ok = ws.ok;
   return s;
 }
 
+void init_set(const IdSet& set, int64_t cap, int64_t filter_words, hipStream_t st) {
+  const int64_t n = cap > filter_words ? cap : filter_words;
+  hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(n, kThreads)), dim3(kThreads), 0, st, set, cap,
+                     filter_words);
+}
+
+// id set from `ids` (cut into B batches at ids_ptr when B > 0), marks of the E edge keys,
+// scan of the tile counts
 template <typename IdT>
-int mark_common(const char* who, const void* key, int64_t E, const void* ids, int64_t n_ids,
-                Scratch& s, hipStream_t st) {
-  hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(s.cap, kThreads)), dim3(kThreads), 0, st,
-                     s.set, s.cap);
-  if (n_ids > 0)
-    hipLaunchKernelGGL(set_insert_kernel<IdT>, dim3(blocks_for(n_ids, kThreads)), dim3(kThreads), 0,
-                       st, s.set, static_cast<const IdT*>(ids), n_ids);
-  if (E > 0)
-    hipLaunchKernelGGL(mark_kernel<IdT>, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st, s.set,
-                       static_cast<const IdT*>(key), E, s.val);
+int mark_common(const char* who, const void* key, int64_t E, const int64_t* key_ptr, const void* ids,
+                int64_t n_ids, const int64_t* ids_ptr, int64_t B, bool with_values, MarkScratch& s,
+                hipStream_t st) {
+  init_set(s.set, s.cap, s.filter_words, st);
+  if (n_ids > 0) {
+    if (B > 0)
+      hipLaunchKernelGGL(set_insert_batched_kernel<IdT>, dim3(blocks_for(n_ids, kThreads)),
+                         dim3(kThreads), 0, st, s.set, static_cast<const IdT*>(ids), n_ids, ids_ptr, B,
+                         int64_t(1) << kBatchShift);
+    else
+      hipLaunchKernelGGL(set_insert_kernel<IdT>, dim3(blocks_for(n_ids, kThreads)), dim3(kThreads), 0,
+                         st, s.set, static_cast<const IdT*>(ids), n_ids);
+  }
+  if (E > 0) {
+    const dim3 grid(static_cast<unsigned>(s.m.tiles));
+    IdT* packed = static_cast<IdT*>(s.packed);
+    if (B > 0) {
+      BatchedKey<IdT> k{static_cast<const IdT*>(key), key_ptr, B};
+      hipLaunchKernelGGL((mark_tiles_kernel<IdT, BatchedKey<IdT>, false>), grid, dim3(kThreads), 0, st,
+                         s.set, k, E, s.m, packed);
+    } else {
+      PlainKey<IdT> k{static_cast<const IdT*>(key)};
+      if (with_values)
+        hipLaunchKernelGGL((mark_tiles_kernel<IdT, PlainKey<IdT>, true>), grid, dim3(kThreads), 0, st,
+                           s.set, k, E, s.m, packed);
+      else
+        hipLaunchKernelGGL((mark_tiles_kernel<IdT, PlainKey<IdT>, false>), grid, dim3(kThreads), 0, st,
+                           s.set, k, E, s.m, packed);
+    }
+  }
   GS_RETURN_IF_ERROR(check_launch(who));
-  Kept f{s.val};
-  return exclusive_scan(f, E, s.prefix, s.tiles, st);
+  LoadCounts f{s.m.tile_counts};
+  return exclusive_scan(f, s.m.tiles, s.m.tile_base, s.scan_tiles, st);
 }
 
 }  // namespace
@@ -369,9 +613,7 @@ size_t gs_row_slice_workspace_bytes(int64_t num_row_ids, int64_t nnz, int64_t nu
   (void)num_cols;
   if (num_row_ids < 0) num_row_ids = 0;
   if (nnz < 0) nnz = 0;
-  const int64_t cap = set_capacity(num_row_ids);
-  return 2 * padded(cap * 8) + padded((nnz > 0 ? nnz : 1) * 8) + padded((nnz + 1) * 8) +
-         scan_workspace_bytes(nnz);
+  return set_bytes(num_row_ids) + marks_bytes(nnz);
 }
 
 int gs_row_slice_csc_mark(const int64_t* indptr, const void* indices, int id_bytes,
@@ -383,19 +625,20 @@ int gs_row_slice_csc_mark(const int64_t* indptr, const void* indices, int id_byt
              "gs_row_slice_csc_mark: null pointer");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_row_slice_csc_mark: id_bytes must be 4 or 8, got %d",
              id_bytes);
-  Scratch s = carve(workspace, workspace_bytes, num_row_ids, nnz, true);
+  MarkScratch s = carve_marks(workspace, workspace_bytes, num_row_ids, nnz, true);
   if (!s.ok) {
     set_error_text("gs_row_slice_csc_mark: workspace needs %zu bytes, 256-byte aligned",
                    gs_row_slice_workspace_bytes(num_row_ids, nnz, num_cols));
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  GS_RETURN_IF_ERROR(id_bytes == 8 ? mark_common<int64_t>("row_slice_csc_mark", indices, nnz, row_ids,
-                                                          num_row_ids, s, st)
-                                   : mark_common<int32_t>("row_slice_csc_mark", indices, nnz, row_ids,
-                                                          num_row_ids, s, st));
+  GS_RETURN_IF_ERROR(id_bytes == 8
+                         ? mark_common<int64_t>("row_slice_csc_mark", indices, nnz, nullptr, row_ids,
+                                                num_row_ids, nullptr, 0, true, s, st)
+                         : mark_common<int32_t>("row_slice_csc_mark", indices, nnz, nullptr, row_ids,
+                                                num_row_ids, nullptr, 0, true, s, st));
   hipLaunchKernelGGL(new_indptr_kernel, dim3(blocks_for(num_cols + 1, kThreads)), dim3(kThreads), 0,
-                     st, indptr, num_cols, s.prefix, out_indptr);
+                     st, indptr, num_cols, s.m, out_indptr);
   return check_launch("row_slice_csc_mark");
 }
 
@@ -407,31 +650,33 @@ int gs_row_slice_csc_compact(const int64_t* indptr, int64_t num_cols, int64_t nn
              id_bytes);
   if (nnz == 0) return GS_OK;
   GS_REQUIRE(out_indices && select_index, "gs_row_slice_csc_compact: null output");
-  Scratch s = carve(workspace, workspace_bytes, 0, nnz, false);
+  MarkScratch s = carve_marks(workspace, workspace_bytes, 0, nnz, false);
   if (!s.ok) {
     set_error_text("gs_row_slice_csc_compact: pass the workspace given to gs_row_slice_csc_mark");
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid(blocks_for(nnz, kTile));
+  const dim3 grid(static_cast<unsigned>(s.m.tiles));
   if (id_bytes == 8) {
     int64_t* oi = static_cast<int64_t*>(out_indices);
     int64_t* cc = static_cast<int64_t*>(coo_col);
+    const int64_t* pk = static_cast<const int64_t*>(s.packed);
     if (coo_col)
       hipLaunchKernelGGL((csc_compact_kernel<true, int64_t>), grid, dim3(kThreads), 0, st, indptr,
-                         num_cols, nnz, s.val, s.prefix, oi, select_index, cc);
+                         num_cols, nnz, s.m, pk, oi, select_index, cc);
     else
       hipLaunchKernelGGL((csc_compact_kernel<false, int64_t>), grid, dim3(kThreads), 0, st, indptr,
-                         num_cols, nnz, s.val, s.prefix, oi, select_index, cc);
+                         num_cols, nnz, s.m, pk, oi, select_index, cc);
   } else {
     int32_t* oi = static_cast<int32_t*>(out_indices);
     int32_t* cc = static_cast<int32_t*>(coo_col);
+    const int32_t* pk = static_cast<const int32_t*>(s.packed);
     if (coo_col)
       hipLaunchKernelGGL((csc_compact_kernel<true, int32_t>), grid, dim3(kThreads), 0, st, indptr,
-                         num_cols, nnz, s.val, s.prefix, oi, select_index, cc);
+                         num_cols, nnz, s.m, pk, oi, select_index, cc);
     else
       hipLaunchKernelGGL((csc_compact_kernel<false, int32_t>), grid, dim3(kThreads), 0, st, indptr,
-                         num_cols, nnz, s.val, s.prefix, oi, select_index, cc);
+                         num_cols, nnz, s.m, pk, oi, select_index, cc);
   }
   return check_launch("row_slice_csc_compact");
 }
@@ -443,17 +688,18 @@ int gs_row_slice_coo_mark(const void* key, int id_bytes, int64_t E, const void* 
   GS_REQUIRE((E == 0 || key) && (num_ids == 0 || ids), "gs_row_slice_coo_mark: null pointer");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_row_slice_coo_mark: id_bytes must be 4 or 8, got %d",
              id_bytes);
-  Scratch s = carve(workspace, workspace_bytes, num_ids, E, true);
+  MarkScratch s = carve_marks(workspace, workspace_bytes, num_ids, E, true);
   if (!s.ok) {
     set_error_text("gs_row_slice_coo_mark: workspace needs %zu bytes, 256-byte aligned",
                    gs_row_slice_workspace_bytes(num_ids, E, 0));
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  GS_RETURN_IF_ERROR(id_bytes == 8
-                         ? mark_common<int64_t>("row_slice_coo_mark", key, E, ids, num_ids, s, st)
-                         : mark_common<int32_t>("row_slice_coo_mark", key, E, ids, num_ids, s, st));
-  hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(64), 0, st, s.prefix, E, num_kept);
+  GS_RETURN_IF_ERROR(id_bytes == 8 ? mark_common<int64_t>("row_slice_coo_mark", key, E, nullptr, ids,
+                                                          num_ids, nullptr, 0, true, s, st)
+                                   : mark_common<int32_t>("row_slice_coo_mark", key, E, nullptr, ids,
+                                                          num_ids, nullptr, 0, true, s, st));
+  hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(kWave), 0, st, s.m, num_kept);
   return check_launch("row_slice_coo_mark");
 }
 
@@ -465,23 +711,23 @@ int gs_row_slice_coo_compact(const void* other, int id_bytes, int64_t E, void* o
              id_bytes);
   if (E == 0) return GS_OK;
   GS_REQUIRE(other && out_key && out_other && select_index, "gs_row_slice_coo_compact: null pointer");
-  Scratch s = carve(workspace, workspace_bytes, 0, E, false);
+  MarkScratch s = carve_marks(workspace, workspace_bytes, 0, E, false);
   if (!s.ok) {
     set_error_text("gs_row_slice_coo_compact: pass the workspace given to gs_row_slice_coo_mark");
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid(blocks_for(E, kThreads));
+  const dim3 grid(static_cast<unsigned>(s.m.tiles));
   if (id_bytes == 8)
-    hipLaunchKernelGGL(coo_compact_kernel<int64_t>, grid, dim3(kThreads), 0, st,
-                       static_cast<const int64_t*>(other), E, s.val, s.prefix,
-                       static_cast<int64_t*>(out_key), static_cast<int64_t*>(out_other),
-                       select_index);
+    hipLaunchKernelGGL((coo_compact_kernel<true, int64_t>), grid, dim3(kThreads), 0, st,
+                       static_cast<const int64_t*>(nullptr), static_cast<const int64_t*>(other), E,
+                       s.m, static_cast<const int64_t*>(s.packed), static_cast<int64_t*>(out_key),
+                       static_cast<int64_t*>(out_other), select_index);
   else
-    hipLaunchKernelGGL(coo_compact_kernel<int32_t>, grid, dim3(kThreads), 0, st,
-                       static_cast<const int32_t*>(other), E, s.val, s.prefix,
-                       static_cast<int32_t*>(out_key), static_cast<int32_t*>(out_other),
-                       select_index);
+    hipLaunchKernelGGL((coo_compact_kernel<true, int32_t>), grid, dim3(kThreads), 0, st,
+                       static_cast<const int32_t*>(nullptr), static_cast<const int32_t*>(other), E,
+                       s.m, static_cast<const int32_t*>(s.packed), static_cast<int32_t*>(out_key),
+                       static_cast<int32_t*>(out_other), select_index);
   return check_launch("row_slice_coo_compact");
 }
 
@@ -507,15 +753,14 @@ int gs_col_row_slice_mark(const int64_t* indptr, int64_t num_cols, const void* i
              "gs_col_row_slice_mark: a batched call needs both batch offsets and an encoding size");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_col_row_slice_mark: id_bytes must be 4 or 8, got %d",
              id_bytes);
-  Scratch s = carve(workspace, workspace_bytes, num_row_ids, D, true, true);
+  MarkScratch s = carve_marks(workspace, workspace_bytes, num_row_ids, D, true, true);
   if (!s.ok) {
     set_error_text("gs_col_row_slice_mark: workspace needs %zu bytes, 256-byte aligned",
                    gs_col_row_slice_workspace_bytes(num_row_ids, D));
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(s.cap, kThreads)), dim3(kThreads), 0, st,
-                     s.set, s.cap);
+  init_set(s.set, s.cap, s.filter_words, st);
   auto run = [&](auto tag) {
     using IdT = decltype(tag);
     const IdT* ids = static_cast<const IdT*>(row_ids);
@@ -529,17 +774,17 @@ int gs_col_row_slice_mark(const int64_t* indptr, int64_t num_cols, const void* i
                            dim3(kThreads), 0, st, s.set, ids, num_row_ids);
     }
     if (D > 0)
-      hipLaunchKernelGGL(sliced_mark_kernel<IdT>, dim3(blocks_for(D, kTile)), dim3(kThreads), 0, st,
-                         s.set, indptr, static_cast<const IdT*>(indices),
+      hipLaunchKernelGGL(sliced_mark_kernel<IdT>, dim3(static_cast<unsigned>(s.m.tiles)),
+                         dim3(kThreads), 0, st, s.set, indptr, static_cast<const IdT*>(indices),
                          static_cast<const IdT*>(column_ids), S, sub_indptr, D, col_batch_ptr,
-                         num_batches, encoding_size, s.val, s.src);
+                         num_batches, encoding_size, s.m, static_cast<IdT*>(s.packed), s.packed_src);
   };
   if (id_bytes == 8) run(int64_t{}); else run(int32_t{});
   GS_RETURN_IF_ERROR(check_launch("col_row_slice_mark"));
-  Kept f{s.val};
-  GS_RETURN_IF_ERROR(exclusive_scan(f, D, s.prefix, s.tiles, st));
+  LoadCounts f{s.m.tile_counts};
+  GS_RETURN_IF_ERROR(exclusive_scan(f, s.m.tiles, s.m.tile_base, s.scan_tiles, st));
   hipLaunchKernelGGL(sliced_indptr_kernel, dim3(blocks_for(S + 1, kThreads)), dim3(kThreads), 0, st,
-                     sub_indptr, S, s.prefix, out_indptr);
+                     sub_indptr, S, s.m, out_indptr);
   return check_launch("col_row_slice_mark");
 }
 
@@ -551,21 +796,21 @@ int gs_col_row_slice_compact(int64_t D, int id_bytes, void* out_indices, int64_t
              id_bytes);
   if (D == 0) return GS_OK;
   GS_REQUIRE(out_indices, "gs_col_row_slice_compact: null output");
-  Scratch s = carve(workspace, workspace_bytes, 0, D, false, true);
+  MarkScratch s = carve_marks(workspace, workspace_bytes, 0, D, false, true);
   if (!s.ok) {
     set_error_text("gs_col_row_slice_compact: pass the workspace given to gs_col_row_slice_mark");
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid(blocks_for(D, kThreads));
+  const dim3 grid(static_cast<unsigned>(s.m.tiles));
   if (id_bytes == 8)
-    hipLaunchKernelGGL(sliced_compact_kernel<int64_t>, grid, dim3(kThreads), 0, st, D, s.val,
-                       s.prefix, s.src, static_cast<int64_t*>(out_indices), select_index,
-                       parent_index);
+    hipLaunchKernelGGL(sliced_compact_kernel<int64_t>, grid, dim3(kThreads), 0, st, D, s.m,
+                       static_cast<const int64_t*>(s.packed), s.packed_src,
+                       static_cast<int64_t*>(out_indices), select_index, parent_index);
   else
-    hipLaunchKernelGGL(sliced_compact_kernel<int32_t>, grid, dim3(kThreads), 0, st, D, s.val,
-                       s.prefix, s.src, static_cast<int32_t*>(out_indices), select_index,
-                       parent_index);
+    hipLaunchKernelGGL(sliced_compact_kernel<int32_t>, grid, dim3(kThreads), 0, st, D, s.m,
+                       static_cast<const int32_t*>(s.packed), s.packed_src,
+                       static_cast<int32_t*>(out_indices), select_index, parent_index);
   return check_launch("col_row_slice_compact");
 }
 
@@ -582,46 +827,19 @@ int gs_coo_filter_mark(const void* key, int id_bytes, int64_t E, const int64_t* 
              "gs_coo_filter_mark: too many batches");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_coo_filter_mark: id_bytes must be 4 or 8, got %d",
              id_bytes);
-  if (num_batches == 0) {
-    Scratch s0 = carve(workspace, workspace_bytes, num_ids, E, true);
-    if (!s0.ok) {
-      set_error_text("gs_coo_filter_mark: workspace needs %zu bytes, 256-byte aligned",
-                     gs_row_slice_workspace_bytes(num_ids, E, 0));
-      return GS_ERR_WORKSPACE;
-    }
-    hipStream_t st0 = static_cast<hipStream_t>(stream);
-    GS_RETURN_IF_ERROR(id_bytes == 8 ? mark_common<int64_t>("coo_filter_mark", key, E, ids, num_ids,
-                                                            s0, st0)
-                                     : mark_common<int32_t>("coo_filter_mark", key, E, ids, num_ids,
-                                                            s0, st0));
-    hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(64), 0, st0, s0.prefix, E, num_kept);
-    return check_launch("coo_filter_mark");
-  }
-  Scratch s = carve(workspace, workspace_bytes, num_ids, E, true);
+  MarkScratch s = carve_marks(workspace, workspace_bytes, num_ids, E, true);
   if (!s.ok) {
     set_error_text("gs_coo_filter_mark: workspace needs %zu bytes, 256-byte aligned",
                    gs_row_slice_workspace_bytes(num_ids, E, 0));
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(s.cap, kThreads)), dim3(kThreads), 0, st,
-                     s.set, s.cap);
-  auto run = [&](auto tag) {
-    using IdT = decltype(tag);
-    if (num_ids > 0)
-      hipLaunchKernelGGL(set_insert_batched_kernel<IdT>, dim3(blocks_for(num_ids, kThreads)),
-                         dim3(kThreads), 0, st, s.set, static_cast<const IdT*>(ids), num_ids,
-                         ids_batch_ptr, num_batches, int64_t(1) << kBatchShift);
-    if (E > 0)
-      hipLaunchKernelGGL(mark_batched_kernel<IdT>, dim3(blocks_for(E, kThreads)), dim3(kThreads), 0,
-                         st, s.set, static_cast<const IdT*>(key), E, key_batch_ptr, num_batches,
-                         s.val);
-  };
-  if (id_bytes == 8) run(int64_t{}); else run(int32_t{});
-  GS_RETURN_IF_ERROR(check_launch("coo_filter_mark"));
-  Kept f{s.val};
-  GS_RETURN_IF_ERROR(exclusive_scan(f, E, s.prefix, s.tiles, st));
-  hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(64), 0, st, s.prefix, E, num_kept);
+  GS_RETURN_IF_ERROR(id_bytes == 8
+                         ? mark_common<int64_t>("coo_filter_mark", key, E, key_batch_ptr, ids, num_ids,
+                                                ids_batch_ptr, num_batches, false, s, st)
+                         : mark_common<int32_t>("coo_filter_mark", key, E, key_batch_ptr, ids, num_ids,
+                                                ids_batch_ptr, num_batches, false, s, st));
+  hipLaunchKernelGGL(copy_total_kernel, dim3(1), dim3(kWave), 0, st, s.m, num_kept);
   return check_launch("coo_filter_mark");
 }
 
@@ -634,7 +852,7 @@ int gs_coo_filter_compact(const void* row, const void* col, int id_bytes, int64_
              id_bytes);
   GS_REQUIRE(!out_batch_ptr || (num_batches > 0 && key_batch_ptr),
              "gs_coo_filter_compact: batch offsets of the result need those of the input");
-  Scratch s = carve(workspace, workspace_bytes, 0, E, false);
+  MarkScratch s = carve_marks(workspace, workspace_bytes, 0, E, false);
   if (!s.ok) {
     set_error_text("gs_coo_filter_compact: pass the workspace given to gs_coo_filter_mark");
     return GS_ERR_WORKSPACE;
@@ -642,19 +860,19 @@ int gs_coo_filter_compact(const void* row, const void* col, int id_bytes, int64_
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (out_batch_ptr)
     hipLaunchKernelGGL(filter_batch_ptr_kernel, dim3(blocks_for(num_batches + 1, kThreads)),
-                       dim3(kThreads), 0, st, key_batch_ptr, num_batches, s.prefix, out_batch_ptr);
+                       dim3(kThreads), 0, st, key_batch_ptr, num_batches, s.m, out_batch_ptr);
   if (E > 0) {
     GS_REQUIRE(row && col && out_row && out_col, "gs_coo_filter_compact: null pointer");
-    const dim3 grid(blocks_for(E, kThreads));
+    const dim3 grid(static_cast<unsigned>(s.m.tiles));
     if (id_bytes == 8)
-      hipLaunchKernelGGL(filter_compact_kernel<int64_t>, grid, dim3(kThreads), 0, st,
-                         static_cast<const int64_t*>(row), static_cast<const int64_t*>(col), E,
-                         s.val, s.prefix, static_cast<int64_t*>(out_row),
+      hipLaunchKernelGGL((coo_compact_kernel<false, int64_t>), grid, dim3(kThreads), 0, st,
+                         static_cast<const int64_t*>(row), static_cast<const int64_t*>(col), E, s.m,
+                         static_cast<const int64_t*>(nullptr), static_cast<int64_t*>(out_row),
                          static_cast<int64_t*>(out_col), select_index);
     else
-      hipLaunchKernelGGL(filter_compact_kernel<int32_t>, grid, dim3(kThreads), 0, st,
-                         static_cast<const int32_t*>(row), static_cast<const int32_t*>(col), E,
-                         s.val, s.prefix, static_cast<int32_t*>(out_row),
+      hipLaunchKernelGGL((coo_compact_kernel<false, int32_t>), grid, dim3(kThreads), 0, st,
+                         static_cast<const int32_t*>(row), static_cast<const int32_t*>(col), E, s.m,
+                         static_cast<const int32_t*>(nullptr), static_cast<int32_t*>(out_row),
                          static_cast<int32_t*>(out_col), select_index);
   }
   return check_launch("coo_filter_compact");
@@ -667,15 +885,14 @@ int gs_index_search(const void* data, int64_t n, const void* keys, int64_t m, in
   GS_REQUIRE(n >= 0 && m >= 0, "gs_index_search: negative size");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_index_search: id_bytes must be 4 or 8, got %d", id_bytes);
   GS_REQUIRE((n == 0 || data) && (m == 0 || (keys && out)), "gs_index_search: null pointer");
-  Scratch s = carve(workspace, workspace_bytes, n, 0, true);
+  MarkScratch s = carve_marks(workspace, workspace_bytes, n, 0, true);
   if (!s.ok) {
     set_error_text("gs_index_search: workspace needs %zu bytes, 256-byte aligned",
                    gs_index_search_workspace_bytes(n));
     return GS_ERR_WORKSPACE;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(set_init_kernel, dim3(blocks_for(s.cap, kThreads)), dim3(kThreads), 0, st,
-                     s.set, s.cap);
+  init_set(s.set, s.cap, s.filter_words, st);
   auto run = [&](auto tag) {
     using IdT = decltype(tag);
     if (n > 0)
