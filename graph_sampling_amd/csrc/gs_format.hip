@@ -14,8 +14,11 @@
 //    (format_transform.cu:58-72 also sorts just the significant bits).  Each
 //    pass is histogram -> scan -> stable scatter; the scatter ranks equal digits
 //    inside a wave with 8 ballots (no LDS atomics, order preserved) and across
-//    waves with a small LDS table.  indptr then comes from one binary search
-//    per column in the sorted keys.
+//    waves with a small LDS table.  What moves is one 64-bit word per edge, key
+//    above and original position below, so a pass is 8 bytes in and 8 bytes out per
+//    edge and the permutation falls out of the last pass.  indptr then comes from
+//    one search per column in the sorted keys, confined to the keys of the
+//    workgroup's 1024 columns (in LDS when they are few).
 #include "gs_common.hpp"
 
 namespace gs {
@@ -131,41 +134,131 @@ compress_kernel(const int64_t* __restrict__ indptr, int64_t num_cols,
   }
 }
 
-// indptr from sorted keys: indptr[c] = number of keys < c, one binary search per
-// column (format_transform.cu:123-156 does the same).  A boundary-driven fill
-// (every edge writes the offsets of the columns between it and its predecessor)
-// was tried first and is worse at both ends: with few edges and millions of
-// columns one lane fills a gap of a million offsets by itself, with many edges
-// and few columns it reads every key to find a handful of boundaries.
+// Sorted keys as the kernels below read them: an id array, or the sort's own words
+// (key above the low idx_bits bits).
 template <typename KeyT>
-__global__ void __launch_bounds__(kThreads)
-indptr_from_sorted_kernel(const KeyT* __restrict__ key, int64_t E, int64_t num_keys,
-                          int64_t* __restrict__ indptr) {
-  const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (c > num_keys) return;
-  int64_t lo = 0, hi = E;  // first position whose key is >= c
+struct PlainKeys {
+  const KeyT* key;
+  __device__ __forceinline__ int64_t operator()(int64_t i) const {
+    return static_cast<int64_t>(key[i]);
+  }
+};
+struct WordKeys {
+  const unsigned long long* word;
+  int idx_bits;
+  __device__ __forceinline__ int64_t operator()(int64_t i) const {
+    return static_cast<int64_t>(word[i] >> idx_bits);
+  }
+};
+
+template <typename Keys>
+__device__ __forceinline__ int64_t first_not_below(const Keys& key, int64_t lo, int64_t hi,
+                                                   int64_t c) {
   while (lo < hi) {
     const int64_t mid = (lo + hi) >> 1;
-    if (static_cast<int64_t>(key[mid]) < c) lo = mid + 1; else hi = mid;
+    if (key(mid) < c) lo = mid + 1; else hi = mid;
   }
-  indptr[c] = lo;
+  return lo;
+}
+
+// First position in [0, E) whose key is >= c, found by a whole wave: 64 probes split the
+// range per step, so 2.7 M keys take four dependent loads instead of twenty-two.  Every
+// lane of the wave calls this and gets the answer.
+template <typename Keys>
+__device__ __forceinline__ int64_t wave_first_not_below(const Keys& key, int64_t E, int64_t c) {
+  const int lane = threadIdx.x & (kWave - 1);
+  int64_t lo = 0, hi = E;
+  while (lo < hi) {
+    const int64_t step = (hi - lo + kWave - 1) / kWave;
+    const int64_t at = lo + lane * step;
+    const bool below = at < hi && key(at) < c;
+    const int count = __popcll(__ballot(below));  // probes are sorted: the first `count` are below
+    const int64_t new_lo = count > 0 ? lo + (count - 1) * step + 1 : lo;
+    const int64_t end = lo + count * step;        // first probe that is not below, if there is one
+    hi = (count < kWave && end < hi) ? end : hi;
+    lo = new_lo;
+  }
+  return lo;
+}
+
+// indptr from sorted keys: indptr[c] = number of keys < c (format_transform.cu:123-156
+// searches the whole key array once per column).  A workgroup owns 256 consecutive
+// columns: two wave-wide searches bound the keys that belong to them, and the per-column
+// searches run inside that range -- in LDS when it holds at most 4096 keys, which is every
+// tile but those of hub columns.  A boundary-driven fill (every edge writes the offsets of
+// the columns between it and its predecessor) was tried first and is worse at both ends:
+// with few edges and millions of columns one lane fills a gap of a million offsets by
+// itself, with many edges and few columns it reads every key to find a handful of
+// boundaries.
+constexpr int kPtrCols = kThreads;
+constexpr int kPtrStage = 4096;
+
+template <typename Keys>
+__global__ void __launch_bounds__(kThreads)
+indptr_from_sorted_kernel(Keys key, int64_t E, int64_t num_keys, int64_t* __restrict__ indptr) {
+  __shared__ int64_t s_range[2];
+  __shared__ int s_key[kPtrStage];
+  const int64_t c0 = static_cast<int64_t>(blockIdx.x) * kPtrCols;
+  const int64_t c1 = c0 + kPtrCols < num_keys + 1 ? c0 + kPtrCols : num_keys + 1;
+  const int wave = threadIdx.x / kWave;
+  if (wave < 2) {
+    const int64_t at = wave_first_not_below(key, E, wave == 0 ? c0 : c1);
+    if ((threadIdx.x & (kWave - 1)) == 0) s_range[wave] = at;
+  }
+  __syncthreads();
+  const int64_t lo = s_range[0], hi = s_range[1];
+  const int n = static_cast<int>(hi - lo <= kPtrStage ? hi - lo : -1);
+  if (n >= 0) {
+    for (int i = threadIdx.x; i < n; i += kThreads) s_key[i] = static_cast<int>(key(lo + i) - c0);
+    __syncthreads();
+  }
+  const int64_t c = c0 + threadIdx.x;
+  if (c >= c1) return;
+  if (n >= 0) {
+    const int want = static_cast<int>(c - c0);
+    int a = 0, b = n;
+    while (a < b) {
+      const int mid = (a + b) >> 1;
+      if (s_key[mid] < want) a = mid + 1; else b = mid;
+    }
+    indptr[c] = lo + a;
+  } else {
+    indptr[c] = first_not_below(key, lo, hi, c);
+  }
 }
 
 // ------------------------------------------------------------ radix sort ----
+// The sort moves ONE 64-bit word per edge: key above, position of the edge below
+// (idx_bits = bits of the edge count).  Sorting the words is the stable sort of the keys,
+// the low bits of the result are the permutation, and a pass reads and writes 8 bytes per
+// edge instead of a widened key and a permutation entry each way.
 constexpr int kRadixBits = 8;
 constexpr int kRadix = 1 << kRadixBits;
 constexpr int kWaves = kThreads / kWave;
 
-__device__ __forceinline__ int digit_of(int64_t key, int shift) {
-  return static_cast<int>((static_cast<uint64_t>(key) >> shift) & (kRadix - 1));
+__device__ __forceinline__ int digit_of(unsigned long long word, int shift) {
+  return static_cast<int>((word >> shift) & (kRadix - 1));
 }
 
-// counts[d * num_blocks + b] = items of tile b with digit d.  KeyT is the
-// caller's id type in the first pass and int64 (the ping-pong buffers) after it.
-template <typename KeyT>
+// words of the first pass, made from the caller's keys on the fly
+template <typename IdT>
+struct FreshWords {
+  const IdT* key;
+  int idx_bits;
+  __device__ __forceinline__ unsigned long long operator()(int64_t i) const {
+    return (static_cast<unsigned long long>(key[i]) << idx_bits) |
+           static_cast<unsigned long long>(i);
+  }
+};
+struct StoredWords {
+  const unsigned long long* word;
+  __device__ __forceinline__ unsigned long long operator()(int64_t i) const { return word[i]; }
+};
+
+// counts[d * num_blocks + b] = items of tile b with digit d
+template <typename Src>
 __global__ void __launch_bounds__(kThreads)
-radix_hist_kernel(const KeyT* __restrict__ keys, int64_t E, int shift, int64_t num_blocks,
-                  int64_t* __restrict__ counts) {
+radix_hist_kernel(Src src, int64_t E, int shift, int64_t num_blocks, int64_t* __restrict__ counts) {
   __shared__ int s_hist[kRadix];
   s_hist[threadIdx.x] = 0;
   __syncthreads();
@@ -173,7 +266,7 @@ radix_hist_kernel(const KeyT* __restrict__ keys, int64_t E, int shift, int64_t n
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
     const int64_t i = base + k * kThreads + threadIdx.x;
-    if (i < E) atomicAdd(&s_hist[digit_of(static_cast<int64_t>(keys[i]), shift)], 1);
+    if (i < E) atomicAdd(&s_hist[digit_of(src(i), shift)], 1);
   }
   __syncthreads();
   counts[static_cast<int64_t>(threadIdx.x) * num_blocks + blockIdx.x] = s_hist[threadIdx.x];
@@ -187,30 +280,31 @@ struct LoadI64 {
 // Stable scatter of one tile.  Items are visited in index order, 256 per round;
 // inside a round the rank of an item among equal digits is (earlier waves'
 // count) + (lower lanes of its wave with the same digit).
-template <typename KeyT>
+template <typename Src>
 __global__ void __launch_bounds__(kThreads)
-radix_scatter_kernel(const KeyT* __restrict__ keys_in, const int64_t* __restrict__ perm_in,
-                     int64_t E, int shift, int64_t num_blocks, const int64_t* __restrict__ offsets,
-                     int64_t* __restrict__ keys_out, int64_t* __restrict__ perm_out) {
+radix_scatter_kernel(Src src, int64_t E, int shift, int64_t num_blocks,
+                     const int64_t* __restrict__ offsets, unsigned long long* __restrict__ out) {
   __shared__ int64_t s_base[kRadix];
   __shared__ int s_cnt[kWaves][kRadix];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   s_base[threadIdx.x] = offsets[static_cast<int64_t>(threadIdx.x) * num_blocks + blockIdx.x];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kTile;
+  unsigned long long words[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = base + k * kThreads + threadIdx.x;
+    words[k] = i < E ? src(i) : 0ull;
+  }
+#pragma unroll
   for (int k = 0; k < kItems; ++k) {
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) s_cnt[w][threadIdx.x] = 0;
     __syncthreads();
     const int64_t i = base + k * kThreads + threadIdx.x;
     const bool live = i < E;
-    int64_t key = 0;
-    int d = 0;
+    const int d = live ? digit_of(words[k], shift) : 0;
     unsigned long long peers = __ballot(live);
-    if (live) {
-      key = static_cast<int64_t>(keys_in[i]);
-      d = digit_of(key, shift);
-    }
 #pragma unroll
     for (int b = 0; b < kRadixBits; ++b) {
       const bool bit = (d >> b) & 1;
@@ -223,8 +317,7 @@ radix_scatter_kernel(const KeyT* __restrict__ keys_in, const int64_t* __restrict
     if (live) {
       int64_t dst = s_base[d] + rank;
       for (int w = 0; w < wave; ++w) dst += s_cnt[w][d];
-      keys_out[dst] = key;
-      perm_out[dst] = perm_in ? perm_in[i] : i;
+      out[dst] = words[k];
     }
     __syncthreads();
     int add = 0;
@@ -235,18 +328,27 @@ radix_scatter_kernel(const KeyT* __restrict__ keys_in, const int64_t* __restrict
   }
 }
 
+// perm[i] = position the i-th edge of the result had; out[i] = value of that edge
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
-gather_kernel(const IdT* __restrict__ value, const int64_t* __restrict__ perm, int64_t E,
-              IdT* __restrict__ out) {
+unpack_gather_kernel(const unsigned long long* __restrict__ word, int idx_bits,
+                     const IdT* __restrict__ value, int64_t E, int64_t* __restrict__ perm,
+                     IdT* __restrict__ out) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (i < E) out[i] = value[perm[i]];
+  if (i >= E) return;
+  const int64_t from = static_cast<int64_t>(word[i] & ((1ull << idx_bits) - 1ull));
+  perm[i] = from;
+  out[i] = value[from];
+}
+
+int bits_for(int64_t n) {  // smallest b with 2^b >= n
+  int bits = 0;
+  while ((int64_t(1) << bits) < n) ++bits;
+  return bits;
 }
 
 int num_passes(int64_t num_keys) {
-  int bits = 0;
-  while ((int64_t(1) << bits) < num_keys) ++bits;  // format_transform.cu:58-72
-  return (bits + kRadixBits - 1) / kRadixBits;
+  return (bits_for(num_keys) + kRadixBits - 1) / kRadixBits;  // format_transform.cu:58-72
 }
 
 // Offsets of B consecutive column ranges, each re-based to start at 0 and laid
@@ -270,16 +372,25 @@ template <typename IdT>
 int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, int sorted,
                  int64_t* indptr, IdT* out_value, int64_t* perm, void* workspace,
                  size_t workspace_bytes, hipStream_t st) {
+  const dim3 ptr_grid(blocks_for(num_keys + 1, kPtrCols));
   if (sorted || E == 0) {
-    hipLaunchKernelGGL((indptr_from_sorted_kernel<IdT>), dim3(blocks_for(num_keys + 1, kThreads)),
-                       dim3(kThreads), 0, st, key, E, num_keys, indptr);
+    PlainKeys<IdT> keys{key};
+    hipLaunchKernelGGL((indptr_from_sorted_kernel<PlainKeys<IdT>>), ptr_grid, dim3(kThreads), 0, st,
+                       keys, E, num_keys, indptr);
     return check_launch("coo2csc");
+  }
+  const int idx_bits = bits_for(E);
+  int passes = num_passes(num_keys);
+  if (passes == 0) passes = 1;  // one key: still produces perm = identity
+  if (idx_bits + passes * kRadixBits > 64) {
+    set_error_text("gs_coo2csc: %lld edges with keys below %lld do not fit the sort's 64-bit words",
+                   static_cast<long long>(E), static_cast<long long>(num_keys));
+    return GS_ERR_UNSUPPORTED;
   }
   const int64_t blocks = blocks_for(E, kTile);
   const int64_t table = kRadix * blocks;
   Carver ws(workspace, workspace_bytes);
-  int64_t* kbuf[2] = {ws.take<int64_t>(E), ws.take<int64_t>(E)};
-  int64_t* pbuf = ws.take<int64_t>(E);
+  unsigned long long* wbuf[2] = {ws.take<unsigned long long>(E), ws.take<unsigned long long>(E)};
   int64_t* counts = ws.take<int64_t>(table);
   int64_t* offsets = ws.take<int64_t>(table + 1);
   int64_t* tiles = ws.take<int64_t>(scan_num_tiles(table) + 1);
@@ -288,36 +399,38 @@ int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, 
                    gs_coo2csc_workspace_bytes(E, num_keys));
     return GS_ERR_WORKSPACE;
   }
-  int passes = num_passes(num_keys);
-  if (passes == 0) passes = 1;  // one key: still produces perm = identity
-  const int64_t* kin = nullptr;  // null: the first pass reads the caller's keys
-  const int64_t* pin = nullptr;
-  // perm alternates between `perm` and pbuf so that the last pass lands in `perm`
+  const dim3 grid(static_cast<unsigned>(blocks));
+  const unsigned long long* win = nullptr;  // null: the first pass reads the caller's keys
   for (int p = 0; p < passes; ++p) {
-    int64_t* kout = kbuf[p & 1];
-    int64_t* pout = ((passes - 1 - p) & 1) ? pbuf : perm;
-    if (p == 0)
-      hipLaunchKernelGGL((radix_hist_kernel<IdT>), dim3(static_cast<unsigned>(blocks)),
-                         dim3(kThreads), 0, st, key, E, 0, blocks, counts);
-    else
-      hipLaunchKernelGGL((radix_hist_kernel<int64_t>), dim3(static_cast<unsigned>(blocks)),
-                         dim3(kThreads), 0, st, kin, E, p * kRadixBits, blocks, counts);
+    unsigned long long* wout = wbuf[p & 1];
+    const int shift = idx_bits + p * kRadixBits;
+    if (p == 0) {
+      FreshWords<IdT> src{key, idx_bits};
+      hipLaunchKernelGGL((radix_hist_kernel<FreshWords<IdT>>), grid, dim3(kThreads), 0, st, src, E,
+                         shift, blocks, counts);
+    } else {
+      StoredWords src{win};
+      hipLaunchKernelGGL((radix_hist_kernel<StoredWords>), grid, dim3(kThreads), 0, st, src, E, shift,
+                         blocks, counts);
+    }
     LoadI64 f{counts};
     GS_RETURN_IF_ERROR(exclusive_scan(f, table, offsets, tiles, st));
-    if (p == 0)
-      hipLaunchKernelGGL((radix_scatter_kernel<IdT>), dim3(static_cast<unsigned>(blocks)),
-                         dim3(kThreads), 0, st, key, pin, E, 0, blocks, offsets, kout, pout);
-    else
-      hipLaunchKernelGGL((radix_scatter_kernel<int64_t>), dim3(static_cast<unsigned>(blocks)),
-                         dim3(kThreads), 0, st, kin, pin, E, p * kRadixBits, blocks, offsets, kout,
-                         pout);
-    kin = kout;
-    pin = pout;
+    if (p == 0) {
+      FreshWords<IdT> src{key, idx_bits};
+      hipLaunchKernelGGL((radix_scatter_kernel<FreshWords<IdT>>), grid, dim3(kThreads), 0, st, src, E,
+                         shift, blocks, offsets, wout);
+    } else {
+      StoredWords src{win};
+      hipLaunchKernelGGL((radix_scatter_kernel<StoredWords>), grid, dim3(kThreads), 0, st, src, E,
+                         shift, blocks, offsets, wout);
+    }
+    win = wout;
   }
-  hipLaunchKernelGGL((gather_kernel<IdT>), dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st,
-                     value, perm, E, out_value);
-  hipLaunchKernelGGL((indptr_from_sorted_kernel<int64_t>), dim3(blocks_for(num_keys + 1, kThreads)),
-                     dim3(kThreads), 0, st, kin, E, num_keys, indptr);
+  hipLaunchKernelGGL((unpack_gather_kernel<IdT>), dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st,
+                     win, idx_bits, value, E, perm, out_value);
+  WordKeys keys{win, idx_bits};
+  hipLaunchKernelGGL((indptr_from_sorted_kernel<WordKeys>), ptr_grid, dim3(kThreads), 0, st, keys, E,
+                     num_keys, indptr);
   return check_launch("coo2csc");
 }
 
@@ -403,7 +516,7 @@ size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys) {
   if (E < 0) E = 0;
   const int64_t blocks = blocks_for(E, kTile);
   const int64_t table = kRadix * blocks;
-  return 3 * padded(static_cast<size_t>(E > 0 ? E : 1) * 8) +  // keys ping-pong, perm pong
+  return 2 * padded(static_cast<size_t>(E > 0 ? E : 1) * 8) +  // the sort's words, ping-pong
          padded(static_cast<size_t>(table) * 8) + padded(static_cast<size_t>(table + 1) * 8) +
          scan_workspace_bytes(table);
 }
