@@ -12,9 +12,11 @@
 // (list_sampling_probs.cu:76-86).  Here the k-th largest 64-bit composite
 // (ordered key << 32 | ~position) is found by a six-level radix SELECT
 // (11+11+10 bits of key, 11+11+10 bits of position): each level is one pass
-// over the 4-byte keys with LDS-private histograms plus a one-workgroup pick,
-// then exactly k survivors are gathered and only those k are sorted (bitonic,
-// in LDS).  Algorithmic traffic is 4 B/item/level instead of 12 B/item per
+// over the 4-byte keys with LDS-private histograms; the pick of a level (which
+// bin holds the k-th item) is made at the head of the NEXT level's kernel, by every
+// workgroup for itself from the finished histogram, so a level is one launch and
+// not two.  Then exactly k survivors are gathered and only those k are sorted
+// (bitonic, in LDS).  Algorithmic traffic is 4 B/item/level instead of 12 B/item per
 // radix-sort pass over key+index pairs.
 #include "gs_common.hpp"
 
@@ -75,10 +77,11 @@ list_gather_kernel(const IdT* __restrict__ data, const int64_t* __restrict__ ind
 }
 
 // ------------------------------------------------------------ weighted -----
+// state[L]: the selection after the picks of levels 0 .. L-1 (state[0]: nothing picked)
 struct SelectState {
   unsigned long long prefix;     // digits chosen so far, in place
   unsigned long long remaining;  // how many of the matching items are still wanted
-  unsigned long long gathered;   // survivor counter
+  unsigned long long gathered;   // survivor counter (state[0] only)
   unsigned long long done;       // every item under the prefix is wanted: lower digits do not matter
 };
 
@@ -126,15 +129,68 @@ keys_hist_kernel(const float* __restrict__ probs, int64_t n, uint64_t seed,
     if (s_hist[i]) atomicAdd(&hist[i], s_hist[i]);
 }
 
-// Levels 1..5: histogram of the next digit over the items that match the prefix.
+// The bin of `level` that holds the `remaining`-th largest item under the prefix, from the
+// finished histogram of that level.  Called by every thread of a workgroup; every
+// workgroup of a launch arrives at the same answer.
+struct PickScratch {
+  int64_t scan[kThreads / kWave + 1];
+  SelectState out;
+};
+
+__device__ __forceinline__ SelectState pick_level(const uint32_t* __restrict__ hist, int level,
+                                                  const SelectState& in, PickScratch* lds) {
+  if (in.done) return in;
+  const uint32_t* h = hist + level * kBins;
+  constexpr int kPer = kBins / kThreads;  // 8 consecutive bins per thread
+  int64_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) mine += h[threadIdx.x * kPer + j];
+  int64_t total;
+  const int64_t below = block_exclusive_scan<kThreads>(mine, &total, lds->scan);
+  if (threadIdx.x == 0) lds->out = in;
+  __syncthreads();
+  const unsigned long long want = in.remaining;
+  unsigned long long above = static_cast<unsigned long long>(total - below - mine);  // bins of threads > t
+  if (above < want && want <= above + static_cast<unsigned long long>(mine)) {
+    for (int j = kPer - 1; j >= 0; --j) {
+      const unsigned long long cnt = h[threadIdx.x * kPer + j];
+      if (want <= above + cnt) {
+        SelectState s = in;
+        s.prefix |= static_cast<unsigned long long>(threadIdx.x * kPer + j) << c_shift[level];
+        s.remaining = want - above;
+        // all of the bin is wanted (typically a bin of one): with the lower digits left at zero
+        // "composite >= prefix" already selects exactly the wanted items
+        if (want - above == cnt) s.done = 1;
+        lds->out = s;
+        break;
+      }
+      above += cnt;
+    }
+  }
+  __syncthreads();
+  const SelectState r = lds->out;
+  __syncthreads();
+  return r;
+}
+
+// Levels 1..5: the pick of the level before, then the histogram of this level's digit over
+// the items that match the prefix.  Workgroup 0 leaves the state after the pick in
+// state[level] for the next launch.
 __global__ void __launch_bounds__(kThreads)
-level_hist_kernel(const uint32_t* __restrict__ okey, int64_t n, int level,
-                  const SelectState* __restrict__ st, uint32_t* __restrict__ hist) {
+level_hist_kernel(const uint32_t* __restrict__ okey, int64_t n, int level, SelectState* state,
+                  uint32_t* __restrict__ hist) {
   __shared__ uint32_t s_hist[kBins];
-  if (st->done) return;  // the pick of an earlier level took its whole bin: nothing left to split
+  __shared__ PickScratch s_pick;
+  const SelectState st = pick_level(hist, level - 1, state[level - 1], &s_pick);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    state[level].prefix = st.prefix;
+    state[level].remaining = st.remaining;
+    state[level].done = st.done;
+  }
+  if (st.done) return;  // a pick took its whole bin: nothing left to split
   for (int i = threadIdx.x; i < kBins; i += kThreads) s_hist[i] = 0;
   __syncthreads();
-  const unsigned long long prefix = st->prefix;
+  const unsigned long long prefix = st.prefix;
   const int up = c_shift[level - 1];
   const int sh = c_shift[level];
   const uint32_t mask = (1u << c_width[level]) - 1u;
@@ -149,54 +205,19 @@ level_hist_kernel(const uint32_t* __restrict__ okey, int64_t n, int level,
     if (s_hist[i]) atomicAdd(&h[i], s_hist[i]);
 }
 
-// One workgroup: the bin holding the `remaining`-th largest item of this level.
+// The pick of the last level, then the items at or above the k-th.
 __global__ void __launch_bounds__(kThreads)
-level_pick_kernel(const uint32_t* __restrict__ hist, int level, SelectState* st) {
-  __shared__ unsigned long long s_tail[kThreads];  // items in the bins owned by threads > t
-  if (st->done) return;
-  const unsigned long long want = st->remaining;   // read before anyone updates it
-  const uint32_t* h = hist + level * kBins;
-  constexpr int kPer = kBins / kThreads;  // 8 consecutive bins per thread
-  unsigned long long mine = 0;
-#pragma unroll
-  for (int j = 0; j < kPer; ++j) mine += h[threadIdx.x * kPer + j];
-  s_tail[threadIdx.x] = mine;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned long long acc = 0;
-    for (int t = kThreads - 1; t >= 0; --t) {
-      const unsigned long long v = s_tail[t];
-      s_tail[t] = acc;
-      acc += v;
-    }
-  }
-  __syncthreads();
-  unsigned long long above = s_tail[threadIdx.x];
-  if (above < want && want <= above + mine) {
-    for (int j = kPer - 1; j >= 0; --j) {
-      const unsigned long long cnt = h[threadIdx.x * kPer + j];
-      if (want <= above + cnt) {
-        st->prefix |= static_cast<unsigned long long>(threadIdx.x * kPer + j) << c_shift[level];
-        st->remaining = want - above;
-        // all of the bin is wanted (typically a bin of one): with the lower digits left at zero
-        // "composite >= prefix" already selects exactly the wanted items
-        if (want - above == cnt) st->done = 1;
-        break;
-      }
-      above += cnt;
-    }
-  }
-}
-
-__global__ void __launch_bounds__(kThreads)
-survivors_kernel(const uint32_t* __restrict__ okey, int64_t n, SelectState* st,
-                 unsigned long long* __restrict__ cand, int64_t k) {
-  const unsigned long long kth = st->prefix;
+survivors_kernel(const uint32_t* __restrict__ okey, int64_t n, SelectState* state,
+                 const uint32_t* __restrict__ hist, unsigned long long* __restrict__ cand,
+                 int64_t k) {
+  __shared__ PickScratch s_pick;
+  const SelectState st = pick_level(hist, kLevels - 1, state[kLevels - 1], &s_pick);
+  const unsigned long long kth = st.prefix;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n;
        i += static_cast<int64_t>(gridDim.x) * kThreads) {
     const unsigned long long c = list_composite(okey[i], i);
     if (c >= kth) {
-      const unsigned long long slot = atomicAdd(&st->gathered, 1ull);
+      const unsigned long long slot = atomicAdd(&state[0].gathered, 1ull);
       if (static_cast<int64_t>(slot) < k) cand[slot] = c;
     }
   }
@@ -246,7 +267,7 @@ WeightedScratch carve_weighted(void* ws_ptr, size_t bytes, int64_t n, int64_t k)
   WeightedScratch s;
   s.okey = ws.take<uint32_t>(n > 0 ? n : 1);
   s.hist = ws.take<uint32_t>(kLevels * kBins);
-  s.state = ws.take<SelectState>(1);
+  s.state = ws.take<SelectState>(kLevels);
   s.cand = ws.take<unsigned long long>(k > 0 ? k : 1);
   s.ok = ws.ok;
   return s;
@@ -283,14 +304,11 @@ int list_weighted_impl(const void* data, const float* probs, int64_t n, int64_t 
   hipLaunchKernelGGL(select_init_kernel, dim3(1), dim3(kThreads), 0, st, s.hist, s.state, k);
   hipLaunchKernelGGL(keys_hist_kernel, dim3(grid), dim3(kThreads), 0, st, probs, n, seed, replay,
                      s.okey, s.hist);
-  for (int level = 0; level < kLevels; ++level) {
-    if (level > 0)
-      hipLaunchKernelGGL(level_hist_kernel, dim3(grid), dim3(kThreads), 0, st, s.okey, n, level,
-                         s.state, s.hist);
-    hipLaunchKernelGGL(level_pick_kernel, dim3(1), dim3(kThreads), 0, st, s.hist, level, s.state);
-  }
-  hipLaunchKernelGGL(survivors_kernel, dim3(grid), dim3(kThreads), 0, st, s.okey, n, s.state, s.cand,
-                     k);
+  for (int level = 1; level < kLevels; ++level)
+    hipLaunchKernelGGL(level_hist_kernel, dim3(grid), dim3(kThreads), 0, st, s.okey, n, level,
+                       s.state, s.hist);
+  hipLaunchKernelGGL(survivors_kernel, dim3(grid), dim3(kThreads), 0, st, s.okey, n, s.state, s.hist,
+                     s.cand, k);
   int padded_k = 2;
   while (padded_k < k) padded_k <<= 1;
   hipLaunchKernelGGL((sort_emit_kernel<IdT>), dim3(1), dim3(1024),
@@ -310,7 +328,7 @@ size_t gs_list_sample_workspace_bytes(int64_t n, int64_t k) {
   if (n < 1) n = 1;
   if (k < 1) k = 1;
   return padded(static_cast<size_t>(n) * 4) + padded(kLevels * kBins * 4) +
-         padded(sizeof(SelectState)) + padded(static_cast<size_t>(k) * 8);
+         padded(kLevels * sizeof(SelectState)) + padded(static_cast<size_t>(k) * 8);
 }
 
 int gs_list_sample_uniform(const void* data, int id_bytes, int64_t n, int64_t k, int replace,
