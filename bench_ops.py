@@ -89,18 +89,20 @@ def main():
     c100k, r200k = perm_ids(100_000), perm_ids(200_000)
     D = int(capi.slice_count(indptr, c100k)[-1].item())
     run("col_row_slice", "gs_col_row_slice_*: 100k columns x 200k rows, D = %d edges looked at; "
-        "b + 16 B per edge looked at (id read, mark, scan), 2b + 16 per edge kept" % D,
+        "b B per edge looked at (id read; one mark bit), 2b + 16 per edge kept twice (packed, "
+        "then placed)" % D,
         lambda: capi.col_row_slice(indptr, indices, c100k, r200k),
-        lambda o: (D * (b + 16) + o[1].numel() * (2 * b + 16), D, "edges"))
+        lambda o: (D * b + o[1].numel() * 2 * (2 * b + 16), D, "edges"))
 
     # ---- row slicing of a column slice (FastGCN layer: keep 512 sampled rows) -----------------
     sp = capi.slice_count(indptr, cols45k)
     nnz = int(sp[-1].item())
     s_idx, s_sel, s_col = capi.slice_fill(indptr, indices, cols45k, sp, nnz, True)
     rows512 = perm_ids(512)
-    run("row_slice_coo", "gs_row_slice_coo_*: %d edges, 512 row ids; b + 16 B per edge" % nnz,
+    run("row_slice_coo", "gs_row_slice_coo_*: %d edges, 512 row ids; b B per edge looked at, "
+        "3b + 8 per edge kept" % nnz,
         lambda: capi.row_slice_coo(s_idx, s_col, rows512),
-        lambda o: (nnz * (b + 16), nnz, "edges"))
+        lambda o: (nnz * b + o[0].numel() * (3 * b + 8), nnz, "edges"))
 
     # ---- weighted sampling of the same slice ---------------------------------------------------
     w_slice = weights[:nnz].contiguous()
@@ -161,9 +163,9 @@ def main():
     ids_ptr = (torch.arange(B + 1, device=dev, dtype=torch.int64) * 4000)
     chosen = rand_ids(B * 4000)
     run("coo_filter_batched", "gs_coo_filter_*: 14M edges in 64 batches against 4000 chosen ids per "
-        "batch; b + 16 B per edge (key, mark, scan)",
+        "batch; b B per edge looked at (key read; one mark bit), 4b + 8 per edge kept",
         lambda: capi.coo_filter(data, data, col14, chosen, ptr, ids_ptr),
-        lambda o: (M * (b + 16) + o[0].numel() * 4 * b, M, "edges"))
+        lambda o: (M * b + o[0].numel() * (4 * b + 8), M, "edges"))
     run("index_search", "gs_index_search: 14M keys against 256k stored ids; 2b per key",
         lambda: capi.index_search(chosen, data),
         lambda o: (M * 2 * b, M, "keys"))
@@ -245,10 +247,11 @@ def main():
         lambda: capi.segment_normalize(indptr, None, weights, out_nrm),
         lambda o: (E * 12 + N * 16, E, "edges"))
     keep_rows = torch.randperm(N, generator=gen, device=dev)[:200_000].to(idt)
-    run("row_slice_csc", "gs_row_slice_csc_*: the whole graph cut down to 200k of its rows (mark, scan, "
-        "compact); b + 16 B per edge looked at, 2b + 8 per edge kept",
+    run("row_slice_csc", "gs_row_slice_csc_*: the whole graph cut down to 200k of its rows (mark, scan "
+        "of the tile counts, compact); b B per edge looked at, 4b + 8 per edge kept (new id packed and "
+        "placed, column, position)",
         lambda: capi.row_slice_csc(indptr, indices, keep_rows, True),
-        lambda o: (E * (b + 16) + int(o[2].numel()) * (2 * b + 8), E, "edges"))
+        lambda o: (E * b + int(o[2].numel()) * (4 * b + 8), E, "edges"))
     out_n = torch.empty(N, device=dev)
     run("segment_sum", "gs_segment_sum of w^2 over every column of the graph; 4 B per edge + 20 B "
         "per column",
