@@ -10,15 +10,17 @@
 // composite (ordered key << 32 | ~position): composites are distinct, so
 // "largest k" is unambiguous and bit-reproducible.
 //
-// Selection is a wave-level top-k: each of the 64 lanes streams a strided share
-// of the candidates and keeps its own sorted top-k list in LDS
-// (list[j * 64 + lane], conflict-free, touched by its lane only); the final k
-// rounds take the wave-wide maximum of the list heads (6 xor-shuffles of a
-// 64-bit value) and pop it.  Rows up to 2048 edges are one wave each.  Longer
-// rows are cut into 2048-edge chunks that go through a device queue: one wave
-// per chunk writes its local top-k composites, then one wave per long row
-// merges them.  That spreads a 10^5-edge hub over hundreds of waves instead of
-// pinning one warp on it.
+// Selection is a wave-level top-k over at most 2048 candidates, 32 per lane, held in
+// registers: the k-th largest of the 64 lanes' own maxima is a floor that at least k
+// candidates reach, so everything below it is dropped at once; the few survivors
+// (between k and 32 k, typically about 2 k) are packed into LDS with ballots and each
+// one counts how many survivors beat it -- that count is its place in the output.  No
+// per-lane sorted lists, no k rounds of wave-wide maxima.  Rows up to 2048 edges are
+// one wave each.  Longer rows are cut into 2048-edge chunks that go through a device
+// queue: one wave per chunk writes its local top-k composites, then one wave per
+// long row merges them (per-lane sorted lists in LDS and k rounds of "largest head
+// wins": the candidates of a hub's chunks can be many more than 2048).  That spreads a
+// 10^5-edge hub over hundreds of waves instead of pinning one warp on it.
 #include "gs_common.hpp"
 
 namespace gs {
@@ -104,37 +106,97 @@ __device__ __forceinline__ unsigned long long edge_composite(const WArgs<IdT>& a
   return composite(ares_key(xv, a.probs[start + i]), static_cast<uint32_t>(i));
 }
 
-// stream edges [lo, hi) of row r into the per-lane lists
-template <typename IdT>
-__device__ __forceinline__ void stream_edges(const WArgs<IdT>& a, int64_t r, int64_t start,
-                                             int64_t lo, int64_t hi, unsigned long long* list,
-                                             int lane, int& cnt) {
+constexpr int kTrips = kChunk / (4 * kWave);  // a lane holds 4 consecutive edges per trip
+constexpr int64_t kSmall = 4 * kWave;         // rows of one trip: selected where they are found
+
+// composites of edges [lo, hi) of row r (lo a multiple of 2048, hi - lo <= TRIPS * 256):
+// the lane's share, 0 where it has none.  A lane takes 4 consecutive edges (one Philox
+// block) per trip.
+template <int TRIPS, typename IdT>
+__device__ __forceinline__ void load_items(const WArgs<IdT>& a, int64_t r, int64_t start,
+                                           int64_t lo, int64_t hi, int lane,
+                                           unsigned long long (&items)[TRIPS][4]) {
   const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[r] : nullptr;
-  // a lane takes 4 consecutive edges (one Philox block) per trip
-  for (int64_t q = (lo >> 2) + lane; q * 4 < hi; q += kWave) {
-    U4 x;
-    if (!rp) x = draw_block(a.seed, kTagWeighted, static_cast<uint64_t>(r), static_cast<uint64_t>(q));
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const int64_t i = q * 4 + t;
-      if (i >= lo && i < hi) lane_insert(list, lane, cnt, a.k, edge_composite(a, r, start, rp, i, x));
+  for (int t = 0; t < TRIPS; ++t) {
+    const int64_t q = (lo >> 2) + lane + t * kWave;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) items[t][j] = 0ull;
+    if (q * 4 < hi) {
+      U4 x;
+      if (!rp) x = draw_block(a.seed, kTagWeighted, static_cast<uint64_t>(r), static_cast<uint64_t>(q));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t i = q * 4 + j;
+        if (i < hi) items[t][j] = edge_composite(a, r, start, rp, i, x);
+      }
     }
   }
 }
 
-template <typename IdT, bool WITH_COO>
-__device__ __forceinline__ void emit_final(const WArgs<IdT>& a, int64_t r, int64_t start,
-                                           int64_t out_start, int lane, int j,
-                                           unsigned long long c) {
-  if (lane == (j & (kWave - 1)) && c != 0ull) {
-    const int64_t q = start + composite_pos(c);
-    a.sub_indices[out_start + j] = a.indices[q];
-    a.select_index[out_start + j] = q;
-    if (WITH_COO) a.coo_col[out_start + j] = static_cast<IdT>(r);
-  }
+__device__ __forceinline__ unsigned long long lane_value(unsigned long long v, int l) {
+  const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(v), l);
+  const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(v >> 32), l);
+  return (static_cast<unsigned long long>(hi) << 32) | lo;
 }
 
-// One wave per row.  deg <= k: copy; deg <= kChunk: select here; longer: queue.
+// The k largest of the wave's items, in descending order: emit(place, composite) is called
+// once per winner by the lane that holds it in the end; returns how many there were
+// (fewer than k when the wave holds fewer items).  `list` is the wave's k * 64 LDS words.
+// Every lane of the wave calls this.
+template <int TRIPS, typename Emit>
+__device__ __forceinline__ int wave_topk(const unsigned long long (&items)[TRIPS][4],
+                                         unsigned long long* list, int lane, int k, Emit emit) {
+  unsigned long long mx = 0ull;
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mx = items[t][j] > mx ? items[t][j] : mx;
+  // floor: the k-th largest of the lanes' maxima (composites are distinct; lanes without
+  // items hold 0 and never qualify).  At least k items reach it, so the winners do.
+  int greater = 0;
+#pragma unroll 8
+  for (int l = 0; l < kWave; ++l) greater += lane_value(mx, l) > mx ? 1 : 0;
+  const unsigned long long holder = __ballot(mx != 0ull && greater == k - 1);
+  const unsigned long long floor_c = holder ? lane_value(mx, __ffsll(holder) - 1) : 0ull;
+  // survivors, packed into LDS in (trip, item, lane) order
+  const unsigned long long lower = (1ull << lane) - 1ull;
+  int n = 0;
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool keep = items[t][j] != 0ull && items[t][j] >= floor_c;
+      const unsigned long long votes = __ballot(keep);
+      if (keep) list[n + __popcll(votes & lower)] = items[t][j];
+      n += __popcll(votes);
+    }
+  }
+  // the wave's own stores must have landed before other lanes read them back
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+  for (int i = lane; i < n; i += kWave) {
+    const unsigned long long mine = list[i];
+    int place = 0;
+    for (int x = 0; x < n; ++x) place += list[x] > mine ? 1 : 0;
+    if (place < k) emit(place, mine);
+  }
+  // the list is free again only when every lane has finished reading it
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+  return n < k ? n : k;
+}
+
+// pick number j of row r is the edge the composite names; called by one lane
+template <typename IdT, bool WITH_COO>
+__device__ __forceinline__ void emit_final(const WArgs<IdT>& a, int64_t r, int64_t start,
+                                           int64_t out_start, int j, unsigned long long c) {
+  const int64_t q = start + composite_pos(c);
+  a.sub_indices[out_start + j] = a.indices[q];
+  a.select_index[out_start + j] = q;
+  if (WITH_COO) a.coo_col[out_start + j] = static_cast<IdT>(r);
+}
+
+// One wave per row.  deg <= k: copy; deg <= 256: select here; longer: queue (rows up to
+// 2048 edges as one chunk that the chunk pass finishes by itself).
 template <typename IdT, bool WITH_COO>
 __global__ void weighted_rows_kernel(WArgs<IdT> a) {
   extern __shared__ unsigned long long s_lists[];
@@ -158,7 +220,7 @@ __global__ void weighted_rows_kernel(WArgs<IdT> a) {
     }
     return;
   }
-  bool here = deg <= kChunk;
+  bool here = deg <= kSmall;
   if (!here) {
     const int64_t nchunks = (deg + kChunk - 1) / kChunk;
     unsigned long long base = 0;
@@ -167,7 +229,7 @@ __global__ void weighted_rows_kernel(WArgs<IdT> a) {
     if (static_cast<int64_t>(base) + nchunks <= a.chunk_cap) {
       for (int64_t ch = lane; ch < nchunks; ch += kWave)
         a.chunk_queue[base + ch] = static_cast<long long>((r << 20) | ch);
-      if (lane == 0) {
+      if (lane == 0 && nchunks > 1) {
         const unsigned long long slot = atomicAdd(&a.counters[1], 1ull);
         a.long_rows[slot * 3 + 0] = r;
         a.long_rows[slot * 3 + 1] = static_cast<long long>(base);
@@ -181,17 +243,31 @@ __global__ void weighted_rows_kernel(WArgs<IdT> a) {
       here = true;
     }
   }
-  if (here) {
+  if (here && deg <= kSmall) {
+    unsigned long long items[1][4];
+    load_items<1>(a, r, start, 0, deg, lane, items);
+    wave_topk<1>(items, list, lane, a.k, [&](int j, unsigned long long c) {
+      emit_final<IdT, WITH_COO>(a, r, start, out_start, j, c);
+    });
+  } else if (here) {
+    // a row that found the queue full: this wave streams it whole
     int cnt = 0;
-    stream_edges(a, r, start, 0, deg, list, lane, cnt);
+    for (int64_t i = lane; i < deg; i += kWave) {
+      U4 x;
+      const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[r] : nullptr;
+      if (!rp) x = draw_block(a.seed, kTagWeighted, static_cast<uint64_t>(r), static_cast<uint64_t>(i >> 2));
+      lane_insert(list, lane, cnt, a.k, edge_composite(a, r, start, rp, i, x));
+    }
     wave_drain(list, lane, cnt, a.k, [&](int j, unsigned long long best) {
-      emit_final<IdT, WITH_COO>(a, r, start, out_start, lane, j, best);
+      if (lane == (j & (kWave - 1)) && best != 0ull)
+        emit_final<IdT, WITH_COO>(a, r, start, out_start, j, best);
     });
   }
 }
 
-// One wave per queued chunk: local top-k composites -> cand[slot * k + j].
-template <typename IdT>
+// One wave per queued chunk: local top-k composites -> cand[slot * k + j]; the only chunk
+// of a row is final and goes to the output.
+template <typename IdT, bool WITH_COO>
 __global__ void weighted_chunks_kernel(WArgs<IdT> a) {
   extern __shared__ unsigned long long s_lists[];
   const int lane = threadIdx.x & (kWave - 1);
@@ -213,12 +289,19 @@ __global__ void weighted_chunks_kernel(WArgs<IdT> a) {
     const int64_t deg = a.indptr[c + 1] - start;
     const int64_t lo = ch * kChunk;
     const int64_t hi = lo + kChunk < deg ? lo + kChunk : deg;
-    int cnt = 0;
-    stream_edges(a, r, start, lo, hi, list, lane, cnt);
+    unsigned long long items[kTrips][4];
+    load_items<kTrips>(a, r, start, lo, hi, lane, items);
+    if (deg <= kChunk) {
+      const int64_t out_start = a.sub_indptr[r];
+      wave_topk<kTrips>(items, list, lane, a.k, [&](int j, unsigned long long c) {
+        emit_final<IdT, WITH_COO>(a, r, start, out_start, j, c);
+      });
+      continue;
+    }
     unsigned long long* out = a.cand + static_cast<size_t>(t) * a.k;
-    wave_drain(list, lane, cnt, a.k, [&](int j, unsigned long long best) {
-      if (lane == (j & (kWave - 1))) out[j] = best;
-    });
+    const int found = wave_topk<kTrips>(items, list, lane, a.k,
+                                        [&](int j, unsigned long long c) { out[j] = c; });
+    for (int j = found + lane; j < a.k; j += kWave) out[j] = 0ull;  // fewer than k edges
   }
 }
 
@@ -240,13 +323,29 @@ __global__ void weighted_merge_kernel(WArgs<IdT> a) {
     const int64_t start = a.indptr[c];
     const int64_t out_start = a.sub_indptr[r];
     const unsigned long long* src = a.cand + static_cast<size_t>(base) * a.k;
+    if (m <= kChunk) {
+      // few enough candidates for the register-resident selection (0 = an empty slot)
+      unsigned long long items[kTrips][4];
+#pragma unroll
+      for (int tr = 0; tr < kTrips; ++tr)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int64_t i = (static_cast<int64_t>(tr) * 4 + j) * kWave + lane;
+          items[tr][j] = i < m ? src[i] : 0ull;
+        }
+      wave_topk<kTrips>(items, list, lane, a.k, [&](int j, unsigned long long cmp) {
+        emit_final<IdT, WITH_COO>(a, r, start, out_start, j, cmp);
+      });
+      continue;
+    }
     int cnt = 0;
     for (int64_t i = lane; i < m; i += kWave) {
       const unsigned long long cmp = src[i];
       if (cmp != 0ull) lane_insert(list, lane, cnt, a.k, cmp);
     }
     wave_drain(list, lane, cnt, a.k, [&](int j, unsigned long long best) {
-      emit_final<IdT, WITH_COO>(a, r, start, out_start, lane, j, best);
+      if (lane == (j & (kWave - 1)) && best != 0ull)
+        emit_final<IdT, WITH_COO>(a, r, start, out_start, j, best);
     });
   }
 }
@@ -270,7 +369,7 @@ int weighted_launch(const WArgs<IdT>& a, hipStream_t st) {
   hipLaunchKernelGGL(zero2_kernel, dim3(1), dim3(64), 0, st, a.counters);
   hipLaunchKernelGGL((weighted_rows_kernel<IdT, WITH_COO>),
                      dim3(static_cast<unsigned>((a.S + waves - 1) / waves)), block, lds, st, a);
-  hipLaunchKernelGGL((weighted_chunks_kernel<IdT>), dim3(kQueueGrid), block, lds, st, a);
+  hipLaunchKernelGGL((weighted_chunks_kernel<IdT, WITH_COO>), dim3(kQueueGrid), block, lds, st, a);
   hipLaunchKernelGGL((weighted_merge_kernel<IdT, WITH_COO>), dim3(kQueueGrid), block, lds, st, a);
   return check_launch("sample_weighted");
 }
