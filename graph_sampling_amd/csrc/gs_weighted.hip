@@ -411,12 +411,59 @@ int weighted_impl(const int64_t* indptr, int64_t num_cols, const void* indices, 
 
 // ------------------------------------------------ with replacement (inverse CDF) ----
 // Replaces _CSRRowWiseSampleReplaceKernel (reference src/cuda/sampling_probs.cu:112-183).
-// One wave per column: the prefix sums of max(prob, 0) are built 64 edges at a time with a
+// The prefix sums of max(prob, 0) over a column are built 64 edges at a time with a
 // Kogge-Stone scan over the wave (x[i] += x[i-d], d = 1..32; the running total enters the
 // next chunk through its first element, as in the reference's WarpScan loop :147-160) and
-// kept in the caller's scratch; then every lane draws picks and searches them.  The order
-// of the float additions is fixed by that scheme, so a host evaluation of the same steps
-// gives the same bits.
+// kept in the caller's scratch; then every lane draws picks and searches them.  That chain
+// is sequential, so a column is cut into blocks of 2048 edges: each block is scanned from
+// zero by a wave of its own, the blocks' totals are added up in order, and entry i of block
+// b stands for (sum of the totals before b) + (its value inside the block).  Columns up to
+// 2048 edges are one block and one wave; a hub of 300 k edges is 146 waves instead of one
+// wave walking 4640 chunks.  The order of the float additions is fixed by that scheme, so a
+// host evaluation of the same steps gives the same bits.
+constexpr int64_t kCdfBlock = 2048;
+constexpr int kMaxBases = 2048;  // block sums of a column kept in LDS: columns up to 4 M edges
+
+// prefix sums of max(prob, 0) over edges [lo, hi) of a column, from zero; returns their total
+__device__ __forceinline__ float scan_block(const float* __restrict__ prob, int64_t lo, int64_t hi,
+                                            float* __restrict__ out, int lane) {
+  float carry = 0.0f;
+  for (int64_t base = lo; base < hi; base += kWave) {
+    float x = base + lane < hi ? prob[base + lane] : 0.0f;
+    if (lane == 0) x += carry;
+    x = x > 0.0f ? x : 0.0f;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const float y = __shfl_up(x, d, kWave);
+      if (lane >= d) x += y;
+    }
+    carry = __shfl(x, kWave - 1, kWave);
+    if (base + lane < hi) out[base + lane] = x;
+  }
+  return carry;
+}
+
+// pick number j of row r: position `at` of the column that starts at `start`
+template <typename IdT, bool WITH_COO>
+__device__ __forceinline__ void emit_pick(const IdT* __restrict__ indices, int64_t start, int64_t at,
+                                          int64_t r, int64_t slot, IdT* __restrict__ sub_indices,
+                                          int64_t* __restrict__ select_index,
+                                          IdT* __restrict__ coo_col) {
+  sub_indices[slot] = indices[start + at];
+  select_index[slot] = start + at;
+  if (WITH_COO) coo_col[slot] = static_cast<IdT>(r);
+}
+
+__device__ __forceinline__ float pick_point(uint64_t seed, const uint32_t* __restrict__ replay,
+                                            int64_t r, int64_t k, int64_t j, float total) {
+  const uint32_t xd = replay ? replay[r * k + j]
+                             : draw_one(seed, kTagWeighted, static_cast<uint64_t>(r),
+                                        static_cast<uint64_t>(j));
+  const float u = static_cast<float>((xd >> 8) + 1u) * 5.9604644775390625e-08f;
+  return u * total;
+}
+
+// One wave per column of at most 2048 edges: scan, then picks.
 template <typename IdT, bool WITH_COO>
 __global__ void __launch_bounds__(256)
 weighted_replace_kernel(const int64_t* __restrict__ indptr, int64_t num_cols,
@@ -433,41 +480,174 @@ weighted_replace_kernel(const int64_t* __restrict__ indptr, int64_t num_cols,
   if (c < 0 || c >= num_cols) return;
   const int64_t start = indptr[c];
   const int64_t deg = indptr[c + 1] - start;
-  if (deg <= 0) return;
+  if (deg <= 0 || deg > kCdfBlock) return;  // longer columns: the two kernels below
   float* my_cdf = cdf + cdf_ptr[r];
-  float carry = 0.0f;
-  for (int64_t base = 0; base < deg; base += kWave) {
-    float x = base + lane < deg ? probs[start + base + lane] : 0.0f;
-    if (lane == 0) x += carry;
-    x = x > 0.0f ? x : 0.0f;
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const float y = __shfl_up(x, d, kWave);
-      if (lane >= d) x += y;
-    }
-    carry = __shfl(x, kWave - 1, kWave);
-    if (base + lane < deg) my_cdf[base + lane] = x;
-  }
+  const float total = scan_block(probs + start, 0, deg, my_cdf, lane);
   // the wave's own stores must have landed before other lanes read them back
   __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
-  const float total = carry;
   const int64_t out_start = sub_indptr[r];
   for (int64_t j = lane; j < k; j += kWave) {
-    const uint32_t xd = replay ? replay[r * k + j]
-                               : draw_one(seed, kTagWeighted, static_cast<uint64_t>(r),
-                                          static_cast<uint64_t>(j));
-    const float u = static_cast<float>((xd >> 8) + 1u) * 5.9604644775390625e-08f;
-    const float rnd = u * total;
-    int64_t lo = 0, hi = deg;
+    const float rnd = pick_point(seed, replay, r, k, j, total);
+    // first the block (here the only one) whose last entry exceeds rnd, then inside it: the
+    // same steps as for the longer columns.  Prefix sums made by different addition trees
+    // need not be monotone to the last bit, so the order of the probes is part of the result.
+    int64_t lo = deg, hi = deg;
+    if (total > rnd) lo = 0;
     while (lo < hi) {
       const int64_t mid = (lo + hi) >> 1;
       if (my_cdf[mid] <= rnd) lo = mid + 1; else hi = mid;
     }
     if (lo > deg - 1) lo = deg - 1;
-    sub_indices[out_start + j] = indices[start + lo];
-    select_index[out_start + j] = start + lo;
-    if (WITH_COO) coo_col[out_start + j] = static_cast<IdT>(r);
+    emit_pick<IdT, WITH_COO>(indices, start, lo, r, out_start + j, sub_indices, select_index, coo_col);
   }
+}
+
+// Blocks of the longer columns.  The scratch `cdf` is the columns' edges one after the
+// other (cdf_ptr), so the work is found without a queue: a wave takes 2048 consecutive
+// scratch positions, and at most two columns longer than that can touch them -- the one
+// that holds the first position and the one that holds the last.  Of each, at most one
+// block STARTS inside the wave's positions; that block is the wave's.
+template <typename IdT>
+__global__ void __launch_bounds__(256)
+replace_blocks_kernel(const int64_t* __restrict__ indptr, const float* __restrict__ probs,
+                      const IdT* __restrict__ cols, int64_t S, const int64_t* __restrict__ cdf_ptr,
+                      float* __restrict__ cdf) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t waves = static_cast<int64_t>(gridDim.x) * (blockDim.x / kWave);
+  const int64_t D = cdf_ptr[S];
+  for (int64_t g = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+       g * kCdfBlock < D; g += waves) {
+    const int64_t t0 = g * kCdfBlock;
+    const int64_t t1 = t0 + kCdfBlock < D ? t0 + kCdfBlock : D;
+    int64_t owner[2];
+#pragma unroll
+    for (int side = 0; side < 2; ++side) {
+      const int64_t at = side == 0 ? t0 : t1 - 1;
+      int64_t lo = 0, hi = S + 1;  // first r with cdf_ptr[r] > at
+      while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (cdf_ptr[mid] <= at) lo = mid + 1; else hi = mid;
+      }
+      owner[side] = lo - 1;
+    }
+#pragma unroll
+    for (int side = 0; side < 2; ++side) {
+      const int64_t r = owner[side];
+      if (side == 1 && r == owner[0]) break;
+      if (r < 0 || r >= S) continue;
+      const int64_t region = cdf_ptr[r];
+      const int64_t deg = cdf_ptr[r + 1] - region;
+      if (deg <= kCdfBlock) continue;
+      const int64_t from = (t0 > region ? t0 : region) - region;
+      const int64_t p = (from + kCdfBlock - 1) / kCdfBlock * kCdfBlock;  // block start in the column
+      if (region + p >= t1 || p >= deg) continue;
+      const int64_t c = cols ? static_cast<int64_t>(cols[r]) : r;
+      scan_block(probs + indptr[c], p, p + kCdfBlock < deg ? p + kCdfBlock : deg, cdf + region, lane);
+    }
+  }
+}
+
+// One wave per column longer than 2048 edges, after its blocks have been scanned: the
+// blocks' totals are added up in order (LDS), then the picks search first the block, then
+// inside it, comparing (sum before the block) + (value inside the block).
+template <typename IdT, bool WITH_COO>
+__global__ void __launch_bounds__(256)
+replace_long_kernel(const int64_t* __restrict__ indptr, int64_t num_cols,
+                    const IdT* __restrict__ indices, const IdT* __restrict__ cols, int64_t S,
+                    int64_t k, uint64_t seed, const uint32_t* __restrict__ replay,
+                    const int64_t* __restrict__ sub_indptr, const int64_t* __restrict__ cdf_ptr,
+                    const float* __restrict__ cdf, IdT* __restrict__ sub_indices,
+                    int64_t* __restrict__ select_index, IdT* __restrict__ coo_col) {
+  __shared__ float s_base[256 / kWave][kMaxBases + 1];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + wave;
+  if (r >= S) return;
+  const int64_t c = cols ? static_cast<int64_t>(cols[r]) : r;
+  if (c < 0 || c >= num_cols) return;
+  const int64_t start = indptr[c];
+  const int64_t deg = indptr[c + 1] - start;
+  if (deg <= kCdfBlock) return;
+  const float* my_cdf = cdf + cdf_ptr[r];
+  const int64_t nblocks = (deg + kCdfBlock - 1) / kCdfBlock;
+  const bool staged = nblocks <= kMaxBases;
+  float* base = s_base[wave];  // base[b] = sum of the totals of blocks 0 .. b-1
+  float total = 0.0f;
+  if (staged) {
+    for (int64_t b = lane; b < nblocks; b += kWave) {
+      const int64_t end = (b + 1) * kCdfBlock < deg ? (b + 1) * kCdfBlock : deg;
+      base[b + 1] = my_cdf[end - 1];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+    if (lane == 0) {
+      float acc = 0.0f;
+      base[0] = 0.0f;
+      for (int64_t b = 0; b < nblocks; ++b) {
+        acc = acc + base[b + 1];
+        base[b + 1] = acc;
+      }
+      total = acc;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+  } else if (lane == 0) {
+    for (int64_t b = 0; b < nblocks; ++b) {
+      const int64_t end = (b + 1) * kCdfBlock < deg ? (b + 1) * kCdfBlock : deg;
+      total = total + my_cdf[end - 1];
+    }
+  }
+  total = __shfl(total, 0, kWave);
+  const int64_t out_start = sub_indptr[r];
+  for (int64_t j = lane; j < k; j += kWave) {
+    const float rnd = pick_point(seed, replay, r, k, j, total);
+    // first block whose last entry exceeds rnd, and the sum before it
+    int64_t b = 0;
+    float before = 0.0f;
+    if (staged) {
+      int64_t lo = 0, hi = nblocks;
+      while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (base[mid + 1] <= rnd) lo = mid + 1; else hi = mid;
+      }
+      b = lo;
+      before = b < nblocks ? base[b] : 0.0f;
+    } else {
+      for (; b < nblocks; ++b) {
+        const int64_t end = (b + 1) * kCdfBlock < deg ? (b + 1) * kCdfBlock : deg;
+        const float next = before + my_cdf[end - 1];
+        if (next > rnd) break;
+        before = next;
+      }
+    }
+    int64_t at = deg - 1;
+    if (b < nblocks) {
+      int64_t lo = b * kCdfBlock;
+      int64_t hi = lo + kCdfBlock < deg ? lo + kCdfBlock : deg;
+      while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (before + my_cdf[mid] <= rnd) lo = mid + 1; else hi = mid;
+      }
+      at = lo > deg - 1 ? deg - 1 : lo;
+    }
+    emit_pick<IdT, WITH_COO>(indices, start, at, r, out_start + j, sub_indices, select_index, coo_col);
+  }
+}
+
+template <typename IdT, bool WITH_COO>
+int weighted_replace_launch(const int64_t* indptr, int64_t num_cols, const IdT* indices,
+                            const float* probs, const IdT* cols, int64_t S, int64_t k, uint64_t seed,
+                            const uint32_t* replay, const int64_t* sub_indptr, const int64_t* cdf_ptr,
+                            float* cdf, IdT* sub_indices, int64_t* select_index, IdT* coo_col,
+                            hipStream_t st) {
+  const dim3 grid(static_cast<unsigned>((S + 3) / 4)), block(4 * kWave);
+  hipLaunchKernelGGL((weighted_replace_kernel<IdT, WITH_COO>), grid, block, 0, st, indptr, num_cols,
+                     indices, probs, cols, S, k, seed, replay, sub_indptr, cdf_ptr, cdf, sub_indices,
+                     select_index, coo_col);
+  hipLaunchKernelGGL((replace_blocks_kernel<IdT>), dim3(512), block, 0, st, indptr, probs, cols, S,
+                     cdf_ptr, cdf);
+  hipLaunchKernelGGL((replace_long_kernel<IdT, WITH_COO>), grid, block, 0, st, indptr, num_cols,
+                     indices, cols, S, k, seed, replay, sub_indptr, cdf_ptr, cdf, sub_indices,
+                     select_index, coo_col);
+  return check_launch("sample_weighted_replace");
 }
 
 template <typename IdT>
@@ -476,18 +656,16 @@ int weighted_replace_impl(const int64_t* indptr, int64_t num_cols, const void* i
                           const uint32_t* replay, const int64_t* sub_indptr, const int64_t* cdf_ptr,
                           float* cdf, void* sub_indices, int64_t* select_index, void* coo_col,
                           hipStream_t st) {
-  const dim3 grid(static_cast<unsigned>((S + 3) / 4)), block(4 * kWave);
-  if (coo_col)
-    hipLaunchKernelGGL((weighted_replace_kernel<IdT, true>), grid, block, 0, st, indptr, num_cols,
-                       static_cast<const IdT*>(indices), probs, static_cast<const IdT*>(cols), S, k,
-                       seed, replay, sub_indptr, cdf_ptr, cdf, static_cast<IdT*>(sub_indices),
-                       select_index, static_cast<IdT*>(coo_col));
-  else
-    hipLaunchKernelGGL((weighted_replace_kernel<IdT, false>), grid, block, 0, st, indptr, num_cols,
-                       static_cast<const IdT*>(indices), probs, static_cast<const IdT*>(cols), S, k,
-                       seed, replay, sub_indptr, cdf_ptr, cdf, static_cast<IdT*>(sub_indices),
-                       select_index, static_cast<IdT*>(coo_col));
-  return check_launch("sample_weighted_replace");
+  const IdT* ind = static_cast<const IdT*>(indices);
+  const IdT* cl = static_cast<const IdT*>(cols);
+  IdT* si = static_cast<IdT*>(sub_indices);
+  IdT* cc = static_cast<IdT*>(coo_col);
+  return coo_col ? weighted_replace_launch<IdT, true>(indptr, num_cols, ind, probs, cl, S, k, seed,
+                                                     replay, sub_indptr, cdf_ptr, cdf, si,
+                                                     select_index, cc, st)
+                 : weighted_replace_launch<IdT, false>(indptr, num_cols, ind, probs, cl, S, k, seed,
+                                                      replay, sub_indptr, cdf_ptr, cdf, si,
+                                                      select_index, cc, st);
 }
 
 }  // namespace

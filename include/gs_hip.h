@@ -229,9 +229,13 @@ int gs_sample_weighted_fill(const int64_t* indptr, int64_t num_cols, const void*
  * _CSRRowWiseSampleReplaceKernel (src/cuda/sampling_probs.cu:112-183).  A column with
  * deg > 0 gets fanout picks.  cdf = inclusive prefix of max(probs, 0) over the column's
  * edges, built 64 edges at a time by a Kogge-Stone scan (x[i] += x[i-d], d = 1, 2, .., 32)
- * whose running total enters the next chunk through its first element.  Pick j of row r:
- * u = ((draw(r, j) >> 8) + 1) * 2^-24, rand = u * cdf[deg-1], item = first position with
- * cdf > rand, clamped to deg-1.  sub_indptr comes from gs_sample_count(replace = 1).
+ * whose running total enters the next chunk through its first element.  A column longer
+ * than 2048 edges is cut into blocks of 2048: every block is scanned from zero, the blocks'
+ * totals are added up in order, and entry i of block b is (sum of the totals before b) +
+ * (its value inside the block).  Pick j of row r: u = ((draw(r, j) >> 8) + 1) * 2^-24,
+ * rand = u * cdf[deg-1], item = first position with cdf > rand (binary search for the
+ * block whose last entry exceeds rand, then inside it), clamped to deg-1.  sub_indptr
+ * comes from gs_sample_count(replace = 1).
  * cdf_ptr[S+1]: offsets of the columns' edges inside the scratch `cdf` (cdf_ptr[S] floats):
  * indptr itself when column_ids == NULL, else the sub_indptr of gs_slice_count.
  * replay: S * fanout draws, [r * fanout + j]. */

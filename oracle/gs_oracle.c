@@ -381,6 +381,11 @@ void gso_sample_weighted_fill(const i64* indptr, i64 num_cols, const i64* indice
 /* element of the next chunk (:147-160); restated here with 64-wide chunks    */
 /* and the scan written out as its Kogge-Stone steps (x[i] += x[i-d] for      */
 /* d = 1, 2, .., 32), so that the float additions happen in one fixed order.  */
+/* That chain is sequential along the column; so that a hub column is not one  */
+/* chain of thousands of steps, a column is cut into blocks of 2048 edges:     */
+/* every block is scanned from zero, the blocks' totals are added up in order, */
+/* and entry i of block b is (sum of the totals before b) + (its value inside  */
+/* the block).  Columns up to 2048 edges are one block: nothing changes there. */
 /* Pick j of row r: u = ((draw >> 8) + 1) * 2^-24 in (0, 1], rand = u * total,*/
 /* item = first position with cdf > rand, clamped to deg-1 (:164-171).        */
 /* Replay: replay[r * k + j].  The concrete picks are parity unpinned         */
@@ -404,6 +409,18 @@ static void cdf_chunks64(const float* prob, i64 deg, float* cdf) {
   }
 }
 
+static void cdf_column(const float* prob, i64 deg, float* cdf) {
+  float before = 0.0f;
+  for (i64 lo = 0; lo < deg; lo += 2048) {
+    i64 len = deg - lo < 2048 ? deg - lo : 2048;
+    cdf_chunks64(prob + lo, len, cdf + lo);
+    float block_total = cdf[lo + len - 1];
+    if (lo > 0)
+      for (i64 i = 0; i < len; ++i) cdf[lo + i] = before + cdf[lo + i];
+    before = before + block_total;
+  }
+}
+
 void gso_sample_weighted_replace(const i64* indptr, i64 num_cols, const i64* indices,
                                  const float* probs, const i64* cols, i64 S, i64 k, u64 seed,
                                  const u32* replay, const i64* sub_indptr, i64* sub_indices,
@@ -417,16 +434,32 @@ void gso_sample_weighted_replace(const i64* indptr, i64 num_cols, const i64* ind
     if (deg <= 0) continue;
     i64 out_start = sub_indptr[r];
     float* cdf = (float*)malloc(sizeof(float) * (size_t)deg);
-    cdf_chunks64(probs + in_start, deg, cdf);
+    cdf_column(probs + in_start, deg, cdf);
     const float total = cdf[deg - 1];
     for (i64 j = 0; j < k; ++j) {
       u32 x = replay ? replay[r * k + j] : gso_draw(seed, GSO_TAG_WEIGHTED, (u64)r, (u64)j);
       float u = (float)((x >> 8) + 1u) * 5.9604644775390625e-08f; /* 2^-24, exact */
       float rnd = u * total;
-      i64 lo = 0, hi = deg; /* first position with cdf > rnd */
+      /* first position with cdf > rnd: first the block whose last entry exceeds rnd,
+       * then inside it.  Prefix sums made by different addition trees need not be
+       * monotone to the last bit, so the probe sequence is part of the definition. */
+      i64 nblocks = (deg + 2047) / 2048;
+      i64 lo = 0, hi = nblocks;
       while (lo < hi) {
         i64 mid = (lo + hi) >> 1;
-        if (cdf[mid] <= rnd) lo = mid + 1; else hi = mid;
+        i64 end = (mid + 1) * 2048 < deg ? (mid + 1) * 2048 : deg;
+        if (cdf[end - 1] <= rnd) lo = mid + 1; else hi = mid;
+      }
+      if (lo < nblocks) {
+        i64 b = lo;
+        lo = b * 2048;
+        hi = lo + 2048 < deg ? lo + 2048 : deg;
+        while (lo < hi) {
+          i64 mid = (lo + hi) >> 1;
+          if (cdf[mid] <= rnd) lo = mid + 1; else hi = mid;
+        }
+      } else {
+        lo = deg;
       }
       if (lo > deg - 1) lo = deg - 1;
       sub_indices[out_start + j] = indices[in_start + lo];

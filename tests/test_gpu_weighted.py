@@ -229,6 +229,33 @@ def test_weighted_replace_hub_column_and_frequencies(dev):
     assert counts.min() > 0.8 * k * p / 10 and counts.max() < 1.2 * k * p / 10
 
 
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+def test_weighted_replace_long_columns_block_by_block(dev, idt):
+    # columns of several 2048-edge blocks between short ones, real-valued weights: the
+    # blocks are scanned by separate waves and their sums added up in order, and every
+    # pick must be the oracle's (same additions, same bits); lengths around the block size
+    degs = [5, 2048, 0, 2049, 40000, 3, 4096, 4097, 1, 10000, 0, 70]
+    indptr = np.concatenate([[0], np.cumsum(degs)]).astype(np.int64)
+    rng = np.random.default_rng(8)
+    indices = rng.integers(0, 1000, size=int(indptr[-1])).astype(np.int64)
+    probs = rng.random(indices.size).astype(np.float32)
+    probs[rng.random(indices.size) < 0.05] = -0.5
+    k = 300
+    for cols in (None, np.array([4, 9, 1, 4, 11, 3, 7, 2], dtype=np.int64)):
+        S = len(degs) if cols is None else cols.size
+        replay = u32_draws(S * k, seed=12)
+        t_cols = None if cols is None else to_dev(cols, dev, idt)
+        got = capi.sample_weighted_replace(to_dev(indptr, dev), to_dev(indices, dev, idt),
+                                           to_dev(probs, dev), t_cols, k,
+                                           replay=to_dev(replay, dev), with_coo=True)
+        want = O.sample_weighted_replace(indptr, indices, probs, cols, k, replay=replay)
+        nnz = int(want[0][-1])
+        assert np.array_equal(got[0].cpu().numpy(), want[0])
+        assert np.array_equal(got[2][:nnz].cpu().numpy(), want[3])
+        assert np.array_equal(got[1][:nnz].cpu().numpy().astype(np.int64), want[2])
+        assert np.array_equal(got[3][:nnz].cpu().numpy().astype(np.int64), want[1])
+
+
 def test_graph_sampling_with_probs_replace(dev):
     import graph_sampling_amd as gs
     n = 1 << 10

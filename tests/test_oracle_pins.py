@@ -212,6 +212,19 @@ def test_weighted_replace_closed_form_and_special_cases():
     one = np.zeros(deg, dtype=np.float32)
     one[42] = 2.5
     assert (O.sample_weighted_replace(indptr, indices, one, None, 50, seed=1)[3] == 42).all()
+    # a column of several 2048-edge blocks (their sums are added up block by block): with
+    # integer weights the order of additions cannot matter, so plain cumsum + searchsorted
+    # must give the same picks
+    big = 2048 * 3 + 700
+    bptr = np.array([0, big], dtype=np.int64)
+    bind = np.arange(big, dtype=np.int64)
+    bw = rng.integers(0, 4, size=big).astype(np.float32)
+    bdraws = u32_draws(5000, seed=10)
+    bsel = O.sample_weighted_replace(bptr, bind, bw, None, 5000, replay=bdraws)[3]
+    bcdf = np.cumsum(bw, dtype=np.float64).astype(np.float32)     # exact: integers below 2^24
+    bu = ((bdraws >> 8).astype(np.float32) + np.float32(1)) * np.float32(2.0 ** -24)
+    assert np.array_equal(bsel, np.minimum(np.searchsorted(bcdf, bu * bcdf[-1], side="right"),
+                                           big - 1))
     # the Philox draw of pick j of row r is draw(seed, tag 2, r, j)
     _, _, _, a = O.sample_weighted_replace(indptr, indices, w, None, 8, seed=77)
     d = np.array([O.draw(77, 2, 1, j) for j in range(8)], dtype=np.uint32)
