@@ -98,13 +98,23 @@ short_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restr
     for (int64_t c = c0 + 1; c <= c1; ++c) ck.incoming[c] = static_cast<int>(s);
     return;
   }
+  // at most kLaneMaxLen edges: a fixed number of predicated reads, all in flight together,
+  // added up in edge order
+  float v[kLaneMaxLen];
+  int64_t at[kLaneMaxLen];
+#pragma unroll
+  for (int k = 0; k < kLaneMaxLen; ++k) {
+    at[k] = begin + k < end ? (emap ? emap[begin + k] : begin + k) : -1;
+    v[k] = at[k] >= 0 ? data[at[k]] : 0.0f;
+  }
   float acc = 0.0f;
-  for (int64_t e = begin; e < end; ++e) acc += powk_f(data[emap ? emap[e] : e], powk);
+#pragma unroll
+  for (int k = 0; k < kLaneMaxLen; ++k)
+    if (at[k] >= 0) acc += powk_f(v[k], powk);
   if (NORMALIZE) {
-    for (int64_t e = begin; e < end; ++e) {
-      const int64_t d = emap ? emap[e] : e;
-      out[d] = data[d] / acc;
-    }
+#pragma unroll
+    for (int k = 0; k < kLaneMaxLen; ++k)
+      if (at[k] >= 0) out[at[k]] = v[k] / acc;
   } else {
     out[nmap ? static_cast<int64_t>(nmap[s]) : s] = acc;
   }
@@ -176,16 +186,46 @@ __device__ __forceinline__ LaneMarks scan_lane_marks(const int (&m)[kLaneEdges],
   return lm;
 }
 
+// Value of the lane `CTRL` names (a data-parallel-primitive move inside the vector ALU, no
+// trip through the LDS crossbar); lanes without a source, or outside ROWS, get `fill`.
+// 0x111/0x112/0x114/0x118: the lane 1/2/4/8 below in the same row of 16; 0x142: lane 15 of
+// the row below (rows 1 and 3 with ROWS = 0xa); 0x143: lane 31 (rows 2 and 3 with 0xc).
+template <int CTRL, int ROWS>
+__device__ __forceinline__ int lane_move(int fill, int v) {
+  return __builtin_amdgcn_update_dpp(fill, v, CTRL, ROWS, 0xf, false);
+}
+
 // latest mark at or before the end of each lane (inclusive) given the lanes' own last marks;
-// positions grow with the lane, so a maximum is "the latest"
-__device__ __forceinline__ int latest_inclusive(int last_packed, int carried, int lane) {
-  int packed = last_packed;
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const int y = __shfl_up(packed, d, kWave);
-    if (lane >= d && y > packed) packed = y;
+// positions grow with the lane, so a maximum is "the latest".  Marks are >= 0.
+__device__ __forceinline__ int latest_inclusive(int last_packed, int carried, int) {
+  int p = last_packed;
+  int y;
+  y = lane_move<0x111, 0xf>(0, p); p = y > p ? y : p;
+  y = lane_move<0x112, 0xf>(0, p); p = y > p ? y : p;
+  y = lane_move<0x114, 0xf>(0, p); p = y > p ? y : p;
+  y = lane_move<0x118, 0xf>(0, p); p = y > p ? y : p;
+  y = lane_move<0x142, 0xa>(0, p); p = y > p ? y : p;
+  y = lane_move<0x143, 0xc>(0, p); p = y > p ? y : p;
+  return p > carried ? p : carried;
+}
+
+// inclusive sums of x over the lanes below that share the lane's key; keys do not decrease
+// with the lane and are >= 0
+__device__ __forceinline__ float keyed_inclusive_sum(float x, int key) {
+#define GS_KEYED_STEP(CTRL, ROWS)                                                       \
+  {                                                                                     \
+    const int ky = lane_move<CTRL, ROWS>(-1, key);                                      \
+    const float y = __builtin_bit_cast(float, lane_move<CTRL, ROWS>(0, __builtin_bit_cast(int, x))); \
+    if (ky == key) x += y;                                                              \
   }
-  return packed > carried ? packed : carried;
+  GS_KEYED_STEP(0x111, 0xf)
+  GS_KEYED_STEP(0x112, 0xf)
+  GS_KEYED_STEP(0x114, 0xf)
+  GS_KEYED_STEP(0x118, 0xf)
+  GS_KEYED_STEP(0x142, 0xa)
+  GS_KEYED_STEP(0x143, 0xc)
+#undef GS_KEYED_STEP
+  return x;
 }
 
 __device__ __forceinline__ int owner_of_mark(int packed) { return (packed & 0xFF) - 2; }
@@ -206,16 +246,50 @@ long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restri
   const int64_t end = begin + kChunk < nnz ? begin + kChunk : nnz;
   int* mark = s_mark[threadIdx.x / kWave];
   const Owned own = load_owned(indptr, ck, c, lane);
+  // The whole chunk lies inside the incoming segment (most chunks of a hub column do): one
+  // sum, no marks, no scans.
+  if (__shfl(own.g >= 0 ? own.e : int64_t(0), kIncomingLane, kWave) >= end) {
+    float acc = 0.0f;
+    if (!emap && end - begin == kChunk && (reinterpret_cast<uintptr_t>(data) & 15u) == 0) {
+#pragma unroll
+      for (int t = 0; t < kChunk / kStep; ++t) {
+        const float4 v = *reinterpret_cast<const float4*>(data + begin + t * kStep + lane * kLaneEdges);
+        acc += (powk_f(v.x, powk) + powk_f(v.y, powk)) + (powk_f(v.z, powk) + powk_f(v.w, powk));
+      }
+    } else {
+      for (int64_t e = begin + lane; e < end; e += kWave)
+        acc += powk_f(data[emap ? emap[e] : e], powk);
+    }
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) acc += __shfl_xor(acc, d, kWave);
+    if (lane == 0) {
+      ck.carry[2 * c] = acc;
+      ck.outgoing[c] = -1;
+    }
+    return;
+  }
   // An incoming segment of which fewer than four edges are left would start and stop inside
   // the first lane, the one case of a run that does not reach beyond a lane: it gets no marks
   // and lane 0 adds it up by itself.
   const int64_t in_left = __shfl(own.g >= 0 ? own.e - begin : int64_t(0), kIncomingLane, kWave);
   const int tiny = in_left < kLaneEdges ? static_cast<int>(in_left) : 0;
+  // a full chunk of plain data: all four steps' reads are issued before the marks are made,
+  // so that the scans below do not wait for memory step by step
+  const bool ahead = !emap && end - begin == kChunk && (reinterpret_cast<uintptr_t>(data) & 15u) == 0;
+  float4 early[kChunk / kStep];
+  if (ahead) {
+#pragma unroll
+    for (int t = 0; t < kChunk / kStep; ++t)
+      early[t] = *reinterpret_cast<const float4*>(data + begin + t * kStep + lane * kLaneEdges);
+  }
   write_marks(mark, own, begin, end, lane, tiny > 0 && lane == kIncomingLane);
   int carried = 0;       // latest mark at the end of the step before
   bool open = false;     // that mark's segment is a long one: its run goes on
   float acc_open = 0.0f;
-  for (int64_t base = begin; base < end; base += kStep) {
+#pragma unroll
+  for (int t = 0; t < kChunk / kStep; ++t) {
+    const int64_t base = begin + t * kStep;
+    if (base >= end) break;
     const int at0 = static_cast<int>(base - begin) + lane * kLaneEdges;
     const int64_t e0 = base + lane * kLaneEdges;
     int m[kLaneEdges];
@@ -224,11 +298,18 @@ long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restri
       const int4 mm = *reinterpret_cast<const int4*>(mark + at0);
       m[0] = mm.x; m[1] = mm.y; m[2] = mm.z; m[3] = mm.w;
     }
+    if (ahead) {
+      v[0] = powk_f(early[t].x, powk);
+      v[1] = powk_f(early[t].y, powk);
+      v[2] = powk_f(early[t].z, powk);
+      v[3] = powk_f(early[t].w, powk);
+    } else {
 #pragma unroll
-    for (int k = 0; k < kLaneEdges; ++k) {
-      const int64_t e = e0 + k;
-      if (e >= end) m[k] = 0;
-      v[k] = e < end ? powk_f(data[emap ? emap[e] : e], powk) : 0.0f;
+      for (int k = 0; k < kLaneEdges; ++k) {
+        const int64_t e = e0 + k;
+        if (e >= end) m[k] = 0;
+        v[k] = e < end ? powk_f(data[emap ? emap[e] : e], powk) : 0.0f;
+      }
     }
     if (tiny > 0 && base == begin && lane == 0) {
       float piece = 0.0f;
@@ -246,19 +327,15 @@ long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restri
       if (has_mark && k >= lm.last_k) post += v[k];
     }
     const int incl = latest_inclusive(lm.last_packed, carried, lane);
-    int in_packed = __shfl_up(incl, 1, kWave);  // the mark in force where the lane begins
-    if (lane == 0) in_packed = carried;
+    // the mark in force where the lane begins: the lane below's (0x138: the whole wave
+    // moved up by one lane), the step before's for lane 0
+    const int in_packed = lane_move<0x138, 0xf>(carried, incl);
     const int in_owner = owner_of_mark(in_packed);
     // one value per lane: the start of a run where the lane holds a mark, else its four edges
     float x = has_mark ? (owner_of_mark(incl) >= 0 ? post : 0.0f) : (in_owner >= 0 ? pre : 0.0f);
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const float y = __shfl_up(x, d, kWave);
-      const int iy = __shfl_up(incl, d, kWave);
-      if (lane >= d && iy == incl) x += y;
-    }
-    float x_prev = __shfl_up(x, 1, kWave);  // the incoming run's sum over the lanes before
-    if (lane == 0) x_prev = 0.0f;
+    x = keyed_inclusive_sum(x, incl);
+    // the incoming run's sum over the lanes before
+    const float x_prev = __builtin_bit_cast(float, lane_move<0x138, 0xf>(0, __builtin_bit_cast(int, x)));
     const int src = in_owner >= 0 ? in_owner : 0;
     const int64_t in_b = __shfl(own.b, src, kWave);
     const int in_g = __shfl(own.g, src, kWave);
@@ -270,8 +347,9 @@ long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restri
       else
         ck.carry[2 * c] = total;
     }
-    const int last = __shfl(incl, kWave - 1, kWave);
-    const float x_last = __shfl(x, kWave - 1, kWave);
+    const int last = __builtin_amdgcn_readlane(incl, kWave - 1);
+    const float x_last =
+        __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), kWave - 1));
     const bool goes_on = owner_of_mark(last) >= 0;
     acc_open = goes_on ? x_last + (open && last == carried ? acc_open : 0.0f) : 0.0f;
     open = goes_on;
@@ -299,22 +377,43 @@ long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restri
   if (lane == 0) ck.outgoing[c] = out_g;
 }
 
-// one lane per chunk: a chunk that holds the head of a long segment going on after it adds
-// up the pieces, in chunk order
+constexpr int64_t kCarryAlone = 16;  // pieces a single lane adds up by itself
+
+// One lane per chunk: a chunk that holds the head of a long segment going on after it adds
+// up the pieces, in chunk order.  A segment that goes on over more than 16 chunks (a hub
+// column: hundreds) is added up by the whole wave instead of one lane walking the pieces.
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 carry_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ nmap, int64_t num_seg,
              int64_t nnz, float* __restrict__ sums, Chunks ck) {
   if (*ck.any_long == 0u) return;
   if (indptr[num_seg] < nnz) nnz = indptr[num_seg];
+  const int lane = threadIdx.x & (kWave - 1);
   const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (c * kChunk >= nnz) return;
-  const int g = ck.outgoing[c];
-  if (g < 0) return;
-  const int64_t seg_e = indptr[g + 1];
-  float total = ck.carry[2 * c + 1];
-  for (int64_t k = c + 1; k * kChunk < seg_e; ++k) total += ck.carry[2 * k];
-  sums[nmap ? static_cast<int64_t>(nmap[g]) : g] = total;
+  int g = -1;
+  int64_t last = 0;  // last chunk the segment reaches
+  if (c * kChunk < nnz) {
+    g = ck.outgoing[c];
+    if (g >= 0) last = (indptr[g + 1] - 1) / kChunk;
+  }
+  const bool wide = g >= 0 && last - c > kCarryAlone;
+  if (g >= 0 && !wide) {
+    float total = ck.carry[2 * c + 1];
+    for (int64_t k = c + 1; k <= last; ++k) total += ck.carry[2 * k];
+    sums[nmap ? static_cast<int64_t>(nmap[g]) : g] = total;
+  }
+  unsigned long long todo = __ballot(wide);
+  while (todo) {
+    const int l = __ffsll(static_cast<long long>(todo)) - 1;
+    todo &= todo - 1;
+    const int64_t from = __shfl(c, l, kWave) + 1;
+    const int64_t to = __shfl(last, l, kWave);
+    float part = 0.0f;
+    for (int64_t k = from + lane; k <= to; k += kWave) part += ck.carry[2 * k];
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) part += __shfl_xor(part, d, kWave);
+    if (lane == l) sums[nmap ? static_cast<int64_t>(nmap[g]) : g] = ck.carry[2 * c + 1] + part;
+  }
 }
 
 // out[d] = data[d] / sums[segment of e] for the edges of long segments
@@ -332,10 +431,34 @@ long_divide_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict
   const int64_t end = begin + kChunk < nnz ? begin + kChunk : nnz;
   int* mark = s_mark[threadIdx.x / kWave];
   const Owned own = load_owned(indptr, ck, c, lane);
-  write_marks(mark, own, begin, end, lane);
   const float own_sum = own.g >= 0 ? sums[own.g] : 0.0f;
+  // the whole chunk lies inside the incoming segment: one divisor, no marks
+  if (__shfl(own.g >= 0 ? own.e : int64_t(0), kIncomingLane, kWave) >= end) {
+    const float total = __shfl(own_sum, kIncomingLane, kWave);
+    for (int64_t e = begin + lane; e < end; e += kWave) {
+      const int64_t d = emap ? emap[e] : e;
+      out[d] = data[d] / total;
+    }
+    return;
+  }
+  // a full chunk of plain data: all four steps' reads are issued before the marks are made
+  const bool ahead = !emap && end - begin == kChunk &&
+                     ((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  float4 early[kChunk / kStep];
+  if (ahead) {
+#pragma unroll
+    for (int t = 0; t < kChunk / kStep; ++t)
+      early[t] = *reinterpret_cast<const float4*>(data + begin + t * kStep + lane * kLaneEdges);
+  } else {
+#pragma unroll
+    for (int t = 0; t < kChunk / kStep; ++t) early[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  }
+  write_marks(mark, own, begin, end, lane);
   int carried = 0;
-  for (int64_t base = begin; base < end; base += kStep) {
+#pragma unroll
+  for (int t = 0; t < kChunk / kStep; ++t) {
+    const int64_t base = begin + t * kStep;
+    if (base >= end) break;
     const int at0 = static_cast<int>(base - begin) + lane * kLaneEdges;
     const int64_t e0 = base + lane * kLaneEdges;
     int m[kLaneEdges];
@@ -348,19 +471,28 @@ long_divide_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict
       if (e0 + k >= end) m[k] = 0;
     const LaneMarks lm = scan_lane_marks(m, at0);
     const int incl = latest_inclusive(lm.last_packed, carried, lane);
-    int cur = __shfl_up(incl, 1, kWave);
-    if (lane == 0) cur = carried;
-    carried = __shfl(incl, kWave - 1, kWave);
+    int cur = lane_move<0x138, 0xf>(carried, incl);
+    carried = __builtin_amdgcn_readlane(incl, kWave - 1);
+    const float have[kLaneEdges] = {early[t].x, early[t].y, early[t].z, early[t].w};
+    float res[kLaneEdges];
+    bool mine[kLaneEdges];
 #pragma unroll
     for (int k = 0; k < kLaneEdges; ++k) {
       if (m[k]) cur = (at0 + k + 1) << 8 | m[k];
       const int owner = owner_of_mark(cur);
       const float total = __shfl(own_sum, owner >= 0 ? owner : 0, kWave);
       const int64_t e = e0 + k;
-      if (e < end && owner >= 0) {
-        const int64_t d = emap ? emap[e] : e;
-        out[d] = data[d] / total;
-      }
+      mine[k] = e < end && owner >= 0;
+      res[k] = 0.0f;
+      if (ahead) res[k] = have[k] / total;
+      else if (mine[k]) res[k] = data[emap ? emap[e] : e] / total;
+    }
+    if (ahead && mine[0] && mine[1] && mine[2] && mine[3]) {
+      *reinterpret_cast<float4*>(out + e0) = make_float4(res[0], res[1], res[2], res[3]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < kLaneEdges; ++k)
+        if (mine[k]) out[emap ? emap[e0 + k] : e0 + k] = res[k];
     }
   }
 }
