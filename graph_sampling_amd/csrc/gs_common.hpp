@@ -171,6 +171,42 @@ inline int blocks_for(int64_t n, int per_block) {
   return static_cast<int>(b < 1 ? 1 : b);
 }
 
+// ------------------------------------------------------- wave-wide search ----
+// Number of leading elements of the sorted a[0..n) that are <= v (the first index whose
+// element exceeds v), found by a whole wave: 64 probes split the range per step, so
+// 2.45 M offsets take four dependent reads instead of twenty-two.  Every lane of the wave
+// calls this and gets the answer.
+__device__ __forceinline__ int64_t wave_upper_bound(const int64_t* __restrict__ a, int64_t n,
+                                                    int64_t v) {
+  const int lane = threadIdx.x & (kWave - 1);
+  int64_t lo = 0, hi = n;
+  while (lo < hi) {
+    const int64_t step = (hi - lo + kWave - 1) / kWave;
+    const int64_t at = lo + lane * step;
+    const bool le = at < hi && a[at] <= v;
+    const int count = __popcll(__ballot(le));  // probes are sorted: the first `count` are <= v
+    const int64_t new_lo = count > 0 ? lo + (count - 1) * step + 1 : lo;
+    const int64_t end = lo + count * step;     // first probe that exceeds v, if there is one
+    hi = (count < kWave && end < hi) ? end : hi;
+    lo = new_lo;
+  }
+  return lo;
+}
+
+// Rows (segments of the offsets ptr[0..n]) that hold positions p_first and p_last, into
+// s_rows[0..1]: the first two waves of the workgroup search, every thread calls this and
+// the values are there after the call (it ends with a workgroup barrier).
+__device__ __forceinline__ void block_row_range(const int64_t* __restrict__ ptr, int64_t n,
+                                                int64_t p_first, int64_t p_last,
+                                                int64_t* s_rows) {
+  const int wave = threadIdx.x / kWave;
+  if (wave < 2) {
+    const int64_t r = wave_upper_bound(ptr, n + 1, wave == 0 ? p_first : p_last) - 1;
+    if ((threadIdx.x & (kWave - 1)) == 0) s_rows[wave] = r;
+  }
+  __syncthreads();
+}
+
 // ------------------------------------------------------------ block scan ----
 // Exclusive scan of one int64 per thread over a block of kThreads threads
 // (multiple of 64).  Returns the exclusive prefix; *total gets the block sum.

@@ -55,10 +55,8 @@ csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz
   __shared__ int s_wave[kThreads / kWave];
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kCooTile;
   const int64_t p1 = p0 + kCooTile < nnz ? p0 + kCooTile : nnz;
-  if (threadIdx.x < 2)
-    s_rows[threadIdx.x] = upper_bound(indptr, num_cols + 1, threadIdx.x == 0 ? p0 : p1 - 1) - 1;
   for (int i = threadIdx.x; i < kCooTile; i += kThreads) s_mark[i] = 0;
-  __syncthreads();
+  block_row_range(indptr, num_cols, p0, p1 - 1, s_rows);
   const int64_t row_lo = s_rows[0], row_hi = s_rows[1];
   // columns row_lo + 1 .. row_hi start inside the tile (row_lo holds its first edge)
   for (int64_t r = row_lo + 1 + threadIdx.x; r <= row_hi; r += kThreads)

@@ -283,9 +283,7 @@ csc_compact_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t
   int64_t row_lo = 0, nrows = 0;
   bool staged = false;
   if (WITH_COO) {
-    if (threadIdx.x < 2)
-      s_rows[threadIdx.x] = upper_bound(indptr, num_cols + 1, threadIdx.x == 0 ? p0 : p1 - 1) - 1;
-    __syncthreads();
+    block_row_range(indptr, num_cols, p0, p1 - 1, s_rows);
     row_lo = s_rows[0];
     nrows = s_rows[1] - row_lo + 1;
     staged = nrows <= kStage;
@@ -387,9 +385,7 @@ sliced_mark_kernel(IdSet t, const int64_t* __restrict__ indptr, const IdT* __res
   __shared__ int s_rank[kWords];
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
   const int64_t p1 = p0 + kTile < D ? p0 + kTile : D;
-  if (threadIdx.x < 2)
-    s_rows[threadIdx.x] = upper_bound(sub_indptr, S + 1, threadIdx.x == 0 ? p0 : p1 - 1) - 1;
-  __syncthreads();
+  block_row_range(sub_indptr, S, p0, p1 - 1, s_rows);
   const int64_t row_lo = s_rows[0];
   const int64_t nrows = s_rows[1] - row_lo + 1;
   const bool staged = nrows <= kStage;

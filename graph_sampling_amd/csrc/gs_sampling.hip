@@ -90,11 +90,7 @@ slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ in
   __shared__ int64_t s_rows[2];
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kFillTile;
   const int64_t p1 = p0 + kFillTile < nnz ? p0 + kFillTile : nnz;
-  if (threadIdx.x < 2) {
-    int64_t p = threadIdx.x == 0 ? p0 : p1 - 1;
-    s_rows[threadIdx.x] = upper_bound(sub_indptr, S + 1, p) - 1;
-  }
-  __syncthreads();
+  block_row_range(sub_indptr, S, p0, p1 - 1, s_rows);
   const int64_t row_lo = s_rows[0];
   const int64_t nrows = s_rows[1] - row_lo + 1;
   const bool staged = nrows <= kFillStage;

@@ -107,11 +107,20 @@ __device__ __forceinline__ void block_column_range(const SddmmArgs<IdT>& a, int6
   }
 }
 
+// need_src / need_dst: whether an operand is taken at that end of the edge; an end nobody
+// asks for is not looked up (the row ids of a CSC are a third of the bytes of a scalar
+// operator over its edges)
 template <typename IdT>
 __device__ __forceinline__ void edge_endpoints(const SddmmArgs<IdT>& a, int64_t e,
                                                const int64_t* s_range, const int64_t* s_ptr,
-                                               int64_t* src, int64_t* dst, int64_t* eid) {
-  *src = static_cast<int64_t>(a.row[e]);
+                                               bool need_src, bool need_dst, int64_t* src,
+                                               int64_t* dst, int64_t* eid) {
+  *src = need_src ? static_cast<int64_t>(a.row[e]) : 0;
+  *eid = a.e_ids ? a.e_ids[e] : e;
+  if (!need_dst) {
+    *dst = 0;
+    return;
+  }
   if (a.indptr) {
     const int64_t n = s_range[1] - s_range[0] + 1;
     const int64_t c = n <= kStageCols ? s_range[0] + column_of(s_ptr, 0, n - 1, e)
@@ -120,7 +129,6 @@ __device__ __forceinline__ void edge_endpoints(const SddmmArgs<IdT>& a, int64_t 
   } else {
     *dst = static_cast<int64_t>(a.col[e]);
   }
-  *eid = a.e_ids ? a.e_ids[e] : e;
 }
 
 // blockDim = (tx, 256/tx): tx walks the out_len positions of an edge, every thread row takes
@@ -132,19 +140,30 @@ __global__ void __launch_bounds__(kThreads) sddmm_generic_kernel(SddmmArgs<IdT> 
   __shared__ int64_t s_ptr[kStageCols];
   const int64_t per_block = static_cast<int64_t>(blockDim.y) * kEdgesPerRow;
   const int64_t e0 = static_cast<int64_t>(blockIdx.x) * per_block;
-  block_column_range(a, e0, e0 + per_block - 1, s_range, s_ptr);
+  const bool need_src = (OP != GS_OP_COPY_RHS && a.lhs_target == 0) ||
+                        (OP != GS_OP_COPY_LHS && a.rhs_target == 0);
+  const bool need_dst = (OP != GS_OP_COPY_RHS && a.lhs_target == 2) ||
+                        (OP != GS_OP_COPY_LHS && a.rhs_target == 2);
+  if (need_dst) block_column_range(a, e0, e0 + per_block - 1, s_range, s_ptr);
+  // the ends of all eight edges first, so that their reads are in flight together
+  int64_t src[kEdgesPerRow], dst[kEdgesPerRow], eid[kEdgesPerRow];
+#pragma unroll
   for (int j = 0; j < kEdgesPerRow; ++j) {
     const int64_t e = e0 + static_cast<int64_t>(j) * blockDim.y + threadIdx.y;
-    if (e >= a.E) return;
-    int64_t src, dst, eid;
-    edge_endpoints(a, e, s_range, s_ptr, &src, &dst, &eid);
+    src[j] = dst[j] = 0;
+    eid[j] = -1;
+    if (e < a.E) edge_endpoints(a, e, s_range, s_ptr, need_src, need_dst, &src[j], &dst[j], &eid[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < kEdgesPerRow; ++j) {
+    if (eid[j] < 0) continue;
     const float* l = (OP == GS_OP_COPY_RHS)
                          ? nullptr
-                         : a.lhs + select3(a.lhs_target, src, eid, dst) * a.lhs_len;
+                         : a.lhs + select3(a.lhs_target, src[j], eid[j], dst[j]) * a.lhs_len;
     const float* r = (OP == GS_OP_COPY_LHS)
                          ? nullptr
-                         : a.rhs + select3(a.rhs_target, src, eid, dst) * a.rhs_len;
-    float* o = a.out + eid * a.out_len;
+                         : a.rhs + select3(a.rhs_target, src[j], eid[j], dst[j]) * a.rhs_len;
+    float* o = a.out + eid[j] * a.out_len;
     for (int64_t k = threadIdx.x; k < a.out_len; k += blockDim.x) {
       const int64_t la = a.lhs_off ? a.lhs_off[k] : k;
       const int64_t ra = a.rhs_off ? a.rhs_off[k] : k;
@@ -168,7 +187,7 @@ __global__ void __launch_bounds__(kThreads) sddmm_dot_rows_kernel(SddmmArgs<IdT>
     const int64_t e = e0 + j * kGroups + threadIdx.x / kDotGroup;
     if (e >= a.E) return;
     int64_t src, dst, eid;
-    edge_endpoints(a, e, s_range, s_ptr, &src, &dst, &eid);
+    edge_endpoints(a, e, s_range, s_ptr, true, true, &src, &dst, &eid);
     const float4* l =
         reinterpret_cast<const float4*>(a.lhs + select3(a.lhs_target, src, eid, dst) * a.lhs_len);
     const float4* r =
