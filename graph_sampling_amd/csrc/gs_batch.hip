@@ -7,14 +7,17 @@
 //   split                       src/cuda/batch_split2.cu:12-100
 //
 // A "batched" array is one flat array plus int64 offsets [B+1] cutting it into B
-// batches.  Everything here is one pass over the items: a workgroup finds the
-// batches of its first and last item once and its lanes search in between.
+// batches.  Everything here is one pass over the items, 2048 per workgroup: the items
+// are read first, then the workgroup finds the batches of its first and last item
+// once and its lanes search in between (the reads do not wait for the searches).
 #include "gs_common.hpp"
 
 namespace gs {
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kItems = 8;
+constexpr int kTile = kThreads * kItems;
 
 // last b in [lo, hi] with ptr[b] <= i
 __device__ __forceinline__ int64_t batch_of(const int64_t* __restrict__ ptr, int64_t i, int64_t lo,
@@ -41,13 +44,21 @@ __global__ void __launch_bounds__(kThreads)
 encode_kernel(const IdT* __restrict__ data, int64_t n, const int64_t* __restrict__ ptr, int64_t B,
               int64_t enc, IdT* __restrict__ out) {
   __shared__ int64_t s_range[2];
-  const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads;
-  const int64_t last = first + kThreads - 1 < n ? first + kThreads - 1 : n - 1;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kTile;
+  const int64_t last = first + kTile - 1 < n ? first + kTile - 1 : n - 1;
+  IdT v[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = first + k * kThreads + threadIdx.x;
+    v[k] = i < n ? data[i] : IdT(0);
+  }
   int64_t lo, hi;
   block_batches(ptr, B, first, last, s_range, &lo, &hi);
-  const int64_t i = first + threadIdx.x;
-  if (i >= n) return;
-  out[i] = static_cast<IdT>(static_cast<int64_t>(data[i]) + batch_of(ptr, i, lo, hi) * enc);
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = first + k * kThreads + threadIdx.x;
+    if (i < n) out[i] = static_cast<IdT>(static_cast<int64_t>(v[k]) + batch_of(ptr, i, lo, hi) * enc);
+  }
 }
 
 template <typename IdT>
@@ -104,19 +115,29 @@ concat_fill_kernel(Segments seg, int64_t B, const int64_t* __restrict__ out_ptr,
   const int s = blockIdx.y;
   const int64_t* ptr = seg.ptr[s];
   const int64_t n = ptr[B];
-  const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kTile;
   if (first >= n) return;
-  const int64_t last = first + kThreads - 1 < n ? first + kThreads - 1 : n - 1;
+  const int64_t last = first + kTile - 1 < n ? first + kTile - 1 : n - 1;
+  const IdT* in = static_cast<const IdT*>(seg.data[s]);
+  IdT v[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = first + k * kThreads + threadIdx.x;
+    v[k] = i < n ? in[i] : IdT(0);
+  }
   int64_t lo, hi;
   block_batches(ptr, B, first, last, s_range, &lo, &hi);
-  const int64_t i = first + threadIdx.x;
-  if (i >= n) return;
-  const int64_t b = batch_of(ptr, i, lo, hi);
-  int64_t before = 0;
-  for (int t = 0; t < s; ++t) before += seg.ptr[t][b + 1] - seg.ptr[t][b];
-  const int64_t w = out_ptr[b] + before + (i - ptr[b]);
-  out[w] = static_cast<const IdT*>(seg.data[s])[i];
-  if (key) key[w] = static_cast<IdT>(b);
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = first + k * kThreads + threadIdx.x;
+    if (i >= n) continue;
+    const int64_t b = batch_of(ptr, i, lo, hi);
+    int64_t before = 0;
+    for (int t = 0; t < s; ++t) before += seg.ptr[t][b + 1] - seg.ptr[t][b];
+    const int64_t w = out_ptr[b] + before + (i - ptr[b]);
+    out[w] = v[k];
+    if (key) key[w] = static_cast<IdT>(b);
+  }
 }
 
 struct OutSegments {
@@ -132,22 +153,32 @@ __global__ void __launch_bounds__(kThreads)
 split_kernel(const IdT* __restrict__ data, const int64_t* __restrict__ data_ptr,
              const IdT* __restrict__ key, int64_t n, int64_t B, OutSegments seg) {
   __shared__ int64_t s_range[2];
-  const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads;
-  const int64_t last = first + kThreads - 1 < n ? first + kThreads - 1 : n - 1;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * kTile;
+  const int64_t last = first + kTile - 1 < n ? first + kTile - 1 : n - 1;
+  IdT v[kItems], kb[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = first + k * kThreads + threadIdx.x;
+    v[k] = i < n ? data[i] : IdT(0);
+    kb[k] = (key && i < n) ? key[i] : IdT(0);
+  }
   int64_t lo = 0, hi = 0;
   if (!key) block_batches(data_ptr, B, first, last, s_range, &lo, &hi);
-  const int64_t i = first + threadIdx.x;
-  if (i >= n) return;
-  const int64_t b = key ? static_cast<int64_t>(key[i]) : batch_of(data_ptr, i, lo, hi);
-  if (b < 0 || b >= B) return;
-  int64_t local = i - data_ptr[b];
-  for (int s = 0; s < seg.n; ++s) {
-    const int64_t len = seg.ptr[s][b + 1] - seg.ptr[s][b];
-    if (local < len) {
-      static_cast<IdT*>(seg.data[s])[seg.ptr[s][b] + local] = data[i];
-      return;
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t i = first + k * kThreads + threadIdx.x;
+    if (i >= n) continue;
+    const int64_t b = key ? static_cast<int64_t>(kb[k]) : batch_of(data_ptr, i, lo, hi);
+    if (b < 0 || b >= B) continue;
+    int64_t local = i - data_ptr[b];
+    for (int s = 0; s < seg.n; ++s) {
+      const int64_t len = seg.ptr[s][b + 1] - seg.ptr[s][b];
+      if (local < len) {
+        static_cast<IdT*>(seg.data[s])[seg.ptr[s][b] + local] = v[k];
+        break;
+      }
+      local -= len;
     }
-    local -= len;
   }
 }
 
@@ -175,7 +206,7 @@ int gs_batch_encode(const void* data, int id_bytes, int64_t n, const int64_t* pt
   if (n == 0) return GS_OK;
   GS_REQUIRE(data && ptr && out, "gs_batch_encode: null pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid(blocks_for(n, kThreads));
+  const dim3 grid(blocks_for(n, kTile));
   if (id_bytes == 8)
     hipLaunchKernelGGL(encode_kernel<int64_t>, grid, dim3(kThreads), 0, st,
                        static_cast<const int64_t*>(data), n, ptr, num_batches, encoding_size,
@@ -263,7 +294,7 @@ int gs_batch_concat_fill(const void* const* segment_data_host,
                                    num_segments, &seg));
   if (max_segment_len == 0) return GS_OK;
   GS_REQUIRE(out, "gs_batch_concat_fill: null output");
-  const dim3 grid(blocks_for(max_segment_len, kThreads), num_segments);
+  const dim3 grid(blocks_for(max_segment_len, kTile), num_segments);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (id_bytes == 8)
     hipLaunchKernelGGL(concat_fill_kernel<int64_t>, grid, dim3(kThreads), 0, st, seg, num_batches,
@@ -291,7 +322,7 @@ int gs_batch_split(const void* data, const int64_t* data_ptr, const void* data_k
   }
   if (n == 0) return GS_OK;
   GS_REQUIRE(data, "gs_batch_split: null input");
-  const dim3 grid(blocks_for(n, kThreads));
+  const dim3 grid(blocks_for(n, kTile));
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (id_bytes == 8)
     hipLaunchKernelGGL(split_kernel<int64_t>, grid, dim3(kThreads), 0, st,
