@@ -123,16 +123,25 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
                        static_cast<int64_t>(threadIdx.x) * kCompactItems;
   bool first[kCompactItems];
   int64_t mine = 0;
+  // slot numbers, then the slots' words, then the stores: three batches, so that the eight
+  // trips to the table are in flight together and none waits for a store before it
+  uint32_t at[kCompactItems], fi[kCompactItems];
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) at[k] = base + k < M_bound ? pos[base + k] : 0u;
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) {
+    // read under the host's bound, not the device-side length, so that the reads do not wait
+    // for it; a slot number beyond the length is whatever the workspace held: masked
+    fi[k] = base + k < M_bound ? t.first_index(at[k] & t.mask) : 0u;
+  }
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) {
     const int64_t i = base + k;
-    // read under the host's bound, not the device-side length, so that the reads do not wait
-    // for it; a slot number beyond the length is whatever the workspace held: masked
-    const uint32_t fi = i < M_bound ? t.first_index(pos[i] & t.mask) : 0u;
-    first[k] = i < M && fi == static_cast<uint32_t>(i);
+    first[k] = i < M && fi[k] == static_cast<uint32_t>(i);
     mine += first[k] ? 1 : 0;
-    // kept for a last pass that must not read the table any more (it empties it)
-    if (first_out && i < M) first_out[i] = fi;
+    // kept for the passes after this one: they need no second trip to the table (and the
+    // last pass of gs_relabel_sampled must not read it any more: it empties it)
+    if (first_out && i < M) first_out[i] = fi[k];
   }
   int64_t tile_total;
   const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
@@ -167,8 +176,8 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
 // Relabel lookups (unique_reindex.cu:162-170): rank of a key = prefix[its first index].
 template <typename IdT, typename T>
 __global__ void __launch_bounds__(kThreads)
-lookup_kernel(T t, const uint32_t* __restrict__ pos, const int64_t* __restrict__ prefix, Query qs,
-              int64_t Q_bound, const int64_t* __restrict__ q_len, int64_t M) {
+lookup_kernel(T t, const uint32_t* __restrict__ first_of, const int64_t* __restrict__ prefix,
+              Query qs, int64_t Q_bound, const int64_t* __restrict__ q_len, int64_t M) {
   const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   int64_t Q = Q_bound;
   if (q_len) {  // one query that aliases the device-sized last mapping span
@@ -188,7 +197,8 @@ lookup_kernel(T t, const uint32_t* __restrict__ pos, const int64_t* __restrict__
   const int64_t local = j - begin;
   int64_t first;
   if (qs.alias[s] >= 0) {
-    first = t.first_index(pos[qs.alias[s] + local]);
+    // a query that is one of the mapping spans: the compaction has set its first indices aside
+    first = first_of[qs.alias[s] + local];
   } else {
     const IdT key = static_cast<const IdT*>(qs.in[s])[local];
     const bool fits = sizeof(IdT) == 4 || !std::is_same<T, PackedTable>::value ||
@@ -242,7 +252,7 @@ template <typename IdT>
 size_t workspace_bytes_for(int64_t M) {
   using T = typename TableFor<IdT>::type;
   const int64_t cap = table_capacity(M);
-  return T::bytes(cap) + padded((M > 0 ? M : 1) * 4) + padded((M + 1) * 8) +
+  return T::bytes(cap) + 2 * padded((M > 0 ? M : 1) * 4) + padded((M + 1) * 8) +
          lookback_state_bytes(compact_num_tiles(M));
 }
 
@@ -270,6 +280,7 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   T t;
   t.carve(ws, cap);
   uint32_t* pos = ws.take<uint32_t>(M > 0 ? M : 1);
+  uint32_t* first = ws.take<uint32_t>(M > 0 ? M : 1);  // index of the first occurrence of item i's key
   int64_t* prefix = ws.take<int64_t>(M + 1);
   const int64_t tiles = compact_num_tiles(M);
   LookbackState lb = carve_lookback(ws, tiles, 1u);  // cleared by table_init on every call
@@ -318,12 +329,12 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
     ProfileScope prof("unique_compact", stream);
     hipLaunchKernelGGL((compact_kernel<IdT, T>), dim3(static_cast<unsigned>(tiles)), dim3(kThreads),
                        0, stream, x, M, t, pos, prefix, static_cast<IdT*>(frontier), num_unique, lb,
-                       box, box_ticket, static_cast<uint32_t*>(nullptr));
+                       box, box_ticket, first);
   }
   if (Q > 0) {
     ProfileScope prof("unique_finish", stream);
     hipLaunchKernelGGL((lookup_kernel<IdT, T>), dim3(blocks_for(Q, kThreads)), dim3(kThreads), 0,
-                       stream, t, pos, prefix, qs, Q, last_span_len, M);
+                       stream, t, first, prefix, qs, Q, last_span_len, M);
   }
   return check_launch("unique_relabel");
 }
@@ -589,7 +600,7 @@ batch_insert_kernel(BatchItems<IdT> x, int64_t M, R t, uint32_t* __restrict__ po
 // flags, chained scan and compaction over all batches at once (see compact_kernel)
 template <typename IdT, typename R>
 __global__ void __launch_bounds__(kThreads)
-batch_compact_kernel(BatchItems<IdT> x, int64_t M, R t, const uint32_t* __restrict__ pos,
+batch_compact_kernel(BatchItems<IdT> x, int64_t M, R t, uint32_t* __restrict__ pos,
                      int64_t* __restrict__ prefix, IdT* __restrict__ unique,
                      int64_t* __restrict__ num_unique, LookbackState lb, gs_mailbox* box,
                      int64_t box_ticket) {
@@ -604,11 +615,20 @@ batch_compact_kernel(BatchItems<IdT> x, int64_t M, R t, const uint32_t* __restri
   const int64_t base = tile_first + static_cast<int64_t>(threadIdx.x) * kCompactItems;
   bool first[kCompactItems];
   int64_t mine = 0;
+  // The slots' words are read here once, eight trips in flight together: from now on pos[i]
+  // is the index of the first occurrence of item i's key, and the lookups of the last pass
+  // need no second trip to the table.
+  uint32_t at[kCompactItems], fi[kCompactItems];
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) at[k] = base + k < M ? pos[base + k] : 0u;
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) fi[k] = base + k < M ? t.first_index(at[k]) : 0u;
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) {
     const int64_t i = base + k;
-    first[k] = i < M && t.first_index(pos[i]) == static_cast<uint32_t>(i);
+    first[k] = i < M && fi[k] == static_cast<uint32_t>(i);
     mine += first[k] ? 1 : 0;
+    if (i < M) pos[i] = fi[k];
   }
   int64_t tile_total;
   const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
@@ -673,9 +693,10 @@ batch_finish_kernel(BatchItems<IdT> x, int64_t num_ids, int64_t M, R t,
     const int64_t b = lo;
     const int64_t begin = x.start(b);
     const int64_t p = begin + (x.seeds_ptr[b + 1] - x.seeds_ptr[b]) + (j - x.ids_ptr[b]);
-    // an index beyond M only when the insert pass gave up (an id too wide for the slots): the
-    // outputs are void then, but no index may leave the arrays
-    const uint32_t fi = t.first_index(pos[p]);
+    // pos holds first-occurrence indices since the compaction.  An index beyond M only when
+    // the insert pass gave up (an id too wide for the slots): the outputs are void then, but
+    // no index may leave the arrays
+    const uint32_t fi = pos[p];
     out_ids[j] = static_cast<IdT>(fi < M ? prefix[fi] - prefix[begin] : -1);
     if (extra) {
       // a second array cut like the ids (the other end of a COO edge): looked up, -1 if absent
