@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0
 # counters (2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE; the factors come from a device copy of
 # known size): profiles/sample_fused_rmat-2.45M-124M_hbm_counters.txt.  The counters cannot
 # be read from inside this process, so the figure is carried here.
-TRAFFIC_BYTES_PER_LAUNCH = {("rmat-2.45M-124M", "sample_fused"): 11627810}
+TRAFFIC_BYTES_PER_LAUNCH = {("rmat-2.45M-124M", "sample_fused"): 11629119}
 
 
 def parse():
