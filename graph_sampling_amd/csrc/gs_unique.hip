@@ -428,6 +428,8 @@ int relabel_sampled_impl(const void* seed_keys, int64_t S, const void* sampled, 
 //    its lanes search inside it.
 constexpr int64_t kRegionFactor = 2;
 
+constexpr int64_t kStagedBatches = 511;  // batch offsets a workgroup keeps in LDS (2 x 4 KB)
+
 template <typename IdT>
 struct BatchItems {
   const IdT* seeds;
@@ -448,6 +450,19 @@ struct BatchItems {
     const int64_t off = i - start(b);
     const int64_t n_seeds = seeds_ptr[b + 1] - seeds_ptr[b];
     return off < n_seeds ? seeds[seeds_ptr[b] + off] : ids[ids_ptr[b] + off - n_seeds];
+  }
+  // The batch offsets copied into LDS (when there are at most kStagedBatches batches), and
+  // this object re-pointed at the copy: the searches and the offset reads that stand between
+  // a lane and its key then cost no trip to memory.  Every thread of the workgroup calls it.
+  __device__ __forceinline__ void stage_offsets(int64_t* lds_seeds_ptr, int64_t* lds_ids_ptr) {
+    if (B > kStagedBatches) return;
+    for (int64_t b = threadIdx.x; b <= B; b += blockDim.x) {
+      lds_seeds_ptr[b] = seeds_ptr[b];
+      lds_ids_ptr[b] = ids_ptr[b];
+    }
+    __syncthreads();
+    seeds_ptr = lds_seeds_ptr;
+    ids_ptr = lds_ids_ptr;
   }
   // batches of the first and the last item of a workgroup's range, through LDS
   __device__ __forceinline__ void block_range(int64_t first, int64_t last, int64_t* lds2,
@@ -579,6 +594,8 @@ __global__ void __launch_bounds__(kThreads)
 batch_insert_kernel(BatchItems<IdT> x, int64_t M, R t, uint32_t* __restrict__ pos,
                     unsigned int* __restrict__ too_wide) {
   __shared__ int64_t s_range[2];
+  __shared__ int64_t s_seeds_ptr[kStagedBatches + 1], s_ids_ptr[kStagedBatches + 1];
+  x.stage_offsets(s_seeds_ptr, s_ids_ptr);
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads;
   const int64_t last = first + kThreads - 1 < M ? first + kThreads - 1 : M - 1;
   int64_t lo, hi;
@@ -607,6 +624,8 @@ batch_compact_kernel(BatchItems<IdT> x, int64_t M, R t, uint32_t* __restrict__ p
   __shared__ int64_t s_scan[kThreads / kWave + 1];
   __shared__ int64_t s_prefix;
   __shared__ int64_t s_range[2];
+  __shared__ int64_t s_seeds_ptr[kStagedBatches + 1], s_ids_ptr[kStagedBatches + 1];
+  x.stage_offsets(s_seeds_ptr, s_ids_ptr);
   const unsigned int tile = blockIdx.x;
   const int64_t tile_first = static_cast<int64_t>(tile) * kCompactTile;
   const int64_t tile_last = tile_first + kCompactTile - 1 < M ? tile_first + kCompactTile - 1 : M - 1;
@@ -670,6 +689,8 @@ batch_finish_kernel(BatchItems<IdT> x, int64_t num_ids, int64_t M, R t,
                     int64_t* __restrict__ unique_ptr, const IdT* __restrict__ extra,
                     IdT* __restrict__ out_extra) {
   __shared__ int64_t s_range[2];
+  __shared__ int64_t s_seeds_ptr[kStagedBatches + 1], s_ids_ptr[kStagedBatches + 1];
+  x.stage_offsets(s_seeds_ptr, s_ids_ptr);
   const int64_t first = static_cast<int64_t>(blockIdx.x) * kThreads;
   if (first < num_ids) {  // a workgroup of id lookups
     const int64_t last = first + kThreads - 1 < num_ids ? first + kThreads - 1 : num_ids - 1;
