@@ -236,7 +236,7 @@ def test_sddmm_coo_ops_targets(dev, op, targets):
 
 @pytest.mark.parametrize("idt", ID_DTYPES)
 def test_sddmm_dot_64_fast_path(dev, idt):
-    # u_dot_v with 64-wide fp32 features (BASELINE config 5)
+    # u_dot_v with 64-wide fp32 features (the large-graph configuration of the benchmark)
     indptr, indices = rmat_csc_np(1 << 11, 1 << 16, seed=8)
     col = O.csc2coo(indptr, indices.size)
     rng = np.random.default_rng(4)
