@@ -317,7 +317,7 @@ coo_compact_kernel(const IdT* __restrict__ key, const IdT* __restrict__ other, i
                    IdT* __restrict__ out_other, int64_t* __restrict__ select_index) {
   const int64_t base = m.tile_base[blockIdx.x];
   const int64_t count = m.tile_base[blockIdx.x + 1] - base;
-  if (count == 0) return;
+  if (count == 0 || !out_key || !out_other) return;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
@@ -858,7 +858,8 @@ int gs_coo_filter_compact(const void* row, const void* col, int id_bytes, int64_
     hipLaunchKernelGGL(filter_batch_ptr_kernel, dim3(blocks_for(num_batches + 1, kThreads)),
                        dim3(kThreads), 0, st, key_batch_ptr, num_batches, s.m, out_batch_ptr);
   if (E > 0) {
-    GS_REQUIRE(row && col && out_row && out_col, "gs_coo_filter_compact: null pointer");
+    GS_REQUIRE(row && col, "gs_coo_filter_compact: null pointer");
+    // no edge kept: the outputs are empty arrays and may be null (the kernel writes nothing)
     const dim3 grid(static_cast<unsigned>(s.m.tiles));
     if (id_bytes == 8)
       hipLaunchKernelGGL((coo_compact_kernel<false, int64_t>), grid, dim3(kThreads), 0, st,

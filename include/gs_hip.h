@@ -515,7 +515,8 @@ int gs_col_row_slice_compact(int64_t D, int id_bytes, void* out_indices, int64_t
  * the ids of its own batch (ids below 2^44).  mark: *num_kept (device scalar).  compact
  * (same workspace, gs_row_slice_workspace_bytes(num_ids, E, 0)): out_row / out_col = the
  * surviving edges in order, select_index (may be NULL) their positions, out_batch_ptr (may
- * be NULL) the batch offsets of the result. */
+ * be NULL) the batch offsets of the result.  When no edge survives the outputs are empty
+ * and may be NULL. */
 int gs_coo_filter_mark(const void* key, int id_bytes, int64_t E, const int64_t* key_batch_ptr,
                        const void* ids, int64_t num_ids, const int64_t* ids_batch_ptr,
                        int64_t num_batches, int64_t* num_kept, void* workspace,

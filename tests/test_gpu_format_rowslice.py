@@ -113,3 +113,36 @@ def test_row_slice_coo(dev, idt):
         assert np.array_equal(g.cpu().numpy(), w)
     mask = np.isin(indices, ids)
     assert np.array_equal(want[1], col[mask])
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("E", [0, 1, 63, 64, 65, 2047, 2048, 2049, 3 * 2048, 3 * 2048 + 64, 9001])
+def test_row_slice_sizes_around_words_and_tiles(dev, E, idt):
+    # the mark pass leaves one bit per edge in 64-edge words and counts per 2048-edge tile:
+    # edge counts on both sides of those boundaries, kept edges everywhere / nowhere / mixed,
+    # ids beyond 2^32 for the 64-bit type, duplicates among the row ids (largest position wins)
+    rng = np.random.default_rng(E)
+    big = (1 << 40) if idt == torch.int64 else 0
+    key = rng.integers(0, 50, size=E).astype(np.int64) + big
+    other = rng.integers(0, 1000, size=E).astype(np.int64)
+    for ids in (np.arange(50, dtype=np.int64) + big,                       # everything kept
+                np.array([77, 78], dtype=np.int64) + big,                  # nothing kept
+                np.array([3, 17, 3, 42, 8, 17], dtype=np.int64) + big):    # mixed, duplicates
+        got = capi.row_slice_coo(to_dev(key, dev, idt), to_dev(other, dev, idt), to_dev(ids, dev, idt))
+        want = O.row_slice_coo(key, other, ids)
+        for g, w in zip(got, want):
+            assert np.array_equal(g.cpu().numpy(), w)
+        # the same edges as a CSC of 7 columns with empty ones in between
+        cuts = np.sort(rng.integers(0, E + 1, size=6))
+        indptr = np.concatenate([[0], cuts, [E]]).astype(np.int64)
+        got = capi.row_slice_csc(to_dev(indptr, dev), to_dev(key, dev, idt), to_dev(ids, dev, idt), True)
+        want = O.row_slice_csc(indptr, key, ids, True)
+        for g, w in zip(got, want):
+            assert np.array_equal(g.cpu().numpy(), w)
+        # membership filter: both ends kept as they are
+        got = capi.coo_filter(to_dev(key, dev, idt), to_dev(key, dev, idt), to_dev(other, dev, idt),
+                              to_dev(ids, dev, idt))
+        mask = np.isin(key, ids)
+        assert np.array_equal(got[0].cpu().numpy(), key[mask])
+        assert np.array_equal(got[1].cpu().numpy(), other[mask])
+        assert np.array_equal(got[3].cpu().numpy(), np.nonzero(mask)[0])
