@@ -58,6 +58,30 @@ def test_coo2csc_unsorted_matches_stable_sort(dev, num_keys, E, idt):
 
 
 @pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("num_keys,E", [(2, 1), (3, 2047), (255, 2048), (256, 2049), (257, 4096),
+                                        (65536, 6000), (65537, 6000), ((1 << 20) + 1, 70000),
+                                        (10, 100000), (5000, 300000)])
+def test_coo2csc_sizes_and_skew(dev, num_keys, E, idt):
+    # edge counts around the 2048-edge sort tiles, key counts around the 8-bit digits (1, 2 and
+    # 3 passes), and keys piled on few columns: the offsets of a 256-column workgroup are then
+    # searched in more than the 4096 keys it can stage
+    rng = np.random.default_rng(num_keys + E)
+    key = (rng.random(E) ** 3 * num_keys).astype(np.int64)        # skewed towards the low keys
+    key[rng.random(E) < 0.01] = num_keys - 1
+    value = rng.integers(0, 1 << 31, size=E).astype(np.int64)
+    ip, val, perm = capi.coo2csc(to_dev(key, dev, idt), to_dev(value, dev, idt), num_keys, False)
+    want_perm = np.argsort(key, kind="stable")
+    assert np.array_equal(perm.cpu().numpy(), want_perm)
+    assert np.array_equal(val.cpu().numpy(), value[want_perm])
+    want_ip = np.concatenate([[0], np.cumsum(np.bincount(key, minlength=num_keys))])
+    assert np.array_equal(ip.cpu().numpy(), want_ip)
+    # the same keys already sorted: offsets only
+    ip2, _, _ = capi.coo2csc(to_dev(key[want_perm], dev, idt), to_dev(value[want_perm], dev, idt),
+                             num_keys, True)
+    assert np.array_equal(ip2.cpu().numpy(), want_ip)
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
 def test_coo2csc_sorted(dev, idt):
     indptr, indices = rmat_csc_np(1 << 12, 1 << 15, seed=3)
     col = np.repeat(np.arange(indptr.size - 1), np.diff(indptr))
