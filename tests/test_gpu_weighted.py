@@ -64,6 +64,37 @@ def test_weighted_hub_many_chunks(dev):
         assert np.array_equal(g, w)
 
 
+@pytest.mark.parametrize("k", [1, 9, 63, 64, 65, 96])
+def test_weighted_degrees_around_the_selection_paths(dev, k):
+    # 256 edges: the last column a wave selects where it finds it; 257 .. 2048: one chunk that
+    # the chunk pass finishes by itself; 2049 and up: several chunks and a merge (4196 edges
+    # with fanout 96 leave 3 * 96 candidates, 40000 edges with fanout 96 more than the 2048 the
+    # register-resident merge holds).  Fanouts on both sides of the 64 lanes (the floor for
+    # dropping candidates comes from the lanes' maxima, and exists only up to 64), equal
+    # weights everywhere in one column (keys differ by the draws only) and a column whose
+    # positive weights are fewer than the fanout.
+    degs = np.array([0, 1, k, k + 1, 255, 256, 257, 1000, 2047, 2048, 2049, 4196, 40000, 300, 600],
+                    dtype=np.int64)
+    indptr = np.concatenate([[0], np.cumsum(degs)])
+    rng = np.random.default_rng(k)
+    indices = rng.integers(0, 1 << 20, int(indptr[-1])).astype(np.int64)
+    probs = (1.0 - rng.random(indices.size)).astype(np.float32)
+    probs[indptr[13]:indptr[14]] = 0.25                      # all weights equal
+    probs[indptr[14]:indptr[15]] = 0.0                       # ... and few positive ones
+    probs[indptr[14] + rng.permutation(600)[:5]] = 0.5
+    rp = O.weighted_replay_ptr(indptr, None, k)
+    replay = u32_draws(int(rp[-1]), k)
+    for idt in (torch.int64, torch.int32):
+        got = _weighted_gpu(dev, indptr, indices, probs, None, k, idt, replay=replay, replay_ptr=rp)
+        want = O.sample_weighted(indptr, indices, probs, None, k, replay=replay)
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w)
+        got = _weighted_gpu(dev, indptr, indices, probs, None, k, idt, seed=31)
+        want = O.sample_weighted(indptr, indices, probs, None, k, seed=31)
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w)
+
+
 def test_weighted_special_cases(dev):
     # one dominant weight is always selected; equal weights -> uniform inclusion
     d, k, trials = 30, 5, 3000
