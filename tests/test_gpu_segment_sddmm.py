@@ -122,6 +122,41 @@ def test_segment_sum_random_layouts(dev, seed):
         np.testing.assert_allclose(out.cpu().numpy(), want_n, rtol=RTOL)
 
 
+@pytest.mark.parametrize("shift", [0, 1, 3])
+def test_segment_sum_hubs_and_unaligned_data(dev, shift):
+    # segments of many whole 1024-edge chunks (summed without marks), their partial chunks at
+    # both ends shared with short and just-long neighbours, and weights that start 4 or 12 bytes
+    # off a 16-byte boundary (the by-edge pass then reads edge by edge instead of four at a time)
+    rng = np.random.default_rng(shift)
+    deg = np.array([3, 5000, 17, 0, 20000, 1, 1024, 1024, 40, 3 * 1024 + 1, 16, 70000, 2],
+                   dtype=np.int64)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    nnz = int(indptr[-1])
+    data = (rng.random(nnz, dtype=np.float32) + np.float32(0.05))
+    base = torch.empty(nnz + 8, dtype=torch.float32, device=dev)
+    d_data = base[shift:shift + nnz]
+    d_data.copy_(to_dev(data, dev))
+    out_base = torch.empty(nnz + 8, dtype=torch.float32, device=dev)
+    for powk in (1, 2):
+        got = torch.empty(deg.size, dtype=torch.float32, device=dev)
+        capi.segment_sum(to_dev(indptr, dev), None, None, d_data, powk, got)
+        want = np.array([(data[indptr[s]:indptr[s + 1]].astype(np.float64) ** powk).sum()
+                         for s in range(deg.size)])
+        np.testing.assert_allclose(got.cpu().numpy(), want, rtol=RTOL)
+    want = np.array([data[indptr[s]:indptr[s + 1]].astype(np.float64).sum() for s in range(deg.size)])
+    out = out_base[shift:shift + nnz]
+    capi.segment_normalize(to_dev(indptr, dev), None, d_data, out)
+    np.testing.assert_allclose(out.cpu().numpy(), data.astype(np.float64) / np.repeat(want, deg),
+                               rtol=RTOL)
+    # through an edge map: weights stored in another order
+    perm = rng.permutation(nnz).astype(np.int64)
+    stored = np.empty_like(data)
+    stored[perm] = data
+    got = torch.empty(deg.size, dtype=torch.float32, device=dev)
+    capi.segment_sum(to_dev(indptr, dev), to_dev(perm, dev), None, to_dev(stored, dev), 1, got)
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=RTOL)
+
+
 def test_segment_sum_edge_count_is_an_upper_bound(dev):
     # the data array may be longer than the offsets cover: the rest is not read into any sum
     indptr = np.array([0, 2000, 2003], dtype=np.int64)
