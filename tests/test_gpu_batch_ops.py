@@ -95,11 +95,11 @@ def test_ops_concat_split_unique(dev, idt):
 
 
 @pytest.mark.parametrize("idt", ID_DTYPES)
-@pytest.mark.parametrize("B", [1, 5, 64])
+@pytest.mark.parametrize("B", [1, 5, 64, 700])
 def test_batch_coo_relabel(dev, B, idt):
     rng = np.random.default_rng(B)
     seeds_ptr = _ptr(rng.integers(0, 50, size=B))
-    coo_ptr = _ptr(rng.integers(0, 900, size=B))
+    coo_ptr = _ptr(rng.integers(0, 900 if B < 100 else 60, size=B))
     seeds = rng.integers(0, 500, size=seeds_ptr[-1]).astype(np.int64)
     row = rng.integers(0, 500, size=coo_ptr[-1]).astype(np.int64)
     # columns are mostly seeds of the same batch; some are strangers and come back as -1

@@ -123,7 +123,11 @@ def _batches(rng, B, n_nodes, max_seeds, max_ids, empty_every=0):
 
 @pytest.mark.parametrize("idt", [torch.int64, torch.int32])
 @pytest.mark.parametrize("B,max_seeds,max_ids,empty_every", [(1, 50, 400, 0), (7, 30, 300, 3),
-                                                               (64, 256, 4000, 0), (300, 8, 40, 5)])
+                                                               (64, 256, 4000, 0), (300, 8, 40, 5),
+                                                               # both sides of the 511 batches whose
+                                                               # offsets a workgroup keeps in LDS
+                                                               (511, 6, 30, 7), (512, 6, 30, 7),
+                                                               (1500, 4, 12, 4)])
 def test_batch_csr_relabel_matches_oracle(dev, idt, B, max_seeds, max_ids, empty_every):
     """Every batch is relabelled on its own: the same id in two batches gets two ranks."""
     rng = np.random.default_rng(B)
