@@ -351,18 +351,29 @@ int num_passes(int64_t num_keys) {
 
 // Offsets of B consecutive column ranges, each re-based to start at 0 and laid
 // out one after the other (batch b: offsets[b+1]-offsets[b]+1 entries starting
-// at offsets[b] + b).  One output entry per lane, batch by binary search.
+// at offsets[b] + b).  One output entry per lane, batch by binary search -- over a
+// copy of the batch offsets in LDS when there are at most 1023 batches, so that only
+// the two reads of indptr go to memory.
+constexpr int kSplitStage = 1024;
+
 __global__ void __launch_bounds__(kThreads)
 indptr_split_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ offsets,
                     int64_t B, int64_t total, int64_t* __restrict__ out) {
+  __shared__ int64_t s_off[kSplitStage];
+  const bool staged = B <= kSplitStage;
+  if (staged) {
+    for (int64_t b = threadIdx.x; b < B; b += kThreads) s_off[b] = offsets[b];
+    __syncthreads();
+  }
+  const int64_t* off = staged ? s_off : offsets;
   const int64_t q = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (q >= total) return;
   int64_t lo = 0, hi = B - 1;  // last b with offsets[b] + b <= q
   while (lo < hi) {
     const int64_t mid = (lo + hi + 1) >> 1;
-    if (offsets[mid] + mid <= q) lo = mid; else hi = mid - 1;
+    if (off[mid] + mid <= q) lo = mid; else hi = mid - 1;
   }
-  const int64_t begin = offsets[lo];
+  const int64_t begin = off[lo];
   out[q] = indptr[begin + (q - begin - lo)] - indptr[begin];
 }
 
