@@ -246,6 +246,11 @@ long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restri
   const int64_t end = begin + kChunk < nnz ? begin + kChunk : nnz;
   int* mark = s_mark[threadIdx.x / kWave];
   const Owned own = load_owned(indptr, ck, c, lane);
+  // no long segment touches the chunk (a chunk of a thousand one-edge rows): nothing to do
+  if (__ballot(own.g >= 0) == 0ull) {
+    if (lane == 0) ck.outgoing[c] = -1;
+    return;
+  }
   // The whole chunk lies inside the incoming segment (most chunks of a hub column do): one
   // sum, no marks, no scans.
   if (__shfl(own.g >= 0 ? own.e : int64_t(0), kIncomingLane, kWave) >= end) {
@@ -431,6 +436,7 @@ long_divide_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict
   const int64_t end = begin + kChunk < nnz ? begin + kChunk : nnz;
   int* mark = s_mark[threadIdx.x / kWave];
   const Owned own = load_owned(indptr, ck, c, lane);
+  if (__ballot(own.g >= 0) == 0ull) return;  // no long segment touches the chunk
   const float own_sum = own.g >= 0 ? sums[own.g] : 0.0f;
   // the whole chunk lies inside the incoming segment: one divisor, no marks
   if (__shfl(own.g >= 0 ? own.e : int64_t(0), kIncomingLane, kWave) >= end) {
