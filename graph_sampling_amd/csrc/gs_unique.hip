@@ -93,6 +93,63 @@ table_insert_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ p
   pos[i] = t.template insert<PEEK>(static_cast<long long>(key), static_cast<uint32_t>(i));
 }
 
+// The same for inputs where keys repeat a lot (the general relabel: edge ends of a block,
+// node lists with hubs).  Thousands of occurrences of one key are thousands of atomics on
+// one table word, and those queue up at the memory side (~11 ns each: 90 k edge ends over
+// 1000 nodes took 58 us, 220 k copies of one key 1.2 ms).  Here the workgroup's 256 items
+// first meet in a small LDS table; of the items that share a key only the one with the
+// lowest index goes to the table in memory, and hands the slot it found to the others.
+constexpr int kGroupSlots = 1024;
+constexpr int kGroupProbes = 4;
+
+template <typename IdT, typename T>
+__global__ void __launch_bounds__(kThreads)
+table_insert_grouped_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ pos,
+                            unsigned int* __restrict__ too_wide) {
+  __shared__ unsigned long long s_key[kGroupSlots];
+  __shared__ unsigned int s_min[kGroupSlots];
+  __shared__ unsigned int s_pos[kGroupSlots];
+  for (int j = threadIdx.x; j < kGroupSlots; j += kThreads) {
+    s_key[j] = ~0ull;
+    s_min[j] = 0xFFFFFFFFu;
+  }
+  __syncthreads();
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  bool live = i < x.items(M_bound);  // the last span's length may live on the device
+  IdT key = IdT(0);
+  if (live) {
+    key = x.get(i);
+    if (sizeof(IdT) == 8 && too_wide && (static_cast<unsigned long long>(key) >> 32) != 0ull) {
+      *too_wide = 2u;
+      pos[i] = 0u;
+      live = false;
+    }
+  }
+  const unsigned long long k64 = static_cast<unsigned long long>(static_cast<long long>(key));
+  int slot = -1;  // the LDS slot of the item's key; none after a few probes: the item goes alone
+  if (live && k64 != ~0ull) {
+    unsigned int h = static_cast<unsigned int>((k64 * 0x9E3779B97F4A7C15ull) >> 40) & (kGroupSlots - 1);
+    for (int probe = 0; probe < kGroupProbes; ++probe) {
+      const unsigned long long seen = atomicCAS(&s_key[h], ~0ull, k64);
+      if (seen == ~0ull || seen == k64) {
+        slot = static_cast<int>(h);
+        atomicMin(&s_min[h], static_cast<unsigned int>(i));
+        break;
+      }
+      h = (h + 1) & (kGroupSlots - 1);
+    }
+  }
+  __syncthreads();
+  const bool leads = live && (slot < 0 || s_min[slot] == static_cast<unsigned int>(i));
+  uint32_t p = 0u;
+  if (leads) {
+    p = t.template insert<true>(static_cast<long long>(key), static_cast<uint32_t>(i));
+    if (slot >= 0) s_pos[slot] = p;
+  }
+  __syncthreads();
+  if (live) pos[i] = leads ? p : s_pos[slot];
+}
+
 struct Query {
   const void* in[GS_MAX_SPANS];
   void* out[GS_MAX_SPANS];
@@ -321,7 +378,7 @@ int unique_relabel_impl(const gs_span* mapping, int n_mapping, const gs_span* qu
   if (M > 0) {
     ProfileScope prof("table_insert", stream);
     constexpr bool kNarrow = sizeof(IdT) == 8 && std::is_same<T, PackedTable>::value;
-    hipLaunchKernelGGL((table_insert_kernel<IdT, T, true>), dim3(blocks_for(M, kThreads)),
+    hipLaunchKernelGGL((table_insert_grouped_kernel<IdT, T>), dim3(blocks_for(M, kThreads)),
                        dim3(kThreads), 0, stream, x, M, t, pos,
                        kNarrow ? lb.error : static_cast<unsigned int*>(nullptr));
   }
