@@ -172,6 +172,77 @@ __global__ void __launch_bounds__(kThreads) sddmm_generic_kernel(SddmmArgs<IdT> 
   }
 }
 
+// Scalar operands on a CSC (weight / per-column sum, weight * per-row factor ...): one value
+// per edge in, one out.  The column of an edge is found as in the CSC -> COO expansion: a
+// workgroup owns 4096 consecutive edges, the columns that start among them mark their first
+// edge in LDS and a running maximum over the marks gives every edge its column -- no search
+// per edge.  Then a pass with consecutive lanes on consecutive edges does the arithmetic.
+constexpr int kScalarItems = 16;
+constexpr int kScalarTile = kThreads * kScalarItems;
+
+template <int OP, typename IdT>
+__global__ void __launch_bounds__(kThreads) sddmm_scalar_csc_kernel(SddmmArgs<IdT> a) {
+  __shared__ int s_mark[kScalarTile];
+  __shared__ int64_t s_rows[2];
+  __shared__ int s_wave[kThreads / kWave];
+  const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kScalarTile;
+  const int64_t p1 = p0 + kScalarTile < a.E ? p0 + kScalarTile : a.E;
+  for (int i = threadIdx.x; i < kScalarTile; i += kThreads) s_mark[i] = 0;
+  block_row_range(a.indptr, a.num_cols, p0, p1 - 1, s_rows);
+  const int64_t row_lo = s_rows[0], row_hi = s_rows[1];
+  // columns row_lo + 1 .. row_hi start inside the tile (row_lo holds its first edge); of
+  // several empty columns at one position the highest wins, which is the owner
+  for (int64_t r = row_lo + 1 + threadIdx.x; r <= row_hi; r += kThreads)
+    atomicMax(&s_mark[a.indptr[r] - p0], static_cast<int>(r - row_lo));
+  __syncthreads();
+  const int at0 = threadIdx.x * kScalarItems;
+  int m[kScalarItems];
+  int run = 0;
+#pragma unroll
+  for (int k = 0; k < kScalarItems; ++k) {
+    const int v = s_mark[at0 + k];
+    run = v > run ? v : run;
+    m[k] = run;
+  }
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  int incl = run;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int y = __shfl_up(incl, d, kWave);
+    if (lane >= d && y > incl) incl = y;
+  }
+  if (lane == kWave - 1) s_wave[wave] = incl;
+  __syncthreads();
+  int before = __shfl_up(incl, 1, kWave);
+  if (lane == 0) before = 0;
+  for (int w = 0; w < wave; ++w) before = s_wave[w] > before ? s_wave[w] : before;
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kScalarItems; ++k) s_mark[at0 + k] = m[k] > before ? m[k] : before;
+  __syncthreads();
+  const bool need_src = (OP != GS_OP_COPY_RHS && a.lhs_target == 0) ||
+                        (OP != GS_OP_COPY_LHS && a.rhs_target == 0);
+#pragma unroll
+  for (int k = 0; k < kScalarItems; ++k) {
+    const int i = k * kThreads + threadIdx.x;
+    const int64_t e = p0 + i;
+    if (e >= p1) continue;
+    const int64_t c = row_lo + s_mark[i];
+    const int64_t dst = a.nid_map ? static_cast<int64_t>(a.nid_map[c]) : c;
+    const int64_t src = need_src ? static_cast<int64_t>(a.row[e]) : 0;
+    const int64_t eid = a.e_ids ? a.e_ids[e] : e;
+    const float* l = (OP == GS_OP_COPY_RHS) ? nullptr : a.lhs + select3(a.lhs_target, src, eid, dst);
+    const float* r = (OP == GS_OP_COPY_LHS) ? nullptr : a.rhs + select3(a.rhs_target, src, eid, dst);
+    a.out[eid] = apply_op<OP>(l, r, 1);
+  }
+}
+
+template <int OP, typename IdT>
+void launch_scalar_csc(const SddmmArgs<IdT>& a, hipStream_t st) {
+  const unsigned grid = static_cast<unsigned>((a.E + kScalarTile - 1) / kScalarTile);
+  hipLaunchKernelGGL((sddmm_scalar_csc_kernel<OP, IdT>), dim3(grid), dim3(kThreads), 0, st, a);
+}
+
 // dot, no broadcast, out_len == 1, R % 4 == 0 and 16-byte aligned rows.
 constexpr int kDotGroup = 16;
 constexpr int kDotEdges = 4;  // edges per 16-lane group
@@ -227,6 +298,17 @@ int sddmm_dispatch(int op, const SddmmArgs<IdT>& a, hipStream_t st) {
     ProfileScope prof("sddmm_dot", st);
     hipLaunchKernelGGL(sddmm_dot_rows_kernel<IdT>, dim3(grid), dim3(kThreads), 0, st, a);
     return check_launch("sddmm_dot");
+  }
+  const bool to_dst = a.lhs_target == 2 || a.rhs_target == 2;
+  if (a.indptr && to_dst && a.out_len == 1 && a.R == 1 && a.lhs_len == 1 && a.rhs_len == 1 &&
+      !a.lhs_off && !a.rhs_off && a.num_cols < (int64_t(1) << 31)) {
+    switch (op) {
+      case GS_OP_ADD: launch_scalar_csc<GS_OP_ADD, IdT>(a, st); return check_launch("sddmm");
+      case GS_OP_SUB: launch_scalar_csc<GS_OP_SUB, IdT>(a, st); return check_launch("sddmm");
+      case GS_OP_MUL: launch_scalar_csc<GS_OP_MUL, IdT>(a, st); return check_launch("sddmm");
+      case GS_OP_DIV: launch_scalar_csc<GS_OP_DIV, IdT>(a, st); return check_launch("sddmm");
+      default: break;  // the copies and a one-element dot go the general way
+    }
   }
   switch (op) {
     case GS_OP_ADD: launch_generic<GS_OP_ADD, IdT>(a, st); break;
