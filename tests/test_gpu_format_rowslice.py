@@ -5,7 +5,8 @@ import torch
 
 from oracle import oracle as O
 from graph_sampling_amd import capi
-from tests.util import graph_12col_4edge, graph_20x5, rmat_csc_np, to_dev
+from tests.util import (graph_12col_4edge, graph_20x5, rmat_csc_np, row_slice_coo_closed_form,
+                        to_dev)
 
 pytestmark = pytest.mark.gpu
 
@@ -135,8 +136,9 @@ def test_row_slice_coo(dev, idt):
     want = O.row_slice_coo(indices, col, ids)
     for g, w in zip(got, want):
         assert np.array_equal(g.cpu().numpy(), w)
-    mask = np.isin(indices, ids)
-    assert np.array_equal(want[1], col[mask])
+    # and against the closed form that does not go through the oracle, all three outputs
+    for g, w in zip(got, row_slice_coo_closed_form(indices, col, ids)):
+        assert np.array_equal(g.cpu().numpy(), w)
 
 
 @pytest.mark.parametrize("idt", ID_DTYPES)
@@ -154,8 +156,9 @@ def test_row_slice_sizes_around_words_and_tiles(dev, E, idt):
                 np.array([3, 17, 3, 42, 8, 17], dtype=np.int64) + big):    # mixed, duplicates
         got = capi.row_slice_coo(to_dev(key, dev, idt), to_dev(other, dev, idt), to_dev(ids, dev, idt))
         want = O.row_slice_coo(key, other, ids)
-        for g, w in zip(got, want):
+        for g, w, c in zip(got, want, row_slice_coo_closed_form(key, other, ids)):
             assert np.array_equal(g.cpu().numpy(), w)
+            assert np.array_equal(w, c)
         # the same edges as a CSC of 7 columns with empty ones in between
         cuts = np.sort(rng.integers(0, E + 1, size=6))
         indptr = np.concatenate([[0], cuts, [E]]).astype(np.int64)

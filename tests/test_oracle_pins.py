@@ -10,7 +10,8 @@ import numpy as np
 import pytest
 
 from oracle import oracle as O
-from tests.util import graph_12col_4edge, graph_20x5, rmat_csc_np, u32_draws
+from tests.util import (graph_12col_4edge, graph_20x5, rmat_csc_np, row_slice_coo_closed_form,
+                        u32_draws)
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 REF = json.load(open(os.path.join(HERE, "golden", "reference_vectors.json")))
@@ -390,6 +391,35 @@ def test_row_slicing_reference_vector():
     ip, coo, ix, sel = O.row_slice_csc(g["indptr"], g["indices"], v["rows"])
     assert ip.tolist() == v["indptr"] and ix.tolist() == v["indices"]
     assert sel.tolist() == v["rows"] and coo.tolist() == list(range(20))
+
+
+def test_row_slice_coo_closed_form():
+    rng = np.random.default_rng(11)
+    cases = []
+    # distinct ids in random order: position != value, so value-for-position mistakes show
+    key = rng.integers(0, 300, size=5000)
+    cases.append((key, rng.integers(0, 10 ** 6, size=5000), rng.permutation(300)[:97]))
+    # duplicate ids: first-vs-last occurrence mistakes show (3 at 0 and 2, 17 at 1 and 5)
+    cases.append((key, np.arange(5000), np.array([3, 17, 3, 42, 8, 17, 299, 0])))
+    # nothing kept / everything kept / ids the edges never mention / no edges / no ids
+    cases.append((key, np.arange(5000), np.array([1000, 2000])))
+    cases.append((key, np.arange(5000), np.arange(299, -1, -1)))
+    cases.append((key, np.arange(5000), np.array([5, 100000, 7])))
+    cases.append((np.zeros(0, dtype=np.int64), np.zeros(0, dtype=np.int64), np.array([1, 2])))
+    cases.append((key, np.arange(5000), np.zeros(0, dtype=np.int64)))
+    # the reference's own graph (tests/test_rowwise_slicing.cc) as a COO
+    g = REF["graph_20x5"]
+    indptr = np.asarray(g["indptr"])
+    cases.append((np.asarray(g["indices"]), np.repeat(np.arange(indptr.size - 1), np.diff(indptr)),
+                  np.asarray(REF["rowwise_slicing_test1"]["rows"])))
+    for key, other, ids in cases:
+        want = row_slice_coo_closed_form(key, other, ids)
+        got = O.row_slice_coo(key, other, ids)
+        for g_, w_ in zip(got, want):
+            assert np.array_equal(g_, w_)
+    # a worked example by hand: ids [7, 5, 7]; 7 -> position 2 (last), 5 -> position 1
+    k, o, s = O.row_slice_coo([5, 6, 7, 5, 9, 7], [10, 11, 12, 13, 14, 15], [7, 5, 7])
+    assert k.tolist() == [1, 2, 1, 2] and o.tolist() == [10, 12, 13, 15] and s.tolist() == [0, 2, 3, 5]
 
 
 def test_format_transform_reference_vectors():

@@ -48,3 +48,15 @@ def to_dev(a, dev, dtype=None):
     if dtype is not None:
         t = t.to(dtype)
     return t.to(dev)
+
+
+def row_slice_coo_closed_form(key, other, ids):
+    """Row slice of a COO from first principles, no oracle involved: an edge is kept when its
+    key is among `ids`; the kept key is renamed to its POSITION in `ids` (the value stored by
+    hashmap.Insert(key[i], i), src/cuda/slicing.cu:744; of duplicate ids the last position
+    wins), the other end is carried, select_index is the edge's place in the input."""
+    key, other, ids = (np.asarray(a, dtype=np.int64) for a in (key, other, ids))
+    place = {int(v): i for i, v in enumerate(ids.tolist())}  # a later duplicate overwrites
+    mask = np.isin(key, ids)
+    renamed = np.array([place[int(v)] for v in key[mask]], dtype=np.int64)
+    return renamed, other[mask], np.nonzero(mask)[0].astype(np.int64)
