@@ -54,6 +54,55 @@ struct ProfileScope {
   }
 };
 
+// ---------------------------------------------------------- phase stamps ----
+// Only in builds with -DGS_PHASE_STAMPS (a measuring build, never the shipped library):
+// thread 0 of every workgroup reads the 100 MHz wall clock at the marked places of a kernel,
+// after waiting for its outstanding memory operations, and appends one record
+// {kind, tile, tiles, stamps...} to a buffer the host registered per translation unit.
+// Without the flag every macro below expands to nothing.
+#ifdef GS_PHASE_STAMPS
+constexpr int kStampSlots = 12;
+constexpr int kStampRecordWords = 16;  // kind, tile, tiles, n, then the stamps
+#define GS_STAMPS_DEFINE(tu)                                                            \
+  namespace gs {                                                                        \
+  static __device__ unsigned long long* g_stamp_buf;                                    \
+  }                                                                                     \
+  extern "C" int gs_debug_set_stamps_##tu(void* buf) {                                  \
+    unsigned long long* p = static_cast<unsigned long long*>(buf);                      \
+    return hipMemcpyToSymbol(HIP_SYMBOL(gs::g_stamp_buf), &p, sizeof(p)) == hipSuccess  \
+               ? GS_OK                                                                  \
+               : GS_ERR_LAUNCH;                                                         \
+  }
+#define GS_STAMP_BEGIN() unsigned long long _st[::gs::kStampSlots] = {}
+#define GS_STAMP(k)                                                \
+  do {                                                             \
+    if (threadIdx.x == 0) {                                        \
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  \
+      _st[k] = wall_clock64();                                     \
+    }                                                              \
+  } while (0)
+#define GS_STAMP_END(kind, n)                                                                 \
+  do {                                                                                        \
+    unsigned long long* _b = ::gs::g_stamp_buf;                                               \
+    if (threadIdx.x == 0 && _b) {                                                             \
+      const unsigned long long _r = atomicAdd(&_b[0], 1ull);                                  \
+      if (_r < _b[1]) {                                                                       \
+        unsigned long long* _w = _b + ::gs::kStampRecordWords * (_r + 1);                     \
+        _w[0] = (kind);                                                                       \
+        _w[1] = blockIdx.x;                                                                   \
+        _w[2] = gridDim.x;                                                                    \
+        _w[3] = (n);                                                                          \
+        for (int _k = 0; _k < ::gs::kStampSlots; ++_k) _w[4 + _k] = _st[_k];                  \
+      }                                                                                       \
+    }                                                                                         \
+  } while (0)
+#else
+#define GS_STAMPS_DEFINE(tu)
+#define GS_STAMP_BEGIN() do {} while (0)
+#define GS_STAMP(k) do {} while (0)
+#define GS_STAMP_END(kind, n) do {} while (0)
+#endif
+
 // Carves 256-byte aligned pieces out of the caller's workspace.
 struct Carver {
   char* base;

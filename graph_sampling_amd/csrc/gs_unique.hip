@@ -27,6 +27,8 @@
 
 #include "gs_table.hpp"
 
+GS_STAMPS_DEFINE(unique)
+
 namespace gs {
 namespace {
 
@@ -81,16 +83,23 @@ table_insert_kernel(Spans<IdT> x, int64_t M_bound, T t, uint32_t* __restrict__ p
                     unsigned int* __restrict__ too_wide) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i >= M_bound) return;
+  GS_STAMP_BEGIN();
+  GS_STAMP(0);
   // the key is read before the device-side length is known (the buffers hold M_bound items
   // whatever the length turns out to be): one round trip instead of two
   const IdT key = x.get(i);
   if (i >= x.items(M_bound)) return;
+  GS_STAMP(1);  // key and length are here
   if (sizeof(IdT) == 8 && too_wide && (static_cast<unsigned long long>(key) >> 32) != 0ull) {
     *too_wide = 2u;
     pos[i] = 0u;
     return;
   }
-  pos[i] = t.template insert<PEEK>(static_cast<long long>(key), static_cast<uint32_t>(i));
+  const uint32_t slot = t.template insert<PEEK>(static_cast<long long>(key), static_cast<uint32_t>(i));
+  GS_STAMP(2);  // the slot is known
+  pos[i] = slot;
+  GS_STAMP(3);
+  GS_STAMP_END(2, 4);
 }
 
 // The same for inputs where keys repeat a lot (the general relabel: edge ends of a block,
@@ -174,6 +183,8 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
                int64_t box_ticket, uint32_t* __restrict__ first_out) {
   __shared__ int64_t s_scan[kThreads / kWave + 1];
   __shared__ int64_t s_prefix;
+  GS_STAMP_BEGIN();
+  GS_STAMP(0);
   const int64_t M = x.items(M_bound);
   const unsigned int tile = blockIdx.x;
   const int64_t base = static_cast<int64_t>(tile) * kCompactTile +
@@ -185,6 +196,7 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
   uint32_t at[kCompactItems], fi[kCompactItems];
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) at[k] = base + k < M_bound ? pos[base + k] : 0u;
+  GS_STAMP(1);  // slot numbers (and the device-side length) are here
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) {
     // read under the host's bound, not the device-side length, so that the reads do not wait
@@ -200,9 +212,11 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
     // last pass of gs_relabel_sampled must not read it any more: it empties it)
     if (first_out && i < M) first_out[i] = fi[k];
   }
+  GS_STAMP(2);  // the slots' words are here
   int64_t tile_total;
   const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
   if (threadIdx.x == 0) lookback_publish_sum(lb, tile, tile_total);
+  GS_STAMP(3);  // flags scanned, tile sum published
   IdT key[kCompactItems];  // in flight while wave 0 walks back
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) key[k] = first[k] ? x.get(base + k) : IdT(0);
@@ -210,7 +224,9 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
     const int64_t before = lookback_exclusive_prefix(lb, tile, tile_total);
     if (threadIdx.x == 0) s_prefix = before;
   }
+  GS_STAMP(4);  // look-back done (and thread 0's keys)
   __syncthreads();
+  GS_STAMP(5);
   int64_t run = s_prefix + local;
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) {
@@ -228,6 +244,8 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
     *num_unique = total;
     post_mailbox(box, total, box_ticket);
   }
+  GS_STAMP(6);  // stores done
+  GS_STAMP_END(3, 7);
 }
 
 // Relabel lookups (unique_reindex.cu:162-170): rank of a key = prefix[its first index].
@@ -279,20 +297,26 @@ finish_linked_kernel(T t, const uint32_t* __restrict__ pos, const uint32_t* __re
                      const int64_t* __restrict__ sampled_len, IdT* __restrict__ out_ids,
                      int64_t* __restrict__ offsets_copy) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  GS_STAMP_BEGIN();
+  GS_STAMP(0);
   // the sampler's S + 1 offsets end at sampled_len: a second copy for the caller who hands
   // the relabelled block out beside the sampled graph (saves a device copy per call)
   if (offsets_copy && i <= S) offsets_copy[i] = (sampled_len - S)[i];
   // reads go by the host's bound so that they do not wait for the device-side length
   const uint32_t f = i < M_bound ? first[i] : 0u;
+  GS_STAMP(1);  // first-occurrence index is here
   const int64_t rank = prefix[f < M_bound ? f : 0u];
   const uint32_t p = i < M_bound ? pos[i] : 0u;
   int64_t n = *sampled_len;
   if (n < 0) n = 0;
   int64_t M = S + n;
   if (M > M_bound) M = M_bound;
+  GS_STAMP(2);  // rank, slot and length are here
   if (i >= M) return;
   if (i >= S) out_ids[i - S] = static_cast<IdT>(rank);
   t.clear(p);
+  GS_STAMP(3);
+  GS_STAMP_END(4, 4);
 }
 
 template <typename T>
