@@ -23,6 +23,8 @@
 //    and a last pass gathers the ids.
 #include "gs_common.hpp"
 
+GS_STAMPS_DEFINE(sampling)
+
 namespace gs {
 namespace {
 
@@ -569,6 +571,8 @@ __global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<I
   const int64_t row0 = static_cast<int64_t>(tile) * kFusedRows;
   const int k = static_cast<int>(a.k);
   const int64_t my_row = row0 + threadIdx.x;
+  GS_STAMP_BEGIN();
+  GS_STAMP(0);
 
   // ---- 1. one row per lane
   int64_t start = 0, deg = 0, cnt = 0;
@@ -580,9 +584,11 @@ __global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<I
     }
     cnt = REPLACE ? (deg > 0 ? a.k : 0) : (deg < a.k ? deg : a.k);
   }
+  GS_STAMP(1);  // column id and offsets are here
   int64_t tile_total;
   const int64_t local = block_exclusive_scan<kFusedThreads>(cnt, &tile_total, s_scan);
   if (threadIdx.x == 0) lookback_publish_sum(a.lb, tile, tile_total);
+  GS_STAMP(2);  // counts scanned, tile sum published
   s_start[threadIdx.x] = start;
   s_deg[threadIdx.x] = static_cast<uint32_t>(deg);
   s_rel[threadIdx.x] = static_cast<uint32_t>(local);
@@ -614,11 +620,14 @@ __global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<I
       }
     }
   }
+  GS_STAMP(3);  // selection done (thread 0's own row)
   if (threadIdx.x < kWave) {
     const int64_t before = lookback_exclusive_prefix(a.lb, tile, tile_total);
     if (threadIdx.x == 0) s_prefix = before;
   }
+  GS_STAMP(4);  // look-back done
   __syncthreads();
+  GS_STAMP(5);  // every wave's selection done
   const int64_t out0 = s_prefix;
   if (my_row < a.S) a.sub_indptr[my_row] = out0 + local;
   if (tile == tiles - 1 && threadIdx.x == 0) {
@@ -661,6 +670,7 @@ __global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<I
         v[u] = indices[q[u]];
       }
     }
+    if (base == threadIdx.x) GS_STAMP(6);  // first batch of gathers back
 #pragma unroll
     for (int u = 0; u < kFusedBatch; ++u) {
       const uint32_t e = base + u * kFusedThreads;
@@ -671,6 +681,8 @@ __global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<I
       }
     }
   }
+  GS_STAMP(7);  // stores done
+  GS_STAMP_END(1, 8);
 }
 
 template <typename IdT>
@@ -928,7 +940,6 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
                                        seed, replay, replay_ptr, sub_indptr, sub_indices,
                                        select_index, coo_col, lb, mailbox, mailbox_ticket, st);
 }
-
 
 int gs_sample_one_keepdim(const int64_t* indptr, int64_t num_cols, const void* indices,
                           const void* column_ids, int id_bytes, int64_t S, uint64_t seed,
