@@ -276,6 +276,27 @@ def sample_uniform_fused(indptr, indices, column_ids, fanout, replace, seed=0, r
     return sub_indptr, sub_indices, select_index, coo_col
 
 
+def sample_uniform_fused_static(indptr, indices, column_ids, fanout, replace, out, seed=0,
+                                replay=None, replay_ptr=None, mailbox=None):
+    """gs_sample_uniform_fused_static: the one-launch sampler on the library's own state, for
+    callers that cannot allocate.  `out` = (sub_indptr[S + 1], sub_indices[cap], select_index[cap]
+    or None, coo_col[cap] or None), all the caller's; nothing is allocated here or in the call."""
+    _need(indptr, torch.int64, "indptr")
+    idb = _ids(indices, "indices")
+    dev = indptr.device
+    S = indptr.numel() - 1 if column_ids is None else column_ids.numel()
+    sub_indptr, sub_indices, select_index, coo_col = out
+    ticket = mailbox.ticket() if mailbox is not None else 0
+    _check(lib().gs_sample_uniform_fused_static(
+        _ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(column_ids), idb, _i64(S),
+        _i64(fanout), int(bool(replace)), _u64(seed), _ptr(replay), _ptr(replay_ptr),
+        _ptr(sub_indptr), _ptr(sub_indices), _ptr(select_index), _ptr(coo_col),
+        _i64(sub_indices.numel()),
+        mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0), _i64(ticket), _stream(dev)),
+        "gs_sample_uniform_fused_static")
+    return ticket
+
+
 class RelabelTable:
     """The persistent hash table of gs_relabel_sampled (prepared once, left empty by every call)."""
 

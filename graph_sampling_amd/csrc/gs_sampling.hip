@@ -23,6 +23,8 @@
 //    and a last pass gathers the ids.
 #include "gs_common.hpp"
 
+#include <mutex>
+
 GS_STAMPS_DEFINE(sampling)
 
 namespace gs {
@@ -772,6 +774,33 @@ static int sample_uniform_fill_t(const int64_t* indptr, int64_t num_cols, const 
                  : sample_fill_impl<IdT, false>(a, replace, algo, st);
 }
 
+// ---- the same sampler for callers that cannot allocate ----
+// Its look-back state (what gs_sample_uniform_fused takes as `state`) lives in a device
+// array of this library instead of a caller's buffer: room for GS_FUSED_STATIC_MAX_COLUMNS
+// columns.  In host code the array's name is only a stand-in; its device address is asked
+// for once per device (hipGetSymbolAddress) and kept.
+namespace gs {
+namespace {
+constexpr int64_t kStaticTiles = (GS_FUSED_STATIC_MAX_COLUMNS + kFusedRows - 1) / kFusedRows;
+constexpr size_t kStaticStateBytes = ((kStaticTiles * 8 + 255) / 256) * 256 + 256 + 256;
+constexpr int kMaxDevices = 64;
+
+struct StaticState {
+  void* ptr = nullptr;  // device address of `scratch` on this device
+  uint32_t epoch = 0;   // last epoch handed out; 0 = the array has to be zero-filled first
+};
+StaticState g_static_state[kMaxDevices];
+std::mutex g_static_mu;
+
+static __global__ void __launch_bounds__(256) zero_words_kernel(unsigned long long* p, size_t n) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0ull;
+}
+}  // namespace
+}  // namespace gs
+
+static __device__ __align__(256) unsigned char scratch[gs::kStaticStateBytes];
+
 extern "C" {
 
 size_t gs_slice_workspace_bytes(int64_t num_cols) { return scan_workspace_bytes(num_cols); }
@@ -939,6 +968,61 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
              : sample_fused_t<int32_t>(indptr, num_cols, indices, column_ids, S, fanout, replace,
                                        seed, replay, replay_ptr, sub_indptr, sub_indices,
                                        select_index, coo_col, lb, mailbox, mailbox_ticket, st);
+}
+
+int gs_sample_uniform_fused_static(const int64_t* indptr, int64_t num_cols, const void* indices,
+                                   const void* column_ids, int id_bytes, int64_t S,
+                                   int64_t fanout, int replace, uint64_t seed,
+                                   const uint32_t* replay, const int64_t* replay_ptr,
+                                   int64_t* sub_indptr, void* sub_indices,
+                                   int64_t* select_index, void* coo_col, int64_t capacity,
+                                   gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream) {
+  if (S > GS_FUSED_STATIC_MAX_COLUMNS) {
+    set_error_text("gs_sample_uniform_fused_static: %lld columns exceed the %lld the library's "
+                   "own state holds; use gs_sample_uniform_fused with a caller's state buffer",
+                   static_cast<long long>(S), static_cast<long long>(GS_FUSED_STATIC_MAX_COLUMNS));
+    return GS_ERR_UNSUPPORTED;
+  }
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    set_error_text("gs_sample_uniform_fused_static: no current device (or its number is above %d)",
+                   kMaxDevices - 1);
+    return GS_ERR_LAUNCH;
+  }
+  void* state = nullptr;
+  uint32_t epoch = 0;
+  {
+    std::lock_guard<std::mutex> lock(g_static_mu);
+    StaticState& st = g_static_state[device];
+    if (!st.ptr) {
+      void* p = nullptr;
+      const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || !p) {
+        set_error_text("gs_sample_uniform_fused_static: hipGetSymbolAddress: %s",
+                       hipGetErrorString(e));
+        return GS_ERR_LAUNCH;
+      }
+      st.ptr = p;
+      st.epoch = 0;
+    }
+    if (st.epoch == 0 || st.epoch >= kLbMaxEpoch) {
+      // first use on this device, or every epoch has been used: start again from zeroes (a
+      // fill kernel on the caller's stream, so that a caller who records the call gets a
+      // kernel node)
+      const size_t words = kStaticStateBytes / 8;
+      hipLaunchKernelGGL(zero_words_kernel, dim3(static_cast<unsigned>((words + 255) / 256)),
+                         dim3(256), 0, static_cast<hipStream_t>(stream),
+                         static_cast<unsigned long long*>(st.ptr), words);
+      GS_RETURN_IF_ERROR(check_launch("gs_sample_uniform_fused_static (state fill)"));
+      st.epoch = 0;
+    }
+    state = st.ptr;
+    epoch = ++st.epoch;
+  }
+  return gs_sample_uniform_fused(indptr, num_cols, indices, column_ids, id_bytes, S, fanout,
+                                 replace, seed, replay, replay_ptr, sub_indptr, sub_indices,
+                                 select_index, coo_col, capacity, state, kStaticStateBytes, epoch,
+                                 mailbox, mailbox_ticket, stream);
 }
 
 int gs_sample_one_keepdim(const int64_t* indptr, int64_t num_cols, const void* indices,

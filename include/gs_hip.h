@@ -197,6 +197,27 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
                             void* state, size_t state_bytes, uint32_t epoch,
                             gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
 
+/* gs_sample_uniform_fused for callers that cannot allocate (no counterpart in the
+ * reference: it is for code under HIP graph capture, tight serving loops and harnesses
+ * that forbid hipMalloc, which can bring outputs but no state buffer of the right age).
+ * The look-back state lives in a device array of the library itself
+ * (GS_FUSED_STATIC_MAX_COLUMNS columns, about 130 KB per device, held until the process
+ * ends) and the library counts the epochs; the call allocates nothing, on the host side
+ * of the device or on the device.  Same arguments, results and status codes as
+ * gs_sample_uniform_fused otherwise; S above GS_FUSED_STATIC_MAX_COLUMNS is refused with
+ * GS_ERR_UNSUPPORTED.  Runs on the current device.  Every call on a device shares that
+ * device's array: calls that overlap in time on one device (two streams, two threads)
+ * race; calls on one stream, or ordered by events, are fine.  Once per 16383 calls, and at
+ * the first call on a device, a fill kernel on `stream` zeroes the array first. */
+#define GS_FUSED_STATIC_MAX_COLUMNS ((int64_t)1 << 22)
+int gs_sample_uniform_fused_static(const int64_t* indptr, int64_t num_cols, const void* indices,
+                                   const void* column_ids, int id_bytes, int64_t S,
+                                   int64_t fanout, int replace, uint64_t seed,
+                                   const uint32_t* replay, const int64_t* replay_ptr,
+                                   int64_t* sub_indptr, void* sub_indices,
+                                   int64_t* select_index, void* coo_col, int64_t capacity,
+                                   gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
+
 /* fanout == 1 with replacement through the fused entry: exactly one slot per
  * column, -1 in both outputs for an empty column; sub_indptr = 0..S.  Replaces
  * impl::fusion::FusedCSCColSlicingSamplingOneKeepDimCUDA
