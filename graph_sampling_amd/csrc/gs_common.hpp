@@ -84,7 +84,10 @@ constexpr int kStampRecordWords = 16;  // kind, tile, tiles, n, then the stamps
 #define GS_STAMP_END(kind, n)                                                                 \
   do {                                                                                        \
     unsigned long long* _b = ::gs::g_stamp_buf;                                               \
-    if (threadIdx.x == 0 && _b) {                                                             \
+    /* in large grids one workgroup in 16 (and the last) reports: the shared cursor is a */  \
+    /* same-address atomic, and thousands of those would be what the stamps measure      */  \
+    if (threadIdx.x == 0 && _b &&                                                             \
+        (gridDim.x <= 256 || (blockIdx.x & 15u) == 0 || blockIdx.x == gridDim.x - 1)) {       \
       const unsigned long long _r = atomicAdd(&_b[0], 1ull);                                  \
       if (_r < _b[1]) {                                                                       \
         unsigned long long* _w = _b + ::gs::kStampRecordWords * (_r + 1);                     \

@@ -521,24 +521,48 @@ int sample_fill_impl(const SampleArgs<IdT>& a, int replace, int algo, hipStream_
 
 
 // ------------------------------------------- one-launch slice + sample ----
-// Counting, the scan of the counts and the fill in ONE kernel.  A workgroup
-// takes a tile of 256 rows:
-//  1. one row per lane reads its column id and offsets (256 independent random
-//     reads in flight per workgroup), the tile's counts are scanned in LDS and
-//     the tile prefix comes from a look-back over earlier tiles;
-//  2. without replacement every lane runs Floyd's selection for its own row in
-//     registers (a fully unrolled k x k duplicate check, four draws per Philox
-//     block) and parks the k chosen positions in LDS;
-//  3. the tile's outputs are then written edge-parallel: lane e finds its row by
-//     binary search in the LDS offsets, so every gather of a lane is independent
-//     of the others and every store is fully coalesced.
-// The outputs must hold S * fanout entries; the true total lands in
-// sub_indptr[S] (and in the host mailbox when one is given).  No workgroup does a
-// read-modify-write on a shared address (see the look-back notes).
-constexpr int kFusedThreads = 256;
-constexpr int kFusedRows = 256;
-constexpr int kFusedBatch = 8;  // gathers a lane keeps in flight in the fill
-constexpr int kPickStride = kFusedRows + 1;  // odd stride: conflict-free by row and by step
+// Counting, the scan of the counts and the fill in ONE kernel.  G lanes share a
+// row (G = 1, 2, 4, 8 for a fanout up to 4, 8, 16, 32); a workgroup takes a tile of
+// THREADS / G rows:
+//  1. every lane of a row reads its column id and offsets (the lanes of a row ask for the
+//     same addresses, which cost one request); the tile's counts are scanned and
+//     the tile's sum is published for the look-back of the later tiles;
+//  2. without replacement the row's lanes run Floyd's selection together: lane s
+//     makes the Philox block of draws 4s..4s+3 and reduces them to their ranges
+//     (the quarter-rate multiplies and the divisions, the bulk of the arithmetic,
+//     spread over the lanes), then the "already chosen?" chain runs step by step
+//     with one in-register lane move per step (quad_perm for G <= 4);
+//  3. wave 0 walks back over the earlier tiles for the tile's output offset while
+//     the other waves already gather;
+//  4. lane s gathers and stores outputs 4s..4s+3 of its row: no search for the row
+//     of an output, nothing parked in LDS.
+// With replacement a lane makes 4 picks per round and a row takes as many rounds
+// as its fanout needs.  The outputs must hold S * fanout entries; the true total
+// lands in sub_indptr[S] (and in the host mailbox when one is given).  No
+// workgroup does a read-modify-write on a shared address (see the look-back
+// notes).  Launches of up to 2^17 lanes use 256-thread tiles (a minibatch layer of
+// 1024 columns becomes 16 workgroups, not 4), larger ones 1024-thread tiles so that the
+// chain of tiles stays short.
+constexpr int kGroupThreadsSmall = 256;
+constexpr int kGroupThreadsLarge = 1024;
+constexpr int64_t kGroupSmallLanes = int64_t(1) << 17;
+constexpr int kGroupMaxLanes = 8;
+
+inline int group_lanes_for(int64_t fanout) {
+  return fanout <= 4 ? 1 : (fanout <= 8 ? 2 : (fanout <= 16 ? 4 : 8));
+}
+// tiles of the launch that samples S columns with G lanes each
+inline int64_t group_tiles(int64_t S, int G) {
+  const int64_t threads = S * G > kGroupSmallLanes ? kGroupThreadsLarge : kGroupThreadsSmall;
+  const int64_t rows = threads / G;
+  return (S + rows - 1) / rows;
+}
+// most tiles any fanout can ask for
+inline int64_t group_tiles_bound(int64_t S) {
+  const int64_t large = (S * kGroupMaxLanes + kGroupThreadsLarge - 1) / kGroupThreadsLarge;
+  const int64_t small = kGroupSmallLanes / kGroupThreadsSmall;
+  return (large > small ? large : small) + 1;
+}
 
 template <typename IdT>
 struct FusedArgs {
@@ -560,23 +584,41 @@ struct FusedArgs {
   int64_t box_ticket;
 };
 
-template <typename IdT, int KMAX, bool REPLACE>
-__global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<IdT> a) {
-  extern __shared__ uint32_t s_pick[];  // [k][kPickStride], without replacement only
-  __shared__ int64_t s_start[kFusedRows];
-  __shared__ uint32_t s_deg[kFusedRows];
-  __shared__ uint32_t s_rel[kFusedRows + 1];  // output offsets relative to the tile's first
-  __shared__ int64_t s_scan[kFusedThreads / kWave + 1];
+// the value lane `owner` of every G-lane group holds (owner is a constant after unrolling)
+template <int G>
+__device__ __forceinline__ uint32_t group_broadcast(uint32_t v, int owner) {
+  if (G == 1) return v;
+  const int x = static_cast<int>(v);
+  if (G == 2) {  // pairs inside a quad: lanes (0,1) read lane owner, lanes (2,3) lane 2 + owner
+    return static_cast<uint32_t>(owner == 0 ? __builtin_amdgcn_update_dpp(0, x, 0xA0, 0xF, 0xF, false)
+                                            : __builtin_amdgcn_update_dpp(0, x, 0xF5, 0xF, 0xF, false));
+  }
+  if (G == 4) {
+    switch (owner) {
+      case 0: return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, x, 0x00, 0xF, 0xF, false));
+      case 1: return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, x, 0x55, 0xF, 0xF, false));
+      case 2: return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, x, 0xAA, 0xF, 0xF, false));
+      default: return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, x, 0xFF, 0xF, 0xF, false));
+    }
+  }
+  return static_cast<uint32_t>(__shfl(x, ((threadIdx.x & (kWave - 1)) & ~(G - 1)) | owner, kWave));
+}
+
+template <typename IdT, int G, bool REPLACE, int THREADS>
+__global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a) {
+  constexpr int kRows = THREADS / G;
+  constexpr int KMAX = 4 * G;
+  __shared__ int64_t s_scan[THREADS / kWave + 1];
   __shared__ int64_t s_prefix;
   const unsigned int tile = blockIdx.x;
   const unsigned int tiles = gridDim.x;
-  const int64_t row0 = static_cast<int64_t>(tile) * kFusedRows;
+  const int sub = threadIdx.x & (G - 1);
+  const int64_t my_row = static_cast<int64_t>(tile) * kRows + threadIdx.x / G;
   const int k = static_cast<int>(a.k);
-  const int64_t my_row = row0 + threadIdx.x;
   GS_STAMP_BEGIN();
   GS_STAMP(0);
 
-  // ---- 1. one row per lane
+  // ---- 1. the row's column and offsets
   int64_t start = 0, deg = 0, cnt = 0;
   if (my_row < a.S) {
     const int64_t c = a.cols ? static_cast<int64_t>(a.cols[my_row]) : my_row;
@@ -588,125 +630,158 @@ __global__ void __launch_bounds__(kFusedThreads) sample_fused_kernel(FusedArgs<I
   }
   GS_STAMP(1);  // column id and offsets are here
   int64_t tile_total;
-  const int64_t local = block_exclusive_scan<kFusedThreads>(cnt, &tile_total, s_scan);
+  const int64_t ex = block_exclusive_scan<THREADS>(sub == 0 ? cnt : 0, &tile_total, s_scan);
+  const int64_t local = sub == 0 ? ex : ex - cnt;  // the row's first output, relative to the tile's
   if (threadIdx.x == 0) lookback_publish_sum(a.lb, tile, tile_total);
   GS_STAMP(2);  // counts scanned, tile sum published
-  s_start[threadIdx.x] = start;
-  s_deg[threadIdx.x] = static_cast<uint32_t>(deg);
-  s_rel[threadIdx.x] = static_cast<uint32_t>(local);
-  if (threadIdx.x == 0) s_rel[kFusedRows] = static_cast<uint32_t>(tile_total);
 
-  // ---- 2. Floyd's selection, one row per lane, positions to LDS
+  // ---- 2. Floyd's selection by the row's lanes: mine[u] = position of output 4*sub+u
+  uint32_t mine[4] = {0u, 0u, 0u, 0u};
   if (!REPLACE && cnt > 0) {
     if (deg <= a.k) {
-      for (int i = 0; i < static_cast<int>(deg); ++i) s_pick[i * kPickStride + threadIdx.x] = i;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) mine[u] = static_cast<uint32_t>(4 * sub + u);
     } else {
-      const uint32_t* rp = a.replay ? a.replay + a.replay_ptr[my_row] : nullptr;
+      const uint32_t lowest = static_cast<uint32_t>(deg - a.k);  // step i draws from [0, lowest + i]
+      uint32_t t[4] = {0u, 0u, 0u, 0u};
+      if (4 * sub < k) {
+        U4 blk;
+        if (a.replay) {
+          const uint32_t* rp = a.replay + a.replay_ptr[my_row];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) blk.v[u] = 4 * sub + u < k ? rp[4 * sub + u] : 0u;
+        } else {
+          blk = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(my_row),
+                           static_cast<uint64_t>(sub));
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) t[u] = blk.v[u] % (lowest + static_cast<uint32_t>(4 * sub + u) + 1u);
+      }
       uint32_t chosen[KMAX];
-      U4 blk;
 #pragma unroll
       for (int i = 0; i < KMAX; ++i) {
         if (i < k) {
-          if ((i & 3) == 0 && !rp)
-            blk = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(my_row),
-                             static_cast<uint64_t>(i >> 2));
-          const uint32_t xv = rp ? rp[i] : blk.v[i & 3];
-          const uint32_t j = static_cast<uint32_t>(deg - a.k + i);
-          const uint32_t t = xv % (j + 1u);
+          const uint32_t ti = t[i & 3];  // the owner's lane holds the step's draw
           bool taken = false;
 #pragma unroll
-          for (int m = 0; m < i; ++m) taken |= chosen[m] == t;
-          chosen[i] = taken ? j : t;
-          s_pick[i * kPickStride + threadIdx.x] = chosen[i];
+          for (int m = 0; m < i; ++m) taken |= chosen[m] == ti;
+          const uint32_t c = group_broadcast<G>(taken ? lowest + static_cast<uint32_t>(i) : ti, i >> 2);
+          chosen[i] = c;
+          if (sub == (i >> 2)) mine[i & 3] = c;
         }
       }
     }
   }
-  GS_STAMP(3);  // selection done (thread 0's own row)
+  GS_STAMP(3);  // selection done
   if (threadIdx.x < kWave) {
     const int64_t before = lookback_exclusive_prefix(a.lb, tile, tile_total);
     if (threadIdx.x == 0) s_prefix = before;
   }
   GS_STAMP(4);  // look-back done
+
+  // ---- 3. gather: outputs 4*sub .. 4*sub+3 of the row (round 0)
+  const IdT* __restrict__ indices = a.indices;
+  const uint32_t* rp_replace = REPLACE && a.replay && cnt > 0 ? a.replay + a.replay_ptr[my_row] : nullptr;
+  int64_t q[4];
+  IdT v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) q[u] = -1;
+  if (cnt > 0) {
+    if (REPLACE) {
+      U4 blk;
+      if (rp_replace) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) blk.v[u] = 4 * sub + u < k ? rp_replace[4 * sub + u] : 0u;
+      } else {
+        blk = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(my_row),
+                         static_cast<uint64_t>(sub));
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) mine[u] = blk.v[u] % static_cast<uint32_t>(deg);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (4 * sub + u < cnt) {
+        q[u] = start + mine[u];
+        v[u] = indices[q[u]];
+      }
+    }
+  }
   __syncthreads();
-  GS_STAMP(5);  // every wave's selection done
   const int64_t out0 = s_prefix;
-  if (my_row < a.S) a.sub_indptr[my_row] = out0 + local;
+  GS_STAMP(5);  // the tile's offset is known to every wave, the first gathers are back
+  if (my_row < a.S && sub == 0) a.sub_indptr[my_row] = out0 + local;
   if (tile == tiles - 1 && threadIdx.x == 0) {
     int64_t total = out0 + tile_total;
     if (__hip_atomic_load(a.lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) total = -1;
     a.sub_indptr[a.S] = total;
     post_mailbox(a.box, total, a.box_ticket);
   }
-
-  // ---- 3. edge-parallel gather and store, kFusedBatch gathers in flight per lane
-  const uint32_t n_out = static_cast<uint32_t>(tile_total);
-  const IdT* __restrict__ indices = a.indices;
-  for (uint32_t base = threadIdx.x; base < n_out; base += kFusedThreads * kFusedBatch) {
-    int64_t q[kFusedBatch];
-    int64_t r[kFusedBatch];
-    IdT v[kFusedBatch];
+  const int64_t row_out = out0 + local;
 #pragma unroll
-    for (int u = 0; u < kFusedBatch; ++u) {
-      const uint32_t e = base + u * kFusedThreads;
-      q[u] = -1;
-      if (e < n_out) {
-        int lo = 0, hi = kFusedRows;  // last row with s_rel[row] <= e
-        while (lo < hi) {
-          const int mid = (lo + hi) >> 1;
-          if (s_rel[mid] <= e) lo = mid + 1; else hi = mid;
-        }
-        const int row = lo - 1;
-        const uint32_t j = e - s_rel[row];
-        r[u] = row0 + row;
-        uint32_t pick;
-        if (REPLACE) {
-          const uint32_t xv = a.replay ? a.replay[a.replay_ptr[r[u]] + j]
-                                       : draw_one(a.seed, kTagUniform, static_cast<uint64_t>(r[u]),
-                                                  static_cast<uint64_t>(j));
-          pick = xv % s_deg[row];
-        } else {
-          pick = s_pick[j * kPickStride + row];
-        }
-        q[u] = s_start[row] + pick;
-        v[u] = indices[q[u]];
-      }
+  for (int u = 0; u < 4; ++u) {
+    if (q[u] >= 0) {
+      const int64_t o = row_out + 4 * sub + u;
+      a.sub_indices[o] = v[u];
+      if (a.select_index) a.select_index[o] = q[u];
+      if (a.coo_col) a.coo_col[o] = static_cast<IdT>(my_row);
     }
-    if (base == threadIdx.x) GS_STAMP(6);  // first batch of gathers back
+  }
+  if (REPLACE) {
+    // further rounds of a fanout above 4 * G picks: 4 * G more outputs of the row each
+    for (int j0 = KMAX; j0 < cnt; j0 += KMAX) {
+      const int j = j0 + 4 * sub;
+      U4 blk;
+      if (rp_replace) {
 #pragma unroll
-    for (int u = 0; u < kFusedBatch; ++u) {
-      const uint32_t e = base + u * kFusedThreads;
-      if (q[u] >= 0) {
-        a.sub_indices[out0 + e] = v[u];
-        if (a.select_index) a.select_index[out0 + e] = q[u];
-        if (a.coo_col) a.coo_col[out0 + e] = static_cast<IdT>(r[u]);
+        for (int u = 0; u < 4; ++u) blk.v[u] = j + u < cnt ? rp_replace[j + u] : 0u;
+      } else {
+        blk = draw_block(a.seed, kTagUniform, static_cast<uint64_t>(my_row),
+                         static_cast<uint64_t>(j >> 2));
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (j + u < cnt) {
+          const int64_t p = start + blk.v[u] % static_cast<uint32_t>(deg);
+          const int64_t o = row_out + j + u;
+          a.sub_indices[o] = indices[p];
+          if (a.select_index) a.select_index[o] = p;
+          if (a.coo_col) a.coo_col[o] = static_cast<IdT>(my_row);
+        }
       }
     }
   }
-  GS_STAMP(7);  // stores done
-  GS_STAMP_END(1, 8);
+  GS_STAMP(6);  // stores done
+  GS_STAMP_END(1, 7);
+}
+
+template <typename IdT, int G, bool REPLACE>
+int sample_group_launch(const FusedArgs<IdT>& a, hipStream_t stream) {
+  const unsigned grid = static_cast<unsigned>(group_tiles(a.S, G));
+  if (a.S * G > kGroupSmallLanes)
+    hipLaunchKernelGGL((sample_group_kernel<IdT, G, REPLACE, kGroupThreadsLarge>), dim3(grid),
+                       dim3(kGroupThreadsLarge), 0, stream, a);
+  else
+    hipLaunchKernelGGL((sample_group_kernel<IdT, G, REPLACE, kGroupThreadsSmall>), dim3(grid),
+                       dim3(kGroupThreadsSmall), 0, stream, a);
+  return check_launch("sample_fused");
+}
+
+template <typename IdT, bool REPLACE>
+int sample_fused_dispatch(const FusedArgs<IdT>& a, hipStream_t stream) {
+  switch (group_lanes_for(a.k)) {
+    case 1: return sample_group_launch<IdT, 1, REPLACE>(a, stream);
+    case 2: return sample_group_launch<IdT, 2, REPLACE>(a, stream);
+    case 4: return sample_group_launch<IdT, 4, REPLACE>(a, stream);
+    default: return sample_group_launch<IdT, 8, REPLACE>(a, stream);
+  }
 }
 
 template <typename IdT>
 int sample_fused_launch(const FusedArgs<IdT>& a, bool replace, hipStream_t stream) {
-  const unsigned grid = static_cast<unsigned>((a.S + kFusedRows - 1) / kFusedRows);
   ProfileScope prof("sample_fused", stream);
-  if (replace) {
-    hipLaunchKernelGGL((sample_fused_kernel<IdT, 1, true>), dim3(grid), dim3(kFusedThreads), 0,
-                       stream, a);
-    return check_launch("sample_fused");
-  }
-  const size_t lds = static_cast<size_t>(a.k) * kPickStride * sizeof(uint32_t);
-  if (a.k <= 8)
-    hipLaunchKernelGGL((sample_fused_kernel<IdT, 8, false>), dim3(grid), dim3(kFusedThreads), lds,
-                       stream, a);
-  else if (a.k <= 16)
-    hipLaunchKernelGGL((sample_fused_kernel<IdT, 16, false>), dim3(grid), dim3(kFusedThreads), lds,
-                       stream, a);
-  else
-    hipLaunchKernelGGL((sample_fused_kernel<IdT, 32, false>), dim3(grid), dim3(kFusedThreads), lds,
-                       stream, a);
-  return check_launch("sample_fused");
+  return replace ? sample_fused_dispatch<IdT, true>(a, stream)
+                 : sample_fused_dispatch<IdT, false>(a, stream);
 }
 
 static __global__ void post_zero_kernel(int64_t* sub_indptr, gs_mailbox* box, int64_t ticket) {
@@ -781,7 +856,7 @@ static int sample_uniform_fill_t(const int64_t* indptr, int64_t num_cols, const 
 // for once per device (hipGetSymbolAddress) and kept.
 namespace gs {
 namespace {
-constexpr int64_t kStaticTiles = (GS_FUSED_STATIC_MAX_COLUMNS + kFusedRows - 1) / kFusedRows;
+constexpr int64_t kStaticTiles = (GS_FUSED_STATIC_MAX_COLUMNS * kGroupMaxLanes) / kGroupThreadsLarge + 1;
 constexpr size_t kStaticStateBytes = ((kStaticTiles * 8 + 255) / 256) * 256 + 256 + 256;
 constexpr int kMaxDevices = 64;
 
@@ -915,7 +990,7 @@ int gs_sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const void* 
 
 size_t gs_sample_fused_state_bytes(int64_t S) {
   const int64_t s = S < 0 ? 0 : S;
-  return lookback_state_bytes((s + kFusedRows - 1) / kFusedRows);
+  return lookback_state_bytes(group_tiles_bound(s));
 }
 
 int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void* indices,
@@ -955,7 +1030,8 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
   GS_REQUIRE(S * fanout <= static_cast<int64_t>(kLbValue),
              "gs_sample_uniform_fused: S * fanout exceeds 2^48");
   Carver ws(state, state_bytes);
-  LookbackState lb = carve_lookback(ws, (S + kFusedRows - 1) / kFusedRows, epoch);
+  // carved for the most tiles any fanout asks for, so that the size does not depend on it
+  LookbackState lb = carve_lookback(ws, group_tiles_bound(S), epoch);
   if (!ws.ok) {
     set_error_text("gs_sample_uniform_fused: state needs %zu bytes, 256-byte aligned",
                    gs_sample_fused_state_bytes(S));

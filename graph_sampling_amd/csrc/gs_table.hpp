@@ -160,7 +160,8 @@ inline void table_shape(T& t, int64_t cap) {
 // user, never as a whole, so its size costs nothing per call; it is kept four times
 // sparser than a one-call table (load <= 1/8): fewer than one insert in ten walks past its
 // home slot, and every such step is a round trip to memory that a whole wave waits for.
-inline int64_t linked_table_capacity(int64_t items) { return table_capacity(4 * items); }
+constexpr int64_t kLinkedFactor = 4;
+inline int64_t linked_table_capacity(int64_t items) { return table_capacity(kLinkedFactor * items); }
 
 // Laid out for the largest capacity the buffer can hold, used with the capacity the call
 // needs.  False when it does not fit.

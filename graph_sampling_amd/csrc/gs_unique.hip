@@ -1082,14 +1082,14 @@ int gs_relabel_table_init(void* table, size_t table_bytes, int id_bytes, void* s
   if (id_bytes == 4) {
     const int64_t cap = linked_table_slots<PackedTable>(table_bytes);
     PackedTable t;
-    GS_REQUIRE(cap > 0 && shape_linked_table<PackedTable>(table, table_bytes, cap / 8, &t),
+    GS_REQUIRE(cap > 0 && shape_linked_table<PackedTable>(table, table_bytes, cap / (2 * kLinkedFactor), &t),
                "gs_relabel_table_init: buffer too small or misaligned");
     hipLaunchKernelGGL(table_clear_kernel<PackedTable>, dim3(blocks_for(cap, kThreads)),
                        dim3(kThreads), 0, st, t, cap);
   } else {
     const int64_t cap = linked_table_slots<WideTable>(table_bytes);
     WideTable t;
-    GS_REQUIRE(cap > 0 && shape_linked_table<WideTable>(table, table_bytes, cap / 8, &t),
+    GS_REQUIRE(cap > 0 && shape_linked_table<WideTable>(table, table_bytes, cap / (2 * kLinkedFactor), &t),
                "gs_relabel_table_init: buffer too small or misaligned");
     hipLaunchKernelGGL(table_clear_kernel<WideTable>, dim3(blocks_for(cap, kThreads)),
                        dim3(kThreads), 0, st, t, cap);
