@@ -35,7 +35,8 @@ def lib():
                      "gs_coo2csc_workspace_bytes", "gs_col_row_slice_workspace_bytes",
                      "gs_index_search_workspace_bytes", "gs_relabel_table_bytes",
                      "gs_relabel_sampled_workspace_bytes", "gs_relabel_sampled_state_bytes",
-                     "gs_segment_workspace_bytes"):
+                     "gs_segment_workspace_bytes", "gs_layer_workspace_bytes",
+                     "gs_layer_sample_state_bytes", "gs_layer_relabel_state_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
     return _lib
@@ -350,6 +351,96 @@ def relabel_sampled(seed_keys, sub_indptr, sub_indices, table, mailbox=None, off
     if mailbox is not None:
         return frontier, num_unique, out_ids, ticket
     return frontier, num_unique, out_ids
+
+
+# ----------------------------------- a whole minibatch queued with no host read ----
+class LayerBuffers:
+    """What one layer of sample_layers owns: outputs at their bounds, device-side counts."""
+
+    def __init__(self, S_bound, fanout, id_dtype, device):
+        self.S_bound = int(S_bound)
+        self.fanout = int(fanout)
+        self.capacity = self.S_bound * self.fanout
+        self.sub_indptr = torch.empty(self.S_bound + 1, dtype=torch.int64, device=device)
+        self.sub_indices = torch.empty(self.capacity, dtype=id_dtype, device=device)
+        self.out_ids = torch.empty(self.capacity, dtype=id_dtype, device=device)
+        self.frontier = torch.empty(self.S_bound + self.capacity, dtype=id_dtype, device=device)
+        self.offsets_copy = torch.empty(self.S_bound + 1, dtype=torch.int64, device=device)
+        self.counts = torch.zeros(2, dtype=torch.int64, device=device)  # num_edges, num_unique
+        self.workspace = torch.empty(
+            int(lib().gs_layer_workspace_bytes(_i64(self.S_bound), _i64(self.fanout))),
+            dtype=torch.uint8, device=device)
+
+    def num_edges_ptr(self):
+        return ctypes.c_void_p(self.counts.data_ptr())
+
+    def num_unique_ptr(self):
+        return ctypes.c_void_p(self.counts.data_ptr() + 8)
+
+
+def sample_layers(indptr, indices, seeds, fanouts, replace=False, seed=0, mailbox=None,
+                  tables=None):
+    """gs_layer_sample + gs_layer_relabel for every layer of a minibatch, queued back to back:
+    layer l + 1 takes its column ids and their number from layer l's frontier and num_unique on
+    the device.  Layer l draws with seed + l.  Returns (layers: list of LayerBuffers, ticket of
+    the last relabel or None); sizes are the device-side counts of each layer."""
+    _need(indptr, torch.int64, "indptr")
+    idb = _ids(indices, "indices")
+    _ids(seeds, "seeds", like=indices)
+    dev = indptr.device
+    L = lib()
+    bounds = [seeds.numel()]
+    for k in fanouts:
+        bounds.append(bounds[-1] * (1 + int(k)))
+    layers = [LayerBuffers(bounds[l], k, indices.dtype, dev) for l, k in enumerate(fanouts)]
+    if tables is None:
+        tables = [RelabelTable(bounds[-1], torch.int32, dev) for _ in range(2)]
+    state_bytes = max(max(L.gs_layer_sample_state_bytes(_i64(b.S_bound)),
+                          L.gs_layer_relabel_state_bytes(_i64(b.S_bound), _i64(b.fanout)))
+                      for b in layers)
+    cols, S_dev = seeds, ctypes.c_void_p(0)
+    ticket = None
+    null = ctypes.c_void_p(0)
+    for l, b in enumerate(layers):
+        table = tables[l % 2]
+        state, epoch = fused_state(state_bytes, dev)
+        _check(L.gs_layer_sample(
+            _ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(cols), idb,
+            _i64(b.S_bound), S_dev, _i64(b.fanout), int(bool(replace)), _u64(seed + l), null, null,
+            _ptr(b.sub_indptr), _ptr(b.sub_indices), _i64(b.capacity), b.num_edges_ptr(),
+            _ptr(table.buf), ctypes.c_size_t(table.buf.numel()), _ptr(b.workspace),
+            ctypes.c_size_t(b.workspace.numel()), _ptr(state), ctypes.c_size_t(state.numel()),
+            ctypes.c_uint32(epoch), null, _i64(0), _stream(dev)), "gs_layer_sample")
+        state, epoch = fused_state(state_bytes, dev)
+        last = l == len(layers) - 1
+        box, ticket = null, None
+        if last and mailbox is not None:
+            ticket = mailbox.ticket()
+            box = mailbox.ptr()
+        prev = layers[l - 1] if l > 0 else None
+        prev_S_dev = null if l < 2 else layers[l - 2].num_unique_ptr()
+        _check(L.gs_layer_relabel(
+            idb, _i64(b.S_bound), S_dev, _i64(b.capacity), b.num_edges_ptr(), _ptr(b.sub_indptr),
+            _ptr(table.buf), ctypes.c_size_t(table.buf.numel()), _ptr(b.workspace),
+            ctypes.c_size_t(b.workspace.numel()), _ptr(b.frontier), _ptr(b.out_ids),
+            b.num_unique_ptr(), _ptr(b.offsets_copy), _ptr(state), ctypes.c_size_t(state.numel()),
+            ctypes.c_uint32(epoch),
+            _ptr(tables[(l - 1) % 2].buf) if prev else null,
+            ctypes.c_size_t(tables[(l - 1) % 2].buf.numel() if prev else 0),
+            _ptr(prev.workspace) if prev else null,
+            ctypes.c_size_t(prev.workspace.numel() if prev else 0),
+            _i64(prev.S_bound if prev else 0), prev_S_dev, _i64(prev.capacity if prev else 0),
+            prev.num_edges_ptr() if prev else null, box, _i64(ticket or 0), _stream(dev)),
+            "gs_layer_relabel")
+        cols, S_dev = b.frontier, b.num_unique_ptr()
+    b = layers[-1]
+    _check(L.gs_layer_table_sweep(
+        _ptr(tables[(len(layers) - 1) % 2].buf),
+        ctypes.c_size_t(tables[(len(layers) - 1) % 2].buf.numel()), _ptr(b.workspace),
+        ctypes.c_size_t(b.workspace.numel()), _i64(b.S_bound),
+        null if len(layers) < 2 else layers[-2].num_unique_ptr(), _i64(b.capacity),
+        b.num_edges_ptr(), _stream(dev)), "gs_layer_table_sweep")
+    return layers, ticket
 
 
 def sample_one_keepdim(indptr, indices, column_ids, seed=0, replay=None):

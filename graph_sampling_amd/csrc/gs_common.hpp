@@ -477,18 +477,53 @@ __device__ __forceinline__ void lb_store(unsigned long long* p, unsigned long lo
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// A tile gives up: the error word is raised and made visible to the whole device before
+// anything the tile publishes afterwards (the one place that pays for a device-scope fence).
+__device__ __forceinline__ void lookback_raise(const LookbackState& st) {
+  __hip_atomic_store(st.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+}
+
 // Any one thread: makes the tile's own sum visible to its successors.  Call it as
 // early as possible; whatever the tile does between this and the walk below
 // gives its predecessors time to publish theirs.
+// may_close = false: tile 0 too publishes its sum as a sum only (for callers that close their
+// tiles themselves, later, with lookback_publish_inclusive).
 __device__ __forceinline__ void lookback_publish_sum(const LookbackState& st, unsigned int tile,
-                                                     int64_t total) {
-  lb_store(&st.status[tile], lb_word(tile == 0 ? 2u : 1u, st.epoch, total));
+                                                     int64_t total, bool may_close = true) {
+  lb_store(&st.status[tile], lb_word(tile == 0 && may_close ? 2u : 1u, st.epoch, total));
+}
+
+// Any one thread: closes the tile (its inclusive prefix).  Only for callers that asked
+// lookback_exclusive_prefix not to do it, because something else of the tile has to be
+// complete first.
+__device__ __forceinline__ void lookback_publish_inclusive(const LookbackState& st,
+                                                           unsigned int tile, int64_t inclusive) {
+  lb_store(&st.status[tile], lb_word(2u, st.epoch, inclusive));
+}
+
+// A closed tile's inclusive prefix, for readers other than the look-back itself: waits (with
+// the same bound) until `tile` is closed.  Returns 0 after giving up, with *st.error raised.
+__device__ __forceinline__ int64_t lookback_wait_inclusive(const LookbackState& st,
+                                                           unsigned long long seen,
+                                                           unsigned int tile) {
+  int polls = 0;
+  while (lb_flag(seen, st.epoch) != 2u) {
+    if (++polls > kLookbackSpinLimit) {
+      lookback_raise(st);
+      return 0;
+    }
+    if (polls > 16) __builtin_amdgcn_s_sleep(32);
+    seen = lb_load(&st.status[tile]);
+  }
+  return static_cast<int64_t>(seen & kLbValue);
 }
 
 // Call with all 64 lanes of wave 0, after lookback_publish_sum.  Returns the sum
-// of all earlier tiles and publishes the tile's inclusive prefix.
+// of all earlier tiles and (unless publish is false) publishes the tile's inclusive prefix.
 __device__ __forceinline__ int64_t lookback_exclusive_prefix(const LookbackState& st,
-                                                             unsigned int tile, int64_t total) {
+                                                             unsigned int tile, int64_t total,
+                                                             bool publish = true) {
   const int lane = threadIdx.x & (kWave - 1);
   if (tile == 0) return 0;
   const unsigned long long before_first = lb_word(2u, st.epoch, 0);  // "tile -1": inclusive 0
@@ -510,7 +545,7 @@ __device__ __forceinline__ int64_t lookback_exclusive_prefix(const LookbackState
         int polls = 0;
         while (lb_flag(s[w], st.epoch) == 0) {
           if (++polls > kLookbackSpinLimit) {
-            __hip_atomic_store(st.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lookback_raise(st);
             s[w] = before_first;
             break;
           }
@@ -531,7 +566,7 @@ __device__ __forceinline__ int64_t lookback_exclusive_prefix(const LookbackState
   }
   // (an error raised above was stored with device scope before this point)
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  if (lane == 0) lb_store(&st.status[tile], lb_word(2u, st.epoch, running + total));
+  if (publish && lane == 0) lb_store(&st.status[tile], lb_word(2u, st.epoch, running + total));
   return running;
 }
 

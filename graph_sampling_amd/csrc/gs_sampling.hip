@@ -25,6 +25,8 @@
 
 #include <mutex>
 
+#include "gs_table.hpp"
+
 GS_STAMPS_DEFINE(sampling)
 
 namespace gs {
@@ -551,16 +553,24 @@ constexpr int kGroupMaxLanes = 8;
 inline int group_lanes_for(int64_t fanout) {
   return fanout <= 4 ? 1 : (fanout <= 8 ? 2 : (fanout <= 16 ? 4 : 8));
 }
+// A linked launch is sized for a bound on the columns, of which the live ones are usually
+// a fraction: it keeps the small tiles up to a larger bound (workgroups beyond the count
+// leave at once and take no part in the look-back).
+constexpr int64_t kGroupSmallLanesLinked = int64_t(1) << 21;
+inline int group_tile_threads(int64_t S, int G, bool linked) {
+  return S * G > (linked ? kGroupSmallLanesLinked : kGroupSmallLanes) ? kGroupThreadsLarge
+                                                                      : kGroupThreadsSmall;
+}
 // tiles of the launch that samples S columns with G lanes each
-inline int64_t group_tiles(int64_t S, int G) {
-  const int64_t threads = S * G > kGroupSmallLanes ? kGroupThreadsLarge : kGroupThreadsSmall;
-  const int64_t rows = threads / G;
-  return (S + rows - 1) / rows;
+inline int64_t group_tiles(int64_t S, int G, bool linked) {
+  const int64_t rows = group_tile_threads(S, G, linked) / G;
+  const int64_t tiles = (S + rows - 1) / rows;
+  return tiles > 0 ? tiles : 1;
 }
 // most tiles any fanout can ask for
-inline int64_t group_tiles_bound(int64_t S) {
+inline int64_t group_tiles_bound(int64_t S, bool linked) {
   const int64_t large = (S * kGroupMaxLanes + kGroupThreadsLarge - 1) / kGroupThreadsLarge;
-  const int64_t small = kGroupSmallLanes / kGroupThreadsSmall;
+  const int64_t small = (linked ? kGroupSmallLanesLinked : kGroupSmallLanes) / kGroupThreadsSmall;
   return (large > small ? large : small) + 1;
 }
 
@@ -582,7 +592,27 @@ struct FusedArgs {
   LookbackState lb;
   gs_mailbox* box;
   int64_t box_ticket;
+  // LINKED kernels only (gs_layer_sample): the number of columns may live on the device (S is
+  // then the bound the launch and the buffers are sized for), and every seed and every
+  // sampled id is entered into the hash table of the relabel that follows: item r < S is
+  // seed r, item S + e is output e; pos[item] = its slot; *num_edges = the total
+  const int64_t* S_dev;
+  PackedTable table;
+  uint32_t* pos;
+  int64_t* num_edges;
 };
+
+// Enters `key` as item `item` (one compare-and-swap in the common case); the slot goes to pos.
+template <typename IdT>
+__device__ __forceinline__ void linked_insert(const PackedTable& t, IdT key, int64_t item,
+                                              uint32_t* __restrict__ pos, unsigned int* too_wide) {
+  if (sizeof(IdT) == 8 && (static_cast<unsigned long long>(key) >> 32) != 0ull) {
+    *too_wide = 2u;  // a 64-bit id that does not fit the one-word slots: reported as -2
+    pos[item] = 0u;
+    return;
+  }
+  pos[item] = t.template insert<false>(static_cast<long long>(key), static_cast<uint32_t>(item));
+}
 
 // the value lane `owner` of every G-lane group holds (owner is a constant after unrolling)
 template <int G>
@@ -604,14 +634,14 @@ __device__ __forceinline__ uint32_t group_broadcast(uint32_t v, int owner) {
   return static_cast<uint32_t>(__shfl(x, ((threadIdx.x & (kWave - 1)) & ~(G - 1)) | owner, kWave));
 }
 
-template <typename IdT, int G, bool REPLACE, int THREADS>
+template <typename IdT, int G, bool REPLACE, int THREADS, bool LINKED>
 __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a) {
   constexpr int kRows = THREADS / G;
   constexpr int KMAX = 4 * G;
   __shared__ int64_t s_scan[THREADS / kWave + 1];
   __shared__ int64_t s_prefix;
   const unsigned int tile = blockIdx.x;
-  const unsigned int tiles = gridDim.x;
+  unsigned int tiles = gridDim.x;
   const int sub = threadIdx.x & (G - 1);
   const int64_t my_row = static_cast<int64_t>(tile) * kRows + threadIdx.x / G;
   const int k = static_cast<int>(a.k);
@@ -619,15 +649,27 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
   GS_STAMP(0);
 
   // ---- 1. the row's column and offsets
+  // (with a device-side column count the reads below go by the bound, under which every
+  // buffer is sized, and do not wait for the count; what lies beyond it is masked afterwards)
   int64_t start = 0, deg = 0, cnt = 0;
+  int64_t c = -1;
   if (my_row < a.S) {
-    const int64_t c = a.cols ? static_cast<int64_t>(a.cols[my_row]) : my_row;
+    c = a.cols ? static_cast<int64_t>(a.cols[my_row]) : my_row;
     if (valid_col(c, a.num_cols)) {
       start = a.indptr[c];
       deg = a.indptr[c + 1] - start;
     }
-    cnt = REPLACE ? (deg > 0 ? a.k : 0) : (deg < a.k ? deg : a.k);
   }
+  int64_t S = a.S;
+  if (LINKED && a.S_dev) {
+    const int64_t s_dev = *a.S_dev;
+    S = s_dev < 0 ? 0 : (s_dev < a.S ? s_dev : a.S);
+    const int64_t live = (S + kRows - 1) / kRows;
+    tiles = static_cast<unsigned int>(live > 0 ? live : 1);
+    if (tile >= tiles) return;  // the whole workgroup: nothing of it is below the count
+    if (my_row >= S) deg = 0;
+  }
+  cnt = REPLACE ? (deg > 0 ? a.k : 0) : (deg < a.k ? deg : a.k);
   GS_STAMP(1);  // column id and offsets are here
   int64_t tile_total;
   const int64_t ex = block_exclusive_scan<THREADS>(sub == 0 ? cnt : 0, &tile_total, s_scan);
@@ -710,11 +752,13 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
   __syncthreads();
   const int64_t out0 = s_prefix;
   GS_STAMP(5);  // the tile's offset is known to every wave, the first gathers are back
-  if (my_row < a.S && sub == 0) a.sub_indptr[my_row] = out0 + local;
+  if (my_row < S && sub == 0) a.sub_indptr[my_row] = out0 + local;
   if (tile == tiles - 1 && threadIdx.x == 0) {
     int64_t total = out0 + tile_total;
-    if (__hip_atomic_load(a.lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) total = -1;
-    a.sub_indptr[a.S] = total;
+    if (!LINKED && __hip_atomic_load(a.lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+      total = -1;  // (a linked launch leaves the verdict to the relabel behind it)
+    a.sub_indptr[S] = total;
+    if (LINKED) *a.num_edges = total;
     post_mailbox(a.box, total, a.box_ticket);
   }
   const int64_t row_out = out0 + local;
@@ -725,6 +769,55 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
       a.sub_indices[o] = v[u];
       if (a.select_index) a.select_index[o] = q[u];
       if (a.coo_col) a.coo_col[o] = static_cast<IdT>(my_row);
+    }
+  }
+  if (LINKED) {
+    // the compare-and-swaps of a lane (its four outputs; the row's first lane also enters the
+    // seed) go out together; what they found is looked at after
+    uint32_t p[4], seed_p = 0u;
+    unsigned long long prev[4], seed_prev = 0ull;
+    bool seed_live = sub == 0 && my_row < S;
+    if (seed_live) {
+      if (sizeof(IdT) == 8 && (static_cast<unsigned long long>(c) >> 32) != 0ull) {
+        *a.lb.error = 2u;
+        a.pos[my_row] = 0u;
+        seed_live = false;
+      } else {
+        seed_p = a.table.home(c);
+        seed_prev = a.table.probe(c, static_cast<uint32_t>(my_row), seed_p);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (q[u] >= 0) {
+        if (sizeof(IdT) == 8 && (static_cast<unsigned long long>(v[u]) >> 32) != 0ull) {
+          *a.lb.error = 2u;
+          a.pos[S + row_out + 4 * sub + u] = 0u;
+          q[u] = -1;
+        } else {
+          p[u] = a.table.home(static_cast<long long>(v[u]));
+          prev[u] = a.table.probe(static_cast<long long>(v[u]),
+                                  static_cast<uint32_t>(S + row_out + 4 * sub + u), p[u]);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (q[u] >= 0) {
+        const uint32_t item = static_cast<uint32_t>(S + row_out + 4 * sub + u);
+        while (!a.table.landed(static_cast<long long>(v[u]), item, p[u], prev[u])) {
+          p[u] = (p[u] + 1) & a.table.mask;
+          prev[u] = a.table.probe(static_cast<long long>(v[u]), item, p[u]);
+        }
+        a.pos[item] = p[u];
+      }
+    }
+    if (seed_live) {
+      while (!a.table.landed(c, static_cast<uint32_t>(my_row), seed_p, seed_prev)) {
+        seed_p = (seed_p + 1) & a.table.mask;
+        seed_prev = a.table.probe(c, static_cast<uint32_t>(my_row), seed_p);
+      }
+      a.pos[my_row] = seed_p;
     }
   }
   if (REPLACE) {
@@ -744,9 +837,11 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
         if (j + u < cnt) {
           const int64_t p = start + blk.v[u] % static_cast<uint32_t>(deg);
           const int64_t o = row_out + j + u;
-          a.sub_indices[o] = indices[p];
+          const IdT got = indices[p];
+          a.sub_indices[o] = got;
           if (a.select_index) a.select_index[o] = p;
           if (a.coo_col) a.coo_col[o] = static_cast<IdT>(my_row);
+          if (LINKED) linked_insert<IdT>(a.table, got, S + o, a.pos, a.lb.error);
         }
       }
     }
@@ -755,33 +850,36 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
   GS_STAMP_END(1, 7);
 }
 
-template <typename IdT, int G, bool REPLACE>
+template <typename IdT, int G, bool REPLACE, bool LINKED>
 int sample_group_launch(const FusedArgs<IdT>& a, hipStream_t stream) {
-  const unsigned grid = static_cast<unsigned>(group_tiles(a.S, G));
-  if (a.S * G > kGroupSmallLanes)
-    hipLaunchKernelGGL((sample_group_kernel<IdT, G, REPLACE, kGroupThreadsLarge>), dim3(grid),
-                       dim3(kGroupThreadsLarge), 0, stream, a);
+  const unsigned grid = static_cast<unsigned>(group_tiles(a.S, G, LINKED));
+  if (group_tile_threads(a.S, G, LINKED) == kGroupThreadsLarge)
+    hipLaunchKernelGGL((sample_group_kernel<IdT, G, REPLACE, kGroupThreadsLarge, LINKED>),
+                       dim3(grid), dim3(kGroupThreadsLarge), 0, stream, a);
   else
-    hipLaunchKernelGGL((sample_group_kernel<IdT, G, REPLACE, kGroupThreadsSmall>), dim3(grid),
-                       dim3(kGroupThreadsSmall), 0, stream, a);
+    hipLaunchKernelGGL((sample_group_kernel<IdT, G, REPLACE, kGroupThreadsSmall, LINKED>),
+                       dim3(grid), dim3(kGroupThreadsSmall), 0, stream, a);
   return check_launch("sample_fused");
 }
 
-template <typename IdT, bool REPLACE>
+template <typename IdT, bool REPLACE, bool LINKED>
 int sample_fused_dispatch(const FusedArgs<IdT>& a, hipStream_t stream) {
   switch (group_lanes_for(a.k)) {
-    case 1: return sample_group_launch<IdT, 1, REPLACE>(a, stream);
-    case 2: return sample_group_launch<IdT, 2, REPLACE>(a, stream);
-    case 4: return sample_group_launch<IdT, 4, REPLACE>(a, stream);
-    default: return sample_group_launch<IdT, 8, REPLACE>(a, stream);
+    case 1: return sample_group_launch<IdT, 1, REPLACE, LINKED>(a, stream);
+    case 2: return sample_group_launch<IdT, 2, REPLACE, LINKED>(a, stream);
+    case 4: return sample_group_launch<IdT, 4, REPLACE, LINKED>(a, stream);
+    default: return sample_group_launch<IdT, 8, REPLACE, LINKED>(a, stream);
   }
 }
 
 template <typename IdT>
-int sample_fused_launch(const FusedArgs<IdT>& a, bool replace, hipStream_t stream) {
-  ProfileScope prof("sample_fused", stream);
-  return replace ? sample_fused_dispatch<IdT, true>(a, stream)
-                 : sample_fused_dispatch<IdT, false>(a, stream);
+int sample_fused_launch(const FusedArgs<IdT>& a, bool replace, bool linked, hipStream_t stream) {
+  ProfileScope prof(linked ? "layer_sample" : "sample_fused", stream);
+  if (linked)
+    return replace ? sample_fused_dispatch<IdT, true, true>(a, stream)
+                   : sample_fused_dispatch<IdT, false, true>(a, stream);
+  return replace ? sample_fused_dispatch<IdT, true, false>(a, stream)
+                 : sample_fused_dispatch<IdT, false, false>(a, stream);
 }
 
 static __global__ void post_zero_kernel(int64_t* sub_indptr, gs_mailbox* box, int64_t ticket) {
@@ -796,7 +894,9 @@ int sample_fused_t(const int64_t* indptr, int64_t num_cols, const void* indices,
                    const void* column_ids, int64_t S, int64_t fanout, int replace, uint64_t seed,
                    const uint32_t* replay, const int64_t* replay_ptr, int64_t* sub_indptr,
                    void* sub_indices, int64_t* select_index, void* coo_col, LookbackState lb,
-                   gs_mailbox* box, int64_t ticket, hipStream_t st) {
+                   gs_mailbox* box, int64_t ticket, hipStream_t st, bool linked = false,
+                   const int64_t* S_dev = nullptr, PackedTable table = PackedTable(),
+                   uint32_t* pos = nullptr, int64_t* num_edges = nullptr) {
   FusedArgs<IdT> a{indptr,
                    static_cast<const IdT*>(indices),
                    static_cast<const IdT*>(column_ids),
@@ -812,8 +912,12 @@ int sample_fused_t(const int64_t* indptr, int64_t num_cols, const void* indices,
                    static_cast<IdT*>(coo_col),
                    lb,
                    box,
-                   ticket};
-  return sample_fused_launch<IdT>(a, replace != 0, st);
+                   ticket,
+                   S_dev,
+                   table,
+                   pos,
+                   num_edges};
+  return sample_fused_launch<IdT>(a, replace != 0, linked, st);
 }
 
 }  // namespace
@@ -856,7 +960,7 @@ static int sample_uniform_fill_t(const int64_t* indptr, int64_t num_cols, const 
 // for once per device (hipGetSymbolAddress) and kept.
 namespace gs {
 namespace {
-constexpr int64_t kStaticTiles = (GS_FUSED_STATIC_MAX_COLUMNS * kGroupMaxLanes) / kGroupThreadsLarge + 1;
+constexpr int64_t kStaticTiles = (GS_FUSED_STATIC_MAX_COLUMNS * kGroupMaxLanes) / kGroupThreadsLarge + 1;  // = group_tiles_bound of the maximum
 constexpr size_t kStaticStateBytes = ((kStaticTiles * 8 + 255) / 256) * 256 + 256 + 256;
 constexpr int kMaxDevices = 64;
 
@@ -990,7 +1094,7 @@ int gs_sample_uniform_fill(const int64_t* indptr, int64_t num_cols, const void* 
 
 size_t gs_sample_fused_state_bytes(int64_t S) {
   const int64_t s = S < 0 ? 0 : S;
-  return lookback_state_bytes(group_tiles_bound(s));
+  return lookback_state_bytes(group_tiles_bound(s, false));
 }
 
 int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void* indices,
@@ -1031,7 +1135,7 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
              "gs_sample_uniform_fused: S * fanout exceeds 2^48");
   Carver ws(state, state_bytes);
   // carved for the most tiles any fanout asks for, so that the size does not depend on it
-  LookbackState lb = carve_lookback(ws, group_tiles_bound(S), epoch);
+  LookbackState lb = carve_lookback(ws, group_tiles_bound(S, false), epoch);
   if (!ws.ok) {
     set_error_text("gs_sample_uniform_fused: state needs %zu bytes, 256-byte aligned",
                    gs_sample_fused_state_bytes(S));
@@ -1044,6 +1148,68 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
              : sample_fused_t<int32_t>(indptr, num_cols, indices, column_ids, S, fanout, replace,
                                        seed, replay, replay_ptr, sub_indptr, sub_indices,
                                        select_index, coo_col, lb, mailbox, mailbox_ticket, st);
+}
+
+size_t gs_layer_sample_state_bytes(int64_t S_bound) {
+  return lookback_state_bytes(group_tiles_bound(S_bound < 0 ? 0 : S_bound, true));
+}
+
+int gs_layer_sample(const int64_t* indptr, int64_t num_cols, const void* indices,
+                    const void* column_ids, int id_bytes, int64_t S_bound, const int64_t* S_dev,
+                    int64_t fanout, int replace, uint64_t seed, const uint32_t* replay,
+                    const int64_t* replay_ptr, int64_t* sub_indptr, void* sub_indices,
+                    int64_t capacity, int64_t* num_edges, void* table, size_t table_bytes,
+                    void* workspace, size_t workspace_bytes, void* state, size_t state_bytes,
+                    uint32_t epoch, gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream) {
+  GS_REQUIRE(indptr && sub_indptr && num_edges && table && workspace && state && S_bound >= 0 &&
+                 fanout >= 0 && num_cols >= 0,
+             "gs_layer_sample: null pointer or negative size");
+  GS_REQUIRE(S_bound == 0 || column_ids, "gs_layer_sample: column_ids is null");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_layer_sample: id_bytes must be 4 or 8, got %d", id_bytes);
+  GS_REQUIRE((replay == nullptr) == (replay_ptr == nullptr),
+             "gs_layer_sample: replay and replay_ptr must be given together");
+  if (!replace && fanout > GS_FUSED_MAX_FANOUT) {
+    set_error_text("gs_layer_sample: fanout %lld without replacement exceeds %d",
+                   static_cast<long long>(fanout), GS_FUSED_MAX_FANOUT);
+    return GS_ERR_UNSUPPORTED;
+  }
+  GS_REQUIRE(capacity >= S_bound * fanout,
+             "gs_layer_sample: outputs must hold S_bound * fanout = %lld entries, capacity is %lld",
+             static_cast<long long>(S_bound * fanout), static_cast<long long>(capacity));
+  GS_REQUIRE(S_bound == 0 || fanout == 0 || (indices && sub_indices), "gs_layer_sample: null buffer");
+  GS_REQUIRE(epoch >= 1 && epoch <= kLbMaxEpoch, "gs_layer_sample: epoch must be 1..%u, got %u",
+             kLbMaxEpoch, epoch);
+  const int64_t M_bound = S_bound + capacity;
+  if (M_bound >= (int64_t(1) << 31)) {
+    set_error_text("gs_layer_sample: %lld items exceed the supported 2^31",
+                   static_cast<long long>(M_bound));
+    return GS_ERR_UNSUPPORTED;
+  }
+  PackedTable t;
+  if (!shape_linked_table<PackedTable>(table, table_bytes, M_bound, &t)) {
+    set_error_text("gs_layer_sample: the table holds fewer than the %lld slots this call needs "
+                   "(or is misaligned)",
+                   static_cast<long long>(linked_table_capacity(M_bound)));
+    return GS_ERR_WORKSPACE;
+  }
+  uint32_t* pos = nullptr;
+  Carver ws(state, state_bytes);
+  LookbackState lb = carve_lookback(ws, group_tiles_bound(S_bound, true), epoch);
+  if (!carve_layer_workspace(workspace, workspace_bytes, M_bound, &pos) || !ws.ok) {
+    set_error_text("gs_layer_sample: workspace needs %zu bytes and state %zu bytes, 256-byte aligned",
+                   layer_workspace_bytes(M_bound), gs_layer_sample_state_bytes(S_bound));
+    return GS_ERR_WORKSPACE;
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return id_bytes == 8
+             ? sample_fused_t<int64_t>(indptr, num_cols, indices, column_ids, S_bound, fanout,
+                                       replace, seed, replay, replay_ptr, sub_indptr, sub_indices,
+                                       nullptr, nullptr, lb, mailbox, mailbox_ticket, st, true,
+                                       S_dev, t, pos, num_edges)
+             : sample_fused_t<int32_t>(indptr, num_cols, indices, column_ids, S_bound, fanout,
+                                       replace, seed, replay, replay_ptr, sub_indptr, sub_indices,
+                                       nullptr, nullptr, lb, mailbox, mailbox_ticket, st, true,
+                                       S_dev, t, pos, num_edges);
 }
 
 int gs_sample_uniform_fused_static(const int64_t* indptr, int64_t num_cols, const void* indices,

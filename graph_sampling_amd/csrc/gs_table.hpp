@@ -179,6 +179,19 @@ inline bool shape_linked_table(void* buffer, size_t bytes, int64_t items, T* t) 
   return true;
 }
 
+// Workspace a layer's two launches share (gs_layer_sample, gs_layer_relabel): the slot of
+// every item.
+inline size_t layer_workspace_bytes(int64_t items) {
+  if (items < 1) items = 1;
+  return padded(static_cast<size_t>(items) * 4);
+}
+inline bool carve_layer_workspace(void* workspace, size_t bytes, int64_t items, uint32_t** pos) {
+  if (items < 1) items = 1;
+  Carver ws(workspace, bytes);
+  *pos = ws.take<uint32_t>(static_cast<size_t>(items));
+  return ws.ok;
+}
+
 template <typename T>
 inline int64_t linked_table_slots(size_t bytes) {
   int64_t cap_max = 1024;

@@ -485,6 +485,220 @@ int relabel_sampled_impl(const void* seed_keys, int64_t S, const void* sampled, 
   return check_launch("relabel_sampled");
 }
 
+// ------------------------------------------- the relabel of gs_layer_relabel ----
+// Second launch of a layer whose first (gs_layer_sample) has already entered every seed and
+// every sampled id into the table: flags, their scan, the frontier AND the renaming of the
+// sampled ids in one kernel.  The rank of a key is the rank of its first occurrence f, and
+// f <= i for every item i that carries the key, so an item only ever needs results of its own
+// or of EARLIER tiles -- the same dependence the look-back has:
+//  * a tile stores, for each of its first occurrences, how far it stands from the tile's end
+//    (12 bits per item, four items to a 64-bit word, the launch's epoch above them: a word
+//    says by itself whether it is this launch's), then closes itself (inclusive prefix);
+//  * rank(f) = inclusive prefix of f's tile - that distance: two reads in flight together for
+//    an f of another tile, each polled until it is this launch's (bounded like the
+//    look-back's waits), LDS for an f of the same tile.
+// The key of an item is the upper half of its slot's word, so neither the seeds nor the
+// sampled ids are read again.  The table is NOT emptied here (a later tile may still have to
+// read a slot): the caller names it as `prev` in its next gs_layer_relabel on ANOTHER table,
+// or sweeps it with gs_layer_table_sweep.
+struct RankCounts {
+  int64_t S_bound;
+  const int64_t* S_dev;
+  int64_t cap;
+  const int64_t* E_dev;
+  __device__ __forceinline__ void get(int64_t* S, int64_t* M) const {
+    int64_t s = S_bound;
+    if (S_dev) {
+      s = *S_dev;
+      s = s < 0 ? 0 : (s < S_bound ? s : S_bound);
+    }
+    int64_t e = *E_dev;
+    e = e < 0 ? 0 : (e < cap ? e : cap);
+    *S = s;
+    *M = s + e;
+  }
+};
+
+template <typename IdT>
+struct RankArgs {
+  PackedTable t;
+  const uint32_t* pos;
+  RankCounts n;
+  unsigned long long* back;  // one 64-bit word per four items, in the look-back state
+  IdT* frontier;
+  IdT* out_ids;
+  int64_t* num_unique;
+  const int64_t* offsets;  // the sampler's offsets (S + 1 of them), copied to offsets_copy
+  int64_t* offsets_copy;
+  LookbackState lb;
+  gs_mailbox* box;
+  int64_t box_ticket;
+  // the table of an earlier layer, emptied on the side
+  PackedTable prev_t;
+  const uint32_t* prev_pos;
+  RankCounts prev_n;
+};
+
+// distances of a tile's first occurrences from its end: 1..2048, four to a word under the epoch
+constexpr int kBackBits = 12;
+constexpr unsigned long long kBackMask = (1ull << kBackBits) - 1;
+constexpr int kBackEpochShift = 48;
+static_assert(kCompactTile < (1 << kBackBits), "a distance must fit its field");
+
+// the word of four items once its tile has stored it in this launch (0 after giving up, with
+// the error raised)
+__device__ __forceinline__ unsigned long long back_wait(const LookbackState& st,
+                                                        const unsigned long long* back,
+                                                        unsigned long long seen, uint32_t at) {
+  int polls = 0;
+  while (((seen >> kBackEpochShift) & kLbMaxEpoch) != st.epoch) {
+    if (++polls > kLookbackSpinLimit) {
+      lookback_raise(st);
+      return 0ull;
+    }
+    if (polls > 16) __builtin_amdgcn_s_sleep(32);
+    seen = lb_load(&back[at]);
+  }
+  return seen;
+}
+
+template <typename IdT>
+__global__ void __launch_bounds__(kThreads) rank_linked_kernel(RankArgs<IdT> a) {
+  __shared__ int64_t s_scan[kThreads / kWave + 1];
+  __shared__ int64_t s_prefix;
+  __shared__ unsigned short s_back[kCompactTile];
+  GS_STAMP_BEGIN();
+  GS_STAMP(0);
+  const unsigned int tile = blockIdx.x;
+  const int64_t M_bound = a.n.S_bound + a.n.cap;
+  const int64_t base = static_cast<int64_t>(tile) * kCompactTile +
+                       static_cast<int64_t>(threadIdx.x) * kCompactItems;
+  // slot numbers go by the bound (the array is sized for it), so that they are on their way
+  // together with the counts
+  uint32_t at[kCompactItems];
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) at[k] = base + k < M_bound ? a.pos[base + k] : 0u;
+  int64_t S, M;
+  a.n.get(&S, &M);
+  const int64_t live = (M + kCompactTile - 1) / kCompactTile;
+  const unsigned int tiles = static_cast<unsigned int>(live > 0 ? live : 1);
+  if (tile >= tiles) return;
+  GS_STAMP(1);  // slot numbers and counts are here
+  unsigned long long w[kCompactItems];
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k)
+    w[k] = base + k < M ? a.t.slots[at[k] & a.t.mask] : ~0ull;
+  bool first[kCompactItems];
+  int64_t mine = 0;
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) {
+    first[k] = base + k < M && static_cast<uint32_t>(w[k]) == static_cast<uint32_t>(base + k);
+    mine += first[k] ? 1 : 0;
+  }
+  GS_STAMP(2);  // the slots' words are here
+  int64_t tile_total;
+  const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
+  if (threadIdx.x == 0) lookback_publish_sum(a.lb, tile, tile_total, /*may_close=*/false);
+  // distance of every first occurrence from the tile's end: to LDS for this tile's own
+  // lookups, to memory (device-scope stores, four items a word) for those of later tiles
+  {
+    const unsigned long long tag = static_cast<unsigned long long>(a.lb.epoch) << kBackEpochShift;
+    unsigned long long word[2] = {tag, tag};
+    int64_t run = local;
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+      const unsigned int d = first[k] ? static_cast<unsigned int>(tile_total - run) : 0u;
+      s_back[threadIdx.x * kCompactItems + k] = static_cast<unsigned short>(d);
+      word[k >> 2] |= static_cast<unsigned long long>(d) << (kBackBits * (k & 3));
+      run += first[k] ? 1 : 0;
+    }
+    if (base < M) lb_store(&a.back[base >> 2], word[0]);
+    if (base + 4 < M) lb_store(&a.back[(base >> 2) + 1], word[1]);
+  }
+  GS_STAMP(3);  // flags scanned, sum published, distances stored
+  if (threadIdx.x < kWave) {
+    const int64_t before = lookback_exclusive_prefix(a.lb, tile, tile_total, /*publish=*/false);
+    if (threadIdx.x == 0) s_prefix = before;
+  }
+  GS_STAMP(4);  // look-back done
+  // every wave's distance stores have completed before the tile closes
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  const int64_t tile_excl = s_prefix;
+  const int64_t tile_incl = tile_excl + tile_total;
+  if (threadIdx.x == 0) lookback_publish_inclusive(a.lb, tile, tile_incl);
+  GS_STAMP(5);
+  // lookups of the sampled ids: both reads of every item first, the waits after
+  unsigned long long bw[kCompactItems], st[kCompactItems];
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) {
+    const int64_t i = base + k;
+    const uint32_t f = static_cast<uint32_t>(w[k]);
+    bw[k] = 0ull;
+    st[k] = 0ull;
+    if (i >= S && i < M && (f >> 11) != tile && f < i) {
+      bw[k] = lb_load(&a.back[f >> 2]);
+      st[k] = lb_load(&a.lb.status[f >> 11]);
+    }
+  }
+  {
+    int64_t run = tile_excl + local;
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+      if (first[k]) a.frontier[run] = static_cast<IdT>(w[k] >> 32);
+      run += first[k] ? 1 : 0;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) {
+    const int64_t i = base + k;
+    if (i >= S && i < M) {
+      const uint32_t f = static_cast<uint32_t>(w[k]);
+      int64_t rank = -1;
+      if (f <= static_cast<uint32_t>(i)) {  // (anything else: the insert pass gave up on this id)
+        if ((f >> 11) == tile) {
+          rank = tile_incl - s_back[f & (kCompactTile - 1)];
+        } else {
+          const int64_t incl = lookback_wait_inclusive(a.lb, st[k], f >> 11);
+          const unsigned long long b = back_wait(a.lb, a.back, bw[k], f >> 2);
+          rank = incl - static_cast<int64_t>((b >> (kBackBits * (f & 3))) & kBackMask);
+        }
+      }
+      a.out_ids[i - S] = static_cast<IdT>(rank);
+    }
+  }
+  if (a.offsets_copy) {
+    const int64_t g = static_cast<int64_t>(tile) * kThreads + threadIdx.x;
+    for (int64_t r = g; r <= S; r += static_cast<int64_t>(tiles) * kThreads)
+      a.offsets_copy[r] = a.offsets[r];
+  }
+  if (tile == tiles - 1 && threadIdx.x == 0) {
+    int64_t total = tile_incl;
+    const unsigned int err = __hip_atomic_load(a.lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (err) total = err == 2u ? -2 : -1;  // 2: a key did not fit the one-word slots
+    *a.num_unique = total;
+    post_mailbox(a.box, total, a.box_ticket);
+  }
+  if (a.prev_pos) {
+    int64_t pS, pM;
+    a.prev_n.get(&pS, &pM);
+    const int64_t g = static_cast<int64_t>(tile) * kThreads + threadIdx.x;
+    for (int64_t j = g; j < pM; j += static_cast<int64_t>(tiles) * kThreads)
+      a.prev_t.clear(a.prev_pos[j] & a.prev_t.mask);
+  }
+  GS_STAMP(6);
+  GS_STAMP_END(5, 7);
+}
+
+// empties the slots a layer used (the last layer of a minibatch has no later relabel to do it)
+__global__ void __launch_bounds__(kThreads)
+layer_sweep_kernel(PackedTable t, const uint32_t* __restrict__ pos, RankCounts n) {
+  int64_t S, M;
+  n.get(&S, &M);
+  const int64_t j = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (j < M) t.clear(pos[j] & t.mask);
+}
+
 // ------------------------------------------------ batched (super-batch) relabel ----
 // B independent relabels in one pass: replaces impl::BatchCSRRelabelCUDA (reference
 // src/cuda/batch_relabel.cu:331; kernels :90-232).  Batch b owns seeds
@@ -1095,6 +1309,121 @@ int gs_relabel_table_init(void* table, size_t table_bytes, int id_bytes, void* s
                        dim3(kThreads), 0, st, t, cap);
   }
   return check_launch("relabel_table_init");
+}
+
+size_t gs_layer_workspace_bytes(int64_t S_bound, int64_t fanout) {
+  if (S_bound < 0) S_bound = 0;
+  if (fanout < 0) fanout = 0;
+  return layer_workspace_bytes(S_bound + S_bound * fanout);
+}
+
+namespace {
+// look-back status words, then the tiles' distance words (one per four items)
+inline size_t layer_relabel_state_bytes(int64_t items) {
+  return gs::lookback_state_bytes(gs::compact_num_tiles(items)) +
+         gs::padded(static_cast<size_t>(items / 4 + 2) * 8);
+}
+}  // namespace
+
+size_t gs_layer_relabel_state_bytes(int64_t S_bound, int64_t fanout) {
+  if (S_bound < 0) S_bound = 0;
+  if (fanout < 0) fanout = 0;
+  return layer_relabel_state_bytes(S_bound + S_bound * fanout);
+}
+
+int gs_layer_relabel(int id_bytes, int64_t S_bound, const int64_t* S_dev, int64_t capacity,
+                     const int64_t* num_edges, const int64_t* sub_indptr, void* table,
+                     size_t table_bytes, void* workspace, size_t workspace_bytes, void* frontier,
+                     void* out_ids, int64_t* num_unique, int64_t* offsets_copy, void* state,
+                     size_t state_bytes, uint32_t epoch, void* prev_table, size_t prev_table_bytes,
+                     const void* prev_workspace, size_t prev_workspace_bytes, int64_t prev_S_bound,
+                     const int64_t* prev_S_dev, int64_t prev_capacity,
+                     const int64_t* prev_num_edges, gs_mailbox* mailbox, int64_t mailbox_ticket,
+                     void* stream) {
+  GS_REQUIRE(S_bound >= 0 && capacity >= 0 && num_edges && table && workspace && num_unique && state,
+             "gs_layer_relabel: null pointer or negative size");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_layer_relabel: id_bytes must be 4 or 8, got %d", id_bytes);
+  GS_REQUIRE((capacity == 0 || out_ids) && (S_bound + capacity == 0 || frontier),
+             "gs_layer_relabel: null buffer");
+  GS_REQUIRE(!offsets_copy || sub_indptr, "gs_layer_relabel: offsets_copy without sub_indptr");
+  GS_REQUIRE(epoch >= 1 && epoch <= kLbMaxEpoch, "gs_layer_relabel: epoch must be in 1..%u",
+             kLbMaxEpoch);
+  const int64_t M_bound = S_bound + capacity;
+  if (M_bound >= (int64_t(1) << 31)) {
+    set_error_text("gs_layer_relabel: %lld items exceed the supported 2^31",
+                   static_cast<long long>(M_bound));
+    return GS_ERR_UNSUPPORTED;
+  }
+  PackedTable t, prev_t;
+  prev_t.slots = nullptr;
+  prev_t.mask = 0;
+  prev_t.shift = 0;
+  if (!shape_linked_table<PackedTable>(table, table_bytes, M_bound, &t)) {
+    set_error_text("gs_layer_relabel: the table holds fewer than the %lld slots this call needs "
+                   "(or is misaligned)",
+                   static_cast<long long>(linked_table_capacity(M_bound)));
+    return GS_ERR_WORKSPACE;
+  }
+  uint32_t* pos = nullptr;
+  Carver sc(state, state_bytes);
+  LookbackState lb = carve_lookback(sc, compact_num_tiles(M_bound), epoch);
+  unsigned long long* back = sc.take<unsigned long long>(static_cast<size_t>(M_bound / 4 + 2));
+  if (!carve_layer_workspace(workspace, workspace_bytes, M_bound, &pos) || !sc.ok) {
+    set_error_text("gs_layer_relabel: workspace needs %zu bytes and state %zu bytes, 256-byte "
+                   "aligned", layer_workspace_bytes(M_bound), layer_relabel_state_bytes(M_bound));
+    return GS_ERR_WORKSPACE;
+  }
+  uint32_t* prev_pos = nullptr;
+  const int64_t prev_bound = prev_S_bound + prev_capacity;
+  if (prev_table) {
+    GS_REQUIRE(prev_table != table, "gs_layer_relabel: the table to empty must be another table");
+    GS_REQUIRE(prev_workspace && prev_num_edges && prev_S_bound >= 0 && prev_capacity >= 0,
+               "gs_layer_relabel: the table to empty needs its layer's workspace and counts");
+    if (!shape_linked_table<PackedTable>(prev_table, prev_table_bytes, prev_bound, &prev_t) ||
+        !carve_layer_workspace(const_cast<void*>(prev_workspace), prev_workspace_bytes, prev_bound,
+                               &prev_pos)) {
+      set_error_text("gs_layer_relabel: the table to empty or its workspace is smaller than its "
+                     "layer needed");
+      return GS_ERR_WORKSPACE;
+    }
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const RankCounts n{S_bound, S_dev, capacity, num_edges};
+  const RankCounts pn{prev_S_bound, prev_S_dev, prev_capacity, prev_num_edges};
+  const dim3 grid(static_cast<unsigned>(compact_num_tiles(M_bound)));
+  ProfileScope prof("layer_relabel", st);
+  if (id_bytes == 8) {
+    RankArgs<int64_t> a{t, pos, n, back, static_cast<int64_t*>(frontier),
+                        static_cast<int64_t*>(out_ids), num_unique, sub_indptr, offsets_copy, lb,
+                        mailbox, mailbox_ticket, prev_t, prev_pos, pn};
+    hipLaunchKernelGGL((rank_linked_kernel<int64_t>), grid, dim3(kThreads), 0, st, a);
+    return check_launch("layer_relabel");
+  }
+  RankArgs<int32_t> a{t, pos, n, back, static_cast<int32_t*>(frontier),
+                      static_cast<int32_t*>(out_ids), num_unique, sub_indptr, offsets_copy, lb,
+                      mailbox, mailbox_ticket, prev_t, prev_pos, pn};
+  hipLaunchKernelGGL((rank_linked_kernel<int32_t>), grid, dim3(kThreads), 0, st, a);
+  return check_launch("layer_relabel");
+}
+
+int gs_layer_table_sweep(void* table, size_t table_bytes, const void* workspace,
+                         size_t workspace_bytes, int64_t S_bound, const int64_t* S_dev,
+                         int64_t capacity, const int64_t* num_edges, void* stream) {
+  GS_REQUIRE(table && workspace && num_edges && S_bound >= 0 && capacity >= 0,
+             "gs_layer_table_sweep: null pointer or negative size");
+  const int64_t M_bound = S_bound + capacity;
+  PackedTable t;
+  uint32_t* pos = nullptr;
+  if (!shape_linked_table<PackedTable>(table, table_bytes, M_bound, &t) ||
+      !carve_layer_workspace(const_cast<void*>(workspace), workspace_bytes, M_bound, &pos)) {
+    set_error_text("gs_layer_table_sweep: the table or the workspace is smaller than the layer needed");
+    return GS_ERR_WORKSPACE;
+  }
+  if (M_bound == 0) return GS_OK;
+  const RankCounts n{S_bound, S_dev, capacity, num_edges};
+  hipLaunchKernelGGL(layer_sweep_kernel, dim3(blocks_for(M_bound, kThreads)), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), t, pos, n);
+  return check_launch("layer_table_sweep");
 }
 
 size_t gs_relabel_sampled_workspace_bytes(int64_t num_items) {

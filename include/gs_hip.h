@@ -373,6 +373,73 @@ int gs_relabel_sampled_narrow(const void* seed_keys, int64_t S, const void* samp
                               uint32_t epoch, gs_mailbox* mailbox, int64_t mailbox_ticket,
                               void* stream);
 
+/* ------------------------------------------------------------------------- */
+/* One GraphSAGE layer -- column slice + uniform sample, then relabel -- as TWO  */
+/* launches that need no host read, so that a caller can queue all layers of a  */
+/* minibatch back to back and wait once.  Replaces, for the loop of              */
+/* examples/graphsage/batching.py:125-138, the pair                              */
+/* impl::fusion::FusedCSCColSlicingSamplingCUDA (src/cuda/fusion/slice_sampling.cu:146) */
+/* + impl::RelabelCUDA (src/cuda/unique_reindex.cu:179); results are those of    */
+/* gs_sample_uniform_fused followed by gs_relabel_sampled, bit for bit.          */
+/*                                                                               */
+/* Sizes may live on the device: S_bound bounds the number of columns (launches  */
+/* and buffers are sized for it), S_dev (NULL = S_bound is the number) is its    */
+/* device address -- typically the num_unique of the previous layer, whose       */
+/* frontier is this layer's column_ids.  A negative *S_dev counts as 0.          */
+/*   table: gs_relabel_table_bytes(max S_bound + capacity, 4), prepared once with */
+/*     gs_relabel_table_init(..., id_bytes = 4, ...): one-word slots.  64-bit ids */
+/*     (id_bytes 8) must fit 32 bits; if one does not, *num_unique reads -2 (as   */
+/*     gs_relabel_sampled_narrow).  gs_layer_sample fills it, gs_layer_relabel    */
+/*     reads it and does NOT empty it: name it as `prev_table` (with that layer's */
+/*     workspace and counts) in a later gs_layer_relabel on ANOTHER table, which  */
+/*     empties it on the side, or call gs_layer_table_sweep.  Two tables used in  */
+/*     turn keep every emptying off the critical path.                           */
+/*   workspace: gs_layer_workspace_bytes(S_bound, fanout), shared by the layer's  */
+/*     two calls and kept until the table has been emptied.                      */
+/*   state / epoch: as for gs_sample_uniform_fused (zero-filled once, a fresh     */
+/*     epoch per call); one buffer of max(gs_layer_sample_state_bytes,            */
+/*     gs_layer_relabel_state_bytes) serves both calls and every layer, each call */
+/*     with an epoch of its own: every word in it carries the epoch it was        */
+/*     written under.                                                            */
+/*   num_edges (device int64): written by gs_layer_sample (also at               */
+/*     sub_indptr[S]), read by gs_layer_relabel.                                 */
+/* ------------------------------------------------------------------------- */
+size_t gs_layer_workspace_bytes(int64_t S_bound, int64_t fanout);
+size_t gs_layer_sample_state_bytes(int64_t S_bound);
+size_t gs_layer_relabel_state_bytes(int64_t S_bound, int64_t fanout);
+
+/* First launch: the one-launch sampler (see gs_sample_uniform_fused: same draws, same
+ * outputs; sub_indices holds `capacity` >= S_bound * fanout entries) which also enters
+ * every seed (item r = seed r) and every sampled id (item S + e = output e) into `table`. */
+int gs_layer_sample(const int64_t* indptr, int64_t num_cols, const void* indices,
+                    const void* column_ids, int id_bytes, int64_t S_bound, const int64_t* S_dev,
+                    int64_t fanout, int replace, uint64_t seed, const uint32_t* replay,
+                    const int64_t* replay_ptr, int64_t* sub_indptr, void* sub_indices,
+                    int64_t capacity, int64_t* num_edges, void* table, size_t table_bytes,
+                    void* workspace, size_t workspace_bytes, void* state, size_t state_bytes,
+                    uint32_t epoch, gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
+
+/* Second launch: frontier (capacity S_bound + capacity; distinct ids of (seeds, sampled ids)
+ * in first-occurrence order), *num_unique (device; -1 / -2 as gs_relabel_sampled_narrow),
+ * out_ids[e] = rank of sampled id e, offsets_copy (NULL, or S + 1 slots that receive
+ * sub_indptr[0..S]).  prev_*: NULL / 0, or the table, workspace and counts of an earlier
+ * layer, whose slots are emptied here. */
+int gs_layer_relabel(int id_bytes, int64_t S_bound, const int64_t* S_dev, int64_t capacity,
+                     const int64_t* num_edges, const int64_t* sub_indptr, void* table,
+                     size_t table_bytes, void* workspace, size_t workspace_bytes, void* frontier,
+                     void* out_ids, int64_t* num_unique, int64_t* offsets_copy, void* state,
+                     size_t state_bytes, uint32_t epoch, void* prev_table, size_t prev_table_bytes,
+                     const void* prev_workspace, size_t prev_workspace_bytes, int64_t prev_S_bound,
+                     const int64_t* prev_S_dev, int64_t prev_capacity,
+                     const int64_t* prev_num_edges, gs_mailbox* mailbox, int64_t mailbox_ticket,
+                     void* stream);
+
+/* Empties the slots a layer filled (for the last layer of a run, which no later
+ * gs_layer_relabel empties). */
+int gs_layer_table_sweep(void* table, size_t table_bytes, const void* workspace,
+                         size_t workspace_bytes, int64_t S_bound, const int64_t* S_dev,
+                         int64_t capacity, const int64_t* num_edges, void* stream);
+
 /* B relabels in one pass ("super-batch"): replaces impl::BatchCSRRelabelCUDA
  * (src/cuda/batch_relabel.cu:331).  Batch b owns seeds[seeds_ptr[b]..seeds_ptr[b+1])
  * and ids[ids_ptr[b]..ids_ptr[b+1]) (both *_ptr: device int64[num_batches+1]).

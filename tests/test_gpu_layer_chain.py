@@ -1,0 +1,96 @@
+"""GPU parity: a whole minibatch queued with no host read (gs_layer_sample + gs_layer_relabel
+per layer, sizes handed from layer to layer on the device) against the CPU oracle, which runs
+the layers one by one: sample_uniform on the frontier, then relabel of (frontier, sampled ids)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from graph_sampling_amd import capi
+from tests.util import rmat_csc_np, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_layers(indptr, indices, seeds, fanouts, replace, seed):
+    out = []
+    cols = seeds
+    for l, k in enumerate(fanouts):
+        sp, _, si, _ = O.sample_uniform(indptr, indices, cols, k, replace, seed=seed + l,
+                                        with_coo=False)
+        frontier, (renamed,) = O.relabel([cols, si], [si])
+        out.append((cols.size, sp, si, frontier, renamed))
+        cols = frontier
+    return out
+
+
+def _check_layers(layers, want):
+    for b, (S, sp, si, frontier, renamed) in zip(layers, want):
+        E, U = (int(v) for v in b.counts.cpu())
+        assert E == si.size and U == frontier.size, (E, si.size, U, frontier.size)
+        assert np.array_equal(b.sub_indptr[:S + 1].cpu().numpy(), sp)
+        assert np.array_equal(b.offsets_copy[:S + 1].cpu().numpy(), sp)
+        assert np.array_equal(b.sub_indices[:E].cpu().numpy().astype(np.int64), si)
+        assert np.array_equal(b.frontier[:U].cpu().numpy().astype(np.int64), frontier)
+        assert np.array_equal(b.out_ids[:E].cpu().numpy().astype(np.int64), renamed)
+
+
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+@pytest.mark.parametrize("num_seeds,fanouts,replace", [
+    (1024, (15, 10, 5), False),   # the benchmark's minibatch
+    (512, (10, 5), False),
+    (1, (3,), False),
+    (0, (4, 4), False),
+    (300, (4, 4, 4, 4), True),
+    (3000, (32,), False),
+    (257, (1, 1, 1), False),
+])
+def test_chain_matches_the_oracle_layer_by_layer(dev, idt, num_seeds, fanouts, replace):
+    n = 1 << 14
+    indptr, indices = rmat_csc_np(n, 1 << 19, seed=21)
+    seeds = np.random.default_rng(num_seeds).permutation(n)[:num_seeds].astype(np.int64)
+    t_ptr, t_idx, t_seeds = to_dev(indptr, dev), to_dev(indices, dev, idt), to_dev(seeds, dev, idt)
+    bound = num_seeds
+    for k in fanouts:
+        bound *= 1 + k
+    tables = [capi.RelabelTable(bound, torch.int32, dev) for _ in range(2)]
+    box = capi.Mailbox()
+    # several minibatches in a row on the same two tables: every one leaves them empty
+    for seed in (40, 50):
+        layers, ticket = capi.sample_layers(t_ptr, t_idx, t_seeds, fanouts, replace, seed=seed,
+                                            mailbox=box, tables=tables)
+        U_last = box.wait(ticket, dev)
+        want = _oracle_layers(indptr, indices, seeds, fanouts, replace, seed)
+        assert U_last == want[-1][3].size
+        _check_layers(layers, want)
+    torch.cuda.synchronize()
+    for t in tables:
+        assert bool((t.buf.view(torch.int64) == -1).all())
+
+
+def test_chain_with_repeated_seeds_and_hub_columns(dev):
+    """Seeds that repeat (the frontier is shorter than the seed list) and the graph's largest
+    columns among them."""
+    n = 1 << 13
+    indptr, indices = rmat_csc_np(n, 1 << 18, seed=3)
+    rng = np.random.default_rng(8)
+    seeds = rng.integers(0, n, size=5000).astype(np.int64)
+    seeds[:16] = np.argsort(np.diff(indptr))[-16:]
+    seeds[100:200] = seeds[0]
+    d = (to_dev(indptr, dev), to_dev(indices, dev, torch.int32), to_dev(seeds, dev, torch.int32))
+    layers, _ = capi.sample_layers(*d, (6, 3), False, seed=9)
+    _check_layers(layers, _oracle_layers(indptr, indices, seeds, (6, 3), False, 9))
+
+
+def test_chain_reports_an_id_beyond_32_bits(dev):
+    """64-bit ids ride on one-word slots; one that does not fit is reported as -2, not truncated."""
+    indptr = np.array([0, 2, 4, 6], dtype=np.int64)
+    indices = np.array([1, 2, 0, (1 << 33) + 5, 0, 1], dtype=np.int64)
+    seeds = np.array([0, 1, 2], dtype=np.int64)
+    d = (to_dev(indptr, dev), to_dev(indices, dev), to_dev(seeds, dev))
+    box = capi.Mailbox()
+    layers, ticket = capi.sample_layers(*d, (2,), False, seed=1, mailbox=box)
+    assert box.wait(ticket, dev) == -2
+    assert int(layers[0].counts[1]) == -2
+    torch.cuda.synchronize()
+    capi._fused_state.clear()  # the error word of the look-back state is sticky
