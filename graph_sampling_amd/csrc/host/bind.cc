@@ -20,6 +20,7 @@ void SetSeed(int64_t seed) { hip::SetSeed(static_cast<uint64_t>(seed)); }
 void SetThreadSeed(int64_t seed) { hip::SetThreadSeed(static_cast<uint64_t>(seed)); }
 void SetSampleAlgo(int64_t algo) { hip::SetSampleAlgo(algo); }
 void SetDeferredSampling(bool on) { hip::SetDeferredSampling(on); }
+void DebugRaiseLookbackError(torch::Tensor like) { hip::DebugRaiseLookbackError(like); }
 torch::Tensor UniqueOp(torch::Tensor ids) { return TensorUnique(ids); }
 }  // namespace
 
@@ -38,6 +39,8 @@ TORCH_LIBRARY(gs_classes, m) {
       GS_DEF2("_CAPI_SamplingWithProbs", "_CAPI_sampling_with_probs", &Graph::SamplingProbs)
       GS_DEF2("_CAPI_FusedColumnwiseSlicingSampling", "_CAPI_fused_columnwise_slicing_sampling",
               &Graph::ColumnwiseFusedSlicingAndSampling)
+      // not in the reference: the per-layer loop of its GraphSAGE examples as one call
+      GS_DEF2("_CAPI_SampleLayers", "_CAPI_sample_layers", &Graph::SampleLayers)
       GS_DEF2("_CAPI_FusionSlicing", "_CAPI_fusion_slicing", &Graph::FusedBidirSlicing)
       GS_DEF2("_CAPI_BatchFusionSlicing", "_CAPI_batch_fusion_slicing",
               &Graph::BatchFusedBidirSlicing)
@@ -141,4 +144,6 @@ TORCH_LIBRARY(gs_ops, m) {
   m.def("_CAPI_SetSampleAlgo", &SetSampleAlgo);
   // not in the reference: off = every sampling call settles its edge count before returning
   m.def("_CAPI_SetDeferredSampling", &SetDeferredSampling);
+  // not in the reference: test hook for the recovery from a look-back that gave up
+  m.def("_CAPI_DebugRaiseLookbackError", &DebugRaiseLookbackError);
 }

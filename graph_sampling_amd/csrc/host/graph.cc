@@ -423,6 +423,53 @@ c10::intrusive_ptr<Graph> Graph::ColumnwiseFusedSlicingAndSampling(torch::Tensor
   return ret;
 }
 
+std::shared_ptr<hip::PendingLayers> Graph::QueueLayers(const torch::Tensor& seeds,
+                                                       const std::vector<int64_t>& fanouts,
+                                                       bool replace) {
+  Settle();
+  TORCH_CHECK(csc_ != nullptr, "fused slicing + sampling needs the CSC format");
+  // a root graph: local ids are the global ones, and no edge data follows the samples
+  if (col_ids_.has_value() || row_ids_.has_value() || data_.has_value() ||
+      val_col_ids_.has_value() || !hip::DeferredSampling())
+    return nullptr;
+  for (int64_t k : fanouts)
+    if (k == 1 && replace) return nullptr;  // (one slot per column, -1 for an empty one)
+  if (!hip::LayerChainApplies(seeds.numel(), fanouts, replace)) return nullptr;
+  return hip::SampleLayersQueued(csc_->indptr, csc_->indices, seeds, fanouts, replace);
+}
+
+std::vector<torch::Tensor> Graph::SampleLayersLoop(torch::Tensor seeds,
+                                                   const std::vector<int64_t>& fanouts,
+                                                   bool replace) {
+  std::vector<torch::Tensor> out;
+  out.reserve(3 * fanouts.size());
+  for (int64_t k : fanouts) {
+    auto sub = ColumnwiseFusedSlicingAndSampling(seeds, k, replace);
+    auto r = sub->Relabel();
+    out.push_back(std::get<0>(r));  // frontier: source ids of the block, seeds first
+    out.push_back(std::get<3>(r));  // offsets over the destinations
+    out.push_back(std::get<4>(r));  // source positions in the frontier
+    seeds = std::get<0>(r);
+  }
+  return out;
+}
+
+std::vector<torch::Tensor> Graph::SampleLayers(torch::Tensor seeds, std::vector<int64_t> fanouts,
+                                               bool replace) {
+  auto pending = QueueLayers(seeds, fanouts, replace);
+  if (!pending) return SampleLayersLoop(seeds, fanouts, replace);
+  try {
+    return pending->Collect();
+  } catch (const hip::IdsTooWide&) {
+    // the same minibatch again, layer by layer, under the seeds the chain drew with
+    const hip::SeedState saved = hip::SaveSeedState();
+    hip::SetThreadSeed(pending->first_seed);
+    auto out = SampleLayersLoop(seeds, fanouts, replace);
+    hip::RestoreSeedState(saved);
+    return out;
+  }
+}
+
 // The reference hands the kernel the GLOBAL ids of the seeds (src/graph.cc:120-128), which
 // only works on a graph without id maps, and gathers the parent's edge data with positions
 // of the virtual column slice (:131-137).  Here the kernel gets the local seeds and edge

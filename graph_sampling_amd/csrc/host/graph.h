@@ -26,6 +26,7 @@ namespace gs {
 
 namespace hip {
 struct PendingSample;
+struct PendingLayers;
 }
 
 class Graph : public torch::CustomClassHolder {
@@ -112,6 +113,24 @@ class Graph : public torch::CustomClassHolder {
                                           bool replace, int64_t on_format, int64_t output_format);
   c10::intrusive_ptr<Graph> ColumnwiseFusedSlicingAndSampling(torch::Tensor column_index,
                                                               int64_t fanout, bool replace);
+  // Every layer of a GraphSAGE-style minibatch in one call: what the loop of the reference's
+  // examples (examples/graphsage/batching.py:125-138) does layer by layer with
+  // ColumnwiseFusedSlicingAndSampling + Relabel, next seeds = frontier.  Returns the flat list
+  // [frontier, offsets, indices] x layers (elements 0, 3, 4 of Relabel()'s tuple); layer l
+  // draws with the l-th seed the calling thread hands out next, so the result equals the
+  // loop's.  On a graph without id maps or edge data all layers are queued with no host read
+  // in between and the sizes are collected once at the end.
+  std::vector<torch::Tensor> SampleLayers(torch::Tensor seeds, std::vector<int64_t> fanouts,
+                                          bool replace);
+  // The first half of SampleLayers when the whole minibatch can be queued (else nullptr, and
+  // no seed is consumed): the caller collects later, other minibatches may be queued
+  // meanwhile.  A collect that throws hip::IdsTooWide is answered with SampleLayersLoop under
+  // the seed the chain started from.
+  std::shared_ptr<hip::PendingLayers> QueueLayers(const torch::Tensor& seeds,
+                                                  const std::vector<int64_t>& fanouts,
+                                                  bool replace);
+  std::vector<torch::Tensor> SampleLayersLoop(torch::Tensor seeds,
+                                              const std::vector<int64_t>& fanouts, bool replace);
   // induced subgraph: columns column_seeds, rows row_seeds (renamed to their position in
   // row_seeds), CSC only (reference src/graph.cc:116-141)
   c10::intrusive_ptr<Graph> FusedBidirSlicing(torch::Tensor column_seeds, torch::Tensor row_seeds);

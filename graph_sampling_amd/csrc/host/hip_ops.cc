@@ -72,9 +72,10 @@ torch::Tensor Scratch(size_t bytes, const torch::Tensor& like) {
 // A ring of kBoxes {total, ticket} pairs per (thread, device); call number t posts
 // to slot t % kBoxes, so a total stays readable until kBoxes later calls have
 // been issued.
-constexpr int64_t kBoxes = 64;
+constexpr int64_t kBoxes = 1024;
 constexpr int64_t kLost = -3;     // the slot was reused before anyone read it
 constexpr int64_t kTooWide = -2;  // posted by the narrow relabel: a key needs more than 32 bits
+constexpr int64_t kGaveUp = -1;   // posted when a tile's bounded wait ran out
 
 // 64-bit ids go on the one-word table slots of 32-bit ids (GS_NARROW_IDS) until this thread
 // meets one that does not fit 32 bits; from then on it asks for the two-array slots.
@@ -122,9 +123,18 @@ int64_t WaitBox(const gs_mailbox* box, int64_t ticket, void* stream, const char*
   const int64_t total = __atomic_load_n(&box->total, __ATOMIC_RELAXED);
   // the slot may have been rewritten between the two loads
   if (__atomic_load_n(&box->ticket, __ATOMIC_ACQUIRE) != ticket) return kLost;
-  TORCH_CHECK(total >= 0 || total == kTooWide, what,
-              ": a tile gave up waiting for its predecessors");
-  return total;
+  return total;  // kGaveUp and kTooWide are the caller's to act on
+}
+
+// A tile gave up waiting for its predecessors: the error word it raised stays in the
+// look-back state until that is zero-filled, and would fail every later launch on it.  Clears
+// it behind the failed launch (an all-zero state is valid under any epoch) and reports.
+[[noreturn]] void GaveUp(const torch::Tensor& state, void* stream, const char* what) {
+  if (state.defined())
+    (void)hipMemsetAsync(state.data_ptr(), 0, static_cast<size_t>(state.numel()),
+                         static_cast<hipStream_t>(stream));
+  TORCH_CHECK(false, what, ": a tile gave up waiting for its predecessors; the look-back state "
+              "has been cleared and the call can be repeated");
 }
 
 // Look-back state of the one-launch sampler, one per (device, stream): zero-filled
@@ -282,11 +292,9 @@ SliceResult SampleInto(const torch::Tensor& indptr, const torch::Tensor& indices
 }  // namespace
 
 int64_t PendingSample::Wait() const {
-  int64_t nnz = WaitBox(Boxes(device).slot(ticket), ticket, stream, "gs_sample_uniform_fused");
-  if (nnz == kLost) {
-    nnz = sub_indptr[S].item<int64_t>();
-    TORCH_CHECK(nnz >= 0, "gs_sample_uniform_fused: a tile gave up waiting for its predecessors");
-  }
+  int64_t nnz = WaitBox(static_cast<const gs_mailbox*>(box), ticket, stream, "gs_sample_uniform_fused");
+  if (nnz == kLost) nnz = sub_indptr[S].item<int64_t>();
+  if (nnz < 0) GaveUp(state_owner, stream, "gs_sample_uniform_fused");
   return nnz;
 }
 
@@ -324,6 +332,9 @@ std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
   FusedStateBuf& state = FusedState(gs_sample_fused_state_bytes(p->S), indptr, p->stream);
   HostBoxes& boxes = Boxes(p->device);
   p->ticket = boxes.next++;
+  p->box = boxes.slot(p->ticket);
+  p->box_owner = boxes.buf;
+  p->state_owner = state.buf;
   Check(gs_sample_uniform_fused(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(),
                                 fused ? column_ids.data_ptr() : nullptr, idb, p->S, fanout,
                                 replace ? 1 : 0, NextSeed(), nullptr, nullptr,
@@ -536,9 +547,212 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred
       FusedState(gs_relabel_sampled_state_bytes(M), col_ids, p.stream);       // next epoch
     }
   }
-  TORCH_CHECK(U >= 0, "gs_relabel_sampled: a tile gave up waiting for its predecessors");
+  if (U < 0) GaveUp(state.buf, p.stream, "gs_relabel_sampled");  // (the table stays marked)
   table.clean = true;
   return {frontier.narrow(0, 0, U), renamed.narrow(0, 0, nnz), nnz, offsets_copy};
+}
+
+
+// ---- a whole minibatch queued with no host read -------------------------------------
+namespace {
+
+// 64-bit ids ride on the chain's one-word table slots until this thread meets one that
+// does not fit 32 bits; from then on its minibatches go layer by layer.
+thread_local bool t_chain_ids_fit = true;
+// the chain's launches and tables are sized for the bounds S * prod(1 + fanout); beyond this
+// many items per layer the layer-by-layer path, which sizes by what was sampled, is used
+constexpr int64_t kChainMaxItems = int64_t(1) << 23;
+
+// the two tables a chain uses in turn (a layer's relabel empties the table of the layer
+// before it), one pair per (thread, device, stream); a chain in flight holds on to its pair
+struct ChainTables {
+  torch::Tensor buf[2];
+  int64_t items = 0;
+  bool clean = false;
+};
+
+std::shared_ptr<ChainTables> ChainTablesFor(const torch::Tensor& like, void* stream,
+                                            int64_t items) {
+  thread_local std::map<std::pair<int, void*>, std::shared_ptr<ChainTables>> tables;
+  std::shared_ptr<ChainTables>& t = tables[{like.device().index(), stream}];
+  if (!t) t = std::make_shared<ChainTables>();
+  if (!t->buf[0].defined() || t->items < items) {
+    int64_t want = 1 << 16;
+    while (want < items) want <<= 1;
+    for (auto& b : t->buf)
+      b = torch::empty({static_cast<int64_t>(gs_relabel_table_bytes(want, 4))},
+                       torch::dtype(torch::kUInt8).device(like.device()));
+    t->items = want;
+    t->clean = false;
+  }
+  if (!t->clean) {
+    for (auto& b : t->buf)
+      Check(gs_relabel_table_init(b.data_ptr(), b.numel(), 4, stream), "gs_relabel_table_init");
+    t->clean = true;
+  }
+  return t;
+}
+
+inline size_t Pad256(size_t n) { return (n + 255) / 256 * 256; }
+
+}  // namespace
+
+void DebugRaiseLookbackError(const torch::Tensor& like) {
+  FusedStateBuf& s = FusedState(65536, like, Stream(like));
+  // the error word is the first word of the state (carve_lookback)
+  s.buf.narrow(0, 0, 4).view(torch::kInt32).fill_(1);
+}
+
+SeedState SaveSeedState() { return {t_own_seed, t_seed}; }
+void RestoreSeedState(const SeedState& s) {
+  t_own_seed = s.own;
+  t_seed = s.seed;
+}
+
+bool LayerChainApplies(int64_t num_seeds, const std::vector<int64_t>& fanouts, bool replace) {
+  if (g_algo.load() != GS_SAMPLE_AUTO || !t_chain_ids_fit || fanouts.empty()) return false;
+  int64_t bound = num_seeds;
+  for (int64_t k : fanouts) {
+    if (k < 0 || (!replace && k > GS_FUSED_MAX_FANOUT)) return false;
+    if (bound > kChainMaxItems / (1 + k)) return false;
+    bound *= 1 + k;
+  }
+  return true;
+}
+
+std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
+                                                  const torch::Tensor& indices,
+                                                  const torch::Tensor& seeds,
+                                                  const std::vector<int64_t>& fanouts,
+                                                  bool replace) {
+  NeedI64(indptr, "indptr");
+  const int idb = IdBytes(indices, "indices");
+  TORCH_CHECK(IdBytes(seeds, "seeds") == idb, "seeds and indices differ in dtype");
+  const int64_t L = static_cast<int64_t>(fanouts.size());
+  TORCH_CHECK(LayerChainApplies(seeds.numel(), fanouts, replace),
+              "SampleLayersQueued: this minibatch has to go layer by layer");
+  auto p = std::make_shared<PendingLayers>();
+  p->layers.resize(L);
+  p->stream = Stream(indptr);
+  p->device = indptr.device().index();
+  p->num_seeds = seeds.numel();
+  // bounds: S_0 = #seeds, capacity_l = S_l * fanout_l, S_{l+1} = S_l + capacity_l
+  std::vector<int64_t> S(L + 1);
+  S[0] = seeds.numel();
+  for (int64_t l = 0; l < L; ++l) S[l + 1] = S[l] * (1 + fanouts[l]);
+  // one allocation for what no caller sees: per layer the sampled ids before renaming, the
+  // items' table slots and the two counts
+  std::vector<size_t> off_ids(L), off_ws(L), ws_bytes(L), off_counts(L);
+  size_t bytes = 0, state_bytes = 0;
+  for (int64_t l = 0; l < L; ++l) {
+    off_ids[l] = bytes;
+    bytes += Pad256(static_cast<size_t>(S[l] * fanouts[l]) * idb);
+    ws_bytes[l] = gs_layer_workspace_bytes(S[l], fanouts[l]);
+    off_ws[l] = bytes;
+    bytes += Pad256(ws_bytes[l]);
+    off_counts[l] = bytes;
+    bytes += 256;
+    state_bytes = std::max(state_bytes, std::max(gs_layer_sample_state_bytes(S[l]),
+                                                 gs_layer_relabel_state_bytes(S[l], fanouts[l])));
+  }
+  p->scratch = Scratch(bytes, indptr);
+  char* base = static_cast<char*>(p->scratch.data_ptr());
+  auto tables = ChainTablesFor(indptr, p->stream, S[L]);
+  p->tables = tables;
+  HostBoxes& boxes = Boxes(p->device);
+  p->box_owner = boxes.buf;
+  p->ring = boxes.ring;
+  const void* cols = seeds.data_ptr();
+  const int64_t* S_dev = nullptr;
+  for (int64_t l = 0; l < L; ++l) {
+    PendingLayers::Layer& y = p->layers[l];
+    const int64_t cap = S[l] * fanouts[l];
+    y.offsets = torch::empty({S[l] + 1}, I64(indptr));
+    y.renamed = torch::empty({cap}, indices.options());
+    y.frontier = torch::empty({S[l] + cap}, indices.options());
+    int64_t* counts = reinterpret_cast<int64_t*>(base + off_counts[l]);
+    void* table = tables->buf[l & 1].data_ptr();
+    const size_t table_bytes = tables->buf[l & 1].numel();
+    const uint64_t seed = NextSeed();
+    if (l == 0) p->first_seed = seed;
+    FusedStateBuf& st1 = FusedState(state_bytes, indptr, p->stream);
+    if (l == 0) p->state_owner = st1.buf;
+    y.ticket_edges = boxes.next++;
+    Check(gs_layer_sample(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), cols,
+                          idb, S[l], S_dev, fanouts[l], replace ? 1 : 0, seed, nullptr, nullptr,
+                          y.offsets.data_ptr<int64_t>(), base + off_ids[l], cap, counts, table,
+                          table_bytes, base + off_ws[l], ws_bytes[l], st1.buf.data_ptr(),
+                          st1.buf.numel(), st1.epoch, boxes.slot(y.ticket_edges), y.ticket_edges,
+                          p->stream),
+          "gs_layer_sample");
+    FusedStateBuf& st2 = FusedState(state_bytes, indptr, p->stream);
+    y.ticket_unique = boxes.next++;
+    const bool has_prev = l > 0;
+    Check(gs_layer_relabel(
+              idb, S[l], S_dev, cap, counts, y.offsets.data_ptr<int64_t>(), table, table_bytes,
+              base + off_ws[l], ws_bytes[l], y.frontier.data_ptr(), y.renamed.data_ptr(),
+              counts + 1, nullptr, st2.buf.data_ptr(), st2.buf.numel(), st2.epoch,
+              has_prev ? tables->buf[(l - 1) & 1].data_ptr() : nullptr,
+              has_prev ? static_cast<size_t>(tables->buf[(l - 1) & 1].numel()) : 0,
+              has_prev ? base + off_ws[l - 1] : nullptr, has_prev ? ws_bytes[l - 1] : 0,
+              has_prev ? S[l - 1] : 0,
+              l >= 2 ? reinterpret_cast<int64_t*>(base + off_counts[l - 2]) + 1 : nullptr,
+              has_prev ? S[l - 1] * fanouts[l - 1] : 0,
+              has_prev ? reinterpret_cast<int64_t*>(base + off_counts[l - 1]) : nullptr,
+              boxes.slot(y.ticket_unique), y.ticket_unique, p->stream),
+          "gs_layer_relabel");
+    cols = y.frontier.data_ptr();
+    S_dev = counts + 1;
+  }
+  // the last layer's table has no later relabel to empty it
+  Check(gs_layer_table_sweep(
+            tables->buf[(L - 1) & 1].data_ptr(), tables->buf[(L - 1) & 1].numel(),
+            base + off_ws[L - 1], ws_bytes[L - 1], S[L - 1],
+            L >= 2 ? reinterpret_cast<int64_t*>(base + off_counts[L - 2]) + 1 : nullptr,
+            S[L - 1] * fanouts[L - 1], reinterpret_cast<int64_t*>(base + off_counts[L - 1]),
+            p->stream),
+        "gs_layer_table_sweep");
+  return p;
+}
+
+std::vector<torch::Tensor> PendingLayers::Collect() {
+  const gs_mailbox* boxes = static_cast<const gs_mailbox*>(ring);
+  std::vector<torch::Tensor> out;
+  out.reserve(3 * layers.size());
+  int64_t S = num_seeds;
+  int64_t worst = 0;
+  std::vector<int64_t> E(layers.size()), U(layers.size());
+  // the last count first: once it is here every earlier one is
+  for (size_t l = layers.size(); l-- > 0;) {
+    U[l] = WaitBox(boxes + layers[l].ticket_unique % kBoxes, layers[l].ticket_unique, stream,
+                   "gs_layer_relabel");
+    E[l] = WaitBox(boxes + layers[l].ticket_edges % kBoxes, layers[l].ticket_edges, stream,
+                   "gs_layer_sample");
+    TORCH_CHECK(U[l] != kLost && E[l] != kLost,
+                "more minibatches in flight than the ring of result mailboxes holds");
+    worst = std::min(worst, U[l]);
+  }
+  if (worst < 0) {
+    // an id beyond 32 bits (-2) or a tile that gave up (-1): either way the tables hold
+    // leftovers and the look-back state a raised error word
+    auto t = std::static_pointer_cast<ChainTables>(tables);
+    if (t) t->clean = false;
+    if (worst == kTooWide) {
+      if (state_owner.defined())
+        (void)hipMemsetAsync(state_owner.data_ptr(), 0, static_cast<size_t>(state_owner.numel()),
+                             static_cast<hipStream_t>(stream));
+      t_chain_ids_fit = false;
+      throw IdsTooWide();
+    }
+    GaveUp(state_owner, stream, "gs_layer_relabel");
+  }
+  for (size_t l = 0; l < layers.size(); ++l) {
+    out.push_back(layers[l].frontier.narrow(0, 0, U[l]));
+    out.push_back(layers[l].offsets.narrow(0, 0, S + 1));
+    out.push_back(layers[l].renamed.narrow(0, 0, E[l]));
+    S = U[l];
+  }
+  return out;
 }
 
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(

@@ -50,6 +50,13 @@ struct PendingSample {
   int64_t ticket = 0;
   void* stream = nullptr;
   int device = 0;
+  // where the kernel posts the total: a slot of the launching thread's ring of pinned
+  // mailboxes, kept alive here so that any thread may wait on it
+  const void* box = nullptr;
+  torch::Tensor box_owner;
+  // the look-back state the launch used: zero-filled again (on `stream`) when a tile of the
+  // launch gave up, since the error word in it is sticky
+  torch::Tensor state_owner;
   int64_t Wait() const;
 };
 // Whether the fused sampler may hand back a graph before its edge count has reached the
@@ -67,6 +74,54 @@ std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
 // reading its total
 std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred(
     const torch::Tensor& col_ids, const PendingSample& p);
+
+// Every layer of a minibatch queued back to back with no host read in between (per layer
+// gs_layer_sample + gs_layer_relabel: the frontier of one layer and its length feed the next
+// on the device).  Collect() waits for the counts and narrows.  Same draws and same results
+// as ColSamplingDeferred + RelabelDeferred layer by layer with the seeds NextSeed() hands out.
+struct PendingLayers {
+  struct Layer {
+    torch::Tensor frontier, offsets, renamed;  // at their bounds until collected
+    int64_t ticket_edges = 0, ticket_unique = 0;
+  };
+  std::vector<Layer> layers;
+  torch::Tensor scratch;    // sampled ids, slot numbers, counts: kept until collected
+  torch::Tensor box_owner;  // the pinned ring the tickets go to
+  const void* ring = nullptr;
+  torch::Tensor state_owner;     // the look-back state of the launches
+  std::shared_ptr<void> tables;  // the pair of hash tables the layers used in turn
+  void* stream = nullptr;
+  int device = 0;
+  int64_t num_seeds = 0;
+  uint64_t first_seed = 0;  // layer l drew with first_seed + l
+  // {frontier, offsets over the layer's seeds, sampled ids renamed} per layer.  Throws
+  // IdsTooWide when a 64-bit id does not fit the chain's one-word table slots (the caller
+  // repeats the minibatch layer by layer), c10::Error when a tile gave up waiting.
+  std::vector<torch::Tensor> Collect();
+};
+struct IdsTooWide : public std::exception {
+  const char* what() const noexcept override { return "an id beyond 32 bits"; }
+};
+// whether SampleLayersQueued takes this minibatch (uniform sampling by the one-launch
+// kernel, bounds within the chain's table limit, ids that have fitted 32 bits so far)
+bool LayerChainApplies(int64_t num_seeds, const std::vector<int64_t>& fanouts, bool replace);
+std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
+                                                  const torch::Tensor& indices,
+                                                  const torch::Tensor& seeds,
+                                                  const std::vector<int64_t>& fanouts,
+                                                  bool replace);
+// For tests of the recovery path: raises the sticky error word in the look-back state of the
+// calling thread's current stream on `like`'s device, as a tile that gave up waiting would.
+// The next one-launch sampler or relabel on that state reports failure (every kernel still
+// runs to its end), after which the host layer clears the state.
+void DebugRaiseLookbackError(const torch::Tensor& like);
+// the calling thread's seed counter as SetThreadSeed / SetSeed left it, to put it back
+struct SeedState {
+  bool own;
+  uint64_t seed;
+};
+SeedState SaveSeedState();
+void RestoreSeedState(const SeedState& s);
 
 SliceResult ColSamplingProbs(const torch::Tensor& indptr, const torch::Tensor& indices,
                              const torch::Tensor& probs, const torch::Tensor& column_ids,

@@ -126,19 +126,41 @@ std::vector<std::vector<torch::Tensor>> SampleBlocks(const c10::intrusive_ptr<Gr
       c10::hip::HIPStreamGuard stream_guard(stream);
       TORCH_CHECK(hipStreamWaitEvent(stream.stream(), ready, 0) == hipSuccess,
                   "hipStreamWaitEvent failed");
+      // Minibatches whose layers can all be queued without a host read are queued a few
+      // ahead of the one being collected, so the stream never waits for this thread.
+      constexpr int64_t kAhead = 8;
+      std::vector<std::pair<int64_t, std::shared_ptr<hip::PendingLayers>>> window;
+      auto collect_oldest = [&] {
+        const int64_t i = window.front().first;
+        auto pending = std::move(window.front().second);
+        window.erase(window.begin());
+        try {
+          out[i] = pending->Collect();
+        } catch (const hip::IdsTooWide&) {
+          // ids beyond 32 bits: what was queued behind it used the same tables, so all of it
+          // is done again, layer by layer, like every later minibatch of this thread
+          std::vector<int64_t> redo{i};
+          for (auto& w : window) redo.push_back(w.first);
+          window.clear();
+          for (int64_t j : redo) {
+            hip::SetThreadSeed(static_cast<uint64_t>(first_seed + j * layers));
+            out[j] = graph->SampleLayersLoop(seed_sets[j], fanouts, replace);
+          }
+        }
+      };
       for (int64_t i = k; i < n; i += nthreads) {
         hip::SetThreadSeed(static_cast<uint64_t>(first_seed + i * layers));
-        torch::Tensor seeds = seed_sets[i];
-        out[i].reserve(3 * layers);
-        for (int64_t l = 0; l < layers; ++l) {
-          auto sub = graph->ColumnwiseFusedSlicingAndSampling(seeds, fanouts[l], replace);
-          auto r = sub->Relabel();
-          out[i].push_back(std::get<0>(r));  // frontier: source ids of the block, seeds first
-          out[i].push_back(std::get<3>(r));  // offsets over the destinations
-          out[i].push_back(std::get<4>(r));  // source positions in the frontier
-          seeds = std::get<0>(r);
+        auto pending = graph->QueueLayers(seed_sets[i], fanouts, replace);
+        if (pending) {
+          window.emplace_back(i, std::move(pending));
+          if (static_cast<int64_t>(window.size()) > kAhead) collect_oldest();
+        } else {
+          while (!window.empty()) collect_oldest();
+          hip::SetThreadSeed(static_cast<uint64_t>(first_seed + i * layers));
+          out[i] = graph->SampleLayersLoop(seed_sets[i], fanouts, replace);
         }
       }
+      while (!window.empty()) collect_oldest();
       TORCH_CHECK(hipStreamSynchronize(stream.stream()) == hipSuccess, "hipStreamSynchronize failed");
     } catch (...) {
       std::lock_guard<std::mutex> hold(failure_lock);

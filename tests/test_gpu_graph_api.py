@@ -844,3 +844,125 @@ def test_relabel_falls_back_when_64_bit_ids_exceed_32_bits(dev):
     frontier = sub._CAPI_Relabel()[0]
     sp, _, rows, _ = O.sample_uniform(indptr, indices, seeds, 6, False, seed=95, with_coo=False)
     assert np.array_equal(frontier.cpu().numpy(), O.relabel([seeds, rows], [rows])[0])
+
+
+# ------------------------------------- a whole minibatch in one call (no host read per layer)
+def _oracle_minibatch(indptr, indices, seeds, fanouts, replace, seed, col_ids=None):
+    want = []
+    cols = seeds
+    keys = seeds if col_ids is None else col_ids[seeds]
+    for l, k in enumerate(fanouts):
+        sp, _, rows, _ = O.sample_uniform(indptr, indices, cols, k, replace, seed=seed + l,
+                                          with_coo=False)
+        frontier, (renamed,) = O.relabel([keys, rows], [rows])
+        want += [frontier, sp, renamed]
+        cols = keys = frontier
+    return want
+
+
+def _same(got, want):
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy().astype(np.int64), w)
+
+
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+@pytest.mark.parametrize("fanouts,replace", [((15, 10, 5), False), ((4, 4), True), ((32,), False),
+                                             ((40, 3), False), ((1, 2), True)])
+def test_sample_layers_equals_the_layer_loop_and_the_oracle(dev, idt, fanouts, replace):
+    """_CAPI_SampleLayers against the oracle run layer by layer and against the Graph methods
+    called layer by layer under the same seeds.  Fanouts above 32 without replacement and a
+    fanout of 1 with replacement take the loop inside the call."""
+    n = 1 << 13
+    indptr, indices = rmat_csc_np(n, 1 << 18, seed=17)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev, idt))
+    seeds = np.random.default_rng(5).permutation(n)[:700].astype(np.int64)
+    t_seeds = to_dev(seeds, dev, idt)
+    for first in (300, 310):
+        gs.set_seed(first)
+        got = g._CAPI_SampleLayers(t_seeds, list(fanouts), replace)
+        if not (replace and 1 in fanouts):  # (the keep-dim sampler is not the oracle's sample_uniform)
+            _same(got, _oracle_minibatch(indptr, indices, seeds, fanouts, replace, first))
+        gs.set_seed(first)
+        cols, loop = t_seeds, []
+        for k in fanouts:
+            sub = g._CAPI_FusedColumnwiseSlicingSampling(cols, k, replace)
+            r = sub._CAPI_Relabel()
+            loop += [r[0], r[3], r[4]]
+            cols = r[0]
+        for a, b in zip(got, loop):
+            assert torch.equal(a, b)
+
+
+def test_sample_layers_on_a_graph_with_column_ids_takes_the_loop(dev):
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 16, seed=13)
+    col_ids = np.random.default_rng(1).permutation(1 << 12).astype(np.int64)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSCWithColIds(to_dev(col_ids, dev), to_dev(indptr, dev), to_dev(indices, dev))
+    seeds = np.arange(200, dtype=np.int64)
+    gs.set_seed(77)
+    got = g._CAPI_SampleLayers(to_dev(seeds, dev), [5], False)
+    _same(got, _oracle_minibatch(indptr, indices, seeds, (5,), False, 77, col_ids=col_ids))
+
+
+def test_sample_layers_repeats_layer_by_layer_when_an_id_exceeds_32_bits(dev):
+    """The queued layers keep 64-bit ids on one-word table slots.  A neighbour id beyond 32 bits
+    is reported by the kernels, the minibatch is sampled again layer by layer under the same
+    seeds, and the calling thread stays on that path.  (Run in a thread of its own: the switch is
+    per thread.)"""
+    import threading
+    indptr = np.array([0, 2, 4, 6, 6], dtype=np.int64)
+    indices = np.array([1, 2, 0, (1 << 33) + 5, 0, 1], dtype=np.int64)
+    seeds = np.array([0, 1, 2], dtype=np.int64)
+    failure = []
+
+    def body():
+        try:
+            torch.cuda.set_device(dev)
+            g = gs.Graph(False)
+            g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev))
+            for first in (11, 12):
+                torch.ops.gs_ops._CAPI_SetThreadSeed(first)
+                got = g._CAPI_SampleLayers(to_dev(seeds, dev), [2, 2], False)
+                _same(got, _oracle_minibatch(indptr, indices, seeds, (2, 2), False, first))
+        except BaseException as e:  # noqa: BLE001
+            failure.append(e)
+
+    t = threading.Thread(target=body)
+    t.start()
+    t.join()
+    if failure:
+        raise failure[0]
+
+
+@pytest.mark.parametrize("whole_minibatch", [True, False])
+def test_a_look_back_that_gave_up_is_reported_and_does_not_stick(dev, whole_minibatch):
+    """The error word a tile raises when its bounded wait runs out stays in the look-back state.
+    Raised here from the host (every kernel runs to its end): the call that meets it fails with an
+    exception, the host layer clears the state behind it, and the next call is right again."""
+    n = 1 << 12
+    indptr, indices = rmat_csc_np(n, 1 << 16, seed=4)
+    g = gs.Graph(False)
+    t_ptr = to_dev(indptr, dev)
+    g._CAPI_LoadCSC(t_ptr, to_dev(indices, dev, torch.int32))
+    seeds = np.random.default_rng(0).permutation(n)[:500].astype(np.int64)
+    t_seeds = to_dev(seeds, dev, torch.int32)
+
+    def run(first):
+        gs.set_seed(first)
+        if whole_minibatch:
+            return g._CAPI_SampleLayers(t_seeds, [6, 4], False)
+        out, cols = [], t_seeds
+        for k in (6, 4):
+            r = g._CAPI_FusedColumnwiseSlicingSampling(cols, k, False)._CAPI_Relabel()
+            out += [r[0], r[3], r[4]]
+            cols = r[0]
+        return out
+
+    _same(run(20), _oracle_minibatch(indptr, indices, seeds, (6, 4), False, 20))
+    torch.ops.gs_ops._CAPI_DebugRaiseLookbackError(t_ptr)
+    with pytest.raises(RuntimeError, match="gave up"):
+        run(21)
+    for first in (22, 23):
+        _same(run(first), _oracle_minibatch(indptr, indices, seeds, (6, 4), False, first))
