@@ -258,16 +258,6 @@ def main():
         lambda: capi.segment_sum(indptr, None, None, weights, 2, out_n),
         lambda o: (E * 4 + N * 20, E, "edges"))
 
-    # ---- what the memory system gives for 8-byte accesses at random positions of a 256 MB table
-    table = torch.full((1 << 25,), -1, dtype=torch.int64, device=dev)
-    pkeys = rand_ids(16 << 20)
-    for kind, name in ((0, "compare-and-swap"), (1, "atomic minimum"), (2, "read"), (3, "write")):
-        run("probe_" + name.replace(" ", "_").replace("-", "_"),
-            "gs_probe_random_access: 16.8M 8-byte %ss at hashed slots of a 32M-slot table; 8 B each" % name,
-            lambda kind=kind: capi.probe_random_access(kind, table, pkeys),
-            lambda o: ((16 << 20) * 8, 16 << 20, "items"))
-    del table
-
     # ---- whole samplers through the Matrix layer (wall clock, device drained around each) -------
     import graph_sampling_amd as gs
     from graph_sampling_amd import jit

@@ -828,17 +828,6 @@ def sddmm_csc(op, indptr, indices, e_ids, nid_map, lhs, rhs, out, lhs_target, rh
                               _ptr(rhs_off), _stream(dev)), "gs_sddmm_csc")
 
 
-def probe_random_access(kind, table, keys):
-    """gs_probe_random_access: one 8-byte access per key at a hashed slot of `table` (int64, a
-    power of two long); kind 0 compare-and-swap, 1 atomic minimum, 2 read, 3 write."""
-    _need(table, torch.int64, "table")
-    _need(keys, torch.int32, "keys")
-    _check(lib().gs_probe_random_access(int(kind), _ptr(table), _i64(table.numel()), _ptr(keys),
-                                        _i64(keys.numel()), _stream(table.device)),
-           "gs_probe_random_access")
-
-
-# ------------------------------------------------------------ segment ops ----
 def segment_sum(indptr, e_ids, n_ids, data, powk, out):
     _need(indptr, torch.int64, "indptr")
     _need(data, torch.float32, "data")

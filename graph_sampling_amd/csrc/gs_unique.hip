@@ -1062,19 +1062,28 @@ int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* 
   BatchItems<IdT> x{static_cast<const IdT*>(seeds), seeds_ptr, static_cast<const IdT*>(ids), ids_ptr,
                     B};
   const int64_t n_init = cap > tiles ? cap : tiles;
-  hipLaunchKernelGGL((regions_init_kernel<R>), dim3(blocks_for(n_init, kThreads)), dim3(kThreads),
-                     0, stream, t, cap, lb, tiles);
-  if (M > 0)
+  {
+    ProfileScope prof("batch_init", stream);
+    hipLaunchKernelGGL((regions_init_kernel<R>), dim3(blocks_for(n_init, kThreads)),
+                       dim3(kThreads), 0, stream, t, cap, lb, tiles);
+  }
+  if (M > 0) {
+    ProfileScope prof("batch_insert", stream);
     hipLaunchKernelGGL((batch_insert_kernel<IdT, R>), dim3(blocks_for(M, kThreads)), dim3(kThreads),
                        0, stream, x, M, t, pos,
                        sizeof(IdT) == 8 && std::is_same<R, PackedRegions>::value
                            ? lb.error
                            : static_cast<unsigned int*>(nullptr));
-  hipLaunchKernelGGL((batch_compact_kernel<IdT, R>), dim3(static_cast<unsigned>(tiles)),
-                     dim3(kThreads), 0, stream, x, M, t, pos, prefix, static_cast<IdT*>(unique),
-                     num_unique, lb, box, box_ticket);
+  }
+  {
+    ProfileScope prof("batch_compact", stream);
+    hipLaunchKernelGGL((batch_compact_kernel<IdT, R>), dim3(static_cast<unsigned>(tiles)),
+                       dim3(kThreads), 0, stream, x, M, t, pos, prefix, static_cast<IdT*>(unique),
+                       num_unique, lb, box, box_ticket);
+  }
   const int64_t id_blocks = (num_ids + kThreads - 1) / kThreads;
   const int64_t ptr_blocks = (B + 1 + kThreads - 1) / kThreads;
+  ProfileScope prof("batch_finish", stream);
   hipLaunchKernelGGL((batch_finish_kernel<IdT, R>), dim3(static_cast<unsigned>(id_blocks + ptr_blocks)),
                      dim3(kThreads), 0, stream, x, num_ids, M, t, pos, prefix, num_unique,
                      static_cast<IdT*>(out_ids), unique_ptr, static_cast<const IdT*>(extra),
@@ -1087,52 +1096,7 @@ int batch_relabel_impl(const void* seeds, const int64_t* seeds_ptr, const void* 
 
 using namespace gs;
 
-namespace gs {
-namespace {
-// kind: 0 compare-and-swap, 1 atomic minimum, 2 read, 3 write
-template <int KIND>
-__global__ void __launch_bounds__(kThreads)
-probe_kernel(unsigned long long* __restrict__ table, uint32_t mask,
-             const uint32_t* __restrict__ keys, int64_t n) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (i >= n) return;
-  const uint32_t key = keys[i];
-  unsigned long long* slot = table + (fib_home(key, 32) & mask);
-  const unsigned long long word = (static_cast<unsigned long long>(key) << 32) | static_cast<uint32_t>(i);
-  if (KIND == 0) {
-    if (atomicCAS(slot, ~0ull, word) == 1ull) table[0] = 0ull;  // keeps the result alive
-  } else if (KIND == 1) {
-    if (atomicMin(slot, word) == 1ull) table[0] = 0ull;
-  } else if (KIND == 2) {
-    if (*slot == 1ull) table[0] = 0ull;
-  } else {
-    *slot = word;
-  }
-}
-}  // namespace
-}  // namespace gs
-
 extern "C" {
-
-int gs_probe_random_access(int kind, uint64_t* table, int64_t slots, const uint32_t* keys,
-                           int64_t n, void* stream) {
-  GS_REQUIRE(kind >= 0 && kind <= 3, "gs_probe_random_access: kind must be 0..3, got %d", kind);
-  GS_REQUIRE(table && keys && n >= 0 && slots >= 1 && slots <= (int64_t(1) << 32) &&
-                 (slots & (slots - 1)) == 0,
-             "gs_probe_random_access: null pointer or a slot count that is not a power of two");
-  if (n == 0) return GS_OK;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  unsigned long long* t = reinterpret_cast<unsigned long long*>(table);
-  const uint32_t mask = static_cast<uint32_t>(slots - 1);
-  const dim3 grid(blocks_for(n, kThreads)), block(kThreads);
-  switch (kind) {
-    case 0: hipLaunchKernelGGL(probe_kernel<0>, grid, block, 0, st, t, mask, keys, n); break;
-    case 1: hipLaunchKernelGGL(probe_kernel<1>, grid, block, 0, st, t, mask, keys, n); break;
-    case 2: hipLaunchKernelGGL(probe_kernel<2>, grid, block, 0, st, t, mask, keys, n); break;
-    default: hipLaunchKernelGGL(probe_kernel<3>, grid, block, 0, st, t, mask, keys, n); break;
-  }
-  return check_launch("probe_random_access");
-}
 
 size_t gs_unique_workspace_bytes(int64_t M) {
   if (M < 0) M = 0;
@@ -1421,6 +1385,7 @@ int gs_layer_table_sweep(void* table, size_t table_bytes, const void* workspace,
   }
   if (M_bound == 0) return GS_OK;
   const RankCounts n{S_bound, S_dev, capacity, num_edges};
+  ProfileScope prof("layer_sweep", static_cast<hipStream_t>(stream));
   hipLaunchKernelGGL(layer_sweep_kernel, dim3(blocks_for(M_bound, kThreads)), dim3(kThreads), 0,
                      static_cast<hipStream_t>(stream), t, pos, n);
   return check_launch("layer_table_sweep");

@@ -82,8 +82,9 @@ typedef struct gs_mailbox {
  * reference).  gs_profile_enable("name") makes every later launch of that site
  * record a hipEvent pair on its stream (up to 4096 launches); NULL or ""
  * disables.  Sites: "sample_fused", "sample_floyd", "table_init", "table_insert",
- * "unique_compact", "unique_finish", "scan_tile_sums", "scan_apply", "random_walk",
- * "metapath_walk", "sddmm_dot".  gs_profile_collect waits for the recorded
+ * "unique_compact", "unique_finish", "layer_sample", "layer_relabel", "layer_sweep",
+ * "batch_init", "batch_insert", "batch_compact", "batch_finish", "scan_tile_sums",
+ * "scan_apply", "random_walk", "metapath_walk", "sddmm_dot".  gs_profile_collect waits for the recorded
  * events, returns their summed duration and count (and, when per_launch_ms is
  * given, the first `cap` individual durations in launch order) and clears the
  * ring.  The events are created by the library and live until the process ends. */
@@ -93,13 +94,6 @@ int gs_profile_enable(const char* launch_site);
  * are themselves that short. */
 int gs_profile_stride(int every);
 int gs_profile_collect(double* total_ms, int64_t* launches, double* per_launch_ms, int64_t cap);
-
-/* Memory-system probe for benchmarks (no counterpart in the reference): n accesses of 8 bytes
- * at hashed positions of a table of `slots` 64-bit words (a power of two), one per key, so
- * that the rates of the hash-table kernels can be read against what the memory system gives:
- * kind 0 = compare-and-swap, 1 = atomic minimum, 2 = plain read, 3 = plain write. */
-int gs_probe_random_access(int kind, uint64_t* table, int64_t slots, const uint32_t* keys,
-                           int64_t n, void* stream);
 
 typedef enum gs_op {
   GS_OP_ADD = 0, GS_OP_SUB = 1, GS_OP_MUL = 2, GS_OP_DIV = 3,
