@@ -287,3 +287,156 @@ def test_segment_sums_and_column_expansion_full_size(dev, sage_graph):
     picks = torch.randint(0, E, (1_000_000,), generator=gen, device=dev)
     want = w[picks].double() / torch.segment_reduce(w.double(), "sum", lengths=lens, initial=0.0)[seg[picks]]
     assert float(((norm[picks].double() - want).abs() / want).max()) < 1e-5
+
+
+# ------------------------------------------------ configuration 5: 111 M nodes / 1.6 B edges
+LARGE_NODES, LARGE_EDGES = 111_000_000, 1_600_000_000
+
+
+@pytest.fixture(scope="module")
+def large_graph(dev):
+    """R-MAT 111 M nodes / 1.6 B edges, int64 offsets, int32 ids, 64-d fp32 node features
+    (0.89 + 6.4 + 28.4 GB on the device; nothing of it is copied to the host)."""
+    free, _ = torch.cuda.mem_get_info(dev)
+    if free < 120 * (1 << 30):
+        pytest.skip("needs about 120 GB of free device memory (graph, features, generator scratch)")
+    indptr, indices = rmat.rmat_csc(LARGE_NODES, LARGE_EDGES, seed=0, device=dev,
+                                    index_dtype=torch.int32)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(3)
+    features = torch.rand(LARGE_NODES, 64, generator=gen, device=dev) - 0.5
+    yield indptr, indices, features
+    del indptr, indices, features
+    torch.cuda.empty_cache()
+
+
+def _oracle_layer(indptr, indices, cols_dev, h_cols, k, seed):
+    """One layer by the oracle on the columns' own small graph (tests/util.py)."""
+    from tests.util import columns_as_a_graph
+    h_ptr, h_idx = columns_as_a_graph(indptr, indices, cols_dev)
+    sp, _, rows, _ = O.sample_uniform(h_ptr, h_idx, np.arange(h_cols.size, dtype=np.int64), k,
+                                      False, seed=seed, with_coo=False)
+    frontier, (renamed,) = O.relabel([h_cols, rows], [rows])
+    return sp, rows, frontier, renamed
+
+
+def test_large_graph_minibatch_relabel_and_u_dot_v(dev, large_graph):
+    """Configuration 5 through the calls of the reference's samplers: per layer the fused slice +
+    sample of 1024 seeds' frontier, u_dot_v of the 64-d features on the sampled block
+    (examples/as-gcn/train_minibatch.py:39-41 computes its attention the same way: source
+    features by global row id, destination features by column), then Relabel.  Ids are bit-exact
+    against the oracle, the dot products within 1e-5 of a torch gather-and-dot."""
+    indptr, indices, features = large_graph
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(indptr, indices)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2)
+    seeds = torch.randperm(LARGE_NODES, generator=gen, device=dev)[:1024].to(torch.int32)
+    h_seeds = _host(seeds)
+    torch.ops.gs_ops._CAPI_SetSeed(900)
+    total = 0
+    for l, k in enumerate(FANOUTS):
+        sub = g._CAPI_FusedColumnwiseSlicingSampling(seeds, k, False)
+        sp, rows, want_frontier, want_idx = _oracle_layer(indptr, indices, seeds, h_seeds, k, 900 + l)
+        E = sub._CAPI_GetNumEdges()
+        assert E == rows.size
+        out = torch.zeros(E, 1, device=dev)
+        rhs = features[seeds.long()]
+        sub._CAPI_SDDMM("dot", features, rhs, out, 0, 2, _CSC)
+        got_ptr, got_rows = sub._CAPI_GetCSC()[:2]
+        assert np.array_equal(_host(got_ptr), sp) and np.array_equal(_host(got_rows), rows)
+        col = torch.repeat_interleave(torch.arange(seeds.numel(), device=dev),
+                                      got_ptr[1:] - got_ptr[:-1])
+        want = (features[got_rows.long()] * rhs[col]).sum(-1, keepdim=True)
+        assert torch.allclose(out, want, rtol=1e-5, atol=1e-6)
+        frontier, n_src, n_dst, ptr, idx, e_ids, fmt = sub._CAPI_Relabel()
+        assert fmt == "csc" and n_dst == h_seeds.size and n_src == want_frontier.size
+        assert np.array_equal(_host(ptr), sp)
+        assert np.array_equal(_host(idx), want_idx)
+        assert np.array_equal(_host(frontier), want_frontier)
+        total += E
+        seeds, h_seeds = frontier, want_frontier
+    assert total > 100_000  # a real minibatch: about 150 k sampled edges on this graph
+
+
+def test_large_graph_whole_minibatch_call_and_block_sddmm(dev, large_graph):
+    """The same configuration through one _CAPI_SampleLayers call (every layer queued on the
+    device), then u_dot_v on each relabelled block with the features gathered by the frontier."""
+    indptr, indices, features = large_graph
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(indptr, indices)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(12)
+    for rep in range(2):
+        seeds = torch.randperm(LARGE_NODES, generator=gen, device=dev)[:1024].to(torch.int32)
+        torch.ops.gs_ops._CAPI_SetSeed(40 + 3 * rep)
+        parts = g._CAPI_SampleLayers(seeds, list(FANOUTS), False)
+        cols, h_cols = seeds, _host(seeds)
+        for l, k in enumerate(FANOUTS):
+            frontier, offsets, renamed = parts[3 * l:3 * l + 3]
+            sp, rows, want_frontier, want_idx = _oracle_layer(indptr, indices, cols, h_cols, k,
+                                                              40 + 3 * rep + l)
+            assert np.array_equal(_host(offsets), sp)
+            assert np.array_equal(_host(renamed), want_idx)
+            assert np.array_equal(_host(frontier), want_frontier)
+            h = features[frontier.long()]
+            out = torch.zeros(renamed.numel(), 1, device=dev)
+            capi.sddmm_csc("dot", offsets, renamed, None, None, h, h[:offsets.numel() - 1], out,
+                           0, 2, 64, 64, 1, 64)
+            col = torch.repeat_interleave(torch.arange(offsets.numel() - 1, device=dev),
+                                          offsets[1:] - offsets[:-1])
+            want = (features[torch.from_numpy(rows).to(dev)] * features[cols.long()][col]).sum(-1, keepdim=True)
+            assert torch.allclose(out, want, rtol=1e-5, atol=1e-6)
+            cols, h_cols = frontier, want_frontier
+
+
+def test_large_graph_sampler_and_walk_properties(dev, large_graph):
+    """2^18 columns of the 1.6 B-edge graph (positions beyond 2^31 in `indices` occur): counts,
+    positions inside the column, ids read from those positions, distinct positions per row."""
+    indptr, indices, _ = large_graph
+    S, k = 1 << 18, 10
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(9)
+    cols = torch.randint(0, LARGE_NODES, (S,), generator=gen, device=dev).to(torch.int32)
+    sub_indptr, sub, sel, coo = capi.sample_uniform_fused(indptr, indices, cols, k, False, seed=4,
+                                                          with_coo=True)
+    nnz = int(sub_indptr[-1].item())
+    sub, sel, coo = sub[:nnz], sel[:nnz], coo[:nnz].long()
+    c = cols.long()
+    start, deg = indptr[c], indptr[c + 1] - indptr[c]
+    assert torch.equal(sub_indptr[1:] - sub_indptr[:-1], deg.clamp(max=k))
+    assert bool(((sel >= start[coo]) & (sel < start[coo] + deg[coo])).all())
+    assert bool((sel > (1 << 31)).any())
+    assert torch.equal(indices[sel], sub)
+    assert torch.unique(coo * (1 << 31) + (sel - start[coo])).numel() == nnz
+
+
+# ------------------------------------------------ configuration 1 at its exact shape
+def test_config_1_exact_shape_matches_oracle(dev):
+    """R-MAT 2^17 nodes / 2^21 edges, int64 offsets, int32 ids, two layers [10, 5], 512 seeds,
+    relabel per block: through the per-layer calls and through the one-call minibatch."""
+    n = 1 << 17
+    indptr, indices = rmat.rmat_csc(n, 1 << 21, seed=0, device=dev, index_dtype=torch.int32)
+    h_indptr, h_indices = _host(indptr), _host(indices)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(indptr, indices)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2)
+    for rep in range(3):
+        seeds = torch.randperm(n, generator=gen, device=dev)[:512].to(torch.int32)
+        first = 70 + 2 * rep
+        torch.ops.gs_ops._CAPI_SetSeed(first)
+        parts = g._CAPI_SampleLayers(seeds, [10, 5], False)
+        torch.ops.gs_ops._CAPI_SetSeed(first)
+        cols, h_cols = seeds, _host(seeds)
+        for l, k in enumerate((10, 5)):
+            sub = g._CAPI_FusedColumnwiseSlicingSampling(cols, k, False)
+            frontier, n_src, n_dst, ptr, idx, e_ids, fmt = sub._CAPI_Relabel()
+            sp, _, rows, _ = O.sample_uniform(h_indptr, h_indices, h_cols, k, False, seed=first + l,
+                                              with_coo=False)
+            want_frontier, (want_idx,) = O.relabel([h_cols, rows], [rows])
+            for got in ((frontier, ptr, idx), parts[3 * l:3 * l + 3]):
+                assert np.array_equal(_host(got[0]), want_frontier)
+                assert np.array_equal(_host(got[1]), sp)
+                assert np.array_equal(_host(got[2]), want_idx)
+            cols, h_cols = frontier, want_frontier

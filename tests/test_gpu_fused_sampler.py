@@ -73,6 +73,20 @@ def test_fused_tile_boundaries_and_long_lookback(dev, S):
         _cmp(got, O.sample_uniform(indptr, indices, cols, 7, replace, seed=S))
 
 
+@pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("k,replace", [(7, False), (16, False), (32, False), (3, True), (40, True)])
+def test_fused_very_many_columns_take_the_row_per_lane_kernel(dev, idt, k, replace):
+    """From 2^18 columns on, the launch runs one row per lane with an edge-parallel fill; same
+    draws and outputs as below that size (the oracle knows one definition only)."""
+    indptr, indices = rmat_csc_np(1 << 13, 1 << 17, seed=2)
+    S = (1 << 18) + 77
+    cols = np.random.default_rng(k).integers(0, 1 << 13, size=S).astype(np.int64)
+    cols[::1000] = -5
+    d = (to_dev(indptr, dev), to_dev(indices, dev, idt), to_dev(cols, dev, idt))
+    got = _narrow(capi.sample_uniform_fused(*d, k, replace, seed=S + k, with_coo=True))
+    _cmp(got, O.sample_uniform(indptr, indices, cols, k, replace, seed=S + k))
+
+
 def test_fused_equals_two_phase_at_benchmark_shape(dev):
     """Layer-3-like shape: 45k seed columns, fanout 5; the two entry points agree bit for bit."""
     indptr, indices = rmat_csc_np(1 << 16, 1 << 21, seed=4)

@@ -60,3 +60,25 @@ def row_slice_coo_closed_form(key, other, ids):
     mask = np.isin(key, ids)
     renamed = np.array([place[int(v)] for v in key[mask]], dtype=np.int64)
     return renamed, other[mask], np.nonzero(mask)[0].astype(np.int64)
+
+
+def columns_as_a_graph(indptr, indices, cols):
+    """(offsets, neighbour ids) of the columns `cols` of a device CSC as numpy arrays, cut out
+    with plain torch indexing (no library kernel).  The oracle's samplers address a column by
+    its place in the call, so sampling columns 0..len(cols)-1 of this small graph with the same
+    seed gives what sampling `cols` of the whole graph gives: graphs too large to copy to the
+    host are checked this way.  Ids outside the graph count as empty columns."""
+    import torch
+    n = indptr.numel() - 1
+    cols = cols.long()
+    ok = (cols >= 0) & (cols < n)
+    safe = torch.where(ok, cols, torch.zeros_like(cols))
+    starts = indptr[safe]
+    deg = torch.where(ok, indptr[safe + 1] - starts, torch.zeros_like(starts))
+    offsets = torch.zeros(cols.numel() + 1, dtype=torch.int64, device=indptr.device)
+    torch.cumsum(deg, 0, out=offsets[1:])
+    total = int(offsets[-1])
+    owner = torch.repeat_interleave(torch.arange(cols.numel(), device=indptr.device), deg,
+                                    output_size=total)
+    pos = torch.arange(total, device=indptr.device) - offsets[owner] + starts[owner]
+    return offsets.cpu().numpy(), indices[pos].cpu().numpy().astype(np.int64)
