@@ -113,7 +113,7 @@ def build_host(verbose=False):
         # only this library would find no GPU
         "-Wl,--no-as-needed", "-ltorch_hip", "-Wl,--as-needed",
         "-Wl,-rpath," + torch_lib,
-        "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib",
+        "-L/opt/rocm/lib", "-lamdhip64", "-lrocprofiler-sdk-roctx", "-Wl,-rpath,/opt/rocm/lib",
     ]
     _run(link)
     return HOST_LIB
@@ -149,7 +149,34 @@ def build_cpp_check(verbose=False):
     return CPP_CHECK_BIN
 
 
+STAMP = os.path.join(_PKG, "libgs.stamp")
+
+
+def source_hash():
+    """sha256 over every source the two libraries are built from (csrc/, include/)."""
+    import hashlib
+    h = hashlib.sha256()
+    files = sorted(glob.glob(os.path.join(_CSRC, "**", "*"), recursive=True) +
+                   glob.glob(os.path.join(_ROOT, "include", "*.h")))
+    for path in files:
+        if os.path.isfile(path):
+            h.update(os.path.relpath(path, _ROOT).encode())
+            with open(path, "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def built_from_current_sources():
+    """Whether both libraries exist and were built from the sources as they are now (the
+    build leaves the hash of its sources beside the libraries)."""
+    if not (os.path.exists(KERNEL_LIB) and os.path.exists(HOST_LIB) and os.path.exists(STAMP)):
+        return False
+    with open(STAMP) as f:
+        return f.read().strip() == source_hash()
+
+
 def build_all(verbose=False):
+    digest = source_hash()
     libs = [build_kernels(verbose)]
     host = build_host(verbose)
     if host:
@@ -157,6 +184,8 @@ def build_all(verbose=False):
         check = build_cpp_check(verbose)
         if check:
             libs.append(check)
+    with open(STAMP, "w") as f:
+        f.write(digest + "\n")
     return libs
 
 

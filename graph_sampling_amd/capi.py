@@ -215,6 +215,16 @@ def fused_state(nbytes, device):
     return buf, epoch
 
 
+def selftest_lookback(state, epoch, tiles, missing_tile, spin_limit):
+    """gs_selftest_lookback on the caller's state buffer; returns the total as a device scalar."""
+    total = torch.full((1,), -7, dtype=torch.int64, device=state.device)
+    _check(lib().gs_selftest_lookback(_ptr(state), ctypes.c_size_t(state.numel()),
+                                      ctypes.c_uint32(epoch), _i64(tiles), _i64(missing_tile),
+                                      int(spin_limit), _ptr(total), _stream(state.device)),
+           "gs_selftest_lookback")
+    return total
+
+
 class Mailbox:
     """gs_mailbox in pinned host memory plus the host side of the protocol."""
 

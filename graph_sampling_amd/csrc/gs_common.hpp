@@ -442,6 +442,7 @@ struct LookbackState {
   unsigned long long* status;  // one per tile
   unsigned int* error;
   unsigned int epoch;
+  int spin_limit;  // polls of one status word before a tile gives up (kLookbackSpinLimit)
 };
 
 constexpr int kLbValueBits = 48;
@@ -457,6 +458,7 @@ inline LookbackState carve_lookback(Carver& ws, int64_t tiles, unsigned int epoc
   st.error = ws.take<unsigned int>(64);  // first, so that it does not move with the tile count
   st.status = ws.take<unsigned long long>(tiles > 0 ? tiles : 1);
   st.epoch = epoch;
+  st.spin_limit = kLookbackSpinLimit;
   return st;
 }
 
@@ -509,7 +511,7 @@ __device__ __forceinline__ int64_t lookback_wait_inclusive(const LookbackState& 
                                                            unsigned int tile) {
   int polls = 0;
   while (lb_flag(seen, st.epoch) != 2u) {
-    if (++polls > kLookbackSpinLimit) {
+    if (++polls > st.spin_limit) {
       lookback_raise(st);
       return 0;
     }
@@ -544,7 +546,7 @@ __device__ __forceinline__ int64_t lookback_exclusive_prefix(const LookbackState
         const int64_t j = newest - w * kWave - lane;
         int polls = 0;
         while (lb_flag(s[w], st.epoch) == 0) {
-          if (++polls > kLookbackSpinLimit) {
+          if (++polls > st.spin_limit) {
             lookback_raise(st);
             s[w] = before_first;
             break;

@@ -382,6 +382,7 @@ int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, 
                  int64_t* indptr, IdT* out_value, int64_t* perm, void* workspace,
                  size_t workspace_bytes, hipStream_t st) {
   const dim3 ptr_grid(blocks_for(num_keys + 1, kPtrCols));
+  if (E == 0 && !indptr) return GS_OK;
   if (sorted || E == 0) {
     PlainKeys<IdT> keys{key};
     hipLaunchKernelGGL((indptr_from_sorted_kernel<PlainKeys<IdT>>), ptr_grid, dim3(kThreads), 0, st,
@@ -437,9 +438,11 @@ int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, 
   }
   hipLaunchKernelGGL((unpack_gather_kernel<IdT>), dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st,
                      win, idx_bits, value, E, perm, out_value);
-  WordKeys keys{win, idx_bits};
-  hipLaunchKernelGGL((indptr_from_sorted_kernel<WordKeys>), ptr_grid, dim3(kThreads), 0, st, keys, E,
-                     num_keys, indptr);
+  if (indptr) {  // (null: the caller wants the sorted order only)
+    WordKeys keys{win, idx_bits};
+    hipLaunchKernelGGL((indptr_from_sorted_kernel<WordKeys>), ptr_grid, dim3(kThreads), 0, st, keys,
+                       E, num_keys, indptr);
+  }
   return check_launch("coo2csc");
 }
 
@@ -533,7 +536,8 @@ size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys) {
 int gs_coo2csc(const void* key, const void* value, int id_bytes, int64_t E, int64_t num_keys,
                int sorted, int64_t* indptr, void* out_value, int64_t* perm, void* workspace,
                size_t workspace_bytes, void* stream) {
-  GS_REQUIRE(E >= 0 && num_keys >= 0 && indptr, "gs_coo2csc: negative size or null indptr");
+  GS_REQUIRE(E >= 0 && num_keys >= 0, "gs_coo2csc: negative size");
+  GS_REQUIRE(indptr || !sorted, "gs_coo2csc: sorted keys and no indptr leave nothing to do");
   GS_REQUIRE(E == 0 || key, "gs_coo2csc: key is null");
   GS_REQUIRE(sorted || E == 0 || (value && out_value && perm),
              "gs_coo2csc: value/out_value/perm required when the keys are not sorted");

@@ -1451,3 +1451,51 @@ int gs_sample_one_keepdim(const int64_t* indptr, int64_t num_cols, const void* i
 }
 
 }  // extern "C"
+
+// ---- self-test of the bounded wait: the chained scan alone, one tile left out ----
+namespace gs {
+namespace {
+__global__ void __launch_bounds__(kWave) lookback_selftest_kernel(LookbackState lb, int64_t tiles,
+                                                                   int64_t missing,
+                                                                   int64_t* total) {
+  // workgroup b plays tile b, or b + 1 from the missing tile on: that tile's status word is
+  // never written, so its first successor waits for it in vain
+  const int64_t tile = missing >= 0 && static_cast<int64_t>(blockIdx.x) >= missing
+                           ? static_cast<int64_t>(blockIdx.x) + 1
+                           : static_cast<int64_t>(blockIdx.x);
+  if (threadIdx.x == 0) lookback_publish_sum(lb, static_cast<unsigned int>(tile), 1);
+  const int64_t before = lookback_exclusive_prefix(lb, static_cast<unsigned int>(tile), 1);
+  if (tile == tiles - 1 && threadIdx.x == 0) {
+    int64_t t = before + 1;
+    if (__hip_atomic_load(lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) t = -1;
+    *total = t;
+  }
+}
+}  // namespace
+}  // namespace gs
+
+extern "C" int gs_selftest_lookback(void* state, size_t state_bytes, uint32_t epoch, int64_t tiles,
+                                    int64_t missing_tile, int spin_limit, int64_t* total,
+                                    void* stream) {
+  using namespace gs;
+  GS_REQUIRE(state && total && tiles >= 2 && tiles <= (int64_t(1) << 20),
+             "gs_selftest_lookback: null pointer, or tiles outside 2..2^20");
+  GS_REQUIRE(missing_tile >= -1 && missing_tile < tiles - 1,
+             "gs_selftest_lookback: the missing tile must not be the last one");
+  GS_REQUIRE(spin_limit >= 1 && spin_limit <= kLookbackSpinLimit,
+             "gs_selftest_lookback: spin_limit must be in 1..%d", kLookbackSpinLimit);
+  GS_REQUIRE(epoch >= 1 && epoch <= kLbMaxEpoch, "gs_selftest_lookback: epoch must be 1..%u",
+             kLbMaxEpoch);
+  Carver ws(state, state_bytes);
+  LookbackState lb = carve_lookback(ws, tiles, epoch);
+  if (!ws.ok) {
+    set_error_text("gs_selftest_lookback: state needs %zu bytes, 256-byte aligned",
+                   lookback_state_bytes(tiles));
+    return GS_ERR_WORKSPACE;
+  }
+  lb.spin_limit = spin_limit;
+  const unsigned grid = static_cast<unsigned>(missing_tile >= 0 ? tiles - 1 : tiles);
+  hipLaunchKernelGGL(lookback_selftest_kernel, dim3(grid), dim3(kWave), 0,
+                     static_cast<hipStream_t>(stream), lb, tiles, missing_tile, total);
+  return check_launch("selftest_lookback");
+}

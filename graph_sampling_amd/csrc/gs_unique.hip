@@ -552,7 +552,7 @@ __device__ __forceinline__ unsigned long long back_wait(const LookbackState& st,
                                                         unsigned long long seen, uint32_t at) {
   int polls = 0;
   while (((seen >> kBackEpochShift) & kLbMaxEpoch) != st.epoch) {
-    if (++polls > kLookbackSpinLimit) {
+    if (++polls > st.spin_limit) {
       lookback_raise(st);
       return 0ull;
     }

@@ -5,63 +5,65 @@
 namespace gs {
 
 namespace {
-int64_t FeatureLen(const torch::Tensor& t) {
+
+// feature shape of an operand (everything after the node/edge axis), right-aligned to `rank`
+// axes with leading ones
+std::vector<int64_t> FeatureShape(const torch::Tensor& t, int64_t rank) {
+  std::vector<int64_t> shape(static_cast<size_t>(rank), 1);
+  const int64_t have = t.dim() - 1;
+  for (int64_t d = 0; d < have; ++d) shape[rank - have + d] = t.size(1 + d);
+  return shape;
+}
+
+int64_t Product(const std::vector<int64_t>& v) {
   int64_t n = 1;
-  for (int64_t d = 1; d < t.dim(); ++d) n *= t.size(d);
+  for (int64_t x : v) n *= x;
   return n;
 }
 
-// size of feature axis `back` counted from the last one (0 = last); axis 0 of
-// the tensor is the node/edge axis and never broadcasts
-int64_t AxisFromBack(const torch::Tensor& t, int64_t back) {
-  const int64_t d = t.dim() - 1 - back;
-  return d < 1 ? 1 : t.size(d);
-}
 }  // namespace
 
-// Same offsets as the reference's src/bcast.cc:24-75 (NumPy broadcasting of the
-// feature shapes, last axis fastest; `dot` keeps its reduction axis out).
+// Which scalar (for dot: which reduce_size-long vector) of each operand feeds output position
+// i, under NumPy broadcasting of the feature shapes; the table the reference builds in
+// src/bcast.cc:24-75.  Written per output position: i is taken apart into its coordinates
+// (row-major, last axis fastest), and an operand's offset is the row-major index of the same
+// coordinates in its own shape, with 0 on every axis it has only one entry of.
 BcastOff CalcBcastOff(const std::string& op, torch::Tensor lhs, torch::Tensor rhs) {
   BcastOff b;
-  b.lhs_len = FeatureLen(lhs);
-  b.rhs_len = FeatureLen(rhs);
-  b.reduce_size = 1;
-  const bool copy = (op == "copy_lhs" || op == "copy_rhs");
-  bool differs = lhs.dim() != rhs.dim();
-  for (int64_t d = 1; !differs && d < lhs.dim(); ++d) differs = lhs.size(d) != rhs.size(d);
-  b.use_bcast = !copy && differs;
-  const bool dot = (op == "dot");
+  const bool dot = op == "dot";
+  const bool copy = op == "copy_lhs" || op == "copy_rhs";
+  const int64_t rank = std::max(lhs.dim(), rhs.dim()) - 1;
+  std::vector<int64_t> ls = FeatureShape(lhs, rank), rs = FeatureShape(rhs, rank);
+  b.lhs_len = Product(ls);
+  b.rhs_len = Product(rs);
+  b.reduce_size = dot ? lhs.size(lhs.dim() - 1) : 1;
+  b.use_bcast = !copy && (lhs.dim() != rhs.dim() || ls != rs);
   if (!b.use_bcast) {
-    b.out_len = (op == "copy_rhs") ? b.rhs_len : b.lhs_len;
-    if (dot) {
-      b.reduce_size = lhs.size(lhs.dim() - 1);
-      b.out_len /= b.reduce_size;
-    }
+    b.out_len = (op == "copy_rhs" ? b.rhs_len : b.lhs_len) / b.reduce_size;
     return b;
   }
-  const int64_t naxes = std::max(lhs.dim(), rhs.dim()) - 1;
-  int64_t first = 0;
-  if (dot) {
-    b.reduce_size = lhs.size(lhs.dim() - 1);
-    first = 1;
+  if (dot) {  // the reduced axis is not an output axis; offsets count whole vectors
+    ls.pop_back();
+    rs.pop_back();
   }
-  b.lhs_offset.assign(1, 0);
-  b.rhs_offset.assign(1, 0);
-  int64_t out_len = 1, stride_l = 1, stride_r = 1;
-  for (int64_t back = first; back < naxes; ++back) {
-    const int64_t dl = AxisFromBack(lhs, back), dr = AxisFromBack(rhs, back);
-    const int64_t extent = std::max(dl, dr);
-    for (int64_t i = 1; i < extent; ++i) {
-      for (int64_t k = 0; k < out_len; ++k) {
-        b.lhs_offset.push_back(b.lhs_offset[k] + (i < dl ? i * stride_l : 0));
-        b.rhs_offset.push_back(b.rhs_offset[k] + (i < dr ? i * stride_r : 0));
-      }
+  std::vector<int64_t> os(ls.size());
+  for (size_t d = 0; d < ls.size(); ++d) os[d] = std::max(ls[d], rs[d]);
+  b.out_len = Product(os);
+  b.lhs_offset.resize(static_cast<size_t>(b.out_len));
+  b.rhs_offset.resize(static_cast<size_t>(b.out_len));
+  for (int64_t i = 0; i < b.out_len; ++i) {
+    int64_t rest = i, at_l = 0, at_r = 0, step_l = 1, step_r = 1;
+    for (size_t d = os.size(); d-- > 0;) {
+      const int64_t coord = rest % os[d];
+      rest /= os[d];
+      if (coord < ls[d]) at_l += coord * step_l;
+      if (coord < rs[d]) at_r += coord * step_r;
+      step_l *= ls[d];
+      step_r *= rs[d];
     }
-    out_len *= extent;
-    stride_l *= dl;
-    stride_r *= dr;
+    b.lhs_offset[static_cast<size_t>(i)] = at_l;
+    b.rhs_offset[static_cast<size_t>(i)] = at_r;
   }
-  b.out_len = out_len;
   return b;
 }
 

@@ -1,4 +1,5 @@
 #include "graph.h"
+#include "range.h"
 
 #include "bcast.h"
 #include "graph_ops.h"
@@ -128,6 +129,7 @@ void Graph::CSR2DCSC() {
 
 // reference src/graph.cc:585-644
 void Graph::CreateSparseFormat(int64_t format) {
+  Range range("gs::CreateSparseFormat");
   Settle();
   if (format == _COO) {
     if (coo_) return;
@@ -234,6 +236,7 @@ c10::intrusive_ptr<Graph> Graph::SameShape(torch::Tensor data) {
 // ------------------------------------------------------------------ slicing
 c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int64_t on_format,
                                          int64_t output_format, bool relabel) {
+  Range range("gs::Slicing");
   Settle();
   TORCH_CHECK(axis == 0 || axis == 1, "axis must be 0 (columns) or 1 (rows)");
   CreateSparseFormat(on_format);
@@ -342,6 +345,7 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
 c10::intrusive_ptr<Graph> Graph::SampleImpl(int64_t axis, const torch::Tensor* edge_probs,
                                             int64_t fanout, bool replace, int64_t on_format,
                                             int64_t output_format) {
+  Range range("gs::Sampling");
   Settle();
   CreateSparseFormat(on_format);
   const bool on_csc = (axis == 0 && on_format == _CSC);
@@ -402,6 +406,7 @@ void Graph::Settle() {
 
 c10::intrusive_ptr<Graph> Graph::ColumnwiseFusedSlicingAndSampling(torch::Tensor column_index,
                                                                    int64_t fanout, bool replace) {
+  Range range("gs::FusedSlicingSampling");
   Settle();
   TORCH_CHECK(csc_ != nullptr, "fused slicing + sampling needs the CSC format");
   torch::Tensor col_ids = Pick(col_ids_, column_index);
@@ -456,6 +461,7 @@ std::vector<torch::Tensor> Graph::SampleLayersLoop(torch::Tensor seeds,
 
 std::vector<torch::Tensor> Graph::SampleLayers(torch::Tensor seeds, std::vector<int64_t> fanouts,
                                                bool replace) {
+  Range range("gs::SampleLayers");
   auto pending = QueueLayers(seeds, fanouts, replace);
   if (!pending) return SampleLayersLoop(seeds, fanouts, replace);
   try {
@@ -476,6 +482,7 @@ std::vector<torch::Tensor> Graph::SampleLayers(torch::Tensor seeds, std::vector<
 // data follows the position in the parent's indices.
 c10::intrusive_ptr<Graph> Graph::FusedBidirSlicing(torch::Tensor column_seeds,
                                                    torch::Tensor row_seeds) {
+  Range range("gs::FusedBidirSlicing");
   Settle();
   CreateSparseFormat(_CSC);
   auto ret = Child(Pick(col_ids_, column_seeds), Pick(row_ids_, row_seeds), column_seeds.numel(),
@@ -510,6 +517,7 @@ c10::intrusive_ptr<Graph> Graph::BatchFusedBidirSlicing(torch::Tensor column_see
 std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> Graph::BatchSlicing(
     torch::Tensor n_ids, torch::Tensor nid_ptr, int64_t axis, int64_t on_format,
     int64_t output_format, bool relabel, bool encoding) {
+  Range range("gs::BatchSlicing");
   Settle();
   TORCH_CHECK(axis == 0, "batch slicing only suppurt column slicing now");  // src/graph.cc:335
   TORCH_CHECK(on_format == _CSC, "Not Implementatin Error");                // src/graph.cc:364
@@ -597,6 +605,7 @@ std::tuple<torch::Tensor, torch::Tensor> Graph::GetBatchCOO() {
 }
 
 torch::Tensor Graph::RandomWalk(torch::Tensor seeds, int64_t walk_length) {
+  Range range("gs::RandomWalk");
   Settle();
   TORCH_CHECK(csc_ != nullptr, "random walks need the CSC format");
   return FusedRandomWalk(csc_, seeds, walk_length);
@@ -604,6 +613,7 @@ torch::Tensor Graph::RandomWalk(torch::Tensor seeds, int64_t walk_length) {
 
 // --------------------------------------------------------- edge-data operators
 torch::Tensor Graph::Sum(int64_t axis, int64_t powk, int64_t on_format) {
+  Range range("gs::Sum");
   Settle();
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
@@ -622,6 +632,7 @@ torch::Tensor Graph::Sum(int64_t axis, int64_t powk, int64_t on_format) {
 }
 
 c10::intrusive_ptr<Graph> Graph::Normalize(int64_t axis, int64_t on_format) {
+  Range range("gs::Normalize");
   Settle();
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
@@ -636,6 +647,7 @@ c10::intrusive_ptr<Graph> Graph::Normalize(int64_t axis, int64_t on_format) {
 }
 
 c10::intrusive_ptr<Graph> Graph::Divide(torch::Tensor divisor, int64_t axis, int64_t on_format) {
+  Range range("gs::Divide");
   Settle();
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
@@ -650,6 +662,7 @@ c10::intrusive_ptr<Graph> Graph::Divide(torch::Tensor divisor, int64_t axis, int
 }
 
 std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> Graph::EDivUSum(torch::Tensor divisor) {
+  Range range("gs::EDivUSum");
   Settle();
   CreateSparseFormat(_COO);
   torch::Tensor data = DataOrOnes();
@@ -663,6 +676,7 @@ std::tuple<c10::intrusive_ptr<Graph>, torch::Tensor> Graph::EDivUSum(torch::Tens
 // CSR the compressed axis is the row, so 0 and 2 swap (reference src/graph.cc:975-976)
 void Graph::SDDMM(const std::string& op, torch::Tensor lhs, torch::Tensor rhs, torch::Tensor out,
                   int64_t lhs_target, int64_t rhs_target, int64_t on_format) {
+  Range range("gs::SDDMM");
   Settle();
   CreateSparseFormat(on_format);
   const hip::Bcast b = ToDevice(CalcBcastOff(op, lhs, rhs), out);
@@ -684,6 +698,7 @@ void Graph::SDDMM(const std::string& op, torch::Tensor lhs, torch::Tensor rhs, t
 
 // ---------------------------------------------------------------- node queries
 torch::Tensor Graph::AllValidNode() {
+  Range range("gs::AllValidNode");
   Settle();
   TORCH_CHECK(col_ids_.has_value(), "For sampling, col_ids_ is necessary!");
   torch::Tensor rows;
@@ -701,6 +716,7 @@ torch::Tensor Graph::AllValidNode() {
 std::tuple<torch::Tensor, int64_t, int64_t, torch::Tensor, torch::Tensor,
            torch::optional<torch::Tensor>, std::string>
 Graph::Relabel() {
+  Range range("gs::Relabel");
   TORCH_CHECK(col_ids_.has_value(), "For sampling, col_ids_ is necessary!");
   torch::Tensor col_ids = col_ids_.value();
   torch::Tensor frontier;

@@ -1,4 +1,5 @@
 #include "hetero_graph.h"
+#include "range.h"
 
 #include "hip_ops.h"
 
@@ -46,6 +47,7 @@ c10::intrusive_ptr<Graph> HeteroGraph::GetHomoGraph(const std::string& edge_type
 
 torch::Tensor HeteroGraph::MetapathRandomWalkFused(torch::Tensor seeds,
                                                    const std::vector<std::string>& metapath) {
+  Range range("gs::MetapathRandomWalk");
   auto cached = metapath_cache_.find(metapath);
   if (cached == metapath_cache_.end()) {
     std::vector<int64_t> ids;

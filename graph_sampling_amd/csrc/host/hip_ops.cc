@@ -1090,6 +1090,23 @@ std::tuple<torch::Tensor, torch::Tensor, torch::optional<torch::Tensor>> Coo2Csc
   return {indptr, out_value, perm};
 }
 
+std::tuple<torch::Tensor, torch::Tensor> SortValuesByKey(const torch::Tensor& key,
+                                                         const torch::Tensor& value,
+                                                         int64_t num_keys) {
+  const int idb = IdBytes(key, "sort key");
+  TORCH_CHECK(IdBytes(value, "sort value") == idb, "sort key and value differ in dtype");
+  const int64_t E = key.numel();
+  auto out_value = torch::empty({E}, value.options());
+  auto perm = torch::empty({E}, I64(key));
+  if (E == 0) return {out_value, perm};
+  auto ws = Scratch(gs_coo2csc_workspace_bytes(E, num_keys), key);
+  Check(gs_coo2csc(key.data_ptr(), value.data_ptr(), idb, E, num_keys, 0, nullptr,
+                   out_value.data_ptr(), perm.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(),
+                   Stream(key)),
+        "gs_coo2csc");
+  return {out_value, perm};
+}
+
 std::tuple<torch::Tensor, torch::Tensor> ListSampling(const torch::Tensor& data, int64_t k,
                                                       bool replace) {
   const int idb = IdBytes(data, "data");

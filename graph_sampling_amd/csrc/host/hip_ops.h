@@ -204,6 +204,12 @@ torch::Tensor Csc2CooCols(const torch::Tensor& indptr, int64_t nnz, const torch:
 std::tuple<torch::Tensor, torch::Tensor, torch::optional<torch::Tensor>> Coo2Csc(
     const torch::Tensor& key, const torch::Tensor& value, int64_t num_keys, bool sorted);
 
+// {`value` in the stable order of `key` (keys below num_keys), the permutation}: the
+// library's radix sort alone, no offsets built
+std::tuple<torch::Tensor, torch::Tensor> SortValuesByKey(const torch::Tensor& key,
+                                                         const torch::Tensor& value,
+                                                         int64_t num_keys);
+
 std::tuple<torch::Tensor, torch::Tensor> ListSampling(const torch::Tensor& data, int64_t k,
                                                       bool replace);
 std::tuple<torch::Tensor, torch::Tensor> ListSamplingProbs(const torch::Tensor& data,

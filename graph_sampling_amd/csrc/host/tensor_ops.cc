@@ -114,12 +114,14 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchUnique2(torch::Tens
   torch::Tensor unique, unique_ptr, unique_key;
   std::tie(unique, unique_ptr, unique_key) = BatchUnique(data, data_ptr);
   if (unique.numel() == 0) return {unique, unique_ptr, unique_key};
-  // order inside the batches: sort on (batch, value) as one key
+  // order inside the batches: the library's stable radix sort by value, then by batch
   const int64_t span = unique.max().item<int64_t>() + 1;
-  auto wide = unique.to(torch::kInt64) + unique_key.to(torch::kInt64) * span;
-  auto sorted = std::get<0>(torch::sort(wide));
-  return {(sorted - unique_key.to(torch::kInt64) * span).to(unique.scalar_type()), unique_ptr,
-          unique_key};
+  const int64_t batches = unique_ptr.numel() - 1;
+  torch::Tensor by_value, order;
+  std::tie(by_value, order) = hip::SortValuesByKey(unique, unique, span);
+  auto batch_of = unique_key.to(unique.scalar_type()).index({order});
+  auto sorted = std::get<0>(hip::SortValuesByKey(batch_of, by_value, batches));
+  return {sorted, unique_ptr, unique_key};
 }
 
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchUniqueByKey2(torch::Tensor data,

@@ -212,6 +212,17 @@ int gs_sample_uniform_fused_static(const int64_t* indptr, int64_t num_cols, cons
                                    int64_t* select_index, void* coo_col, int64_t capacity,
                                    gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
 
+/* Self-test of the one-launch kernels' bounded wait (no counterpart in the reference; for
+ * test suites, not for the sampling path).  Runs the chained scan of gs_sample_uniform_fused
+ * over `tiles` tiles that each contribute 1, on `state` under `epoch`, with tile
+ * `missing_tile` left out of the launch (-1: none) and a tile giving up after `spin_limit`
+ * polls of a predecessor's status word.  Every workgroup runs to its end whatever is
+ * missing.  *total (device) receives `tiles` when every tile was there, -1 when a wait ran
+ * out; the error word a give-up raises stays in `state` (every later one-launch call on it
+ * reports -1) until the caller zero-fills it. */
+int gs_selftest_lookback(void* state, size_t state_bytes, uint32_t epoch, int64_t tiles,
+                         int64_t missing_tile, int spin_limit, int64_t* total, void* stream);
+
 /* fanout == 1 with replacement through the fused entry: exactly one slot per
  * column, -1 in both outputs for an empty column; sub_indptr = 0..S.  Replaces
  * impl::fusion::FusedCSCColSlicingSamplingOneKeepDimCUDA
@@ -641,7 +652,8 @@ size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys);
 /* Stable counting sort of (key -> value), both id_bytes wide: indptr[num_keys+1],
  * out_value[E], perm[E] (int64; = stable argsort of key, the reference's
  * sort_index).  sorted != 0: only indptr is computed (out_value / perm
- * untouched, may be NULL). */
+ * untouched, may be NULL).  indptr NULL (unsorted keys only): the sort alone, for keys with
+ * no offsets to build (num_keys then only bounds the keys: the sort runs over its bits). */
 int gs_coo2csc(const void* key, const void* value, int id_bytes, int64_t E, int64_t num_keys,
                int sorted, int64_t* indptr, void* out_value, int64_t* perm, void* workspace,
                size_t workspace_bytes, void* stream);

@@ -12,13 +12,24 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+BUILD_MODE = "unknown"
+
+
 def pytest_sessionstart(session):
-    """The tests load the libraries that are built; only when there are none do they build."""
-    pkg = os.path.join(ROOT, "graph_sampling_amd")
-    if all(os.path.exists(os.path.join(pkg, name)) for name in ("libgs_hip.so", "libgs.so")):
-        return
+    """The tests load the libraries that are built, as long as they were built from the sources
+    as they are now (the build leaves a hash of csrc/ and include/ beside them); when the
+    libraries are missing or stale they are built first."""
+    global BUILD_MODE
     from graph_sampling_amd import build
+    if build.built_from_current_sources():
+        BUILD_MODE = "prebuilt libraries, source hash %s" % build.source_hash()[:16]
+        return
     build.build_all()
+    BUILD_MODE = "built at session start, source hash %s" % build.source_hash()[:16]
+
+
+def pytest_report_header(config):
+    return "graph_sampling_amd native libraries: " + BUILD_MODE
 
 
 @pytest.fixture(scope="session")

@@ -256,3 +256,35 @@ def test_relabel_sampled_narrow_slots_for_64_bit_ids(dev):
     torch.cuda.synchronize()
     # the sticky error word of the look-back state must not leak into later calls of this process
     capi._fused_state.clear()
+
+
+def test_bounded_wait_gives_up_and_the_error_sticks_until_the_state_is_cleared(dev):
+    """The chained scan's wait for a predecessor is bounded.  gs_selftest_lookback leaves one tile
+    out of the launch (every workgroup that does run reaches its end): the tiles behind it give
+    up after the spin limit, the total reads -1, and the error word stays in the state -- a
+    complete scan and the sampler itself report -1 on it -- until the state is zero-filled."""
+    indptr, indices = rmat_csc_np(1 << 10, 1 << 14, seed=3)
+    cols = np.random.default_rng(1).integers(0, 1 << 10, size=700).astype(np.int64)
+    d = (to_dev(indptr, dev), to_dev(indices, dev), to_dev(cols, dev))
+    want = O.sample_uniform(indptr, indices, cols, 3, False, seed=5, with_coo=False)
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    state = torch.zeros(1 << 16, dtype=torch.uint8, device=dev)
+    saved = capi._fused_state.get(key)
+    try:
+        assert int(capi.selftest_lookback(state, 1, 700, -1, 1 << 20)) == 700
+        for missing in (0, 5, 698):
+            state.zero_()
+            assert int(capi.selftest_lookback(state, 2, 700, missing, 48)) == -1
+        assert int(capi.selftest_lookback(state, 3, 700, -1, 1 << 20)) == -1      # sticky
+        capi._fused_state[key] = (state, 3)
+        got = capi.sample_uniform_fused(*d, 3, False, seed=5)
+        assert int(got[0][-1]) == -1                                                # sticky
+        state.zero_()
+        capi._fused_state[key] = (state, 0)
+        _cmp(_narrow(capi.sample_uniform_fused(*d, 3, False, seed=5)), want)
+        assert int(capi.selftest_lookback(state, 9, 700, -1, 1 << 20)) == 700
+    finally:
+        if saved is None:
+            capi._fused_state.pop(key, None)
+        else:
+            capi._fused_state[key] = saved
