@@ -183,6 +183,16 @@ def main():
         lambda: capi.random_walk(indptr, indices, starts, 80, seed=3),
         lambda o: (int((o[1_000_000:] >= 0).sum().item()) * 28,
                    int((o[1_000_000:] >= 0).sum().item()), "steps"))
+    if not only or "random_walk_4M_200M" in only:
+        # the walk configuration's own graph: R-MAT 4 M nodes / 200 M edges
+        w_ptr, w_idx = rmat.rmat_csc(4_000_000, 200_000_000, seed=0, device=dev, index_dtype=idt)
+        w_starts = rand_ids(1_000_000, 4_000_000)
+        run("random_walk_4M_200M", "gs_random_walk: 1M walkers x 80 steps on R-MAT 4M nodes / 200M "
+            "edges (the walk configuration's graph); 28 B per live step",
+            lambda: capi.random_walk(w_ptr, w_idx, w_starts, 80, seed=3),
+            lambda o: (int((o[1_000_000:] >= 0).sum().item()) * 28,
+                       int((o[1_000_000:] >= 0).sum().item()), "steps"))
+        del w_ptr, w_idx
     if not only or "metapath_walk" in only:
         # three bipartite relations (1M x 2M nodes, 50M edges each), metapath of 4 repeated 4 times
         rels = [rmat.rmat_csc(2_000_000, 50_000_000, seed=30 + r, device=dev, index_dtype=idt,

@@ -91,6 +91,7 @@ def build_host(verbose=False):
     abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
     flags = ["-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
              "-D_GLIBCXX_USE_CXX11_ABI=%d" % abi, "-Wno-deprecated-declarations"]
+    flags += os.environ.get("GS_HOST_CXXFLAGS", "").split()
     objs, procs = [], []
     for src in srcs:
         obj = os.path.join(objdir, "host_" + os.path.basename(src) + ".o")

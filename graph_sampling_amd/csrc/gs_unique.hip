@@ -562,6 +562,25 @@ __device__ __forceinline__ unsigned long long back_wait(const LookbackState& st,
   return seen;
 }
 
+// workgroup `part` of `parts` empties its share of the slots a layer's items went to
+__device__ __forceinline__ void sweep_slots(const PackedTable& t, const uint32_t* __restrict__ pos,
+                                            const RankCounts& n, unsigned int part,
+                                            unsigned int parts) {
+  int64_t S, M;
+  n.get(&S, &M);
+  const int64_t g = static_cast<int64_t>(part) * kThreads + threadIdx.x;
+  const int64_t stride = static_cast<int64_t>(parts) * kThreads;
+  constexpr int kInFlight = 8;  // slot numbers a lane reads before it stores
+  for (int64_t j = g; j < M; j += kInFlight * stride) {
+    uint32_t slot[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) slot[u] = j + u * stride < M ? pos[j + u * stride] : 0u;
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u)
+      if (j + u * stride < M) t.clear(slot[u] & t.mask);
+  }
+}
+
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads) rank_linked_kernel(RankArgs<IdT> a) {
   __shared__ int64_t s_scan[kThreads / kWave + 1];
@@ -582,7 +601,16 @@ __global__ void __launch_bounds__(kThreads) rank_linked_kernel(RankArgs<IdT> a) 
   a.n.get(&S, &M);
   const int64_t live = (M + kCompactTile - 1) / kCompactTile;
   const unsigned int tiles = static_cast<unsigned int>(live > 0 ? live : 1);
-  if (tile >= tiles) return;
+  // The launch is sized for the bound, so most of its workgroups usually have no items: those
+  // empty the slots of the earlier layer while the others work.  Only when too few are idle
+  // do the working ones share that job, at their ends.
+  const unsigned int idle = gridDim.x - tiles;
+  const bool idle_sweep = idle * 4u >= tiles;
+  if (tile >= tiles) {
+    if (a.prev_pos && idle_sweep)
+      sweep_slots(a.prev_t, a.prev_pos, a.prev_n, tile - tiles, idle);
+    return;
+  }
   GS_STAMP(1);  // slot numbers and counts are here
   unsigned long long w[kCompactItems];
 #pragma unroll
@@ -679,13 +707,7 @@ __global__ void __launch_bounds__(kThreads) rank_linked_kernel(RankArgs<IdT> a) 
     *a.num_unique = total;
     post_mailbox(a.box, total, a.box_ticket);
   }
-  if (a.prev_pos) {
-    int64_t pS, pM;
-    a.prev_n.get(&pS, &pM);
-    const int64_t g = static_cast<int64_t>(tile) * kThreads + threadIdx.x;
-    for (int64_t j = g; j < pM; j += static_cast<int64_t>(tiles) * kThreads)
-      a.prev_t.clear(a.prev_pos[j] & a.prev_t.mask);
-  }
+  if (a.prev_pos && !idle_sweep) sweep_slots(a.prev_t, a.prev_pos, a.prev_n, tile, tiles);
   GS_STAMP(6);
   GS_STAMP_END(5, 7);
 }

@@ -4,14 +4,20 @@
 // profiler attached a range is two calls into a library that has no subscriber.
 #pragma once
 
+#ifndef GS_NO_RANGES
 #include <rocprofiler-sdk-roctx/roctx.h>
+#endif
 
 namespace gs {
 
 class Range {
  public:
+#ifndef GS_NO_RANGES
   explicit Range(const char* name) { roctxRangePushA(name); }
   ~Range() { roctxRangePop(); }
+#else
+  explicit Range(const char*) {}
+#endif
   Range(const Range&) = delete;
   Range& operator=(const Range&) = delete;
 };
