@@ -47,28 +47,40 @@ def kernel_sources():
     return sorted(glob.glob(os.path.join(_CSRC, "*.hip"))) + [os.path.join(_CSRC, "gs_api.cpp")]
 
 
-def build_kernels(verbose=False):
+STAMPS_LIB = os.path.join(_PKG, "libgs_hip_stamps.so")
+
+
+def build_stamps(verbose=False):
+    """The measuring build of the kernel library: the same sources with -DGS_PHASE_STAMPS, which
+    compiles wall-clock marks into the minibatch kernels (graph_sampling_amd/phase_stamps.py
+    reads them).  Never loaded by the package itself."""
+    return build_kernels(verbose, extra_flags=("-DGS_PHASE_STAMPS",), out=STAMPS_LIB,
+                         objdir=os.path.join(_PKG, "build", "stamps"))
+
+
+def build_kernels(verbose=False, extra_flags=(), out=None, objdir=None):
     """Compile every HIP translation unit for gfx950 and link libgs_hip.so."""
-    objdir = os.path.join(_PKG, "build")
+    out = out or KERNEL_LIB
+    objdir = objdir or os.path.join(_PKG, "build")
     os.makedirs(objdir, exist_ok=True)
     objs = []
     procs = []
     for src in kernel_sources():
         obj = os.path.join(objdir, os.path.basename(src) + ".o")
         objs.append(obj)
-        cmd = [HIPCC] + HIP_FLAGS + ["-x", "hip", "-c", src, "-o", obj]
+        cmd = [HIPCC] + HIP_FLAGS + list(extra_flags) + ["-x", "hip", "-c", src, "-o", obj]
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
                                             text=True)))
     for cmd, p in procs:
-        out, _ = p.communicate()
-        out = "\n".join(l for l in out.splitlines()
+        log, _ = p.communicate()
+        log = "\n".join(l for l in log.splitlines()
                         if "is not a recognized feature for this target" not in l)
         if p.returncode != 0:
-            raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
-        if verbose and out.strip():
-            print(out)
-    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", KERNEL_LIB] + objs)
-    return KERNEL_LIB
+            raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), log))
+        if verbose and log.strip():
+            print(log)
+    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", out] + objs)
+    return out
 
 
 def host_sources():
@@ -191,5 +203,8 @@ def build_all(verbose=False):
 
 
 if __name__ == "__main__":
-    for lib in build_all(verbose="-v" in sys.argv):
-        print("built", lib)
+    if "--stamps" in sys.argv:
+        print("built", build_stamps(verbose="-v" in sys.argv))
+    else:
+        for lib in build_all(verbose="-v" in sys.argv):
+            print("built", lib)
