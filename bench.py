@@ -327,7 +327,8 @@ def saturated(torch, graph, timer, nodes, idt, dev, b):
     timer.enable("")
     t = min(per[1:]) * 1e-3
     achieved = sample_bytes(b, S, E, 0) / t / 1e9
-    return {"kernel": SITE_KERNEL["sample_fused"], "seeds": S, "fanout": 10, "sampled_edges": E,
+    return {"kernel": "sample_row_lane_kernel (the one-launch sampler from 2^18 columns on: one row "
+                      "per lane, edge-parallel fill)", "seeds": S, "fanout": 10, "sampled_edges": E,
             "launch_us": t * 1e6, "achieved": achieved, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS}
 

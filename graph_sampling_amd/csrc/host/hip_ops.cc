@@ -640,13 +640,23 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
   std::vector<int64_t> S(L + 1);
   S[0] = seeds.numel();
   for (int64_t l = 0; l < L; ++l) S[l + 1] = S[l] * (1 + fanouts[l]);
-  // one allocation for what no caller sees: per layer the sampled ids before renaming, the
-  // items' table slots and the two counts
-  std::vector<size_t> off_ids(L), off_ws(L), ws_bytes(L), off_counts(L);
+  // ONE allocation for the whole minibatch, made before the first launch: per layer the
+  // three outputs at their bounds (offsets, renamed ids, frontier) and what no caller sees (the
+  // sampled ids before renaming, the items' table slots, the two counts).  The output tensors
+  // are cut out of it after the last launch, while the device is already at work.
+  std::vector<size_t> off_ids(L), off_ws(L), ws_bytes(L), off_counts(L), off_offsets(L),
+      off_renamed(L), off_frontier(L);
   size_t bytes = 0, state_bytes = 0;
   for (int64_t l = 0; l < L; ++l) {
+    const size_t cap = static_cast<size_t>(S[l] * fanouts[l]);
+    off_offsets[l] = bytes;
+    bytes += Pad256(static_cast<size_t>(S[l] + 1) * 8);
+    off_renamed[l] = bytes;
+    bytes += Pad256(cap * idb);
+    off_frontier[l] = bytes;
+    bytes += Pad256((static_cast<size_t>(S[l]) + cap) * idb);
     off_ids[l] = bytes;
-    bytes += Pad256(static_cast<size_t>(S[l] * fanouts[l]) * idb);
+    bytes += Pad256(cap * idb);
     ws_bytes[l] = gs_layer_workspace_bytes(S[l], fanouts[l]);
     off_ws[l] = bytes;
     bytes += Pad256(ws_bytes[l]);
@@ -667,9 +677,8 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
   for (int64_t l = 0; l < L; ++l) {
     PendingLayers::Layer& y = p->layers[l];
     const int64_t cap = S[l] * fanouts[l];
-    y.offsets = torch::empty({S[l] + 1}, I64(indptr));
-    y.renamed = torch::empty({cap}, indices.options());
-    y.frontier = torch::empty({S[l] + cap}, indices.options());
+    int64_t* offsets = reinterpret_cast<int64_t*>(base + off_offsets[l]);
+    void* frontier = base + off_frontier[l];
     int64_t* counts = reinterpret_cast<int64_t*>(base + off_counts[l]);
     void* table = tables->buf[l & 1].data_ptr();
     const size_t table_bytes = tables->buf[l & 1].numel();
@@ -680,7 +689,7 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
     y.ticket_edges = boxes.next++;
     Check(gs_layer_sample(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), cols,
                           idb, S[l], S_dev, fanouts[l], replace ? 1 : 0, seed, nullptr, nullptr,
-                          y.offsets.data_ptr<int64_t>(), base + off_ids[l], cap, counts, table,
+                          offsets, base + off_ids[l], cap, counts, table,
                           table_bytes, base + off_ws[l], ws_bytes[l], st1.buf.data_ptr(),
                           st1.buf.numel(), st1.epoch, boxes.slot(y.ticket_edges), y.ticket_edges,
                           p->stream),
@@ -689,9 +698,8 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
     y.ticket_unique = boxes.next++;
     const bool has_prev = l > 0;
     Check(gs_layer_relabel(
-              idb, S[l], S_dev, cap, counts, y.offsets.data_ptr<int64_t>(), table, table_bytes,
-              base + off_ws[l], ws_bytes[l], y.frontier.data_ptr(), y.renamed.data_ptr(),
-              counts + 1, nullptr, st2.buf.data_ptr(), st2.buf.numel(), st2.epoch,
+              idb, S[l], S_dev, cap, counts, offsets, table, table_bytes, base + off_ws[l],
+              ws_bytes[l], frontier, base + off_renamed[l], counts + 1, nullptr, st2.buf.data_ptr(), st2.buf.numel(), st2.epoch,
               has_prev ? tables->buf[(l - 1) & 1].data_ptr() : nullptr,
               has_prev ? static_cast<size_t>(tables->buf[(l - 1) & 1].numel()) : 0,
               has_prev ? base + off_ws[l - 1] : nullptr, has_prev ? ws_bytes[l - 1] : 0,
@@ -701,7 +709,7 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
               has_prev ? reinterpret_cast<int64_t*>(base + off_counts[l - 1]) : nullptr,
               boxes.slot(y.ticket_unique), y.ticket_unique, p->stream),
           "gs_layer_relabel");
-    cols = y.frontier.data_ptr();
+    cols = frontier;
     S_dev = counts + 1;
   }
   // the last layer's table has no later relabel to empty it
@@ -712,8 +720,31 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
             S[L - 1] * fanouts[L - 1], reinterpret_cast<int64_t*>(base + off_counts[L - 1]),
             p->stream),
         "gs_layer_table_sweep");
+  p->id_type = indices.scalar_type();
+  for (int64_t l = 0; l < L; ++l) {
+    p->layers[l].off_offsets = off_offsets[l];
+    p->layers[l].off_renamed = off_renamed[l];
+    p->layers[l].off_frontier = off_frontier[l];
+  }
   return p;
 }
+
+namespace {
+// `count` elements of `type` starting `byte_offset` bytes into the 1-d byte tensor `base`, as
+// a tensor that shares its storage: what base.narrow(...).view(type) gives, made directly (two
+// trips through the operator dispatcher per output are a tenth of a minibatch's host time)
+torch::Tensor Window(const torch::Tensor& base, size_t byte_offset, int64_t count,
+                     c10::ScalarType type) {
+  const auto meta = c10::scalarTypeToTypeMeta(type);
+  auto t = at::detail::make_tensor<c10::TensorImpl>(c10::Storage(base.storage()), base.key_set(),
+                                                    meta);
+  auto* impl = t.unsafeGetTensorImpl();
+  impl->set_storage_offset(
+      base.storage_offset() + static_cast<int64_t>(byte_offset / meta.itemsize()));
+  impl->set_sizes_contiguous({count});
+  return t;
+}
+}  // namespace
 
 std::vector<torch::Tensor> PendingLayers::Collect() {
   const gs_mailbox* boxes = static_cast<const gs_mailbox*>(ring);
@@ -747,9 +778,9 @@ std::vector<torch::Tensor> PendingLayers::Collect() {
     GaveUp(state_owner, stream, "gs_layer_relabel");
   }
   for (size_t l = 0; l < layers.size(); ++l) {
-    out.push_back(layers[l].frontier.narrow(0, 0, U[l]));
-    out.push_back(layers[l].offsets.narrow(0, 0, S + 1));
-    out.push_back(layers[l].renamed.narrow(0, 0, E[l]));
+    out.push_back(Window(scratch, layers[l].off_frontier, U[l], id_type));
+    out.push_back(Window(scratch, layers[l].off_offsets, S + 1, c10::ScalarType::Long));
+    out.push_back(Window(scratch, layers[l].off_renamed, E[l], id_type));
     S = U[l];
   }
   return out;

@@ -81,11 +81,15 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred
 // as ColSamplingDeferred + RelabelDeferred layer by layer with the seeds NextSeed() hands out.
 struct PendingLayers {
   struct Layer {
-    torch::Tensor frontier, offsets, renamed;  // at their bounds until collected
+    // where the layer's outputs start in `scratch` (bytes); their lengths come with the counts
+    size_t off_frontier = 0, off_offsets = 0, off_renamed = 0;
     int64_t ticket_edges = 0, ticket_unique = 0;
   };
   std::vector<Layer> layers;
-  torch::Tensor scratch;    // sampled ids, slot numbers, counts: kept until collected
+  // the minibatch's one allocation: every layer's outputs at their bounds, the sampled ids
+  // before renaming, slot numbers, counts; the collected tensors are windows of it
+  torch::Tensor scratch;
+  c10::ScalarType id_type = c10::ScalarType::Long;
   torch::Tensor box_owner;  // the pinned ring the tickets go to
   const void* ring = nullptr;
   torch::Tensor state_owner;     // the look-back state of the launches
