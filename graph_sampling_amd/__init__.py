@@ -53,23 +53,34 @@ def set_seed(seed):
     torch.ops.gs_ops._CAPI_SetSeed(int(seed))
 
 
+def _blocks_of(parts, num_layers):
+    from .block import Block
+    blocks = []
+    for l in range(num_layers):
+        frontier, indptr, indices = parts[3 * l:3 * l + 3]
+        blocks.insert(0, Block(frontier.numel(), indptr.numel() - 1, "csc", indptr, indices, frontier))
+    return parts[-3], blocks
+
+
+def sample_layers(matrix, seeds, fanouts, replace=False):
+    """One GraphSAGE-style minibatch in one call of the C++ layer (fused slice + sample, relabel,
+    next seeds = frontier, per layer): what the per-layer loop of the reference's examples does
+    (examples/graphsage/batching.py:125-138), with every layer queued on the device and the
+    sizes collected once.  Returns (input_nodes, [Block, ...] innermost layer first); the draws
+    are those of the loop under the same seed."""
+    load_library()
+    graph = getattr(matrix, "_graph", matrix)
+    return _blocks_of(graph._CAPI_SampleLayers(seeds, list(fanouts), bool(replace)), len(fanouts))
+
+
 def sample_blocks(matrix, seed_sets, fanouts, replace=False, workers=4, seed=0):
     """GraphSAGE-style minibatches sampled side by side by `workers` host threads of the C++
     layer, one stream each (fused slice + sample, relabel, next seeds = frontier, per layer).
     Returns [(input_nodes, [Block, ...] innermost layer first)] in the order of `seed_sets`;
     minibatch i draws with seeds `seed + i * len(fanouts) + layer` whichever thread runs it."""
     import torch
-    from .block import Block
     load_library()
     graph = getattr(matrix, "_graph", matrix)
     flat = torch.ops.gs_ops._CAPI_SampleBlocks(graph, list(seed_sets), list(fanouts), bool(replace),
                                                int(workers), int(seed))
-    out = []
-    for parts in flat:
-        blocks = []
-        for l in range(len(fanouts)):
-            frontier, indptr, indices = parts[3 * l:3 * l + 3]
-            blocks.insert(0, Block(frontier.numel(), indptr.numel() - 1, "csc", indptr, indices,
-                                   frontier))
-        out.append((parts[-3], blocks))
-    return out
+    return [_blocks_of(parts, len(fanouts)) for parts in flat]

@@ -895,6 +895,18 @@ def test_sample_layers_equals_the_layer_loop_and_the_oracle(dev, idt, fanouts, r
             assert torch.equal(a, b)
 
 
+def test_sample_layers_python_helper_returns_blocks(dev):
+    m, indptr, indices, _ = _rmat_matrix(dev, 12, 16, 3)
+    seeds = to_dev(np.arange(100, dtype=np.int64), dev)
+    gs.set_seed(5)
+    nodes, blocks = gs.sample_layers(m, seeds, [4, 3])
+    gs.set_seed(5)
+    want = _oracle_minibatch(indptr, indices, np.arange(100, dtype=np.int64), (4, 3), False, 5)
+    assert np.array_equal(nodes.cpu().numpy(), want[3])
+    assert [b.num_dst_nodes() for b in blocks] == [want[0].size, 100]
+    assert np.array_equal(blocks[1].csc()[1].cpu().numpy(), want[2])
+
+
 def test_sample_layers_on_a_graph_with_column_ids_takes_the_loop(dev):
     indptr, indices = rmat_csc_np(1 << 12, 1 << 16, seed=13)
     col_ids = np.random.default_rng(1).permutation(1 << 12).astype(np.int64)
