@@ -123,12 +123,13 @@ def main():
     # CSC -> CSR of a slice: sort 14M (row, column) pairs by row, stable, with the permutation
     s_rows, s_cols = rand_ids(14_000_000), torch.sort(rand_ids(14_000_000, 45_000)).values.to(idt)
     run("coo2csr_sort", "gs_coo2csc on 14M unsorted edges (stable radix sort by row over 2.45M "
-        "rows + offsets + permutation): one 8-byte word (key, position) per edge read by the "
-        "histogram and read and written by the scatter of each of the 3 passes for 22-bit keys "
-        "(the first reads the b-byte key instead), then permutation and gathered ids written",
+        "rows + offsets + permutation), 3 passes for 22-bit keys: a pass's histogram reads the "
+        "8-byte word (key, position) of every edge (the first pass the b-byte key), the pass "
+        "itself reads word and value and writes them (the last: value, permutation, key), then "
+        "the offsets read the sorted keys",
         lambda: capi.coo2csc(s_rows, s_cols, N, False),
-        lambda o: (14_000_000 * ((2 * b + 8) + 2 * 24 + (8 + 8 + 2 * b)) + N * 8, 14_000_000,
-                   "edges"))
+        lambda o: (14_000_000 * ((b + 2 * b + 8 + b) + (8 + 2 * (8 + b)) + (8 + 8 + b + 8 + 2 * b)
+                                 + b) + N * 8, 14_000_000, "edges"))
 
     # ---- super-batch helpers on a third-layer super-batch (64 x 45k columns, 14M edges) -------
     B = 64

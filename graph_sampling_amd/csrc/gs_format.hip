@@ -253,16 +253,25 @@ struct StoredWords {
   __device__ __forceinline__ unsigned long long operator()(int64_t i) const { return word[i]; }
 };
 
+// A tile of the sort: 256 threads, 16 items each with 4-byte values, 8 with 8-byte values (the
+// tile's words and values pass through LDS on their way out).
+template <typename IdT>
+struct SortTile {
+  static constexpr int kPerThread = sizeof(IdT) == 4 ? 16 : 8;
+  static constexpr int kSize = kThreads * kPerThread;
+  static constexpr int kRounds = kSize / kWaves / kWave;  // rounds of 64 consecutive items per wave
+};
+
 // counts[d * num_blocks + b] = items of tile b with digit d
-template <typename Src>
+template <typename Src, int TILE>
 __global__ void __launch_bounds__(kThreads)
 radix_hist_kernel(Src src, int64_t E, int shift, int64_t num_blocks, int64_t* __restrict__ counts) {
   __shared__ int s_hist[kRadix];
   s_hist[threadIdx.x] = 0;
   __syncthreads();
-  const int64_t base = static_cast<int64_t>(blockIdx.x) * kTile;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * TILE;
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
+  for (int k = 0; k < TILE / kThreads; ++k) {
     const int64_t i = base + k * kThreads + threadIdx.x;
     if (i < E) atomicAdd(&s_hist[digit_of(src(i), shift)], 1);
   }
@@ -275,33 +284,61 @@ struct LoadI64 {
   __device__ __forceinline__ int64_t operator()(int64_t i) const { return p[i]; }
 };
 
-// Stable scatter of one tile.  Items are visited in index order, 256 per round;
-// inside a round the rank of an item among equal digits is (earlier waves'
-// count) + (lower lanes of its wave with the same digit).
-template <typename Src>
+// where the last pass of the sort writes: the values in key order, the permutation, and
+// the sorted keys themselves (for the offsets; null when nobody builds any)
+template <typename IdT>
+struct SortOutputs {
+  IdT* value;
+  int64_t* perm;
+  IdT* key;
+  int idx_bits;
+};
+
+// One pass of the sort over one tile, stable.  A wave owns a quarter of the tile, in index
+// order, and visits it 64 consecutive items at a time: the rank of an item among the equal
+// digits of its round comes from 8 ballots, the count of the wave's earlier rounds from a
+// small LDS table only that wave touches (no workgroup barrier per round).  One barrier
+// later the digits' totals are scanned, every item knows its place in the tile's sorted
+// order and goes there in LDS together with its value; the tile then leaves in that
+// order, so that the items of a digit are written as one run -- coalesced stores, where a
+// scatter straight from registers wrote 8 bytes here and 8 bytes there.
+// The value rides along with its word from the first pass on (read in input order then), so
+// no pass gathers it by position; the LAST pass writes values, permutation and keys instead
+// of words.
+template <typename IdT, typename Src, bool LAST>
 __global__ void __launch_bounds__(kThreads)
-radix_scatter_kernel(Src src, int64_t E, int shift, int64_t num_blocks,
-                     const int64_t* __restrict__ offsets, unsigned long long* __restrict__ out) {
-  __shared__ int64_t s_base[kRadix];
-  __shared__ int s_cnt[kWaves][kRadix];
+radix_pass_kernel(Src src, const IdT* __restrict__ val_in, int64_t E, int shift,
+                  int64_t num_blocks, const int64_t* __restrict__ offsets,
+                  unsigned long long* __restrict__ out, IdT* __restrict__ val_out,
+                  SortOutputs<IdT> last) {
+  using T = SortTile<IdT>;
+  __shared__ unsigned long long s_word[T::kSize];
+  __shared__ IdT s_val[T::kSize];
+  __shared__ int64_t s_base[kRadix];     // where the tile's run of a digit starts in memory
+  __shared__ int s_cnt[kWaves][kRadix];  // per wave: count, then count of the earlier waves
+  __shared__ int s_start[kRadix];        // where the run of a digit starts in the tile
+  __shared__ int s_scan[kWaves];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   s_base[threadIdx.x] = offsets[static_cast<int64_t>(threadIdx.x) * num_blocks + blockIdx.x];
-  const int64_t base = static_cast<int64_t>(blockIdx.x) * kTile;
-  unsigned long long words[kItems];
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
-    const int64_t i = base + k * kThreads + threadIdx.x;
-    words[k] = i < E ? src(i) : 0ull;
+  for (int w = 0; w < kWaves; ++w) s_cnt[w][threadIdx.x] = 0;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * T::kSize;
+  const int64_t wave_base = base + static_cast<int64_t>(wave) * (T::kSize / kWaves);
+  unsigned long long word[T::kRounds];
+  IdT val[T::kRounds];
+#pragma unroll
+  for (int r = 0; r < T::kRounds; ++r) {
+    const int64_t i = wave_base + r * kWave + lane;
+    word[r] = i < E ? src(i) : ~0ull;
+    val[r] = i < E ? val_in[i] : IdT(0);
   }
+  __syncthreads();  // the tables are zero
+  int place[T::kRounds];
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) s_cnt[w][threadIdx.x] = 0;
-    __syncthreads();
-    const int64_t i = base + k * kThreads + threadIdx.x;
-    const bool live = i < E;
-    const int d = live ? digit_of(words[k], shift) : 0;
+  for (int r = 0; r < T::kRounds; ++r) {
+    const bool live = wave_base + r * kWave + lane < E;
+    const int d = digit_of(word[r], shift);
     unsigned long long peers = __ballot(live);
 #pragma unroll
     for (int b = 0; b < kRadixBits; ++b) {
@@ -310,33 +347,59 @@ radix_scatter_kernel(Src src, int64_t E, int shift, int64_t num_blocks,
       peers &= bit ? bal : ~bal;
     }
     const int rank = __popcll(peers & ((1ull << lane) - 1ull));
-    if (live && rank == 0) s_cnt[wave][d] = __popcll(peers);
-    __syncthreads();
-    if (live) {
-      int64_t dst = s_base[d] + rank;
-      for (int w = 0; w < wave; ++w) dst += s_cnt[w][d];
-      out[dst] = words[k];
-    }
-    __syncthreads();
-    int add = 0;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) add += s_cnt[w][threadIdx.x];
-    s_base[threadIdx.x] += add;
-    __syncthreads();
+    const int before = s_cnt[wave][d];  // the wave's earlier rounds (LDS operations of a wave keep their order)
+    place[r] = before + rank;
+    if (live && rank == 0) s_cnt[wave][d] = before + __popcll(peers);
   }
-}
-
-// perm[i] = position the i-th edge of the result had; out[i] = value of that edge
-template <typename IdT>
-__global__ void __launch_bounds__(kThreads)
-unpack_gather_kernel(const unsigned long long* __restrict__ word, int idx_bits,
-                     const IdT* __restrict__ value, int64_t E, int64_t* __restrict__ perm,
-                     IdT* __restrict__ out) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (i >= E) return;
-  const int64_t from = static_cast<int64_t>(word[i] & ((1ull << idx_bits) - 1ull));
-  perm[i] = from;
-  out[i] = value[from];
+  __syncthreads();
+  // digit threadIdx.x: counts of the waves -> counts of the earlier waves, total -> start
+  int total = 0;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    const int c = s_cnt[w][threadIdx.x];
+    s_cnt[w][threadIdx.x] = total;
+    total += c;
+  }
+  int incl = total;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int y = __shfl_up(incl, d, kWave);
+    if (lane >= d) incl += y;
+  }
+  if (lane == kWave - 1) s_scan[wave] = incl;
+  __syncthreads();
+  int start = incl - total;
+  for (int w = 0; w < wave; ++w) start += s_scan[w];
+  s_start[threadIdx.x] = start;
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < T::kRounds; ++r) {
+    if (wave_base + r * kWave + lane < E) {
+      const int d = digit_of(word[r], shift);
+      const int at = s_start[d] + s_cnt[wave][d] + place[r];
+      s_word[at] = word[r];
+      s_val[at] = val[r];
+    }
+  }
+  __syncthreads();
+  const int n = static_cast<int>(E - base < T::kSize ? E - base : T::kSize);
+#pragma unroll
+  for (int k = 0; k < T::kPerThread; ++k) {
+    const int j = k * kThreads + threadIdx.x;
+    if (j < n) {
+      const unsigned long long w = s_word[j];
+      const int d = digit_of(w, shift);
+      const int64_t dst = s_base[d] + (j - s_start[d]);
+      if (LAST) {
+        last.value[dst] = s_val[j];
+        last.perm[dst] = static_cast<int64_t>(w & ((1ull << last.idx_bits) - 1ull));
+        if (last.key) last.key[dst] = static_cast<IdT>(w >> last.idx_bits);
+      } else {
+        out[dst] = w;
+        val_out[dst] = s_val[j];
+      }
+    }
+  }
 }
 
 int bits_for(int64_t n) {  // smallest b with 2^b >= n
@@ -397,10 +460,12 @@ int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, 
                    static_cast<long long>(E), static_cast<long long>(num_keys));
     return GS_ERR_UNSUPPORTED;
   }
-  const int64_t blocks = blocks_for(E, kTile);
+  using T = SortTile<IdT>;
+  const int64_t blocks = blocks_for(E, T::kSize);
   const int64_t table = kRadix * blocks;
   Carver ws(workspace, workspace_bytes);
   unsigned long long* wbuf[2] = {ws.take<unsigned long long>(E), ws.take<unsigned long long>(E)};
+  IdT* vbuf[2] = {ws.take<IdT>(E), ws.take<IdT>(E)};
   int64_t* counts = ws.take<int64_t>(table);
   int64_t* offsets = ws.take<int64_t>(table + 1);
   int64_t* tiles = ws.take<int64_t>(scan_num_tiles(table) + 1);
@@ -409,39 +474,52 @@ int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, 
                    gs_coo2csc_workspace_bytes(E, num_keys));
     return GS_ERR_WORKSPACE;
   }
+  // the sorted keys (for the offsets) land where the last pass would have put its words
+  IdT* sorted_keys = indptr ? reinterpret_cast<IdT*>(wbuf[(passes - 1) & 1]) : nullptr;
+  const SortOutputs<IdT> outs{out_value, perm, sorted_keys, idx_bits};
   const dim3 grid(static_cast<unsigned>(blocks));
   const unsigned long long* win = nullptr;  // null: the first pass reads the caller's keys
+  const IdT* vin = value;
   for (int p = 0; p < passes; ++p) {
     unsigned long long* wout = wbuf[p & 1];
+    IdT* vout = vbuf[p & 1];
     const int shift = idx_bits + p * kRadixBits;
+    const bool last = p == passes - 1;
     if (p == 0) {
       FreshWords<IdT> src{key, idx_bits};
-      hipLaunchKernelGGL((radix_hist_kernel<FreshWords<IdT>>), grid, dim3(kThreads), 0, st, src, E,
-                         shift, blocks, counts);
+      hipLaunchKernelGGL((radix_hist_kernel<FreshWords<IdT>, T::kSize>), grid, dim3(kThreads), 0, st,
+                         src, E, shift, blocks, counts);
     } else {
       StoredWords src{win};
-      hipLaunchKernelGGL((radix_hist_kernel<StoredWords>), grid, dim3(kThreads), 0, st, src, E, shift,
-                         blocks, counts);
+      hipLaunchKernelGGL((radix_hist_kernel<StoredWords, T::kSize>), grid, dim3(kThreads), 0, st, src,
+                         E, shift, blocks, counts);
     }
     LoadI64 f{counts};
     GS_RETURN_IF_ERROR(exclusive_scan(f, table, offsets, tiles, st));
     if (p == 0) {
       FreshWords<IdT> src{key, idx_bits};
-      hipLaunchKernelGGL((radix_scatter_kernel<FreshWords<IdT>>), grid, dim3(kThreads), 0, st, src, E,
-                         shift, blocks, offsets, wout);
+      if (last)
+        hipLaunchKernelGGL((radix_pass_kernel<IdT, FreshWords<IdT>, true>), grid, dim3(kThreads), 0,
+                           st, src, vin, E, shift, blocks, offsets, wout, vout, outs);
+      else
+        hipLaunchKernelGGL((radix_pass_kernel<IdT, FreshWords<IdT>, false>), grid, dim3(kThreads), 0,
+                           st, src, vin, E, shift, blocks, offsets, wout, vout, outs);
     } else {
       StoredWords src{win};
-      hipLaunchKernelGGL((radix_scatter_kernel<StoredWords>), grid, dim3(kThreads), 0, st, src, E,
-                         shift, blocks, offsets, wout);
+      if (last)
+        hipLaunchKernelGGL((radix_pass_kernel<IdT, StoredWords, true>), grid, dim3(kThreads), 0, st,
+                           src, vin, E, shift, blocks, offsets, wout, vout, outs);
+      else
+        hipLaunchKernelGGL((radix_pass_kernel<IdT, StoredWords, false>), grid, dim3(kThreads), 0, st,
+                           src, vin, E, shift, blocks, offsets, wout, vout, outs);
     }
     win = wout;
+    vin = vout;
   }
-  hipLaunchKernelGGL((unpack_gather_kernel<IdT>), dim3(blocks_for(E, kThreads)), dim3(kThreads), 0, st,
-                     win, idx_bits, value, E, perm, out_value);
   if (indptr) {  // (null: the caller wants the sorted order only)
-    WordKeys keys{win, idx_bits};
-    hipLaunchKernelGGL((indptr_from_sorted_kernel<WordKeys>), ptr_grid, dim3(kThreads), 0, st, keys,
-                       E, num_keys, indptr);
+    PlainKeys<IdT> keys{sorted_keys};
+    hipLaunchKernelGGL((indptr_from_sorted_kernel<PlainKeys<IdT>>), ptr_grid, dim3(kThreads), 0, st,
+                       keys, E, num_keys, indptr);
   }
   return check_launch("coo2csc");
 }
@@ -526,9 +604,12 @@ int gs_csc_compress(const int64_t* indptr, int64_t num_cols, int id_bytes, void*
 size_t gs_coo2csc_workspace_bytes(int64_t E, int64_t num_keys) {
   (void)num_keys;
   if (E < 0) E = 0;
-  const int64_t blocks = blocks_for(E, kTile);
+  // sized for the smaller tile (8-byte ids), which has the larger table
+  const int64_t blocks = blocks_for(E, SortTile<int64_t>::kSize);
   const int64_t table = kRadix * blocks;
-  return 2 * padded(static_cast<size_t>(E > 0 ? E : 1) * 8) +  // the sort's words, ping-pong
+  const size_t n = static_cast<size_t>(E > 0 ? E : 1);
+  return 2 * padded(n * 8) +  // the sort's words, ping-pong
+         2 * padded(n * 8) +  // the values riding along, ping-pong
          padded(static_cast<size_t>(table) * 8) + padded(static_cast<size_t>(table + 1) * 8) +
          scan_workspace_bytes(table);
 }

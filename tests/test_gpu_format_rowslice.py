@@ -60,12 +60,14 @@ def test_coo2csc_unsorted_matches_stable_sort(dev, num_keys, E, idt):
 
 @pytest.mark.parametrize("idt", ID_DTYPES)
 @pytest.mark.parametrize("num_keys,E", [(2, 1), (3, 2047), (255, 2048), (256, 2049), (257, 4096),
+                                        (300, 4095), (70000, 4097), (5, 8191), (99, 8193),
                                         (65536, 6000), (65537, 6000), ((1 << 20) + 1, 70000),
                                         (10, 100000), (5000, 300000)])
 def test_coo2csc_sizes_and_skew(dev, num_keys, E, idt):
-    # edge counts around the 2048-edge sort tiles, key counts around the 8-bit digits (1, 2 and
-    # 3 passes), and keys piled on few columns: the offsets of a 256-column workgroup are then
-    # searched in more than the 4096 keys it can stage
+    # edge counts around the sort tiles (2048 edges with 8-byte ids, 4096 with 4-byte ids) and
+    # around a wave's share of a tile, key counts around the 8-bit digits (1, 2 and 3 passes),
+    # and keys piled on few columns: the offsets of a 256-column workgroup are then searched in
+    # more than the 4096 keys it can stage
     rng = np.random.default_rng(num_keys + E)
     key = (rng.random(E) ** 3 * num_keys).astype(np.int64)        # skewed towards the low keys
     key[rng.random(E) < 0.01] = num_keys - 1
@@ -80,6 +82,20 @@ def test_coo2csc_sizes_and_skew(dev, num_keys, E, idt):
     ip2, _, _ = capi.coo2csc(to_dev(key[want_perm], dev, idt), to_dev(value[want_perm], dev, idt),
                              num_keys, True)
     assert np.array_equal(ip2.cpu().numpy(), want_ip)
+
+
+def test_coo2csc_one_key_many_edges_keeps_input_order(dev):
+    """Every edge under the same key (and under two keys at the ends of the digit range): the
+    stable order is the input order, across waves, rounds and tiles."""
+    E = 3 * 4096 + 77
+    value = np.arange(E, dtype=np.int64)[::-1].copy()
+    for keys in (np.zeros(E, dtype=np.int64), np.where(np.arange(E) % 3 == 0, 255, 0)):
+        for idt in ID_DTYPES:
+            ip, val, perm = capi.coo2csc(to_dev(keys, dev, idt), to_dev(value, dev, idt), 256, False)
+            want = np.argsort(keys, kind="stable")
+            assert np.array_equal(perm.cpu().numpy(), want)
+            assert np.array_equal(val.cpu().numpy(), value[want])
+            assert int(ip[-1]) == E
 
 
 @pytest.mark.parametrize("idt", ID_DTYPES)
