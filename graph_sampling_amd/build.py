@@ -80,6 +80,8 @@ def build_kernels(verbose=False, extra_flags=(), out=None, objdir=None):
         if verbose and log.strip():
             print(log)
     _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", out] + objs)
+    if out == KERNEL_LIB and not extra_flags:
+        _stamp("kernels")
     return out
 
 
@@ -129,6 +131,7 @@ def build_host(verbose=False):
         "-L/opt/rocm/lib", "-lamdhip64", "-lrocprofiler-sdk-roctx", "-Wl,-rpath,/opt/rocm/lib",
     ]
     _run(link)
+    _stamp("host")
     return HOST_LIB
 
 
@@ -165,13 +168,10 @@ def build_cpp_check(verbose=False):
 STAMP = os.path.join(_PKG, "libgs.stamp")
 
 
-def source_hash():
-    """sha256 over every source the two libraries are built from (csrc/, include/)."""
+def _hash_of(paths):
     import hashlib
     h = hashlib.sha256()
-    files = sorted(glob.glob(os.path.join(_CSRC, "**", "*"), recursive=True) +
-                   glob.glob(os.path.join(_ROOT, "include", "*.h")))
-    for path in files:
+    for path in sorted(paths):
         if os.path.isfile(path):
             h.update(os.path.relpath(path, _ROOT).encode())
             with open(path, "rb") as f:
@@ -179,17 +179,52 @@ def source_hash():
     return h.hexdigest()
 
 
-def built_from_current_sources():
-    """Whether both libraries exist and were built from the sources as they are now (the
-    build leaves the hash of its sources beside the libraries)."""
-    if not (os.path.exists(KERNEL_LIB) and os.path.exists(HOST_LIB) and os.path.exists(STAMP)):
-        return False
-    with open(STAMP) as f:
-        return f.read().strip() == source_hash()
+def _headers():
+    return glob.glob(os.path.join(_ROOT, "include", "*.h"))
+
+
+def source_hashes():
+    """sha256 over what each library is built from: {"kernels": ..., "host": ...}."""
+    kernels = [p for p in glob.glob(os.path.join(_CSRC, "*")) if os.path.isfile(p)]
+    host = glob.glob(os.path.join(_CSRC, "host", "*"))
+    return {"kernels": _hash_of(kernels + _headers()), "host": _hash_of(host + _headers())}
+
+
+def source_hash():
+    h = source_hashes()
+    return h["kernels"][:8] + h["host"][:8]
+
+
+def _read_stamp():
+    try:
+        with open(STAMP) as f:
+            return dict(line.split() for line in f if len(line.split()) == 2)
+    except OSError:
+        return None
+
+
+def _stamp(which):
+    """Records that library `which` has just been built from the sources as they are."""
+    have = _read_stamp() or {}
+    have[which] = source_hashes()[which]
+    with open(STAMP, "w") as f:
+        for k in sorted(have):
+            f.write("%s %s\n" % (k, have[k]))
+
+
+def build_state():
+    """"current": both libraries exist and were built from the sources as they are now (each
+    build leaves the hash of its sources beside the libraries); "stale": one was built from
+    other sources; "unknown": libraries without hashes beside them; "missing"."""
+    if not (os.path.exists(KERNEL_LIB) and os.path.exists(HOST_LIB)):
+        return "missing"
+    have = _read_stamp()
+    if not have:
+        return "unknown"
+    return "current" if have == source_hashes() else "stale"
 
 
 def build_all(verbose=False):
-    digest = source_hash()
     libs = [build_kernels(verbose)]
     host = build_host(verbose)
     if host:
@@ -197,8 +232,6 @@ def build_all(verbose=False):
         check = build_cpp_check(verbose)
         if check:
             libs.append(check)
-    with open(STAMP, "w") as f:
-        f.write(digest + "\n")
     return libs
 
 

@@ -21,11 +21,15 @@ def pytest_sessionstart(session):
     libraries are missing or stale they are built first."""
     global BUILD_MODE
     from graph_sampling_amd import build
-    if build.built_from_current_sources():
+    state = build.build_state()
+    if state == "current":
         BUILD_MODE = "prebuilt libraries, source hash %s" % build.source_hash()[:16]
-        return
-    build.build_all()
-    BUILD_MODE = "built at session start, source hash %s" % build.source_hash()[:16]
+    elif state == "unknown":
+        BUILD_MODE = "prebuilt libraries with no source hash beside them (not rebuilt)"
+    else:
+        build.build_all()
+        BUILD_MODE = "%s libraries: built at session start, source hash %s" % (
+            state, build.source_hash()[:16])
 
 
 def pytest_report_header(config):
