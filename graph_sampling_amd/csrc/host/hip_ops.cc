@@ -291,6 +291,36 @@ SliceResult SampleInto(const torch::Tensor& indptr, const torch::Tensor& indices
 
 }  // namespace
 
+namespace {
+inline size_t Pad256(size_t n) { return (n + 255) / 256 * 256; }
+
+// `count` elements of `type` starting `byte_offset` bytes into the 1-d byte tensor `base`, as
+// a tensor that shares its storage: what base.narrow(...).view(type) gives, made directly (two
+// trips through the operator dispatcher per output are a tenth of a minibatch's host time)
+torch::Tensor Window(const torch::Tensor& base, size_t byte_offset, int64_t count,
+                     c10::ScalarType type) {
+  const auto meta = c10::scalarTypeToTypeMeta(type);
+  auto t = at::detail::make_tensor<c10::TensorImpl>(c10::Storage(base.storage()), base.key_set(),
+                                                    meta);
+  auto* impl = t.unsafeGetTensorImpl();
+  impl->set_storage_offset(
+      base.storage_offset() + static_cast<int64_t>(byte_offset / meta.itemsize()));
+  impl->set_sizes_contiguous({count});
+  return t;
+}
+
+// One allocation cut into 256-byte aligned pieces: the outputs and the scratch of a call that
+// would otherwise ask the allocator five times.
+struct Pieces {
+  size_t bytes = 0;
+  size_t Add(size_t n) {
+    const size_t at = bytes;
+    bytes += Pad256(n > 0 ? n : 1);
+    return at;
+  }
+};
+}  // namespace
+
 int64_t PendingSample::Wait() const {
   int64_t nnz = WaitBox(static_cast<const gs_mailbox*>(box), ticket, stream, "gs_sample_uniform_fused");
   if (nnz == kLost) nnz = sub_indptr[S].item<int64_t>();
@@ -322,11 +352,19 @@ std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
   TORCH_CHECK(fanout >= 0, "fanout must be non-negative");
   auto p = std::make_shared<PendingSample>();
   p->S = fused ? column_ids.numel() : indptr.numel() - 1;
-  p->sub_indptr = torch::empty({p->S + 1}, I64(indptr));
   const int64_t cap = p->S * fanout;
-  p->indices = torch::empty({cap}, indices.options());
-  if (with_select) p->select_index = torch::empty({cap}, I64(indptr));
-  if (with_coo) p->coo_col = torch::empty({cap}, indices.options());
+  {
+    Pieces at;
+    const size_t o_ptr = at.Add(static_cast<size_t>(p->S + 1) * 8);
+    const size_t o_idx = at.Add(static_cast<size_t>(cap) * idb);
+    const size_t o_sel = with_select ? at.Add(static_cast<size_t>(cap) * 8) : 0;
+    const size_t o_coo = with_coo ? at.Add(static_cast<size_t>(cap) * idb) : 0;
+    auto buf = Scratch(at.bytes, indptr);
+    p->sub_indptr = Window(buf, o_ptr, p->S + 1, torch::kInt64);
+    p->indices = Window(buf, o_idx, cap, indices.scalar_type());
+    if (with_select) p->select_index = Window(buf, o_sel, cap, torch::kInt64);
+    if (with_coo) p->coo_col = Window(buf, o_coo, cap, indices.scalar_type());
+  }
   p->stream = Stream(indptr);
   p->device = indptr.device().index();
   FusedStateBuf& state = FusedState(gs_sample_fused_state_bytes(p->S), indptr, p->stream);
@@ -502,11 +540,20 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred
   const int64_t cap = p.indices.numel();
   const int64_t S = col_ids.numel();
   const int64_t M = S + cap;
-  auto renamed = torch::empty_like(p.indices);
-  auto frontier = torch::empty({M}, col_ids.options());
-  auto num = torch::empty({1}, I64(col_ids));
-  auto offsets_copy = torch::empty_like(p.sub_indptr);
-  auto ws = Scratch(gs_relabel_sampled_workspace_bytes(M), col_ids);
+  Pieces at;
+  const size_t o_renamed = at.Add(static_cast<size_t>(cap) * idb);
+  const size_t o_frontier = at.Add(static_cast<size_t>(M) * idb);
+  const size_t o_num = at.Add(8);
+  const size_t o_offsets = at.Add(static_cast<size_t>(p.sub_indptr.numel()) * 8);
+  const size_t ws_bytes = gs_relabel_sampled_workspace_bytes(M);
+  const size_t o_ws = at.Add(ws_bytes);
+  auto buf = Scratch(at.bytes, col_ids);
+  const auto id_type = col_ids.scalar_type();
+  auto renamed = Window(buf, o_renamed, cap, id_type);
+  auto frontier = Window(buf, o_frontier, M, id_type);
+  auto num = Window(buf, o_num, 1, torch::kInt64);
+  auto offsets_copy = Window(buf, o_offsets, p.sub_indptr.numel(), torch::kInt64);
+  auto ws = Window(buf, o_ws, static_cast<int64_t>(ws_bytes), torch::kUInt8);
   RelabelTable& table = RelabelTableFor(col_ids, p.stream, idb, M);
   FusedStateBuf& state = FusedState(gs_relabel_sampled_state_bytes(M), col_ids, p.stream);
   HostBoxes& boxes = Boxes(p.device);
@@ -549,7 +596,8 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred
   }
   if (U < 0) GaveUp(state.buf, p.stream, "gs_relabel_sampled");  // (the table stays marked)
   table.clean = true;
-  return {frontier.narrow(0, 0, U), renamed.narrow(0, 0, nnz), nnz, offsets_copy};
+  return {Window(buf, o_frontier, U, id_type), Window(buf, o_renamed, nnz, id_type), nnz,
+          offsets_copy};
 }
 
 
@@ -592,8 +640,6 @@ std::shared_ptr<ChainTables> ChainTablesFor(const torch::Tensor& like, void* str
   }
   return t;
 }
-
-inline size_t Pad256(size_t n) { return (n + 255) / 256 * 256; }
 
 }  // namespace
 
@@ -728,23 +774,6 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
   }
   return p;
 }
-
-namespace {
-// `count` elements of `type` starting `byte_offset` bytes into the 1-d byte tensor `base`, as
-// a tensor that shares its storage: what base.narrow(...).view(type) gives, made directly (two
-// trips through the operator dispatcher per output are a tenth of a minibatch's host time)
-torch::Tensor Window(const torch::Tensor& base, size_t byte_offset, int64_t count,
-                     c10::ScalarType type) {
-  const auto meta = c10::scalarTypeToTypeMeta(type);
-  auto t = at::detail::make_tensor<c10::TensorImpl>(c10::Storage(base.storage()), base.key_set(),
-                                                    meta);
-  auto* impl = t.unsafeGetTensorImpl();
-  impl->set_storage_offset(
-      base.storage_offset() + static_cast<int64_t>(byte_offset / meta.itemsize()));
-  impl->set_sizes_contiguous({count});
-  return t;
-}
-}  // namespace
 
 std::vector<torch::Tensor> PendingLayers::Collect() {
   const gs_mailbox* boxes = static_cast<const gs_mailbox*>(ring);
