@@ -895,6 +895,21 @@ def test_sample_layers_equals_the_layer_loop_and_the_oracle(dev, idt, fanouts, r
             assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+def test_sample_layers_with_no_seeds_and_with_isolated_seeds(dev, idt):
+    """No seeds at all, and seeds without neighbours (every later layer is then empty too):
+    lengths 0 all the way, offsets of the right length, no launch goes wrong."""
+    indptr = np.array([0, 0, 2, 2, 3], dtype=np.int64)   # columns 0 and 2 have no edges
+    indices = np.array([3, 1, 1], dtype=np.int64)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev, idt))
+    for seeds in (np.zeros(0, dtype=np.int64), np.array([0, 2], dtype=np.int64),
+                  np.array([1, 3, 0], dtype=np.int64)):
+        gs.set_seed(3)
+        got = g._CAPI_SampleLayers(to_dev(seeds, dev, idt), [2, 2, 2], False)
+        _same(got, _oracle_minibatch(indptr, indices, seeds, (2, 2, 2), False, 3))
+
+
 def test_sample_layers_python_helper_returns_blocks(dev):
     m, indptr, indices, _ = _rmat_matrix(dev, 12, 16, 3)
     seeds = to_dev(np.arange(100, dtype=np.int64), dev)
