@@ -44,6 +44,8 @@ def _check_layers(layers, want):
     (300, (4, 4, 4, 4), True),
     (3000, (32,), False),
     (257, (1, 1, 1), False),
+    (1024, (16, 2), False),
+    (1000, (16,), True),
 ])
 def test_chain_matches_the_oracle_layer_by_layer(dev, idt, num_seeds, fanouts, replace):
     n = 1 << 14
@@ -68,15 +70,17 @@ def test_chain_matches_the_oracle_layer_by_layer(dev, idt, num_seeds, fanouts, r
         assert bool((t.buf.view(torch.int64) == -1).all())
 
 
-def test_chain_with_repeated_seeds_and_hub_columns(dev):
-    """Seeds that repeat (the frontier is shorter than the seed list) and the graph's largest
-    columns among them."""
+@pytest.mark.parametrize("num_seeds", [5000, 1000])
+def test_chain_with_repeated_seeds_and_hub_columns(dev, num_seeds):
+    """Seeds that repeat (the frontier is shorter than the seed list), seeds that the sampled
+    ids name again, and the graph's largest columns among them."""
     n = 1 << 13
     indptr, indices = rmat_csc_np(n, 1 << 18, seed=3)
     rng = np.random.default_rng(8)
-    seeds = rng.integers(0, n, size=5000).astype(np.int64)
+    seeds = rng.integers(0, n, size=num_seeds).astype(np.int64)
     seeds[:16] = np.argsort(np.diff(indptr))[-16:]
     seeds[100:200] = seeds[0]
+    seeds[300:400] = indices[indptr[seeds[0]]:indptr[seeds[0]] + 100]  # neighbours of a hub
     d = (to_dev(indptr, dev), to_dev(indices, dev, torch.int32), to_dev(seeds, dev, torch.int32))
     layers, _ = capi.sample_layers(*d, (6, 3), False, seed=9)
     _check_layers(layers, _oracle_layers(indptr, indices, seeds, (6, 3), False, 9))
