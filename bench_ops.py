@@ -234,7 +234,7 @@ def main():
     row_prob[torch.rand(N, generator=gen, device=dev) < 0.7] = 0.0  # most rows unreachable
     all_rows = torch.arange(N, device=dev, dtype=idt)
     run("list_sample_weighted", "gs_list_sample_weighted: 512 of 2.45M rows without replacement "
-        "(70% of the weights zero); 4 B per row and select level + 16 B per pick",
+        "(70% of the weights zero); 4 B per row (the weight, read once) + 16 B per pick",
         lambda: capi.list_sample_weighted(all_rows, row_prob, 512, seed=3),
         lambda o: (N * 4 + 512 * 16, N, "items"))
     run("list_sample_uniform", "gs_list_sample_uniform: 512 of 2.45M rows without replacement",

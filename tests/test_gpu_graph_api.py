@@ -13,6 +13,11 @@ from tests.util import rmat_csc_np, to_dev
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, scope="module")
+def _ops_library():
+    gs.load_library()  # torch.ops.gs_ops is used directly below, before any gs.Graph is made
+
+
 def I(dev):
     return dict(dtype=torch.int64, device=dev)
 

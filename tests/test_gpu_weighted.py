@@ -180,6 +180,61 @@ def test_list_weighted_massive_ties(dev):
     assert np.array_equal(O.list_sample_weighted(data, probs, k, seed=1)[1], np.arange(k))
 
 
+@pytest.mark.parametrize("n,k,positive", [
+    (300000, 512, 100),     # fewer positive weights than picks: the rest by position
+    (300000, 512, 511),
+    (2500000, 2000, 700),
+    (3000, 2999, 10),
+    (70000, 8192, 8000),    # more picked items above the k-th key's class than one sort holds
+])
+def test_list_weighted_with_few_positive_weights(dev, n, k, positive):
+    rng = np.random.default_rng(n + positive)
+    data = rng.integers(0, 1 << 30, n).astype(np.int64)
+    probs = np.zeros(n, dtype=np.float32)
+    at = rng.permutation(n)[:positive]
+    probs[at] = rng.random(positive, dtype=np.float32) + 1e-3
+    probs[rng.integers(0, n, 50)] = -1.0   # not positive: as good as zero
+    sel, idx = capi.list_sample_weighted(to_dev(data, dev), to_dev(probs, dev), k, seed=5)
+    w_sel, w_idx = O.list_sample_weighted(data, probs, k, seed=5)
+    assert np.array_equal(idx.cpu().numpy(), w_idx)
+    assert np.array_equal(sel.cpu().numpy(), w_sel)
+    # closed form: every positive weight is picked, then the lowest positions without one
+    n_pos = int((probs > 0).sum())
+    assert set(w_idx[:n_pos].tolist()) == set(np.flatnonzero(probs > 0).tolist())
+    assert np.array_equal(w_idx[n_pos:], np.flatnonzero(~(probs > 0))[:k - n_pos])
+
+
+@pytest.mark.parametrize("n,k,distinct", [(60000, 700, 3), (20000, 5000, 1), (100000, 8192, 40)])
+def test_list_weighted_keys_that_repeat_thousands_of_times(dev, n, k, distinct):
+    """Replayed draws that are nearly all alike over equal weights: the class of the k-th key
+    holds far more items than one sort takes, and positions decide inside a key."""
+    rng = np.random.default_rng(n)
+    data = np.arange(n, dtype=np.int64) * 7
+    probs = np.full(n, 0.5, dtype=np.float32)
+    values = rng.integers(1 << 30, 1 << 32, distinct, dtype=np.uint64).astype(np.uint32)
+    replay = values[rng.integers(0, distinct, n)]
+    sel, idx = capi.list_sample_weighted(to_dev(data, dev), to_dev(probs, dev), k,
+                                         replay=to_dev(replay, dev))
+    w_sel, w_idx = O.list_sample_weighted(data, probs, k, replay=replay)
+    assert np.array_equal(idx.cpu().numpy(), w_idx)
+    assert np.array_equal(sel.cpu().numpy(), w_sel)
+    # closed form: equal weights, so the larger draw wins and the position breaks ties
+    order = np.lexsort((np.arange(n), -(replay >> 8).astype(np.int64)))
+    assert np.array_equal(w_idx, order[:k])
+
+
+def test_list_weighted_weights_at_any_alignment(dev):
+    n, k = 100003, 300
+    rng = np.random.default_rng(3)
+    data = rng.integers(0, 1 << 30, n).astype(np.int64)
+    probs = rng.random(n + 3, dtype=np.float32)
+    t_probs = to_dev(probs, dev)
+    for off in (1, 2, 3):
+        sel, idx = capi.list_sample_weighted(to_dev(data, dev), t_probs[off:off + n], k, seed=2)
+        assert np.array_equal(idx.cpu().numpy(),
+                              O.list_sample_weighted(data, probs[off:off + n], k, seed=2)[1])
+
+
 def test_list_weighted_replay(dev):
     n, k = 20000, 300
     rng = np.random.default_rng(8)
