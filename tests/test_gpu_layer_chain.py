@@ -86,6 +86,23 @@ def test_chain_with_repeated_seeds_and_hub_columns(dev, num_seeds):
     _check_layers(layers, _oracle_layers(indptr, indices, seeds, (6, 3), False, 9))
 
 
+def test_chain_with_seeds_that_are_no_columns(dev):
+    """Seeds outside the graph are empty columns in every layer they reach."""
+    n = 1 << 12
+    indptr, indices = rmat_csc_np(n, 1 << 16, seed=5)
+    seeds = np.array([5, -1, n, 17, n + 100, 900, 5], dtype=np.int64)
+    d = (to_dev(indptr, dev), to_dev(indices, dev, torch.int32), to_dev(seeds, dev, torch.int32))
+    layers, _ = capi.sample_layers(*d, (3, 3), False, seed=2)
+    want = _oracle_layers(indptr, indices, seeds, (3, 3), False, 2)
+    for b, (S, sp, si, frontier, renamed) in zip(layers, want):
+        E, U = (int(v) for v in b.counts.cpu())
+        assert (E, U) == (si.size, frontier.size)
+        assert np.array_equal(b.sub_indptr[:S + 1].cpu().numpy(), sp)
+        assert np.array_equal(b.sub_indices[:E].cpu().numpy().astype(np.int64), si)
+        assert np.array_equal(b.frontier[:U].cpu().numpy().astype(np.int32), frontier.astype(np.int32))
+        assert np.array_equal(b.out_ids[:E].cpu().numpy().astype(np.int64), renamed)
+
+
 def test_chain_reports_an_id_beyond_32_bits(dev):
     """64-bit ids ride on one-word slots; one that does not fit is reported as -2, not truncated."""
     indptr = np.array([0, 2, 4, 6], dtype=np.int64)
