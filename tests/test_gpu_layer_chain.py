@@ -87,10 +87,11 @@ def test_chain_with_repeated_seeds_and_hub_columns(dev, num_seeds):
 
 
 def test_chain_with_seeds_that_are_no_columns(dev):
-    """Seeds outside the graph are empty columns in every layer they reach."""
+    """Seeds beyond the graph's last column are empty columns in every layer they reach.  (-1,
+    the reference's mark of an empty table slot, unique_reindex.cu:52-54, is no id to relabel.)"""
     n = 1 << 12
     indptr, indices = rmat_csc_np(n, 1 << 16, seed=5)
-    seeds = np.array([5, -1, n, 17, n + 100, 900, 5], dtype=np.int64)
+    seeds = np.array([5, 1 << 20, n, 17, n + 100, 900, 5], dtype=np.int64)
     d = (to_dev(indptr, dev), to_dev(indices, dev, torch.int32), to_dev(seeds, dev, torch.int32))
     layers, _ = capi.sample_layers(*d, (3, 3), False, seed=2)
     want = _oracle_layers(indptr, indices, seeds, (3, 3), False, 2)
