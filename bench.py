@@ -495,10 +495,10 @@ def main():
     per_step = LAUNCHES_PER_STEP.get(dominant, len(FANOUTS))
 
     torch.ops.gs_ops._CAPI_SetSeed(first_seed)
-    # every 4th launch of the dominant site is bracketed by an event pair: with three
+    # every 7th launch of the dominant site is bracketed by an event pair: with three
     # launches per step that visits the three layers in turn, and keeps the pairs' own
     # queue time (about 6 us each, as long as the kernel) mostly out of the measurement
-    timer.enable(dominant, every=4 if per_step == len(FANOUTS) else 1)
+    timer.enable(dominant, every=7 if per_step == len(FANOUTS) else 1)
     sampled = 0
     layer_sizes = None
     first = None
@@ -506,23 +506,27 @@ def main():
     whole_step_bytes = 0
     torch.cuda.synchronize()
     t_begin = time.perf_counter()
+    all_sizes = []
     for s in timed_sets:
         # a step ends when the host holds every tensor size of the minibatch (the call hands
-        # back tensors of their final lengths); nothing else synchronises inside the loop
+        # back tensors of their final lengths); nothing else synchronises inside the loop,
+        # and the byte counts are made from the sizes afterwards
         n, sizes, parts = step_fn(graph, s)
         sampled += n
-        layer_sizes = sizes
-        if per_step == 1:
-            algo_bytes += SITE_BYTES[api][dominant](b, *sizes[-1])
-        else:
-            algo_bytes += sum(SITE_BYTES[api][dominant](b, *z) for z in sizes)
-        whole_step_bytes += step_bytes(sizes)
+        all_sizes.append(sizes)
         if first is None:
             first = (n, parts)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t_begin
     k_ms, k_launches, _ = timer.collect()
     timer.enable("")
+    layer_sizes = all_sizes[-1]
+    for sizes in all_sizes:
+        if per_step == 1:
+            algo_bytes += SITE_BYTES[api][dominant](b, *sizes[-1])
+        else:
+            algo_bytes += sum(SITE_BYTES[api][dominant](b, *z) for z in sizes)
+        whole_step_bytes += step_bytes(sizes)
 
     # the checker: step 0 of the timed region must agree with the oracle bit for bit
     if O is not None and not check_against_oracle(torch, np, O, indptr, indices, timed_sets[0],
@@ -659,21 +663,24 @@ def main():
     pool = None
     if extras:
         DEPTH = 32
-        ops._CAPI_SampleBlocks(graph, seed_sets[:DEPTH], FANOUTS, False, WORKERS, 0)
+        # three sampler threads: a process has four hardware queues, one of them the null
+        # stream's, and a fourth worker shares a queue with another one
+        POOL = 3
+        ops._CAPI_SampleBlocks(graph, seed_sets[:DEPTH], FANOUTS, False, POOL, 0)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         pool_edges = 0
         for c0 in range(0, len(timed_sets), DEPTH):
-            res = ops._CAPI_SampleBlocks(graph, timed_sets[c0:c0 + DEPTH], FANOUTS, False, WORKERS,
+            res = ops._CAPI_SampleBlocks(graph, timed_sets[c0:c0 + DEPTH], FANOUTS, False, POOL,
                                          c0 * len(FANOUTS))
             pool_edges += sum(int(parts[3 * l + 2].numel()) for parts in res
                               for l in range(len(FANOUTS)))
             del res
         torch.cuda.synchronize()
         pool_s = time.perf_counter() - t1
-        pool = {"workers": WORKERS, "minibatches_per_call": DEPTH,
+        pool = {"workers": POOL, "minibatches_per_call": DEPTH,
                 "ms_per_step": pool_s / len(timed_sets) * 1e3, "value": pool_edges / pool_s,
-                "what": "the timed minibatches through gs_ops._CAPI_SampleBlocks: four host threads "
+                "what": "the timed minibatches through gs_ops._CAPI_SampleBlocks: three host threads "
                         "of the C++ layer, one stream each, every minibatch queued whole"}
 
     out = {
