@@ -367,7 +367,7 @@ def large_graph(torch, np, gs, capi, rmat, timer, args, dev, O):
         outs = []
         for l in range(len(FANOUTS)):
             frontier, offsets, renamed = parts[3 * l:3 * l + 3]
-            h = features.index_select(0, frontier.long())  # source features; seeds come first
+            h = features.index_select(0, frontier)  # source features; seeds come first
             out = torch.empty(renamed.numel(), 1, device=dev)
             capi.sddmm_csc("dot", offsets, renamed, None, None, h, h[:offsets.numel() - 1], out,
                            0, 2, FEATURE_DIM, FEATURE_DIM, 1, FEATURE_DIM)

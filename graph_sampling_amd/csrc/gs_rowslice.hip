@@ -34,13 +34,19 @@ constexpr int kTile = kThreads * kItems;
 constexpr int kStage = 1024;
 
 struct IdSet {
-  long long* keys;  // -1 empty
-  long long* vals;
+  // slot p: key (-1 empty) at slots[2 p], value at slots[2 p + 1] -- one 16-byte read for a
+  // lookup that finds its key in its home slot
+  long long* slots;
   uint32_t mask;
   int shift;
   // bit (hash of key) is set for every key of the set: a clear bit proves absence
   uint32_t* filter;
   int filter_shift;
+  // The filter folded down to at most kLdsFilterWords words (bit b of the filter is bit
+  // b mod its size of this one): what a workgroup keeps in LDS.  The filter itself when that
+  // is no larger.
+  uint32_t* coarse;
+  uint32_t coarse_mask;  // its number of bits - 1
   __device__ __forceinline__ uint32_t home(long long key) const {
     return static_cast<uint32_t>((static_cast<uint64_t>(key) * 0x9E3779B97F4A7C15ull) >> shift);
   }
@@ -55,15 +61,41 @@ struct IdSet {
   __device__ __forceinline__ void admit(long long key) const {
     const uint32_t b = filter_bit(key);
     atomicOr(&filter[b >> 5], 1u << (b & 31));
+    if (coarse != filter) atomicOr(&coarse[(b & coarse_mask) >> 5], 1u << (b & 31));
+  }
+  // the same test against a copy of `coarse` in LDS
+  __device__ __forceinline__ bool maybe_lds(const uint32_t* lds, long long key) const {
+    const uint32_t b = filter_bit(key) & coarse_mask;
+    return (lds[b >> 5] >> (b & 31)) & 1u;
+  }
+  __device__ __forceinline__ longlong2 slot(uint32_t p) const {
+    return reinterpret_cast<const longlong2*>(slots)[p];
+  }
+  // value of `key` (-1: absent) given what its home slot holds; walks on in the rare case
+  // that the slot belongs to another key
+  __device__ __forceinline__ int64_t resolve(long long key, longlong2 kv) const {
+    uint32_t p = home(key);
+    while (kv.x != key && kv.x != -1) {
+      p = (p + 1) & mask;
+      kv = slot(p);
+    }
+    return kv.x == key ? kv.y : -1;
   }
   __device__ __forceinline__ int64_t query(long long key) const {
-    uint32_t p = home(key);
-    while (true) {
-      const long long cur = keys[p];
-      if (cur == key) return vals[p];
-      if (cur == -1) return -1;
-      p = (p + 1) & mask;
-    }
+    return resolve(key, slot(home(key)));
+  }
+  // N lookups of a thread: the home slots of all of them are read together (a lookup written
+  // as one loop after the other makes N round trips, since a wave nearly always has some lane
+  // with a key to look up in each)
+  template <int N>
+  __device__ __forceinline__ void query_all(const long long (&key)[N], const bool (&want)[N],
+                                            int64_t (&val)[N]) const {
+    longlong2 kv[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+      if (want[k]) kv[k] = slot(home(key[k]));
+#pragma unroll
+    for (int k = 0; k < N; ++k) val[k] = want[k] ? resolve(key[k], kv[k]) : -1;
   }
 };
 
@@ -80,15 +112,34 @@ int64_t filter_bits(int64_t n) {
   return bits;
 }
 
-// clears the table and the filter; the grid covers the longer of the two
+// A workgroup's copy of the folded filter: 128 KB of the 160 KB of LDS a compute unit has, so
+// that one workgroup of 1024 lanes is resident per unit.  It pays where most keys are in no
+// set: the index search (14 M keys against 256 k ids: 184 -> 98 us together with reading the
+// home slots of a thread's eight keys at once), less so the mark pass of a row slice (whole
+// graph, 200 k row ids: 0.84 -> 0.77 ms), and not the batched filter (0.10 -> 0.14 ms), which
+// keeps the one-tile workgroups.
+constexpr int kLdsFilterWords = 32768;
+constexpr int kBigThreads = 1024;
+constexpr int64_t kLdsSearchMinKeys = int64_t(1) << 20;  // below: not worth 128 KB per workgroup
+
+// clears the table and the filters; the grid covers the longer of them
 __global__ void __launch_bounds__(kThreads)
 set_init_kernel(IdSet t, int64_t cap, int64_t filter_words) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i < cap) {
-    t.keys[i] = -1;
-    t.vals[i] = -1;
+    reinterpret_cast<longlong2*>(t.slots)[i] = make_longlong2(-1, -1);
   }
   if (i < filter_words) t.filter[i] = 0;
+  if (t.coarse != t.filter && i < kLdsFilterWords) t.coarse[i] = 0;
+}
+
+// every thread of a workgroup of kBigThreads: the folded filter into LDS
+__device__ __forceinline__ void load_filter(const IdSet& t, uint32_t* lds) {
+  const int words = static_cast<int>((t.coarse_mask + 1u) >> 5);
+  const uint4* src = reinterpret_cast<const uint4*>(t.coarse);
+  for (int i = threadIdx.x; i < words / 4; i += kBigThreads)
+    reinterpret_cast<uint4*>(lds)[i] = src[i];
+  __syncthreads();
 }
 
 template <typename IdT>
@@ -100,12 +151,12 @@ set_insert_kernel(IdSet t, const IdT* __restrict__ ids, int64_t n) {
   uint32_t p = t.home(key);
   while (true) {
     const unsigned long long prev =
-        atomicCAS(reinterpret_cast<unsigned long long*>(&t.keys[p]), ~0ull,
+        atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[2 * p]), ~0ull,
                   static_cast<unsigned long long>(key));
     if (prev == ~0ull || prev == static_cast<unsigned long long>(key)) break;
     p = (p + 1) & t.mask;
   }
-  atomicMax(&t.vals[p], static_cast<long long>(i));
+  atomicMax(&t.slots[2 * p + 1], static_cast<long long>(i));
   t.admit(key);
 }
 
@@ -149,7 +200,8 @@ struct LoadCounts {
 template <typename IdT>
 struct PlainKey {
   const IdT* key;
-  __device__ __forceinline__ bool operator()(int64_t e, long long* out) const {
+  __device__ __forceinline__ int64_t tile_hint(int64_t, int64_t) const { return 0; }
+  __device__ __forceinline__ bool operator()(int64_t e, int64_t, long long* out) const {
     *out = static_cast<long long>(key[e]);
     return true;
   }
@@ -163,13 +215,20 @@ struct BatchedKey {
   const IdT* key;
   const int64_t* key_ptr;
   int64_t B;
-  __device__ __forceinline__ bool operator()(int64_t e, long long* out) const {
-    int64_t lo = 0, hi = B + 1;  // first b with key_ptr[b] > e
+  // the batch of the tile's first edge (-1: before the first batch), searched once per tile;
+  // an edge of the tile then steps on from there, which is seldom a step at all
+  __device__ __forceinline__ int64_t tile_hint(int64_t p0, int64_t E) const {
+    if (p0 >= E) return B;
+    int64_t lo = 0, hi = B + 1;  // first b with key_ptr[b] > p0
     while (lo < hi) {
       const int64_t mid = (lo + hi) >> 1;
-      if (key_ptr[mid] <= e) lo = mid + 1; else hi = mid;
+      if (key_ptr[mid] <= p0) lo = mid + 1; else hi = mid;
     }
-    const int64_t b = lo - 1;
+    return lo - 1;
+  }
+  __device__ __forceinline__ bool operator()(int64_t e, int64_t hint, long long* out) const {
+    int64_t b = hint;
+    while (b < B && key_ptr[b + 1] <= e) ++b;
     if (b < 0 || b >= B) return false;
     *out = static_cast<long long>(key[e]) + (static_cast<long long>(b) << kBatchShift);
     return true;
@@ -180,15 +239,16 @@ struct BatchedKey {
 // p0 + k * 256 + thread in round k, so that a wave's ballot in round k is the word of 64
 // consecutive positions (word k * 4 + wave of the tile).  vals[k] >= 0: kept, and the
 // value to pack to the front of the tile's range (with src[k] beside it when WITH_SRC).
-// Every thread of the workgroup calls this.
+// Every thread of the workgroup calls this; `tid` is the thread's number among the 256 that
+// own tile `tile`.
 template <typename IdT, bool WITH_VALUES, bool WITH_SRC>
 __device__ __forceinline__ void publish_marks(const int64_t (&vals)[kItems],
                                               const int64_t (&src)[kItems], int64_t p0, int64_t n,
                                               const Marks& m, IdT* __restrict__ packed,
                                               int64_t* __restrict__ packed_src, int* s_pop,
-                                              int* s_rank) {
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+                                              int* s_rank, int tid, int64_t tile) {
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
   unsigned long long bal[kItems];
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
@@ -200,20 +260,19 @@ __device__ __forceinline__ void publish_marks(const int64_t (&vals)[kItems],
     }
   }
   __syncthreads();
-  if (threadIdx.x < kWave) {
-    const int v = threadIdx.x < kWords ? s_pop[threadIdx.x] : 0;
+  if (tid < kWave) {
+    const int v = tid < kWords ? s_pop[tid] : 0;
     int incl = v;
 #pragma unroll
     for (int d = 1; d < kWords; d <<= 1) {
       const int o = __shfl_up(incl, d, kWave);
       if (lane >= d) incl += o;
     }
-    if (threadIdx.x < kWords) {
-      s_rank[threadIdx.x] = incl - v;
-      if (p0 + static_cast<int64_t>(threadIdx.x) * kWave < n)
-        m.word_rank[(p0 >> 6) + threadIdx.x] = incl - v;
+    if (tid < kWords) {
+      s_rank[tid] = incl - v;
+      if (p0 + static_cast<int64_t>(tid) * kWave < n) m.word_rank[(p0 >> 6) + tid] = incl - v;
     }
-    if (threadIdx.x == kWords - 1) m.tile_counts[blockIdx.x] = incl;
+    if (tid == kWords - 1 && tile < m.tiles) m.tile_counts[tile] = incl;
   }
   if (WITH_VALUES || WITH_SRC) {
     __syncthreads();
@@ -237,21 +296,64 @@ mark_tiles_kernel(IdSet t, KeyOf key_of, int64_t E, Marks m, IdT* __restrict__ p
   __shared__ int s_pop[kWords];
   __shared__ int s_rank[kWords];
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
+  const int64_t hint = key_of.tile_hint(p0, E);
   long long keys[kItems];
   bool pass[kItems];
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
     const int64_t e = p0 + k * kThreads + threadIdx.x;
     keys[k] = -1;
-    pass[k] = e < E && key_of(e, &keys[k]);
+    pass[k] = e < E && key_of(e, hint, &keys[k]);
   }
 #pragma unroll
   for (int k = 0; k < kItems; ++k)
     if (pass[k]) pass[k] = t.maybe(keys[k]);
   int64_t vals[kItems];
+  t.query_all<kItems>(keys, pass, vals);
+  publish_marks<IdT, WITH_VALUES, false>(vals, vals, p0, E, m, packed, nullptr, s_pop, s_rank,
+                                         threadIdx.x, blockIdx.x);
+}
+
+// The same for many edges: workgroups of 1024 lanes that stay (four tiles at a time, then the
+// next four, ...) and test the keys against the folded filter in LDS first.
+template <typename IdT, typename KeyOf, bool WITH_VALUES>
+__global__ void __launch_bounds__(kBigThreads)
+mark_tiles_lds_kernel(IdSet t, KeyOf key_of, int64_t E, Marks m, IdT* __restrict__ packed) {
+  constexpr int kSub = kBigThreads / kThreads;
+  __shared__ uint32_t s_filter[kLdsFilterWords];
+  __shared__ int s_pop[kSub][kWords];
+  __shared__ int s_rank[kSub][kWords];
+  load_filter(t, s_filter);
+  const int sub = threadIdx.x / kThreads;
+  const int tid = threadIdx.x % kThreads;
+  const bool two_levels = t.coarse != t.filter;
+  for (int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kSub; tile0 < m.tiles;
+       tile0 += static_cast<int64_t>(gridDim.x) * kSub) {
+    const int64_t tile = tile0 + sub;
+    const int64_t p0 = tile * kTile;
+    const int64_t hint = key_of.tile_hint(p0, E);
+    long long keys[kItems];
+    bool pass[kItems];
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) vals[k] = pass[k] ? t.query(keys[k]) : -1;
-  publish_marks<IdT, WITH_VALUES, false>(vals, vals, p0, E, m, packed, nullptr, s_pop, s_rank);
+    for (int k = 0; k < kItems; ++k) {
+      const int64_t e = p0 + k * kThreads + tid;
+      keys[k] = -1;
+      pass[k] = e < E && key_of(e, hint, &keys[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < kItems; ++k)
+      if (pass[k]) pass[k] = t.maybe_lds(s_filter, keys[k]);
+    if (two_levels) {
+#pragma unroll
+      for (int k = 0; k < kItems; ++k)
+        if (pass[k]) pass[k] = t.maybe(keys[k]);
+    }
+    int64_t vals[kItems];
+    t.query_all<kItems>(keys, pass, vals);
+    publish_marks<IdT, WITH_VALUES, false>(vals, vals, p0, E, m, packed, nullptr, s_pop[sub],
+                                           s_rank[sub], tid, tile);
+    __syncthreads();  // s_pop and s_rank are written again in the next round
+  }
 }
 
 __global__ void __launch_bounds__(kThreads)
@@ -364,12 +466,12 @@ set_insert_batched_kernel(IdSet t, const IdT* __restrict__ ids, int64_t n,
   uint32_t p = t.home(key);
   while (true) {
     const unsigned long long prev =
-        atomicCAS(reinterpret_cast<unsigned long long*>(&t.keys[p]), ~0ull,
+        atomicCAS(reinterpret_cast<unsigned long long*>(&t.slots[2 * p]), ~0ull,
                   static_cast<unsigned long long>(key));
     if (prev == ~0ull || prev == static_cast<unsigned long long>(key)) break;
     p = (p + 1) & t.mask;
   }
-  atomicMax(&t.vals[p], id);
+  atomicMax(&t.slots[2 * p + 1], id);
   t.admit(key);
 }
 
@@ -423,12 +525,14 @@ sliced_mark_kernel(IdSet t, const int64_t* __restrict__ indptr, const IdT* __res
   for (int k = 0; k < kItems; ++k)
     if (pass[k]) pass[k] = t.maybe(keys[k]);
   int64_t vals[kItems];
+  t.query_all<kItems>(keys, pass, vals);
+  if (B > 0) {
 #pragma unroll
-  for (int k = 0; k < kItems; ++k) {
-    const int64_t v = pass[k] ? t.query(keys[k]) : -1;
-    vals[k] = (B > 0 && v >= 0) ? ids[k] : v;  // batched: rows keep their id
+    for (int k = 0; k < kItems; ++k)
+      if (vals[k] >= 0) vals[k] = ids[k];  // batched: rows keep their id
   }
-  publish_marks<IdT, true, true>(vals, src, p0, D, m, packed, packed_src, s_pop, s_rank);
+  publish_marks<IdT, true, true>(vals, src, p0, D, m, packed, packed_src, s_pop, s_rank, threadIdx.x,
+                                 blockIdx.x);
 }
 
 __global__ void __launch_bounds__(kThreads)
@@ -488,14 +592,47 @@ search_kernel(IdSet t, const IdT* __restrict__ keys, int64_t m, IdT* __restrict_
   if (i < m) out[i] = static_cast<IdT>(t.query(static_cast<long long>(keys[i])));
 }
 
+// The same for many keys: most of them are in no set, and the folded filter in LDS says so
+// without a trip to memory.
+template <typename IdT>
+__global__ void __launch_bounds__(kBigThreads)
+search_lds_kernel(IdSet t, const IdT* __restrict__ keys, int64_t m, IdT* __restrict__ out) {
+  __shared__ uint32_t s_filter[kLdsFilterWords];
+  load_filter(t, s_filter);
+  const bool two_levels = t.coarse != t.filter;
+  constexpr int kPer = 8;
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * kBigThreads * kPer; base < m;
+       base += static_cast<int64_t>(gridDim.x) * kBigThreads * kPer) {
+    long long key[kPer];
+    bool pass[kPer];
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+      const int64_t i = base + u * kBigThreads + threadIdx.x;
+      key[u] = i < m ? static_cast<long long>(keys[i]) : -1;
+      pass[u] = i < m && t.maybe_lds(s_filter, key[u]);
+    }
+    if (two_levels) {
+#pragma unroll
+      for (int u = 0; u < kPer; ++u)
+        if (pass[u]) pass[u] = t.maybe(key[u]);
+    }
+    int64_t val[kPer];
+    t.query_all<kPer>(key, pass, val);
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+      const int64_t i = base + u * kBigThreads + threadIdx.x;
+      if (i < m) out[i] = static_cast<IdT>(val[u]);
+    }
+  }
+}
+
 // Workspace layout: [marks | (parent positions) | id-set keys | id-set values | filter].
 // The marks (bit words, word ranks, tile counts and bases, scan tiles, packed new ids)
 // and the parent positions depend on the edge count only, so the compact call finds them
 // again without knowing how many ids the mark call was given.
 void carve_set(Carver& ws, int64_t n_ids, IdSet* set, int64_t* cap, int64_t* filter_words) {
   *cap = set_capacity(n_ids);
-  set->keys = ws.take<long long>(*cap);
-  set->vals = ws.take<long long>(*cap);
+  set->slots = ws.take<long long>(2 * *cap);
   set->mask = static_cast<uint32_t>(*cap - 1);
   int lg = 0;
   while ((int64_t(1) << lg) < *cap) ++lg;
@@ -506,10 +643,19 @@ void carve_set(Carver& ws, int64_t n_ids, IdSet* set, int64_t* cap, int64_t* fil
   lg = 0;
   while ((int64_t(1) << lg) < bits) ++lg;
   set->filter_shift = 64 - lg;
+  if (*filter_words > kLdsFilterWords) {
+    set->coarse = ws.take<uint32_t>(kLdsFilterWords);
+    set->coarse_mask = static_cast<uint32_t>(kLdsFilterWords) * 32u - 1u;
+  } else {
+    set->coarse = set->filter;
+    set->coarse_mask = static_cast<uint32_t>(bits - 1);
+  }
 }
 
 size_t set_bytes(int64_t n_ids) {
-  return 2 * padded(set_capacity(n_ids) * 8) + padded(filter_bits(n_ids) / 8);
+  const int64_t words = filter_bits(n_ids) / 32;
+  return padded(set_capacity(n_ids) * 16) + padded(words * 4) +
+         (words > kLdsFilterWords ? padded(kLdsFilterWords * 4) : 0);
 }
 
 struct MarkScratch {
@@ -576,7 +722,19 @@ int mark_common(const char* who, const void* key, int64_t E, const int64_t* key_
       hipLaunchKernelGGL(set_insert_kernel<IdT>, dim3(blocks_for(n_ids, kThreads)), dim3(kThreads), 0,
                          st, s.set, static_cast<const IdT*>(ids), n_ids);
   }
-  if (E > 0) {
+  if (E >= kLdsSearchMinKeys && B == 0) {
+    // few workgroups that stay, one per compute unit and a second one waiting
+    const int64_t groups = (s.m.tiles + kBigThreads / kThreads - 1) / (kBigThreads / kThreads);
+    const dim3 grid(static_cast<unsigned>(groups < 512 ? groups : 512));
+    IdT* packed = static_cast<IdT*>(s.packed);
+    PlainKey<IdT> k{static_cast<const IdT*>(key)};
+    if (with_values)
+      hipLaunchKernelGGL((mark_tiles_lds_kernel<IdT, PlainKey<IdT>, true>), grid, dim3(kBigThreads),
+                         0, st, s.set, k, E, s.m, packed);
+    else
+      hipLaunchKernelGGL((mark_tiles_lds_kernel<IdT, PlainKey<IdT>, false>), grid, dim3(kBigThreads),
+                         0, st, s.set, k, E, s.m, packed);
+  } else if (E > 0) {
     const dim3 grid(static_cast<unsigned>(s.m.tiles));
     IdT* packed = static_cast<IdT*>(s.packed);
     if (B > 0) {
@@ -895,9 +1053,15 @@ int gs_index_search(const void* data, int64_t n, const void* keys, int64_t m, in
     if (n > 0)
       hipLaunchKernelGGL(set_insert_kernel<IdT>, dim3(blocks_for(n, kThreads)), dim3(kThreads), 0,
                          st, s.set, static_cast<const IdT*>(data), n);
-    if (m > 0)
+    if (m >= kLdsSearchMinKeys) {
+      const int64_t groups = (m + kBigThreads * 8 - 1) / (kBigThreads * 8);
+      hipLaunchKernelGGL(search_lds_kernel<IdT>, dim3(static_cast<unsigned>(groups < 512 ? groups : 512)),
+                         dim3(kBigThreads), 0, st, s.set, static_cast<const IdT*>(keys), m,
+                         static_cast<IdT*>(out));
+    } else if (m > 0) {
       hipLaunchKernelGGL(search_kernel<IdT>, dim3(blocks_for(m, kThreads)), dim3(kThreads), 0, st,
                          s.set, static_cast<const IdT*>(keys), m, static_cast<IdT*>(out));
+    }
   };
   if (id_bytes == 8) run(int64_t{}); else run(int32_t{});
   return check_launch("index_search");

@@ -150,6 +150,52 @@ def test_coo_filter(dev, B, idt):
             assert np.array_equal(_np(g), w)
 
 
+@pytest.mark.parametrize("B,ids_per_batch", [(0, 50000), (64, 300), (64, 4000), (3000, 40)])
+def test_coo_filter_many_edges(dev, B, ids_per_batch):
+    """From 2^20 edges on: workgroups that stay, the filter (or its folded copy) in LDS, and the
+    batch of an edge found by stepping on from the batch of its tile's first edge."""
+    rng = np.random.default_rng(B + ids_per_batch)
+    n = 1 << 17
+    E = (1 << 20) + 12345
+    if B == 0:
+        key_ptr = ids_ptr = None
+        ids = rng.permutation(n)[:ids_per_batch].astype(np.int64)
+    else:
+        cuts = np.sort(rng.integers(0, E, size=B - 1))
+        key_ptr = np.concatenate([[0], cuts, [E]]).astype(np.int64)
+        id_sizes = rng.integers(0, 2 * ids_per_batch, size=B)
+        ids_ptr = _ptr(id_sizes)
+        ids = np.concatenate([rng.integers(0, n, size=s) for s in id_sizes]).astype(np.int64)
+    row = rng.integers(0, n, size=E).astype(np.int64)
+    col = rng.integers(0, n, size=E).astype(np.int64)
+    got = capi.coo_filter(to_dev(row, dev, torch.int32), to_dev(row, dev, torch.int32),
+                          to_dev(col, dev, torch.int32), to_dev(ids, dev, torch.int32),
+                          None if B == 0 else to_dev(key_ptr, dev),
+                          None if B == 0 else to_dev(ids_ptr, dev))
+    want = O.coo_filter(row, row, col, ids, key_ptr, ids_ptr)
+    for g, w in zip(got, want):
+        if w is None:
+            assert g is None
+        else:
+            assert np.array_equal(_np(g), w)
+    if B == 0:   # closed form
+        keep = np.isin(row, ids)
+        assert np.array_equal(want[0], row[keep]) and np.array_equal(want[1], col[keep])
+
+
+@pytest.mark.parametrize("n_data", [3000, 200000])
+def test_index_search_many_keys(dev, n_data):
+    rng = np.random.default_rng(n_data)
+    data = rng.permutation(1 << 20)[:n_data].astype(np.int64)
+    keys = rng.integers(0, 1 << 20, size=(1 << 20) + 999).astype(np.int64)
+    got = capi.index_search(to_dev(data, dev, torch.int32), to_dev(keys, dev, torch.int32))
+    want = O.index_search(data, keys)
+    assert np.array_equal(_np(got), want)
+    lut = np.full(1 << 20, -1)
+    lut[data] = np.arange(n_data)
+    assert np.array_equal(want, lut[keys])
+
+
 def test_ops_coo_slicing_and_global_id(dev):
     import graph_sampling_amd as gs
     gs.load_library()

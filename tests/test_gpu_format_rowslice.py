@@ -144,6 +144,26 @@ def test_row_slice_csc_rmat(dev, with_coo, n_rows, idt):
 
 
 @pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("n_rows", [300, 20000, 150000])
+def test_row_slice_csc_many_edges(dev, n_rows, idt):
+    """From 2^20 edges on the keys are tested by workgroups that stay, against a copy of the
+    filter in LDS: the filter itself for few row ids, a folded one in front of it for many."""
+    n = 1 << 18
+    indptr, indices = rmat_csc_np(n, (1 << 21) + 777, seed=6)
+    rows = np.random.default_rng(n_rows).permutation(n)[:n_rows].astype(np.int64)
+    got = capi.row_slice_csc(to_dev(indptr, dev), to_dev(indices, dev, idt), to_dev(rows, dev, idt),
+                             True)
+    want = O.row_slice_csc(indptr, indices, rows, True)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+    mask = np.isin(indices, rows)
+    lut = np.full(n, -1)
+    lut[rows] = np.arange(n_rows)
+    assert np.array_equal(want[2], lut[indices[mask]])
+    assert np.array_equal(want[3], np.nonzero(mask)[0])
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
 def test_row_slice_coo(dev, idt):
     indptr, indices = rmat_csc_np(1 << 12, 1 << 16, seed=5)
     col = np.repeat(np.arange(indptr.size - 1), np.diff(indptr))
