@@ -25,6 +25,8 @@
 // (slicing.cu:56); here the largest position wins (atomicMax), deterministically.
 #include "gs_common.hpp"
 
+GS_STAMPS_DEFINE(rowslice)
+
 namespace gs {
 namespace {
 
@@ -120,7 +122,11 @@ int64_t filter_bits(int64_t n) {
 // keeps the one-tile workgroups.
 constexpr int kLdsFilterWords = 32768;
 constexpr int kBigThreads = 1024;
+#ifdef GS_PHASE_STAMPS
+constexpr int64_t kLdsSearchMinKeys = int64_t(1) << 62;  // the marked kernels are the one-tile ones
+#else
 constexpr int64_t kLdsSearchMinKeys = int64_t(1) << 20;  // below: not worth 128 KB per workgroup
+#endif
 
 // clears the table and the filters; the grid covers the longer of them
 __global__ void __launch_bounds__(kThreads)
@@ -295,6 +301,8 @@ __global__ void __launch_bounds__(kThreads)
 mark_tiles_kernel(IdSet t, KeyOf key_of, int64_t E, Marks m, IdT* __restrict__ packed) {
   __shared__ int s_pop[kWords];
   __shared__ int s_rank[kWords];
+  GS_STAMP_BEGIN();
+  GS_STAMP(0);
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
   const int64_t hint = key_of.tile_hint(p0, E);
   long long keys[kItems];
@@ -305,13 +313,18 @@ mark_tiles_kernel(IdSet t, KeyOf key_of, int64_t E, Marks m, IdT* __restrict__ p
     keys[k] = -1;
     pass[k] = e < E && key_of(e, hint, &keys[k]);
   }
+  GS_STAMP(1);  // keys are here
 #pragma unroll
   for (int k = 0; k < kItems; ++k)
     if (pass[k]) pass[k] = t.maybe(keys[k]);
+  GS_STAMP(2);  // filter bits are here
   int64_t vals[kItems];
   t.query_all<kItems>(keys, pass, vals);
+  GS_STAMP(3);  // table lookups done
   publish_marks<IdT, WITH_VALUES, false>(vals, vals, p0, E, m, packed, nullptr, s_pop, s_rank,
                                          threadIdx.x, blockIdx.x);
+  GS_STAMP(4);  // marks, ranks and packed ids stored
+  GS_STAMP_END(9, 5);
 }
 
 // The same for many edges: workgroups of 1024 lanes that stay (four tiles at a time, then the
