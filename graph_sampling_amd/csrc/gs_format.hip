@@ -305,7 +305,11 @@ struct SortOutputs {
 // The value rides along with its word from the first pass on (read in input order then), so
 // no pass gathers it by position; the LAST pass writes values, permutation and keys instead
 // of words.
-template <typename IdT, typename Src, bool LAST>
+// SELF: `offsets` holds the tiles' raw counts and every workgroup adds up for itself where its
+// runs start (a sort of few tiles: two launches less per pass than scanning the counts first).
+constexpr int64_t kSelfScanTiles = 64;
+
+template <typename IdT, typename Src, bool LAST, bool SELF>
 __global__ void __launch_bounds__(kThreads)
 radix_pass_kernel(Src src, const IdT* __restrict__ val_in, int64_t E, int shift,
                   int64_t num_blocks, const int64_t* __restrict__ offsets,
@@ -320,7 +324,30 @@ radix_pass_kernel(Src src, const IdT* __restrict__ val_in, int64_t E, int shift,
   __shared__ int s_scan[kWaves];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  s_base[threadIdx.x] = offsets[static_cast<int64_t>(threadIdx.x) * num_blocks + blockIdx.x];
+  if (SELF) {
+    // digit threadIdx.x: its items in all tiles, and in the tiles before this one
+    __shared__ int64_t s_digits[kWaves];
+    const int64_t* row = offsets + static_cast<int64_t>(threadIdx.x) * num_blocks;
+    int64_t all = 0, before = 0;
+    for (int64_t b = 0; b < num_blocks; ++b) {
+      const int64_t c = row[b];
+      all += c;
+      before += b < static_cast<int64_t>(blockIdx.x) ? c : 0;
+    }
+    int64_t incl = all;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int64_t y = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl += y;
+    }
+    if (lane == kWave - 1) s_digits[wave] = incl;
+    __syncthreads();
+    int64_t lower = incl - all;  // items of the smaller digits
+    for (int w = 0; w < wave; ++w) lower += s_digits[w];
+    s_base[threadIdx.x] = lower + before;
+  } else {
+    s_base[threadIdx.x] = offsets[static_cast<int64_t>(threadIdx.x) * num_blocks + blockIdx.x];
+  }
 #pragma unroll
   for (int w = 0; w < kWaves; ++w) s_cnt[w][threadIdx.x] = 0;
   const int64_t base = static_cast<int64_t>(blockIdx.x) * T::kSize;
@@ -440,6 +467,20 @@ indptr_split_kernel(const int64_t* __restrict__ indptr, const int64_t* __restric
   out[q] = indptr[begin + (q - begin - lo)] - indptr[begin];
 }
 
+template <typename IdT, typename Src>
+void launch_pass(Src src, bool last, bool self, dim3 grid, hipStream_t st, const IdT* vin, int64_t E,
+                 int shift, int64_t blocks, const int64_t* where, unsigned long long* wout,
+                 IdT* vout, const SortOutputs<IdT>& outs) {
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), 0, st, src, vin, E, shift, blocks, where, wout,
+                       vout, outs);
+  };
+  if (last && self) go(radix_pass_kernel<IdT, Src, true, true>);
+  else if (last) go(radix_pass_kernel<IdT, Src, true, false>);
+  else if (self) go(radix_pass_kernel<IdT, Src, false, true>);
+  else go(radix_pass_kernel<IdT, Src, false, false>);
+}
+
 template <typename IdT>
 int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, int sorted,
                  int64_t* indptr, IdT* out_value, int64_t* perm, void* workspace,
@@ -494,24 +535,18 @@ int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, 
       hipLaunchKernelGGL((radix_hist_kernel<StoredWords, T::kSize>), grid, dim3(kThreads), 0, st, src,
                          E, shift, blocks, counts);
     }
-    LoadI64 f{counts};
-    GS_RETURN_IF_ERROR(exclusive_scan(f, table, offsets, tiles, st));
+    const bool self = blocks <= kSelfScanTiles;
+    if (!self) {
+      LoadI64 f{counts};
+      GS_RETURN_IF_ERROR(exclusive_scan(f, table, offsets, tiles, st));
+    }
+    const int64_t* where = self ? counts : offsets;
     if (p == 0) {
       FreshWords<IdT> src{key, idx_bits};
-      if (last)
-        hipLaunchKernelGGL((radix_pass_kernel<IdT, FreshWords<IdT>, true>), grid, dim3(kThreads), 0,
-                           st, src, vin, E, shift, blocks, offsets, wout, vout, outs);
-      else
-        hipLaunchKernelGGL((radix_pass_kernel<IdT, FreshWords<IdT>, false>), grid, dim3(kThreads), 0,
-                           st, src, vin, E, shift, blocks, offsets, wout, vout, outs);
+      launch_pass<IdT>(src, last, self, grid, st, vin, E, shift, blocks, where, wout, vout, outs);
     } else {
       StoredWords src{win};
-      if (last)
-        hipLaunchKernelGGL((radix_pass_kernel<IdT, StoredWords, true>), grid, dim3(kThreads), 0, st,
-                           src, vin, E, shift, blocks, offsets, wout, vout, outs);
-      else
-        hipLaunchKernelGGL((radix_pass_kernel<IdT, StoredWords, false>), grid, dim3(kThreads), 0, st,
-                           src, vin, E, shift, blocks, offsets, wout, vout, outs);
+      launch_pass<IdT>(src, last, self, grid, st, vin, E, shift, blocks, where, wout, vout, outs);
     }
     win = wout;
     vin = vout;
