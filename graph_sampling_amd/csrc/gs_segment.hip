@@ -62,12 +62,17 @@ __global__ void __launch_bounds__(kThreads) clear_chunks_kernel(Chunks ck, int64
   }
 }
 
+// four floats side by side at any 4-byte boundary
+struct __attribute__((packed, aligned(4))) Four {
+  float a, b, c, d;
+};
+
 // ---- by segment: the short ones.  NORMALIZE writes out[d] = data[d] / sum instead.
 template <bool NORMALIZE, typename IdT>
 __global__ void __launch_bounds__(kThreads)
 short_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ emap,
                       const IdT* __restrict__ nmap, const float* __restrict__ data,
-                      int64_t num_seg, int powk, float* __restrict__ out, Chunks ck) {
+                      int64_t num_seg, int64_t nnz, int powk, float* __restrict__ out, Chunks ck) {
   const int64_t s = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   int64_t begin = 0, end = 0;
   if (s < num_seg) {
@@ -99,13 +104,33 @@ short_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restr
     return;
   }
   // at most kLaneMaxLen edges: a fixed number of predicated reads, all in flight together,
-  // added up in edge order
+  // added up in edge order.  Without an edge map the lane's edges lie side by side and are
+  // read four at a time (a lane's reads are scattered from its neighbours' either way: every
+  // read instruction is a line access per lane, and this makes four of sixteen).
   float v[kLaneMaxLen];
   int64_t at[kLaneMaxLen];
+  if (!emap) {
 #pragma unroll
-  for (int k = 0; k < kLaneMaxLen; ++k) {
-    at[k] = begin + k < end ? (emap ? emap[begin + k] : begin + k) : -1;
-    v[k] = at[k] >= 0 ? data[at[k]] : 0.0f;
+    for (int j = 0; j < kLaneMaxLen / 4; ++j) {
+      const int64_t p = begin + 4 * j;
+      Four q{0.0f, 0.0f, 0.0f, 0.0f};
+      if (p + 3 < nnz && p < end) {
+        q = *reinterpret_cast<const Four*>(data + p);
+      } else {
+        if (p < end) q.a = data[p];
+        if (p + 1 < end) q.b = data[p + 1];
+        if (p + 2 < end) q.c = data[p + 2];
+      }
+      v[4 * j] = q.a, v[4 * j + 1] = q.b, v[4 * j + 2] = q.c, v[4 * j + 3] = q.d;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) at[4 * j + u] = p + u < end ? p + u : -1;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < kLaneMaxLen; ++k) {
+      at[k] = begin + k < end ? emap[begin + k] : -1;
+      v[k] = at[k] >= 0 ? data[at[k]] : 0.0f;
+    }
   }
   float acc = 0.0f;
 #pragma unroll
@@ -542,7 +567,7 @@ int segment_sum_impl(const int64_t* indptr, const int64_t* emap, const void* nma
   hipLaunchKernelGGL(clear_chunks_kernel, dim3(blocks_for(chunks, kThreads)), dim3(kThreads), 0, st,
                      s.ck, chunks);
   hipLaunchKernelGGL((short_segments_kernel<false, IdT>), dim3(blocks_for(num_seg, kThreads)),
-                     dim3(kThreads), 0, st, indptr, emap, nm, data, num_seg, powk, out, s.ck);
+                     dim3(kThreads), 0, st, indptr, emap, nm, data, num_seg, nnz, powk, out, s.ck);
   if (nnz > kLaneMaxLen) {
     hipLaunchKernelGGL(long_segments_kernel<IdT>, dim3(blocks_for(chunks, kWaves)), dim3(kThreads),
                        0, st, indptr, emap, nm, data, num_seg, nnz, powk, out, s.ck);
@@ -710,7 +735,7 @@ int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const floa
   hipLaunchKernelGGL(clear_chunks_kernel, dim3(blocks_for(chunks, kThreads)), dim3(kThreads), 0, st,
                      s.ck, chunks);
   hipLaunchKernelGGL((short_segments_kernel<true, int64_t>), dim3(blocks_for(num_segments, kThreads)),
-                     dim3(kThreads), 0, st, indptr, e_ids, no_map, data, num_segments, 1, out, s.ck);
+                     dim3(kThreads), 0, st, indptr, e_ids, no_map, data, num_segments, nnz, 1, out, s.ck);
   if (nnz > kLaneMaxLen) {
     hipLaunchKernelGGL(long_segments_kernel<int64_t>, dim3(blocks_for(chunks, kWaves)),
                        dim3(kThreads), 0, st, indptr, e_ids, no_map, data, num_segments, nnz, 1,
