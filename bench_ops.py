@@ -320,6 +320,33 @@ def main():
     flow("flow_ladies", "LADIES, 2 layers of 512 picks from 512 seeds (slice, row sums of w^2 over "
          "2.45M rows, weighted pick, row slice, divide, normalise, relabel)",
          lambda: ladies(A, seeds512, [512, 512]), edges_of, "edges")
+    if not only or "config3" in only:
+        # the layer-wise sampler's configuration as a line of its own, in the shape of bench.py's:
+        # fresh seeds every step, the steps back to back, one synchronisation on either side
+        steps, warm = max(args.reps, 10) * 5, 5
+        sets = [torch.randperm(N, generator=gen, device=dev)[:512].to(idt)
+                for _ in range(warm + steps)]
+        for s_ in sets[:warm]:
+            ladies(A, s_, [512, 512])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        block_edges = 0
+        for s_ in sets[warm:]:
+            block_edges += edges_of(ladies(A, s_, [512, 512]))
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        print(json.dumps({
+            "metric": "block edges/sec, LADIES 2 layers x 512 weighted picks, batch 512",
+            "value": block_edges / dt, "unit": "edges/s", "n_gpus": 1, "steps": steps,
+            "warmup": warm, "ms_per_step": dt / steps * 1e3, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "int32 ids, fp32 weights",
+            "data": "synthetic R-MAT (a=.57,b=.19,c=.19), generated on device, seed 0",
+            "config": {"workload": "rmat-%.2fM-%dM ladies" % (N / 1e6, E // 1_000_000),
+                       "batch": 512, "picks_per_layer": [512, 512],
+                       "api": "gs.Matrix: A[:, seeds], sum(axis=1, powk=2), "
+                              "list_sampling_with_probs, U[nodes, :], divide, normalize, "
+                              "all_indices, to_dgl_block (examples/ladies/ladies_raw.py:8-27)"}}),
+              flush=True)
     ladies_c = jit.compile(ladies, (A, seeds512, [512, 512]))
     flow("flow_ladies_compiled", "the same sampler through jit.compile",
          lambda: ladies_c(A, seeds512, [512, 512]), edges_of, "edges")
