@@ -104,6 +104,30 @@ def test_chain_with_seeds_that_are_no_columns(dev):
         assert np.array_equal(b.out_ids[:E].cpu().numpy().astype(np.int64), renamed)
 
 
+@pytest.mark.parametrize("case", range(24))
+def test_chain_on_seeded_random_shapes(dev, case):
+    """Graph size, skew, seed count (with repeats), depth, fanouts and the replace flag drawn
+    from a seeded generator: every case against the oracle, layer by layer."""
+    rng = np.random.default_rng(1000 + case)
+    n = int(rng.choice([64, 1 << 10, 1 << 13, 1 << 15]))
+    e = int(n * rng.choice([1, 4, 30]))
+    indptr, indices = rmat_csc_np(n, e, seed=case)
+    num_seeds = int(rng.choice([1, 7, 100, 1500, 4000]))
+    seeds = rng.integers(0, n, size=num_seeds).astype(np.int64)
+    depth = int(rng.integers(1, 4))
+    replace = bool(rng.integers(0, 2))
+    fanouts = tuple(int(rng.choice([2, 3, 5, 8, 12, 20, 32])) for _ in range(depth))
+    bound = num_seeds
+    for k in fanouts:
+        bound *= 1 + k
+    if bound > 1 << 22:
+        fanouts = fanouts[:1]
+    idt = torch.int32 if case % 2 == 0 else torch.int64
+    d = (to_dev(indptr, dev), to_dev(indices, dev, idt), to_dev(seeds, dev, idt))
+    layers, _ = capi.sample_layers(*d, fanouts, replace, seed=case)
+    _check_layers(layers, _oracle_layers(indptr, indices, seeds, fanouts, replace, case))
+
+
 def test_chain_reports_an_id_beyond_32_bits(dev):
     """64-bit ids ride on one-word slots; one that does not fit is reported as -2, not truncated."""
     indptr = np.array([0, 2, 4, 6], dtype=np.int64)

@@ -223,6 +223,29 @@ def test_list_weighted_keys_that_repeat_thousands_of_times(dev, n, k, distinct):
     assert np.array_equal(w_idx, order[:k])
 
 
+@pytest.mark.parametrize("case", range(16))
+def test_list_weighted_on_seeded_random_shapes(dev, case):
+    """n, k, the share of items without weight and the spread of the weights drawn from a seeded
+    generator; half of the cases replay given draws."""
+    rng = np.random.default_rng(500 + case)
+    n = int(rng.choice([50, 3000, 70000, 400000]))
+    k = int(min(n - 1, rng.choice([1, 10, 512, 3000, 8192])))
+    data = rng.integers(0, 1 << 30, n).astype(np.int64)
+    probs = (rng.random(n, dtype=np.float32) ** int(rng.choice([1, 4, 12]))).astype(np.float32)
+    probs[rng.random(n) < rng.choice([0.0, 0.5, 0.97])] = 0.0
+    idt = torch.int32 if case % 2 else torch.int64
+    if case % 2:
+        replay = u32_draws(n, case)
+        sel, idx = capi.list_sample_weighted(to_dev(data, dev, idt), to_dev(probs, dev), k,
+                                             replay=to_dev(replay, dev))
+        w_sel, w_idx = O.list_sample_weighted(data, probs, k, replay=replay)
+    else:
+        sel, idx = capi.list_sample_weighted(to_dev(data, dev, idt), to_dev(probs, dev), k, seed=case)
+        w_sel, w_idx = O.list_sample_weighted(data, probs, k, seed=case)
+    assert np.array_equal(idx.cpu().numpy(), w_idx)
+    assert np.array_equal(sel.cpu().numpy().astype(np.int64), w_sel)
+
+
 def test_list_weighted_weights_at_any_alignment(dev):
     n, k = 100003, 300
     rng = np.random.default_rng(3)
