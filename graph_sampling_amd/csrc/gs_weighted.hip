@@ -30,6 +30,7 @@ constexpr int64_t kChunk = 2048;          // edges per wave task
 constexpr int64_t kMaxFanout = 96;        // 64 lanes * 96 * 8 B = 48 KB of LDS per wave
 constexpr int kQueueGrid = 1024;          // workgroups draining a queue
 constexpr int64_t kQueueExtra = 1 << 19;  // chunk-queue capacity = S + kQueueExtra
+constexpr int kQueueParts = 64;           // one lane per part where the parts are added up
 
 template <typename IdT>
 struct WArgs {
@@ -48,9 +49,13 @@ struct WArgs {
   int64_t* select_index;
   IdT* coo_col;
   // long rows
-  unsigned long long* counters;  // [0] chunks reserved, [1] long rows
+  // [1] long rows, [2 + q] chunks reserved in part q of the queue.  The queue is kept in
+  // kQueueParts parts, each with a counter of its own (a workgroup reserves in part
+  // blockIdx % kQueueParts): reservations at ONE counter queue up at its address, 11 ns
+  // apiece, and 2000 rows above 256 edges among 45 k made that the rows kernel's last 20 us.
+  unsigned long long* counters;
   long long* chunk_queue;        // row << 20 | chunk, -1 = void
-  int64_t chunk_cap;
+  int64_t chunk_cap;             // slots of one part
   long long* long_rows;          // 3 entries per long row: row, first queue slot, #chunks
   unsigned long long* cand;      // chunk_cap * k composites
 };
@@ -223,23 +228,27 @@ __global__ void weighted_rows_kernel(WArgs<IdT> a) {
   bool here = deg <= kSmall;
   if (!here) {
     const int64_t nchunks = (deg + kChunk - 1) / kChunk;
+    const int64_t part = blockIdx.x & (kQueueParts - 1);
+    const int64_t part0 = part * a.chunk_cap;
     unsigned long long base = 0;
-    if (lane == 0) base = atomicAdd(&a.counters[0], static_cast<unsigned long long>(nchunks));
+    if (lane == 0)
+      base = atomicAdd(&a.counters[2 + part], static_cast<unsigned long long>(nchunks));
     base = __shfl(base, 0, kWave);
     if (static_cast<int64_t>(base) + nchunks <= a.chunk_cap) {
       for (int64_t ch = lane; ch < nchunks; ch += kWave)
-        a.chunk_queue[base + ch] = static_cast<long long>((r << 20) | ch);
+        a.chunk_queue[part0 + base + ch] = static_cast<long long>((r << 20) | ch);
       if (lane == 0 && nchunks > 1) {
         const unsigned long long slot = atomicAdd(&a.counters[1], 1ull);
         a.long_rows[slot * 3 + 0] = r;
-        a.long_rows[slot * 3 + 1] = static_cast<long long>(base);
+        a.long_rows[slot * 3 + 1] = part0 + static_cast<long long>(base);
         a.long_rows[slot * 3 + 2] = nchunks;
       }
     } else {
-      // queue full: void the reserved tail and select the whole row with this wave
+      // this part of the queue is full: void the reserved tail and select the whole row with
+      // this wave
       for (int64_t ch = static_cast<int64_t>(base) + lane;
            ch < a.chunk_cap && ch < static_cast<int64_t>(base) + nchunks; ch += kWave)
-        a.chunk_queue[ch] = -1;
+        a.chunk_queue[part0 + ch] = -1;
       here = true;
     }
   }
@@ -274,12 +283,29 @@ __global__ void weighted_chunks_kernel(WArgs<IdT> a) {
   const int wave = threadIdx.x / kWave;
   const int waves = blockDim.x / kWave;
   unsigned long long* list = s_lists + static_cast<size_t>(wave) * a.k * kWave;
-  const unsigned long long reserved = a.counters[0];
-  const int64_t n = reserved < static_cast<unsigned long long>(a.chunk_cap)
-                        ? static_cast<int64_t>(reserved)
-                        : a.chunk_cap;
-  for (int64_t t = static_cast<int64_t>(blockIdx.x) * waves + wave; t < n;
-       t += static_cast<int64_t>(gridDim.x) * waves) {
+  // lane q: entries of part q, and how many lie in the parts before it
+  static_assert(kQueueParts == kWave, "one lane per part of the queue");
+  const unsigned long long reserved = a.counters[2 + lane];
+  const int64_t mine = reserved < static_cast<unsigned long long>(a.chunk_cap)
+                           ? static_cast<int64_t>(reserved)
+                           : a.chunk_cap;
+  int64_t incl = mine;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int64_t o = __shfl_up(incl, d, kWave);
+    if (lane >= d) incl += o;
+  }
+  const int64_t before = incl - mine;
+  const int64_t n = __shfl(incl, kWave - 1, kWave);
+  for (int64_t v = static_cast<int64_t>(blockIdx.x) * waves + wave; v < n;
+       v += static_cast<int64_t>(gridDim.x) * waves) {
+    int lo_part = 0, hi_part = kQueueParts;  // the last part that starts at or before v
+#pragma unroll
+    for (int step = 0; step < 6; ++step) {
+      const int mid = (lo_part + hi_part) >> 1;
+      if (__shfl(before, mid, kWave) <= v) lo_part = mid; else hi_part = mid;
+    }
+    const int64_t t = static_cast<int64_t>(lo_part) * a.chunk_cap + (v - __shfl(before, lo_part, kWave));
     const long long e = a.chunk_queue[t];
     if (e < 0) continue;
     const int64_t r = e >> 20;
@@ -351,7 +377,7 @@ __global__ void weighted_merge_kernel(WArgs<IdT> a) {
 }
 
 static __global__ void zero2_kernel(unsigned long long* p) {
-  if (threadIdx.x < 2) p[threadIdx.x] = 0;
+  for (int i = threadIdx.x; i < 2 + kQueueParts; i += blockDim.x) p[i] = 0;
 }
 
 int waves_per_block(int64_t k) {
@@ -396,11 +422,11 @@ int weighted_impl(const int64_t* indptr, int64_t num_cols, const void* indices, 
   a.sub_indices = static_cast<IdT*>(sub_indices);
   a.select_index = select_index;
   a.coo_col = static_cast<IdT*>(coo_col);
-  a.chunk_cap = S + kQueueExtra;
-  a.counters = ws.take<unsigned long long>(2);
-  a.chunk_queue = ws.take<long long>(static_cast<size_t>(a.chunk_cap));
+  a.chunk_cap = (S + kQueueExtra) / kQueueParts;
+  a.counters = ws.take<unsigned long long>(2 + kQueueParts);
+  a.chunk_queue = ws.take<long long>(static_cast<size_t>(a.chunk_cap) * kQueueParts);
   a.long_rows = ws.take<long long>(static_cast<size_t>(S) * 3);
-  a.cand = ws.take<unsigned long long>(static_cast<size_t>(a.chunk_cap) * k);
+  a.cand = ws.take<unsigned long long>(static_cast<size_t>(a.chunk_cap) * kQueueParts * k);
   if (!ws.ok) {
     set_error_text("gs_sample_weighted_fill: workspace needs %zu bytes, 256-byte aligned",
                    gs_sample_weighted_workspace_bytes(S, k));
@@ -679,7 +705,7 @@ size_t gs_sample_weighted_workspace_bytes(int64_t S, int64_t fanout) {
   if (S < 0) S = 0;
   if (fanout < 1) fanout = 1;
   const size_t cap = static_cast<size_t>(S + kQueueExtra);
-  return padded(16) + padded(cap * 8) + padded(static_cast<size_t>(S) * 24) +
+  return padded((2 + kQueueParts) * 8) + padded(cap * 8) + padded(static_cast<size_t>(S) * 24) +
          padded(cap * static_cast<size_t>(fanout) * 8);
 }
 
