@@ -507,30 +507,42 @@ sliced_mark_kernel(IdSet t, const int64_t* __restrict__ indptr, const IdT* __res
   if (staged)
     for (int64_t i = threadIdx.x; i <= nrows; i += kThreads) s_ptr[i] = sub_indptr[row_lo + i];
   __syncthreads();
+  // The eight positions of a thread go through the same chain of reads (row of the position,
+  // the row's column, the column's start, the edge's id): every link for all eight before the
+  // next, so that eight reads are in flight at a time instead of one.
   long long keys[kItems], ids[kItems];
-  int64_t src[kItems];
+  int64_t src[kItems], row[kItems], off[kItems];
   bool pass[kItems];
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
     const int64_t p = p0 + k * kThreads + threadIdx.x;
     keys[k] = ids[k] = -1;
-    src[k] = 0;
-    pass[k] = false;
-    if (p >= p1) continue;
+    src[k] = row[k] = off[k] = 0;
+    pass[k] = p < p1;
+    if (!pass[k]) continue;
     const int64_t lr = (staged ? upper_bound(s_ptr, nrows + 1, p)
                                : upper_bound(sub_indptr + row_lo, nrows + 1, p)) - 1;
-    const int64_t r = row_lo + lr;
-    const int64_t first = staged ? s_ptr[lr] : sub_indptr[r];
-    // a column that owns a position of the slice has passed the range check of the count
-    const int64_t c = static_cast<int64_t>(cols[r]);
-    src[k] = indptr[c] + (p - first);
-    ids[k] = static_cast<long long>(indices[src[k]]);
+    row[k] = row_lo + lr;
+    off[k] = p - (staged ? s_ptr[lr] : sub_indptr[row[k]]);
+  }
+  // a column that owns a position of the slice has passed the range check of the count
+  int64_t col[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) col[k] = pass[k] ? static_cast<int64_t>(cols[row[k]]) : 0;
+#pragma unroll
+  for (int k = 0; k < kItems; ++k)
+    if (pass[k]) src[k] = indptr[col[k]] + off[k];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k)
+    if (pass[k]) ids[k] = static_cast<long long>(indices[src[k]]);
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    if (!pass[k]) continue;
     if (B > 0) {
-      const int64_t b = upper_bound(col_ptr, B + 1, r) - 1;
+      const int64_t b = upper_bound(col_ptr, B + 1, row[k]) - 1;
       pass[k] = b >= 0 && b < B;
       keys[k] = ids[k] + b * enc;
     } else {
-      pass[k] = true;
       keys[k] = ids[k];
     }
   }
