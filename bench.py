@@ -155,6 +155,20 @@ def step_bytes(sizes):
     return sum(32 * S + 16 * E + 64 * (S + E) + 32 * E + 16 * U for S, E, U in sizes)
 
 
+def empty_pair_us(torch):
+    """What an event pair with nothing between reads on the current stream: the share of
+    avg_launch_us that is the two records' own (a kernel trace does not have it)."""
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+             for _ in range(20)]
+    torch.cuda.synchronize()
+    for a, b in pairs:
+        a.record()
+        b.record()
+    torch.cuda.synchronize()
+    reads = sorted(a.elapsed_time(b) for a, b in pairs)
+    return reads[len(reads) // 2] * 1e3
+
+
 def traffic_from_profile(site, workload):
     """HBM bytes per launch of `site` as the hardware counters gave them (FETCH_SIZE and
     WRITE_SIZE passes scaled by a device copy of known size): the line
@@ -741,6 +755,7 @@ def main():
             "launches": per_step * args.steps,
             "launches_timed": k_launches,
             "avg_launch_us": avg_s * 1e6,
+            "empty_event_pair_us": empty_pair_us(torch),
             "algorithmic_bytes_per_launch": bytes_per_launch,
             "gpu_ms_per_step_by_site": {k: round(v, 4) for k, v in site_ms.items()},
         }
