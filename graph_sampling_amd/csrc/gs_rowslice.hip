@@ -395,6 +395,20 @@ csc_compact_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t
   const int wave = threadIdx.x / kWave;
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kTile;
   const int64_t p1 = p0 + kTile < nnz ? p0 + kTile : nnz;
+  // the tile's marks, ranks and packed ids are asked for before the search for its columns
+  // (four dependent reads and a barrier), not behind it
+  unsigned long long bits[kItems];
+  int rank[kItems];
+  IdT mine[kItems];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int w = k * (kThreads / kWave) + wave;
+    const bool in = p0 + static_cast<int64_t>(w) * kWave < p1;
+    bits[k] = in ? m.mask[(p0 >> 6) + w] : 0ull;
+    rank[k] = in ? m.word_rank[(p0 >> 6) + w] : 0;
+    const int64_t r = threadIdx.x + static_cast<int64_t>(k) * kThreads;
+    mine[k] = r < count ? packed[p0 + r] : IdT(0);
+  }
   int64_t row_lo = 0, nrows = 0;
   bool staged = false;
   if (WITH_COO) {
@@ -406,16 +420,18 @@ csc_compact_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t
       for (int64_t i = threadIdx.x; i <= nrows; i += kThreads) s_ptr[i] = indptr[row_lo + i];
     __syncthreads();
   }
-  for (int64_t r = threadIdx.x; r < count; r += kThreads) out_indices[base + r] = packed[p0 + r];
+#pragma unroll
+  for (int k = 0; k < kItems; ++k) {
+    const int64_t r = threadIdx.x + static_cast<int64_t>(k) * kThreads;
+    if (r < count) out_indices[base + r] = mine[k];
+  }
   const unsigned long long lower = (1ull << lane) - 1ull;
 #pragma unroll
   for (int k = 0; k < kItems; ++k) {
     const int w = k * (kThreads / kWave) + wave;
     const int64_t e = p0 + static_cast<int64_t>(w) * kWave + lane;
-    if (e - lane >= p1) break;
-    const unsigned long long bits = m.mask[(p0 >> 6) + w];
-    if (!((bits >> lane) & 1ull)) continue;
-    const int64_t pos = base + m.word_rank[(p0 >> 6) + w] + __popcll(bits & lower);
+    if (!((bits[k] >> lane) & 1ull)) continue;
+    const int64_t pos = base + rank[k] + __popcll(bits[k] & lower);
     select_index[pos] = e;
     if (WITH_COO)
       coo_col[pos] = static_cast<IdT>(row_lo + (staged ? upper_bound(s_ptr, nrows + 1, e)
