@@ -350,12 +350,18 @@ def main():
     ladies_c = jit.compile(ladies, (A, seeds512, [512, 512]))
     flow("flow_ladies_compiled", "the same sampler through jit.compile",
          lambda: ladies_c(A, seeds512, [512, 512]), edges_of, "edges")
+    # the GraphSAGE examples load the adjacency alone (examples/graphsage/graphsage_fused.py:23-26):
+    # no edge data follows the samples
+    P = gs.Matrix().load_csc(indptr, indices)
     flow("flow_graphsage_unfused", "GraphSAGE [15,10,5], 1024 seeds, written as slice -> sample -> "
          "all_indices -> block through the Matrix layer",
-         lambda: graphsage(A, seeds1024, [15, 10, 5]), edges_of, "edges")
-    sage_c = jit.compile(graphsage, (A, seeds1024, [15, 10, 5]))
-    flow("flow_graphsage_compiled", "the same sampler through jit.compile (fused slice+sample, one "
-         "relabel per layer)",
+         lambda: graphsage(P, seeds1024, [15, 10, 5]), edges_of, "edges")
+    sage_c = jit.compile(graphsage, (P, seeds1024, [15, 10, 5]))
+    flow("flow_graphsage_compiled", "the same sampler through jit.compile (its three layers as one "
+         "chain call)",
+         lambda: sage_c(P, seeds1024, [15, 10, 5]), edges_of, "edges")
+    flow("flow_graphsage_compiled_weights", "the compiled sampler on the graph with edge weights "
+         "(the weights follow the samples: layer by layer)",
          lambda: sage_c(A, seeds1024, [15, 10, 5]), edges_of, "edges")
 
 

@@ -41,6 +41,8 @@ TORCH_LIBRARY(gs_classes, m) {
               &Graph::ColumnwiseFusedSlicingAndSampling)
       // not in the reference: the per-layer loop of its GraphSAGE examples as one call
       GS_DEF2("_CAPI_SampleLayers", "_CAPI_sample_layers", &Graph::SampleLayers)
+      GS_DEF2("_CAPI_SampleLayersIfQueued", "_CAPI_sample_layers_if_queued",
+              &Graph::SampleLayersIfQueued)
       GS_DEF2("_CAPI_FusionSlicing", "_CAPI_fusion_slicing", &Graph::FusedBidirSlicing)
       GS_DEF2("_CAPI_BatchFusionSlicing", "_CAPI_batch_fusion_slicing",
               &Graph::BatchFusedBidirSlicing)

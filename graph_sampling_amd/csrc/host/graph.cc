@@ -459,11 +459,11 @@ std::vector<torch::Tensor> Graph::SampleLayersLoop(torch::Tensor seeds,
   return out;
 }
 
-std::vector<torch::Tensor> Graph::SampleLayers(torch::Tensor seeds, std::vector<int64_t> fanouts,
-                                               bool replace) {
-  Range range("gs::SampleLayers");
+std::vector<torch::Tensor> Graph::SampleLayersIfQueued(torch::Tensor seeds,
+                                                        std::vector<int64_t> fanouts,
+                                                        bool replace) {
   auto pending = QueueLayers(seeds, fanouts, replace);
-  if (!pending) return SampleLayersLoop(seeds, fanouts, replace);
+  if (!pending) return {};
   try {
     return pending->Collect();
   } catch (const hip::IdsTooWide&) {
@@ -474,6 +474,14 @@ std::vector<torch::Tensor> Graph::SampleLayers(torch::Tensor seeds, std::vector<
     hip::RestoreSeedState(saved);
     return out;
   }
+}
+
+std::vector<torch::Tensor> Graph::SampleLayers(torch::Tensor seeds, std::vector<int64_t> fanouts,
+                                               bool replace) {
+  Range range("gs::SampleLayers");
+  auto out = SampleLayersIfQueued(seeds, fanouts, replace);
+  if (out.empty() && !fanouts.empty()) return SampleLayersLoop(seeds, fanouts, replace);
+  return out;
 }
 
 // The reference hands the kernel the GLOBAL ids of the seeds (src/graph.cc:120-128), which

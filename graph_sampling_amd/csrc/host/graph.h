@@ -122,6 +122,12 @@ class Graph : public torch::CustomClassHolder {
   // in between and the sizes are collected once at the end.
   std::vector<torch::Tensor> SampleLayers(torch::Tensor seeds, std::vector<int64_t> fanouts,
                                           bool replace);
+  // SampleLayers where the whole minibatch can be queued on the device (a root graph without
+  // edge data or id maps, sizes the layer chain takes); otherwise nothing is sampled, no seed
+  // is consumed and the list is empty, so that a caller who needs edge data or edge ids for
+  // its blocks goes layer by layer itself.
+  std::vector<torch::Tensor> SampleLayersIfQueued(torch::Tensor seeds,
+                                                  std::vector<int64_t> fanouts, bool replace);
   // The first half of SampleLayers when the whole minibatch can be queued (else nullptr, and
   // no seed is consumed): the caller collects later, other minibatches may be queued
   // meanwhile.  A collect that throws hip::IdsTooWide is answered with SampleLayersLoop under

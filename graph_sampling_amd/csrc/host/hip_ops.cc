@@ -63,6 +63,14 @@ const void* OptIds(const torch::optional<torch::Tensor>& t, int idb, const char*
   return t.value().data_ptr();
 }
 
+// The edge array (or edge weights) of a graph for a sampling call.  A graph without edges has
+// an empty tensor there, whose pointer is null, and the entry points refuse a null array as
+// long as there are columns; no degree is above zero then, so nothing is read through the
+// pointer, and the offsets' address stands in.
+const void* EdgeArray(const torch::Tensor& edges, const torch::Tensor& indptr) {
+  return edges.numel() > 0 ? edges.data_ptr() : indptr.data_ptr();
+}
+
 torch::Tensor Scratch(size_t bytes, const torch::Tensor& like) {
   return torch::empty({static_cast<int64_t>(bytes < 256 ? 256 : bytes)},
                       torch::dtype(torch::kUInt8).device(like.device()));
@@ -373,7 +381,7 @@ std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
   p->box = boxes.slot(p->ticket);
   p->box_owner = boxes.buf;
   p->state_owner = state.buf;
-  Check(gs_sample_uniform_fused(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(),
+  Check(gs_sample_uniform_fused(indptr.data_ptr<int64_t>(), indptr.numel() - 1, EdgeArray(indices, indptr),
                                 fused ? column_ids.data_ptr() : nullptr, idb, p->S, fanout,
                                 replace ? 1 : 0, NextSeed(), nullptr, nullptr,
                                 p->sub_indptr.data_ptr<int64_t>(), p->indices.data_ptr(),
@@ -410,7 +418,7 @@ SliceResult ColSampling(const torch::Tensor& indptr, const torch::Tensor& indice
       indptr, indices, column_ids, fanout, replace, with_coo, 0,
       [&](const void* cols, int idb, int64_t S, torch::Tensor& sub_indptr, torch::Tensor& sub_indices,
           torch::Tensor& select_index, torch::Tensor& coo_col, torch::Tensor& ws, void* st) {
-        Check(gs_sample_uniform_fill(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), cols, idb, S,
+        Check(gs_sample_uniform_fill(indptr.data_ptr<int64_t>(), indptr.numel() - 1, EdgeArray(indices, indptr), cols, idb, S,
                                      fanout, replace ? 1 : 0, static_cast<int>(g_algo.load()),
                                      NextSeed(), nullptr, nullptr, sub_indptr.data_ptr<int64_t>(),
                                      sub_indices.data_ptr(), select_index.data_ptr<int64_t>(),
@@ -447,8 +455,8 @@ SliceResult ColSamplingProbs(const torch::Tensor& indptr, const torch::Tensor& i
             torch::Tensor& sub_indices, torch::Tensor& select_index, torch::Tensor& coo_col,
             torch::Tensor&, void* st) {
           Check(gs_sample_weighted_replace(
-                    indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(),
-                    probs.data_ptr<float>(), cols, idb, S_, fanout, NextSeed(), nullptr,
+                    indptr.data_ptr<int64_t>(), indptr.numel() - 1, EdgeArray(indices, indptr),
+                    static_cast<const float*>(EdgeArray(probs, indptr)), cols, idb, S_, fanout, NextSeed(), nullptr,
                     sub_indptr.data_ptr<int64_t>(), cdf_ptr.data_ptr<int64_t>(),
                     cdf.data_ptr<float>(), sub_indices.data_ptr(),
                     select_index.data_ptr<int64_t>(), with_coo ? coo_col.data_ptr() : nullptr, st),
@@ -461,8 +469,8 @@ SliceResult ColSamplingProbs(const torch::Tensor& indptr, const torch::Tensor& i
       [&](const void* cols, int idb, int64_t S_, torch::Tensor& sub_indptr,
           torch::Tensor& sub_indices, torch::Tensor& select_index, torch::Tensor& coo_col,
           torch::Tensor& ws, void* st) {
-        Check(gs_sample_weighted_fill(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(),
-                                      probs.data_ptr<float>(), cols, idb, S_, fanout, NextSeed(),
+        Check(gs_sample_weighted_fill(indptr.data_ptr<int64_t>(), indptr.numel() - 1, EdgeArray(indices, indptr),
+                                      static_cast<const float*>(EdgeArray(probs, indptr)), cols, idb, S_, fanout, NextSeed(),
                                       nullptr, nullptr, sub_indptr.data_ptr<int64_t>(),
                                       sub_indices.data_ptr(), select_index.data_ptr<int64_t>(),
                                       with_coo ? coo_col.data_ptr() : nullptr, ws.data_ptr(),
@@ -480,7 +488,7 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> SampleOneKeepDim(
   auto sub_indptr = torch::empty({S + 1}, I64(indptr));
   auto sub_indices = torch::empty({S}, indices.options());
   auto select_index = torch::empty({S}, I64(indptr));
-  Check(gs_sample_one_keepdim(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), column_ids.data_ptr(),
+  Check(gs_sample_one_keepdim(indptr.data_ptr<int64_t>(), indptr.numel() - 1, EdgeArray(indices, indptr), column_ids.data_ptr(),
                               idb, S, NextSeed(), nullptr, sub_indptr.data_ptr<int64_t>(),
                               sub_indices.data_ptr(), select_index.data_ptr<int64_t>(),
                               Stream(indptr)),
@@ -733,7 +741,7 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
     FusedStateBuf& st1 = FusedState(state_bytes, indptr, p->stream);
     if (l == 0) p->state_owner = st1.buf;
     y.ticket_edges = boxes.next++;
-    Check(gs_layer_sample(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), cols,
+    Check(gs_layer_sample(indptr.data_ptr<int64_t>(), indptr.numel() - 1, EdgeArray(indices, indptr), cols,
                           idb, S[l], S_dev, fanouts[l], replace ? 1 : 0, seed, nullptr, nullptr,
                           offsets, base + off_ids[l], cap, counts, table,
                           table_bytes, base + off_ws[l], ws_bytes[l], st1.buf.data_ptr(),

@@ -8,6 +8,10 @@
   next layer's seeds, which is what keeps consecutive blocks aligned.
 * `fuse_slicing_and_sampling` -- a column slice whose only consumer is a uniform column
   sampling becomes the fused operator that never writes the slice (optimize.py:62-82).
+* `chain_sampled_layers` -- consecutive layers of the GraphSAGE loop (fused slice + sample of
+  one graph, `Relabel`, next seeds = the frontier; examples/graphsage/batching.py:125-138)
+  become one `sample_layer_chain` call, which queues every layer on the device at once where
+  the graph allows it and goes layer by layer where it does not.  Not in the reference.
 * `common_subexpressions` -- repeated pure queries of one graph (valid rows, sums, ...) are
   made once (python/gs/jit/passes.py:40-58, restricted here to calls known to be pure:
   sampling calls draw fresh random numbers and must stay apart).
@@ -16,6 +20,7 @@
 """
 import operator
 
+import torch
 import torch.fx as fx
 
 from ..format import _COO, _CSC
@@ -108,6 +113,90 @@ def fuse_slicing_and_sampling(gm: fx.GraphModule) -> fx.GraphModule:
     return dead_code(gm)
 
 
+def sample_layer_chain(graph, seeds, fanouts, replace):
+    """[(tuple of `Graph::Relabel`, edge data)] per layer of a GraphSAGE-style minibatch, the
+    values the per-layer calls `_CAPI_FusedColumnwiseSlicingSampling` -> `_CAPI_Relabel` /
+    `_CAPI_GetData('default')` give under the same seed.  A root graph without edge data takes
+    the whole minibatch in one call of the C++ layer; its blocks have no edge ids and ones as
+    edge data, as the per-layer calls find on a graph without data (src/graph.cc:68-73)."""
+    fanouts = list(fanouts)
+    parts = graph._CAPI_SampleLayersIfQueued(seeds, fanouts, bool(replace))
+    layers = []
+    if parts:
+        num_dst = seeds.numel()
+        for l in range(len(fanouts)):
+            frontier, indptr, indices = parts[3 * l:3 * l + 3]
+            ones = torch.ones(indices.numel(), dtype=torch.float32, device=indices.device)
+            layers.append(((frontier, frontier.numel(), num_dst, indptr, indices, None, "csc"), ones))
+            num_dst = frontier.numel()
+        return layers
+    for k in fanouts:
+        sub = graph._CAPI_FusedColumnwiseSlicingSampling(seeds, k, replace)
+        relabel = sub._CAPI_Relabel()
+        layers.append((relabel, sub._CAPI_GetData("default")))
+        seeds = relabel[0]
+    return layers
+
+
+def _layer_of(fused):
+    """(relabel, [data queries]) when `fused` is used for its block only, else None."""
+    relabel, data = None, []
+    for user in fused.users:
+        if _is_method(user, RELABEL) and relabel is None and user.args == (fused,):
+            relabel = user
+        elif (_is_method(user, ("_CAPI_GetData", "_CAPI_get_data")) and
+              user.args == (fused, "default") and not user.kwargs):
+            data.append(user)
+        else:
+            return None
+    return (relabel, data) if relabel is not None else None
+
+
+def chain_sampled_layers(gm: fx.GraphModule) -> fx.GraphModule:
+    layer_of = {n: _layer_of(n) for n in gm.graph.nodes
+                if _is_method(n, (FUSED,)) and len(n.args) == 4 and not n.kwargs}
+    layer_of = {n: l for n, l in layer_of.items() if l is not None}
+
+    def follower(fused):
+        # the layer whose seeds are this layer's frontier, on the same graph and replace flag
+        for item in layer_of[fused][0].users:
+            if not (item.op == "call_function" and item.target is operator.getitem and
+                    item.args[1] == 0):
+                continue
+            for nxt in item.users:
+                if (nxt in layer_of and nxt.args[1] is item and nxt.args[0] is fused.args[0] and
+                        nxt.args[3] == fused.args[3] and isinstance(nxt.args[2], int)):
+                    return nxt
+        return None
+
+    followers = {n: follower(n) for n in layer_of}
+    followed = set(f for f in followers.values() if f is not None)
+    for head in [n for n in layer_of if n not in followed and isinstance(n.args[2], int)]:
+        chain = [head]
+        while followers.get(chain[-1]) is not None:
+            chain.append(followers[chain[-1]])
+        if len(chain) < 2:
+            continue
+        parent, seeds, _, replace = head.args
+        with gm.graph.inserting_before(head):
+            layers = gm.graph.call_function(
+                sample_layer_chain, (parent, seeds, [n.args[2] for n in chain], replace))
+            for l, fused in enumerate(chain):
+                layer = gm.graph.call_function(operator.getitem, (layers, l))
+                relabel, data = layer_of[fused]
+                relabel.replace_all_uses_with(gm.graph.call_function(operator.getitem, (layer, 0)))
+                if data:
+                    values = gm.graph.call_function(operator.getitem, (layer, 1))
+                    for query in data:
+                        query.replace_all_uses_with(values)
+        # later layers first: each one's seeds are a use of the layer before
+        for fused in reversed(chain):
+            relabel, data = layer_of[fused]
+            for node in data + [relabel, fused]:
+                gm.graph.erase_node(node)
+    return dead_code(gm)
+
+
 def common_subexpressions(gm: fx.GraphModule) -> fx.GraphModule:
     seen = {}
     for node in list(gm.graph.nodes):
@@ -126,5 +215,5 @@ def common_subexpressions(gm: fx.GraphModule) -> fx.GraphModule:
     return _finish(gm)
 
 
-DEFAULT = (merge_relabel_and_all_indices, fuse_slicing_and_sampling, common_subexpressions,
-           dead_code)
+DEFAULT = (merge_relabel_and_all_indices, fuse_slicing_and_sampling, chain_sampled_layers,
+           common_subexpressions, dead_code)

@@ -915,6 +915,32 @@ def test_sample_layers_with_no_seeds_and_with_isolated_seeds(dev, idt):
         _same(got, _oracle_minibatch(indptr, indices, seeds, (2, 2, 2), False, 3))
 
 
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+@pytest.mark.parametrize("fanout,replace", [(2, False), (2, True), (1, True), (40, False)])
+def test_sampling_a_slice_without_edges(dev, idt, fanout, replace):
+    """Slice first, then sample (the sampler without the fused operator): when none of the
+    seeds has a neighbour the slice holds no edge at all, and every kind of column sampling
+    of it is an empty graph over the same columns."""
+    indptr = np.array([0, 0, 2, 2, 3], dtype=np.int64)   # columns 0 and 2 have no edges
+    indices = np.array([3, 1, 1], dtype=np.int64)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev, idt))
+    sliced = g._CAPI_Slicing(to_dev(np.array([0, 2, 0], dtype=np.int64), dev, idt), 0, _CSC, _COO,
+                             False)
+    assert sliced._CAPI_GetNumEdges() == 0
+    probs = torch.zeros(0, **F(dev))
+    for sub in (sliced._CAPI_Sampling(0, fanout, replace, _CSC, _COO),
+                sliced._CAPI_Sampling(0, fanout, replace, _CSC, _CSC),
+                sliced._CAPI_SamplingWithProbs(0, probs, min(fanout, 32), replace, _CSC, _COO)):
+        ptr, idx, _ = sub._CAPI_GetCSC()
+        if fanout == 1 and replace and idx.numel():  # one slot per column, -1 where it is empty
+            assert idx.cpu().tolist() == [-1, -1, -1] and ptr.cpu().tolist() == [0, 1, 2, 3]
+            continue
+        assert ptr.cpu().tolist() == [0, 0, 0, 0] and idx.numel() == 0
+        frontier = sub._CAPI_Relabel()[0]
+        assert frontier.cpu().tolist() == [0, 2]
+
+
 def test_sample_layers_python_helper_returns_blocks(dev):
     m, indptr, indices, _ = _rmat_matrix(dev, 12, 16, 3)
     seeds = to_dev(np.arange(100, dtype=np.int64), dev)

@@ -31,10 +31,12 @@ def _same_block(a, b):
 
 
 @pytest.mark.parametrize("with_data", [False, True])
-def test_compiled_graphsage_equals_eager(dev, with_data):
+@pytest.mark.parametrize("chained", [False, True])
+def test_compiled_graphsage_equals_eager(dev, with_data, chained):
     A = _matrix(dev, 13, 17, 1, with_data)
-    compiled = jit.compile(graphsage, (A, torch.arange(4, device=dev), [10, 5]))
-    assert passes.FUSED in compiled.code
+    rewrites = tuple(p for p in passes.DEFAULT if chained or p is not passes.chain_sampled_layers)
+    compiled = jit.compile(graphsage, (A, torch.arange(4, device=dev), [10, 5]), passes=rewrites)
+    assert ("sample_layer_chain" if chained else passes.FUSED) in compiled.code
     for trial in range(3):  # replays: fresh seeds and sizes on the same trace
         seeds = torch.randperm(1 << 13, device=dev)[:200 + 50 * trial]
         gs.set_seed(40 + trial)
@@ -44,6 +46,46 @@ def test_compiled_graphsage_equals_eager(dev, with_data):
         assert torch.equal(got_nodes, want_nodes)
         for g, w in zip(got_blocks, want_blocks):
             _same_block(g, w)
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_chained_layers_of_three_on_a_root_and_on_a_slice(dev, replace):
+    """The chain call takes a root graph in one call of the C++ layer and a row slice (a graph
+    with an id map, whose columns are still all the nodes) layer by layer: both give the
+    per-layer sampler's minibatch, and the next call draws with the seed the loop would have
+    reached."""
+    def sampler(A, seeds, fanouts):
+        blocks = []
+        for k in fanouts:
+            sub = A[:, seeds].columnwise_sampling(k, replace)
+            seeds = sub.all_indices()
+            blocks.insert(0, sub.to_dgl_block())
+        return seeds, blocks
+
+    root = _matrix(dev, 14, 19, 3)
+    fanouts = [15, 10, 5]
+    compiled = jit.compile(sampler, (root, torch.arange(4, device=dev), fanouts))
+    assert "sample_layer_chain(" in compiled.code and passes.FUSED not in compiled.code
+    # on a graph with a row id list the sampler itself orders the next seeds by that list, the
+    # rewritten one by the block (merge_relabel_and_all_indices): the yardstick there is the
+    # rewritten sampler without the chain
+    per_layer = jit.compile(sampler, (root, torch.arange(4, device=dev), fanouts),
+                            passes=tuple(p for p in passes.DEFAULT
+                                         if p is not passes.chain_sampled_layers))
+    # (the fused operator reads a CSC: the rows are sliced on that format and kept in it)
+    kept = torch.arange(0, 1 << 14, 2, device=dev)
+    sliced = gs.Matrix(root._graph._CAPI_Slicing(kept, 1, gs._CSC, gs._CSC, False))
+    for A in (root, sliced):
+        for trial, count in enumerate((1024, 1, 3000)):
+            seeds = torch.randperm(1 << 13, device=dev)[:count]
+            gs.set_seed(90 + trial)
+            want = [(sampler if A is root else per_layer)(A, seeds, fanouts) for _ in range(2)]
+            gs.set_seed(90 + trial)
+            got = [compiled(A, seeds, fanouts) for _ in range(2)]
+            for (got_nodes, got_blocks), (want_nodes, want_blocks) in zip(got, want):
+                assert torch.equal(got_nodes, want_nodes)
+                for g, w in zip(got_blocks, want_blocks):
+                    _same_block(g, w)
 
 
 def ladies_one_frontier(A, seeds, fanouts):

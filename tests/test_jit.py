@@ -42,8 +42,11 @@ def test_raw_trace_records_the_calls_of_the_matrix_api():
     assert t.count("_CAPI_Relabel") == 2 and t.count("_CAPI_AllValidNode") == 2
 
 
+PER_LAYER = tuple(p for p in passes.DEFAULT if p is not passes.chain_sampled_layers)
+
+
 def test_rewrites_fuse_slice_with_sample_and_share_one_relabel():
-    c = jit.compile(graphsage, (gs.Matrix(), torch.arange(4), [10, 5]))
+    c = jit.compile(graphsage, (gs.Matrix(), torch.arange(4), [10, 5]), passes=PER_LAYER)
     t = _targets(c)
     assert t.count(passes.FUSED) == 2
     assert "_CAPI_Slicing" not in t and "_CAPI_Sampling" not in t
@@ -51,6 +54,69 @@ def test_rewrites_fuse_slice_with_sample_and_share_one_relabel():
     # the fused call takes (seeds, fanout, replace) of the pair it replaces
     fused = [n for n in c.gm.graph.nodes if n.target == passes.FUSED]
     assert [n.args[2:] for n in fused] == [(10, False), (5, False)]
+
+
+def _functions(compiled):
+    return [n for n in compiled.gm.graph.nodes if n.op == "call_function"]
+
+
+def test_consecutive_layers_become_one_chain_call():
+    c = jit.compile(graphsage, (gs.Matrix(), torch.arange(4), [10, 5, 3]))
+    assert _targets(c) == []  # no per-layer call is left
+    chains = [n for n in _functions(c) if n.target is passes.sample_layer_chain]
+    assert len(chains) == 1
+    graph, seeds, fanouts, replace = chains[0].args
+    assert fanouts == [10, 5, 3] and replace is False
+    # the three blocks are made of layers 0, 1, 2 of the chain, and the sampler's seeds are
+    # the last layer's frontier
+    blocks = [n for n in _functions(c) if n.target is gs.block.make_block]
+    assert [b.args[0].args[0].args for b in blocks] == [(chains[0], l) for l in range(3)]
+    nodes, made = c.gm.graph.output_node().args[0]
+    assert made == blocks[::-1] and nodes.args == (blocks[2].args[0], 0)
+
+
+def test_layers_are_chained_only_where_the_loop_is_the_plain_one():
+    def one_layer(A, seeds):
+        return A[:, seeds].columnwise_sampling(3, False).to_dgl_block()
+
+    def sample_kept(A, seeds):  # the sampled matrix itself is asked for its rows as well
+        blocks, rows = [], []
+        for k in (4, 2):
+            sub = A[:, seeds].columnwise_sampling(k, False)
+            rows.append(sub.row_ids())
+            seeds = sub.all_indices()
+            blocks.append(sub.to_dgl_block())
+        return blocks, rows
+
+    def two_graphs(A, B, seeds):
+        sub = A[:, seeds].columnwise_sampling(4, False)
+        nxt = B[:, sub.all_indices()].columnwise_sampling(2, False)
+        return sub.to_dgl_block(), nxt.to_dgl_block()
+
+    def mixed_replace(A, seeds):
+        sub = A[:, seeds].columnwise_sampling(4, False)
+        nxt = A[:, sub.all_indices()].columnwise_sampling(2, True)
+        return sub.to_dgl_block(), nxt.to_dgl_block()
+
+    for sampler, args in ((one_layer, (gs.Matrix(), torch.arange(4))),
+                          (sample_kept, (gs.Matrix(), torch.arange(4))),
+                          (two_graphs, (gs.Matrix(), gs.Matrix(), torch.arange(4))),
+                          (mixed_replace, (gs.Matrix(), torch.arange(4)))):
+        c = jit.compile(sampler, args)
+        assert not [n for n in _functions(c) if n.target is passes.sample_layer_chain], sampler
+        assert passes.FUSED in _targets(c)
+
+
+def test_a_chain_may_start_behind_other_work_and_two_chains_stay_apart():
+    def sampler(A, seeds, more):
+        first = graphsage(A, torch.cat((seeds, more)), [4, 2])
+        second = graphsage(A, more, [3, 3, 3])
+        return first, second
+
+    c = jit.compile(sampler, (gs.Matrix(), torch.arange(4), torch.arange(2)))
+    chains = [n for n in _functions(c) if n.target is passes.sample_layer_chain]
+    assert [n.args[2] for n in chains] == [[4, 2], [3, 3, 3]]
+    assert passes.FUSED not in _targets(c)
 
 
 def test_slice_with_a_second_consumer_is_not_fused():
