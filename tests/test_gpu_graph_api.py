@@ -646,6 +646,48 @@ def test_pending_graph_outlives_its_mailbox_slot(dev):
     assert np.array_equal(sub._CAPI_GetCSC()[1].cpu().numpy(), rows)
 
 
+def test_pending_graph_settled_by_another_thread(dev):
+    """A producer thread samples and hands the unsettled graphs over; the consumer (here the
+    main thread, after the producer has exited and after calls of its own have used the same
+    ticket numbers) relabels them and asks for their edges: it must wait on the producer's
+    mailbox slots, not on its own."""
+    import threading
+    m, indptr, indices, _ = _rmat_matrix(dev, 12, 16, 9)
+    rng = np.random.default_rng(11)
+    seed_sets = [rng.permutation(1 << 12)[:200 + 40 * i].astype(np.int64) for i in range(4)]
+    handed, errors = [], []
+
+    def producer():
+        try:
+            for i, seeds in enumerate(seed_sets):
+                torch.ops.gs_ops._CAPI_SetThreadSeed(600 + i)
+                handed.append(m._graph._CAPI_FusedColumnwiseSlicingSampling(to_dev(seeds, dev), 5,
+                                                                            False))
+        except Exception as e:
+            errors.append(e)
+
+    t = threading.Thread(target=producer)
+    t.start()
+    t.join()
+    assert not errors, errors
+    # calls of the consumer's own: its ring hands out the ticket numbers the producer's did
+    for _ in range(3):
+        m._graph._CAPI_FusedColumnwiseSlicingSampling(to_dev(seed_sets[0][:7], dev), 2,
+                                                      False)._CAPI_GetNumEdges()
+    for i, (sub, seeds) in enumerate(zip(handed, seed_sets)):
+        w_ptr, _, w_rows, _ = O.sample_uniform(indptr, indices, seeds, 5, False, seed=600 + i,
+                                               with_coo=False)
+        if i % 2 == 0:
+            frontier, n_src, n_dst, ptr, idx, _, _ = sub._CAPI_Relabel()
+            w_frontier, (w_idx,) = O.relabel([seeds, w_rows], [w_rows])
+            assert n_dst == seeds.size and n_src == w_frontier.size
+            assert np.array_equal(frontier.cpu().numpy(), w_frontier)
+            assert np.array_equal(ptr.cpu().numpy(), w_ptr)
+            assert np.array_equal(idx.cpu().numpy(), w_idx)
+        assert sub._CAPI_GetNumEdges() == w_rows.size
+        assert np.array_equal(sub._CAPI_GetCSC()[1].cpu().numpy(), w_rows)
+
+
 def test_deferred_sampling_switch_gives_identical_results(dev):
     outs = []
     for mode in (True, False):
