@@ -980,6 +980,16 @@ def csc2coo(indptr, nnz, id_dtype=torch.int64):
     return col
 
 
+def dcsc2coo(indptr, nnz, ids):
+    """Column of every edge of a doubly-compressed CSC: `ids[c]` for the edges of stored
+    column c (`indptr` runs over the stored columns only)."""
+    _need(indptr, torch.int64, "indptr")
+    col = torch.empty(nnz, dtype=ids.dtype, device=indptr.device)
+    _check(lib().gs_dcsc2coo(_ptr(indptr), _i64(indptr.numel() - 1), _i64(nnz), _ptr(ids),
+                             _ptr(col), _id_bytes(col), _stream(indptr.device)), "gs_dcsc2coo")
+    return col
+
+
 def coo2csc(key, value, num_keys, is_sorted):
     """Returns (indptr, sorted value | value, perm | None)."""
     idb = _ids(key, "key")

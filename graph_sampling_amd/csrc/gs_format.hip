@@ -5,11 +5,11 @@
 // src/cuda/format_transform.cu:35,135; the reference leans on cub radix sort,
 // whose stability pins the edge order, format_transform.cu:81-100).
 //
-//  * csc2coo: edge-balanced.  A workgroup owns 4096 consecutive edges, finds the
-//    columns they span with two binary searches, lets those columns mark their
-//    first edge in LDS and turns the marks into column numbers with a running
-//    maximum (the reference runs a full global binary search per edge,
-//    format_transform.cu:24-33).
+//  * csc2coo: edge-balanced.  A workgroup owns 4096 consecutive edges; a first
+//    launch over the columns has left the column of each tile's first edge in the
+//    output, the offsets are read in order from there, the columns mark their first
+//    edge in LDS and a running maximum turns the marks into column numbers (the
+//    reference runs a full global binary search per edge, format_transform.cu:24-33).
 //  * coo2csc: 8-bit digits, only ceil(log2(num_keys)/8) passes
 //    (format_transform.cu:58-72 also sorts just the significant bits).  Each
 //    pass is histogram -> scan -> stable scatter; the scatter ranks equal digits
@@ -41,28 +41,79 @@ __device__ __forceinline__ int64_t upper_bound(P a, int64_t n, int64_t v) {
 constexpr int kCooItems = 16;
 constexpr int kCooTile = kThreads * kCooItems;
 
-// A workgroup owns kCooTile consecutive edges.  The columns that start inside the tile mark
-// their first edge in LDS (column-parallel, coalesced reads of the offsets; of several empty
-// columns at one position the highest wins, which is the owner), and a running maximum
-// over the marks gives every edge its column: sixteen consecutive edges per thread, one
-// maximum per thread across the workgroup.  No search per edge.
+// (A thread's sixteen marks lie side by side; one spare word after every sixteen keeps the
+// threads of a wave on different LDS banks when each walks its own run.)
+__device__ __forceinline__ int coo_slot(int i) { return i + (i >> 4); }
+
+// First of two launches: every column with edges writes its number at the first position of
+// each 4096-edge tile that begins inside it, so that the tile's workgroup finds the column
+// of its first edge with one read instead of a search through the offsets.  The numbers go
+// into the output itself (the tile overwrites its own first entry at the end).  A column
+// that spans more than 64 tiles is written by its whole wave.
 template <typename IdT>
+__global__ void __launch_bounds__(kThreads)
+coo_tile_heads_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, IdT* __restrict__ col) {
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  int64_t t0 = 0, t1 = -1;
+  if (c < num_cols) {
+    const int64_t s = indptr[c], e = indptr[c + 1];
+    if (e > s) {
+      t0 = (s + kCooTile - 1) / kCooTile;
+      t1 = (e - 1) / kCooTile;
+    }
+  }
+  const bool wide = t1 - t0 >= kWave;
+  if (!wide)
+    for (int64_t t = t0; t <= t1; ++t) col[t * kCooTile] = static_cast<IdT>(c);
+  unsigned long long todo = __ballot(wide);
+  const int lane = threadIdx.x & (kWave - 1);
+  while (todo) {
+    const int src = __ffsll(static_cast<long long>(todo)) - 1;
+    todo &= todo - 1;
+    const int64_t w0 = __shfl(t0, src, kWave), w1 = __shfl(t1, src, kWave);
+    const int64_t wc = __shfl(c, src, kWave);
+    for (int64_t t = w0 + lane; t <= w1; t += kWave) col[t * kCooTile] = static_cast<IdT>(wc);
+  }
+}
+
+// A workgroup owns kCooTile consecutive edges.  The first entry of its output holds the last
+// column that starts at or before the tile (left there by the launch above); from there the
+// offsets are read in order, 256 at a time.  The columns that start inside the tile mark
+// their first edge in LDS (of several empty columns at one position the highest wins, which
+// is the owner), and a running maximum over the marks gives every edge its column: sixteen
+// consecutive edges per thread, one maximum per thread across the workgroup.  No search.
+// (DCSC: stored column c stands for node ids[c], format_transform.cu:48-60; a switch at
+// compile time, because a load that may or may not happen before a store makes every store
+// wait for everything in flight.)
+template <typename IdT, bool DCSC>
 __global__ void __launch_bounds__(kThreads)
 csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz,
                const IdT* __restrict__ ids, IdT* __restrict__ col) {
-  __shared__ int s_mark[kCooTile];
-  __shared__ int64_t s_rows[2];
+  __shared__ int s_mark[kCooTile + kCooTile / 16];
   __shared__ int s_wave[kThreads / kWave];
+  __shared__ bool s_more;
   const int64_t p0 = static_cast<int64_t>(blockIdx.x) * kCooTile;
   const int64_t p1 = p0 + kCooTile < nnz ? p0 + kCooTile : nnz;
-  for (int i = threadIdx.x; i < kCooTile; i += kThreads) s_mark[i] = 0;
-  block_row_range(indptr, num_cols, p0, p1 - 1, s_rows);
-  const int64_t row_lo = s_rows[0], row_hi = s_rows[1];
-  // columns row_lo + 1 .. row_hi start inside the tile (row_lo holds its first edge)
-  for (int64_t r = row_lo + 1 + threadIdx.x; r <= row_hi; r += kThreads)
-    atomicMax(&s_mark[indptr[r] - p0], static_cast<int>(r - row_lo));
+  const int64_t base = static_cast<int64_t>(col[p0]);  // holds edge p0
+  for (int i = threadIdx.x; i < kCooTile + kCooTile / 16; i += kThreads) s_mark[i] = 0;
+  const int64_t kNone = INT64_MAX;
+  int64_t ahead = base + 1 + threadIdx.x <= num_cols ? indptr[base + 1 + threadIdx.x] : kNone;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   __syncthreads();
-  const int at0 = threadIdx.x * kCooItems;
+  // columns base + 1 ... that start before p1 start inside the tile (after p0: the last one
+  // that starts at p0 is the base); the offsets are in order, so the last thread tells
+  // whether the next 256 have to be looked at as well
+  for (int64_t r = base + 1 + threadIdx.x;; r += kThreads) {
+    const bool inside = ahead < p1;
+    if (inside)
+      atomicMax(&s_mark[coo_slot(static_cast<int>(ahead - p0))], static_cast<int>(r - base));
+    if (threadIdx.x == kThreads - 1) s_more = inside;
+    __syncthreads();
+    if (!s_more) break;
+    ahead = r + kThreads <= num_cols ? indptr[r + kThreads] : kNone;
+    __syncthreads();  // (everyone has read the flag before it is written again)
+  }
+  const int at0 = threadIdx.x * (kCooItems + 1);
   int m[kCooItems];
   int run = 0;
 #pragma unroll
@@ -72,7 +123,6 @@ csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz
     m[k] = run;  // relative to what holds where the thread begins
   }
   // exclusive running maximum of the threads' last values
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   int incl = run;
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
@@ -84,22 +134,34 @@ csc2coo_kernel(const int64_t* __restrict__ indptr, int64_t num_cols, int64_t nnz
   int before = __shfl_up(incl, 1, kWave);
   if (lane == 0) before = 0;
   for (int w = 0; w < wave; ++w) before = s_wave[w] > before ? s_wave[w] : before;
-  // column numbers (relative to row_lo) go back into the marks' place, so that the stores
+  // column numbers (relative to base) go back into the marks' place, so that the stores
   // below are coalesced whatever the id width
-  __syncthreads();
 #pragma unroll
   for (int k = 0; k < kCooItems; ++k) s_mark[at0 + k] = m[k] > before ? m[k] : before;
   __syncthreads();
+  IdT out[kCooItems];
 #pragma unroll
   for (int k = 0; k < kCooItems; ++k) {
-    const int i = k * kThreads + threadIdx.x;
-    const int64_t p = p0 + i;
-    if (p < p1) {
-      const int64_t c = row_lo + s_mark[i];
-      // doubly-compressed: stored column c stands for node ids[c] (format_transform.cu:48-60)
-      col[p] = ids ? ids[c] : static_cast<IdT>(c);
-    }
+    const int64_t c = base + s_mark[coo_slot(k * kThreads + threadIdx.x)];
+    if (DCSC)
+      out[k] = p0 + k * kThreads + threadIdx.x < p1 ? ids[c] : IdT(0);
+    else
+      out[k] = static_cast<IdT>(c);
   }
+#pragma unroll
+  for (int k = 0; k < kCooItems; ++k) {
+    const int64_t p = p0 + k * kThreads + threadIdx.x;
+    if (p < p1) col[p] = out[k];
+  }
+}
+
+template <typename IdT, bool DCSC>
+void launch_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, const IdT* ids, IdT* col,
+                    hipStream_t st) {
+  hipLaunchKernelGGL((coo_tile_heads_kernel<IdT>), dim3(blocks_for(num_cols, kThreads)),
+                     dim3(kThreads), 0, st, indptr, num_cols, col);
+  hipLaunchKernelGGL((csc2coo_kernel<IdT, DCSC>), dim3(blocks_for(nnz, kCooTile)), dim3(kThreads),
+                     0, st, indptr, num_cols, nnz, ids, col);
 }
 
 // CSC -> doubly-compressed CSC: the columns that own at least one edge, in order, and
@@ -575,13 +637,9 @@ int gs_csc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, void* col, 
   if (nnz == 0) return GS_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (id_bytes == 8)
-    hipLaunchKernelGGL((csc2coo_kernel<int64_t>), dim3(blocks_for(nnz, kCooTile)), dim3(kThreads), 0,
-                       st, indptr, num_cols, nnz, static_cast<const int64_t*>(nullptr),
-                       static_cast<int64_t*>(col));
+    launch_csc2coo<int64_t, false>(indptr, num_cols, nnz, nullptr, static_cast<int64_t*>(col), st);
   else
-    hipLaunchKernelGGL((csc2coo_kernel<int32_t>), dim3(blocks_for(nnz, kCooTile)), dim3(kThreads), 0,
-                       st, indptr, num_cols, nnz, static_cast<const int32_t*>(nullptr),
-                       static_cast<int32_t*>(col));
+    launch_csc2coo<int32_t, false>(indptr, num_cols, nnz, nullptr, static_cast<int32_t*>(col), st);
   return check_launch("csc2coo");
 }
 
@@ -594,13 +652,11 @@ int gs_dcsc2coo(const int64_t* indptr, int64_t num_cols, int64_t nnz, const void
   if (nnz == 0) return GS_OK;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (id_bytes == 8)
-    hipLaunchKernelGGL((csc2coo_kernel<int64_t>), dim3(blocks_for(nnz, kCooTile)), dim3(kThreads), 0,
-                       st, indptr, num_cols, nnz, static_cast<const int64_t*>(ids),
-                       static_cast<int64_t*>(col));
+    launch_csc2coo<int64_t, true>(indptr, num_cols, nnz, static_cast<const int64_t*>(ids),
+                              static_cast<int64_t*>(col), st);
   else
-    hipLaunchKernelGGL((csc2coo_kernel<int32_t>), dim3(blocks_for(nnz, kCooTile)), dim3(kThreads), 0,
-                       st, indptr, num_cols, nnz, static_cast<const int32_t*>(ids),
-                       static_cast<int32_t*>(col));
+    launch_csc2coo<int32_t, true>(indptr, num_cols, nnz, static_cast<const int32_t*>(ids),
+                              static_cast<int32_t*>(col), st);
   return check_launch("dcsc2coo");
 }
 

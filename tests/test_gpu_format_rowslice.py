@@ -31,6 +31,36 @@ def test_csc2coo_rmat(dev, seed, idt):
     assert np.array_equal(col, O.csc2coo(indptr, indices.size))
 
 
+@pytest.mark.parametrize("idt", ID_DTYPES)
+def test_csc2coo_runs_of_tiles_with_hubs_and_empty_columns(dev, idt):
+    """From 2 x 4096 x 2048 edges on a workgroup walks through several 4096-edge tiles: hubs that
+    cover many tiles, runs of more than 256 empty columns (several reads of the offsets for one
+    tile), columns that start exactly on tile and span boundaries, empty columns at both ends."""
+    rng = np.random.default_rng(3)
+    deg = rng.integers(0, 60, size=700_000).astype(np.int64)
+    deg[rng.integers(0, deg.size, size=40)] = rng.integers(20_000, 400_000, size=40)
+    for at in rng.integers(0, deg.size - 2000, size=30):
+        deg[at:at + rng.integers(257, 1500)] = 0
+    deg[:300] = 0
+    deg[-700:] = 0
+    # make some columns start exactly on multiples of 4096 and of 3 x 4096
+    ptr = np.concatenate([[0], np.cumsum(deg)])
+    for c in rng.integers(1000, deg.size - 1000, size=200):
+        pad = (-ptr[c]) % (4096 * (3 if c % 2 else 1))
+        deg[c - 1] += pad
+        ptr = np.concatenate([[0], np.cumsum(deg)])
+    nnz = int(ptr[-1])
+    assert nnz >= 3 * 4096 * 2048
+    col = capi.csc2coo(to_dev(ptr, dev), nnz, idt)
+    want = torch.repeat_interleave(torch.arange(deg.size, device=dev), to_dev(deg, dev))
+    assert col.dtype == idt and torch.equal(col.long(), want)
+    # the doubly-compressed form of the same: only the columns with edges are stored
+    kept = np.flatnonzero(deg)
+    d_ptr = np.concatenate([[0], np.cumsum(deg[kept])])
+    d_col = capi.dcsc2coo(to_dev(d_ptr, dev), nnz, to_dev(kept, dev, idt))
+    assert torch.equal(d_col.long(), want)
+
+
 def test_coo2csc_reference_eids(dev):
     # reference tests/test_format_transform.cc:54-74: CSC -> CSR of the 12-column graph
     indptr, indices = graph_12col_4edge()
