@@ -222,18 +222,51 @@ __global__ void __launch_bounds__(kThreads) sddmm_scalar_csc_kernel(SddmmArgs<Id
   __syncthreads();
   const bool need_src = (OP != GS_OP_COPY_RHS && a.lhs_target == 0) ||
                         (OP != GS_OP_COPY_LHS && a.rhs_target == 0);
+  // In three sweeps over the thread's sixteen edges -- where the operands are, the operands,
+  // the results -- so that the reads of one edge do not wait for the store of the one before
+  // (the output may overlap an operand: a read cannot be moved ahead of a store by itself).
+  // The optional id maps are read without a branch (a branch before a read makes the read
+  // wait for all before it): an absent map is read at a stride of zero from the offsets,
+  // which are always there, and the value is then not used.
+  const IdT* nid_from = a.nid_map ? a.nid_map : reinterpret_cast<const IdT*>(a.indptr);
+  const int64_t* eid_from = a.e_ids ? a.e_ids : a.indptr;
+  const IdT* src_from = need_src ? a.row : reinterpret_cast<const IdT*>(a.indptr);
+  const int64_t nid_step = a.nid_map ? 1 : 0, eid_step = a.e_ids ? 1 : 0, src_step = need_src ? 1 : 0;
+  constexpr int kHalf = kScalarItems / 2;  // (eight edges at a time keep the registers few)
+#pragma unroll 1
+  for (int k0 = 0; k0 < kScalarItems; k0 += kHalf) {
+    int64_t at_l[kHalf], at_r[kHalf], at_o[kHalf];
+    IdT nid_v[kHalf], src_v[kHalf];
 #pragma unroll
-  for (int k = 0; k < kScalarItems; ++k) {
-    const int i = k * kThreads + threadIdx.x;
-    const int64_t e = p0 + i;
-    if (e >= p1) continue;
-    const int64_t c = row_lo + s_mark[i];
-    const int64_t dst = a.nid_map ? static_cast<int64_t>(a.nid_map[c]) : c;
-    const int64_t src = need_src ? static_cast<int64_t>(a.row[e]) : 0;
-    const int64_t eid = a.e_ids ? a.e_ids[e] : e;
-    const float* l = (OP == GS_OP_COPY_RHS) ? nullptr : a.lhs + select3(a.lhs_target, src, eid, dst);
-    const float* r = (OP == GS_OP_COPY_LHS) ? nullptr : a.rhs + select3(a.rhs_target, src, eid, dst);
-    a.out[eid] = apply_op<OP>(l, r, 1);
+    for (int k = 0; k < kHalf; ++k) {
+      const int i = (k0 + k) * kThreads + threadIdx.x;
+      const int64_t e = p0 + i < p1 ? p0 + i : p1 - 1;  // (past the end: the last edge again)
+      at_l[k] = row_lo + s_mark[e - p0];
+      nid_v[k] = nid_from[at_l[k] * nid_step];
+      src_v[k] = src_from[e * src_step];
+      at_o[k] = eid_from[e * eid_step];
+    }
+#pragma unroll
+    for (int k = 0; k < kHalf; ++k) {
+      const int i = (k0 + k) * kThreads + threadIdx.x;
+      const int64_t e = p0 + i < p1 ? p0 + i : p1 - 1;
+      const int64_t dst = a.nid_map ? static_cast<int64_t>(nid_v[k]) : at_l[k];
+      const int64_t src = static_cast<int64_t>(src_v[k]);
+      const int64_t eid = a.e_ids ? at_o[k] : e;
+      at_l[k] = select3(a.lhs_target, src, eid, dst);
+      at_r[k] = select3(a.rhs_target, src, eid, dst);
+      at_o[k] = eid;
+    }
+    float lv[kHalf], rv[kHalf];
+#pragma unroll
+    for (int k = 0; k < kHalf; ++k) {
+      lv[k] = (OP == GS_OP_COPY_RHS) ? 0.0f : a.lhs[at_l[k]];
+      rv[k] = (OP == GS_OP_COPY_LHS) ? 0.0f : a.rhs[at_r[k]];
+    }
+#pragma unroll
+    for (int k = 0; k < kHalf; ++k)
+      if (p0 + (k0 + k) * kThreads + threadIdx.x < p1)
+        a.out[at_o[k]] = apply_op<OP>(&lv[k], &rv[k], 1);
   }
 }
 
