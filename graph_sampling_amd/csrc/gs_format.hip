@@ -379,7 +379,6 @@ radix_pass_kernel(Src src, const IdT* __restrict__ val_in, int64_t E, int shift,
                   SortOutputs<IdT> last) {
   using T = SortTile<IdT>;
   __shared__ unsigned long long s_word[T::kSize];
-  __shared__ IdT s_val[T::kSize];
   __shared__ int64_t s_base[kRadix];     // where the tile's run of a digit starts in memory
   __shared__ int s_cnt[kWaves][kRadix];  // per wave: count, then count of the earlier waves
   __shared__ int s_start[kRadix];        // where the run of a digit starts in the tile
@@ -461,34 +460,43 @@ radix_pass_kernel(Src src, const IdT* __restrict__ val_in, int64_t E, int shift,
   for (int w = 0; w < wave; ++w) start += s_scan[w];
   s_start[threadIdx.x] = start;
   __syncthreads();
+  // (words first, then the values through the same LDS: half the footprint of staging both
+  // at once, and twice the workgroups per compute unit)
 #pragma unroll
   for (int r = 0; r < T::kRounds; ++r) {
-    if (wave_base + r * kWave + lane < E) {
-      const int d = digit_of(word[r], shift);
-      const int at = s_start[d] + s_cnt[wave][d] + place[r];
-      s_word[at] = word[r];
-      s_val[at] = val[r];
-    }
+    const int d = digit_of(word[r], shift);
+    place[r] += s_start[d] + s_cnt[wave][d];
+    if (wave_base + r * kWave + lane < E) s_word[place[r]] = word[r];
   }
   __syncthreads();
   const int n = static_cast<int>(E - base < T::kSize ? E - base : T::kSize);
+  int64_t dst[T::kPerThread];
 #pragma unroll
   for (int k = 0; k < T::kPerThread; ++k) {
     const int j = k * kThreads + threadIdx.x;
+    dst[k] = -1;
     if (j < n) {
       const unsigned long long w = s_word[j];
       const int d = digit_of(w, shift);
-      const int64_t dst = s_base[d] + (j - s_start[d]);
+      dst[k] = s_base[d] + (j - s_start[d]);
       if (LAST) {
-        last.value[dst] = s_val[j];
-        last.perm[dst] = static_cast<int64_t>(w & ((1ull << last.idx_bits) - 1ull));
-        if (last.key) last.key[dst] = static_cast<IdT>(w >> last.idx_bits);
+        last.perm[dst[k]] = static_cast<int64_t>(w & ((1ull << last.idx_bits) - 1ull));
+        if (last.key) last.key[dst[k]] = static_cast<IdT>(w >> last.idx_bits);
       } else {
-        out[dst] = w;
-        val_out[dst] = s_val[j];
+        out[dst[k]] = w;
       }
     }
   }
+  __syncthreads();
+  IdT* s_val = reinterpret_cast<IdT*>(s_word);
+#pragma unroll
+  for (int r = 0; r < T::kRounds; ++r)
+    if (wave_base + r * kWave + lane < E) s_val[place[r]] = val[r];
+  __syncthreads();
+  IdT* to = LAST ? last.value : val_out;
+#pragma unroll
+  for (int k = 0; k < T::kPerThread; ++k)
+    if (dst[k] >= 0) to[dst[k]] = s_val[k * kThreads + threadIdx.x];
 }
 
 int bits_for(int64_t n) {  // smallest b with 2^b >= n
