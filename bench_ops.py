@@ -243,7 +243,7 @@ def main():
     # row probabilities straight off a column slice's COO rows (atomic adds into 2.45M sums)
     out_p = torch.zeros(N, device=dev)
     run("coo_sum", "gs_coo_sum of w^2 over the rows of a 512-column slice's edges into 2.45M sums",
-        lambda: capi.coo_sum(indices[:2_000_000], None, weights[:2_000_000], 2, out_p),
+        lambda: capi.coo_sum_binned(indices[:2_000_000], None, weights[:2_000_000], 2, out_p),
         lambda o: (2_000_000 * (b + 4 + 8), 2_000_000, "edges"))
     coo_cols2m = capi.csc2coo(indptr, E, idt)[:2_000_000]
     out_c = torch.zeros(N, device=dev)

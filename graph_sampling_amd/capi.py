@@ -36,7 +36,8 @@ def lib():
                      "gs_index_search_workspace_bytes", "gs_relabel_table_bytes",
                      "gs_relabel_sampled_workspace_bytes", "gs_relabel_sampled_state_bytes",
                      "gs_segment_workspace_bytes", "gs_layer_workspace_bytes",
-                     "gs_layer_sample_state_bytes", "gs_layer_relabel_state_bytes"):
+                     "gs_layer_sample_state_bytes", "gs_layer_relabel_state_bytes",
+                     "gs_coo_sum_workspace_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
     return _lib
@@ -858,6 +859,21 @@ def coo_sum(target, e_ids, data, powk, out):
     _need(out, torch.float32, "out")
     _check(lib().gs_coo_sum(_ptr(target), idb, _ptr(e_ids), _ptr(data), _i64(target.numel()),
                             _i64(powk), _ptr(out), _stream(target.device)), "gs_coo_sum")
+
+
+def coo_sum_binned(target, e_ids, data, powk, out):
+    """`coo_sum` through the entry point that knows the number of targets (`out.numel()`) and
+    brings a workspace: large inputs are binned by target and added up without atomics."""
+    idb = _ids(target, "target")
+    _need(data, torch.float32, "data")
+    _need(out, torch.float32, "out")
+    L = lib()
+    ws = workspace(L.gs_coo_sum_workspace_bytes(_i64(target.numel()), _i64(out.numel())),
+                   target.device)
+    _check(L.gs_coo_sum_binned(_ptr(target), idb, _ptr(e_ids), _ptr(data), _i64(target.numel()),
+                               _i64(powk), _i64(out.numel()), _ptr(out), _ptr(ws),
+                               ctypes.c_size_t(ws.numel()), _stream(target.device)),
+           "gs_coo_sum_binned")
 
 
 def segment_normalize(indptr, e_ids, data, out):

@@ -206,6 +206,14 @@ __device__ __forceinline__ float ares_key(uint32_t x, float w) {
   return __fdiv_rn(log2_u24(x), w);
 }
 
+// x^powk of the edge-data reductions (graph_ops.cu:30)
+__device__ __forceinline__ float powk_f(float x, int powk) {
+  if (powk == 1) return x;
+  float p = x;
+  for (int i = 1; i < powk; ++i) p *= x;
+  return p;
+}
+
 // Order-preserving map float -> uint32 (larger float => larger uint).
 __device__ __forceinline__ uint32_t float_to_ordered(float f) {
   uint32_t b = __float_as_uint(f);

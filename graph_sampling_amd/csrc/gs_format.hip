@@ -629,6 +629,107 @@ int coo2csc_impl(const IdT* key, const IdT* value, int64_t E, int64_t num_keys, 
   return check_launch("coo2csc");
 }
 
+// ---------------------------------------------------- binned scatter-add ----
+// out[target[e]] += data[e]^powk without an atomic to memory: one partition pass of the sort
+// above brings the edges of every run of 2^bin_shift targets together (at most 256 runs),
+// and a workgroup then adds a run's edges up in LDS and writes its sums with plain stores.
+// Atomics to memory run at about ten per nanosecond on this part whatever the kernel does
+// around them; edges that mostly hit different targets paid that price one by one.
+constexpr int kBinThreads = 1024;
+// A run with many edges (the hubs' run of a skewed graph holds a third of them) is shared by
+// several workgroups, which then add their sums to memory with atomics: the additions to one
+// LDS word queue up, and 16 k edges a workgroup measured fastest (2 M edges over 2.45 M
+// targets: 0.32 ms with one workgroup a run, 0.14 at 64 k edges, 0.10 at 16 k or 8 k).
+constexpr int kBinParts = 64;             // workgroups that may share one run of targets
+constexpr int64_t kBinPartItems = 16384;  // edges a workgroup takes before a run is shared
+constexpr int kBinMaxShift = 15;         // 2^15 sums = 128 KB of LDS
+
+__global__ void __launch_bounds__(kBinThreads)
+bin_sum_kernel(const unsigned long long* __restrict__ words, const int32_t* __restrict__ vals,
+               const int64_t* __restrict__ offsets, int64_t num_blocks, int idx_bits,
+               int bin_shift, int powk, int64_t num_targets, float* __restrict__ out) {
+  extern __shared__ float s_sum[];
+  const int bin = blockIdx.x;
+  const int64_t lo = offsets[bin * num_blocks], hi = offsets[(bin + 1) * num_blocks];
+  const int64_t n = hi - lo;
+  int64_t parts = (n + kBinPartItems - 1) / kBinPartItems;
+  if (parts > kBinParts) parts = kBinParts;
+  if (static_cast<int64_t>(blockIdx.y) >= parts) return;
+  const int width = 1 << bin_shift;
+  for (int j = threadIdx.x; j < width; j += kBinThreads) s_sum[j] = 0.0f;
+  __syncthreads();
+  const int64_t per = (n + parts - 1) / parts;
+  const int64_t begin = lo + blockIdx.y * per;
+  const int64_t end = begin + per < hi ? begin + per : hi;
+  const int64_t first = static_cast<int64_t>(bin) << bin_shift;
+  for (int64_t i = begin + threadIdx.x; i < end; i += kBinThreads) {
+    const int64_t t = static_cast<int64_t>(words[i] >> idx_bits) - first;
+    // (a target beyond num_targets has no sum to go to: left out, as out has no room for it)
+    if (t >= 0 && t < width) atomicAdd(&s_sum[t], powk_f(__int_as_float(vals[i]), powk));
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < width; j += kBinThreads) {
+    const float x = s_sum[j];
+    if (x != 0.0f && first + j < num_targets) {
+      if (parts == 1)
+        out[first + j] += x;
+      else
+        unsafeAtomicAdd(out + first + j, x);
+    }
+  }
+}
+
+// whether the binned path takes the call: 4-byte ids (the value rides along in an id-sized
+// word), plain edge order, few enough targets for 256 runs of at most 2^15, enough edges
+// for five launches to pay
+inline bool bin_sum_applies(int id_bytes, const int64_t* e_ids, int64_t E, int64_t num_targets) {
+  return id_bytes == 4 && !e_ids && E >= (int64_t(1) << 17) && num_targets > 0 &&
+         num_targets <= (int64_t(kRadix) << kBinMaxShift) && E < (int64_t(1) << 31);
+}
+
+int bin_sum_impl(const int32_t* target, const float* data, int64_t E, int powk, int64_t num_targets,
+                 float* out, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  using T = SortTile<int32_t>;
+  const int64_t blocks = blocks_for(E, T::kSize);
+  const int64_t table = kRadix * blocks;
+  Carver ws(workspace, workspace_bytes);
+  unsigned long long* words = ws.take<unsigned long long>(E);
+  int32_t* vals = ws.take<int32_t>(E);
+  int64_t* counts = ws.take<int64_t>(table);
+  int64_t* offsets = ws.take<int64_t>(table + 1);
+  int64_t* tiles = ws.take<int64_t>(scan_num_tiles(table) + 1);
+  if (!ws.ok) {
+    set_error_text("gs_coo_sum_binned: workspace needs %zu bytes, 256-byte aligned",
+                   gs_coo_sum_workspace_bytes(E, num_targets));
+    return GS_ERR_WORKSPACE;
+  }
+  const int idx_bits = bits_for(E);
+  int bin_shift = bits_for(num_targets) - kRadixBits;
+  if (bin_shift < 0) bin_shift = 0;
+  const int shift = idx_bits + bin_shift;
+  const dim3 grid(static_cast<unsigned>(blocks));
+  FreshWords<int32_t> src{target, idx_bits};
+  hipLaunchKernelGGL((radix_hist_kernel<FreshWords<int32_t>, T::kSize>), grid, dim3(kThreads), 0, st,
+                     src, E, shift, blocks, counts);
+  LoadI64 f{counts};
+  GS_RETURN_IF_ERROR(exclusive_scan(f, table, offsets, tiles, st));
+  const SortOutputs<int32_t> none{nullptr, nullptr, nullptr, idx_bits};
+  launch_pass<int32_t>(src, false, false, grid, st, reinterpret_cast<const int32_t*>(data), E, shift,
+                       blocks, offsets, words, vals, none);
+  const int bins = static_cast<int>(((num_targets - 1) >> bin_shift) + 1);
+  static const hipError_t lds_allowed = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(bin_sum_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+      static_cast<int>(sizeof(float) << kBinMaxShift));
+  if (lds_allowed != hipSuccess) {
+    set_error_text("gs_coo_sum_binned: %s", hipGetErrorString(lds_allowed));
+    return GS_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(bin_sum_kernel, dim3(bins, kBinParts), dim3(kBinThreads),
+                     sizeof(float) << bin_shift, st, words, vals, offsets, blocks, idx_bits,
+                     bin_shift, powk, num_targets, out);
+  return check_launch("coo_sum_binned");
+}
+
 }  // namespace
 }  // namespace gs
 
@@ -742,6 +843,32 @@ int gs_indptr_split(const int64_t* indptr, const int64_t* offsets, int64_t num_b
   hipLaunchKernelGGL(indptr_split_kernel, dim3(blocks_for(total, kThreads)), dim3(kThreads), 0,
                      static_cast<hipStream_t>(stream), indptr, offsets, num_batches, total, out);
   return check_launch("indptr_split");
+}
+
+size_t gs_coo_sum_workspace_bytes(int64_t E, int64_t num_targets) {
+  if (E < 0) E = 0;
+  if (!bin_sum_applies(4, nullptr, E, num_targets)) return 256;
+  const int64_t blocks = blocks_for(E, SortTile<int32_t>::kSize);
+  const int64_t table = kRadix * blocks;
+  return padded(static_cast<size_t>(E) * 8) + padded(static_cast<size_t>(E) * 4) +
+         padded(static_cast<size_t>(table) * 8) + padded(static_cast<size_t>(table + 1) * 8) +
+         scan_workspace_bytes(table);
+}
+
+int gs_coo_sum_binned(const void* target, int id_bytes, const int64_t* e_ids, const float* data,
+                      int64_t E, int64_t powk, int64_t num_targets, float* out, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  GS_REQUIRE(E >= 0 && powk >= 1 && num_targets >= 0,
+             "gs_coo_sum_binned: negative size or powk < 1");
+  GS_REQUIRE(E == 0 || (target && data && out), "gs_coo_sum_binned: null pointer");
+  GS_REQUIRE(valid_id_bytes(id_bytes), "gs_coo_sum_binned: id_bytes must be 4 or 8, got %d",
+             id_bytes);
+  if (E == 0) return GS_OK;
+  if (!bin_sum_applies(id_bytes, e_ids, E, num_targets))
+    return gs_coo_sum(target, id_bytes, e_ids, data, E, powk, out, stream);
+  return bin_sum_impl(static_cast<const int32_t*>(target), data, E, static_cast<int>(powk),
+                      num_targets, out, workspace, workspace_bytes,
+                      static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

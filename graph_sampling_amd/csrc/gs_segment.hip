@@ -36,13 +36,6 @@ constexpr int64_t kChunk = 1024;   // edges per wave in the by-edge pass
 constexpr int kChunkList = 64;     // list slots per chunk: 1024 / 17 + 1 = 61 segments can start in one
 constexpr int kIncomingLane = kWave - 1;
 
-__device__ __forceinline__ float powk_f(float x, int powk) {
-  if (powk == 1) return x;  // graph_ops.cu:30
-  float p = x;
-  for (int i = 1; i < powk; ++i) p *= x;
-  return p;
-}
-
 // Per-chunk bookkeeping of the by-edge pass, all in the caller's workspace.
 struct Chunks {
   unsigned int* any_long;  // does any segment exceed kLaneMaxLen?

@@ -962,9 +962,11 @@ void CooSum(const torch::Tensor& target, const torch::optional<torch::Tensor>& e
   const int idb = IdBytes(target, "coo target");
   NeedF32(data, "data");
   NeedF32(out, "out");
-  Check(gs_coo_sum(target.data_ptr(), idb, OptI64(e_ids, "e_ids"), data.data_ptr<float>(),
-                   target.numel(), powk, out.data_ptr<float>(), Stream(target)),
-        "gs_coo_sum");
+  auto ws = Scratch(gs_coo_sum_workspace_bytes(target.numel(), out.numel()), target);
+  Check(gs_coo_sum_binned(target.data_ptr(), idb, OptI64(e_ids, "e_ids"), data.data_ptr<float>(),
+                          target.numel(), powk, out.numel(), out.data_ptr<float>(), ws.data_ptr(),
+                          ws.numel(), Stream(target)),
+        "gs_coo_sum_binned");
 }
 
 void SegmentNormalize(const torch::Tensor& indptr, const torch::optional<torch::Tensor>& e_ids,

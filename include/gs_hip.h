@@ -535,6 +535,19 @@ int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const void* n_id
 int gs_coo_sum(const void* target, int id_bytes, const int64_t* e_ids, const float* data, int64_t E,
                int64_t powk, float* out, void* stream);
 
+/* The same sums for callers that know how many targets there are (out has num_targets
+ * entries; a target beyond is left out) and bring a workspace: with 4-byte ids, no e_ids,
+ * at least 2^17 edges and at most 2^23 targets the edges are first brought together by runs
+ * of targets (one partition pass of the sort behind gs_coo2csc) and then added up in LDS, a
+ * run per workgroup, with no atomic to memory -- several times faster than gs_coo_sum when
+ * most edges hit different targets.  Any other call is passed on to gs_coo_sum.  The order of
+ * the additions is not fixed in either (impl::COOSumCUDA, src/cuda/graph_ops.cu:45-64, adds
+ * with atomics too). */
+size_t gs_coo_sum_workspace_bytes(int64_t E, int64_t num_targets);
+int gs_coo_sum_binned(const void* target, int id_bytes, const int64_t* e_ids, const float* data,
+                      int64_t E, int64_t powk, int64_t num_targets, float* out, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
 /* out[d] = data[d] / sum of its segment, d = e_ids ? e_ids[e] : e */
 int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const float* data,
                          int64_t num_segments, int64_t nnz, float* out, void* workspace,

@@ -213,6 +213,45 @@ def test_coo_sum_and_e_div_u_sum(dev, idt):
     np.testing.assert_allclose(osum.cpu().numpy(), ws, rtol=1e-4)
 
 
+@pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("targets,edges,skew", [
+    (2_450_000, 1 << 20, True),    # a LADIES row sum: many targets, hubs among them
+    (2_450_000, 1 << 20, False),
+    (1000, 1 << 18, False),        # fewer targets than runs: every run is one target
+    (1 << 23, 300_000, True),      # the widest runs (2^15 sums in LDS)
+    ((1 << 23) + 1, 300_000, False),  # one target too many for the runs: the plain kernel
+    (70_000, (1 << 17) - 1, False),   # one edge short of the binned path
+    (5, 1 << 19, False),           # one run shared by several workgroups
+])
+def test_coo_sum_binned(dev, idt, targets, edges, skew):
+    """The sums with a known number of targets: against float64 sums of the same products (the
+    order of the additions is not fixed, so a tolerance), on top of what `out` held, for sizes
+    on both sides of every switch between the binned and the plain kernel."""
+    rng = np.random.default_rng(edges + targets)
+    if skew:
+        t = (rng.random(edges) ** 6 * targets).astype(np.int64)  # most edges on a few low targets
+    else:
+        t = rng.integers(0, targets, size=edges)
+    t[:3] = [0, targets - 1, targets - 1]
+    data = (rng.random(edges, dtype=np.float32) + 0.25).astype(np.float32)
+    for powk in (1, 2):
+        before = rng.random(targets, dtype=np.float32)
+        out = to_dev(before, dev)
+        capi.coo_sum_binned(to_dev(t, dev, idt), None, to_dev(data, dev), powk, out)
+        want = before.astype(np.float64) + np.bincount(t, weights=data.astype(np.float64) ** powk,
+                                                       minlength=targets)
+        np.testing.assert_allclose(out.cpu().numpy(), want, rtol=2e-5)
+        # targets nobody hits keep exactly what they held
+        idle = np.bincount(t, minlength=targets) == 0
+        assert np.array_equal(out.cpu().numpy()[idle], before[idle])
+    # with an edge-id map the plain kernel takes the call, whatever the size
+    e_ids = rng.permutation(edges)
+    out = torch.zeros(targets, dtype=torch.float32, device=dev)
+    capi.coo_sum_binned(to_dev(t, dev, idt), to_dev(e_ids, dev), to_dev(data, dev), 1, out)
+    want = np.bincount(t, weights=data[e_ids].astype(np.float64), minlength=targets)
+    np.testing.assert_allclose(out.cpu().numpy(), want, rtol=2e-5)
+
+
 # ------------------------------------------------------------------ SDDMM
 def _sddmm_coo_gpu(dev, op, row, col, e_ids, lhs, rhs, lt, rt, idt=torch.int64):
     ls = lhs.shape if lhs.ndim > 1 else lhs.shape + (1,)
