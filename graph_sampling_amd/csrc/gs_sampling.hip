@@ -110,23 +110,35 @@ slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ in
     }
   }
   __syncthreads();
+  // where each of the thread's edges comes from, then all the reads, then all the stores: a
+  // read issued behind a store waits for it, and eight edges one after the other would wait
+  // eight times
+  int64_t row[kFillItems], q[kFillItems];
+#pragma unroll
+  for (int k = 0; k < kFillItems; ++k) {
+    int64_t p = p0 + k * kFillThreads + threadIdx.x;
+    if (p >= p1) p = p1 - 1;  // (past the end: the last edge again, read but not stored)
+    if (staged) {
+      int64_t i = upper_bound(s_ptr, nrows + 1, p) - 1;
+      row[k] = row_lo + i;
+      q[k] = s_in[i] + (p - s_ptr[i]);
+    } else {
+      row[k] = row_lo + upper_bound(sub_indptr + row_lo, nrows + 1, p) - 1;
+      int64_t c = cols ? static_cast<int64_t>(cols[row[k]]) : row[k];  // non-empty row => valid id
+      q[k] = indptr[c] + (p - sub_indptr[row[k]]);
+    }
+  }
+  IdT v[kFillItems];
+#pragma unroll
+  for (int k = 0; k < kFillItems; ++k) v[k] = indices[q[k]];
 #pragma unroll
   for (int k = 0; k < kFillItems; ++k) {
     const int64_t p = p0 + k * kFillThreads + threadIdx.x;
-    if (p >= p1) break;
-    int64_t row, q;
-    if (staged) {
-      int64_t i = upper_bound(s_ptr, nrows + 1, p) - 1;
-      row = row_lo + i;
-      q = s_in[i] + (p - s_ptr[i]);
-    } else {
-      row = row_lo + upper_bound(sub_indptr + row_lo, nrows + 1, p) - 1;
-      int64_t c = cols ? static_cast<int64_t>(cols[row]) : row;  // non-empty row => valid id
-      q = indptr[c] + (p - sub_indptr[row]);
+    if (p < p1) {
+      sub_indices[p] = v[k];
+      if (select_index) select_index[p] = q[k];
+      if (WITH_COO) coo_col[p] = static_cast<IdT>(row[k]);
     }
-    sub_indices[p] = indices[q];
-    if (select_index) select_index[p] = q;
-    if (WITH_COO) coo_col[p] = static_cast<IdT>(row);
   }
 }
 
