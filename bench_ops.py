@@ -240,9 +240,9 @@ def main():
     run("list_sample_uniform", "gs_list_sample_uniform: 512 of 2.45M rows without replacement",
         lambda: capi.list_sample_uniform(all_rows, 512, False, seed=3),
         lambda o: (512 * (b + 16), 512, "items"))
-    # row probabilities straight off a column slice's COO rows (atomic adds into 2.45M sums)
+    # row probabilities straight off a column slice's COO rows (binned by row, added up in LDS)
     out_p = torch.zeros(N, device=dev)
-    run("coo_sum", "gs_coo_sum of w^2 over the rows of a 512-column slice's edges into 2.45M sums",
+    run("coo_sum", "gs_coo_sum_binned of w^2 over the rows of a 512-column slice's edges into 2.45M sums",
         lambda: capi.coo_sum_binned(indices[:2_000_000], None, weights[:2_000_000], 2, out_p),
         lambda o: (2_000_000 * (b + 4 + 8), 2_000_000, "edges"))
     coo_cols2m = capi.csc2coo(indptr, E, idt)[:2_000_000]
