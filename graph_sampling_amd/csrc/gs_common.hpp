@@ -3,6 +3,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
+#include <utility>
 #include <stdint.h>
 
 #include "../../include/gs_hip.h"
@@ -312,6 +314,36 @@ constexpr int kScanTile = kScanThreads * kScanItems;
 inline int64_t scan_num_tiles(int64_t n) { return n <= 0 ? 1 : (n + kScanTile - 1) / kScanTile; }
 inline size_t scan_workspace_bytes(int64_t n) { return padded((scan_num_tiles(n) + 1) * 8); }
 
+// A scan functor is either `int64_t operator()(i)` or, when it chases a pointer, the pair
+// `where(i)` (first read: which entry) and `count(entry)` (second read: its value).  The pair
+// lets a thread issue the first reads of all its items, then all second reads, instead of
+// walking two dependent reads per item one item after the other; neither may carry a
+// condition of its own (a read that may or may not happen makes every later one wait for all
+// that is in flight), so indices past the end are clamped and their values dropped.
+template <typename F, typename = void>
+struct scan_two_phase : std::false_type {};
+template <typename F>
+struct scan_two_phase<F, std::void_t<decltype(std::declval<const F&>().where(int64_t(0)))>>
+    : std::true_type {};
+
+// v[k] = f(at(k)) for at(k) < n, else 0; n > 0
+template <typename F, int ITEMS, typename At>
+__device__ __forceinline__ void scan_load(const F& f, int64_t n, At at, int64_t (&v)[ITEMS]) {
+  if constexpr (scan_two_phase<F>::value) {
+    decltype(f.where(int64_t(0))) key[ITEMS];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) key[k] = f.where(at(k) < n ? at(k) : n - 1);
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) v[k] = f.count(key[k]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) v[k] = f(at(k) < n ? at(k) : n - 1);
+  }
+#pragma unroll
+  for (int k = 0; k < ITEMS; ++k)
+    if (at(k) >= n) v[k] = 0;
+}
+
 // Evaluates f once per item (f may chase pointers), parks the value in out[i]
 // for the apply pass and reduces the tile.
 template <typename F>
@@ -320,14 +352,15 @@ __global__ void __launch_bounds__(kScanThreads) scan_tile_sums_kernel(F f, int64
                                                                       int64_t* out) {
   __shared__ int64_t lds[kScanThreads / kWave + 1];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kScanTile;
+  auto at = [&](int k) { return base + k * kScanThreads + threadIdx.x; };
+  int64_t v[kScanItems];
   int64_t acc = 0;
+  if (n > 0) {
+    scan_load(f, n, at, v);
 #pragma unroll
-  for (int k = 0; k < kScanItems; ++k) {
-    int64_t i = base + k * kScanThreads + threadIdx.x;
-    if (i < n) {
-      const int64_t v = f(i);
-      out[i] = v;
-      acc += v;
+    for (int k = 0; k < kScanItems; ++k) {
+      if (at(k) < n) out[at(k)] = v[k];
+      acc += v[k];
     }
   }
   int64_t total;
@@ -374,14 +407,24 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(F f, int64_t n
   }
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kScanTile +
                        static_cast<int64_t>(threadIdx.x) * kScanItems;
+  auto at = [&](int k) { return base + k; };
   int64_t v[kScanItems];
   int64_t acc = 0;
 #pragma unroll
-  for (int k = 0; k < kScanItems; ++k) {
-    int64_t i = base + k;
-    v[k] = i < n ? (tiles ? out[i] : f(i)) : 0;
-    acc += v[k];
+  for (int k = 0; k < kScanItems; ++k) v[k] = 0;
+  if (n > 0) {
+    if (tiles) {  // the values were parked in out by the sums pass
+#pragma unroll
+      for (int k = 0; k < kScanItems; ++k) v[k] = out[at(k) < n ? at(k) : n - 1];
+#pragma unroll
+      for (int k = 0; k < kScanItems; ++k)
+        if (at(k) >= n) v[k] = 0;
+    } else {
+      scan_load(f, n, at, v);
+    }
   }
+#pragma unroll
+  for (int k = 0; k < kScanItems; ++k) acc += v[k];
   int64_t total;
   int64_t ex = block_exclusive_scan<kScanThreads>(acc, &total, lds);
   int64_t run = ex + tile_base;

@@ -40,16 +40,35 @@ __device__ __forceinline__ bool valid_col(int64_t c, int64_t num_cols) {
   return static_cast<uint64_t>(c) < static_cast<uint64_t>(num_cols);
 }
 
+// (Read without a branch: an absent id list is read at a stride of zero from the offsets,
+// an id outside the graph reads entry 0 twice, and the value is then not used.)
+template <typename IdT>
+struct ColIds {
+  const IdT* from;
+  int64_t step;
+  bool given;
+  __device__ __forceinline__ ColIds(const IdT* cols, const int64_t* indptr)
+      : from(cols ? cols : reinterpret_cast<const IdT*>(indptr)), step(cols ? 1 : 0), given(cols) {}
+  __device__ __forceinline__ int64_t operator()(int64_t r) const {
+    const IdT c = from[r * step];
+    return given ? static_cast<int64_t>(c) : r;
+  }
+};
+
+__device__ __forceinline__ int64_t degree_of(const int64_t* indptr, int64_t c, int64_t num_cols) {
+  const bool ok = valid_col(c, num_cols);
+  const int64_t lo = indptr[ok ? c : 0], hi = indptr[ok ? c + 1 : 0];
+  return ok ? hi - lo : 0;
+}
+
 template <typename IdT>
 struct ColDegree {
   const int64_t* indptr;
   const IdT* cols;  // nullptr: identity
   int64_t num_cols;
-  __device__ __forceinline__ int64_t operator()(int64_t r) const {
-    int64_t c = cols ? static_cast<int64_t>(cols[r]) : r;
-    if (!valid_col(c, num_cols)) return 0;
-    return indptr[c + 1] - indptr[c];
-  }
+  __device__ __forceinline__ int64_t where(int64_t r) const { return ColIds<IdT>(cols, indptr)(r); }
+  __device__ __forceinline__ int64_t count(int64_t c) const { return degree_of(indptr, c, num_cols); }
+  __device__ __forceinline__ int64_t operator()(int64_t r) const { return count(where(r)); }
 };
 
 template <typename IdT>
@@ -59,12 +78,13 @@ struct ColCount {
   int64_t num_cols;
   int64_t k;
   int replace;
-  __device__ __forceinline__ int64_t operator()(int64_t r) const {
-    int64_t c = cols ? static_cast<int64_t>(cols[r]) : r;
-    int64_t deg = valid_col(c, num_cols) ? indptr[c + 1] - indptr[c] : 0;
+  __device__ __forceinline__ int64_t where(int64_t r) const { return ColIds<IdT>(cols, indptr)(r); }
+  __device__ __forceinline__ int64_t count(int64_t c) const {
+    const int64_t deg = degree_of(indptr, c, num_cols);
     if (replace) return deg == 0 ? 0 : k;
     return deg < k ? deg : k;
   }
+  __device__ __forceinline__ int64_t operator()(int64_t r) const { return count(where(r)); }
 };
 
 // first index i in [0, n) with a[i] > v (n if none)

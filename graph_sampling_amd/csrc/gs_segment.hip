@@ -60,8 +60,10 @@ struct __attribute__((packed, aligned(4))) Four {
   float a, b, c, d;
 };
 
-// ---- by segment: the short ones.  NORMALIZE writes out[d] = data[d] / sum instead.
-template <bool NORMALIZE, typename IdT>
+// ---- by segment: the short ones.  NORMALIZE writes out[d] = data[d] / sum instead.  EMAP:
+// with an edge map (a compile-time switch: the two ways of reading hold different things in
+// registers, and one kernel for both would run both at the occupancy of the larger).
+template <bool NORMALIZE, bool EMAP, typename IdT>
 __global__ void __launch_bounds__(kThreads)
 short_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ emap,
                       const IdT* __restrict__ nmap, const float* __restrict__ data,
@@ -99,10 +101,13 @@ short_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restr
   // at most kLaneMaxLen edges: a fixed number of predicated reads, all in flight together,
   // added up in edge order.  Without an edge map the lane's edges lie side by side and are
   // read four at a time (a lane's reads are scattered from its neighbours' either way: every
-  // read instruction is a line access per lane, and this makes four of sixteen).
+  // read instruction is a line access per lane, and this makes four of sixteen).  With one,
+  // the map's entries are read in one sweep and the data in a second (clamped to the
+  // segment, so that no read carries a condition: sixteen dependent pairs, each behind a
+  // condition of its own, were sixteen round trips one after the other).
   float v[kLaneMaxLen];
   int64_t at[kLaneMaxLen];
-  if (!emap) {
+  if (!EMAP) {
 #pragma unroll
     for (int j = 0; j < kLaneMaxLen / 4; ++j) {
       const int64_t p = begin + 4 * j;
@@ -121,8 +126,18 @@ short_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restr
   } else {
 #pragma unroll
     for (int k = 0; k < kLaneMaxLen; ++k) {
-      at[k] = begin + k < end ? emap[begin + k] : -1;
-      v[k] = at[k] >= 0 ? data[at[k]] : 0.0f;
+      v[k] = 0.0f;
+      at[k] = -1;
+    }
+    if (len > 0) {
+      int64_t from[kLaneMaxLen];
+#pragma unroll
+      for (int k = 0; k < kLaneMaxLen; ++k) from[k] = emap[begin + k < end ? begin + k : end - 1];
+#pragma unroll
+      for (int k = 0; k < kLaneMaxLen; ++k) {
+        v[k] = data[from[k]];
+        if (begin + k < end) at[k] = from[k];
+      }
     }
   }
   float acc = 0.0f;
@@ -439,6 +454,62 @@ carry_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ nmap, i
   }
 }
 
+// The steps of a chunk in the divide pass.  AHEAD: a full chunk of plain, aligned data, whose
+// four reads were issued before the marks were made; that variant contains no read at all, so
+// its stores follow one another without waiting (in one body with the other variant every
+// step waited for the store of the step before: a read that may happen makes the compiler
+// wait for all that is in flight).
+template <bool AHEAD>
+__device__ __forceinline__ void divide_steps(const int* mark, const Owned& own, float own_sum,
+                                             const float4 (&early)[kChunk / kStep],
+                                             const int64_t* __restrict__ emap,
+                                             const float* __restrict__ data, int64_t begin,
+                                             int64_t end, int lane, float* __restrict__ out) {
+  int carried = 0;
+#pragma unroll
+  for (int t = 0; t < kChunk / kStep; ++t) {
+    const int64_t base = begin + t * kStep;
+    if (!AHEAD && base >= end) break;
+    const int at0 = static_cast<int>(base - begin) + lane * kLaneEdges;
+    const int64_t e0 = base + lane * kLaneEdges;
+    int m[kLaneEdges];
+    {
+      const int4 mm = *reinterpret_cast<const int4*>(mark + at0);
+      m[0] = mm.x; m[1] = mm.y; m[2] = mm.z; m[3] = mm.w;
+    }
+    if (!AHEAD) {
+#pragma unroll
+      for (int k = 0; k < kLaneEdges; ++k)
+        if (e0 + k >= end) m[k] = 0;
+    }
+    const LaneMarks lm = scan_lane_marks(m, at0);
+    const int incl = latest_inclusive(lm.last_packed, carried, lane);
+    int cur = lane_move<0x138, 0xf>(carried, incl);
+    carried = __builtin_amdgcn_readlane(incl, kWave - 1);
+    const float have[kLaneEdges] = {early[t].x, early[t].y, early[t].z, early[t].w};
+    float res[kLaneEdges];
+    bool mine[kLaneEdges];
+#pragma unroll
+    for (int k = 0; k < kLaneEdges; ++k) {
+      if (m[k]) cur = (at0 + k + 1) << 8 | m[k];
+      const int owner = owner_of_mark(cur);
+      const float total = __shfl(own_sum, owner >= 0 ? owner : 0, kWave);
+      const int64_t e = e0 + k;
+      mine[k] = (AHEAD || e < end) && owner >= 0;
+      res[k] = 0.0f;
+      if (AHEAD) res[k] = have[k] / total;
+      else if (mine[k]) res[k] = data[emap ? emap[e] : e] / total;
+    }
+    if (AHEAD && mine[0] && mine[1] && mine[2] && mine[3]) {
+      *reinterpret_cast<float4*>(out + e0) = make_float4(res[0], res[1], res[2], res[3]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < kLaneEdges; ++k)
+        if (mine[k]) out[!AHEAD && emap ? emap[e0 + k] : e0 + k] = res[k];
+    }
+  }
+}
+
 // out[d] = data[d] / sums[segment of e] for the edges of long segments
 __global__ void __launch_bounds__(kThreads)
 long_divide_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ emap,
@@ -456,69 +527,42 @@ long_divide_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict
   const Owned own = load_owned(indptr, ck, c, lane);
   if (__ballot(own.g >= 0) == 0ull) return;  // no long segment touches the chunk
   const float own_sum = own.g >= 0 ? sums[own.g] : 0.0f;
+  // a full chunk of plain data: all four steps' reads are issued together
+  const bool ahead = !emap && end - begin == kChunk &&
+                     ((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  float4 early[kChunk / kStep];
+#pragma unroll
+  for (int t = 0; t < kChunk / kStep; ++t) early[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
   // the whole chunk lies inside the incoming segment: one divisor, no marks
   if (__shfl(own.g >= 0 ? own.e : int64_t(0), kIncomingLane, kWave) >= end) {
     const float total = __shfl(own_sum, kIncomingLane, kWave);
+    if (ahead) {
+#pragma unroll
+      for (int t = 0; t < kChunk / kStep; ++t)
+        early[t] = *reinterpret_cast<const float4*>(data + begin + t * kStep + lane * kLaneEdges);
+#pragma unroll
+      for (int t = 0; t < kChunk / kStep; ++t)
+        *reinterpret_cast<float4*>(out + begin + t * kStep + lane * kLaneEdges) =
+            make_float4(early[t].x / total, early[t].y / total, early[t].z / total,
+                        early[t].w / total);
+      return;
+    }
     for (int64_t e = begin + lane; e < end; e += kWave) {
       const int64_t d = emap ? emap[e] : e;
       out[d] = data[d] / total;
     }
     return;
   }
-  // a full chunk of plain data: all four steps' reads are issued before the marks are made
-  const bool ahead = !emap && end - begin == kChunk &&
-                     ((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
-  float4 early[kChunk / kStep];
   if (ahead) {
 #pragma unroll
     for (int t = 0; t < kChunk / kStep; ++t)
       early[t] = *reinterpret_cast<const float4*>(data + begin + t * kStep + lane * kLaneEdges);
-  } else {
-#pragma unroll
-    for (int t = 0; t < kChunk / kStep; ++t) early[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
   }
   write_marks(mark, own, begin, end, lane);
-  int carried = 0;
-#pragma unroll
-  for (int t = 0; t < kChunk / kStep; ++t) {
-    const int64_t base = begin + t * kStep;
-    if (base >= end) break;
-    const int at0 = static_cast<int>(base - begin) + lane * kLaneEdges;
-    const int64_t e0 = base + lane * kLaneEdges;
-    int m[kLaneEdges];
-    {
-      const int4 mm = *reinterpret_cast<const int4*>(mark + at0);
-      m[0] = mm.x; m[1] = mm.y; m[2] = mm.z; m[3] = mm.w;
-    }
-#pragma unroll
-    for (int k = 0; k < kLaneEdges; ++k)
-      if (e0 + k >= end) m[k] = 0;
-    const LaneMarks lm = scan_lane_marks(m, at0);
-    const int incl = latest_inclusive(lm.last_packed, carried, lane);
-    int cur = lane_move<0x138, 0xf>(carried, incl);
-    carried = __builtin_amdgcn_readlane(incl, kWave - 1);
-    const float have[kLaneEdges] = {early[t].x, early[t].y, early[t].z, early[t].w};
-    float res[kLaneEdges];
-    bool mine[kLaneEdges];
-#pragma unroll
-    for (int k = 0; k < kLaneEdges; ++k) {
-      if (m[k]) cur = (at0 + k + 1) << 8 | m[k];
-      const int owner = owner_of_mark(cur);
-      const float total = __shfl(own_sum, owner >= 0 ? owner : 0, kWave);
-      const int64_t e = e0 + k;
-      mine[k] = e < end && owner >= 0;
-      res[k] = 0.0f;
-      if (ahead) res[k] = have[k] / total;
-      else if (mine[k]) res[k] = data[emap ? emap[e] : e] / total;
-    }
-    if (ahead && mine[0] && mine[1] && mine[2] && mine[3]) {
-      *reinterpret_cast<float4*>(out + e0) = make_float4(res[0], res[1], res[2], res[3]);
-    } else {
-#pragma unroll
-      for (int k = 0; k < kLaneEdges; ++k)
-        if (mine[k]) out[emap ? emap[e0 + k] : e0 + k] = res[k];
-    }
-  }
+  if (ahead)
+    divide_steps<true>(mark, own, own_sum, early, emap, data, begin, end, lane, out);
+  else
+    divide_steps<false>(mark, own, own_sum, early, emap, data, begin, end, lane, out);
 }
 
 inline int64_t num_chunks(int64_t nnz) { return nnz <= 0 ? 1 : (nnz + kChunk - 1) / kChunk; }
@@ -559,8 +603,12 @@ int segment_sum_impl(const int64_t* indptr, const int64_t* emap, const void* nma
   const int64_t chunks = num_chunks(nnz);
   hipLaunchKernelGGL(clear_chunks_kernel, dim3(blocks_for(chunks, kThreads)), dim3(kThreads), 0, st,
                      s.ck, chunks);
-  hipLaunchKernelGGL((short_segments_kernel<false, IdT>), dim3(blocks_for(num_seg, kThreads)),
-                     dim3(kThreads), 0, st, indptr, emap, nm, data, num_seg, nnz, powk, out, s.ck);
+  if (emap)
+    hipLaunchKernelGGL((short_segments_kernel<false, true, IdT>), dim3(blocks_for(num_seg, kThreads)),
+                       dim3(kThreads), 0, st, indptr, emap, nm, data, num_seg, nnz, powk, out, s.ck);
+  else
+    hipLaunchKernelGGL((short_segments_kernel<false, false, IdT>), dim3(blocks_for(num_seg, kThreads)),
+                       dim3(kThreads), 0, st, indptr, emap, nm, data, num_seg, nnz, powk, out, s.ck);
   if (nnz > kLaneMaxLen) {
     hipLaunchKernelGGL(long_segments_kernel<IdT>, dim3(blocks_for(chunks, kWaves)), dim3(kThreads),
                        0, st, indptr, emap, nm, data, num_seg, nnz, powk, out, s.ck);
@@ -727,8 +775,14 @@ int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const floa
   const int64_t chunks = num_chunks(nnz);
   hipLaunchKernelGGL(clear_chunks_kernel, dim3(blocks_for(chunks, kThreads)), dim3(kThreads), 0, st,
                      s.ck, chunks);
-  hipLaunchKernelGGL((short_segments_kernel<true, int64_t>), dim3(blocks_for(num_segments, kThreads)),
-                     dim3(kThreads), 0, st, indptr, e_ids, no_map, data, num_segments, nnz, 1, out, s.ck);
+  if (e_ids)
+    hipLaunchKernelGGL((short_segments_kernel<true, true, int64_t>),
+                       dim3(blocks_for(num_segments, kThreads)), dim3(kThreads), 0, st, indptr,
+                       e_ids, no_map, data, num_segments, nnz, 1, out, s.ck);
+  else
+    hipLaunchKernelGGL((short_segments_kernel<true, false, int64_t>),
+                       dim3(blocks_for(num_segments, kThreads)), dim3(kThreads), 0, st, indptr,
+                       e_ids, no_map, data, num_segments, nnz, 1, out, s.ck);
   if (nnz > kLaneMaxLen) {
     hipLaunchKernelGGL(long_segments_kernel<int64_t>, dim3(blocks_for(chunks, kWaves)),
                        dim3(kThreads), 0, st, indptr, e_ids, no_map, data, num_segments, nnz, 1,

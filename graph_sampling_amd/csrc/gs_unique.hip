@@ -594,9 +594,16 @@ __global__ void __launch_bounds__(kThreads) rank_linked_kernel(RankArgs<IdT> a) 
                        static_cast<int64_t>(threadIdx.x) * kCompactItems;
   // slot numbers go by the bound (the array is sized for it), so that they are on their way
   // together with the counts
+  // (read without a branch, the last entry again past the end: a read that may or may not
+  // happen makes every later one wait for all that is in flight)
   uint32_t at[kCompactItems];
 #pragma unroll
-  for (int k = 0; k < kCompactItems; ++k) at[k] = base + k < M_bound ? a.pos[base + k] : 0u;
+  for (int k = 0; k < kCompactItems; ++k) at[k] = 0u;
+  if (M_bound > 0) {
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k)
+      at[k] = a.pos[base + k < M_bound ? base + k : M_bound - 1];
+  }
   int64_t S, M;
   a.n.get(&S, &M);
   const int64_t live = (M + kCompactTile - 1) / kCompactTile;
@@ -614,8 +621,10 @@ __global__ void __launch_bounds__(kThreads) rank_linked_kernel(RankArgs<IdT> a) 
   GS_STAMP(1);  // slot numbers and counts are here
   unsigned long long w[kCompactItems];
 #pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) w[k] = a.t.slots[at[k] & a.t.mask];  // (any slot will do past M)
+#pragma unroll
   for (int k = 0; k < kCompactItems; ++k)
-    w[k] = base + k < M ? a.t.slots[at[k] & a.t.mask] : ~0ull;
+    if (base + k >= M) w[k] = ~0ull;
   bool first[kCompactItems];
   int64_t mine = 0;
 #pragma unroll
