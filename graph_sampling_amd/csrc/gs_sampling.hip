@@ -806,8 +806,8 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
   if (LINKED) {
     // the compare-and-swaps of a lane (its four outputs; the row's first lane also enters the
     // seed) go out together; what they found is looked at after
-    uint32_t p[4], seed_p = 0u;
-    unsigned long long prev[4], seed_prev = 0ull;
+    uint32_t p[4] = {0u, 0u, 0u, 0u}, seed_p = 0u;
+    unsigned long long prev[4] = {0ull, 0ull, 0ull, 0ull}, seed_prev = 0ull;
     bool seed_live = sub == 0 && my_row < S;
     if (seed_live) {
       if (sizeof(IdT) == 8 && (static_cast<unsigned long long>(c) >> 32) != 0ull) {
@@ -833,23 +833,56 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
         }
       }
     }
+    // What the five compare-and-swaps found is sorted out in rounds over all of them, not item
+    // by item: the items that have their slot store it (and lower the index there where
+    // theirs is smaller) one after the other with nothing to wait for in between; those that
+    // met another key probe the next slot, all together, and come round again.  Item by item,
+    // every item's store waited for the one before, because a loop that may issue another
+    // compare-and-swap stood between them.
+    long long key[5];
+    uint32_t item[5], at[5];
+    unsigned long long seen[5];
+    unsigned int open = 0u;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      if (q[u] >= 0) {
-        const uint32_t item = static_cast<uint32_t>(S + row_out + 4 * sub + u);
-        while (!a.table.landed(static_cast<long long>(v[u]), item, p[u], prev[u])) {
-          p[u] = (p[u] + 1) & a.table.mask;
-          prev[u] = a.table.probe(static_cast<long long>(v[u]), item, p[u]);
-        }
-        a.pos[item] = p[u];
-      }
+      key[u] = static_cast<long long>(v[u]);
+      item[u] = static_cast<uint32_t>(S + row_out + 4 * sub + u);
+      at[u] = p[u];
+      seen[u] = prev[u];
+      if (q[u] >= 0) open |= 1u << u;
     }
-    if (seed_live) {
-      while (!a.table.landed(c, static_cast<uint32_t>(my_row), seed_p, seed_prev)) {
-        seed_p = (seed_p + 1) & a.table.mask;
-        seed_prev = a.table.probe(c, static_cast<uint32_t>(my_row), seed_p);
+    key[4] = c;
+    item[4] = static_cast<uint32_t>(my_row);
+    at[4] = seed_p;
+    seen[4] = seed_prev;
+    if (seed_live) open |= 1u << 4;
+    while (open) {
+      // what every open probe found, before anything is stored: the first look waits for the
+      // compare-and-swaps, and nothing below reads memory until the next round's probes
+      unsigned int home = 0u, down = 0u;
+#pragma unroll
+      for (int u = 0; u < 5; ++u) {
+        if (open >> u & 1u) {
+          const unsigned int f = a.table.found(key[u], item[u], seen[u]);
+          home |= (f & 1u) << u;
+          down |= (f >> 1) << u;
+        }
       }
-      a.pos[my_row] = seed_p;
+#pragma unroll
+      for (int u = 0; u < 5; ++u) {
+        if (home >> u & 1u) {
+          if (down >> u & 1u) a.table.lower(key[u], item[u], at[u]);
+          a.pos[item[u]] = at[u];
+        }
+      }
+      open &= ~home;
+#pragma unroll
+      for (int u = 0; u < 5; ++u) {
+        if (open >> u & 1u) {
+          at[u] = (at[u] + 1) & a.table.mask;
+          seen[u] = a.table.probe(key[u], item[u], at[u]);
+        }
+      }
     }
   }
   if (REPLACE) {

@@ -58,6 +58,18 @@ struct PackedTable {
     if (static_cast<uint32_t>(prev) > i) atomicMin(&slots[p], hi | i);
     return true;
   }
+  // `landed` in two steps for callers that sort out several probes at once: what a probe found
+  // (no memory access: 0 = another key's slot, 1 = the key's slot, 3 = the key's slot and the
+  // index there is to be lowered), and the lowering itself.
+  __device__ __forceinline__ unsigned int found(long long key, uint32_t i,
+                                                unsigned long long prev) const {
+    if (prev == ~0ull) return 1u;
+    if (static_cast<uint32_t>(prev >> 32) != static_cast<uint32_t>(key)) return 0u;
+    return static_cast<uint32_t>(prev) > i ? 3u : 1u;
+  }
+  __device__ __forceinline__ void lower(long long key, uint32_t i, uint32_t p) const {
+    atomicMin(&slots[p], (static_cast<unsigned long long>(static_cast<uint32_t>(key)) << 32) | i);
+  }
   __device__ __forceinline__ uint32_t first_index(uint32_t p) const {
     return static_cast<uint32_t>(slots[p]);
   }
