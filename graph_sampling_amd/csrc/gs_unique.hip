@@ -678,6 +678,26 @@ __global__ void __launch_bounds__(kThreads) rank_linked_kernel(RankArgs<IdT> a) 
       st[k] = lb_load(&a.lb.status[f >> 11]);
     }
   }
+  // every rank first (the reads, and the waits for tiles that have not closed yet), then all
+  // the stores: a store between two items' reads would make the later read wait for it
+  int64_t rank[kCompactItems];
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) {
+    const int64_t i = base + k;
+    rank[k] = -1;
+    if (i >= S && i < M) {
+      const uint32_t f = static_cast<uint32_t>(w[k]);
+      if (f <= static_cast<uint32_t>(i)) {  // (anything else: the insert pass gave up on this id)
+        if ((f >> 11) == tile) {
+          rank[k] = tile_incl - s_back[f & (kCompactTile - 1)];
+        } else {
+          const int64_t incl = lookback_wait_inclusive(a.lb, st[k], f >> 11);
+          const unsigned long long b = back_wait(a.lb, a.back, bw[k], f >> 2);
+          rank[k] = incl - static_cast<int64_t>((b >> (kBackBits * (f & 3))) & kBackMask);
+        }
+      }
+    }
+  }
   {
     int64_t run = tile_excl + local;
 #pragma unroll
@@ -689,20 +709,7 @@ __global__ void __launch_bounds__(kThreads) rank_linked_kernel(RankArgs<IdT> a) 
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) {
     const int64_t i = base + k;
-    if (i >= S && i < M) {
-      const uint32_t f = static_cast<uint32_t>(w[k]);
-      int64_t rank = -1;
-      if (f <= static_cast<uint32_t>(i)) {  // (anything else: the insert pass gave up on this id)
-        if ((f >> 11) == tile) {
-          rank = tile_incl - s_back[f & (kCompactTile - 1)];
-        } else {
-          const int64_t incl = lookback_wait_inclusive(a.lb, st[k], f >> 11);
-          const unsigned long long b = back_wait(a.lb, a.back, bw[k], f >> 2);
-          rank = incl - static_cast<int64_t>((b >> (kBackBits * (f & 3))) & kBackMask);
-        }
-      }
-      a.out_ids[i - S] = static_cast<IdT>(rank);
-    }
+    if (i >= S && i < M) a.out_ids[i - S] = static_cast<IdT>(rank[k]);
   }
   if (a.offsets_copy) {
     const int64_t g = static_cast<int64_t>(tile) * kThreads + threadIdx.x;
