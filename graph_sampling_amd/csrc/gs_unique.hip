@@ -779,11 +779,14 @@ struct BatchItems {
     }
     return lo;
   }
-  __device__ __forceinline__ IdT get_in(int64_t b, int64_t i) const {
+  // (one read through a chosen address, not one of two reads: a read that may or may not
+  // happen makes every later one wait for all that is in flight)
+  __device__ __forceinline__ const IdT* where_in(int64_t b, int64_t i) const {
     const int64_t off = i - start(b);
     const int64_t n_seeds = seeds_ptr[b + 1] - seeds_ptr[b];
-    return off < n_seeds ? seeds[seeds_ptr[b] + off] : ids[ids_ptr[b] + off - n_seeds];
+    return off < n_seeds ? seeds + seeds_ptr[b] + off : ids + ids_ptr[b] + off - n_seeds;
   }
+  __device__ __forceinline__ IdT get_in(int64_t b, int64_t i) const { return *where_in(b, i); }
   // The batch offsets copied into LDS (when there are at most kStagedBatches batches), and
   // this object re-pointed at the copy: the searches and the offset reads that stand between
   // a lane and its key then cost no trip to memory.  Every thread of the workgroup calls it.
@@ -970,25 +973,39 @@ batch_compact_kernel(BatchItems<IdT> x, int64_t M, R t, uint32_t* __restrict__ p
   // The slots' words are read here once, eight trips in flight together: from now on pos[i]
   // is the index of the first occurrence of item i's key, and the lookups of the last pass
   // need no second trip to the table.
+  // All reads carry no condition of their own (the last item again past the end; a read that
+  // may or may not happen makes every later one wait for all that is in flight), and every
+  // read of the thread's eight items stands before its first store.
   uint32_t at[kCompactItems], fi[kCompactItems];
+  IdT key[kCompactItems];
 #pragma unroll
-  for (int k = 0; k < kCompactItems; ++k) at[k] = base + k < M ? pos[base + k] : 0u;
+  for (int k = 0; k < kCompactItems; ++k) at[k] = fi[k] = 0u;
+  if (M > 0) {
+    const IdT* from[kCompactItems];
 #pragma unroll
-  for (int k = 0; k < kCompactItems; ++k) fi[k] = base + k < M ? t.first_index(at[k]) : 0u;
+    for (int k = 0; k < kCompactItems; ++k) {
+      const int64_t i = base + k < M ? base + k : M - 1;
+      at[k] = pos[i];
+      from[k] = x.where_in(x.batch_of(i, lo, hi), i);
+    }
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) {
+      fi[k] = t.first_index(at[k]);
+      key[k] = *from[k];  // in flight while wave 0 walks back
+    }
+  }
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) {
     const int64_t i = base + k;
     first[k] = i < M && fi[k] == static_cast<uint32_t>(i);
     mine += first[k] ? 1 : 0;
-    if (i < M) pos[i] = fi[k];
   }
   int64_t tile_total;
   const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
   if (threadIdx.x == 0) lookback_publish_sum(lb, tile, tile_total);
-  IdT key[kCompactItems];  // in flight while wave 0 walks back
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k)
-    key[k] = first[k] ? x.get_in(x.batch_of(base + k, lo, hi), base + k) : IdT(0);
+    if (base + k < M) pos[base + k] = fi[k];
   if (threadIdx.x < kWave) {
     const int64_t before = lookback_exclusive_prefix(lb, tile, tile_total);
     if (threadIdx.x == 0) s_prefix = before;
