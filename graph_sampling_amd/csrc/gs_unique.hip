@@ -193,33 +193,45 @@ compact_kernel(Spans<IdT> x, int64_t M_bound, T t, const uint32_t* __restrict__ 
   int64_t mine = 0;
   // slot numbers, then the slots' words, then the stores: three batches, so that the eight
   // trips to the table are in flight together and none waits for a store before it
+  // (no read carries a condition of its own -- the last entry again past the end: a read that
+  // may or may not happen makes every later one wait for all that is in flight)
   uint32_t at[kCompactItems], fi[kCompactItems];
 #pragma unroll
-  for (int k = 0; k < kCompactItems; ++k) at[k] = base + k < M_bound ? pos[base + k] : 0u;
-  GS_STAMP(1);  // slot numbers (and the device-side length) are here
+  for (int k = 0; k < kCompactItems; ++k) at[k] = 0u;
+  if (M_bound > 0) {
 #pragma unroll
-  for (int k = 0; k < kCompactItems; ++k) {
-    // read under the host's bound, not the device-side length, so that the reads do not wait
-    // for it; a slot number beyond the length is whatever the workspace held: masked
-    fi[k] = base + k < M_bound ? t.first_index(at[k] & t.mask) : 0u;
+    for (int k = 0; k < kCompactItems; ++k) at[k] = pos[base + k < M_bound ? base + k : M_bound - 1];
   }
+  GS_STAMP(1);  // slot numbers (and the device-side length) are here
+  // read under the host's bound, not the device-side length, so that the reads do not wait
+  // for it; a slot number beyond the length is whatever the workspace held: masked
+#pragma unroll
+  for (int k = 0; k < kCompactItems; ++k) fi[k] = t.first_index(at[k] & t.mask);
 #pragma unroll
   for (int k = 0; k < kCompactItems; ++k) {
     const int64_t i = base + k;
     first[k] = i < M && fi[k] == static_cast<uint32_t>(i);
     mine += first[k] ? 1 : 0;
-    // kept for the passes after this one: they need no second trip to the table (and the
-    // last pass of gs_relabel_sampled must not read it any more: it empties it)
-    if (first_out && i < M) first_out[i] = fi[k];
+  }
+  // kept for the passes after this one: they need no second trip to the table (and the
+  // last pass of gs_relabel_sampled must not read it any more: it empties it)
+  if (first_out) {
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k)
+      if (base + k < M) first_out[base + k] = fi[k];
   }
   GS_STAMP(2);  // the slots' words are here
   int64_t tile_total;
   const int64_t local = block_exclusive_scan<kThreads>(mine, &tile_total, s_scan);
   if (threadIdx.x == 0) lookback_publish_sum(lb, tile, tile_total);
   GS_STAMP(3);  // flags scanned, tile sum published
-  IdT key[kCompactItems];  // in flight while wave 0 walks back
+  IdT key[kCompactItems];  // in flight while wave 0 walks back (every item's key, needed or not)
 #pragma unroll
-  for (int k = 0; k < kCompactItems; ++k) key[k] = first[k] ? x.get(base + k) : IdT(0);
+  for (int k = 0; k < kCompactItems; ++k) key[k] = IdT(0);
+  if (M > 0) {
+#pragma unroll
+    for (int k = 0; k < kCompactItems; ++k) key[k] = x.get(base + k < M ? base + k : M - 1);
+  }
   if (threadIdx.x < kWave) {
     const int64_t before = lookback_exclusive_prefix(lb, tile, tile_total);
     if (threadIdx.x == 0) s_prefix = before;
