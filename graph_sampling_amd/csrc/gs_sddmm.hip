@@ -276,6 +276,56 @@ void launch_scalar_csc(const SddmmArgs<IdT>& a, hipStream_t st) {
   hipLaunchKernelGGL((sddmm_scalar_csc_kernel<OP, IdT>), dim3(grid), dim3(kThreads), 0, st, a);
 }
 
+// Scalar operands where no column has to be found (a COO, or a CSC whose operands sit on the
+// edge and on its row): eight edges per thread, strided by the workgroup, in three sweeps --
+// the ends and the edge id, the operands, the results -- so that all reads of a sweep are in
+// flight together and no read stands behind a store (the general kernel walks an edge at a
+// time; one scalar per row over 124 M edges: 0.89 ms there).
+constexpr int kFlatItems = 8;
+constexpr int kFlatTile = kThreads * kFlatItems;
+
+template <int OP, typename IdT>
+__global__ void __launch_bounds__(kThreads) sddmm_scalar_flat_kernel(SddmmArgs<IdT> a) {
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kFlatTile + threadIdx.x;
+  const bool need_src = (OP != GS_OP_COPY_RHS && a.lhs_target == 0) ||
+                        (OP != GS_OP_COPY_LHS && a.rhs_target == 0);
+  const bool need_dst = (OP != GS_OP_COPY_RHS && a.lhs_target == 2) ||
+                        (OP != GS_OP_COPY_LHS && a.rhs_target == 2);
+  // an end nobody asks for is read at a stride of zero (the row ids are always there)
+  const IdT* dst_from = need_dst ? a.col : a.row;
+  const int64_t src_step = need_src ? 1 : 0, dst_step = need_dst ? 1 : 0;
+  int64_t e[kFlatItems], eid[kFlatItems];
+  IdT src[kFlatItems], dst[kFlatItems];
+#pragma unroll
+  for (int k = 0; k < kFlatItems; ++k) {
+    e[k] = base + static_cast<int64_t>(k) * kThreads;
+    if (e[k] >= a.E) e[k] = a.E - 1;  // (past the end: the last edge again, not stored)
+    src[k] = a.row[e[k] * src_step];
+    dst[k] = dst_from[e[k] * dst_step];
+    eid[k] = e[k];
+  }
+  if (a.e_ids) {
+#pragma unroll
+    for (int k = 0; k < kFlatItems; ++k) eid[k] = a.e_ids[e[k]];
+  }
+  float lv[kFlatItems], rv[kFlatItems];
+#pragma unroll
+  for (int k = 0; k < kFlatItems; ++k) {
+    const int64_t s = static_cast<int64_t>(src[k]), d = static_cast<int64_t>(dst[k]);
+    lv[k] = (OP == GS_OP_COPY_RHS) ? 0.0f : a.lhs[select3(a.lhs_target, s, eid[k], d)];
+    rv[k] = (OP == GS_OP_COPY_LHS) ? 0.0f : a.rhs[select3(a.rhs_target, s, eid[k], d)];
+  }
+#pragma unroll
+  for (int k = 0; k < kFlatItems; ++k)
+    if (base + static_cast<int64_t>(k) * kThreads < a.E) a.out[eid[k]] = apply_op<OP>(&lv[k], &rv[k], 1);
+}
+
+template <int OP, typename IdT>
+void launch_scalar_flat(const SddmmArgs<IdT>& a, hipStream_t st) {
+  const unsigned grid = static_cast<unsigned>((a.E + kFlatTile - 1) / kFlatTile);
+  hipLaunchKernelGGL((sddmm_scalar_flat_kernel<OP, IdT>), dim3(grid), dim3(kThreads), 0, st, a);
+}
+
 // dot, no broadcast, out_len == 1, R % 4 == 0 and 16-byte aligned rows.
 constexpr int kDotGroup = 16;
 constexpr int kDotEdges = 4;  // edges per 16-lane group
@@ -340,6 +390,16 @@ int sddmm_dispatch(int op, const SddmmArgs<IdT>& a, hipStream_t st) {
       case GS_OP_SUB: launch_scalar_csc<GS_OP_SUB, IdT>(a, st); return check_launch("sddmm");
       case GS_OP_MUL: launch_scalar_csc<GS_OP_MUL, IdT>(a, st); return check_launch("sddmm");
       case GS_OP_DIV: launch_scalar_csc<GS_OP_DIV, IdT>(a, st); return check_launch("sddmm");
+      default: break;  // the copies and a one-element dot go the general way
+    }
+  }
+  if ((!a.indptr || !to_dst) && a.row && (a.indptr || a.col) && a.out_len == 1 && a.R == 1 &&
+      a.lhs_len == 1 && a.rhs_len == 1 && !a.lhs_off && !a.rhs_off) {
+    switch (op) {
+      case GS_OP_ADD: launch_scalar_flat<GS_OP_ADD, IdT>(a, st); return check_launch("sddmm");
+      case GS_OP_SUB: launch_scalar_flat<GS_OP_SUB, IdT>(a, st); return check_launch("sddmm");
+      case GS_OP_MUL: launch_scalar_flat<GS_OP_MUL, IdT>(a, st); return check_launch("sddmm");
+      case GS_OP_DIV: launch_scalar_flat<GS_OP_DIV, IdT>(a, st); return check_launch("sddmm");
       default: break;  // the copies and a one-element dot go the general way
     }
   }
