@@ -717,7 +717,8 @@ int bin_sum_impl(const int32_t* target, const float* data, int64_t E, int powk, 
   launch_pass<int32_t>(src, false, false, grid, st, reinterpret_cast<const int32_t*>(data), E, shift,
                        blocks, offsets, words, vals, none);
   const int bins = static_cast<int>(((num_targets - 1) >> bin_shift) + 1);
-  static const hipError_t lds_allowed = hipFuncSetAttribute(
+  // (per call: the attribute belongs to the device the call runs on)
+  const hipError_t lds_allowed = hipFuncSetAttribute(
       reinterpret_cast<const void*>(bin_sum_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
       static_cast<int>(sizeof(float) << kBinMaxShift));
   if (lds_allowed != hipSuccess) {
