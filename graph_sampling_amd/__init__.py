@@ -56,10 +56,13 @@ def set_seed(seed):
 def _blocks_of(parts, num_layers):
     from .block import Block
     blocks = []
+    per = len(parts) // num_layers  # 3, or 4 when the graph has edge data (the samples' share)
     for l in range(num_layers):
-        frontier, indptr, indices = parts[3 * l:3 * l + 3]
-        blocks.insert(0, Block(frontier.numel(), indptr.numel() - 1, "csc", indptr, indices, frontier))
-    return parts[-3], blocks
+        frontier, indptr, indices = parts[per * l:per * l + 3]
+        data = parts[per * l + 3] if per == 4 else None
+        blocks.insert(0, Block(frontier.numel(), indptr.numel() - 1, "csc", indptr, indices, frontier,
+                               weights=data))
+    return parts[-per], blocks
 
 
 def sample_layers(matrix, seeds, fanouts, replace=False):

@@ -255,9 +255,12 @@ class Mailbox:
 
 
 def sample_uniform_fused(indptr, indices, column_ids, fanout, replace, seed=0, replay=None,
-                         replay_ptr=None, with_coo=False, mailbox=None):
+                         replay_ptr=None, with_coo=False, mailbox=None, edge_data=None,
+                         edge_ids=None):
     """gs_sample_uniform_fused: one launch.  Same return shape as sample_uniform; with a
-    Mailbox also returns the ticket to wait on as a fifth element."""
+    Mailbox also returns the ticket to wait on as a fifth element.  With edge_data (fp32, and
+    optionally the int64 edge-id map edge_ids) the call is gs_sample_uniform_fused_data and the
+    samples' edge data, at capacity, comes back as the last element."""
     _need(indptr, torch.int64, "indptr")
     idb = _ids(indices, "indices")
     dev = indptr.device
@@ -276,12 +279,28 @@ def sample_uniform_fused(indptr, indices, column_ids, fanout, replace, seed=0, r
     coo_col = torch.empty(cap, dtype=indices.dtype, device=dev) if with_coo else None
     state, epoch = fused_state(lib().gs_sample_fused_state_bytes(_i64(S)), dev)
     ticket = mailbox.ticket() if mailbox is not None else 0
+    box = mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0)
+    if edge_data is not None:
+        _need(edge_data, torch.float32, "edge_data")
+        if edge_ids is not None:
+            _need(edge_ids, torch.int64, "edge_ids")
+        data_out = torch.empty(cap, dtype=torch.float32, device=dev)
+        _check(lib().gs_sample_uniform_fused_data(
+            _ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(column_ids), idb, _i64(S),
+            _i64(fanout), int(bool(replace)), _u64(seed), _ptr(replay), _ptr(replay_ptr),
+            _ptr(sub_indptr), _ptr(sub_indices), _ptr(select_index), _ptr(coo_col), _i64(cap),
+            _ptr(edge_data), _ptr(edge_ids), _ptr(data_out),
+            _ptr(state), ctypes.c_size_t(state.numel()), ctypes.c_uint32(epoch),
+            box, _i64(ticket), _stream(dev)), "gs_sample_uniform_fused_data")
+        if mailbox is not None:
+            return sub_indptr, sub_indices, select_index, coo_col, ticket, data_out
+        return sub_indptr, sub_indices, select_index, coo_col, data_out
     _check(lib().gs_sample_uniform_fused(
         _ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(column_ids), idb, _i64(S),
         _i64(fanout), int(bool(replace)), _u64(seed), _ptr(replay), _ptr(replay_ptr),
         _ptr(sub_indptr), _ptr(sub_indices), _ptr(select_index), _ptr(coo_col), _i64(cap),
         _ptr(state), ctypes.c_size_t(state.numel()), ctypes.c_uint32(epoch),
-        mailbox.ptr() if mailbox is not None else ctypes.c_void_p(0), _i64(ticket), _stream(dev)),
+        box, _i64(ticket), _stream(dev)),
         "gs_sample_uniform_fused")
     if mailbox is not None:
         return sub_indptr, sub_indices, select_index, coo_col, ticket
@@ -368,7 +387,7 @@ def relabel_sampled(seed_keys, sub_indptr, sub_indices, table, mailbox=None, off
 class LayerBuffers:
     """What one layer of sample_layers owns: outputs at their bounds, device-side counts."""
 
-    def __init__(self, S_bound, fanout, id_dtype, device):
+    def __init__(self, S_bound, fanout, id_dtype, device, with_data=False):
         self.S_bound = int(S_bound)
         self.fanout = int(fanout)
         self.capacity = self.S_bound * self.fanout
@@ -378,6 +397,11 @@ class LayerBuffers:
         self.frontier = torch.empty(self.S_bound + self.capacity, dtype=id_dtype, device=device)
         self.offsets_copy = torch.empty(self.S_bound + 1, dtype=torch.int64, device=device)
         self.counts = torch.zeros(2, dtype=torch.int64, device=device)  # num_edges, num_unique
+        # only with edge data: positions of the samples in the graph's indices, and their data
+        self.select_index = self.data = None
+        if with_data:
+            self.select_index = torch.empty(self.capacity, dtype=torch.int64, device=device)
+            self.data = torch.empty(self.capacity, dtype=torch.float32, device=device)
         self.workspace = torch.empty(
             int(lib().gs_layer_workspace_bytes(_i64(self.S_bound), _i64(self.fanout))),
             dtype=torch.uint8, device=device)
@@ -390,11 +414,17 @@ class LayerBuffers:
 
 
 def sample_layers(indptr, indices, seeds, fanouts, replace=False, seed=0, mailbox=None,
-                  tables=None):
+                  tables=None, edge_data=None, edge_ids=None):
     """gs_layer_sample + gs_layer_relabel for every layer of a minibatch, queued back to back:
     layer l + 1 takes its column ids and their number from layer l's frontier and num_unique on
     the device.  Layer l draws with seed + l.  Returns (layers: list of LayerBuffers, ticket of
-    the last relabel or None); sizes are the device-side counts of each layer."""
+    the last relabel or None); sizes are the device-side counts of each layer.  With edge_data
+    (fp32; edge_ids: the optional int64 edge-id map) every layer also leaves the positions of
+    its samples (select_index) and their edge data (data), both at capacity."""
+    if edge_data is not None:
+        _need(edge_data, torch.float32, "edge_data")
+        if edge_ids is not None:
+            _need(edge_ids, torch.int64, "edge_ids")
     _need(indptr, torch.int64, "indptr")
     idb = _ids(indices, "indices")
     _ids(seeds, "seeds", like=indices)
@@ -403,7 +433,8 @@ def sample_layers(indptr, indices, seeds, fanouts, replace=False, seed=0, mailbo
     bounds = [seeds.numel()]
     for k in fanouts:
         bounds.append(bounds[-1] * (1 + int(k)))
-    layers = [LayerBuffers(bounds[l], k, indices.dtype, dev) for l, k in enumerate(fanouts)]
+    layers = [LayerBuffers(bounds[l], k, indices.dtype, dev, edge_data is not None)
+              for l, k in enumerate(fanouts)]
     if tables is None:
         tables = [RelabelTable(bounds[-1], torch.int32, dev) for _ in range(2)]
     state_bytes = max(max(L.gs_layer_sample_state_bytes(_i64(b.S_bound)),
@@ -419,6 +450,7 @@ def sample_layers(indptr, indices, seeds, fanouts, replace=False, seed=0, mailbo
             _ptr(indptr), _i64(indptr.numel() - 1), _ptr(indices), _ptr(cols), idb,
             _i64(b.S_bound), S_dev, _i64(b.fanout), int(bool(replace)), _u64(seed + l), null, null,
             _ptr(b.sub_indptr), _ptr(b.sub_indices), _i64(b.capacity), b.num_edges_ptr(),
+            _ptr(b.select_index), _ptr(edge_data), _ptr(edge_ids), _ptr(b.data),
             _ptr(table.buf), ctypes.c_size_t(table.buf.numel()), _ptr(b.workspace),
             ctypes.c_size_t(b.workspace.numel()), _ptr(state), ctypes.c_size_t(state.numel()),
             ctypes.c_uint32(epoch), null, _i64(0), _stream(dev)), "gs_layer_sample")

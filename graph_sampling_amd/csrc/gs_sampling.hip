@@ -632,6 +632,12 @@ struct FusedArgs {
   PackedTable table;
   uint32_t* pos;
   int64_t* num_edges;
+  // edge data that follows the samples (reference src/graph.cc:544-557): data_out[o] =
+  // edge_data[edge_ids ? edge_ids[q] : q] for the output o taken at position q of `indices`;
+  // data_out == nullptr: none
+  const float* edge_data;
+  const int64_t* edge_ids;
+  float* data_out;
 };
 
 // Enters `key` as item `item` (one compare-and-swap in the common case); the slot goes to pos.
@@ -781,6 +787,21 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
       }
     }
   }
+  // the edge data of the same four picks, asked for while the ids are on their way
+  float w[4] = {0.f, 0.f, 0.f, 0.f};
+  if (a.data_out && cnt > 0) {
+    int64_t at_data[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) at_data[u] = q[u];
+    if (a.edge_ids) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (q[u] >= 0) at_data[u] = a.edge_ids[q[u]];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (q[u] >= 0) w[u] = a.edge_data[at_data[u]];
+  }
   __syncthreads();
   const int64_t out0 = s_prefix;
   GS_STAMP(5);  // the tile's offset is known to every wave, the first gathers are back
@@ -801,6 +822,7 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
       a.sub_indices[o] = v[u];
       if (a.select_index) a.select_index[o] = q[u];
       if (a.coo_col) a.coo_col[o] = static_cast<IdT>(my_row);
+      if (a.data_out) a.data_out[o] = w[u];
     }
   }
   if (LINKED) {
@@ -906,6 +928,7 @@ __global__ void __launch_bounds__(THREADS) sample_group_kernel(FusedArgs<IdT> a)
           a.sub_indices[o] = got;
           if (a.select_index) a.select_index[o] = p;
           if (a.coo_col) a.coo_col[o] = static_cast<IdT>(my_row);
+          if (a.data_out) a.data_out[o] = a.edge_data[a.edge_ids ? a.edge_ids[p] : p];
           if (LINKED) linked_insert<IdT>(a.table, got, S + o, a.pos, a.lb.error);
         }
       }
@@ -1059,6 +1082,19 @@ __global__ void __launch_bounds__(kFusedThreads) sample_row_lane_kernel(FusedArg
         v[u] = indices[q[u]];
       }
     }
+    float w[kFusedBatch];
+    if (a.data_out) {
+      int64_t at_data[kFusedBatch];
+#pragma unroll
+      for (int u = 0; u < kFusedBatch; ++u) at_data[u] = q[u];
+      if (a.edge_ids) {
+#pragma unroll
+        for (int u = 0; u < kFusedBatch; ++u)
+          if (q[u] >= 0) at_data[u] = a.edge_ids[q[u]];
+      }
+#pragma unroll
+      for (int u = 0; u < kFusedBatch; ++u) w[u] = q[u] >= 0 ? a.edge_data[at_data[u]] : 0.f;
+    }
 #pragma unroll
     for (int u = 0; u < kFusedBatch; ++u) {
       const uint32_t e = base + u * kFusedThreads;
@@ -1066,6 +1102,7 @@ __global__ void __launch_bounds__(kFusedThreads) sample_row_lane_kernel(FusedArg
         a.sub_indices[out0 + e] = v[u];
         if (a.select_index) a.select_index[out0 + e] = q[u];
         if (a.coo_col) a.coo_col[out0 + e] = static_cast<IdT>(r[u]);
+        if (a.data_out) a.data_out[out0 + e] = w[u];
       }
     }
   }
@@ -1117,7 +1154,9 @@ int sample_fused_t(const int64_t* indptr, int64_t num_cols, const void* indices,
                    void* sub_indices, int64_t* select_index, void* coo_col, LookbackState lb,
                    gs_mailbox* box, int64_t ticket, hipStream_t st, bool linked = false,
                    const int64_t* S_dev = nullptr, PackedTable table = PackedTable(),
-                   uint32_t* pos = nullptr, int64_t* num_edges = nullptr) {
+                   uint32_t* pos = nullptr, int64_t* num_edges = nullptr,
+                   const float* edge_data = nullptr, const int64_t* edge_ids = nullptr,
+                   float* data_out = nullptr) {
   FusedArgs<IdT> a{indptr,
                    static_cast<const IdT*>(indices),
                    static_cast<const IdT*>(column_ids),
@@ -1137,7 +1176,10 @@ int sample_fused_t(const int64_t* indptr, int64_t num_cols, const void* indices,
                    S_dev,
                    table,
                    pos,
-                   num_edges};
+                   num_edges,
+                   edge_data,
+                   edge_ids,
+                   data_out};
   return sample_fused_launch<IdT>(a, replace != 0, linked, st);
 }
 
@@ -1325,6 +1367,23 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
                             int64_t* select_index, void* coo_col, int64_t capacity,
                             void* state, size_t state_bytes, uint32_t epoch,
                             gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream) {
+  return gs_sample_uniform_fused_data(indptr, num_cols, indices, column_ids, id_bytes, S, fanout,
+                                      replace, seed, replay, replay_ptr, sub_indptr, sub_indices,
+                                      select_index, coo_col, capacity, nullptr, nullptr, nullptr,
+                                      state, state_bytes, epoch, mailbox, mailbox_ticket, stream);
+}
+
+int gs_sample_uniform_fused_data(const int64_t* indptr, int64_t num_cols, const void* indices,
+                                 const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+                                 int replace, uint64_t seed, const uint32_t* replay,
+                                 const int64_t* replay_ptr, int64_t* sub_indptr,
+                                 void* sub_indices, int64_t* select_index, void* coo_col,
+                                 int64_t capacity, const float* edge_data,
+                                 const int64_t* edge_ids, float* data_out, void* state,
+                                 size_t state_bytes, uint32_t epoch, gs_mailbox* mailbox,
+                                 int64_t mailbox_ticket, void* stream) {
+  GS_REQUIRE(edge_data ? (data_out != nullptr || S * fanout == 0) : (!data_out && !edge_ids),
+             "gs_sample_uniform_fused_data: edge_data and data_out go together (edge_ids needs both)");
   GS_REQUIRE(indptr && sub_indptr && S >= 0 && fanout >= 0 && num_cols >= 0,
              "gs_sample_uniform_fused: null pointer or negative size");
   GS_REQUIRE(column_ids || S <= num_cols,
@@ -1365,10 +1424,14 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
   return id_bytes == 8
              ? sample_fused_t<int64_t>(indptr, num_cols, indices, column_ids, S, fanout, replace,
                                        seed, replay, replay_ptr, sub_indptr, sub_indices,
-                                       select_index, coo_col, lb, mailbox, mailbox_ticket, st)
+                                       select_index, coo_col, lb, mailbox, mailbox_ticket, st,
+                                       false, nullptr, PackedTable(), nullptr, nullptr, edge_data,
+                                       edge_ids, data_out)
              : sample_fused_t<int32_t>(indptr, num_cols, indices, column_ids, S, fanout, replace,
                                        seed, replay, replay_ptr, sub_indptr, sub_indices,
-                                       select_index, coo_col, lb, mailbox, mailbox_ticket, st);
+                                       select_index, coo_col, lb, mailbox, mailbox_ticket, st,
+                                       false, nullptr, PackedTable(), nullptr, nullptr, edge_data,
+                                       edge_ids, data_out);
 }
 
 size_t gs_layer_sample_state_bytes(int64_t S_bound) {
@@ -1379,9 +1442,13 @@ int gs_layer_sample(const int64_t* indptr, int64_t num_cols, const void* indices
                     const void* column_ids, int id_bytes, int64_t S_bound, const int64_t* S_dev,
                     int64_t fanout, int replace, uint64_t seed, const uint32_t* replay,
                     const int64_t* replay_ptr, int64_t* sub_indptr, void* sub_indices,
-                    int64_t capacity, int64_t* num_edges, void* table, size_t table_bytes,
-                    void* workspace, size_t workspace_bytes, void* state, size_t state_bytes,
-                    uint32_t epoch, gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream) {
+                    int64_t capacity, int64_t* num_edges, int64_t* select_index,
+                    const float* edge_data, const int64_t* edge_ids, float* data_out, void* table,
+                    size_t table_bytes, void* workspace, size_t workspace_bytes, void* state,
+                    size_t state_bytes, uint32_t epoch, gs_mailbox* mailbox,
+                    int64_t mailbox_ticket, void* stream) {
+  GS_REQUIRE(edge_data ? (data_out != nullptr || capacity == 0) : (!data_out && !edge_ids),
+             "gs_layer_sample: edge_data and data_out go together (edge_ids needs both)");
   GS_REQUIRE(indptr && sub_indptr && num_edges && table && workspace && state && S_bound >= 0 &&
                  fanout >= 0 && num_cols >= 0,
              "gs_layer_sample: null pointer or negative size");
@@ -1425,12 +1492,12 @@ int gs_layer_sample(const int64_t* indptr, int64_t num_cols, const void* indices
   return id_bytes == 8
              ? sample_fused_t<int64_t>(indptr, num_cols, indices, column_ids, S_bound, fanout,
                                        replace, seed, replay, replay_ptr, sub_indptr, sub_indices,
-                                       nullptr, nullptr, lb, mailbox, mailbox_ticket, st, true,
-                                       S_dev, t, pos, num_edges)
+                                       select_index, nullptr, lb, mailbox, mailbox_ticket, st, true,
+                                       S_dev, t, pos, num_edges, edge_data, edge_ids, data_out)
              : sample_fused_t<int32_t>(indptr, num_cols, indices, column_ids, S_bound, fanout,
                                        replace, seed, replay, replay_ptr, sub_indptr, sub_indices,
-                                       nullptr, nullptr, lb, mailbox, mailbox_ticket, st, true,
-                                       S_dev, t, pos, num_edges);
+                                       select_index, nullptr, lb, mailbox, mailbox_ticket, st, true,
+                                       S_dev, t, pos, num_edges, edge_data, edge_ids, data_out);
 }
 
 int gs_sample_uniform_fused_static(const int64_t* indptr, int64_t num_cols, const void* indices,

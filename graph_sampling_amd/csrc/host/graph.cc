@@ -402,6 +402,7 @@ void Graph::Settle() {
   csc->indices = p->indices.narrow(0, 0, nnz);
   csc_ = csc;
   num_edges_ = nnz;
+  if (p->data.defined()) data_ = p->data.narrow(0, 0, nnz);
 }
 
 c10::intrusive_ptr<Graph> Graph::ColumnwiseFusedSlicingAndSampling(torch::Tensor column_index,
@@ -411,12 +412,20 @@ c10::intrusive_ptr<Graph> Graph::ColumnwiseFusedSlicingAndSampling(torch::Tensor
   TORCH_CHECK(csc_ != nullptr, "fused slicing + sampling needs the CSC format");
   torch::Tensor col_ids = Pick(col_ids_, column_index);
   auto ret = Child(col_ids, row_ids_, col_ids.numel(), num_rows_);
-  // No edge data to carry over: nothing on the host needs the edge count yet, so the
-  // child is handed back while the sampler runs and settles when it is first used.
-  if (hip::DeferredSampling() && !data_.has_value() && !(fanout == 1 && replace) &&
+  // Nothing on the host needs the edge count yet, so the child is handed back while the
+  // sampler runs and settles when it is first used.  Edge data follows the samples inside the
+  // sampler's launch (the gathers of src/graph.cc:544-557) when the kernels can read it.
+  const bool data_fits = !data_.has_value() || hip::EdgeData::Fits(data_.value(), csc_->e_ids);
+  if (hip::DeferredSampling() && data_fits && !(fanout == 1 && replace) &&
       hip::OneLaunchApplies(column_index.numel(), fanout, replace)) {
-    ret->pending_ = hip::ColSamplingDeferred(csc_->indptr, csc_->indices, column_index, fanout,
-                                             replace, false, false);
+    if (data_.has_value()) {
+      const hip::EdgeData edge{data_.value(), csc_->e_ids};
+      ret->pending_ = hip::ColSamplingDeferred(csc_->indptr, csc_->indices, column_index, fanout,
+                                               replace, false, false, &edge);
+    } else {
+      ret->pending_ = hip::ColSamplingDeferred(csc_->indptr, csc_->indices, column_index, fanout,
+                                               replace, false, false);
+    }
     return ret;
   }
   std::shared_ptr<CSC> sampled;
@@ -433,13 +442,19 @@ std::shared_ptr<hip::PendingLayers> Graph::QueueLayers(const torch::Tensor& seed
                                                        bool replace) {
   Settle();
   TORCH_CHECK(csc_ != nullptr, "fused slicing + sampling needs the CSC format");
-  // a root graph: local ids are the global ones, and no edge data follows the samples
-  if (col_ids_.has_value() || row_ids_.has_value() || data_.has_value() ||
-      val_col_ids_.has_value() || !hip::DeferredSampling())
+  // a root graph: local ids are the global ones; edge data, when there is any, must be what
+  // the sampler kernels can carry over themselves
+  if (col_ids_.has_value() || row_ids_.has_value() || val_col_ids_.has_value() ||
+      !hip::DeferredSampling())
     return nullptr;
+  if (data_.has_value() && !hip::EdgeData::Fits(data_.value(), csc_->e_ids)) return nullptr;
   for (int64_t k : fanouts)
     if (k == 1 && replace) return nullptr;  // (one slot per column, -1 for an empty one)
   if (!hip::LayerChainApplies(seeds.numel(), fanouts, replace)) return nullptr;
+  if (data_.has_value()) {
+    const hip::EdgeData edge{data_.value(), csc_->e_ids};
+    return hip::SampleLayersQueued(csc_->indptr, csc_->indices, seeds, fanouts, replace, &edge);
+  }
   return hip::SampleLayersQueued(csc_->indptr, csc_->indices, seeds, fanouts, replace);
 }
 
@@ -447,13 +462,15 @@ std::vector<torch::Tensor> Graph::SampleLayersLoop(torch::Tensor seeds,
                                                    const std::vector<int64_t>& fanouts,
                                                    bool replace) {
   std::vector<torch::Tensor> out;
-  out.reserve(3 * fanouts.size());
+  out.reserve(4 * fanouts.size());
   for (int64_t k : fanouts) {
     auto sub = ColumnwiseFusedSlicingAndSampling(seeds, k, replace);
     auto r = sub->Relabel();
     out.push_back(std::get<0>(r));  // frontier: source ids of the block, seeds first
     out.push_back(std::get<3>(r));  // offsets over the destinations
     out.push_back(std::get<4>(r));  // source positions in the frontier
+    // the samples' edge data, in the order of the sampled edges (the sample has no edge-id map)
+    if (data_.has_value()) out.push_back(sub->GetData("default").value());
     seeds = std::get<0>(r);
   }
   return out;
@@ -741,6 +758,7 @@ Graph::Relabel() {
     csc->indices = p->indices.narrow(0, 0, nnz);
     csc_ = csc;
     num_edges_ = nnz;
+    if (p->data.defined()) data_ = p->data.narrow(0, 0, nnz);
     return {frontier, frontier.numel(), col_ids.numel(), indptr_copy, relabeled, csc_->e_ids, "csc"};
   }
   Settle();

@@ -61,7 +61,10 @@ class Graph : public torch::CustomClassHolder {
   }
   void SetCOOByTensor(torch::Tensor row, torch::Tensor col, torch::optional<torch::Tensor> e_ids,
                       bool row_sorted, bool col_sorted);
-  void SetData(torch::Tensor data) { data_ = data; }
+  void SetData(torch::Tensor data) {
+    Settle();
+    data_ = data;
+  }
   // ids of the stored columns / rows when the CSC / CSR is doubly compressed
   void SetValidCols(torch::Tensor val_cols) { val_col_ids_ = val_cols; }
   void SetValidRows(torch::Tensor val_rows) { val_row_ids_ = val_rows; }
@@ -116,16 +119,18 @@ class Graph : public torch::CustomClassHolder {
   // Every layer of a GraphSAGE-style minibatch in one call: what the loop of the reference's
   // examples (examples/graphsage/batching.py:125-138) does layer by layer with
   // ColumnwiseFusedSlicingAndSampling + Relabel, next seeds = frontier.  Returns the flat list
-  // [frontier, offsets, indices] x layers (elements 0, 3, 4 of Relabel()'s tuple); layer l
-  // draws with the l-th seed the calling thread hands out next, so the result equals the
-  // loop's.  On a graph without id maps or edge data all layers are queued with no host read
-  // in between and the sizes are collected once at the end.
+  // [frontier, offsets, indices] x layers (elements 0, 3, 4 of Relabel()'s tuple), and on a
+  // graph with edge data [frontier, offsets, indices, data] x layers, data being the sampled
+  // edges' share of it (what GetData("default") of the layer's sample gives); layer l draws
+  // with the l-th seed the calling thread hands out next, so the result equals the loop's.
+  // On a graph without id maps all layers are queued with no host read in between and the
+  // sizes are collected once at the end.
   std::vector<torch::Tensor> SampleLayers(torch::Tensor seeds, std::vector<int64_t> fanouts,
                                           bool replace);
   // SampleLayers where the whole minibatch can be queued on the device (a root graph without
-  // edge data or id maps, sizes the layer chain takes); otherwise nothing is sampled, no seed
-  // is consumed and the list is empty, so that a caller who needs edge data or edge ids for
-  // its blocks goes layer by layer itself.
+  // id maps, sizes the layer chain takes, edge data -- if any -- one fp32 value per edge);
+  // otherwise nothing is sampled, no seed is consumed and the list is empty, so that the
+  // caller goes layer by layer itself.
   std::vector<torch::Tensor> SampleLayersIfQueued(torch::Tensor seeds,
                                                   std::vector<int64_t> fanouts, bool replace);
   // The first half of SampleLayers when the whole minibatch can be queued (else nullptr, and

@@ -311,8 +311,11 @@ torch::Tensor Window(const torch::Tensor& base, size_t byte_offset, int64_t coun
   auto t = at::detail::make_tensor<c10::TensorImpl>(c10::Storage(base.storage()), base.key_set(),
                                                     meta);
   auto* impl = t.unsafeGetTensorImpl();
-  impl->set_storage_offset(
-      base.storage_offset() + static_cast<int64_t>(byte_offset / meta.itemsize()));
+  const size_t at_byte = static_cast<size_t>(base.storage_offset()) * base.element_size() + byte_offset;
+  TORCH_CHECK(at_byte % meta.itemsize() == 0, "Window: misaligned for the element type");
+  TORCH_CHECK(count >= 0 && byte_offset + static_cast<size_t>(count) * meta.itemsize() <= base.nbytes(),
+              "Window: ", count, " elements at byte ", byte_offset, " do not fit the buffer");
+  impl->set_storage_offset(static_cast<int64_t>(at_byte / meta.itemsize()));
   impl->set_sizes_contiguous({count});
   return t;
 }
@@ -347,11 +350,24 @@ bool OneLaunchApplies(int64_t S, int64_t fanout, bool replace) {
          (replace || fanout <= GS_FUSED_MAX_FANOUT);
 }
 
+bool EdgeData::Fits(const torch::Tensor& data, const torch::optional<torch::Tensor>& e_ids) {
+  if (!data.defined() || !data.is_cuda() || data.dim() != 1 || !data.is_contiguous() ||
+      data.scalar_type() != torch::kFloat32)
+    return false;
+  if (e_ids.has_value() && e_ids.value().defined()) {
+    const torch::Tensor& e = e_ids.value();
+    if (!e.is_cuda() || e.dim() != 1 || !e.is_contiguous() || e.scalar_type() != torch::kInt64)
+      return false;
+  }
+  return true;
+}
+
 // One launch, no host read: the total is posted to a mailbox and collected by Wait().
 std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
                                                    const torch::Tensor& indices,
                                                    const torch::Tensor& column_ids, int64_t fanout,
-                                                   bool replace, bool with_coo, bool with_select) {
+                                                   bool replace, bool with_coo, bool with_select,
+                                                   const EdgeData* edge) {
   NeedI64(indptr, "indptr");
   const int idb = IdBytes(indices, "indices");
   const bool fused = column_ids.defined();
@@ -367,12 +383,15 @@ std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
     const size_t o_idx = at.Add(static_cast<size_t>(cap) * idb);
     const size_t o_sel = with_select ? at.Add(static_cast<size_t>(cap) * 8) : 0;
     const size_t o_coo = with_coo ? at.Add(static_cast<size_t>(cap) * idb) : 0;
+    const size_t o_data = edge ? at.Add(static_cast<size_t>(cap) * 4) : 0;
     auto buf = Scratch(at.bytes, indptr);
     p->sub_indptr = Window(buf, o_ptr, p->S + 1, torch::kInt64);
     p->indices = Window(buf, o_idx, cap, indices.scalar_type());
     if (with_select) p->select_index = Window(buf, o_sel, cap, torch::kInt64);
     if (with_coo) p->coo_col = Window(buf, o_coo, cap, indices.scalar_type());
+    if (edge) p->data = Window(buf, o_data, cap, torch::kFloat32);
   }
+  if (edge) TORCH_CHECK(EdgeData::Fits(edge->data, edge->e_ids), "edge data the sampler cannot read");
   p->stream = Stream(indptr);
   p->device = indptr.device().index();
   FusedStateBuf& state = FusedState(gs_sample_fused_state_bytes(p->S), indptr, p->stream);
@@ -381,14 +400,16 @@ std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
   p->box = boxes.slot(p->ticket);
   p->box_owner = boxes.buf;
   p->state_owner = state.buf;
-  Check(gs_sample_uniform_fused(indptr.data_ptr<int64_t>(), indptr.numel() - 1, EdgeArray(indices, indptr),
-                                fused ? column_ids.data_ptr() : nullptr, idb, p->S, fanout,
-                                replace ? 1 : 0, NextSeed(), nullptr, nullptr,
-                                p->sub_indptr.data_ptr<int64_t>(), p->indices.data_ptr(),
-                                with_select ? p->select_index.data_ptr<int64_t>() : nullptr,
-                                with_coo ? p->coo_col.data_ptr() : nullptr, cap,
-                                state.buf.data_ptr(), state.buf.numel(), state.epoch,
-                                boxes.slot(p->ticket), p->ticket, p->stream),
+  Check(gs_sample_uniform_fused_data(
+            indptr.data_ptr<int64_t>(), indptr.numel() - 1, EdgeArray(indices, indptr),
+            fused ? column_ids.data_ptr() : nullptr, idb, p->S, fanout, replace ? 1 : 0, NextSeed(),
+            nullptr, nullptr, p->sub_indptr.data_ptr<int64_t>(), p->indices.data_ptr(),
+            with_select ? p->select_index.data_ptr<int64_t>() : nullptr,
+            with_coo ? p->coo_col.data_ptr() : nullptr, cap,
+            edge ? static_cast<const float*>(EdgeArray(edge->data, indptr)) : nullptr,
+            edge ? OptI64(edge->e_ids, "e_ids") : nullptr,
+            edge ? p->data.data_ptr<float>() : nullptr, state.buf.data_ptr(), state.buf.numel(),
+            state.epoch, boxes.slot(p->ticket), p->ticket, p->stream),
         "gs_sample_uniform_fused");
   return p;
 }
@@ -678,10 +699,13 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
                                                   const torch::Tensor& indices,
                                                   const torch::Tensor& seeds,
                                                   const std::vector<int64_t>& fanouts,
-                                                  bool replace) {
+                                                  bool replace, const EdgeData* edge) {
   NeedI64(indptr, "indptr");
   const int idb = IdBytes(indices, "indices");
   TORCH_CHECK(IdBytes(seeds, "seeds") == idb, "seeds and indices differ in dtype");
+  if (edge) TORCH_CHECK(EdgeData::Fits(edge->data, edge->e_ids), "edge data the sampler cannot read");
+  const float* edge_data = edge ? static_cast<const float*>(EdgeArray(edge->data, indptr)) : nullptr;
+  const int64_t* edge_ids = edge ? OptI64(edge->e_ids, "e_ids") : nullptr;
   const int64_t L = static_cast<int64_t>(fanouts.size());
   TORCH_CHECK(LayerChainApplies(seeds.numel(), fanouts, replace),
               "SampleLayersQueued: this minibatch has to go layer by layer");
@@ -699,7 +723,7 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
   // sampled ids before renaming, the items' table slots, the two counts).  The output tensors
   // are cut out of it after the last launch, while the device is already at work.
   std::vector<size_t> off_ids(L), off_ws(L), ws_bytes(L), off_counts(L), off_offsets(L),
-      off_renamed(L), off_frontier(L);
+      off_renamed(L), off_frontier(L), off_data(L);
   size_t bytes = 0, state_bytes = 0;
   for (int64_t l = 0; l < L; ++l) {
     const size_t cap = static_cast<size_t>(S[l] * fanouts[l]);
@@ -711,6 +735,8 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
     bytes += Pad256((static_cast<size_t>(S[l]) + cap) * idb);
     off_ids[l] = bytes;
     bytes += Pad256(cap * idb);
+    off_data[l] = bytes;
+    if (edge) bytes += Pad256(cap * 4);
     ws_bytes[l] = gs_layer_workspace_bytes(S[l], fanouts[l]);
     off_ws[l] = bytes;
     bytes += Pad256(ws_bytes[l]);
@@ -743,7 +769,8 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
     y.ticket_edges = boxes.next++;
     Check(gs_layer_sample(indptr.data_ptr<int64_t>(), indptr.numel() - 1, EdgeArray(indices, indptr), cols,
                           idb, S[l], S_dev, fanouts[l], replace ? 1 : 0, seed, nullptr, nullptr,
-                          offsets, base + off_ids[l], cap, counts, table,
+                          offsets, base + off_ids[l], cap, counts, nullptr, edge_data, edge_ids,
+                          edge ? reinterpret_cast<float*>(base + off_data[l]) : nullptr, table,
                           table_bytes, base + off_ws[l], ws_bytes[l], st1.buf.data_ptr(),
                           st1.buf.numel(), st1.epoch, boxes.slot(y.ticket_edges), y.ticket_edges,
                           p->stream),
@@ -775,7 +802,9 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
             p->stream),
         "gs_layer_table_sweep");
   p->id_type = indices.scalar_type();
+  p->with_data = edge != nullptr;
   for (int64_t l = 0; l < L; ++l) {
+    p->layers[l].off_data = off_data[l];
     p->layers[l].off_offsets = off_offsets[l];
     p->layers[l].off_renamed = off_renamed[l];
     p->layers[l].off_frontier = off_frontier[l];
@@ -786,7 +815,7 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
 std::vector<torch::Tensor> PendingLayers::Collect() {
   const gs_mailbox* boxes = static_cast<const gs_mailbox*>(ring);
   std::vector<torch::Tensor> out;
-  out.reserve(3 * layers.size());
+  out.reserve(4 * layers.size());
   int64_t S = num_seeds;
   int64_t worst = 0;
   std::vector<int64_t> E(layers.size()), U(layers.size());
@@ -818,6 +847,7 @@ std::vector<torch::Tensor> PendingLayers::Collect() {
     out.push_back(Window(scratch, layers[l].off_frontier, U[l], id_type));
     out.push_back(Window(scratch, layers[l].off_offsets, S + 1, c10::ScalarType::Long));
     out.push_back(Window(scratch, layers[l].off_renamed, E[l], id_type));
+    if (with_data) out.push_back(Window(scratch, layers[l].off_data, E[l], c10::ScalarType::Float));
     S = U[l];
   }
   return out;

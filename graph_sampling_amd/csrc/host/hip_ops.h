@@ -38,6 +38,16 @@ SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices
 SliceResult ColSampling(const torch::Tensor& indptr, const torch::Tensor& indices,
                         const torch::Tensor& column_ids, int64_t fanout, bool replace,
                         bool with_coo);
+// The edge data of a graph for a sampler to carry over to its samples in the same launch
+// (what the reference gathers afterwards, src/graph.cc:544-557): data[e_ids ? e_ids[q] : q]
+// for a sample taken at position q of the CSC's indices.
+struct EdgeData {
+  torch::Tensor data;                    // fp32, one value per edge id
+  torch::optional<torch::Tensor> e_ids;  // the CSC's edge-id map, when it has one
+  // whether the sampler kernels can read it: one contiguous fp32 value per edge on the device
+  static bool Fits(const torch::Tensor& data, const torch::optional<torch::Tensor>& e_ids);
+};
+
 // A one-launch sample whose total the host has not read yet.  The buffers have
 // the capacity S * fanout; Wait() collects the total from its mailbox (no stream
 // synchronisation), after which the caller narrows them.
@@ -46,6 +56,7 @@ struct PendingSample {
   torch::Tensor indices;       // capacity
   torch::Tensor select_index;  // capacity; undefined when not requested
   torch::Tensor coo_col;       // capacity; undefined when not requested
+  torch::Tensor data;          // capacity; the samples' edge data, undefined without any
   int64_t S = 0;
   int64_t ticket = 0;
   void* stream = nullptr;
@@ -68,7 +79,8 @@ bool OneLaunchApplies(int64_t S, int64_t fanout, bool replace);
 std::shared_ptr<PendingSample> ColSamplingDeferred(const torch::Tensor& indptr,
                                                    const torch::Tensor& indices,
                                                    const torch::Tensor& column_ids, int64_t fanout,
-                                                   bool replace, bool with_coo, bool with_select);
+                                                   bool replace, bool with_coo, bool with_select,
+                                                   const EdgeData* edge = nullptr);
 // {frontier, relabelled sampled ids, number of sampled ids, copy of the sampler's
 // offsets}: unique / relabel of (column ids, sampled ids) queued behind the sampler without
 // reading its total
@@ -82,7 +94,7 @@ std::tuple<torch::Tensor, torch::Tensor, int64_t, torch::Tensor> RelabelDeferred
 struct PendingLayers {
   struct Layer {
     // where the layer's outputs start in `scratch` (bytes); their lengths come with the counts
-    size_t off_frontier = 0, off_offsets = 0, off_renamed = 0;
+    size_t off_frontier = 0, off_offsets = 0, off_renamed = 0, off_data = 0;
     int64_t ticket_edges = 0, ticket_unique = 0;
   };
   std::vector<Layer> layers;
@@ -98,7 +110,9 @@ struct PendingLayers {
   int device = 0;
   int64_t num_seeds = 0;
   uint64_t first_seed = 0;  // layer l drew with first_seed + l
-  // {frontier, offsets over the layer's seeds, sampled ids renamed} per layer.  Throws
+  bool with_data = false;   // the graph has edge data: every layer also holds its samples' data
+  // {frontier, offsets over the layer's seeds, sampled ids renamed[, edge data of the samples
+  // when the graph has edge data]} per layer.  Throws
   // IdsTooWide when a 64-bit id does not fit the chain's one-word table slots (the caller
   // repeats the minibatch layer by layer), c10::Error when a tile gave up waiting.
   std::vector<torch::Tensor> Collect();
@@ -113,7 +127,7 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
                                                   const torch::Tensor& indices,
                                                   const torch::Tensor& seeds,
                                                   const std::vector<int64_t>& fanouts,
-                                                  bool replace);
+                                                  bool replace, const EdgeData* edge = nullptr);
 // For tests of the recovery path: raises the sticky error word in the look-back state of the
 // calling thread's current stream on `like`'s device, as a tile that gave up waiting would.
 // The next one-launch sampler or relabel on that state reports failure (every kernel still

@@ -116,18 +116,21 @@ def fuse_slicing_and_sampling(gm: fx.GraphModule) -> fx.GraphModule:
 def sample_layer_chain(graph, seeds, fanouts, replace):
     """[(tuple of `Graph::Relabel`, edge data)] per layer of a GraphSAGE-style minibatch, the
     values the per-layer calls `_CAPI_FusedColumnwiseSlicingSampling` -> `_CAPI_Relabel` /
-    `_CAPI_GetData('default')` give under the same seed.  A root graph without edge data takes
-    the whole minibatch in one call of the C++ layer; its blocks have no edge ids and ones as
-    edge data, as the per-layer calls find on a graph without data (src/graph.cc:68-73)."""
+    `_CAPI_GetData('default')` give under the same seed.  A root graph takes the whole
+    minibatch in one call of the C++ layer; its blocks have no edge ids, and as edge data the
+    sampled edges' share of the graph's, or ones on a graph without data, as the per-layer
+    calls find there (src/graph.cc:68-73)."""
     fanouts = list(fanouts)
     parts = graph._CAPI_SampleLayersIfQueued(seeds, fanouts, bool(replace))
     layers = []
     if parts:
         num_dst = seeds.numel()
+        per = len(parts) // len(fanouts)  # 4 with edge data
         for l in range(len(fanouts)):
-            frontier, indptr, indices = parts[3 * l:3 * l + 3]
-            ones = torch.ones(indices.numel(), dtype=torch.float32, device=indices.device)
-            layers.append(((frontier, frontier.numel(), num_dst, indptr, indices, None, "csc"), ones))
+            frontier, indptr, indices = parts[per * l:per * l + 3]
+            data = parts[per * l + 3] if per == 4 else torch.ones(
+                indices.numel(), dtype=torch.float32, device=indices.device)
+            layers.append(((frontier, frontier.numel(), num_dst, indptr, indices, None, "csc"), data))
             num_dst = frontier.numel()
         return layers
     for k in fanouts:

@@ -191,6 +191,23 @@ int gs_sample_uniform_fused(const int64_t* indptr, int64_t num_cols, const void*
                             void* state, size_t state_bytes, uint32_t epoch,
                             gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
 
+/* gs_sample_uniform_fused that also carries the graph's edge data over to the samples, in
+ * the same launch: data_out[o] = edge_data[edge_ids ? edge_ids[q] : q] for the output o taken
+ * at position q of `indices` (q is what select_index[o] receives).  Replaces the two torch
+ * `index` gathers Graph::ColumnwiseFusedSlicingAndSampling makes after the sampler
+ * (src/graph.cc:544-557: data_[e_ids[select_index]]).  edge_data: fp32, one value per edge id;
+ * edge_ids: NULL, or the CSC's edge-id map (int64, one per position of `indices`); data_out:
+ * `capacity` floats.  All three NULL: exactly gs_sample_uniform_fused. */
+int gs_sample_uniform_fused_data(const int64_t* indptr, int64_t num_cols, const void* indices,
+                                 const void* column_ids, int id_bytes, int64_t S, int64_t fanout,
+                                 int replace, uint64_t seed, const uint32_t* replay,
+                                 const int64_t* replay_ptr, int64_t* sub_indptr,
+                                 void* sub_indices, int64_t* select_index, void* coo_col,
+                                 int64_t capacity, const float* edge_data,
+                                 const int64_t* edge_ids, float* data_out, void* state,
+                                 size_t state_bytes, uint32_t epoch, gs_mailbox* mailbox,
+                                 int64_t mailbox_ticket, void* stream);
+
 /* gs_sample_uniform_fused for callers that cannot allocate (no counterpart in the
  * reference: it is for code under HIP graph capture, tight serving loops and harnesses
  * that forbid hipMalloc, which can bring outputs but no state buffer of the right age).
@@ -415,14 +432,21 @@ size_t gs_layer_relabel_state_bytes(int64_t S_bound, int64_t fanout);
 
 /* First launch: the one-launch sampler (see gs_sample_uniform_fused: same draws, same
  * outputs; sub_indices holds `capacity` >= S_bound * fanout entries) which also enters
- * every seed (item r = seed r) and every sampled id (item S + e = output e) into `table`. */
+ * every seed (item r = seed r) and every sampled id (item S + e = output e) into `table`.
+ * select_index (NULL, or `capacity` slots): position of every sample in `indices`.
+ * edge_data / edge_ids / data_out (all NULL, or as for gs_sample_uniform_fused_data): the
+ * edge data of the samples, data_[e_ids[select_index]] of src/graph.cc:544-557, written by
+ * the lane that holds the position; output e of the layer keeps its place through
+ * gs_layer_relabel, so data_out[e] belongs to out_ids[e]. */
 int gs_layer_sample(const int64_t* indptr, int64_t num_cols, const void* indices,
                     const void* column_ids, int id_bytes, int64_t S_bound, const int64_t* S_dev,
                     int64_t fanout, int replace, uint64_t seed, const uint32_t* replay,
                     const int64_t* replay_ptr, int64_t* sub_indptr, void* sub_indices,
-                    int64_t capacity, int64_t* num_edges, void* table, size_t table_bytes,
-                    void* workspace, size_t workspace_bytes, void* state, size_t state_bytes,
-                    uint32_t epoch, gs_mailbox* mailbox, int64_t mailbox_ticket, void* stream);
+                    int64_t capacity, int64_t* num_edges, int64_t* select_index,
+                    const float* edge_data, const int64_t* edge_ids, float* data_out, void* table,
+                    size_t table_bytes, void* workspace, size_t workspace_bytes, void* state,
+                    size_t state_bytes, uint32_t epoch, gs_mailbox* mailbox,
+                    int64_t mailbox_ticket, void* stream);
 
 /* Second launch: frontier (capacity S_bound + capacity; distinct ids of (seeds, sampled ids)
  * in first-occurrence order), *num_unique (device; -1 / -2 as gs_relabel_sampled_narrow),

@@ -87,6 +87,30 @@ def test_fused_very_many_columns_take_the_row_per_lane_kernel(dev, idt, k, repla
     _cmp(got, O.sample_uniform(indptr, indices, cols, k, replace, seed=S + k))
 
 
+@pytest.mark.parametrize("with_edge_ids", [False, True])
+@pytest.mark.parametrize("S,k,replace", [(3000, 15, False), (3000, 4, True), (3000, 70, True),
+                                         ((1 << 18) + 77, 7, False), ((1 << 18) + 5, 3, True),
+                                         (0, 5, False)])
+def test_fused_carries_edge_data(dev, S, k, replace, with_edge_ids):
+    """gs_sample_uniform_fused_data: the same samples as gs_sample_uniform_fused plus
+    data[e_ids[select_index]] (reference src/graph.cc:544-557), by both kernels of the launch
+    (G lanes per row; one row per lane from 2^18 columns on)."""
+    indptr, indices = rmat_csc_np(1 << 13, 1 << 17, seed=6)
+    rng = np.random.default_rng(S + k)
+    cols = rng.integers(0, 1 << 13, size=S).astype(np.int64)
+    data = (1.0 - rng.random(indices.size)).astype(np.float32)
+    e_ids = rng.permutation(indices.size).astype(np.int64) if with_edge_ids else None
+    d = (to_dev(indptr, dev), to_dev(indices, dev, torch.int32), to_dev(cols, dev, torch.int32))
+    res = capi.sample_uniform_fused(*d, k, replace, seed=S + k, with_coo=True,
+                                    edge_data=to_dev(data, dev),
+                                    edge_ids=None if e_ids is None else to_dev(e_ids, dev))
+    want = O.sample_uniform(indptr, indices, cols, k, replace, seed=S + k)
+    _cmp(_narrow(res), want)
+    sel = want[3]
+    picked = data[sel] if e_ids is None else data[e_ids[sel]]
+    assert np.array_equal(res[-1][:sel.size].cpu().numpy(), picked)
+
+
 def test_fused_equals_two_phase_at_benchmark_shape(dev):
     """Layer-3-like shape: 45k seed columns, fanout 5; the two entry points agree bit for bit."""
     indptr, indices = rmat_csc_np(1 << 16, 1 << 21, seed=4)

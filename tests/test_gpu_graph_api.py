@@ -943,6 +943,89 @@ def test_sample_layers_equals_the_layer_loop_and_the_oracle(dev, idt, fanouts, r
 
 
 @pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+@pytest.mark.parametrize("from_coo", [False, True])
+@pytest.mark.parametrize("fanouts,replace", [((15, 10, 5), False), ((4, 4), True), ((40, 3), False)])
+def test_sample_layers_on_a_graph_with_edge_data(dev, idt, from_coo, fanouts, replace):
+    """A graph with fp32 edge data (BASELINE configurations 3 and 5 carry weights): the whole
+    minibatch still goes in one call, every layer hands back the sampled edges' share of the data
+    (`data_[e_ids[select_index]]`, reference src/graph.cc:544-557), and the result equals the
+    per-layer calls and the oracle.  Loaded as an unsorted COO the CSC has an edge-id map, and
+    the data stays in COO order."""
+    n = 1 << 12
+    indptr, indices = rmat_csc_np(n, 1 << 17, seed=31)
+    rng = np.random.default_rng(9)
+    g = gs.Graph(False)
+    if from_coo:
+        col = np.repeat(np.arange(n, dtype=np.int64), np.diff(indptr))
+        perm = rng.permutation(indices.size)
+        g._CAPI_LoadCOO(to_dev(indices[perm], dev, idt), to_dev(col[perm], dev, idt))
+        g._CAPI_SetMetadata(None, None, n, n)
+        g._CAPI_CreateSparseFormat(_CSC)
+        t_ptr, t_idx, t_eid = g._CAPI_GetCSC()
+        indptr = t_ptr.cpu().numpy()
+        indices = t_idx.cpu().numpy().astype(np.int64)
+        e_ids = t_eid.cpu().numpy()
+        assert not np.array_equal(e_ids, np.arange(e_ids.size))
+    else:
+        g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev, idt))
+        e_ids = None
+    data = (1.0 - rng.random(indices.size)).astype(np.float32)
+    g._CAPI_SetData(to_dev(data, dev))
+    seeds = rng.permutation(n)[:600].astype(np.int64)
+    t_seeds = to_dev(seeds, dev, idt)
+    for first in (410, 420):
+        gs.set_seed(first)
+        got = g._CAPI_SampleLayers(t_seeds, list(fanouts), replace)
+        assert len(got) == 4 * len(fanouts)
+        _same([t for i, t in enumerate(got) if i % 4 != 3],
+              _oracle_minibatch(indptr, indices, seeds, fanouts, replace, first))
+        cols = seeds
+        for l, k in enumerate(fanouts):
+            sel = O.sample_uniform(indptr, indices, cols, k, replace, seed=first + l,
+                                   with_coo=False)[3]
+            picked = data[sel] if e_ids is None else data[e_ids[sel]]
+            assert np.array_equal(got[4 * l + 3].cpu().numpy(), picked)
+            cols = got[4 * l].cpu().numpy().astype(np.int64)
+        gs.set_seed(first)
+        cols, loop = t_seeds, []
+        for k in fanouts:
+            sub = g._CAPI_FusedColumnwiseSlicingSampling(cols, k, replace)
+            r = sub._CAPI_Relabel()
+            loop += [r[0], r[3], r[4], sub._CAPI_GetData("default")]
+            cols = r[0]
+        for a, b in zip(got, loop):
+            assert torch.equal(a, b)
+    # the blocks of the Python helper carry the data as edge weights
+    gs.set_seed(410)
+    _, blocks = gs.sample_layers(g, t_seeds, list(fanouts), replace)
+    gs.set_seed(410)
+    got = g._CAPI_SampleLayers(t_seeds, list(fanouts), replace)
+    assert torch.equal(blocks[-1].edata["w"], got[3])
+
+
+def test_fused_sampling_settles_its_edge_data_whichever_method_comes_first(dev):
+    """The fused sampler hands its child back before the edge count is known; the child's data
+    is there whether Relabel, GetData or GetCSC is the first method called on it."""
+    n = 1 << 11
+    indptr, indices = rmat_csc_np(n, 1 << 15, seed=2)
+    data = (1.0 - np.random.default_rng(1).random(indices.size)).astype(np.float32)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev))
+    g._CAPI_SetData(to_dev(data, dev))
+    seeds = np.arange(0, n, 3, dtype=np.int64)
+    sel = O.sample_uniform(indptr, indices, seeds, 5, False, seed=8, with_coo=False)[3]
+    for first_call in ("relabel", "data", "csc"):
+        gs.set_seed(8)
+        sub = g._CAPI_FusedColumnwiseSlicingSampling(to_dev(seeds, dev), 5, False)
+        if first_call == "relabel":
+            sub._CAPI_Relabel()
+        elif first_call == "csc":
+            sub._CAPI_GetCSC()
+        assert np.array_equal(sub._CAPI_GetData("default").cpu().numpy(), data[sel])
+        assert sub._CAPI_GetNumEdges() == sel.size
+
+
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
 def test_sample_layers_with_no_seeds_and_with_isolated_seeds(dev, idt):
     """No seeds at all, and seeds without neighbours (every later layer is then empty too):
     lengths 0 all the way, offsets of the right length, no launch goes wrong."""

@@ -70,6 +70,43 @@ def test_chain_matches_the_oracle_layer_by_layer(dev, idt, num_seeds, fanouts, r
         assert bool((t.buf.view(torch.int64) == -1).all())
 
 
+@pytest.mark.parametrize("idt", [torch.int32, torch.int64])
+@pytest.mark.parametrize("with_edge_ids", [False, True])
+@pytest.mark.parametrize("num_seeds,fanouts,replace", [
+    (1024, (15, 10, 5), False),
+    (700, (3, 40), True),      # fanout 40 with replacement: further rounds of a row's lanes
+    (0, (4, 4), False),
+    (257, (1, 6), False),
+])
+def test_chain_carries_the_edge_data_of_its_samples(dev, idt, with_edge_ids, num_seeds, fanouts,
+                                                    replace):
+    """With edge data the sampler leaves, per layer, the position of every sample in the graph's
+    indices and data[e_ids[position]] (the gathers of the reference's src/graph.cc:544-557), at
+    the same place as the sample's renamed id."""
+    n = 1 << 13
+    indptr, indices = rmat_csc_np(n, 1 << 18, seed=23)
+    rng = np.random.default_rng(77)
+    data = (1.0 - rng.random(indices.size)).astype(np.float32)
+    e_ids = rng.permutation(indices.size).astype(np.int64) if with_edge_ids else None
+    seeds = rng.permutation(n)[:num_seeds].astype(np.int64)
+    layers, _ = capi.sample_layers(
+        to_dev(indptr, dev), to_dev(indices, dev, idt), to_dev(seeds, dev, idt), fanouts, replace,
+        seed=61, edge_data=to_dev(data, dev), edge_ids=None if e_ids is None else to_dev(e_ids, dev))
+    want = _oracle_layers(indptr, indices, seeds, fanouts, replace, 61)
+    _check_layers(layers, want)
+    cols = seeds
+    for l, (b, k) in enumerate(zip(layers, fanouts)):
+        _, _, si, sel = O.sample_uniform(indptr, indices, cols, k, replace, seed=61 + l,
+                                         with_coo=False)
+        E = int(b.counts[0])
+        assert E == sel.size
+        assert np.array_equal(b.select_index[:E].cpu().numpy(), sel)
+        assert np.array_equal(indices[sel], si)
+        picked = data[sel] if e_ids is None else data[e_ids[sel]]
+        assert np.array_equal(b.data[:E].cpu().numpy(), picked)
+        cols = want[l][3]
+
+
 @pytest.mark.parametrize("num_seeds", [5000, 1000])
 def test_chain_with_repeated_seeds_and_hub_columns(dev, num_seeds):
     """Seeds that repeat (the frontier is shorter than the seed list), seeds that the sampled
