@@ -390,6 +390,63 @@ def test_large_graph_whole_minibatch_call_and_block_sddmm(dev, large_graph):
             cols, h_cols = frontier, want_frontier
 
 
+def _check_weighted_minibatch(dev, indptr, indices, weights, num_nodes, first_seed):
+    """One [15, 10, 5] x 1024 minibatch on a graph that carries fp32 edge weights, through
+    _CAPI_SampleLayers and through the per-layer calls: ids against the oracle bit for bit, and
+    every layer's data equal to weights[select_index] (reference src/graph.cc:544-557), the
+    oracle's select_index taken to positions of the whole graph."""
+    from tests.util import columns_as_a_graph
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(indptr, indices)
+    g._CAPI_SetData(weights)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(first_seed)
+    seeds = torch.randperm(num_nodes, generator=gen, device=dev)[:1024].to(indices.dtype)
+    torch.ops.gs_ops._CAPI_SetSeed(first_seed)
+    parts = g._CAPI_SampleLayers(seeds, list(FANOUTS), False)
+    assert len(parts) == 4 * len(FANOUTS)
+    torch.ops.gs_ops._CAPI_SetSeed(first_seed)
+    cols, h_cols, total = seeds, _host(seeds), 0
+    for l, k in enumerate(FANOUTS):
+        h_ptr, h_idx, pos = columns_as_a_graph(indptr, indices, cols, with_positions=True)
+        sp, _, rows, sel = O.sample_uniform(h_ptr, h_idx, np.arange(h_cols.size, dtype=np.int64),
+                                            k, False, seed=first_seed + l, with_coo=False)
+        want_frontier, (want_idx,) = O.relabel([h_cols, rows], [rows])
+        want_data = weights[pos[torch.from_numpy(sel).to(dev)]]
+        sub = g._CAPI_FusedColumnwiseSlicingSampling(cols, k, False)
+        r = sub._CAPI_Relabel()
+        for frontier, offsets, renamed, data in (parts[4 * l:4 * l + 4],
+                                                 (r[0], r[3], r[4], sub._CAPI_GetData("default"))):
+            assert np.array_equal(_host(offsets), sp)
+            assert np.array_equal(_host(renamed), want_idx)
+            assert np.array_equal(_host(frontier), want_frontier)
+            assert torch.equal(data, want_data)
+        total += rows.size
+        cols, h_cols = parts[4 * l], want_frontier
+    return total
+
+
+def test_large_graph_with_edge_weights_keeps_the_queued_path(dev, large_graph):
+    """Configuration 5 as BASELINE.json states it: the 111 M / 1.6 B graph WITH its fp32 edge
+    weights attached (6.4 GB)."""
+    indptr, indices, _ = large_graph
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    weights = 1.0 - torch.rand(indices.numel(), generator=gen, device=dev)
+    assert _check_weighted_minibatch(dev, indptr, indices, weights, LARGE_NODES, 500) > 100_000
+    del weights
+
+
+def test_config_2_graph_with_edge_weights(dev, sage_graph):
+    """The same on configuration 2's graph (2.45 M nodes / 124 M edges, int32 ids) with weights,
+    which is configuration 3's graph."""
+    indptr, indices = sage_graph[:2]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    weights = 1.0 - torch.rand(indices.numel(), generator=gen, device=dev)
+    assert _check_weighted_minibatch(dev, indptr, indices, weights, 2_450_000, 600) > 200_000
+
+
 def test_large_graph_sampler_properties(dev, large_graph):
     """2^18 columns of the 1.6 B-edge graph (positions up to 1.6 * 10^9 in `indices`): counts,
     positions inside the column, ids read from those positions, distinct positions per row."""

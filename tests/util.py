@@ -62,12 +62,14 @@ def row_slice_coo_closed_form(key, other, ids):
     return renamed, other[mask], np.nonzero(mask)[0].astype(np.int64)
 
 
-def columns_as_a_graph(indptr, indices, cols):
+def columns_as_a_graph(indptr, indices, cols, with_positions=False):
     """(offsets, neighbour ids) of the columns `cols` of a device CSC as numpy arrays, cut out
     with plain torch indexing (no library kernel).  The oracle's samplers address a column by
     its place in the call, so sampling columns 0..len(cols)-1 of this small graph with the same
     seed gives what sampling `cols` of the whole graph gives: graphs too large to copy to the
-    host are checked this way.  Ids outside the graph count as empty columns."""
+    host are checked this way.  Ids outside the graph count as empty columns.
+    with_positions: also the place of every edge of the small graph in the whole graph's
+    `indices` (a device tensor), which turns the oracle's select_index into the graph's."""
     import torch
     n = indptr.numel() - 1
     cols = cols.long()
@@ -81,4 +83,6 @@ def columns_as_a_graph(indptr, indices, cols):
     owner = torch.repeat_interleave(torch.arange(cols.numel(), device=indptr.device), deg,
                                     output_size=total)
     pos = torch.arange(total, device=indptr.device) - offsets[owner] + starts[owner]
+    if with_positions:
+        return offsets.cpu().numpy(), indices[pos].cpu().numpy().astype(np.int64), pos
     return offsets.cpu().numpy(), indices[pos].cpu().numpy().astype(np.int64)
