@@ -328,6 +328,24 @@ def sample_uniform_fused_static(indptr, indices, column_ids, fanout, replace, ou
     return ticket
 
 
+def static_init():
+    """gs_sample_uniform_fused_static_init: resolves the library's state array on the current
+    device (to be called before a stream capture that records the static sampler)."""
+    _check(lib().gs_sample_uniform_fused_static_init(), "gs_sample_uniform_fused_static_init")
+
+
+def static_reset():
+    """gs_sample_uniform_fused_static_reset: the next static call starts from a zero-filled
+    state (after a call that reported -1)."""
+    _check(lib().gs_sample_uniform_fused_static_reset(), "gs_sample_uniform_fused_static_reset")
+
+
+def static_debug_raise(device):
+    """Raises the sticky error word in the library's own look-back state (test hook)."""
+    _check(lib().gs_sample_uniform_fused_static_debug_raise(_stream(device)),
+           "gs_sample_uniform_fused_static_debug_raise")
+
+
 class RelabelTable:
     """The persistent hash table of gs_relabel_sampled (prepared once, left empty by every call)."""
 

@@ -631,4 +631,9 @@ __device__ __forceinline__ void post_mailbox(gs_mailbox* box, int64_t total, int
   __hip_atomic_store(&box->ticket, ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// gs_coo_sum with a bound on the targets: one outside [0, num_targets) is left out
+// (gs_segment.hip; gs_coo_sum_binned passes the calls it does not bin on to it)
+int coo_sum_bounded(const void* target, int id_bytes, const int64_t* e_ids, const float* data,
+                    int64_t E, int64_t powk, int64_t num_targets, float* out, void* stream);
+
 }  // namespace gs

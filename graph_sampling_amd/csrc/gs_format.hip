@@ -866,7 +866,7 @@ int gs_coo_sum_binned(const void* target, int id_bytes, const int64_t* e_ids, co
              id_bytes);
   if (E == 0) return GS_OK;
   if (!bin_sum_applies(id_bytes, e_ids, E, num_targets))
-    return gs_coo_sum(target, id_bytes, e_ids, data, E, powk, out, stream);
+    return coo_sum_bounded(target, id_bytes, e_ids, data, E, powk, num_targets, out, stream);
   return bin_sum_impl(static_cast<const int32_t*>(target), data, E, static_cast<int>(powk),
                       num_targets, out, workspace, workspace_bytes,
                       static_cast<hipStream_t>(stream));

@@ -208,10 +208,12 @@ keys_hist_kernel(const float* __restrict__ probs, int64_t n, int run_shift, int6
     if (s_hist[i]) atomicAdd(&hist[i], s_hist[i]);
   // The workgroup that finishes last sees every count and makes the pick for the later
   // launches.  The additions are device-scope operations, done where every workgroup sees them
-  // once they are acknowledged: waiting for the acknowledgements (what a workgroup-scope
-  // release amounts to) is enough, and a device-scope fence would write the L2's dirty lines
-  // back first -- all the keys just stored, 60 us of it at 2.45 M items.  The pick reads the
-  // counts past the caches (device-scope loads).
+  // once they are acknowledged, so every thread waits for the acknowledgements of its OWN
+  // additions (the vector-memory counter; a workgroup-scope release alone need not wait for
+  // them) before the barrier that precedes the ticket.  A device-scope fence would do too, but
+  // writes the L2's dirty lines back first -- all the keys just stored, 60 us of it at
+  // 2.45 M items.  The pick reads the counts past the caches (device-scope loads).
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (threadIdx.x == 0) s_last = atomicAdd(&st->finished, 1u) == gridDim.x - 1;

@@ -1500,6 +1500,81 @@ int gs_layer_sample(const int64_t* indptr, int64_t num_cols, const void* indices
                                        S_dev, t, pos, num_edges, edge_data, edge_ids, data_out);
 }
 
+// device address of `scratch` on the current device, resolved once per device (not under
+// stream capture: the lookup is a runtime call of its own)
+// (stream_known: `stream` is the stream of a launch and is asked whether it is being captured;
+// the calls that launch nothing leave every stream alone)
+static int static_state_of_current_device(const char* who, bool stream_known, hipStream_t stream,
+                                          bool* capturing, gs::StaticState** out) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    set_error_text("%s: no current device (or its number is above %d)", who, kMaxDevices - 1);
+    return GS_ERR_LAUNCH;
+  }
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (stream_known && hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+    set_error_text("%s: hipStreamIsCapturing failed", who);
+    return GS_ERR_LAUNCH;
+  }
+  *capturing = cap != hipStreamCaptureStatusNone;
+  StaticState& st = g_static_state[device];
+  if (!st.ptr) {
+    if (*capturing) {
+      set_error_text("%s: the first call on a device resolves the address of the library's "
+                     "state array, which cannot be done while the stream is being captured; call "
+                     "gs_sample_uniform_fused_static_init before the capture", who);
+      return GS_ERR_UNSUPPORTED;
+    }
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      set_error_text("%s: hipGetSymbolAddress: %s", who, hipGetErrorString(e));
+      return GS_ERR_LAUNCH;
+    }
+    st.ptr = p;
+    st.epoch = 0;
+  }
+  *out = &st;
+  return GS_OK;
+}
+
+int gs_sample_uniform_fused_static_init(void) {
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  bool capturing = false;
+  StaticState* st = nullptr;
+  return static_state_of_current_device("gs_sample_uniform_fused_static_init", false, nullptr,
+                                        &capturing, &st);
+}
+
+int gs_sample_uniform_fused_static_reset(void) {
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  bool capturing = false;
+  StaticState* st = nullptr;
+  GS_RETURN_IF_ERROR(static_state_of_current_device("gs_sample_uniform_fused_static_reset", false,
+                                                    nullptr, &capturing, &st));
+  st->epoch = 0;  // the next call zero-fills the array (error word included) before it runs
+  return GS_OK;
+}
+
+namespace gs {
+namespace {
+static __global__ void raise_error_word_kernel(unsigned int* error) { *error = 1u; }
+}  // namespace
+}  // namespace gs
+
+int gs_sample_uniform_fused_static_debug_raise(void* stream) {
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  bool capturing = false;
+  StaticState* st = nullptr;
+  GS_RETURN_IF_ERROR(static_state_of_current_device("gs_sample_uniform_fused_static_debug_raise",
+                                                    true, static_cast<hipStream_t>(stream),
+                                                    &capturing, &st));
+  // the error word is the first word of a look-back state (carve_lookback)
+  hipLaunchKernelGGL(raise_error_word_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream),
+                     static_cast<unsigned int*>(st->ptr));
+  return check_launch("gs_sample_uniform_fused_static_debug_raise");
+}
+
 int gs_sample_uniform_fused_static(const int64_t* indptr, int64_t num_cols, const void* indices,
                                    const void* column_ids, int id_bytes, int64_t S,
                                    int64_t fanout, int replace, uint64_t seed,
@@ -1513,41 +1588,32 @@ int gs_sample_uniform_fused_static(const int64_t* indptr, int64_t num_cols, cons
                    static_cast<long long>(S), static_cast<long long>(GS_FUSED_STATIC_MAX_COLUMNS));
     return GS_ERR_UNSUPPORTED;
   }
-  int device = -1;
-  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
-    set_error_text("gs_sample_uniform_fused_static: no current device (or its number is above %d)",
-                   kMaxDevices - 1);
-    return GS_ERR_LAUNCH;
-  }
   void* state = nullptr;
   uint32_t epoch = 0;
   {
     std::lock_guard<std::mutex> lock(g_static_mu);
-    StaticState& st = g_static_state[device];
-    if (!st.ptr) {
-      void* p = nullptr;
-      const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-      if (e != hipSuccess || !p) {
-        set_error_text("gs_sample_uniform_fused_static: hipGetSymbolAddress: %s",
-                       hipGetErrorString(e));
-        return GS_ERR_LAUNCH;
-      }
-      st.ptr = p;
-      st.epoch = 0;
-    }
-    if (st.epoch == 0 || st.epoch >= kLbMaxEpoch) {
-      // first use on this device, or every epoch has been used: start again from zeroes (a
-      // fill kernel on the caller's stream, so that a caller who records the call gets a
-      // kernel node)
+    bool capturing = false;
+    StaticState* st = nullptr;
+    GS_RETURN_IF_ERROR(static_state_of_current_device("gs_sample_uniform_fused_static", true,
+                                                      static_cast<hipStream_t>(stream), &capturing,
+                                                      &st));
+    // The epochs are counted here, on the host, and go into the launch as an argument.  A call
+    // that is being recorded into a graph will run again, as often as the graph is replayed,
+    // with that same argument: so a recorded call always starts from a zero-filled array under
+    // epoch 1 (the fill kernel is recorded in front of it), which is right on every replay,
+    // and leaves the count at "fill first" for whatever call comes next.  Otherwise the array
+    // is filled on first use, when every epoch has been used, and after a reset.
+    if (capturing || st->epoch == 0 || st->epoch >= kLbMaxEpoch) {
       const size_t words = kStaticStateBytes / 8;
       hipLaunchKernelGGL(zero_words_kernel, dim3(static_cast<unsigned>((words + 255) / 256)),
                          dim3(256), 0, static_cast<hipStream_t>(stream),
-                         static_cast<unsigned long long*>(st.ptr), words);
+                         static_cast<unsigned long long*>(st->ptr), words);
       GS_RETURN_IF_ERROR(check_launch("gs_sample_uniform_fused_static (state fill)"));
-      st.epoch = 0;
+      st->epoch = 0;
     }
-    state = st.ptr;
-    epoch = ++st.epoch;
+    state = st->ptr;
+    epoch = st->epoch + 1;
+    st->epoch = capturing ? 0 : epoch;
   }
   return gs_sample_uniform_fused(indptr, num_cols, indices, column_ids, id_bytes, S, fanout,
                                  replace, seed, replay, replay_ptr, sub_indptr, sub_indices,

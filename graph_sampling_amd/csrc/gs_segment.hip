@@ -24,6 +24,7 @@
 //    edge.  A 300 000-edge hub is 290 chunks of work for 290 waves, millions of
 //    empty segments cost the by-edge pass nothing, and the order of the additions
 //    is fixed by the layout alone, so results repeat from run to run.
+#include <limits>
 #include "gs_common.hpp"
 
 namespace gs {
@@ -646,17 +647,20 @@ __device__ __forceinline__ void keyed_add(KeyedSums& t, long long key, float v) 
   unsafeAtomicAdd(&t.sum[h], v);
 }
 
-__device__ __forceinline__ void keyed_flush(KeyedSums& t, float* __restrict__ out) {
+// (a key outside [0, bound) is left out)
+__device__ __forceinline__ void keyed_flush(KeyedSums& t, float* __restrict__ out,
+                                            long long bound = 0x7FFFFFFFFFFFFFFFll) {
   __syncthreads();
   for (int i = threadIdx.x; i < kAggSlots; i += kThreads)
-    if (t.key[i] != -1) unsafeAtomicAdd(out + t.key[i], t.sum[i]);
+    if (t.key[i] >= 0 && t.key[i] < bound) unsafeAtomicAdd(out + t.key[i], t.sum[i]);
 }
 
 // out[target[e]] += f(data[emap ? emap[e] : e])   (graph_ops.cu:45-64)
 template <typename IdT>
 __global__ void __launch_bounds__(kThreads)
 coo_sum_kernel(const IdT* __restrict__ target, const int64_t* __restrict__ emap,
-               const float* __restrict__ data, int64_t E, int powk, float* __restrict__ out) {
+               const float* __restrict__ data, int64_t E, int powk, float* __restrict__ out,
+               int64_t bound) {
   __shared__ KeyedSums table;
   keyed_clear(table);
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kAggTile + threadIdx.x;
@@ -667,7 +671,7 @@ coo_sum_kernel(const IdT* __restrict__ target, const int64_t* __restrict__ emap,
       keyed_add(table, static_cast<long long>(target[e]),
                 powk_f(data[emap ? emap[e] : e], powk));
   }
-  keyed_flush(table, out);
+  keyed_flush(table, out, bound);
 }
 
 // edge_map_reduce.cu:15-23
@@ -729,6 +733,15 @@ int gs_segment_sum(const int64_t* indptr, const int64_t* e_ids, const void* n_id
 
 int gs_coo_sum(const void* target, int id_bytes, const int64_t* e_ids, const float* data, int64_t E,
                int64_t powk, float* out, void* stream) {
+  return gs::coo_sum_bounded(target, id_bytes, e_ids, data, E, powk,
+                             std::numeric_limits<int64_t>::max(), out, stream);
+}
+
+}  // extern "C"
+
+// gs_coo_sum with targets outside [0, num_targets) left out (gs_coo_sum_binned's other path)
+int gs::coo_sum_bounded(const void* target, int id_bytes, const int64_t* e_ids, const float* data,
+                        int64_t E, int64_t powk, int64_t num_targets, float* out, void* stream) {
   GS_REQUIRE(E >= 0 && powk >= 1, "gs_coo_sum: negative size or powk < 1");
   GS_REQUIRE(E == 0 || (target && data && out), "gs_coo_sum: null pointer");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_coo_sum: id_bytes must be 4 or 8, got %d", id_bytes);
@@ -738,13 +751,16 @@ int gs_coo_sum(const void* target, int id_bytes, const int64_t* e_ids, const flo
   if (id_bytes == 8)
     hipLaunchKernelGGL(coo_sum_kernel<int64_t>, grid, dim3(kThreads), 0, st,
                        static_cast<const int64_t*>(target), e_ids, data, E, static_cast<int>(powk),
-                       out);
+                       out, num_targets);
   else
     hipLaunchKernelGGL(coo_sum_kernel<int32_t>, grid, dim3(kThreads), 0, st,
                        static_cast<const int32_t*>(target), e_ids, data, E, static_cast<int>(powk),
-                       out);
+                       out, num_targets);
   return check_launch("coo_sum");
 }
+
+extern "C" {
+
 
 int gs_segment_normalize(const int64_t* indptr, const int64_t* e_ids, const float* data,
                          int64_t num_segments, int64_t nnz, float* out, void* workspace,

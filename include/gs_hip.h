@@ -218,9 +218,27 @@ int gs_sample_uniform_fused_data(const int64_t* indptr, int64_t num_cols, const 
  * gs_sample_uniform_fused otherwise; S above GS_FUSED_STATIC_MAX_COLUMNS is refused with
  * GS_ERR_UNSUPPORTED.  Runs on the current device.  Every call on a device shares that
  * device's array: calls that overlap in time on one device (two streams, two threads)
- * race; calls on one stream, or ordered by events, are fine.  Once per 16383 calls, and at
- * the first call on a device, a fill kernel on `stream` zeroes the array first. */
+ * race; calls on one stream, or ordered by events, are fine.  Once per 16383 calls, at the
+ * first call on a device and after a reset, a fill kernel on `stream` zeroes the array first.
+ *
+ * Under stream capture (hipStreamIsCapturing): the epoch is an argument of the launch, and a
+ * recorded launch runs again on every replay, so a recorded call always consists of the fill
+ * kernel followed by the sampler under epoch 1 -- two kernel nodes, right on every replay
+ * whatever ran in between.  The address of the array is looked up at the first call on a
+ * device, which must therefore come before the capture: call
+ * gs_sample_uniform_fused_static_init() (idempotent, allocates nothing) on the device first;
+ * a first call under capture is refused with GS_ERR_UNSUPPORTED.  A mailbox ticket recorded
+ * into a graph is posted again on every replay.
+ *
+ * When a call reports a total of -1 (a tile's bounded wait ran out), the error word stays in
+ * the library's array, which the caller cannot reach: call
+ * gs_sample_uniform_fused_static_reset() and the next call starts from a zero-filled array.
+ * gs_sample_uniform_fused_static_debug_raise(stream) raises that error word from the host
+ * (test suites: every kernel still runs to its end). */
 #define GS_FUSED_STATIC_MAX_COLUMNS ((int64_t)1 << 22)
+int gs_sample_uniform_fused_static_init(void);
+int gs_sample_uniform_fused_static_reset(void);
+int gs_sample_uniform_fused_static_debug_raise(void* stream);
 int gs_sample_uniform_fused_static(const int64_t* indptr, int64_t num_cols, const void* indices,
                                    const void* column_ids, int id_bytes, int64_t S,
                                    int64_t fanout, int replace, uint64_t seed,

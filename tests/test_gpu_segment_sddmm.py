@@ -252,6 +252,25 @@ def test_coo_sum_binned(dev, idt, targets, edges, skew):
     np.testing.assert_allclose(out.cpu().numpy(), want, rtol=2e-5)
 
 
+@pytest.mark.parametrize("edges", [1 << 18, 5000])
+def test_coo_sum_binned_leaves_out_targets_beyond_the_output(dev, edges):
+    """A target outside [0, num_targets) is left out on the binned path (2^18 edges) and on the
+    plain kernel the smaller call is passed on to; the slots behind `out` stay untouched."""
+    targets = 1000
+    rng = np.random.default_rng(edges)
+    t = rng.integers(0, targets + 200, size=edges)
+    t[:4] = [-1, -5, targets, 1 << 30]
+    data = (rng.random(edges, dtype=np.float32) + 0.25).astype(np.float32)
+    buf = torch.full((targets + 4096,), 7.0, dtype=torch.float32, device=dev)
+    out = buf[:targets]
+    out.zero_()
+    capi.coo_sum_binned(to_dev(t, dev, torch.int32), None, to_dev(data, dev), 1, out)
+    ok = (t >= 0) & (t < targets)
+    want = np.bincount(t[ok], weights=data[ok].astype(np.float64), minlength=targets)
+    np.testing.assert_allclose(out.cpu().numpy(), want, rtol=2e-5)
+    assert bool((buf[targets:] == 7.0).all())
+
+
 # ------------------------------------------------------------------ SDDMM
 def _sddmm_coo_gpu(dev, op, row, col, e_ids, lhs, rhs, lt, rt, idt=torch.int64):
     ls = lhs.shape if lhs.ndim > 1 else lhs.shape + (1,)

@@ -68,3 +68,83 @@ def test_static_state_sampler_refuses_more_columns_than_its_state_holds(dev):
     torch.cuda.synchronize()
     n = int(want[0][-1])
     assert torch.equal(want[0], out[0][:(1 << 22) + 1]) and torch.equal(want[1][:n], out[1][:n])
+
+
+def test_static_state_sampler_allocates_nothing(dev):
+    """Free device memory is the same before and after static calls of several sizes (the
+    outputs are made beforehand; the call itself must not reach the allocator)."""
+    h_indptr, h_indices = rmat_csc_np(1 << 13, 1 << 17, seed=5)
+    indptr, indices = to_dev(h_indptr, dev), to_dev(h_indices, dev, torch.int32)
+    sizes = (30_000, 500, 12_000)
+    cols = [to_dev(np.random.default_rng(s).integers(0, 1 << 13, size=s), dev, torch.int32)
+            for s in sizes]
+    outs = [(torch.empty(s + 1, dtype=torch.int64, device=dev),
+             torch.empty(s * 8, dtype=torch.int32, device=dev),
+             torch.empty(s * 8, dtype=torch.int64, device=dev), None) for s in sizes]
+    capi.sample_uniform_fused_static(indptr, indices, cols[0], 8, False, outs[0], seed=1)  # warm-up
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    reserved_before = torch.cuda.memory_reserved(dev)
+    for rep in range(3):
+        for c, o in zip(cols, outs):
+            capi.sample_uniform_fused_static(indptr, indices, c, 8, rep == 1, o, seed=rep)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
+    assert torch.cuda.memory_reserved(dev) == reserved_before
+
+
+def test_static_state_sampler_recovers_after_a_reset(dev):
+    """The error word a give-up leaves is in the library's own array: every later call reports
+    -1 until gs_sample_uniform_fused_static_reset, after which results are right again."""
+    h_indptr, h_indices = rmat_csc_np(1 << 12, 1 << 16, seed=6)
+    indptr, indices = to_dev(h_indptr, dev), to_dev(h_indices, dev, torch.int32)
+    cols = to_dev(np.random.default_rng(2).integers(0, 1 << 12, size=3000), dev, torch.int32)
+    _both(indptr, indices, cols, 6, False, 30, dev, False)
+    capi.static_debug_raise(dev)
+    out = (torch.empty(3001, dtype=torch.int64, device=dev),
+           torch.empty(18000, dtype=torch.int32, device=dev), None, None)
+    for seed in (31, 32):  # sticky: both report the failure
+        capi.sample_uniform_fused_static(indptr, indices, cols, 6, False, out, seed=seed)
+        torch.cuda.synchronize()
+        assert int(out[0][-1]) == -1
+    capi.static_reset()
+    _both(indptr, indices, cols, 6, False, 33, dev, False)
+    _both(indptr, indices, cols[:100], 6, False, 34, dev, True)
+
+
+def test_static_state_sampler_recorded_into_a_graph_is_right_on_every_replay(dev):
+    """One static call recorded into a HIP graph, the column ids rewritten in place between the
+    replays, eager static calls of other sizes in between (they leave other epochs in the shared
+    state): every replay equals gs_sample_uniform_fused on the same columns."""
+    h_indptr, h_indices = rmat_csc_np(1 << 13, 1 << 17, seed=7)
+    indptr, indices = to_dev(h_indptr, dev), to_dev(h_indices, dev, torch.int32)
+    rng = np.random.default_rng(8)
+    S, k = 20_000, 10
+    cols = to_dev(rng.integers(0, 1 << 13, size=S), dev, torch.int32)
+    out = (torch.full((S + 1,), -7, dtype=torch.int64, device=dev),
+           torch.full((S * k,), -7, dtype=torch.int32, device=dev),
+           torch.full((S * k,), -7, dtype=torch.int64, device=dev), None)
+    other = to_dev(rng.integers(0, 1 << 13, size=900), dev, torch.int32)
+    other_out = (torch.empty(901, dtype=torch.int64, device=dev),
+                 torch.empty(900 * k, dtype=torch.int32, device=dev), None, None)
+    capi.static_init()
+    capi.sample_uniform_fused_static(indptr, indices, other, k, False, other_out, seed=1)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        capi.sample_uniform_fused_static(indptr, indices, cols, k, False, out, seed=21)
+    for rep in range(3):
+        cols.copy_(to_dev(rng.integers(0, 1 << 13, size=S), dev, torch.int32))
+        for o in out[:3]:
+            o.fill_(-7)
+        capi.sample_uniform_fused_static(indptr, indices, other, k, False, other_out, seed=rep)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = capi.sample_uniform_fused(indptr, indices, cols, k, False, seed=21)
+        n = int(want[0][-1])
+        assert int(out[0][-1]) == n > 0
+        assert torch.equal(want[0], out[0])
+        assert torch.equal(want[1][:n], out[1][:n]) and torch.equal(want[2][:n], out[2][:n])
+    # an eager call after the recorded one still works (the epoch count was left at "fill first")
+    _both(indptr, indices, cols[:5000], k, False, 40, dev, True)
