@@ -662,10 +662,16 @@ def unique_relabel(mapping, queries, mailbox=None, last_span_len=None, narrow=Fa
     return frontier, num_unique, outs
 
 
-def batch_csr_relabel(seeds, seeds_ptr, ids, ids_ptr, mailbox=None, narrow=False):
+RELABEL_REGIONS = 0x200
+RELABEL_BINS = 0x400
+
+
+def batch_csr_relabel(seeds, seeds_ptr, ids, ids_ptr, mailbox=None, narrow=False, path=None):
     """gs_batch_csr_relabel.  Returns (unique_buf, unique_ptr, relabelled ids, num_unique_dev
-    [, ticket]); unique_buf has the capacity len(seeds) + len(ids)."""
+    [, ticket]); unique_buf has the capacity len(seeds) + len(ids).  path: None (the library
+    chooses), "bins" or "regions"."""
     idb = _ids(seeds, "seeds") | (NARROW_IDS if narrow else 0)
+    idb |= {None: 0, "bins": RELABEL_BINS, "regions": RELABEL_REGIONS}[path]
     _ids(ids, "ids", like=seeds)
     _need(seeds_ptr, torch.int64, "seeds_ptr")
     _need(ids_ptr, torch.int64, "ids_ptr")

@@ -636,4 +636,16 @@ __device__ __forceinline__ void post_mailbox(gs_mailbox* box, int64_t total, int
 int coo_sum_bounded(const void* target, int id_bytes, const int64_t* e_ids, const float* data,
                     int64_t E, int64_t powk, int64_t num_targets, float* out, void* stream);
 
+// The batched relabel by hash classes and LDS tables (gs_binrelabel.hip): same outputs as
+// the one on hash regions (gs_unique.hip), no memory-side atomic per item.  Ids must fit 32
+// bits (id_bytes 8: the 64-bit ids are read and written as such).  *num_unique = -4 when a
+// class held more distinct ids than its table: the call has to be repeated on hash regions.
+size_t binned_relabel_workspace_bytes(int64_t M, int64_t B);
+bool binned_relabel_applies(int64_t M, int64_t B);
+int batch_relabel_binned(const void* seeds, const int64_t* seeds_ptr, const void* ids,
+                         const int64_t* ids_ptr, int64_t B, int64_t num_seeds, int64_t num_ids,
+                         int id_bytes, void* unique, int64_t* unique_ptr, void* out_ids,
+                         int64_t* num_unique, void* workspace, size_t workspace_bytes,
+                         gs_mailbox* box, int64_t box_ticket, hipStream_t stream);
+
 }  // namespace gs

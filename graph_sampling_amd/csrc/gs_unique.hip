@@ -23,6 +23,7 @@
 //    so every relabel lookup is two gathers in a last kernel, and a query that
 //    aliases a mapping span is relabelled by slot gather instead of probing.
 #include "gs_common.hpp"
+#include "gs_batch_items.hpp"
 #include <type_traits>
 
 #include "gs_table.hpp"
@@ -773,59 +774,6 @@ layer_sweep_kernel(PackedTable t, const uint32_t* __restrict__ pos, RankCounts n
 //    its lanes search inside it.
 constexpr int64_t kRegionFactor = 2;
 
-constexpr int64_t kStagedBatches = 511;  // batch offsets a workgroup keeps in LDS (2 x 4 KB)
-
-template <typename IdT>
-struct BatchItems {
-  const IdT* seeds;
-  const int64_t* seeds_ptr;
-  const IdT* ids;
-  const int64_t* ids_ptr;
-  int64_t B;
-  __device__ __forceinline__ int64_t start(int64_t b) const { return seeds_ptr[b] + ids_ptr[b]; }
-  // last b in [lo, hi] with start(b) <= i
-  __device__ __forceinline__ int64_t batch_of(int64_t i, int64_t lo, int64_t hi) const {
-    while (lo < hi) {
-      const int64_t mid = (lo + hi + 1) >> 1;
-      if (start(mid) <= i) lo = mid; else hi = mid - 1;
-    }
-    return lo;
-  }
-  // (one read through a chosen address, not one of two reads: a read that may or may not
-  // happen makes every later one wait for all that is in flight)
-  __device__ __forceinline__ const IdT* where_in(int64_t b, int64_t i) const {
-    const int64_t off = i - start(b);
-    const int64_t n_seeds = seeds_ptr[b + 1] - seeds_ptr[b];
-    return off < n_seeds ? seeds + seeds_ptr[b] + off : ids + ids_ptr[b] + off - n_seeds;
-  }
-  __device__ __forceinline__ IdT get_in(int64_t b, int64_t i) const { return *where_in(b, i); }
-  // The batch offsets copied into LDS (when there are at most kStagedBatches batches), and
-  // this object re-pointed at the copy: the searches and the offset reads that stand between
-  // a lane and its key then cost no trip to memory.  Every thread of the workgroup calls it.
-  __device__ __forceinline__ void stage_offsets(int64_t* lds_seeds_ptr, int64_t* lds_ids_ptr) {
-    if (B > kStagedBatches) return;
-    for (int64_t b = threadIdx.x; b <= B; b += blockDim.x) {
-      lds_seeds_ptr[b] = seeds_ptr[b];
-      lds_ids_ptr[b] = ids_ptr[b];
-    }
-    __syncthreads();
-    seeds_ptr = lds_seeds_ptr;
-    ids_ptr = lds_ids_ptr;
-  }
-  // batches of the first and the last item of a workgroup's range, through LDS
-  __device__ __forceinline__ void block_range(int64_t first, int64_t last, int64_t* lds2,
-                                              int64_t* lo, int64_t* hi) const {
-    if (threadIdx.x < 2) lds2[threadIdx.x] = batch_of(threadIdx.x == 0 ? first : last, 0, B - 1);
-    __syncthreads();
-    *lo = lds2[0];
-    *hi = lds2[1];
-  }
-};
-
-__device__ __forceinline__ uint32_t hash32(unsigned long long key) {
-  return static_cast<uint32_t>((key * 0x9E3779B97F4A7C15ull) >> 32);
-}
-
 // one region per batch, slots (key << 32 | first index), all ones = empty
 struct PackedRegions {
   unsigned long long* slots;
@@ -1236,7 +1184,8 @@ size_t gs_batch_relabel_workspace_bytes(int64_t num_items) {
   if (num_items < 0) num_items = 0;
   const size_t a = batch_workspace_bytes_for<int64_t>(num_items);
   const size_t b = batch_workspace_bytes_for<int32_t>(num_items);
-  return a > b ? a : b;
+  const size_t c = binned_relabel_workspace_bytes(num_items, kStagedBatches);
+  return a > b ? (a > c ? a : c) : (b > c ? b : c);
 }
 
 int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void* ids,
@@ -1252,15 +1201,32 @@ int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void
                  (num_seeds + num_ids == 0 || unique),
              "gs_batch_csr_relabel: null buffer");
   const bool narrow = (id_bytes & GS_NARROW_IDS) != 0;
-  id_bytes &= ~GS_NARROW_IDS;
+  const bool want_regions = (id_bytes & GS_RELABEL_REGIONS) != 0;
+  const bool want_bins = (id_bytes & GS_RELABEL_BINS) != 0;
+  id_bytes &= ~(GS_NARROW_IDS | GS_RELABEL_REGIONS | GS_RELABEL_BINS);
   GS_REQUIRE(valid_id_bytes(id_bytes) && (!narrow || id_bytes == 8),
              "gs_batch_csr_relabel: id_bytes must be 4, 8 or 8 | GS_NARROW_IDS, got %d", id_bytes);
+  GS_REQUIRE(!(want_regions && want_bins),
+             "gs_batch_csr_relabel: GS_RELABEL_REGIONS and GS_RELABEL_BINS exclude each other");
   if (num_seeds + num_ids >= (int64_t(1) << 30)) {
     set_error_text("gs_batch_csr_relabel: %lld items exceed the supported 2^30",
                    static_cast<long long>(num_seeds + num_ids));
     return GS_ERR_UNSUPPORTED;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // ids that ride in 32 bits go through the bins from about half a million items on
+  const bool can_bin = (id_bytes == 4 || narrow) && num_seeds + num_ids > 0 &&
+                       num_batches <= kStagedBatches;
+  if (want_bins && !can_bin) {
+    set_error_text("gs_batch_csr_relabel: GS_RELABEL_BINS needs ids that fit 32 bits, at least "
+                   "one item and at most %lld batches", static_cast<long long>(kStagedBatches));
+    return GS_ERR_UNSUPPORTED;
+  }
+  if (can_bin && !want_regions &&
+      (want_bins || binned_relabel_applies(num_seeds + num_ids, num_batches)))
+    return batch_relabel_binned(seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds, num_ids,
+                                id_bytes, unique, unique_ptr, out_ids, num_unique, workspace,
+                                workspace_bytes, mailbox, mailbox_ticket, st);
   if (id_bytes == 4)
     return batch_relabel_impl<int32_t, PackedRegions>(
         seeds, seeds_ptr, ids, ids_ptr, num_batches, num_seeds, num_ids, unique, unique_ptr, out_ids,

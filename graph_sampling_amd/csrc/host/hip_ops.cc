@@ -82,6 +82,7 @@ torch::Tensor Scratch(size_t bytes, const torch::Tensor& like) {
 // been issued.
 constexpr int64_t kBoxes = 1024;
 constexpr int64_t kLost = -3;     // the slot was reused before anyone read it
+constexpr int64_t kBinsFull = -4; // posted by the binned batch relabel: repeat on hash regions
 constexpr int64_t kTooWide = -2;  // posted by the narrow relabel: a key needs more than 32 bits
 constexpr int64_t kGaveUp = -1;   // posted when a tile's bounded wait ran out
 
@@ -872,17 +873,20 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(
   void* st = Stream(seeds);
   HostBoxes& boxes = Boxes(seeds.device().index());
   int64_t U = kTooWide;
-  for (int attempt = 0; attempt < 2 && U == kTooWide; ++attempt) {
+  int path = 0;  // the library chooses between bins and hash regions
+  for (int attempt = 0; attempt < 3 && (U == kTooWide || U == kBinsFull); ++attempt) {
     const int64_t ticket = boxes.next++;
     Check(gs_batch_csr_relabel(seeds.data_ptr(), seeds_ptr.data_ptr<int64_t>(), ids.data_ptr(),
                                ids_ptr.data_ptr<int64_t>(), B, seeds.numel(), ids.numel(),
-                               TableIds(idb), unique.data_ptr(), unique_ptr.data_ptr<int64_t>(),
-                               out_ids.data_ptr(), num.data_ptr<int64_t>(), ws.data_ptr(),
-                               ws.numel(), boxes.slot(ticket), ticket, st),
+                               TableIds(idb) | path, unique.data_ptr(),
+                               unique_ptr.data_ptr<int64_t>(), out_ids.data_ptr(),
+                               num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(),
+                               boxes.slot(ticket), ticket, st),
           "gs_batch_csr_relabel");
     U = WaitBox(boxes.slot(ticket), ticket, st, "gs_batch_csr_relabel");
     if (U == kLost) U = num.item<int64_t>();
     if (U == kTooWide) t_narrow_ids = false;
+    if (U == kBinsFull) path = GS_RELABEL_REGIONS;  // a class outgrew its LDS table
   }
   TORCH_CHECK(U >= 0, "gs_batch_csr_relabel: a tile gave up waiting for its predecessors");
   return {unique.narrow(0, 0, U), unique_ptr, out_ids};

@@ -78,6 +78,18 @@ typedef struct gs_mailbox {
  * int64 throughout; this is how that costs no more than int32.) */
 #define GS_NARROW_IDS 0x100
 
+/* Or-ed into id_bytes of gs_batch_csr_relabel: which of its two implementations runs.  By
+ * default ids that fit 32 bits (id_bytes 4, or 8 | GS_NARROW_IDS), from about half a million
+ * items on and with at most 511 batches, are relabelled through bins (the items of a batch
+ * are brought together by hash class and deduplicated in LDS: no atomic on memory per item);
+ * everything else through one hash region per batch.  GS_RELABEL_REGIONS forces the second,
+ * GS_RELABEL_BINS the first (refused with GS_ERR_UNSUPPORTED where it cannot run).  The bins
+ * report *num_unique = -4 (mailbox too) when one class of one batch holds more distinct ids
+ * than its LDS table (a single batch of more than ~16 M distinct ids): nothing else written is
+ * valid then; call again with GS_RELABEL_REGIONS. */
+#define GS_RELABEL_REGIONS 0x200
+#define GS_RELABEL_BINS 0x400
+
 /* Optional timing of one launch site, for benchmarks (no counterpart in the
  * reference).  gs_profile_enable("name") makes every later launch of that site
  * record a hipEvent pair on its stream (up to 4096 launches); NULL or ""

@@ -148,6 +148,96 @@ def test_batch_csr_relabel_matches_oracle(dev, idt, B, max_seeds, max_ids, empty
         assert np.array_equal(f[w_out[ip[b]:ip[b + 1]]], ids[ip[b]:ip[b + 1]])
 
 
+def _check_batch_relabel(dev, idt, seeds, sp, ids, ip, narrow, path):
+    unique, unique_ptr, out_ids, num = capi.batch_csr_relabel(
+        to_dev(seeds, dev, idt), to_dev(sp, dev), to_dev(ids, dev, idt), to_dev(ip, dev),
+        narrow=narrow, path=path)
+    w_unique, w_ptr, w_out = O.batch_csr_relabel(seeds, sp, ids, ip)
+    U = int(num.item())
+    assert U == w_unique.size
+    assert np.array_equal(unique_ptr.cpu().numpy(), w_ptr)
+    assert np.array_equal(unique[:U].cpu().numpy().astype(np.int64), w_unique)
+    assert np.array_equal(out_ids.cpu().numpy().astype(np.int64), w_out)
+
+
+@pytest.mark.parametrize("idt,narrow", [(torch.int32, False), (torch.int64, True)])
+@pytest.mark.parametrize("B,max_seeds,max_ids,empty_every", [(1, 50, 400, 0), (7, 30, 300, 3),
+                                                               (64, 256, 4000, 0), (300, 8, 40, 5),
+                                                               (511, 6, 30, 7), (3, 3000, 50000, 0)])
+def test_batch_csr_relabel_through_bins_small(dev, idt, narrow, B, max_seeds, max_ids, empty_every):
+    """The binned relabel (hash classes + LDS tables) forced on inputs far below the size it is
+    chosen for: same frontiers, offsets and ranks as the oracle, empty batches included."""
+    rng = np.random.default_rng(B + 1)
+    seeds, sp, ids, ip = _batches(rng, B, 3000, max_seeds, max_ids, empty_every)
+    _check_batch_relabel(dev, idt, seeds, sp, ids, ip, narrow, "bins")
+
+
+@pytest.mark.parametrize("idt,narrow", [(torch.int32, False), (torch.int64, True)])
+@pytest.mark.parametrize("shape", ["even", "one_large", "hubs", "single", "all_same"])
+def test_batch_csr_relabel_through_bins_at_size(dev, idt, narrow, shape):
+    """From 2^19 items on the library takes the bins by itself: batches of equal size, one batch
+    that holds nearly everything (thousands of classes) beside tiny and empty ones, ids that
+    repeat tens of thousands of times, one batch only, one id only; the last batches empty."""
+    rng = np.random.default_rng(len(shape))
+    n_nodes = 1 << 21
+    if shape == "even":
+        sizes = [(1000, 60000)] * 16
+    elif shape == "one_large":
+        sizes = [(5, 40), (0, 0), (2000, 1_500_000), (1, 0), (0, 7), (300, 9000), (0, 0)]
+    elif shape == "hubs":
+        sizes = [(500, 200000)] * 4
+    elif shape == "single":
+        sizes = [(4096, 900000)]
+    else:
+        sizes = [(1, 300000), (1, 300000)]
+    seeds, ids, sp, ip = [], [], [0], [0]
+    for ns, ni in sizes:
+        seeds.append(rng.permutation(n_nodes)[:ns])
+        if shape == "hubs":     # a few ids hold most of the positions
+            x = (rng.random(ni) ** 8 * n_nodes).astype(np.int64)
+        elif shape == "all_same":
+            x = np.full(ni, 77, dtype=np.int64)
+        else:
+            x = rng.integers(0, n_nodes, size=ni)
+        ids.append(x)
+        sp.append(sp[-1] + ns)
+        ip.append(ip[-1] + ni)
+    seeds = np.concatenate(seeds).astype(np.int64)
+    ids = np.concatenate(ids).astype(np.int64)
+    assert seeds.size + ids.size >= 1 << 19
+    _check_batch_relabel(dev, idt, seeds, np.array(sp, dtype=np.int64), ids,
+                         np.array(ip, dtype=np.int64), narrow, None)
+
+
+def test_batch_csr_relabel_bins_report_what_they_cannot_take(dev):
+    """An id beyond 32 bits among 64-bit ids promised to be narrow: -2, as on the hash regions.  A
+    class with more distinct ids than its LDS table holds: -4 from the C ABI, and the host
+    layer's operator repeats the call on hash regions by itself."""
+    import graph_sampling_amd as gs
+    gs.load_library()
+    rng = np.random.default_rng(5)
+    seeds = rng.permutation(1 << 20)[:100].astype(np.int64)
+    ids = rng.integers(0, 1 << 20, size=(1 << 19) + 5).astype(np.int64)
+    ids[1234] = (1 << 35) + 3
+    sp, ip = np.array([0, 100], dtype=np.int64), np.array([0, ids.size], dtype=np.int64)
+    num = capi.batch_csr_relabel(to_dev(seeds, dev), to_dev(sp, dev), to_dev(ids, dev),
+                                 to_dev(ip, dev), narrow=True)[3]
+    assert int(num.item()) == -2
+    # one batch of 20 M distinct ids: 4096 classes of ~4900 distinct ids each, tables of 4096 slots
+    n = 20_000_000
+    ids = torch.randperm(n, device=dev, dtype=torch.int64).to(torch.int32)
+    seeds = ids[:10].clone()
+    t_sp = torch.tensor([0, 10], device=dev)
+    t_ip = torch.tensor([0, n], device=dev)
+    num = capi.batch_csr_relabel(seeds, t_sp, ids, t_ip)[3]
+    assert int(num.item()) == -4
+    uni, uni_ptr, rel, _ = torch.ops.gs_ops.BatchCSRRelabel(seeds, t_sp, ids, t_ip)
+    # closed form: the seeds are the first ten ids, every other id is new, in order
+    assert uni_ptr.cpu().tolist() == [0, n]
+    assert torch.equal(uni, ids)
+    assert torch.equal(rel, torch.arange(n, device=dev, dtype=torch.int32))
+
+
 # a few tiles of the compaction, with keys all distinct, in long runs, and in between
 @pytest.mark.parametrize("idt", [torch.int64, torch.int32])
 @pytest.mark.parametrize("n", [8191, 8192, 8193, 16383, 16384, 16385])
