@@ -563,6 +563,10 @@ def graphsage(cx, workload, weighted, with_features, full, cpu_budget):
                     "reference's GraphSAGE examples load it): nothing follows the samples"}
         del other
 
+    # the throughput form on the same graph: 64 minibatches per call
+    if extras and full != "config2":
+        out["super_batch"] = super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted)
+
     # u_dot_v with 64-d fp32 node features on every block (the large configuration's second half)
     if extras and with_features:
         gen.manual_seed(3)
@@ -668,44 +672,7 @@ def graphsage(cx, workload, weighted, with_features, full, cpu_budget):
             "ms_per_step": nf_s / nf_steps * 1e3, "value": nf_e / nf_s, "steps": nf_steps,
             "what": "Slicing -> Sampling -> Relabel per layer instead of the fused sampler"}
 
-        # SUPER minibatches per call through the batch operators, on seed sets of its own
-        groups = [[fresh_seeds() for _ in range(SUPER)] for _ in range(3)]
-        super_batch(torch, graph, groups[0])
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        sb_edges = 0
-        sb_sizes = None
-        for grp in groups:
-            n, sb_sizes, _ = super_batch(torch, graph, grp)
-            sb_edges += n
-        torch.cuda.synchronize()
-        sb_s = time.perf_counter() - t1
-        sb_sites = {}
-        for site in SUPER_SITES:
-            timer.enable(site)
-            super_batch(torch, graph, groups[0])
-            torch.cuda.synchronize()
-            ms, n, per_l = timer.collect()
-            if n:
-                sb_sites[site] = (ms, per_l)
-        timer.enable("")
-        sb_dom = max(sb_sites, key=lambda k: sb_sites[k][0])
-        # the dominant site's largest launch (the third layer) against its bytes
-        S3, E3, U3 = sb_sizes[-1]
-        sb_bytes = SUPER_SITES[sb_dom](b, S3, E3, U3)
-        t3 = max(sb_sites[sb_dom][1]) * 1e-3
-        out["super_batch"] = {
-            "minibatches_per_call": SUPER, "calls": len(groups),
-            "ms_per_minibatch": sb_s / (len(groups) * SUPER) * 1e3, "value": sb_edges / sb_s,
-            "layers_S_E_U": sb_sizes,
-            "roofline": {"bound": "hbm", "kernel": sb_dom + " (third layer's launch)",
-                         "achieved": sb_bytes / t3 / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": sb_bytes / t3 / 1e9 / HBM_PEAK_GBS, "launch_us": t3 * 1e6,
-                         "algorithmic_bytes": sb_bytes,
-                         "gpu_ms_by_site": {k: round(v[0], 4) for k, v in sb_sites.items()}},
-            "what": "fused sampling + GetBatchCSC + BatchCSRRelabel + splits over 64 minibatches "
-                    "of 1024 seeds at once; every minibatch is relabelled on its own"}
-        del groups
+        out["super_batch"] = super_batch_leg(torch, graph, timer, fresh_seeds, b, False)
 
         # the same minibatches with 64-bit ids, the reference's only id type
         if idt == torch.int32:
@@ -791,13 +758,103 @@ def graphsage(cx, workload, weighted, with_features, full, cpu_budget):
     return out
 
 
+def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted):
+    """SUPER minibatches per call on seed sets of its own: what the kernels reach once a launch
+    holds enough work for the chip."""
+    per = 4 if weighted else 3
+    # SUPER minibatches per call (a "super-batch"), on seed sets of its own: the C++ layer's
+    # own loop (_CAPI_SampleLayersBatched), and the same flow written with the reference's
+    # operators in Python (examples/graphsage/batching.py:59-88)
+    groups = [[fresh_seeds() for _ in range(SUPER)] for _ in range(5)]
+
+    def batched(grp):
+        return graph._CAPI_SampleLayersBatched(grp, list(FANOUTS), False)
+
+    def sizes_of(res):  # per layer (S, E, U) over all minibatches of a call
+        sizes = [[sum(int(parts[per * l + j].numel()) for parts in res) for j in (1, 2, 0)]
+                 for l in range(len(FANOUTS))]
+        return [(S - len(res), E, U) for S, E, U in sizes]  # (offsets hold one entry more per batch)
+
+    # warm-up with every call's result kept, as in the timed loop: the allocator then holds the
+    # blocks of all of them (a fresh hipMalloc of a few hundred MB costs milliseconds)
+    results = [batched(grp) for grp in groups]
+    del results
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    results = [batched(grp) for grp in groups]  # a call ends with every minibatch's views made
+    torch.cuda.synchronize()
+    sb_s = time.perf_counter() - t1
+    sb_sizes = sizes_of(results[-1])
+    sb_edges = sum(sum(z[1] for z in sizes_of(res)) for res in results)
+    del results
+    super_batch(torch, graph, groups[0])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    py_edges = 0
+    for grp in groups:
+        py_edges += super_batch(torch, graph, grp)[0]
+    torch.cuda.synchronize()
+    py_s = time.perf_counter() - t1
+    sb_sites = {}
+    for site in SUPER_SITES:
+        timer.enable(site)
+        batched(groups[0])
+        torch.cuda.synchronize()
+        ms, n, per_l = timer.collect()
+        if n:
+            sb_sites[site] = (ms, per_l)
+    timer.enable("")
+    sb_dom = max(sb_sites, key=lambda k: sb_sites[k][0])
+    # the dominant site's largest launch (the third layer) against its bytes
+    S3, E3, U3 = sb_sizes[-1]
+    sb_bytes = SUPER_SITES[sb_dom](b, S3, E3, U3)
+    t3 = max(sb_sites[sb_dom][1]) * 1e-3
+    gpu_ms = sum(v[0] for v in sb_sites.values())
+    call_bytes = step_bytes(sb_sizes, weighted)
+    out = {
+        "minibatches_per_call": SUPER, "calls": len(groups),
+        "ms_per_minibatch": sb_s / (len(groups) * SUPER) * 1e3, "value": sb_edges / sb_s,
+        "ms_per_call": sb_s / len(groups) * 1e3,
+        "layers_S_E_U": sb_sizes,
+        "api": "gs_classes.Graph._CAPI_SampleLayersBatched (one call per super-batch)",
+        "through_python_ops": {
+            "ms_per_minibatch": py_s / (len(groups) * SUPER) * 1e3, "value": py_edges / py_s,
+            "what": "the same flow as _CAPI_FusedColumnwiseSlicingSampling + GetBatchCSC + "
+                    "BatchCSRRelabel + SplitByOffset / IndptrSplitByOffset calls from Python"},
+        "roofline": {"bound": "hbm", "kernel": sb_dom + " (third layer's launch)",
+                     "achieved": sb_bytes / t3 / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": sb_bytes / t3 / 1e9 / HBM_PEAK_GBS, "launch_us": t3 * 1e6,
+                     "algorithmic_bytes": sb_bytes,
+                     "gpu_ms_by_site": {k: round(v[0], 4) for k, v in sb_sites.items()}},
+        "step_roofline": {"bound": "hbm", "achieved": call_bytes / (sb_s / len(groups)) / 1e9,
+                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": call_bytes / (sb_s / len(groups)) / 1e9 / HBM_PEAK_GBS,
+                          "gpu_busy_frac": gpu_ms * 1e-3 / (sb_s / len(groups)),
+                          "what": "the scope table's bytes of the whole call (as step_roofline) "
+                                  "over its wall time; gpu_busy_frac = the sites' kernel time "
+                                  "over the same"},
+        "what": "fused sampling over the concatenated seeds + the batches' edge cuts + one relabel "
+                "per minibatch in one pass (through hash classes and LDS tables from 2^19 items "
+                "on) + per-minibatch views, 64 minibatches of 1024 seeds at once"}
+    return out
+
+
 def _sb_sample(b, S, E, U):
     return sample_bytes(b, 0, S, E, U)
 
 
 # launch sites of the super-batch flow and the least bytes of each one's third-layer launch
+# (M = S + E items; the binned relabel: count reads the ids, scatter reads them and writes an
+# 8-byte record each, flag reads and rewrites the records and marks first occurrences, rank
+# reads a byte and writes 16 bytes per 64 items, rename reads the records and a 16-byte entry
+# each and writes the renamed ids and the frontier)
 SUPER_SITES = {
     "sample_fused": _sb_sample,
+    "bins_count": lambda b, S, E, U: (S + E) * b,
+    "bins_scatter": lambda b, S, E, U: (S + E) * (b + 8),
+    "bins_flag": lambda b, S, E, U: (S + E) * 16 + U,
+    "bins_rank": lambda b, S, E, U: (S + E) * (1 + 0.25),
+    "bins_rename": lambda b, S, E, U: (S + E) * (8 + 16) + E * b + U * b,
     "batch_init": lambda b, S, E, U: 4 * (S + E) * 8,            # 8-byte slots, 4 per item
     "batch_insert": lambda b, S, E, U: (S + E) * (b + 16 + 4 + 8),  # id, slot RMW, slot index, offsets
     "batch_compact": lambda b, S, E, U: (S + E) * 20 + U * b,

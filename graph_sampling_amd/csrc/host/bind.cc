@@ -43,6 +43,9 @@ TORCH_LIBRARY(gs_classes, m) {
       GS_DEF2("_CAPI_SampleLayers", "_CAPI_sample_layers", &Graph::SampleLayers)
       GS_DEF2("_CAPI_SampleLayersIfQueued", "_CAPI_sample_layers_if_queued",
               &Graph::SampleLayersIfQueued)
+      // not in the reference: its super-batch flow (examples/graphsage/batching.py:59-98) as one call
+      GS_DEF2("_CAPI_SampleLayersBatched", "_CAPI_sample_layers_batched",
+              &Graph::SampleLayersBatched)
       GS_DEF2("_CAPI_FusionSlicing", "_CAPI_fusion_slicing", &Graph::FusedBidirSlicing)
       GS_DEF2("_CAPI_BatchFusionSlicing", "_CAPI_batch_fusion_slicing",
               &Graph::BatchFusedBidirSlicing)

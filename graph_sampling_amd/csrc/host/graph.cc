@@ -501,6 +501,88 @@ std::vector<torch::Tensor> Graph::SampleLayers(torch::Tensor seeds, std::vector<
   return out;
 }
 
+std::vector<std::vector<torch::Tensor>> Graph::SampleLayersBatched(
+    const std::vector<torch::Tensor>& seed_sets, const std::vector<int64_t>& fanouts,
+    bool replace) {
+  Range range("gs::SampleLayersBatched");
+  Settle();
+  TORCH_CHECK(csc_ != nullptr, "fused slicing + sampling needs the CSC format");
+  const int64_t B = static_cast<int64_t>(seed_sets.size());
+  const int64_t L = static_cast<int64_t>(fanouts.size());
+  std::vector<std::vector<torch::Tensor>> out(B);
+  if (B == 0 || L == 0) return out;
+  // what the one launch sequence cannot take goes minibatch by minibatch
+  bool one_sequence = !col_ids_.has_value() && !row_ids_.has_value() && !val_col_ids_.has_value() &&
+                      hip::DeferredSampling() &&
+                      (!data_.has_value() || hip::EdgeData::Fits(data_.value(), csc_->e_ids));
+  int64_t bound = 0;
+  for (const auto& s : seed_sets) {
+    TORCH_CHECK(s.defined() && s.dim() == 1 && s.device() == csc_->indptr.device() &&
+                    s.scalar_type() == csc_->indices.scalar_type(),
+                "every seed set must be a 1-d tensor of the graph's id type on its device");
+    bound += s.numel();
+  }
+  for (int64_t k : fanouts) {
+    one_sequence = one_sequence && !(k == 1 && replace) && hip::OneLaunchApplies(bound, k, replace);
+    bound *= 1 + k;
+  }
+  if (!one_sequence) {
+    for (int64_t b = 0; b < B; ++b) out[b] = SampleLayers(seed_sets[b], fanouts, replace);
+    return out;
+  }
+  const bool with_data = data_.has_value();
+  const hip::EdgeData edge{with_data ? data_.value() : torch::Tensor(), csc_->e_ids};
+  auto pinned = torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true);
+  std::vector<int64_t> cut(B + 1, 0);
+  for (int64_t b = 0; b < B; ++b) cut[b + 1] = cut[b] + seed_sets[b].numel();
+  auto host_ptr = torch::empty({B + 1}, pinned);
+  std::copy(cut.begin(), cut.end(), host_ptr.data_ptr<int64_t>());
+  torch::Tensor ptr = host_ptr.to(csc_->indptr.device(), /*non_blocking=*/true);
+  torch::Tensor seeds = torch::cat(seed_sets);
+  struct Layer {
+    torch::Tensor frontier, offsets, renamed, data;
+    torch::Tensor cuts;  // pinned: [seed cuts | edge cuts | frontier cuts], B + 1 each
+  };
+  std::vector<Layer> layers(L);
+  for (int64_t l = 0; l < L; ++l) {
+    Layer& y = layers[l];
+    const int64_t S = seeds.numel();
+    auto p = hip::ColSamplingDeferred(csc_->indptr, csc_->indices, seeds, fanouts[l], replace, false,
+                                      false, with_data ? &edge : nullptr);
+    // queued behind the sampler while its edge count is on its way: where every minibatch's
+    // edges start, and the offsets of every minibatch re-based to its own first edge
+    torch::Tensor ids_ptr = p->sub_indptr.index_select(0, ptr);
+    y.offsets = hip::IndptrSplit(p->sub_indptr, ptr, S + B);
+    const int64_t nnz = p->Wait();
+    torch::Tensor ids = hip::Slice1d(p->indices, 0, nnz);
+    if (with_data) y.data = hip::Slice1d(p->data, 0, nnz);
+    torch::Tensor uni_ptr;
+    std::tie(y.frontier, uni_ptr, y.renamed) = hip::BatchCsrRelabel(seeds, ptr, ids, ids_ptr);
+    y.cuts = torch::empty({3 * (B + 1)}, pinned);
+    y.cuts.narrow(0, 0, B + 1).copy_(ptr, /*non_blocking=*/true);
+    y.cuts.narrow(0, B + 1, B + 1).copy_(ids_ptr, /*non_blocking=*/true);
+    y.cuts.narrow(0, 2 * (B + 1), B + 1).copy_(uni_ptr, /*non_blocking=*/true);
+    seeds = y.frontier;
+    ptr = uni_ptr;
+  }
+  // one wait for the cuts of all layers, then views
+  hip::SyncCurrentStream(seeds);
+  for (int64_t b = 0; b < B; ++b) out[b].reserve((with_data ? 4 : 3) * L);
+  for (int64_t l = 0; l < L; ++l) {
+    const Layer& y = layers[l];
+    const int64_t* s_cut = y.cuts.data_ptr<int64_t>();
+    const int64_t* e_cut = s_cut + (B + 1);
+    const int64_t* u_cut = e_cut + (B + 1);
+    for (int64_t b = 0; b < B; ++b) {
+      out[b].push_back(hip::Slice1d(y.frontier, u_cut[b], u_cut[b + 1] - u_cut[b]));
+      out[b].push_back(hip::Slice1d(y.offsets, s_cut[b] + b, s_cut[b + 1] - s_cut[b] + 1));
+      out[b].push_back(hip::Slice1d(y.renamed, e_cut[b], e_cut[b + 1] - e_cut[b]));
+      if (with_data) out[b].push_back(hip::Slice1d(y.data, e_cut[b], e_cut[b + 1] - e_cut[b]));
+    }
+  }
+  return out;
+}
+
 // The reference hands the kernel the GLOBAL ids of the seeds (src/graph.cc:120-128), which
 // only works on a graph without id maps, and gathers the parent's edge data with positions
 // of the virtual column slice (:131-137).  Here the kernel gets the local seeds and edge

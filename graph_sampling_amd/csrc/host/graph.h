@@ -142,6 +142,17 @@ class Graph : public torch::CustomClassHolder {
                                                   bool replace);
   std::vector<torch::Tensor> SampleLayersLoop(torch::Tensor seeds,
                                               const std::vector<int64_t>& fanouts, bool replace);
+  // Many minibatches as ONE launch sequence per layer (a "super-batch", the flow of the
+  // reference's examples/graphsage/batching.py:59-98: fused sampling over the concatenated
+  // seeds, the batches' edge offsets, one relabel per minibatch done in one pass, the splits),
+  // run inside this layer: no interpreter between the launches, two host waits per layer (the
+  // edge count, the frontier length), the per-minibatch cuts read back once at the end.
+  // Returns per seed set what SampleLayers returns; minibatch b draws as row range
+  // [ptr[b], ptr[b+1]) of one sampler call per layer, so its samples differ from those of a
+  // SampleLayers call on the same seeds, while every block is a valid sample of its seeds.
+  std::vector<std::vector<torch::Tensor>> SampleLayersBatched(
+      const std::vector<torch::Tensor>& seed_sets, const std::vector<int64_t>& fanouts,
+      bool replace);
   // induced subgraph: columns column_seeds, rows row_seeds (renamed to their position in
   // row_seeds), CSC only (reference src/graph.cc:116-141)
   c10::intrusive_ptr<Graph> FusedBidirSlicing(torch::Tensor column_seeds, torch::Tensor row_seeds);

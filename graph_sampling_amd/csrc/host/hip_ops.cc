@@ -333,6 +333,22 @@ struct Pieces {
 };
 }  // namespace
 
+void SyncCurrentStream(const torch::Tensor& like) {
+  TORCH_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream(like))) == hipSuccess,
+              "hipStreamSynchronize failed");
+}
+
+torch::Tensor Slice1d(const torch::Tensor& t, int64_t first, int64_t count) {
+  TORCH_CHECK(t.dim() == 1 && t.is_contiguous() && first >= 0 && count >= 0 &&
+                  first + count <= t.numel(),
+              "Slice1d: [", first, ", ", first + count, ") of a 1-d tensor of ", t.numel());
+  auto v = at::detail::make_tensor<c10::TensorImpl>(c10::Storage(t.storage()), t.key_set(), t.dtype());
+  auto* impl = v.unsafeGetTensorImpl();
+  impl->set_storage_offset(t.storage_offset() + first);
+  impl->set_sizes_contiguous({count});
+  return v;
+}
+
 int64_t PendingSample::Wait() const {
   int64_t nnz = WaitBox(static_cast<const gs_mailbox*>(box), ticket, stream, "gs_sample_uniform_fused");
   if (nnz == kLost) nnz = sub_indptr[S].item<int64_t>();

@@ -128,6 +128,12 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
                                                   const torch::Tensor& seeds,
                                                   const std::vector<int64_t>& fanouts,
                                                   bool replace, const EdgeData* edge = nullptr);
+// waits until everything queued on the calling thread's current stream of `like`'s device is done
+void SyncCurrentStream(const torch::Tensor& like);
+// t[first : first + count] of a contiguous 1-d tensor, sharing its storage: what narrow()
+// gives, made without a trip through the operator dispatcher (a super-batch hands back a few
+// hundred such views per call).
+torch::Tensor Slice1d(const torch::Tensor& t, int64_t first, int64_t count);
 // For tests of the recovery path: raises the sticky error word in the look-back state of the
 // calling thread's current stream on `like`'s device, as a tile that gave up waiting would.
 // The next one-launch sampler or relabel on that state reports failure (every kernel still

@@ -363,3 +363,81 @@ def test_batch_relabel_64_bit_ids_narrow_and_fallback(dev):
             lo, hi = int(uni_ptr[b]), int(uni_ptr[b + 1])
             assert np.array_equal(uni[lo:hi].cpu().numpy(), f)
             assert np.array_equal(rel[ids_ptr[b]:ids_ptr[b + 1]].cpu().numpy(), r)
+
+
+def _oracle_super_batch(indptr, indices, seed_sets, fanouts, replace, first_seed, data=None):
+    """The super-batch flow by the oracle: one sampler call per layer over the concatenated seeds
+    (row r of the call draws as row r), one relabel per minibatch, next seeds = the frontiers."""
+    sizes = [s.size for s in seed_sets]
+    seeds = np.concatenate(seed_sets).astype(np.int64) if seed_sets else np.empty(0, np.int64)
+    sp = _ptr(sizes)
+    out = [[] for _ in seed_sets]
+    for l, k in enumerate(fanouts):
+        sub_ptr, _, rows, sel = O.sample_uniform(indptr, indices, seeds, k, replace,
+                                                 seed=first_seed + l, with_coo=False)
+        ip = sub_ptr[sp]
+        uni, uni_ptr, rel = O.batch_csr_relabel(seeds, sp, rows, ip)
+        for b in range(len(seed_sets)):
+            out[b] += [uni[uni_ptr[b]:uni_ptr[b + 1]], sub_ptr[sp[b]:sp[b + 1] + 1] - sub_ptr[sp[b]],
+                       rel[ip[b]:ip[b + 1]]]
+            if data is not None:
+                out[b].append(data[sel][ip[b]:ip[b + 1]])
+        seeds, sp = uni, uni_ptr
+    return out
+
+
+@pytest.mark.parametrize("idt", ID_DTYPES)
+@pytest.mark.parametrize("with_data", [False, True])
+@pytest.mark.parametrize("sizes,fanouts,replace", [([300, 0, 1, 1024, 77], (4, 3), False),
+                                                   ([1024] * 64, (15, 10), False),
+                                                   ([50, 60], (3, 3, 3), True)])
+def test_sample_layers_batched_equals_the_oracle_flow(dev, idt, with_data, sizes, fanouts, replace):
+    """_CAPI_SampleLayersBatched (the super-batch flow inside the C++ layer: fused sampling over
+    the concatenated seeds, the batches' edge cuts, one relabel per minibatch in one pass -- through
+    the bins from 2^19 items on --, the per-minibatch views) against the oracle doing the same."""
+    import graph_sampling_amd as gs
+    n = 1 << 15
+    indptr, indices = rmat_csc_np(n, 1 << 20, seed=41)
+    rng = np.random.default_rng(len(sizes))
+    data = (1.0 - rng.random(indices.size)).astype(np.float32) if with_data else None
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev, idt))
+    if with_data:
+        g._CAPI_SetData(to_dev(data, dev))
+    seed_sets = [rng.permutation(n)[:s].astype(np.int64) for s in sizes]
+    for first in (700, 710):
+        gs.set_seed(first)
+        got = g._CAPI_SampleLayersBatched([to_dev(s, dev, idt) for s in seed_sets], list(fanouts),
+                                          replace)
+        want = _oracle_super_batch(indptr, indices, seed_sets, fanouts, replace, first, data)
+        assert len(got) == len(want)
+        for b, (g_b, w_b) in enumerate(zip(got, want)):
+            assert len(g_b) == len(w_b)
+            for j, (x, y) in enumerate(zip(g_b, w_b)):
+                if y.dtype == np.float32:
+                    assert np.array_equal(x.cpu().numpy(), y), (b, j)
+                else:
+                    assert np.array_equal(_np(x), y), (b, j)
+    # the Python helper hands back blocks, innermost layer first
+    gs.set_seed(700)
+    res = gs.sample_blocks_batched(g, [to_dev(s, dev, idt) for s in seed_sets], fanouts, replace)
+    want = _oracle_super_batch(indptr, indices, seed_sets, fanouts, replace, 700, data)
+    nodes, blocks = res[0]
+    assert np.array_equal(_np(nodes), want[0][-(4 if with_data else 3)])
+    assert blocks[-1].num_dst_nodes() == sizes[0]
+
+
+def test_sample_layers_batched_on_a_graph_with_id_maps_goes_minibatch_by_minibatch(dev):
+    import graph_sampling_amd as gs
+    indptr, indices = rmat_csc_np(1 << 12, 1 << 16, seed=13)
+    col_ids = np.random.default_rng(1).permutation(1 << 12).astype(np.int64)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSCWithColIds(to_dev(col_ids, dev), to_dev(indptr, dev), to_dev(indices, dev))
+    sets = [to_dev(np.arange(100, dtype=np.int64), dev), to_dev(np.arange(50, 90, dtype=np.int64), dev)]
+    gs.set_seed(5)
+    got = g._CAPI_SampleLayersBatched(sets, [4], False)
+    gs.set_seed(5)
+    want = [g._CAPI_SampleLayers(s, [4], False) for s in sets]
+    for a, b in zip(got, want):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
