@@ -655,7 +655,7 @@ namespace {
 thread_local bool t_chain_ids_fit = true;
 // the chain's launches and tables are sized for the bounds S * prod(1 + fanout); beyond this
 // many items per layer the layer-by-layer path, which sizes by what was sampled, is used
-constexpr int64_t kChainMaxItems = int64_t(1) << 23;
+constexpr int64_t kChainMaxItems = int64_t(1) << 24;  // (8192 seeds x [15, 10, 5] is 8.65 M)
 
 // the two tables a chain uses in turn (a layer's relabel empties the table of the layer
 // before it), one pair per (thread, device, stream); a chain in flight holds on to its pair

@@ -1025,6 +1025,24 @@ def test_fused_sampling_settles_its_edge_data_whichever_method_comes_first(dev):
         assert sub._CAPI_GetNumEdges() == sel.size
 
 
+def test_sample_layers_keeps_8192_seeds_on_the_queued_path(dev):
+    """8192 seeds x [15, 10, 5]: bounds of 8.65 M items in the third layer, which the queued chain
+    takes (its limit is 2^24 items); the result is the oracle's, and _CAPI_SampleLayersIfQueued
+    answers (an empty list would mean the loop)."""
+    n = 1 << 17
+    indptr, indices = rmat_csc_np(n, 1 << 21, seed=3)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev, torch.int32))
+    seeds = np.random.default_rng(1).permutation(n)[:8192].astype(np.int64)
+    gs.set_seed(90)
+    got = g._CAPI_SampleLayersIfQueued(to_dev(seeds, dev, torch.int32), [15, 10, 5], False)
+    assert len(got) == 9
+    _same(got, _oracle_minibatch(indptr, indices, seeds, (15, 10, 5), False, 90))
+    # and one seed more than the bound allows goes layer by layer, with the same result shape
+    many = np.random.default_rng(2).permutation(n)[:16000].astype(np.int64)
+    assert g._CAPI_SampleLayersIfQueued(to_dev(many, dev, torch.int32), [15, 10, 5], False) == []
+
+
 @pytest.mark.parametrize("idt", [torch.int32, torch.int64])
 def test_sample_layers_with_no_seeds_and_with_isolated_seeds(dev, idt):
     """No seeds at all, and seeds without neighbours (every later layer is then empty too):
