@@ -863,13 +863,17 @@ SUPER_SITES = {
 
 
 # ---------------------------------------------------------------------------------------
-def make_ladies_sampler(torch):
+def make_ladies_sampler(torch, seen_probs=None):
+    """`seen_probs` (a list): the run's row probabilities are appended to it, layer by layer,
+    for the checker (they are sums by float atomics: another run's differ in the last bits)."""
     def ladies_sampler(A, seeds, fanouts):
         """The sampler of examples/ladies/ladies_raw.py:8-27, written against Matrix."""
         ret = []
         for fanout in fanouts:
             U = A[:, seeds]
             prob = U.sum(axis=1, powk=2)
+            if seen_probs is not None:
+                seen_probs.append(prob)
             selected, _ = torch.ops.gs_ops.list_sampling_with_probs(U.row_ids(unique=False), prob,
                                                                     fanout, False)
             nodes = torch.cat((seeds, selected)).unique()
@@ -945,7 +949,8 @@ def ladies(cx, cpu_budget):
         for s in sets[:warm]:
             fn(A, s, PICKS)
         gs.set_seed(first_seed)
-        first = fn(A, sets[warm], PICKS)
+        seen = []
+        first = (make_ladies_sampler(torch, seen) if name == "as_written" else fn)(A, sets[warm], PICKS)
         gs.set_seed(first_seed)
         e, t = timed(torch, lambda s: edges_of(fn(A, s, PICKS)), sets[warm:])
         out[name] = {"ms_per_step": t / steps * 1e3, "value": e / t, "unit": "block edges/s"}
@@ -954,17 +959,9 @@ def ladies(cx, cpu_budget):
             h_indices = indices.cpu().numpy().astype(np.int64)
             h_w = weights.cpu().numpy()
             h_seeds = sets[warm].cpu().numpy().astype(np.int64)
-            # the device's row probabilities decide the picks (they differ from the oracle's in
-            # the last bits, float sums in another order): recomputed here stage by stage
-            probs, cols = [], sets[warm]
-            gs.set_seed(first_seed)
-            for l, k in enumerate(PICKS):
-                U = A[:, cols]
-                prob = U.sum(axis=1, powk=2)
-                probs.append(prob.cpu().numpy())
-                picked, _ = torch.ops.gs_ops.list_sampling_with_probs(U.row_ids(unique=False), prob,
-                                                                      k, False)
-                cols = U[torch.cat((cols, picked)).unique(), :].all_indices()
+            # the checked run's own row probabilities decide the oracle's picks (they differ
+            # from the oracle's in the last bits: float sums in another order)
+            probs = [p.cpu().numpy() for p in seen]
             want = cpu_ladies(O, np, h_indptr, h_indices, h_w, h_seeds, PICKS, first_seed, probs)
             bad = []
             for l, (frontier, rel_row, rel_col, w_norm, prob) in enumerate(want):

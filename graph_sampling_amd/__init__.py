@@ -53,6 +53,15 @@ def set_seed(seed):
     torch.ops.gs_ops._CAPI_SetSeed(int(seed))
 
 
+def set_ordered_sums(on):
+    """on: `sum(axis)` of a matrix held as a COO only sorts its edges first and adds in edge
+    order, so two runs give the same bits; off (the default): it adds edge by edge with float
+    atomics, faster, and a sum of three or more addends may differ in its last bit run to run."""
+    import torch
+    load_library()
+    torch.ops.gs_ops._CAPI_SetOrderedSums(bool(on))
+
+
 def _blocks_of(parts, num_layers):
     from .block import Block
     blocks = []

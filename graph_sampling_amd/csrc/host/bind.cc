@@ -19,6 +19,7 @@ namespace {
 void SetSeed(int64_t seed) { hip::SetSeed(static_cast<uint64_t>(seed)); }
 void SetThreadSeed(int64_t seed) { hip::SetThreadSeed(static_cast<uint64_t>(seed)); }
 void SetSampleAlgo(int64_t algo) { hip::SetSampleAlgo(algo); }
+void SetOrderedSums(bool on) { hip::SetOrderedSums(on); }
 void SetDeferredSampling(bool on) { hip::SetDeferredSampling(on); }
 void DebugRaiseLookbackError(torch::Tensor like) { hip::DebugRaiseLookbackError(like); }
 torch::Tensor UniqueOp(torch::Tensor ids) { return TensorUnique(ids); }
@@ -147,6 +148,9 @@ TORCH_LIBRARY(gs_ops, m) {
   m.def("_CAPI_SetThreadSeed", &SetThreadSeed);
   m.def("_CAPI_SampleBlocks", &SampleBlocks);
   m.def("_CAPI_SetSampleAlgo", &SetSampleAlgo);
+  // not in the reference: on = float sums of a COO-only graph add in edge order (same bits
+  // every run) at the price of sorting its edges first
+  m.def("_CAPI_SetOrderedSums", &SetOrderedSums);
   // not in the reference: off = every sampling call settles its edge count before returning
   m.def("_CAPI_SetDeferredSampling", &SetDeferredSampling);
   // not in the reference: test hook for the recovery from a look-back that gave up

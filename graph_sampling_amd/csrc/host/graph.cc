@@ -239,6 +239,10 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
   Range range("gs::Slicing");
   Settle();
   TORCH_CHECK(axis == 0 || axis == 1, "axis must be 0 (columns) or 1 (rows)");
+  if (axis == 1 && on_format == _CSR && output_format == _COO && !relabel) {
+    auto sliced = RowSliceOfCoo(n_ids);
+    if (sliced) return sliced;
+  }
   CreateSparseFormat(on_format);
   const bool with_coo = output_format & _COO;
   torch::optional<torch::Tensor> new_val_cols, new_val_rows;
@@ -338,6 +342,40 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
   if (out_csc) ret->val_col_ids_ = new_val_cols;
   if (out_csr) ret->val_row_ids_ = new_val_rows;
   InheritData(ret.get(), e_ids, select_index);
+  return ret;
+}
+
+// Rows n_ids of a graph that is held as a COO only (a column slice, as `U[nodes, :]` of the
+// layer-wise samplers meets it: python/gs/matrix_api/matrix.py:104-105), without the CSR the
+// reference builds of the whole slice first (src/graph.cc:258-283, a sort of every edge): the
+// edges are filtered by the id set, and only the kept ones are sorted by their new row.  The
+// filter keeps the COO's order and the sort is stable, so the result holds the same edges in
+// the same order as the CSR and its slice give.  Only for ids that are strictly increasing
+// (distinct: a row asked for twice appears twice in the reference's result); returns null
+// when it does not apply, and the caller goes the reference's way.
+c10::intrusive_ptr<Graph> Graph::RowSliceOfCoo(const torch::Tensor& n_ids) {
+  if (csr_ || spare_csr_ || !coo_ || val_row_ids_.has_value() || n_ids.numel() == 0 ||
+      coo_->row.numel() == 0)
+    return nullptr;
+  torch::Tensor increasing;  // device flag, read together with the count of kept edges
+  if (n_ids.numel() > 1)
+    increasing = (n_ids.narrow(0, 1, n_ids.numel() - 1) > n_ids.narrow(0, 0, n_ids.numel() - 1)).all();
+  torch::Tensor new_row, cols, select_index;
+  bool distinct = true;
+  std::tie(new_row, cols, select_index) =
+      hip::RowSlicingCoo(coo_->row, coo_->col, n_ids, increasing.defined() ? &increasing : nullptr,
+                         &distinct);
+  if (!distinct) return nullptr;
+  torch::Tensor indptr, sorted_cols;
+  torch::optional<torch::Tensor> perm;
+  std::tie(indptr, sorted_cols, perm) = hip::Coo2Csc(new_row, cols, n_ids.numel(), false);
+  if (perm.has_value()) select_index = select_index.index({perm.value()});
+  auto ret = Child(col_ids_, Pick(row_ids_, n_ids), num_cols_, n_ids.numel());
+  ret->SetNumEdges(sorted_cols.numel());
+  ret->SetCOO(std::make_shared<COO>(COO{hip::Csc2CooCols(indptr, sorted_cols.numel(), sorted_cols),
+                                        sorted_cols, torch::nullopt, true, false}));
+  ret->spare_csr_ = std::make_shared<CSR>(CSR{indptr, sorted_cols, torch::nullopt});
+  InheritData(ret.get(), coo_->e_ids, select_index);
   return ret;
 }
 
@@ -722,6 +760,16 @@ torch::Tensor Graph::RandomWalk(torch::Tensor seeds, int64_t walk_length) {
 torch::Tensor Graph::Sum(int64_t axis, int64_t powk, int64_t on_format) {
   Range range("gs::Sum");
   Settle();
+  // Sums along the rows (columns) of a graph held as a COO only are added up by edge, straight
+  // off the COO, instead of sorting every edge into a CSR (CSC) first: the row probabilities
+  // of a layer-wise sampler's column slice are 2.8 M edges over 2.45 M rows.  The same sums,
+  // the order of the float additions aside (as on the reference's own COO path, which adds
+  // with atomics, src/cuda/graph_ops.cu:45-64).
+  // hip::SetOrderedSums(true) keeps the sorted route, whose sums are the same bits every run.
+  if (!hip::OrderedSums() &&
+      ((axis == 1 && on_format == _CSR && !csr_ && !spare_csr_ && coo_ && !val_row_ids_.has_value()) ||
+       (axis == 0 && on_format == _CSC && !csc_ && !spare_csc_ && coo_ && !val_col_ids_.has_value())))
+    on_format = _COO;
   CreateSparseFormat(on_format);
   torch::Tensor data = DataOrOnes();
   // one entry per column (axis 0) / row (axis 1) OF THIS GRAPH OBJECT, so a

@@ -208,6 +208,7 @@ class Graph : public torch::CustomClassHolder {
   torch::TensorOptions IdOptions() const;
   void InheritData(Graph* child, const torch::optional<torch::Tensor>& e_ids,
                    const torch::Tensor& select_index) const;
+  c10::intrusive_ptr<Graph> RowSliceOfCoo(const torch::Tensor& n_ids);
   c10::intrusive_ptr<Graph> SampleImpl(int64_t axis, const torch::Tensor* edge_probs,
                                        int64_t fanout, bool replace, int64_t on_format,
                                        int64_t output_format);

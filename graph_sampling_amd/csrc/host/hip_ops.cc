@@ -233,6 +233,12 @@ void SetThreadSeed(uint64_t seed) {
   t_seed = seed;
 }
 uint64_t NextSeed() { return t_own_seed ? t_seed++ : g_seed.fetch_add(1); }
+
+namespace {
+std::atomic<bool> g_ordered_sums{false};
+}
+void SetOrderedSums(bool on) { g_ordered_sums.store(on); }
+bool OrderedSums() { return g_ordered_sums.load(); }
 void SetSampleAlgo(int64_t algo) {
   TORCH_CHECK(algo == GS_SAMPLE_AUTO || algo == GS_SAMPLE_RESERVOIR, "unknown sampling algorithm ", algo);
   g_algo.store(algo);
@@ -1072,9 +1078,9 @@ SliceResult RowSlicingCsc(const torch::Tensor& indptr, const torch::Tensor& indi
   return {out_indptr, coo_col, out_indices, select_index};
 }
 
-std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(const torch::Tensor& key,
-                                                                      const torch::Tensor& other,
-                                                                      const torch::Tensor& ids) {
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(
+    const torch::Tensor& key, const torch::Tensor& other, const torch::Tensor& ids,
+    const torch::Tensor* flag, bool* flag_value) {
   const int idb = IdBytes(key, "coo ids");
   TORCH_CHECK(IdBytes(other, "coo ids") == idb && IdBytes(ids, "node ids") == idb,
               "coo ids and node ids differ in dtype");
@@ -1085,7 +1091,15 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(const torc
   Check(gs_row_slice_coo_mark(key.data_ptr(), idb, E, ids.data_ptr(), n, num.data_ptr<int64_t>(),
                               ws.data_ptr(), ws.numel(), st),
         "gs_row_slice_coo_mark");
-  const int64_t kept = num.item<int64_t>();
+  int64_t kept;
+  if (flag) {
+    auto both = torch::stack({num.reshape({}), flag->to(torch::kInt64).reshape({})}).cpu();
+    kept = both.data_ptr<int64_t>()[0];
+    *flag_value = both.data_ptr<int64_t>()[1] != 0;
+    if (!*flag_value) return {torch::Tensor(), torch::Tensor(), torch::Tensor()};
+  } else {
+    kept = num.item<int64_t>();
+  }
   auto out_key = torch::empty({kept}, key.options());
   auto out_other = torch::empty({kept}, key.options());
   auto select_index = torch::empty({kept}, I64(key));

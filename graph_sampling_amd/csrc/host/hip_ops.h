@@ -28,6 +28,12 @@ void SetSeed(uint64_t seed);
 // not depend on how they interleave.
 void SetThreadSeed(uint64_t seed);
 uint64_t NextSeed();
+// off (default): Graph::Sum along the rows (columns) of a graph held as a COO only adds edge
+// by edge with float atomics, so a sum of three or more addends can differ in its last bit
+// from run to run (as on the reference's COO path, src/cuda/graph_ops.cu:45-64).  on: such a
+// sum goes through the sorted format and adds in edge order, the same bits every run.
+void SetOrderedSums(bool on);
+bool OrderedSums();
 // 0: Floyd selection for deg > fanout (default), 1: the reference's Algorithm R.
 void SetSampleAlgo(int64_t algo);
 
@@ -196,10 +202,13 @@ void EDivUSum(const torch::Tensor& row, const torch::Tensor& col, const torch::T
 
 SliceResult RowSlicingCsc(const torch::Tensor& indptr, const torch::Tensor& indices,
                           const torch::Tensor& row_ids, bool with_coo);
-// {relabelled key, other, select_index}
-std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(const torch::Tensor& key,
-                                                                      const torch::Tensor& other,
-                                                                      const torch::Tensor& ids);
+// {relabelled key, other, select_index}.  `flag` (a device scalar of any integer / bool type,
+// or null) is read back in the same transfer as the count of kept edges and lands in
+// *flag_value: a caller's own device-side check at no extra host wait; when it reads false the
+// compaction is skipped and the three tensors come back undefined.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(
+    const torch::Tensor& key, const torch::Tensor& other, const torch::Tensor& ids,
+    const torch::Tensor* flag = nullptr, bool* flag_value = nullptr);
 
 // Induced-subgraph slice (columns column_ids, rows in row_ids) without writing the column
 // slice: {out_indptr, out_indices, select_index, parent_index}.  select_index counts

@@ -523,6 +523,63 @@ def test_ladies_flow_matches_oracle(dev):
     assert np.array_equal(block.edges()[1].cpu().numpy(), rel_col)
 
 
+@pytest.mark.parametrize("ids", ["increasing", "shuffled", "repeated"])
+def test_row_slice_of_a_column_slice_is_the_same_by_filter_and_by_sorted_rows(dev, ids):
+    """`U[nodes, :]` of a column slice (a COO) filters the COO and sorts the kept edges when the
+    ids increase, and goes through the CSR of all of U otherwise (or when ordered sums have
+    built that CSR): the same edges in the same order with the same data, and both equal the
+    oracle's row slice of U's CSR (src/graph.cc:258-283)."""
+    m, indptr, indices, data = _rmat_matrix(dev, 12, 16, 9, with_data=True)
+    N = 1 << 12
+    rng = np.random.default_rng(3)
+    seeds = rng.permutation(N)[:200].astype(np.int64)
+    nodes = np.sort(rng.permutation(N)[:700]).astype(np.int64)
+    if ids == "shuffled":
+        nodes = rng.permutation(nodes)
+    elif ids == "repeated":
+        nodes = np.sort(np.concatenate([nodes, nodes[:50]]))
+    sp, coo, si, sel = O.slice_columns(indptr, indices, seeds)
+    r_ip, r_col, r_perm = O.coo2csc(si, coo, N, False)
+    s_ip, s_row, s_col, s_sel = O.slice_columns(r_ip, r_col, nodes)
+    got = []
+    for ordered in (False, True):
+        gs.set_ordered_sums(ordered)
+        try:
+            U = m[:, to_dev(seeds, dev)]
+            U.sum(axis=1)  # ordered: builds the CSR of U, which the slice then uses
+            sub = U[to_dev(nodes, dev), :]
+        finally:
+            gs.set_ordered_sums(False)
+        assert sub.get_num_rows() == nodes.size and sub.get_num_edges() == s_col.size
+        assert np.array_equal(sub.get_data().cpu().numpy(), data[sel][r_perm][s_sel])
+        block = sub.to_dgl_block()
+        got.append([t.cpu().numpy() for t in (block.srcdata["_ID"], *block.edges(), block.edata["w"])])
+    for a, b in zip(*got):
+        assert np.array_equal(a, b)
+
+
+def test_sum_over_the_rows_of_a_column_slice_adds_edge_by_edge_or_in_order(dev):
+    """`U.sum(axis=1)` of a column slice held as a COO adds straight off the COO (float atomics)
+    unless ordered sums are on (CSR of U, one row after the other): the oracle's sums to 1e-5
+    either way, and with ordered sums the same bits on every run."""
+    m, indptr, indices, data = _rmat_matrix(dev, 14, 19, 6, with_data=True)
+    N = 1 << 14
+    seeds = np.random.default_rng(8).permutation(N)[:6000].astype(np.int64)
+    sp, coo, si, sel = O.slice_columns(indptr, indices, seeds)
+    assert si.size >= 1 << 17  # enough edges for the sum through bins
+    want = O.coo_sum(si, None, data[sel], 2, N)
+    runs = []
+    for ordered in (False, True, True):
+        gs.set_ordered_sums(ordered)
+        try:
+            prob = m[:, to_dev(seeds, dev)].sum(axis=1, powk=2)
+        finally:
+            gs.set_ordered_sums(False)
+        np.testing.assert_allclose(prob.cpu().numpy(), want, rtol=1e-5)
+        runs.append(prob)
+    assert torch.equal(runs[1], runs[2])
+
+
 def test_fastgcn_coo_row_slicing_flow(dev):
     """examples/fastgcn/unbatching_training.py:18-31: _CAPI_slicing(selected, 1, _COO, _COO, False)."""
     m, indptr, indices, _ = _rmat_matrix(dev, 11, 15, 5)
