@@ -37,9 +37,10 @@ def lib():
                      "gs_relabel_sampled_workspace_bytes", "gs_relabel_sampled_state_bytes",
                      "gs_segment_workspace_bytes", "gs_layer_workspace_bytes",
                      "gs_layer_sample_state_bytes", "gs_layer_relabel_state_bytes",
-                     "gs_coo_sum_workspace_bytes"):
+                     "gs_coo_sum_workspace_bytes", "gs_coo_pick_rows_workspace_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
+        _lib.gs_sorted_union_max.restype = ctypes.c_int64
     return _lib
 
 
@@ -825,6 +826,59 @@ def index_search(data, keys):
                                  _ptr(out), _ptr(ws), ctypes.c_size_t(ws.numel()),
                                  _stream(data.device)), "gs_index_search")
     return out
+
+
+# ------------------------------------------------- layer-wise sampler tail ----
+def sorted_union_max(id_bytes):
+    return int(lib().gs_sorted_union_max(int(id_bytes)))
+
+
+def sorted_union(a, b):
+    """gs_sorted_union.  Returns (out with room for len(a) + len(b), count: device int64[1])."""
+    idb = _ids(a, "a")
+    _ids(b, "b", like=a)
+    out = torch.empty(a.numel() + b.numel(), dtype=a.dtype, device=a.device)
+    count = torch.empty(1, dtype=torch.int64, device=a.device)
+    _check(lib().gs_sorted_union(_ptr(a), _i64(a.numel()), _ptr(b), _i64(b.numel()), idb, _ptr(out),
+                                 _ptr(count), _stream(a.device)), "gs_sorted_union")
+    return out, count
+
+
+def coo_pick_rows(row, col, nodes, count, max_nodes):
+    """gs_coo_pick_rows.  Returns (kept_key, kept_pos, totals: device int64[2])."""
+    idb = _ids(row, "row")
+    _ids(col, "col", like=row)
+    _ids(nodes, "nodes", like=row)
+    _need(count, torch.int64, "count")
+    E = row.numel()
+    key = torch.empty(E, dtype=row.dtype, device=row.device)
+    pos = torch.empty(E, dtype=row.dtype, device=row.device)
+    totals = torch.empty(2, dtype=torch.int64, device=row.device)
+    ws = workspace(lib().gs_coo_pick_rows_workspace_bytes(_i64(E)), row.device)
+    _check(lib().gs_coo_pick_rows(_ptr(row), _ptr(col), idb, _i64(E), _ptr(nodes), _ptr(count),
+                                  _i64(max_nodes), _ptr(key), _ptr(pos), _ptr(totals), _ptr(ws),
+                                  ctypes.c_size_t(ws.numel()), _stream(row.device)),
+           "gs_coo_pick_rows")
+    return key, pos, totals
+
+
+def coo_block_values(kept_key, kept_pos, max_nodes, row, data, divisor, num_cols):
+    """gs_coo_block_values.  Returns (out_row, out_value, out_indptr)."""
+    idb = _ids(row, "row")
+    _ids(kept_key, "kept_key", like=row)
+    _ids(kept_pos, "kept_pos", like=row)
+    _need(divisor, torch.float32, "divisor")
+    if data is not None:
+        _need(data, torch.float32, "data")
+    kept = kept_key.numel()
+    out_row = torch.empty(kept, dtype=row.dtype, device=row.device)
+    out_value = torch.empty(kept, dtype=torch.float32, device=row.device)
+    out_indptr = torch.empty(num_cols + 1, dtype=torch.int64, device=row.device)
+    _check(lib().gs_coo_block_values(_ptr(kept_key), _ptr(kept_pos), _i64(kept), _i64(max_nodes),
+                                     _ptr(row), idb, _ptr(data), _ptr(divisor), _i64(num_cols),
+                                     _ptr(out_row), _ptr(out_value), _ptr(out_indptr),
+                                     _stream(row.device)), "gs_coo_block_values")
+    return out_row, out_value, out_indptr
 
 
 # ------------------------------------------------------------------ walks ----

@@ -104,13 +104,14 @@ constexpr int kFillItems = 8;
 constexpr int kFillTile = kFillThreads * kFillItems;
 constexpr int kFillStage = 1024;  // rows of offsets staged in LDS
 
-template <typename IdT, bool WITH_COO>
+template <typename IdT, bool WITH_COO, bool WITH_DATA>
 __global__ void __launch_bounds__(kFillThreads)
 slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
                   const IdT* __restrict__ cols, int64_t num_cols, int64_t S,
                   const int64_t* __restrict__ sub_indptr,
                   int64_t nnz, IdT* __restrict__ sub_indices, int64_t* __restrict__ select_index,
-                  IdT* __restrict__ coo_col) {
+                  IdT* __restrict__ coo_col, const float* __restrict__ edge_data,
+                  const int64_t* __restrict__ edge_ids, float* __restrict__ data_out) {
   __shared__ int64_t s_ptr[kFillStage + 1];
   __shared__ int64_t s_in[kFillStage];
   __shared__ int64_t s_rows[2];
@@ -151,6 +152,20 @@ slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ in
   IdT v[kFillItems];
 #pragma unroll
   for (int k = 0; k < kFillItems; ++k) v[k] = indices[q[k]];
+  // the edges' data along with them (what the reference gathers afterwards from
+  // select_index, src/graph.cc:68-73): data[e_ids ? e_ids[q] : q]
+  float w[kFillItems];
+  if (WITH_DATA) {
+    int64_t at[kFillItems];
+#pragma unroll
+    for (int k = 0; k < kFillItems; ++k) at[k] = q[k];
+    if (edge_ids) {
+#pragma unroll
+      for (int k = 0; k < kFillItems; ++k) at[k] = edge_ids[q[k]];
+    }
+#pragma unroll
+    for (int k = 0; k < kFillItems; ++k) w[k] = edge_data[at[k]];
+  }
 #pragma unroll
   for (int k = 0; k < kFillItems; ++k) {
     const int64_t p = p0 + k * kFillThreads + threadIdx.x;
@@ -158,6 +173,7 @@ slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ in
       sub_indices[p] = v[k];
       if (select_index) select_index[p] = q[k];
       if (WITH_COO) coo_col[p] = static_cast<IdT>(row[k]);
+      if (WITH_DATA) data_out[p] = w[k];
     }
   }
 }
@@ -477,24 +493,43 @@ int slice_count_impl(const int64_t* indptr, int64_t num_cols, const void* cols, 
   return exclusive_scan(f, S, sub_indptr, tile_ws, stream);
 }
 
+template <typename IdT, bool WITH_COO, bool WITH_DATA>
+void slice_fill_launch(const int64_t* indptr, int64_t num_cols, const void* indices,
+                       const void* cols, int64_t S, const int64_t* sub_indptr, int64_t nnz,
+                       void* sub_indices, int64_t* select_index, void* coo_col,
+                       const float* edge_data, const int64_t* edge_ids, float* data_out,
+                       hipStream_t stream) {
+  const unsigned grid = static_cast<unsigned>((nnz + kFillTile - 1) / kFillTile);
+  hipLaunchKernelGGL((slice_fill_kernel<IdT, WITH_COO, WITH_DATA>), dim3(grid), dim3(kFillThreads),
+                     0, stream, indptr, static_cast<const IdT*>(indices),
+                     static_cast<const IdT*>(cols), num_cols, S, sub_indptr, nnz,
+                     static_cast<IdT*>(sub_indices), select_index, static_cast<IdT*>(coo_col),
+                     edge_data, edge_ids, data_out);
+}
+
 template <typename IdT>
 int slice_fill_impl(const int64_t* indptr, int64_t num_cols, const void* indices,
                     const void* cols, int64_t S, const int64_t* sub_indptr, int64_t nnz,
-                    void* sub_indices,
-                    int64_t* select_index, void* coo_col, hipStream_t stream) {
+                    void* sub_indices, int64_t* select_index, void* coo_col,
+                    const float* edge_data, const int64_t* edge_ids, float* data_out,
+                    hipStream_t stream) {
   if (nnz == 0) return GS_OK;
-  const unsigned grid = static_cast<unsigned>((nnz + kFillTile - 1) / kFillTile);
-  if (coo_col) {
-    hipLaunchKernelGGL((slice_fill_kernel<IdT, true>), dim3(grid), dim3(kFillThreads), 0, stream,
-                       indptr, static_cast<const IdT*>(indices), static_cast<const IdT*>(cols),
-                       num_cols, S, sub_indptr, nnz, static_cast<IdT*>(sub_indices), select_index,
-                       static_cast<IdT*>(coo_col));
-  } else {
-    hipLaunchKernelGGL((slice_fill_kernel<IdT, false>), dim3(grid), dim3(kFillThreads), 0, stream,
-                       indptr, static_cast<const IdT*>(indices), static_cast<const IdT*>(cols),
-                       num_cols, S, sub_indptr, nnz, static_cast<IdT*>(sub_indices), select_index,
-                       static_cast<IdT*>(nullptr));
-  }
+  if (coo_col && data_out)
+    slice_fill_launch<IdT, true, true>(indptr, num_cols, indices, cols, S, sub_indptr, nnz,
+                                       sub_indices, select_index, coo_col, edge_data, edge_ids,
+                                       data_out, stream);
+  else if (coo_col)
+    slice_fill_launch<IdT, true, false>(indptr, num_cols, indices, cols, S, sub_indptr, nnz,
+                                        sub_indices, select_index, coo_col, edge_data, edge_ids,
+                                        data_out, stream);
+  else if (data_out)
+    slice_fill_launch<IdT, false, true>(indptr, num_cols, indices, cols, S, sub_indptr, nnz,
+                                        sub_indices, select_index, coo_col, edge_data, edge_ids,
+                                        data_out, stream);
+  else
+    slice_fill_launch<IdT, false, false>(indptr, num_cols, indices, cols, S, sub_indptr, nnz,
+                                         sub_indices, select_index, coo_col, edge_data, edge_ids,
+                                         data_out, stream);
   return check_launch("slice_fill");
 }
 
@@ -1271,18 +1306,30 @@ int gs_slice_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
                   const void* column_ids, int id_bytes, int64_t S, const int64_t* sub_indptr,
                   int64_t nnz, void* sub_indices, int64_t* select_index, void* coo_col,
                   void* stream) {
+  return gs_slice_fill_data(indptr, num_cols, indices, column_ids, id_bytes, S, sub_indptr, nnz,
+                            sub_indices, select_index, coo_col, nullptr, nullptr, nullptr, stream);
+}
+
+int gs_slice_fill_data(const int64_t* indptr, int64_t num_cols, const void* indices,
+                       const void* column_ids, int id_bytes, int64_t S, const int64_t* sub_indptr,
+                       int64_t nnz, void* sub_indices, int64_t* select_index, void* coo_col,
+                       const float* edge_data, const int64_t* edge_ids, float* data_out,
+                       void* stream) {
   GS_REQUIRE(indptr && sub_indptr && S >= 0 && nnz >= 0 && num_cols >= 0,
              "gs_slice_fill: null pointer or negative size");
   GS_REQUIRE(nnz == 0 || (indices && column_ids && sub_indices),
              "gs_slice_fill: null buffer with nnz > 0");
+  GS_REQUIRE(edge_data ? (data_out != nullptr || nnz == 0) : (!data_out && !edge_ids),
+             "gs_slice_fill: edge_data, its output and the edge-id map go together");
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_slice_fill: id_bytes must be 4 or 8, got %d", id_bytes);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!edge_data) data_out = nullptr;
   return id_bytes == 8 ? slice_fill_impl<int64_t>(indptr, num_cols, indices, column_ids, S,
                                                   sub_indptr, nnz, sub_indices, select_index,
-                                                  coo_col, st)
+                                                  coo_col, edge_data, edge_ids, data_out, st)
                        : slice_fill_impl<int32_t>(indptr, num_cols, indices, column_ids, S,
                                                   sub_indptr, nnz, sub_indices, select_index,
-                                                  coo_col, st);
+                                                  coo_col, edge_data, edge_ids, data_out, st);
 }
 
 size_t gs_sample_workspace_bytes(int64_t S, int64_t fanout) {

@@ -285,6 +285,17 @@ long_segments_kernel(const int64_t* __restrict__ indptr, const int64_t* __restri
         const float4 v = *reinterpret_cast<const float4*>(data + begin + t * kStep + lane * kLaneEdges);
         acc += (powk_f(v.x, powk) + powk_f(v.y, powk)) + (powk_f(v.z, powk) + powk_f(v.w, powk));
       }
+    } else if (end - begin == kChunk) {
+      // the same additions in the same order through an edge map (or from unaligned data), so
+      // that a sum does not depend on which of its layouts a graph holds
+#pragma unroll
+      for (int t = 0; t < kChunk / kStep; ++t) {
+        const int64_t e = begin + t * kStep + lane * kLaneEdges;
+        float v[kLaneEdges];
+#pragma unroll
+        for (int k = 0; k < kLaneEdges; ++k) v[k] = powk_f(data[emap ? emap[e + k] : e + k], powk);
+        acc += (v[0] + v[1]) + (v[2] + v[3]);
+      }
     } else {
       for (int64_t e = begin + lane; e < end; e += kWave)
         acc += powk_f(data[emap ? emap[e] : e], powk);

@@ -47,6 +47,8 @@ TORCH_LIBRARY(gs_classes, m) {
       // not in the reference: its super-batch flow (examples/graphsage/batching.py:59-98) as one call
       GS_DEF2("_CAPI_SampleLayersBatched", "_CAPI_sample_layers_batched",
               &Graph::SampleLayersBatched)
+      GS_DEF2("_CAPI_LayerwiseBlockIfFused", "_CAPI_layerwise_block_if_fused",
+              &Graph::LayerwiseBlockIfFused)
       GS_DEF2("_CAPI_FusionSlicing", "_CAPI_fusion_slicing", &Graph::FusedBidirSlicing)
       GS_DEF2("_CAPI_BatchFusionSlicing", "_CAPI_batch_fusion_slicing",
               &Graph::BatchFusedBidirSlicing)

@@ -261,6 +261,7 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
   std::shared_ptr<CSR> out_csr, spare_csr;
   std::shared_ptr<COO> out_coo;
   torch::Tensor select_index;
+  torch::Tensor carried;  // the slice's share of the edge data, when its own pass brought it
   torch::optional<torch::Tensor> e_ids;
   int64_t num_edges = 0;
 
@@ -286,7 +287,11 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
       if (stored.has_value())
         std::tie(tmp, select_index) =
             DCSCColSlicing(fmt, stored.value(), n_ids, with_coo, data_.has_value());
-      else
+      else if (data_.has_value() && hip::EdgeData::Fits(data_.value(), fmt->e_ids)) {
+        // the edges' data ride along in the slice's own pass: no select_index, no gather
+        const hip::EdgeData edge{data_.value(), fmt->e_ids};
+        std::tie(tmp, select_index) = CSCColSlicing(fmt, n_ids, with_coo, false, &edge, &carried);
+      } else
         std::tie(tmp, select_index) = CSCColSlicing(fmt, n_ids, with_coo, data_.has_value());
       if (relabel) {
         // the other side is renumbered by first occurrence (reference src/graph.cc:219-227)
@@ -341,7 +346,10 @@ c10::intrusive_ptr<Graph> Graph::Slicing(torch::Tensor n_ids, int64_t axis, int6
   ret->spare_csr_ = spare_csr;
   if (out_csc) ret->val_col_ids_ = new_val_cols;
   if (out_csr) ret->val_row_ids_ = new_val_rows;
-  InheritData(ret.get(), e_ids, select_index);
+  if (carried.defined())
+    ret->SetData(carried);
+  else
+    InheritData(ret.get(), e_ids, select_index);
   return ret;
 }
 
@@ -377,6 +385,57 @@ c10::intrusive_ptr<Graph> Graph::RowSliceOfCoo(const torch::Tensor& n_ids) {
   ret->spare_csr_ = std::make_shared<CSR>(CSR{indptr, sorted_cols, torch::nullopt});
   InheritData(ret.get(), coo_->e_ids, select_index);
   return ret;
+}
+
+std::vector<torch::Tensor> Graph::LayerwiseBlockIfFused(torch::Tensor seeds, int64_t fanout) {
+  Range range("gs::LayerwiseBlock");
+  Settle();
+  if (col_ids_.has_value() || row_ids_.has_value() || val_col_ids_.has_value() ||
+      val_row_ids_.has_value() || !(csc_ || coo_ || csr_))
+    return {};
+  const int64_t S = seeds.numel();
+  const int64_t picks = std::min<int64_t>(fanout, num_rows_);
+  if (S == 0 || picks <= 0 || seeds.dim() != 1 || !seeds.is_contiguous() ||
+      seeds.scalar_type() != IdOptions().dtype().toScalarType() ||
+      !hip::SortedUnionFits(S + picks, seeds))
+    return {};
+  int key_bits = 0;  // of column << bits(S + picks) | place among the nodes
+  while ((int64_t(1) << key_bits) < S + picks) ++key_bits;
+  int col_bits = 0;
+  while ((int64_t(1) << col_bits) < S) ++col_bits;
+  if (key_bits + col_bits > (seeds.element_size() == 4 ? 30 : 62)) return {};
+
+  auto U = Slicing(seeds, 0, _CSC, _COO, false);
+  // (the edges of a column slice come by column, which the block's ordering relies on)
+  if (!U->coo_ || U->num_edges_ == 0 || U->coo_->e_ids.has_value() || !U->coo_->col_sorted) return {};
+  if (U->data_.has_value() &&
+      (U->data_.value().scalar_type() != torch::kFloat32 || U->data_.value().dim() != 1))
+    return {};
+  const hip::SeedState before = hip::SaveSeedState();
+  torch::Tensor prob = U->Sum(1, 2, _CSR);
+  torch::Tensor picked = std::get<0>(hip::ListSamplingProbs(GetRows(), prob, fanout, false));
+  torch::Tensor nodes, count, kept_key, kept_pos, totals;
+  std::tie(nodes, count) = hip::SortedUnion(seeds, picked);
+  std::tie(kept_key, kept_pos, totals) =
+      hip::CooPickRows(U->coo_->row, U->coo_->col, nodes, count, S + picks);
+  const torch::Tensor h_totals = totals.cpu();  // the host waits here
+  const int64_t kept = h_totals.data_ptr<int64_t>()[1];
+  if (kept == 0) {
+    hip::RestoreSeedState(before);
+    return {};
+  }
+  torch::Tensor rows, values, indptr;
+  std::tie(rows, values, indptr) = hip::CooBlockValues(
+      hip::Slice1d(kept_key, 0, kept), hip::Slice1d(kept_pos, 0, kept), S + picks, U->coo_->row,
+      U->data_.has_value() ? torch::optional<torch::Tensor>(U->data_.value().contiguous())
+                           : torch::nullopt,
+      prob, S);
+  torch::Tensor normalized = torch::empty_like(values);
+  hip::SegmentNormalize(indptr, torch::nullopt, values, normalized);
+  torch::Tensor frontier;
+  std::vector<torch::Tensor> renamed;
+  std::tie(frontier, renamed) = BatchTensorRelabel({seeds, rows}, {rows});
+  return {frontier, indptr, renamed[0], normalized};
 }
 
 // ----------------------------------------------------------------- sampling
@@ -910,7 +969,12 @@ Graph::Relabel() {
 }
 
 torch::Tensor Graph::GetRows() {
-  return row_ids_.has_value() ? row_ids_.value() : torch::arange(num_rows_, IdOptions());
+  if (row_ids_.has_value()) return row_ids_.value();
+  if (!all_rows_.defined() || all_rows_.numel() != num_rows_ ||
+      all_rows_.options().dtype() != IdOptions().dtype() ||
+      all_rows_.device() != IdOptions().device())
+    all_rows_ = torch::arange(num_rows_, IdOptions());
+  return all_rows_;
 }
 
 torch::Tensor Graph::GetCols() {

@@ -153,6 +153,21 @@ class Graph : public torch::CustomClassHolder {
   std::vector<std::vector<torch::Tensor>> SampleLayersBatched(
       const std::vector<torch::Tensor>& seed_sets, const std::vector<int64_t>& fanouts,
       bool replace);
+  // One layer of a layer-wise (LADIES-style) sampler as ONE call, the operator chain of the
+  // reference's examples/ladies/ladies_raw.py:10-25 on a root graph:
+  //   U = this[:, seeds]; prob = U.sum(axis=1, powk=2);
+  //   picked = list_sampling_with_probs(all rows, prob, fanout, replace=false);
+  //   nodes = unique(cat(seeds, picked));
+  //   block of U[nodes, :].divide(prob[nodes], axis=1).normalize(axis=0)
+  // Returns {frontier, offsets of the seeds' columns, renamed row ends, values}: what
+  // Relabel() and GetData("default") of that chain's result give, the values already in the
+  // order of the block's edges (so there is no edge-id map).  The slice, the sum and the pick
+  // are the same calls as in the chain; behind them the edges of U are tested against the
+  // node set and only the kept ones are put in order, and the host waits twice more (kept
+  // count, frontier length).  Takes the list-sampling seed the chain would take.  Empty (nothing
+  // drawn, no seed consumed) where it does not apply: a graph with id maps, more than
+  // gs_sorted_union_max seeds + picks, a slice or a block without edges.
+  std::vector<torch::Tensor> LayerwiseBlockIfFused(torch::Tensor seeds, int64_t fanout);
   // induced subgraph: columns column_seeds, rows row_seeds (renamed to their position in
   // row_seeds), CSC only (reference src/graph.cc:116-141)
   c10::intrusive_ptr<Graph> FusedBidirSlicing(torch::Tensor column_seeds, torch::Tensor row_seeds);
@@ -226,6 +241,10 @@ class Graph : public torch::CustomClassHolder {
   // installs instead of converting the COO back.
   std::shared_ptr<CSC> spare_csc_;
   std::shared_ptr<CSR> spare_csr_;
+
+  // 0 .. num_rows - 1 of a graph without a row id list, made once (GetRows hands it to the
+  // list samplers of every layer)
+  torch::Tensor all_rows_;
 
   bool is_subgraph_ = false;
   int64_t num_cols_ = 0;

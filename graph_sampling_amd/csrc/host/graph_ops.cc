@@ -17,8 +17,11 @@ std::pair<std::shared_ptr<_TMP>, torch::Tensor> Wrap(hip::SliceResult r) {
 
 std::pair<std::shared_ptr<_TMP>, torch::Tensor> CSCColSlicing(std::shared_ptr<CSC> csc,
                                                               torch::Tensor node_ids,
-                                                              bool with_coo, bool with_select) {
-  return Wrap(hip::ColSlicing(csc->indptr, csc->indices, node_ids, with_coo, with_select));
+                                                              bool with_coo, bool with_select,
+                                                              const hip::EdgeData* edge,
+                                                              torch::Tensor* data_out) {
+  return Wrap(hip::ColSlicing(csc->indptr, csc->indices, node_ids, with_coo, with_select, edge,
+                              data_out));
 }
 
 std::pair<std::shared_ptr<_TMP>, torch::Tensor> CSCRowSlicing(std::shared_ptr<CSC> csc,

@@ -15,10 +15,17 @@
 
 namespace gs {
 
-// with_select false: the returned select_index is undefined (the caller has no edge data)
+namespace hip {
+struct EdgeData;  // hip_ops.h
+}
+
+// with_select false: the returned select_index is undefined (the caller has no edge data, or
+// hands it in as `edge` and gets the slice's share back in *data_out from the same pass)
 std::pair<std::shared_ptr<_TMP>, torch::Tensor> CSCColSlicing(std::shared_ptr<CSC> csc,
                                                               torch::Tensor node_ids,
-                                                              bool with_coo, bool with_select = true);
+                                                              bool with_coo, bool with_select = true,
+                                                              const hip::EdgeData* edge = nullptr,
+                                                              torch::Tensor* data_out = nullptr);
 
 std::pair<std::shared_ptr<_TMP>, torch::Tensor> CSCRowSlicing(std::shared_ptr<CSC> csc,
                                                               torch::Tensor node_ids,

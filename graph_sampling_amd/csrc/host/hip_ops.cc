@@ -245,7 +245,8 @@ void SetSampleAlgo(int64_t algo) {
 }
 
 SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
-                       const torch::Tensor& column_ids, bool with_coo, bool with_select) {
+                       const torch::Tensor& column_ids, bool with_coo, bool with_select,
+                       const EdgeData* edge, torch::Tensor* data_out) {
   NeedI64(indptr, "indptr");
   const int idb = IdBytes(indices, "indices");
   TORCH_CHECK(IdBytes(column_ids, "column ids") == idb, "column ids and indices differ in dtype");
@@ -262,10 +263,16 @@ SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices
   if (with_select) select_index = torch::empty({nnz}, I64(indptr));
   torch::Tensor coo_col;
   if (with_coo) coo_col = torch::empty({nnz}, indices.options());
-  Check(gs_slice_fill(indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), column_ids.data_ptr(), idb, S,
-                      sub_indptr.data_ptr<int64_t>(), nnz, sub_indices.data_ptr(),
-                      with_select ? select_index.data_ptr<int64_t>() : nullptr,
-                      with_coo ? coo_col.data_ptr() : nullptr, st),
+  const bool with_data = edge != nullptr && data_out != nullptr;
+  if (with_data) *data_out = torch::empty({nnz}, edge->data.options());
+  Check(gs_slice_fill_data(
+            indptr.data_ptr<int64_t>(), indptr.numel() - 1, indices.data_ptr(), column_ids.data_ptr(),
+            idb, S, sub_indptr.data_ptr<int64_t>(), nnz, sub_indices.data_ptr(),
+            with_select ? select_index.data_ptr<int64_t>() : nullptr,
+            with_coo ? coo_col.data_ptr() : nullptr,
+            with_data ? edge->data.data_ptr<float>() : nullptr,
+            with_data && edge->e_ids.has_value() ? edge->e_ids.value().data_ptr<int64_t>() : nullptr,
+            with_data ? data_out->data_ptr<float>() : nullptr, st),
         "gs_slice_fill");
   return {sub_indptr, coo_col, sub_indices, select_index};
 }
@@ -1239,6 +1246,71 @@ std::tuple<torch::Tensor, torch::Tensor> SortValuesByKey(const torch::Tensor& ke
                    Stream(key)),
         "gs_coo2csc");
   return {out_value, perm};
+}
+
+bool SortedUnionFits(int64_t count, const torch::Tensor& ids_like) {
+  return count >= 1 && count <= gs_sorted_union_max(IdBytes(ids_like, "ids"));
+}
+
+std::tuple<torch::Tensor, torch::Tensor> SortedUnion(const torch::Tensor& a, const torch::Tensor& b) {
+  const int idb = IdBytes(a, "a");
+  TORCH_CHECK(IdBytes(b, "b") == idb, "SortedUnion: the two id lists differ in dtype");
+  TORCH_CHECK(a.is_contiguous() && b.is_contiguous(), "SortedUnion: id lists must be contiguous");
+  auto out = torch::empty({a.numel() + b.numel()}, a.options());
+  auto count = torch::empty({1}, I64(a));
+  Check(gs_sorted_union(a.data_ptr(), a.numel(), b.data_ptr(), b.numel(), idb, out.data_ptr(),
+                        count.data_ptr<int64_t>(), Stream(a)),
+        "gs_sorted_union");
+  return {out, count};
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> CooPickRows(
+    const torch::Tensor& row, const torch::Tensor& col, const torch::Tensor& nodes,
+    const torch::Tensor& count, int64_t max_nodes) {
+  const int idb = IdBytes(row, "row");
+  TORCH_CHECK(IdBytes(col, "col") == idb && IdBytes(nodes, "nodes") == idb,
+              "CooPickRows: ids differ in dtype");
+  NeedI64(count, "count");
+  const int64_t E = row.numel();
+  TORCH_CHECK(col.numel() == E && nodes.numel() >= max_nodes && count.numel() >= 1,
+              "CooPickRows: sizes do not fit");
+  auto key = torch::empty({E}, row.options());
+  auto pos = torch::empty({E}, row.options());
+  auto totals = torch::empty({2}, I64(row));
+  auto ws = Scratch(gs_coo_pick_rows_workspace_bytes(E), row);
+  Check(gs_coo_pick_rows(row.data_ptr(), col.data_ptr(), idb, E, nodes.data_ptr(),
+                         count.data_ptr<int64_t>(), max_nodes, key.data_ptr(), pos.data_ptr(),
+                         totals.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), Stream(row)),
+        "gs_coo_pick_rows");
+  return {key, pos, totals};
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> CooBlockValues(
+    const torch::Tensor& kept_key, const torch::Tensor& kept_pos, int64_t max_nodes,
+    const torch::Tensor& row, const torch::optional<torch::Tensor>& data,
+    const torch::Tensor& divisor, int64_t num_cols) {
+  const int idb = IdBytes(row, "row");
+  TORCH_CHECK(IdBytes(kept_key, "keys") == idb && IdBytes(kept_pos, "positions") == idb,
+              "CooBlockValues: ids differ in dtype");
+  NeedF32(divisor, "divisor");
+  const int64_t kept = kept_key.numel();
+  TORCH_CHECK(kept_pos.numel() == kept, "CooBlockValues: one position per key");
+  const float* values = nullptr;
+  if (data.has_value()) {
+    NeedF32(data.value(), "data");
+    TORCH_CHECK(data.value().numel() == row.numel() && data.value().is_contiguous(),
+                "CooBlockValues: one contiguous value per edge");
+    values = data.value().data_ptr<float>();
+  }
+  auto out_row = torch::empty({kept}, row.options());
+  auto out_value = torch::empty({kept}, divisor.options());
+  auto out_indptr = torch::empty({num_cols + 1}, I64(row));
+  Check(gs_coo_block_values(kept_key.data_ptr(), kept_pos.data_ptr(), kept, max_nodes, row.data_ptr(),
+                            idb, values, divisor.data_ptr<float>(), num_cols, out_row.data_ptr(),
+                            out_value.data_ptr<float>(), out_indptr.data_ptr<int64_t>(),
+                            Stream(row)),
+        "gs_coo_block_values");
+  return {out_row, out_value, out_indptr};
 }
 
 std::tuple<torch::Tensor, torch::Tensor> ListSampling(const torch::Tensor& data, int64_t k,

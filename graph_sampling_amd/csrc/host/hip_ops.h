@@ -38,8 +38,11 @@ bool OrderedSums();
 void SetSampleAlgo(int64_t algo);
 
 // with_select false: select_index comes back undefined (nothing to gather edge data for)
+struct EdgeData;
+// edge (with data_out): the slice carries the edges' data over in the same pass, into *data_out
 SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
-                       const torch::Tensor& column_ids, bool with_coo, bool with_select = true);
+                       const torch::Tensor& column_ids, bool with_coo, bool with_select = true,
+                       const EdgeData* edge = nullptr, torch::Tensor* data_out = nullptr);
 // column_ids undefined: every column of the CSC
 SliceResult ColSampling(const torch::Tensor& indptr, const torch::Tensor& indices,
                         const torch::Tensor& column_ids, int64_t fanout, bool replace,
@@ -242,6 +245,26 @@ std::tuple<torch::Tensor, torch::Tensor, torch::optional<torch::Tensor>> Coo2Csc
 std::tuple<torch::Tensor, torch::Tensor> SortValuesByKey(const torch::Tensor& key,
                                                          const torch::Tensor& value,
                                                          int64_t num_keys);
+
+// ---- the tail of a layer-wise sampler on a column slice held as a COO (gs_layerwise.hip)
+// whether na + nb ids of this width fit the one-workgroup sort of SortedUnion
+bool SortedUnionFits(int64_t count, const torch::Tensor& ids_like);
+// {distinct values of a and b in increasing order (room for all; the first *count hold),
+// count: device int64[1]}
+std::tuple<torch::Tensor, torch::Tensor> SortedUnion(const torch::Tensor& a, const torch::Tensor& b);
+// the edges of (row, col) whose row is among the first *count of nodes (SortedUnion's pair),
+// in edge order: {key = col << bits(max_nodes) | place of the row in nodes, position of the
+// edge; both with room for every edge, totals: device int64[2] = {*count, kept edges}}
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> CooPickRows(
+    const torch::Tensor& row, const torch::Tensor& col, const torch::Tensor& nodes,
+    const torch::Tensor& count, int64_t max_nodes);
+// the block of the kept edges of a COO whose edges come by column (CooPickRows' pair, cut to
+// the kept count; the same max_nodes): inside every column in the order of the rows,
+// {their row ids, data / divisor[row] (data undefined: ones), offsets of the num_cols columns}
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> CooBlockValues(
+    const torch::Tensor& kept_key, const torch::Tensor& kept_pos, int64_t max_nodes,
+    const torch::Tensor& row, const torch::optional<torch::Tensor>& data,
+    const torch::Tensor& divisor, int64_t num_cols);
 
 std::tuple<torch::Tensor, torch::Tensor> ListSampling(const torch::Tensor& data, int64_t k,
                                                       bool replace);

@@ -12,6 +12,12 @@
   one graph, `Relabel`, next seeds = the frontier; examples/graphsage/batching.py:125-138)
   become one `sample_layer_chain` call, which queues every layer on the device at once where
   the graph allows it and goes layer by layer where it does not.  Not in the reference.
+* `fuse_layerwise_block` -- a whole layer of a layer-wise sampler (column slice, row
+  probabilities, weighted pick of rows, node set, row slice, division by the probabilities,
+  column normalisation, block: examples/ladies/ladies_raw.py:10-25) whose intermediate
+  results serve nothing else becomes one `layerwise_block` call, which hands the layer to one
+  call of the C++ layer where the graph allows it and runs the same chain where it does not.
+  Not in the reference.
 * `common_subexpressions` -- repeated pure queries of one graph (valid rows, sums, ...) are
   made once (python/gs/jit/passes.py:40-58, restricted here to calls known to be pure:
   sampling calls draw fresh random numbers and must stay apart).
@@ -23,7 +29,7 @@ import operator
 import torch
 import torch.fx as fx
 
-from ..format import _COO, _CSC
+from ..format import _COO, _CSC, _CSR
 
 RELABEL = ("_CAPI_Relabel", "_CAPI_relabel")
 ALL_VALID = ("_CAPI_AllValidNode", "_CAPI_all_valid_node")
@@ -200,6 +206,122 @@ def chain_sampled_layers(gm: fx.GraphModule) -> fx.GraphModule:
     return dead_code(gm)
 
 
+def layerwise_block(graph, seeds, fanout):
+    """(tuple of `Graph::Relabel`, edge data) of one layer of a layer-wise sampler: what
+    the chain below returns under the same seed.  A root graph takes the layer in one call of
+    the C++ layer; its block has no edge-id map, the values come in the order of its edges."""
+    parts = graph._CAPI_LayerwiseBlockIfFused(seeds, int(fanout))
+    if parts:
+        frontier, indptr, rows, values = parts
+        return (frontier, frontier.numel(), seeds.numel(), indptr, rows, None, "csc"), values
+    U = graph._CAPI_Slicing(seeds, 0, _CSC, _COO, False)
+    prob = U._CAPI_Sum(1, 2, _CSR)
+    picked = torch.ops.gs_ops.list_sampling_with_probs(U._CAPI_GetRows(), prob, fanout, False)[0]
+    nodes = torch.cat((seeds, picked)).unique()
+    sub = U._CAPI_Slicing(nodes, 1, _CSR, _COO, False)
+    sub = sub._CAPI_Divide(prob[nodes], 1, _COO)._CAPI_Normalize(0, _CSC)
+    return sub._CAPI_Relabel(), sub._CAPI_GetData("default")
+
+
+def _only_users(node, *users):
+    return set(node.users) == set(users)
+
+
+def _match_layerwise_block(norm):
+    """The nodes of one layer that ends in `norm` (a column normalisation), or None."""
+    if not (_is_method(norm, ("_CAPI_Normalize", "_CAPI_normalize")) and norm.args[1:] == (0, _CSC)):
+        return None
+    relabel = [u for u in norm.users if _is_method(u, RELABEL) and u.args == (norm,)]
+    data = [u for u in norm.users if _is_method(u, ("_CAPI_GetData", "_CAPI_get_data")) and
+            u.args == (norm, "default") and not u.kwargs]
+    if len(relabel) != 1 or len(relabel) + len(data) != len(norm.users):
+        return None
+    div = norm.args[0]
+    if not (isinstance(div, fx.Node) and _is_method(div, ("_CAPI_Divide", "_CAPI_divide")) and
+            len(div.args) == 4 and div.args[2:] == (1, _COO) and _only_users(div, norm)):
+        return None
+    sub, scale = div.args[0], div.args[1]
+    if not (isinstance(sub, fx.Node) and _is_method(sub, SLICING) and len(sub.args) == 6 and
+            sub.args[2:] == (1, _CSR, _COO, False) and _only_users(sub, div)):
+        return None
+    U, nodes = sub.args[0], sub.args[1]
+    if not (isinstance(scale, fx.Node) and scale.op == "call_function" and
+            scale.target is operator.getitem and scale.args[1] is nodes and _only_users(scale, div)):
+        return None
+    prob = scale.args[0]
+    if not (isinstance(nodes, fx.Node) and nodes.op == "call_method" and nodes.target == "unique" and
+            len(nodes.args) == 1 and not nodes.kwargs and _only_users(nodes, sub, scale)):
+        return None
+    cat = nodes.args[0]
+    if not (isinstance(cat, fx.Node) and cat.op == "call_function" and cat.target is torch.cat and
+            len(cat.args) == 1 and not cat.kwargs and isinstance(cat.args[0], (tuple, list)) and
+            len(cat.args[0]) == 2 and _only_users(cat, nodes)):
+        return None
+    seeds, picked = cat.args[0]
+    if not (isinstance(picked, fx.Node) and picked.op == "call_function" and
+            picked.target is operator.getitem and picked.args[1] == 0 and _only_users(picked, cat)):
+        return None
+    pick = picked.args[0]
+    if not (isinstance(pick, fx.Node) and pick.op == "call_function" and
+            pick.target in _LIST_SAMPLING_WITH_PROBS and len(pick.args) == 4 and
+            pick.args[1] is prob and isinstance(pick.args[2], int) and pick.args[3] is False and
+            _only_users(pick, picked)):
+        return None
+    rows = pick.args[0]
+    if not (isinstance(U, fx.Node) and _is_method(U, SLICING) and len(U.args) == 6 and
+            U.args[1] is seeds and U.args[2:] == (0, _CSC, _COO, False)):
+        return None
+    if not (isinstance(rows, fx.Node) and _is_method(rows, ("_CAPI_GetRows", "_CAPI_get_rows")) and
+            rows.args == (U,) and _only_users(rows, pick)):
+        return None
+    if not (isinstance(prob, fx.Node) and _is_method(prob, ("_CAPI_Sum", "_CAPI_sum")) and
+            prob.args == (U, 1, 2, _CSR) and _only_users(prob, pick, scale)):
+        return None
+    if not _only_users(U, prob, rows, sub):
+        return None
+    # users first, so that the nodes can be erased in this order
+    return {"relabel": relabel[0], "data": data, "graph": U.args[0], "seeds": seeds,
+            "fanout": pick.args[2],
+            "nodes": [norm, div, scale, sub, nodes, cat, picked, pick, rows, prob, U]}
+
+
+def _list_sampling_targets():
+    names = ("list_sampling_with_probs", "_CAPI_ListSamplingWithProbs")
+    found = []
+    for name in names:
+        try:
+            packet = getattr(torch.ops.gs_ops, name)
+        except (AttributeError, RuntimeError):
+            continue
+        found.append(packet)
+        found.extend(getattr(packet, o) for o in packet.overloads())
+    return tuple(found)
+
+
+_LIST_SAMPLING_WITH_PROBS = ()
+
+
+def fuse_layerwise_block(gm: fx.GraphModule) -> fx.GraphModule:
+    global _LIST_SAMPLING_WITH_PROBS
+    if not _LIST_SAMPLING_WITH_PROBS:
+        _LIST_SAMPLING_WITH_PROBS = _list_sampling_targets()
+    for norm in list(gm.graph.nodes):
+        layer = _match_layerwise_block(norm)
+        if layer is None:
+            continue
+        with gm.graph.inserting_before(layer["relabel"]):
+            fused = gm.graph.call_function(layerwise_block,
+                                           (layer["graph"], layer["seeds"], layer["fanout"]))
+            layer["relabel"].replace_all_uses_with(gm.graph.call_function(operator.getitem, (fused, 0)))
+            if layer["data"]:
+                values = gm.graph.call_function(operator.getitem, (fused, 1))
+                for query in layer["data"]:
+                    query.replace_all_uses_with(values)
+        for node in layer["data"] + [layer["relabel"]] + layer["nodes"]:
+            gm.graph.erase_node(node)
+    return dead_code(gm)
+
+
 def common_subexpressions(gm: fx.GraphModule) -> fx.GraphModule:
     seen = {}
     for node in list(gm.graph.nodes):
@@ -219,4 +341,4 @@ def common_subexpressions(gm: fx.GraphModule) -> fx.GraphModule:
 
 
 DEFAULT = (merge_relabel_and_all_indices, fuse_slicing_and_sampling, chain_sampled_layers,
-           common_subexpressions, dead_code)
+           fuse_layerwise_block, common_subexpressions, dead_code)

@@ -130,6 +130,16 @@ int gs_slice_fill(const int64_t* indptr, int64_t num_cols, const void* indices,
                   const void* column_ids, int id_bytes, int64_t S, const int64_t* sub_indptr,
                   int64_t nnz, void* sub_indices, int64_t* select_index, void* coo_col,
                   void* stream);
+/* gs_slice_fill that also carries the edges' data over in the same pass: data_out[p] =
+ * edge_data[edge_ids ? edge_ids[q] : q] for the edge copied from position q of indices --
+ * the gather the reference makes afterwards from select_index (src/graph.cc:68-73), which
+ * the caller then need not ask for.  edge_data NULL (then edge_ids and data_out too):
+ * gs_slice_fill. */
+int gs_slice_fill_data(const int64_t* indptr, int64_t num_cols, const void* indices,
+                       const void* column_ids, int id_bytes, int64_t S, const int64_t* sub_indptr,
+                       int64_t nnz, void* sub_indices, int64_t* select_index, void* coo_col,
+                       const float* edge_data, const int64_t* edge_ids, float* data_out,
+                       void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Uniform neighbour sampling: replaces impl::CSCColSamplingCUDA              */
@@ -692,6 +702,42 @@ int gs_coo_filter_compact(const void* row, const void* col, int id_bytes, int64_
 size_t gs_index_search_workspace_bytes(int64_t n);
 int gs_index_search(const void* data, int64_t n, const void* keys, int64_t m, int id_bytes,
                     void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* The rows of a column slice that a layer-wise sampler keeps, as the block's   */
+/* values: what examples/ladies/ladies_raw.py:15-22 reaches through              */
+/*   nodes = unique(cat(seeds, picked)); U[nodes, :].divide(prob[nodes], 1)      */
+/* (a CSR of all of U, src/graph.cc:258-283 -> impl::CSCColSlicingCUDA,          */
+/* src/cuda/graph_ops.cu division by row, then the CSC of the result,            */
+/* src/graph.cc:585-644) without sorting the edges that are not kept.            */
+/* ------------------------------------------------------------------------- */
+/* out = the distinct values of a[na] and b[nb] in increasing order (torch.unique of their
+ * concatenation, for ids >= 0), *count (device) = how many; out has room for na + nb.
+ * 1 <= na + nb <= gs_sorted_union_max(id_bytes) (8192 / 4096 for 4- / 8-byte ids: one
+ * workgroup sorts them in LDS). */
+int64_t gs_sorted_union_max(int id_bytes);
+int gs_sorted_union(const void* a, int64_t na, const void* b, int64_t nb, int id_bytes, void* out,
+                    int64_t* count, void* stream);
+/* Of the COO (row, col)[E], the edges whose row is among nodes[*num_nodes] (sorted, distinct,
+ * at most max_nodes <= gs_sorted_union_max: the output of gs_sorted_union with its count
+ * still on the device), in edge order: kept_key = col << bits | position of the row in
+ * nodes, with bits = the smallest b that has 2^b >= max_nodes (the caller makes sure
+ * num_cols << bits fits the id type), and kept_pos = the edge's position.  Both have room
+ * for E entries.  totals (device int64[2]) = {*num_nodes, number of kept edges}. */
+size_t gs_coo_pick_rows_workspace_bytes(int64_t E);
+int gs_coo_pick_rows(const void* row, const void* col, int id_bytes, int64_t E, const void* nodes,
+                     const int64_t* num_nodes, int64_t max_nodes, void* kept_key, void* kept_pos,
+                     int64_t* totals, void* workspace, size_t workspace_bytes, void* stream);
+/* The block of the kept edges (kept_key / kept_pos [kept] as gs_coo_pick_rows leaves them for a
+ * COO whose edges come by column, with the same max_nodes): inside every column the edges are
+ * put in the order of their rows (ties: of their positions) -- the order of a stable sort of
+ * all kept edges by kept_key, done column by column in LDS -- and leave as out_row = their row
+ * ids and out_value = data[pos] / divisor[row] (data NULL: ones; divisor is indexed by row id);
+ * out_indptr[num_cols + 1] = the offsets of the columns. */
+int gs_coo_block_values(const void* kept_key, const void* kept_pos, int64_t kept, int64_t max_nodes,
+                        const void* row, int id_bytes, const float* data, const float* divisor,
+                        int64_t num_cols, void* out_row, float* out_value, int64_t* out_indptr,
+                        void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Format conversion: replaces impl::CSC2COOCUDA and impl::COO2CSCCUDA          */

@@ -125,8 +125,12 @@ def _compiled_ladies_equals_eager(dev, rtol):
     plain = jit.compile(ladies, (A, torch.arange(4, device=dev), [64, 64]),
                         passes=(passes.fuse_slicing_and_sampling, passes.common_subexpressions,
                                 passes.dead_code))
-    merged = jit.compile(ladies, (A, torch.arange(4, device=dev), [64, 64]))
-    for compiled, eager in ((plain, ladies), (merged, ladies_one_frontier)):
+    merged = jit.compile(ladies, (A, torch.arange(4, device=dev), [64, 64]),
+                         passes=tuple(p for p in passes.DEFAULT if p is not passes.fuse_layerwise_block))
+    one_call = jit.compile(ladies, (A, torch.arange(4, device=dev), [64, 64]))
+    assert "layerwise_block" in one_call.code and "layerwise_block" not in merged.code
+    for compiled, eager in ((plain, ladies), (merged, ladies_one_frontier),
+                            (one_call, ladies_one_frontier)):
         gs.set_seed(5)
         want_nodes, want_blocks = eager(A, seeds, [64, 64])
         gs.set_seed(5)

@@ -128,11 +128,52 @@ def test_slice_with_a_second_consumer_is_not_fused():
     assert "_CAPI_Slicing" in t and "_CAPI_Sampling" in t and passes.FUSED not in t
 
 
+NO_LAYERWISE = tuple(p for p in passes.DEFAULT if p is not passes.fuse_layerwise_block)
+
+
 def test_weighted_and_row_slices_are_left_alone():
-    c = jit.compile(ladies, (gs.Matrix(), torch.arange(4), [64, 64]))
+    c = jit.compile(ladies, (gs.Matrix(), torch.arange(4), [64, 64]), passes=NO_LAYERWISE)
     t = _targets(c)
     assert t.count("_CAPI_Slicing") == 4 and t.count("_CAPI_Relabel") == 2
     assert "_CAPI_AllValidNode" not in t and t.count("_CAPI_Sum") == 2
+
+
+def test_a_layer_of_a_layerwise_sampler_becomes_one_call():
+    c = jit.compile(ladies, (gs.Matrix(), torch.arange(4), [64, 32]))
+    assert _targets(c) == []  # nothing of the operator chain is left
+    layers = [n for n in _functions(c) if n.target is passes.layerwise_block]
+    assert [n.args[2] for n in layers] == [64, 32]
+    # the second layer's seeds are the first layer's frontier; the blocks are made of the
+    # layers' (relabel, data) pairs
+    first_relabel = [u for u in layers[0].users if u.args[1] == 0][0]
+    assert layers[1].args[1].args == (first_relabel, 0)
+    blocks = [n for n in _functions(c) if n.target is gs.block.make_block]
+    assert [b.args[0].args for b in blocks] == [(l, 0) for l in layers]
+    assert [b.args[1].args for b in blocks] == [(l, 1) for l in layers]
+
+
+def test_a_layer_whose_parts_are_used_elsewhere_stays_a_chain():
+    def keeps_the_probabilities(A, seeds, fanouts):
+        U = A[:, seeds]
+        prob = U.sum(axis=1, powk=2)
+        picked, _ = torch.ops.gs_ops.list_sampling_with_probs(U.row_ids(unique=False), prob,
+                                                              fanouts[0], False)
+        nodes = torch.cat((seeds, picked)).unique()
+        sub = U[nodes, :].divide(prob[nodes], axis=1).normalize(axis=0)
+        return sub.to_dgl_block(), prob
+
+    def other_power(A, seeds, fanouts):
+        U = A[:, seeds]
+        prob = U.sum(axis=1, powk=1)
+        picked, _ = torch.ops.gs_ops.list_sampling_with_probs(U.row_ids(unique=False), prob,
+                                                              fanouts[0], False)
+        nodes = torch.cat((seeds, picked)).unique()
+        return U[nodes, :].divide(prob[nodes], axis=1).normalize(axis=0).to_dgl_block()
+
+    for sampler in (keeps_the_probabilities, other_power):
+        c = jit.compile(sampler, (gs.Matrix(), torch.arange(4), [64]))
+        assert not [n for n in _functions(c) if n.target is passes.layerwise_block], sampler
+        assert _targets(c).count("_CAPI_Slicing") == 2
 
 
 def test_repeated_queries_are_made_once_but_samples_stay_apart():
