@@ -844,8 +844,18 @@ def sorted_union(a, b):
     return out, count
 
 
-def coo_pick_rows(row, col, nodes, count, max_nodes):
-    """gs_coo_pick_rows.  Returns (kept_key, kept_pos, totals: device int64[2])."""
+def post_total(values, at, box):
+    """gs_post_total: values[at] (device int64) through the mailbox `box`; returns it."""
+    _need(values, torch.int64, "values")
+    ticket = box.ticket()
+    _check(lib().gs_post_total(ctypes.c_void_p(values.data_ptr() + 8 * int(at)), box.ptr(),
+                               _i64(ticket), _stream(values.device)), "gs_post_total")
+    return box.wait(ticket, values.device)
+
+
+def coo_pick_rows(row, col, nodes, count, max_nodes, box=None):
+    """gs_coo_pick_rows.  Returns (kept_key, kept_pos, totals: device int64[2]); with a
+    mailbox `box` the number of kept edges is waited for and returned as a fourth value."""
     idb = _ids(row, "row")
     _ids(col, "col", like=row)
     _ids(nodes, "nodes", like=row)
@@ -855,10 +865,15 @@ def coo_pick_rows(row, col, nodes, count, max_nodes):
     pos = torch.empty(E, dtype=row.dtype, device=row.device)
     totals = torch.empty(2, dtype=torch.int64, device=row.device)
     ws = workspace(lib().gs_coo_pick_rows_workspace_bytes(_i64(E)), row.device)
+    ticket = box.ticket() if box is not None else 0
     _check(lib().gs_coo_pick_rows(_ptr(row), _ptr(col), idb, _i64(E), _ptr(nodes), _ptr(count),
-                                  _i64(max_nodes), _ptr(key), _ptr(pos), _ptr(totals), _ptr(ws),
+                                  _i64(max_nodes), _ptr(key), _ptr(pos), _ptr(totals),
+                                  box.ptr() if box is not None else ctypes.c_void_p(0),
+                                  _i64(ticket), _ptr(ws),
                                   ctypes.c_size_t(ws.numel()), _stream(row.device)),
            "gs_coo_pick_rows")
+    if box is not None:
+        return key, pos, totals, box.wait(ticket, row.device)
     return key, pos, totals
 
 

@@ -132,7 +132,8 @@ __global__ void __launch_bounds__(kPickThreads)
 pick_fill_kernel(const int* __restrict__ place, const IdT* __restrict__ col, int64_t E,
                  int node_bits, const int64_t* __restrict__ tile_offsets, int64_t num_tiles,
                  const int64_t* __restrict__ num_nodes, IdT* __restrict__ kept_key,
-                 IdT* __restrict__ kept_pos, int64_t* __restrict__ totals) {
+                 IdT* __restrict__ kept_pos, int64_t* __restrict__ totals, gs_mailbox* box,
+                 int64_t ticket) {
   __shared__ int64_t s_scan[kPickThreads / kWave + 1];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kPickTile + threadIdx.x * kPickItems;
   int at[kPickItems];
@@ -154,8 +155,10 @@ pick_fill_kernel(const int* __restrict__ place, const IdT* __restrict__ col, int
     }
   }
   if (blockIdx.x == 0 && threadIdx.x == 0) {
+    const int64_t kept = tile_offsets[num_tiles];
     totals[0] = *num_nodes;
-    totals[1] = tile_offsets[num_tiles];
+    totals[1] = kept;
+    post_mailbox(box, kept, ticket);
   }
 }
 
@@ -335,7 +338,8 @@ int sorted_union_t(const void* a, int64_t na, const void* b, int64_t nb, void* o
 template <typename IdT>
 int pick_rows_t(const void* row, const void* col, int64_t E, const void* nodes,
                 const int64_t* num_nodes, int max_nodes, void* kept_key, void* kept_pos,
-                int64_t* totals, void* workspace, size_t workspace_bytes, hipStream_t st) {
+                int64_t* totals, gs_mailbox* box, int64_t ticket, void* workspace,
+                size_t workspace_bytes, hipStream_t st) {
   const int64_t tiles = blocks_for(E, kPickTile);
   Carver ws(workspace, workspace_bytes);
   int64_t* counts = ws.take<int64_t>(tiles);
@@ -358,7 +362,7 @@ int pick_rows_t(const void* row, const void* col, int64_t E, const void* nodes,
   hipLaunchKernelGGL(pick_fill_kernel<IdT>, grid, dim3(kPickThreads), 0, st,
                      static_cast<const int*>(place), static_cast<const IdT*>(col), E, node_bits,
                      static_cast<const int64_t*>(offsets), tiles, num_nodes,
-                     static_cast<IdT*>(kept_key), static_cast<IdT*>(kept_pos), totals);
+                     static_cast<IdT*>(kept_key), static_cast<IdT*>(kept_pos), totals, box, ticket);
   return check_launch("coo_pick_rows");
 }
 
@@ -393,7 +397,8 @@ size_t gs_coo_pick_rows_workspace_bytes(int64_t E) {
 
 int gs_coo_pick_rows(const void* row, const void* col, int id_bytes, int64_t E, const void* nodes,
                      const int64_t* num_nodes, int64_t max_nodes, void* kept_key, void* kept_pos,
-                     int64_t* totals, void* workspace, size_t workspace_bytes, void* stream) {
+                     int64_t* totals, gs_mailbox* mailbox, int64_t ticket, void* workspace,
+                     size_t workspace_bytes, void* stream) {
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_coo_pick_rows: id_bytes must be 4 or 8, got %d", id_bytes);
   GS_REQUIRE(E >= 1 && (id_bytes == 8 || E < (int64_t(1) << 31)),
              "gs_coo_pick_rows: %lld edges (at least one; below 2^31 with 4-byte ids)",
@@ -406,9 +411,9 @@ int gs_coo_pick_rows(const void* row, const void* col, int id_bytes, int64_t E, 
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int n = static_cast<int>(max_nodes);
   return id_bytes == 8 ? pick_rows_t<int64_t>(row, col, E, nodes, num_nodes, n, kept_key, kept_pos,
-                                              totals, workspace, workspace_bytes, st)
+                                              totals, mailbox, ticket, workspace, workspace_bytes, st)
                        : pick_rows_t<int32_t>(row, col, E, nodes, num_nodes, n, kept_key, kept_pos,
-                                              totals, workspace, workspace_bytes, st);
+                                              totals, mailbox, ticket, workspace, workspace_bytes, st);
 }
 
 int gs_coo_block_values(const void* kept_key, const void* kept_pos, int64_t kept, int64_t max_nodes,

@@ -104,6 +104,11 @@ constexpr int kFillItems = 8;
 constexpr int kFillTile = kFillThreads * kFillItems;
 constexpr int kFillStage = 1024;  // rows of offsets staged in LDS
 
+__global__ void post_total_kernel(const int64_t* __restrict__ value, gs_mailbox* box,
+                                  int64_t ticket) {
+  post_mailbox(box, *value, ticket);
+}
+
 template <typename IdT, bool WITH_COO, bool WITH_DATA>
 __global__ void __launch_bounds__(kFillThreads)
 slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
@@ -1300,6 +1305,13 @@ int gs_slice_count(const int64_t* indptr, int64_t num_cols, const void* column_i
   return id_bytes == 8
              ? slice_count_impl<int64_t>(indptr, num_cols, column_ids, S, sub_indptr, tiles, st)
              : slice_count_impl<int32_t>(indptr, num_cols, column_ids, S, sub_indptr, tiles, st);
+}
+
+int gs_post_total(const int64_t* value, gs_mailbox* mailbox, int64_t ticket, void* stream) {
+  GS_REQUIRE(value && mailbox, "gs_post_total: null pointer");
+  hipLaunchKernelGGL(post_total_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), value,
+                     mailbox, ticket);
+  return check_launch("post_total");
 }
 
 int gs_slice_fill(const int64_t* indptr, int64_t num_cols, const void* indices,

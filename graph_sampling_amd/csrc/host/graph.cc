@@ -416,10 +416,9 @@ std::vector<torch::Tensor> Graph::LayerwiseBlockIfFused(torch::Tensor seeds, int
   torch::Tensor picked = std::get<0>(hip::ListSamplingProbs(GetRows(), prob, fanout, false));
   torch::Tensor nodes, count, kept_key, kept_pos, totals;
   std::tie(nodes, count) = hip::SortedUnion(seeds, picked);
+  int64_t kept = 0;  // (the host waits here)
   std::tie(kept_key, kept_pos, totals) =
-      hip::CooPickRows(U->coo_->row, U->coo_->col, nodes, count, S + picks);
-  const torch::Tensor h_totals = totals.cpu();  // the host waits here
-  const int64_t kept = h_totals.data_ptr<int64_t>()[1];
+      hip::CooPickRows(U->coo_->row, U->coo_->col, nodes, count, S + picks, &kept);
   if (kept == 0) {
     hip::RestoreSeedState(before);
     return {};

@@ -244,6 +244,19 @@ void SetSampleAlgo(int64_t algo) {
   g_algo.store(algo);
 }
 
+namespace {
+// values[at] of a device int64 array, through a mailbox: a one-thread kernel behind the producer
+// posts it and the host spins on pinned memory, instead of a copy to pageable memory and a
+// stream synchronisation
+int64_t ReadTotal(const torch::Tensor& values, int64_t at, void* stream, const char* what) {
+  HostBoxes& boxes = Boxes(values.get_device());
+  const int64_t ticket = boxes.next++;
+  Check(gs_post_total(values.data_ptr<int64_t>() + at, boxes.slot(ticket), ticket, stream), what);
+  const int64_t total = WaitBox(boxes.slot(ticket), ticket, stream, what);
+  return total == kLost ? values[at].item<int64_t>() : total;
+}
+}  // namespace
+
 SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
                        const torch::Tensor& column_ids, bool with_coo, bool with_select,
                        const EdgeData* edge, torch::Tensor* data_out) {
@@ -257,7 +270,7 @@ SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices
   Check(gs_slice_count(indptr.data_ptr<int64_t>(), indptr.numel() - 1, column_ids.data_ptr(), idb, S,
                        sub_indptr.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
         "gs_slice_count");
-  const int64_t nnz = sub_indptr[S].item<int64_t>();
+  const int64_t nnz = ReadTotal(sub_indptr, S, st, "gs_slice_count");
   auto sub_indices = torch::empty({nnz}, indices.options());
   torch::Tensor select_index;
   if (with_select) select_index = torch::empty({nnz}, I64(indptr));
@@ -306,7 +319,7 @@ SliceResult SampleInto(const torch::Tensor& indptr, const torch::Tensor& indices
                         sub_indptr.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
         "gs_sample_count");
   fill(cols, idb, S, sub_indptr, sub_indices, select_index, coo_col, ws, st);
-  const int64_t nnz = sub_indptr[S].item<int64_t>();  // the only host read of the call
+  const int64_t nnz = ReadTotal(sub_indptr, S, Stream(sub_indptr), "total");  // the only host read of the call
   if (with_coo) coo_col = coo_col.narrow(0, 0, nnz);
   return {sub_indptr, coo_col, sub_indices.narrow(0, 0, nnz), select_index.narrow(0, 0, nnz)};
 }
@@ -497,7 +510,7 @@ SliceResult ColSamplingProbs(const torch::Tensor& indptr, const torch::Tensor& i
                            IdBytes(column_ids, "column ids"), S, cdf_ptr.data_ptr<int64_t>(),
                            sws.data_ptr(), sws.numel(), Stream(indptr)),
             "gs_slice_count");
-      cdf_len = cdf_ptr[S].item<int64_t>();
+      cdf_len = ReadTotal(cdf_ptr, S, Stream(cdf_ptr), "total");
     }
     auto cdf = torch::empty({cdf_len > 0 ? cdf_len : 1}, probs.options());
     return SampleInto(
@@ -1071,7 +1084,7 @@ SliceResult RowSlicingCsc(const torch::Tensor& indptr, const torch::Tensor& indi
                               row_ids.data_ptr(), nr, out_indptr.data_ptr<int64_t>(), ws.data_ptr(),
                               ws.numel(), st),
         "gs_row_slice_csc_mark");
-  const int64_t kept = out_indptr[ncols].item<int64_t>();
+  const int64_t kept = ReadTotal(out_indptr, ncols, Stream(out_indptr), "total");
   auto out_indices = torch::empty({kept}, indices.options());
   auto select_index = torch::empty({kept}, I64(indptr));
   torch::Tensor coo_col;
@@ -1105,7 +1118,7 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> RowSlicingCoo(
     *flag_value = both.data_ptr<int64_t>()[1] != 0;
     if (!*flag_value) return {torch::Tensor(), torch::Tensor(), torch::Tensor()};
   } else {
-    kept = num.item<int64_t>();
+    kept = ReadTotal(num, 0, Stream(num), "total");
   }
   auto out_key = torch::empty({kept}, key.options());
   auto out_other = torch::empty({kept}, key.options());
@@ -1143,7 +1156,7 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ColRowSli
                          sub_indptr.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
           "gs_slice_count");
   }
-  const int64_t D = sub_indptr[S].item<int64_t>();
+  const int64_t D = ReadTotal(sub_indptr, S, Stream(sub_indptr), "total");
   auto out_indptr = torch::empty({S + 1}, I64(indptr));
   auto ws = Scratch(gs_col_row_slice_workspace_bytes(nr, D), indptr);
   Check(gs_col_row_slice_mark(indptr.data_ptr<int64_t>(), ncols, indices.data_ptr(), idb,
@@ -1152,7 +1165,7 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ColRowSli
                               OptI64(row_ptr, "row batch offsets"), B, encoding_size,
                               out_indptr.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), st),
         "gs_col_row_slice_mark");
-  const int64_t kept = out_indptr[S].item<int64_t>();
+  const int64_t kept = ReadTotal(out_indptr, S, Stream(out_indptr), "total");
   auto out_indices = torch::empty({kept}, indices.options());
   auto select_index = torch::empty({kept}, I64(indptr));
   auto parent_index = torch::empty({kept}, I64(indptr));
@@ -1195,7 +1208,7 @@ std::tuple<torch::Tensor, torch::Tensor> CscCompress(const torch::Tensor& indptr
                         out_indptr.data_ptr<int64_t>(), num.data_ptr<int64_t>(), ws.data_ptr(),
                         ws.numel(), Stream(indptr)),
         "gs_csc_compress");
-  const int64_t kept = num.item<int64_t>();
+  const int64_t kept = ReadTotal(num, 0, Stream(num), "total");
   return {out_indptr.narrow(0, 0, kept + 1), val_ids.narrow(0, 0, kept)};
 }
 
@@ -1266,7 +1279,7 @@ std::tuple<torch::Tensor, torch::Tensor> SortedUnion(const torch::Tensor& a, con
 
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> CooPickRows(
     const torch::Tensor& row, const torch::Tensor& col, const torch::Tensor& nodes,
-    const torch::Tensor& count, int64_t max_nodes) {
+    const torch::Tensor& count, int64_t max_nodes, int64_t* kept) {
   const int idb = IdBytes(row, "row");
   TORCH_CHECK(IdBytes(col, "col") == idb && IdBytes(nodes, "nodes") == idb,
               "CooPickRows: ids differ in dtype");
@@ -1278,10 +1291,17 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> CooPickRows(
   auto pos = torch::empty({E}, row.options());
   auto totals = torch::empty({2}, I64(row));
   auto ws = Scratch(gs_coo_pick_rows_workspace_bytes(E), row);
+  HostBoxes& boxes = Boxes(row.get_device());
+  const int64_t ticket = boxes.next++;
   Check(gs_coo_pick_rows(row.data_ptr(), col.data_ptr(), idb, E, nodes.data_ptr(),
                          count.data_ptr<int64_t>(), max_nodes, key.data_ptr(), pos.data_ptr(),
-                         totals.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(), Stream(row)),
+                         totals.data_ptr<int64_t>(), boxes.slot(ticket), ticket, ws.data_ptr(),
+                         ws.numel(), Stream(row)),
         "gs_coo_pick_rows");
+  if (kept) {
+    *kept = WaitBox(boxes.slot(ticket), ticket, Stream(row), "gs_coo_pick_rows");
+    if (*kept == kLost) *kept = totals[1].item<int64_t>();
+  }
   return {key, pos, totals};
 }
 
@@ -1508,7 +1528,7 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> CooFilter
                            OptI64(ids_ptr, "neighbors_ptr"), B, num.data_ptr<int64_t>(),
                            ws.data_ptr(), ws.numel(), st),
         "gs_coo_filter_mark");
-  const int64_t kept = num.item<int64_t>();
+  const int64_t kept = ReadTotal(num, 0, Stream(num), "total");
   auto out_row = torch::empty({kept}, key.options());
   auto out_col = torch::empty({kept}, key.options());
   auto select_index = torch::empty({kept}, I64(key));

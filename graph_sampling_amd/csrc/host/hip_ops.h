@@ -254,10 +254,11 @@ bool SortedUnionFits(int64_t count, const torch::Tensor& ids_like);
 std::tuple<torch::Tensor, torch::Tensor> SortedUnion(const torch::Tensor& a, const torch::Tensor& b);
 // the edges of (row, col) whose row is among the first *count of nodes (SortedUnion's pair),
 // in edge order: {key = col << bits(max_nodes) | place of the row in nodes, position of the
-// edge; both with room for every edge, totals: device int64[2] = {*count, kept edges}}
+// edge; both with room for every edge, totals: device int64[2] = {*count, kept edges}}.
+// kept (may be null): the host waits for the number of kept edges (a mailbox) and puts it there.
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> CooPickRows(
     const torch::Tensor& row, const torch::Tensor& col, const torch::Tensor& nodes,
-    const torch::Tensor& count, int64_t max_nodes);
+    const torch::Tensor& count, int64_t max_nodes, int64_t* kept = nullptr);
 // the block of the kept edges of a COO whose edges come by column (CooPickRows' pair, cut to
 // the kept count; the same max_nodes): inside every column in the order of the rows,
 // {their row ids, data / divisor[row] (data undefined: ones), offsets of the num_cols columns}

@@ -123,6 +123,12 @@ int gs_slice_count(const int64_t* indptr, int64_t num_cols, const void* column_i
                    int64_t S, int64_t* sub_indptr, void* workspace, size_t workspace_bytes,
                    void* stream);
 
+/* Posts *value (a device int64, e.g. sub_indptr + S after gs_slice_count) to a mailbox from a
+ * one-thread kernel queued on the stream: the host then spins on the mailbox instead of
+ * copying the value back and synchronising the stream (the blocking read of
+ * src/cuda/slicing.cu:147). */
+int gs_post_total(const int64_t* value, gs_mailbox* mailbox, int64_t ticket, void* stream);
+
 /* Neighbour copy (slicing.cu:101-119).  nnz = sub_indptr[S] as read back by the
  * caller.  coo_col may be NULL (WITH_COO = false); select_index may be NULL when
  * the caller has no edge data to gather. */
@@ -723,11 +729,13 @@ int gs_sorted_union(const void* a, int64_t na, const void* b, int64_t nb, int id
  * still on the device), in edge order: kept_key = col << bits | position of the row in
  * nodes, with bits = the smallest b that has 2^b >= max_nodes (the caller makes sure
  * num_cols << bits fits the id type), and kept_pos = the edge's position.  Both have room
- * for E entries.  totals (device int64[2]) = {*num_nodes, number of kept edges}. */
+ * for E entries.  totals (device int64[2]) = {*num_nodes, number of kept edges}; the number of
+ * kept edges also goes to the mailbox (may be NULL). */
 size_t gs_coo_pick_rows_workspace_bytes(int64_t E);
 int gs_coo_pick_rows(const void* row, const void* col, int id_bytes, int64_t E, const void* nodes,
                      const int64_t* num_nodes, int64_t max_nodes, void* kept_key, void* kept_pos,
-                     int64_t* totals, void* workspace, size_t workspace_bytes, void* stream);
+                     int64_t* totals, gs_mailbox* mailbox, int64_t ticket, void* workspace,
+                     size_t workspace_bytes, void* stream);
 /* The block of the kept edges (kept_key / kept_pos [kept] as gs_coo_pick_rows leaves them for a
  * COO whose edges come by column, with the same max_nodes): inside every column the edges are
  * put in the order of their rows (ties: of their positions) -- the order of a stable sort of

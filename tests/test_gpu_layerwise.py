@@ -72,6 +72,11 @@ def test_pick_rows_and_block_values_against_numpy(dev, idb, E, num_nodes, room):
     want_key, want_pos = _np_pick(row, col, nodes, bits)
     got_n, kept = [int(x) for x in totals.cpu()]
     assert got_n == num_nodes and kept == want_pos.size
+    # the same count through a mailbox, and any device value through gs_post_total
+    box = capi.Mailbox()
+    assert capi.coo_pick_rows(to_dev(row, dev), to_dev(col, dev), to_dev(padded, dev), count, room,
+                              box)[3] == kept
+    assert capi.post_total(totals, 0, box) == num_nodes and capi.post_total(totals, 1, box) == kept
     assert np.array_equal(key[:kept].cpu().numpy().astype(np.int64), want_key)
     assert np.array_equal(pos[:kept].cpu().numpy().astype(np.int64), want_pos)
 
