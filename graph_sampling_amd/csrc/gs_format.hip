@@ -646,36 +646,90 @@ constexpr int kBinMaxShift = 15;         // 2^15 sums = 128 KB of LDS
 
 __global__ void __launch_bounds__(kBinThreads)
 bin_sum_kernel(const unsigned long long* __restrict__ words, const int32_t* __restrict__ vals,
-               const int64_t* __restrict__ offsets, int64_t num_blocks, int idx_bits,
+               const int64_t* __restrict__ offsets, int64_t num_blocks, int num_bins, int idx_bits,
                int bin_shift, int powk, int64_t num_targets, float* __restrict__ out) {
   extern __shared__ float s_sum[];
-  const int bin = blockIdx.x;
+  // Which run, and which share of it, this workgroup takes: the launch has one workgroup per
+  // share that can exist (a run of n edges has ceil(n / 16 k) of them, 64 at most), and every
+  // workgroup works the numbering out for itself from the runs' sizes.  (A launch of 64
+  // workgroups per run, most of which left at once, spent 30 of its 48 us handing 64 KB of LDS
+  // to workgroups with nothing to do.)
+  __shared__ int64_t s_scan[kBinThreads / kWave + 1];
+  __shared__ int s_first[kRadix + 1];
+  {
+    int64_t mine = 0;
+    if (threadIdx.x < num_bins) {
+      const int64_t n = offsets[(threadIdx.x + 1) * num_blocks] - offsets[threadIdx.x * num_blocks];
+      mine = (n + kBinPartItems - 1) / kBinPartItems;
+      if (mine > kBinParts) mine = kBinParts;
+    }
+    int64_t total;
+    const int64_t before = block_exclusive_scan<kBinThreads>(mine, &total, s_scan);
+    if (threadIdx.x <= num_bins) s_first[threadIdx.x] = static_cast<int>(before);
+    __syncthreads();
+  }
+  if (static_cast<int>(blockIdx.x) >= s_first[num_bins]) return;
+  int bin = 0;
+  for (int step = kRadix / 2; step > 0; step >>= 1)
+    if (bin + step <= num_bins && s_first[bin + step] <= static_cast<int>(blockIdx.x)) bin += step;
+  const int part = static_cast<int>(blockIdx.x) - s_first[bin];
   const int64_t lo = offsets[bin * num_blocks], hi = offsets[(bin + 1) * num_blocks];
   const int64_t n = hi - lo;
   int64_t parts = (n + kBinPartItems - 1) / kBinPartItems;
   if (parts > kBinParts) parts = kBinParts;
-  if (static_cast<int64_t>(blockIdx.y) >= parts) return;
   const int width = 1 << bin_shift;
   for (int j = threadIdx.x; j < width; j += kBinThreads) s_sum[j] = 0.0f;
   __syncthreads();
   const int64_t per = (n + parts - 1) / parts;
-  const int64_t begin = lo + blockIdx.y * per;
+  const int64_t begin = lo + part * per;
   const int64_t end = begin + per < hi ? begin + per : hi;
   const int64_t first = static_cast<int64_t>(bin) << bin_shift;
-  for (int64_t i = begin + threadIdx.x; i < end; i += kBinThreads) {
-    const int64_t t = static_cast<int64_t>(words[i] >> idx_bits) - first;
-    // (a target beyond num_targets has no sum to go to: left out, as out has no room for it)
-    if (t >= 0 && t < width) atomicAdd(&s_sum[t], powk_f(__int_as_float(vals[i]), powk));
+  // a thread's edges eight at a time, all reads (clamped to the part) before the first
+  // addition: one edge at a time every addition waits for its own trip to memory
+  constexpr int kBatch = 8;
+  for (int64_t i0 = begin + threadIdx.x; i0 < end; i0 += kBinThreads * kBatch) {
+    unsigned long long w[kBatch];
+    int v[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int64_t i = i0 + u * kBinThreads;
+      w[u] = words[i < end ? i : end - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int64_t i = i0 + u * kBinThreads;
+      v[u] = vals[i < end ? i : end - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int64_t t = static_cast<int64_t>(w[u] >> idx_bits) - first;
+      // (a target beyond num_targets has no sum to go to: left out, as out has no room for it)
+      if (i0 + u * kBinThreads < end && t >= 0 && t < width)
+        atomicAdd(&s_sum[t], powk_f(__int_as_float(v[u]), powk));
+    }
   }
   __syncthreads();
-  for (int j = threadIdx.x; j < width; j += kBinThreads) {
-    const float x = s_sum[j];
-    if (x != 0.0f && first + j < num_targets) {
-      if (parts == 1)
-        out[first + j] += x;
-      else
-        unsafeAtomicAdd(out + first + j, x);
+  if (parts > 1) {
+    for (int j = threadIdx.x; j < width; j += kBinThreads) {
+      const float x = s_sum[j];
+      if (x != 0.0f && first + j < num_targets) unsafeAtomicAdd(out + first + j, x);
     }
+    return;
+  }
+  // the run is this workgroup's alone: plain read, add, write -- a thread's sums eight at a
+  // time, the reads (of a word that is always there where the sum is zero) before the writes
+  for (int j0 = threadIdx.x; j0 < width; j0 += kBinThreads * kBatch) {
+    float x[kBatch], was[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int j = j0 + u * kBinThreads;
+      x[u] = (j < width && first + j < num_targets) ? s_sum[j] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) was[u] = out[x[u] != 0.0f ? first + j0 + u * kBinThreads : first];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+      if (x[u] != 0.0f) out[first + j0 + u * kBinThreads] = was[u] + x[u];
   }
 }
 
@@ -725,8 +779,9 @@ int bin_sum_impl(const int32_t* target, const float* data, int64_t E, int powk, 
     set_error_text("gs_coo_sum_binned: %s", hipGetErrorString(lds_allowed));
     return GS_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL(bin_sum_kernel, dim3(bins, kBinParts), dim3(kBinThreads),
-                     sizeof(float) << bin_shift, st, words, vals, offsets, blocks, idx_bits,
+  const int64_t shares = E / kBinPartItems + bins;  // at most: sum of ceil(n / 16 k) over the runs
+  hipLaunchKernelGGL(bin_sum_kernel, dim3(static_cast<unsigned>(shares)), dim3(kBinThreads),
+                     sizeof(float) << bin_shift, st, words, vals, offsets, blocks, bins, idx_bits,
                      bin_shift, powk, num_targets, out);
   return check_launch("coo_sum_binned");
 }
