@@ -192,15 +192,20 @@ column_offsets_kernel(const IdT* __restrict__ kept_key, int64_t kept, int node_b
 // position) -- the order of a stable sort of all kept edges by key, which for a few tens of
 // thousands of edges is three radix passes of two launches each -- by a counting sort in LDS:
 // a histogram over the 2^node_bits places, its scan, then the edges in their own order, 4096
-// at a time: wave 0 walks them 64 at a time, a lane finds the lanes that hold the same place
+// at a time: a wave walks them 64 at a time, a lane finds the lanes that hold the same place
 // with one ballot per key bit and takes the bin's next free places in lane order; then all
 // lanes write row id and value data / divisor[row] to where the edges go.  Work grows with the
 // column's length, not its square: the hubs among a layer's seeds keep tens of thousands of
-// edges (parallel edges included), most columns a few dozen.
+// edges (parallel edges included), most columns a few dozen.  FOUR_WAVES (up to 2048 places):
+// each wave walks a quarter of the 4096 and counts per place in 16-bit counters of its own; an
+// edge's place is the bin's start + the counts of the quarters before its own + its rank
+// inside its quarter.
 constexpr int kColumnStage = 4096;
 constexpr int kColumnBatch = 4;
+constexpr int kFourWavesBits = 11;
+constexpr int kRankShift = 13;  // a key has at most 13 bits, a rank inside a quarter 12
 
-template <typename IdT>
+template <typename IdT, bool FOUR_WAVES>
 __global__ void __launch_bounds__(256)
 order_columns_kernel(const IdT* __restrict__ kept_key, const IdT* __restrict__ kept_pos,
                      int node_bits, const int64_t* __restrict__ indptr,
@@ -266,8 +271,48 @@ order_columns_kernel(const IdT* __restrict__ kept_key, const IdT* __restrict__ k
       for (int u = 0; u < kColumnBatch; ++u)
         if (j0 + u * 256 < n) s_key[j0 + u * 256] = k[u];
     }
+    if (FOUR_WAVES) {
+      unsigned int* zero = s_key + kColumnStage;  // the four waves' counters: 2 * places words
+      for (int j = threadIdx.x; j < 2 * places; j += 256) zero[j] = 0u;
+    }
     __syncthreads();
-    if (threadIdx.x < kWave) {
+    if (FOUR_WAVES) {
+      unsigned short* s_count = reinterpret_cast<unsigned short*>(s_key + kColumnStage);
+      const int wave = threadIdx.x / kWave;
+      const int quarter = ((n + 4 * kWave - 1) / (4 * kWave)) * kWave;
+      const int q_hi = (wave + 1) * quarter < n ? (wave + 1) * quarter : n;
+      unsigned short* mine = s_count + wave * places;
+      for (int c = wave * quarter; c < q_hi; c += kWave) {
+        const bool valid = c + lane < q_hi;
+        const unsigned int k = valid ? s_key[c + lane] : 0u;
+        unsigned long long peers = __ballot(valid);
+        for (int b = 0; b < node_bits; ++b) {
+          const bool bit = (k >> b) & 1u;
+          const unsigned long long with_bit = __ballot(valid && bit);
+          peers &= bit ? with_bit : ~with_bit;
+        }
+        if (valid) {
+          const unsigned int ahead = __popcll(peers & ((1ull << lane) - 1ull));
+          const unsigned int start = mine[k];
+          s_key[c + lane] = k | ((start + ahead) << kRankShift);
+          if (lane == 63 - __clzll(peers))
+            mine[k] = static_cast<unsigned short>(start + __popcll(peers));
+        }
+      }
+      __syncthreads();
+      for (int j = threadIdx.x; j < n; j += 256) {
+        const unsigned int v = s_key[j];
+        const unsigned int k = v & ((1u << kRankShift) - 1u);
+        unsigned int place = s_bin[k] + (v >> kRankShift);
+        const int w = j / quarter;
+        for (int before = 0; before < w; ++before) place += s_count[before * places + k];
+        s_key[j] = place;
+      }
+      __syncthreads();
+      for (int k = threadIdx.x; k < places; k += 256)
+        s_bin[k] += static_cast<unsigned int>(s_count[k]) + s_count[places + k] +
+                    s_count[2 * places + k] + s_count[3 * places + k];
+    } else if (threadIdx.x < kWave) {
       for (int c = 0; c < n; c += kWave) {
         const bool valid = c + lane < n;
         const unsigned int k = valid ? s_key[c + lane] : 0u;
@@ -314,6 +359,25 @@ order_columns_kernel(const IdT* __restrict__ kept_key, const IdT* __restrict__ k
     }
     __syncthreads();
   }
+}
+
+template <typename IdT>
+void order_columns_launch(dim3 grid, int node_bits, hipStream_t st, const void* kept_key,
+                          const void* kept_pos, const int64_t* indptr, const void* row,
+                          const float* data, const float* divisor, void* out_row, float* out_value) {
+  const size_t places = size_t(1) << node_bits;
+  if (node_bits <= kFourWavesBits)
+    hipLaunchKernelGGL((order_columns_kernel<IdT, true>), grid, dim3(256),
+                       (places + kColumnStage + 2 * places) * sizeof(unsigned int), st,
+                       static_cast<const IdT*>(kept_key), static_cast<const IdT*>(kept_pos), node_bits,
+                       indptr, static_cast<const IdT*>(row), data, divisor,
+                       static_cast<IdT*>(out_row), out_value);
+  else
+    hipLaunchKernelGGL((order_columns_kernel<IdT, false>), grid, dim3(256),
+                       (places + kColumnStage) * sizeof(unsigned int), st,
+                       static_cast<const IdT*>(kept_key), static_cast<const IdT*>(kept_pos), node_bits,
+                       indptr, static_cast<const IdT*>(row), data, divisor,
+                       static_cast<IdT*>(out_row), out_value);
 }
 
 inline int bits_of(int64_t n) {  // smallest b with 2^b >= n
@@ -432,25 +496,18 @@ int gs_coo_block_values(const void* kept_key, const void* kept_pos, int64_t kept
   const int node_bits = bits_of(max_nodes);
   const dim3 by_edge(static_cast<unsigned>(blocks_for(kept, 256)));
   const dim3 by_column(static_cast<unsigned>(num_cols));
-  const size_t column_lds = ((size_t(1) << node_bits) + kColumnStage) * sizeof(unsigned int);
   if (id_bytes == 8) {
     hipLaunchKernelGGL(column_offsets_kernel<int64_t>, by_edge, dim3(256), 0, st,
                        static_cast<const int64_t*>(kept_key), kept, node_bits, num_cols, out_indptr);
     if (kept > 0 && num_cols > 0)
-      hipLaunchKernelGGL(order_columns_kernel<int64_t>, by_column, dim3(256), column_lds, st,
-                         static_cast<const int64_t*>(kept_key), static_cast<const int64_t*>(kept_pos),
-                         node_bits, static_cast<const int64_t*>(out_indptr),
-                         static_cast<const int64_t*>(row), data, divisor,
-                         static_cast<int64_t*>(out_row), out_value);
+      order_columns_launch<int64_t>(by_column, node_bits, st, kept_key, kept_pos, out_indptr, row, data,
+                                    divisor, out_row, out_value);
   } else {
     hipLaunchKernelGGL(column_offsets_kernel<int32_t>, by_edge, dim3(256), 0, st,
                        static_cast<const int32_t*>(kept_key), kept, node_bits, num_cols, out_indptr);
     if (kept > 0 && num_cols > 0)
-      hipLaunchKernelGGL(order_columns_kernel<int32_t>, by_column, dim3(256), column_lds, st,
-                         static_cast<const int32_t*>(kept_key), static_cast<const int32_t*>(kept_pos),
-                         node_bits, static_cast<const int64_t*>(out_indptr),
-                         static_cast<const int32_t*>(row), data, divisor,
-                         static_cast<int32_t*>(out_row), out_value);
+      order_columns_launch<int32_t>(by_column, node_bits, st, kept_key, kept_pos, out_indptr, row, data,
+                                    divisor, out_row, out_value);
   }
   return check_launch("coo_block_values");
 }
