@@ -567,7 +567,7 @@ def sample_weighted_replace(indptr, indices, probs, column_ids, fanout, seed=0, 
         _ids(column_ids, "column_ids", like=indices)
         S = column_ids.numel()
         cdf_ptr = slice_count(indptr, column_ids)
-        cdf_len = int(cdf_ptr[-1].item())
+        cdf_len = _total(cdf_ptr, cdf_ptr.numel() - 1)
     sub_indptr = torch.empty(S + 1, dtype=torch.int64, device=dev)
     cap = S * int(fanout)
     sub_indices = torch.empty(cap, dtype=indices.dtype, device=dev)
@@ -805,7 +805,7 @@ def coo_filter(key, row, col, ids, key_ptr=None, ids_ptr=None):
     _check(lib().gs_coo_filter_mark(_ptr(key), idb, _i64(E), _ptr(key_ptr), _ptr(ids), _i64(n),
                                     _ptr(ids_ptr), _i64(B), _ptr(num_kept), _ptr(ws),
                                     ctypes.c_size_t(ws.numel()), st), "gs_coo_filter_mark")
-    kept = int(num_kept.item())
+    kept = _total(num_kept, 0)
     out_row = torch.empty(kept, dtype=key.dtype, device=dev)
     out_col = torch.empty(kept, dtype=key.dtype, device=dev)
     select_index = torch.empty(kept, dtype=torch.int64, device=dev)
@@ -842,6 +842,17 @@ def sorted_union(a, b):
     _check(lib().gs_sorted_union(_ptr(a), _i64(a.numel()), _ptr(b), _i64(b.numel()), idb, _ptr(out),
                                  _ptr(count), _stream(a.device)), "gs_sorted_union")
     return out, count
+
+
+_boxes = {}
+
+
+def _total(values, at):
+    """values[at] read back through a mailbox (gs_post_total) instead of a blocking copy."""
+    box = _boxes.get(values.device)
+    if box is None:
+        box = _boxes[values.device] = Mailbox()
+    return post_total(values, at, box)
 
 
 def post_total(values, at, box):
@@ -1037,7 +1048,7 @@ def row_slice_csc(indptr, indices, row_ids, with_coo):
     _check(lib().gs_row_slice_csc_mark(_ptr(indptr), _ptr(indices), idb, _i64(ncols), _i64(nnz),
                                        _ptr(row_ids), _i64(nr), _ptr(out_indptr), _ptr(ws),
                                        ctypes.c_size_t(ws.numel()), st), "gs_row_slice_csc_mark")
-    kept = int(out_indptr[-1].item())
+    kept = _total(out_indptr, out_indptr.numel() - 1)
     out_indices = torch.empty(kept, dtype=indices.dtype, device=dev)
     select_index = torch.empty(kept, dtype=torch.int64, device=dev)
     coo_col = torch.empty(kept, dtype=indices.dtype, device=dev) if with_coo else None
@@ -1063,7 +1074,7 @@ def row_slice_coo(key, other, ids):
     _check(lib().gs_row_slice_coo_mark(_ptr(key), idb, _i64(E), _ptr(ids), _i64(n), _ptr(num_kept),
                                        _ptr(ws), ctypes.c_size_t(ws.numel()), st),
            "gs_row_slice_coo_mark")
-    kept = int(num_kept.item())
+    kept = _total(num_kept, 0)
     out_key = torch.empty(kept, dtype=key.dtype, device=dev)
     out_other = torch.empty(kept, dtype=key.dtype, device=dev)
     select_index = torch.empty(kept, dtype=torch.int64, device=dev)
@@ -1091,7 +1102,7 @@ def col_row_slice(indptr, indices, column_ids, row_ids, col_ptr=None, row_ptr=No
         _need(row_ptr, torch.int64, "row_ptr")
         B = col_ptr.numel() - 1
     sub_indptr = slice_count(indptr, column_ids)
-    D = int(sub_indptr[-1].item())
+    D = _total(sub_indptr, sub_indptr.numel() - 1)
     out_indptr = torch.empty(S + 1, dtype=torch.int64, device=dev)
     ws = workspace(lib().gs_col_row_slice_workspace_bytes(_i64(nr), _i64(D)), dev)
     st = _stream(dev)
@@ -1100,7 +1111,7 @@ def col_row_slice(indptr, indices, column_ids, row_ids, col_ptr=None, row_ptr=No
                                        _ptr(row_ids), _i64(nr), _ptr(col_ptr), _ptr(row_ptr),
                                        _i64(B), _i64(encoding_size), _ptr(out_indptr), _ptr(ws),
                                        ctypes.c_size_t(ws.numel()), st), "gs_col_row_slice_mark")
-    kept = int(out_indptr[-1].item())
+    kept = _total(out_indptr, out_indptr.numel() - 1)
     out_indices = torch.empty(kept, dtype=indices.dtype, device=dev)
     select_index = torch.empty(kept, dtype=torch.int64, device=dev)
     parent_index = torch.empty(kept, dtype=torch.int64, device=dev)
