@@ -109,6 +109,17 @@ __global__ void post_total_kernel(const int64_t* __restrict__ value, gs_mailbox*
   post_mailbox(box, *value, ticket);
 }
 
+// values[0..n) to pinned host memory with system-scope stores, then the mailbox
+__global__ void __launch_bounds__(256)
+post_values_kernel(const int64_t* __restrict__ values, int64_t n, int64_t* out, gs_mailbox* box,
+                   int64_t ticket) {
+  for (int64_t i = threadIdx.x; i < n; i += 256)
+    __hip_atomic_store(&out[i], values[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  __threadfence_system();
+  __syncthreads();
+  if (threadIdx.x == 0) post_mailbox(box, n, ticket);
+}
+
 template <typename IdT, bool WITH_COO, bool WITH_DATA>
 __global__ void __launch_bounds__(kFillThreads)
 slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
@@ -1312,6 +1323,14 @@ int gs_post_total(const int64_t* value, gs_mailbox* mailbox, int64_t ticket, voi
   hipLaunchKernelGGL(post_total_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), value,
                      mailbox, ticket);
   return check_launch("post_total");
+}
+
+int gs_post_values(const int64_t* values, int64_t n, int64_t* host_out, gs_mailbox* mailbox,
+                   int64_t ticket, void* stream) {
+  GS_REQUIRE(n >= 0 && (n == 0 || (values && host_out)), "gs_post_values: null pointer or negative size");
+  hipLaunchKernelGGL(post_values_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     values, n, host_out, mailbox, ticket);
+  return check_launch("post_values");
 }
 
 int gs_slice_fill(const int64_t* indptr, int64_t num_cols, const void* indices,

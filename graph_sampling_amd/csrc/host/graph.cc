@@ -654,15 +654,17 @@ std::vector<std::vector<torch::Tensor>> Graph::SampleLayersBatched(
     if (with_data) y.data = hip::Slice1d(p->data, 0, nnz);
     torch::Tensor uni_ptr;
     std::tie(y.frontier, uni_ptr, y.renamed) = hip::BatchCsrRelabel(seeds, ptr, ids, ids_ptr);
+    // the cuts go to pinned memory by small kernels of the library (a copy call of the runtime
+    // per array cost the host 30-60 us each, a third of the call)
     y.cuts = torch::empty({3 * (B + 1)}, pinned);
-    y.cuts.narrow(0, 0, B + 1).copy_(ptr, /*non_blocking=*/true);
-    y.cuts.narrow(0, B + 1, B + 1).copy_(ids_ptr, /*non_blocking=*/true);
-    y.cuts.narrow(0, 2 * (B + 1), B + 1).copy_(uni_ptr, /*non_blocking=*/true);
+    hip::PostValues(ptr, y.cuts, 0);
+    hip::PostValues(ids_ptr, y.cuts, B + 1);
+    hip::PostValues(uni_ptr, y.cuts, 2 * (B + 1));
     seeds = y.frontier;
     ptr = uni_ptr;
   }
   // one wait for the cuts of all layers, then views
-  hip::SyncCurrentStream(seeds);
+  hip::WaitPosted(seeds);
   for (int64_t b = 0; b < B; ++b) out[b].reserve((with_data ? 4 : 3) * L);
   for (int64_t l = 0; l < L; ++l) {
     const Layer& y = layers[l];

@@ -257,6 +257,33 @@ int64_t ReadTotal(const torch::Tensor& values, int64_t at, void* stream, const c
 }
 }  // namespace
 
+namespace {
+thread_local std::map<int, int64_t> t_last_posted;  // device -> ticket of the last PostValues
+}
+
+void PostValues(const torch::Tensor& values, torch::Tensor& pinned, int64_t at) {
+  NeedI64(values, "values");
+  TORCH_CHECK(pinned.is_pinned() && pinned.scalar_type() == torch::kInt64 && pinned.is_contiguous() &&
+                  at >= 0 && at + values.numel() <= pinned.numel(),
+              "PostValues: the target must be pinned int64 memory with room for the values");
+  HostBoxes& boxes = Boxes(values.get_device());
+  const int64_t ticket = boxes.next++;
+  Check(gs_post_values(values.data_ptr<int64_t>(), values.numel(), pinned.data_ptr<int64_t>() + at,
+                       boxes.slot(ticket), ticket, Stream(values)),
+        "gs_post_values");
+  t_last_posted[values.get_device()] = ticket;
+}
+
+void WaitPosted(const torch::Tensor& like) {
+  const int device = like.get_device();
+  auto it = t_last_posted.find(device);
+  if (it == t_last_posted.end()) return;
+  HostBoxes& boxes = Boxes(device);
+  if (WaitBox(boxes.slot(it->second), it->second, Stream(like), "gs_post_values") == kLost)
+    SyncCurrentStream(like);  // the slot went to a later call: wait for the stream instead
+  t_last_posted.erase(it);
+}
+
 SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
                        const torch::Tensor& column_ids, bool with_coo, bool with_select,
                        const EdgeData* edge, torch::Tensor* data_out) {

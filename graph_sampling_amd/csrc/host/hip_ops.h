@@ -137,6 +137,12 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
                                                   const torch::Tensor& seeds,
                                                   const std::vector<int64_t>& fanouts,
                                                   bool replace, const EdgeData* edge = nullptr);
+// values (device int64) -> pinned[at ...] (pinned host memory) by a small kernel on the current
+// stream, without a copy call of the runtime.  WaitPosted() then waits (a mailbox) until the
+// last PostValues of the calling thread on that device has landed, and with it everything
+// queued before it on the same stream.
+void PostValues(const torch::Tensor& values, torch::Tensor& pinned, int64_t at);
+void WaitPosted(const torch::Tensor& like);
 // waits until everything queued on the calling thread's current stream of `like`'s device is done
 void SyncCurrentStream(const torch::Tensor& like);
 // t[first : first + count] of a contiguous 1-d tensor, sharing its storage: what narrow()

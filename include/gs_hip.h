@@ -128,6 +128,11 @@ int gs_slice_count(const int64_t* indptr, int64_t num_cols, const void* column_i
  * copying the value back and synchronising the stream (the blocking read of
  * src/cuda/slicing.cu:147). */
 int gs_post_total(const int64_t* value, gs_mailbox* mailbox, int64_t ticket, void* stream);
+/* The same for an array: values[0..n) (device) are stored to host_out (pinned host memory, mapped
+ * for the device) by one small kernel on the stream, and then {n, ticket} to the mailbox (may be
+ * NULL): offsets a caller cuts its results by reach the host without a copy call. */
+int gs_post_values(const int64_t* values, int64_t n, int64_t* host_out, gs_mailbox* mailbox,
+                   int64_t ticket, void* stream);
 
 /* Neighbour copy (slicing.cu:101-119).  nnz = sub_indptr[S] as read back by the
  * caller.  coo_col may be NULL (WITH_COO = false); select_index may be NULL when
