@@ -427,7 +427,7 @@ def _check_weighted_minibatch(dev, indptr, indices, weights, num_nodes, first_se
 
 
 def test_large_graph_with_edge_weights_keeps_the_queued_path(dev, large_graph):
-    """Configuration 5 as BASELINE.json states it: the 111 M / 1.6 B graph WITH its fp32 edge
+    """Configuration 5 in full: the 111 M / 1.6 B graph WITH its fp32 edge
     weights attached (6.4 GB)."""
     indptr, indices, _ = large_graph
     gen = torch.Generator(device=dev)

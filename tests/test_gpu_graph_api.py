@@ -1003,7 +1003,7 @@ def test_sample_layers_equals_the_layer_loop_and_the_oracle(dev, idt, fanouts, r
 @pytest.mark.parametrize("from_coo", [False, True])
 @pytest.mark.parametrize("fanouts,replace", [((15, 10, 5), False), ((4, 4), True), ((40, 3), False)])
 def test_sample_layers_on_a_graph_with_edge_data(dev, idt, from_coo, fanouts, replace):
-    """A graph with fp32 edge data (BASELINE configurations 3 and 5 carry weights): the whole
+    """A graph with fp32 edge data (configurations 3 and 5 carry weights): the whole
     minibatch still goes in one call, every layer hands back the sampled edges' share of the data
     (`data_[e_ids[select_index]]`, reference src/graph.cc:544-557), and the result equals the
     per-layer calls and the oracle.  Loaded as an unsorted COO the CSC has an edge-id map, and
