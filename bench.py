@@ -549,6 +549,35 @@ def graphsage(cx, workload, weighted, with_features, full, cpu_budget):
                     "per layer (examples/graphsage/batching.py:125-138)%s: one host wait per layer"
                     % (" + _CAPI_GetData of every sample" if weighted else "")}
 
+    # the same minibatches with the next one queued before this one is collected
+    if extras:
+        per = 4 if weighted else 3
+
+        def pipelined(sets):
+            edges, ahead = 0, graph._CAPI_QueueSampleLayers(sets[0], list(FANOUTS), False)
+            for nxt in list(sets[1:]) + [None]:
+                following = (graph._CAPI_QueueSampleLayers(nxt, list(FANOUTS), False)
+                             if nxt is not None else None)
+                parts = ahead.collect()
+                edges += sum(parts[per * l + 2].numel() for l in range(len(FANOUTS)))
+                ahead = following
+            return edges
+
+        ops._CAPI_SetSeed(0)
+        pipelined(seed_sets[:args.warmup])
+        ops._CAPI_SetSeed(first_seed)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        q_e = pipelined(timed_sets)
+        torch.cuda.synchronize()
+        q_s = time.perf_counter() - t1
+        out["queued_ahead"] = {
+            "ms_per_step": q_s / args.steps * 1e3, "value": q_e / q_s,
+            "same_edges_as_headline": bool(q_e == sampled),
+            "what": "_CAPI_QueueSampleLayers of minibatch i + 1 before .collect() of minibatch i (one "
+                    "thread, one stream): the same minibatches, the stream does not wait for the "
+                    "host between them"}
+
     # the same graph without its weights / with them, whichever the headline is not
     if extras and full != "config2":
         other = gs.Graph(False)

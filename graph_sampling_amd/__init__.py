@@ -98,6 +98,28 @@ def sample_blocks(matrix, seed_sets, fanouts, replace=False, workers=4, seed=0):
     return [_blocks_of(parts, len(fanouts)) for parts in flat]
 
 
+class _QueuedMinibatch(object):
+    """A minibatch whose launches are queued; `collect()` waits for it and returns
+    (input_nodes, [Block, ...]) as `sample_layers` does."""
+
+    def __init__(self, handle, num_layers):
+        self._handle, self._num_layers = handle, num_layers
+
+    def collect(self):
+        return _blocks_of(self._handle.collect(), self._num_layers)
+
+
+def queue_sample_layers(matrix, seeds, fanouts, replace=False):
+    """`sample_layers` in two halves: the call queues every layer's launches and returns at
+    once (the draws' seeds are taken now, in call order); `.collect()` of the returned object
+    waits and hands over the minibatch.  Queue minibatch i + 1 before collecting minibatch i
+    and the stream never waits for the host between them.  Not in the reference."""
+    load_library()
+    graph = getattr(matrix, "_graph", matrix)
+    fanouts = list(fanouts)
+    return _QueuedMinibatch(graph._CAPI_QueueSampleLayers(seeds, fanouts, bool(replace)), len(fanouts))
+
+
 def sample_blocks_batched(matrix, seed_sets, fanouts, replace=False):
     """GraphSAGE-style minibatches sampled as ONE launch sequence per layer (a "super-batch": the
     flow of the reference's examples/graphsage/batching.py:59-98 -- fused sampling over the

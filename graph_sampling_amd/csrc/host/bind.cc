@@ -28,6 +28,10 @@ torch::Tensor UniqueOp(torch::Tensor ids) { return TensorUnique(ids); }
 #define GS_DEF2(camel, snake, fn) .def(camel, fn).def(snake, fn)
 
 TORCH_LIBRARY(gs_classes, m) {
+  // not in the reference: a minibatch whose launches are queued and whose results are
+  // collected later (Graph::QueueSampleLayers)
+  m.class_<QueuedLayers>("QueuedLayers") GS_DEF2("_CAPI_Collect", "collect", &QueuedLayers::Collect);
+
   m.class_<Graph>("Graph")
       .def(torch::init<bool>())
       GS_DEF2("_CAPI_SetData", "_CAPI_set_data", &Graph::SetData)
@@ -49,6 +53,7 @@ TORCH_LIBRARY(gs_classes, m) {
               &Graph::SampleLayersBatched)
       GS_DEF2("_CAPI_LayerwiseBlockIfFused", "_CAPI_layerwise_block_if_fused",
               &Graph::LayerwiseBlockIfFused)
+      GS_DEF2("_CAPI_QueueSampleLayers", "_CAPI_queue_sample_layers", &Graph::QueueSampleLayers)
       GS_DEF2("_CAPI_FusionSlicing", "_CAPI_fusion_slicing", &Graph::FusedBidirSlicing)
       GS_DEF2("_CAPI_BatchFusionSlicing", "_CAPI_batch_fusion_slicing",
               &Graph::BatchFusedBidirSlicing)

@@ -589,6 +589,39 @@ std::vector<torch::Tensor> Graph::SampleLayersIfQueued(torch::Tensor seeds,
   }
 }
 
+c10::intrusive_ptr<QueuedLayers> Graph::QueueSampleLayers(torch::Tensor seeds,
+                                                          std::vector<int64_t> fanouts,
+                                                          bool replace) {
+  Range range("gs::QueueSampleLayers");
+  auto q = c10::make_intrusive<QueuedLayers>();
+  q->graph = c10::intrusive_ptr<Graph>::reclaim_copy(this);
+  q->seeds = seeds;
+  q->fanouts = fanouts;
+  q->replace = replace;
+  q->pending = QueueLayers(seeds, fanouts, replace);
+  if (!q->pending) q->ready = SampleLayersLoop(seeds, fanouts, replace);
+  return q;
+}
+
+std::vector<torch::Tensor> QueuedLayers::Collect() {
+  TORCH_CHECK(!collected, "this minibatch has been collected already");
+  collected = true;
+  if (!pending) return std::move(ready);
+  try {
+    auto out = pending->Collect();
+    pending.reset();
+    return out;
+  } catch (const hip::IdsTooWide&) {
+    // the same minibatch again, layer by layer, under the seeds the chain drew with
+    const hip::SeedState saved = hip::SaveSeedState();
+    hip::SetThreadSeed(pending->first_seed);
+    auto out = graph->SampleLayersLoop(seeds, fanouts, replace);
+    hip::RestoreSeedState(saved);
+    pending.reset();
+    return out;
+  }
+}
+
 std::vector<torch::Tensor> Graph::SampleLayers(torch::Tensor seeds, std::vector<int64_t> fanouts,
                                                bool replace) {
   Range range("gs::SampleLayers");

@@ -29,6 +29,19 @@ struct PendingSample;
 struct PendingLayers;
 }
 
+class Graph;
+// a minibatch queued by Graph::QueueSampleLayers (TORCH_LIBRARY class gs_classes.QueuedLayers)
+struct QueuedLayers : public torch::CustomClassHolder {
+  c10::intrusive_ptr<Graph> graph;
+  torch::Tensor seeds;
+  std::vector<int64_t> fanouts;
+  bool replace = false;
+  std::shared_ptr<hip::PendingLayers> pending;  // null: `ready` holds the result
+  std::vector<torch::Tensor> ready;
+  bool collected = false;
+  std::vector<torch::Tensor> Collect();
+};
+
 class Graph : public torch::CustomClassHolder {
  public:
   explicit Graph(bool is_subgraph) : is_subgraph_(is_subgraph) {}
@@ -142,6 +155,13 @@ class Graph : public torch::CustomClassHolder {
                                                   bool replace);
   std::vector<torch::Tensor> SampleLayersLoop(torch::Tensor seeds,
                                               const std::vector<int64_t>& fanouts, bool replace);
+  // SampleLayers in two halves for a caller that wants the next minibatch queued before it
+  // collects this one (one thread, one stream: the stream then never waits for the host
+  // between minibatches).  The seeds of the draws are taken here, in call order; collect()
+  // gives what SampleLayers would have returned.  Where the minibatch cannot be queued it is
+  // sampled at once and collect() hands the result over.
+  c10::intrusive_ptr<QueuedLayers> QueueSampleLayers(torch::Tensor seeds,
+                                                     std::vector<int64_t> fanouts, bool replace);
   // Many minibatches as ONE launch sequence per layer (a "super-batch", the flow of the
   // reference's examples/graphsage/batching.py:59-98: fused sampling over the concatenated
   // seeds, the batches' edge offsets, one relabel per minibatch done in one pass, the splits),

@@ -1100,6 +1100,42 @@ def test_sample_layers_keeps_8192_seeds_on_the_queued_path(dev):
     assert g._CAPI_SampleLayersIfQueued(to_dev(many, dev, torch.int32), [15, 10, 5], False) == []
 
 
+@pytest.mark.parametrize("with_data", [False, True])
+def test_queued_minibatches_equal_sample_layers_whatever_is_in_flight(dev, with_data):
+    """Four minibatches queued before the first is collected, collected out of order: each is
+    the minibatch `_CAPI_SampleLayers` gives under the seeds the queue calls took, in call order.
+    A graph that cannot be queued (column ids) is sampled at the queue call."""
+    m, indptr, indices, data = _rmat_matrix(dev, 13, 17, 21, with_data=with_data)
+    g = m._graph
+    fanouts = [10, 5, 3]
+    sets = [torch.randperm(1 << 13, device=dev)[:300 + 17 * i] for i in range(4)]
+    gs.set_seed(400)
+    want = [g._CAPI_SampleLayers(s, fanouts, False) for s in sets]
+    gs.set_seed(400)
+    handles = [g._CAPI_QueueSampleLayers(s, fanouts, False) for s in sets]
+    for i in (2, 0, 3, 1):
+        got = handles[i].collect()
+        assert len(got) == len(want[i]) == (4 if with_data else 3) * len(fanouts)
+        for a, b in zip(got, want[i]):
+            assert torch.equal(a, b)
+    with pytest.raises(RuntimeError, match="collected already"):
+        handles[0].collect()
+    # the Python helper returns blocks
+    gs.set_seed(400)
+    nodes, blocks = gs.queue_sample_layers(m, sets[0], fanouts).collect()
+    assert torch.equal(nodes, want[0][-(4 if with_data else 3)]) and len(blocks) == 3
+    # a graph with column ids is sampled layer by layer at the queue call
+    col_ids = to_dev(np.random.default_rng(1).permutation(1 << 13).astype(np.int64), dev)
+    sub = gs.Graph(False)
+    sub._CAPI_LoadCSCWithColIds(col_ids, to_dev(indptr, dev), to_dev(indices, dev))
+    seeds = torch.arange(100, device=dev)
+    gs.set_seed(77)
+    loop = sub._CAPI_SampleLayers(seeds, [4], False)
+    gs.set_seed(77)
+    for a, b in zip(sub._CAPI_QueueSampleLayers(seeds, [4], False).collect(), loop):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("idt", [torch.int32, torch.int64])
 def test_sample_layers_with_no_seeds_and_with_isolated_seeds(dev, idt):
     """No seeds at all, and seeds without neighbours (every later layer is then empty too):
