@@ -118,11 +118,16 @@ struct TileWalk {
   int64_t lo, hi;          // batches of the tile's first and last item
   uint32_t first_bucket;   // bucket_base[lo]
   uint32_t span;           // buckets of batches lo..hi, cut to the LDS counters
-  __device__ __forceinline__ void open(BatchItems<IdT>& x, const Plan& p, int64_t M,
+  // M comes in as the caller's count of items, which may be a bound: the offsets hold the
+  // true one.  False: the tile lies beyond the items (the whole workgroup leaves).
+  __device__ __forceinline__ bool open(BatchItems<IdT>& x, const Plan& p, int64_t& M,
                                        int64_t* s_seeds_ptr, int64_t* s_ids_ptr,
                                        uint32_t* s_base, uint32_t* s_lg, int64_t* s_range,
                                        uint32_t* s_cnt) {
     x.stage_offsets(s_seeds_ptr, s_ids_ptr);
+    const int64_t held = x.seeds_ptr[x.B] + x.ids_ptr[x.B];
+    if (held < M) M = held;
+    if (static_cast<int64_t>(blockIdx.x) * kPartTile >= M) return false;
     for (int64_t b = threadIdx.x; b <= x.B; b += kThreads) {
       s_base[b] = p.bucket_base[b];
       s_lg[b] = b < x.B ? p.classes_log2[b] : 0u;
@@ -135,6 +140,7 @@ struct TileWalk {
     span = all < static_cast<uint32_t>(kCounterCap) ? all : static_cast<uint32_t>(kCounterCap);
     for (uint32_t c = threadIdx.x; c < span; c += kThreads) s_cnt[c] = 0u;
     __syncthreads();
+    return true;
   }
 };
 
@@ -158,7 +164,7 @@ __global__ void __launch_bounds__(kThreads)
 bins_partition_kernel(BatchItems<IdT> x, int64_t M, Bins s) {
   __shared__ PartShared sh;
   TileWalk<IdT> w;
-  w.open(x, s.plan, M, sh.seeds_ptr, sh.ids_ptr, sh.base, sh.lg, sh.range, sh.cnt);
+  if (!w.open(x, s.plan, M, sh.seeds_ptr, sh.ids_ptr, sh.base, sh.lg, sh.range, sh.cnt)) return;
   const int64_t tile_first = static_cast<int64_t>(blockIdx.x) * kPartTile;
   // where every item is: all reads of the thread's items stand together, none behind a
   // condition of its own (the last item again past the end)
@@ -416,6 +422,10 @@ __global__ void __launch_bounds__(kThreads)
 bins_rename_kernel(BatchItems<IdT> x, int64_t M, Bins s, IdT* __restrict__ unique,
                    IdT* __restrict__ out_ids, const int64_t* __restrict__ unique_ptr) {
   __shared__ RenameShared sh;
+  {  // (M may be a bound: the offsets hold the true count)
+    const int64_t held = x.seeds_ptr[x.B] + x.ids_ptr[x.B];
+    if (held < M) M = held;
+  }
   const int64_t chunks = (M + kRenameTile - 1) / kRenameTile;
   const int64_t per = (chunks + kXcds - 1) / kXcds;
   const int64_t chunk = static_cast<int64_t>(blockIdx.x % kXcds) * per + blockIdx.x / kXcds;

@@ -1188,6 +1188,10 @@ size_t gs_batch_relabel_workspace_bytes(int64_t num_items) {
   return a > b ? (a > c ? a : c) : (b > c ? b : c);
 }
 
+size_t gs_batch_relabel_bins_workspace_bytes(int64_t num_items, int64_t num_batches) {
+  return binned_relabel_workspace_bytes(num_items, num_batches);
+}
+
 int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void* ids,
                          const int64_t* ids_ptr, int64_t num_batches, int64_t num_seeds,
                          int64_t num_ids, int id_bytes, void* unique, int64_t* unique_ptr,

@@ -20,6 +20,8 @@ void SetSeed(int64_t seed) { hip::SetSeed(static_cast<uint64_t>(seed)); }
 void SetThreadSeed(int64_t seed) { hip::SetThreadSeed(static_cast<uint64_t>(seed)); }
 void SetSampleAlgo(int64_t algo) { hip::SetSampleAlgo(algo); }
 void SetOrderedSums(bool on) { hip::SetOrderedSums(on); }
+void SetBatchedNoWait(bool on) { hip::SetBatchedNoWait(on); }
+std::vector<int64_t> BatchedNoWaitCounts() { return hip::BatchedNoWaitCounts(); }
 void SetDeferredSampling(bool on) { hip::SetDeferredSampling(on); }
 void DebugRaiseLookbackError(torch::Tensor like) { hip::DebugRaiseLookbackError(like); }
 torch::Tensor UniqueOp(torch::Tensor ids) { return TensorUnique(ids); }
@@ -158,6 +160,11 @@ TORCH_LIBRARY(gs_ops, m) {
   // not in the reference: on = float sums of a COO-only graph add in edge order (same bits
   // every run) at the price of sorting its edges first
   m.def("_CAPI_SetOrderedSums", &SetOrderedSums);
+  // not in the reference: off = _CAPI_SampleLayersBatched waits for every layer's edge count
+  // before its relabel (buffers of the exact sizes) instead of queueing the relabel behind
+  // the sampler
+  m.def("_CAPI_SetBatchedNoWait", &SetBatchedNoWait);
+  m.def("_CAPI_BatchedNoWaitCounts", &BatchedNoWaitCounts);
   // not in the reference: off = every sampling call settles its edge count before returning
   m.def("_CAPI_SetDeferredSampling", &SetDeferredSampling);
   // not in the reference: test hook for the recovery from a look-back that gave up

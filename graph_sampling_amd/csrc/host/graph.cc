@@ -411,7 +411,7 @@ std::vector<torch::Tensor> Graph::LayerwiseBlockIfFused(torch::Tensor seeds, int
   if (U->data_.has_value() &&
       (U->data_.value().scalar_type() != torch::kFloat32 || U->data_.value().dim() != 1))
     return {};
-  const hip::SeedState before = hip::SaveSeedState();
+  const uint64_t seed_before = hip::PeekSeed();
   torch::Tensor prob = U->Sum(1, 2, _CSR);
   torch::Tensor picked = std::get<0>(hip::ListSamplingProbs(GetRows(), prob, fanout, false));
   torch::Tensor nodes, count, kept_key, kept_pos, totals;
@@ -420,7 +420,7 @@ std::vector<torch::Tensor> Graph::LayerwiseBlockIfFused(torch::Tensor seeds, int
   std::tie(kept_key, kept_pos, totals) =
       hip::CooPickRows(U->coo_->row, U->coo_->col, nodes, count, S + picks, &kept);
   if (kept == 0) {
-    hip::RestoreSeedState(before);
+    hip::RewindSeeds(hip::PeekSeed() - seed_before);  // the chain draws for itself
     return {};
   }
   torch::Tensor rows, values, indptr;
@@ -671,8 +671,24 @@ std::vector<std::vector<torch::Tensor>> Graph::SampleLayersBatched(
   struct Layer {
     torch::Tensor frontier, offsets, renamed, data;
     torch::Tensor cuts;  // pinned: [seed cuts | edge cuts | frontier cuts], B + 1 each
+    std::shared_ptr<hip::PendingSample> sample;  // (queued form: kept until the cuts are back)
   };
   std::vector<Layer> layers(L);
+  auto hand_out = [&]() {
+    for (int64_t b = 0; b < B; ++b) out[b].reserve((with_data ? 4 : 3) * L);
+    for (int64_t l = 0; l < L; ++l) {
+      const Layer& y = layers[l];
+      const int64_t* s_cut = y.cuts.data_ptr<int64_t>();
+      const int64_t* e_cut = s_cut + (B + 1);
+      const int64_t* u_cut = e_cut + (B + 1);
+      for (int64_t b = 0; b < B; ++b) {
+        out[b].push_back(hip::Slice1d(y.frontier, u_cut[b], u_cut[b + 1] - u_cut[b]));
+        out[b].push_back(hip::Slice1d(y.offsets, s_cut[b] + b, s_cut[b + 1] - s_cut[b] + 1));
+        out[b].push_back(hip::Slice1d(y.renamed, e_cut[b], e_cut[b + 1] - e_cut[b]));
+        if (with_data) out[b].push_back(hip::Slice1d(y.data, e_cut[b], e_cut[b + 1] - e_cut[b]));
+      }
+    }
+  };
   for (int64_t l = 0; l < L; ++l) {
     Layer& y = layers[l];
     const int64_t S = seeds.numel();
@@ -682,11 +698,28 @@ std::vector<std::vector<torch::Tensor>> Graph::SampleLayersBatched(
     // edges start, and the offsets of every minibatch re-based to its own first edge
     torch::Tensor ids_ptr = p->sub_indptr.index_select(0, ptr);
     y.offsets = hip::IndptrSplit(p->sub_indptr, ptr, S + B);
-    const int64_t nnz = p->Wait();
-    torch::Tensor ids = hip::Slice1d(p->indices, 0, nnz);
-    if (with_data) y.data = hip::Slice1d(p->data, 0, nnz);
+    // The relabel is queued behind the sampler with the edge count still on the device (it
+    // reads its items' number from the offsets; launches and buffers take the sampler's
+    // capacity, which a layer fills to nine tenths and more), so a layer has ONE host wait, for
+    // the frontier's length, which sizes the next layer's launches.  Where that form does not
+    // apply (ids beyond 32 bits, more than 511 minibatches) or reports a status (a bucket's
+    // table full), the edge count is waited for and the relabel done with the exact sizes.
     torch::Tensor uni_ptr;
-    std::tie(y.frontier, uni_ptr, y.renamed) = hip::BatchCsrRelabel(seeds, ptr, ids, ids_ptr);
+    int64_t U = -1;
+    if (hip::BatchedNoWait())
+      std::tie(y.frontier, uni_ptr, y.renamed) =
+          hip::BatchCsrRelabelQueued(seeds, ptr, p->indices, ids_ptr, &U);
+    hip::CountBatchedNoWait(U >= 0);
+    if (U >= 0) {
+      y.frontier = hip::Slice1d(y.frontier, 0, U);
+      if (with_data) y.data = p->data;
+      y.sample = p;
+    } else {
+      const int64_t nnz = p->Wait();
+      torch::Tensor ids = hip::Slice1d(p->indices, 0, nnz);
+      if (with_data) y.data = hip::Slice1d(p->data, 0, nnz);
+      std::tie(y.frontier, uni_ptr, y.renamed) = hip::BatchCsrRelabel(seeds, ptr, ids, ids_ptr);
+    }
     // the cuts go to pinned memory by small kernels of the library (a copy call of the runtime
     // per array cost the host 30-60 us each, a third of the call)
     y.cuts = torch::empty({3 * (B + 1)}, pinned);
@@ -698,19 +731,7 @@ std::vector<std::vector<torch::Tensor>> Graph::SampleLayersBatched(
   }
   // one wait for the cuts of all layers, then views
   hip::WaitPosted(seeds);
-  for (int64_t b = 0; b < B; ++b) out[b].reserve((with_data ? 4 : 3) * L);
-  for (int64_t l = 0; l < L; ++l) {
-    const Layer& y = layers[l];
-    const int64_t* s_cut = y.cuts.data_ptr<int64_t>();
-    const int64_t* e_cut = s_cut + (B + 1);
-    const int64_t* u_cut = e_cut + (B + 1);
-    for (int64_t b = 0; b < B; ++b) {
-      out[b].push_back(hip::Slice1d(y.frontier, u_cut[b], u_cut[b + 1] - u_cut[b]));
-      out[b].push_back(hip::Slice1d(y.offsets, s_cut[b] + b, s_cut[b + 1] - s_cut[b] + 1));
-      out[b].push_back(hip::Slice1d(y.renamed, e_cut[b], e_cut[b + 1] - e_cut[b]));
-      if (with_data) out[b].push_back(hip::Slice1d(y.data, e_cut[b], e_cut[b + 1] - e_cut[b]));
-    }
-  }
+  hand_out();
   return out;
 }
 

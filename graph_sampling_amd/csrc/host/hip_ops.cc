@@ -233,6 +233,23 @@ void SetThreadSeed(uint64_t seed) {
   t_seed = seed;
 }
 uint64_t NextSeed() { return t_own_seed ? t_seed++ : g_seed.fetch_add(1); }
+uint64_t PeekSeed() { return t_own_seed ? t_seed : g_seed.load(); }
+void RewindSeeds(uint64_t n) {
+  if (t_own_seed)
+    t_seed -= n;
+  else
+    g_seed.fetch_sub(n);
+}
+namespace {
+std::atomic<bool> g_batched_no_wait{true};
+std::atomic<int64_t> g_no_wait_counts[2];
+}  // namespace
+std::vector<int64_t> BatchedNoWaitCounts() {
+  return {g_no_wait_counts[0].load(), g_no_wait_counts[1].load()};
+}
+void CountBatchedNoWait(bool went_through) { g_no_wait_counts[went_through ? 0 : 1].fetch_add(1); }
+void SetBatchedNoWait(bool on) { g_batched_no_wait.store(on); }
+bool BatchedNoWait() { return g_batched_no_wait.load(); }
 
 namespace {
 std::atomic<bool> g_ordered_sums{false};
@@ -959,6 +976,46 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(
   }
   TORCH_CHECK(U >= 0, "gs_batch_csr_relabel: a tile gave up waiting for its predecessors");
   return {unique.narrow(0, 0, U), unique_ptr, out_ids};
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabelQueued(
+    const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& ids,
+    const torch::Tensor& ids_ptr, int64_t* num_unique) {
+  const int idb = IdBytes(seeds, "seeds");
+  TORCH_CHECK(IdBytes(ids, "indices") == idb, "seeds and indices differ in dtype");
+  NeedI64(seeds_ptr, "seeds_ptr");
+  NeedI64(ids_ptr, "indices_ptr");
+  TORCH_CHECK(seeds_ptr.numel() == ids_ptr.numel() && seeds_ptr.numel() >= 2,
+              "seeds_ptr and indices_ptr must both hold num_batches + 1 offsets");
+  const int64_t B = seeds_ptr.numel() - 1;
+  const int64_t M = seeds.numel() + ids.numel();
+  const int table_ids = TableIds(idb);
+  // (below half a million items the relabel on hash regions, three launches, is the quicker one:
+  // there the caller's wait for the edge count costs less than the bins' eight launches)
+  if ((idb == 8 && !(table_ids & GS_NARROW_IDS)) || B > 511 || M < (int64_t(1) << 19) ||
+      M >= (int64_t(1) << 30))
+    return {torch::Tensor(), torch::Tensor(), torch::Tensor()};
+  auto unique = torch::empty({M}, seeds.options());
+  auto unique_ptr = torch::empty({B + 1}, I64(seeds));
+  auto out_ids = torch::empty_like(ids);
+  auto ws = Scratch(gs_batch_relabel_bins_workspace_bytes(M, B), seeds);
+  void* st = Stream(seeds);
+  auto num = torch::empty({1}, I64(seeds));
+  HostBoxes& boxes = Boxes(seeds.device().index());
+  const int64_t ticket = boxes.next++;
+  Check(gs_batch_csr_relabel(seeds.data_ptr(), seeds_ptr.data_ptr<int64_t>(), ids.data_ptr(),
+                             ids_ptr.data_ptr<int64_t>(), B, seeds.numel(), ids.numel(),
+                             table_ids | GS_RELABEL_BINS, unique.data_ptr(),
+                             unique_ptr.data_ptr<int64_t>(), out_ids.data_ptr(),
+                             num.data_ptr<int64_t>(), ws.data_ptr(), ws.numel(),
+                             boxes.slot(ticket), ticket, st),
+        "gs_batch_csr_relabel");
+  int64_t U = WaitBox(boxes.slot(ticket), ticket, st, "gs_batch_csr_relabel");
+  if (U == kLost) U = num.item<int64_t>();
+  if (U == kTooWide) t_narrow_ids = false;
+  TORCH_CHECK(U != kGaveUp, "gs_batch_csr_relabel: a tile gave up waiting for its predecessors");
+  *num_unique = U;
+  return {unique, unique_ptr, out_ids};
 }
 
 torch::Tensor IndptrSplit(const torch::Tensor& indptr, const torch::Tensor& offsets,

@@ -28,6 +28,17 @@ void SetSeed(uint64_t seed);
 // not depend on how they interleave.
 void SetThreadSeed(uint64_t seed);
 uint64_t NextSeed();
+// the seed the next NextSeed() of the calling thread will hand out, and n seeds handed back
+// (for a call that drew, found it cannot go on this way, and leaves the draw to another path)
+uint64_t PeekSeed();
+void RewindSeeds(uint64_t n);
+// whether Graph::SampleLayersBatched may queue a layer's relabel behind its sampler without
+// waiting for the edge count (default on)
+void SetBatchedNoWait(bool on);
+bool BatchedNoWait();
+// {layers whose relabel was queued that way, layers that waited for the edge count}, since load
+std::vector<int64_t> BatchedNoWaitCounts();
+void CountBatchedNoWait(bool went_through);
 // off (default): Graph::Sum along the rows (columns) of a graph held as a COO only adds edge
 // by edge with float atomics, so a sum of three or more addends can differ in its last bit
 // from run to run (as on the reference's COO path, src/cuda/graph_ops.cu:45-64).  on: such a
@@ -176,6 +187,17 @@ std::tuple<torch::Tensor, std::vector<torch::Tensor>> Relabel(
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(
     const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& ids,
     const torch::Tensor& ids_ptr);
+// BatchCsrRelabel queued behind a sampler whose edge count has not been read: `ids` is the
+// sampler's buffer, of which the first ids_ptr[B] entries (a device value) count; launches and
+// outputs are sized by the buffer.  {unique (room for all items), unique_ptr, renamed ids (room
+// for all ids)}; *num_unique = the frontiers' total length, waited for here, or a status the
+// caller answers by waiting for the edge count and calling BatchCsrRelabel: -2 an id too wide,
+// -4 a bucket's table full.  Undefined tensors and *num_unique untouched when the path through
+// bins is not the one to take the call (ids that do not ride in 32 bits, more than 511 batches,
+// fewer than 2^19 items by the buffers' sizes).
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabelQueued(
+    const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& ids,
+    const torch::Tensor& ids_ptr, int64_t* num_unique);
 // the batches' offsets, re-based, back to back (host_offsets: the same offsets on the host)
 torch::Tensor IndptrSplit(const torch::Tensor& indptr, const torch::Tensor& offsets,
                           int64_t total);

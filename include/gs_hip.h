@@ -529,6 +529,12 @@ int gs_layer_table_sweep(void* table, size_t table_bytes, const void* workspace,
  * batch's frontier; *num_unique (and the mailbox, when given) = total frontier length.
  * Ids must not be -1.  Workspace: gs_batch_relabel_workspace_bytes(num_seeds+num_ids). */
 size_t gs_batch_relabel_workspace_bytes(int64_t num_items);
+/* With GS_RELABEL_BINS, num_seeds and num_ids may be upper bounds (the sizes of the buffers):
+ * the true counts are seeds_ptr[num_batches] and ids_ptr[num_batches] on the device, launches
+ * and workspace (gs_batch_relabel_bins_workspace_bytes(bound, num_batches) suffices) are sized
+ * by the bounds.  A caller can so queue a relabel behind a sampler whose edge count it has not
+ * read. */
+size_t gs_batch_relabel_bins_workspace_bytes(int64_t num_items, int64_t num_batches);
 int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void* ids,
                          const int64_t* ids_ptr, int64_t num_batches, int64_t num_seeds,
                          int64_t num_ids, int id_bytes, void* unique, int64_t* unique_ptr,

@@ -405,10 +405,25 @@ def test_sample_layers_batched_equals_the_oracle_flow(dev, idt, with_data, sizes
     if with_data:
         g._CAPI_SetData(to_dev(data, dev))
     seed_sets = [rng.permutation(n)[:s].astype(np.int64) for s in sizes]
-    for first in (700, 710):
-        gs.set_seed(first)
-        got = g._CAPI_SampleLayersBatched([to_dev(s, dev, idt) for s in seed_sets], list(fanouts),
-                                          replace)
+    ops = torch.ops.gs_ops
+    # first with every layer's relabel queued behind its sampler (sized by the sampler's capacity,
+    # one host wait a layer), then with the wait for the edge count too (exact sizes): the same
+    # minibatches either way, and from 2^19 items on the first way is the one taken
+    for first, no_wait in ((700, True), (710, False)):
+        through, repeated = ops._CAPI_BatchedNoWaitCounts()
+        ops._CAPI_SetBatchedNoWait(no_wait)
+        try:
+            gs.set_seed(first)
+            got = g._CAPI_SampleLayersBatched([to_dev(s, dev, idt) for s in seed_sets],
+                                              list(fanouts), replace)
+        finally:
+            ops._CAPI_SetBatchedNoWait(True)
+        now = ops._CAPI_BatchedNoWaitCounts()
+        assert now[0] + now[1] == through + repeated + len(fanouts)  # one count per layer
+        if not no_wait:
+            assert now[0] == through
+        elif idt == torch.int32 and len(sizes) == 64:
+            assert now == [through + len(fanouts), repeated]  # 2^19 items and more: all queued
         want = _oracle_super_batch(indptr, indices, seed_sets, fanouts, replace, first, data)
         assert len(got) == len(want)
         for b, (g_b, w_b) in enumerate(zip(got, want)):
