@@ -252,6 +252,31 @@ def main():
         lambda: capi.e_div_u_sum(indices[:2_000_000], coo_cols2m, weights[:2_000_000], divisor,
                                  out_d, out_c),
         lambda o: (2_000_000 * (2 * b + 4 + 4 + 4 + 8), 2_000_000, "edges"))
+    # ---- the tail of a layer-wise sampler on that slice: node set, kept rows, block values --------
+    seeds1k, picks512 = perm_ids(1024), perm_ids(512)
+    run("sorted_union", "gs_sorted_union: 1024 seeds + 512 picked rows, sorted and distinct (one "
+        "workgroup, LDS); 2b per id",
+        lambda: capi.sorted_union(seeds1k, picks512),
+        lambda o: (1536 * 2 * b, 1536, "ids"))
+    hub_rows = torch.sort(torch.unique(indices[:2_000_000])[:1536]).values.contiguous()
+    n_nodes = torch.tensor([hub_rows.numel()], dtype=torch.int64, device=dev)
+    picked = capi.coo_pick_rows(indices[:2_000_000], coo_cols2m, hub_rows, n_nodes, hub_rows.numel())
+    kept = int(picked[2][1])
+    run("coo_pick_rows", "gs_coo_pick_rows: the 2M edges of the slice against 1536 rows (binary "
+        "search of the set in LDS; count, scan, fill), %d kept; b B per edge looked at + 4 (its "
+        "place, written and read), 3b per edge kept" % kept,
+        lambda: capi.coo_pick_rows(indices[:2_000_000], coo_cols2m, hub_rows, n_nodes,
+                                   hub_rows.numel()),
+        lambda o: (2_000_000 * (b + 8) + kept * 3 * b, 2_000_000, "edges"))
+    k_key, k_pos = picked[0][:kept].contiguous(), picked[1][:kept].contiguous()
+    num_cols2m = int(coo_cols2m.max()) + 1
+    run("coo_block_values", "gs_coo_block_values: those kept edges put in block order column by "
+        "column (counting sort in LDS) with value = w / divisor[row]; 2b read, b + 4 + 8 "
+        "gathered, b + 4 written per kept edge, 8 B per column",
+        lambda: capi.coo_block_values(k_key, k_pos, hub_rows.numel(), indices[:2_000_000],
+                                      weights[:2_000_000], divisor, num_cols2m),
+        lambda o: (kept * (4 * b + 16) + num_cols2m * 8, kept, "edges"))
+
     out_nrm = torch.empty(E, device=dev)
     run("segment_normalize", "gs_segment_normalize over every column of the graph; 4 B read twice + "
         "4 B written per edge, 16 B per column",

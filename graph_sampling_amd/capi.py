@@ -37,7 +37,8 @@ def lib():
                      "gs_relabel_sampled_workspace_bytes", "gs_relabel_sampled_state_bytes",
                      "gs_segment_workspace_bytes", "gs_layer_workspace_bytes",
                      "gs_layer_sample_state_bytes", "gs_layer_relabel_state_bytes",
-                     "gs_coo_sum_workspace_bytes", "gs_coo_pick_rows_workspace_bytes"):
+                     "gs_coo_sum_workspace_bytes", "gs_coo_pick_rows_workspace_bytes",
+                     "gs_coo_block_values_workspace_bytes"):
             if hasattr(_lib, name):
                 getattr(_lib, name).restype = ctypes.c_size_t
         _lib.gs_sorted_union_max.restype = ctypes.c_int64
@@ -900,10 +901,12 @@ def coo_block_values(kept_key, kept_pos, max_nodes, row, data, divisor, num_cols
     out_row = torch.empty(kept, dtype=row.dtype, device=row.device)
     out_value = torch.empty(kept, dtype=torch.float32, device=row.device)
     out_indptr = torch.empty(num_cols + 1, dtype=torch.int64, device=row.device)
+    ws = workspace(lib().gs_coo_block_values_workspace_bytes(_i64(kept)), row.device)
     _check(lib().gs_coo_block_values(_ptr(kept_key), _ptr(kept_pos), _i64(kept), _i64(max_nodes),
                                      _ptr(row), idb, _ptr(data), _ptr(divisor), _i64(num_cols),
-                                     _ptr(out_row), _ptr(out_value), _ptr(out_indptr),
-                                     _stream(row.device)), "gs_coo_block_values")
+                                     _ptr(out_row), _ptr(out_value), _ptr(out_indptr), _ptr(ws),
+                                     ctypes.c_size_t(ws.numel()), _stream(row.device)),
+           "gs_coo_block_values")
     return out_row, out_value, out_indptr
 
 

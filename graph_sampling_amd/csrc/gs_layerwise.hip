@@ -174,8 +174,10 @@ struct LoadCounts {
 template <typename IdT>
 __global__ void __launch_bounds__(256)
 column_offsets_kernel(const IdT* __restrict__ kept_key, int64_t kept, int node_bits,
-                      int64_t num_cols, int64_t* __restrict__ out_indptr) {
+                      int64_t num_cols, int64_t* __restrict__ out_indptr,
+                      unsigned int* __restrict__ num_long) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i == 0) *num_long = 0u;  // (the list of long columns is made by the next launch)
   if (kept == 0) {
     for (int64_t c = i; c <= num_cols; c += static_cast<int64_t>(gridDim.x) * 256) out_indptr[c] = 0;
     return;
@@ -205,18 +207,73 @@ constexpr int kColumnBatch = 4;
 constexpr int kFourWavesBits = 11;
 constexpr int kRankShift = 13;  // a key has at most 13 bits, a rank inside a quarter 12
 
+constexpr int kShortColumn = 256;
+
+// The columns with more than kShortColumn kept edges, listed for the workgroups that order them
+// in LDS (a thread a column).
+__global__ void __launch_bounds__(256)
+long_columns_kernel(const int64_t* __restrict__ indptr, int64_t num_cols,
+                    unsigned int* __restrict__ num_long, unsigned int* __restrict__ long_columns) {
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (c < num_cols && indptr[c + 1] - indptr[c] > kShortColumn)
+    long_columns[atomicAdd(num_long, 1u)] = static_cast<unsigned int>(c);
+}
+
+// The short columns (up to 256 kept edges: nearly all of them) by edge: a thread takes one kept
+// edge, finds its column's range in the offsets, and counts the column's edges that come before
+// its own by (key, position) -- the keys of a column lie side by side and the threads of a
+// column read the same ones, out of the caches.  (A workgroup per column, long or short, cost
+// 116 us for 82 k edges over 40 k columns: tens of thousands of workgroups with two edges each.)
+template <typename IdT>
+__device__ __forceinline__ void order_short_edge(int64_t i, const IdT* __restrict__ kept_key,
+                                                 const IdT* __restrict__ kept_pos, int node_bits,
+                                                 const int64_t* __restrict__ indptr,
+                                                 const IdT* __restrict__ row,
+                                                 const float* __restrict__ data,
+                                                 const float* __restrict__ divisor,
+                                                 IdT* __restrict__ out_row,
+                                                 float* __restrict__ out_value) {
+  const unsigned long long key = static_cast<unsigned long long>(kept_key[i]);
+  const int64_t e = static_cast<int64_t>(kept_pos[i]);
+  const int64_t column = static_cast<int64_t>(key >> node_bits);
+  const int64_t lo = indptr[column], hi = indptr[column + 1];
+  if (hi - lo > kShortColumn) return;  // (a long column: its own workgroup's)
+  const IdT r = row[e];
+  const float w = data ? data[e] : 1.0f;
+  const float d = divisor[r];
+  int64_t before = 0;
+  for (int64_t j = lo; j < hi; ++j) {
+    const unsigned long long y = static_cast<unsigned long long>(kept_key[j]);
+    before += (y < key) || (y == key && j < i);  // (one column: the keys differ in the place only)
+  }
+  out_row[lo + before] = r;
+  out_value[lo + before] = w / d;
+}
+
 template <typename IdT, bool FOUR_WAVES>
 __global__ void __launch_bounds__(256)
 order_columns_kernel(const IdT* __restrict__ kept_key, const IdT* __restrict__ kept_pos,
                      int node_bits, const int64_t* __restrict__ indptr,
                      const IdT* __restrict__ row, const float* __restrict__ data,
                      const float* __restrict__ divisor, IdT* __restrict__ out_row,
-                     float* __restrict__ out_value) {
+                     float* __restrict__ out_value, const unsigned int* __restrict__ num_long,
+                     const unsigned int* __restrict__ long_columns, unsigned int long_blocks,
+                     int64_t kept) {
   extern __shared__ unsigned long long s_raw[];
   __shared__ int64_t s_scan[256 / kWave + 1];
-  const int64_t lo = indptr[blockIdx.x], hi = indptr[blockIdx.x + 1];
+  // the launch's first long_blocks workgroups take a listed long column each, the others 256
+  // kept edges of short columns: both kinds run side by side
+  if (blockIdx.x >= long_blocks) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x - long_blocks) * 256 + threadIdx.x;
+    if (i < kept)
+      order_short_edge(i, kept_key, kept_pos, node_bits, indptr, row, data, divisor, out_row,
+                       out_value);
+    return;
+  }
+  if (blockIdx.x >= *num_long) return;
+  const unsigned int column = long_columns[blockIdx.x];
+  const int64_t lo = indptr[column], hi = indptr[column + 1];
   const int64_t len = hi - lo;
-  if (len == 0) return;
   const int places = 1 << node_bits;
   const unsigned int mask = static_cast<unsigned int>(places) - 1u;
   unsigned int* s_bin = reinterpret_cast<unsigned int*>(s_raw);
@@ -362,22 +419,30 @@ order_columns_kernel(const IdT* __restrict__ kept_key, const IdT* __restrict__ k
 }
 
 template <typename IdT>
-void order_columns_launch(dim3 grid, int node_bits, hipStream_t st, const void* kept_key,
-                          const void* kept_pos, const int64_t* indptr, const void* row,
-                          const float* data, const float* divisor, void* out_row, float* out_value) {
+void order_columns_launch(int64_t num_cols, int64_t kept, int node_bits, hipStream_t st,
+                          const void* kept_key, const void* kept_pos, const int64_t* indptr,
+                          const void* row, const float* data, const float* divisor, void* out_row,
+                          float* out_value, unsigned int* num_long, unsigned int* long_columns) {
+  hipLaunchKernelGGL(long_columns_kernel, dim3(static_cast<unsigned>(blocks_for(num_cols, 256))),
+                     dim3(256), 0, st, indptr, num_cols, num_long, long_columns);
+  // at most kept / 257 columns are long
+  const unsigned int long_blocks = static_cast<unsigned int>(kept / (kShortColumn + 1) + 1);
+  const dim3 grid(long_blocks + static_cast<unsigned>(blocks_for(kept, 256)));
   const size_t places = size_t(1) << node_bits;
   if (node_bits <= kFourWavesBits)
     hipLaunchKernelGGL((order_columns_kernel<IdT, true>), grid, dim3(256),
                        (places + kColumnStage + 2 * places) * sizeof(unsigned int), st,
                        static_cast<const IdT*>(kept_key), static_cast<const IdT*>(kept_pos), node_bits,
                        indptr, static_cast<const IdT*>(row), data, divisor,
-                       static_cast<IdT*>(out_row), out_value);
+                       static_cast<IdT*>(out_row), out_value, num_long, long_columns, long_blocks,
+                       kept);
   else
     hipLaunchKernelGGL((order_columns_kernel<IdT, false>), grid, dim3(256),
                        (places + kColumnStage) * sizeof(unsigned int), st,
                        static_cast<const IdT*>(kept_key), static_cast<const IdT*>(kept_pos), node_bits,
                        indptr, static_cast<const IdT*>(row), data, divisor,
-                       static_cast<IdT*>(out_row), out_value);
+                       static_cast<IdT*>(out_row), out_value, num_long, long_columns, long_blocks,
+                       kept);
 }
 
 inline int bits_of(int64_t n) {  // smallest b with 2^b >= n
@@ -480,10 +545,16 @@ int gs_coo_pick_rows(const void* row, const void* col, int id_bytes, int64_t E, 
                                               totals, mailbox, ticket, workspace, workspace_bytes, st);
 }
 
+size_t gs_coo_block_values_workspace_bytes(int64_t kept) {
+  if (kept < 0) kept = 0;
+  return 256 + ((static_cast<size_t>(kept / (kShortColumn + 1) + 1) * sizeof(unsigned int) + 255u) &
+                ~size_t(255));
+}
+
 int gs_coo_block_values(const void* kept_key, const void* kept_pos, int64_t kept, int64_t max_nodes,
                         const void* row, int id_bytes, const float* data, const float* divisor,
                         int64_t num_cols, void* out_row, float* out_value, int64_t* out_indptr,
-                        void* stream) {
+                        void* workspace, size_t workspace_bytes, void* stream) {
   GS_REQUIRE(valid_id_bytes(id_bytes), "gs_coo_block_values: id_bytes must be 4 or 8, got %d",
              id_bytes);
   GS_REQUIRE(kept >= 0 && num_cols >= 0, "gs_coo_block_values: negative size");
@@ -492,22 +563,31 @@ int gs_coo_block_values(const void* kept_key, const void* kept_pos, int64_t kept
              static_cast<long long>(max_nodes), static_cast<long long>(gs_sorted_union_max(id_bytes)));
   GS_REQUIRE(out_indptr && (kept == 0 || (kept_key && kept_pos && row && divisor && out_row && out_value)),
              "gs_coo_block_values: null pointer");
+  Carver ws(workspace, workspace_bytes);
+  unsigned int* num_long = ws.take<unsigned int>(1);
+  unsigned int* long_columns = ws.take<unsigned int>(static_cast<size_t>(kept / (kShortColumn + 1) + 1));
+  if (!ws.ok) {
+    set_error_text("gs_coo_block_values: workspace needs %zu bytes, 256-byte aligned",
+                   gs_coo_block_values_workspace_bytes(kept));
+    return GS_ERR_WORKSPACE;
+  }
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int node_bits = bits_of(max_nodes);
   const dim3 by_edge(static_cast<unsigned>(blocks_for(kept, 256)));
-  const dim3 by_column(static_cast<unsigned>(num_cols));
   if (id_bytes == 8) {
     hipLaunchKernelGGL(column_offsets_kernel<int64_t>, by_edge, dim3(256), 0, st,
-                       static_cast<const int64_t*>(kept_key), kept, node_bits, num_cols, out_indptr);
+                       static_cast<const int64_t*>(kept_key), kept, node_bits, num_cols, out_indptr,
+                       num_long);
     if (kept > 0 && num_cols > 0)
-      order_columns_launch<int64_t>(by_column, node_bits, st, kept_key, kept_pos, out_indptr, row, data,
-                                    divisor, out_row, out_value);
+      order_columns_launch<int64_t>(num_cols, kept, node_bits, st, kept_key, kept_pos, out_indptr, row,
+                                    data, divisor, out_row, out_value, num_long, long_columns);
   } else {
     hipLaunchKernelGGL(column_offsets_kernel<int32_t>, by_edge, dim3(256), 0, st,
-                       static_cast<const int32_t*>(kept_key), kept, node_bits, num_cols, out_indptr);
+                       static_cast<const int32_t*>(kept_key), kept, node_bits, num_cols, out_indptr,
+                       num_long);
     if (kept > 0 && num_cols > 0)
-      order_columns_launch<int32_t>(by_column, node_bits, st, kept_key, kept_pos, out_indptr, row, data,
-                                    divisor, out_row, out_value);
+      order_columns_launch<int32_t>(num_cols, kept, node_bits, st, kept_key, kept_pos, out_indptr, row,
+                                    data, divisor, out_row, out_value, num_long, long_columns);
   }
   return check_launch("coo_block_values");
 }

@@ -1409,10 +1409,11 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> CooBlockValues(
   auto out_row = torch::empty({kept}, row.options());
   auto out_value = torch::empty({kept}, divisor.options());
   auto out_indptr = torch::empty({num_cols + 1}, I64(row));
+  auto ws = Scratch(gs_coo_block_values_workspace_bytes(kept), row);
   Check(gs_coo_block_values(kept_key.data_ptr(), kept_pos.data_ptr(), kept, max_nodes, row.data_ptr(),
                             idb, values, divisor.data_ptr<float>(), num_cols, out_row.data_ptr(),
                             out_value.data_ptr<float>(), out_indptr.data_ptr<int64_t>(),
-                            Stream(row)),
+                            ws.data_ptr(), ws.numel(), Stream(row)),
         "gs_coo_block_values");
   return {out_row, out_value, out_indptr};
 }

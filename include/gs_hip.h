@@ -753,10 +753,11 @@ int gs_coo_pick_rows(const void* row, const void* col, int id_bytes, int64_t E, 
  * all kept edges by kept_key, done column by column in LDS -- and leave as out_row = their row
  * ids and out_value = data[pos] / divisor[row] (data NULL: ones; divisor is indexed by row id);
  * out_indptr[num_cols + 1] = the offsets of the columns. */
+size_t gs_coo_block_values_workspace_bytes(int64_t kept);
 int gs_coo_block_values(const void* kept_key, const void* kept_pos, int64_t kept, int64_t max_nodes,
                         const void* row, int id_bytes, const float* data, const float* divisor,
                         int64_t num_cols, void* out_row, float* out_value, int64_t* out_indptr,
-                        void* stream);
+                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Format conversion: replaces impl::CSC2COOCUDA and impl::COO2CSCCUDA          */
