@@ -95,7 +95,8 @@ typedef struct gs_mailbox {
  * record a hipEvent pair on its stream (up to 4096 launches); NULL or ""
  * disables.  Sites: "sample_fused", "sample_floyd", "table_init", "table_insert",
  * "unique_compact", "unique_finish", "layer_sample", "layer_relabel", "layer_sweep",
- * "batch_init", "batch_insert", "batch_compact", "batch_finish", "scan_tile_sums",
+ * "batch_init", "batch_insert", "batch_compact", "batch_finish", "bins_init", "bins_count",
+ * "bins_scatter", "bins_flag", "bins_rank", "bins_rename", "scan_tile_sums",
  * "scan_apply", "random_walk", "metapath_walk", "sddmm_dot".  gs_profile_collect waits for the recorded
  * events, returns their summed duration and count (and, when per_launch_ms is
  * given, the first `cap` individual durations in launch order) and clears the
@@ -750,9 +751,10 @@ int gs_coo_pick_rows(const void* row, const void* col, int id_bytes, int64_t E, 
 /* The block of the kept edges (kept_key / kept_pos [kept] as gs_coo_pick_rows leaves them for a
  * COO whose edges come by column, with the same max_nodes): inside every column the edges are
  * put in the order of their rows (ties: of their positions) -- the order of a stable sort of
- * all kept edges by kept_key, done column by column in LDS -- and leave as out_row = their row
+ * all kept edges by kept_key, done column by column -- and leave as out_row = their row
  * ids and out_value = data[pos] / divisor[row] (data NULL: ones; divisor is indexed by row id);
- * out_indptr[num_cols + 1] = the offsets of the columns. */
+ * out_indptr[num_cols + 1] = the offsets of the columns.  Workspace (the list of the columns
+ * with more than 256 kept edges): gs_coo_block_values_workspace_bytes(kept). */
 size_t gs_coo_block_values_workspace_bytes(int64_t kept);
 int gs_coo_block_values(const void* kept_key, const void* kept_pos, int64_t kept, int64_t max_nodes,
                         const void* row, int id_bytes, const float* data, const float* divisor,
