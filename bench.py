@@ -816,6 +816,24 @@ def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted):
     sb_sizes = sizes_of(results[-1])
     sb_edges = sum(sum(z[1] for z in sizes_of(res)) for res in results)
     del results
+    # the same calls in two halves, super-batch i + 1 queued before super-batch i is collected:
+    # the host's share of a call then runs while the stream works on the last layer
+    def queued(grp):
+        return graph._CAPI_QueueSampleLayersBatched(grp, list(FANOUTS), False)
+
+    results = []
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ahead = queued(groups[0])
+    for grp in groups[1:]:
+        nxt = queued(grp)
+        results.append(ahead.collect())
+        ahead = nxt
+    results.append(ahead.collect())
+    torch.cuda.synchronize()
+    qa_s = time.perf_counter() - t1
+    qa_edges = sum(sum(z[1] for z in sizes_of(res)) for res in results)
+    del results, ahead, nxt
     super_batch(torch, graph, groups[0])
     torch.cuda.synchronize()
     t1 = time.perf_counter()
@@ -846,6 +864,10 @@ def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted):
         "ms_per_call": sb_s / len(groups) * 1e3,
         "layers_S_E_U": sb_sizes,
         "api": "gs_classes.Graph._CAPI_SampleLayersBatched (one call per super-batch)",
+        "queued_ahead": {
+            "ms_per_call": qa_s / len(groups) * 1e3, "value": qa_edges / qa_s,
+            "what": "_CAPI_QueueSampleLayersBatched of super-batch i + 1 before .collect() of "
+                    "super-batch i (one thread, one stream)"},
         "through_python_ops": {
             "ms_per_minibatch": py_s / (len(groups) * SUPER) * 1e3, "value": py_edges / py_s,
             "what": "the same flow as _CAPI_FusedColumnwiseSlicingSampling + GetBatchCSC + "

@@ -120,6 +120,30 @@ def queue_sample_layers(matrix, seeds, fanouts, replace=False):
     return _QueuedMinibatch(graph._CAPI_QueueSampleLayers(seeds, fanouts, bool(replace)), len(fanouts))
 
 
+class _QueuedSuperBatch(object):
+    """A super-batch whose launches are queued; `collect()` waits for it and returns what
+    `sample_blocks_batched` returns."""
+
+    def __init__(self, handle, num_layers):
+        self._handle, self._num_layers = handle, num_layers
+
+    def collect(self):
+        return [_blocks_of(parts, self._num_layers) for parts in self._handle.collect()]
+
+
+def queue_sample_blocks_batched(matrix, seed_sets, fanouts, replace=False):
+    """`sample_blocks_batched` in two halves: the call returns when the last layer's launches
+    are queued, `.collect()` of the returned object waits for them and hands over the
+    minibatches.  Queue super-batch i + 1 before collecting super-batch i and the host's share
+    of a call (concatenating the seeds, the per-minibatch views) runs while the stream is busy.
+    Not in the reference."""
+    load_library()
+    graph = getattr(matrix, "_graph", matrix)
+    fanouts = list(fanouts)
+    return _QueuedSuperBatch(
+        graph._CAPI_QueueSampleLayersBatched(list(seed_sets), fanouts, bool(replace)), len(fanouts))
+
+
 def sample_blocks_batched(matrix, seed_sets, fanouts, replace=False):
     """GraphSAGE-style minibatches sampled as ONE launch sequence per layer (a "super-batch": the
     flow of the reference's examples/graphsage/batching.py:59-98 -- fused sampling over the

@@ -865,6 +865,60 @@ def post_total(values, at, box):
     return box.wait(ticket, values.device)
 
 
+def post_values(values, box):
+    """gs_post_values: a device int64 array to pinned host memory; returns the pinned tensor once
+    the mailbox says it has landed."""
+    _need(values, torch.int64, "values")
+    out = torch.empty(values.numel(), dtype=torch.int64).pin_memory()
+    ticket = box.ticket()
+    _check(lib().gs_post_values(_ptr(values), _i64(values.numel()),
+                                ctypes.c_void_p(out.data_ptr()), box.ptr(), _i64(ticket),
+                                _stream(values.device)), "gs_post_values")
+    got = box.wait(ticket, values.device)
+    if got != values.numel():
+        raise GsError("gs_post_values posted %d values, expected %d" % (got, values.numel()))
+    return out
+
+
+def post_value_sets(sets, box):
+    """gs_post_value_sets: several device int64 arrays of one length to pinned host memory by
+    one launch; returns a pinned [len(sets), n] tensor once the mailbox says it has landed."""
+    n = sets[0].numel() if sets else 0
+    for t in sets:
+        _need(t, torch.int64, "values")
+        if t.numel() != n:
+            raise ValueError("the arrays must have one length")
+    out = torch.empty((len(sets), n), dtype=torch.int64).pin_memory()
+    at = (ctypes.c_void_p * max(len(sets), 1))(*[t.data_ptr() for t in sets])
+    ticket = box.ticket()
+    dev = sets[0].device if sets else torch.device("cuda", torch.cuda.current_device())
+    _check(lib().gs_post_value_sets(at, len(sets), _i64(n), ctypes.c_void_p(out.data_ptr()),
+                                    box.ptr(), _i64(ticket), _stream(dev)), "gs_post_value_sets")
+    got = box.wait(ticket, dev)
+    if got != len(sets) * n:
+        raise GsError("gs_post_value_sets posted %d values, expected %d" % (got, len(sets) * n))
+    return out
+
+
+def indptr_split(indptr, offsets, with_cuts=False):
+    """gs_indptr_split / gs_indptr_split_cuts: the batches' offsets re-based and laid out back to
+    back; with_cuts also returns indptr[offsets] from the same launch."""
+    _need(indptr, torch.int64, "indptr")
+    _need(offsets, torch.int64, "offsets")
+    B = offsets.numel() - 1
+    span = int(offsets[-1] - offsets[0]) if B >= 1 else 0
+    total = span + B
+    out = torch.empty(total, dtype=torch.int64, device=indptr.device)
+    if not with_cuts:
+        _check(lib().gs_indptr_split(_ptr(indptr), _ptr(offsets), _i64(B), _i64(total), _ptr(out),
+                                     _stream(indptr.device)), "gs_indptr_split")
+        return out
+    cuts = torch.empty(B + 1, dtype=torch.int64, device=indptr.device)
+    _check(lib().gs_indptr_split_cuts(_ptr(indptr), _ptr(offsets), _i64(B), _i64(total), _ptr(out),
+                                      _ptr(cuts), _stream(indptr.device)), "gs_indptr_split_cuts")
+    return out, cuts
+
+
 def coo_pick_rows(row, col, nodes, count, max_nodes, box=None):
     """gs_coo_pick_rows.  Returns (kept_key, kept_pos, totals: device int64[2]); with a
     mailbox `box` the number of kept edges is waited for and returned as a fourth value."""

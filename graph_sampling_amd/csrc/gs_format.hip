@@ -518,7 +518,8 @@ constexpr int kSplitStage = 1024;
 
 __global__ void __launch_bounds__(kThreads)
 indptr_split_kernel(const int64_t* __restrict__ indptr, const int64_t* __restrict__ offsets,
-                    int64_t B, int64_t total, int64_t* __restrict__ out) {
+                    int64_t B, int64_t total, int64_t* __restrict__ out,
+                    int64_t* __restrict__ cuts) {
   __shared__ int64_t s_off[kSplitStage];
   const bool staged = B <= kSplitStage;
   if (staged) {
@@ -527,6 +528,8 @@ indptr_split_kernel(const int64_t* __restrict__ indptr, const int64_t* __restric
   }
   const int64_t* off = staged ? s_off : offsets;
   const int64_t q = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  // where every batch's entries start (and the last one's end), for the caller's next cut
+  if (cuts && q <= B) cuts[q] = indptr[offsets[q]];
   if (q >= total) return;
   int64_t lo = 0, hi = B - 1;  // last b with offsets[b] + b <= q
   while (lo < hi) {
@@ -893,11 +896,18 @@ int gs_coo2csc(const void* key, const void* value, int id_bytes, int64_t E, int6
 
 int gs_indptr_split(const int64_t* indptr, const int64_t* offsets, int64_t num_batches,
                     int64_t total, int64_t* out, void* stream) {
+  return gs_indptr_split_cuts(indptr, offsets, num_batches, total, out, nullptr, stream);
+}
+
+int gs_indptr_split_cuts(const int64_t* indptr, const int64_t* offsets, int64_t num_batches,
+                         int64_t total, int64_t* out, int64_t* cuts, void* stream) {
   GS_REQUIRE(num_batches >= 0 && total >= 0, "gs_indptr_split: negative size");
-  if (num_batches == 0 || total == 0) return GS_OK;
-  GS_REQUIRE(indptr && offsets && out, "gs_indptr_split: null pointer");
-  hipLaunchKernelGGL(indptr_split_kernel, dim3(blocks_for(total, kThreads)), dim3(kThreads), 0,
-                     static_cast<hipStream_t>(stream), indptr, offsets, num_batches, total, out);
+  if (num_batches == 0 || (total == 0 && !cuts)) return GS_OK;
+  GS_REQUIRE(indptr && offsets && (out || total == 0), "gs_indptr_split: null pointer");
+  const int64_t lanes = cuts && num_batches + 1 > total ? num_batches + 1 : total;
+  hipLaunchKernelGGL(indptr_split_kernel, dim3(blocks_for(lanes, kThreads)), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), indptr, offsets, num_batches, total, out,
+                     cuts);
   return check_launch("indptr_split");
 }
 

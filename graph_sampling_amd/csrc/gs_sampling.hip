@@ -120,6 +120,25 @@ post_values_kernel(const int64_t* __restrict__ values, int64_t n, int64_t* out, 
   if (threadIdx.x == 0) post_mailbox(box, n, ticket);
 }
 
+// several arrays of n values each, one after the other, by one workgroup
+constexpr int kPostSetsMax = 32;
+struct PostSets {
+  const int64_t* set[kPostSetsMax];
+};
+
+__global__ void __launch_bounds__(256)
+post_value_sets_kernel(PostSets sets, int num_sets, int64_t n, int64_t* out, gs_mailbox* box,
+                       int64_t ticket) {
+  for (int s = 0; s < num_sets; ++s) {
+    const int64_t* __restrict__ values = sets.set[s];
+    for (int64_t i = threadIdx.x; i < n; i += 256)
+      __hip_atomic_store(&out[s * n + i], values[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+  __threadfence_system();
+  __syncthreads();
+  if (threadIdx.x == 0) post_mailbox(box, static_cast<int64_t>(num_sets) * n, ticket);
+}
+
 template <typename IdT, bool WITH_COO, bool WITH_DATA>
 __global__ void __launch_bounds__(kFillThreads)
 slice_fill_kernel(const int64_t* __restrict__ indptr, const IdT* __restrict__ indices,
@@ -1330,6 +1349,22 @@ int gs_post_values(const int64_t* values, int64_t n, int64_t* host_out, gs_mailb
   GS_REQUIRE(n >= 0 && (n == 0 || (values && host_out)), "gs_post_values: null pointer or negative size");
   hipLaunchKernelGGL(post_values_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream),
                      values, n, host_out, mailbox, ticket);
+  return check_launch("post_values");
+}
+
+int gs_post_value_sets(const int64_t* const* sets, int num_sets, int64_t n, int64_t* host_out,
+                       gs_mailbox* mailbox, int64_t ticket, void* stream) {
+  GS_REQUIRE(num_sets >= 0 && num_sets <= kPostSetsMax && n >= 0,
+             "gs_post_value_sets: between 0 and %d arrays of a non-negative length", kPostSetsMax);
+  GS_REQUIRE(num_sets == 0 || n == 0 || (sets && host_out), "gs_post_value_sets: null pointer");
+  PostSets by_value = {};
+  for (int s = 0; s < num_sets; ++s) {
+    GS_REQUIRE(n == 0 || sets[s], "gs_post_value_sets: null array");
+    by_value.set[s] = sets[s];
+  }
+  hipLaunchKernelGGL(post_value_sets_kernel, dim3(1), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), by_value, num_sets, n, host_out, mailbox,
+                     ticket);
   return check_launch("post_values");
 }
 

@@ -33,6 +33,9 @@ TORCH_LIBRARY(gs_classes, m) {
   // not in the reference: a minibatch whose launches are queued and whose results are
   // collected later (Graph::QueueSampleLayers)
   m.class_<QueuedLayers>("QueuedLayers") GS_DEF2("_CAPI_Collect", "collect", &QueuedLayers::Collect);
+  // the same for a super-batch (Graph::QueueSampleLayersBatched)
+  m.class_<QueuedSuperBatch>("QueuedSuperBatch")
+      GS_DEF2("_CAPI_Collect", "collect", &QueuedSuperBatch::Collect);
 
   m.class_<Graph>("Graph")
       .def(torch::init<bool>())
@@ -56,6 +59,8 @@ TORCH_LIBRARY(gs_classes, m) {
       GS_DEF2("_CAPI_LayerwiseBlockIfFused", "_CAPI_layerwise_block_if_fused",
               &Graph::LayerwiseBlockIfFused)
       GS_DEF2("_CAPI_QueueSampleLayers", "_CAPI_queue_sample_layers", &Graph::QueueSampleLayers)
+      GS_DEF2("_CAPI_QueueSampleLayersBatched", "_CAPI_queue_sample_layers_batched",
+              &Graph::QueueSampleLayersBatched)
       GS_DEF2("_CAPI_FusionSlicing", "_CAPI_fusion_slicing", &Graph::FusedBidirSlicing)
       GS_DEF2("_CAPI_BatchFusionSlicing", "_CAPI_batch_fusion_slicing",
               &Graph::BatchFusedBidirSlicing)

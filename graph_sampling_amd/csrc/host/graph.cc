@@ -633,13 +633,21 @@ std::vector<torch::Tensor> Graph::SampleLayers(torch::Tensor seeds, std::vector<
 std::vector<std::vector<torch::Tensor>> Graph::SampleLayersBatched(
     const std::vector<torch::Tensor>& seed_sets, const std::vector<int64_t>& fanouts,
     bool replace) {
+  return QueueSampleLayersBatched(seed_sets, fanouts, replace)->Collect();
+}
+
+c10::intrusive_ptr<QueuedSuperBatch> Graph::QueueSampleLayersBatched(
+    const std::vector<torch::Tensor>& seed_sets, const std::vector<int64_t>& fanouts,
+    bool replace) {
   Range range("gs::SampleLayersBatched");
   Settle();
   TORCH_CHECK(csc_ != nullptr, "fused slicing + sampling needs the CSC format");
   const int64_t B = static_cast<int64_t>(seed_sets.size());
   const int64_t L = static_cast<int64_t>(fanouts.size());
-  std::vector<std::vector<torch::Tensor>> out(B);
-  if (B == 0 || L == 0) return out;
+  auto q = c10::make_intrusive<QueuedSuperBatch>();
+  q->num_batches = B;
+  q->ready.resize(B);
+  if (B == 0 || L == 0) return q;
   // what the one launch sequence cannot take goes minibatch by minibatch
   bool one_sequence = !col_ids_.has_value() && !row_ids_.has_value() && !val_col_ids_.has_value() &&
                       hip::DeferredSampling() &&
@@ -656,10 +664,11 @@ std::vector<std::vector<torch::Tensor>> Graph::SampleLayersBatched(
     bound *= 1 + k;
   }
   if (!one_sequence) {
-    for (int64_t b = 0; b < B; ++b) out[b] = SampleLayers(seed_sets[b], fanouts, replace);
-    return out;
+    for (int64_t b = 0; b < B; ++b) q->ready[b] = SampleLayers(seed_sets[b], fanouts, replace);
+    return q;
   }
   const bool with_data = data_.has_value();
+  q->with_data = with_data;
   const hip::EdgeData edge{with_data ? data_.value() : torch::Tensor(), csc_->e_ids};
   auto pinned = torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true);
   std::vector<int64_t> cut(B + 1, 0);
@@ -668,36 +677,20 @@ std::vector<std::vector<torch::Tensor>> Graph::SampleLayersBatched(
   std::copy(cut.begin(), cut.end(), host_ptr.data_ptr<int64_t>());
   torch::Tensor ptr = host_ptr.to(csc_->indptr.device(), /*non_blocking=*/true);
   torch::Tensor seeds = torch::cat(seed_sets);
-  struct Layer {
-    torch::Tensor frontier, offsets, renamed, data;
-    torch::Tensor cuts;  // pinned: [seed cuts | edge cuts | frontier cuts], B + 1 each
-    std::shared_ptr<hip::PendingSample> sample;  // (queued form: kept until the cuts are back)
-  };
-  std::vector<Layer> layers(L);
-  auto hand_out = [&]() {
-    for (int64_t b = 0; b < B; ++b) out[b].reserve((with_data ? 4 : 3) * L);
-    for (int64_t l = 0; l < L; ++l) {
-      const Layer& y = layers[l];
-      const int64_t* s_cut = y.cuts.data_ptr<int64_t>();
-      const int64_t* e_cut = s_cut + (B + 1);
-      const int64_t* u_cut = e_cut + (B + 1);
-      for (int64_t b = 0; b < B; ++b) {
-        out[b].push_back(hip::Slice1d(y.frontier, u_cut[b], u_cut[b + 1] - u_cut[b]));
-        out[b].push_back(hip::Slice1d(y.offsets, s_cut[b] + b, s_cut[b + 1] - s_cut[b] + 1));
-        out[b].push_back(hip::Slice1d(y.renamed, e_cut[b], e_cut[b + 1] - e_cut[b]));
-        if (with_data) out[b].push_back(hip::Slice1d(y.data, e_cut[b], e_cut[b + 1] - e_cut[b]));
-      }
-    }
-  };
+  q->layers.resize(L);
+  // per layer [seed cuts | edge cuts | frontier cuts], B + 1 each: device arrays, all sent to
+  // pinned memory by ONE launch behind the last layer (a launch per array after every layer
+  // stood between a layer's relabel and the next layer's sampler)
+  q->cut_sets.reserve(3 * L);
   for (int64_t l = 0; l < L; ++l) {
-    Layer& y = layers[l];
+    QueuedSuperBatch::Layer& y = q->layers[l];
     const int64_t S = seeds.numel();
     auto p = hip::ColSamplingDeferred(csc_->indptr, csc_->indices, seeds, fanouts[l], replace, false,
                                       false, with_data ? &edge : nullptr);
     // queued behind the sampler while its edge count is on its way: where every minibatch's
     // edges start, and the offsets of every minibatch re-based to its own first edge
-    torch::Tensor ids_ptr = p->sub_indptr.index_select(0, ptr);
-    y.offsets = hip::IndptrSplit(p->sub_indptr, ptr, S + B);
+    torch::Tensor ids_ptr;
+    y.offsets = hip::IndptrSplit(p->sub_indptr, ptr, S + B, &ids_ptr);
     // The relabel is queued behind the sampler with the edge count still on the device (it
     // reads its items' number from the offsets; launches and buffers take the sampler's
     // capacity, which a layer fills to nine tenths and more), so a layer has ONE host wait, for
@@ -720,18 +713,44 @@ std::vector<std::vector<torch::Tensor>> Graph::SampleLayersBatched(
       if (with_data) y.data = hip::Slice1d(p->data, 0, nnz);
       std::tie(y.frontier, uni_ptr, y.renamed) = hip::BatchCsrRelabel(seeds, ptr, ids, ids_ptr);
     }
-    // the cuts go to pinned memory by small kernels of the library (a copy call of the runtime
-    // per array cost the host 30-60 us each, a third of the call)
-    y.cuts = torch::empty({3 * (B + 1)}, pinned);
-    hip::PostValues(ptr, y.cuts, 0);
-    hip::PostValues(ids_ptr, y.cuts, B + 1);
-    hip::PostValues(uni_ptr, y.cuts, 2 * (B + 1));
+    q->cut_sets.push_back(ptr);
+    q->cut_sets.push_back(ids_ptr);
+    q->cut_sets.push_back(uni_ptr);
     seeds = y.frontier;
     ptr = uni_ptr;
   }
+  // the cuts of all layers go to pinned memory by a small kernel of the library (a copy call of
+  // the runtime per array cost the host 30-60 us each, a third of the call)
+  q->cuts = torch::empty({3 * L * (B + 1)}, pinned);
+  q->posted = std::make_shared<hip::Posted>(hip::PostValueSets(q->cut_sets, q->cuts));
+  return q;
+}
+
+std::vector<std::vector<torch::Tensor>> QueuedSuperBatch::Collect() {
+  TORCH_CHECK(!collected, "this super-batch has been collected already");
+  collected = true;
+  if (!posted) return std::move(ready);
   // one wait for the cuts of all layers, then views
-  hip::WaitPosted(seeds);
-  hand_out();
+  hip::WaitPosted(*std::static_pointer_cast<hip::Posted>(posted));
+  const int64_t B = num_batches;
+  const int64_t L = static_cast<int64_t>(layers.size());
+  std::vector<std::vector<torch::Tensor>> out(B);
+  for (int64_t b = 0; b < B; ++b) out[b].reserve((with_data ? 4 : 3) * L);
+  for (int64_t l = 0; l < L; ++l) {
+    const Layer& y = layers[l];
+    const int64_t* s_cut = cuts.data_ptr<int64_t>() + 3 * l * (B + 1);
+    const int64_t* e_cut = s_cut + (B + 1);
+    const int64_t* u_cut = e_cut + (B + 1);
+    for (int64_t b = 0; b < B; ++b) {
+      out[b].push_back(hip::Slice1d(y.frontier, u_cut[b], u_cut[b + 1] - u_cut[b]));
+      out[b].push_back(hip::Slice1d(y.offsets, s_cut[b] + b, s_cut[b + 1] - s_cut[b] + 1));
+      out[b].push_back(hip::Slice1d(y.renamed, e_cut[b], e_cut[b + 1] - e_cut[b]));
+      if (with_data) out[b].push_back(hip::Slice1d(y.data, e_cut[b], e_cut[b + 1] - e_cut[b]));
+    }
+  }
+  layers.clear();
+  cut_sets.clear();
+  posted.reset();
   return out;
 }
 

@@ -42,6 +42,25 @@ struct QueuedLayers : public torch::CustomClassHolder {
   std::vector<torch::Tensor> Collect();
 };
 
+// a super-batch queued by Graph::QueueSampleLayersBatched (TORCH_LIBRARY class
+// gs_classes.QueuedSuperBatch): every layer is launched, the per-minibatch cuts are on their
+// way to pinned memory; Collect() waits for them and hands out the per-minibatch views
+struct QueuedSuperBatch : public torch::CustomClassHolder {
+  struct Layer {
+    torch::Tensor frontier, offsets, renamed, data;
+    std::shared_ptr<hip::PendingSample> sample;  // (queued form: kept until the cuts are back)
+  };
+  std::vector<Layer> layers;
+  std::vector<torch::Tensor> cut_sets;  // device arrays the post reads
+  torch::Tensor cuts;                   // pinned: per layer [seed | edge | frontier cuts]
+  std::shared_ptr<void> posted;         // hip::Posted; null: `ready` holds the result
+  int64_t num_batches = 0;
+  bool with_data = false;
+  std::vector<std::vector<torch::Tensor>> ready;
+  bool collected = false;
+  std::vector<std::vector<torch::Tensor>> Collect();
+};
+
 class Graph : public torch::CustomClassHolder {
  public:
   explicit Graph(bool is_subgraph) : is_subgraph_(is_subgraph) {}
@@ -171,6 +190,15 @@ class Graph : public torch::CustomClassHolder {
   // [ptr[b], ptr[b+1]) of one sampler call per layer, so its samples differ from those of a
   // SampleLayers call on the same seeds, while every block is a valid sample of its seeds.
   std::vector<std::vector<torch::Tensor>> SampleLayersBatched(
+      const std::vector<torch::Tensor>& seed_sets, const std::vector<int64_t>& fanouts,
+      bool replace);
+  // The same in two halves: the call returns once the last layer is launched (the waits for
+  // the earlier layers' frontier lengths are inside it), Collect() of the result waits for the
+  // cuts and makes the views.  A caller that queues super-batch i + 1 before it collects
+  // super-batch i has the host's work before the first and after the last launch of a call
+  // (concatenating the seeds, some hundred views and their Python wrappers) run while the
+  // stream is busy with the last layer.
+  c10::intrusive_ptr<QueuedSuperBatch> QueueSampleLayersBatched(
       const std::vector<torch::Tensor>& seed_sets, const std::vector<int64_t>& fanouts,
       bool replace);
   // One layer of a layer-wise (LADIES-style) sampler as ONE call, the operator chain of the

@@ -274,31 +274,44 @@ int64_t ReadTotal(const torch::Tensor& values, int64_t at, void* stream, const c
 }
 }  // namespace
 
-namespace {
-thread_local std::map<int, int64_t> t_last_posted;  // device -> ticket of the last PostValues
-}
-
-void PostValues(const torch::Tensor& values, torch::Tensor& pinned, int64_t at) {
-  NeedI64(values, "values");
+Posted PostValueSets(const std::vector<torch::Tensor>& sets, torch::Tensor& pinned) {
+  Posted posted;
+  if (sets.empty()) return posted;
+  const int64_t n = sets[0].numel();
+  const int device = sets[0].get_device();
+  std::vector<const int64_t*> at(sets.size());
+  for (size_t s = 0; s < sets.size(); ++s) {
+    NeedI64(sets[s], "values");
+    TORCH_CHECK(sets[s].numel() == n && sets[s].get_device() == device,
+                "PostValueSets: the arrays must have one length and one device");
+    at[s] = sets[s].data_ptr<int64_t>();
+  }
   TORCH_CHECK(pinned.is_pinned() && pinned.scalar_type() == torch::kInt64 && pinned.is_contiguous() &&
-                  at >= 0 && at + values.numel() <= pinned.numel(),
-              "PostValues: the target must be pinned int64 memory with room for the values");
-  HostBoxes& boxes = Boxes(values.get_device());
-  const int64_t ticket = boxes.next++;
-  Check(gs_post_values(values.data_ptr<int64_t>(), values.numel(), pinned.data_ptr<int64_t>() + at,
-                       boxes.slot(ticket), ticket, Stream(values)),
-        "gs_post_values");
-  t_last_posted[values.get_device()] = ticket;
+                  static_cast<int64_t>(sets.size()) * n <= pinned.numel(),
+              "PostValueSets: the target must be pinned int64 memory with room for the values");
+  HostBoxes& boxes = Boxes(device);
+  posted.ring = boxes.buf;
+  posted.stream = Stream(sets[0]);
+  constexpr size_t kPerLaunch = 32;  // arrays one launch of the library takes
+  for (size_t first = 0; first < sets.size(); first += kPerLaunch) {
+    const size_t count = std::min(kPerLaunch, sets.size() - first);
+    posted.ticket = boxes.next++;
+    posted.slot = boxes.slot(posted.ticket);
+    Check(gs_post_value_sets(at.data() + first, static_cast<int>(count), n,
+                             pinned.data_ptr<int64_t>() + static_cast<int64_t>(first) * n,
+                             boxes.slot(posted.ticket), posted.ticket, posted.stream),
+          "gs_post_value_sets");
+  }
+  return posted;
 }
 
-void WaitPosted(const torch::Tensor& like) {
-  const int device = like.get_device();
-  auto it = t_last_posted.find(device);
-  if (it == t_last_posted.end()) return;
-  HostBoxes& boxes = Boxes(device);
-  if (WaitBox(boxes.slot(it->second), it->second, Stream(like), "gs_post_values") == kLost)
-    SyncCurrentStream(like);  // the slot went to a later call: wait for the stream instead
-  t_last_posted.erase(it);
+void WaitPosted(const Posted& posted) {
+  if (!posted.slot) return;
+  // (the slot went to a later call: wait for the stream instead)
+  if (WaitBox(static_cast<const gs_mailbox*>(posted.slot), posted.ticket, posted.stream,
+              "gs_post_value_sets") == kLost)
+    TORCH_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(posted.stream)) == hipSuccess,
+                "gs_post_value_sets: the stream failed");
 }
 
 SliceResult ColSlicing(const torch::Tensor& indptr, const torch::Tensor& indices,
@@ -402,11 +415,6 @@ struct Pieces {
   }
 };
 }  // namespace
-
-void SyncCurrentStream(const torch::Tensor& like) {
-  TORCH_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(Stream(like))) == hipSuccess,
-              "hipStreamSynchronize failed");
-}
 
 torch::Tensor Slice1d(const torch::Tensor& t, int64_t first, int64_t count) {
   TORCH_CHECK(t.dim() == 1 && t.is_contiguous() && first >= 0 && count >= 0 &&
@@ -1019,12 +1027,14 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabelQueued(
 }
 
 torch::Tensor IndptrSplit(const torch::Tensor& indptr, const torch::Tensor& offsets,
-                          int64_t total) {
+                          int64_t total, torch::Tensor* cuts) {
   NeedI64(indptr, "indptr");
   NeedI64(offsets, "offsets");
   auto out = torch::empty({total}, I64(indptr));
-  Check(gs_indptr_split(indptr.data_ptr<int64_t>(), offsets.data_ptr<int64_t>(),
-                        offsets.numel() - 1, total, out.data_ptr<int64_t>(), Stream(indptr)),
+  if (cuts) *cuts = torch::empty({offsets.numel()}, I64(indptr));
+  Check(gs_indptr_split_cuts(indptr.data_ptr<int64_t>(), offsets.data_ptr<int64_t>(),
+                             offsets.numel() - 1, total, out.data_ptr<int64_t>(),
+                             cuts ? cuts->data_ptr<int64_t>() : nullptr, Stream(indptr)),
         "gs_indptr_split");
   return out;
 }

@@ -148,14 +148,18 @@ std::shared_ptr<PendingLayers> SampleLayersQueued(const torch::Tensor& indptr,
                                                   const torch::Tensor& seeds,
                                                   const std::vector<int64_t>& fanouts,
                                                   bool replace, const EdgeData* edge = nullptr);
-// values (device int64) -> pinned[at ...] (pinned host memory) by a small kernel on the current
-// stream, without a copy call of the runtime.  WaitPosted() then waits (a mailbox) until the
-// last PostValues of the calling thread on that device has landed, and with it everything
-// queued before it on the same stream.
-void PostValues(const torch::Tensor& values, torch::Tensor& pinned, int64_t at);
-void WaitPosted(const torch::Tensor& like);
-// waits until everything queued on the calling thread's current stream of `like`'s device is done
-void SyncCurrentStream(const torch::Tensor& like);
+// Device int64 arrays of one length -> pinned host memory, back to back, by a small kernel on
+// the current stream (one launch per 32 arrays), without a copy call of the runtime.
+// WaitPosted() then waits (a mailbox) until the last of them has landed, and with it everything
+// queued before it on the same stream; any thread may wait.
+struct Posted {
+  const void* slot = nullptr;  // the mailbox of the last launch; null: nothing was posted
+  torch::Tensor ring;          // keeps the mailbox alive
+  int64_t ticket = 0;
+  void* stream = nullptr;
+};
+Posted PostValueSets(const std::vector<torch::Tensor>& sets, torch::Tensor& pinned);
+void WaitPosted(const Posted& posted);
 // t[first : first + count] of a contiguous 1-d tensor, sharing its storage: what narrow()
 // gives, made without a trip through the operator dispatcher (a super-batch hands back a few
 // hundred such views per call).
@@ -199,8 +203,9 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabelQueued(
     const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& ids,
     const torch::Tensor& ids_ptr, int64_t* num_unique);
 // the batches' offsets, re-based, back to back (host_offsets: the same offsets on the host)
+// cuts (optional): receives indptr[offsets], where every batch's edges start, from the same launch
 torch::Tensor IndptrSplit(const torch::Tensor& indptr, const torch::Tensor& offsets,
-                          int64_t total);
+                          int64_t total, torch::Tensor* cuts = nullptr);
 
 torch::Tensor RandomWalk(const torch::Tensor& seeds, int64_t length, const torch::Tensor& indptr,
                          const torch::Tensor& indices);

@@ -134,6 +134,12 @@ int gs_post_total(const int64_t* value, gs_mailbox* mailbox, int64_t ticket, voi
  * NULL): offsets a caller cuts its results by reach the host without a copy call. */
 int gs_post_values(const int64_t* values, int64_t n, int64_t* host_out, gs_mailbox* mailbox,
                    int64_t ticket, void* stream);
+/* Several arrays of the same length in one launch: sets is a HOST array of num_sets (at most 32)
+ * device pointers, host_out receives sets[0][0..n), sets[1][0..n), ... one after the other, then
+ * {num_sets * n, ticket} goes to the mailbox.  No counterpart in the reference (it reads
+ * such offsets back one tensor at a time, examples/graphsage/batching.py:75-80). */
+int gs_post_value_sets(const int64_t* const* sets, int num_sets, int64_t n, int64_t* host_out,
+                       gs_mailbox* mailbox, int64_t ticket, void* stream);
 
 /* Neighbour copy (slicing.cu:101-119).  nnz = sub_indptr[S] as read back by the
  * caller.  coo_col may be NULL (WITH_COO = false); select_index may be NULL when
@@ -800,6 +806,12 @@ int gs_coo2csc(const void* key, const void* value, int id_bytes, int64_t E, int6
  * offsets[b+1]-offsets[b]+1 entries, re-based to start at 0, one batch after the other. */
 int gs_indptr_split(const int64_t* indptr, const int64_t* offsets, int64_t num_batches,
                     int64_t total, int64_t* out, void* stream);
+/* The same launch also leaves cuts[b] = indptr[offsets[b]], b = 0..num_batches (device int64,
+ * may be NULL): where every batch's edges start, the third result of the GetBatchCSC call in
+ * the reference's super-batch example (examples/graphsage/batching.py:67), without a separate
+ * indexing launch. */
+int gs_indptr_split_cuts(const int64_t* indptr, const int64_t* offsets, int64_t num_batches,
+                         int64_t total, int64_t* out, int64_t* cuts, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Super-batch plumbing.  A batched array is a flat array plus device int64     */

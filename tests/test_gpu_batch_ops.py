@@ -456,3 +456,87 @@ def test_sample_layers_batched_on_a_graph_with_id_maps_goes_minibatch_by_minibat
     for a, b in zip(got, want):
         for x, y in zip(a, b):
             assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("with_data", [False, True])
+def test_super_batches_queued_ahead_equal_the_calls_one_by_one(dev, with_data):
+    """_CAPI_QueueSampleLayersBatched: three super-batches, each queued before the one before it
+    is collected (and the last two collected out of order), give what three
+    _CAPI_SampleLayersBatched calls give under the same seeds; a handle collects once; a graph
+    with id maps (minibatch by minibatch inside) goes through the same two halves."""
+    import graph_sampling_amd as gs
+    n = 1 << 15
+    indptr, indices = rmat_csc_np(n, 1 << 20, seed=43)
+    rng = np.random.default_rng(9)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(to_dev(indptr, dev), to_dev(indices, dev, torch.int32))
+    if with_data:
+        g._CAPI_SetData(to_dev((1.0 - rng.random(indices.size)).astype(np.float32), dev))
+    fanouts = [15, 10]
+    groups = [[to_dev(rng.permutation(n)[:s].astype(np.int64), dev, torch.int32) for s in sizes]
+              for sizes in ([1024] * 64, [300, 0, 1, 1024, 77], [1024] * 48)]
+    gs.set_seed(900)
+    want = [g._CAPI_SampleLayersBatched(sets, fanouts, False) for sets in groups]
+    gs.set_seed(900)
+    h0 = g._CAPI_QueueSampleLayersBatched(groups[0], fanouts, False)
+    h1 = g._CAPI_QueueSampleLayersBatched(groups[1], fanouts, False)
+    got = [h0.collect()]
+    h2 = g._CAPI_QueueSampleLayersBatched(groups[2], fanouts, False)
+    last = h2.collect()
+    got += [h1.collect(), last]
+    for a, b in zip(got, want):
+        assert len(a) == len(b)
+        for x, y in zip(a, b):
+            assert len(x) == len(y) == (4 if with_data else 3) * len(fanouts)
+            for u, v in zip(x, y):
+                assert torch.equal(u, v)
+    with pytest.raises(RuntimeError, match="collected already"):
+        h1.collect()
+    gs.set_seed(900)
+    res = gs.queue_sample_blocks_batched(g, groups[0], fanouts).collect()
+    assert len(res) == 64 and torch.equal(res[3][0], want[0][3][-(4 if with_data else 3)])
+    # a graph the one launch sequence does not take
+    col_ids = to_dev(np.random.default_rng(1).permutation(n).astype(np.int64), dev)
+    m = gs.Graph(False)
+    m._CAPI_LoadCSCWithColIds(col_ids, to_dev(indptr, dev), to_dev(indices, dev))
+    sets = [to_dev(np.arange(100, dtype=np.int64), dev), to_dev(np.arange(50, 90, dtype=np.int64), dev)]
+    gs.set_seed(5)
+    loop = [m._CAPI_SampleLayers(x, [4], False) for x in sets]
+    gs.set_seed(5)
+    queued = m._CAPI_QueueSampleLayersBatched(sets, [4], False).collect()
+    for a, b in zip(queued, loop):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("sizes", [[5], [0, 3, 0, 0, 7], [300, 1, 0, 5000, 257, 256], [0, 0, 0]])
+def test_indptr_split_with_cuts_through_the_c_abi(dev, sizes):
+    """gs_indptr_split_cuts: the re-based offsets of every batch back to back, and where each
+    batch's edges start (indptr[offsets]) from the same launch; closed form in numpy."""
+    rng = np.random.default_rng(sum(sizes) + len(sizes))
+    cols = int(sum(sizes))
+    deg = rng.integers(0, 9, size=cols)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    ptr = _ptr(sizes)
+    want = np.concatenate([indptr[ptr[b]:ptr[b + 1] + 1] - indptr[ptr[b]] for b in range(len(sizes))])
+    plain = capi.indptr_split(to_dev(indptr, dev), to_dev(ptr, dev))
+    out, cuts = capi.indptr_split(to_dev(indptr, dev), to_dev(ptr, dev), with_cuts=True)
+    assert np.array_equal(_np(plain), want)
+    assert np.array_equal(_np(out), want)
+    assert np.array_equal(_np(cuts), indptr[ptr])
+
+
+def test_offsets_reach_pinned_memory_by_one_launch(dev):
+    """gs_post_values / gs_post_value_sets: device arrays arrive in pinned host memory, in order,
+    with the mailbox telling how many values were stored."""
+    rng = np.random.default_rng(5)
+    box = capi.Mailbox()
+    for n, k in [(65, 9), (1, 1), (1000, 32), (0, 3)]:
+        sets = [rng.integers(-2**62, 2**62, size=n).astype(np.int64) for _ in range(k)]
+        got = capi.post_value_sets([to_dev(s, dev) for s in sets], box)
+        assert (got.is_pinned() or n == 0) and tuple(got.shape) == (k, n)
+        assert np.array_equal(got.numpy(), np.stack(sets) if n else np.zeros((k, 0), np.int64))
+        one = capi.post_values(to_dev(sets[0], dev), box)
+        assert np.array_equal(one.numpy(), sets[0])
+    with pytest.raises(capi.GsError):
+        capi.post_value_sets([to_dev(np.zeros(4, np.int64), dev)] * 33, box)
