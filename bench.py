@@ -824,8 +824,9 @@ def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted):
     results = []
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    ahead = queued(groups[0])
-    for grp in groups[1:]:
+    qa_groups = groups + groups  # (every call draws with fresh seeds: no call repeats another)
+    ahead = queued(qa_groups[0])
+    for grp in qa_groups[1:]:
         nxt = queued(grp)
         results.append(ahead.collect())
         ahead = nxt
@@ -865,7 +866,9 @@ def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted):
         "layers_S_E_U": sb_sizes,
         "api": "gs_classes.Graph._CAPI_SampleLayersBatched (one call per super-batch)",
         "queued_ahead": {
-            "ms_per_call": qa_s / len(groups) * 1e3, "value": qa_edges / qa_s,
+            "calls": len(qa_groups), "ms_per_call": qa_s / len(qa_groups) * 1e3,
+            "value": qa_edges / qa_s,
+            "gpu_busy_frac": gpu_ms * 1e-3 / (qa_s / len(qa_groups)),
             "what": "_CAPI_QueueSampleLayersBatched of super-batch i + 1 before .collect() of "
                     "super-batch i (one thread, one stream)"},
         "through_python_ops": {
