@@ -594,7 +594,7 @@ def graphsage(cx, workload, weighted, with_features, full, cpu_budget):
 
     # the throughput form on the same graph: 64 minibatches per call
     if extras and full != "config2":
-        out["super_batch"] = super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted)
+        out["super_batch"] = super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted, workload)
 
     # u_dot_v with 64-d fp32 node features on every block (the large configuration's second half)
     if extras and with_features:
@@ -701,7 +701,7 @@ def graphsage(cx, workload, weighted, with_features, full, cpu_budget):
             "ms_per_step": nf_s / nf_steps * 1e3, "value": nf_e / nf_s, "steps": nf_steps,
             "what": "Slicing -> Sampling -> Relabel per layer instead of the fused sampler"}
 
-        out["super_batch"] = super_batch_leg(torch, graph, timer, fresh_seeds, b, False)
+        out["super_batch"] = super_batch_leg(torch, graph, timer, fresh_seeds, b, False, workload)
 
         # the same minibatches with 64-bit ids, the reference's only id type
         if idt == torch.int32:
@@ -787,7 +787,7 @@ def graphsage(cx, workload, weighted, with_features, full, cpu_budget):
     return out
 
 
-def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted):
+def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted, workload):
     """SUPER minibatches per call on seed sets of its own: what the kernels reach once a launch
     holds enough work for the chip."""
     per = 4 if weighted else 3
@@ -879,6 +879,9 @@ def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted):
                      "achieved": sb_bytes / t3 / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": sb_bytes / t3 / 1e9 / HBM_PEAK_GBS, "launch_us": t3 * 1e6,
                      "algorithmic_bytes": sb_bytes,
+                     "traffic": traffic_from_profile("super_batch", workload)
+                     if sb_dom == "sample_fused" and not weighted else None,
+                     "traffic_source": "profiles/super_batch_%s_hbm_counters.txt" % workload,
                      "gpu_ms_by_site": {k: round(v[0], 4) for k, v in sb_sites.items()}},
         "step_roofline": {"bound": "hbm", "achieved": call_bytes / (sb_s / len(groups)) / 1e9,
                           "peak": HBM_PEAK_GBS, "unit": "GB/s",
