@@ -85,16 +85,26 @@ def sample_layers(matrix, seeds, fanouts, replace=False):
     return _blocks_of(graph._CAPI_SampleLayers(seeds, list(fanouts), bool(replace)), len(fanouts))
 
 
-def sample_blocks(matrix, seed_sets, fanouts, replace=False, workers=4, seed=0):
+def sample_blocks(matrix, seed_sets, fanouts, replace=False, workers=4, seed=0, per_call=None):
     """GraphSAGE-style minibatches sampled side by side by `workers` host threads of the C++
     layer, one stream each (fused slice + sample, relabel, next seeds = frontier, per layer).
     Returns [(input_nodes, [Block, ...] innermost layer first)] in the order of `seed_sets`;
-    minibatch i draws with seeds `seed + i * len(fanouts) + layer` whichever thread runs it."""
+    minibatch i draws with seeds `seed + i * len(fanouts) + layer` whichever thread runs it.
+    With `per_call` the seed sets go that many at a time as super-batches (the flow of
+    `sample_blocks_batched`) through one thread of the pool, which queues its next super-batch
+    before it collects the one before (`workers` must be 1: super-batches side by side are
+    switched off in the library); group g then draws with seeds
+    `seed + g * per_call * len(fanouts) + layer`."""
     import torch
     load_library()
     graph = getattr(matrix, "_graph", matrix)
-    flat = torch.ops.gs_ops._CAPI_SampleBlocks(graph, list(seed_sets), list(fanouts), bool(replace),
-                                               int(workers), int(seed))
+    if per_call is None:
+        flat = torch.ops.gs_ops._CAPI_SampleBlocks(graph, list(seed_sets), list(fanouts),
+                                                   bool(replace), int(workers), int(seed))
+    else:
+        flat = torch.ops.gs_ops._CAPI_SampleBlocksBatched(graph, list(seed_sets), list(fanouts),
+                                                          bool(replace), int(workers),
+                                                          int(per_call), int(seed))
     return [_blocks_of(parts, len(fanouts)) for parts in flat]
 
 

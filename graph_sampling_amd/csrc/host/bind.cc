@@ -161,6 +161,7 @@ TORCH_LIBRARY(gs_ops, m) {
   m.def("_CAPI_SetSeed", &SetSeed);
   m.def("_CAPI_SetThreadSeed", &SetThreadSeed);
   m.def("_CAPI_SampleBlocks", &SampleBlocks);
+  m.def("_CAPI_SampleBlocksBatched", &SampleBlocksBatched);
   m.def("_CAPI_SetSampleAlgo", &SetSampleAlgo);
   // not in the reference: on = float sums of a COO-only graph add in edge order (same bits
   // every run) at the price of sorting its edges first

@@ -93,6 +93,44 @@ c10::hip::HIPStream WorkerStream(int device) {
   return it->second;
 }
 
+// Runs work(k), k = 0..nthreads-1, on the pool's threads, each under its own stream of `device`
+// behind everything the caller's current stream holds so far; rethrows the first failure.
+void RunOnPool(int64_t nthreads, const c10::Device& device,
+               const std::function<void(int64_t)>& work) {
+  // what the caller queued so far (the seeds) must be visible to the workers' streams
+  const auto caller = c10::hip::getCurrentHIPStream(device.index());
+  hipEvent_t ready;
+  TORCH_CHECK(hipEventCreateWithFlags(&ready, hipEventDisableTiming) == hipSuccess,
+              "hipEventCreate failed");
+  TORCH_CHECK(hipEventRecord(ready, caller.stream()) == hipSuccess, "hipEventRecord failed");
+  std::exception_ptr failure;
+  std::mutex failure_lock;
+  auto guarded = [&](int64_t k) {
+    try {
+      c10::hip::HIPGuard device_guard(device.index());
+      const auto stream = WorkerStream(device.index());
+      c10::hip::HIPStreamGuard stream_guard(stream);
+      TORCH_CHECK(hipStreamWaitEvent(stream.stream(), ready, 0) == hipSuccess,
+                  "hipStreamWaitEvent failed");
+      work(k);
+      TORCH_CHECK(hipStreamSynchronize(stream.stream()) == hipSuccess, "hipStreamSynchronize failed");
+    } catch (...) {
+      std::lock_guard<std::mutex> hold(failure_lock);
+      if (!failure) failure = std::current_exception();
+    }
+  };
+  {
+    Pool& pool = ThePool();
+    std::lock_guard<std::mutex> turn(pool.one_call);
+    while (static_cast<int64_t>(pool.workers.size()) < nthreads)
+      pool.workers.push_back(std::make_unique<Worker>());
+    for (int64_t k = 0; k < nthreads; ++k) pool.workers[k]->Start([&guarded, k] { guarded(k); });
+    for (int64_t k = 0; k < nthreads; ++k) pool.workers[k]->Wait();
+  }
+  (void)hipEventDestroy(ready);
+  if (failure) std::rethrow_exception(failure);
+}
+
 }  // namespace
 
 std::vector<std::vector<torch::Tensor>> SampleBlocks(const c10::intrusive_ptr<Graph>& graph,
@@ -109,74 +147,98 @@ std::vector<std::vector<torch::Tensor>> SampleBlocks(const c10::intrusive_ptr<Gr
                 "every seed set must be a tensor on the same GPU");
   const auto device = seed_sets[0].device();
   graph->CreateSparseFormat(_CSC);  // the one lazy step of the shared graph, done before the threads start
-  // what the caller queued so far (the seeds) must be visible to the workers' streams
-  const auto caller = c10::hip::getCurrentHIPStream(device.index());
-  hipEvent_t ready;
-  TORCH_CHECK(hipEventCreateWithFlags(&ready, hipEventDisableTiming) == hipSuccess,
-              "hipEventCreate failed");
-  TORCH_CHECK(hipEventRecord(ready, caller.stream()) == hipSuccess, "hipEventRecord failed");
-
   const int64_t nthreads = workers < n ? workers : n;
-  std::exception_ptr failure;
-  std::mutex failure_lock;
-  auto work = [&](int64_t k) {
-    try {
-      c10::hip::HIPGuard device_guard(device.index());
-      const auto stream = WorkerStream(device.index());
-      c10::hip::HIPStreamGuard stream_guard(stream);
-      TORCH_CHECK(hipStreamWaitEvent(stream.stream(), ready, 0) == hipSuccess,
-                  "hipStreamWaitEvent failed");
-      // Minibatches whose layers can all be queued without a host read are queued a few
-      // ahead of the one being collected, so the stream never waits for this thread.
-      constexpr int64_t kAhead = 8;
-      std::vector<std::pair<int64_t, std::shared_ptr<hip::PendingLayers>>> window;
-      auto collect_oldest = [&] {
-        const int64_t i = window.front().first;
-        auto pending = std::move(window.front().second);
-        window.erase(window.begin());
-        try {
-          out[i] = pending->Collect();
-        } catch (const hip::IdsTooWide&) {
-          // ids beyond 32 bits: what was queued behind it used the same tables, so all of it
-          // is done again, layer by layer, like every later minibatch of this thread
-          std::vector<int64_t> redo{i};
-          for (auto& w : window) redo.push_back(w.first);
-          window.clear();
-          for (int64_t j : redo) {
-            hip::SetThreadSeed(static_cast<uint64_t>(first_seed + j * layers));
-            out[j] = graph->SampleLayersLoop(seed_sets[j], fanouts, replace);
-          }
-        }
-      };
-      for (int64_t i = k; i < n; i += nthreads) {
-        hip::SetThreadSeed(static_cast<uint64_t>(first_seed + i * layers));
-        auto pending = graph->QueueLayers(seed_sets[i], fanouts, replace);
-        if (pending) {
-          window.emplace_back(i, std::move(pending));
-          if (static_cast<int64_t>(window.size()) > kAhead) collect_oldest();
-        } else {
-          while (!window.empty()) collect_oldest();
-          hip::SetThreadSeed(static_cast<uint64_t>(first_seed + i * layers));
-          out[i] = graph->SampleLayersLoop(seed_sets[i], fanouts, replace);
+  RunOnPool(nthreads, device, [&](int64_t k) {
+    // Minibatches whose layers can all be queued without a host read are queued a few
+    // ahead of the one being collected, so the stream never waits for this thread.
+    constexpr int64_t kAhead = 8;
+    std::vector<std::pair<int64_t, std::shared_ptr<hip::PendingLayers>>> window;
+    auto collect_oldest = [&] {
+      const int64_t i = window.front().first;
+      auto pending = std::move(window.front().second);
+      window.erase(window.begin());
+      try {
+        out[i] = pending->Collect();
+      } catch (const hip::IdsTooWide&) {
+        // ids beyond 32 bits: what was queued behind it used the same tables, so all of it
+        // is done again, layer by layer, like every later minibatch of this thread
+        std::vector<int64_t> redo{i};
+        for (auto& w : window) redo.push_back(w.first);
+        window.clear();
+        for (int64_t j : redo) {
+          hip::SetThreadSeed(static_cast<uint64_t>(first_seed + j * layers));
+          out[j] = graph->SampleLayersLoop(seed_sets[j], fanouts, replace);
         }
       }
-      while (!window.empty()) collect_oldest();
-      TORCH_CHECK(hipStreamSynchronize(stream.stream()) == hipSuccess, "hipStreamSynchronize failed");
-    } catch (...) {
-      std::lock_guard<std::mutex> hold(failure_lock);
-      if (!failure) failure = std::current_exception();
+    };
+    for (int64_t i = k; i < n; i += nthreads) {
+      hip::SetThreadSeed(static_cast<uint64_t>(first_seed + i * layers));
+      auto pending = graph->QueueLayers(seed_sets[i], fanouts, replace);
+      if (pending) {
+        window.emplace_back(i, std::move(pending));
+        if (static_cast<int64_t>(window.size()) > kAhead) collect_oldest();
+      } else {
+        while (!window.empty()) collect_oldest();
+        hip::SetThreadSeed(static_cast<uint64_t>(first_seed + i * layers));
+        out[i] = graph->SampleLayersLoop(seed_sets[i], fanouts, replace);
+      }
     }
-  };
-  {
-    Pool& pool = ThePool();
-    std::lock_guard<std::mutex> turn(pool.one_call);
-    while (static_cast<int64_t>(pool.workers.size()) < nthreads)
-      pool.workers.push_back(std::make_unique<Worker>());
-    for (int64_t k = 0; k < nthreads; ++k) pool.workers[k]->Start([&work, k] { work(k); });
-    for (int64_t k = 0; k < nthreads; ++k) pool.workers[k]->Wait();
-  }
-  (void)hipEventDestroy(ready);
-  if (failure) std::rethrow_exception(failure);
+    while (!window.empty()) collect_oldest();
+  });
+  return out;
+}
+
+// The same pool, a super-batch per task: the seed sets are cut into groups of `per_call`, a
+// group is one Graph::QueueSampleLayersBatched call, and a thread queues its next group before
+// it collects the one before.  Written for several threads (two super-batches in flight: the
+// kernels of one -- a sampler that waits for HBM, relabel passes that wait for the L2s -- fill
+// what the other leaves idle), of which only one is admitted for now, see below.  Group g draws with the seeds first_seed + g * per_call * layers + layer (a
+// group that has to go minibatch by minibatch takes layers seeds per minibatch from there),
+// whatever thread runs it.
+std::vector<std::vector<torch::Tensor>> SampleBlocksBatched(
+    const c10::intrusive_ptr<Graph>& graph, std::vector<torch::Tensor> seed_sets,
+    std::vector<int64_t> fanouts, bool replace, int64_t workers, int64_t per_call,
+    int64_t first_seed) {
+  const int64_t n = static_cast<int64_t>(seed_sets.size());
+  const int64_t layers = static_cast<int64_t>(fanouts.size());
+  std::vector<std::vector<torch::Tensor>> out(n);
+  if (n == 0 || layers == 0) return out;
+  TORCH_CHECK(workers >= 1 && workers <= 16, "workers must be in 1..16, got ", workers);
+  TORCH_CHECK(per_call >= 1, "per_call must be positive, got ", per_call);
+  // Switched off: with two workers this call gave the expected results in its tests and
+  // 0.98 ms per super-batch on a weighted 111 M-node graph, and then, repeated on the same
+  // graph with ten groups per call, the process ended with a GPU memory fault whose cause
+  // has not been found.  One worker (one super-batch ahead on the pool's stream) stays.
+  TORCH_CHECK(workers == 1,
+              "super-batches side by side (workers > 1) are switched off: a run of two in flight "
+              "ended in a GPU memory fault that is not explained yet; use workers = 1, or "
+              "_CAPI_QueueSampleLayersBatched from the calling thread");
+  for (const auto& s : seed_sets)
+    TORCH_CHECK(s.defined() && s.is_cuda() && s.device() == seed_sets[0].device(),
+                "every seed set must be a tensor on the same GPU");
+  const auto device = seed_sets[0].device();
+  graph->CreateSparseFormat(_CSC);  // the one lazy step of the shared graph, done before the threads start
+  const int64_t groups = (n + per_call - 1) / per_call;
+  const int64_t nthreads = workers < groups ? workers : groups;
+  RunOnPool(nthreads, device, [&](int64_t k) {
+    int64_t ahead_group = -1;
+    c10::intrusive_ptr<QueuedSuperBatch> ahead;
+    auto collect = [&] {
+      auto parts = ahead->Collect();
+      for (size_t b = 0; b < parts.size(); ++b) out[ahead_group * per_call + b] = std::move(parts[b]);
+      ahead.reset();
+    };
+    for (int64_t g = k; g < groups; g += nthreads) {
+      const int64_t lo = g * per_call, hi = std::min(n, lo + per_call);
+      std::vector<torch::Tensor> sets(seed_sets.begin() + lo, seed_sets.begin() + hi);
+      hip::SetThreadSeed(static_cast<uint64_t>(first_seed + g * per_call * layers));
+      auto queued = graph->QueueSampleLayersBatched(sets, fanouts, replace);
+      if (ahead) collect();
+      ahead = std::move(queued);
+      ahead_group = g;
+    }
+    if (ahead) collect();
+  });
   return out;
 }
 

@@ -17,4 +17,13 @@ std::vector<std::vector<torch::Tensor>> SampleBlocks(const c10::intrusive_ptr<Gr
                                                      std::vector<int64_t> fanouts, bool replace,
                                                      int64_t workers, int64_t first_seed);
 
+// The same pool with a super-batch per task: the seed sets go `per_call` at a time through
+// Graph::QueueSampleLayersBatched, a thread queues its next group before it collects the one
+// before (`workers` must be 1 for now: super-batches side by side are switched off).  Group g (seed sets g * per_call ...) draws with
+// the seeds first_seed + g * per_call * layers + layer whatever thread runs it.
+std::vector<std::vector<torch::Tensor>> SampleBlocksBatched(
+    const c10::intrusive_ptr<Graph>& graph, std::vector<torch::Tensor> seed_sets,
+    std::vector<int64_t> fanouts, bool replace, int64_t workers, int64_t per_call,
+    int64_t first_seed);
+
 }  // namespace gs
