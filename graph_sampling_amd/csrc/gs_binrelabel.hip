@@ -31,6 +31,11 @@
 // buckets store to (flags, renamed ids, frontier) are a megabyte or two that stays in that
 // XCD's L2 until its lines are full.
 //
+// The ids may come from a sampler that is still running when the relabel is queued, and whose
+// total is then read from the offsets on the device.  A sampler that failed leaves a negative
+// last offset: every pass then leaves at once and the call reports -1, as a look-back of its
+// own that gave up would.
+//
 // An LDS table that fills up (a bucket with more than its slots' worth of distinct ids: only
 // a batch beyond ~16 M distinct ids can do that) raises an error word and the call reports
 // -4: the caller repeats it on hash regions (GS_RELABEL_REGIONS).
@@ -100,7 +105,7 @@ __global__ void __launch_bounds__(512) bins_plan_kernel(BatchItems<IdT> x, Plan 
   int64_t classes = 0;
   uint32_t lg = 0;
   if (b < x.B) {
-    const int64_t m = x.start(b + 1) - x.start(b);
+    const int64_t m = x.ids_ptr[x.B] < 0 ? 0 : x.start(b + 1) - x.start(b);
     const int64_t want = (m + (int64_t(1) << kBucketItemsLog2) - 1) >> kBucketItemsLog2;
     while ((int64_t(1) << lg) < want && lg < kMaxClassesLog2) ++lg;
     classes = int64_t(1) << lg;
@@ -127,6 +132,7 @@ struct TileWalk {
     x.stage_offsets(s_seeds_ptr, s_ids_ptr);
     const int64_t held = x.seeds_ptr[x.B] + x.ids_ptr[x.B];
     if (held < M) M = held;
+    if (x.ids_ptr[x.B] < 0) return false;  // the producer of the ids failed
     if (static_cast<int64_t>(blockIdx.x) * kPartTile >= M) return false;
     for (int64_t b = threadIdx.x; b <= x.B; b += kThreads) {
       s_base[b] = p.bucket_base[b];
@@ -397,6 +403,7 @@ bins_rank_kernel(Bins s, int64_t M, int64_t B, const int64_t* __restrict__ seeds
     int64_t total = s_prefix + tile_total;
     const unsigned int err = __hip_atomic_load(lb.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (err) total = err == 2u ? -2 : (err == 3u ? -4 : -1);
+    if (ids_ptr[B] < 0) total = -1;  // the producer of the ids failed: nothing was relabelled
     *num_unique = total;
     unique_ptr[B] = total;
     post_mailbox(box, total, box_ticket);
@@ -425,6 +432,7 @@ bins_rename_kernel(BatchItems<IdT> x, int64_t M, Bins s, IdT* __restrict__ uniqu
   {  // (M may be a bound: the offsets hold the true count)
     const int64_t held = x.seeds_ptr[x.B] + x.ids_ptr[x.B];
     if (held < M) M = held;
+    if (x.ids_ptr[x.B] < 0) return;  // the producer of the ids failed: no records were made
   }
   const int64_t chunks = (M + kRenameTile - 1) / kRenameTile;
   const int64_t per = (chunks + kXcds - 1) / kXcds;

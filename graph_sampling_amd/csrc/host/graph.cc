@@ -701,7 +701,7 @@ c10::intrusive_ptr<QueuedSuperBatch> Graph::QueueSampleLayersBatched(
     int64_t U = -1;
     if (hip::BatchedNoWait())
       std::tie(y.frontier, uni_ptr, y.renamed) =
-          hip::BatchCsrRelabelQueued(seeds, ptr, p->indices, ids_ptr, &U);
+          hip::BatchCsrRelabelQueued(seeds, ptr, p->indices, ids_ptr, &U, p.get());
     hip::CountBatchedNoWait(U >= 0);
     if (U >= 0) {
       y.frontier = hip::Slice1d(y.frontier, 0, U);

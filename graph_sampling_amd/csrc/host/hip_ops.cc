@@ -988,7 +988,7 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(
 
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabelQueued(
     const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& ids,
-    const torch::Tensor& ids_ptr, int64_t* num_unique) {
+    const torch::Tensor& ids_ptr, int64_t* num_unique, const PendingSample* producer) {
   const int idb = IdBytes(seeds, "seeds");
   TORCH_CHECK(IdBytes(ids, "indices") == idb, "seeds and indices differ in dtype");
   NeedI64(seeds_ptr, "seeds_ptr");
@@ -1021,7 +1021,13 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabelQueued(
   int64_t U = WaitBox(boxes.slot(ticket), ticket, st, "gs_batch_csr_relabel");
   if (U == kLost) U = num.item<int64_t>();
   if (U == kTooWide) t_narrow_ids = false;
-  TORCH_CHECK(U != kGaveUp, "gs_batch_csr_relabel: a tile gave up waiting for its predecessors");
+  if (U == kGaveUp) {
+    // either the sampler the ids come from failed (its last offset is negative and the relabel
+    // left at once: Wait() reports it and clears the sampler's look-back state) or a tile of
+    // the relabel's own scan gave up (its state lives in the workspace and is gone with it)
+    if (producer) producer->Wait();
+    TORCH_CHECK(false, "gs_batch_csr_relabel: a tile gave up waiting for its predecessors");
+  }
   *num_unique = U;
   return {unique, unique_ptr, out_ids};
 }

@@ -196,12 +196,14 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabel(
 // outputs are sized by the buffer.  {unique (room for all items), unique_ptr, renamed ids (room
 // for all ids)}; *num_unique = the frontiers' total length, waited for here, or a status the
 // caller answers by waiting for the edge count and calling BatchCsrRelabel: -2 an id too wide,
-// -4 a bucket's table full.  Undefined tensors and *num_unique untouched when the path through
+// -4 a bucket's table full.  `producer`: the sampler the ids come from; when the relabel reports
+// that it left because that sampler failed, the sampler is waited for, which raises its error
+// and clears its look-back state.  Undefined tensors and *num_unique untouched when the path through
 // bins is not the one to take the call (ids that do not ride in 32 bits, more than 511 batches,
 // fewer than 2^19 items by the buffers' sizes).
 std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> BatchCsrRelabelQueued(
     const torch::Tensor& seeds, const torch::Tensor& seeds_ptr, const torch::Tensor& ids,
-    const torch::Tensor& ids_ptr, int64_t* num_unique);
+    const torch::Tensor& ids_ptr, int64_t* num_unique, const PendingSample* producer = nullptr);
 // the batches' offsets, re-based, back to back (host_offsets: the same offsets on the host)
 // cuts (optional): receives indptr[offsets], where every batch's edges start, from the same launch
 torch::Tensor IndptrSplit(const torch::Tensor& indptr, const torch::Tensor& offsets,

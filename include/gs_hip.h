@@ -540,7 +540,8 @@ size_t gs_batch_relabel_workspace_bytes(int64_t num_items);
  * the true counts are seeds_ptr[num_batches] and ids_ptr[num_batches] on the device, launches
  * and workspace (gs_batch_relabel_bins_workspace_bytes(bound, num_batches) suffices) are sized
  * by the bounds.  A caller can so queue a relabel behind a sampler whose edge count it has not
- * read. */
+ * read.  A negative ids_ptr[num_batches] (the total a failed one-launch sampler leaves in its
+ * offsets) makes every pass leave at once and *num_unique = -1. */
 size_t gs_batch_relabel_bins_workspace_bytes(int64_t num_items, int64_t num_batches);
 int gs_batch_csr_relabel(const void* seeds, const int64_t* seeds_ptr, const void* ids,
                          const int64_t* ids_ptr, int64_t num_batches, int64_t num_seeds,

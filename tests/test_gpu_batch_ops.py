@@ -540,3 +540,33 @@ def test_offsets_reach_pinned_memory_by_one_launch(dev):
         assert np.array_equal(one.numpy(), sets[0])
     with pytest.raises(capi.GsError):
         capi.post_value_sets([to_dev(np.zeros(4, np.int64), dev)] * 33, box)
+
+
+def test_super_batch_reports_a_sampler_that_gave_up(dev):
+    """A layer's relabel is queued behind its sampler before anyone has read the sampler's total.
+    With the sampler's error word raised from the host (every kernel runs to its end) the total it
+    leaves is negative: the relabel's passes leave at once, the call raises, the host layer clears
+    the sampler's state behind it, and the next call is right again."""
+    import graph_sampling_amd as gs
+    n = 1 << 15
+    indptr, indices = rmat_csc_np(n, 1 << 20, seed=47)
+    rng = np.random.default_rng(4)
+    t_ptr = to_dev(indptr, dev)
+    g = gs.Graph(False)
+    g._CAPI_LoadCSC(t_ptr, to_dev(indices, dev, torch.int32))
+    sets = [to_dev(rng.permutation(n)[:1024].astype(np.int64), dev, torch.int32) for _ in range(64)]
+    fanouts = [15, 10]
+    gs.set_seed(40)
+    want = g._CAPI_SampleLayersBatched(sets, fanouts, False)
+    torch.ops.gs_ops._CAPI_DebugRaiseLookbackError(t_ptr)
+    through, _ = torch.ops.gs_ops._CAPI_BatchedNoWaitCounts()
+    with pytest.raises(RuntimeError, match="gave up"):
+        g._CAPI_SampleLayersBatched(sets, fanouts, False)
+    for _ in range(2):
+        gs.set_seed(40)
+        got = g._CAPI_SampleLayersBatched(sets, fanouts, False)
+        for a, b in zip(got, want):
+            for x, y in zip(a, b):
+                assert torch.equal(x, y)
+    # (the calls that went through did so with every layer's relabel queued behind its sampler)
+    assert torch.ops.gs_ops._CAPI_BatchedNoWaitCounts()[0] >= through + 2 * len(fanouts)
