@@ -879,8 +879,10 @@ def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted, workload):
                      "achieved": sb_bytes / t3 / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": sb_bytes / t3 / 1e9 / HBM_PEAK_GBS, "launch_us": t3 * 1e6,
                      "algorithmic_bytes": sb_bytes,
+                     # (the summaries were taken on the large graph with its edge weights and on
+                     # config 2 without any)
                      "traffic": traffic_from_profile("super_batch", workload)
-                     if sb_dom == "sample_fused" and not weighted else None,
+                     if sb_dom == "sample_fused" and weighted == (workload == LARGE) else None,
                      "traffic_source": "profiles/super_batch_%s_hbm_counters.txt" % workload,
                      "gpu_ms_by_site": {k: round(v[0], 4) for k, v in sb_sites.items()}},
         "step_roofline": {"bound": "hbm", "achieved": call_bytes / (sb_s / len(groups)) / 1e9,
