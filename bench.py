@@ -856,6 +856,8 @@ def super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted, workload):
     # the dominant site's largest launch (the third layer) against its bytes
     S3, E3, U3 = sb_sizes[-1]
     sb_bytes = SUPER_SITES[sb_dom](b, S3, E3, U3)
+    if weighted and sb_dom == "sample_fused":
+        sb_bytes += 8 * E3  # a weight read and written per sampled edge
     t3 = max(sb_sites[sb_dom][1]) * 1e-3
     gpu_ms = sum(v[0] for v in sb_sites.values())
     call_bytes = step_bytes(sb_sizes, weighted)
