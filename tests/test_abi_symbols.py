@@ -57,3 +57,18 @@ def test_python_binding_rejects_cpu_tensors():
     indptr = torch.zeros(3, dtype=torch.int64)
     with pytest.raises(capi.GsError, match="no CPU path"):
         capi.slice_count(indptr, torch.zeros(2, dtype=torch.int64))
+
+
+def test_every_entry_point_names_what_it_replaces():
+    """Each declaration of the header stands under a comment (its own or its section's) that cites
+    the reference interface it replaces as file:line, or says that it has no counterpart there."""
+    lines = open(os.path.join(ROOT, "include", "gs_hip.h")).read().split("\n")
+    uncited = []
+    for i, line in enumerate(lines):
+        m = re.match(r"^(int|size_t|int64_t|const char\*)\s+(gs_[a-z0-9_]+)\s*\(", line)
+        if not m:
+            continue
+        above = "\n".join(lines[max(0, i - 60):i])
+        if not re.search(r"(src/|examples/|tests/|python/)[A-Za-z_/\.]+:\d+|counterpart", above, re.I):
+            uncited.append(m.group(2))
+    assert not uncited, uncited
