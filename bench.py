@@ -353,6 +353,17 @@ def saturated(torch, graph, timer, nodes, idt, dev, b):
             "frac": achieved / HBM_PEAK_GBS}
 
 
+def leg(fn):
+    """A secondary leg must not take the headline with it: when it raises, the traceback goes to
+    stderr and the line carries {"error": ...} under the leg's key."""
+    try:
+        return fn()
+    except Exception as e:  # noqa: BLE001 -- whatever it is, the headline is still worth printing
+        import traceback
+        traceback.print_exc()
+        return {"error": "%s: %s" % (type(e).__name__, str(e)[:500])}
+
+
 def timed(torch, fn, sets):
     torch.cuda.synchronize()
     t1 = time.perf_counter()
@@ -594,7 +605,8 @@ def graphsage(cx, workload, weighted, with_features, full, cpu_budget):
 
     # the throughput form on the same graph: 64 minibatches per call
     if extras and full != "config2":
-        out["super_batch"] = super_batch_leg(torch, graph, timer, fresh_seeds, b, weighted, workload)
+        out["super_batch"] = leg(lambda: super_batch_leg(torch, graph, timer, fresh_seeds, b,
+                                                         weighted, workload))
 
     # u_dot_v with 64-d fp32 node features on every block (the large configuration's second half)
     if extras and with_features:
@@ -701,7 +713,8 @@ def graphsage(cx, workload, weighted, with_features, full, cpu_budget):
             "ms_per_step": nf_s / nf_steps * 1e3, "value": nf_e / nf_s, "steps": nf_steps,
             "what": "Slicing -> Sampling -> Relabel per layer instead of the fused sampler"}
 
-        out["super_batch"] = super_batch_leg(torch, graph, timer, fresh_seeds, b, False, workload)
+        out["super_batch"] = leg(lambda: super_batch_leg(torch, graph, timer, fresh_seeds, b, False,
+                                                         workload))
 
         # the same minibatches with 64-bit ids, the reference's only id type
         if idt == torch.int32:
@@ -1224,12 +1237,12 @@ def main():
     out.update(head)
     if not args.headline_only:
         if "config_2" in legs and args.workload != SAGE:
-            out["config_2"] = graphsage(cx, SAGE, False, with_features=False, full="config2",
-                                        cpu_budget=6.0)
+            out["config_2"] = leg(lambda: graphsage(cx, SAGE, False, with_features=False,
+                                                    full="config2", cpu_budget=6.0))
         if "ladies" in legs:
-            out["ladies"] = ladies(cx, cpu_budget=6.0)
+            out["ladies"] = leg(lambda: ladies(cx, cpu_budget=6.0))
         if "walks" in legs:
-            out["walks"] = walks(cx, cpu_budget=1.0)
+            out["walks"] = leg(lambda: walks(cx, cpu_budget=1.0))
     print(json.dumps(out))
 
 

@@ -51,3 +51,9 @@ def test_byte_models_are_the_stated_formulas():
     assert bench.compact_bytes(4, 0, S, E, U) == 20 * (S + E) + 4 * U
     # the published peak the fractions are taken against
     assert bench.HBM_PEAK_GBS == 8000.0
+
+
+def test_a_failing_secondary_leg_is_recorded_and_does_not_raise():
+    assert bench.leg(lambda: {"value": 1}) == {"value": 1}
+    got = bench.leg(lambda: [][1])
+    assert set(got) == {"error"} and got["error"].startswith("IndexError")
