@@ -207,8 +207,11 @@ std::vector<std::vector<torch::Tensor>> SampleBlocksBatched(
   TORCH_CHECK(per_call >= 1, "per_call must be positive, got ", per_call);
   // Switched off: with two workers this call gave the expected results in its tests and
   // 0.98 ms per super-batch on a weighted 111 M-node graph, and then, repeated on the same
-  // graph with ten groups per call, the process ended with a GPU memory fault whose cause
-  // has not been found.  One worker (one super-batch ahead on the pool's stream) stays.
+  // graph with ten groups per call, the process ended with a GPU memory fault.  The likely
+  // mechanism: two chip-filling launches with chained scans share the workgroup slots, the
+  // waiting tiles of one can keep the other's lowest tile from starting and the other way
+  // round, and after the bounded wait the tiles give up and leave offsets that are none.
+  // One worker (one super-batch ahead on the pool's stream) stays.
   TORCH_CHECK(workers == 1,
               "super-batches side by side (workers > 1) are switched off: a run of two in flight "
               "ended in a GPU memory fault that is not explained yet; use workers = 1, or "
