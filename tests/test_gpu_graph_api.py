@@ -908,8 +908,9 @@ def test_sample_blocks_pool_equals_the_python_loop(dev, workers):
 
 
 _TWO_IN_FLIGHT_OFF = ("switched off in the library: two super-batches in flight passed here and then "
-                      "ended a bench run on the weighted 111 M-node graph with a GPU memory fault "
-                      "whose cause has not been found")
+                      "ended a bench run on the weighted 111 M-node graph with a GPU memory fault; the "
+                      "likely cause (chained scans of two chip-filling launches starving each other) "
+                      "has not been shown on the device")
 
 
 @pytest.mark.parametrize("workers", [1, pytest.param(2, marks=pytest.mark.skip(reason=_TWO_IN_FLIGHT_OFF)),
